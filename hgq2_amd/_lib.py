@@ -1,0 +1,102 @@
+"""ctypes binding of ``libhgq_hip.so`` (declared in ``include/hgq_hip.h``).
+
+There is no CPU fallback: if the library is missing or a call fails, this raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'libhgq_hip.so')
+
+# mode bits, mirrored from include/hgq_hip.h
+TRN, RND, RND_CONV = 0, 1, 2
+WRAP, SAT, SAT_SYM = 0, 1, 2
+MODE_TRAINING = 1 << 8
+MODE_KBI = 1 << 9
+MODE_ROUND_PARAMS = 1 << 10
+MODE_K_U8 = 1 << 11
+MODE_SYMMETRIC = 1 << 12
+MODE_TRACING = 1 << 13
+ACT_NONE, ACT_RELU = 0, 1
+
+ROUND_MODES = {'TRN': TRN, 'RND': RND, 'RND_CONV': RND_CONV}
+OVERFLOW_MODES = {'WRAP': WRAP, 'SAT': SAT, 'SAT_SYM': SAT_SYM}
+
+ERRORS = {-1: 'HGQ_ERR_ARG', -2: 'HGQ_ERR_LAUNCH', -3: 'HGQ_ERR_UNSUPPORTED'}
+
+# name -> (restype, argtypes); exactly the declarations of include/hgq_hip.h
+SIGNATURES = {
+    'hgq_version': (c_int, []),
+    'hgq_last_error': (c_char_p, []),
+    'hgq_quantize_fwd': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    'hgq_quantize_bwd': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    'hgq_wrap_track_i': (c_int, [c_void_p] * 5 + [c_int64, c_float, c_float, c_float, c_int, c_void_p]),
+    'hgq_qdense_fwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 4 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_qdense_bwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_dense_ebops': (
+        c_int,
+        [c_void_p] * 3 + [c_int64, c_int, c_int] + [c_void_p] * 4 + [c_float, c_float, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p],
+    ),
+    'hgq_sparse_ce_fwd_bwd': (c_int, [c_void_p] * 4 + [c_int64, c_int, c_void_p]),
+    'hgq_sgd_update': (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_float, c_void_p]),
+    'hgq_fill_u32': (c_int, [c_void_p, ctypes.c_uint32, c_int64, c_void_p]),
+}
+
+_lib = None
+
+
+class HGQLibraryError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library; raise if it has not been built (``python -c 'import __graft_entry__ as g; g.build()'``)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HGQLibraryError(
+            f'{LIB_PATH} not found: the HIP extension is not built. Run `make -C hgq2_amd/csrc` '
+            '(or __graft_entry__.build()). There is no CPU fallback.'
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().hgq_last_error()
+        raise HGQLibraryError(f'{what} failed with {ERRORS.get(rc, rc)}: {msg.decode() if msg else ""}')
+
+
+def mode_bits(round_mode: str, overflow_mode: str, *, training=False, kbi=False, round_params=False, k_u8=False,
+              symmetric=False, tracing=False) -> int:
+    rm = round_mode.upper()
+    if rm.startswith('S_'):
+        rm = rm[2:]
+    try:
+        m = ROUND_MODES[rm] | (OVERFLOW_MODES[overflow_mode.upper()] << 4)
+    except KeyError as e:
+        raise ValueError(f'unsupported round/overflow mode {round_mode}/{overflow_mode}') from e
+    if training:
+        m |= MODE_TRAINING
+    if kbi:
+        m |= MODE_KBI
+    if round_params:
+        m |= MODE_ROUND_PARAMS
+    if k_u8:
+        m |= MODE_K_U8
+    if symmetric:
+        m |= MODE_SYMMETRIC
+    if tracing:
+        m |= MODE_TRACING
+    return m

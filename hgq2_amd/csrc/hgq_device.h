@@ -1,0 +1,146 @@
+// Device-side core of the fixed-point quantizer, shared by every kernel family.
+//
+// All arithmetic is the same sequence of IEEE-754 fp32 operations the reference's eager
+// Keras path performs (scale by an exact power of two, add 0.5, floor, scale back, compare,
+// select), so results are bit-identical to it; powers of two are built from the exponent
+// (v_ldexp_f32) and never through exp2f/powf/log2f.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/hgq_hip.h"
+
+#define HGQ_LN2 0.69314718055994530942f
+
+namespace hgq {
+
+struct Mode {
+    int round_mode, overflow_mode;
+    bool training, kbi, round_params, k_u8, symmetric, tracing;
+    __host__ __device__ explicit Mode(int m)
+        : round_mode(m & 0xf), overflow_mode((m >> 4) & 0xf), training(m & HGQ_MODE_TRAINING),
+          kbi(m & HGQ_MODE_KBI), round_params(m & HGQ_MODE_ROUND_PARAMS), k_u8(m & HGQ_MODE_K_U8),
+          symmetric(m & HGQ_MODE_SYMMETRIC), tracing(m & HGQ_MODE_TRACING) {}
+};
+
+// 2**e for an integer-valued float e (exact, including subnormal results).
+__device__ __forceinline__ float pow2(float e) { return ldexpf(1.0f, (int)e); }
+
+template <int RM>
+__device__ __forceinline__ float round_scaled(float t) {
+    if (RM == HGQ_TRN) return floorf(t);
+    if (RM == HGQ_RND) return floorf(__fadd_rn(t, 0.5f));
+    return rintf(t);  // RND_CONV: round half to even
+}
+
+// xq = R(x * 2**f) / 2**f.  Scaling by ldexp equals the multiply / divide by the fp32 value
+// 2**f wherever that value is finite and the result normal.
+template <int RM>
+__device__ __forceinline__ float fixed_round(float x, float f) {
+    const int fi = (int)f;
+    return ldexpf(round_scaled<RM>(ldexpf(x, fi)), -fi);
+}
+
+__device__ __forceinline__ float load_k(const void *k, int64_t idx, bool k_u8) {
+    return k_u8 ? (float)((const uint8_t *)k)[idx] : ((const float *)k)[idx];
+}
+
+// Resolve (k, i, f) of one bit-width entry from the stored operands.
+struct KIF {
+    float k, i, f;
+};
+
+__device__ __forceinline__ KIF resolve_kif(float k, float i, float fb, bool kbi, bool round_params) {
+    if (round_params) {
+        i = rintf(i);
+        fb = rintf(fb);
+    }
+    KIF r;
+    r.k = k;
+    r.i = i;
+    r.f = kbi ? __fsub_rn(fb, i) : fb;
+    return r;
+}
+
+// Overflow handling of an already-rounded value.  Returns the output; `state` is 0 inside the
+// range, bit 0 set above the upper bound, bit 1 set below the lower bound (SAT modes only).
+template <int OM>
+__device__ __forceinline__ float overflow(float xq, const KIF &p, bool training, int &state) {
+    state = 0;
+    if (OM == HGQ_WRAP) {
+        if (training) return xq;
+        const float bias = p.k * pow2(p.i);
+        const float ik = __fadd_rn(p.i, p.k);
+        const float m = pow2(ik);
+        const float a = __fadd_rn(xq, bias);
+        // floor-mod by a power of two: a - floor(a / m) * m is exact
+        const float q = floorf(ldexpf(a, -(int)ik));
+        return __fsub_rn(__fmaf_rn(-q, m, a), bias);
+    }
+    const float eps = pow2(-p.f);
+    const float hi = __fsub_rn(pow2(p.i), eps);
+    const float lo = (OM == HGQ_SAT) ? -p.k * pow2(p.i) : -p.k * hi;
+    // both comparisons are evaluated: for an empty word (upper bound below the lower bound) a
+    // value can violate both, the upper bound wins in the forward and both bounds take gradient
+    const bool over = xq > hi, under = xq < lo;
+    state = (over ? 1 : 0) | (under ? 2 : 0);
+    return over ? hi : (under ? lo : xq);
+}
+
+template <int RM, int OM>
+__device__ __forceinline__ float quantize(float x, const KIF &p, bool training) {
+    int st;
+    float y = overflow<OM>(fixed_round<RM>(x, p.f), p, training, st);
+    if (!training && !(p.k + p.i + p.f > 0.0f)) y = 0.0f;
+    return y;
+}
+
+// Surrogate backward of one element (training mode).  Outputs the gradients w.r.t. x, i, f.
+template <int RM, int OM>
+__device__ __forceinline__ void quantize_grad(float x, float dy, const KIF &p, float &dx, float &di, float &df) {
+    const float xq = fixed_round<RM>(x, p.f);
+    int st = 0;
+    if (OM != HGQ_WRAP) (void)overflow<OM>(xq, p, true, st);
+    if (st == 0) {
+        dx = dy;
+        di = 0.0f;
+        df = -HGQ_LN2 * (xq - x) * dy;
+    } else {
+        dx = 0.0f;
+        const float gi = HGQ_LN2 * pow2(p.i) * dy;
+        const float gf = HGQ_LN2 * pow2(-p.f) * dy;
+        di = 0.0f, df = 0.0f;
+        if (st & 1) {
+            di += gi;
+            df += gf;
+        }
+        if (st & 2) {
+            di += -p.k * gi;
+            if (OM == HGQ_SAT_SYM) df += -p.k * gf;
+        }
+    }
+}
+
+// Bit pattern of |v| as an unsigned integer: monotone for non-negative floats, so an integer
+// atomic max is a float max.  NaN payloads compare above every finite value and propagate.
+__device__ __forceinline__ uint32_t abs_bits(float v) { return __float_as_uint(v) & 0x7fffffffu; }
+
+}  // namespace hgq
+
+// dispatch a (round_mode, overflow_mode) pair to template arguments
+#define HGQ_DISPATCH_RM_OM(RMV, OMV, ...)                                   \
+    do {                                                                    \
+        switch ((RMV) * 4 + (OMV)) {                                        \
+            case HGQ_TRN * 4 + HGQ_WRAP: { constexpr int RM = HGQ_TRN, OM = HGQ_WRAP; __VA_ARGS__; } break;         \
+            case HGQ_TRN * 4 + HGQ_SAT: { constexpr int RM = HGQ_TRN, OM = HGQ_SAT; __VA_ARGS__; } break;           \
+            case HGQ_TRN * 4 + HGQ_SAT_SYM: { constexpr int RM = HGQ_TRN, OM = HGQ_SAT_SYM; __VA_ARGS__; } break;   \
+            case HGQ_RND * 4 + HGQ_WRAP: { constexpr int RM = HGQ_RND, OM = HGQ_WRAP; __VA_ARGS__; } break;         \
+            case HGQ_RND * 4 + HGQ_SAT: { constexpr int RM = HGQ_RND, OM = HGQ_SAT; __VA_ARGS__; } break;           \
+            case HGQ_RND * 4 + HGQ_SAT_SYM: { constexpr int RM = HGQ_RND, OM = HGQ_SAT_SYM; __VA_ARGS__; } break;   \
+            case HGQ_RND_CONV * 4 + HGQ_WRAP: { constexpr int RM = HGQ_RND_CONV, OM = HGQ_WRAP; __VA_ARGS__; } break;       \
+            case HGQ_RND_CONV * 4 + HGQ_SAT: { constexpr int RM = HGQ_RND_CONV, OM = HGQ_SAT; __VA_ARGS__; } break;         \
+            case HGQ_RND_CONV * 4 + HGQ_SAT_SYM: { constexpr int RM = HGQ_RND_CONV, OM = HGQ_SAT_SYM; __VA_ARGS__; } break; \
+            default: return hgq::fail(HGQ_ERR_ARG, "unknown round/overflow mode");                                          \
+        }                                                                   \
+    } while (0)

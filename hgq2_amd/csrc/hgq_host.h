@@ -1,0 +1,47 @@
+// Host-side helpers shared by the C-ABI entry points: error reporting and launch checks.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/hgq_hip.h"
+
+namespace hgq {
+
+int fail(int code, const char *fmt, ...);  // records a thread-local message, returns `code`
+
+inline int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HGQ_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return HGQ_OK;
+}
+
+// Number of workgroups for a persistent (grid-stride) launch: enough to fill all 256 CUs of
+// an MI355X several times over without exceeding the work available.
+inline int persistent_grid(int64_t work_items, int per_cu = 4) {
+    static int n_cu = 0;
+    if (n_cu == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n_cu = prop.multiProcessorCount;
+        if (n_cu <= 0) n_cu = 256;
+    }
+    int64_t g = (int64_t)n_cu * per_cu;
+    if (g > work_items) g = work_items;
+    if (g < 1) g = 1;
+    return (int)g;
+}
+
+__global__ void fill_u32_kernel(uint32_t *p, uint32_t v, int64_t n);
+int fill_u32(uint32_t *p, uint32_t v, int64_t n, hipStream_t s);
+inline int fill_f32(float *p, float v, int64_t n, hipStream_t s) {
+    union {
+        float f;
+        uint32_t u;
+    } c;
+    c.f = v;
+    return fill_u32((uint32_t *)p, c.u, n, s);
+}
+
+}  // namespace hgq

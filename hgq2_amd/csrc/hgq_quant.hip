@@ -1,0 +1,571 @@
+// Fixed-point quantizer kernels: forward, surrogate backward, integer-bit tracking.
+//
+// Three layouts of the bit-width operands are served:
+//   per-element  (bw_size == n)            1-D kernel, 128-bit loads of x, k, i, f
+//   shared       (bw_size == 1)            1-D kernel, operands in registers, one reduction per launch
+//   per-column   (bw_inner == 1, x = [rows, bw_size])  2-D kernel: a thread owns fixed columns
+//                and walks down the rows, so bit-widths and the partial reductions stay in
+//                registers; one atomic per column per workgroup at the end
+// plus a scalar fallback for bw_inner > 1.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "hgq_device.h"
+#include "hgq_host.h"
+
+namespace hgq {
+
+static thread_local char g_err[256] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+__global__ void fill_u32_kernel(uint32_t *p, uint32_t v, int64_t n) {
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (int64_t)gridDim.x * blockDim.x) p[t] = v;
+}
+
+int fill_u32(uint32_t *p, uint32_t v, int64_t n, hipStream_t s) {
+    if (n <= 0) return HGQ_OK;
+    int grid = (int)((n + 255) / 256);
+    if (grid > 2048) grid = 2048;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(grid), dim3(256), 0, s, p, v, n);
+    return check_launch("fill");
+}
+
+// ------------------------------------------------------------------------------------------
+// wavefront (64 lanes) and workgroup reductions
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        uint32_t t = (uint32_t)__shfl_xor((int)v, o, 64);
+        v = t > v ? t : v;
+    }
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_or_u32(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v |= (uint32_t)__shfl_xor((int)v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+template <int VEC>
+struct VecIO;
+template <>
+struct VecIO<1> {
+    static __device__ __forceinline__ void load(const float *p, int64_t v, float *o) { o[0] = p[v]; }
+    static __device__ __forceinline__ void store(float *p, int64_t v, const float *o) { p[v] = o[0]; }
+    static __device__ __forceinline__ void load_k(const void *k, int64_t v, bool u8, float *o) { o[0] = hgq::load_k(k, v, u8); }
+    static __device__ __forceinline__ void store_u32(uint32_t *p, int64_t v, const uint32_t *o) { p[v] = o[0]; }
+};
+template <>
+struct VecIO<4> {
+    static __device__ __forceinline__ void load(const float *p, int64_t v, float *o) {
+        float4 t = ((const float4 *)p)[v];
+        o[0] = t.x, o[1] = t.y, o[2] = t.z, o[3] = t.w;
+    }
+    static __device__ __forceinline__ void store(float *p, int64_t v, const float *o) {
+        ((float4 *)p)[v] = make_float4(o[0], o[1], o[2], o[3]);
+    }
+    static __device__ __forceinline__ void load_k(const void *k, int64_t v, bool u8, float *o) {
+        if (u8) {
+            uchar4 t = ((const uchar4 *)k)[v];
+            o[0] = t.x, o[1] = t.y, o[2] = t.z, o[3] = t.w;
+        } else {
+            load((const float *)k, v, o);
+        }
+    }
+    static __device__ __forceinline__ void store_u32(uint32_t *p, int64_t v, const uint32_t *o) {
+        ((uint4 *)p)[v] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+};
+
+// ------------------------------------------------------------------------------------------
+// 1-D kernels: per-element or shared bit-widths
+// ------------------------------------------------------------------------------------------
+template <int RM, int OM, int VEC, bool SHARED>
+__global__ __launch_bounds__(256) void quant_fwd_1d(const float *__restrict__ x, const void *__restrict__ k,
+                                                    const float *__restrict__ i, const float *__restrict__ fb,
+                                                    float *__restrict__ y, uint32_t *amax, uint32_t *anyneg,
+                                                    int64_t nvec, int mode) {
+    const Mode m(mode);
+    KIF ps;
+    if (SHARED) ps = resolve_kif(load_k(k, 0, m.k_u8), i[0], fb[0], m.kbi, m.round_params);
+    uint32_t lmax = 0, lneg = 0;
+    for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+        float xv[VEC], kv[VEC], iv[VEC], fv[VEC], yv[VEC];
+        VecIO<VEC>::load(x, v, xv);
+        if (!SHARED) {
+            VecIO<VEC>::load_k(k, v, m.k_u8, kv);
+            VecIO<VEC>::load(i, v, iv);
+            VecIO<VEC>::load(fb, v, fv);
+        }
+        uint32_t ab[VEC], ng[VEC];
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            const KIF p = SHARED ? ps : resolve_kif(kv[c], iv[c], fv[c], m.kbi, m.round_params);
+            yv[c] = quantize<RM, OM>(xv[c], p, m.training);
+            ab[c] = abs_bits(yv[c]);
+            ng[c] = yv[c] < 0.0f ? 1u : 0u;
+            lmax = ab[c] > lmax ? ab[c] : lmax;
+            lneg |= ng[c];
+        }
+        VecIO<VEC>::store(y, v, yv);
+        if (!SHARED) {
+            if (amax) VecIO<VEC>::store_u32(amax, v, ab);
+            if (anyneg) VecIO<VEC>::store_u32(anyneg, v, ng);
+        }
+    }
+    if (SHARED && (amax || anyneg)) {
+        __shared__ uint32_t smax[4], sneg[4];
+        lmax = wave_max_u32(lmax);
+        lneg = wave_or_u32(lneg);
+        if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = lmax, sneg[threadIdx.x >> 6] = lneg;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint32_t a = smax[0], g = sneg[0];
+            for (int w = 1; w < 4; ++w) a = smax[w] > a ? smax[w] : a, g |= sneg[w];
+            if (amax) atomicMax(amax, a);
+            if (anyneg && g) atomicOr(anyneg, 1u);
+        }
+    }
+}
+
+template <int RM, int OM, int VEC, bool SHARED>
+__global__ __launch_bounds__(256) void quant_bwd_1d(const float *__restrict__ dy, const float *__restrict__ x,
+                                                    const void *__restrict__ k, const float *__restrict__ i,
+                                                    const float *__restrict__ fb, float *__restrict__ dx,
+                                                    float *di, float *dfb, int64_t nvec, int mode) {
+    const Mode m(mode);
+    KIF ps;
+    if (SHARED) ps = resolve_kif(load_k(k, 0, m.k_u8), i[0], fb[0], m.kbi, m.round_params);
+    float si = 0.0f, sf = 0.0f;
+    for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+        float gv[VEC], xv[VEC], kv[VEC], iv[VEC], fv[VEC], dxv[VEC], div[VEC], dfv[VEC];
+        VecIO<VEC>::load(dy, v, gv);
+        VecIO<VEC>::load(x, v, xv);
+        if (!SHARED) {
+            VecIO<VEC>::load_k(k, v, m.k_u8, kv);
+            VecIO<VEC>::load(i, v, iv);
+            VecIO<VEC>::load(fb, v, fv);
+        }
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            const KIF p = SHARED ? ps : resolve_kif(kv[c], iv[c], fv[c], m.kbi, m.round_params);
+            float gi, gf;
+            quantize_grad<RM, OM>(xv[c], gv[c], p, dxv[c], gi, gf);
+            if (m.kbi) gi -= gf;  // f = b - i
+            div[c] = gi, dfv[c] = gf;
+            si += gi, sf += gf;
+        }
+        if (dx) VecIO<VEC>::store(dx, v, dxv);
+        if (!SHARED) {
+            if (di) VecIO<VEC>::store(di, v, div);
+            if (dfb) VecIO<VEC>::store(dfb, v, dfv);
+        }
+    }
+    if (SHARED) {
+        __shared__ float ssi[4], ssf[4];
+        si = wave_sum_f32(si);
+        sf = wave_sum_f32(sf);
+        if ((threadIdx.x & 63) == 0) ssi[threadIdx.x >> 6] = si, ssf[threadIdx.x >> 6] = sf;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            if (di) atomicAdd(di, ssi[0] + ssi[1] + ssi[2] + ssi[3]);
+            if (dfb) atomicAdd(dfb, ssf[0] + ssf[1] + ssf[2] + ssf[3]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// 2-D kernels: x = [rows, M], one bit-width entry per column
+// thread (tx, ty): tx walks column groups of VEC, ty walks rows; TX is a power of two <= 64
+// ------------------------------------------------------------------------------------------
+template <int RM, int OM, int VEC>
+__global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ x, const void *__restrict__ k,
+                                                      const float *__restrict__ i, const float *__restrict__ fb,
+                                                      float *__restrict__ y, uint32_t *amax, uint32_t *anyneg,
+                                                      int64_t rows, int64_t M, int TX, int mode) {
+    const Mode m(mode);
+    const int TY = 256 / TX;
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t cg = M / VEC;
+    const int64_t c = (int64_t)blockIdx.x * TX + tx;
+    const bool active = c < cg;
+    KIF p[VEC];
+    uint32_t lmax[VEC], lneg[VEC];
+    if (active) {
+        float kv[VEC], iv[VEC], fv[VEC];
+        VecIO<VEC>::load_k(k, c, m.k_u8, kv);
+        VecIO<VEC>::load(i, c, iv);
+        VecIO<VEC>::load(fb, c, fv);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) p[e] = resolve_kif(kv[e], iv[e], fv[e], m.kbi, m.round_params);
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) lmax[e] = 0, lneg[e] = 0;
+    if (active) {
+        for (int64_t r = (int64_t)blockIdx.y * TY + ty; r < rows; r += (int64_t)gridDim.y * TY) {
+            float xv[VEC], yv[VEC];
+            VecIO<VEC>::load(x, r * cg + c, xv);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                yv[e] = quantize<RM, OM>(xv[e], p[e], m.training);
+                const uint32_t ab = abs_bits(yv[e]);
+                lmax[e] = ab > lmax[e] ? ab : lmax[e];
+                lneg[e] |= yv[e] < 0.0f ? 1u : 0u;
+            }
+            VecIO<VEC>::store(y, r * cg + c, yv);
+        }
+    }
+    if (amax || anyneg) {
+        __shared__ uint32_t smax[256 * VEC], sneg[256 * VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) smax[threadIdx.x * VEC + e] = lmax[e], sneg[threadIdx.x * VEC + e] = lneg[e];
+        __syncthreads();
+        for (int s = TY / 2; s > 0; s >>= 1) {
+            if (ty < s) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const uint32_t o = smax[(threadIdx.x + s * TX) * VEC + e];
+                    uint32_t &mine = smax[threadIdx.x * VEC + e];
+                    mine = o > mine ? o : mine;
+                    sneg[threadIdx.x * VEC + e] |= sneg[(threadIdx.x + s * TX) * VEC + e];
+                }
+            }
+            __syncthreads();
+        }
+        if (ty == 0 && active) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if (amax) atomicMax(&amax[c * VEC + e], smax[tx * VEC + e]);
+                if (anyneg && sneg[tx * VEC + e]) atomicOr(&anyneg[c * VEC + e], 1u);
+            }
+        }
+    }
+}
+
+template <int RM, int OM, int VEC>
+__global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ dy, const float *__restrict__ x,
+                                                      const void *__restrict__ k, const float *__restrict__ i,
+                                                      const float *__restrict__ fb, float *__restrict__ dx, float *di,
+                                                      float *dfb, int64_t rows, int64_t M, int TX, int mode) {
+    const Mode m(mode);
+    const int TY = 256 / TX;
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t cg = M / VEC;
+    const int64_t c = (int64_t)blockIdx.x * TX + tx;
+    const bool active = c < cg;
+    KIF p[VEC];
+    float si[VEC], sf[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) si[e] = 0.0f, sf[e] = 0.0f;
+    if (active) {
+        float kv[VEC], iv[VEC], fv[VEC];
+        VecIO<VEC>::load_k(k, c, m.k_u8, kv);
+        VecIO<VEC>::load(i, c, iv);
+        VecIO<VEC>::load(fb, c, fv);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) p[e] = resolve_kif(kv[e], iv[e], fv[e], m.kbi, m.round_params);
+        for (int64_t r = (int64_t)blockIdx.y * TY + ty; r < rows; r += (int64_t)gridDim.y * TY) {
+            float gv[VEC], xv[VEC], dxv[VEC];
+            VecIO<VEC>::load(dy, r * cg + c, gv);
+            VecIO<VEC>::load(x, r * cg + c, xv);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float gi, gf;
+                quantize_grad<RM, OM>(xv[e], gv[e], p[e], dxv[e], gi, gf);
+                if (m.kbi) gi -= gf;
+                si[e] += gi, sf[e] += gf;
+            }
+            if (dx) VecIO<VEC>::store(dx, r * cg + c, dxv);
+        }
+    }
+    __shared__ float ssi[256 * VEC], ssf[256 * VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ssi[threadIdx.x * VEC + e] = si[e], ssf[threadIdx.x * VEC + e] = sf[e];
+    __syncthreads();
+    for (int s = TY / 2; s > 0; s >>= 1) {
+        if (ty < s) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                ssi[threadIdx.x * VEC + e] += ssi[(threadIdx.x + s * TX) * VEC + e];
+                ssf[threadIdx.x * VEC + e] += ssf[(threadIdx.x + s * TX) * VEC + e];
+            }
+        }
+        __syncthreads();
+    }
+    if (ty == 0 && active) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            if (di) atomicAdd(&di[c * VEC + e], ssi[tx * VEC + e]);
+            if (dfb) atomicAdd(&dfb[c * VEC + e], ssf[tx * VEC + e]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// scalar fallback: arbitrary (bw_size, bw_inner); reductions go straight to global atomics
+// ------------------------------------------------------------------------------------------
+template <int RM, int OM>
+__global__ __launch_bounds__(256) void quant_fwd_generic(const float *__restrict__ x, const void *k, const float *i,
+                                                         const float *fb, float *__restrict__ y, uint32_t *amax,
+                                                         uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner,
+                                                         int mode) {
+    const Mode m(mode);
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+        const int64_t b = (e / bw_inner) % bw_size;
+        const KIF p = resolve_kif(load_k(k, b, m.k_u8), i[b], fb[b], m.kbi, m.round_params);
+        const float yv = quantize<RM, OM>(x[e], p, m.training);
+        y[e] = yv;
+        if (amax) atomicMax(&amax[b], abs_bits(yv));
+        if (anyneg && yv < 0.0f) atomicOr(&anyneg[b], 1u);
+    }
+}
+
+template <int RM, int OM>
+__global__ __launch_bounds__(256) void quant_bwd_generic(const float *__restrict__ dy, const float *__restrict__ x,
+                                                         const void *k, const float *i, const float *fb,
+                                                         float *__restrict__ dx, float *di, float *dfb, int64_t n,
+                                                         int64_t bw_size, int64_t bw_inner, int mode) {
+    const Mode m(mode);
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+        const int64_t b = (e / bw_inner) % bw_size;
+        const KIF p = resolve_kif(load_k(k, b, m.k_u8), i[b], fb[b], m.kbi, m.round_params);
+        float gx, gi, gf;
+        quantize_grad<RM, OM>(x[e], dy[e], p, gx, gi, gf);
+        if (m.kbi) gi -= gf;
+        if (dx) dx[e] = gx;
+        if (di && gi != 0.0f) atomicAdd(&di[b], gi);
+        if (dfb && gf != 0.0f) atomicAdd(&dfb[b], gf);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// integer-bit tracking
+// ------------------------------------------------------------------------------------------
+// ceil(log2(v)) for v > 0 from the exponent field: exact, where log2f is only faithfully rounded.
+__device__ __forceinline__ float ceil_log2(float v) {
+    if (!(v > 0.0f)) return v == 0.0f ? -INFINITY : NAN;
+    if (!(v < INFINITY)) return v;
+    int e;
+    const float mant = frexpf(v, &e);  // v = mant * 2**e, mant in [0.5, 1)
+    return (float)(mant == 0.5f ? e - 1 : e);
+}
+
+__global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__restrict__ amax,
+                                                           const uint32_t *__restrict__ anyneg, float *i_var,
+                                                           const float *__restrict__ fb, uint8_t *k_var, int64_t n,
+                                                           float decay, float c_lo, float c_hi, int mode) {
+    const Mode m(mode);
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n) return;
+    const float xr = __uint_as_float(amax[t]);
+    const float raw_i = i_var[t];
+    float mi;
+    if (!m.kbi) {
+        const float f = rintf(fb[t]);
+        mi = ceil_log2(__fadd_rn(xr, pow2(-f)));
+    } else {
+        const float b = rintf(fb[t]);
+        const float eps = 1e-7f;
+        const float num = __fadd_rn(xr, eps);
+        const float den = __fadd_rn(__fsub_rn(1.0f, pow2(-b)), eps);
+        mi = ceilf(log2f(__fdiv_rn(num, den)));
+        if (!m.symmetric && !(b > 0.0f)) mi = 32.0f;
+    }
+    float ni;
+    if (!m.tracing) {
+        ni = fmaxf(__fsub_rn(raw_i, decay), mi);
+        if (m.kbi) ni = fminf(fmaxf(ni, c_lo), c_hi);
+    } else {
+        if (!m.kbi) {
+            mi = fminf(fmaxf(mi, c_lo), c_hi);
+            ni = fmaxf(rintf(raw_i), mi);
+        } else {
+            ni = fminf(fmaxf(fmaxf(rintf(raw_i), mi), c_lo), c_hi);
+        }
+        if (k_var && anyneg && anyneg[t]) k_var[t] = 1;
+    }
+    i_var[t] = ni;
+}
+
+static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+static inline int pow2_floor_le64(int64_t v) {
+    int t = 1;
+    while (t * 2 <= v && t < 64) t *= 2;
+    return t;
+}
+
+}  // namespace hgq
+
+using namespace hgq;
+
+extern "C" int hgq_version(void) { return 1; }
+extern "C" const char *hgq_last_error(void) { return g_err; }
+
+extern "C" int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream) {
+    if (n < 0 || (n > 0 && !p)) return fail(HGQ_ERR_ARG, "hgq_fill_u32: bad arguments");
+    return fill_u32(p, value, n, (hipStream_t)stream);
+}
+
+extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, const float *fb, float *y,
+                                uint32_t *amax, uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner,
+                                int mode, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (n < 0 || bw_size < 1 || bw_inner < 1) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd: bad sizes");
+    if (n == 0) return HGQ_OK;
+    if (!x || !k || !i || !fb || !y) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd: null pointer");
+    if (bw_size * bw_inner > n || n % (bw_size * bw_inner) != 0)
+        return fail(HGQ_ERR_ARG, "hgq_quantize_fwd: n=%lld is not a multiple of bw_size*bw_inner", (long long)n);
+    const Mode m(mode);
+    const bool reduce = bw_size < n;
+    if (reduce) {
+        int rc;
+        if (amax && (rc = fill_u32(amax, 0, bw_size, s))) return rc;
+        if (anyneg && (rc = fill_u32(anyneg, 0, bw_size, s))) return rc;
+    }
+    if (bw_size == n || bw_size == 1) {
+        const bool shared = bw_size == 1 && n > 1;
+        bool vec = aligned16(x) && aligned16(y) && n >= 4;
+        if (!shared) vec = vec && aligned16(i) && aligned16(fb) && ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0 &&
+                           (!amax || aligned16(amax)) && (!anyneg || aligned16(anyneg));
+        const int64_t n4 = vec ? (n / 4) : 0;
+        const int64_t tail0 = n4 * 4, tail = n - tail0;
+        HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+            if (n4 > 0) {
+                const int grid = persistent_grid((n4 + 255) / 256, 8);
+                if (shared)
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 4, true>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n4, mode);
+                else
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 4, false>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n4, mode);
+            }
+            if (tail > 0) {
+                const int grid = persistent_grid((tail + 255) / 256, 8);
+                if (shared) {
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 1, true>), dim3(grid), dim3(256), 0, s, x + tail0, k, i, fb, y + tail0, amax, anyneg, tail, mode);
+                } else {
+                    const void *kt = m.k_u8 ? (const void *)((const uint8_t *)k + tail0) : (const void *)((const float *)k + tail0);
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 1, false>), dim3(grid), dim3(256), 0, s, x + tail0, kt, i + tail0, fb + tail0, y + tail0,
+                                       amax ? amax + tail0 : nullptr, anyneg ? anyneg + tail0 : nullptr, tail, mode);
+                }
+            }
+        });
+        return check_launch("hgq_quantize_fwd");
+    }
+    if (bw_inner == 1) {
+        const int64_t M = bw_size, rows = n / M;
+        const bool vec = (M % 4 == 0) && aligned16(x) && aligned16(y) && aligned16(i) && aligned16(fb) &&
+                         ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0;
+        const int64_t cg = vec ? M / 4 : M;
+        const int TX = pow2_floor_le64(cg), TY = 256 / TX;
+        const int64_t gx = (cg + TX - 1) / TX;
+        int64_t gy = (rows + TY - 1) / TY;
+        const int64_t cap = (int64_t)persistent_grid(1 << 30, 8) / gx;
+        if (gy > cap) gy = cap < 1 ? 1 : cap;
+        HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+            if (vec)
+                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, mode);
+            else
+                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, mode);
+        });
+        return check_launch("hgq_quantize_fwd");
+    }
+    HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+        const int grid = persistent_grid((n + 255) / 256, 8);
+        hipLaunchKernelGGL((quant_fwd_generic<RM, OM>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n, bw_size, bw_inner, mode);
+    });
+    return check_launch("hgq_quantize_fwd");
+}
+
+extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,
+                                float *dx, float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner,
+                                int mode, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (n < 0 || bw_size < 1 || bw_inner < 1) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd: bad sizes");
+    if (n == 0) return HGQ_OK;
+    if (!dy || !x || !k || !i || !fb) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd: null pointer");
+    if (bw_size * bw_inner > n || n % (bw_size * bw_inner) != 0)
+        return fail(HGQ_ERR_ARG, "hgq_quantize_bwd: n=%lld is not a multiple of bw_size*bw_inner", (long long)n);
+    const Mode m(mode);
+    if (!m.training) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd: the surrogate gradient is defined for training mode only");
+    if (bw_size < n) {
+        int rc;
+        if (di && (rc = fill_f32(di, 0.0f, bw_size, s))) return rc;
+        if (dfb && (rc = fill_f32(dfb, 0.0f, bw_size, s))) return rc;
+    }
+    if (bw_size == n || bw_size == 1) {
+        const bool shared = bw_size == 1 && n > 1;
+        bool vec = aligned16(x) && aligned16(dy) && (!dx || aligned16(dx)) && n >= 4;
+        if (!shared) vec = vec && aligned16(i) && aligned16(fb) && ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0 &&
+                           (!di || aligned16(di)) && (!dfb || aligned16(dfb));
+        const int64_t n4 = vec ? (n / 4) : 0;
+        const int64_t tail0 = n4 * 4, tail = n - tail0;
+        HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+            if (n4 > 0) {
+                const int grid = persistent_grid((n4 + 255) / 256, 8);
+                if (shared)
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 4, true>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n4, mode);
+                else
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 4, false>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n4, mode);
+            }
+            if (tail > 0) {
+                const int grid = persistent_grid((tail + 255) / 256, 8);
+                if (shared) {
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 1, true>), dim3(grid), dim3(256), 0, s, dy + tail0, x + tail0, k, i, fb,
+                                       dx ? dx + tail0 : nullptr, di, dfb, tail, mode);
+                } else {
+                    const void *kt = m.k_u8 ? (const void *)((const uint8_t *)k + tail0) : (const void *)((const float *)k + tail0);
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 1, false>), dim3(grid), dim3(256), 0, s, dy + tail0, x + tail0, kt, i + tail0, fb + tail0,
+                                       dx ? dx + tail0 : nullptr, di ? di + tail0 : nullptr, dfb ? dfb + tail0 : nullptr, tail, mode);
+                }
+            }
+        });
+        return check_launch("hgq_quantize_bwd");
+    }
+    if (bw_inner == 1) {
+        const int64_t M = bw_size, rows = n / M;
+        const bool vec = (M % 4 == 0) && aligned16(x) && aligned16(dy) && (!dx || aligned16(dx)) && aligned16(i) &&
+                         aligned16(fb) && ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0;
+        const int64_t cg = vec ? M / 4 : M;
+        const int TX = pow2_floor_le64(cg), TY = 256 / TX;
+        const int64_t gx = (cg + TX - 1) / TX;
+        int64_t gy = (rows + TY - 1) / TY;
+        const int64_t cap = (int64_t)persistent_grid(1 << 30, 8) / gx;
+        if (gy > cap) gy = cap < 1 ? 1 : cap;
+        HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+            if (vec)
+                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, mode);
+            else
+                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, mode);
+        });
+        return check_launch("hgq_quantize_bwd");
+    }
+    HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+        const int grid = persistent_grid((n + 255) / 256, 8);
+        hipLaunchKernelGGL((quant_bwd_generic<RM, OM>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n, bw_size, bw_inner, mode);
+    });
+    return check_launch("hgq_quantize_bwd");
+}
+
+extern "C" int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, float *i_var, const float *fb,
+                                uint8_t *k_var, int64_t m, float decay, float c_lo, float c_hi, int mode, void *stream) {
+    if (m < 0) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i: bad size");
+    if (m == 0) return HGQ_OK;
+    if (!amax || !i_var || !fb) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i: null pointer");
+    hipLaunchKernelGGL(wrap_track_i_kernel, dim3((unsigned)((m + 255) / 256)), dim3(256), 0, (hipStream_t)stream, amax, anyneg, i_var, fb,
+                       k_var, m, decay, c_lo, c_hi, mode);
+    return check_launch("hgq_wrap_track_i");
+}

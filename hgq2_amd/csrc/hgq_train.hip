@@ -1,0 +1,154 @@
+// Training-step kernels around the contractions: EBOPs of a dense contraction (value and
+// gradient in one pass), sparse categorical cross-entropy (value and gradient in one pass),
+// SGD update with the bit-width constraint and MonoL1 gradient folded in.
+#include <math.h>
+
+#include "hgq_device.h"
+#include "hgq_host.h"
+
+namespace hgq {
+
+__device__ __forceinline__ float block_sum_256(float v, float *scratch4) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if ((threadIdx.x & 63) == 0) scratch4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = scratch4[0] + scratch4[1] + scratch4[2] + scratch4[3];
+    __syncthreads();
+    return v;
+}
+
+// bits of one entry and the derivative of bits w.r.t. the fractional / total-bits variable
+__device__ __forceinline__ float entry_bits(const void *k, const float *i, const float *fb, int64_t idx, const Mode &m,
+                                            float &dbits) {
+    float b;
+    if (m.kbi) {
+        b = rintf(fb[idx]);
+        dbits = 1.0f;
+    } else {
+        const float s = __fadd_rn(rintf(i[idx]), rintf(fb[idx]));
+        b = s > 0.0f ? s : 0.0f;
+        dbits = s > 0.0f ? 1.0f : 0.0f;
+    }
+    if (m.overflow_mode == HGQ_SAT) b += load_k(k, idx, m.k_u8);
+    return b;
+}
+
+#define HGQ_EBOPS_MAXK 4096
+
+__global__ __launch_bounds__(256) void dense_ebops_kernel(const void *k_in, const float *i_in, const float *f_in,
+                                                          int64_t P, int K, int N, const void *k_ker,
+                                                          const float *b_ker, const void *k_bias, const float *b_bias,
+                                                          float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
+                                                          float *ebops, uint32_t *ebops_u32, float *g_f_in,
+                                                          float *g_b_ker, float *g_b_bias) {
+    __shared__ float colsum[HGQ_EBOPS_MAXK];  // sum_n bits_ker[k, n]
+    __shared__ float insum[HGQ_EBOPS_MAXK];   // sum_p bits_in[p, k]
+    __shared__ float red[4];
+    const Mode mi(mode_in), mk(mode_ker), mb(mode_bias);
+    const int t = threadIdx.x;
+    for (int k = t; k < K; k += 256) {
+        float s = 0.0f, d;
+        for (int n = 0; n < N; ++n) s += entry_bits(k_ker, nullptr, b_ker, (int64_t)k * N + n, mk, d);
+        colsum[k] = s;
+        float a = 0.0f;
+        for (int64_t p = 0; p < P; ++p) {
+            const float b = entry_bits(k_in, i_in, f_in, p * K + k, mi, d);
+            a += b;
+            if (g_f_in) g_f_in[p * K + k] = d * s * scale;
+        }
+        insum[k] = a;
+    }
+    __syncthreads();
+    float part = 0.0f;
+    for (int k = t; k < K; k += 256) part += insum[k] * colsum[k];
+    float total = block_sum_256(part, red);
+    if (g_b_ker)
+        for (int64_t e = t; e < (int64_t)K * N; e += 256) g_b_ker[e] = insum[e / N] * scale;
+    if (b_bias) {
+        float bs = 0.0f, d;
+        for (int n = t; n < N; n += 256) {
+            bs += entry_bits(k_bias, nullptr, b_bias, n, mb, d);
+            if (g_b_bias) g_b_bias[n] = bias_size / (float)N * scale;
+        }
+        bs = block_sum_256(bs, red);
+        total += bs / (float)N * bias_size;
+    }
+    if (t == 0) {
+        const float e = total * scale;
+        ebops[0] = e;
+        if (ebops_u32) ebops_u32[0] = (uint32_t)e;
+    }
+}
+
+// one thread per row; C is small (class count)
+__global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict__ logits,
+                                                        const int64_t *__restrict__ labels, float *loss,
+                                                        float *__restrict__ dlogits, int64_t rows, int C) {
+    __shared__ float red[4];
+    const float inv_rows = 1.0f / (float)rows;
+    float acc = 0.0f;
+    for (int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x; r < rows; r += (int64_t)gridDim.x * 256) {
+        const float *z = logits + r * C;
+        float mx = z[0];
+        for (int c = 1; c < C; ++c) mx = fmaxf(mx, z[c]);
+        float se = 0.0f;
+        for (int c = 0; c < C; ++c) se += expf(z[c] - mx);
+        const float lse = logf(se);
+        const int64_t lab = labels[r];
+        acc += lse - (z[lab] - mx);
+        if (dlogits) {
+            float *d = dlogits + r * C;
+            const float inv = 1.0f / se;
+            for (int c = 0; c < C; ++c) d[c] = (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows;
+        }
+    }
+    acc = block_sum_256(acc, red);
+    if (threadIdx.x == 0) atomicAdd(loss, acc * inv_rows);
+}
+
+__global__ __launch_bounds__(256) void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, int64_t n,
+                                                  float lr, float l1, float lo, float hi) {
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < n; t += (int64_t)gridDim.x * 256) {
+        const float v = __fsub_rn(w[t], __fmul_rn(lr, __fadd_rn(g[t], l1)));
+        w[t] = fminf(fmaxf(v, lo), hi);
+    }
+}
+
+}  // namespace hgq
+
+using namespace hgq;
+
+extern "C" int hgq_dense_ebops(const void *k_in, const float *i_in, const float *f_in, int64_t P, int K, int N,
+                               const void *k_ker, const float *b_ker, const void *k_bias, const float *b_bias,
+                               float scale, float bias_size, int mode_in, int mode_ker, int mode_bias, float *ebops,
+                               uint32_t *ebops_u32, float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream) {
+    if (P < 1 || K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_dense_ebops: bad sizes");
+    if (!i_in || !f_in || !b_ker || !ebops || !k_in || !k_ker) return fail(HGQ_ERR_ARG, "hgq_dense_ebops: null pointer");
+    if (K > HGQ_EBOPS_MAXK) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops: K=%d > %d", K, HGQ_EBOPS_MAXK);
+    if (!(Mode(mode_ker).kbi) || (b_bias && !(Mode(mode_bias).kbi))) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops: kernel/bias bit-widths must use the KBI parametrisation");
+    hipLaunchKernelGGL(dense_ebops_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, k_in, i_in, f_in, P, K, N, k_ker, b_ker,
+                       k_bias, b_bias, scale, bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
+    return check_launch("hgq_dense_ebops");
+}
+
+extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *loss, float *dlogits,
+                                     int64_t rows, int C, void *stream) {
+    if (rows < 1 || C < 1) return fail(HGQ_ERR_ARG, "hgq_sparse_ce_fwd_bwd: bad sizes");
+    if (!logits || !labels || !loss) return fail(HGQ_ERR_ARG, "hgq_sparse_ce_fwd_bwd: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int rc = fill_f32(loss, 0.0f, 1, s);
+    if (rc) return rc;
+    const int grid = persistent_grid((rows + 255) / 256, 4);
+    hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C);
+    return check_launch("hgq_sparse_ce_fwd_bwd");
+}
+
+extern "C" int hgq_sgd_update(float *w, const float *g, int64_t n, float lr, float l1, float lo, float hi, void *stream) {
+    if (n < 0) return fail(HGQ_ERR_ARG, "hgq_sgd_update: bad size");
+    if (n == 0) return HGQ_OK;
+    if (!w || !g) return fail(HGQ_ERR_ARG, "hgq_sgd_update: null pointer");
+    const int grid = persistent_grid((n + 255) / 256, 8);
+    hipLaunchKernelGGL(sgd_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, w, g, n, lr, l1, lo, hi);
+    return check_launch("hgq_sgd_update");
+}

@@ -1,0 +1,328 @@
+"""``torch.library`` operators over the C ABI of ``libhgq_hip.so``.
+
+Every operator validates its arguments on the host (device, dtype, contiguity, sizes),
+allocates its outputs with torch, and enqueues the HIP kernels on torch's current stream.
+Autograd is attached with ``register_autograd``; the backward formulas call the backward
+entry points of the same library.  There is no CPU implementation: tensors must be on a GPU.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+__all__ = [
+    'quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_',
+]
+
+
+def _ptr(t: Tensor | None):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_f32(name: str, t: Tensor):
+    _need(t.is_cuda, f'{name} must be a GPU tensor (there is no CPU implementation), got device {t.device}')
+    _need(t.dtype == torch.float32, f'{name} must be float32, got {t.dtype}')
+    _need(t.is_contiguous(), f'{name} must be contiguous')
+
+
+def _check_k(name: str, t: Tensor):
+    _need(t.is_cuda, f'{name} must be a GPU tensor')
+    _need(t.dtype in (torch.float32, torch.uint8), f'{name} must be float32 or uint8, got {t.dtype}')
+    _need(t.is_contiguous(), f'{name} must be contiguous')
+
+
+def _kmode(mode: int, k: Tensor) -> int:
+    return (mode | _lib.MODE_K_U8) if k.dtype == torch.uint8 else (mode & ~_lib.MODE_K_U8)
+
+
+# --------------------------------------------------------------------------------------
+# quantizer
+# --------------------------------------------------------------------------------------
+@torch.library.custom_op('hgq::quantize_fwd', mutates_args=())
+def quantize_fwd(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, track: bool) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
+    bw_size = i.numel()
+    _need(k.numel() == bw_size and fb.numel() == bw_size, 'k, i, f must have the same number of elements')
+    n = x.numel()
+    _need(bw_size >= 1 and bw_inner >= 1 and (n == 0 or n % (bw_size * bw_inner) == 0),
+          f'x has {n} elements, not a multiple of bw_size*bw_inner = {bw_size}*{bw_inner}')
+    y = torch.empty_like(x)
+    amax = torch.empty(bw_size if track else 0, dtype=torch.int32, device=x.device)
+    neg = torch.empty(bw_size if track else 0, dtype=torch.int32, device=x.device)
+    rc = _lib.load().hgq_quantize_fwd(_ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(y), _ptr(amax), _ptr(neg), n, bw_size,
+                                      bw_inner, _kmode(mode, k), _stream())
+    _lib.check(rc, 'hgq_quantize_fwd')
+    return y, amax, neg
+
+
+@quantize_fwd.register_fake
+def _(x, k, i, fb, mode, bw_inner, track):
+    m = i.numel() if track else 0
+    return torch.empty_like(x), x.new_empty(m, dtype=torch.int32), x.new_empty(m, dtype=torch.int32)
+
+
+@torch.library.custom_op('hgq::quantize_bwd', mutates_args=())
+def quantize_bwd(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('dy', dy), _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
+    _need(dy.numel() == x.numel(), 'dy and x differ in size')
+    dx = torch.empty_like(x)
+    di = torch.empty_like(i)
+    dfb = torch.empty_like(fb)
+    rc = _lib.load().hgq_quantize_bwd(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), _ptr(di), _ptr(dfb),
+                                      x.numel(), i.numel(), bw_inner, _kmode(mode, k), _stream())
+    _lib.check(rc, 'hgq_quantize_bwd')
+    return dx, di, dfb
+
+
+@quantize_bwd.register_fake
+def _(dy, x, k, i, fb, mode, bw_inner):
+    return torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+
+
+def _quantize_setup(ctx, inputs, output):
+    x, k, i, fb, mode, bw_inner, track = inputs
+    ctx.save_for_backward(x, k, i, fb)
+    ctx.mode, ctx.bw_inner = mode, bw_inner
+
+
+def _quantize_backward(ctx, gy, g_amax, g_neg):
+    x, k, i, fb = ctx.saved_tensors
+    if not (ctx.mode & _lib.MODE_TRAINING):
+        raise RuntimeError('hgq::quantize_fwd: gradients are defined for the training-mode forward only')
+    dx, di, dfb = quantize_bwd(gy.contiguous(), x, k, i, fb, ctx.mode, ctx.bw_inner)
+    return dx, None, di, dfb, None, None, None
+
+
+quantize_fwd.register_autograd(_quantize_backward, setup_context=_quantize_setup)
+
+
+def quantize(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int = 1, track: bool = False):
+    """Fixed-point quantizer.  Returns ``(y, amax_bits, anyneg)``; the last two are empty unless ``track``."""
+    return quantize_fwd(x.contiguous(), k.contiguous(), i.contiguous(), fb.contiguous(), mode, bw_inner, track)
+
+
+@torch.library.custom_op('hgq::wrap_track_i', mutates_args=('i_var', 'k_var'))
+def wrap_track_i_op(amax: Tensor, anyneg: Tensor, i_var: Tensor, fb: Tensor, k_var: Tensor, decay: float, c_lo: float,
+                    c_hi: float, mode: int) -> None:
+    _check_f32('i_var', i_var), _check_f32('fb', fb)
+    m = i_var.numel()
+    _need(amax.numel() == m and amax.dtype == torch.int32 and amax.is_cuda, 'amax must be an int32 GPU tensor matching i_var')
+    _need(fb.numel() == m, 'fb must match i_var')
+    if k_var.numel():
+        _need(k_var.dtype == torch.uint8 and k_var.numel() == m and anyneg.numel() == m, 'k_var must be uint8 matching i_var')
+    rc = _lib.load().hgq_wrap_track_i(_ptr(amax), _ptr(anyneg), _ptr(i_var), _ptr(fb), _ptr(k_var), m, decay, c_lo, c_hi,
+                                      mode, _stream())
+    _lib.check(rc, 'hgq_wrap_track_i')
+
+
+def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('inf'), anyneg=None, k_var=None):
+    empty_i = amax.new_empty(0)
+    empty_k = torch.empty(0, dtype=torch.uint8, device=amax.device)
+    wrap_track_i_op(amax, anyneg if anyneg is not None else empty_i, i_var, fb, k_var if k_var is not None else empty_k,
+                    float(decay), float(c_lo), float(c_hi), mode)
+
+
+# --------------------------------------------------------------------------------------
+# dense contraction with the input quantizer fused into the operand load
+# --------------------------------------------------------------------------------------
+@torch.library.custom_op('hgq::qdense_fwd', mutates_args=())
+def qdense_fwd(x: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, qw: Tensor, qb: Tensor, act: int, mode: int,
+               bw_rows: int, track: bool) -> tuple[Tensor, Tensor]:
+    _check_f32('x', x), _check_f32('qw', qw)
+    _need(x.dim() == 2 and qw.dim() == 2 and x.shape[1] == qw.shape[0], f'shape mismatch {tuple(x.shape)} @ {tuple(qw.shape)}')
+    rows, K = x.shape
+    N = qw.shape[1]
+    if qb.numel():
+        _check_f32('qb', qb)
+        _need(qb.numel() == N, 'bias size mismatch')
+    if bw_rows > 0:
+        _check_k('k_in', k_in), _check_f32('i_in', i_in), _check_f32('f_in', f_in)
+        _need(i_in.numel() == bw_rows * K and f_in.numel() == bw_rows * K and k_in.numel() == bw_rows * K,
+              'input bit-widths must have bw_rows*K elements')
+        _need(rows % bw_rows == 0, 'rows must be a multiple of bw_rows')
+        mode = _kmode(mode, k_in)
+    y = torch.empty((rows, N), dtype=torch.float32, device=x.device)
+    amax = torch.empty(bw_rows * K if (track and bw_rows > 0) else 0, dtype=torch.int32, device=x.device)
+    rc = _lib.load().hgq_qdense_fwd(_ptr(x), _ptr(k_in), _ptr(i_in), _ptr(f_in), bw_rows, _ptr(qw), _ptr(qb), _ptr(y),
+                                    _ptr(amax), rows, K, N, act, mode, _stream())
+    _lib.check(rc, 'hgq_qdense_fwd')
+    return y, amax
+
+
+@qdense_fwd.register_fake
+def _(x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track):
+    return x.new_empty((x.shape[0], qw.shape[1])), x.new_empty(bw_rows * x.shape[1] if (track and bw_rows > 0) else 0, dtype=torch.int32)
+
+
+@torch.library.custom_op('hgq::qdense_bwd', mutates_args=())
+def qdense_bwd(dy: Tensor, y: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_bias: bool, act: int, mode: int,
+               bw_rows: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    _check_f32('dy', dy), _check_f32('x', x), _check_f32('qw', qw), _check_f32('y', y)
+    rows, K = x.shape
+    N = qw.shape[1]
+    _need(tuple(dy.shape) == (rows, N), 'dy shape mismatch')
+    dx = torch.empty_like(x)
+    dqw = torch.empty_like(qw)
+    dqb = torch.empty(N if has_bias else 0, dtype=torch.float32, device=x.device)
+    df = torch.empty(bw_rows * K, dtype=torch.float32, device=x.device)
+    rc = _lib.load().hgq_qdense_bwd(_ptr(dy), _ptr(y), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(dqw),
+                                    _ptr(dqb), _ptr(df), rows, K, N, act, mode, _stream())
+    _lib.check(rc, 'hgq_qdense_bwd')
+    return dx, dqw, dqb, df
+
+
+@qdense_bwd.register_fake
+def _(dy, y, x, f_in, qw, has_bias, act, mode, bw_rows):
+    return (torch.empty_like(x), torch.empty_like(qw), x.new_empty(qw.shape[1] if has_bias else 0),
+            x.new_empty(bw_rows * x.shape[1]))
+
+
+def _qdense_setup(ctx, inputs, output):
+    x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track = inputs
+    y, _ = output
+    ctx.save_for_backward(x, f_in, qw, y)
+    ctx.has_bias = qb.numel() > 0
+    ctx.act, ctx.mode, ctx.bw_rows = act, mode, bw_rows
+    ctx.f_shape = f_in.shape
+
+
+def _qdense_backward(ctx, gy, g_amax):
+    x, f_in, qw, y = ctx.saved_tensors
+    dx, dqw, dqb, df = qdense_bwd(gy.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows)
+    return (dx, None, None, df.view(ctx.f_shape) if ctx.bw_rows > 0 else None, dqw, dqb if ctx.has_bias else None,
+            None, None, None, None)
+
+
+qdense_fwd.register_autograd(_qdense_backward, setup_context=_qdense_setup)
+
+FUSED_BWD_MAX = 64  # hgq_qdense_bwd covers K <= 64 and N <= 64
+
+
+def qdense(x2d, k_in, i_in, f_in, qw, qb, act: int, mode: int, bw_rows: int, track: bool):
+    """y = act(q_in(x) @ qw + qb) on a [rows, K] view; returns ``(y, amax_bits)``."""
+    empty = x2d.new_empty(0)
+    return qdense_fwd(x2d, k_in if k_in is not None else empty, i_in if i_in is not None else empty,
+                      f_in if f_in is not None else empty, qw, qb if qb is not None else empty, act, mode, bw_rows, track)
+
+
+# --------------------------------------------------------------------------------------
+# EBOPs of a dense contraction
+# --------------------------------------------------------------------------------------
+@torch.library.custom_op('hgq::dense_ebops', mutates_args=())
+def dense_ebops_op(k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor, b_ker: Tensor, k_bias: Tensor, b_bias: Tensor,
+                   P: int, K: int, N: int, scale: float, bias_size: float, mode_in: int, mode_ker: int,
+                   mode_bias: int) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
+    _check_k('k_in', k_in), _check_f32('i_in', i_in), _check_f32('f_in', f_in), _check_k('k_ker', k_ker), _check_f32('b_ker', b_ker)
+    _need(i_in.numel() == P * K and f_in.numel() == P * K and k_in.numel() == P * K, 'input bit-width size mismatch')
+    _need(b_ker.numel() == K * N and k_ker.numel() == K * N, 'kernel bit-width size mismatch')
+    has_bias = b_bias.numel() > 0
+    if has_bias:
+        _check_f32('b_bias', b_bias), _check_k('k_bias', k_bias)
+        _need(b_bias.numel() == N and k_bias.numel() == N, 'bias bit-width size mismatch')
+        mode_bias = _kmode(mode_bias, k_bias)
+    ebops = torch.empty((), dtype=torch.float32, device=f_in.device)
+    ebops_u32 = torch.empty((), dtype=torch.int32, device=f_in.device)  # bit pattern of the uint32 value
+    g_f = torch.empty_like(f_in)
+    g_bk = torch.empty_like(b_ker)
+    g_bb = torch.empty_like(b_bias)
+    rc = _lib.load().hgq_dense_ebops(_ptr(k_in), _ptr(i_in), _ptr(f_in), P, K, N, _ptr(k_ker), _ptr(b_ker), _ptr(k_bias),
+                                     _ptr(b_bias), scale, bias_size, _kmode(mode_in, k_in), _kmode(mode_ker, k_ker), mode_bias,
+                                     _ptr(ebops), _ptr(ebops_u32), _ptr(g_f), _ptr(g_bk), _ptr(g_bb), _stream())
+    _lib.check(rc, 'hgq_dense_ebops')
+    return ebops, ebops_u32, g_f, g_bk, g_bb
+
+
+@dense_ebops_op.register_fake
+def _(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, bias_size, mode_in, mode_ker, mode_bias):
+    return f_in.new_empty(()), f_in.new_empty((), dtype=torch.int32), torch.empty_like(f_in), torch.empty_like(b_ker), torch.empty_like(b_bias)
+
+
+def _ebops_setup(ctx, inputs, output):
+    _, _, g_f, g_bk, g_bb = output
+    ctx.save_for_backward(g_f, g_bk, g_bb)
+    ctx.i_needs = inputs[1].requires_grad and not (inputs[12] & _lib.MODE_KBI)
+
+
+def _ebops_backward(ctx, g, *_unused):
+    g_f, g_bk, g_bb = ctx.saved_tensors
+    gf = g * g_f
+    return (None, gf if ctx.i_needs else None, gf, None, g * g_bk, None, g * g_bb if g_bb.numel() else None,
+            None, None, None, None, None, None, None, None)
+
+
+dense_ebops_op.register_autograd(_ebops_backward, setup_context=_ebops_setup)
+
+
+def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, bias_size, mode_in, mode_ker, mode_bias):
+    """Returns ``(ebops fp32 scalar, ebops truncated to uint32 as an int32 bit pattern)``."""
+    dev = f_in.device
+    e_f = torch.empty(0, dtype=torch.float32, device=dev)
+    e_k = torch.empty(0, dtype=torch.uint8, device=dev)
+    out = dense_ebops_op(k_in, i_in, f_in, k_ker, b_ker, k_bias if k_bias is not None else e_k,
+                         b_bias if b_bias is not None else e_f, P, K, N,
+                         float(scale), float(bias_size), mode_in, mode_ker, mode_bias)
+    return out[0], out[1]
+
+
+# --------------------------------------------------------------------------------------
+# loss and optimizer step
+# --------------------------------------------------------------------------------------
+@torch.library.custom_op('hgq::sparse_ce', mutates_args=())
+def sparse_ce_op(logits: Tensor, labels: Tensor) -> tuple[Tensor, Tensor]:
+    _check_f32('logits', logits)
+    _need(logits.dim() == 2 and labels.dim() == 1 and labels.shape[0] == logits.shape[0], 'logits [rows, C], labels [rows]')
+    _need(labels.dtype == torch.int64 and labels.is_cuda and labels.is_contiguous(), 'labels must be a contiguous int64 GPU tensor')
+    loss = torch.empty((), dtype=torch.float32, device=logits.device)
+    dlogits = torch.empty_like(logits)
+    rc = _lib.load().hgq_sparse_ce_fwd_bwd(_ptr(logits), _ptr(labels), _ptr(loss), _ptr(dlogits), logits.shape[0],
+                                           logits.shape[1], _stream())
+    _lib.check(rc, 'hgq_sparse_ce_fwd_bwd')
+    return loss, dlogits
+
+
+@sparse_ce_op.register_fake
+def _(logits, labels):
+    return logits.new_empty(()), torch.empty_like(logits)
+
+
+def _ce_setup(ctx, inputs, output):
+    ctx.save_for_backward(output[1])
+
+
+def _ce_backward(ctx, g, _):
+    (dlogits,) = ctx.saved_tensors
+    return g * dlogits, None
+
+
+sparse_ce_op.register_autograd(_ce_backward, setup_context=_ce_setup)
+
+
+def sparse_ce(logits: Tensor, labels: Tensor) -> Tensor:
+    """Mean sparse categorical cross-entropy from logits."""
+    return sparse_ce_op(logits.contiguous(), labels)[0]
+
+
+@torch.library.custom_op('hgq::sgd_update', mutates_args=('w',))
+def sgd_update_op(w: Tensor, g: Tensor, lr: float, l1: float, lo: float, hi: float) -> None:
+    _check_f32('w', w), _check_f32('g', g)
+    _need(w.numel() == g.numel(), 'gradient size mismatch')
+    rc = _lib.load().hgq_sgd_update(_ptr(w), _ptr(g), w.numel(), lr, l1, lo, hi, _stream())
+    _lib.check(rc, 'hgq_sgd_update')
+
+
+def sgd_update_(w, g, lr, l1=0.0, lo=float('-inf'), hi=float('inf')):
+    sgd_update_op(w, g.contiguous(), float(lr), float(l1), float(lo), float(hi))

@@ -1,0 +1,171 @@
+/*
+ * hgq_hip.h - C ABI of libhgq_hip.so: the HGQ2 quantized-training hot path on MI355X (gfx950).
+ *
+ * The reference (calad0i/HGQ2) is pure Python and has no FFI; the seam these entry points sit
+ * behind is the stateless quantizer callable it imports from the third-party package
+ * `quantizers` and the chains of eager keras.ops calls inside its layers.  Each declaration
+ * cites the reference code it replaces (paths relative to the reference root).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer to contiguous memory, fp32 unless stated otherwise;
+ *   - the library never allocates, never frees and never synchronises; all work is enqueued on
+ *     `stream` (a hipStream_t passed as void*; NULL = the default stream);
+ *   - every function returns HGQ_OK (0) or a negative HGQ_ERR_* code; hgq_last_error() returns a
+ *     thread-local description of the last failure;
+ *   - outputs that are reductions (bit-width gradients, abs-max trackers) are cleared by the
+ *     entry point itself with a fill kernel (safe under HIP graph capture), then accumulated;
+ *   - bit-width operands (k, i, f or b) must hold integer-valued floats after the optional
+ *     rounding selected by HGQ_MODE_ROUND_PARAMS; powers of two are formed exactly from them.
+ *
+ * Bit-width broadcasting: element `e` of a tensor with `n` elements uses bit-width entry
+ * `(e / bw_inner) % bw_size`.  bw_size == n, bw_inner == 1 is the per-element case;
+ * bw_size == 1 a single shared bit-width; a tensor [B, ...] with bit-widths [1, ...] has
+ * bw_size = n / B, bw_inner = 1.
+ */
+#ifndef HGQ_HIP_H
+#define HGQ_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HGQ_OK 0
+#define HGQ_ERR_ARG (-1)         /* null pointer, negative size, unknown mode */
+#define HGQ_ERR_LAUNCH (-2)      /* the HIP runtime refused a launch; see hgq_last_error() */
+#define HGQ_ERR_UNSUPPORTED (-3) /* shape outside what the kernel family covers */
+
+/* rounding modes (low nibble of `mode`) */
+#define HGQ_TRN 0
+#define HGQ_RND 1
+#define HGQ_RND_CONV 2
+/* overflow modes (second nibble of `mode`) */
+#define HGQ_WRAP 0
+#define HGQ_SAT 1
+#define HGQ_SAT_SYM 2
+
+#define HGQ_MODE(round_mode, overflow_mode) ((round_mode) | ((overflow_mode) << 4))
+#define HGQ_MODE_TRAINING (1 << 8)     /* training-mode forward: WRAP is round-only, no zeroing of empty words */
+#define HGQ_MODE_KBI (1 << 9)          /* third bit-width operand is b (total bits); f = b - i */
+#define HGQ_MODE_ROUND_PARAMS (1 << 10) /* operands are the raw trainable variables: round half-even first */
+#define HGQ_MODE_K_U8 (1 << 11)        /* k operand is uint8 (the reference's `_k` variable dtype) */
+#define HGQ_MODE_SYMMETRIC (1 << 12)   /* hgq_wrap_track_i: the symmetric minimal-i formula */
+#define HGQ_MODE_TRACING (1 << 13)     /* hgq_wrap_track_i: calibration ("tracing") update rule */
+
+#define HGQ_ACT_NONE 0
+#define HGQ_ACT_RELU 1
+
+int hgq_version(void);
+const char *hgq_last_error(void);
+
+/*
+ * Fixed-point quantizer, forward.  Replaces the callable returned by
+ * quantizers.fixed_point._fixed_point_ops._get_fixed_quantizer(round_mode, overflow_mode),
+ * i.e. `q(x, k, i, f, training, seed_gen)` and `q.round(x, f, ...)` (imported at
+ * src/hgq/quantizer/internal/fixed_point_quantizer.py:9, called at :147, :288, :305, :405),
+ * together with the broadcast of k/i/f and the inference-time zeroing around it
+ * (fixed_point_quantizer.py:142-150) and the `round_conv` of the raw variables (:250,:254,:441,:445).
+ *
+ *   y      [n]        quantized values
+ *   amax   [bw_size]  optional (NULL to skip): max |y| over the elements sharing each bit-width
+ *                     entry, as the uint32 bit pattern of a non-negative float - the reduction of
+ *                     DefaultBitwidthMapper.x_to_bw_absmax (src/hgq/quantizer/internal/base.py:185-186)
+ *   anyneg [bw_size]  optional: 1 where any y < 0 (x_to_bw_sign, internal/base.py:188-189)
+ */
+int hgq_quantize_fwd(const float *x, const void *k, const float *i, const float *fb, float *y,
+                     uint32_t *amax, uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner,
+                     int mode, void *stream);
+
+/*
+ * Fixed-point quantizer, surrogate backward (training mode only).  Replaces the custom
+ * gradients of the same third-party callable plus autograd through broadcast_to (the sum over
+ * the homogeneous axes) and through `f = b - i` for the KBI parametrisation
+ * (fixed_point_quantizer.py:256-265).
+ *
+ *   dx  [n];  di, dfb [bw_size]  (either may be NULL to skip).  With HGQ_MODE_KBI `dfb` is the
+ *   gradient w.r.t. b and `di` the total gradient w.r.t. i (direct - via f).
+ */
+int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,
+                     float *dx, float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner,
+                     int mode, void *stream);
+
+/*
+ * Integer-bit tracking of WRAP quantizers.  Replaces minimal_i_given_xf / minimal_i_given_xb
+ * (fixed_point_quantizer.py:16-31) and the `_i.assign(...)` recurrences of
+ * FixedPointQuantizerKIF.call (:406-422) and FixedPointQuantizerKBI.call (:280-300).
+ *
+ *   i_var [m]  in/out: the raw `_i` variable;   fb [m]: raw `_f` (KIF) or `_b` (KBI)
+ *   training : i_var <- max(i_var - decay, minimal_i)            (KBI: then clipped to [c_lo, c_hi])
+ *   tracing  : i_var <- max(round(i_var), clip(minimal_i)),  k_var |= anyneg   (k_var uint8, optional)
+ */
+int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, float *i_var, const float *fb,
+                     uint8_t *k_var, int64_t m, float decay, float c_lo, float c_hi, int mode, void *stream);
+
+/*
+ * QDense / QEinsumDense contraction, forward, with the input quantizer fused into the operand
+ * load.  Replaces `ops.matmul(self.iq(inputs), self.qkernel) + self.qbias` and the activation
+ * (src/hgq/layers/core/dense.py:60-68; einsum_dense.py:72-83 for equations that reshape to a
+ * GEMM), including the abs-max reduction the WRAP input quantizer needs
+ * (fixed_point_quantizer.py:405-408).
+ *
+ *   x [rows, K];  k_in/i_in/f_in [bw_rows, K] input-quantizer operands (row r uses entry
+ *   r % bw_rows); bw_rows == 0 means x is used as is;  qw [K, N] quantized kernel;
+ *   qb [N] quantized bias or NULL;  y [rows, N];  amax [bw_rows*K] optional.
+ *   The input quantizer must be a training-mode WRAP quantizer or any inference/SAT mode
+ *   selected by `mode`; act is HGQ_ACT_*.
+ */
+int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_in, const float *f_in, int64_t bw_rows,
+                   const float *qw, const float *qb, float *y, uint32_t *amax, int64_t rows, int K, int N,
+                   int act, int mode, void *stream);
+
+/*
+ * QDense / QEinsumDense contraction, backward: autograd of the same expression.
+ *   dx [rows, K] gradient w.r.t. the un-quantized input (straight-through);
+ *   dqw [K, N], dqb [N] (NULL if no bias): gradients w.r.t. the quantized kernel / bias;
+ *   df_in [bw_rows*K]: gradient w.r.t. the input quantizer's fractional bits (NULL if bw_rows == 0).
+ * Supported: K <= 64 and N <= 64, training-mode WRAP input quantizer (round-only).
+ */
+int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
+                   const float *qw, float *dx, float *dqw, float *dqb, float *df_in, int64_t rows, int K,
+                   int N, int act, int mode, void *stream);
+
+/*
+ * EBOPs of a dense contraction and its gradient.  Replaces QDense._compute_ebops
+ * (src/hgq/layers/core/dense.py:70-80) / QEinsumDense._compute_ebops for GEMM-shaped equations
+ * (einsum_dense.py:85-93) evaluated on bit-width tensors, i.e.
+ *     ebops = (sum_p sum_k bits_in[p,k] * sum_n bits_ker[k,n] + mean(bits_bias) * bias_size) * scale
+ * with bits_in = relu(round(i_in)+round(f_in)) (+k for SAT), bits_ker / bits_bias = round(b) (+k for SAT).
+ *
+ *   ebops [1] fp32;  ebops_u32 [1] optional: the value cast to uint32 (the `_ebops` variable,
+ *   src/hgq/layers/core/base.py:103);  g_f_in [P*K], g_b_ker [K*N], g_b_bias [N]: d ebops / d variable.
+ */
+int hgq_dense_ebops(const void *k_in, const float *i_in, const float *f_in, int64_t P, int K, int N,
+                    const void *k_ker, const float *b_ker, const void *k_bias, const float *b_bias,
+                    float scale, float bias_size, int mode_in, int mode_ker, int mode_bias, float *ebops,
+                    uint32_t *ebops_u32,
+                    float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream);
+
+/*
+ * Mean sparse categorical cross-entropy from logits, forward and gradient in one pass.
+ *   logits [rows, C]; labels [rows] int64;  loss [1] = mean_r(-log softmax(logits_r)[label_r]);
+ *   dlogits [rows, C] = (softmax - onehot) / rows.
+ */
+int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *loss, float *dlogits, int64_t rows,
+                          int C, void *stream);
+
+/*
+ * Plain SGD update with the reference's post-update constraint and MonoL1 regulariser folded in.
+ * Replaces `optimizer.apply` + Constraint.__call__ (src/hgq/constraints/__init__.py:19-21) +
+ * the gradient of MonoL1 (src/hgq/regularizers/__init__.py:13-14) for one variable:
+ *     w <- clip(w - lr * (g + l1), lo, hi)          (pass lo = -inf, hi = +inf for no constraint)
+ */
+int hgq_sgd_update(float *w, const float *g, int64_t n, float lr, float l1, float lo, float hi, void *stream);
+
+/* Fill kernel (graph-capture safe replacement for a memset). */
+int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HGQ_HIP_H */

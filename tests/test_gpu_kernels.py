@@ -1,0 +1,284 @@
+"""GPU parity of the HIP kernels (through torch.library -> ctypes -> C ABI) against the CPU oracle.
+
+Bar: quantized values, tracked integer bits and EBOPs bit-exact; contractions and gradients
+within 1e-5 relative (fp32; the reference statement is evaluated in float64 where a sum is
+involved so that the tolerance measures the kernel, not the checker)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fixed_point as ofp
+from oracle import hgq_ref as ref
+
+pytestmark = pytest.mark.gpu
+
+ROUND = ('TRN', 'RND', 'RND_CONV')
+OVER = ('WRAP', 'SAT', 'SAT_SYM')
+RTOL = 1e-5
+
+
+def _ops():
+    from hgq2_amd import _lib, ops
+
+    return _lib, ops
+
+
+def _rand_kif(shape, g, kbi=False):
+    k = torch.randint(0, 2, shape, generator=g).float()
+    i = torch.randint(-2, 5, shape, generator=g).float()
+    f = torch.randint(0, 9, shape, generator=g).float()
+    if kbi:
+        return k, i, i + f  # b = i + f >= 0
+    return k, i, f
+
+
+def _assert_close_sum(got, want64, scale64, what):
+    """|got - want| <= RTOL * sum|terms| : a relative bound that is meaningful under cancellation."""
+    err = (got.double().cpu() - want64).abs()
+    tol = RTOL * scale64 + 1e-30
+    assert torch.all(err <= tol), f'{what}: max err {err.max().item():.3e} tol {tol.min().item():.3e}'
+
+
+@pytest.mark.parametrize('round_mode', ROUND)
+@pytest.mark.parametrize('overflow_mode', OVER)
+@pytest.mark.parametrize('training', (False, True))
+@pytest.mark.parametrize('n', (1, 3, 4099, 1 << 16))
+def test_quantize_per_element_values(dev, round_mode, overflow_mode, training, n):
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(n, generator=g) * 4
+    x[::7] = torch.round(x[::7] * 8) / 8 + 1 / 16  # exact ties for small f
+    k, i, f = _rand_kif((n,), g)
+    want = ofp.get_fixed_quantizer(round_mode, overflow_mode)(x, k, i, f, training, None)
+    if not training:
+        want = torch.where(k + i + f > 0, want, torch.zeros_like(want))
+    mode = _lib.mode_bits(round_mode, overflow_mode, training=training)
+    y, _, _ = ops.quantize(x.to(dev), k.to(dev), i.to(dev), f.to(dev), mode)
+    assert torch.equal(y.cpu(), want)
+    # uint8 k and raw (un-rounded) variables
+    noise = (torch.rand(n, generator=g) - 0.5) * 0.8
+    y2, _, _ = ops.quantize(x.to(dev), k.to(torch.uint8).to(dev), (i + noise).to(dev), (f - noise).to(dev),
+                            mode | _lib.MODE_ROUND_PARAMS)
+    assert torch.equal(y2.cpu(), want)
+
+
+@pytest.mark.parametrize('overflow_mode', OVER)
+@pytest.mark.parametrize('kbi', (False, True))
+def test_quantize_per_element_gradients(dev, overflow_mode, kbi):
+    _lib, ops = _ops()
+    n = 50000
+    g = torch.Generator().manual_seed(7)
+    x = (torch.randn(n, generator=g) * 4).requires_grad_(True)
+    k, i, fb = _rand_kif((n,), g, kbi)
+    i.requires_grad_(True), fb.requires_grad_(True)
+    f = fb - i if kbi else fb
+    y = ofp.get_fixed_quantizer('RND', overflow_mode)(x, k, i, f, True, None)
+    gy = torch.randn(n, generator=g)
+    y.backward(gy)
+    mode = _lib.mode_bits('RND', overflow_mode, training=True, kbi=kbi)
+    xd = x.detach().to(dev).requires_grad_(True)
+    idv = i.detach().to(dev).requires_grad_(True)
+    fd = fb.detach().to(dev).requires_grad_(True)
+    yd, _, _ = ops.quantize(xd, k.to(dev), idv, fd, mode)
+    assert torch.equal(yd.detach().cpu(), y.detach())
+    yd.backward(gy.to(dev))
+    for got, want, name in ((xd.grad, x.grad, 'dx'), (idv.grad, i.grad, 'di'), (fd.grad, fb.grad, 'dfb')):
+        want = torch.zeros(n) if want is None else want
+        np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=RTOL, atol=1e-30, err_msg=name)
+
+
+@pytest.mark.parametrize('shape,bw_shape', [((4096, 16), (1, 16)), ((1000, 7), (1, 7)), ((64, 12, 20), (1, 12, 20)),
+                                            ((3000,), ()), ((33, 5, 8), (1, 1, 1)), ((50, 6, 4), (1, 6, 1))])
+@pytest.mark.parametrize('overflow_mode', ('WRAP', 'SAT'))
+def test_quantize_broadcast_bitwidths(dev, shape, bw_shape, overflow_mode):
+    """Bit-widths shared along the homogeneous axes: values, abs-max / any-negative trackers, reduced gradients."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(shape, generator=g) * 3).requires_grad_(True)
+    k, i, f = _rand_kif(bw_shape, g)
+    i.requires_grad_(True), f.requires_grad_(True)
+    q = ofp.get_fixed_quantizer('RND', overflow_mode)
+    kb, ib, fb = (torch.broadcast_to(t, shape) for t in (k, i, f))
+    y = q(x, kb, ib, fb, True, None)
+    gy = torch.randn(shape, generator=g)
+    y.backward(gy)
+    bw_size = max(1, int(np.prod(bw_shape)))
+    # position of the heterogeneous block -> (bw_size, bw_inner)
+    inner = 1
+    for ax in range(len(shape) - 1, -1, -1):
+        if len(bw_shape) and bw_shape[ax] != 1:
+            break
+        inner *= shape[ax]
+    if bw_size == 1:
+        inner = 1
+    mode = _lib.mode_bits('RND', overflow_mode, training=True)
+    xd = x.detach().to(dev).requires_grad_(True)
+    idv = i.detach().reshape(-1).to(dev).requires_grad_(True)
+    fd = f.detach().reshape(-1).to(dev).requires_grad_(True)
+    yd, amax, neg = ops.quantize(xd, k.reshape(-1).to(dev), idv, fd, mode, bw_inner=inner, track=True)
+    assert torch.equal(yd.detach().cpu(), y.detach())
+    hom = tuple(a for a in range(len(shape)) if not len(bw_shape) or bw_shape[a] == 1)
+    want_amax = torch.amax(y.detach().abs(), dim=hom).reshape(-1)
+    want_neg = torch.amax((y.detach() < 0).int(), dim=hom).reshape(-1)
+    assert torch.equal(amax.view(torch.float32).cpu(), want_amax)
+    assert torch.equal(neg.cpu(), want_neg.int())
+    yd.backward(gy.to(dev))
+    np.testing.assert_allclose(xd.grad.cpu().numpy(), x.grad.numpy(), rtol=RTOL, atol=1e-30)
+    # reduced gradients: float64 statement of the same per-element terms
+    x64, gy64 = x.detach().double(), gy.double()
+    delta = y.detach().double() - x64
+    over = (y.detach() != ofp.fixed_round(x.detach(), fb, 'RND', False))
+    f_terms = torch.where(over, torch.zeros_like(delta), -np.log(2) * delta * gy64)
+    if overflow_mode == 'WRAP':
+        want_df = f_terms.sum(dim=hom).reshape(-1)
+        scale = f_terms.abs().sum(dim=hom).reshape(-1)
+        _assert_close_sum(fd.grad, want_df, scale, 'df')
+        assert torch.all(idv.grad == 0)
+    else:
+        np.testing.assert_allclose(fd.grad.cpu().numpy(), f.grad.reshape(-1).numpy(), rtol=2e-4, atol=1e-4)
+        np.testing.assert_allclose(idv.grad.cpu().numpy(), i.grad.reshape(-1).numpy(), rtol=2e-4, atol=1e-4)
+
+
+def test_wrap_track_i_matches_reference_recurrence(dev):
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(3)
+    q = ref.default_quantizer('datalane', (None, 40), q_type='kif', overflow_mode='WRAP')
+    with torch.no_grad():
+        q.quantizer._f.copy_(torch.randint(0, 9, (1, 40), generator=g).float())
+        q.quantizer._i.copy_(torch.randint(-3, 3, (1, 40), generator=g).float() + 0.37)
+    x = torch.randn(512, 40, generator=g) * torch.logspace(-2, 2, 40)
+    x[:, 5] = 0.0
+    x[:, 6] = 2.0 - 2.0 ** -float(q.quantizer._f[0, 6])  # exactly at 2**1 - 2**-f
+    i_dev = q.quantizer._i.detach().clone().reshape(-1).to(dev)
+    f_dev = q.quantizer._f.detach().clone().reshape(-1).to(dev)
+    k_dev = q.quantizer._k.reshape(-1).to(dev)
+    mode = _lib.mode_bits('RND', 'WRAP', training=True, round_params=True)
+    for _ in range(3):
+        want_y = q(x, training=True)
+        y, amax, _ = ops.quantize(x.to(dev), k_dev, i_dev, f_dev, mode, track=True)
+        ops.wrap_track_i_(amax, i_dev, f_dev, 0.01, mode)
+        assert torch.equal(y.cpu(), want_y.detach())
+        assert torch.equal(i_dev.cpu(), q.quantizer._i.detach().reshape(-1))
+        x = x * 0.5
+
+
+@pytest.mark.parametrize('rows,K,N,P', [(16384, 16, 64, 1), (1000, 64, 32, 1), (777, 32, 5, 1), (512, 12, 8, 1),
+                                        (64 * 30, 16, 64, 64), (12 * 50, 8, 8, 12), (300, 7, 3, 1), (256, 40, 33, 1)])
+@pytest.mark.parametrize('act', ('relu', None))
+def test_qdense_forward_backward(dev, rows, K, N, P, act):
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(rows + K)
+    x = (torch.randn(rows, K, generator=g) * 2).requires_grad_(True)
+    f = torch.randint(0, 7, (P, K), generator=g).float().requires_grad_(True)
+    qw = (torch.round(torch.randn(K, N, generator=g) * 16) / 32).requires_grad_(True)
+    qb = (torch.round(torch.randn(N, generator=g) * 16) / 32).requires_grad_(True)
+    fb = f.repeat(rows // P, 1)
+    rx = ofp.get_fixed_quantizer('RND', 'WRAP').round(x, fb, False, None)
+    z = rx.double() @ qw.double() + qb.double()
+    y = torch.relu(z) if act else z
+    gy = torch.randn(rows, N, generator=g)
+    y.backward(gy.double())
+    mode = _lib.mode_bits('RND', 'WRAP', training=True)
+    xd = x.detach().to(dev).requires_grad_(True)
+    fd = f.detach().to(dev).requires_grad_(True)
+    wd = qw.detach().to(dev).requires_grad_(True)
+    bd = qb.detach().to(dev).requires_grad_(True)
+    kd = torch.ones(P, K, device=dev)
+    idv = torch.zeros(P, K, device=dev)
+    yd, amax = ops.qdense(xd, kd, idv, fd, wd, bd, _lib.ACT_RELU if act else _lib.ACT_NONE, mode, P, True)
+    scale = (rx.detach().double().abs() @ qw.detach().double().abs()) + qb.detach().double().abs()
+    _assert_close_sum(yd.detach(), y.detach(), scale, 'y')
+    want_amax = rx.detach().abs().reshape(rows // P, P, K).amax(dim=0).reshape(-1)
+    assert torch.equal(amax.view(torch.float32).cpu(), want_amax)
+    # The kernel's relu mask comes from its own fp32 output; rows where the sign of the
+    # pre-activation is not decided at fp32 accuracy are excluded from the gradient check.
+    yd.backward(gy.to(dev))
+    if act:
+        decided = (z.detach().abs() > RTOL * scale).all(dim=1)
+    else:
+        decided = torch.ones(rows, dtype=torch.bool)
+    dz = gy.double() * ((z.detach() > 0) if act else 1.0)
+    dx_scale = dz.abs() @ qw.detach().double().abs().T
+    err = (xd.grad.cpu().double() - x.grad.double()).abs()
+    assert torch.all(err[decided] <= RTOL * dx_scale[decided] + 1e-30)
+    if bool(decided.all()):
+        _assert_close_sum(wd.grad, qw.grad.double(), rx.detach().double().abs().T @ dz.abs(), 'dqw')
+        _assert_close_sum(bd.grad, qb.grad.double(), dz.abs().sum(0), 'dqb')
+        delta = rx.detach().double() - x.detach().double()
+        terms = (-np.log(2) * delta * x.grad.double()).reshape(rows // P, P, K)
+        _assert_close_sum(fd.grad.reshape(-1), terms.sum(0).reshape(-1), terms.abs().sum(0).reshape(-1) + 1e-12, 'df')
+
+
+def test_qdense_exact_in_small_bitwidth_regime(dev):
+    """Operands with few significant bits: every product and partial sum is exact in fp32, so the
+    contraction must be bit-identical whatever the accumulation order."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(4096, 64, generator=g) * 2
+    f = torch.full((1, 64), 3.0)
+    qw = torch.round(torch.randn(64, 64, generator=g) * 8) / 16
+    qb = torch.round(torch.randn(64, generator=g) * 8) / 16
+    want = torch.relu(ofp.fixed_round(x, f.expand_as(x), 'RND', False) @ qw + qb)
+    mode = _lib.mode_bits('RND', 'WRAP', training=True)
+    y, _ = ops.qdense(x.to(dev), torch.ones(1, 64, device=dev), torch.zeros(1, 64, device=dev), f.to(dev), qw.to(dev),
+                      qb.to(dev), _lib.ACT_RELU, mode, 1, False)
+    assert torch.equal(y.cpu(), want)
+
+
+def test_qdense_large_shapes_forward_only(dev):
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(500, 300, generator=g)
+    f = torch.randint(2, 6, (1, 300), generator=g).float()
+    qw = torch.round(torch.randn(300, 130, generator=g) * 16) / 32
+    want = ofp.fixed_round(x, f.expand_as(x), 'RND', False).double() @ qw.double()
+    mode = _lib.mode_bits('RND', 'WRAP', training=True)
+    y, _ = ops.qdense(x.to(dev), torch.ones(1, 300, device=dev), torch.zeros(1, 300, device=dev), f.to(dev), qw.to(dev),
+                      None, _lib.ACT_NONE, mode, 1, False)
+    scale = x.double().abs() @ qw.double().abs()
+    _assert_close_sum(y, want, scale, 'y')
+
+
+def test_dense_ebops_exact_and_gradients(dev):
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(13)
+    layer = ref.RefMLP(dims=(24, 10)).layers[0]
+    with torch.no_grad():
+        layer.iq.quantizer._f.copy_(torch.randint(-3, 7, (1, 24), generator=g).float() + 0.2)
+        layer.iq.quantizer._i.copy_(torch.randint(-2, 4, (1, 24), generator=g).float() - 0.3)
+        layer.kq.quantizer._b.copy_(torch.randint(0, 9, (24, 10), generator=g).float() + 0.1)
+        layer.bq.quantizer._b.copy_(torch.randint(0, 9, (10,), generator=g).float())
+    e = layer._compute_ebops((1, 24))
+    e.backward()
+    iq, kq, bq = layer.iq.quantizer, layer.kq.quantizer, layer.bq.quantizer
+    d = lambda t: t.detach().reshape(-1).to(dev).requires_grad_(t.requires_grad)  # noqa: E731
+    fi, bk, bb = d(iq._f), d(kq._b), d(bq._b)
+    m_in = _lib.mode_bits('RND', 'WRAP', training=True, round_params=True)
+    m_k = _lib.mode_bits('RND', 'SAT_SYM', training=True, round_params=True, kbi=True)
+    val, u32 = ops.dense_ebops(iq._k.reshape(-1).to(dev), d(iq._i), fi, kq._k.reshape(-1).to(dev), bk,
+                               bq._k.to(dev), bb, 1, 24, 10, 1.0, 10.0, m_in, m_k, m_k)
+    assert val.item() == e.item() and u32.item() == int(e.item())
+    val.backward()
+    assert torch.equal(fi.grad.cpu(), iq._f.grad.reshape(-1))
+    assert torch.equal(bk.grad.cpu(), kq._b.grad.reshape(-1))
+    assert torch.equal(bb.grad.cpu(), bq._b.grad.reshape(-1))
+
+
+def test_sparse_ce_and_sgd(dev):
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(17)
+    logits = (torch.randn(16384, 5, generator=g) * 3).requires_grad_(True)
+    labels = torch.randint(0, 5, (16384,), generator=g)
+    loss = torch.nn.functional.cross_entropy(logits.double(), labels)
+    loss.backward()
+    ld = logits.detach().to(dev).requires_grad_(True)
+    got = ops.sparse_ce(ld, labels.to(dev))
+    got.backward()
+    assert abs(got.item() - loss.item()) <= RTOL * abs(loss.item())
+    np.testing.assert_allclose(ld.grad.cpu().numpy(), logits.grad.numpy(), rtol=1e-4, atol=1e-9)
+    w = torch.randn(1000, generator=g) * 10
+    gr = torch.randn(1000, generator=g) * 100
+    wd = w.to(dev)
+    ops.sgd_update_(wd, gr.to(dev), 0.01, 1e-8, -2.0, 2.0)
+    assert torch.equal(wd.cpu(), torch.clamp(w - 0.01 * (gr + 1e-8), -2.0, 2.0))
