@@ -21,6 +21,7 @@ MODE_ROUND_PARAMS = 1 << 10
 MODE_K_U8 = 1 << 11
 MODE_SYMMETRIC = 1 << 12
 MODE_TRACING = 1 << 13
+MODE_TRACK_INPUT = 1 << 14
 ACT_NONE, ACT_RELU = 0, 1
 
 ROUND_MODES = {'TRN': TRN, 'RND': RND, 'RND_CONV': RND_CONV}
@@ -79,7 +80,7 @@ def check(rc: int, what: str) -> None:
 
 
 def mode_bits(round_mode: str, overflow_mode: str, *, training=False, kbi=False, round_params=False, k_u8=False,
-              symmetric=False, tracing=False) -> int:
+              symmetric=False, tracing=False, track_input=False) -> int:
     rm = round_mode.upper()
     if rm.startswith('S_'):
         rm = rm[2:]
@@ -99,4 +100,6 @@ def mode_bits(round_mode: str, overflow_mode: str, *, training=False, kbi=False,
         m |= MODE_SYMMETRIC
     if tracing:
         m |= MODE_TRACING
+    if track_input:
+        m |= MODE_TRACK_INPUT
     return m

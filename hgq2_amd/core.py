@@ -1,0 +1,272 @@
+"""Minimal layer runtime the API mirror sits on (Keras v3 is not required on the host).
+
+It reproduces the few Keras behaviours the hot path relies on:
+
+* lazy ``build(input_shape)`` on first call and ``add_weight(...)`` with per-variable
+  ``constraint`` / ``regularizer`` / ``trainable``;
+* the ``training`` flag is inherited by nested layer calls through a call context, so
+  ``self.kq(self._kernel)`` inside a layer sees the outer call's flag;
+* ``add_loss`` terms are collected per top-level call; variable regularizers are summed into
+  the loss; constraints are applied after the optimizer update.
+"""
+
+from __future__ import annotations
+
+import math
+import threading
+from typing import Any
+
+import numpy as np
+import torch
+from torch import nn
+
+_ctx = threading.local()
+
+EPSILON = 1e-7  # keras.backend.epsilon() default
+
+
+def epsilon() -> float:
+    return EPSILON
+
+
+def _training_ctx():
+    return getattr(_ctx, 'training', None)
+
+
+class TrainingFlagWrapper:
+    """Falsy object that compares equal to a string; used for ``training='tracing'``
+    (reference src/hgq/utils/minmax_trace.py:24-32)."""
+
+    def __init__(self, value):
+        self.value = value
+
+    def __bool__(self):
+        return self.value is True
+
+    def __eq__(self, other):
+        return self.value == other
+
+    def __hash__(self):
+        return hash(self.value)
+
+
+# ------------------------------------------------------------------------------------------
+# initializers
+# ------------------------------------------------------------------------------------------
+class Initializer:
+    def __call__(self, shape, dtype, device, generator=None):
+        raise NotImplementedError
+
+    def clone(self):
+        return self
+
+
+class Constant(Initializer):
+    def __init__(self, value=0.0):
+        self.value = value
+
+    def __call__(self, shape, dtype, device, generator=None):
+        return torch.full(tuple(shape), self.value, dtype=torch.float32).to(dtype).to(device)
+
+    def clone(self):
+        return Constant(self.value)
+
+
+class GlorotUniform(Initializer):
+    def __init__(self, seed=None):
+        self.seed = seed
+
+    def __call__(self, shape, dtype, device, generator=None):
+        shape = tuple(shape)
+        if len(shape) < 1:
+            fan_in = fan_out = 1
+        elif len(shape) == 1:
+            fan_in = fan_out = shape[0]
+        elif len(shape) == 2:
+            fan_in, fan_out = shape
+        else:  # conv kernels: receptive field * channels
+            rf = int(np.prod(shape[:-2]))
+            fan_in, fan_out = shape[-2] * rf, shape[-1] * rf
+        limit = math.sqrt(6.0 / (fan_in + fan_out))
+        g = generator
+        if self.seed is not None:
+            g = torch.Generator().manual_seed(self.seed)
+        return ((torch.rand(shape, generator=g) * 2 - 1) * limit).to(dtype).to(device)
+
+
+_INITIALIZERS = {
+    'zeros': lambda: Constant(0.0),
+    'ones': lambda: Constant(1.0),
+    'glorot_uniform': lambda: GlorotUniform(),
+}
+
+
+def get_initializer(spec) -> Initializer:
+    if isinstance(spec, Initializer):
+        return spec
+    if isinstance(spec, (int, float, np.number)):
+        return Constant(float(spec))
+    if isinstance(spec, str) and spec in _INITIALIZERS:
+        return _INITIALIZERS[spec]()
+    raise ValueError(f'unknown initializer {spec!r}')
+
+
+_DTYPES = {'float32': torch.float32, 'uint8': torch.uint8, 'uint32': torch.uint32, 'int32': torch.int32, None: torch.float32}
+
+_default_device = None
+
+
+def set_default_device(device):
+    """Device on which layers create their variables when built without seeing a tensor."""
+    global _default_device
+    _default_device = torch.device(device) if device is not None else None
+
+
+def default_device():
+    if _default_device is not None:
+        return _default_device
+    return torch.device('cuda', torch.cuda.current_device()) if torch.cuda.is_available() else torch.device('cpu')
+
+
+_name_counts: dict[str, int] = {}
+
+
+def _auto_name(cls_name: str) -> str:
+    base = ''.join('_' + c.lower() if c.isupper() and i else c.lower() for i, c in enumerate(cls_name))
+    n = _name_counts.get(base, 0)
+    _name_counts[base] = n + 1
+    return base if n == 0 else f'{base}_{n}'
+
+
+class Layer(nn.Module):
+    """Keras-like layer on top of ``torch.nn.Module``."""
+
+    def __init__(self, name: str | None = None, trainable: bool = True, dtype: Any = None, **kwargs):
+        super().__init__()
+        if kwargs:
+            raise TypeError(f'unexpected keyword arguments {sorted(kwargs)} for {type(self).__name__}')
+        self.name = name or _auto_name(type(self).__name__)
+        self._layer_trainable = trainable
+        self.built = False
+        self._losses: list[torch.Tensor] = []
+        self._build_device = None
+
+    # ---- variables
+    @property
+    def trainable(self):
+        return self._layer_trainable
+
+    def add_weight(self, name, shape=(), initializer='zeros', trainable=True, dtype=None, constraint=None,
+                   regularizer=None, **_unused):
+        dt = _DTYPES[dtype] if not isinstance(dtype, torch.dtype) else dtype
+        device = self._build_device or default_device()
+        value = get_initializer(initializer)(shape, dt, device)
+        attr = f'_var_{name}'
+        if dt.is_floating_point:
+            p = nn.Parameter(value, requires_grad=bool(trainable) and self._layer_trainable)
+            p.constraint = constraint
+            p.regularizer = regularizer
+            p.var_name = name
+            self.register_parameter(attr, p)
+            return p
+        self.register_buffer(attr, value)
+        return getattr(self, attr)
+
+    # ---- losses
+    def add_loss(self, value):
+        self._losses.append(value)
+
+    @property
+    def losses(self):
+        """``add_loss`` terms of the last call of this layer and its sub-layers, plus the
+        regularization losses of all variables."""
+        out = []
+        for m in self.modules():
+            if isinstance(m, Layer):
+                out += m._losses
+        for p in self.parameters():
+            r = getattr(p, 'regularizer', None)
+            if r is not None:
+                out.append(r(p))
+        return out
+
+    def _clear_losses(self):
+        for m in self.modules():
+            if isinstance(m, Layer):
+                m._losses = []
+
+    def apply_constraints(self):
+        """What a Keras optimizer does after each update."""
+        with torch.no_grad():
+            for p in self.parameters():
+                c = getattr(p, 'constraint', None)
+                if c is not None and p.requires_grad:
+                    p.copy_(c(p))
+
+    # ---- build / call
+    def build(self, input_shape=None):
+        self.built = True
+
+    def compute_output_shape(self, input_shape):
+        return input_shape
+
+    def _maybe_build(self, args):
+        if self.built:
+            return
+        first = args[0]
+        if isinstance(first, (tuple, list)) and len(first) and isinstance(first[0], torch.Tensor):
+            self._build_device = first[0].device
+            self.build([tuple(t.shape) for t in first])
+        elif isinstance(first, torch.Tensor):
+            self._build_device = first.device
+            self.build(tuple(first.shape))
+        else:
+            self.build(None)
+        self.built = True
+
+    def __call__(self, *args, training=None, **kwargs):
+        outer = _training_ctx()
+        if training is None:
+            training = outer if outer is not None else False
+        top = getattr(_ctx, 'depth', 0) == 0
+        if top:
+            self._clear_losses()
+        else:
+            self._losses = []
+        _ctx.training = training
+        _ctx.depth = getattr(_ctx, 'depth', 0) + 1
+        try:
+            self._maybe_build(args)
+            return self._wrapped_call(*args, training=training, **kwargs)
+        finally:
+            _ctx.depth -= 1
+            _ctx.training = outer
+
+    def _wrapped_call(self, *args, training=None, **kwargs):
+        return self.call(*args, training=training, **kwargs)
+
+    def call(self, *args, **kwargs):
+        raise NotImplementedError
+
+    def forward(self, *args, **kwargs):  # nn.Module API
+        return self(*args, **kwargs)
+
+    def extra_repr(self):
+        return f'name={self.name}'
+
+
+class Sequential(Layer):
+    def __init__(self, layers=(), **kwargs):
+        super().__init__(**kwargs)
+        self.layers = nn.ModuleList(list(layers))
+
+    def add(self, layer):
+        self.layers.append(layer)
+
+    def build(self, input_shape=None):
+        self.built = True
+
+    def call(self, x, training=None):
+        for layer in self.layers:
+            x = layer(x) if not isinstance(layer, Layer) else layer(x, training=training)
+        return x

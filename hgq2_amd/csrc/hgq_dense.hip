@@ -359,9 +359,19 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
     else if (m.round_mode == HGQ_RND_CONV) fn = qdense_bwd_kernel<HGQ_RND_CONV, true>;
     else return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: unknown round mode");
     if (dyn > 8192) {
-        // static LDS is ~50 KB; ask for the part of the 160 KB per-CU LDS beyond the default 64 KB window
-        hipError_t e = hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
-        if (e != hipSuccess) return fail(HGQ_ERR_LAUNCH, "hgq_qdense_bwd: hipFuncSetAttribute: %s", hipGetErrorString(e));
+        // static LDS is ~50 KB; ask once per kernel for the part of the 160 KB LDS beyond the default 64 KB window
+        static const void *raised[8] = {nullptr};
+        bool done = false;
+        int slot = -1;
+        for (int t = 0; t < 8; ++t) {
+            if (raised[t] == (const void *)fn) done = true;
+            if (raised[t] == nullptr && slot < 0) slot = t;
+        }
+        if (!done) {
+            hipError_t e = hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, DF_LDS_MAX * 4);
+            if (e != hipSuccess) return fail(HGQ_ERR_LAUNCH, "hgq_qdense_bwd: hipFuncSetAttribute: %s", hipGetErrorString(e));
+            if (slot >= 0) raised[slot] = (const void *)fn;
+        }
     }
     hipLaunchKernelGGL(fn, grid, dim3(256), dyn, s, dy, y, x, f_in, quant ? bw_rows : (int64_t)1, qw, dx, dqw, dqb, df_in, rows, K, N, act,
                        mode, df_lds);

@@ -17,11 +17,11 @@ namespace hgq {
 
 struct Mode {
     int round_mode, overflow_mode;
-    bool training, kbi, round_params, k_u8, symmetric, tracing;
+    bool training, kbi, round_params, k_u8, symmetric, tracing, track_input;
     __host__ __device__ explicit Mode(int m)
         : round_mode(m & 0xf), overflow_mode((m >> 4) & 0xf), training(m & HGQ_MODE_TRAINING),
           kbi(m & HGQ_MODE_KBI), round_params(m & HGQ_MODE_ROUND_PARAMS), k_u8(m & HGQ_MODE_K_U8),
-          symmetric(m & HGQ_MODE_SYMMETRIC), tracing(m & HGQ_MODE_TRACING) {}
+          symmetric(m & HGQ_MODE_SYMMETRIC), tracing(m & HGQ_MODE_TRACING), track_input(m & HGQ_MODE_TRACK_INPUT) {}
 };
 
 // 2**e for an integer-valued float e (exact, including subnormal results).

@@ -116,8 +116,9 @@ __global__ __launch_bounds__(256) void quant_fwd_1d(const float *__restrict__ x,
         for (int c = 0; c < VEC; ++c) {
             const KIF p = SHARED ? ps : resolve_kif(kv[c], iv[c], fv[c], m.kbi, m.round_params);
             yv[c] = quantize<RM, OM>(xv[c], p, m.training);
-            ab[c] = abs_bits(yv[c]);
-            ng[c] = yv[c] < 0.0f ? 1u : 0u;
+            const float tv = m.track_input ? xv[c] : yv[c];
+            ab[c] = abs_bits(tv);
+            ng[c] = tv < 0.0f ? 1u : 0u;
             lmax = ab[c] > lmax ? ab[c] : lmax;
             lneg |= ng[c];
         }
@@ -222,9 +223,10 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 yv[e] = quantize<RM, OM>(xv[e], p[e], m.training);
-                const uint32_t ab = abs_bits(yv[e]);
+                const float tv = m.track_input ? xv[e] : yv[e];
+                const uint32_t ab = abs_bits(tv);
                 lmax[e] = ab > lmax[e] ? ab : lmax[e];
-                lneg[e] |= yv[e] < 0.0f ? 1u : 0u;
+                lneg[e] |= tv < 0.0f ? 1u : 0u;
             }
             VecIO<VEC>::store(y, r * cg + c, yv);
         }
@@ -329,8 +331,9 @@ __global__ __launch_bounds__(256) void quant_fwd_generic(const float *__restrict
         const KIF p = resolve_kif(load_k(k, b, m.k_u8), i[b], fb[b], m.kbi, m.round_params);
         const float yv = quantize<RM, OM>(x[e], p, m.training);
         y[e] = yv;
-        if (amax) atomicMax(&amax[b], abs_bits(yv));
-        if (anyneg && yv < 0.0f) atomicOr(&anyneg[b], 1u);
+        const float tv = m.track_input ? x[e] : yv;
+        if (amax) atomicMax(&amax[b], abs_bits(tv));
+        if (anyneg && tv < 0.0f) atomicOr(&anyneg[b], 1u);
     }
 }
 

@@ -1,0 +1,203 @@
+"""QEinsumDense (reference src/hgq/layers/core/einsum_dense.py:10-115).
+
+Equations whose kernel axes are ``<contracted axes><new output axes>`` and whose input ends with
+the contracted axes (``'bpf,fh->bph'``, ``'abc,cde->abde'``, ``'abcd,cde->abe'`` ...) reshape to
+one GEMM and run through the fused dense kernels; every other equation quantizes the operands
+with the quantizer kernels and contracts with ``torch.einsum``.
+"""
+
+from __future__ import annotations
+
+import re
+from math import prod
+
+import torch
+
+from ...core import get_initializer
+from ...quantizer import Quantizer
+from ...quantizer.config import QuantizerConfig
+from ._contraction import dense_contraction, dense_ebops_fast, get_activation
+from .base import QLayerBaseSingleInput
+
+
+def _einsum_free0_size(equation: str, input_shape) -> int:
+    """Number of times the kernel is reused across the non-batch input axes."""
+    _inp, _ker_out = equation.split(',', 1)
+    _ker, _out = _ker_out.split('->', 1)
+    elided_size = len(input_shape) - len(_inp) + 3
+    _inp = _inp.replace('...', '?' * elided_size)
+    n_parallel = 1
+    for ax, dim in zip(_inp[1:], input_shape[1:]):
+        if ax not in _ker and (ax in _out or ax == '?'):
+            assert dim is not None, f'Cannot determine input loop size for einsum eq: {equation} with input shape {input_shape}'
+            n_parallel *= dim
+    return n_parallel
+
+
+def analyze_einsum_string(equation, bias_axes, input_shape, output_shape):
+    """Kernel shape, bias shape and full output shape of an EinsumDense equation (no ellipsis)."""
+    m = re.match(r'([a-zA-Z]+),([a-zA-Z]+)->([a-zA-Z]+)', equation)
+    if not m or '...' in equation:
+        raise NotImplementedError(f'einsum equation {equation!r}: only ellipsis-free "ab,bc->ac" forms are supported')
+    in_spec, w_spec, out_spec = m.groups()
+    output_shape = [output_shape] if isinstance(output_shape, int) else list(output_shape)
+    output_shape.insert(0, input_shape[0])
+    if len(in_spec) != len(input_shape) or len(out_spec) != len(output_shape):
+        raise ValueError(f'equation {equation} does not match input shape {input_shape} / output shape {output_shape}')
+    in_map = {d: i for i, d in enumerate(in_spec)}
+    out_map = {d: i for i, d in enumerate(out_spec)}
+    for d in out_spec:
+        if d not in in_spec and d not in w_spec:
+            raise ValueError(f"Dimension '{d}' was specified in the output '{out_spec}' but has no corresponding dim")
+    w_shape = []
+    for d in w_spec:
+        if d in in_map:
+            w_shape.append(input_shape[in_map[d]])
+        elif d in out_map:
+            w_shape.append(output_shape[out_map[d]])
+        else:
+            raise ValueError(f"Weight dimension '{d}' did not have a match in either the input or the output spec")
+    bias_shape = None
+    if bias_axes is not None:
+        for c in bias_axes:
+            if c not in out_spec:
+                raise ValueError(f"Bias dimension '{c}' was requested, but is not part of the output spec '{out_spec}'")
+        first = min(out_spec.find(c) for c in bias_axes)
+        bias_shape = [output_shape[out_map[c]] if c in bias_axes else 1 for c in out_spec[first:]]
+    return tuple(w_shape), None if bias_shape is None else tuple(bias_shape), tuple(output_shape)
+
+
+def gemm_form(equation):
+    """(n_contract, n_new) if the equation is ``<free><C>,<C><O>-><free><O>``, else None."""
+    in_spec, rest = equation.split(',', 1)
+    w_spec, out_spec = rest.split('->', 1)
+    for nc in range(1, len(w_spec)):
+        c, o = w_spec[:nc], w_spec[nc:]
+        if in_spec.endswith(c) and out_spec == in_spec[:len(in_spec) - nc] + o and not (set(o) & set(in_spec)):
+            return nc, len(o)
+    return None
+
+
+class QEinsumDense(QLayerBaseSingleInput):
+    def __init__(self, equation, output_shape, activation=None, bias_axes=None, kernel_initializer='glorot_uniform',
+                 bias_initializer='zeros', kernel_regularizer=None, bias_regularizer=None, kernel_constraint=None,
+                 bias_constraint=None, kq_conf: None | QuantizerConfig = None, iq_conf: None | QuantizerConfig = None,
+                 bq_conf: None | QuantizerConfig = None, parallelization_factor: int = -1, **kwargs):
+        super().__init__(iq_conf=iq_conf, **kwargs)
+        self.equation = equation
+        self.partial_output_shape = (output_shape,) if isinstance(output_shape, int) else tuple(output_shape)
+        self.bias_axes = bias_axes
+        self.activation, self._act_name = get_activation(activation)
+        self.kernel_initializer = get_initializer(kernel_initializer)
+        self.bias_initializer = get_initializer(bias_initializer)
+        self.kernel_regularizer, self.bias_regularizer = kernel_regularizer, bias_regularizer
+        self.kernel_constraint, self.bias_constraint = kernel_constraint, bias_constraint
+        kq_conf = kq_conf or QuantizerConfig('default', 'weight')
+        self._kq = Quantizer(kq_conf, name=f'{self.name}_kq')
+        bq_conf = bq_conf or QuantizerConfig('default', 'bias')
+        self._bq = None if bias_axes is None else Quantizer(bq_conf, name=f'{self.name}_bq')
+        self.parallelization_factor = parallelization_factor
+        self.bias = None
+
+    @property
+    def kq(self):
+        return self._kq
+
+    @property
+    def bq(self):
+        return self._bq
+
+    @property
+    def kernel(self):
+        return self._kernel
+
+    def build(self, input_shape):
+        super().build(input_shape)
+        kernel_shape, bias_shape, full_output_shape = analyze_einsum_string(
+            self.equation, self.bias_axes, tuple(input_shape), self.partial_output_shape)
+        self.full_output_shape = tuple(full_output_shape)
+        self._kernel = self.add_weight(name='kernel', shape=kernel_shape, initializer=self.kernel_initializer,
+                                       regularizer=self.kernel_regularizer, constraint=self.kernel_constraint)
+        if bias_shape is not None:
+            self.bias = self.add_weight(name='bias', shape=bias_shape, initializer=self.bias_initializer,
+                                        regularizer=self.bias_regularizer, constraint=self.bias_constraint)
+        self.n_parallel = _einsum_free0_size(self.equation, input_shape)
+        if self.parallelization_factor < 0:
+            self.parallelization_factor = self.n_parallel
+        for q, shape in ((self.kq, kernel_shape), (self.bq, bias_shape)):
+            if q is not None:
+                q._build_device = self._build_device
+                q.build(tuple(shape))
+                q.built = True
+        self.ebops_equation = self.equation.split('->')[0] + '->'
+        self._gemm = gemm_form(self.equation)
+        if self._gemm is not None:
+            nc, _ = self._gemm
+            self._K = prod(kernel_shape[:nc])
+            self._N = prod(kernel_shape[nc:])
+            # the bias rides in the GEMM epilogue only when it is exactly one value per output column
+            self._bias_in_gemm = bias_shape is not None and prod(bias_shape) == self._N and \
+                tuple(s for s in bias_shape if s != 1) == tuple(s for s in kernel_shape[nc:] if s != 1)
+
+    def compute_output_shape(self, input_shape):
+        return (input_shape[0],) + tuple(self.full_output_shape[1:])
+
+    def _contract(self, inputs, qkernel, qbias, training):
+        iq = self.iq if self.enable_iq else None
+        if self._gemm is not None:
+            nc, _ = self._gemm
+            x = inputs  # the contracted axes are trailing and contiguous: a [rows, K] view of the same memory
+            b1d = qbias.reshape(-1) if (qbias is not None and self._bias_in_gemm) else None
+            fuse_act = self._act_name if (qbias is None or self._bias_in_gemm) else None
+            y, act_done = dense_contraction(x, iq, qkernel.reshape(self._K, self._N), b1d, fuse_act, training)
+            y = y.view(inputs.shape[0], *self.full_output_shape[1:])
+            if qbias is not None and not self._bias_in_gemm:
+                y = y + qbias
+            return y, act_done
+        if iq is not None:
+            inputs = iq(inputs, training=training)
+        y = torch.einsum(self.equation, inputs, qkernel)
+        if qbias is not None:
+            y = y + qbias
+        return y, False
+
+    def call(self, inputs, training=None):
+        qkernel = self.kq(self._kernel, training=training)
+        qbias = self.bq(self.bias, training=training) if self.bias is not None else None
+        y, act_done = self._contract(inputs, qkernel, qbias, training)
+        if self.activation is not None and not act_done:
+            y = self.activation(y)
+        return y
+
+    def _compute_ebops(self, shape):
+        scale = self.parallelization_factor / self.n_parallel
+        out_size = float(prod(self.full_output_shape[1:]))
+        if self._gemm is not None and (self.bq is None or self._bias_in_gemm):
+            fast = dense_ebops_fast(self.iq, self.kq, self.bq, self._K, self._N, scale, out_size)
+            if fast is not None:
+                return fast
+        bw_inp = self.iq.bits_(shape)
+        bw_ker = self.kq.bits_(self._kernel.shape)
+        ebops = torch.einsum(self.ebops_equation, bw_inp, bw_ker)
+        if self.bq is not None:
+            bw_bias = self.bq.bits_(self.bias.shape)
+            ebops = ebops + torch.mean(bw_bias) * out_size
+        return ebops * scale
+
+    def get_config(self):
+        config = super().get_config()
+        config.update({'equation': self.equation, 'output_shape': self.partial_output_shape, 'bias_axes': self.bias_axes,
+                       'activation': self._act_name, 'kq_conf': self.kq.config,
+                       'bq_conf': self.bq.config if self.bq is not None else None,
+                       'parallelization_factor': self.parallelization_factor})
+        return config
+
+    @property
+    def qkernel(self):
+        return self.kq(self._kernel)
+
+    @property
+    def qbias(self):
+        if self.bias is None:
+            return None
+        return self.bq(self.bias)

@@ -1,0 +1,94 @@
+"""The generic quantizer layer (reference src/hgq/quantizer/quantizer.py:10-104): wraps an
+internal quantizer and adds the optional scaler, quantization-noise blend and affine map."""
+
+from __future__ import annotations
+
+import torch
+
+from ..core import Layer
+from .config import QuantizerConfig, all_quantizer_keys
+
+
+class Quantizer(Layer):
+    """``Quantizer(config)`` or ``Quantizer(q_type=..., place=..., **quantizer_kwargs)``."""
+
+    def __init__(self, *args, **kwargs):
+        self.supports_masking = True
+        config, kwargs = self.get_quantizer_config_kwargs(*args, **kwargs)
+        super().__init__(**kwargs)
+        self.config = config
+        self.qnoise_factor = config.qnoise_factor
+        self.scaler = config.scaler
+        self.affine = config.affine
+        self.quantizer = config.get_quantizer()
+
+    def build(self, input_shape):
+        if not self.quantizer.built:
+            self.quantizer._build_device = self._build_device
+            self.quantizer.build(tuple(input_shape))
+            self.quantizer.built = True
+        self.built = True
+
+    def get_quantizer_config_kwargs(self, *args, **kwargs):
+        if len(args) == 1 and isinstance(args[0], QuantizerConfig):
+            return args[0], kwargs
+        config = kwargs.pop('config', None)
+        if isinstance(config, QuantizerConfig):
+            return config, kwargs
+        assert config is None, f'config must be a QuantizerConfig object, got {config}'
+        q_kwargs = {k: kwargs.pop(k) for k in list(kwargs) if k in all_quantizer_keys}
+        return QuantizerConfig(*args, **q_kwargs), kwargs
+
+    def call(self, inputs, training=None):
+        if self.scaler is not None:
+            inputs = inputs / self.scaler
+        outputs = self.quantizer(inputs, training=training)
+        if self.scaler is not None:
+            outputs = outputs * self.scaler
+        if self.qnoise_factor is not None and training:
+            outputs = inputs + self.qnoise_factor * (outputs - inputs)
+        if self.affine is not None:
+            outputs = outputs * self.affine[0] + self.affine[1]
+        return outputs
+
+    @property
+    def plain(self) -> bool:
+        """No scaler / noise blend / affine: the call is exactly the internal quantizer."""
+        return self.scaler is None and self.qnoise_factor is None and self.affine is None
+
+    def get_config(self):
+        return {'config': self.config}
+
+    @property
+    def bits(self):
+        return self.quantizer.bits
+
+    @property
+    def fbits(self):
+        return self.quantizer.fbits
+
+    @property
+    def q_type(self):
+        return self.config.q_type
+
+    def __repr__(self):
+        return f'{self.__class__.__name__}(q_type={self.config.q_type}, name={self.name}, built={self.built})'
+
+    def _bw_to_x(self, t, shape):
+        t = torch.as_tensor(t)
+        return self.quantizer.bw_mapper.bw_to_x(t, shape)
+
+    def bits_(self, shape):
+        return self._bw_to_x(self.bits, shape)
+
+    def fbits_(self, shape):
+        return self._bw_to_x(self.fbits, shape)
+
+    def min_(self, shape):
+        return self._bw_to_x(self.quantizer.min, shape)
+
+    def max_(self, shape):
+        return self._bw_to_x(self.quantizer.max, shape)
+
+    def epsilon_(self, shape):
+        return self._bw_to_x(self.quantizer.epsilon, shape)

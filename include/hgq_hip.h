@@ -52,6 +52,7 @@ extern "C" {
 #define HGQ_MODE_K_U8 (1 << 11)        /* k operand is uint8 (the reference's `_k` variable dtype) */
 #define HGQ_MODE_SYMMETRIC (1 << 12)   /* hgq_wrap_track_i: the symmetric minimal-i formula */
 #define HGQ_MODE_TRACING (1 << 13)     /* hgq_wrap_track_i: calibration ("tracing") update rule */
+#define HGQ_MODE_TRACK_INPUT (1 << 14) /* hgq_quantize_fwd: amax / anyneg observe x instead of y (KBI WRAP tracks the un-rounded input) */
 
 #define HGQ_ACT_NONE 0
 #define HGQ_ACT_RELU 1

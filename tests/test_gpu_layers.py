@@ -1,0 +1,143 @@
+"""GPU parity of the layer API (hgq2_amd.layers / quantizer / config) against the CPU oracle's
+restatement of the reference's Python, on identical weights and inputs."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hgq_ref as ref
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+def _copy_mlp(src: 'ref.RefMLP', model, dev):
+    """Load the oracle's weights and bit-widths into the product model."""
+    with torch.no_grad():
+        for rl, pl in zip(src.layers, model.layers):
+            pl._kernel.copy_(rl.kernel.detach().to(dev))
+            pl.bias.copy_(rl.bias.detach().to(dev))
+            for rq, pq in ((rl.iq, pl.iq), (rl.kq, pl.kq), (rl.bq, pl.bq)):
+                for name, t in rq.quantizer.variables().items():
+                    getattr(pq.quantizer, name).copy_(t.detach().to(dev))
+
+
+def _close(got, want, scale=None, rtol=RTOL, what=''):
+    got, want = got.detach().double().cpu(), want.detach().double()
+    tol = rtol * (want.abs() if scale is None else scale) + 1e-12
+    err = (got - want).abs()
+    assert torch.all(err <= tol), f'{what}: max err {err.max():.3e}, tol {tol.max():.3e}'
+
+
+def test_scopes_produce_reference_default_configs():
+    from hgq2_amd.utils.models import qdense_mlp
+    from hgq2_amd.quantizer.internal import FixedPointQuantizerKBI, FixedPointQuantizerKIF
+
+    m = qdense_mlp(device='cpu')
+    l0 = m.layers[0]
+    assert isinstance(l0.iq.quantizer, FixedPointQuantizerKIF) and l0.iq.quantizer.overflow_mode == 'WRAP'
+    assert isinstance(l0.kq.quantizer, FixedPointQuantizerKBI) and l0.kq.quantizer.overflow_mode == 'SAT_SYM'
+    assert isinstance(l0.bq.quantizer, FixedPointQuantizerKBI) and l0.bq.quantizer.overflow_mode == 'SAT_SYM'
+    assert tuple(l0.iq.quantizer._i.shape) == (1, 16) and tuple(l0.kq.quantizer._b.shape) == (16, 64)
+    assert l0.iq.quantizer._k.dtype == torch.uint8 and l0._ebops.dtype == torch.uint32
+
+
+@pytest.mark.parametrize('batch', (16384, 1000))
+def test_mlp_training_steps_match_oracle(dev, batch):
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, model_loss
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(batch, 16, generator=g)
+    labels = torch.randint(0, 5, (batch,), generator=g)
+    oracle = ref.RefMLP(seed=1)
+    model = qdense_mlp(device=dev)
+    _copy_mlp(oracle, model, dev)
+    opt = SGD(model.parameters(), lr=0.01)
+    xd, yd = x.to(dev), labels.to(dev)
+    for step in range(3):
+        want_loss, want_logits = oracle.train_step(x, labels, lr=0.01)
+        opt.zero_grad()
+        logits = model(xd, training=True)
+        loss = model_loss(model, ops.sparse_ce(logits, yd))
+        loss.backward()
+        opt.step()
+        _close(logits, want_logits, scale=want_logits.abs() + 1.0, rtol=2e-5, what=f'logits step {step}')
+        assert abs(loss.item() - want_loss.item()) <= 2e-5 * abs(want_loss.item())
+        for n, (rl, pl) in enumerate(zip(oracle.layers, model.layers)):
+            # tracked integer bits and EBOPs: exact
+            assert torch.equal(pl.iq.quantizer._i.cpu(), rl.iq.quantizer._i.detach()), f'layer {n} _i step {step}'
+            assert int(pl.ebops.cpu().view(torch.int32)) == int(rl.ebops_value), f'layer {n} ebops step {step}'
+            _close(pl._kernel, rl.kernel, scale=rl.kernel.detach().abs() + 1e-3, what=f'kernel {n}')
+            _close(pl.bias, rl.bias, scale=rl.bias.detach().abs() + 1e-3, what=f'bias {n}')
+            _close(pl.iq.quantizer._f, rl.iq.quantizer._f, scale=rl.iq.quantizer._f.detach().abs() + 1e-3, what=f'iq._f {n}')
+            _close(pl.kq.quantizer._b, rl.kq.quantizer._b, scale=rl.kq.quantizer._b.detach().abs() + 1e-3, what=f'kq._b {n}')
+            _close(pl.kq.quantizer._i, rl.kq.quantizer._i, scale=rl.kq.quantizer._i.detach().abs() + 1e-3, what=f'kq._i {n}')
+            _close(pl.bq.quantizer._b, rl.bq.quantizer._b, scale=rl.bq.quantizer._b.detach().abs() + 1e-3, what=f'bq._b {n}')
+
+
+def test_mlp_inference_matches_oracle_bitexact_inputs(dev):
+    """Inference mode (WRAP applied, empty words zeroed): quantized activations are exact; the
+    logits are compared at 1e-5."""
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4096, 16, generator=g) * 3
+    oracle = ref.RefMLP(seed=2)
+    model = qdense_mlp(device=dev)
+    with torch.no_grad():
+        for layer in oracle.layers:  # make the first layer overflow and one lane empty
+            layer.iq.quantizer._i.fill_(1.0)
+        oracle.layers[0].iq.quantizer._f[0, 3] = -2.0
+        oracle.layers[0].iq.quantizer._k[0, 3] = 0
+    _copy_mlp(oracle, model, dev)
+    with torch.no_grad():
+        want = oracle.forward(x, training=False)
+        got = model(x.to(dev), training=False)
+        q0 = model.layers[0].iq(x.to(dev), training=False)
+        w0 = oracle.layers[0].iq(x, training=False)
+    assert torch.equal(q0.cpu(), w0)
+    assert torch.all(q0[:, 3] == 0)
+    _close(got, want, scale=want.abs() + 1.0, rtol=2e-5, what='logits')
+
+
+def test_graphed_step_equals_eager_steps(dev):
+    """HIP-graph replays of the training step give the same trajectory as eager steps."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, GraphedTrainStep, model_loss
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(5)
+    xs = [torch.randn(2048, 16, generator=g).to(dev) for _ in range(4)]
+    ys = [torch.randint(0, 5, (2048,), generator=g).to(dev) for _ in range(4)]
+    src = ref.RefMLP(seed=4)
+
+    eager = qdense_mlp(device=dev)
+    _copy_mlp(src, eager, dev)
+    opt = SGD(eager.parameters(), lr=0.01, fold_regularizers=True)
+    graphed = qdense_mlp(device=dev)
+    _copy_mlp(src, graphed, dev)
+    gopt = SGD(graphed.parameters(), lr=0.01, fold_regularizers=True)
+    # capture warms up on (and therefore trains on) its example batch: give both models the same history
+    warm = 3
+    for _ in range(warm + 1):
+        opt.zero_grad()
+        loss = model_loss(eager, ops.sparse_ce(eager(xs[0], training=True), ys[0]), True)
+        loss.backward()
+        opt.step()
+    step = GraphedTrainStep(graphed, ops.sparse_ce, gopt, xs[0], ys[0], warmup=warm)
+    step()  # first replay = the (warm+1)-th step on the example batch
+    for x, y in zip(xs[1:], ys[1:]):
+        opt.zero_grad()
+        loss = model_loss(eager, ops.sparse_ce(eager(x, training=True), y), True)
+        loss.backward()
+        opt.step()
+        gl = step(x, y)
+        torch.cuda.synchronize()
+        assert abs(gl.item() - loss.item()) <= 1e-5 * abs(loss.item())
+        for pe, pg in zip(eager.parameters(), graphed.parameters()):
+            np.testing.assert_allclose(pg.detach().cpu().numpy(), pe.detach().cpu().numpy(), rtol=1e-4, atol=1e-6)
+        for le, lg in zip(eager.layers, graphed.layers):
+            assert torch.equal(le.iq.quantizer._i, lg.iq.quantizer._i)
+            assert int(le.ebops.cpu().view(torch.int32)) == int(lg.ebops.cpu().view(torch.int32))
