@@ -1,0 +1,191 @@
+"""Benchmark: QDense MLP 16-64-32-32-5 training step at batch 16384 (samples/s), plus the
+quantizer kernels' achieved HBM bandwidth on the 4 Mi-element standalone case, plus the CPU
+oracle timed on the host cores as a baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints one JSON line.  Everything is synthetic (seeded) data with inputs resident in HBM.
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+BATCH = 16384
+DIMS = (16, 64, 32, 32, 5)
+QN = 4 * 1024 * 1024  # standalone quantizer case: 4 Mi fp32 elements
+
+
+def _events_ms(fn, iters):
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def quantizer_roofline(iters=200):
+    """Standalone KIF quantizer, RND/WRAP, per-element k, i, f, training forward + surrogate
+    backward, launched straight through the C ABI on torch's current stream and timed with HIP
+    events on that stream."""
+    import torch
+
+    from hgq2_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(0)
+    # The MI355X has a 256 MB memory-side cache; one launch touches 80-128 MB, so re-running on
+    # one buffer set would be served from that cache.  Rotate over enough distinct sets (> 1 GB in
+    # total) that every launch streams from HBM.
+    n_sets = 10
+    sets = []
+    for _ in range(n_sets):
+        x = (torch.randn(QN, generator=g) * 2.0).to(dev)  # N(0, sigma^2 = 4)
+        k = torch.ones(QN, device=dev)
+        i = torch.randint(0, 5, (QN,), generator=g).float().to(dev)
+        f = torch.randint(0, 9, (QN,), generator=g).float().to(dev)
+        dy = torch.randn(QN, generator=g).to(dev)
+        sets.append((x, k, i, f, dy) + tuple(torch.empty(QN, device=dev) for _ in range(4)))
+    mode = _lib.mode_bits('RND', 'WRAP', training=True)
+    s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    state = {'n': 0}
+
+    def fwd():
+        x, k, i, f, dy, y, dx, di, df = sets[state['n'] % n_sets]
+        state['n'] += 1
+        rc = lib.hgq_quantize_fwd(p(x), p(k), p(i), p(f), p(y), None, None, QN, QN, 1, mode, s)
+        assert rc == 0
+
+    def bwd():
+        x, k, i, f, dy, y, dx, di, df = sets[state['n'] % n_sets]
+        state['n'] += 1
+        rc = lib.hgq_quantize_bwd(p(dy), p(x), p(k), p(i), p(f), p(dx), p(di), p(df), QN, QN, 1, mode, s)
+        assert rc == 0
+
+    for _ in range(10):
+        fwd(), bwd()
+    t_fwd = _events_ms(fwd, iters)
+    t_bwd = _events_ms(bwd, iters)
+    out = {}
+    for name, ms, bpe in (('quant_fwd_1d', t_fwd, 20), ('quant_bwd_1d', t_bwd, 32)):
+        gbs = bpe * QN / (ms * 1e-3) / 1e9
+        out[name] = {'ms': ms, 'bytes': bpe * QN, 'GBps': gbs, 'frac': gbs / HBM_PEAK_GBS}
+    return out
+
+
+def cpu_baseline(budget_s=20.0):
+    """The oracle's eager torch-CPU restatement of the reference path, same model and batch."""
+    import torch
+
+    from oracle import hgq_ref as ref
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(BATCH, DIMS[0], generator=g)
+    labels = torch.randint(0, DIMS[-1], (BATCH,), generator=g)
+    mlp = ref.RefMLP(dims=DIMS, seed=1)
+    for _ in range(3):
+        mlp.train_step(x, labels)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        mlp.train_step(x, labels)
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 200:
+            break
+    return {'value': BATCH * n / el, 'unit': 'samples/s', 'cores': cores, 'kind': 'port',
+            'sample': f'{n} training steps of the same MLP at batch {BATCH} (eager torch-CPU restatement of the reference path)'}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=300)
+    ap.add_argument('--warmup', type=int, default=30)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--eager', action='store_true', help='time eager steps instead of HIP-graph replays')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f'bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported', file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, GraphedTrainStep, model_loss
+    from hgq2_amd.utils.models import qdense_mlp
+
+    dev = torch.device('cuda:0')
+    torch.cuda.set_device(dev)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(BATCH, DIMS[0], generator=g).to(dev)
+    labels = torch.randint(0, DIMS[-1], (BATCH,), generator=g).to(dev)
+    torch.manual_seed(1)
+    model = qdense_mlp(DIMS, beta0=1e-5, device=dev)
+    opt = SGD(model.parameters(), lr=0.01, fold_regularizers=True)
+
+    if args.eager:
+        def step():
+            opt.zero_grad()
+            loss = model_loss(model, ops.sparse_ce(model(x, training=True), labels), True)
+            loss.backward()
+            opt.step()
+            return loss
+    else:
+        step = GraphedTrainStep(model, ops.sparse_ce, opt, x, labels, warmup=3)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    el = time.perf_counter() - t0
+    ms_per_step = el / args.steps * 1e3
+    value = BATCH * args.steps / el
+
+    qr = quantizer_roofline()
+    dom = qr['quant_bwd_1d']
+    roofline = {'bound': 'hbm', 'kernel': 'quant_bwd_1d', 'achieved': dom['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                'frac': dom['frac'], 'traffic': None,
+                'workload': 'standalone kif quantizer RND/WRAP, 4 Mi fp32 elements, per-element k/i/f: backward 32 B/elem'}
+    out = {
+        'metric': 'QDense MLP train samples/s @bs16384; quantizer HBM GB/s vs peak',
+        'value': value, 'unit': 'samples/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32',
+        'data': 'synthetic',
+        'config': {'workload': 'QDense MLP 16-64-32-32-5 (ReLU hidden, linear out), batch 16384, kbi SAT_SYM weights, '
+                               'kif WRAP datalanes, EBOPs beta0=1e-5, sparse CE, one fwd+bwd+SGD step'
+                               + (' (eager launches)' if args.eager else ' (HIP-graph replay)')},
+        'final_loss': float(loss),
+        'roofline': roofline,
+        'quantizer_kernels': qr,
+    }
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline()
+        out['gpu_over_cpu'] = value / out['cpu_baseline']['value']
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

@@ -35,15 +35,19 @@ SIGNATURES = {
     'hgq_last_error': (c_char_p, []),
     'hgq_quantize_fwd': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_bwd': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
-    'hgq_wrap_track_i': (c_int, [c_void_p] * 5 + [c_int64, c_float, c_float, c_float, c_int, c_void_p]),
+    'hgq_wrap_track_i': (c_int, [c_void_p] * 2 + [c_int] + [c_void_p] * 3 + [c_int64, c_float, c_float, c_float, c_int, c_void_p]),
+    'hgq_qdense_fwd_parts': (c_int, [c_int64]),
+    'hgq_qdense_bwd_workspace': (c_int64, [c_int64, c_int, c_int, c_int64]),
     'hgq_qdense_fwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 4 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
-    'hgq_qdense_bwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_qdense_bwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 6 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     'hgq_dense_ebops': (
         c_int,
-        [c_void_p] * 3 + [c_int64, c_int, c_int] + [c_void_p] * 4 + [c_float, c_float, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p],
+        [c_void_p, c_int, c_float, c_void_p, c_void_p] + [c_void_p] * 3 + [c_int64, c_int, c_int] + [c_void_p] * 4
+        + [c_float, c_float, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p],
     ),
     'hgq_sparse_ce_fwd_bwd': (c_int, [c_void_p] * 4 + [c_int64, c_int, c_void_p]),
     'hgq_sgd_update': (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_float, c_void_p]),
+    'hgq_sgd_update_multi': (c_int, [c_void_p, c_int, c_float, c_void_p]),
     'hgq_fill_u32': (c_int, [c_void_p, ctypes.c_uint32, c_int64, c_void_p]),
 }
 

@@ -20,39 +20,47 @@ namespace hgq {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-#define FWD_BM 128
+#define FWD_BM 64
 #define FWD_BK 32
 #define FWD_BN 64
 #define AMAX_LDS_MAX 8192
+#define MAX_PARTS 512
 
 __device__ __forceinline__ int acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
 
+// Workgroup `g` of the row grid owns slice `g` of `amax_part` ([gridDim.x, P*K]): no atomics
+// between workgroups, no clearing pass; the integer-bit tracking kernel reduces over the slices.
 template <int RM, int OM, bool QUANT>
 __global__ __launch_bounds__(256) void qdense_fwd_kernel(const float *__restrict__ x, const void *__restrict__ k_in,
                                                          const float *__restrict__ i_in, const float *__restrict__ f_in,
                                                          int64_t P, const float *__restrict__ qw,
                                                          const float *__restrict__ qb, float *__restrict__ y,
-                                                         uint32_t *amax, int64_t rows, int K, int N, int act, int mode,
-                                                         int vec_ok, int amax_lds) {
+                                                         uint32_t *amax_part, int64_t rows, int K, int N, int act,
+                                                         int mode, int vec_ok, int amax_lds) {
     __shared__ float xs[FWD_BM][FWD_BK + 1];
     __shared__ float ws[FWD_BK][FWD_BN];
     extern __shared__ uint32_t amax_s[];  // [P*K] when amax_lds
 
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rh = wave & 1, cb = wave >> 1;  // this wave's 32 x 32 output block of the 64 x 64 tile
     const int n0 = blockIdx.y * FWD_BN;
     const int nw = min(FWD_BN, N - n0);
     const int64_t n_tiles = (rows + FWD_BM - 1) / FWD_BM;
     const int64_t PK = P * (int64_t)K;
-    const bool track = QUANT && amax != nullptr && blockIdx.y == 0;
+    const bool track = QUANT && amax_part != nullptr && blockIdx.y == 0;
+    uint32_t *my_amax = track ? amax_part + (int64_t)blockIdx.x * PK : nullptr;
 
-    if (track && amax_lds)
-        for (int64_t t = tid; t < PK; t += 256) amax_s[t] = 0;
+    if (track) {
+        if (amax_lds) for (int64_t t = tid; t < PK; t += 256) amax_s[t] = 0;
+        else for (int64_t t = tid; t < PK; t += 256) my_amax[t] = 0;
+        __threadfence_block();
+    }
     __syncthreads();
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t r0 = tile * FWD_BM;
-        floatx16 acc0 = {0}, acc1 = {0};
+        floatx16 acc = {0};
         for (int k0 = 0; k0 < K; k0 += FWD_BK) {
             const int kw = min(FWD_BK, K - k0);
             // ---- stage the (quantized) input tile
@@ -71,10 +79,7 @@ __global__ __launch_bounds__(256) void qdense_fwd_kernel(const float *__restrict
                             for (int e = 0; e < 4; ++e) {
                                 const KIF p = resolve_kif(load_k(k_in, b + e, m.k_u8), i_in[b + e], f_in[b + e], m.kbi, m.round_params);
                                 v[e] = quantize<RM, OM>(v[e], p, m.training);
-                                if (track) {
-                                    if (amax_lds) atomicMax(&amax_s[b + e], abs_bits(v[e]));
-                                    else atomicMax(&amax[b + e], abs_bits(v[e]));
-                                }
+                                if (track && P > 1) atomicMax(amax_lds ? &amax_s[b + e] : &my_amax[b + e], abs_bits(v[e]));
                             }
                         }
                     }
@@ -92,10 +97,7 @@ __global__ __launch_bounds__(256) void qdense_fwd_kernel(const float *__restrict
                             const int64_t b = (gr % P) * K + k0 + c;
                             const KIF p = resolve_kif(load_k(k_in, b, m.k_u8), i_in[b], f_in[b], m.kbi, m.round_params);
                             v = quantize<RM, OM>(v, p, m.training);
-                            if (track) {
-                                if (amax_lds) atomicMax(&amax_s[b], abs_bits(v));
-                                else atomicMax(&amax[b], abs_bits(v));
-                            }
+                            if (track && P > 1) atomicMax(amax_lds ? &amax_s[b] : &my_amax[b], abs_bits(v));
                         }
                     }
                     xs[row][c] = v;
@@ -111,32 +113,35 @@ __global__ __launch_bounds__(256) void qdense_fwd_kernel(const float *__restrict
                 ws[kk][nn] = (kk < kw && nn < nw) ? qw[(int64_t)(k0 + kk) * N + n0 + nn] : 0.f;
             }
             __syncthreads();
-            const int ksteps = (kw + 1) & ~1;
-            const int arow = wave * 32 + (lane & 31), kq = lane >> 5, bcol = lane & 31;
-            if (nw > 32) {
-                for (int kk = 0; kk < ksteps; kk += 2) {
-                    const float a = xs[arow][kk + kq];
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, ws[kk + kq][bcol], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, ws[kk + kq][32 + bcol], acc1, 0, 0, 0);
+            // one bit-width entry per column: column maxima straight from the staged tile
+            // (rows past the end were staged as zero, which never raises a maximum)
+            if (track && P == 1 && tid < kw) {
+                uint32_t mx = 0;
+#pragma unroll 8
+                for (int r = 0; r < FWD_BM; ++r) {
+                    const uint32_t a = abs_bits(xs[r][tid]);
+                    mx = a > mx ? a : mx;
                 }
-            } else {
+                uint32_t *dst = amax_lds ? &amax_s[k0 + tid] : &my_amax[k0 + tid];
+                if (mx > *dst) *dst = mx;
+            }
+            if (cb * 32 < nw) {
+                const int ksteps = (kw + 1) & ~1;
+                const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
                 for (int kk = 0; kk < ksteps; kk += 2)
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[arow][kk + kq], ws[kk + kq][bcol], acc0, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[arow][kk + kq], ws[kk + kq][bcol], acc, 0, 0, 0);
             }
             __syncthreads();
         }
         // ---- epilogue: bias, activation, store
-        const int col = lane & 31;
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            const int n = n0 + blk * 32 + col;
-            if (blk * 32 >= nw || n >= N) continue;
+        const int n = n0 + cb * 32 + (lane & 31);
+        if (cb * 32 < nw && n < N) {
             const float bias = qb ? qb[n] : 0.f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int64_t gr = r0 + wave * 32 + acc_row(r, lane);
+                const int64_t gr = r0 + rh * 32 + acc_row(r, lane);
                 if (gr < rows) {
-                    float v = (blk == 0 ? acc0[r] : acc1[r]) + bias;
+                    float v = acc[r] + bias;
                     if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
                     y[gr * N + n] = v;
                 }
@@ -145,10 +150,7 @@ __global__ __launch_bounds__(256) void qdense_fwd_kernel(const float *__restrict
     }
     if (track && amax_lds) {
         __syncthreads();
-        for (int64_t t = tid; t < PK; t += 256) {
-            const uint32_t v = amax_s[t];
-            if (v) atomicMax(&amax[t], v);
-        }
+        for (int64_t t = tid; t < PK; t += 256) my_amax[t] = amax_s[t];
     }
 }
 
@@ -159,12 +161,16 @@ __global__ __launch_bounds__(256) void qdense_fwd_kernel(const float *__restrict
 #define BWD_LD 65
 #define DF_LDS_MAX 4096
 
+// Workgroup `g` accumulates its share of the kernel / bias / fractional-bit gradients over the
+// tiles it walks and writes them to slice `g` of `part` ([gridDim.x, K*N + N + P*K]); a second
+// small kernel sums the slices in a fixed order, so the result is deterministic and no floating
+// point atomics are used.
 template <int RM, bool QUANT>
 __global__ __launch_bounds__(256) void qdense_bwd_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                          const float *__restrict__ x, const float *__restrict__ f_in,
                                                          int64_t P, const float *__restrict__ qw, float *__restrict__ dx,
-                                                         float *dqw, float *dqb, float *df_in, int64_t rows, int K, int N,
-                                                         int act, int mode, int df_lds) {
+                                                         float *part, int has_bias, int64_t rows, int K, int N, int act,
+                                                         int mode, int df_lds) {
     __shared__ float xs[BWD_BM][BWD_LD];   // quantized input tile
     __shared__ float dzs[BWD_BM][BWD_LD];  // gradient at the pre-activation
     __shared__ float ws[64][BWD_LD];       // quantized kernel, zero padded to 64 x 64
@@ -174,16 +180,22 @@ __global__ __launch_bounds__(256) void qdense_bwd_kernel(const float *__restrict
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5;
-    const int64_t PK = P * (int64_t)K;
+    const int64_t PK = QUANT ? P * (int64_t)K : 0;
+    const int64_t M = (int64_t)K * N + N + PK;
     const int64_t n_tiles = (rows + BWD_BM - 1) / BWD_BM;
-    const bool want_df = QUANT && df_in != nullptr;
+    float *my_dw = part + (int64_t)blockIdx.x * M;
+    float *my_db = my_dw + (int64_t)K * N;
+    float *my_df = my_db + N;
 
     for (int id = tid; id < 64 * 64; id += 256) {
         const int kk = id >> 6, nn = id & 63;
         ws[kk][nn] = (kk < K && nn < N) ? qw[(int64_t)kk * N + nn] : 0.f;
     }
-    if (want_df && df_lds)
-        for (int64_t t = tid; t < PK; t += 256) df_s[t] = 0.f;
+    if (QUANT) {
+        if (df_lds) for (int64_t t = tid; t < PK; t += 256) df_s[t] = 0.f;
+        else for (int64_t t = tid; t < PK; t += 256) my_df[t] = 0.f;
+        __threadfence_block();
+    }
 
     // kernel-gradient block owned by this wave
     const int nblk = K32 * N32;        // 1, 2 or 4 blocks of 32 x 32
@@ -233,68 +245,105 @@ __global__ __launch_bounds__(256) void qdense_bwd_kernel(const float *__restrict
                     const int64_t gr = r0 + row;
                     if (gr < rows && kcol < K) {
                         dx[gr * K + kcol] = acc[r];
-                        if (want_df) {
+                        if (QUANT) {
                             const float delta = xs[row][kcol] - x[gr * K + kcol];
                             const float g = -HGQ_LN2 * delta * acc[r];
                             if (P == 1) dfsum += g;
-                            else if (df_lds) atomicAdd(&df_s[(gr % P) * K + kcol], g);
-                            else atomicAdd(&df_in[(gr % P) * K + kcol], g);
+                            else atomicAdd(df_lds ? &df_s[(gr % P) * K + kcol] : &my_df[(gr % P) * K + kcol], g);
                         }
                     }
                 }
-                if (want_df && P == 1) {
+                if (QUANT && P == 1) {
                     dfsum += __shfl_xor(dfsum, 32, 64);
-                    if (lane < 32 && kcol < K) {
-                        if (df_lds) atomicAdd(&df_s[kcol], dfsum);
-                        else atomicAdd(&df_in[kcol], dfsum);
-                    }
+                    if (lane < 32 && kcol < K) atomicAdd(df_lds ? &df_s[kcol] : &my_df[kcol], dfsum);
                 }
             }
         }
         // ---- dW += rx^T @ dz : this wave's block, its slice of the tile's rows
-        if (dqw) {
+        {
             const int rbeg = sub * rows_per;
             const int kq = lane >> 5, c32 = lane & 31;
             for (int rr = rbeg; rr < rbeg + rows_per; rr += 2)
                 accw = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[rr + kq][wkb * 32 + c32], dzs[rr + kq][wnb * 32 + c32], accw, 0, 0, 0);
         }
         // ---- bias gradient partial sums
-        if (dqb) {
+        if (has_bias) {
 #pragma unroll
             for (int j = 0; j < BWD_BM / 4; ++j) accb += dzs[bq * (BWD_BM / 4) + j][bn];
         }
     }
-    // ---- flush
-    if (dqw) {
-        const int n = wnb * 32 + (lane & 31);
+    // ---- write this workgroup's slice.  Waves sharing a kernel-gradient block combine through LDS.
+    __syncthreads();
+    float *comb = &xs[0][0];  // 64 x 65 floats, free now
+    for (int pass = 0; pass < wpb; ++pass) {
+        if (sub == pass) {
+            const int n = wnb * 32 + (lane & 31);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int k = wkb * 32 + acc_row(r, lane);
-            if (k < K && n < N) atomicAdd(&dqw[(int64_t)k * N + n], accw[r]);
+            for (int r = 0; r < 16; ++r) {
+                const int k = wkb * 32 + acc_row(r, lane);
+                if (pass == 0) comb[k * BWD_LD + n] = accw[r];
+                else comb[k * BWD_LD + n] += accw[r];
+            }
         }
-    }
-    if (dqb) {
-        bred[tid] = accb;
         __syncthreads();
-        if (tid < 64 && tid < N) atomicAdd(&dqb[tid], bred[tid] + bred[tid + 64] + bred[tid + 128] + bred[tid + 192]);
     }
-    if (want_df && df_lds) {
-        __syncthreads();
-        for (int64_t t = tid; t < PK; t += 256) {
-            const float v = df_s[t];
-            if (v != 0.f) atomicAdd(&df_in[t], v);
+    for (int id = tid; id < K * N; id += 256) my_dw[id] = comb[(id / N) * BWD_LD + (id % N)];
+    bred[tid] = accb;
+    __syncthreads();
+    if (tid < N) my_db[tid] = has_bias ? bred[tid] + bred[tid + 64] + bred[tid + 128] + bred[tid + 192] : 0.f;
+    if (QUANT && df_lds)
+        for (int64_t t = tid; t < PK; t += 256) my_df[t] = df_s[t];
+}
+
+// out[e] = sum over slices of part[g][e], in slice order.  256 threads = 64 elements x 4 slice groups.
+__global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restrict__ part, int n_parts, int64_t M,
+                                                           float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb,
+                                                           float *df, int64_t n_df) {
+    __shared__ float red[256];
+    const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
+    float s = 0.f;
+    if (e < M) {
+        const int per = (n_parts + 3) / 4;
+        const int g0 = grp * per, g1 = min(n_parts, g0 + per);
+        for (int g = g0; g < g1; ++g) s += part[(int64_t)g * M + e];
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    if (grp == 0 && e < M) {
+        const float v = (red[e_local] + red[e_local + 64]) + (red[e_local + 128] + red[e_local + 192]);
+        if (e < n_dqw) {
+            if (dqw) dqw[e] = v;
+        } else if (e < n_dqw + n_dqb) {
+            if (dqb) dqb[e - n_dqw] = v;
+        } else if (df) {
+            df[e - n_dqw - n_dqb] = v;
         }
     }
 }
 
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+static inline int row_parts(int64_t rows, int bm) {
+    const int64_t n_tiles = (rows + bm - 1) / bm;
+    int g = persistent_grid(n_tiles, 2);
+    if (g > MAX_PARTS) g = MAX_PARTS;
+    return g;
+}
+
 }  // namespace hgq
 
 using namespace hgq;
 
+extern "C" int hgq_qdense_fwd_parts(int64_t rows) { return rows > 0 ? row_parts(rows, FWD_BM) : 1; }
+
+extern "C" int64_t hgq_qdense_bwd_workspace(int64_t rows, int K, int N, int64_t bw_rows) {
+    const int64_t M = (int64_t)K * N + N + bw_rows * (int64_t)K;
+    return (rows > 0 ? row_parts(rows, BWD_BM) : 1) * M;
+}
+
 extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_in, const float *f_in, int64_t bw_rows,
-                              const float *qw, const float *qb, float *y, uint32_t *amax, int64_t rows, int K, int N,
+                              const float *qw, const float *qb, float *y, uint32_t *amax_part, int64_t rows, int K, int N,
                               int act, int mode, void *stream) {
     hipStream_t s = (hipStream_t)stream;
     if (rows < 0 || K < 1 || N < 1 || bw_rows < 0) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd: bad sizes");
@@ -306,32 +355,29 @@ extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_i
     const Mode m(mode);
     const int64_t PK = bw_rows * (int64_t)K;
     const bool quant = bw_rows > 0;
-    int rc;
-    if (quant && amax && (rc = fill_u32(amax, 0, PK, s))) return rc;
-    const int amax_lds = (quant && amax && PK <= AMAX_LDS_MAX) ? 1 : 0;
+    const int amax_lds = (quant && amax_part && PK <= AMAX_LDS_MAX) ? 1 : 0;
     const size_t dyn = amax_lds ? (size_t)PK * 4 : 0;
     const int vec_ok = (K % 4 == 0) && aligned16(x);
-    const int64_t n_tiles = (rows + FWD_BM - 1) / FWD_BM;
-    const dim3 grid((unsigned)persistent_grid(n_tiles, 4), (unsigned)((N + FWD_BN - 1) / FWD_BN));
+    const dim3 grid((unsigned)row_parts(rows, FWD_BM), (unsigned)((N + FWD_BN - 1) / FWD_BN));
     if (!quant) {
         hipLaunchKernelGGL((qdense_fwd_kernel<HGQ_TRN, HGQ_WRAP, false>), grid, dim3(256), dyn, s, x, k_in, i_in, f_in, (int64_t)1, qw, qb, y,
-                           amax, rows, K, N, act, mode, vec_ok, amax_lds);
+                           (uint32_t *)nullptr, rows, K, N, act, mode, vec_ok, amax_lds);
     } else {
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
-            hipLaunchKernelGGL((qdense_fwd_kernel<RM, OM, true>), grid, dim3(256), dyn, s, x, k_in, i_in, f_in, bw_rows, qw, qb, y, amax, rows,
-                               K, N, act, mode, vec_ok, amax_lds);
+            hipLaunchKernelGGL((qdense_fwd_kernel<RM, OM, true>), grid, dim3(256), dyn, s, x, k_in, i_in, f_in, bw_rows, qw, qb, y, amax_part,
+                               rows, K, N, act, mode, vec_ok, amax_lds);
         });
     }
     return check_launch("hgq_qdense_fwd");
 }
 
 extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
-                              const float *qw, float *dx, float *dqw, float *dqb, float *df_in, int64_t rows, int K,
-                              int N, int act, int mode, void *stream) {
+                              const float *qw, float *dx, float *dqw, float *dqb, float *df_in, float *workspace,
+                              int64_t rows, int K, int N, int act, int mode, void *stream) {
     hipStream_t s = (hipStream_t)stream;
     if (rows < 0 || K < 1 || N < 1 || bw_rows < 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: bad sizes");
     if (K > 64 || N > 64) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_bwd: K=%d N=%d exceed the fused kernel's 64 x 64", K, N);
-    if (!dy || !x || !qw || !dx) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: null pointer");
+    if (!dy || !x || !qw || !dx || !workspace) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: null pointer");
     if (act == HGQ_ACT_RELU && !y) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: relu needs the forward output");
     if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: unknown activation %d", act);
     const Mode m(mode);
@@ -341,17 +387,20 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
     if (quant && !f_in) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: null bit-width pointer");
     if (quant && rows % bw_rows != 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: rows not a multiple of bw_rows");
     const int64_t PK = bw_rows * (int64_t)K;
-    int rc;
-    if (dqw && (rc = fill_f32(dqw, 0.f, (int64_t)K * N, s))) return rc;
-    if (dqb && (rc = fill_f32(dqb, 0.f, N, s))) return rc;
-    if (quant && df_in && (rc = fill_f32(df_in, 0.f, PK, s))) return rc;
-    if (rows == 0) return HGQ_OK;
-    const int df_lds = (quant && df_in && PK <= DF_LDS_MAX) ? 1 : 0;
+    const int64_t M = (int64_t)K * N + N + PK;
+    if (rows == 0) {
+        int rc;
+        if (dqw && (rc = fill_f32(dqw, 0.f, (int64_t)K * N, s))) return rc;
+        if (dqb && (rc = fill_f32(dqb, 0.f, N, s))) return rc;
+        if (df_in && (rc = fill_f32(df_in, 0.f, PK, s))) return rc;
+        return HGQ_OK;
+    }
+    const int df_lds = (quant && PK <= DF_LDS_MAX) ? 1 : 0;
     const size_t dyn = df_lds ? (size_t)PK * 4 : 0;
-    const int64_t n_tiles = (rows + BWD_BM - 1) / BWD_BM;
-    const dim3 grid((unsigned)persistent_grid(n_tiles, 3));
-    typedef void (*bwd_fn)(const float *, const float *, const float *, const float *, int64_t, const float *, float *, float *,
-                           float *, float *, int64_t, int, int, int, int, int);
+    const int parts = row_parts(rows, BWD_BM);
+    const dim3 grid((unsigned)parts);
+    typedef void (*bwd_fn)(const float *, const float *, const float *, const float *, int64_t, const float *, float *, float *, int,
+                           int64_t, int, int, int, int, int);
     bwd_fn fn = nullptr;
     if (!quant) fn = qdense_bwd_kernel<HGQ_TRN, false>;
     else if (m.round_mode == HGQ_TRN) fn = qdense_bwd_kernel<HGQ_TRN, true>;
@@ -373,7 +422,11 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
             if (slot >= 0) raised[slot] = (const void *)fn;
         }
     }
-    hipLaunchKernelGGL(fn, grid, dim3(256), dyn, s, dy, y, x, f_in, quant ? bw_rows : (int64_t)1, qw, dx, dqw, dqb, df_in, rows, K, N, act,
-                       mode, df_lds);
-    return check_launch("hgq_qdense_bwd");
+    hipLaunchKernelGGL(fn, grid, dim3(256), dyn, s, dy, y, x, f_in, quant ? bw_rows : (int64_t)1, qw, dx, workspace, dqb ? 1 : 0, rows, K, N,
+                       act, mode, df_lds);
+    int rc = check_launch("hgq_qdense_bwd");
+    if (rc) return rc;
+    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(256), 0, s, workspace, parts, M, dqw, (int64_t)K * N, dqb,
+                       (int64_t)N, quant ? df_in : (float *)nullptr, PK);
+    return check_launch("hgq_qdense_bwd(reduce)");
 }

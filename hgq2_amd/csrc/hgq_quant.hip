@@ -367,14 +367,35 @@ __device__ __forceinline__ float ceil_log2(float v) {
     return (float)(mant == 0.5f ? e - 1 : e);
 }
 
+// 256 threads = 64 entries x 4 slice groups: the abs-max / any-negative trackers arrive as
+// `n_parts` slices of [n] (one per producing workgroup) and are combined here.
 __global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__restrict__ amax,
-                                                           const uint32_t *__restrict__ anyneg, float *i_var,
-                                                           const float *__restrict__ fb, uint8_t *k_var, int64_t n,
-                                                           float decay, float c_lo, float c_hi, int mode) {
+                                                           const uint32_t *__restrict__ anyneg, int n_parts,
+                                                           float *i_var, const float *__restrict__ fb, uint8_t *k_var,
+                                                           int64_t n, float decay, float c_lo, float c_hi, int mode) {
+    __shared__ uint32_t smax[256], sneg[256];
     const Mode m(mode);
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= n) return;
-    const float xr = __uint_as_float(amax[t]);
+    const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int64_t t = (int64_t)blockIdx.x * 64 + e_local;
+    uint32_t mx = 0, ng = 0;
+    if (t < n) {
+        const int per = (n_parts + 3) / 4;
+        const int g0 = grp * per, g1 = min(n_parts, g0 + per);
+        for (int g = g0; g < g1; ++g) {
+            const uint32_t a = amax[(int64_t)g * n + t];
+            mx = a > mx ? a : mx;
+            if (anyneg) ng |= anyneg[(int64_t)g * n + t];
+        }
+    }
+    smax[threadIdx.x] = mx, sneg[threadIdx.x] = ng;
+    __syncthreads();
+    if (grp != 0 || t >= n) return;
+    for (int w = 1; w < 4; ++w) {
+        const uint32_t a = smax[e_local + 64 * w];
+        mx = a > mx ? a : mx;
+        ng |= sneg[e_local + 64 * w];
+    }
+    const float xr = __uint_as_float(mx);
     const float raw_i = i_var[t];
     float mi;
     if (!m.kbi) {
@@ -399,7 +420,7 @@ __global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__res
         } else {
             ni = fminf(fmaxf(fmaxf(rintf(raw_i), mi), c_lo), c_hi);
         }
-        if (k_var && anyneg && anyneg[t]) k_var[t] = 1;
+        if (k_var && anyneg && ng) k_var[t] = 1;
     }
     i_var[t] = ni;
 }
@@ -563,12 +584,12 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
     return check_launch("hgq_quantize_bwd");
 }
 
-extern "C" int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, float *i_var, const float *fb,
+extern "C" int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, int n_parts, float *i_var, const float *fb,
                                 uint8_t *k_var, int64_t m, float decay, float c_lo, float c_hi, int mode, void *stream) {
-    if (m < 0) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i: bad size");
+    if (m < 0 || n_parts < 1) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i: bad size");
     if (m == 0) return HGQ_OK;
     if (!amax || !i_var || !fb) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i: null pointer");
-    hipLaunchKernelGGL(wrap_track_i_kernel, dim3((unsigned)((m + 255) / 256)), dim3(256), 0, (hipStream_t)stream, amax, anyneg, i_var, fb,
-                       k_var, m, decay, c_lo, c_hi, mode);
+    hipLaunchKernelGGL(wrap_track_i_kernel, dim3((unsigned)((m + 63) / 64)), dim3(256), 0, (hipStream_t)stream, amax, anyneg, n_parts,
+                       i_var, fb, k_var, m, decay, c_lo, c_hi, mode);
     return check_launch("hgq_wrap_track_i");
 }

@@ -36,7 +36,18 @@ __device__ __forceinline__ float entry_bits(const void *k, const float *i, const
 
 #define HGQ_EBOPS_MAXK 4096
 
-__global__ __launch_bounds__(256) void dense_ebops_kernel(const void *k_in, const float *i_in, const float *f_in,
+// ceil(log2(v)) for v > 0 from the exponent field (exact).
+__device__ __forceinline__ float ceil_log2_exact(float v) {
+    if (!(v > 0.0f)) return v == 0.0f ? -INFINITY : NAN;
+    if (!(v < INFINITY)) return v;
+    int e;
+    const float mant = frexpf(v, &e);
+    return (float)(mant == 0.5f ? e - 1 : e);
+}
+
+__global__ __launch_bounds__(256) void dense_ebops_kernel(const uint32_t *amax_part, int n_parts, float decay,
+                                                          const float *beta, float *loss_term,
+                                                          const void *k_in, float *i_in, const float *f_in,
                                                           int64_t P, int K, int N, const void *k_ker,
                                                           const float *b_ker, const void *k_bias, const float *b_bias,
                                                           float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
@@ -47,6 +58,23 @@ __global__ __launch_bounds__(256) void dense_ebops_kernel(const void *k_in, cons
     __shared__ float red[4];
     const Mode mi(mode_in), mk(mode_ker), mb(mode_bias);
     const int t = threadIdx.x;
+    // with beta the gradients are those of the loss term ebops * beta
+    const float gscale = beta ? scale * beta[0] : scale;
+    if (amax_part) {
+        // integer-bit tracking of the (KIF, WRAP, training) input quantizer, before its bits are read:
+        // _i <- max(_i - decay, ceil(log2(max|x_q| + 2**-f)))
+        for (int64_t e = t; e < P * K; e += 256) {
+            uint32_t mx = 0;
+            for (int g = 0; g < n_parts; ++g) {
+                const uint32_t a = amax_part[(int64_t)g * P * K + e];
+                mx = a > mx ? a : mx;
+            }
+            const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-rintf(f_in[e]))));
+            i_in[e] = fmaxf(__fsub_rn(i_in[e], decay), mi_);
+        }
+        __threadfence_block();
+        __syncthreads();
+    }
     for (int k = t; k < K; k += 256) {
         float s = 0.0f, d;
         for (int n = 0; n < N; ++n) s += entry_bits(k_ker, nullptr, b_ker, (int64_t)k * N + n, mk, d);
@@ -55,7 +83,7 @@ __global__ __launch_bounds__(256) void dense_ebops_kernel(const void *k_in, cons
         for (int64_t p = 0; p < P; ++p) {
             const float b = entry_bits(k_in, i_in, f_in, p * K + k, mi, d);
             a += b;
-            if (g_f_in) g_f_in[p * K + k] = d * s * scale;
+            if (g_f_in) g_f_in[p * K + k] = d * s * gscale;
         }
         insum[k] = a;
     }
@@ -64,12 +92,12 @@ __global__ __launch_bounds__(256) void dense_ebops_kernel(const void *k_in, cons
     for (int k = t; k < K; k += 256) part += insum[k] * colsum[k];
     float total = block_sum_256(part, red);
     if (g_b_ker)
-        for (int64_t e = t; e < (int64_t)K * N; e += 256) g_b_ker[e] = insum[e / N] * scale;
+        for (int64_t e = t; e < (int64_t)K * N; e += 256) g_b_ker[e] = insum[e / N] * gscale;
     if (b_bias) {
         float bs = 0.0f, d;
         for (int n = t; n < N; n += 256) {
             bs += entry_bits(k_bias, nullptr, b_bias, n, mb, d);
-            if (g_b_bias) g_b_bias[n] = bias_size / (float)N * scale;
+            if (g_b_bias) g_b_bias[n] = bias_size / (float)N * gscale;
         }
         bs = block_sum_256(bs, red);
         total += bs / (float)N * bias_size;
@@ -78,6 +106,7 @@ __global__ __launch_bounds__(256) void dense_ebops_kernel(const void *k_in, cons
         const float e = total * scale;
         ebops[0] = e;
         if (ebops_u32) ebops_u32[0] = (uint32_t)e;
+        if (loss_term && beta) loss_term[0] = e * beta[0];
     }
 }
 
@@ -115,11 +144,47 @@ __global__ __launch_bounds__(256) void sgd_kernel(float *__restrict__ w, const f
     }
 }
 
+struct SgdBatch {
+    hgq_sgd_item item[HGQ_SGD_BATCH];
+};
+
+// grid.y = variable, grid.x strides over its elements; the descriptors travel as a kernel argument
+__global__ __launch_bounds__(256) void sgd_multi_kernel(SgdBatch b, float lr) {
+    const hgq_sgd_item it = b.item[blockIdx.y];
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < it.n; t += (int64_t)gridDim.x * 256) {
+        const float v = __fsub_rn(it.w[t], __fmul_rn(lr, __fadd_rn(it.g[t], it.l1)));
+        it.w[t] = fminf(fmaxf(v, it.lo), it.hi);
+    }
+}
+
 }  // namespace hgq
 
 using namespace hgq;
 
-extern "C" int hgq_dense_ebops(const void *k_in, const float *i_in, const float *f_in, int64_t P, int K, int N,
+extern "C" int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *stream) {
+    if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_sgd_update_multi: bad arguments");
+    for (int base = 0; base < count; base += HGQ_SGD_BATCH) {
+        SgdBatch b;
+        const int nb = count - base < HGQ_SGD_BATCH ? count - base : HGQ_SGD_BATCH;
+        int64_t max_n = 0;
+        for (int t = 0; t < nb; ++t) {
+            b.item[t] = items[base + t];
+            if (b.item[t].n < 0 || (b.item[t].n > 0 && (!b.item[t].w || !b.item[t].g)))
+                return fail(HGQ_ERR_ARG, "hgq_sgd_update_multi: bad item %d", base + t);
+            if (b.item[t].n > max_n) max_n = b.item[t].n;
+        }
+        if (max_n == 0) continue;
+        int64_t gx = (max_n + 1023) / 1024;
+        if (gx > 512) gx = 512;
+        hipLaunchKernelGGL(sgd_multi_kernel, dim3((unsigned)gx, (unsigned)nb), dim3(256), 0, (hipStream_t)stream, b, lr);
+        int rc = check_launch("hgq_sgd_update_multi");
+        if (rc) return rc;
+    }
+    return HGQ_OK;
+}
+
+extern "C" int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const float *beta, float *loss_term,
+                               const void *k_in, float *i_in, const float *f_in, int64_t P, int K, int N,
                                const void *k_ker, const float *b_ker, const void *k_bias, const float *b_bias,
                                float scale, float bias_size, int mode_in, int mode_ker, int mode_bias, float *ebops,
                                uint32_t *ebops_u32, float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream) {
@@ -127,7 +192,10 @@ extern "C" int hgq_dense_ebops(const void *k_in, const float *i_in, const float 
     if (!i_in || !f_in || !b_ker || !ebops || !k_in || !k_ker) return fail(HGQ_ERR_ARG, "hgq_dense_ebops: null pointer");
     if (K > HGQ_EBOPS_MAXK) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops: K=%d > %d", K, HGQ_EBOPS_MAXK);
     if (!(Mode(mode_ker).kbi) || (b_bias && !(Mode(mode_bias).kbi))) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops: kernel/bias bit-widths must use the KBI parametrisation");
-    hipLaunchKernelGGL(dense_ebops_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, k_in, i_in, f_in, P, K, N, k_ker, b_ker,
+    if (amax_part && (n_parts < 1 || Mode(mode_in).kbi || Mode(mode_in).overflow_mode != HGQ_WRAP))
+        return fail(HGQ_ERR_ARG, "hgq_dense_ebops: fused tracking is for KIF WRAP input quantizers");
+    hipLaunchKernelGGL(dense_ebops_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, amax_part, n_parts, decay, beta, loss_term, k_in,
+                       i_in, f_in, P, K, N, k_ker, b_ker,
                        k_bias, b_bias, scale, bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
     return check_launch("hgq_dense_ebops");
 }

@@ -57,8 +57,23 @@ def _covers_trailing(bw_shape, K):
     return False
 
 
+class DeferredTracking:
+    """Abs-max slices of a fused input quantizer whose integer-bit update has not run yet."""
+
+    def __init__(self, quantizer, amax):
+        self.quantizer, self.amax = quantizer, amax
+
+    def flush(self):
+        if self.amax is not None:
+            self.quantizer._track(self.amax, True)
+            self.amax = None
+
+
+FUSED_TRACK_MAX = 65536  # slices * entries the single-workgroup EBOPs kernel is allowed to walk
+
+
 def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training):
-    """x [..., K] -> [..., N].  Returns the 2-D result [rows, N]."""
+    """x [..., K] -> [rows, N].  Returns ``(y, activation applied, DeferredTracking or None)``."""
     K, N = qkernel2d.shape
     x2d = x.reshape(-1, K)
     if not x2d.is_contiguous():
@@ -70,25 +85,25 @@ def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training):
         q = iq.quantizer
         y, amax = ops.qdense(x2d, q._k.view(-1), q._i.view(-1), q._f.view(-1), qkernel2d, qbias1d, act_code,
                              q._mode(True), bw_rows, True)
-        q._track(amax, True)
-        return y, act_code != _lib.ACT_NONE
+        return y, act_code != _lib.ACT_NONE, DeferredTracking(q, amax)
     if iq is not None:
         x2d = iq(x, training=training).reshape(-1, K)
         if not x2d.is_contiguous():
             x2d = x2d.contiguous()
     if fused_bwd:
         y, _ = ops.qdense(x2d, None, None, None, qkernel2d, qbias1d, act_code, 0, 0, False)
-        return y, act_code != _lib.ACT_NONE
+        return y, act_code != _lib.ACT_NONE, None
     # shapes beyond the fused backward kernel: plain library GEMM on the quantized operands
     y = x2d @ qkernel2d
     if qbias1d is not None:
         y = y + qbias1d
-    return y, False
+    return y, False, None
 
 
-def dense_ebops_fast(iq, kq, bq, K, N, scale, bias_size):
-    """EBOPs through the fused kernel when the quantizers are the fixed-point kinds it covers.
-    Returns ``(ebops, uint32 bit pattern)`` or ``None`` when the generic path must be used."""
+def dense_ebops_term(layer, iq, kq, bq, K, N, scale, bias_size, deferred):
+    """``ebops * beta`` through the fused kernel (which also assigns the layer's ``_ebops`` and, when
+    ``deferred`` tracking is pending and small enough, updates the input quantizer's ``_i`` first).
+    Returns ``None`` when the quantizers are not the fixed-point kinds the kernel covers."""
     qi, qk = iq.quantizer, kq.quantizer
     if not isinstance(qi, (FixedPointQuantizerKIF, FixedPointQuantizerKBI)) or not isinstance(qk, FixedPointQuantizerKBI):
         return None
@@ -100,7 +115,16 @@ def dense_ebops_fast(iq, kq, bq, K, N, scale, bias_size):
     if qb is not None and qb._b.numel() != N:
         return None
     P = qi._i.numel() // K
-    return ops.dense_ebops(
+    amax = None
+    if deferred is not None and deferred.amax is not None:
+        if deferred.quantizer is qi and deferred.amax.numel() <= FUSED_TRACK_MAX:
+            amax, deferred.amax = deferred.amax, None
+        else:
+            deferred.flush()
+    decay = qi._decay_host if amax is not None else 0.0
+    _, term = ops.dense_ebops(
         qi._k.view(-1), qi._i.view(-1), qi._third().view(-1), qk._k.view(-1), qk._b.view(-1),
-        qb._k.view(-1) if qb is not None else None, qb._b.view(-1) if qb is not None else None, P, K, N, scale,
-        bias_size, qi._mode(True), qk._mode(True), qb._mode(True) if qb is not None else 0)
+        qb._k.view(-1) if qb is not None else None, qb._b.view(-1) if qb is not None else None, P, K, N,
+        scale * layer.ebops_factor, bias_size, qi._mode(True), qk._mode(True), qb._mode(True) if qb is not None else 0,
+        amax=amax, decay=decay, beta=layer._beta, ebops_var=layer._ebops.view(torch.int32))
+    return term

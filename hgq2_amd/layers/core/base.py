@@ -90,33 +90,30 @@ class QLayerBase(Layer):
         self.oq.build(tuple(output_shape))
         self.oq.built = True
 
-    def _set_ebops(self, ebops, ebops_bits=None):
-        """``_ebops.assign(cast(ebops, uint32))`` and ``add_loss(ebops * beta)`` (reference :103-104)."""
+    def _ebops_loss_term(self, *shapes):
+        """``ebops = _compute_ebops(...) * ebops_factor; _ebops.assign(cast(ebops, uint32))``; returns
+        the loss term ``ebops * beta`` (reference :101-104).  Layers with a fused kernel override this."""
+        ebops = self._compute_ebops(*shapes) * self.ebops_factor
         with torch.no_grad():
-            if ebops_bits is None:
-                ebops_bits = ebops.detach().to(torch.int64).to(torch.int32)
-            self._ebops.view(torch.int32).copy_(ebops_bits)
-        self.add_loss(ebops * self._beta)
+            self._ebops.view(torch.int32).copy_(ebops.detach().to(torch.int64).to(torch.int32))
+        return ebops * self._beta
 
     def _wrapped_call(self, *args, training=None, **kwargs):
         r = self.call(*args, training=training, **kwargs)
         if (training or training == 'tracing') and self.enable_ebops:
             tensors = args[0] if isinstance(args[0], (tuple, list)) else [a for a in args if isinstance(a, torch.Tensor)]
             shapes = [(1,) + tuple(t.shape[1:]) for t in tensors]
-            out = self._compute_ebops(*shapes)
-            if isinstance(out, tuple):
-                ebops, bits = out
-            else:
-                ebops, bits = out, None
-            if self.ebops_factor != 1.0:
-                ebops, bits = ebops * self.ebops_factor, None
-            self._set_ebops(ebops, bits)
+            self.add_loss(self._ebops_loss_term(*shapes))
+        self._finish_call()
         if not self.enable_oq or self.__output_quantizer_handled__:
             return r
         assert not isinstance(r, (tuple, list)), (
             f'Layer {self.name}({type(self)}) returns multiple outputs, which must be handled in subclasses.'
         )
         return self.oq(r, training=training)
+
+    def _finish_call(self):
+        """Hook: state updates a layer deferred so they could be fused with the EBOPs kernel."""
 
     def get_config(self):
         return {

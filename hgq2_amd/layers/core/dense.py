@@ -9,7 +9,7 @@ import torch
 from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
-from ._contraction import dense_contraction, dense_ebops_fast, get_activation
+from ._contraction import dense_contraction, dense_ebops_term, get_activation
 from .base import QLayerBaseSingleInput
 
 
@@ -70,18 +70,30 @@ class QDense(QLayerBaseSingleInput):
 
     def call(self, inputs, training=None):
         iq = self.iq if self.enable_iq else None
-        y, act_done = dense_contraction(inputs, iq, self.qkernel, self.qbias, self._act_name, training)
+        y, act_done, self._deferred = dense_contraction(inputs, iq, self.qkernel, self.qbias, self._act_name, training)
         y = y.view(*inputs.shape[:-1], self.units)
         if self.activation is not None and not act_done:
             y = self.activation(y)
         return y
 
+    def _finish_call(self):
+        d, self._deferred = getattr(self, '_deferred', None), None
+        if d is not None:
+            d.flush()
+
+    def _ebops_loss_term(self, shape):
+        out_size = float(prod(shape[:-1]) * self.units)
+        scale = self.parallelization_factor / self.n_parallel
+        term = dense_ebops_term(self, self.iq, self.kq, self.bq, shape[-1], self.units, scale, out_size,
+                                getattr(self, '_deferred', None))
+        if term is not None:
+            return term
+        self._finish_call()  # the generic path reads the integer bits: track first
+        return super()._ebops_loss_term(shape)
+
     def _compute_ebops(self, shape):
         out_size = float(prod(shape[:-1]) * self.units)
         scale = self.parallelization_factor / self.n_parallel
-        fast = dense_ebops_fast(self.iq, self.kq, self.bq, shape[-1], self.units, scale, out_size)
-        if fast is not None:
-            return fast
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self._kernel.shape).to(bw_inp.device)
         ebops = torch.sum(torch.matmul(bw_inp, bw_ker))

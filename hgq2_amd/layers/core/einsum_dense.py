@@ -16,7 +16,7 @@ import torch
 from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
-from ._contraction import dense_contraction, dense_ebops_fast, get_activation
+from ._contraction import dense_contraction, dense_ebops_term, get_activation
 from .base import QLayerBaseSingleInput
 
 
@@ -149,7 +149,7 @@ class QEinsumDense(QLayerBaseSingleInput):
             x = inputs  # the contracted axes are trailing and contiguous: a [rows, K] view of the same memory
             b1d = qbias.reshape(-1) if (qbias is not None and self._bias_in_gemm) else None
             fuse_act = self._act_name if (qbias is None or self._bias_in_gemm) else None
-            y, act_done = dense_contraction(x, iq, qkernel.reshape(self._K, self._N), b1d, fuse_act, training)
+            y, act_done, self._deferred = dense_contraction(x, iq, qkernel.reshape(self._K, self._N), b1d, fuse_act, training)
             y = y.view(inputs.shape[0], *self.full_output_shape[1:])
             if qbias is not None and not self._bias_in_gemm:
                 y = y + qbias
@@ -169,13 +169,25 @@ class QEinsumDense(QLayerBaseSingleInput):
             y = self.activation(y)
         return y
 
-    def _compute_ebops(self, shape):
+    def _finish_call(self):
+        d, self._deferred = getattr(self, '_deferred', None), None
+        if d is not None:
+            d.flush()
+
+    def _ebops_loss_term(self, shape):
         scale = self.parallelization_factor / self.n_parallel
         out_size = float(prod(self.full_output_shape[1:]))
         if self._gemm is not None and (self.bq is None or self._bias_in_gemm):
-            fast = dense_ebops_fast(self.iq, self.kq, self.bq, self._K, self._N, scale, out_size)
-            if fast is not None:
-                return fast
+            term = dense_ebops_term(self, self.iq, self.kq, self.bq, self._K, self._N, scale, out_size,
+                                    getattr(self, '_deferred', None))
+            if term is not None:
+                return term
+        self._finish_call()
+        return super()._ebops_loss_term(shape)
+
+    def _compute_ebops(self, shape):
+        scale = self.parallelization_factor / self.n_parallel
+        out_size = float(prod(self.full_output_shape[1:]))
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self._kernel.shape)
         ebops = torch.einsum(self.ebops_equation, bw_inp, bw_ker)

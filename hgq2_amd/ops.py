@@ -1,23 +1,23 @@
-"""``torch.library`` operators over the C ABI of ``libhgq_hip.so``.
+"""``torch.library`` operators over the C ABI of ``libhgq_hip.so`` and their autograd wrappers.
 
-Every operator validates its arguments on the host (device, dtype, contiguity, sizes),
-allocates its outputs with torch, and enqueues the HIP kernels on torch's current stream.
-Autograd is attached with ``register_autograd``; the backward formulas call the backward
-entry points of the same library.  There is no CPU implementation: tensors must be on a GPU.
+Layering: ``hgq::*`` custom operators are thin, validated launches of one C-ABI entry point
+(outputs allocated with torch, kernels enqueued on torch's current stream); the
+``torch.autograd.Function`` classes below pair each forward operator with its backward
+operator.  There is no CPU implementation: tensors must live on a GPU and a missing library
+raises.
 """
 
 from __future__ import annotations
 
 import ctypes
+from typing import Sequence
 
 import torch
 from torch import Tensor
 
 from . import _lib
 
-__all__ = [
-    'quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_',
-]
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_']
 
 
 def _ptr(t: Tensor | None):
@@ -49,9 +49,9 @@ def _kmode(mode: int, k: Tensor) -> int:
     return (mode | _lib.MODE_K_U8) if k.dtype == torch.uint8 else (mode & ~_lib.MODE_K_U8)
 
 
-# --------------------------------------------------------------------------------------
-# quantizer
-# --------------------------------------------------------------------------------------
+# ======================================================================================
+# raw operators (one C-ABI call each)
+# ======================================================================================
 @torch.library.custom_op('hgq::quantize_fwd', mutates_args=())
 def quantize_fwd(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, track: bool) -> tuple[Tensor, Tensor, Tensor]:
     _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
@@ -93,52 +93,22 @@ def _(dy, x, k, i, fb, mode, bw_inner):
     return torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
 
 
-def _quantize_setup(ctx, inputs, output):
-    x, k, i, fb, mode, bw_inner, track = inputs
-    ctx.save_for_backward(x, k, i, fb)
-    ctx.mode, ctx.bw_inner = mode, bw_inner
-
-
-def _quantize_backward(ctx, gy, g_amax, g_neg):
-    x, k, i, fb = ctx.saved_tensors
-    if not (ctx.mode & _lib.MODE_TRAINING):
-        raise RuntimeError('hgq::quantize_fwd: gradients are defined for the training-mode forward only')
-    dx, di, dfb = quantize_bwd(gy.contiguous(), x, k, i, fb, ctx.mode, ctx.bw_inner)
-    return dx, None, di, dfb, None, None, None
-
-
-quantize_fwd.register_autograd(_quantize_backward, setup_context=_quantize_setup)
-
-
-def quantize(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int = 1, track: bool = False):
-    """Fixed-point quantizer.  Returns ``(y, amax_bits, anyneg)``; the last two are empty unless ``track``."""
-    return quantize_fwd(x.contiguous(), k.contiguous(), i.contiguous(), fb.contiguous(), mode, bw_inner, track)
-
-
 @torch.library.custom_op('hgq::wrap_track_i', mutates_args=('i_var', 'k_var'))
-def wrap_track_i_op(amax: Tensor, anyneg: Tensor, i_var: Tensor, fb: Tensor, k_var: Tensor, decay: float, c_lo: float,
-                    c_hi: float, mode: int) -> None:
+def wrap_track_i_op(amax: Tensor, anyneg: Tensor, n_parts: int, i_var: Tensor, fb: Tensor, k_var: Tensor, decay: float,
+                    c_lo: float, c_hi: float, mode: int) -> None:
     _check_f32('i_var', i_var), _check_f32('fb', fb)
     m = i_var.numel()
-    _need(amax.numel() == m and amax.dtype == torch.int32 and amax.is_cuda, 'amax must be an int32 GPU tensor matching i_var')
+    _need(amax.numel() == m * n_parts and amax.dtype == torch.int32 and amax.is_cuda,
+          'amax must be an int32 GPU tensor of n_parts slices matching i_var')
     _need(fb.numel() == m, 'fb must match i_var')
     if k_var.numel():
-        _need(k_var.dtype == torch.uint8 and k_var.numel() == m and anyneg.numel() == m, 'k_var must be uint8 matching i_var')
-    rc = _lib.load().hgq_wrap_track_i(_ptr(amax), _ptr(anyneg), _ptr(i_var), _ptr(fb), _ptr(k_var), m, decay, c_lo, c_hi,
-                                      mode, _stream())
+        _need(k_var.dtype == torch.uint8 and k_var.numel() == m and anyneg.numel() == m * n_parts,
+              'k_var must be uint8 matching i_var')
+    rc = _lib.load().hgq_wrap_track_i(_ptr(amax), _ptr(anyneg), n_parts, _ptr(i_var), _ptr(fb), _ptr(k_var), m, decay,
+                                      c_lo, c_hi, mode, _stream())
     _lib.check(rc, 'hgq_wrap_track_i')
 
 
-def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('inf'), anyneg=None, k_var=None):
-    empty_i = amax.new_empty(0)
-    empty_k = torch.empty(0, dtype=torch.uint8, device=amax.device)
-    wrap_track_i_op(amax, anyneg if anyneg is not None else empty_i, i_var, fb, k_var if k_var is not None else empty_k,
-                    float(decay), float(c_lo), float(c_hi), mode)
-
-
-# --------------------------------------------------------------------------------------
-# dense contraction with the input quantizer fused into the operand load
-# --------------------------------------------------------------------------------------
 @torch.library.custom_op('hgq::qdense_fwd', mutates_args=())
 def qdense_fwd(x: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, qw: Tensor, qb: Tensor, act: int, mode: int,
                bw_rows: int, track: bool) -> tuple[Tensor, Tensor]:
@@ -155,17 +125,21 @@ def qdense_fwd(x: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, qw: Tensor, 
               'input bit-widths must have bw_rows*K elements')
         _need(rows % bw_rows == 0, 'rows must be a multiple of bw_rows')
         mode = _kmode(mode, k_in)
+    lib = _lib.load()
     y = torch.empty((rows, N), dtype=torch.float32, device=x.device)
-    amax = torch.empty(bw_rows * K if (track and bw_rows > 0) else 0, dtype=torch.int32, device=x.device)
-    rc = _lib.load().hgq_qdense_fwd(_ptr(x), _ptr(k_in), _ptr(i_in), _ptr(f_in), bw_rows, _ptr(qw), _ptr(qb), _ptr(y),
-                                    _ptr(amax), rows, K, N, act, mode, _stream())
+    if track and bw_rows > 0:
+        amax = torch.empty((lib.hgq_qdense_fwd_parts(rows), bw_rows * K), dtype=torch.int32, device=x.device)
+    else:
+        amax = torch.empty((0, 0), dtype=torch.int32, device=x.device)
+    rc = lib.hgq_qdense_fwd(_ptr(x), _ptr(k_in), _ptr(i_in), _ptr(f_in), bw_rows, _ptr(qw), _ptr(qb), _ptr(y), _ptr(amax),
+                            rows, K, N, act, mode, _stream())
     _lib.check(rc, 'hgq_qdense_fwd')
     return y, amax
 
 
 @qdense_fwd.register_fake
 def _(x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track):
-    return x.new_empty((x.shape[0], qw.shape[1])), x.new_empty(bw_rows * x.shape[1] if (track and bw_rows > 0) else 0, dtype=torch.int32)
+    return x.new_empty((x.shape[0], qw.shape[1])), x.new_empty((0, 0), dtype=torch.int32)
 
 
 @torch.library.custom_op('hgq::qdense_bwd', mutates_args=())
@@ -175,12 +149,14 @@ def qdense_bwd(dy: Tensor, y: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_b
     rows, K = x.shape
     N = qw.shape[1]
     _need(tuple(dy.shape) == (rows, N), 'dy shape mismatch')
+    lib = _lib.load()
     dx = torch.empty_like(x)
     dqw = torch.empty_like(qw)
     dqb = torch.empty(N if has_bias else 0, dtype=torch.float32, device=x.device)
     df = torch.empty(bw_rows * K, dtype=torch.float32, device=x.device)
-    rc = _lib.load().hgq_qdense_bwd(_ptr(dy), _ptr(y), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(dqw),
-                                    _ptr(dqb), _ptr(df), rows, K, N, act, mode, _stream())
+    ws = torch.empty(lib.hgq_qdense_bwd_workspace(rows, K, N, bw_rows), dtype=torch.float32, device=x.device)
+    rc = lib.hgq_qdense_bwd(_ptr(dy), _ptr(y), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(dqw), _ptr(dqb),
+                            _ptr(df), _ptr(ws), rows, K, N, act, mode, _stream())
     _lib.check(rc, 'hgq_qdense_bwd')
     return dx, dqw, dqb, df
 
@@ -191,41 +167,12 @@ def _(dy, y, x, f_in, qw, has_bias, act, mode, bw_rows):
             x.new_empty(bw_rows * x.shape[1]))
 
 
-def _qdense_setup(ctx, inputs, output):
-    x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track = inputs
-    y, _ = output
-    ctx.save_for_backward(x, f_in, qw, y)
-    ctx.has_bias = qb.numel() > 0
-    ctx.act, ctx.mode, ctx.bw_rows = act, mode, bw_rows
-    ctx.f_shape = f_in.shape
-
-
-def _qdense_backward(ctx, gy, g_amax):
-    x, f_in, qw, y = ctx.saved_tensors
-    dx, dqw, dqb, df = qdense_bwd(gy.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows)
-    return (dx, None, None, df.view(ctx.f_shape) if ctx.bw_rows > 0 else None, dqw, dqb if ctx.has_bias else None,
-            None, None, None, None)
-
-
-qdense_fwd.register_autograd(_qdense_backward, setup_context=_qdense_setup)
-
-FUSED_BWD_MAX = 64  # hgq_qdense_bwd covers K <= 64 and N <= 64
-
-
-def qdense(x2d, k_in, i_in, f_in, qw, qb, act: int, mode: int, bw_rows: int, track: bool):
-    """y = act(q_in(x) @ qw + qb) on a [rows, K] view; returns ``(y, amax_bits)``."""
-    empty = x2d.new_empty(0)
-    return qdense_fwd(x2d, k_in if k_in is not None else empty, i_in if i_in is not None else empty,
-                      f_in if f_in is not None else empty, qw, qb if qb is not None else empty, act, mode, bw_rows, track)
-
-
-# --------------------------------------------------------------------------------------
-# EBOPs of a dense contraction
-# --------------------------------------------------------------------------------------
-@torch.library.custom_op('hgq::dense_ebops', mutates_args=())
-def dense_ebops_op(k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor, b_ker: Tensor, k_bias: Tensor, b_bias: Tensor,
-                   P: int, K: int, N: int, scale: float, bias_size: float, mode_in: int, mode_ker: int,
-                   mode_bias: int) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
+@torch.library.custom_op('hgq::dense_ebops', mutates_args=('i_in', 'ebops_var'))
+def dense_ebops_op(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor,
+                   b_ker: Tensor, k_bias: Tensor, b_bias: Tensor, ebops_var: Tensor, P: int, K: int, N: int, scale: float,
+                   bias_size: float, mode_in: int, mode_ker: int, mode_bias: int) -> tuple[Tensor, Tensor, Tensor]:
+    """Returns (ebops, ebops*beta, [g_f_in | g_b_ker | g_b_bias] in one buffer); with ``beta`` the
+    gradient buffer holds d(ebops*beta)/d variable, else d ebops / d variable."""
     _check_k('k_in', k_in), _check_f32('i_in', i_in), _check_f32('f_in', f_in), _check_k('k_ker', k_ker), _check_f32('b_ker', b_ker)
     _need(i_in.numel() == P * K and f_in.numel() == P * K and k_in.numel() == P * K, 'input bit-width size mismatch')
     _need(b_ker.numel() == K * N and k_ker.numel() == K * N, 'kernel bit-width size mismatch')
@@ -234,53 +181,28 @@ def dense_ebops_op(k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor, b_ke
         _check_f32('b_bias', b_bias), _check_k('k_bias', k_bias)
         _need(b_bias.numel() == N and k_bias.numel() == N, 'bias bit-width size mismatch')
         mode_bias = _kmode(mode_bias, k_bias)
-    ebops = torch.empty((), dtype=torch.float32, device=f_in.device)
-    ebops_u32 = torch.empty((), dtype=torch.int32, device=f_in.device)  # bit pattern of the uint32 value
-    g_f = torch.empty_like(f_in)
-    g_bk = torch.empty_like(b_ker)
-    g_bb = torch.empty_like(b_bias)
-    rc = _lib.load().hgq_dense_ebops(_ptr(k_in), _ptr(i_in), _ptr(f_in), P, K, N, _ptr(k_ker), _ptr(b_ker), _ptr(k_bias),
-                                     _ptr(b_bias), scale, bias_size, _kmode(mode_in, k_in), _kmode(mode_ker, k_ker), mode_bias,
-                                     _ptr(ebops), _ptr(ebops_u32), _ptr(g_f), _ptr(g_bk), _ptr(g_bb), _stream())
-    _lib.check(rc, 'hgq_dense_ebops')
-    return ebops, ebops_u32, g_f, g_bk, g_bb
-
-
-@dense_ebops_op.register_fake
-def _(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, bias_size, mode_in, mode_ker, mode_bias):
-    return f_in.new_empty(()), f_in.new_empty((), dtype=torch.int32), torch.empty_like(f_in), torch.empty_like(b_ker), torch.empty_like(b_bias)
-
-
-def _ebops_setup(ctx, inputs, output):
-    _, _, g_f, g_bk, g_bb = output
-    ctx.save_for_backward(g_f, g_bk, g_bb)
-    ctx.i_needs = inputs[1].requires_grad and not (inputs[12] & _lib.MODE_KBI)
-
-
-def _ebops_backward(ctx, g, *_unused):
-    g_f, g_bk, g_bb = ctx.saved_tensors
-    gf = g * g_f
-    return (None, gf if ctx.i_needs else None, gf, None, g * g_bk, None, g * g_bb if g_bb.numel() else None,
-            None, None, None, None, None, None, None, None)
-
-
-dense_ebops_op.register_autograd(_ebops_backward, setup_context=_ebops_setup)
-
-
-def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, bias_size, mode_in, mode_ker, mode_bias):
-    """Returns ``(ebops fp32 scalar, ebops truncated to uint32 as an int32 bit pattern)``."""
+    n_parts = 0
+    if amax.numel():
+        _need(amax.dtype == torch.int32 and amax.is_cuda and amax.numel() % (P * K) == 0, 'amax slices must be [n_parts, P*K] int32')
+        n_parts = amax.numel() // (P * K)
+    if ebops_var.numel():
+        _need(ebops_var.is_cuda and ebops_var.element_size() == 4, 'the ebops variable must be a 4-byte GPU scalar')
+    if beta.numel():
+        _check_f32('beta', beta)
     dev = f_in.device
-    e_f = torch.empty(0, dtype=torch.float32, device=dev)
-    e_k = torch.empty(0, dtype=torch.uint8, device=dev)
-    out = dense_ebops_op(k_in, i_in, f_in, k_ker, b_ker, k_bias if k_bias is not None else e_k,
-                         b_bias if b_bias is not None else e_f, P, K, N,
-                         float(scale), float(bias_size), mode_in, mode_ker, mode_bias)
-    return out[0], out[1]
+    ebops = torch.empty((), dtype=torch.float32, device=dev)
+    term = torch.empty((), dtype=torch.float32, device=dev)
+    nb = N if has_bias else 0
+    g = torch.empty(P * K + K * N + nb, dtype=torch.float32, device=dev)
+    g_f, g_bk, g_bb = g[:P * K], g[P * K:P * K + K * N], g[P * K + K * N:]
+    rc = _lib.load().hgq_dense_ebops(_ptr(amax), n_parts, decay, _ptr(beta), _ptr(term), _ptr(k_in), _ptr(i_in), _ptr(f_in),
+                                     P, K, N, _ptr(k_ker), _ptr(b_ker), _ptr(k_bias), _ptr(b_bias), scale, bias_size,
+                                     _kmode(mode_in, k_in), _kmode(mode_ker, k_ker), mode_bias, _ptr(ebops), _ptr(ebops_var),
+                                     _ptr(g_f), _ptr(g_bk), _ptr(g_bb), _stream())
+    _lib.check(rc, 'hgq_dense_ebops')
+    return ebops, term, g
 
 
-# --------------------------------------------------------------------------------------
-# loss and optimizer step
-# --------------------------------------------------------------------------------------
 @torch.library.custom_op('hgq::sparse_ce', mutates_args=())
 def sparse_ce_op(logits: Tensor, labels: Tensor) -> tuple[Tensor, Tensor]:
     _check_f32('logits', logits)
@@ -299,23 +221,6 @@ def _(logits, labels):
     return logits.new_empty(()), torch.empty_like(logits)
 
 
-def _ce_setup(ctx, inputs, output):
-    ctx.save_for_backward(output[1])
-
-
-def _ce_backward(ctx, g, _):
-    (dlogits,) = ctx.saved_tensors
-    return g * dlogits, None
-
-
-sparse_ce_op.register_autograd(_ce_backward, setup_context=_ce_setup)
-
-
-def sparse_ce(logits: Tensor, labels: Tensor) -> Tensor:
-    """Mean sparse categorical cross-entropy from logits."""
-    return sparse_ce_op(logits.contiguous(), labels)[0]
-
-
 @torch.library.custom_op('hgq::sgd_update', mutates_args=('w',))
 def sgd_update_op(w: Tensor, g: Tensor, lr: float, l1: float, lo: float, hi: float) -> None:
     _check_f32('w', w), _check_f32('g', g)
@@ -324,5 +229,166 @@ def sgd_update_op(w: Tensor, g: Tensor, lr: float, l1: float, lo: float, hi: flo
     _lib.check(rc, 'hgq_sgd_update')
 
 
+class _SgdItem(ctypes.Structure):
+    _fields_ = [('w', ctypes.c_void_p), ('g', ctypes.c_void_p), ('n', ctypes.c_int64), ('l1', ctypes.c_float),
+                ('lo', ctypes.c_float), ('hi', ctypes.c_float)]
+
+
+@torch.library.custom_op('hgq::sgd_update_multi', mutates_args=('ws',))
+def sgd_update_multi_op(ws: Sequence[Tensor], gs: Sequence[Tensor], l1: Sequence[float], lo: Sequence[float],
+                        hi: Sequence[float], lr: float) -> None:
+    n = len(ws)
+    _need(len(gs) == n and len(l1) == n and len(lo) == n and len(hi) == n, 'per-variable lists differ in length')
+    items = (_SgdItem * n)()
+    for t, (w, g) in enumerate(zip(ws, gs)):
+        _check_f32('w', w), _check_f32('g', g)
+        _need(w.numel() == g.numel(), 'gradient size mismatch')
+        items[t] = _SgdItem(w.data_ptr(), g.data_ptr(), w.numel(), l1[t], lo[t], hi[t])
+    rc = _lib.load().hgq_sgd_update_multi(items, n, lr, _stream())
+    _lib.check(rc, 'hgq_sgd_update_multi')
+
+
+# ======================================================================================
+# autograd pairing
+# ======================================================================================
+class _Quantize(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, k, i, fb, mode, bw_inner, track):
+        y, amax, neg = quantize_fwd(x, k, i, fb, mode, bw_inner, track)
+        ctx.save_for_backward(x, k, i, fb)
+        ctx.mode, ctx.bw_inner = mode, bw_inner
+        ctx.mark_non_differentiable(amax, neg)
+        ctx.set_materialize_grads(False)
+        return y, amax, neg
+
+    @staticmethod
+    def backward(ctx, gy, _ga, _gn):
+        if gy is None:
+            return (None,) * 7
+        if not (ctx.mode & _lib.MODE_TRAINING):
+            raise RuntimeError('hgq quantizer: gradients are defined for the training-mode forward only')
+        x, k, i, fb = ctx.saved_tensors
+        dx, di, dfb = quantize_bwd(gy.contiguous(), x, k, i, fb, ctx.mode, ctx.bw_inner)
+        return (dx if ctx.needs_input_grad[0] else None, None, di if ctx.needs_input_grad[2] else None,
+                dfb if ctx.needs_input_grad[3] else None, None, None, None)
+
+
+def quantize(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int = 1, track: bool = False):
+    """Fixed-point quantizer.  Returns ``(y, amax_bits, anyneg)``; the last two are empty unless ``track``."""
+    return _Quantize.apply(x.contiguous(), k.contiguous(), i.contiguous(), fb.contiguous(), mode, bw_inner, track)
+
+
+def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('inf'), anyneg=None, k_var=None):
+    """In-place integer-bit tracking; ``amax`` is [m] or [n_parts, m]."""
+    m = i_var.numel()
+    n_parts = amax.numel() // m
+    empty_i = amax.new_empty(0)
+    empty_k = torch.empty(0, dtype=torch.uint8, device=amax.device)
+    wrap_track_i_op(amax, anyneg if anyneg is not None else empty_i, n_parts, i_var, fb,
+                    k_var if k_var is not None else empty_k, float(decay), float(c_lo), float(c_hi), mode)
+
+
+FUSED_BWD_MAX = 64  # hgq_qdense_bwd covers K <= 64 and N <= 64
+
+
+class _QDense(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track):
+        y, amax = qdense_fwd(x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track)
+        ctx.save_for_backward(x, f_in, qw, y)
+        ctx.has_bias = qb.numel() > 0
+        ctx.act, ctx.mode, ctx.bw_rows, ctx.f_shape = act, mode, bw_rows, f_in.shape
+        ctx.mark_non_differentiable(amax)
+        ctx.set_materialize_grads(False)
+        return y, amax
+
+    @staticmethod
+    def backward(ctx, gy, _ga):
+        if gy is None:
+            return (None,) * 10
+        x, f_in, qw, y = ctx.saved_tensors
+        dx, dqw, dqb, df = qdense_bwd(gy.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows)
+        return (dx, None, None, df.view(ctx.f_shape) if ctx.bw_rows > 0 else None, dqw, dqb if ctx.has_bias else None,
+                None, None, None, None)
+
+
+def qdense(x2d, k_in, i_in, f_in, qw, qb, act: int, mode: int, bw_rows: int, track: bool):
+    """y = act(q_in(x) @ qw + qb) on a [rows, K] view; returns ``(y, amax slices)``."""
+    empty = x2d.new_empty(0)
+    return _QDense.apply(x2d, k_in if k_in is not None else empty, i_in if i_in is not None else empty,
+                         f_in if f_in is not None else empty, qw, qb if qb is not None else empty, act, mode, bw_rows, track)
+
+
+class _DenseEbops(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, i_in, f_in, b_ker, b_bias, amax, decay, beta, k_in, k_ker, k_bias, ebops_var, P, K, N, scale, bias_size,
+                mode_in, mode_ker, mode_bias):
+        ebops, term, g = dense_ebops_op(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N,
+                                        scale, bias_size, mode_in, mode_ker, mode_bias)
+        ctx.save_for_backward(g)
+        ctx.has_beta = beta.numel() > 0
+        ctx.sizes = (P * K, K * N, b_bias.numel())
+        ctx.kbi_in = bool(mode_in & _lib.MODE_KBI)
+        ctx.shapes = (i_in.shape, f_in.shape, b_ker.shape, b_bias.shape)
+        ctx.set_materialize_grads(False)
+        if ctx.has_beta:
+            ctx.mark_non_differentiable(ebops)
+        else:
+            ctx.mark_non_differentiable(term)
+        return ebops, term
+
+    @staticmethod
+    def backward(ctx, g_ebops, g_term):
+        (g,) = ctx.saved_tensors
+        up = g_term if ctx.has_beta else g_ebops
+        if up is None:
+            return (None,) * 19
+        grads = up * g
+        n_f, n_k, n_b = ctx.sizes
+        s_i, s_f, s_k, s_b = ctx.shapes
+        gf = grads[:n_f]
+        gi = gf.view(s_i) if (ctx.needs_input_grad[0] and not ctx.kbi_in) else None
+        return (gi, gf.view(s_f), grads[n_f:n_f + n_k].view(s_k), grads[n_f + n_k:].view(s_b) if n_b else None) + (None,) * 15
+
+
+def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, bias_size, mode_in, mode_ker, mode_bias,
+                amax=None, decay=0.0, beta=None, ebops_var=None):
+    """EBOPs of a dense contraction.  Returns ``(ebops, ebops * beta)``: with ``beta`` the second
+    carries the gradient (and the first is a plain value), without it the first does.  With
+    ``amax`` the input quantizer's integer bits are tracked in place first; with ``ebops_var`` the
+    uint32 variable is assigned."""
+    dev = f_in.device
+    e_f = torch.empty(0, dtype=torch.float32, device=dev)
+    e_i = torch.empty(0, dtype=torch.int32, device=dev)
+    e_k = torch.empty(0, dtype=torch.uint8, device=dev)
+    return _DenseEbops.apply(i_in, f_in, b_ker, b_bias if b_bias is not None else e_f, amax if amax is not None else e_i,
+                             float(decay), beta if beta is not None else e_f, k_in, k_ker,
+                             k_bias if k_bias is not None else e_k, ebops_var if ebops_var is not None else e_i, P, K, N,
+                             float(scale), float(bias_size), mode_in, mode_ker, mode_bias)
+
+
+class _SparseCE(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, labels):
+        loss, dlogits = sparse_ce_op(logits, labels)
+        ctx.save_for_backward(dlogits)
+        return loss
+
+    @staticmethod
+    def backward(ctx, g):
+        (dlogits,) = ctx.saved_tensors
+        return g * dlogits, None
+
+
+def sparse_ce(logits: Tensor, labels: Tensor) -> Tensor:
+    """Mean sparse categorical cross-entropy from logits."""
+    return _SparseCE.apply(logits.contiguous(), labels)
+
+
 def sgd_update_(w, g, lr, l1=0.0, lo=float('-inf'), hi=float('inf')):
     sgd_update_op(w, g.contiguous(), float(lr), float(l1), float(lo), float(hi))
+
+
+def sgd_update_multi_(ws, gs, l1, lo, hi, lr):
+    sgd_update_multi_op(list(ws), [g.contiguous() for g in gs], [float(v) for v in l1], [float(v) for v in lo],
+                        [float(v) for v in hi], float(lr))

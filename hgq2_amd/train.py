@@ -50,18 +50,25 @@ class SGD:
 
     @torch.no_grad()
     def step(self):
+        ws, gs, l1s, los, his, post = [], [], [], [], [], []
         for p in self.params:
             if p.grad is None:
                 continue
             c = getattr(p, 'constraint', None)
             r = getattr(p, 'regularizer', None)
-            l1 = r.l1 if (self.fold_regularizers and isinstance(r, MonoL1)) else 0.0
             bounds = c.bounds() if c is not None else (float('-inf'), float('inf'))
-            if bounds is None:
-                ops.sgd_update_(p.data, p.grad, self.lr, l1)
-                p.copy_(c(p))
-            else:
-                ops.sgd_update_(p.data, p.grad, self.lr, l1, bounds[0], bounds[1])
+            if bounds is None:  # a constraint that is not a clip: applied after the update
+                bounds = (float('-inf'), float('inf'))
+                post.append((p, c))
+            ws.append(p.data)
+            gs.append(p.grad)
+            l1s.append(r.l1 if (self.fold_regularizers and isinstance(r, MonoL1)) else 0.0)
+            los.append(bounds[0])
+            his.append(bounds[1])
+        if ws:
+            ops.sgd_update_multi_(ws, gs, l1s, los, his, self.lr)
+        for p, c in post:
+            p.copy_(c(p))
 
 
 class GraphedTrainStep:

@@ -96,11 +96,13 @@ int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float
  * (fixed_point_quantizer.py:16-31) and the `_i.assign(...)` recurrences of
  * FixedPointQuantizerKIF.call (:406-422) and FixedPointQuantizerKBI.call (:280-300).
  *
+ *   amax / anyneg [n_parts, m]: trackers as produced by hgq_quantize_fwd (n_parts = 1) or by
+ *   hgq_qdense_fwd (one slice per producing workgroup); they are combined here.
  *   i_var [m]  in/out: the raw `_i` variable;   fb [m]: raw `_f` (KIF) or `_b` (KBI)
  *   training : i_var <- max(i_var - decay, minimal_i)            (KBI: then clipped to [c_lo, c_hi])
  *   tracing  : i_var <- max(round(i_var), clip(minimal_i)),  k_var |= anyneg   (k_var uint8, optional)
  */
-int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, float *i_var, const float *fb,
+int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, int n_parts, float *i_var, const float *fb,
                      uint8_t *k_var, int64_t m, float decay, float c_lo, float c_hi, int mode, void *stream);
 
 /*
@@ -112,24 +114,30 @@ int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, float *i_var,
  *
  *   x [rows, K];  k_in/i_in/f_in [bw_rows, K] input-quantizer operands (row r uses entry
  *   r % bw_rows); bw_rows == 0 means x is used as is;  qw [K, N] quantized kernel;
- *   qb [N] quantized bias or NULL;  y [rows, N];  amax [bw_rows*K] optional.
- *   The input quantizer must be a training-mode WRAP quantizer or any inference/SAT mode
- *   selected by `mode`; act is HGQ_ACT_*.
+ *   qb [N] quantized bias or NULL;  y [rows, N];
+ *   amax_part [hgq_qdense_fwd_parts(rows), bw_rows*K] optional: per-workgroup slices of the
+ *   abs-max tracker (no atomics, no clearing pass), to be handed to hgq_wrap_track_i.
+ *   `mode` selects the input quantizer (any round / overflow mode, training or inference);
+ *   act is HGQ_ACT_*.
  */
+int hgq_qdense_fwd_parts(int64_t rows);
 int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_in, const float *f_in, int64_t bw_rows,
-                   const float *qw, const float *qb, float *y, uint32_t *amax, int64_t rows, int K, int N,
+                   const float *qw, const float *qb, float *y, uint32_t *amax_part, int64_t rows, int K, int N,
                    int act, int mode, void *stream);
 
 /*
  * QDense / QEinsumDense contraction, backward: autograd of the same expression.
  *   dx [rows, K] gradient w.r.t. the un-quantized input (straight-through);
  *   dqw [K, N], dqb [N] (NULL if no bias): gradients w.r.t. the quantized kernel / bias;
- *   df_in [bw_rows*K]: gradient w.r.t. the input quantizer's fractional bits (NULL if bw_rows == 0).
+ *   df_in [bw_rows*K]: gradient w.r.t. the input quantizer's fractional bits (NULL if bw_rows == 0);
+ *   workspace: hgq_qdense_bwd_workspace(rows, K, N, bw_rows) floats of scratch for the
+ *   per-workgroup partial sums, which a second kernel adds up in a fixed order (deterministic).
  * Supported: K <= 64 and N <= 64, training-mode WRAP input quantizer (round-only).
  */
+int64_t hgq_qdense_bwd_workspace(int64_t rows, int K, int N, int64_t bw_rows);
 int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
-                   const float *qw, float *dx, float *dqw, float *dqb, float *df_in, int64_t rows, int K,
-                   int N, int act, int mode, void *stream);
+                   const float *qw, float *dx, float *dqw, float *dqb, float *df_in, float *workspace,
+                   int64_t rows, int K, int N, int act, int mode, void *stream);
 
 /*
  * EBOPs of a dense contraction and its gradient.  Replaces QDense._compute_ebops
@@ -139,13 +147,19 @@ int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float 
  * with bits_in = relu(round(i_in)+round(f_in)) (+k for SAT), bits_ker / bits_bias = round(b) (+k for SAT).
  *
  *   ebops [1] fp32;  ebops_u32 [1] optional: the value cast to uint32 (the `_ebops` variable,
- *   src/hgq/layers/core/base.py:103);  g_f_in [P*K], g_b_ker [K*N], g_b_bias [N]: d ebops / d variable.
+ *   src/hgq/layers/core/base.py:103);  g_f_in [P*K], g_b_ker [K*N], g_b_bias [N]: d ebops / d variable;
+ *   beta [1], loss_term [1] optional: loss_term = ebops * beta (the add_loss term, base.py:104);
+ *   when beta is given the three gradient outputs are d loss_term / d variable (scaled by beta).
+ *   amax_part [n_parts, P*K] optional: when given, the input quantizer's integer bits are first
+ *   tracked in place in i_in exactly as hgq_wrap_track_i does in training mode with `decay`
+ *   (the reference updates `_i` in the layer call before EBOPs are computed, base.py:94-104);
+ *   meant for small P*K*n_parts - the single workgroup walks all slices.
  */
-int hgq_dense_ebops(const void *k_in, const float *i_in, const float *f_in, int64_t P, int K, int N,
+int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const float *beta, float *loss_term,
+                    const void *k_in, float *i_in, const float *f_in, int64_t P, int K, int N,
                     const void *k_ker, const float *b_ker, const void *k_bias, const float *b_bias,
                     float scale, float bias_size, int mode_in, int mode_ker, int mode_bias, float *ebops,
-                    uint32_t *ebops_u32,
-                    float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream);
+                    uint32_t *ebops_u32, float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream);
 
 /*
  * Mean sparse categorical cross-entropy from logits, forward and gradient in one pass.
@@ -162,6 +176,19 @@ int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *los
  *     w <- clip(w - lr * (g + l1), lo, hi)          (pass lo = -inf, hi = +inf for no constraint)
  */
 int hgq_sgd_update(float *w, const float *g, int64_t n, float lr, float l1, float lo, float hi, void *stream);
+
+/*
+ * The same update for many variables in one launch (descriptors are read on the host and travel
+ * to the kernel as launch arguments, so the call is safe under HIP graph capture).
+ */
+#define HGQ_SGD_BATCH 48
+typedef struct {
+    float *w;
+    const float *g;
+    int64_t n;
+    float l1, lo, hi;
+} hgq_sgd_item;
+int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *stream);
 
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);

@@ -190,7 +190,7 @@ def test_qdense_forward_backward(dev, rows, K, N, P, act):
     scale = (rx.detach().double().abs() @ qw.detach().double().abs()) + qb.detach().double().abs()
     _assert_close_sum(yd.detach(), y.detach(), scale, 'y')
     want_amax = rx.detach().abs().reshape(rows // P, P, K).amax(dim=0).reshape(-1)
-    assert torch.equal(amax.view(torch.float32).cpu(), want_amax)
+    assert torch.equal(amax.view(torch.float32).reshape(-1, P * K).amax(0).cpu(), want_amax)
     # The kernel's relu mask comes from its own fp32 output; rows where the sign of the
     # pre-activation is not decided at fp32 accuracy are excluded from the gradient check.
     yd.backward(gy.to(dev))
@@ -256,13 +256,35 @@ def test_dense_ebops_exact_and_gradients(dev):
     fi, bk, bb = d(iq._f), d(kq._b), d(bq._b)
     m_in = _lib.mode_bits('RND', 'WRAP', training=True, round_params=True)
     m_k = _lib.mode_bits('RND', 'SAT_SYM', training=True, round_params=True, kbi=True)
-    val, u32 = ops.dense_ebops(iq._k.reshape(-1).to(dev), d(iq._i), fi, kq._k.reshape(-1).to(dev), bk,
-                               bq._k.to(dev), bb, 1, 24, 10, 1.0, 10.0, m_in, m_k, m_k)
-    assert val.item() == e.item() and u32.item() == int(e.item())
+    var = torch.zeros((), dtype=torch.int32, device=dev)
+    val, _ = ops.dense_ebops(iq._k.reshape(-1).to(dev), d(iq._i), fi, kq._k.reshape(-1).to(dev), bk,
+                             bq._k.to(dev), bb, 1, 24, 10, 1.0, 10.0, m_in, m_k, m_k, ebops_var=var)
+    assert val.item() == e.item() and var.item() == int(e.item())
     val.backward()
     assert torch.equal(fi.grad.cpu(), iq._f.grad.reshape(-1))
     assert torch.equal(bk.grad.cpu(), kq._b.grad.reshape(-1))
     assert torch.equal(bb.grad.cpu(), bq._b.grad.reshape(-1))
+    # loss-term form: ebops * beta with the gradient scaled by beta, input integer bits tracked first
+    beta = torch.tensor(0.25, device=dev)
+    amax = torch.randint(0, 2**30, (7, 24), dtype=torch.int32, device=dev)
+    i_track = d(iq._i).clone()
+    want_i = i_track.clone()
+    ops.wrap_track_i_(amax, want_i, fi.detach(), 0.01, _lib.mode_bits('RND', 'WRAP', training=True))
+    with torch.no_grad():
+        layer.iq.quantizer._i.copy_(want_i.cpu().reshape(1, 24))
+    for v in (iq._f, kq._b, bq._b):
+        v.grad = None
+    e2 = layer._compute_ebops((1, 24)) * 0.25
+    e2.backward()
+    fi2, bk2, bb2 = d(iq._f), d(kq._b), d(bq._b)
+    _, term = ops.dense_ebops(iq._k.reshape(-1).to(dev), i_track, fi2, kq._k.reshape(-1).to(dev), bk2, bq._k.to(dev), bb2,
+                              1, 24, 10, 1.0, 10.0, m_in, m_k, m_k, amax=amax, decay=0.01, beta=beta, ebops_var=var)
+    assert torch.equal(i_track, want_i)
+    assert term.item() == e2.item() and var.item() == int(e2.item() / 0.25)
+    term.backward()
+    assert torch.equal(fi2.grad.cpu(), iq._f.grad.reshape(-1))
+    assert torch.equal(bk2.grad.cpu(), kq._b.grad.reshape(-1))
+    assert torch.equal(bb2.grad.cpu(), bq._b.grad.reshape(-1))
 
 
 def test_sparse_ce_and_sgd(dev):
@@ -282,3 +304,11 @@ def test_sparse_ce_and_sgd(dev):
     wd = w.to(dev)
     ops.sgd_update_(wd, gr.to(dev), 0.01, 1e-8, -2.0, 2.0)
     assert torch.equal(wd.cpu(), torch.clamp(w - 0.01 * (gr + 1e-8), -2.0, 2.0))
+    # many variables in one launch (more than one descriptor batch)
+    ws = [torch.randn(n, generator=g) for n in ([5, 1024, 37, 2048] * 15)]
+    gs = [torch.randn(t.shape, generator=g) for t in ws]
+    wds, gds = [t.to(dev) for t in ws], [t.to(dev) for t in gs]
+    n = len(ws)
+    ops.sgd_update_multi_(wds, gds, [1e-8] * n, [-1.0] * n, [float('inf')] * n, 0.05)
+    for wd_, w_, g_ in zip(wds, ws, gs):
+        assert torch.equal(wd_.cpu(), torch.clamp(w_ - 0.05 * (g_ + 1e-8), min=-1.0))
