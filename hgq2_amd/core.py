@@ -186,7 +186,7 @@ class Layer(nn.Module):
                 out += m._losses
         for p in self.parameters():
             r = getattr(p, 'regularizer', None)
-            if r is not None:
+            if r is not None and p.requires_grad:
                 out.append(r(p))
         return out
 

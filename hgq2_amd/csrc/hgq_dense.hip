@@ -306,7 +306,15 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restri
     if (e < M) {
         const int per = (n_parts + 3) / 4;
         const int g0 = grp * per, g1 = min(n_parts, g0 + per);
-        for (int g = g0; g < g1; ++g) s += part[(int64_t)g * M + e];
+        // eight independent loads in flight per thread: the loop is latency-bound otherwise
+        int g = g0;
+        for (; g + 8 <= g1; g += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(int64_t)(g + u) * M + e];
+            s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+        }
+        for (; g < g1; ++g) s += part[(int64_t)g * M + e];
     }
     red[threadIdx.x] = s;
     __syncthreads();

@@ -69,14 +69,21 @@ struct VecIO<1> {
     static __device__ __forceinline__ void load_k(const void *k, int64_t v, bool u8, float *o) { o[0] = hgq::load_k(k, v, u8); }
     static __device__ __forceinline__ void store_u32(uint32_t *p, int64_t v, const uint32_t *o) { p[v] = o[0]; }
 };
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 128-bit accesses.  Loads and stores are non-temporal: every operand is touched once, so the
+// caches are bypassed instead of polluted; measured on MI355X this is worth ~10 % of bandwidth.
 template <>
 struct VecIO<4> {
     static __device__ __forceinline__ void load(const float *p, int64_t v, float *o) {
-        float4 t = ((const float4 *)p)[v];
+        const f32x4 t = __builtin_nontemporal_load((const f32x4 *)p + v);
         o[0] = t.x, o[1] = t.y, o[2] = t.z, o[3] = t.w;
     }
     static __device__ __forceinline__ void store(float *p, int64_t v, const float *o) {
-        ((float4 *)p)[v] = make_float4(o[0], o[1], o[2], o[3]);
+        f32x4 t;
+        t.x = o[0], t.y = o[1], t.z = o[2], t.w = o[3];
+        __builtin_nontemporal_store(t, (f32x4 *)p + v);
     }
     static __device__ __forceinline__ void load_k(const void *k, int64_t v, bool u8, float *o) {
         if (u8) {
@@ -87,15 +94,19 @@ struct VecIO<4> {
         }
     }
     static __device__ __forceinline__ void store_u32(uint32_t *p, int64_t v, const uint32_t *o) {
-        ((uint4 *)p)[v] = make_uint4(o[0], o[1], o[2], o[3]);
+        u32x4 t;
+        t.x = o[0], t.y = o[1], t.z = o[2], t.w = o[3];
+        __builtin_nontemporal_store(t, (u32x4 *)p + v);
     }
 };
 
 // ------------------------------------------------------------------------------------------
 // 1-D kernels: per-element or shared bit-widths
 // ------------------------------------------------------------------------------------------
+#define Q1D_BS 512
+
 template <int RM, int OM, int VEC, bool SHARED>
-__global__ __launch_bounds__(256) void quant_fwd_1d(const float *__restrict__ x, const void *__restrict__ k,
+__global__ __launch_bounds__(Q1D_BS) void quant_fwd_1d(const float *__restrict__ x, const void *__restrict__ k,
                                                     const float *__restrict__ i, const float *__restrict__ fb,
                                                     float *__restrict__ y, uint32_t *amax, uint32_t *anyneg,
                                                     int64_t nvec, int mode) {
@@ -103,7 +114,7 @@ __global__ __launch_bounds__(256) void quant_fwd_1d(const float *__restrict__ x,
     KIF ps;
     if (SHARED) ps = resolve_kif(load_k(k, 0, m.k_u8), i[0], fb[0], m.kbi, m.round_params);
     uint32_t lmax = 0, lneg = 0;
-    for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+    for (int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * Q1D_BS) {
         float xv[VEC], kv[VEC], iv[VEC], fv[VEC], yv[VEC];
         VecIO<VEC>::load(x, v, xv);
         if (!SHARED) {
@@ -129,14 +140,14 @@ __global__ __launch_bounds__(256) void quant_fwd_1d(const float *__restrict__ x,
         }
     }
     if (SHARED && (amax || anyneg)) {
-        __shared__ uint32_t smax[4], sneg[4];
+        __shared__ uint32_t smax[Q1D_BS / 64], sneg[Q1D_BS / 64];
         lmax = wave_max_u32(lmax);
         lneg = wave_or_u32(lneg);
         if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6] = lmax, sneg[threadIdx.x >> 6] = lneg;
         __syncthreads();
         if (threadIdx.x == 0) {
             uint32_t a = smax[0], g = sneg[0];
-            for (int w = 1; w < 4; ++w) a = smax[w] > a ? smax[w] : a, g |= sneg[w];
+            for (int w = 1; w < Q1D_BS / 64; ++w) a = smax[w] > a ? smax[w] : a, g |= sneg[w];
             if (amax) atomicMax(amax, a);
             if (anyneg && g) atomicOr(anyneg, 1u);
         }
@@ -144,7 +155,7 @@ __global__ __launch_bounds__(256) void quant_fwd_1d(const float *__restrict__ x,
 }
 
 template <int RM, int OM, int VEC, bool SHARED>
-__global__ __launch_bounds__(256) void quant_bwd_1d(const float *__restrict__ dy, const float *__restrict__ x,
+__global__ __launch_bounds__(Q1D_BS) void quant_bwd_1d(const float *__restrict__ dy, const float *__restrict__ x,
                                                     const void *__restrict__ k, const float *__restrict__ i,
                                                     const float *__restrict__ fb, float *__restrict__ dx,
                                                     float *di, float *dfb, int64_t nvec, int mode) {
@@ -152,7 +163,7 @@ __global__ __launch_bounds__(256) void quant_bwd_1d(const float *__restrict__ dy
     KIF ps;
     if (SHARED) ps = resolve_kif(load_k(k, 0, m.k_u8), i[0], fb[0], m.kbi, m.round_params);
     float si = 0.0f, sf = 0.0f;
-    for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+    for (int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * Q1D_BS) {
         float gv[VEC], xv[VEC], kv[VEC], iv[VEC], fv[VEC], dxv[VEC], div[VEC], dfv[VEC];
         VecIO<VEC>::load(dy, v, gv);
         VecIO<VEC>::load(x, v, xv);
@@ -177,14 +188,16 @@ __global__ __launch_bounds__(256) void quant_bwd_1d(const float *__restrict__ dy
         }
     }
     if (SHARED) {
-        __shared__ float ssi[4], ssf[4];
+        __shared__ float ssi[Q1D_BS / 64], ssf[Q1D_BS / 64];
         si = wave_sum_f32(si);
         sf = wave_sum_f32(sf);
         if ((threadIdx.x & 63) == 0) ssi[threadIdx.x >> 6] = si, ssf[threadIdx.x >> 6] = sf;
         __syncthreads();
         if (threadIdx.x == 0) {
-            if (di) atomicAdd(di, ssi[0] + ssi[1] + ssi[2] + ssi[3]);
-            if (dfb) atomicAdd(dfb, ssf[0] + ssf[1] + ssf[2] + ssf[3]);
+            float ti = 0.f, tf = 0.f;
+            for (int w = 0; w < Q1D_BS / 64; ++w) ti += ssi[w], tf += ssf[w];
+            if (di) atomicAdd(di, ti);
+            if (dfb) atomicAdd(dfb, tf);
         }
     }
 }
@@ -381,7 +394,19 @@ __global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__res
     if (t < n) {
         const int per = (n_parts + 3) / 4;
         const int g0 = grp * per, g1 = min(n_parts, g0 + per);
-        for (int g = g0; g < g1; ++g) {
+        int g = g0;
+        for (; g + 8 <= g1; g += 8) {  // independent loads in flight
+            uint32_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = amax[(int64_t)(g + u) * n + t];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) mx = v[u] > mx ? v[u] : mx;
+            if (anyneg) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) ng |= anyneg[(int64_t)(g + u) * n + t];
+            }
+        }
+        for (; g < g1; ++g) {
             const uint32_t a = amax[(int64_t)g * n + t];
             mx = a > mx ? a : mx;
             if (anyneg) ng |= anyneg[(int64_t)g * n + t];
@@ -470,19 +495,19 @@ extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, c
         const int64_t tail0 = n4 * 4, tail = n - tail0;
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (n4 > 0) {
-                const int grid = persistent_grid((n4 + 255) / 256, 8);
+                const int grid = persistent_grid((n4 + Q1D_BS - 1) / Q1D_BS, 16);
                 if (shared)
-                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 4, true>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n4, mode);
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 4, true>), dim3(grid), dim3(Q1D_BS), 0, s, x, k, i, fb, y, amax, anyneg, n4, mode);
                 else
-                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 4, false>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n4, mode);
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 4, false>), dim3(grid), dim3(Q1D_BS), 0, s, x, k, i, fb, y, amax, anyneg, n4, mode);
             }
             if (tail > 0) {
-                const int grid = persistent_grid((tail + 255) / 256, 8);
+                const int grid = 1;
                 if (shared) {
-                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 1, true>), dim3(grid), dim3(256), 0, s, x + tail0, k, i, fb, y + tail0, amax, anyneg, tail, mode);
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 1, true>), dim3(grid), dim3(Q1D_BS), 0, s, x + tail0, k, i, fb, y + tail0, amax, anyneg, tail, mode);
                 } else {
                     const void *kt = m.k_u8 ? (const void *)((const uint8_t *)k + tail0) : (const void *)((const float *)k + tail0);
-                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 1, false>), dim3(grid), dim3(256), 0, s, x + tail0, kt, i + tail0, fb + tail0, y + tail0,
+                    hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 1, false>), dim3(grid), dim3(Q1D_BS), 0, s, x + tail0, kt, i + tail0, fb + tail0, y + tail0,
                                        amax ? amax + tail0 : nullptr, anyneg ? anyneg + tail0 : nullptr, tail, mode);
                 }
             }
@@ -539,20 +564,20 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
         const int64_t tail0 = n4 * 4, tail = n - tail0;
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (n4 > 0) {
-                const int grid = persistent_grid((n4 + 255) / 256, 8);
+                const int grid = persistent_grid((n4 + Q1D_BS - 1) / Q1D_BS, 16);
                 if (shared)
-                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 4, true>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n4, mode);
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 4, true>), dim3(grid), dim3(Q1D_BS), 0, s, dy, x, k, i, fb, dx, di, dfb, n4, mode);
                 else
-                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 4, false>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n4, mode);
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 4, false>), dim3(grid), dim3(Q1D_BS), 0, s, dy, x, k, i, fb, dx, di, dfb, n4, mode);
             }
             if (tail > 0) {
-                const int grid = persistent_grid((tail + 255) / 256, 8);
+                const int grid = 1;
                 if (shared) {
-                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 1, true>), dim3(grid), dim3(256), 0, s, dy + tail0, x + tail0, k, i, fb,
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 1, true>), dim3(grid), dim3(Q1D_BS), 0, s, dy + tail0, x + tail0, k, i, fb,
                                        dx ? dx + tail0 : nullptr, di, dfb, tail, mode);
                 } else {
                     const void *kt = m.k_u8 ? (const void *)((const uint8_t *)k + tail0) : (const void *)((const float *)k + tail0);
-                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 1, false>), dim3(grid), dim3(256), 0, s, dy + tail0, x + tail0, kt, i + tail0, fb + tail0,
+                    hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 1, false>), dim3(grid), dim3(Q1D_BS), 0, s, dy + tail0, x + tail0, kt, i + tail0, fb + tail0,
                                        dx ? dx + tail0 : nullptr, di ? di + tail0 : nullptr, dfb ? dfb + tail0 : nullptr, tail, mode);
                 }
             }

@@ -63,14 +63,39 @@ __global__ __launch_bounds__(256) void dense_ebops_kernel(const uint32_t *amax_p
     if (amax_part) {
         // integer-bit tracking of the (KIF, WRAP, training) input quantizer, before its bits are read:
         // _i <- max(_i - decay, ceil(log2(max|x_q| + 2**-f)))
-        for (int64_t e = t; e < P * K; e += 256) {
+        // 256 threads = `ne` entries x `ng` slice groups per pass, combined through LDS
+        __shared__ uint32_t tmax[256];
+        const int64_t PK = P * K;
+        int ne = 1;
+        while (ne < 256 && ne < PK) ne <<= 1;
+        const int ng = 256 / ne, el = t % ne, grp = t / ne;
+        const int per = (n_parts + ng - 1) / ng;
+        for (int64_t e0 = 0; e0 < PK; e0 += ne) {
+            const int64_t e = e0 + el;
             uint32_t mx = 0;
-            for (int g = 0; g < n_parts; ++g) {
-                const uint32_t a = amax_part[(int64_t)g * P * K + e];
-                mx = a > mx ? a : mx;
+            if (e < PK) {
+                const int g0 = grp * per, g1 = min(n_parts, g0 + per);
+                int g = g0;
+                for (; g + 8 <= g1; g += 8) {
+                    uint32_t v[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) v[u] = amax_part[(int64_t)(g + u) * PK + e];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) mx = v[u] > mx ? v[u] : mx;
+                }
+                for (; g < g1; ++g) {
+                    const uint32_t a = amax_part[(int64_t)g * PK + e];
+                    mx = a > mx ? a : mx;
+                }
             }
-            const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-rintf(f_in[e]))));
-            i_in[e] = fmaxf(__fsub_rn(i_in[e], decay), mi_);
+            tmax[t] = mx;
+            __syncthreads();
+            if (grp == 0 && e < PK) {
+                for (int w = 1; w < ng; ++w) mx = tmax[el + w * ne] > mx ? tmax[el + w * ne] : mx;
+                const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-rintf(f_in[e]))));
+                i_in[e] = fmaxf(__fsub_rn(i_in[e], decay), mi_);
+            }
+            __syncthreads();
         }
         __threadfence_block();
         __syncthreads();

@@ -24,9 +24,9 @@ def model_loss(model, base_loss, fold_regularizers: bool = False):
             loss = loss + term
     for p in model.parameters():
         r = getattr(p, 'regularizer', None)
-        if r is None:
+        if r is None or not p.requires_grad:  # Keras regularises trainable variables only
             continue
-        if fold_regularizers and isinstance(r, MonoL1) and p.requires_grad:
+        if fold_regularizers and isinstance(r, MonoL1):
             continue
         loss = loss + r(p)
     return loss

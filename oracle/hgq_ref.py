@@ -223,10 +223,11 @@ class RefFixedPointQuantizer:
         return [v for v in (self._i, self._f, self._b) if v is not None and v.requires_grad]
 
     def regularization_loss(self):
-        """regularizers/__init__.py:13-14 applied to each variable that carries one."""
+        """regularizers/__init__.py:13-14 applied to each trainable variable that carries one
+        (Keras collects regularization losses from trainable weights only)."""
         loss = 0.0
         for v, r in ((self._i, self.i_regularizer), (self._f, self.f_regularizer), (self._b, self.b_regularizer)):
-            if v is not None and r is not None:
+            if v is not None and r is not None and v.requires_grad:
                 loss = loss + r * torch.sum(v)
         return loss
 
