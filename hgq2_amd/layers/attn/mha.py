@@ -1,0 +1,189 @@
+"""QMultiHeadAttention (reference src/hgq/layers/attn/mha.py:27-537) for rank-3 inputs
+``[batch, sequence, features]``: four QEinsumDense projections (query / key / value with output
+quantizers, attention_output), scaled dot-product scores, the table softmax, and the EBOPs of
+the two score contractions.  The einsum strings are those Keras builds for rank-3 inputs."""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ...core import Constant
+from ...quantizer import Quantizer
+from ...quantizer.config import QuantizerConfig
+from ..core.base import QLayerBase
+from ..core.einsum_dense import QEinsumDense
+from ..softmax import QSoftmax
+
+_PROJ_EQ, _PROJ_BIAS = 'abc,cde->abde', 'de'
+_OUT_EQ, _OUT_BIAS = 'abcd,cde->abe', 'e'
+_DOT_EQ = 'aecd,abcd->acbe'      # key [B,S,N,H], query [B,T,N,H] -> scores [B,N,T,S]
+_COMBINE_EQ = 'acbe,aecd->abcd'  # scores [B,N,T,S], value [B,S,N,H] -> [B,T,N,H]
+
+
+class QMultiHeadAttention(QLayerBase):
+    __output_quantizer_handled__ = True
+
+    def __init__(self, num_heads, key_dim, value_dim=None, dropout=0.0, use_bias=True, output_shape=None,
+                 attention_axes=None, kernel_initializer='glorot_uniform', bias_initializer='zeros', seed=None,
+                 fuse='none', qkvo_iq_conf=None, qkvo_kq_conf=None, qkvo_bq_conf=None, qkvo_oq_conf=None,
+                 softmax_iq_conf=None, softmax_exp_iq_conf=None, softmax_exp_oq_conf=None, softmax_inv_iq_conf=None,
+                 softmax_inv_oq_conf=None, softmax_oq_conf=None, stable_softmax=True,
+                 softmax_allow_heterogeneous_table: bool = False, parallelization_factor=-1, **kwargs):
+        super().__init__(**kwargs)
+        if attention_axes is not None:
+            raise NotImplementedError('only attention over the sequence axis of rank-3 inputs is supported')
+        self._num_heads, self._key_dim = int(num_heads), int(key_dim)
+        self._value_dim = int(value_dim) if value_dim else int(key_dim)
+        self._dropout, self._use_bias, self._output_shape = float(dropout), use_bias, output_shape
+        self._kernel_initializer, self._bias_initializer = kernel_initializer, bias_initializer
+        self._qkvo_iq_conf = qkvo_iq_conf or QuantizerConfig(place='datalane')
+        self._qkvo_kq_conf = qkvo_kq_conf or QuantizerConfig(place='weight')
+        self._qkvo_bq_conf = qkvo_bq_conf or QuantizerConfig(place='bias')
+        self._qkvo_oq_conf = qkvo_oq_conf or QuantizerConfig(place='datalane')
+        self._softmax_iq_conf = softmax_iq_conf or QuantizerConfig(place='datalane')
+        self._softmax_exp_iq_conf = softmax_exp_iq_conf or QuantizerConfig(place='datalane', overflow_mode='SAT')
+        self._softmax_exp_oq_conf = softmax_exp_oq_conf or QuantizerConfig(place='table')
+        self._softmax_inv_iq_conf = softmax_inv_iq_conf or QuantizerConfig(place='datalane')
+        self._softmax_inv_oq_conf = softmax_inv_oq_conf or QuantizerConfig(place='table')
+        self._softmax_oq_conf = softmax_oq_conf or QuantizerConfig(place='datalane')
+        self._softmax_allow_heterogeneous_table = softmax_allow_heterogeneous_table
+        self.parallelization_factor = parallelization_factor
+        self._stable_softmax = stable_softmax
+        self._fuse = fuse.lower()
+        self._inverse_sqrt_key_dim = 1.0 / math.sqrt(float(key_dim))
+
+    def _sub_kwargs(self):
+        return dict(kernel_initializer=self._kernel_initializer, bias_initializer=self._bias_initializer,
+                    iq_conf=self._qkvo_iq_conf.copy(), kq_conf=self._qkvo_kq_conf.copy(), bq_conf=self._qkvo_bq_conf.copy(),
+                    oq_conf=self._qkvo_oq_conf.copy(), enable_ebops=self.enable_ebops, beta0=self._beta0.clone(),
+                    parallelization_factor=self.parallelization_factor)
+
+    def _build_sub(self, layer, shape):
+        layer._build_device = self._build_device
+        layer.build(tuple(shape))
+        layer.built = True
+
+    def build(self, query_shape, value_shape=None, key_shape=None):
+        if isinstance(query_shape, list) and query_shape and isinstance(query_shape[0], (tuple, list)):
+            shapes = list(query_shape)
+            query_shape = shapes[0]
+            value_shape = shapes[1] if len(shapes) > 1 else None
+            key_shape = shapes[2] if len(shapes) > 2 else None
+        value_shape = query_shape if value_shape is None else value_shape
+        key_shape = value_shape if key_shape is None else key_shape
+        if len(query_shape) != 3:
+            raise NotImplementedError('QMultiHeadAttention: rank-3 inputs [batch, sequence, features] only')
+        if self._fuse == 'qkv':
+            assert query_shape == value_shape == key_shape, 'For fuse=qkv, query, key and value must have the same shape'
+        if self._fuse == 'kv':
+            assert value_shape == key_shape, 'For fuse=kv, key and value must have the same shape'
+        if tuple(value_shape[1:-1]) != tuple(key_shape[1:-1]):
+            raise ValueError('All dimensions of `value` and `key`, except the last one, must be equal.')
+        T, S = query_shape[1], value_shape[1]
+        N = self._num_heads
+        bias = _PROJ_BIAS if self._use_bias else None
+        self._query_dense = QEinsumDense(_PROJ_EQ, output_shape=[T, N, self._key_dim], bias_axes=bias, name='query',
+                                         enable_iq=self.enable_iq and not self._fuse == 'qkv', enable_oq=True, **self._sub_kwargs())
+        self._key_dense = QEinsumDense(_PROJ_EQ, output_shape=[S, N, self._key_dim], bias_axes=None, name='key',
+                                       enable_iq=self.enable_iq and self._fuse not in ('qkv', 'kv'), enable_oq=True,
+                                       **self._sub_kwargs())
+        self._value_dense = QEinsumDense(_PROJ_EQ, output_shape=[S, N, self._value_dim], bias_axes=bias, name='value',
+                                         enable_iq=self.enable_iq, enable_oq=True, **self._sub_kwargs())
+        self._build_sub(self._value_dense, value_shape)
+        if self._fuse == 'qkv' and self.enable_iq:
+            self._query_dense._iq = self._value_dense._iq
+            self._query_dense._enable_iq = True
+        if self._fuse in ('qkv', 'kv') and self.enable_iq:
+            self._key_dense._iq = self._value_dense._iq
+            self._key_dense._enable_iq = True
+        self._build_sub(self._query_dense, query_shape)
+        self._build_sub(self._key_dense, key_shape)
+
+        self._softmax = QSoftmax(
+            enable_oq=True, axis=(3,), stable=self._stable_softmax, iq_conf=self._softmax_iq_conf,
+            exp_iq_conf=self._softmax_exp_iq_conf, exp_oq_conf=self._softmax_exp_oq_conf,
+            inv_iq_conf=self._softmax_inv_iq_conf, inv_oq_conf=self._softmax_inv_oq_conf, oq_conf=self._softmax_oq_conf,
+            allow_heterogeneous_table=self._softmax_allow_heterogeneous_table, input_scaler=self._inverse_sqrt_key_dim,
+            enable_ebops=self.enable_ebops)
+        self._inverse_sqrt_key_dim = 1.0  # the scale now lives in the softmax's exp table
+        self._build_sub(self._softmax, (query_shape[0], N, T, S))
+
+        out_dim = self._output_shape if self._output_shape else query_shape[-1]
+        if isinstance(out_dim, (tuple, list)):
+            (out_dim,) = out_dim
+        self._output_dense = QEinsumDense(_OUT_EQ, output_shape=[T, out_dim], bias_axes=_OUT_BIAS if self._use_bias else None,
+                                          name='attention_output', enable_iq=True, enable_oq=self.enable_oq,
+                                          **self._sub_kwargs())
+        self._build_sub(self._output_dense, (query_shape[0], T, N, self._value_dim))
+
+        if self.enable_ebops:
+            self._beta = self.add_weight(name='beta', shape=(), initializer=self._beta0, trainable=False)
+            self._ebops = self.add_weight(name='ebops', shape=(), initializer=Constant(0.0), trainable=False, dtype='uint32')
+        self._q_shape = (1, T, N, self._key_dim)
+        self._k_shape = (1, S, N, self._key_dim)
+        self._v_shape = (1, S, N, self._value_dim)
+        self.built = True
+
+    def _maybe_build(self, args):
+        if self.built:
+            return
+        q = args[0]
+        self._build_device = q.device
+        v = args[1] if len(args) > 1 and args[1] is not None else None
+        k = args[2] if len(args) > 2 and args[2] is not None else None
+        self.build(tuple(q.shape), tuple(v.shape) if v is not None else None, tuple(k.shape) if k is not None else None)
+
+    def _compute_ebops(self, query_shape, value_shape=None, key_shape=None):
+        value_shape = query_shape if value_shape is None else value_shape
+        attn_shape = (1, self._num_heads, query_shape[1], value_shape[1])
+        bw_q = self._query_dense.oq.bits_(self._q_shape)
+        bw_k = self._key_dense.oq.bits_(self._k_shape)
+        bw_v = self._value_dense.oq.bits_(self._v_shape)
+        bw_attn = self._softmax.oq.bits_(attn_shape)
+        ebops_qk = torch.einsum(_DOT_EQ.split('->')[0] + '->', bw_k, bw_q)
+        ebops_av = torch.einsum(_COMBINE_EQ.split('->')[0] + '->', bw_attn, bw_v)
+        ebops = ebops_qk + ebops_av
+        if self.parallelization_factor > 0:
+            return ebops * self.parallelization_factor
+        return ebops
+
+    @property
+    def ebops(self):
+        if self._ebops is None:
+            return 0
+        own = int(self._ebops.cpu().view(torch.int32))
+        subs = (self._query_dense, self._key_dense, self._value_dense, self._output_dense)
+        return own + sum(int(s.ebops.cpu().view(torch.int32)) for s in subs) + self._softmax.ebops
+
+    def call(self, query, value=None, key=None, attention_mask=None, return_attention_scores=False, training=None,
+             use_causal_mask=False):
+        if value is None:
+            value = query
+        if key is None:
+            key = value
+        if use_causal_mask:
+            T, S = query.shape[1], value.shape[1]
+            causal = torch.tril(torch.ones((1, T, S), dtype=torch.bool, device=query.device))
+            attention_mask = causal if attention_mask is None else (attention_mask.bool() & causal)
+        q = self._query_dense(query)
+        k = self._key_dense(key)
+        v = self._value_dense(value)
+        out, scores = self._compute_attention(q, k, v, attention_mask, training)
+        out = self._output_dense(out)
+        if self.enable_oq:
+            out = self.oq(out, training=training)
+        if return_attention_scores:
+            return out, scores
+        return out
+
+    def _compute_attention(self, query, key, value, attention_mask=None, training=None):
+        query = query * self._inverse_sqrt_key_dim
+        scores = torch.einsum(_DOT_EQ, key, query)
+        mask = None
+        if attention_mask is not None:
+            mask = attention_mask.unsqueeze(1)  # broadcast over heads
+        scores = self._softmax(scores, mask=mask)
+        final = torch.nn.functional.dropout(scores, self._dropout) if (self._dropout and training) else scores
+        return torch.einsum(_COMBINE_EQ, final, value), scores

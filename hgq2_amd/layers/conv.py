@@ -1,0 +1,140 @@
+"""QConv2D (reference src/hgq/layers/conv.py:12-102,175-200): ``act(conv(iq(x), kq(W)) + bq(b))``
+on channels-last tensors with the kernel in HWIO layout, and the EBOPs obtained by convolving the
+bit-width tensors.  The input / kernel / bias quantizers run in the HIP quantizer kernels; the
+convolution of the quantized operands is the plain library convolution."""
+
+from __future__ import annotations
+
+from math import prod
+
+import torch
+import torch.nn.functional as F
+
+from ..core import get_initializer
+from ..quantizer import Quantizer
+from ..quantizer.config import QuantizerConfig
+from .core._contraction import get_activation
+from .core.base import QLayerBaseSingleInput
+
+
+def _pair(v):
+    return (int(v), int(v)) if isinstance(v, int) else tuple(int(t) for t in v)
+
+
+class QConv2D(QLayerBaseSingleInput):
+    def __init__(self, filters, kernel_size, strides=(1, 1), padding='valid', data_format=None, dilation_rate=(1, 1),
+                 groups=1, activation=None, use_bias=True, kernel_initializer='glorot_uniform', bias_initializer='zeros',
+                 kernel_regularizer=None, bias_regularizer=None, activity_regularizer=None, kernel_constraint=None,
+                 bias_constraint=None, kq_conf: None | QuantizerConfig = None, iq_conf: None | QuantizerConfig = None,
+                 bq_conf: None | QuantizerConfig = None, parallelization_factor=-1, **kwargs):
+        super().__init__(iq_conf=iq_conf, **kwargs)
+        if data_format not in (None, 'channels_last'):
+            raise NotImplementedError('QConv2D: channels_last only')
+        if groups != 1:
+            raise NotImplementedError('QConv2D: groups == 1 only')
+        self.rank = 2
+        self.filters = int(filters)
+        self.kernel_size, self.strides, self.dilation_rate = _pair(kernel_size), _pair(strides), _pair(dilation_rate)
+        self.padding = padding.lower()
+        assert self.padding in ('valid', 'same')
+        self.data_format = 'channels_last'
+        self.activation, self._act_name = get_activation(activation)
+        self.use_bias = use_bias
+        self.kernel_initializer = get_initializer(kernel_initializer)
+        self.bias_initializer = get_initializer(bias_initializer)
+        self.kernel_regularizer, self.bias_regularizer = kernel_regularizer, bias_regularizer
+        self.kernel_constraint, self.bias_constraint = kernel_constraint, bias_constraint
+        kq_conf = kq_conf or QuantizerConfig('default', 'weight')
+        self._kq = Quantizer(kq_conf, name=f'{self.name}_kq')
+        bq_conf = bq_conf or QuantizerConfig('default', 'bias')
+        self._bq = Quantizer(bq_conf, name=f'{self.name}_bq') if use_bias else None
+        self.parallelization_factor = parallelization_factor
+        self.bias = None
+
+    @property
+    def kq(self):
+        return self._kq
+
+    @property
+    def bq(self):
+        return self._bq
+
+    @property
+    def kernel(self):
+        return self._kernel
+
+    def compute_output_shape(self, input_shape):
+        out = [input_shape[0]]
+        for d, (k, s, dil) in enumerate(zip(self.kernel_size, self.strides, self.dilation_rate)):
+            n = input_shape[1 + d]
+            if n is None:
+                out.append(None)
+            elif self.padding == 'same':
+                out.append(-(-n // s))
+            else:
+                out.append((n - dil * (k - 1) - 1) // s + 1)
+        return tuple(out) + (self.filters,)
+
+    def build(self, input_shape):
+        super().build(input_shape)
+        c_in = int(input_shape[-1])
+        self._kernel = self.add_weight(name='kernel', shape=self.kernel_size + (c_in, self.filters),
+                                       initializer=self.kernel_initializer, regularizer=self.kernel_regularizer,
+                                       constraint=self.kernel_constraint)
+        if self.use_bias:
+            self.bias = self.add_weight(name='bias', shape=(self.filters,), initializer=self.bias_initializer,
+                                        regularizer=self.bias_regularizer, constraint=self.bias_constraint)
+        for q, shape in ((self.kq, self._kernel.shape), (self.bq, (self.filters,))):
+            if q is not None:
+                q._build_device = self._build_device
+                q.build(tuple(shape))
+                q.built = True
+        out_shape = self.compute_output_shape(input_shape)
+        self.n_parallel = None if None in out_shape[1:] else prod(out_shape[1:-1])
+        if self.parallelization_factor <= 0:
+            assert self.n_parallel is not None
+            self.parallelization_factor = self.n_parallel
+
+    def convolution_op(self, x_nhwc, kernel_hwio):
+        x = x_nhwc.permute(0, 3, 1, 2)
+        w = kernel_hwio.permute(3, 2, 0, 1)
+        if self.padding == 'same':
+            pads = []
+            for d in (1, 0):  # F.pad wants the last dimension first
+                n, k, s, dil = x.shape[2 + d], self.kernel_size[d], self.strides[d], self.dilation_rate[d]
+                total = max((-(-n // s) - 1) * s + dil * (k - 1) + 1 - n, 0)
+                pads += [total // 2, total - total // 2]
+            x = F.pad(x, pads)
+        y = F.conv2d(x, w, None, self.strides, 0, self.dilation_rate)
+        return y.permute(0, 2, 3, 1)
+
+    def call(self, inputs, training=None):
+        if self.enable_iq:
+            inputs = self.iq(inputs, training=training)
+        outputs = self.convolution_op(inputs, self.qkernel)
+        if self.use_bias:
+            outputs = outputs + self.qbias.reshape(1, 1, 1, self.filters)
+        if self.activation is not None:
+            outputs = self.activation(outputs)
+        return outputs
+
+    def _compute_ebops(self, shape):
+        bw_inp = self.iq.bits_(shape)
+        bw_ker = self.kq.bits_(self._kernel.shape)
+        ebops = torch.sum(self.convolution_op(bw_inp, bw_ker))
+        ebops = ebops * (self.parallelization_factor / self.n_parallel)
+        if self.bq is not None:
+            size = float(prod(shape[:-1]) * self.filters)
+            bw_bias = self.bq.bits_(self.bias.shape)
+            ebops = ebops + torch.mean(bw_bias) * size
+        return ebops
+
+    @property
+    def qkernel(self):
+        return self.kq(self._kernel)
+
+    @property
+    def qbias(self):
+        if self.bias is None:
+            return None
+        return self.bq(self.bias)

@@ -1,0 +1,109 @@
+"""QEinsumDenseBatchnorm (reference src/hgq/layers/einsum_dense_batchnorm.py:11-211): batch
+normalisation folded into the kernel and bias *before* they are quantized.  In training the
+moments come from an un-quantized-kernel contraction of the quantized input, so each step runs
+two contractions."""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..core import epsilon, get_initializer
+from .core.einsum_dense import QEinsumDense, analyze_einsum_string
+
+
+class QEinsumDenseBatchnorm(QEinsumDense):
+    def __init__(self, equation, output_shape, activation=None, bias_axes=None, normalize_axes: str | None = None,
+                 momentum=0.99, epsilon=1e-3, center=True, scale=True, beta_initializer='zeros',
+                 gamma_initializer='ones', moving_mean_initializer='zeros', moving_variance_initializer='ones',
+                 beta_regularizer=None, gamma_regularizer=None, beta_constraint=None, gamma_constraint=None,
+                 synchronized=False, **kwargs):
+        super().__init__(equation=equation, output_shape=output_shape, activation=activation, bias_axes=bias_axes, **kwargs)
+        self.synchronized = synchronized
+        self.momentum = float(momentum)
+        self.epsilon = float(epsilon)  # stored only: the fusion uses the global epsilon, as the reference does (:165)
+        self.center = center
+        self.scale = scale
+        self.gamma_initializer = get_initializer(gamma_initializer)
+        self.moving_mean_initializer = get_initializer(moving_mean_initializer)
+        self.moving_variance_initializer = get_initializer(moving_variance_initializer)
+        self.gamma_regularizer, self.gamma_constraint = gamma_regularizer, gamma_constraint
+        normalize_axes = normalize_axes or bias_axes
+        assert normalize_axes is not None, 'Either normalize_axes or bias_axes must be provided.'
+        self.normalize_axes = normalize_axes
+        self._check_normalize_axes()
+
+    def _check_normalize_axes(self):
+        kernel_axes, output_axes = self.equation.split(',')[1].split('->')
+        for c in self.normalize_axes:
+            if c not in kernel_axes:
+                raise ValueError(f'Axis {c} not found in kernel axes {kernel_axes}')
+            if c not in output_axes:
+                raise ValueError(f'Axis {c} not found in output axes {output_axes}')
+            if self.bias_axes and c not in self.bias_axes:
+                raise ValueError(f'Axis {c} not found in bias axes {self.bias_axes}')
+
+    def _compute_fused_einsum_specs(self, input_shape):
+        kernel_axes, output_axes = self.equation.split(',')[1].split('->')
+        _, norm_cast_shape, output_shape = analyze_einsum_string(self.equation, self.normalize_axes, tuple(input_shape),
+                                                                 self.partial_output_shape)
+        normalize_axes = ''.join(c for c in kernel_axes if c in self.normalize_axes)
+        self._reduction_axes = tuple(i for i, c in enumerate(output_axes) if c not in normalize_axes)
+        norm_shape = tuple(output_shape[i] for i, c in enumerate(output_axes) if c in normalize_axes)
+        assert np.prod(norm_shape) == np.prod(norm_cast_shape), f'{norm_shape} != {norm_cast_shape}'
+        self._norm_offset_cast_shape = norm_cast_shape
+        self.fused_kernel_equation = f'{kernel_axes},{normalize_axes}->{kernel_axes}'
+        return norm_shape
+
+    def build(self, input_shape):
+        super().build(input_shape)
+        norm_shape = self._compute_fused_einsum_specs(input_shape)
+        if self.scale:
+            self.bn_gamma = self.add_weight(shape=norm_shape, name='gamma', initializer=self.gamma_initializer,
+                                            regularizer=self.gamma_regularizer, constraint=self.gamma_constraint)
+        assert self.bias is not None
+        self.bias.requires_grad_(bool(self.center))
+        self.moving_mean = self.add_weight(shape=norm_shape, name='moving_mean', initializer=self.moving_mean_initializer,
+                                           trainable=False)
+        self.moving_variance = self.add_weight(shape=norm_shape, name='moving_variance',
+                                               initializer=self.moving_variance_initializer, trainable=False)
+
+    def get_fused_qkernel_and_qbias(self, training, mean, var):
+        bn_gamma = self.bn_gamma if self.scale else 1
+        scaler = bn_gamma / torch.sqrt(var + epsilon())
+        fused_kernel = torch.einsum(self.fused_kernel_equation, self._kernel, scaler)
+        fused_qkernel = self.kq(fused_kernel, training=training)
+        offset = torch.reshape(-mean * scaler, self._norm_offset_cast_shape)
+        fused_qbias = self.bq(self.bias + offset, training=training)
+        return fused_qkernel, fused_qbias
+
+    @property
+    def qkernel(self):
+        return self.get_fused_qkernel_and_qbias(False, self.moving_mean, self.moving_variance)[0]
+
+    @property
+    def qbias(self):
+        return self.get_fused_qkernel_and_qbias(False, self.moving_mean, self.moving_variance)[1]
+
+    def call(self, inputs, training=None):
+        if self.enable_iq:
+            inputs = self.iq(inputs, training=training)
+        if training and self.trainable:
+            x = torch.einsum(self.equation, inputs, self._kernel)
+            mean = torch.mean(x, dim=self._reduction_axes)
+            var = torch.mean(torch.square(x), dim=self._reduction_axes) - torch.square(mean)
+            with torch.no_grad():
+                self.moving_mean.copy_(self.moving_mean * self.momentum + mean * (1.0 - self.momentum))
+                self.moving_variance.copy_(self.moving_variance * self.momentum + var * (1.0 - self.momentum))
+        else:
+            var, mean = self.moving_variance, self.moving_mean
+        qkernel, qbias = self.get_fused_qkernel_and_qbias(training, mean, var)
+        # the input is already quantized: contract without the fused input quantizer
+        enable_iq, self._enable_iq = self._enable_iq, False
+        try:
+            y, act_done = self._contract(inputs, qkernel, qbias, training)
+        finally:
+            self._enable_iq = enable_iq
+        if self.activation is not None and not act_done:
+            y = self.activation(y)
+        return y

@@ -167,8 +167,7 @@ def _(dy, y, x, f_in, qw, has_bias, act, mode, bw_rows):
             x.new_empty(bw_rows * x.shape[1]))
 
 
-@torch.library.custom_op('hgq::dense_ebops', mutates_args=('i_in', 'ebops_var'))
-def dense_ebops_op(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor,
+def _dense_ebops_impl(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor,
                    b_ker: Tensor, k_bias: Tensor, b_bias: Tensor, ebops_var: Tensor, P: int, K: int, N: int, scale: float,
                    bias_size: float, mode_in: int, mode_ker: int, mode_bias: int) -> tuple[Tensor, Tensor, Tensor]:
     """Returns (ebops, ebops*beta, [g_f_in | g_b_ker | g_b_bias] in one buffer); with ``beta`` the
@@ -201,6 +200,12 @@ def dense_ebops_op(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_in:
                                      _ptr(g_f), _ptr(g_bk), _ptr(g_bb), _stream())
     _lib.check(rc, 'hgq_dense_ebops')
     return ebops, term, g
+
+
+# Two registrations of the same launch: the tracking form updates the input quantizer's integer
+# bits in place (and is declared so), the plain form leaves them alone.
+dense_ebops_track_op = torch.library.custom_op('hgq::dense_ebops_track', _dense_ebops_impl, mutates_args=('i_in', 'ebops_var'))
+dense_ebops_op = torch.library.custom_op('hgq::dense_ebops', _dense_ebops_impl, mutates_args=('ebops_var',))
 
 
 @torch.library.custom_op('hgq::sparse_ce', mutates_args=())
@@ -323,7 +328,8 @@ class _DenseEbops(torch.autograd.Function):
     @staticmethod
     def forward(ctx, i_in, f_in, b_ker, b_bias, amax, decay, beta, k_in, k_ker, k_bias, ebops_var, P, K, N, scale, bias_size,
                 mode_in, mode_ker, mode_bias):
-        ebops, term, g = dense_ebops_op(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N,
+        op = dense_ebops_track_op if amax.numel() else dense_ebops_op
+        ebops, term, g = op(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N,
                                         scale, bias_size, mode_in, mode_ker, mode_bias)
         ctx.save_for_backward(g)
         ctx.has_beta = beta.numel() > 0

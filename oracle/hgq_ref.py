@@ -512,6 +512,247 @@ class RefQEinsumDense(RefQLayer):
         return ebops * self.parallelization_factor / self.n_parallel
 
 
+class RefQEinsumDenseBatchnorm(RefQEinsumDense):
+    """src/hgq/layers/einsum_dense_batchnorm.py:11-211.  ``moments`` is restated as Keras' torch
+    backend computes it: mean, and mean(x**2) - mean**2 (biased variance)."""
+
+    def __init__(self, *args, gamma, moving_mean, moving_variance, normalize_axes, momentum=0.99, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.gamma = None if gamma is None else gamma.detach().clone().requires_grad_(True)
+        self.moving_mean = moving_mean.detach().clone()
+        self.moving_variance = moving_variance.detach().clone()
+        self.momentum = momentum
+        kernel_axes, output_axes = self.equation.split(',')[1].split('->')
+        norm = ''.join(c for c in kernel_axes if c in normalize_axes)
+        self.reduction_axes = tuple(i for i, c in enumerate(output_axes) if c not in norm)
+        self.fused_kernel_equation = f'{kernel_axes},{norm}->{kernel_axes}'
+        first = min(output_axes.find(c) for c in normalize_axes)
+        self.norm_axes_spec = output_axes[first:]
+        self.normalize_axes = normalize_axes
+
+    def weights(self):
+        return super().weights() + ([self.gamma] if self.gamma is not None else [])
+
+    def fused(self, training, mean, var):
+        gamma = self.gamma if self.gamma is not None else 1
+        scaler = gamma / torch.sqrt(var + EPSILON)
+        fused_kernel = torch.einsum(self.fused_kernel_equation, self.kernel, scaler)
+        qkernel = self.kq(fused_kernel, training=training)
+        offset = torch.reshape(-mean * scaler, self.bias.shape)
+        qbias = self.bq(self.bias + offset, training=training)
+        return qkernel, qbias
+
+    def call(self, x, training=None):
+        if self.iq is not None:
+            x = self.iq(x, training=training)
+        if training:
+            z = torch.einsum(self.equation, x, self.kernel)
+            mean = torch.mean(z, dim=self.reduction_axes)
+            var = torch.mean(torch.square(z), dim=self.reduction_axes) - torch.square(mean)
+            with torch.no_grad():
+                self.moving_mean.copy_(self.moving_mean * self.momentum + mean * (1.0 - self.momentum))
+                self.moving_variance.copy_(self.moving_variance * self.momentum + var * (1.0 - self.momentum))
+        else:
+            var, mean = self.moving_variance, self.moving_mean
+        qkernel, qbias = self.fused(training, mean, var)
+        y = torch.einsum(self.equation, x, qkernel) + qbias
+        if self.activation == 'relu':
+            y = torch.relu(y)
+        return y
+
+
+class RefQUnaryFunctionLUT(RefQLayer):
+    """src/hgq/layers/activation.py:18-67."""
+
+    def __init__(self, fn, iq, oq, beta0=1e-5, enable_ebops=True):
+        self._init_common(beta0, enable_ebops)
+        self.fn, self.iq, self.oq = fn, iq, oq
+
+    def weights(self):
+        return []
+
+    def quantizers(self):
+        return [q for q in (self.iq, self.oq) if q is not None]
+
+    def call(self, x, training=None):
+        if self.iq is not None:
+            x = self.iq(x, training=training)
+        return self.fn(x)
+
+    def _compute_ebops(self, shape):
+        bw_inp = self.iq.bits_(shape)
+        bw_out = self.oq.bits_(shape)
+        return torch.sum((2.0**bw_inp) * bw_out) * 1e-4
+
+
+class RefQSoftmax(RefQLayer):
+    """src/hgq/layers/softmax.py:13-161 (stable form)."""
+
+    def __init__(self, axes, exp_table, inv_table, oq, iq=None, input_scaler=1.0, beta0=1e-5, enable_ebops=True,
+                 parallelization_factor=-1):
+        self._init_common(beta0, enable_ebops)
+        self.axes = tuple(axes)
+        self.exp_table, self.inv_table, self.oq, self.iq = exp_table, inv_table, oq, iq
+        self.input_scaler = input_scaler
+        self.parallelization_factor = parallelization_factor
+
+    def weights(self):
+        return []
+
+    def quantizers(self):
+        return [q for q in (self.iq, self.oq) if q is not None] + self.exp_table.quantizers() + self.inv_table.quantizers()
+
+    def __call__(self, x, training=None, mask=None):
+        self._mask = mask
+        return super().__call__(x, training=training)
+
+    def call(self, x, training=None):
+        mask = self._mask
+        if self.iq is not None:
+            x = self.iq(x, training=training)
+        if mask is not None:
+            mask = mask.to(x.dtype)
+            x = mask * x - (1 - mask) * 1e9
+        x = torch.amax(x, dim=self.axes, keepdim=True) - x
+        e = self.exp_table(x, training=training)
+        if mask is not None:
+            e = mask * e
+        s = torch.sum(e, dim=self.axes, keepdim=True)
+        return e * self.inv_table(s, training=training)
+
+    def extra_loss(self):
+        return super().extra_loss() + sum(t for t in self.exp_table.losses) + sum(t for t in self.inv_table.losses)
+
+    def _compute_ebops(self, shape):
+        accum_shape = tuple(1 if i in self.axes else s for i, s in enumerate(shape))
+        max_instance = prod(accum_shape)
+        n_instance = self.parallelization_factor if self.parallelization_factor > 0 else max_instance
+        factor = n_instance / max_instance
+        inp_bits = self.iq.bits_(shape) if self.iq is not None else 0
+        exp_bits = self.exp_table.oq.bits_(shape)
+        inv_bits = self.inv_table.oq.bits_(accum_shape)
+        sub = torch.sum(inp_bits) if self.iq is not None else torch.sum(self.exp_table.iq.bits_(shape))
+        accum = torch.sum(exp_bits) - torch.sum(torch.amin(exp_bits, dim=self.axes))
+        mult = torch.sum(exp_bits * inv_bits)
+        return (sub + accum + mult) * factor
+
+
+class RefQMultiHeadAttention(RefQLayer):
+    """src/hgq/layers/attn/mha.py:27-537 for rank-3 inputs; einsum strings as Keras builds them."""
+
+    def __init__(self, query_dense, key_dense, value_dense, output_dense, softmax, beta0=1e-5, enable_ebops=True,
+                 parallelization_factor=-1):
+        self._init_common(beta0, enable_ebops)
+        self.qd, self.kd, self.vd, self.od, self.softmax = query_dense, key_dense, value_dense, output_dense, softmax
+        self.parallelization_factor = parallelization_factor
+
+    def sublayers(self):
+        return [self.qd, self.kd, self.vd, self.softmax, self.softmax.exp_table, self.softmax.inv_table, self.od]
+
+    def weights(self):
+        return [w for l in (self.qd, self.kd, self.vd, self.od) for w in l.weights()]
+
+    def quantizers(self):
+        seen, out = set(), []
+        for l in (self.qd, self.kd, self.vd, self.od, self.softmax):
+            for q in l.quantizers():
+                if id(q) not in seen:
+                    seen.add(id(q))
+                    out.append(q)
+        return out
+
+    def call(self, x, training=None, mask=None):
+        q = self.qd(x, training=training)
+        k = self.kd(x, training=training)
+        v = self.vd(x, training=training)
+        scores = torch.einsum('aecd,abcd->acbe', k, q * 1.0)
+        m = None if mask is None else mask.unsqueeze(1)
+        scores = self.softmax(scores, training=training, mask=m)
+        out = torch.einsum('acbe,aecd->abcd', scores, v)
+        self._shapes = (q.shape, k.shape, v.shape, scores.shape)
+        return self.od(out, training=training)
+
+    def __call__(self, x, training=None, mask=None):
+        self.losses = []
+        r = self.call(x, training=training, mask=mask)
+        if training and self.enable_ebops:
+            ebops = self._compute_ebops()
+            self.ebops_value = ebops.detach().to(torch.int64)
+            self.losses.append(ebops * self.beta)
+        return r
+
+    def extra_loss(self):
+        loss = 0.0
+        for term in self.losses:
+            loss = loss + term
+        for l in (self.qd, self.kd, self.vd, self.od, self.softmax, self.softmax.exp_table, self.softmax.inv_table):
+            for term in l.losses:
+                loss = loss + term
+        for q in self.quantizers():
+            loss = loss + q.quantizer.regularization_loss()
+        return loss
+
+    def _compute_ebops(self):
+        qs, ks, vs, ss = ((1,) + tuple(s[1:]) for s in self._shapes)
+        bw_q, bw_k, bw_v = self.qd.oq.bits_(qs), self.kd.oq.bits_(ks), self.vd.oq.bits_(vs)
+        bw_attn = self.softmax.oq.bits_(ss)
+        ebops = torch.einsum('aecd,abcd->', bw_k, bw_q) + torch.einsum('acbe,aecd->', bw_attn, bw_v)
+        if self.parallelization_factor > 0:
+            return ebops * self.parallelization_factor
+        return ebops
+
+
+class RefQConv2D(RefQLayer):
+    """src/hgq/layers/conv.py:12-102: channels-last input, HWIO kernel, 'valid' or 'same' padding."""
+
+    def __init__(self, kernel, bias, iq, kq, bq, strides=(1, 1), padding='valid', activation=None, beta0=1e-5,
+                 enable_ebops=True, parallelization_factor=-1, n_parallel=1, oq=None):
+        self._init_common(beta0, enable_ebops and iq is not None)
+        self.kernel = kernel.detach().clone().requires_grad_(True)
+        self.bias = None if bias is None else bias.detach().clone().requires_grad_(True)
+        self.iq, self.kq, self.bq, self.oq = iq, kq, bq, oq
+        self.strides, self.padding, self.activation = tuple(strides), padding, activation
+        self.n_parallel = n_parallel
+        self.parallelization_factor = parallelization_factor if parallelization_factor > 0 else n_parallel
+
+    def weights(self):
+        return [w for w in (self.kernel, self.bias) if w is not None]
+
+    def quantizers(self):
+        return [q for q in (self.iq, self.kq, self.bq, self.oq) if q is not None]
+
+    def conv(self, x, w):
+        x = x.permute(0, 3, 1, 2)
+        w = w.permute(3, 2, 0, 1)
+        if self.padding == 'same':
+            pads = []
+            for d in (1, 0):
+                n, k, st = x.shape[2 + d], w.shape[2 + d], self.strides[d]
+                total = max((-(-n // st) - 1) * st + k - n, 0)
+                pads += [total // 2, total - total // 2]
+            x = F.pad(x, pads)
+        return F.conv2d(x, w, None, self.strides).permute(0, 2, 3, 1)
+
+    def call(self, x, training=None):
+        if self.iq is not None:
+            x = self.iq(x, training=training)
+        y = self.conv(x, self.kq(self.kernel, training=training))
+        if self.bias is not None:
+            y = y + self.bq(self.bias, training=training).reshape(1, 1, 1, -1)
+        if self.activation == 'relu':
+            y = torch.relu(y)
+        return y
+
+    def _compute_ebops(self, shape):
+        bw_inp = self.iq.bits_(shape)
+        bw_ker = self.kq.bits_(self.kernel.shape)
+        ebops = torch.sum(self.conv(bw_inp, bw_ker)) * (self.parallelization_factor / self.n_parallel)
+        if self.bq is not None:
+            size = float(prod(shape[:-1]) * self.kernel.shape[-1])
+            ebops = ebops + torch.mean(self.bq.bits_(self.bias.shape)) * size
+        return ebops
+
+
 # --------------------------------------------------------------------------------------
 # the QDense-MLP training step (reference call stack: tests/base.py:302-321 and README.md:57-67)
 # --------------------------------------------------------------------------------------
