@@ -122,7 +122,9 @@ def main():
     ap.add_argument('--steps', type=int, default=300)
     ap.add_argument('--warmup', type=int, default=30)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--eager', action='store_true', help='time eager steps instead of HIP-graph replays')
+    ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused-graph',
+                    help='fused: whole-step kernels (3 launches); layers: per-layer torch.library operators with autograd; '
+                         '-graph: the step is captured once in a HIP graph and replayed')
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported', file=sys.stderr)
@@ -131,7 +133,7 @@ def main():
     import torch
 
     from hgq2_amd import ops
-    from hgq2_amd.train import SGD, GraphedTrainStep, model_loss
+    from hgq2_amd.train import SGD, FusedQDenseStack, GraphedTrainStep, model_loss
     from hgq2_amd.utils.models import qdense_mlp
 
     dev = torch.device('cuda:0')
@@ -143,15 +145,35 @@ def main():
     model = qdense_mlp(DIMS, beta0=1e-5, device=dev)
     opt = SGD(model.parameters(), lr=0.01, fold_regularizers=True)
 
-    if args.eager:
+    if args.path == 'layers-eager':
         def step():
             opt.zero_grad()
             loss = model_loss(model, ops.sparse_ce(model(x, training=True), labels), True)
             loss.backward()
             opt.step()
             return loss
-    else:
+    elif args.path == 'layers-graph':
         step = GraphedTrainStep(model, ops.sparse_ce, opt, x, labels, warmup=3)
+    else:
+        fused = FusedQDenseStack(model, lr=0.01)
+        if args.path == 'fused':
+            def step():
+                return fused.step(x, labels)
+        else:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    fused.step(x, labels)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fused.step(x, labels)
+
+            def step():
+                graph.replay()
+                return fused.loss
 
     for _ in range(args.warmup):
         step()
@@ -176,7 +198,9 @@ def main():
         'data': 'synthetic',
         'config': {'workload': 'QDense MLP 16-64-32-32-5 (ReLU hidden, linear out), batch 16384, kbi SAT_SYM weights, '
                                'kif WRAP datalanes, EBOPs beta0=1e-5, sparse CE, one fwd+bwd+SGD step'
-                               + (' (eager launches)' if args.eager else ' (HIP-graph replay)')},
+                               + {'fused': ' (whole-step kernels, 3 launches)', 'fused-graph': ' (whole-step kernels, HIP-graph replay)',
+                                  'layers-graph': ' (per-layer operators + autograd, HIP-graph replay)',
+                                  'layers-eager': ' (per-layer operators + autograd, eager launches)'}[args.path]},
         'final_loss': float(loss),
         'roofline': roofline,
         'quantizer_kernels': qr,

@@ -7,6 +7,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stdint.h>
 
 #include "../../include/hgq_hip.h"
@@ -125,6 +126,42 @@ __device__ __forceinline__ void quantize_grad(float x, float dy, const KIF &p, f
 // Bit pattern of |v| as an unsigned integer: monotone for non-negative floats, so an integer
 // atomic max is a float max.  NaN payloads compare above every finite value and propagate.
 __device__ __forceinline__ uint32_t abs_bits(float v) { return __float_as_uint(v) & 0x7fffffffu; }
+
+
+// Runtime-mode forms (for kernels that serve several quantizers with different modes at once).
+__device__ __forceinline__ float fixed_round_dyn(float x, float f, int rm) {
+    return rm == HGQ_TRN ? fixed_round<HGQ_TRN>(x, f) : rm == HGQ_RND ? fixed_round<HGQ_RND>(x, f) : fixed_round<HGQ_RND_CONV>(x, f);
+}
+
+__device__ __forceinline__ float quantize_dyn(float x, const KIF &p, int rm, int om, bool training) {
+    const float xq = fixed_round_dyn(x, p.f, rm);
+    int st;
+    float y = om == HGQ_WRAP ? overflow<HGQ_WRAP>(xq, p, training, st)
+              : om == HGQ_SAT ? overflow<HGQ_SAT>(xq, p, training, st) : overflow<HGQ_SAT_SYM>(xq, p, training, st);
+    if (!training && !(p.k + p.i + p.f > 0.0f)) y = 0.0f;
+    return y;
+}
+
+__device__ __forceinline__ void quantize_grad_dyn(float x, float dy, const KIF &p, int rm, int om, float &dx, float &di, float &df) {
+#define HGQ_QG(RMV, OMV) quantize_grad<RMV, OMV>(x, dy, p, dx, di, df)
+    if (om == HGQ_WRAP) {
+        if (rm == HGQ_TRN) HGQ_QG(HGQ_TRN, HGQ_WRAP); else if (rm == HGQ_RND) HGQ_QG(HGQ_RND, HGQ_WRAP); else HGQ_QG(HGQ_RND_CONV, HGQ_WRAP);
+    } else if (om == HGQ_SAT) {
+        if (rm == HGQ_TRN) HGQ_QG(HGQ_TRN, HGQ_SAT); else if (rm == HGQ_RND) HGQ_QG(HGQ_RND, HGQ_SAT); else HGQ_QG(HGQ_RND_CONV, HGQ_SAT);
+    } else {
+        if (rm == HGQ_TRN) HGQ_QG(HGQ_TRN, HGQ_SAT_SYM); else if (rm == HGQ_RND) HGQ_QG(HGQ_RND, HGQ_SAT_SYM); else HGQ_QG(HGQ_RND_CONV, HGQ_SAT_SYM);
+    }
+#undef HGQ_QG
+}
+
+// ceil(log2(v)) for v > 0 from the exponent field: exact, where log2f is only faithfully rounded.
+__device__ __forceinline__ float ceil_log2_exact(float v) {
+    if (!(v > 0.0f)) return v == 0.0f ? -INFINITY : NAN;
+    if (!(v < INFINITY)) return v;
+    int e;
+    const float mant = frexpf(v, &e);  // v = mant * 2**e, mant in [0.5, 1)
+    return (float)(mant == 0.5f ? e - 1 : e);
+}
 
 }  // namespace hgq
 

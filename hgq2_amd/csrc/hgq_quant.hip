@@ -371,15 +371,6 @@ __global__ __launch_bounds__(256) void quant_bwd_generic(const float *__restrict
 // ------------------------------------------------------------------------------------------
 // integer-bit tracking
 // ------------------------------------------------------------------------------------------
-// ceil(log2(v)) for v > 0 from the exponent field: exact, where log2f is only faithfully rounded.
-__device__ __forceinline__ float ceil_log2(float v) {
-    if (!(v > 0.0f)) return v == 0.0f ? -INFINITY : NAN;
-    if (!(v < INFINITY)) return v;
-    int e;
-    const float mant = frexpf(v, &e);  // v = mant * 2**e, mant in [0.5, 1)
-    return (float)(mant == 0.5f ? e - 1 : e);
-}
-
 // 256 threads = 64 entries x 4 slice groups: the abs-max / any-negative trackers arrive as
 // `n_parts` slices of [n] (one per producing workgroup) and are combined here.
 __global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__restrict__ amax,
@@ -425,7 +416,7 @@ __global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__res
     float mi;
     if (!m.kbi) {
         const float f = rintf(fb[t]);
-        mi = ceil_log2(__fadd_rn(xr, pow2(-f)));
+        mi = ceil_log2_exact(__fadd_rn(xr, pow2(-f)));
     } else {
         const float b = rintf(fb[t]);
         const float eps = 1e-7f;

@@ -36,15 +36,6 @@ __device__ __forceinline__ float entry_bits(const void *k, const float *i, const
 
 #define HGQ_EBOPS_MAXK 4096
 
-// ceil(log2(v)) for v > 0 from the exponent field (exact).
-__device__ __forceinline__ float ceil_log2_exact(float v) {
-    if (!(v > 0.0f)) return v == 0.0f ? -INFINITY : NAN;
-    if (!(v < INFINITY)) return v;
-    int e;
-    const float mant = frexpf(v, &e);
-    return (float)(mant == 0.5f ? e - 1 : e);
-}
-
 __global__ __launch_bounds__(256) void dense_ebops_kernel(const uint32_t *amax_part, int n_parts, float decay,
                                                           const float *beta, float *loss_term,
                                                           const void *k_in, float *i_in, const float *f_in,

@@ -111,3 +111,103 @@ class GraphedTrainStep:
             self.y.copy_(y)
         self.graph.replay()
         return self.loss
+
+
+class FusedQDenseStack:
+    """One SGD training step of a stack of :class:`QDense` layers with mean sparse categorical
+    cross-entropy, executed by the whole-step kernels (three launches, see ``hgq_mlp_train_step``).
+
+    It updates exactly the variables the layer-by-layer path updates (kernels, biases, every
+    bit-width variable, the tracked integer bits, ``ebops``) with the same arithmetic; it exists
+    because at these layer sizes a step made of per-layer launches is bound by launch latency.
+    Requirements (checked): 2-D inputs, widths up to 64, plain KIF/WRAP input quantizers with
+    batch-shared bit-widths, plain KBI SAT / SAT_SYM kernel and bias quantizers, relu or linear
+    activations, no kernel / bias regularizers or constraints, MonoL1 or no regularizer and clip
+    constraints on the bit-widths.
+    """
+
+    def __init__(self, layers, lr: float = 0.01):
+        import ctypes
+
+        from . import _lib
+        from .layers import QDense
+        from .quantizer.internal import FixedPointQuantizerKBI, FixedPointQuantizerKIF
+        from .regularizers import MonoL1 as _L1
+
+        layers = list(getattr(layers, 'layers', layers))
+        if not layers or not all(isinstance(layer, QDense) and layer.built for layer in layers):
+            raise ValueError('FusedQDenseStack needs a non-empty sequence of built QDense layers')
+        self.layers, self.lr = layers, float(lr)
+        self._lib, self._ct = _lib, ctypes
+        arr = (_lib.MlpLayer * len(layers))()
+        inf = float('inf')
+
+        def var_params(p):
+            r, c = getattr(p, 'regularizer', None), getattr(p, 'constraint', None)
+            if r is not None and not isinstance(r, _L1):
+                raise ValueError('only MonoL1 regularizers can be folded into the fused update')
+            b = c.bounds() if c is not None else (-inf, inf)
+            if b is None:
+                raise ValueError('only clip-type constraints can be folded into the fused update')
+            return (r.l1 if (r is not None and p.requires_grad) else 0.0), b[0], b[1]
+
+        ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+        for n, layer in enumerate(layers):
+            qi = layer.iq.quantizer if layer.enable_iq else None
+            qk, qb = layer.kq.quantizer, (layer.bq.quantizer if layer.bq is not None else None)
+            ok = (qi is not None and layer.iq.plain and isinstance(qi, FixedPointQuantizerKIF) and qi.overflow_mode == 'WRAP'
+                  and qi.trainable and tuple(qi._i.shape) == (1, layer._kernel.shape[0])
+                  and layer.kq.plain and isinstance(qk, FixedPointQuantizerKBI) and qk.overflow_mode != 'WRAP'
+                  and (qb is None or (layer.bq.plain and isinstance(qb, FixedPointQuantizerKBI) and qb.overflow_mode != 'WRAP'))
+                  and layer._act_name in ('relu', 'linear') and not layer.enable_oq
+                  and all(getattr(p, 'regularizer', None) is None and getattr(p, 'constraint', None) is None
+                          for p in (layer._kernel, layer.bias) if p is not None))
+            if not ok:
+                raise ValueError(f'layer {n} ({layer.name}) is outside what the fused QDense step covers')
+            it = arr[n]
+            it.K, it.N = layer._kernel.shape
+            it.act = _lib.ACT_RELU if layer._act_name == 'relu' else _lib.ACT_NONE
+            km = lambda q: q._mode(True) | _lib.MODE_K_U8  # noqa: E731  (`_k` variables are uint8)
+            it.mode_in, it.mode_ker, it.mode_bias = km(qi), km(qk), (km(qb) if qb is not None else 0)
+            it.w, it.bias = ptr(layer._kernel), ptr(layer.bias)
+            it.k_in, it.i_in, it.f_in = ptr(qi._k), ptr(qi._i), ptr(qi._f)
+            it.k_ker, it.b_ker, it.i_ker = ptr(qk._k), ptr(qk._b), ptr(qk._i)
+            if qb is not None:
+                it.k_bias, it.b_bias, it.i_bias = ptr(qb._k), ptr(qb._b), ptr(qb._i)
+            it.decay = qi._decay_host
+            if layer.enable_ebops:
+                it.beta, it.ebops = ptr(layer._beta), ptr(layer._ebops)
+            it.ebops_scale = layer.parallelization_factor / layer.n_parallel * layer.ebops_factor
+            it.bias_size = float(layer.units)
+            it.f_in_l1, it.f_in_lo, it.f_in_hi = var_params(qi._f)
+            it.b_ker_l1, it.b_ker_lo, it.b_ker_hi = var_params(qk._b)
+            it.i_ker_l1, it.i_ker_lo, it.i_ker_hi = var_params(qk._i)
+            it.train_i_ker = int(qk._i.requires_grad)
+            if qb is not None:
+                it.b_bias_l1, it.b_bias_lo, it.b_bias_hi = var_params(qb._b)
+                it.i_bias_l1, it.i_bias_lo, it.i_bias_hi = var_params(qb._i)
+                it.train_i_bias = int(qb._i.requires_grad)
+        self._arr = arr
+        self._ws = None
+        self.device = layers[0]._kernel.device
+        self.loss = torch.zeros((), dtype=torch.float32, device=self.device)
+
+    def step(self, x, labels):
+        """Run one training step in place; returns the loss tensor (cross-entropy + sum of EBOPs * beta
+        + MonoL1 regularisation terms, i.e. the full training loss)."""
+        ct, lib = self._ct, self._lib.load()
+        if not (x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == self._arr[0].K):
+            raise ValueError('x must be a contiguous float32 GPU tensor [rows, K]')
+        if not (labels.is_cuda and labels.dtype == torch.int64 and labels.is_contiguous() and labels.shape == (x.shape[0],)):
+            raise ValueError('labels must be a contiguous int64 GPU tensor [rows]')
+        rows = x.shape[0]
+        need = lib.hgq_mlp_workspace(self._arr, len(self.layers), rows)
+        if need < 0:
+            self._lib.check(-3, 'hgq_mlp_workspace')
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.empty(need, dtype=torch.float32, device=self.device)
+        rc = lib.hgq_mlp_train_step(self._arr, len(self.layers), ct.c_void_p(x.data_ptr()), ct.c_void_p(labels.data_ptr()), rows,
+                                    self.lr, ct.c_void_p(self.loss.data_ptr()), ct.c_void_p(self._ws.data_ptr()),
+                                    ct.c_void_p(torch.cuda.current_stream().cuda_stream))
+        self._lib.check(rc, 'hgq_mlp_train_step')
+        return self.loss

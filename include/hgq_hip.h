@@ -190,6 +190,48 @@ typedef struct {
 } hgq_sgd_item;
 int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *stream);
 
+/*
+ * One training step (forward, mean sparse categorical cross-entropy from logits, backward, SGD)
+ * of a stack of QDense layers in three launches.  It performs, in the same order and with the
+ * same arithmetic, what the per-layer entry points above do when the reference's call stack
+ * (src/hgq/layers/core/base.py:88-110 around src/hgq/layers/core/dense.py:60-80, then the
+ * optimizer and the constraints) is followed layer by layer: input quantizer (KIF, WRAP,
+ * training branch, fixed_point_quantizer.py:401-413) with its integer-bit tracking, kernel / bias
+ * quantizers (KBI, SAT or SAT_SYM), contraction, bias, activation, EBOPs * beta added to the loss
+ * and assigned to `ebops`, MonoL1 gradient, SGD update, clip constraints.
+ *
+ * Limits: up to HGQ_MLP_MAX_LAYERS layers, widths up to 64, bit-widths shared along the batch
+ * axis for inputs and individual per weight.  All variables are updated in place.
+ *   x [rows, layers[0].K];  labels [rows] int64 in [0, layers[n-1].N);
+ *   loss [1] optional: cross-entropy + sum of ebops * beta + the MonoL1 terms of the trainable bit-widths;
+ *   workspace: hgq_mlp_workspace(layers, n_layers, rows) floats.
+ */
+#define HGQ_MLP_MAX_LAYERS 8
+typedef struct {
+    int K, N, act;                    /* input width, output width, HGQ_ACT_* */
+    int mode_in, mode_ker, mode_bias; /* HGQ_MODE(...) | HGQ_MODE_KBI | HGQ_MODE_K_U8 as applicable */
+    float *w, *bias;                  /* kernel [K, N]; bias [N] or NULL */
+    const void *k_in;                 /* input quantizer variables, [K] */
+    float *i_in, *f_in;
+    const void *k_ker;                /* kernel quantizer variables, [K, N] */
+    float *b_ker, *i_ker;
+    const void *k_bias;               /* bias quantizer variables, [N] (NULL without bias) */
+    float *b_bias, *i_bias;
+    float decay;                      /* i_decay_speed of the input quantizer */
+    const float *beta;                /* the layer's beta variable [1] */
+    uint32_t *ebops;                  /* the layer's ebops variable [1] */
+    float ebops_scale;                /* parallelization_factor / n_parallel * ebops_factor */
+    float bias_size;                  /* number of bias additions: prod(shape[:-1]) * N for shape (1, ..., K) */
+    /* MonoL1 coefficient and clip bounds of each trainable bit-width variable (-inf / +inf for none) */
+    float f_in_l1, f_in_lo, f_in_hi;
+    float b_ker_l1, b_ker_lo, b_ker_hi, i_ker_l1, i_ker_lo, i_ker_hi;
+    float b_bias_l1, b_bias_lo, b_bias_hi, i_bias_l1, i_bias_lo, i_bias_hi;
+    int train_i_ker, train_i_bias;    /* integer bits of SAT / SAT_SYM quantizers are trainable */
+} hgq_mlp_layer;
+int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, int64_t rows);
+int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
+                       int64_t rows, float lr, float *loss, float *workspace, void *stream);
+
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
 

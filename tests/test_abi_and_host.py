@@ -1,0 +1,130 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares, the
+ctypes table matches the header, and the host logic (config scopes, bit-width layouts, einsum
+analysis) behaves as the reference's does.  No compute call is made here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, 'include', 'hgq_hip.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(hgq_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from hgq2_amd import _lib
+
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f'{n} is declared in include/hgq_hip.h but not exported'
+        assert n in _lib.SIGNATURES, f'{n} has no ctypes signature'
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.hgq_version() >= 1
+
+
+def test_mode_bits_match_header():
+    from hgq2_amd import _lib
+
+    text = open(os.path.join(ROOT, 'include', 'hgq_hip.h')).read()
+    for name in ('TRAINING', 'KBI', 'ROUND_PARAMS', 'K_U8', 'SYMMETRIC', 'TRACING', 'TRACK_INPUT'):
+        shift = int(re.search(rf'#define HGQ_MODE_{name} \(1 << (\d+)\)', text).group(1))
+        assert getattr(_lib, f'MODE_{name}') == 1 << shift
+    assert _lib.mode_bits('RND', 'SAT_SYM', training=True, kbi=True) == 1 | (2 << 4) | (1 << 8) | (1 << 9)
+    with pytest.raises(ValueError):
+        _lib.mode_bits('RND', 'NOPE')
+
+
+def test_ops_refuse_cpu_tensors():
+    from hgq2_amd import _lib, ops
+
+    x = torch.zeros(8)
+    with pytest.raises(ValueError, match='GPU'):
+        ops.quantize(x, x, x, x, _lib.mode_bits('RND', 'WRAP'))
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from hgq2_amd import _lib
+
+    monkeypatch.setattr(_lib, '_lib', None)
+    monkeypatch.setattr(_lib, 'LIB_PATH', '/nonexistent/libhgq_hip.so')
+    with pytest.raises(_lib.HGQLibraryError, match='no CPU fallback'):
+        _lib.load()
+
+
+def test_quantizer_config_scopes_follow_reference_semantics():
+    from hgq2_amd.config import LayerConfigScope, QuantizerConfig, QuantizerConfigScope, global_config
+    from hgq2_amd.quantizer.config import default_configs, default_q_type
+
+    before = {k: dict(v) for k, v in default_configs.items()}
+    with QuantizerConfigScope(place='all', default_q_type='kbi', overflow_mode='SAT_SYM'):
+        with QuantizerConfigScope(place='datalane', default_q_type='kif', overflow_mode='WRAP'):
+            assert QuantizerConfig('default', 'datalane').q_type == 'kif'
+            assert QuantizerConfig('default', 'datalane')['overflow_mode'] == 'WRAP'
+            assert QuantizerConfig('default', 'bias')['overflow_mode'] == 'SAT_SYM'
+            assert QuantizerConfig('default', 'weight').q_type == 'kbi'
+            assert 'overflow_mode' not in default_configs[('float', 'weight')]
+        assert default_q_type['datalane'] == 'kbi'
+    assert {k: dict(v) for k, v in default_configs.items()} == before
+    assert default_q_type == {'weight': 'kbi', 'datalane': 'kif', 'bias': 'kbi', 'table': 'kbi'}
+    # explicit kwargs beat the scope; unknown keys are rejected; two of (i0, f0, b0) imply the third
+    with QuantizerConfigScope(place='datalane', overflow_mode='WRAP'):
+        assert QuantizerConfig(place='datalane', overflow_mode='SAT')['overflow_mode'] == 'SAT'
+    with pytest.raises(ValueError):
+        QuantizerConfig('kif', 'datalane', b0=3)
+    s = QuantizerConfigScope(i0=2, b0=6)
+    assert s.kwargs['f0'] == 4
+    with LayerConfigScope(beta0=0.5, enable_ebops=False):
+        assert global_config['beta0'] == 0.5 and global_config['enable_ebops'] is False
+    assert global_config['beta0'] == 1e-5 and global_config['enable_ebops'] is True
+    d = default_configs[('kif', 'datalane')]
+    assert (d['k0'], d['i0'], d['f0'], d['i_decay_speed'], d['homogeneous_axis']) == (True, 2, 6, 0.01, (0,))
+    w = default_configs[('kbi', 'weight')]
+    assert (w['b0'], w['i0'], w['overflow_mode'], w['bc'].max_value, w['is_weight']) == (8, 2, 'SAT_SYM', 23.0, True)
+
+
+def test_bitwidth_layouts():
+    from hgq2_amd.quantizer.internal import DefaultBitwidthMapper
+    from hgq2_amd.quantizer.internal.base import bw_layout
+
+    m = DefaultBitwidthMapper(None, (0,))
+    assert m.inference_weight_shape((None, 28, 28, 1)) == (1, 28, 28, 1)
+    m = DefaultBitwidthMapper((), None)
+    assert m.inference_weight_shape((None, 4, 64, 64)) == (1, 1, 1, 1)
+    assert bw_layout((1, 16), (4096, 16)) == (16, 1)
+    assert bw_layout((16, 64), (16, 64)) == (1024, 1)
+    assert bw_layout((1, 1, 1), (33, 5, 8)) == (1, 1)
+    assert bw_layout((1, 6, 1), (50, 6, 4)) == (6, 4)
+    assert bw_layout((1, 4, 64, 64), (2048, 4, 64, 64)) == (16384, 1)
+    assert bw_layout((3, 1, 5), (3, 4, 5)) is None
+
+
+def test_einsum_analysis():
+    from hgq2_amd.layers.core.einsum_dense import _einsum_free0_size, analyze_einsum_string, gemm_form
+
+    assert analyze_einsum_string('abc,cde->abde', 'de', (None, 64, 64), (64, 4, 16)) == ((64, 4, 16), (4, 16), (None, 64, 4, 16))
+    assert analyze_einsum_string('abcd,cde->abe', 'e', (None, 64, 4, 16), (64, 64)) == ((4, 16, 64), (64,), (None, 64, 64))
+    assert analyze_einsum_string('Babc,bcd->Babd', 'ad', (None, 3, 4, 5), (3, 4, 2))[1] == (3, 1, 2)
+    assert gemm_form('bpf,fh->bph') == (1, 1) and gemm_form('abc,cde->abde') == (1, 2)
+    assert gemm_form('abcd,cde->abe') == (2, 1) and gemm_form('Bij,ijk->Bik') is None
+    assert _einsum_free0_size('bpf,fh->bph', (None, 64, 16)) == 64
+    assert _einsum_free0_size('Bij,ijk->Bik', (None, 3, 4)) == 1
+
+
+def test_constraints_and_regularizers():
+    from hgq2_amd.constraints import Constant, Max, Min, MinMax
+    from hgq2_amd.regularizers import MonoL1
+
+    w = torch.tensor([-30.0, 0.5, 30.0])
+    assert MinMax(-24, 24)(w).tolist() == [-24.0, 0.5, 24.0] and MinMax(-24, 24).bounds() == (-24.0, 24.0)
+    assert Min(0)(w).tolist() == [0.0, 0.5, 30.0] and Max(1)(w).tolist() == [-30.0, 0.5, 1.0]
+    assert Constant(2)(w).tolist() == [2.0, 2.0, 2.0]
+    assert float(MonoL1(1e-2)(w)) == pytest.approx(0.005)

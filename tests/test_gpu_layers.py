@@ -141,3 +141,33 @@ def test_graphed_step_equals_eager_steps(dev):
         for le, lg in zip(eager.layers, graphed.layers):
             assert torch.equal(le.iq.quantizer._i, lg.iq.quantizer._i)
             assert int(le.ebops.cpu().view(torch.int32)) == int(lg.ebops.cpu().view(torch.int32))
+
+
+@pytest.mark.parametrize('batch,dims', [(16384, (16, 64, 32, 32, 5)), (1000, (16, 64, 32, 32, 5)), (300, (7, 40, 3))])
+def test_fused_qdense_stack_step_matches_oracle(dev, batch, dims):
+    """The whole-step kernels update every variable as the oracle's layer-by-layer step does."""
+    from hgq2_amd.train import FusedQDenseStack
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(batch, dims[0], generator=g)
+    labels = torch.randint(0, dims[-1], (batch,), generator=g)
+    oracle = ref.RefMLP(dims=dims, seed=3)
+    model = qdense_mlp(dims, device=dev)
+    _copy_mlp(oracle, model, dev)
+    fused = FusedQDenseStack(model, lr=0.01)
+    xd, yd = x.to(dev), labels.to(dev)
+    for step in range(3):
+        want_loss, _ = oracle.train_step(x, labels, lr=0.01)
+        loss = fused.step(xd, yd)
+        assert abs(loss.item() - want_loss.item()) <= 2e-5 * abs(want_loss.item()), f'loss step {step}'
+        for n, (rl, pl) in enumerate(zip(oracle.layers, model.layers)):
+            assert torch.equal(pl.iq.quantizer._i.cpu(), rl.iq.quantizer._i.detach()), f'layer {n} _i step {step}'
+            assert int(pl.ebops.cpu().view(torch.int32)) == int(rl.ebops_value), f'layer {n} ebops step {step}'
+            _close(pl._kernel, rl.kernel, scale=rl.kernel.detach().abs() + 1e-3, what=f'kernel {n}')
+            _close(pl.bias, rl.bias, scale=rl.bias.detach().abs() + 1e-3, what=f'bias {n}')
+            _close(pl.iq.quantizer._f, rl.iq.quantizer._f, scale=rl.iq.quantizer._f.detach().abs() + 1e-3, what=f'iq._f {n}')
+            _close(pl.kq.quantizer._b, rl.kq.quantizer._b, scale=rl.kq.quantizer._b.detach().abs() + 1e-3, what=f'kq._b {n}')
+            _close(pl.kq.quantizer._i, rl.kq.quantizer._i, scale=rl.kq.quantizer._i.detach().abs() + 1e-3, what=f'kq._i {n}')
+            _close(pl.bq.quantizer._b, rl.bq.quantizer._b, scale=rl.bq.quantizer._b.detach().abs() + 1e-3, what=f'bq._b {n}')
+            _close(pl.bq.quantizer._i, rl.bq.quantizer._i, scale=rl.bq.quantizer._i.detach().abs() + 1e-3, what=f'bq._i {n}')
