@@ -45,13 +45,42 @@ __device__ __forceinline__ KIF kbi_entry(const void *k, const float *i, const fl
     return resolve_kif(load_k(k, idx, m.k_u8), i[idx], b[idx], true, true);
 }
 
+// Quantize `count` kernel (or bias) entries into their padded LDS image.  The global loads of a
+// batch of four entries are issued before any of them is used: the prologue is latency-bound.
+__device__ __forceinline__ void stage_quantized(float *dst, int n_lds, int ld, int K, int N, const float *w, const void *kq,
+                                                const float *iq, const float *bq, int mode, int tid) {
+    const Mode m(mode);
+    for (int base = tid; base < n_lds; base += 4 * 256) {
+        float wv[4], kv[4], iv[4], bv[4];
+        bool ok[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int id = base + u * 256;
+            const int k = id / ld, n = id - k * ld;
+            ok[u] = id < n_lds && k < K && n < N;
+            if (ok[u]) {
+                const int64_t e = (int64_t)k * N + n;
+                wv[u] = w[e], kv[u] = load_k(kq, e, m.k_u8), iv[u] = iq[e], bv[u] = bq[e];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int id = base + u * 256;
+            if (id < n_lds)
+                dst[id] = ok[u] ? quantize_dyn(wv[u], resolve_kif(kv[u], iv[u], bv[u], true, true), m.round_mode, m.overflow_mode, true) : 0.f;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ x,
                                                           const int64_t *__restrict__ labels, int64_t rows,
                                                           float *part) {
     extern __shared__ float lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int L = d.n_layers;
-    float *raw = lds + d.off_raw, *rx = lds + d.off_rx, *red = lds + d.off_red;
+    float *raw = lds + d.off_raw, *rx = lds + d.off_rx;
+    float *dfs = lds + d.off_red;                                 // [L][64] fractional-bit gradient sums
+    uint32_t *amx = (uint32_t *)(lds + d.off_red) + 64 * HGQ_MLP_MAX_LAYERS;  // [L][64] abs-max of each layer's quantized input
     float *my = part + (int64_t)blockIdx.x * d.M;
     const int64_t n_tiles = (rows + MLP_BM - 1) / MLP_BM;
     const float inv_rows = 1.0f / (float)rows;
@@ -59,83 +88,76 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
     // ---- prologue: quantize every layer's kernel and bias into LDS (zero padded), round f
     for (int l = 0; l < L; ++l) {
         const MlpLayerDev &ly = d.l[l];
-        const Mode mk(ly.h.mode_ker), mb(ly.h.mode_bias);
-        float *ws = lds + ly.off_w;
-        for (int id = tid; id < ly.Kp * ly.ldw; id += 256) {
-            const int k = id / ly.ldw, n = id - k * ly.ldw;
-            float v = 0.f;
-            if (k < ly.h.K && n < ly.h.N) {
-                const int64_t e = (int64_t)k * ly.h.N + n;
-                v = quantize_dyn(ly.h.w[e], kbi_entry(ly.h.k_ker, ly.h.i_ker, ly.h.b_ker, e, ly.h.mode_ker), mk.round_mode,
-                                 mk.overflow_mode, true);
-            }
-            ws[id] = v;
-        }
-        for (int n = tid; n < ly.Np; n += 256) {
-            float v = 0.f;
-            if (n < ly.h.N && ly.h.bias)
-                v = quantize_dyn(ly.h.bias[n], kbi_entry(ly.h.k_bias, ly.h.i_bias, ly.h.b_bias, n, ly.h.mode_bias), mb.round_mode,
-                                 mb.overflow_mode, true);
-            lds[ly.off_qb + n] = v;
-        }
+        stage_quantized(lds + ly.off_w, ly.Kp * ly.ldw, ly.ldw, ly.h.K, ly.h.N, ly.h.w, ly.h.k_ker, ly.h.i_ker, ly.h.b_ker, ly.h.mode_ker, tid);
+        if (ly.h.bias)
+            stage_quantized(lds + ly.off_qb, ly.Np, ly.Np, 1, ly.h.N, ly.h.bias, ly.h.k_bias, ly.h.i_bias, ly.h.b_bias, ly.h.mode_bias, tid);
+        else
+            for (int n = tid; n < ly.Np; n += 256) lds[ly.off_qb + n] = 0.f;
         for (int k = tid; k < ly.Kp; k += 256) lds[ly.off_f + k] = k < ly.h.K ? rintf(ly.h.f_in[k]) : 0.f;
     }
-    for (int id = tid; id < MLP_BM * d.ld_raw; id += 256) raw[id] = 0.f;
+    for (int id = tid; id < MLP_BM * d.ld_rx; id += 256) rx[id] = 0.f;  // padding columns stay zero for good
+    for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += 256) dfs[id] = 0.f, amx[id] = 0u;
     __syncthreads();
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const bool first = tile == blockIdx.x;
         const int64_t r0 = tile * MLP_BM;
-        // ---- stage the input batch tile
+        // ---- stage the input tile: raw value, quantized value, abs-max
         {
-            const int K0 = d.l[0].h.K;
+            const MlpLayerDev &l0 = d.l[0];
+            const int K0 = l0.h.K, rm = Mode(l0.h.mode_in).round_mode;
+            const float *fl = lds + l0.off_f;
             for (int id = tid; id < MLP_BM * K0; id += 256) {
                 const int row = id / K0, k = id - row * K0;
                 const int64_t gr = r0 + row;
-                raw[row * d.ld_raw + d.l[0].acol + k] = gr < rows ? x[gr * K0 + k] : 0.f;
+                float v = 0.f, q = 0.f;
+                if (gr < rows) {
+                    v = x[gr * K0 + k];
+                    q = fixed_round_dyn(v, fl[k], rm);
+                    atomicMax(&amx[k], abs_bits(q));
+                }
+                raw[row * d.ld_raw + l0.acol + k] = v;
+                rx[row * d.ld_rx + l0.acol + k] = q;
             }
         }
         __syncthreads();
         // ================= forward =================
         for (int l = 0; l < L; ++l) {
             const MlpLayerDev &ly = d.l[l];
-            const int K = ly.h.K, N = ly.h.N;
-            const int rm = Mode(ly.h.mode_in).round_mode;
-            const float *fl = lds + ly.off_f;
-            for (int id = tid; id < MLP_BM * ly.Kp; id += 256) {
-                const int row = id / ly.Kp, k = id - row * ly.Kp;
-                float v = 0.f;
-                if (k < K && r0 + row < rows) v = fixed_round_dyn(raw[row * d.ld_raw + ly.acol + k], fl[k], rm);
-                rx[row * d.ld_rx + ly.acol + k] = v;
-            }
-            __syncthreads();
-            if (tid < K) {  // abs-max of the quantized input, per feature
-                uint32_t mx = 0;
-#pragma unroll 8
-                for (int r = 0; r < MLP_BM; ++r) {
-                    const uint32_t a = abs_bits(rx[r * d.ld_rx + ly.acol + tid]);
-                    mx = a > mx ? a : mx;
-                }
-                uint32_t *dst = (uint32_t *)(my + ly.p_amax) + tid;
-                if (first || mx > *dst) *dst = mx;
-            }
-            {
-                const int rh = wave & 1, cb = wave >> 1;
-                if (cb * 32 < ly.Np) {
-                    floatx16 acc = {0};
-                    const float *ws = lds + ly.off_w;
-                    const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
-                    for (int kk = 0; kk < ly.Kp; kk += 2)
-                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(rx[arow * d.ld_rx + ly.acol + kk + kq], ws[(kk + kq) * ly.ldw + bcol], acc, 0, 0, 0);
-                    if (bcol < N) {
-                        const float bias = lds[ly.off_qb + bcol];
-                        const int ocol = (l + 1 < L ? d.l[l + 1].acol : d.acol_out) + bcol;
+            const int N = ly.h.N;
+            const int rh = wave & 1, cb = wave >> 1;
+            if (cb * 32 < ly.Np) {
+                floatx16 acc = {0};
+                const float *ws = lds + ly.off_w;
+                const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
+                const int ksteps = (ly.h.K + 1) & ~1;
+                for (int kk = 0; kk < ksteps; kk += 2)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(rx[arow * d.ld_rx + ly.acol + kk + kq], ws[(kk + kq) * ly.ldw + bcol], acc, 0, 0, 0);
+                if (bcol < N) {
+                    const float bias = lds[ly.off_qb + bcol];
+                    const bool last = l + 1 == L;
+                    const int ocol = (last ? d.acol_out : d.l[l + 1].acol) + bcol;
+                    // the next layer's input quantizer runs here, on the accumulator registers
+                    const float fn = last ? 0.f : lds[d.l[l + 1].off_f + bcol];
+                    const int rm = last ? 0 : Mode(d.l[l + 1].h.mode_in).round_mode;
+                    uint32_t mx = 0;
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            float v = acc[r] + bias;
-                            if (ly.h.act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
-                            raw[(rh * 32 + acc_row_(r, lane)) * d.ld_raw + ocol] = v;
+                    for (int r = 0; r < 16; ++r) {
+                        const int row = rh * 32 + acc_row_(r, lane);
+                        float v = acc[r] + bias;
+                        if (ly.h.act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                        raw[row * d.ld_raw + ocol] = v;
+                        if (!last) {
+                            const float q = (r0 + row < rows) ? fixed_round_dyn(v, fn, rm) : 0.f;
+                            rx[row * d.ld_rx + ocol] = q;
+                            const uint32_t a = abs_bits(q);
+                            mx = a > mx ? a : mx;
                         }
+                    }
+                    if (!last) {
+                        const uint32_t o = (uint32_t)__shfl_xor((int)mx, 32, 64);
+                        mx = o > mx ? o : mx;
+                        if (lane < 32) atomicMax(&amx[(l + 1) * 64 + bcol], mx);
                     }
                 }
             }
@@ -145,6 +167,7 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
         float *cur = lds + d.off_dz0, *nxt = lds + d.off_dz1;
         {
             const int C = d.n_classes;
+            const int Cp = d.l[L - 1].Np;
             float lrow = 0.f;
             if (tid < MLP_BM) {
                 const int64_t gr = r0 + tid;
@@ -159,9 +182,9 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
                     lrow = logf(se) - (z[lab] - mx);
                     const float inv = 1.0f / se;
                     for (int c = 0; c < C; ++c) dz[c] = (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows;
-                    for (int c = C; c < 64; ++c) dz[c] = 0.f;
+                    for (int c = C; c < Cp; ++c) dz[c] = 0.f;
                 } else {
-                    for (int c = 0; c < 64; ++c) dz[c] = 0.f;
+                    for (int c = 0; c < Cp; ++c) dz[c] = 0.f;
                 }
             }
             if (wave == 0) {
@@ -172,132 +195,161 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
         }
         __syncthreads();
         // ================= backward =================
+        // `cur` holds the gradient at this layer's pre-activation (relu mask already applied) in
+        // columns [0, Np); both phases only read it, so one barrier per layer is enough.
         for (int l = L - 1; l >= 0; --l) {
             const MlpLayerDev &ly = d.l[l];
             const int K = ly.h.K, N = ly.h.N;
             const int K32 = ly.Kp >> 5, N32 = ly.Np >> 5;
-            if (ly.h.act == HGQ_ACT_RELU) {
-                const int ocol = l + 1 < L ? d.l[l + 1].acol : d.acol_out;
-                for (int id = tid; id < MLP_BM * N; id += 256) {
-                    const int row = id / N, n = id - row * N;
-                    if (!(raw[row * d.ld_raw + ocol + n] > 0.f)) cur[row * MLP_LDZ + n] = 0.f;
-                }
-                __syncthreads();
-            }
-            for (int id = tid; id < ly.Kp; id += 256) red[id] = 0.f;  // fractional-bit gradient of this layer's input
+            const int nblk = K32 * N32;
             // ---- kernel gradient: one 32 x 32 block per wave over the whole tile
-            {
-                const int nblk = K32 * N32;
-                if (wave < nblk) {
-                    const int wkb = wave / N32, wnb = wave % N32;
-                    floatx16 acc = {0};
-                    const int kq = lane >> 5, c32 = lane & 31;
-                    for (int rr = 0; rr < MLP_BM; rr += 2)
-                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(rx[(rr + kq) * d.ld_rx + ly.acol + wkb * 32 + c32],
-                                                                   cur[(rr + kq) * MLP_LDZ + wnb * 32 + c32], acc, 0, 0, 0);
-                    const int n = wnb * 32 + c32;
-                    if (n < N) {
+            if (wave < nblk) {
+                const int wkb = wave / N32, wnb = wave % N32;
+                floatx16 acc = {0};
+                const int kq = lane >> 5, c32 = lane & 31;
+                for (int rr = 0; rr < MLP_BM; rr += 2)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(rx[(rr + kq) * d.ld_rx + ly.acol + wkb * 32 + c32],
+                                                               cur[(rr + kq) * MLP_LDZ + wnb * 32 + c32], acc, 0, 0, 0);
+                const int n = wnb * 32 + c32;
+                if (n < N) {
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int k = wkb * 32 + acc_row_(r, lane);
-                            if (k < K) {
-                                float *dst = my + ly.p_dw + k * N + n;
-                                *dst = first ? acc[r] : *dst + acc[r];
-                            }
+                    for (int r = 0; r < 16; ++r) {
+                        const int k = wkb * 32 + acc_row_(r, lane);
+                        if (k < K) {
+                            float *dst = my + ly.p_dw + k * N + n;
+                            *dst = first ? acc[r] : *dst + acc[r];
                         }
                     }
                 }
             }
-            // ---- bias gradient
-            if (tid < N) {
-                float s = 0.f;
+            // ---- bias gradient: the last wave is free of kernel-gradient work unless all four blocks exist
+            if (ly.h.bias && wave == 3 && lane < N) {
+                float s0 = 0.f, s1 = 0.f;
 #pragma unroll 8
-                for (int r = 0; r < MLP_BM; ++r) s += cur[r * MLP_LDZ + tid];
-                float *dst = my + ly.p_db + tid;
-                *dst = first ? s : *dst + s;
+                for (int r = 0; r < MLP_BM; r += 2) s0 += cur[r * MLP_LDZ + lane], s1 += cur[(r + 1) * MLP_LDZ + lane];
+                float *dst = my + ly.p_db + lane;
+                *dst = first ? s0 + s1 : *dst + (s0 + s1);
             }
-            __syncthreads();  // red zeroed, cur fully read by the bias sums before nxt/cur swap matters
-            // ---- input gradient and the fractional-bit gradient of the input quantizer
+            // ---- input gradient, the relu mask of the layer below, and this layer's fractional-bit gradient
             {
                 const int rh = wave & 1, kb = wave >> 1;
                 if (kb < K32) {
                     floatx16 acc = {0};
                     const float *ws = lds + ly.off_w;
                     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
-                    for (int nn = 0; nn < ly.Np; nn += 2)
+                    const int nsteps = (N + 1) & ~1;
+                    for (int nn = 0; nn < nsteps; nn += 2)
                         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(cur[arow * MLP_LDZ + nn + kq], ws[wrow * ly.ldw + nn + kq], acc, 0, 0, 0);
                     const int kcol = kb * 32 + (lane & 31);
+                    const bool mask_below = l > 0 && d.l[l - 1].h.act == HGQ_ACT_RELU;
                     float dfsum = 0.f;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int row = rh * 32 + acc_row_(r, lane);
-                        nxt[row * MLP_LDZ + kcol] = acc[r];
-                        const float delta = rx[row * d.ld_rx + ly.acol + kcol] - raw[row * d.ld_raw + ly.acol + kcol];
+                        const float a = raw[row * d.ld_raw + ly.acol + kcol];
+                        const float delta = rx[row * d.ld_rx + ly.acol + kcol] - a;
                         if (kcol < K && r0 + row < rows) dfsum += -HGQ_LN2 * delta * acc[r];
+                        nxt[row * MLP_LDZ + kcol] = (kcol < K && (!mask_below || a > 0.f)) ? acc[r] : 0.f;
                     }
                     dfsum += __shfl_xor(dfsum, 32, 64);
-                    if (lane < 32 && kcol < K) atomicAdd(&red[kcol], dfsum);
+                    if (lane < 32 && kcol < K) atomicAdd(&dfs[l * 64 + kcol], dfsum);
                 }
             }
-            __syncthreads();
-            if (tid < K) {
-                float *dst = my + ly.p_df + tid;
-                *dst = first ? red[tid] : *dst + red[tid];
-            }
-            // columns [Kp, 64) of the next gradient tile must read as zero for a narrower next layer
-            if (ly.Kp < 64)
-                for (int id = tid; id < MLP_BM * (64 - ly.Kp); id += 256) {
-                    const int row = id / (64 - ly.Kp), c = ly.Kp + id % (64 - ly.Kp);
-                    nxt[row * MLP_LDZ + c] = 0.f;
-                }
             __syncthreads();
             float *t = cur;
             cur = nxt;
             nxt = t;
         }
     }
-}
-
-// out[e] = combination over slices of part[g][e]: float sum, or unsigned max inside the abs-max sections
-__global__ __launch_bounds__(256) void mlp_reduce_kernel(MlpDev d, const float *__restrict__ part, int n_parts, float *out) {
-    __shared__ float red[256];
-    const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
-    bool is_max = false;
-    for (int l = 0; l < d.n_layers; ++l) is_max |= (e >= d.l[l].p_amax && e < d.l[l].p_amax + d.l[l].h.K);
-    float s = 0.f;
-    uint32_t mx = 0;
-    if (e < d.M) {
-        const int per = (n_parts + 3) / 4;
-        const int g0 = grp * per, g1 = min(n_parts, g0 + per);
-        int g = g0;
-        for (; g + 8 <= g1; g += 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = part[(int64_t)(g + u) * d.M + e];
-            if (is_max) {
-#pragma unroll
-                for (int u = 0; u < 8; ++u) mx = max(mx, __float_as_uint(v[u]));
-            } else {
-                s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
-            }
-        }
-        for (; g < g1; ++g) {
-            const float v = part[(int64_t)g * d.M + e];
-            if (is_max) mx = max(mx, __float_as_uint(v));
-            else s += v;
+    // ---- this workgroup's abs-max and fractional-bit sums
+    for (int l = 0; l < L; ++l) {
+        const MlpLayerDev &ly = d.l[l];
+        if (tid < ly.h.K) {
+            my[ly.p_df + tid] = dfs[l * 64 + tid];
+            ((uint32_t *)(my + ly.p_amax))[tid] = amx[l * 64 + tid];
         }
     }
-    red[threadIdx.x] = is_max ? __uint_as_float(mx) : s;
-    __syncthreads();
-    if (grp == 0 && e < d.M) {
-        if (is_max) {
-            uint32_t m = __float_as_uint(red[e_local]);
-            for (int w = 1; w < 4; ++w) m = max(m, __float_as_uint(red[e_local + 64 * w]));
-            out[e] = __uint_as_float(m);
-        } else {
-            out[e] = (red[e_local] + red[e_local + 64]) + (red[e_local + 128] + red[e_local + 192]);
+}
+
+#define MLP_AUX 192  // per layer, after the M reduced sums: colsum[64], bits_in[64], dbits_in[64]
+
+// Blocks [0, ceil(M/64)): out[e] = sum over slices of part[g][e] (the abs-max sections are skipped
+// here).  Blocks beyond that, one per layer: reduce the layer's abs-max section, track the input
+// quantizer's integer bits in place, and leave for the update pass - which must not read variables
+// another workgroup is updating - the per-feature bit counts of the input quantizer and the
+// per-row sums of the kernel bit counts, all from the pre-update variables.
+__global__ __launch_bounds__(256) void mlp_reduce_kernel(MlpDev d, const float *__restrict__ part, int n_parts, float *out,
+                                                         float *loss) {
+    __shared__ float red[256];
+    const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int n_main = (d.M + 63) / 64;
+    const int per = (n_parts + 3) / 4;
+    const int g0 = grp * per, g1 = min(n_parts, g0 + per);
+    if ((int)blockIdx.x < n_main) {
+        const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
+        float s = 0.f;
+        if (e < d.M) {
+            int g = g0;
+            for (; g + 8 <= g1; g += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = part[(int64_t)(g + u) * d.M + e];
+                s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+            }
+            for (; g < g1; ++g) s += part[(int64_t)g * d.M + e];
         }
+        red[threadIdx.x] = s;
+        __syncthreads();
+        if (grp == 0 && e < d.M) {
+            const float v = (red[e_local] + red[e_local + 64]) + (red[e_local + 128] + red[e_local + 192]);
+            out[e] = v;
+            if (e == d.p_loss && loss) loss[0] = v;
+        }
+        return;
+    }
+    const int l = blockIdx.x - n_main;
+    const MlpLayerDev &ly = d.l[l];
+    const hgq_mlp_layer &h = ly.h;
+    const int k = e_local, K = h.K, N = h.N;
+    const Mode mk(h.mode_ker), mi(h.mode_in);
+    uint32_t mx = 0;
+    float cs = 0.f;
+    if (k < K) {
+        const uint32_t *pa = (const uint32_t *)part + ly.p_amax + k;
+        int g = g0;
+        for (; g + 8 <= g1; g += 8) {
+            uint32_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = pa[(int64_t)(g + u) * d.M];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) mx = max(mx, v[u]);
+        }
+        for (; g < g1; ++g) mx = max(mx, pa[(int64_t)g * d.M]);
+        // this thread's quarter of row k of the kernel bit counts
+        const int nper = (N + 3) / 4, n0 = grp * nper, n1 = min(N, n0 + nper);
+        for (int n = n0; n < n1; ++n) {
+            float bk = rintf(h.b_ker[k * N + n]);
+            if (mk.overflow_mode == HGQ_SAT) bk += load_k(h.k_ker, k * N + n, mk.k_u8);
+            cs += bk;
+        }
+    }
+    __shared__ uint32_t smx[256];
+    smx[threadIdx.x] = mx;
+    red[threadIdx.x] = cs;
+    __syncthreads();
+    if (grp == 0 && k < K) {
+        for (int w = 1; w < 4; ++w) mx = max(mx, smx[k + 64 * w]);
+        const float f = rintf(h.f_in[k]);
+        const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-f)));
+        const float ni = fmaxf(__fsub_rn(h.i_in[k], h.decay), mi_);
+        h.i_in[k] = ni;
+        const float sfi = __fadd_rn(rintf(ni), f);
+        float b = sfi > 0.f ? sfi : 0.f;
+        if (mi.overflow_mode == HGQ_SAT) b += load_k(h.k_in, k, mi.k_u8);
+        float *aux = out + d.M + l * MLP_AUX;
+        aux[k] = (red[k] + red[k + 64]) + (red[k + 128] + red[k + 192]);
+        aux[64 + k] = b;
+        aux[128 + k] = sfi > 0.f ? 1.f : 0.f;
     }
 }
 
@@ -305,60 +357,61 @@ __device__ __forceinline__ float sgd_clip(float w, float g, float lr, float l1, 
     return fminf(fmaxf(__fsub_rn(w, __fmul_rn(lr, __fadd_rn(g, l1))), lo), hi);
 }
 
-// One workgroup per layer.  All gradients are formed from the pre-update variables (phase 1 and 2
-// only read), then every variable is updated (phase 3).
+#define MLP_UPD_SPLIT 8
+
+// Grid (layers, MLP_UPD_SPLIT).  Each workgroup updates its share of the layer's kernel entries;
+// the first one of a layer also owns EBOPs, the bias and the input quantizer's fractional bits.
+// Everything a workgroup needs about variables it does not own comes from the reduce pass.
 __global__ __launch_bounds__(256) void mlp_update_kernel(MlpDev d, const float *__restrict__ g, float lr, float *loss) {
     __shared__ float colsum[64];   // sum_n bits_ker[k, n]
     __shared__ float bits_in[64];  // relu(round(i) + round(f)) with the tracked i
     __shared__ float dbits_in[64];
-    __shared__ float redbuf[4];
     const MlpLayerDev &ly = d.l[blockIdx.x];
     const hgq_mlp_layer &h = ly.h;
     const int tid = threadIdx.x, K = h.K, N = h.N;
-    const Mode mk(h.mode_ker), mb(h.mode_bias), mi(h.mode_in);
-    // ---- phase 1: integer-bit tracking of the input quantizer, then bit counts
-    if (tid < K) {
-        const float f = rintf(h.f_in[tid]);
-        const float mi_ = ceil_log2_exact(__fadd_rn(g[ly.p_amax + tid], pow2(-f)));
-        const float ni = fmaxf(__fsub_rn(h.i_in[tid], h.decay), mi_);
-        h.i_in[tid] = ni;
-        const float s = __fadd_rn(rintf(ni), f);
-        float b = s > 0.f ? s : 0.f;
-        dbits_in[tid] = s > 0.f ? 1.f : 0.f;
-        if (mi.overflow_mode == HGQ_SAT) b += load_k(h.k_in, tid, mi.k_u8);
-        bits_in[tid] = b;
-        float cs = 0.f;
-        for (int n = 0; n < N; ++n) {
-            float bk = rintf(h.b_ker[tid * N + n]);
-            if (mk.overflow_mode == HGQ_SAT) bk += load_k(h.k_ker, tid * N + n, mk.k_u8);
-            cs += bk;
-        }
-        colsum[tid] = cs;
+    const bool owner = blockIdx.y == 0;
+    const Mode mk(h.mode_ker), mb(h.mode_bias);
+    if (tid < 64) {
+        const float *aux = g + d.M + blockIdx.x * MLP_AUX;
+        colsum[tid] = aux[tid], bits_in[tid] = aux[64 + tid], dbits_in[tid] = aux[128 + tid];
     }
-    __syncthreads();
-    // ---- phase 2: EBOPs value
-    float part = tid < K ? bits_in[tid] * colsum[tid] : 0.f;
-    float bsum = 0.f;
-    if (h.bias && tid < N) {
-        bsum = rintf(h.b_bias[tid]);
-        if (mb.overflow_mode == HGQ_SAT) bsum += load_k(h.k_bias, tid, mb.k_u8);
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64), bsum += __shfl_xor(bsum, o, 64);
-    if ((tid & 63) == 0) redbuf[tid >> 6] = part;  // K, N <= 64: only wave 0 holds non-zero terms
     __syncthreads();
     const float beta = h.beta ? h.beta[0] : 0.f;
-    if (tid == 0) {
-        float total = redbuf[0];
-        if (h.bias) total += bsum / (float)N * h.bias_size;
-        const float e = total * h.ebops_scale;
-        if (h.ebops) h.ebops[0] = (uint32_t)e;
-        if (loss) atomicAdd(loss, e * beta + (blockIdx.x == 0 ? g[d.p_loss] : 0.f));
-    }
     const float gs = h.ebops_scale * beta;  // d(ebops * beta) / d bits
     float reg = 0.f;  // MonoL1 regularisation loss of the trainable bit-width variables (pre-update values)
-    // ---- phase 3: quantizer backward of kernel and bias, SGD + constraints on every variable
-    for (int e = tid; e < K * N; e += 256) {
+    if (owner) {
+        float part = tid < K ? bits_in[tid] * colsum[tid] : 0.f;
+        float bsum = 0.f;
+        if (h.bias && tid < N) {
+            bsum = rintf(h.b_bias[tid]);
+            if (mb.overflow_mode == HGQ_SAT) bsum += load_k(h.k_bias, tid, mb.k_u8);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64), bsum += __shfl_xor(bsum, o, 64);
+        if (tid == 0) {  // K, N <= 64: wave 0 holds every non-zero term
+            float total = part;
+            if (h.bias) total += bsum / (float)N * h.bias_size;
+            const float e = total * h.ebops_scale;
+            if (h.ebops) h.ebops[0] = (uint32_t)e;
+            if (loss) atomicAdd(loss, e * beta);
+        }
+        if (h.bias && tid < N) {
+            const KIF p = kbi_entry(h.k_bias, h.i_bias, h.b_bias, tid, h.mode_bias);
+            float dw, di, db;
+            quantize_grad_dyn(h.bias[tid], g[ly.p_db + tid], p, mb.round_mode, mb.overflow_mode, dw, di, db);
+            di -= db;
+            h.bias[tid] = __fsub_rn(h.bias[tid], __fmul_rn(lr, dw));
+            reg += h.b_bias_l1 * h.b_bias[tid] + (h.train_i_bias ? h.i_bias_l1 * h.i_bias[tid] : 0.f);
+            h.b_bias[tid] = sgd_clip(h.b_bias[tid], db + h.bias_size / (float)N * gs, lr, h.b_bias_l1, h.b_bias_lo, h.b_bias_hi);
+            if (h.train_i_bias) h.i_bias[tid] = sgd_clip(h.i_bias[tid], di, lr, h.i_bias_l1, h.i_bias_lo, h.i_bias_hi);
+        }
+        if (tid < K) {
+            reg += h.f_in_l1 * h.f_in[tid];
+            h.f_in[tid] = sgd_clip(h.f_in[tid], g[ly.p_df + tid] + dbits_in[tid] * colsum[tid] * gs, lr, h.f_in_l1, h.f_in_lo, h.f_in_hi);
+        }
+    }
+    // quantizer backward of this workgroup's kernel entries, SGD + constraints
+    for (int e = blockIdx.y * 256 + tid; e < K * N; e += MLP_UPD_SPLIT * 256) {
         const int k = e / N;
         const KIF p = kbi_entry(h.k_ker, h.i_ker, h.b_ker, e, h.mode_ker);
         float dw, di, db;
@@ -368,20 +421,6 @@ __global__ __launch_bounds__(256) void mlp_update_kernel(MlpDev d, const float *
         reg += h.b_ker_l1 * h.b_ker[e] + (h.train_i_ker ? h.i_ker_l1 * h.i_ker[e] : 0.f);
         h.b_ker[e] = sgd_clip(h.b_ker[e], db + bits_in[k] * gs, lr, h.b_ker_l1, h.b_ker_lo, h.b_ker_hi);
         if (h.train_i_ker) h.i_ker[e] = sgd_clip(h.i_ker[e], di, lr, h.i_ker_l1, h.i_ker_lo, h.i_ker_hi);
-    }
-    if (h.bias && tid < N) {
-        const KIF p = kbi_entry(h.k_bias, h.i_bias, h.b_bias, tid, h.mode_bias);
-        float dw, di, db;
-        quantize_grad_dyn(h.bias[tid], g[ly.p_db + tid], p, mb.round_mode, mb.overflow_mode, dw, di, db);
-        di -= db;
-        h.bias[tid] = __fsub_rn(h.bias[tid], __fmul_rn(lr, dw));
-        reg += h.b_bias_l1 * h.b_bias[tid] + (h.train_i_bias ? h.i_bias_l1 * h.i_bias[tid] : 0.f);
-        h.b_bias[tid] = sgd_clip(h.b_bias[tid], db + h.bias_size / (float)N * gs, lr, h.b_bias_l1, h.b_bias_lo, h.b_bias_hi);
-        if (h.train_i_bias) h.i_bias[tid] = sgd_clip(h.i_bias[tid], di, lr, h.i_bias_l1, h.i_bias_lo, h.i_bias_hi);
-    }
-    if (tid < K) {
-        reg += h.f_in_l1 * h.f_in[tid];
-        h.f_in[tid] = sgd_clip(h.f_in[tid], g[ly.p_df + tid] + dbits_in[tid] * colsum[tid] * gs, lr, h.f_in_l1, h.f_in_lo, h.f_in_hi);
     }
     if (loss) {
 #pragma unroll
@@ -430,7 +469,7 @@ static int mlp_plan(const hgq_mlp_layer *layers, int n_layers, MlpDev &d, size_t
     d.off_rx = off, off += MLP_BM * d.ld_rx;
     d.off_dz0 = off, off += MLP_BM * MLP_LDZ;
     d.off_dz1 = off, off += MLP_BM * MLP_LDZ;
-    d.off_red = off, off += 64;
+    d.off_red = off, off += 2 * 64 * HGQ_MLP_MAX_LAYERS;  // fractional-bit sums and abs-max, [layers][64] each
     lds_bytes = (size_t)off * 4;
     if (lds_bytes > 160 * 1024 - 512) return fail(HGQ_ERR_UNSUPPORTED, "hgq_mlp: the stack needs %zu bytes of LDS", lds_bytes);
     return HGQ_OK;
@@ -449,7 +488,7 @@ extern "C" int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, 
     MlpDev d;
     size_t lds_bytes;
     if (mlp_plan(layers, n_layers, d, lds_bytes)) return -1;
-    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M;
+    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX;
 }
 
 extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
@@ -468,11 +507,10 @@ extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, con
     }
     const int parts = mlp_parts(rows);
     float *reduced = workspace + (int64_t)parts * d.M;
-    if (loss && (rc = fill_f32(loss, 0.f, 1, s))) return rc;
     hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(256), lds_bytes, s, d, x, labels, rows, workspace);
     if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
-    hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64), dim3(256), 0, s, d, workspace, parts, reduced);
+    hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(256), 0, s, d, workspace, parts, reduced, loss);
     if ((rc = check_launch("hgq_mlp_train_step(reduce)"))) return rc;
-    hipLaunchKernelGGL(mlp_update_kernel, dim3(n_layers), dim3(256), 0, s, d, reduced, lr, loss);
+    hipLaunchKernelGGL(mlp_update_kernel, dim3(n_layers, MLP_UPD_SPLIT), dim3(256), 0, s, d, reduced, lr, loss);
     return check_launch("hgq_mlp_train_step(update)");
 }
