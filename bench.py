@@ -21,6 +21,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+# HBM bytes per launch of the 4 Mi-element quantizer kernels from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# counters, each scaled by what the same counter reads for a 16 MiB device copy (FETCH_SIZE x 1.997,
+# WRITE_SIZE x 1.000); summary and commands in profiles/quantizer_4Mi_hbm_counters.md
+TRAFFIC_BYTES = {'quant_fwd_1d': 83.8e6, 'quant_bwd_1d': 117.4e6}
 BATCH = 16384
 DIMS = (16, 64, 32, 32, 5)
 QN = 4 * 1024 * 1024  # standalone quantizer case: 4 Mi fp32 elements
@@ -39,7 +43,7 @@ def _events_ms(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
-def quantizer_roofline(iters=200):
+def quantizer_roofline(iters=200, with_copy=False):
     """Standalone KIF quantizer, RND/WRAP, per-element k, i, f, training forward + surrogate
     backward, launched straight through the C ABI on torch's current stream and timed with HIP
     events on that stream."""
@@ -84,9 +88,18 @@ def quantizer_roofline(iters=200):
     t_fwd = _events_ms(fwd, iters)
     t_bwd = _events_ms(bwd, iters)
     out = {}
+    if with_copy:
+        # calibration for hardware counters: a plain device copy of known size (16 MiB read + 16 MiB written)
+        def cp():
+            x, k, i, f, dy, y, dx, di, df = sets[state['n'] % n_sets]
+            state['n'] += 1
+            y.copy_(x)
+
+        t_cp = _events_ms(cp, iters)
+        out['copy_4Mi_f32'] = {'ms': t_cp, 'bytes': 8 * QN, 'GBps': 8 * QN / (t_cp * 1e-3) / 1e9, 'frac': 8 * QN / (t_cp * 1e-3) / 1e9 / HBM_PEAK_GBS}
     for name, ms, bpe in (('quant_fwd_1d', t_fwd, 20), ('quant_bwd_1d', t_bwd, 32)):
         gbs = bpe * QN / (ms * 1e-3) / 1e9
-        out[name] = {'ms': ms, 'bytes': bpe * QN, 'GBps': gbs, 'frac': gbs / HBM_PEAK_GBS}
+        out[name] = {'ms': ms, 'bytes': bpe * QN, 'GBps': gbs, 'frac': gbs / HBM_PEAK_GBS, 'traffic': TRAFFIC_BYTES[name]}
     return out
 
 
@@ -122,7 +135,9 @@ def main():
     ap.add_argument('--steps', type=int, default=300)
     ap.add_argument('--warmup', type=int, default=30)
     ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused-graph',
+    ap.add_argument('--roofline-only', action='store_true',
+                    help='run only the standalone quantizer kernels and a plain copy of known size (for counter runs)')
+    ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused',
                     help='fused: whole-step kernels (3 launches); layers: per-layer torch.library operators with autograd; '
                          '-graph: the step is captured once in a HIP graph and replayed')
     args = ap.parse_args()
@@ -131,6 +146,11 @@ def main():
         sys.exit(2)
 
     import torch
+
+    if args.roofline_only:
+        torch.cuda.set_device(0)
+        print(json.dumps({'quantizer_kernels': quantizer_roofline(iters=20, with_copy=True)}))
+        return
 
     from hgq2_amd import ops
     from hgq2_amd.train import SGD, FusedQDenseStack, GraphedTrainStep, model_loss
@@ -189,7 +209,7 @@ def main():
     qr = quantizer_roofline()
     dom = qr['quant_bwd_1d']
     roofline = {'bound': 'hbm', 'kernel': 'quant_bwd_1d', 'achieved': dom['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': dom['frac'], 'traffic': None,
+                'frac': dom['frac'], 'traffic': dom['traffic'],
                 'workload': 'standalone kif quantizer RND/WRAP, 4 Mi fp32 elements, per-element k/i/f: backward 32 B/elem'}
     out = {
         'metric': 'QDense MLP train samples/s @bs16384; quantizer HBM GB/s vs peak',

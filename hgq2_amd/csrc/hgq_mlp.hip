@@ -1,4 +1,4 @@
-// One training step of a stack of QDense layers in three launches.
+// One training step of a stack of QDense layers in four launches.
 //
 // At the layer sizes HGQ targets (tens of units per layer) a training step built from per-layer
 // kernels is bound by launch latency, not by HBM or MFMA.  Here the whole data path - every
@@ -45,34 +45,39 @@ __device__ __forceinline__ KIF kbi_entry(const void *k, const float *i, const fl
     return resolve_kif(load_k(k, idx, m.k_u8), i[idx], b[idx], true, true);
 }
 
-// Quantize `count` kernel (or bias) entries into their padded LDS image.  The global loads of a
-// batch of four entries are issued before any of them is used: the prologue is latency-bound.
-__device__ __forceinline__ void stage_quantized(float *dst, int n_lds, int ld, int K, int N, const float *w, const void *kq,
-                                                const float *iq, const float *bq, int mode, int tid) {
-    const Mode m(mode);
-    for (int base = tid; base < n_lds; base += 4 * 256) {
-        float wv[4], kv[4], iv[4], bv[4];
-        bool ok[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int id = base + u * 256;
-            const int k = id / ld, n = id - k * ld;
-            ok[u] = id < n_lds && k < K && n < N;
-            if (ok[u]) {
-                const int64_t e = (int64_t)k * N + n;
-                wv[u] = w[e], kv[u] = load_k(kq, e, m.k_u8), iv[u] = iq[e], bv[u] = bq[e];
-            }
+// The quantized kernels and biases of all layers and the rounded fractional bits of the input
+// quantizers, laid out exactly as the forward/backward kernel keeps them in LDS (zero padded).
+// One thread per entry: every workgroup of the main kernel then fetches the finished image with
+// a single round of wide loads instead of re-quantizing it behind dozens of dependent loads.
+__global__ __launch_bounds__(256) void mlp_prep_kernel(MlpDev d, float *__restrict__ img) {
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= d.off_raw) return;
+    int l = 0;
+    while (l + 1 < d.n_layers && e >= d.l[l + 1].off_w) ++l;
+    const MlpLayerDev &ly = d.l[l];
+    const hgq_mlp_layer &h = ly.h;
+    float v = 0.f;
+    if (e < ly.off_qb) {
+        const int id = e - ly.off_w, k = id / ly.ldw, n = id - k * ly.ldw;
+        if (k < h.K && n < h.N) {
+            const Mode m(h.mode_ker);
+            const int64_t t = (int64_t)k * h.N + n;
+            v = quantize_dyn(h.w[t], kbi_entry(h.k_ker, h.i_ker, h.b_ker, t, h.mode_ker), m.round_mode, m.overflow_mode, true);
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int id = base + u * 256;
-            if (id < n_lds)
-                dst[id] = ok[u] ? quantize_dyn(wv[u], resolve_kif(kv[u], iv[u], bv[u], true, true), m.round_mode, m.overflow_mode, true) : 0.f;
+    } else if (e < ly.off_f) {
+        const int n = e - ly.off_qb;
+        if (n < h.N && h.bias) {
+            const Mode m(h.mode_bias);
+            v = quantize_dyn(h.bias[n], kbi_entry(h.k_bias, h.i_bias, h.b_bias, n, h.mode_bias), m.round_mode, m.overflow_mode, true);
         }
+    } else {
+        const int k = e - ly.off_f;
+        if (k < h.K) v = rintf(h.f_in[k]);
     }
+    img[e] = v;
 }
 
-__global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ x,
+__global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ img, const float *__restrict__ x,
                                                           const int64_t *__restrict__ labels, int64_t rows,
                                                           float *part) {
     extern __shared__ float lds[];
@@ -85,16 +90,8 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
     const int64_t n_tiles = (rows + MLP_BM - 1) / MLP_BM;
     const float inv_rows = 1.0f / (float)rows;
 
-    // ---- prologue: quantize every layer's kernel and bias into LDS (zero padded), round f
-    for (int l = 0; l < L; ++l) {
-        const MlpLayerDev &ly = d.l[l];
-        stage_quantized(lds + ly.off_w, ly.Kp * ly.ldw, ly.ldw, ly.h.K, ly.h.N, ly.h.w, ly.h.k_ker, ly.h.i_ker, ly.h.b_ker, ly.h.mode_ker, tid);
-        if (ly.h.bias)
-            stage_quantized(lds + ly.off_qb, ly.Np, ly.Np, 1, ly.h.N, ly.h.bias, ly.h.k_bias, ly.h.i_bias, ly.h.b_bias, ly.h.mode_bias, tid);
-        else
-            for (int n = tid; n < ly.Np; n += 256) lds[ly.off_qb + n] = 0.f;
-        for (int k = tid; k < ly.Kp; k += 256) lds[ly.off_f + k] = k < ly.h.K ? rintf(ly.h.f_in[k]) : 0.f;
-    }
+    // ---- prologue: fetch the quantized kernels / biases / rounded fractional bits (off_raw is a multiple of 4)
+    for (int id = tid * 4; id < d.off_raw; id += 4 * 256) *(float4 *)(lds + id) = *(const float4 *)(img + id);
     for (int id = tid; id < MLP_BM * d.ld_rx; id += 256) rx[id] = 0.f;  // padding columns stay zero for good
     for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += 256) dfs[id] = 0.f, amx[id] = 0u;
     __syncthreads();
@@ -465,6 +462,7 @@ static int mlp_plan(const hgq_mlp_layer *layers, int n_layers, MlpDev &d, size_t
     d.ld_raw = acol + d.l[n_layers - 1].Np + 1;
     d.p_loss = p, p += 1;
     d.M = p;
+    off = (off + 3) & ~3;
     d.off_raw = off, off += MLP_BM * d.ld_raw;
     d.off_rx = off, off += MLP_BM * d.ld_rx;
     d.off_dz0 = off, off += MLP_BM * MLP_LDZ;
@@ -488,7 +486,7 @@ extern "C" int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, 
     MlpDev d;
     size_t lds_bytes;
     if (mlp_plan(layers, n_layers, d, lds_bytes)) return -1;
-    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX;
+    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX + d.off_raw + 4;
 }
 
 extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
@@ -507,7 +505,11 @@ extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, con
     }
     const int parts = mlp_parts(rows);
     float *reduced = workspace + (int64_t)parts * d.M;
-    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(256), lds_bytes, s, d, x, labels, rows, workspace);
+    float *img = reduced + d.M + (int64_t)n_layers * MLP_AUX;
+    img += (4 - ((uintptr_t)img / 4) % 4) % 4;  // 16-byte aligned
+    hipLaunchKernelGGL(mlp_prep_kernel, dim3((d.off_raw + 255) / 256), dim3(256), 0, s, d, img);
+    if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
+    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(256), lds_bytes, s, d, img, x, labels, rows, workspace);
     if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
     hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(256), 0, s, d, workspace, parts, reduced, loss);
     if ((rc = check_launch("hgq_mlp_train_step(reduce)"))) return rc;
