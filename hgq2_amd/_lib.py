@@ -51,7 +51,18 @@ SIGNATURES = {
     'hgq_mlp_workspace': (c_int64, [c_void_p, c_int, c_int64]),
     'hgq_mlp_train_step': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p]),
     'hgq_fill_u32': (c_int, [c_void_p, ctypes.c_uint32, c_int64, c_void_p]),
+    'hgq_qsoftmax_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_float, c_float] + [c_void_p] * 5
+                         + [c_void_p] * 3 + [c_void_p]),
+    'hgq_qsoftmax_bwd_workspace': (c_int64, [c_int64, c_int, c_int64, c_int]),
+    'hgq_qsoftmax_bwd': (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int64, c_float, c_float] + [c_void_p] * 5
+                         + [c_void_p] * 4 + [c_void_p]),
 }
+
+
+class QDesc(ctypes.Structure):
+    """``hgq_qdesc`` of include/hgq_hip.h: one quantizer's raw variables and mode bits."""
+
+    _fields_ = [('k', c_void_p), ('i', c_void_p), ('fb', c_void_p), ('mode', c_int)]
 
 
 

@@ -99,13 +99,14 @@ class QLayerBase(Layer):
         return ebops * self._beta
 
     def _wrapped_call(self, *args, training=None, **kwargs):
+        self._oq_applied_in_call = False  # a `call` that ran the output quantizer in a fused kernel sets this
         r = self.call(*args, training=training, **kwargs)
         if (training or training == 'tracing') and self.enable_ebops:
             tensors = args[0] if isinstance(args[0], (tuple, list)) else [a for a in args if isinstance(a, torch.Tensor)]
             shapes = [(1,) + tuple(t.shape[1:]) for t in tensors]
             self.add_loss(self._ebops_loss_term(*shapes))
         self._finish_call()
-        if not self.enable_oq or self.__output_quantizer_handled__:
+        if not self.enable_oq or self.__output_quantizer_handled__ or self._oq_applied_in_call:
             return r
         assert not isinstance(r, (tuple, list)), (
             f'Layer {self.name}({type(self)}) returns multiple outputs, which must be handled in subclasses.'

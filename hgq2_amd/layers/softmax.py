@@ -13,11 +13,17 @@ from math import prod
 
 import torch
 
+from .. import ops
 from ..config.layer import global_config
 from ..core import epsilon
 from ..quantizer import QuantizerConfig
+from ..quantizer.internal import FixedPointQuantizerKBI, FixedPointQuantizerKIF
+from ..quantizer.internal.base import bw_layout
 from .activation import QUnaryFunctionLUT
 from .core.base import QLayerBaseSingleInput
+
+
+FUSED = True  # module switch: False forces the per-stage path (used to cross-check the one-pass kernels)
 
 
 class QSoftmax(QLayerBaseSingleInput):
@@ -82,9 +88,73 @@ class QSoftmax(QLayerBaseSingleInput):
         self.inv_table.built = True
         super().build(input_shape)
 
+    # ---- fused kernel path
+    @staticmethod
+    def _fusable_quantizer(q, training, shared: bool):
+        """``(k, i, fb, mode, track)`` if the kernel can run this quantizer in place, else ``None``."""
+        if q is None or not q.plain:
+            return None
+        inner = q.quantizer
+        if not isinstance(inner, (FixedPointQuantizerKIF, FixedPointQuantizerKBI)) or not inner.built:
+            return None
+        if shared and inner._i.numel() != 1:
+            return None
+        track = False
+        if inner.overflow_mode == 'WRAP' and inner.trainable:
+            if training == 'tracing' or (training and not isinstance(inner, FixedPointQuantizerKIF)):
+                return None  # calibration and the KBI tracking rule keep their own call sequence
+            track = training is True
+        return inner._k.view(-1), inner._i.view(-1), inner._third().view(-1), inner._mode(training is True), track
+
+    def _fused_plan(self, x, training, mask):
+        """Descriptors for ``ops.qsoftmax`` when this call maps onto the one-pass kernel, else ``None``."""
+        if not (FUSED and self.stable and mask is None and x.is_cuda and x.dtype == torch.float32 and x.dim() >= 2):
+            return None
+        if self.axes != (x.dim() - 1,) or not 1 <= x.shape[-1] <= 256 or x.numel() == 0:
+            return None
+        if training not in (True, False, None):
+            return None
+        e, v = self.exp_table, self.inv_table
+        if not (e.enable_iq and e.enable_oq and v.enable_iq and v.enable_oq):
+            return None
+        qs = [self._fusable_quantizer(q, training, True) for q in (e.iq, e.oq, v.iq, v.oq)]
+        if any(q is None for q in qs):
+            return None
+        if self.enable_oq:
+            if not self.oq.built:
+                return None
+            qo = self._fusable_quantizer(self.oq, training, False)
+            layout = bw_layout(self.oq.quantizer._i.shape, x.shape)
+            if qo is None or layout is None or layout[1] != 1 or layout[0] % x.shape[-1] != 0:
+                return None
+            qs.append(qo)
+        else:
+            qs.append(None)
+        return qs
+
+    def _call_fused(self, x, training, qs):
+        e, v = self.exp_table, self.inv_table
+        owners = (e.iq, e.oq, v.iq, v.oq, self.oq if self.enable_oq else None)
+        track_mask = sum(bit for bit, q in zip((1, 0, 2, 0, 4), qs) if q is not None and q[4])
+        y, a1, a3, ao = ops.qsoftmax(x, [None if q is None else q[:4] for q in qs], self.input_scaler, epsilon(), track_mask)
+        for amax, n in ((a1, 0), (a3, 2), (ao, 4)):
+            if amax.numel():
+                owners[n].quantizer._track(amax, True)
+        # what the two table layers' own call wrappers do after their call (EBOPs term, uint32 variable)
+        accum_shape = tuple(x.shape[:-1]) + (1,)
+        for table, shape in ((e, tuple(x.shape)), (v, accum_shape)):
+            table._losses = []
+            if training and table.enable_ebops:
+                table.add_loss(table._ebops_loss_term((1,) + shape[1:]))
+        return y
+
     def call(self, inputs, training=None, mask=None):
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
+        qs = self._fused_plan(inputs, training, mask)
+        if qs is not None:
+            self._oq_applied_in_call = self.enable_oq  # the kernel runs the output quantizer itself
+            return self._call_fused(inputs, training, qs)
         if self.stable:
             if mask is not None:
                 mask = mask.to(inputs.dtype)

@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax']
 
 
 def _ptr(t: Tensor | None):
@@ -253,6 +253,90 @@ def sgd_update_multi_op(ws: Sequence[Tensor], gs: Sequence[Tensor], l1: Sequence
     _lib.check(rc, 'hgq_sgd_update_multi')
 
 
+def _qdescs(ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor], modes: Sequence[int]):
+    """Five ``hgq_qdesc`` structures (exp_iq, exp_oq, inv_iq, inv_oq, oq); an empty ``k`` means absent."""
+    _need(len(ks) == 5 and len(is_) == 5 and len(fbs) == 5 and len(modes) == 5, 'five quantizer descriptors are expected')
+    descs = []
+    for n, (k, i, fb, mode) in enumerate(zip(ks, is_, fbs, modes)):
+        if k.numel() == 0:
+            descs.append(_lib.QDesc(None, None, None, 0))
+            continue
+        _check_k(f'k[{n}]', k), _check_f32(f'i[{n}]', i), _check_f32(f'fb[{n}]', fb)
+        _need(k.numel() == i.numel() == fb.numel(), f'quantizer {n}: k, i, fb differ in size')
+        if n < 4:
+            _need(i.numel() == 1, f'quantizer {n}: the table quantizers must have a single bit-width entry')
+        descs.append(_lib.QDesc(k.data_ptr(), i.data_ptr(), fb.data_ptr(), _kmode(mode, k)))
+    return descs
+
+
+def _softmax_bw_rows(x: Tensor, oq_i: Tensor) -> int:
+    L = x.shape[-1]
+    if oq_i.numel() == 0:
+        return 1
+    _need(oq_i.numel() % L == 0, 'the output quantizer table must be [bw_rows, L]')
+    return oq_i.numel() // L
+
+
+@torch.library.custom_op('hgq::qsoftmax_fwd', mutates_args=())
+def qsoftmax_fwd(x: Tensor, ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor], modes: Sequence[int],
+                 input_scaler: float, eps: float, track_mask: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    _check_f32('x', x)
+    _need(x.dim() >= 1 and 1 <= x.shape[-1] <= 256, 'softmax rows of 1..256 elements are supported')
+    L = x.shape[-1]
+    rows = x.numel() // L
+    descs = _qdescs(ks, is_, fbs, modes)
+    bw_rows = _softmax_bw_rows(x, is_[4])
+    _need(rows % bw_rows == 0, 'rows must be a multiple of the output quantizer table rows')
+    y = torch.empty_like(x)
+    i32 = dict(dtype=torch.int32, device=x.device)
+    a1 = torch.empty(1 if track_mask & 1 else 0, **i32)
+    a3 = torch.empty(1 if track_mask & 2 else 0, **i32)
+    ao = torch.empty(bw_rows * L if track_mask & 4 else 0, **i32)
+    rc = _lib.load().hgq_qsoftmax_fwd(_ptr(x), _ptr(y), rows, L, bw_rows, input_scaler, eps,
+                                      *[ctypes.addressof(d) for d in descs], _ptr(a1), _ptr(a3), _ptr(ao), _stream())
+    _lib.check(rc, 'hgq_qsoftmax_fwd')
+    return y, a1, a3, ao
+
+
+@qsoftmax_fwd.register_fake
+def _(x, ks, is_, fbs, modes, input_scaler, eps, track_mask):
+    L = x.shape[-1]
+    n_o = is_[4].numel() if track_mask & 4 else 0
+    return (torch.empty_like(x), x.new_empty(1 if track_mask & 1 else 0, dtype=torch.int32),
+            x.new_empty(1 if track_mask & 2 else 0, dtype=torch.int32), x.new_empty(n_o, dtype=torch.int32))
+
+
+@torch.library.custom_op('hgq::qsoftmax_bwd', mutates_args=())
+def qsoftmax_bwd(dy: Tensor, x: Tensor, ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor],
+                 modes: Sequence[int], input_scaler: float, eps: float) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    _check_f32('dy', dy), _check_f32('x', x)
+    _need(dy.shape == x.shape, 'dy and x differ in shape')
+    L = x.shape[-1]
+    rows = x.numel() // L
+    descs = _qdescs(ks, is_, fbs, modes)
+    has_oq = is_[4].numel() > 0
+    bw_rows = _softmax_bw_rows(x, is_[4])
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    f32 = dict(dtype=torch.float32, device=x.device)
+    g_shared = torch.empty(8, **f32)
+    g_oi = torch.empty(bw_rows * L if has_oq else 0, **f32)
+    g_of = torch.empty(bw_rows * L if has_oq else 0, **f32)
+    n_ws = lib.hgq_qsoftmax_bwd_workspace(rows, L, bw_rows, int(has_oq))
+    _need(n_ws >= 0, 'hgq_qsoftmax_bwd_workspace rejected the shape')
+    ws = torch.empty(max(int(n_ws), 1), **f32)
+    rc = lib.hgq_qsoftmax_bwd(_ptr(dy), _ptr(x), _ptr(dx), rows, L, bw_rows, input_scaler, eps,
+                              *[ctypes.addressof(d) for d in descs], _ptr(g_shared), _ptr(g_oi), _ptr(g_of), _ptr(ws), _stream())
+    _lib.check(rc, 'hgq_qsoftmax_bwd')
+    return dx, g_shared, g_oi, g_of
+
+
+@qsoftmax_bwd.register_fake
+def _(dy, x, ks, is_, fbs, modes, input_scaler, eps):
+    n_o = is_[4].numel()
+    return torch.empty_like(x), x.new_empty(8), x.new_empty(n_o), x.new_empty(n_o)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -371,6 +455,56 @@ def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, 
                              float(decay), beta if beta is not None else e_f, k_in, k_ker,
                              k_bias if k_bias is not None else e_k, ebops_var if ebops_var is not None else e_i, P, K, N,
                              float(scale), float(bias_size), mode_in, mode_ker, mode_bias)
+
+
+class _QSoftmax(torch.autograd.Function):
+    """Arguments after the scalars: k, i, fb of exp_iq, exp_oq, inv_iq, inv_oq, oq (15 tensors, empty = absent)."""
+
+    @staticmethod
+    def forward(ctx, x, modes, input_scaler, eps, track_mask, *qvars):
+        ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
+        y, a1, a3, ao = qsoftmax_fwd(x, ks, is_, fbs, list(modes), input_scaler, eps, track_mask)
+        ctx.save_for_backward(x, *qvars)
+        ctx.modes, ctx.input_scaler, ctx.eps = tuple(modes), input_scaler, eps
+        ctx.mark_non_differentiable(a1, a3, ao)
+        ctx.set_materialize_grads(False)
+        return y, a1, a3, ao
+
+    @staticmethod
+    def backward(ctx, gy, *_unused):
+        n_in = 5 + 15
+        if gy is None:
+            return (None,) * n_in
+        x, *qvars = ctx.saved_tensors
+        ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
+        dx, g_shared, g_oi, g_of = qsoftmax_bwd(gy.contiguous(), x, ks, is_, fbs, list(ctx.modes), ctx.input_scaler, ctx.eps)
+        grads = [dx if ctx.needs_input_grad[0] else None, None, None, None, None]
+        for n in range(5):
+            gi = g_shared[2 * n] if n < 4 else g_oi
+            gf = g_shared[2 * n + 1] if n < 4 else g_of
+            present = ks[n].numel() > 0
+            base = 5 + 3 * n
+            grads.append(None)
+            grads.append(gi.view(is_[n].shape) if present and ctx.needs_input_grad[base + 1] else None)
+            grads.append(gf.view(fbs[n].shape) if present and ctx.needs_input_grad[base + 2] else None)
+        return tuple(grads)
+
+
+def qsoftmax(x: Tensor, quantizers, input_scaler: float, eps: float, track_mask: int = 0):
+    """Table-driven softmax over the last axis.  ``quantizers`` = five entries (exp_iq, exp_oq, inv_iq,
+    inv_oq, oq), each ``None`` or ``(k, i, fb, mode)``.  Returns ``(y, amax_exp_iq, amax_inv_iq, amax_oq)``."""
+    e_f = x.new_empty(0)
+    e_k = torch.empty(0, dtype=torch.uint8, device=x.device)
+    flat, modes = [], []
+    for q in quantizers:
+        if q is None:
+            flat += [e_k, e_f, e_f]
+            modes.append(0)
+        else:
+            k, i, fb, mode = q
+            flat += [k.contiguous(), i.contiguous(), fb.contiguous()]
+            modes.append(int(mode))
+    return _QSoftmax.apply(x.contiguous(), tuple(modes), float(input_scaler), float(eps), int(track_mask), *flat)
 
 
 class _SparseCE(torch.autograd.Function):

@@ -232,6 +232,56 @@ int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, int64_t row
 int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
                        int64_t rows, float lr, float *loss, float *workspace, void *stream);
 
+/*
+ * Table-driven softmax, forward.  Replaces QSoftmax.call for the stable form without a mask
+ * (src/hgq/layers/softmax.py:119-136) together with the two QUnaryFunctionLUT tables it calls
+ * (src/hgq/layers/activation.py:58-61 and the input / output quantizers the layer wrapper applies
+ * around them, src/hgq/layers/core/base.py:88-116), i.e. for every row of L contiguous elements
+ *     d = max(x) - x;  e = Q_exp_oq(exp(-Q_exp_iq(d) * input_scaler));  s = sum(e);
+ *     r = Q_inv_oq(1 / (Q_inv_iq(s) + eps));  y = Q_oq(e * r)
+ * which the reference evaluates as about ten full passes over the score tensor
+ * (QMultiHeadAttention._compute_attention, src/hgq/layers/attn/mha.py:386-416 builds it with
+ * input_scaler = 1 / sqrt(key_dim)).
+ *
+ * A quantizer is described by its raw variables and mode bits; k == NULL (or a NULL descriptor)
+ * means the stage has no quantizer.  The four table quantizers have ONE bit-width entry each
+ * (the reference's default, allow_heterogeneous_table = False, softmax.py:59-63); the output
+ * quantizer has a [bw_rows, L] table, row r using table row r % bw_rows (bw_rows = 1 for a
+ * table shared by all rows).  L <= 256.
+ *
+ *   x, y [rows, L];
+ *   amax_exp_iq [1], amax_inv_iq [1], amax_oq [bw_rows * L]  optional: max |.| of the values the
+ *   respective quantizer produced, as uint32 bit patterns (for hgq_wrap_track_i; pass them for
+ *   KIF quantizers on their WRAP training branch, where the quantizer output is the rounded value).
+ */
+typedef struct {
+    const void *k;   /* keep-negative variable (fp32, or uint8 with HGQ_MODE_K_U8); NULL = no quantizer */
+    const float *i;  /* integer-bits variable */
+    const float *fb; /* fractional-bits (KIF) or total-bits (HGQ_MODE_KBI) variable */
+    int mode;        /* HGQ_MODE(round, overflow) | HGQ_MODE_* flags */
+} hgq_qdesc;
+int hgq_qsoftmax_fwd(const float *x, float *y, int64_t rows, int L, int64_t bw_rows, float input_scaler, float eps,
+                     const hgq_qdesc *exp_iq, const hgq_qdesc *exp_oq, const hgq_qdesc *inv_iq, const hgq_qdesc *inv_oq,
+                     const hgq_qdesc *oq, uint32_t *amax_exp_iq, uint32_t *amax_inv_iq, uint32_t *amax_oq, void *stream);
+
+/*
+ * Table-driven softmax, backward (training mode): autograd of the expression above, including
+ * the even split of the row maximum's gradient among ties (torch.amax) and the surrogate
+ * gradients of the five quantizers.  The forward chain is recomputed from x.
+ *
+ *   dy, x, dx [rows, L];
+ *   g_shared [8]: d loss / d (i, fb) of exp_iq, exp_oq, inv_iq, inv_oq in that order (fb = f or b;
+ *                 with HGQ_MODE_KBI the i entry is the total gradient, direct minus via f = b - i);
+ *   g_oq_i, g_oq_fb [bw_rows * L]: the same for the output quantizer (either may be NULL);
+ *   workspace: hgq_qsoftmax_bwd_workspace(rows, L, bw_rows, has_oq) floats for the per-wavefront
+ *   partial sums, which a second kernel adds up in a fixed order (deterministic).
+ */
+int64_t hgq_qsoftmax_bwd_workspace(int64_t rows, int L, int64_t bw_rows, int has_oq);
+int hgq_qsoftmax_bwd(const float *dy, const float *x, float *dx, int64_t rows, int L, int64_t bw_rows, float input_scaler,
+                     float eps, const hgq_qdesc *exp_iq, const hgq_qdesc *exp_oq, const hgq_qdesc *inv_iq,
+                     const hgq_qdesc *inv_oq, const hgq_qdesc *oq, float *g_shared, float *g_oq_i, float *g_oq_fb,
+                     float *workspace, void *stream);
+
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
 
