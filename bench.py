@@ -103,6 +103,68 @@ def quantizer_roofline(iters=200, with_copy=False):
     return out
 
 
+def softmax_roofline(iters=50, shape=(2048, 4, 64, 64), scaler=0.25):
+    """Table softmax of the attention configuration (scores [2048, 4, 64, 64], 8-bit exp / inverse
+    tables, per-position output quantizer): the one-pass kernels launched through the C ABI on
+    torch's current stream, timed with HIP events on that stream.  Algorithmic bytes: forward
+    8 B/element (scores in, probabilities out), backward 12 B/element (dy, scores in; dx out)."""
+    import torch
+
+    from hgq2_amd import _lib
+    from hgq2_amd.config import LayerConfigScope, QuantizerConfig, QuantizerConfigScope
+    from hgq2_amd.layers import QSoftmax
+
+    lib = _lib.load()
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(0)
+    with QuantizerConfigScope(place='all', default_q_type='kbi', overflow_mode='SAT_SYM'), \
+            QuantizerConfigScope(place='datalane', default_q_type='kif', overflow_mode='WRAP'), \
+            LayerConfigScope(enable_ebops=True, beta0=1e-5):
+        layer = QSoftmax(axis=-1, enable_oq=True, input_scaler=scaler,
+                         exp_iq_conf=QuantizerConfig(place='datalane', overflow_mode='SAT'))
+    n_sets = 3  # 3 x (scores + output + dy + dx) = 1.6 GB: every launch streams from HBM
+    sets = [tuple(torch.randn(shape, generator=g).to(dev) * (3.0 if j == 0 else 1.0) for j in range(2))
+            + (torch.empty(shape, device=dev), torch.empty(shape, device=dev)) for _ in range(n_sets)]
+    layer(sets[0][0], training=True)
+    qs = layer._fused_plan(sets[0][0], True, None)
+    assert qs is not None
+    descs = [_lib.QDesc(q[0].data_ptr(), q[1].data_ptr(), q[2].data_ptr(), q[3] | _lib.MODE_K_U8) for q in qs]
+    refs = [ctypes.addressof(d) for d in descs]
+    L = shape[-1]
+    n = 1
+    for d in shape:
+        n *= d
+    rows, bw_rows = n // L, qs[4][1].numel() // L
+    ws = torch.empty(lib.hgq_qsoftmax_bwd_workspace(rows, L, bw_rows, 1), device=dev)
+    a1, a3 = (torch.empty(1, dtype=torch.int32, device=dev) for _ in range(2))
+    ao = torch.empty(bw_rows * L, dtype=torch.int32, device=dev)
+    gsh, goi, gof = torch.empty(8, device=dev), torch.empty(bw_rows * L, device=dev), torch.empty(bw_rows * L, device=dev)
+    s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    state = {'n': 0}
+
+    def fwd():
+        x, dy, y, dx = sets[state['n'] % n_sets]
+        state['n'] += 1
+        rc = lib.hgq_qsoftmax_fwd(p(x), p(y), rows, L, bw_rows, scaler, 1e-7, *refs, None, p(a3), p(ao), s)
+        assert rc == 0
+
+    def bwd():
+        x, dy, y, dx = sets[state['n'] % n_sets]
+        state['n'] += 1
+        rc = lib.hgq_qsoftmax_bwd(p(dy), p(x), p(dx), rows, L, bw_rows, scaler, 1e-7, *refs, p(gsh), p(goi), p(gof), p(ws), s)
+        assert rc == 0
+
+    for _ in range(3):
+        fwd(), bwd()
+    out = {}
+    for name, fn, bpe in (('qsoftmax_fwd', fwd, 8), ('qsoftmax_bwd', bwd, 12)):
+        ms = _events_ms(fn, iters)
+        gbs = bpe * n / (ms * 1e-3) / 1e9
+        out[name] = {'ms': ms, 'bytes': bpe * n, 'GBps': gbs, 'frac': gbs / HBM_PEAK_GBS}
+    return out
+
+
 def cpu_baseline(budget_s=20.0):
     """The oracle's eager torch-CPU restatement of the reference path, same model and batch."""
     import torch
@@ -137,6 +199,8 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--roofline-only', action='store_true',
                     help='run only the standalone quantizer kernels and a plain copy of known size (for counter runs)')
+    ap.add_argument('--softmax-only', action='store_true',
+                    help='run only the one-pass table-softmax kernels at the attention configuration (for profiler runs)')
     ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused',
                     help='fused: whole-step kernels (3 launches); layers: per-layer torch.library operators with autograd; '
                          '-graph: the step is captured once in a HIP graph and replayed')
@@ -150,6 +214,10 @@ def main():
     if args.roofline_only:
         torch.cuda.set_device(0)
         print(json.dumps({'quantizer_kernels': quantizer_roofline(iters=20, with_copy=True)}))
+        return
+    if args.softmax_only:
+        torch.cuda.set_device(0)
+        print(json.dumps({'softmax_kernels': softmax_roofline(iters=20)}))
         return
 
     from hgq2_amd import ops

@@ -3,12 +3,15 @@
 //   d = max(x) - x;  e = Q_exp_out(exp(-Q_exp_in(d) * scale));  s = sum(e);
 //   r = Q_inv_out(1 / (Q_inv_in(s) + eps));  y = Q_out(e * r)
 //
-// A row (the softmax axis, contiguous, L <= 256 elements) lives in the lanes of one wavefront:
-// SUB lanes per row (a power of two >= L, or 64 lanes holding EPL elements each), 64 / SUB rows
-// side by side.  The four table quantizers have one shared bit-width entry each; the output
-// quantizer has a [P, L] table, row r using entry r % P.  A wavefront owns fixed table rows and
-// walks along the batch, so the output quantizer's operands, its abs-max tracker and its
-// bit-width gradients stay in registers; max / sum over the row are xor-shuffles.
+// Layout.  A row (the softmax axis, contiguous, L <= 256 elements) lives in SUB lanes of a
+// wavefront, VEC consecutive elements per lane (128-bit accesses when L is a multiple of 4), so a
+// wavefront holds 64 / SUB rows side by side and takes NP such groups per step: the row maximum
+// and sum are four DPP steps inside a 16-lane row (plus scalar-register reads across rows when a
+// row spans several), and the per-row stages (inverse table) are evaluated once for all rows of
+// the wavefront.  The four table quantizers have one shared bit-width entry each; the output
+// quantizer has a [P, L] table, row r using entry r % P.  A workgroup owns fixed table rows and
+// its wavefronts walk along the batch, so the output quantizer's operands, its abs-max tracker
+// and its bit-width gradients stay in registers and are combined through LDS once at the end.
 #include <math.h>
 
 #include "hgq_device.h"
@@ -16,245 +19,406 @@
 
 namespace hgq {
 
-// A quantizer with a single shared bit-width entry, resolved once per wavefront.
-struct SharedQ {
-    bool present, training, kbi;
-    int rm, om;
-    KIF p;
-    __device__ __forceinline__ void init(const hgq_qdesc &d) {
+// A quantizer whose mode is uniform over the wavefront, with every mode except inference-time
+// WRAP folded into constants so that the per-element code has no mode branches:
+//   rounding  r = conv ? rint(t) : floor(t + rc)     (rc = 0.5 for RND, -0 for TRN)
+//   overflow  clamp to [lo, hi]; modes that do not saturate use lo = -inf, hi = +inf
+// Arithmetic and operation order are those of quantize<> / quantize_grad<> in hgq_device.h.
+struct UniQ {
+    bool present, conv, sat, sym, kbi, wrap_inf, training;
+    float rc;
+    __device__ __forceinline__ void init_mode(const hgq_qdesc &d) {
         present = d.k != nullptr;
-        training = false, kbi = false, rm = 0, om = 0;
-        p.k = 0.f, p.i = 0.f, p.f = 0.f;
+        const Mode m(present ? d.mode : 0);
+        conv = m.round_mode == HGQ_RND_CONV;
+        rc = m.round_mode == HGQ_RND ? 0.5f : -0.0f;
+        sat = m.overflow_mode != HGQ_WRAP, sym = m.overflow_mode == HGQ_SAT_SYM;
+        kbi = m.kbi, training = m.training;
+        wrap_inf = present && !sat && !m.training;
+    }
+    __device__ __forceinline__ float round_at(float x, int fi) const {
+        const float t = ldexpf(x, fi);
+        const float r = conv ? rintf(t) : floorf(__fadd_rn(t, rc));
+        return ldexpf(r, -fi);
+    }
+    // two's-complement wrap of an already-rounded value (inference only)
+    static __device__ __forceinline__ float wrap(float xq, const KIF &p) {
+        int st;
+        return overflow<HGQ_WRAP>(xq, p, false, st);
+    }
+};
+
+// One shared bit-width entry: bounds and their derivatives are wavefront constants.
+struct SharedQ : UniQ {
+    KIF p;
+    int fi;
+    float hi, lo, gi_hi, gf_hi, gi_lo, gf_lo;
+    bool zero;
+    __device__ __forceinline__ void init(const hgq_qdesc &d) {
+        init_mode(d);
+        p.k = 0.f, p.i = 0.f, p.f = 0.f, fi = 0, zero = false;
+        hi = INFINITY, lo = -INFINITY, gi_hi = gf_hi = gi_lo = gf_lo = 0.f;
         if (!present) return;
         const Mode m(d.mode);
-        rm = m.round_mode, om = m.overflow_mode, training = m.training, kbi = m.kbi;
         p = resolve_kif(load_k(d.k, 0, m.k_u8), d.i[0], d.fb[0], m.kbi, m.round_params);
+        fi = (int)p.f;
+        zero = !training && !(p.k + p.i + p.f > 0.0f);
+        if (sat) {
+            const float eps = pow2(-p.f);
+            hi = __fsub_rn(pow2(p.i), eps);
+            lo = sym ? -p.k * hi : -p.k * pow2(p.i);
+            gi_hi = HGQ_LN2 * pow2(p.i), gf_hi = HGQ_LN2 * eps;
+            gi_lo = -p.k * gi_hi, gf_lo = sym ? -p.k * gf_hi : 0.f;
+        }
+        // the values are the same in every lane: pin them to scalar registers
+        fi = __builtin_amdgcn_readfirstlane(fi);
+        hi = uniform(hi), lo = uniform(lo), gi_hi = uniform(gi_hi), gf_hi = uniform(gf_hi), gi_lo = uniform(gi_lo), gf_lo = uniform(gf_lo);
+        p.k = uniform(p.k), p.i = uniform(p.i), p.f = uniform(p.f);
     }
-    __device__ __forceinline__ float fwd(float x) const { return present ? quantize_dyn(x, p, rm, om, training) : x; }
-    // gradients w.r.t. the input and the two stored variables (i and f, or i and b)
+    static __device__ __forceinline__ float uniform(float v) {
+        return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+    }
+    __device__ __forceinline__ float fwd(float x) const {
+        if (!present) return x;
+        const float xq = round_at(x, fi);
+        float y = xq > hi ? hi : (xq < lo ? lo : xq);
+        if (wrap_inf) y = wrap(xq, p);
+        return zero ? 0.f : y;
+    }
+    // gradients w.r.t. the input and the two stored variables (i and f, or i and b), training mode
     __device__ __forceinline__ void grad(float x, float dy, float &dx, float &di, float &dfb) const {
         if (!present) {
             dx = dy, di = 0.f, dfb = 0.f;
             return;
         }
-        quantize_grad_dyn(x, dy, p, rm, om, dx, di, dfb);
+        const float xq = round_at(x, fi);
+        const bool over = xq > hi, under = xq < lo;
+        const float ste_f = -HGQ_LN2 * (xq - x) * dy;
+        const float oi = over ? gi_hi * dy : 0.f, of = over ? gf_hi * dy : 0.f;
+        const float ui = under ? gi_lo * dy : 0.f, uf = under ? gf_lo * dy : 0.f;
+        const bool in = !(over || under);
+        dx = in ? dy : 0.f;
+        di = oi + ui;
+        dfb = in ? ste_f : of + uf;
         if (kbi) di -= dfb;  // f = b - i
     }
 };
 
-// The output quantizer: per-lane operands.
-struct LaneQ {
-    int rm, om;
-    bool present, training, kbi;
-    __device__ __forceinline__ void init(const hgq_qdesc &d) {
-        present = d.k != nullptr;
-        const Mode m(present ? d.mode : 0);
-        rm = m.round_mode, om = m.overflow_mode, training = m.training, kbi = m.kbi;
-    }
-    __device__ __forceinline__ KIF load(const hgq_qdesc &d, int64_t idx) const {
+// The output quantizer: operands differ per lane (packed into one register per element: f in
+// bits 0-7, i in bits 8-15, both as signed bytes, k in bit 16), the mode is uniform.
+struct LaneQ : UniQ {
+    __device__ __forceinline__ void init(const hgq_qdesc &d) { init_mode(d); }
+    static __device__ __forceinline__ int clamp8(float v) { return (int)fminf(fmaxf(v, -128.f), 127.f); }
+    __device__ __forceinline__ int load(const hgq_qdesc &d, int64_t idx) const {
         const Mode m(d.mode);
-        return resolve_kif(load_k(d.k, idx, m.k_u8), d.i[idx], d.fb[idx], m.kbi, m.round_params);
+        const KIF p = resolve_kif(load_k(d.k, idx, m.k_u8), d.i[idx], d.fb[idx], m.kbi, m.round_params);
+        return (clamp8(p.f) & 0xff) | ((clamp8(p.i) & 0xff) << 8) | (p.k != 0.f ? 1 << 16 : 0);
+    }
+    static __device__ __forceinline__ int f_of(int pk) { return (int)(int8_t)(pk & 0xff); }
+    static __device__ __forceinline__ int i_of(int pk) { return (int)(int8_t)((pk >> 8) & 0xff); }
+    static __device__ __forceinline__ float k_of(int pk) { return (pk >> 16) & 1 ? 1.f : 0.f; }
+    __device__ __forceinline__ float fwd(float x, int pk) const {
+        const int fi = f_of(pk);
+        const float xq = round_at(x, fi);
+        float y = xq;
+        if (sat) {
+            const float k = k_of(pk), pi = ldexpf(1.0f, i_of(pk));
+            const float hi = __fsub_rn(pi, ldexpf(1.0f, -fi));
+            const float lo = sym ? -k * hi : -k * pi;
+            y = xq > hi ? hi : (xq < lo ? lo : xq);
+        } else if (wrap_inf) {
+            KIF p;
+            p.k = k_of(pk), p.i = (float)i_of(pk), p.f = (float)fi;
+            y = wrap(xq, p);
+        }
+        if (!training && !(k_of(pk) + (float)(i_of(pk) + fi) > 0.0f)) y = 0.f;
+        return y;
+    }
+    __device__ __forceinline__ void grad(float x, float dy, int pk, float &dx, float &di, float &dfb) const {
+        const int fi = f_of(pk);
+        const float xq = round_at(x, fi);
+        dx = dy, di = 0.f;
+        dfb = -HGQ_LN2 * (xq - x) * dy;
+        if (sat) {
+            const float k = k_of(pk), eps = ldexpf(1.0f, -fi), pi = ldexpf(1.0f, i_of(pk));
+            const float hi = __fsub_rn(pi, eps);
+            const float lo = sym ? -k * hi : -k * pi;
+            const bool over = xq > hi, under = xq < lo;
+            if (over || under) {
+                const float gi = HGQ_LN2 * pi * dy, gf = HGQ_LN2 * eps * dy;
+                dx = 0.f;
+                di = (over ? gi : 0.f) + (under ? -k * gi : 0.f);
+                dfb = (over ? gf : 0.f) + ((under && sym) ? -k * gf : 0.f);
+            }
+        }
+        if (kbi) di -= dfb;
     }
 };
 
-template <int SUB>
-__device__ __forceinline__ float sub_max(float v) {
-#pragma unroll
-    for (int o = SUB / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+// ------------------------------------------------------------------------------------------
+// all-reduce over the SUB lanes of a row: four DPP steps inside each 16-lane row (xor 1, xor 2,
+// half-row mirror, row mirror), then the row totals are read back through scalar registers
+// ------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+struct OpMax {
+    static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
+};
+struct OpAdd {
+    static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+};
+template <int SUB, class Op>
+__device__ __forceinline__ float sub_reduce(float v) {
+    v = Op::f(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = Op::f(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = Op::f(v, dpp_mov<0x141>(v));  // row_half_mirror
+    v = Op::f(v, dpp_mov<0x140>(v));  // row_mirror
+    if (SUB == 16) return v;
+    const float r0 = lane_value(v, 0), r1 = lane_value(v, 16), r2 = lane_value(v, 32), r3 = lane_value(v, 48);
+    const float a = Op::f(r0, r1), b = Op::f(r2, r3);
+    if (SUB == 32) return (threadIdx.x & 32) ? b : a;
+    return Op::f(a, b);
 }
 template <int SUB>
-__device__ __forceinline__ float sub_sum(float v) {
-#pragma unroll
-    for (int o = SUB / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
-__device__ __forceinline__ float wave_sum(float v) { return sub_sum<64>(v); }
+__device__ __forceinline__ float sub_max(float v) { return sub_reduce<SUB, OpMax>(v); }
+template <int SUB>
+__device__ __forceinline__ float sub_sum(float v) { return sub_reduce<SUB, OpAdd>(v); }
+__device__ __forceinline__ float wave_sum(float v) { return sub_reduce<64, OpAdd>(v); }
 __device__ __forceinline__ uint32_t wave_max_bits(uint32_t v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const uint32_t t = (uint32_t)__shfl_xor((int)v, o, 64);
-        v = t > v ? t : v;
-    }
-    return v;
+    // non-negative floats order like their bit patterns
+    return __float_as_uint(sub_reduce<64, OpMax>(__uint_as_float(v)));
 }
 
-// Work decomposition shared by the forward and backward kernels.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <int VEC>
+__device__ __forceinline__ void row_load(const float *p, float *o) {
+    if (VEC == 4) {
+        const f32x4 t = __builtin_nontemporal_load((const f32x4 *)p);
+        o[0] = t.x, o[1] = t.y, o[2] = t.z, o[3] = t.w;
+    } else {
+        o[0] = __builtin_nontemporal_load(p);
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void row_store(float *p, const float *o) {
+    if (VEC == 4) {
+        f32x4 t;
+        t.x = o[0], t.y = o[1], t.z = o[2], t.w = o[3];
+        __builtin_nontemporal_store(t, (f32x4 *)p);
+    } else {
+        __builtin_nontemporal_store(o[0], p);
+    }
+}
+
+#define SM_WPB 8  // wavefronts per workgroup
+
+// Work decomposition shared by the forward and backward kernels.  Workgroup (pg, chunk) owns the
+// table rows [pg * RI, (pg + 1) * RI) with RI = NP * 64 / SUB and the batches of its chunk;
+// wavefront w of the workgroup takes batches b0 + w, b0 + w + SM_WPB, ...
 struct SoftmaxPlan {
     int64_t rows;       // number of softmax rows
     int L;              // row length
-    int64_t Pq;         // table rows walked by the grid (a multiple of the rows one wavefront takes per step)
+    int64_t Pq;         // table rows walked by the grid (a multiple of RI)
     int64_t P_table;    // rows of the output quantizer's bit-width table (1 if shared or absent)
     int64_t n_batches;  // ceil(rows / Pq)
-    int64_t PG;         // position groups = Pq / (rows per wavefront step)
+    int64_t PG;         // position groups = Pq / RI
     int bpc;            // batches per chunk
     int64_t n_chunks;
-    int SUB, EPL, NP;
-    __host__ __device__ int64_t n_waves() const { return PG * n_chunks; }
+    int SUB, VEC, NP;
+    __host__ __device__ int64_t n_blocks() const { return PG * n_chunks; }
 };
 
-#define SM_WAVES_PER_BLOCK 4
+// Per-wavefront constants of the walk.
+template <int SUB, int VEC, int NP>
+struct Walk {
+    static constexpr int RPW = 64 / SUB;
+    int lane, col;
+    bool col_on;
+    int nb;           // steps of this wavefront
+    int64_t stride;   // elements between consecutive steps
+    int64_t off[NP];  // element offset of this lane's first element at step 0
+    int tcol[NP];     // offset into the output quantizer's table
+    int wcol[NP];     // offset into a [Pq, L] slice
+    int blim[NP];     // number of steps whose row exists
+    __device__ __forceinline__ void init(const SoftmaxPlan &pl) {
+        const int wave = threadIdx.x >> 6;
+        lane = threadIdx.x & 63;
+        const int slot = lane / SUB;
+        col = (lane % SUB) * VEC;
+        col_on = col < pl.L;
+        const int64_t pg = blockIdx.x % pl.PG, chunk = blockIdx.x / pl.PG;
+        const int64_t b0 = chunk * pl.bpc + wave, b1 = min(pl.n_batches, chunk * pl.bpc + pl.bpc);
+        nb = b0 < b1 ? (int)((b1 - b0 + SM_WPB - 1) / SM_WPB) : 0;
+        stride = (int64_t)SM_WPB * pl.Pq * pl.L;
+#pragma unroll
+        for (int np = 0; np < NP; ++np) {
+            const int64_t pos = (pg * NP + np) * RPW + slot;
+            const int64_t first = b0 * pl.Pq + pos;
+            off[np] = first * pl.L + col;
+            tcol[np] = (int)((pos % pl.P_table) * pl.L) + col;
+            wcol[np] = (int)(pos * pl.L) + col;
+            const int64_t step_rows = (int64_t)SM_WPB * pl.Pq;
+            const int64_t left = first < pl.rows ? (pl.rows - first + step_rows - 1) / step_rows : 0;
+            blim[np] = (int)min((int64_t)nb, left);
+        }
+    }
+};
 
-template <int SUB, int EPL, int NP>
-__global__ __launch_bounds__(64 * SM_WAVES_PER_BLOCK) void qsoftmax_fwd_kernel(
+template <int SUB, int VEC, int NP>
+__global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_fwd_kernel(
     const float *__restrict__ x, float *__restrict__ y, SoftmaxPlan pl, float scale, float eps, hgq_qdesc d1, hgq_qdesc d2,
     hgq_qdesc d3, hgq_qdesc d4, hgq_qdesc dq, uint32_t *amax1, uint32_t *amax3, uint32_t *amax_o) {
-    constexpr int RPW = 64 / SUB;
-    const int64_t gw = (int64_t)blockIdx.x * SM_WAVES_PER_BLOCK + (threadIdx.x >> 6);
-    if (gw >= pl.n_waves()) return;
-    const int lane = threadIdx.x & 63, slot = lane / SUB, col = lane % SUB;
-    const int64_t pg = gw % pl.PG, chunk = gw / pl.PG;
+    __shared__ uint32_t lds_max[SM_WPB][NP * VEC][64];
+    __shared__ uint32_t lds_m13[SM_WPB][2];
+    Walk<SUB, VEC, NP> wk;
+    wk.init(pl);
     SharedQ q1, q2, q3, q4;
     q1.init(d1), q2.init(d2), q3.init(d3), q4.init(d4);
     LaneQ qo;
     qo.init(dq);
-    const int L = pl.L;
-    KIF po[NP][EPL];
-    uint32_t mo[NP][EPL];
-    int64_t pos[NP];
+    int po[NP][VEC];
+    uint32_t mo[NP][VEC];
 #pragma unroll
-    for (int np = 0; np < NP; ++np) {
-        pos[np] = (pg * NP + np) * RPW + slot;
+    for (int np = 0; np < NP; ++np)
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            mo[np][e] = 0;
-            const int c = col + 64 * e;
-            po[np][e].k = 0.f, po[np][e].i = 0.f, po[np][e].f = 0.f;
-            if (qo.present && c < L) po[np][e] = qo.load(dq, (pos[np] % pl.P_table) * L + c);
+        for (int e = 0; e < VEC; ++e) {
+            mo[np][e] = 0, po[np][e] = 0;
+            if (qo.present && wk.col_on) po[np][e] = qo.load(dq, wk.tcol[np] + e);
         }
-    }
     uint32_t m1 = 0, m3 = 0;
-    const int64_t b0 = chunk * pl.bpc, b1 = min(pl.n_batches, b0 + pl.bpc);
-    for (int64_t b = b0; b < b1; ++b) {
-        float xv[NP][EPL];
-        bool act[NP][EPL];
+    for (int b = 0; b < wk.nb; ++b) {
+        float xv[NP][VEC];
+        bool act[NP];
 #pragma unroll
         for (int np = 0; np < NP; ++np) {
-            const int64_t r = b * pl.Pq + pos[np];
+            act[np] = b < wk.blim[np] && wk.col_on;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                const int c = col + 64 * e;
-                act[np][e] = r < pl.rows && c < L;
-                xv[np][e] = act[np][e] ? __builtin_nontemporal_load(x + r * L + c) : -INFINITY;
-            }
+            for (int e = 0; e < VEC; ++e) xv[np][e] = -INFINITY;
+            if (act[np]) row_load<VEC>(x + wk.off[np], xv[np]);
         }
 #pragma unroll
         for (int np = 0; np < NP; ++np) {
-            const int64_t r = b * pl.Pq + pos[np];
             float mx = xv[np][0];
 #pragma unroll
-            for (int e = 1; e < EPL; ++e) mx = fmaxf(mx, xv[np][e]);
+            for (int e = 1; e < VEC; ++e) mx = fmaxf(mx, xv[np][e]);
             mx = sub_max<SUB>(mx);
-            float ev[EPL], s = 0.f;
+            float ev[VEC], s = 0.f;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                const float d = __fsub_rn(mx, xv[np][e]);
+            for (int e = 0; e < VEC; ++e) {
+                const float d = act[np] ? __fsub_rn(mx, xv[np][e]) : 0.f;
                 const float a = q1.fwd(d);
                 const float t = expf(__fmul_rn(-a, scale));
-                ev[e] = act[np][e] ? q2.fwd(t) : 0.f;
-                if (act[np][e]) m1 = max(m1, abs_bits(a));
+                ev[e] = act[np] ? q2.fwd(t) : 0.f;
+                m1 = max(m1, abs_bits(a));
                 s += ev[e];
             }
             s = sub_sum<SUB>(s);
             const float sq = q3.fwd(s);
             const float rr = q4.fwd(__fdiv_rn(1.0f, __fadd_rn(sq, eps)));
-            if (r < pl.rows) m3 = max(m3, abs_bits(sq));
+            if (b < wk.blim[np]) m3 = max(m3, abs_bits(sq));
+            float yv[VEC];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                float yv = __fmul_rn(ev[e], rr);
-                if (qo.present) yv = quantize_dyn(yv, po[np][e], qo.rm, qo.om, qo.training);
-                if (act[np][e]) {
-                    __builtin_nontemporal_store(yv, y + r * L + col + 64 * e);
-                    mo[np][e] = max(mo[np][e], abs_bits(yv));
-                }
+            for (int e = 0; e < VEC; ++e) {
+                yv[e] = __fmul_rn(ev[e], rr);
+                if (qo.present) yv[e] = qo.fwd(yv[e], po[np][e]);
+                if (act[np]) mo[np][e] = max(mo[np][e], abs_bits(yv[e]));
             }
+            if (act[np]) row_store<VEC>(y + wk.off[np], yv);
+            wk.off[np] += wk.stride;
         }
     }
-    if (amax1) {
-        m1 = wave_max_bits(m1);
-        if (lane == 0) atomicMax(amax1, m1);
-    }
-    if (amax3) {
-        m3 = wave_max_bits(m3);
-        if (lane == 0) atomicMax(amax3, m3);
+    // combine the trackers of the workgroup's wavefronts, then one atomic per entry
+    const int wave = threadIdx.x >> 6;
+    if (amax1 || amax3) {
+        m1 = wave_max_bits(m1), m3 = wave_max_bits(m3);
+        if (wk.lane == 0) lds_m13[wave][0] = m1, lds_m13[wave][1] = m3;
     }
     if (amax_o) {
 #pragma unroll
         for (int np = 0; np < NP; ++np)
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                const int c = col + 64 * e;
-                if (c < L && mo[np][e]) atomicMax(&amax_o[(pos[np] % pl.P_table) * L + c], mo[np][e]);
+            for (int e = 0; e < VEC; ++e) lds_max[wave][np * VEC + e][wk.lane] = mo[np][e];
+    }
+    __syncthreads();
+    if (threadIdx.x < 2 && (amax1 || amax3)) {
+        uint32_t m = 0;
+        for (int w = 0; w < SM_WPB; ++w) m = max(m, lds_m13[w][threadIdx.x]);
+        uint32_t *dst = threadIdx.x == 0 ? amax1 : amax3;
+        if (dst) atomicMax(dst, m);
+    }
+    if (amax_o && wave == 0 && wk.col_on) {
+#pragma unroll
+        for (int np = 0; np < NP; ++np)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                uint32_t m = 0;
+                for (int w = 0; w < SM_WPB; ++w) m = max(m, lds_max[w][np * VEC + e][wk.lane]);
+                if (m) atomicMax(&amax_o[wk.tcol[np] + e], m);
             }
     }
 }
 
-// Backward: recomputes the forward chain from x, then walks it in reverse.  Per-wavefront
-// partial sums of the bit-width gradients go to workspace slices that a second kernel adds up
-// in a fixed order.
-//   workspace = [n_waves, 8] scalar slices | [n_chunks, Pq * L] d/di of Q_out | [n_chunks, Pq * L] d/df of Q_out
-template <int SUB, int EPL, int NP>
-__global__ __launch_bounds__(64 * SM_WAVES_PER_BLOCK) void qsoftmax_bwd_kernel(
+// Backward: recomputes the forward chain from x, then walks it in reverse.  Partial sums of the
+// bit-width gradients go to workspace slices that a second kernel adds up in a fixed order.
+//   workspace = [n_blocks, 8] shared-quantizer slices | [n_chunks, Pq * L] d/df of Q_out | [n_chunks, Pq * L] d/di of Q_out
+// OQ_GI: the output quantizer saturates, so its integer bits take gradient (else that slice is not written).
+template <int SUB, int VEC, int NP, bool OQ_GI>
+__global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_bwd_kernel(
     const float *__restrict__ dy, const float *__restrict__ x, float *__restrict__ dx, SoftmaxPlan pl, float scale,
     float eps, hgq_qdesc d1, hgq_qdesc d2, hgq_qdesc d3, hgq_qdesc d4, hgq_qdesc dq, float *__restrict__ ws) {
-    constexpr int RPW = 64 / SUB;
-    const int64_t gw = (int64_t)blockIdx.x * SM_WAVES_PER_BLOCK + (threadIdx.x >> 6);
-    if (gw >= pl.n_waves()) return;
-    const int lane = threadIdx.x & 63, slot = lane / SUB, col = lane % SUB;
-    const int64_t pg = gw % pl.PG, chunk = gw / pl.PG;
+    __shared__ float lds_g[SM_WPB][NP * VEC][64];
+    __shared__ float part[SM_WPB][8];
+    Walk<SUB, VEC, NP> wk;
+    wk.init(pl);
     SharedQ q1, q2, q3, q4;
     q1.init(d1), q2.init(d2), q3.init(d3), q4.init(d4);
     LaneQ qo;
     qo.init(dq);
-    const int L = pl.L;
-    KIF po[NP][EPL];
-    float goi[NP][EPL], gof[NP][EPL];
-    int64_t pos[NP];
+    int po[NP][VEC];
+    float gof[NP][VEC], goi[OQ_GI ? NP : 1][VEC];
 #pragma unroll
-    for (int np = 0; np < NP; ++np) {
-        pos[np] = (pg * NP + np) * RPW + slot;
+    for (int np = 0; np < NP; ++np)
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            goi[np][e] = 0.f, gof[np][e] = 0.f;
-            const int c = col + 64 * e;
-            po[np][e].k = 0.f, po[np][e].i = 0.f, po[np][e].f = 0.f;
-            if (qo.present && c < L) po[np][e] = qo.load(dq, (pos[np] % pl.P_table) * L + c);
+        for (int e = 0; e < VEC; ++e) {
+            gof[np][e] = 0.f, po[np][e] = 0;
+            if (OQ_GI) goi[np][e] = 0.f;
+            if (qo.present && wk.col_on) po[np][e] = qo.load(dq, wk.tcol[np] + e);
         }
-    }
     float gs[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) gs[j] = 0.f;
-    const int64_t b0 = chunk * pl.bpc, b1 = min(pl.n_batches, b0 + pl.bpc);
-    for (int64_t b = b0; b < b1; ++b) {
-        float xv[NP][EPL], gv[NP][EPL];
-        bool act[NP][EPL];
+    const bool row_lead = wk.col == 0;
+    for (int b = 0; b < wk.nb; ++b) {
+        float xv[NP][VEC], gv[NP][VEC];
+        bool act[NP];
 #pragma unroll
         for (int np = 0; np < NP; ++np) {
-            const int64_t r = b * pl.Pq + pos[np];
+            act[np] = b < wk.blim[np] && wk.col_on;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                const int c = col + 64 * e;
-                act[np][e] = r < pl.rows && c < L;
-                xv[np][e] = act[np][e] ? __builtin_nontemporal_load(x + r * L + c) : -INFINITY;
-                gv[np][e] = act[np][e] ? __builtin_nontemporal_load(dy + r * L + c) : 0.f;
+            for (int e = 0; e < VEC; ++e) xv[np][e] = -INFINITY, gv[np][e] = 0.f;
+            if (act[np]) {
+                row_load<VEC>(x + wk.off[np], xv[np]);
+                row_load<VEC>(dy + wk.off[np], gv[np]);
             }
         }
 #pragma unroll
         for (int np = 0; np < NP; ++np) {
-            const int64_t r = b * pl.Pq + pos[np];
-            const bool row_on = r < pl.rows;
             // ---- forward chain
             float mx = xv[np][0];
 #pragma unroll
-            for (int e = 1; e < EPL; ++e) mx = fmaxf(mx, xv[np][e]);
+            for (int e = 1; e < VEC; ++e) mx = fmaxf(mx, xv[np][e]);
             mx = sub_max<SUB>(mx);
-            float dv[EPL], av[EPL], tv[EPL], ev[EPL], s = 0.f;
+            float dv[VEC], tv[VEC], ev[VEC], s = 0.f;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                dv[e] = act[np][e] ? __fsub_rn(mx, xv[np][e]) : 0.f;
-                av[e] = q1.fwd(dv[e]);
-                tv[e] = expf(__fmul_rn(-av[e], scale));
-                ev[e] = act[np][e] ? q2.fwd(tv[e]) : 0.f;
+            for (int e = 0; e < VEC; ++e) {
+                dv[e] = act[np] ? __fsub_rn(mx, xv[np][e]) : 0.f;
+                tv[e] = expf(__fmul_rn(-q1.fwd(dv[e]), scale));
+                ev[e] = act[np] ? q2.fwd(tv[e]) : 0.f;
                 s += ev[e];
             }
             s = sub_sum<SUB>(s);
@@ -262,140 +426,211 @@ __global__ __launch_bounds__(64 * SM_WAVES_PER_BLOCK) void qsoftmax_bwd_kernel(
             const float r0 = __fdiv_rn(1.0f, __fadd_rn(sq, eps));
             const float rr = q4.fwd(r0);
             // ---- backward chain
-            float g0[EPL], drr = 0.f;
+            float g0[VEC], drr = 0.f;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                const float y0 = __fmul_rn(ev[e], rr);
+            for (int e = 0; e < VEC; ++e) {
                 float gx = gv[np][e];
                 if (qo.present) {
                     float gi, gf;
-                    quantize_grad_dyn(y0, gv[np][e], po[np][e], qo.rm, qo.om, gx, gi, gf);
-                    if (qo.kbi) gi -= gf;
-                    if (act[np][e]) goi[np][e] += gi, gof[np][e] += gf;
+                    qo.grad(__fmul_rn(ev[e], rr), gv[np][e], po[np][e], gx, gi, gf);
+                    gof[np][e] += gf;  // dy is zero on inactive lanes
+                    if (OQ_GI) goi[np][e] += gi;
                 }
-                g0[e] = act[np][e] ? gx : 0.f;
+                g0[e] = gx;
                 drr += g0[e] * ev[e];
             }
             drr = sub_sum<SUB>(drr);
-            float dr0, gi4, gf4, dsq, gi3, gf3, ds;
+            float dr0, gi4, gf4, ds, gi3, gf3;
             q4.grad(r0, drr, dr0, gi4, gf4);
-            dsq = dr0 * -(r0 * r0);
-            q3.grad(s, dsq, ds, gi3, gf3);
-            if (row_on && col == 0) gs[6] += gi4, gs[7] += gf4, gs[4] += gi3, gs[5] += gf3;
-            float dd[EPL], dm = 0.f, cnt = 0.f;
+            q3.grad(s, dr0 * -(r0 * r0), ds, gi3, gf3);
+            if (b < wk.blim[np] && row_lead) gs[6] += gi4, gs[7] += gf4, gs[4] += gi3, gs[5] += gf3;
+            float dd[VEC], dm = 0.f, cnt = 0.f;
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
+            for (int e = 0; e < VEC; ++e) {
                 const float de = g0[e] * rr + ds;
                 float dt, gi2, gf2, gi1, gf1;
                 q2.grad(tv[e], de, dt, gi2, gf2);
-                const float da = -((dt * tv[e]) * scale);
-                q1.grad(dv[e], da, dd[e], gi1, gf1);
-                if (act[np][e]) {
+                q1.grad(dv[e], -((dt * tv[e]) * scale), dd[e], gi1, gf1);
+                if (act[np]) {
                     gs[2] += gi2, gs[3] += gf2, gs[0] += gi1, gs[1] += gf1;
                     dm += dd[e];
                     cnt += (xv[np][e] == mx) ? 1.f : 0.f;
-                } else {
-                    dd[e] = 0.f;
                 }
             }
             dm = sub_sum<SUB>(dm);
             cnt = sub_sum<SUB>(cnt);
             const float share = dm / cnt;  // the maximum's gradient is split evenly among ties
+            float ov[VEC];
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                if (act[np][e]) {
-                    const float g = (xv[np][e] == mx) ? share - dd[e] : -dd[e];
-                    __builtin_nontemporal_store(g, dx + r * L + col + 64 * e);
-                }
-            }
+            for (int e = 0; e < VEC; ++e) ov[e] = (xv[np][e] == mx) ? share - dd[e] : -dd[e];
+            if (act[np]) row_store<VEC>(dx + wk.off[np], ov);
+            wk.off[np] += wk.stride;
         }
     }
+    // shared-quantizer gradients: wavefront sums, then the workgroup's in a fixed order
+    const int wave = threadIdx.x >> 6;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float v = wave_sum(gs[j]);
-        if (lane == 0) ws[gw * 8 + j] = v;
+        if (wk.lane == 0) part[wave][j] = v;
     }
     if (qo.present) {
-        const int64_t PL = pl.Pq * L;
-        float *wi = ws + pl.n_waves() * 8 + chunk * PL;
-        float *wf = wi + pl.n_chunks * PL;
 #pragma unroll
         for (int np = 0; np < NP; ++np)
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                const int c = col + 64 * e;
-                if (c < L) wi[pos[np] * L + c] = goi[np][e], wf[pos[np] * L + c] = gof[np][e];
+            for (int e = 0; e < VEC; ++e) lds_g[wave][np * VEC + e][wk.lane] = gof[np][e];
+    }
+    __syncthreads();
+    if (threadIdx.x < 8) {
+        float s = 0.f;
+        for (int w = 0; w < SM_WPB; ++w) s += part[w][threadIdx.x];
+        ws[(int64_t)blockIdx.x * 8 + threadIdx.x] = s;
+    }
+    if (!qo.present) return;
+    const int64_t PL = pl.Pq * pl.L;
+    const int64_t chunk = blockIdx.x / pl.PG;
+    float *wf = ws + pl.n_blocks() * 8 + chunk * PL;
+    if (wave == 0 && wk.col_on) {
+#pragma unroll
+        for (int np = 0; np < NP; ++np)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float s = 0.f;
+                for (int w = 0; w < SM_WPB; ++w) s += lds_g[w][np * VEC + e][wk.lane];
+                wf[wk.wcol[np] + e] = s;
             }
+    }
+    if (OQ_GI) {
+        __syncthreads();
+#pragma unroll
+        for (int np = 0; np < NP; ++np)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) lds_g[wave][np * VEC + e][wk.lane] = goi[np][e];
+        __syncthreads();
+        float *wi = wf + pl.n_chunks * PL;
+        if (wave == 0 && wk.col_on) {
+#pragma unroll
+            for (int np = 0; np < NP; ++np)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float s = 0.f;
+                    for (int w = 0; w < SM_WPB; ++w) s += lds_g[w][np * VEC + e][wk.lane];
+                    wi[wk.wcol[np] + e] = s;
+                }
+        }
     }
 }
 
 // Fixed-order sums of the backward kernel's slices.
 //   block 0: the eight shared-quantizer gradients;  blocks 1..: 64 output-quantizer entries each
-__global__ __launch_bounds__(256) void qsoftmax_reduce_kernel(const float *__restrict__ ws, SoftmaxPlan pl, float *g_shared,
-                                                              float *g_oi, float *g_of) {
-    __shared__ float red[256];
+__global__ __launch_bounds__(1024) void qsoftmax_reduce_kernel(const float *__restrict__ ws, SoftmaxPlan pl, float *g_shared,
+                                                               float *g_oi, float *g_of, int oq_gi) {
+    __shared__ float red[1024];
     const int t = threadIdx.x;
-    const int64_t nw = pl.n_waves();
+    const int64_t nblk = pl.n_blocks();
     if (blockIdx.x == 0) {
-        // thread t sums slice entries j = t % 8 of waves t / 8, t / 8 + 32, ...
+        // thread t sums entry j = t % 8 of slices t / 8, t / 8 + 128, ...; eight loads in flight
         const int j = t & 7;
         float s = 0.f;
-        for (int64_t w = t >> 3; w < nw; w += 32) s += ws[w * 8 + j];
+        int64_t w = t >> 3;
+        for (; w + 7 * 128 < nblk; w += 8 * 128) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = ws[(w + u * 128) * 8 + j];
+            s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+        }
+        for (; w < nblk; w += 128) s += ws[w * 8 + j];
         red[t] = s;
         __syncthreads();
-        for (int o = 128; o >= 8; o >>= 1) {
+        for (int o = 512; o >= 8; o >>= 1) {
             if (t < o) red[t] += red[t + o];
             __syncthreads();
         }
         if (t < 8 && g_shared) g_shared[t] = red[t];
         return;
     }
-    if (!g_oi && !g_of) return;
     const int64_t PL = pl.Pq * pl.L, M = pl.P_table * pl.L;
-    const int64_t fold = pl.Pq / pl.P_table;  // table rows aliased by several walked rows (shared table)
+    const int64_t fold = pl.Pq / pl.P_table;  // walked rows that alias one table row (shared table)
     const int64_t n_slices = pl.n_chunks * fold;
-    const int e_local = t & 63, grp = t >> 6;
+    const int e_local = t & 63, grp = t >> 6;  // 16 slice groups x 64 entries
     const int64_t e = (int64_t)(blockIdx.x - 1) * 64 + e_local;
-    const float *wi = ws + nw * 8, *wf = wi + pl.n_chunks * PL;
+    const float *wf = ws + nblk * 8, *wi = wf + pl.n_chunks * PL;
     float si = 0.f, sf = 0.f;
     if (e < M) {
-        for (int64_t sl = grp; sl < n_slices; sl += 4) {
-            const int64_t off = (sl / fold) * PL + (sl % fold) * M + e;
-            si += wi[off], sf += wf[off];
+        for (int64_t sl = grp; sl < n_slices; sl += 16) {
+            const int64_t o = (sl / fold) * PL + (sl % fold) * M + e;
+            sf += wf[o];
+            if (oq_gi) si += wi[o];
         }
     }
-    red[t] = si;
-    __syncthreads();
-    if (grp == 0 && e < M && g_oi) g_oi[e] = (red[e_local] + red[e_local + 64]) + (red[e_local + 128] + red[e_local + 192]);
-    __syncthreads();
     red[t] = sf;
     __syncthreads();
-    if (grp == 0 && e < M && g_of) g_of[e] = (red[e_local] + red[e_local + 64]) + (red[e_local + 128] + red[e_local + 192]);
+    for (int o = 512; o >= 64; o >>= 1) {
+        if (t < o) red[t] += red[t + o];
+        __syncthreads();
+    }
+    if (t < 64 && e < M && g_of) g_of[e] = red[t];
+    __syncthreads();
+    red[t] = si;
+    __syncthreads();
+    for (int o = 512; o >= 64; o >>= 1) {
+        if (t < o) red[t] += red[t + o];
+        __syncthreads();
+    }
+    if (t < 64 && e < M && g_oi) g_oi[e] = red[t];
+}
+
+// Clears up to three tracker arrays in one launch.
+__global__ void fill3_u32_kernel(uint32_t *a, int64_t na, uint32_t *b, int64_t nb, uint32_t *c, int64_t nc) {
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < na + nb + nc; t += (int64_t)gridDim.x * blockDim.x) {
+        if (t < na) a[t] = 0;
+        else if (t < na + nb) b[t - na] = 0;
+        else c[t - na - nb] = 0;
+    }
+}
+
+static int pow2_at_least(int v, int lo) {
+    int t = lo;
+    while (t < v) t *= 2;
+    return t;
 }
 
 static int plan_softmax(int64_t rows, int L, int64_t bw_rows, bool has_oq, SoftmaxPlan &pl, const char *who) {
     if (rows < 0 || L < 1) return fail(HGQ_ERR_ARG, "%s: bad sizes", who);
-    if (L > 256) return fail(HGQ_ERR_UNSUPPORTED, "%s: rows of up to 256 elements are supported, got %d", who, L);
     int64_t P = has_oq ? bw_rows : 1;
-    if (P < 1 || (rows > 0 && rows % P != 0)) return fail(HGQ_ERR_ARG, "%s: rows=%lld is not a multiple of bw_rows=%lld", who, (long long)rows, (long long)P);
+    if (P < 1 || (rows > 0 && rows % P != 0))
+        return fail(HGQ_ERR_ARG, "%s: rows=%lld is not a multiple of bw_rows=%lld", who, (long long)rows, (long long)P);
     pl.rows = rows, pl.L = L, pl.P_table = P;
-    pl.EPL = L <= 64 ? 1 : (L <= 128 ? 2 : 4);
-    pl.SUB = L > 32 ? 64 : (L > 16 ? 32 : 16);
-    if (P > 1 && P % (64 / pl.SUB) != 0) pl.SUB = 64;  // table rows do not tile the wavefront: one row per wavefront
-    const int rpw = 64 / pl.SUB;
-    if (P == 1) {
-        pl.NP = 4, pl.Pq = rpw * 4;
+    if (L % 4 == 0 && L > 16 && L <= 256) {
+        pl.VEC = 4, pl.SUB = pow2_at_least(L / 4, 16);
+    } else if (L <= 64) {
+        pl.VEC = 1, pl.SUB = pow2_at_least(L, 16);
     } else {
-        pl.NP = (P % (rpw * 4) == 0) ? 4 : 1;
+        return fail(HGQ_ERR_UNSUPPORTED, "%s: rows of up to 64 elements, or up to 256 in multiples of 4, are supported, got %d", who, L);
+    }
+    if (P > 1 && P % (64 / pl.SUB) != 0) {
+        // the table rows do not tile the wavefront: fall back to one row per wavefront
+        if (pl.VEC == 4 && L > 64)
+            return fail(HGQ_ERR_UNSUPPORTED, "%s: bw_rows=%lld must be a multiple of %d for rows of %d elements", who, (long long)P, 64 / pl.SUB, L);
+        pl.VEC = 1, pl.SUB = 64;
+    }
+    const int rpw = 64 / pl.SUB;
+    // four row groups per step give a one-element-per-lane wavefront independent work; with four
+    // elements per lane that is already there and more would only cost registers
+    if (P == 1) {
+        pl.NP = pl.VEC == 1 ? 4 : 1, pl.Pq = rpw * pl.NP;
+    } else {
+        pl.NP = (pl.VEC == 1 && P % (rpw * 4) == 0) ? 4 : 1;
         pl.Pq = P;
     }
     pl.PG = pl.Pq / (rpw * pl.NP);
     pl.n_batches = (rows + pl.Pq - 1) / pl.Pq;
     if (pl.n_batches < 1) pl.n_batches = 1;
-    // enough wavefronts to fill the device (256 CUs x 4 SIMDs x ~8), each walking >= 4 batches where possible
-    const int64_t target = 8192;
+    // about 1024 workgroups of 8 wavefronts fill the device; a wavefront should walk >= 4 steps
+    const int64_t target = 1024;
     int64_t chunks = (target + pl.PG - 1) / pl.PG;
-    if (chunks > pl.n_batches) chunks = pl.n_batches;
+    const int64_t max_chunks = (pl.n_batches + SM_WPB * 4 - 1) / (SM_WPB * 4);
+    if (chunks > max_chunks) chunks = max_chunks;
     if (chunks < 1) chunks = 1;
     pl.bpc = (int)((pl.n_batches + chunks - 1) / chunks);
     pl.n_chunks = (pl.n_batches + pl.bpc - 1) / pl.bpc;
@@ -408,6 +643,7 @@ static hgq_qdesc desc_or_none(const hgq_qdesc *d) {
     r.k = nullptr, r.i = nullptr, r.fb = nullptr, r.mode = 0;
     return d ? *d : r;
 }
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 }  // namespace hgq
 
@@ -415,18 +651,17 @@ using namespace hgq;
 
 #define SM_DISPATCH(PLAN, ...)                                                                      \
     do {                                                                                            \
-        const int key = (PLAN).SUB * 100 + (PLAN).EPL * 10 + (PLAN).NP;                             \
+        const int key = (PLAN).SUB * 100 + (PLAN).VEC * 10 + (PLAN).NP;                             \
         switch (key) {                                                                              \
-            case 1611: { constexpr int SUB = 16, EPL = 1, NP = 1; __VA_ARGS__; } break;             \
-            case 1614: { constexpr int SUB = 16, EPL = 1, NP = 4; __VA_ARGS__; } break;             \
-            case 3211: { constexpr int SUB = 32, EPL = 1, NP = 1; __VA_ARGS__; } break;             \
-            case 3214: { constexpr int SUB = 32, EPL = 1, NP = 4; __VA_ARGS__; } break;             \
-            case 6411: { constexpr int SUB = 64, EPL = 1, NP = 1; __VA_ARGS__; } break;             \
-            case 6414: { constexpr int SUB = 64, EPL = 1, NP = 4; __VA_ARGS__; } break;             \
-            case 6421: { constexpr int SUB = 64, EPL = 2, NP = 1; __VA_ARGS__; } break;             \
-            case 6424: { constexpr int SUB = 64, EPL = 2, NP = 4; __VA_ARGS__; } break;             \
-            case 6441: { constexpr int SUB = 64, EPL = 4, NP = 1; __VA_ARGS__; } break;             \
-            case 6444: { constexpr int SUB = 64, EPL = 4, NP = 4; __VA_ARGS__; } break;             \
+            case 1611: { constexpr int SUB = 16, VEC = 1, NP = 1; __VA_ARGS__; } break;             \
+            case 1614: { constexpr int SUB = 16, VEC = 1, NP = 4; __VA_ARGS__; } break;             \
+            case 3211: { constexpr int SUB = 32, VEC = 1, NP = 1; __VA_ARGS__; } break;             \
+            case 3214: { constexpr int SUB = 32, VEC = 1, NP = 4; __VA_ARGS__; } break;             \
+            case 6411: { constexpr int SUB = 64, VEC = 1, NP = 1; __VA_ARGS__; } break;             \
+            case 6414: { constexpr int SUB = 64, VEC = 1, NP = 4; __VA_ARGS__; } break;             \
+            case 1641: { constexpr int SUB = 16, VEC = 4, NP = 1; __VA_ARGS__; } break;             \
+            case 3241: { constexpr int SUB = 32, VEC = 4, NP = 1; __VA_ARGS__; } break;             \
+            case 6441: { constexpr int SUB = 64, VEC = 4, NP = 1; __VA_ARGS__; } break;             \
             default: return fail(HGQ_ERR_UNSUPPORTED, "softmax: no kernel for this row layout");    \
         }                                                                                           \
     } while (0)
@@ -442,14 +677,18 @@ extern "C" int hgq_qsoftmax_fwd(const float *x, float *y, int64_t rows, int L, i
     if (rc) return rc;
     if (rows == 0) return HGQ_OK;
     if (!x || !y) return fail(HGQ_ERR_ARG, "hgq_qsoftmax_fwd: null pointer");
+    if (pl.VEC == 4 && !(aligned16(x) && aligned16(y))) return fail(HGQ_ERR_ARG, "hgq_qsoftmax_fwd: x and y must be 16-byte aligned");
     if (!desc_ok(exp_iq) || !desc_ok(exp_oq) || !desc_ok(inv_iq) || !desc_ok(inv_oq) || !desc_ok(oq))
         return fail(HGQ_ERR_ARG, "hgq_qsoftmax_fwd: a quantizer descriptor has k but not i / fb");
     if (amax_oq && !has_oq) return fail(HGQ_ERR_ARG, "hgq_qsoftmax_fwd: amax_oq without an output quantizer");
-    if (amax_exp_iq && (rc = fill_u32(amax_exp_iq, 0, 1, s))) return rc;
-    if (amax_inv_iq && (rc = fill_u32(amax_inv_iq, 0, 1, s))) return rc;
-    if (amax_oq && (rc = fill_u32(amax_oq, 0, pl.P_table * L, s))) return rc;
-    const unsigned grid = (unsigned)((pl.n_waves() + SM_WAVES_PER_BLOCK - 1) / SM_WAVES_PER_BLOCK);
-    SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_fwd_kernel<SUB, EPL, NP>), dim3(grid), dim3(64 * SM_WAVES_PER_BLOCK), 0, s, x, y, pl,
+    if (amax_exp_iq || amax_inv_iq || amax_oq) {
+        const int64_t n_o = amax_oq ? pl.P_table * L : 0;
+        const int grid = (int)min((int64_t)1024, (n_o + 2 + 255) / 256);
+        hipLaunchKernelGGL(fill3_u32_kernel, dim3(grid), dim3(256), 0, s, amax_exp_iq, (int64_t)(amax_exp_iq ? 1 : 0), amax_inv_iq,
+                           (int64_t)(amax_inv_iq ? 1 : 0), amax_oq, n_o);
+        if ((rc = check_launch("hgq_qsoftmax_fwd(clear)"))) return rc;
+    }
+    SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_fwd_kernel<SUB, VEC, NP>), dim3((unsigned)pl.n_blocks()), dim3(64 * SM_WPB), 0, s, x, y, pl,
                                        input_scaler, eps, desc_or_none(exp_iq), desc_or_none(exp_oq), desc_or_none(inv_iq),
                                        desc_or_none(inv_oq), desc_or_none(oq), amax_exp_iq, amax_inv_iq, amax_oq));
     return check_launch("hgq_qsoftmax_fwd");
@@ -458,7 +697,7 @@ extern "C" int hgq_qsoftmax_fwd(const float *x, float *y, int64_t rows, int L, i
 extern "C" int64_t hgq_qsoftmax_bwd_workspace(int64_t rows, int L, int64_t bw_rows, int has_oq) {
     SoftmaxPlan pl;
     if (plan_softmax(rows, L, bw_rows, has_oq != 0, pl, "hgq_qsoftmax_bwd_workspace")) return -1;
-    return pl.n_waves() * 8 + (has_oq ? 2 * pl.n_chunks * pl.Pq * L : 0);
+    return pl.n_blocks() * 8 + (has_oq ? 2 * pl.n_chunks * pl.Pq * L : 0);
 }
 
 extern "C" int hgq_qsoftmax_bwd(const float *dy, const float *x, float *dx, int64_t rows, int L, int64_t bw_rows,
@@ -483,13 +722,21 @@ extern "C" int hgq_qsoftmax_bwd(const float *dy, const float *x, float *dx, int6
         return HGQ_OK;
     }
     if (!dy || !x || !dx || !workspace) return fail(HGQ_ERR_ARG, "hgq_qsoftmax_bwd: null pointer");
-    const unsigned grid = (unsigned)((pl.n_waves() + SM_WAVES_PER_BLOCK - 1) / SM_WAVES_PER_BLOCK);
-    SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_bwd_kernel<SUB, EPL, NP>), dim3(grid), dim3(64 * SM_WAVES_PER_BLOCK), 0, s, dy, x, dx,
-                                       pl, input_scaler, eps, desc_or_none(exp_iq), desc_or_none(exp_oq), desc_or_none(inv_iq),
-                                       desc_or_none(inv_oq), desc_or_none(oq), workspace));
+    if (pl.VEC == 4 && !(aligned16(x) && aligned16(dy) && aligned16(dx)))
+        return fail(HGQ_ERR_ARG, "hgq_qsoftmax_bwd: dy, x and dx must be 16-byte aligned");
+    const bool oq_gi = has_oq && ((oq->mode >> 4) & 0xf) != HGQ_WRAP;
+    const unsigned grid = (unsigned)pl.n_blocks();
+    if (oq_gi)
+        SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_bwd_kernel<SUB, VEC, NP, true>), dim3(grid), dim3(64 * SM_WPB), 0, s, dy, x, dx, pl,
+                                           input_scaler, eps, desc_or_none(exp_iq), desc_or_none(exp_oq), desc_or_none(inv_iq),
+                                           desc_or_none(inv_oq), desc_or_none(oq), workspace));
+    else
+        SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_bwd_kernel<SUB, VEC, NP, false>), dim3(grid), dim3(64 * SM_WPB), 0, s, dy, x, dx, pl,
+                                           input_scaler, eps, desc_or_none(exp_iq), desc_or_none(exp_oq), desc_or_none(inv_iq),
+                                           desc_or_none(inv_oq), desc_or_none(oq), workspace));
     if ((rc = check_launch("hgq_qsoftmax_bwd"))) return rc;
     const unsigned rgrid = 1 + (has_oq ? (unsigned)((pl.P_table * L + 63) / 64) : 0);
-    hipLaunchKernelGGL(qsoftmax_reduce_kernel, dim3(rgrid), dim3(256), 0, s, workspace, pl, g_shared, has_oq ? g_oq_i : nullptr,
-                       has_oq ? g_oq_fb : nullptr);
+    hipLaunchKernelGGL(qsoftmax_reduce_kernel, dim3(rgrid), dim3(1024), 0, s, workspace, pl, g_shared, has_oq ? g_oq_i : nullptr,
+                       has_oq ? g_oq_fb : nullptr, (int)oq_gi);
     return check_launch("hgq_qsoftmax_bwd(reduce)");
 }

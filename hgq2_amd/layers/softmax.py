@@ -13,7 +13,7 @@ from math import prod
 
 import torch
 
-from .. import ops
+from .. import _lib, ops
 from ..config.layer import global_config
 from ..core import epsilon
 from ..quantizer import QuantizerConfig
@@ -130,6 +130,10 @@ class QSoftmax(QLayerBaseSingleInput):
             qs.append(qo)
         else:
             qs.append(None)
+        L = x.shape[-1]
+        bw_rows = qs[4][1].numel() // L if qs[4] is not None else 1
+        if _lib.load().hgq_qsoftmax_bwd_workspace(x.numel() // L, L, bw_rows, int(qs[4] is not None)) < 0:
+            return None  # a row layout outside the kernel family
         return qs
 
     def _call_fused(self, x, training, qs):

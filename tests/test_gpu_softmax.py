@@ -46,11 +46,11 @@ def _named(layer, r, xp, xr):
 
 
 @pytest.mark.parametrize('shape,enable_oq,exp_overflow,oq_hom', [
-    ((32, 4, 16, 64), True, 'SAT', None),    # one row per wavefront, four table rows per step
+    ((32, 4, 16, 64), True, 'SAT', None),    # 128-bit accesses, four rows side by side
     ((16, 3, 10), True, 'WRAP', None),       # short rows, table rows that do not tile a wavefront
     ((24, 8, 16), True, 'SAT', None),        # four rows side by side in a wavefront
-    ((8, 5, 100), True, 'SAT', None),        # two elements per lane
-    ((4, 8, 200), True, 'WRAP', None),       # four elements per lane
+    ((8, 6, 100), True, 'SAT', None),        # 128-bit accesses, a row spans 32 lanes
+    ((4, 8, 200), True, 'WRAP', None),       # 128-bit accesses, a row spans the wavefront
     ((40, 7, 32), False, 'SAT', None),       # no output quantizer
     ((12, 6, 24), True, 'SAT', (0, 1)),      # output quantizer table shared by all rows
 ])
