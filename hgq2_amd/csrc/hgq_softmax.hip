@@ -78,12 +78,17 @@ struct SharedQ : UniQ {
     static __device__ __forceinline__ float uniform(float v) {
         return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
     }
+    // TRAIN: every quantizer of the launch is in training mode (no wrap, no zeroing of empty words)
+    template <bool TRAIN = true>
     __device__ __forceinline__ float fwd(float x) const {
         if (!present) return x;
         const float xq = round_at(x, fi);
         float y = xq > hi ? hi : (xq < lo ? lo : xq);
-        if (wrap_inf) y = wrap(xq, p);
-        return zero ? 0.f : y;
+        if (!TRAIN) {
+            if (wrap_inf) y = wrap(xq, p);
+            y = zero ? 0.f : y;
+        }
+        return y;
     }
     // gradients w.r.t. the input and the two stored variables (i and f, or i and b), training mode
     __device__ __forceinline__ void grad(float x, float dy, float &dx, float &di, float &dfb) const {
@@ -117,6 +122,7 @@ struct LaneQ : UniQ {
     static __device__ __forceinline__ int f_of(int pk) { return (int)(int8_t)(pk & 0xff); }
     static __device__ __forceinline__ int i_of(int pk) { return (int)(int8_t)((pk >> 8) & 0xff); }
     static __device__ __forceinline__ float k_of(int pk) { return (pk >> 16) & 1 ? 1.f : 0.f; }
+    template <bool TRAIN>
     __device__ __forceinline__ float fwd(float x, int pk) const {
         const int fi = f_of(pk);
         const float xq = round_at(x, fi);
@@ -126,12 +132,12 @@ struct LaneQ : UniQ {
             const float hi = __fsub_rn(pi, ldexpf(1.0f, -fi));
             const float lo = sym ? -k * hi : -k * pi;
             y = xq > hi ? hi : (xq < lo ? lo : xq);
-        } else if (wrap_inf) {
+        } else if (!TRAIN && wrap_inf) {
             KIF p;
             p.k = k_of(pk), p.i = (float)i_of(pk), p.f = (float)fi;
             y = wrap(xq, p);
         }
-        if (!training && !(k_of(pk) + (float)(i_of(pk) + fi) > 0.0f)) y = 0.f;
+        if (!TRAIN && !training && !(k_of(pk) + (float)(i_of(pk) + fi) > 0.0f)) y = 0.f;
         return y;
     }
     __device__ __forceinline__ void grad(float x, float dy, int pk, float &dx, float &di, float &dfb) const {
@@ -152,6 +158,85 @@ struct LaneQ : UniQ {
             }
         }
         if (kbi) di -= dfb;
+    }
+};
+
+// The exp stage as the lookup table it stands for.  The rounded, saturated argument of the exp
+// quantizer is a small non-negative integer code n (d >= 0), and
+//     t(n) = exp(-(n * 2**-f) * scale),   e(n) = Q_exp_oq(t(n))
+// are functions of n alone: a workgroup tabulates the first SM_TABLE codes in LDS with the same
+// device code that evaluates them directly, so looked-up and computed values are identical;
+// codes beyond the table (possible only when the exp input quantizer does not saturate) are
+// computed in place.
+#define SM_TABLE 1024
+struct ExpTable {
+    float code_max;  // largest code the input quantizer lets through (+inf without saturation)
+    bool on;
+    __device__ __forceinline__ void init(const SharedQ &q1) {
+        // the table needs d -> code to be monotone from 0: an input quantizer whose upper bound is
+        // negative (an empty word) keeps the direct evaluation
+        on = q1.present && !(q1.hi < 0.f);
+        code_max = INFINITY;
+        if (on && q1.sat) code_max = SharedQ::uniform(ldexpf(q1.hi, q1.fi));
+    }
+    static __device__ __forceinline__ float code_of(float d, const SharedQ &q1) {
+        return q1.conv ? rintf(ldexpf(d, q1.fi)) : floorf(__fadd_rn(ldexpf(d, q1.fi), q1.rc));
+    }
+    static __device__ __forceinline__ float t_of(float a, float scale) { return expf(__fmul_rn(-a, scale)); }
+
+    // forward: tab[n] = e(n)
+    __device__ __forceinline__ void build_fwd(float *tab, const SharedQ &q1, const SharedQ &q2, float scale) {
+        init(q1);
+        if (!on) return;
+        for (int n = threadIdx.x; n < SM_TABLE; n += blockDim.x) tab[n] = q2.fwd<true>(t_of(ldexpf((float)n, -q1.fi), scale));
+        __syncthreads();
+    }
+    // d >= 0 -> a = Q_exp_iq(d), e
+    __device__ __forceinline__ void eval_fwd(const float *tab, float d, const SharedQ &q1, const SharedQ &q2, float scale,
+                                             float &a, float &e) const {
+        const float rcl = fminf(code_of(d, q1), code_max);
+        a = ldexpf(rcl, -q1.fi);
+        const unsigned n = (unsigned)(int)rcl;
+        e = n < SM_TABLE ? tab[n] : q2.fwd<true>(t_of(a, scale));
+    }
+
+    // backward: tab[n] = (e, d a / d e-gradient, d i2, d fb2) with
+    //   da = -((dt * t) * scale) = ca * de,  gi2 = ci * de,  gf2 = cf * de   for the upstream gradient de of e
+    struct Entry {
+        float e, ca, ci, cf;
+    };
+    static __device__ __forceinline__ Entry entry_of(float a, const SharedQ &q2, float scale) {
+        const float t = t_of(a, scale);
+        Entry r;
+        r.e = q2.fwd<true>(t);
+        float dt;
+        q2.grad(t, 1.0f, dt, r.ci, r.cf);
+        r.ca = -((dt * t) * scale);
+        return r;
+    }
+    __device__ __forceinline__ void build_bwd(Entry *tab, const SharedQ &q1, const SharedQ &q2, float scale) {
+        init(q1);
+        if (!on) return;
+        for (int n = threadIdx.x; n < SM_TABLE; n += blockDim.x) tab[n] = entry_of(ldexpf((float)n, -q1.fi), q2, scale);
+        __syncthreads();
+    }
+    // d >= 0 -> r = un-saturated code, entry of the saturated code
+    __device__ __forceinline__ Entry eval_bwd(const Entry *tab, float d, const SharedQ &q1, const SharedQ &q2, float scale,
+                                              float &r) const {
+        r = code_of(d, q1);
+        const float rcl = fminf(r, code_max);
+        const unsigned n = (unsigned)(int)rcl;
+        if (n < SM_TABLE) return tab[n];
+        return entry_of(ldexpf(rcl, -q1.fi), q2, scale);
+    }
+    // gradients of the exp input quantizer from the un-saturated code r (no lower violation: d >= 0 >= lo)
+    __device__ __forceinline__ void grad_q1(float d, float r, float da, const SharedQ &q1, float &dd, float &gi, float &gf) const {
+        const bool over = r > code_max;
+        const float xq = ldexpf(r, -q1.fi);
+        dd = over ? 0.f : da;
+        gi = over ? q1.gi_hi * da : 0.f;
+        gf = over ? q1.gf_hi * da : -HGQ_LN2 * (xq - d) * da;
+        if (q1.kbi) gi -= gf;
     }
 };
 
@@ -269,12 +354,13 @@ struct Walk {
     }
 };
 
-template <int SUB, int VEC, int NP>
+template <int SUB, int VEC, int NP, bool TRAIN>
 __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_fwd_kernel(
     const float *__restrict__ x, float *__restrict__ y, SoftmaxPlan pl, float scale, float eps, hgq_qdesc d1, hgq_qdesc d2,
     hgq_qdesc d3, hgq_qdesc d4, hgq_qdesc dq, uint32_t *amax1, uint32_t *amax3, uint32_t *amax_o) {
     __shared__ uint32_t lds_max[SM_WPB][NP * VEC][64];
     __shared__ uint32_t lds_m13[SM_WPB][2];
+    __shared__ float lds_tab_e[SM_TABLE];
     Walk<SUB, VEC, NP> wk;
     wk.init(pl);
     SharedQ q1, q2, q3, q4;
@@ -290,6 +376,9 @@ __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_fwd_kernel(
             mo[np][e] = 0, po[np][e] = 0;
             if (qo.present && wk.col_on) po[np][e] = qo.load(dq, wk.tcol[np] + e);
         }
+    ExpTable tab;
+    tab.on = false;
+    if (TRAIN) tab.build_fwd(lds_tab_e, q1, q2, scale);
     uint32_t m1 = 0, m3 = 0;
     for (int b = 0; b < wk.nb; ++b) {
         float xv[NP][VEC];
@@ -311,21 +400,26 @@ __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_fwd_kernel(
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const float d = act[np] ? __fsub_rn(mx, xv[np][e]) : 0.f;
-                const float a = q1.fwd(d);
-                const float t = expf(__fmul_rn(-a, scale));
-                ev[e] = act[np] ? q2.fwd(t) : 0.f;
+                float a, ee;
+                if (TRAIN && tab.on) {
+                    tab.eval_fwd(lds_tab_e, d, q1, q2, scale, a, ee);
+                } else {
+                    a = q1.fwd<TRAIN>(d);
+                    ee = q2.fwd<TRAIN>(ExpTable::t_of(a, scale));
+                }
+                ev[e] = act[np] ? ee : 0.f;
                 m1 = max(m1, abs_bits(a));
                 s += ev[e];
             }
             s = sub_sum<SUB>(s);
-            const float sq = q3.fwd(s);
-            const float rr = q4.fwd(__fdiv_rn(1.0f, __fadd_rn(sq, eps)));
+            const float sq = q3.fwd<TRAIN>(s);
+            const float rr = q4.fwd<TRAIN>(__fdiv_rn(1.0f, __fadd_rn(sq, eps)));
             if (b < wk.blim[np]) m3 = max(m3, abs_bits(sq));
             float yv[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 yv[e] = __fmul_rn(ev[e], rr);
-                if (qo.present) yv[e] = qo.fwd(yv[e], po[np][e]);
+                if (qo.present) yv[e] = qo.fwd<TRAIN>(yv[e], po[np][e]);
                 if (act[np]) mo[np][e] = max(mo[np][e], abs_bits(yv[e]));
             }
             if (act[np]) row_store<VEC>(y + wk.off[np], yv);
@@ -373,6 +467,7 @@ __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_bwd_kernel(
     float eps, hgq_qdesc d1, hgq_qdesc d2, hgq_qdesc d3, hgq_qdesc d4, hgq_qdesc dq, float *__restrict__ ws) {
     __shared__ float lds_g[SM_WPB][NP * VEC][64];
     __shared__ float part[SM_WPB][8];
+    __shared__ ExpTable::Entry lds_tab[SM_TABLE];
     Walk<SUB, VEC, NP> wk;
     wk.init(pl);
     SharedQ q1, q2, q3, q4;
@@ -393,6 +488,8 @@ __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_bwd_kernel(
 #pragma unroll
     for (int j = 0; j < 8; ++j) gs[j] = 0.f;
     const bool row_lead = wk.col == 0;
+    ExpTable tab;
+    tab.build_bwd(lds_tab, q1, q2, scale);
     for (int b = 0; b < wk.nb; ++b) {
         float xv[NP][VEC], gv[NP][VEC];
         bool act[NP];
@@ -413,12 +510,18 @@ __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_bwd_kernel(
 #pragma unroll
             for (int e = 1; e < VEC; ++e) mx = fmaxf(mx, xv[np][e]);
             mx = sub_max<SUB>(mx);
-            float dv[VEC], tv[VEC], ev[VEC], s = 0.f;
+            float dv[VEC], rv[VEC], ev[VEC], s = 0.f;
+            ExpTable::Entry en[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 dv[e] = act[np] ? __fsub_rn(mx, xv[np][e]) : 0.f;
-                tv[e] = expf(__fmul_rn(-q1.fwd(dv[e]), scale));
-                ev[e] = act[np] ? q2.fwd(tv[e]) : 0.f;
+                if (tab.on) {
+                    en[e] = tab.eval_bwd(lds_tab, dv[e], q1, q2, scale, rv[e]);
+                } else {
+                    rv[e] = 0.f;
+                    en[e] = ExpTable::entry_of(q1.fwd(dv[e]), q2, scale);
+                }
+                ev[e] = act[np] ? en[e].e : 0.f;
                 s += ev[e];
             }
             s = sub_sum<SUB>(s);
@@ -448,9 +551,12 @@ __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_bwd_kernel(
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const float de = g0[e] * rr + ds;
-                float dt, gi2, gf2, gi1, gf1;
-                q2.grad(tv[e], de, dt, gi2, gf2);
-                q1.grad(dv[e], -((dt * tv[e]) * scale), dd[e], gi1, gf1);
+                const float gi2 = en[e].ci * de, gf2 = en[e].cf * de, da = en[e].ca * de;
+                float gi1, gf1;
+                if (tab.on)
+                    tab.grad_q1(dv[e], rv[e], da, q1, dd[e], gi1, gf1);
+                else
+                    q1.grad(dv[e], da, dd[e], gi1, gf1);
                 if (act[np]) {
                     gs[2] += gi2, gs[3] += gf2, gs[0] += gi1, gs[1] += gf1;
                     dm += dd[e];
@@ -688,9 +794,19 @@ extern "C" int hgq_qsoftmax_fwd(const float *x, float *y, int64_t rows, int L, i
                            (int64_t)(amax_inv_iq ? 1 : 0), amax_oq, n_o);
         if ((rc = check_launch("hgq_qsoftmax_fwd(clear)"))) return rc;
     }
-    SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_fwd_kernel<SUB, VEC, NP>), dim3((unsigned)pl.n_blocks()), dim3(64 * SM_WPB), 0, s, x, y, pl,
-                                       input_scaler, eps, desc_or_none(exp_iq), desc_or_none(exp_oq), desc_or_none(inv_iq),
-                                       desc_or_none(inv_oq), desc_or_none(oq), amax_exp_iq, amax_inv_iq, amax_oq));
+    // a launch whose quantizers are all in training mode takes the kernel without the inference-only steps
+    bool train = true;
+    const hgq_qdesc *all[5] = {exp_iq, exp_oq, inv_iq, inv_oq, oq};
+    for (const hgq_qdesc *d : all)
+        if (d && d->k && !(d->mode & HGQ_MODE_TRAINING)) train = false;
+    if (train)
+        SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_fwd_kernel<SUB, VEC, NP, true>), dim3((unsigned)pl.n_blocks()), dim3(64 * SM_WPB), 0, s, x, y,
+                                           pl, input_scaler, eps, desc_or_none(exp_iq), desc_or_none(exp_oq), desc_or_none(inv_iq),
+                                           desc_or_none(inv_oq), desc_or_none(oq), amax_exp_iq, amax_inv_iq, amax_oq));
+    else
+        SM_DISPATCH(pl, hipLaunchKernelGGL((qsoftmax_fwd_kernel<SUB, VEC, NP, false>), dim3((unsigned)pl.n_blocks()), dim3(64 * SM_WPB), 0, s, x, y,
+                                           pl, input_scaler, eps, desc_or_none(exp_iq), desc_or_none(exp_oq), desc_or_none(inv_iq),
+                                           desc_or_none(inv_oq), desc_or_none(oq), amax_exp_iq, amax_inv_iq, amax_oq));
     return check_launch("hgq_qsoftmax_fwd");
 }
 
