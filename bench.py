@@ -165,6 +165,57 @@ def softmax_roofline(iters=50, shape=(2048, 4, 64, 64), scaler=0.25):
     return out
 
 
+def config_step_time(name, steps=20, warmup=5):
+    """One forward + backward pass of the configurations other than the headline one, at their full
+    sizes: 'particle' (QEinsumDenseBatchnorm per-particle network, batch 4096 x 64 x 16), 'conv'
+    (QConv2D stack on 28 x 28 x 1, batch 1024), 'mha' (QMultiHeadAttention, batch 2048 x 64 x 64)."""
+    import torch
+
+    from hgq2_amd import ops
+    from hgq2_amd.train import model_loss
+    from hgq2_amd.utils import models
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(0)
+    torch.manual_seed(1)
+    if name == 'particle':
+        batch = 4096
+        x = torch.randn(batch, 64, 16, generator=g).to(dev)
+        labels = torch.randint(0, 5, (batch,), generator=g).to(dev)
+        model = models.particle_mlp(device=dev)
+        loss_fn = lambda out: ops.sparse_ce(out, labels)  # noqa: E731
+    elif name == 'conv':
+        batch = 1024
+        x = torch.rand(batch, 28, 28, 1, generator=g).to(dev)
+        labels = torch.randint(0, 10, (batch,), generator=g).to(dev)
+        model = models.conv_stack(device=dev)
+        loss_fn = lambda out: ops.sparse_ce(out, labels)  # noqa: E731
+    elif name == 'mha':
+        batch = 2048
+        x = torch.randn(batch, 64, 64, generator=g).to(dev)
+        model = models.mha_block(device=dev)
+        loss_fn = lambda out: (out * out).mean()  # noqa: E731
+    else:
+        raise ValueError(name)
+
+    def step():
+        for p in model.parameters():
+            p.grad = None
+        loss = model_loss(model, loss_fn(model(x, training=True)))
+        loss.backward()
+        return loss
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    return {'workload': name, 'batch': batch, 'ms_per_step': ms, 'samples_per_s': batch / ms * 1e3, 'loss': float(loss)}
+
+
 def cpu_baseline(budget_s=20.0):
     """The oracle's eager torch-CPU restatement of the reference path, same model and batch."""
     import torch
@@ -199,6 +250,8 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--roofline-only', action='store_true',
                     help='run only the standalone quantizer kernels and a plain copy of known size (for counter runs)')
+    ap.add_argument('--config-step', choices=('particle', 'conv', 'mha'), default=None,
+                    help='time one forward + backward pass of another configuration at full size instead of the headline run')
     ap.add_argument('--softmax-only', action='store_true',
                     help='run only the one-pass table-softmax kernels at the attention configuration (for profiler runs)')
     ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused',
@@ -214,6 +267,10 @@ def main():
     if args.roofline_only:
         torch.cuda.set_device(0)
         print(json.dumps({'quantizer_kernels': quantizer_roofline(iters=20, with_copy=True)}))
+        return
+    if args.config_step:
+        torch.cuda.set_device(0)
+        print(json.dumps({'config_step': config_step_time(args.config_step, steps=args.steps if args.steps != 300 else 20)}))
         return
     if args.softmax_only:
         torch.cuda.set_device(0)

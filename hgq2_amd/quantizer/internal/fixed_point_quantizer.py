@@ -143,7 +143,7 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
         lo, hi = self._constraint_bounds() if (clip or tracing) else (float('-inf'), float('inf'))
         mode = _lib.mode_bits(self.round_mode, self.overflow_mode, kbi=self._kbi, symmetric=self._symmetric,
                               tracing=tracing)
-        if amax.numel() != self._i.numel():
+        if amax.numel() == 0 or amax.numel() % self._i.numel() != 0:  # one slice, or one per producing workgroup
             raise NotImplementedError('integer-bit tracking needs a bit-width layout the kernels can index')
         with torch.no_grad():
             ops.wrap_track_i_(amax, self._i.data.view(-1), self._third().data.view(-1), self._decay_host, mode, lo, hi,

@@ -4,7 +4,8 @@ from __future__ import annotations
 
 from ..config import LayerConfigScope, QuantizerConfigScope
 from ..core import Sequential, set_default_device
-from ..layers import QDense
+from ..core import Layer
+from ..layers import QConv2D, QDense, QEinsumDenseBatchnorm, QMultiHeadAttention
 
 
 class _Scopes:
@@ -41,3 +42,58 @@ def qdense_mlp(dims=(16, 64, 32, 32, 5), beta0=1e-5, device=None, batch=None):
         layer.built = True
         shape = (batch, d)
     return model
+
+
+class Lambda(Layer):
+    """A parameter-free step between quantized layers (pooling, flatten, mean)."""
+
+    def __init__(self, fn, **kwargs):
+        super().__init__(**kwargs)
+        self.fn = fn
+
+    def call(self, x, training=None):
+        return self.fn(x)
+
+
+def particle_mlp(n_particles=64, n_features=16, hidden=(64, 32), n_out=5, beta0=1e-5, device=None):
+    """Per-particle network: QEinsumDenseBatchnorm('bpf,fh->bph') x len(hidden) with ReLU, mean over the
+    particles, QDense(n_out)."""
+    import torch
+
+    if device is not None:
+        set_default_device(device)
+    with _Scopes(beta0):
+        layers = [QEinsumDenseBatchnorm('bpf,fh->bph', (n_particles, h), bias_axes='h', activation='relu') for h in hidden]
+        layers.append(Lambda(lambda t: torch.mean(t, dim=1), name='mean_over_particles'))
+        layers.append(QDense(n_out))
+    return Sequential(layers)
+
+
+def conv_stack(filters=32, n_out=10, beta0=1e-5, device=None):
+    """QConv2D 3x3 ReLU -> MaxPool 2x2 -> QConv2D 3x3 ReLU -> Flatten -> QDense(n_out), channels-last."""
+    import torch
+    import torch.nn.functional as F
+
+    if device is not None:
+        set_default_device(device)
+
+    def pool(t):  # NHWC max-pool 2x2, stride 2, 'valid'
+        b, h, w, c = t.shape
+        t = t[:, :h // 2 * 2, :w // 2 * 2, :].reshape(b, h // 2, 2, w // 2, 2, c)
+        return torch.amax(t, dim=(2, 4))
+
+    with _Scopes(beta0):
+        layers = [QConv2D(filters, (3, 3), activation='relu'), Lambda(pool, name='max_pool'),
+                  QConv2D(filters, (3, 3), activation='relu'), Lambda(lambda t: t.reshape(t.shape[0], -1), name='flatten'),
+                  QDense(n_out)]
+    del F
+    return Sequential(layers)
+
+
+def mha_block(num_heads=4, key_dim=16, beta0=1e-5, device=None):
+    """Self-attention block: QMultiHeadAttention with the table softmax (8-bit tables by default)."""
+    if device is not None:
+        set_default_device(device)
+    with _Scopes(beta0):
+        layer = QMultiHeadAttention(num_heads=num_heads, key_dim=key_dim)
+    return layer

@@ -190,3 +190,28 @@ def test_conv2d_stack_layer(dev):
         _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=1e-4)
         assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
         assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+
+
+def test_einsum_dense_many_tracker_slices(dev):
+    """A projection of the attention configuration's size: the fused input quantizer produces more
+    abs-max slices than the EBOPs kernel folds in, so the integer bits are tracked by the separate
+    kernel over all slices; output, EBOPs and tracked bits must still match the oracle."""
+    from hgq2_amd.layers import QEinsumDense
+    from hgq2_amd.layers.core import _contraction
+
+    g = torch.Generator().manual_seed(7)
+    with readme_scopes():
+        layer = QEinsumDense('abc,cde->abde', (64, 4, 16), bias_axes='de')
+    x = torch.randn(1024, 64, 64, generator=g) * 2
+    layer(x.to(dev), training=True)
+    r = twin.ref_einsum_dense(layer, tuple(x.shape))
+    from hgq2_amd import _lib
+
+    n_parts = _lib.load().hgq_qdense_fwd_parts(x.shape[0] * x.shape[1])
+    assert n_parts * 64 * 64 > _contraction.FUSED_TRACK_MAX
+    with torch.no_grad():
+        got = layer(x.to(dev), training=True)
+        want = r(x, training=True)
+    _close(got, want, what='output')
+    assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
+    assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)
