@@ -56,7 +56,16 @@ SIGNATURES = {
     'hgq_qsoftmax_bwd_workspace': (c_int64, [c_int64, c_int, c_int64, c_int]),
     'hgq_qsoftmax_bwd': (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int64, c_float, c_float] + [c_void_p] * 5
                          + [c_void_p] * 4 + [c_void_p]),
+    'hgq_conv2d_fwd': (c_int, [c_void_p] * 5 + [c_int, c_int, c_void_p]),
+    'hgq_conv2d_bwd_workspace': (c_int64, [c_void_p, c_int]),
+    'hgq_conv2d_bwd': (c_int, [c_void_p] * 9 + [c_int, c_int, c_void_p]),
 }
+
+
+class ConvGeom(ctypes.Structure):
+    """``hgq_conv_geom`` of include/hgq_hip.h."""
+
+    _fields_ = [(n, c_int) for n in ('B', 'H', 'W', 'C', 'kh', 'kw', 'sy', 'sx', 'py', 'px', 'dly', 'dlx', 'OH', 'OW')]
 
 
 class QDesc(ctypes.Structure):

@@ -330,6 +330,12 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restri
     }
 }
 
+int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb, float *df,
+                 int64_t n_df, hipStream_t s) {
+    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(256), 0, s, part, n_parts, M, dqw, n_dqw, dqb, n_dqb, df, n_df);
+    return check_launch("reduce_parts");
+}
+
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 static inline int row_parts(int64_t rows, int bm) {

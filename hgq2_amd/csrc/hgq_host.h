@@ -44,4 +44,9 @@ inline int fill_f32(float *p, float v, int64_t n, hipStream_t s) {
     return fill_u32((uint32_t *)p, c.u, n, s);
 }
 
+// out[e] = sum over the n_parts slices of part[slice][e] (slice length M), in a fixed order; the
+// first n_dqw entries go to dqw, the next n_dqb to dqb, the remaining n_df to df (null = skip).
+int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb, float *df,
+                 int64_t n_df, hipStream_t s);
+
 }  // namespace hgq

@@ -1,14 +1,16 @@
 """QConv2D (reference src/hgq/layers/conv.py:12-102,175-200): ``act(conv(iq(x), kq(W)) + bq(b))``
 on channels-last tensors with the kernel in HWIO layout, and the EBOPs obtained by convolving the
 bit-width tensors.  The input / kernel / bias quantizers run in the HIP quantizer kernels; the
-convolution of the quantized operands is the plain library convolution."""
+convolution of the quantized operands, the bias add and a ReLU run in the implicit-GEMM kernels
+(``hgq_conv2d_fwd / hgq_conv2d_bwd``), which are also what convolves the bit-width tensors for EBOPs."""
 
 from __future__ import annotations
 
 from math import prod
 
 import torch
-import torch.nn.functional as F
+
+from .. import _lib, ops
 
 from ..core import get_initializer
 from ..quantizer import Quantizer
@@ -95,26 +97,16 @@ class QConv2D(QLayerBaseSingleInput):
             assert self.n_parallel is not None
             self.parallelization_factor = self.n_parallel
 
-    def convolution_op(self, x_nhwc, kernel_hwio):
-        x = x_nhwc.permute(0, 3, 1, 2)
-        w = kernel_hwio.permute(3, 2, 0, 1)
-        if self.padding == 'same':
-            pads = []
-            for d in (1, 0):  # F.pad wants the last dimension first
-                n, k, s, dil = x.shape[2 + d], self.kernel_size[d], self.strides[d], self.dilation_rate[d]
-                total = max((-(-n // s) - 1) * s + dil * (k - 1) + 1 - n, 0)
-                pads += [total // 2, total - total // 2]
-            x = F.pad(x, pads)
-        y = F.conv2d(x, w, None, self.strides, 0, self.dilation_rate)
-        return y.permute(0, 2, 3, 1)
+    def convolution_op(self, x_nhwc, kernel_hwio, bias=None, act_code=_lib.ACT_NONE):
+        """``act(conv(x, kernel) + bias)`` on channels-last tensors through the implicit-GEMM kernels."""
+        return ops.conv2d(x_nhwc, kernel_hwio, bias, self.strides, self.padding, self.dilation_rate, act_code)
 
     def call(self, inputs, training=None):
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
-        outputs = self.convolution_op(inputs, self.qkernel)
-        if self.use_bias:
-            outputs = outputs + self.qbias.reshape(1, 1, 1, self.filters)
-        if self.activation is not None:
+        fused_act = _lib.ACT_RELU if self._act_name == 'relu' else _lib.ACT_NONE
+        outputs = self.convolution_op(inputs, self.qkernel, self.qbias if self.use_bias else None, fused_act)
+        if self.activation is not None and fused_act == _lib.ACT_NONE:
             outputs = self.activation(outputs)
         return outputs
 

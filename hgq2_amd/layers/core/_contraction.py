@@ -93,11 +93,9 @@ def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training):
     if fused_bwd:
         y, _ = ops.qdense(x2d, None, None, None, qkernel2d, qbias1d, act_code, 0, 0, False)
         return y, act_code != _lib.ACT_NONE, None
-    # shapes beyond the fused backward kernel: plain library GEMM on the quantized operands
-    y = x2d @ qkernel2d
-    if qbias1d is not None:
-        y = y + qbias1d
-    return y, False, None
+    # shapes beyond the fused backward kernel: the implicit-GEMM kernels in their 1 x 1 form
+    y = ops.matmul_bias_act(x2d, qkernel2d, qbias1d, act_code)
+    return y, act_code != _lib.ACT_NONE, None
 
 
 def dense_ebops_term(layer, iq, kq, bq, K, N, scale, bias_size, deferred):

@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act']
 
 
 def _ptr(t: Tensor | None):
@@ -337,6 +337,57 @@ def _(dy, x, ks, is_, fbs, modes, input_scaler, eps):
     return torch.empty_like(x), x.new_empty(8), x.new_empty(n_o), x.new_empty(n_o)
 
 
+def _geom(g: Sequence[int]):
+    _need(len(g) == 14, 'a convolution geometry has 14 entries (B, H, W, C, kh, kw, sy, sx, py, px, dly, dlx, OH, OW)')
+    return _lib.ConvGeom(*[int(v) for v in g])
+
+
+@torch.library.custom_op('hgq::conv2d_fwd', mutates_args=())
+def conv2d_fwd(xq: Tensor, qw: Tensor, qb: Tensor, geom: Sequence[int], act: int) -> Tensor:
+    _check_f32('xq', xq), _check_f32('qw', qw)
+    g = _geom(geom)
+    F = qw.shape[-1]
+    _need(xq.numel() == g.B * g.H * g.W * g.C, f'input has {xq.numel()} elements, geometry says {g.B}x{g.H}x{g.W}x{g.C}')
+    _need(qw.numel() == g.kh * g.kw * g.C * F, 'kernel must be [kh, kw, C, F]')
+    if qb.numel():
+        _check_f32('qb', qb)
+        _need(qb.numel() == F, 'bias size mismatch')
+    y = torch.empty((g.B, g.OH, g.OW, F), dtype=torch.float32, device=xq.device)
+    rc = _lib.load().hgq_conv2d_fwd(_ptr(xq), _ptr(qw), _ptr(qb), _ptr(y), ctypes.addressof(g), F, act, _stream())
+    _lib.check(rc, 'hgq_conv2d_fwd')
+    return y
+
+
+@conv2d_fwd.register_fake
+def _(xq, qw, qb, geom, act):
+    return xq.new_empty((geom[0], geom[12], geom[13], qw.shape[-1]))
+
+
+@torch.library.custom_op('hgq::conv2d_bwd', mutates_args=())
+def conv2d_bwd(dy: Tensor, y: Tensor, xq: Tensor, qw: Tensor, geom: Sequence[int], act: int, need_dx: bool, has_bias: bool) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('dy', dy), _check_f32('y', y), _check_f32('xq', xq), _check_f32('qw', qw)
+    g = _geom(geom)
+    F = qw.shape[-1]
+    _need(dy.numel() == g.B * g.OH * g.OW * F and y.numel() == dy.numel(), 'dy / y must be [B, OH, OW, F]')
+    lib = _lib.load()
+    f32 = dict(dtype=torch.float32, device=xq.device)
+    dx = torch.empty(xq.shape if need_dx else (0,), **f32)
+    dqw = torch.empty_like(qw)
+    dqb = torch.empty(F if has_bias else 0, **f32)
+    n_ws = lib.hgq_conv2d_bwd_workspace(ctypes.addressof(g), F)
+    _need(n_ws >= 0, 'hgq_conv2d_bwd_workspace rejected the geometry')
+    ws = torch.empty(max(int(n_ws), 1), **f32)
+    rc = lib.hgq_conv2d_bwd(_ptr(dy), _ptr(y), _ptr(xq), _ptr(qw), _ptr(dx), _ptr(dqw), _ptr(dqb), _ptr(ws),
+                            ctypes.addressof(g), F, act, _stream())
+    _lib.check(rc, 'hgq_conv2d_bwd')
+    return dx, dqw, dqb
+
+
+@conv2d_bwd.register_fake
+def _(dy, y, xq, qw, geom, act, need_dx, has_bias):
+    return (xq.new_empty(xq.shape if need_dx else (0,)), torch.empty_like(qw), xq.new_empty(qw.shape[-1] if has_bias else 0))
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -505,6 +556,49 @@ def qsoftmax(x: Tensor, quantizers, input_scaler: float, eps: float, track_mask:
             flat += [k.contiguous(), i.contiguous(), fb.contiguous()]
             modes.append(int(mode))
     return _QSoftmax.apply(x.contiguous(), tuple(modes), float(input_scaler), float(eps), int(track_mask), *flat)
+
+
+class _Conv2D(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, xq, qw, qb, geom, act):
+        y = conv2d_fwd(xq, qw, qb, list(geom), act)
+        ctx.save_for_backward(xq, qw, y)
+        ctx.geom, ctx.act, ctx.has_bias = tuple(geom), act, qb.numel() > 0
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        xq, qw, y = ctx.saved_tensors
+        dx, dqw, dqb = conv2d_bwd(gy.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, ctx.needs_input_grad[0], ctx.has_bias)
+        return (dx if ctx.needs_input_grad[0] else None, dqw, dqb if ctx.has_bias else None, None, None)
+
+
+def conv2d(xq: Tensor, qw: Tensor, qb, strides=(1, 1), padding='valid', dilation=(1, 1), act: int = 0) -> Tensor:
+    """``act(conv2d(xq, qw) + qb)`` for a channels-last input [B, H, W, C] and an HWIO kernel; 'same'
+    padding puts the odd pad after the last row / column, as Keras / TensorFlow do."""
+    B, H, W, C = xq.shape
+    kh, kw, c2, F = qw.shape
+    _need(c2 == C, f'kernel has {c2} input channels, input has {C}')
+    (sy, sx), (dly, dlx) = strides, dilation
+    eh, ew = dly * (kh - 1) + 1, dlx * (kw - 1) + 1
+    if padding == 'same':
+        OH, OW = -(-H // sy), -(-W // sx)
+        py, px = max((OH - 1) * sy + eh - H, 0) // 2, max((OW - 1) * sx + ew - W, 0) // 2
+    else:
+        OH, OW, py, px = (H - eh) // sy + 1, (W - ew) // sx + 1, 0, 0
+    _need(OH >= 1 and OW >= 1, 'the kernel does not fit the input')
+    geom = (B, H, W, C, kh, kw, sy, sx, py, px, dly, dlx, OH, OW)
+    return _Conv2D.apply(xq.contiguous(), qw.contiguous(), qb.contiguous() if qb is not None else xq.new_empty(0), geom, act)
+
+
+def matmul_bias_act(x2d: Tensor, qw: Tensor, qb, act: int = 0) -> Tensor:
+    """``act(x2d @ qw + qb)`` for any K, N: the 1 x 1 case of the implicit-GEMM kernels."""
+    rows, K = x2d.shape
+    N = qw.shape[1]
+    geom = (rows, 1, 1, K, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1)
+    y = _Conv2D.apply(x2d.contiguous(), qw.contiguous().view(1, 1, K, N), qb.contiguous() if qb is not None else x2d.new_empty(0),
+                      geom, act)
+    return y.view(rows, N)
 
 
 class _SparseCE(torch.autograd.Function):

@@ -282,6 +282,40 @@ int hgq_qsoftmax_bwd(const float *dy, const float *x, float *dx, int64_t rows, i
                      const hgq_qdesc *inv_oq, const hgq_qdesc *oq, float *g_shared, float *g_oq_i, float *g_oq_fb,
                      float *workspace, void *stream);
 
+/*
+ * QConv2D contraction, forward.  Replaces `self.convolution_op(qinputs, self.qkernel)`, the bias
+ * add and the activation of QBaseConv.call (src/hgq/layers/conv.py:72-89; the Keras torch backend
+ * transposes to channels-first around a library convolution) with an implicit GEMM that reads the
+ * channels-last tensors in place.  With a 1 x 1 geometry (H = W = kh = kw = 1, C = K) it is the
+ * dense contraction of any width, `ops.matmul(qinputs, self.qkernel) + self.qbias`
+ * (src/hgq/layers/core/dense.py:60-68), used where K or N exceeds the fused dense kernels.
+ *
+ *   xq [B, H, W, C] quantized input;  qw [kh, kw, C, F] quantized kernel;  qb [F] or NULL;
+ *   y [B, OH, OW, F];  output pixel (oy, ox) reads input rows oy * sy - py + ky * dly (columns alike),
+ *   positions outside the input contribute zero ('same' padding: py, px = the top / left pad).
+ */
+typedef struct {
+    int B, H, W, C;   /* input: batch, height, width, channels */
+    int kh, kw;       /* kernel height, width */
+    int sy, sx;       /* strides */
+    int py, px;       /* zero padding before the first row / column */
+    int dly, dlx;     /* dilation */
+    int OH, OW;       /* output height, width */
+} hgq_conv_geom;
+int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb, float *y, const hgq_conv_geom *g, int F, int act,
+                   void *stream);
+
+/*
+ * QConv2D contraction, backward: autograd of the expression above.
+ *   dy, y [B, OH, OW, F] (y only for HGQ_ACT_RELU);  dxq [B, H, W, C] gradient w.r.t. the quantized
+ *   input (NULL to skip);  dqw [kh, kw, C, F], dqb [F] gradients w.r.t. the quantized kernel / bias
+ *   (NULL to skip);  workspace: hgq_conv2d_bwd_workspace(g, F) floats for the per-workgroup partial
+ *   sums of the weight gradient, added up in a fixed order by a second kernel.
+ */
+int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F);
+int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
+                   float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
+
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
 

@@ -1,0 +1,102 @@
+"""GPU parity of the implicit-GEMM convolution kernels (hgq_conv2d_fwd / hgq_conv2d_bwd) against
+the library routine they reduce to, evaluated in fp64 on the CPU: forward values and all three
+gradients within 1e-5 relative; exact where the operands are small integers (the EBOPs use)."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+
+def _ref_conv(x, w, b, strides, padding, dilation, relu):
+    """Channels-last reference in fp64; 'same' pads like Keras (odd pad after)."""
+    x = x.double().permute(0, 3, 1, 2)
+    wt = w.double().permute(3, 2, 0, 1)
+    if padding == 'same':
+        pads = []
+        for d in (1, 0):
+            n, k, s, dl = x.shape[2 + d], w.shape[d], strides[d], dilation[d]
+            total = max((-(-n // s) - 1) * s + dl * (k - 1) + 1 - n, 0)
+            pads += [total // 2, total - total // 2]
+        x = F.pad(x, pads)
+    y = F.conv2d(x, wt, None if b is None else b.double(), strides, 0, dilation).permute(0, 2, 3, 1)
+    return torch.relu(y) if relu else y
+
+
+CASES = [
+    # B, H, W, C, kh, kw, F, strides, padding, dilation, relu, bias
+    (1024 // 16, 28, 28, 1, 3, 3, 32, (1, 1), 'valid', (1, 1), True, True),    # first layer of the image configuration
+    (16, 13, 13, 32, 3, 3, 32, (1, 1), 'valid', (1, 1), True, True),           # second layer
+    (5, 10, 9, 3, 3, 3, 8, (2, 1), 'same', (1, 1), True, True),
+    (3, 12, 11, 5, 2, 4, 40, (1, 2), 'same', (1, 1), False, False),            # more than 32 filters: 64-wide tiles
+    (2, 9, 14, 40, 3, 3, 70, (2, 2), 'valid', (1, 1), True, True),             # more than 32 channels in the data gradient
+    (4, 11, 11, 6, 3, 3, 10, (1, 1), 'same', (2, 2), False, True),             # dilation
+    (7, 1, 1, 300, 1, 1, 10, (1, 1), 'valid', (1, 1), False, True),            # dense as 1 x 1
+    (0, 5, 5, 3, 3, 3, 4, (1, 1), 'valid', (1, 1), True, True),                # empty batch
+]
+
+
+@pytest.mark.parametrize('case', CASES)
+def test_conv2d_matches_fp64_reference(dev, case):
+    from hgq2_amd import _lib, ops
+
+    B, H, W, C, kh, kw, Fo, strides, padding, dilation, relu, bias = case
+    g = torch.Generator().manual_seed(hash(case) % 1000)
+    x = torch.randn(B, H, W, C, generator=g)
+    w = torch.randn(kh, kw, C, Fo, generator=g) * 0.3
+    b = torch.randn(Fo, generator=g) if bias else None
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    br = b.clone().requires_grad_(True) if bias else None
+    want = _ref_conv(xr, wr, br, strides, padding, dilation, relu)
+    xp, wp = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    bp = b.to(dev).requires_grad_(True) if bias else None
+    got = ops.conv2d(xp, wp, bp, strides, padding, dilation, _lib.ACT_RELU if relu else _lib.ACT_NONE)
+    assert tuple(got.shape) == tuple(want.shape)
+    if B == 0:
+        return
+    scale = want.abs().max().item() + 1e-9
+    assert float((got.detach().cpu().double() - want.detach()).abs().max()) <= 1e-5 * scale
+    up = torch.randn(want.shape, generator=g)
+    (want * up.double()).sum().backward()
+    (got * up.to(dev)).sum().backward()
+    for name, p, r in (('x', xp, xr), ('w', wp, wr)) + ((('b', bp, br),) if bias else ()):
+        gs = r.grad.abs().max().item() + 1e-9
+        err = float((p.grad.cpu().double() - r.grad.double()).abs().max())
+        assert err <= 2e-5 * gs, f'grad {name}: {err:.3e} vs scale {gs:.3e}'
+
+
+def test_conv2d_small_integers_exact(dev):
+    """Bit-width tensors convolved for EBOPs hold small integers: products and sums are exact in fp32."""
+    from hgq2_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randint(0, 12, (1, 28, 28, 4), generator=g).float()
+    w = torch.randint(0, 9, (3, 3, 4, 32), generator=g).float()
+    got = ops.conv2d(x.to(dev), w.to(dev), None)
+    want = _ref_conv(x, w, None, (1, 1), 'valid', (1, 1), False)
+    assert torch.equal(got.cpu().double(), want)
+
+
+def test_wide_dense_layer_matches_oracle(dev):
+    """QDense 3872 -> 10 (the classifier of the image configuration): beyond the fused dense
+    kernels, so the contraction runs in the 1 x 1 implicit-GEMM kernels."""
+    from hgq2_amd.layers import QDense
+    from tests import twin
+    from tests.test_gpu_more_layers import _compare_step, _perturb, readme_scopes
+
+    g = torch.Generator().manual_seed(9)
+    with readme_scopes():
+        layer = QDense(10)
+    x = torch.rand(64, 3872, generator=g)
+    layer(x.to(dev), training=True)
+    _perturb(layer, g)
+    r = twin.ref_dense(layer)
+    xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
+    named_p = [('x', xp), ('kernel', layer._kernel), ('bias', layer.bias), ('iq_f', layer.iq.quantizer._f),
+               ('kq_b', layer.kq.quantizer._b), ('kq_i', layer.kq.quantizer._i)]
+    named_r = [('x', xr), ('kernel', r.kernel), ('bias', r.bias), ('iq_f', r.iq.quantizer._f), ('kq_b', r.kq.quantizer._b),
+               ('kq_i', r.kq.quantizer._i)]
+    _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=1e-4)
+    assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
+    assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)
