@@ -56,7 +56,8 @@ SIGNATURES = {
     'hgq_qsoftmax_bwd_workspace': (c_int64, [c_int64, c_int, c_int64, c_int]),
     'hgq_qsoftmax_bwd': (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int64, c_float, c_float] + [c_void_p] * 5
                          + [c_void_p] * 4 + [c_void_p]),
-    'hgq_conv2d_fwd': (c_int, [c_void_p] * 5 + [c_int, c_int, c_void_p]),
+    'hgq_conv2d_fwd_workspace': (c_int64, [c_void_p, c_int]),
+    'hgq_conv2d_fwd': (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p]),
     'hgq_conv2d_bwd_workspace': (c_int64, [c_void_p, c_int]),
     'hgq_conv2d_bwd': (c_int, [c_void_p] * 9 + [c_int, c_int, c_void_p]),
 }

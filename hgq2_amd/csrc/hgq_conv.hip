@@ -97,8 +97,12 @@ template <int MODE, int WN>
 __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ src, const float *__restrict__ mask,
                                                     const float *__restrict__ w, const float *__restrict__ bias,
                                                     float *__restrict__ out, hgq_conv_geom g, int F, int64_t rows, int K,
-                                                    int N, int act) {
+                                                    int N, int act, int kchunk) {
+    // gridDim.z > 1: split along k; slice z of `out` ([gridDim.z, rows * N]) receives the raw partial sums
     constexpr int WM = 4 / WN, BM = 32 * WM, BN = 32 * WN;
+    const bool split = gridDim.z > 1;
+    const int k_begin = blockIdx.z * kchunk, k_end = min(K, k_begin + kchunk);
+    if (split) out += (int64_t)blockIdx.z * rows * N;
     __shared__ float as[BM][CV_BK + 1];
     __shared__ float bs[CV_BK][BN + 1];
     __shared__ RowInfo rinfo[BM];
@@ -113,8 +117,8 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
         if (tid < BM) rinfo[tid] = decode_row<MODE>(r0 + tid, rows, g);
         __syncthreads();
         floatx16 acc = {0};
-        for (int k0 = 0; k0 < K; k0 += CV_BK) {
-            const ColInfo ci = decode_col<MODE>(k0 + acol, K, g, F);
+        for (int k0 = k_begin; k0 < k_end; k0 += CV_BK) {
+            const ColInfo ci = decode_col<MODE>(k0 + acol, k_end, g, F);
 #pragma unroll 4
             for (int j = 0; j < BM / 8; ++j) {
                 const int row = arow0 + 8 * j;
@@ -127,7 +131,7 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
                 else nn = id / CV_BK, kk = id - nn * CV_BK;
                 const int k = k0 + kk, n = n0 + nn;
                 float v = 0.f;
-                if (k < K && n < N) {
+                if (k < k_end && n < N) {
                     if (MODE == 0) {
                         v = w[(int64_t)k * N + n];
                     } else {
@@ -148,13 +152,13 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
         }
         const int n = n0 + wn * 32 + (lane & 31);
         if (n < N) {
-            const float bv = (MODE == 0 && bias) ? bias[n] : 0.f;
+            const float bv = (MODE == 0 && bias && !split) ? bias[n] : 0.f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int64_t m = r0 + wm * 32 + cv_acc_row(r, lane);
                 if (m < rows) {
                     float v = acc[r] + bv;
-                    if (MODE == 0 && act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                    if (MODE == 0 && act == HGQ_ACT_RELU && !split) v = v > 0.f ? v : 0.f;
                     out[m * N + n] = v;
                 }
             }
@@ -162,19 +166,201 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
     }
 }
 
+// y = act(sum of the k-split slices + bias), slices added in order.
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const float *__restrict__ part, int n_parts, int64_t n,
+                                                            const float *__restrict__ bias, int N, int act,
+                                                            float *__restrict__ out) {
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+        float v = 0.f;
+        for (int p = 0; p < n_parts; ++p) v += part[(int64_t)p * n + e];
+        if (bias) v += bias[e % N];
+        if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+        out[e] = v;
+    }
+}
+
+// Data gradient for inputs with few channels (C <= 4, e.g. the image itself), where a matrix-core
+// tile would be almost empty.  FP = lanes per pixel (a power of two >= F): lane f of a pixel's
+// group keeps the kernel entries W[tap, c, f] in registers, accumulates dz[tap pixel, f] * W over
+// the taps with coalesced reads along f, and the group is summed with DPP steps at the end.
+#define DG_MAXW 8192
+// KH, KW > 0: kernel size known at compile time (all tap loads of a pixel in flight together); 0: any size.
+template <int FP, int KH, int KW>
+__global__ __launch_bounds__(256) void dgrad_smallc_kernel(const float *__restrict__ dz, const float *__restrict__ mask,
+                                                           const float *__restrict__ w, float *__restrict__ out,
+                                                           hgq_conv_geom g, int F, int64_t in_rows) {
+    constexpr int PPW = 64 / FP;  // pixels per wavefront step
+    extern __shared__ float wl[];  // the kernel, kh * kw * C * F floats
+    const int lane = threadIdx.x & 63, f = lane % FP, slot = lane / FP;
+    const int C = g.C, taps = g.kh * g.kw;
+    const bool f_on = f < F;
+    for (int t = threadIdx.x; t < taps * C * F; t += 256) wl[t] = w[t];
+    __syncthreads();
+    const bool unit = g.sy == 1 && g.sx == 1;
+    const int64_t wave_id = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6, n_waves = ((int64_t)gridDim.x * 256) >> 6;
+    for (int64_t m0 = wave_id * PPW; m0 < in_rows; m0 += n_waves * PPW) {
+        const int64_t m = m0 + slot;
+        const RowInfo r = decode_row<1>(m, in_rows, g);
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        if (KH > 0) {
+            constexpr int NT = KH * KW > 0 ? KH * KW : 1, KWD = KW > 0 ? KW : 1;
+            float v[NT], km[NT];
+            bool ok[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int ky = t / KWD, kx = t % KWD;
+                const int ty = r.y0 - ky * g.dly, tx = r.x0 - kx * g.dlx;
+                const int oy = unit ? ty : ty / g.sy, ox = unit ? tx : tx / g.sx;
+                ok[t] = r.base >= 0 && f_on && ty >= 0 && tx >= 0 && oy * g.sy == ty && ox * g.sx == tx && oy < g.OH && ox < g.OW;
+                const int64_t a = ok[t] ? ((int64_t)r.base + oy * g.OW + ox) * F + f : 0;
+                v[t] = dz[a];
+                km[t] = mask ? mask[a] : 1.f;
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const float vv = (ok[t] && km[t] > 0.f) ? v[t] : 0.f;
+                const float *wt = wl + t * C * F + (f_on ? f : 0);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (c < C) acc[c] += vv * wt[c * F];
+            }
+        } else {
+            // three taps at a time, loads issued together and unconditionally (clamped address)
+            for (int ky = 0; ky < g.kh; ++ky) {
+                const int ty = r.y0 - ky * g.dly;
+                const int oy = unit ? ty : ty / g.sy;
+                const bool oky = r.base >= 0 && f_on && ty >= 0 && oy * g.sy == ty && oy < g.OH;
+                for (int kx0 = 0; kx0 < g.kw; kx0 += 3) {
+                    float v[3], km[3];
+                    bool ok[3];
+#pragma unroll
+                    for (int u = 0; u < 3; ++u) {
+                        const int kx = kx0 + u;
+                        const int tx = r.x0 - kx * g.dlx;
+                        const int ox = unit ? tx : tx / g.sx;
+                        ok[u] = oky && kx < g.kw && tx >= 0 && ox * g.sx == tx && ox < g.OW;
+                        const int64_t a = ok[u] ? ((int64_t)r.base + oy * g.OW + ox) * F + f : 0;
+                        v[u] = dz[a];
+                        km[u] = mask ? mask[a] : 1.f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 3; ++u) {
+                        const int kx = kx0 + u;
+                        if (kx < g.kw) {
+                            const float vv = (ok[u] && km[u] > 0.f) ? v[u] : 0.f;
+                            const float *wt = wl + (ky * g.kw + kx) * C * F + (f_on ? f : 0);
+#pragma unroll
+                            for (int c = 0; c < 4; ++c)
+                                if (c < C) acc[c] += vv * wt[c * F];
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (c < C) {
+                const float tot = row_reduce_sum<FP>(acc[c]);
+                if (f == 0 && m < in_rows) out[m * C + c] = tot;
+            }
+        }
+    }
+}
+
+// The same for unit stride and dilation: a workgroup takes an 8 x 32 patch of input pixels,
+// stages the (8 + kh - 1) x (32 + kw - 1) patch of dz it needs (masked, read once, coalesced
+// along f) in LDS with the pixel stride padded to F + 1, and each thread contracts one pixel
+// from LDS.
+#define DP_TH 8
+#define DP_TW 32
+__global__ __launch_bounds__(256) void dgrad_patch_kernel(const float *__restrict__ dz, const float *__restrict__ mask,
+                                                          const float *__restrict__ w, float *__restrict__ out,
+                                                          hgq_conv_geom g, int F, int tiles_x, int tiles_y) {
+    extern __shared__ float lds[];  // [kh * kw * C * F] kernel | [(DP_TH + kh - 1) * (DP_TW + kw - 1)][F + 1] patch
+    const int C = g.C, taps = g.kh * g.kw;
+    float *wl = lds, *patch = lds + taps * C * F;
+    const int PH = DP_TH + g.kh - 1, PW = DP_TW + g.kw - 1, FS = F + 1;
+    for (int t = threadIdx.x; t < taps * C * F; t += 256) wl[t] = w[t];
+    const int tx = threadIdx.x % DP_TW, ty = threadIdx.x / DP_TW;
+    const int64_t n_tiles = (int64_t)g.B * tiles_y * tiles_x;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int b = (int)(tile / (tiles_y * tiles_x)), rem = (int)(tile - (int64_t)b * tiles_y * tiles_x);
+        const int iy0 = (rem / tiles_x) * DP_TH, ix0 = (rem % tiles_x) * DP_TW;
+        // patch origin in output coordinates: oy = iy + py - ky, ky = kh - 1 .. 0
+        const int oy0 = iy0 + g.py - (g.kh - 1), ox0 = ix0 + g.px - (g.kw - 1);
+        __syncthreads();
+        // 32 lanes along f, 8 pixel columns at a time: no per-element index division
+        const int fl = threadIdx.x & 31, pc0 = threadIdx.x >> 5;
+        for (int pr = 0; pr < PH; ++pr) {
+            const int oy = oy0 + pr;
+            const bool row_ok = (unsigned)oy < (unsigned)g.OH;
+            for (int pc = pc0; pc < PW; pc += 8) {
+                const int ox = ox0 + pc;
+                const bool ok = row_ok && (unsigned)ox < (unsigned)g.OW;
+                const int64_t a0 = (((int64_t)b * g.OH + oy) * g.OW + ox) * F;
+                for (int f = fl; f < F; f += 32) {
+                    float v = 0.f;
+                    if (ok) {
+                        v = dz[a0 + f];
+                        if (mask && !(mask[a0 + f] > 0.f)) v = 0.f;
+                    }
+                    patch[(pr * PW + pc) * FS + f] = v;
+                }
+            }
+        }
+        __syncthreads();
+        const int iy = iy0 + ty, ix = ix0 + tx;
+        if (iy < g.H && ix < g.W) {
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int ky = 0; ky < g.kh; ++ky)
+                for (int kx = 0; kx < g.kw; ++kx) {
+                    // oy = iy + py - ky  ->  patch row ty + (kh - 1) - ky
+                    const float *pp = patch + ((ty + g.kh - 1 - ky) * PW + (tx + g.kw - 1 - kx)) * FS;
+                    const float *wt = wl + (ky * g.kw + kx) * C * F;
+                    int f = 0;
+                    for (; f + 8 <= F; f += 8) {  // eight LDS reads in flight per operand
+                        float v[8];
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) v[u] = pp[f + u];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            if (c < C) {
+                                float wv[8];
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) wv[u] = wt[c * F + f + u];
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) acc[c] += v[u] * wv[u];
+                            }
+                        }
+                    }
+                    for (; f < F; ++f) {
+                        const float v = pp[f];
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+                            if (c < C) acc[c] += v * wt[c * F + f];
+                    }
+                }
+            const int64_t o = (((int64_t)b * g.H + iy) * g.W + ix) * C;
+            for (int c = 0; c < C; ++c) out[o + c] = acc[c];
+        }
+    }
+}
+
 // Weight / bias gradient.  Workgroup (kt, nt, split): k tile of 32 * WK columns of the im2col
-// matrix, n tile of 32 * (4 / WK) filters, rows [split * chunk, (split + 1) * chunk).
-// Slice `split` of `part` is [K * F | F].
-template <int WK>
+// matrix, n tile of 32 * WN filters, rows [split * chunk, (split + 1) * chunk) taken 32 * WS at
+// a step, WS wavefronts sharing one output block (combined through LDS at the end);
+// WK * WN * WS = 4.  Slice `split` of `part` is [K * F | F].
+template <int WK, int WN, int WS>
 __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ src, const float *__restrict__ dy,
                                                     const float *__restrict__ y, float *__restrict__ part, hgq_conv_geom g,
                                                     int F, int64_t rows, int K, int64_t chunk, int act, int n_ktiles) {
-    constexpr int WN = 4 / WK, BKT = 32 * WK, BN = 32 * WN, BMS = 32;
+    constexpr int BKT = 32 * WK, BN = 32 * WN, BMS = 32 * WS;
+    static_assert(WK * WN * WS == 4, "four wavefronts");
     __shared__ float as[BMS][BKT + 1];
     __shared__ float zs[BMS][BN + 1];
     __shared__ RowInfo rinfo[BMS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wk = wave / WN, wn = wave % WN;
+    const int wsub = wave / (WK * WN), wk = (wave / WN) % WK, wn = wave % WN;
     const int kt = blockIdx.x % n_ktiles, nt = blockIdx.x / n_ktiles;
     const int k0 = kt * BKT, n0 = nt * BN;
     const int64_t m_begin = (int64_t)blockIdx.y * chunk, m_end = min(rows, m_begin + chunk);
@@ -204,13 +390,31 @@ __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ sr
             bsum += v;
         }
         __syncthreads();
-        const int kq = lane >> 5, c32 = lane & 31;
+        const int kq = lane >> 5, c32 = lane & 31, mb = wsub * 32;
 #pragma unroll
-        for (int mm = 0; mm < BMS; mm += 2)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[mm + kq][wk * 32 + c32], zs[mm + kq][wn * 32 + c32], acc, 0, 0, 0);
+        for (int mm = 0; mm < 32; mm += 2)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[mb + mm + kq][wk * 32 + c32], zs[mb + mm + kq][wn * 32 + c32], acc, 0, 0, 0);
+    }
+    __syncthreads();
+    float *red = &as[0][0];  // BMS * (BKT + 1) >= 4096 floats whenever WS > 1
+    if (WS > 1) {
+        // the WS wavefronts of an output block add up in wavefront order
+        const int blk = wk * WN + wn;  // output block of this wavefront
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[((blk * WS + wsub) * 32 + cv_acc_row(r, lane)) * 32 + (lane & 31)] = acc[r];
+        __syncthreads();
+        if (wsub == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = 0.f;
+                for (int u = 0; u < WS; ++u) v += red[((blk * WS + u) * 32 + cv_acc_row(r, lane)) * 32 + (lane & 31)];
+                acc[r] = v;
+            }
+        }
+        __syncthreads();
     }
     const int n = n0 + wn * 32 + (lane & 31);
-    if (n < F) {
+    if (wsub == 0 && n < F) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int k = k0 + wk * 32 + cv_acc_row(r, lane);
@@ -219,8 +423,6 @@ __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ sr
     }
     if (kt == 0) {
         // bias gradient: threads with the same dz column add up in a fixed order
-        __syncthreads();
-        float *red = &as[0][0];
         red[tid] = bsum;
         __syncthreads();
         if (tid < BN && n0 + tid < F) {
@@ -229,6 +431,30 @@ __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ sr
             my[KF + n0 + tid] = s;
         }
     }
+}
+
+struct WgradCfg {
+    int wk, wn, ws;
+    int n_kt, n_nt;
+};
+static WgradCfg wgrad_cfg(int K, int F) {
+    WgradCfg c;
+    if (F > 32) c.wk = 2, c.wn = 2, c.ws = 1;
+    else if (K <= 32) c.wk = 1, c.wn = 1, c.ws = 4;
+    else if (K <= 64) c.wk = 2, c.wn = 1, c.ws = 2;
+    else c.wk = 4, c.wn = 1, c.ws = 1;
+    c.n_kt = (K + 32 * c.wk - 1) / (32 * c.wk), c.n_nt = (F + 32 * c.wn - 1) / (32 * c.wn);
+    return c;
+}
+
+// k-split of the forward for few output tiles and a long contraction (a wide dense layer on a small batch)
+static int fwd_ksplit(int64_t rows, int K, int F) {
+    const int64_t tiles = F <= 32 ? (rows + 127) / 128 : ((rows + 63) / 64) * ((F + 63) / 64);
+    if (tiles >= 256 || K < 512) return 1;
+    int64_t s = 512 / tiles;
+    if (s > K / 128) s = K / 128;
+    if (s > 64) s = 64;
+    return s < 1 ? 1 : (int)s;
 }
 
 static int check_geom(const hgq_conv_geom *g, int F, const char *who) {
@@ -256,8 +482,15 @@ static int64_t wgrad_splits(int64_t rows, int n_tiles_kn) {
 
 using namespace hgq;
 
-extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb, float *y, const hgq_conv_geom *g, int F,
-                              int act, void *stream) {
+extern "C" int64_t hgq_conv2d_fwd_workspace(const hgq_conv_geom *g, int F) {
+    if (check_geom(g, F, "hgq_conv2d_fwd_workspace")) return -1;
+    const int64_t rows = (int64_t)g->B * g->OH * g->OW;
+    const int ks = fwd_ksplit(rows, g->kh * g->kw * g->C, F);
+    return ks > 1 ? (int64_t)ks * rows * F : 0;
+}
+
+extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb, float *y, float *workspace,
+                              const hgq_conv_geom *g, int F, int act, void *stream) {
     int rc = check_geom(g, F, "hgq_conv2d_fwd");
     if (rc) return rc;
     if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_conv2d_fwd: unknown activation %d", act);
@@ -266,23 +499,35 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
     if (!xq || !qw || !y) return fail(HGQ_ERR_ARG, "hgq_conv2d_fwd: null pointer");
     const int K = g->kh * g->kw * g->C;
     hipStream_t s = (hipStream_t)stream;
+    const int ks = fwd_ksplit(rows, K, F);
+    if (ks > 1 && !workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_fwd: this shape needs the workspace");
+    int kchunk = (K + ks - 1) / ks;
+    kchunk = (kchunk + CV_BK - 1) / CV_BK * CV_BK;
+    const int nz = (K + kchunk - 1) / kchunk;
+    float *dst = nz > 1 ? workspace : y;
     if (F <= 32) {
-        const dim3 grid((unsigned)persistent_grid((rows + 127) / 128, 8), 1);
-        hipLaunchKernelGGL((igemm_kernel<0, 1>), grid, dim3(256), 0, s, xq, (const float *)nullptr, qw, qb, y, *g, F, rows, K, F, act);
+        const dim3 grid((unsigned)persistent_grid((rows + 127) / 128, 8), 1, (unsigned)nz);
+        hipLaunchKernelGGL((igemm_kernel<0, 1>), grid, dim3(256), 0, s, xq, (const float *)nullptr, qw, qb, dst, *g, F, rows, K, F, act, kchunk);
     } else {
-        const dim3 grid((unsigned)persistent_grid((rows + 63) / 64, 8), (unsigned)((F + 63) / 64));
-        hipLaunchKernelGGL((igemm_kernel<0, 2>), grid, dim3(256), 0, s, xq, (const float *)nullptr, qw, qb, y, *g, F, rows, K, F, act);
+        const dim3 grid((unsigned)persistent_grid((rows + 63) / 64, 8), (unsigned)((F + 63) / 64), (unsigned)nz);
+        hipLaunchKernelGGL((igemm_kernel<0, 2>), grid, dim3(256), 0, s, xq, (const float *)nullptr, qw, qb, dst, *g, F, rows, K, F, act, kchunk);
     }
-    return check_launch("hgq_conv2d_fwd");
+    if ((rc = check_launch("hgq_conv2d_fwd"))) return rc;
+    if (nz > 1) {
+        const int64_t n = rows * F;
+        hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)persistent_grid((n + 255) / 256, 8)), dim3(256), 0, s, workspace, nz, n, qb, F,
+                           act, y);
+        return check_launch("hgq_conv2d_fwd(finish)");
+    }
+    return HGQ_OK;
 }
 
 extern "C" int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F) {
     if (check_geom(g, F, "hgq_conv2d_bwd_workspace")) return -1;
     const int64_t rows = (int64_t)g->B * g->OH * g->OW;
     const int K = g->kh * g->kw * g->C;
-    const int wk = F <= 32 ? 4 : 2;
-    const int n_kn = ((K + 32 * wk - 1) / (32 * wk)) * ((F + 32 * (4 / wk) - 1) / (32 * (4 / wk)));
-    return wgrad_splits(rows, n_kn) * ((int64_t)K * F + F);
+    const WgradCfg c = wgrad_cfg(K, F);
+    return wgrad_splits(rows, c.n_kt * c.n_nt) * ((int64_t)K * F + F);
 }
 
 extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw,
@@ -305,27 +550,48 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
     const float *mask = act == HGQ_ACT_RELU ? y : nullptr;
     if (dxq) {
         const int Kt = g->kh * g->kw * F;  // contraction length of the data gradient
-        if (g->C <= 32) {
+        const size_t patch_lds = ((size_t)g->kh * g->kw * g->C * F + (size_t)(DP_TH + g->kh - 1) * (DP_TW + g->kw - 1) * (F + 1)) * sizeof(float);
+        if (g->C <= 4 && g->sy == 1 && g->sx == 1 && g->dly == 1 && g->dlx == 1 && patch_lds <= 64 * 1024) {
+            const int tiles_x = (g->W + DP_TW - 1) / DP_TW, tiles_y = (g->H + DP_TH - 1) / DP_TH;
+            const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
+            hipLaunchKernelGGL(dgrad_patch_kernel, grid, dim3(256), patch_lds, s, dy, mask, qw, dxq, *g, F, tiles_x, tiles_y);
+        } else if (g->C <= 4 && (int64_t)g->kh * g->kw * g->C * F <= DG_MAXW && F <= 64) {
+            const int fp = F <= 16 ? 16 : (F <= 32 ? 32 : 64);
+            const dim3 grid((unsigned)persistent_grid((in_rows * fp + 255) / 256, 16));
+            const size_t lds = (size_t)g->kh * g->kw * g->C * F * sizeof(float);
+            const bool k33 = g->kh == 3 && g->kw == 3;
+#define HGQ_DG(FPV) \
+    do { \
+        if (k33) hipLaunchKernelGGL((dgrad_smallc_kernel<FPV, 3, 3>), grid, dim3(256), lds, s, dy, mask, qw, dxq, *g, F, in_rows); \
+        else hipLaunchKernelGGL((dgrad_smallc_kernel<FPV, 0, 0>), grid, dim3(256), lds, s, dy, mask, qw, dxq, *g, F, in_rows); \
+    } while (0)
+            if (fp == 16) HGQ_DG(16);
+            else if (fp == 32) HGQ_DG(32);
+            else HGQ_DG(64);
+#undef HGQ_DG
+        } else if (g->C <= 32) {
             const dim3 grid((unsigned)persistent_grid((in_rows + 127) / 128, 8), 1);
-            hipLaunchKernelGGL((igemm_kernel<1, 1>), grid, dim3(256), 0, s, dy, mask, qw, (const float *)nullptr, dxq, *g, F, in_rows, Kt, g->C, act);
+            hipLaunchKernelGGL((igemm_kernel<1, 1>), grid, dim3(256), 0, s, dy, mask, qw, (const float *)nullptr, dxq, *g, F, in_rows, Kt, g->C, act, Kt);
         } else {
             const dim3 grid((unsigned)persistent_grid((in_rows + 63) / 64, 8), (unsigned)((g->C + 63) / 64));
-            hipLaunchKernelGGL((igemm_kernel<1, 2>), grid, dim3(256), 0, s, dy, mask, qw, (const float *)nullptr, dxq, *g, F, in_rows, Kt, g->C, act);
+            hipLaunchKernelGGL((igemm_kernel<1, 2>), grid, dim3(256), 0, s, dy, mask, qw, (const float *)nullptr, dxq, *g, F, in_rows, Kt, g->C, act, Kt);
         }
         if ((rc = check_launch("hgq_conv2d_bwd(data)"))) return rc;
     }
     if (dqw || dqb) {
         if (!workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null workspace");
-        const int wk = F <= 32 ? 4 : 2;
-        const int n_kt = (K + 32 * wk - 1) / (32 * wk), n_nt = (F + 32 * (4 / wk) - 1) / (32 * (4 / wk));
-        const int64_t splits = wgrad_splits(rows, n_kt * n_nt);
+        const WgradCfg c = wgrad_cfg(K, F);
+        const int64_t splits = wgrad_splits(rows, c.n_kt * c.n_nt);
         int64_t chunk = (rows + splits - 1) / splits;
-        chunk = (chunk + 31) / 32 * 32;
-        const dim3 grid((unsigned)(n_kt * n_nt), (unsigned)splits);
-        if (wk == 4)
-            hipLaunchKernelGGL((wgrad_kernel<4>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, n_kt);
-        else
-            hipLaunchKernelGGL((wgrad_kernel<2>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, n_kt);
+        chunk = (chunk + 127) / 128 * 128;
+        const dim3 grid((unsigned)(c.n_kt * c.n_nt), (unsigned)splits);
+#define HGQ_WGRAD(WK, WN, WS) \
+    hipLaunchKernelGGL((wgrad_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt)
+        if (c.wk == 2 && c.wn == 2) HGQ_WGRAD(2, 2, 1);
+        else if (c.wk == 1) HGQ_WGRAD(1, 1, 4);
+        else if (c.wk == 2) HGQ_WGRAD(2, 1, 2);
+        else HGQ_WGRAD(4, 1, 1);
+#undef HGQ_WGRAD
         if ((rc = check_launch("hgq_conv2d_bwd(weights)"))) return rc;
         const int64_t M = KF + F;
         if ((rc = reduce_parts(workspace, (int)splits, M, dqw, KF, dqb, (int64_t)F, nullptr, 0, s))) return rc;

@@ -163,6 +163,41 @@ __device__ __forceinline__ float ceil_log2_exact(float v) {
     return (float)(mant == 0.5f ? e - 1 : e);
 }
 
+// ------------------------------------------------------------------------------------------
+// all-reduce over groups of SUB consecutive lanes (SUB = 16, 32 or 64): four DPP steps inside
+// each 16-lane row (xor 1, xor 2, half-row mirror, row mirror), then the row totals are read
+// back through scalar registers
+// ------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+struct OpMax {
+    static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
+};
+struct OpAdd {
+    static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+};
+template <int SUB, class Op>
+__device__ __forceinline__ float sub_reduce(float v) {
+    v = Op::f(v, dpp_mov<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = Op::f(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = Op::f(v, dpp_mov<0x141>(v));  // row_half_mirror
+    v = Op::f(v, dpp_mov<0x140>(v));  // row_mirror
+    if (SUB == 16) return v;
+    const float r0 = lane_value(v, 0), r1 = lane_value(v, 16), r2 = lane_value(v, 32), r3 = lane_value(v, 48);
+    const float a = Op::f(r0, r1), b = Op::f(r2, r3);
+    if (SUB == 32) return (threadIdx.x & 32) ? b : a;
+    return Op::f(a, b);
+}
+template <int SUB>
+__device__ __forceinline__ float row_reduce_sum(float v) { return sub_reduce<SUB, OpAdd>(v); }
+template <int SUB>
+__device__ __forceinline__ float row_reduce_max(float v) { return sub_reduce<SUB, OpMax>(v); }
+
 }  // namespace hgq
 
 // dispatch a (round_mode, overflow_mode) pair to template arguments

@@ -353,7 +353,11 @@ def conv2d_fwd(xq: Tensor, qw: Tensor, qb: Tensor, geom: Sequence[int], act: int
         _check_f32('qb', qb)
         _need(qb.numel() == F, 'bias size mismatch')
     y = torch.empty((g.B, g.OH, g.OW, F), dtype=torch.float32, device=xq.device)
-    rc = _lib.load().hgq_conv2d_fwd(_ptr(xq), _ptr(qw), _ptr(qb), _ptr(y), ctypes.addressof(g), F, act, _stream())
+    lib = _lib.load()
+    n_ws = lib.hgq_conv2d_fwd_workspace(ctypes.addressof(g), F)
+    _need(n_ws >= 0, 'hgq_conv2d_fwd_workspace rejected the geometry')
+    ws = torch.empty(int(n_ws), dtype=torch.float32, device=xq.device)
+    rc = lib.hgq_conv2d_fwd(_ptr(xq), _ptr(qw), _ptr(qb), _ptr(y), _ptr(ws), ctypes.addressof(g), F, act, _stream())
     _lib.check(rc, 'hgq_conv2d_fwd')
     return y
 

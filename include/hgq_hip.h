@@ -292,7 +292,9 @@ int hgq_qsoftmax_bwd(const float *dy, const float *x, float *dx, int64_t rows, i
  *
  *   xq [B, H, W, C] quantized input;  qw [kh, kw, C, F] quantized kernel;  qb [F] or NULL;
  *   y [B, OH, OW, F];  output pixel (oy, ox) reads input rows oy * sy - py + ky * dly (columns alike),
- *   positions outside the input contribute zero ('same' padding: py, px = the top / left pad).
+ *   positions outside the input contribute zero ('same' padding: py, px = the top / left pad);
+ *   workspace: hgq_conv2d_fwd_workspace(g, F) floats (0 for most shapes; a long contraction with few
+ *   output tiles is split along k and the slices are added by a second kernel), may be NULL if 0.
  */
 typedef struct {
     int B, H, W, C;   /* input: batch, height, width, channels */
@@ -302,8 +304,9 @@ typedef struct {
     int dly, dlx;     /* dilation */
     int OH, OW;       /* output height, width */
 } hgq_conv_geom;
-int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb, float *y, const hgq_conv_geom *g, int F, int act,
-                   void *stream);
+int64_t hgq_conv2d_fwd_workspace(const hgq_conv_geom *g, int F);
+int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb, float *y, float *workspace, const hgq_conv_geom *g,
+                   int F, int act, void *stream);
 
 /*
  * QConv2D contraction, backward: autograd of the expression above.

@@ -34,6 +34,10 @@ CASES = [
     (4, 11, 11, 6, 3, 3, 10, (1, 1), 'same', (2, 2), False, True),             # dilation
     (7, 1, 1, 300, 1, 1, 10, (1, 1), 'valid', (1, 1), False, True),            # dense as 1 x 1
     (0, 5, 5, 3, 3, 3, 4, (1, 1), 'valid', (1, 1), True, True),                # empty batch
+    (6, 9, 9, 2, 3, 3, 10, (1, 1), 'same', (1, 1), True, True),                # few channels, filters not a multiple of 4
+    (48, 1, 1, 3872, 1, 1, 10, (1, 1), 'valid', (1, 1), True, True),           # long contraction, few rows: split along k
+    (300, 6, 6, 2, 3, 3, 24, (1, 1), 'valid', (1, 1), True, True),             # K = 18: row-split weight gradient
+    (40, 8, 8, 5, 3, 3, 16, (1, 1), 'valid', (1, 1), False, True),             # K = 45: two k blocks, two row groups
 ]
 
 
