@@ -165,7 +165,7 @@ def softmax_roofline(iters=50, shape=(2048, 4, 64, 64), scaler=0.25):
     return out
 
 
-def config_step_time(name, steps=20, warmup=5):
+def config_step_time(name, steps=20, warmup=5, graph=False):
     """One forward + backward pass of the configurations other than the headline one, at their full
     sizes: 'particle' (QEinsumDenseBatchnorm per-particle network, batch 4096 x 64 x 16), 'conv'
     (QConv2D stack on 28 x 28 x 1, batch 1024), 'mha' (QMultiHeadAttention, batch 2048 x 64 x 64)."""
@@ -205,15 +205,36 @@ def config_step_time(name, steps=20, warmup=5):
         loss.backward()
         return loss
 
+    run = step
+    if graph:
+        # the step is tens to hundreds of small launches: record it once, replay it
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for p in model.parameters():
+            p.grad = None
+        g_ = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_):
+            static_loss = step()
+
+        def run():
+            g_.replay()
+            return static_loss
+
     for _ in range(warmup):
-        step()
+        run()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        loss = step()
+        loss = run()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / steps * 1e3
-    return {'workload': name, 'batch': batch, 'ms_per_step': ms, 'samples_per_s': batch / ms * 1e3, 'loss': float(loss)}
+    return {'workload': name, 'batch': batch, 'ms_per_step': ms, 'samples_per_s': batch / ms * 1e3, 'loss': float(loss),
+            'launch': 'hip-graph replay' if graph else 'eager'}
 
 
 def cpu_baseline(budget_s=20.0):
@@ -252,6 +273,7 @@ def main():
                     help='run only the standalone quantizer kernels and a plain copy of known size (for counter runs)')
     ap.add_argument('--config-step', choices=('particle', 'conv', 'mha'), default=None,
                     help='time one forward + backward pass of another configuration at full size instead of the headline run')
+    ap.add_argument('--graph', action='store_true', help='with --config-step: capture the step in a HIP graph and replay it')
     ap.add_argument('--softmax-only', action='store_true',
                     help='run only the one-pass table-softmax kernels at the attention configuration (for profiler runs)')
     ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused',
@@ -270,7 +292,7 @@ def main():
         return
     if args.config_step:
         torch.cuda.set_device(0)
-        print(json.dumps({'config_step': config_step_time(args.config_step, steps=args.steps if args.steps != 300 else 20)}))
+        print(json.dumps({'config_step': config_step_time(args.config_step, steps=args.steps if args.steps != 300 else 20, graph=args.graph)}))
         return
     if args.softmax_only:
         torch.cuda.set_device(0)

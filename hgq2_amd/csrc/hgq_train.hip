@@ -173,6 +173,72 @@ __global__ __launch_bounds__(256) void sgd_multi_kernel(SgdBatch b, float lr) {
     }
 }
 
+
+// ------------------------------------------------------------------------------------------
+// per-column first and second moments of a [rows, N] matrix (batch-normalisation statistics)
+// ------------------------------------------------------------------------------------------
+// A thread owns VEC adjacent columns and walks down the rows; the workgroup's TY row groups are
+// combined through LDS and written to slice blockIdx.y of `part` ([gridDim.y, 2 * N]: sums, then
+// sums of squares), which reduce_parts adds up in a fixed order.
+template <int VEC>
+__global__ __launch_bounds__(256) void col_moments_kernel(const float *__restrict__ x, int64_t rows, int N, int TX,
+                                                          float *__restrict__ part) {
+    __shared__ float s1[256 * VEC], s2[256 * VEC];
+    const int TY = 256 / TX;
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t cg = N / VEC;
+    const int64_t c = (int64_t)blockIdx.x * TX + tx;
+    float a1[VEC], a2[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) a1[e] = 0.f, a2[e] = 0.f;
+    if (c < cg) {
+        for (int64_t r = (int64_t)blockIdx.y * TY + ty; r < rows; r += (int64_t)gridDim.y * TY) {
+            float v[VEC];
+            if (VEC == 4) {
+                const float4 t = *(const float4 *)(x + (r * cg + c) * 4);
+                v[0] = t.x, v[1 % VEC] = t.y, v[2 % VEC] = t.z, v[3 % VEC] = t.w;
+            } else {
+                v[0] = x[r * cg + c];
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) a1[e] += v[e], a2[e] += v[e] * v[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) s1[threadIdx.x * VEC + e] = a1[e], s2[threadIdx.x * VEC + e] = a2[e];
+    __syncthreads();
+    for (int st = TY / 2; st > 0; st >>= 1) {
+        if (ty < st) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                s1[threadIdx.x * VEC + e] += s1[(threadIdx.x + st * TX) * VEC + e];
+                s2[threadIdx.x * VEC + e] += s2[(threadIdx.x + st * TX) * VEC + e];
+            }
+        }
+        __syncthreads();
+    }
+    if (ty == 0 && c < cg) {
+        float *my = part + (int64_t)blockIdx.y * 2 * N;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) my[c * VEC + e] = s1[tx * VEC + e], my[N + c * VEC + e] = s2[tx * VEC + e];
+    }
+}
+
+__global__ __launch_bounds__(256) void col_moments_scale_kernel(float *mean, float *meansq, int N, float inv_rows) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t < N) mean[t] *= inv_rows, meansq[t] *= inv_rows;
+}
+
+// dx[r, c] = (dmean[c] + 2 x[r, c] dmeansq[c]) / rows
+__global__ __launch_bounds__(256) void col_moments_bwd_kernel(const float *__restrict__ x, const float *__restrict__ dmean,
+                                                              const float *__restrict__ dmeansq, int64_t n, int N,
+                                                              float inv_rows, float *__restrict__ dx) {
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+        const int c = (int)(e % N);
+        dx[e] = (dmean[c] + 2.0f * x[e] * dmeansq[c]) * inv_rows;
+    }
+}
+
 }  // namespace hgq
 
 using namespace hgq;
@@ -235,4 +301,57 @@ extern "C" int hgq_sgd_update(float *w, const float *g, int64_t n, float lr, flo
     const int grid = persistent_grid((n + 255) / 256, 8);
     hipLaunchKernelGGL(sgd_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, w, g, n, lr, l1, lo, hi);
     return check_launch("hgq_sgd_update");
+}
+
+static inline int moments_layout(int64_t rows, int N, bool vec, int &TX, int64_t &gx, int64_t &gy) {
+    const int64_t cg = vec ? N / 4 : N;
+    TX = 1;
+    while (TX * 2 <= cg && TX < 64) TX *= 2;
+    const int TY = 256 / TX;
+    gx = (cg + TX - 1) / TX;
+    gy = (rows + TY - 1) / TY;
+    int64_t cap = (int64_t)persistent_grid(1 << 30, 4) / gx;
+    if (cap > 256) cap = 256;
+    if (gy > cap) gy = cap < 1 ? 1 : cap;
+    return 0;
+}
+
+extern "C" int64_t hgq_col_moments_workspace(int64_t rows, int N) {
+    if (rows < 0 || N < 1) return -1;
+    int TX;
+    int64_t gx, gy;
+    moments_layout(rows, N, N % 4 == 0, TX, gx, gy);
+    return gy * 2 * N;
+}
+
+extern "C" int hgq_col_moments_fwd(const float *x, int64_t rows, int N, float *mean, float *meansq, float *workspace,
+                                   void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (rows < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_col_moments_fwd: bad sizes");
+    if (!x || !mean || !meansq || !workspace) return fail(HGQ_ERR_ARG, "hgq_col_moments_fwd: null pointer");
+    const bool vec = N % 4 == 0 && ((uintptr_t)x & 15u) == 0;
+    int TX;
+    int64_t gx, gy;
+    moments_layout(rows, N, N % 4 == 0, TX, gx, gy);
+    if (!vec && N % 4 == 0) moments_layout(rows, N, false, TX, gx, gy), gy = hgq_col_moments_workspace(rows, N) / (2 * N);
+    if (vec)
+        hipLaunchKernelGGL((col_moments_kernel<4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, rows, N, TX, workspace);
+    else
+        hipLaunchKernelGGL((col_moments_kernel<1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, rows, N, TX, workspace);
+    int rc = check_launch("hgq_col_moments_fwd");
+    if (rc) return rc;
+    if ((rc = reduce_parts(workspace, (int)gy, 2 * (int64_t)N, mean, N, meansq, N, nullptr, 0, s))) return rc;
+    hipLaunchKernelGGL(col_moments_scale_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, mean, meansq, N, 1.0f / (float)rows);
+    return check_launch("hgq_col_moments_fwd(scale)");
+}
+
+extern "C" int hgq_col_moments_bwd(const float *x, const float *dmean, const float *dmeansq, int64_t rows, int N, float *dx,
+                                   void *stream) {
+    if (rows < 0 || N < 1) return fail(HGQ_ERR_ARG, "hgq_col_moments_bwd: bad sizes");
+    if (rows == 0) return HGQ_OK;
+    if (!x || !dmean || !dmeansq || !dx) return fail(HGQ_ERR_ARG, "hgq_col_moments_bwd: null pointer");
+    const int64_t n = rows * N;
+    hipLaunchKernelGGL(col_moments_bwd_kernel, dim3((unsigned)persistent_grid((n + 255) / 256, 16)), dim3(256), 0, (hipStream_t)stream, x, dmean,
+                       dmeansq, n, N, 1.0f / (float)rows, dx);
+    return check_launch("hgq_col_moments_bwd");
 }

@@ -8,6 +8,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
+from .. import _lib, ops
 from ..core import epsilon, get_initializer
 from .core.einsum_dense import QEinsumDense, analyze_einsum_string
 
@@ -85,13 +86,32 @@ class QEinsumDenseBatchnorm(QEinsumDense):
     def qbias(self):
         return self.get_fused_qkernel_and_qbias(False, self.moving_mean, self.moving_variance)[1]
 
+    def _batch_moments(self, qinputs):
+        """Mean and variance of the un-quantized-kernel pre-activation over the non-normalised axes
+        (reference :108-112).  GEMM-shaped equations whose normalised axes are all the new output axes
+        run through the dense and column-moment kernels; others through the library einsum."""
+        n_out = len(self.full_output_shape)
+        trailing = self._gemm is not None and self._reduction_axes == tuple(range(n_out - self._gemm[1]))
+        if trailing and qinputs.is_cuda:
+            x2d = qinputs.reshape(-1, self._K)
+            w2d = self._kernel.reshape(self._K, self._N)
+            if self._K <= ops.FUSED_BWD_MAX and self._N <= ops.FUSED_BWD_MAX:
+                pre, _ = ops.qdense(x2d.contiguous(), None, None, None, w2d, None, _lib.ACT_NONE, 0, 0, False)
+            else:
+                pre = ops.matmul_bias_act(x2d, w2d, None, _lib.ACT_NONE)
+            mean, meansq = ops.col_moments(pre)
+            shape = tuple(self.full_output_shape[n_out - self._gemm[1]:])
+            mean, meansq = mean.view(shape), meansq.view(shape)
+            return mean, meansq - torch.square(mean)
+        x = torch.einsum(self.equation, qinputs, self._kernel)
+        mean = torch.mean(x, dim=self._reduction_axes)
+        return mean, torch.mean(torch.square(x), dim=self._reduction_axes) - torch.square(mean)
+
     def call(self, inputs, training=None):
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
         if training and self.trainable:
-            x = torch.einsum(self.equation, inputs, self._kernel)
-            mean = torch.mean(x, dim=self._reduction_axes)
-            var = torch.mean(torch.square(x), dim=self._reduction_axes) - torch.square(mean)
+            mean, var = self._batch_moments(inputs)
             with torch.no_grad():
                 self.moving_mean.copy_(self.moving_mean * self.momentum + mean * (1.0 - self.momentum))
                 self.moving_variance.copy_(self.moving_variance * self.momentum + var * (1.0 - self.momentum))

@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments']
 
 
 def _ptr(t: Tensor | None):
@@ -392,6 +392,41 @@ def _(dy, y, xq, qw, geom, act, need_dx, has_bias):
     return (xq.new_empty(xq.shape if need_dx else (0,)), torch.empty_like(qw), xq.new_empty(qw.shape[-1] if has_bias else 0))
 
 
+@torch.library.custom_op('hgq::col_moments_fwd', mutates_args=())
+def col_moments_fwd(x: Tensor) -> tuple[Tensor, Tensor]:
+    _check_f32('x', x)
+    _need(x.dim() == 2 and x.shape[0] >= 1, 'x must be [rows >= 1, N]')
+    rows, N = x.shape
+    lib = _lib.load()
+    mean = torch.empty(N, dtype=torch.float32, device=x.device)
+    meansq = torch.empty(N, dtype=torch.float32, device=x.device)
+    ws = torch.empty(int(lib.hgq_col_moments_workspace(rows, N)), dtype=torch.float32, device=x.device)
+    rc = lib.hgq_col_moments_fwd(_ptr(x), rows, N, _ptr(mean), _ptr(meansq), _ptr(ws), _stream())
+    _lib.check(rc, 'hgq_col_moments_fwd')
+    return mean, meansq
+
+
+@col_moments_fwd.register_fake
+def _(x):
+    return x.new_empty(x.shape[1]), x.new_empty(x.shape[1])
+
+
+@torch.library.custom_op('hgq::col_moments_bwd', mutates_args=())
+def col_moments_bwd(x: Tensor, dmean: Tensor, dmeansq: Tensor) -> Tensor:
+    _check_f32('x', x), _check_f32('dmean', dmean), _check_f32('dmeansq', dmeansq)
+    rows, N = x.shape
+    _need(dmean.numel() == N and dmeansq.numel() == N, 'gradient size mismatch')
+    dx = torch.empty_like(x)
+    rc = _lib.load().hgq_col_moments_bwd(_ptr(x), _ptr(dmean), _ptr(dmeansq), rows, N, _ptr(dx), _stream())
+    _lib.check(rc, 'hgq_col_moments_bwd')
+    return dx
+
+
+@col_moments_bwd.register_fake
+def _(x, dmean, dmeansq):
+    return torch.empty_like(x)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -603,6 +638,26 @@ def matmul_bias_act(x2d: Tensor, qw: Tensor, qb, act: int = 0) -> Tensor:
     y = _Conv2D.apply(x2d.contiguous(), qw.contiguous().view(1, 1, K, N), qb.contiguous() if qb is not None else x2d.new_empty(0),
                       geom, act)
     return y.view(rows, N)
+
+
+class _ColMoments(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        mean, meansq = col_moments_fwd(x)
+        ctx.save_for_backward(x)
+        return mean, meansq
+
+    @staticmethod
+    def backward(ctx, gm, gs):
+        (x,) = ctx.saved_tensors
+        gm = torch.zeros(x.shape[1], device=x.device) if gm is None else gm.contiguous()
+        gs = torch.zeros(x.shape[1], device=x.device) if gs is None else gs.contiguous()
+        return col_moments_bwd(x, gm, gs)
+
+
+def col_moments(x2d: Tensor):
+    """``(mean(x, 0), mean(x * x, 0))`` of a [rows, N] matrix in one pass."""
+    return _ColMoments.apply(x2d.contiguous())
 
 
 class _SparseCE(torch.autograd.Function):

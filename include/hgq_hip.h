@@ -319,6 +319,19 @@ int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F);
 int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
                    float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
 
+/*
+ * Per-column mean and mean of squares of a [rows, N] matrix, and the gradient of both.  Replaces
+ * `ops.mean(x, axis)` / `ops.mean(ops.square(x), axis)` and their autograd in
+ * QEinsumDenseBatchnorm.call (src/hgq/layers/einsum_dense_batchnorm.py:99-124, the batch
+ * statistics of the un-quantized pre-activation) when the normalised axes are the trailing ones.
+ *   mean, meansq [N];  workspace: hgq_col_moments_workspace(rows, N) floats (partial sums per
+ *   workgroup, added in a fixed order);  dx[r, c] = (dmean[c] + 2 x[r, c] dmeansq[c]) / rows.
+ */
+int64_t hgq_col_moments_workspace(int64_t rows, int N);
+int hgq_col_moments_fwd(const float *x, int64_t rows, int N, float *mean, float *meansq, float *workspace, void *stream);
+int hgq_col_moments_bwd(const float *x, const float *dmean, const float *dmeansq, int64_t rows, int N, float *dx,
+                        void *stream);
+
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
 
