@@ -295,6 +295,323 @@ __global__ __launch_bounds__(256) void qdense_bwd_kernel(const float *__restrict
         for (int64_t t = tid; t < PK; t += 256) my_df[t] = df_s[t];
 }
 
+// ------------------------------------------------------------------------------------------
+// streaming variants for the common case: K, N <= 64, K a multiple of 4, the input quantizer (if
+// any) on its WRAP training branch (round only) with a bit-width table whose row count divides 64
+// ------------------------------------------------------------------------------------------
+// A tile is 64 rows, so the table row of a staged element, (tile row) % P, is the same in every
+// tile: a thread keeps the fractional bits and the abs-max / gradient accumulators of the elements
+// it stages in registers for the whole launch.  The next tile's global loads are issued before
+// the current tile's MFMAs, and the staged tile is double buffered (one barrier per tile).
+#define FAST_BM 64
+#define FAST_LD 65
+#define FAST_NJ 4  // 128-bit loads per thread and tile: 64 * K / 4 / 256 <= 4
+
+struct FastMap {
+    int row[FAST_NJ], col[FAST_NJ];
+    bool on[FAST_NJ];
+    __device__ __forceinline__ void init(int W) {  // W = row width in floats, a multiple of 4
+        const int w4 = W >> 2;
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            const int id = threadIdx.x + 256 * j;
+            on[j] = id < FAST_BM * w4;
+            row[j] = on[j] ? id / w4 : 0;
+            col[j] = on[j] ? (id - row[j] * w4) << 2 : 0;
+        }
+    }
+};
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld4_or_zero(const float *p, bool ok) {
+    if (!ok) return make_float4(0.f, 0.f, 0.f, 0.f);
+    const f32x4_t t = __builtin_nontemporal_load((const f32x4_t *)p);
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void st4(float *p, const float4 &v) {
+    f32x4_t t;
+    t.x = v.x, t.y = v.y, t.z = v.z, t.w = v.w;
+    __builtin_nontemporal_store(t, (f32x4_t *)p);
+}
+
+template <int RM, bool QUANT>
+__global__ __launch_bounds__(256) void qdense_fwd_fast_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
+                                                              int P, const float *__restrict__ qw,
+                                                              const float *__restrict__ qb, float *__restrict__ y,
+                                                              uint32_t *amax_part, int64_t rows, int K, int N, int act,
+                                                              int mode) {
+    __shared__ float xs[2][FAST_BM][FAST_LD];
+    __shared__ float ws[64][FAST_LD];
+    const Mode m(mode);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rh = wave & 1, cb = wave >> 1;
+    const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
+    for (int id = tid; id < 64 * 64; id += 256) {
+        const int kk = id >> 6, nn = id & 63;
+        ws[kk][nn] = (kk < K && nn < N) ? qw[(int64_t)kk * N + nn] : 0.f;
+        xs[0][kk][nn] = 0.f, xs[1][kk][nn] = 0.f;  // columns >= K stay zero
+    }
+    FastMap mp;
+    mp.init(K);
+    int fi[FAST_NJ][4];
+    uint32_t amx[FAST_NJ][4];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            amx[j][e] = 0, fi[j][e] = 0;
+            if (QUANT && mp.on[j]) {
+                const float f = f_in[(mp.row[j] % P) * K + mp.col[j] + e];
+                fi[j][e] = (int)(m.round_params ? rintf(f) : f);
+            }
+        }
+    float4 raw[FAST_NJ];
+    int64_t tile = blockIdx.x;
+    if (tile < n_tiles) {
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            const int64_t gr = tile * FAST_BM + mp.row[j];
+            raw[j] = ld4_or_zero(x + gr * K + mp.col[j], mp.on[j] && gr < rows);
+        }
+    }
+    const int K2 = (K + 1) & ~1;
+    int buf = 0;
+    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            if (mp.on[j]) {
+                float v[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (QUANT) {
+                        v[e] = ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]);
+                        amx[j][e] = max(amx[j][e], abs_bits(v[e]));
+                    }
+                    xs[buf][mp.row[j]][mp.col[j] + e] = v[e];
+                }
+            }
+        }
+        __syncthreads();
+        const int64_t next = tile + gridDim.x;
+        if (next < n_tiles) {
+#pragma unroll
+            for (int j = 0; j < FAST_NJ; ++j) {
+                const int64_t gr = next * FAST_BM + mp.row[j];
+                raw[j] = ld4_or_zero(x + gr * K + mp.col[j], mp.on[j] && gr < rows);
+            }
+        }
+        if (cb * 32 < N) {
+            floatx16 acc = {0};
+            const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
+            for (int kk = 0; kk < K2; kk += 2)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[buf][arow][kk + kq], ws[kk + kq][bcol], acc, 0, 0, 0);
+            const int n = bcol;
+            if (n < N) {
+                const float bias = qb ? qb[n] : 0.f;
+                const int64_t r0 = tile * FAST_BM + rh * 32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t gr = r0 + acc_row(r, lane);
+                    if (gr < rows) {
+                        float v = acc[r] + bias;
+                        if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                        y[gr * N + n] = v;
+                    }
+                }
+            }
+        }
+    }
+    if (QUANT && amax_part) {
+        // this workgroup's slice: combine the registers of all threads through an LDS table
+        const int PK = P * K;
+        uint32_t *tab = (uint32_t *)&xs[0][0][0];
+        __syncthreads();
+        for (int t = tid; t < PK; t += 256) tab[t] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j)
+            if (mp.on[j])
+#pragma unroll
+                for (int e = 0; e < 4; ++e) atomicMax(&tab[(mp.row[j] % P) * K + mp.col[j] + e], amx[j][e]);
+        __syncthreads();
+        uint32_t *my = amax_part + (int64_t)blockIdx.x * PK;
+        for (int t = tid; t < PK; t += 256) my[t] = tab[t];
+    }
+}
+
+// Backward.  Per tile: stage dz = dy (masked by y for ReLU) and the quantized input; dx = dz W^T
+// and dW += xq^T dz on MFMA; dx goes back through LDS so that it is stored with 128-bit writes and
+// meets the rounding residue (xq - x) of the staging thread for the fractional-bit gradient.
+// Slice blockIdx.x of `part` is [K * N | N | P * K].
+template <int RM, bool QUANT>
+__global__ __launch_bounds__(256) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
+                                                              const float *__restrict__ x, const float *__restrict__ f_in,
+                                                              int P, const float *__restrict__ qw, float *__restrict__ dx,
+                                                              float *part, int has_bias, int64_t rows, int K, int N, int act,
+                                                              int mode) {
+    __shared__ float xs[FAST_BM][FAST_LD];
+    __shared__ float dzs[FAST_BM][FAST_LD];  // dz, then the dx tile
+    __shared__ float ws[64][FAST_LD];
+    const Mode m(mode);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5;
+    const int PK = QUANT ? P * K : 0;
+    const int64_t M = (int64_t)K * N + N + PK;
+    const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
+    float *my_dw = part + (int64_t)blockIdx.x * M;
+    float *my_db = my_dw + (int64_t)K * N;
+    float *my_df = my_db + N;
+    for (int id = tid; id < 64 * 64; id += 256) {
+        const int kk = id >> 6, nn = id & 63;
+        ws[kk][nn] = (kk < K && nn < N) ? qw[(int64_t)kk * N + nn] : 0.f;
+        xs[kk][nn] = 0.f, dzs[kk][nn] = 0.f;
+    }
+    FastMap mx, mz;
+    mx.init(K), mz.init(N);
+    int fi[FAST_NJ][4];
+    float gf[FAST_NJ][4];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            gf[j][e] = 0.f, fi[j][e] = 0;
+            if (QUANT && mx.on[j]) {
+                const float f = f_in[(mx.row[j] % P) * K + mx.col[j] + e];
+                fi[j][e] = (int)(m.round_params ? rintf(f) : f);
+            }
+        }
+    // kernel-gradient block owned by this wave
+    const int nblk = K32 * N32, wpb = 4 / nblk;
+    const int blk = wave / wpb, sub = wave % wpb;
+    const int wkb = blk / N32, wnb = blk % N32;
+    const int rows_per = FAST_BM / wpb;
+    floatx16 accw = {0};
+    float accb = 0.f;
+    const int bn = tid & 63, bq = tid >> 6;
+    const bool relu = act == HGQ_ACT_RELU;
+
+    float4 rx[FAST_NJ], rg[FAST_NJ], ry[FAST_NJ];
+    int64_t tile = blockIdx.x;
+    auto load_tile = [&](int64_t t) {
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            const int64_t gx = t * FAST_BM + mx.row[j], gz = t * FAST_BM + mz.row[j];
+            rx[j] = ld4_or_zero(x + gx * K + mx.col[j], mx.on[j] && gx < rows);
+            rg[j] = ld4_or_zero(dy + gz * N + mz.col[j], mz.on[j] && gz < rows);
+            ry[j] = relu ? ld4_or_zero(y + gz * N + mz.col[j], mz.on[j] && gz < rows) : make_float4(1.f, 1.f, 1.f, 1.f);
+        }
+    };
+    if (tile < n_tiles) load_tile(tile);
+    for (; tile < n_tiles; tile += gridDim.x) {
+        float dlt[FAST_NJ][4];  // xq - x of the elements this thread stages
+        __syncthreads();        // previous tile's dx has been read back
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            if (mx.on[j]) {
+                const float v[4] = {rx[j].x, rx[j].y, rx[j].z, rx[j].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float q = QUANT ? ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]) : v[e];
+                    dlt[j][e] = q - v[e];
+                    xs[mx.row[j]][mx.col[j] + e] = q;
+                }
+            }
+            if (mz.on[j]) {
+                const float g[4] = {rg[j].x, rg[j].y, rg[j].z, rg[j].w};
+                const float a[4] = {ry[j].x, ry[j].y, ry[j].z, ry[j].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dzs[mz.row[j]][mz.col[j] + e] = a[e] > 0.f ? g[e] : 0.f;
+            }
+        }
+        __syncthreads();
+        const int64_t next = tile + gridDim.x;
+        const int64_t r0 = tile * FAST_BM;
+        if (next < n_tiles) load_tile(next);
+        // ---- dx = dz @ qW^T : blocks (row half, k block), kept in registers until dz is no longer needed
+        floatx16 acc = {0};
+        const int rh = wave & 1, kb = wave >> 1;
+        if (kb < K32) {
+            const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
+            const int nsteps = N32 * 32;
+            for (int nn = 0; nn < nsteps; nn += 2)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(dzs[arow][nn + kq], ws[wrow][nn + kq], acc, 0, 0, 0);
+        }
+        // ---- dW += xq^T @ dz : this wave's block, its slice of the tile's rows
+        {
+            const int rbeg = sub * rows_per;
+            const int kq = lane >> 5, c32 = lane & 31;
+            for (int rr = rbeg; rr < rbeg + rows_per; rr += 2)
+                accw = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[rr + kq][wkb * 32 + c32], dzs[rr + kq][wnb * 32 + c32], accw, 0, 0, 0);
+        }
+        if (has_bias) {
+#pragma unroll
+            for (int j = 0; j < FAST_BM / 4; ++j) accb += dzs[bq * (FAST_BM / 4) + j][bn];
+        }
+        __syncthreads();  // dz consumed: the dx tile takes its place
+        if (kb < K32) {
+            const int kcol = kb * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dzs[rh * 32 + acc_row(r, lane)][kcol] = acc[r];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            if (mx.on[j]) {
+                const int64_t gr = r0 + mx.row[j];
+                float4 o;
+                o.x = dzs[mx.row[j]][mx.col[j]], o.y = dzs[mx.row[j]][mx.col[j] + 1];
+                o.z = dzs[mx.row[j]][mx.col[j] + 2], o.w = dzs[mx.row[j]][mx.col[j] + 3];
+                if (gr < rows) {
+                    st4(dx + gr * K + mx.col[j], o);
+                    if (QUANT) {
+                        gf[j][0] += -HGQ_LN2 * dlt[j][0] * o.x, gf[j][1] += -HGQ_LN2 * dlt[j][1] * o.y;
+                        gf[j][2] += -HGQ_LN2 * dlt[j][2] * o.z, gf[j][3] += -HGQ_LN2 * dlt[j][3] * o.w;
+                    }
+                }
+            }
+        }
+    }
+    // ---- write this workgroup's slice.  Waves sharing a kernel-gradient block combine through LDS.
+    __syncthreads();
+    float *comb = &xs[0][0];
+    for (int pass = 0; pass < wpb; ++pass) {
+        if (sub == pass) {
+            const int n = wnb * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int k = wkb * 32 + acc_row(r, lane);
+                if (pass == 0) comb[k * FAST_LD + n] = accw[r];
+                else comb[k * FAST_LD + n] += accw[r];
+            }
+        }
+        __syncthreads();
+    }
+    for (int id = tid; id < K * N; id += 256) my_dw[id] = comb[(id / N) * FAST_LD + (id % N)];
+    float *bred = &ws[0][0];
+    __syncthreads();
+    bred[tid] = accb;
+    __syncthreads();
+    if (tid < N) my_db[tid] = has_bias ? bred[tid] + bred[tid + 64] + bred[tid + 128] + bred[tid + 192] : 0.f;
+    if (QUANT) {
+        // fractional-bit gradient: every (tile row, column) has one owner thread; rows that share a
+        // table row are added in row order
+        float *gt = &dzs[0][0];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j)
+            if (mx.on[j])
+#pragma unroll
+                for (int e = 0; e < 4; ++e) gt[mx.row[j] * FAST_LD + mx.col[j] + e] = gf[j][e];
+        __syncthreads();
+        for (int t = tid; t < PK; t += 256) {
+            const int p = t / K, c = t - p * K;
+            float s = 0.f;
+            for (int r = p; r < FAST_BM; r += P) s += gt[r * FAST_LD + c];
+            my_df[t] = s;
+        }
+    }
+}
+
 // out[e] = sum over slices of part[g][e], in slice order.  256 threads = 64 elements x 4 slice groups.
 __global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restrict__ part, int n_parts, int64_t M,
                                                            float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb,
@@ -372,6 +689,18 @@ extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_i
     const int amax_lds = (quant && amax_part && PK <= AMAX_LDS_MAX) ? 1 : 0;
     const size_t dyn = amax_lds ? (size_t)PK * 4 : 0;
     const int vec_ok = (K % 4 == 0) && aligned16(x);
+    const bool wrap_train = quant && m.overflow_mode == HGQ_WRAP && m.training && !m.kbi;
+    const bool fast = (!quant || wrap_train) && K <= 64 && N <= 64 && K % 4 == 0 && aligned16(x) &&
+                      (!quant || (bw_rows <= 64 && 64 % bw_rows == 0));
+    if (fast) {
+        const dim3 fgrid((unsigned)row_parts(rows, FWD_BM));
+        const int P = quant ? (int)bw_rows : 1;
+        if (!quant) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_TRN, false>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, (uint32_t *)nullptr, rows, K, N, act, mode);
+        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_TRN, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode);
+        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_RND, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode);
+        else hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_RND_CONV, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode);
+        return check_launch("hgq_qdense_fwd");
+    }
     const dim3 grid((unsigned)row_parts(rows, FWD_BM), (unsigned)((N + FWD_BN - 1) / FWD_BN));
     if (!quant) {
         hipLaunchKernelGGL((qdense_fwd_kernel<HGQ_TRN, HGQ_WRAP, false>), grid, dim3(256), dyn, s, x, k_in, i_in, f_in, (int64_t)1, qw, qb, y,
@@ -408,6 +737,23 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
         if (dqb && (rc = fill_f32(dqb, 0.f, N, s))) return rc;
         if (df_in && (rc = fill_f32(df_in, 0.f, PK, s))) return rc;
         return HGQ_OK;
+    }
+    const bool fast = K % 4 == 0 && N % 4 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx) && (act != HGQ_ACT_RELU || aligned16(y)) &&
+                      (!quant || (bw_rows <= 64 && 64 % bw_rows == 0));
+    if (fast) {
+        const int parts = row_parts(rows, BWD_BM);
+        const int P = quant ? (int)bw_rows : 1;
+        const dim3 fgrid((unsigned)parts);
+#define HGQ_BWD_FAST(RMV, QV) \
+    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, dqb ? 1 : 0, rows, K, N, act, mode)
+        if (!quant) HGQ_BWD_FAST(HGQ_TRN, false);
+        else if (m.round_mode == HGQ_TRN) HGQ_BWD_FAST(HGQ_TRN, true);
+        else if (m.round_mode == HGQ_RND) HGQ_BWD_FAST(HGQ_RND, true);
+        else HGQ_BWD_FAST(HGQ_RND_CONV, true);
+#undef HGQ_BWD_FAST
+        int rc = check_launch("hgq_qdense_bwd");
+        if (rc) return rc;
+        return reduce_parts(workspace, parts, M, dqw, (int64_t)K * N, dqb, (int64_t)N, quant ? df_in : (float *)nullptr, PK, s);
     }
     const int df_lds = (quant && PK <= DF_LDS_MAX) ? 1 : 0;
     const size_t dyn = df_lds ? (size_t)PK * 4 : 0;
