@@ -9,6 +9,7 @@ import math
 
 import torch
 
+from ... import ops
 from ...core import Constant
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
@@ -179,11 +180,13 @@ class QMultiHeadAttention(QLayerBase):
         return out
 
     def _compute_attention(self, query, key, value, attention_mask=None, training=None):
-        query = query * self._inverse_sqrt_key_dim
-        scores = torch.einsum(_DOT_EQ, key, query)
+        if self._inverse_sqrt_key_dim != 1.0:  # 1 after build: the scale lives in the softmax's exp table
+            query = query * self._inverse_sqrt_key_dim
+        own = query.is_cuda and max(query.shape[1], key.shape[1], query.shape[3], value.shape[3]) <= ops.ATTN_MAX
+        scores = ops.attn_scores(query, key) if own else torch.einsum(_DOT_EQ, key, query)
         mask = None
         if attention_mask is not None:
             mask = attention_mask.unsqueeze(1)  # broadcast over heads
         scores = self._softmax(scores, mask=mask)
         final = torch.nn.functional.dropout(scores, self._dropout) if (self._dropout and training) else scores
-        return torch.einsum(_COMBINE_EQ, final, value), scores
+        return (ops.attn_combine(final, value) if own else torch.einsum(_COMBINE_EQ, final, value)), scores

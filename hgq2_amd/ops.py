@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX']
 
 
 def _ptr(t: Tensor | None):
@@ -427,6 +427,81 @@ def _(x, dmean, dmeansq):
     return torch.empty_like(x)
 
 
+ATTN_MAX = 64  # the attention contraction kernels cover sequence lengths and head sizes up to 64
+
+
+def _attn_dims(a: Tensor, b: Tensor):
+    """a [B, T, N, H], b [B, S, N, H] -> (B, T, S, N, H)"""
+    _need(a.dim() == 4 and b.dim() == 4 and a.shape[0] == b.shape[0] and a.shape[2:] == b.shape[2:], 'operands must be [B, seq, N, H]')
+    return a.shape[0], a.shape[1], b.shape[1], a.shape[2], a.shape[3]
+
+
+@torch.library.custom_op('hgq::attn_scores_fwd', mutates_args=())
+def attn_scores_fwd(query: Tensor, key: Tensor) -> Tensor:
+    _check_f32('query', query), _check_f32('key', key)
+    B, T, S, N, H = _attn_dims(query, key)
+    scores = torch.empty((B, N, T, S), dtype=torch.float32, device=query.device)
+    rc = _lib.load().hgq_attn_scores_fwd(_ptr(query), _ptr(key), _ptr(scores), B, T, S, N, H, _stream())
+    _lib.check(rc, 'hgq_attn_scores_fwd')
+    return scores
+
+
+@attn_scores_fwd.register_fake
+def _(query, key):
+    return query.new_empty((query.shape[0], query.shape[2], query.shape[1], key.shape[1]))
+
+
+@torch.library.custom_op('hgq::attn_scores_bwd', mutates_args=())
+def attn_scores_bwd(dscores: Tensor, query: Tensor, key: Tensor) -> tuple[Tensor, Tensor]:
+    _check_f32('dscores', dscores), _check_f32('query', query), _check_f32('key', key)
+    B, T, S, N, H = _attn_dims(query, key)
+    _need(tuple(dscores.shape) == (B, N, T, S), 'dscores must be [B, N, T, S]')
+    dq, dk = torch.empty_like(query), torch.empty_like(key)
+    rc = _lib.load().hgq_attn_scores_bwd(_ptr(dscores), _ptr(query), _ptr(key), _ptr(dq), _ptr(dk), B, T, S, N, H, _stream())
+    _lib.check(rc, 'hgq_attn_scores_bwd')
+    return dq, dk
+
+
+@attn_scores_bwd.register_fake
+def _(dscores, query, key):
+    return torch.empty_like(query), torch.empty_like(key)
+
+
+@torch.library.custom_op('hgq::attn_combine_fwd', mutates_args=())
+def attn_combine_fwd(probs: Tensor, value: Tensor) -> Tensor:
+    _check_f32('probs', probs), _check_f32('value', value)
+    _need(probs.dim() == 4 and value.dim() == 4, 'probs [B, N, T, S], value [B, S, N, H]')
+    B, N, T, S = probs.shape
+    _need(value.shape[0] == B and value.shape[1] == S and value.shape[2] == N, 'value must be [B, S, N, H]')
+    H = value.shape[3]
+    out = torch.empty((B, T, N, H), dtype=torch.float32, device=probs.device)
+    rc = _lib.load().hgq_attn_combine_fwd(_ptr(probs), _ptr(value), _ptr(out), B, T, S, N, H, _stream())
+    _lib.check(rc, 'hgq_attn_combine_fwd')
+    return out
+
+
+@attn_combine_fwd.register_fake
+def _(probs, value):
+    return probs.new_empty((probs.shape[0], probs.shape[2], probs.shape[1], value.shape[3]))
+
+
+@torch.library.custom_op('hgq::attn_combine_bwd', mutates_args=())
+def attn_combine_bwd(dout: Tensor, probs: Tensor, value: Tensor) -> tuple[Tensor, Tensor]:
+    _check_f32('dout', dout), _check_f32('probs', probs), _check_f32('value', value)
+    B, N, T, S = probs.shape
+    H = value.shape[3]
+    _need(tuple(dout.shape) == (B, T, N, H), 'dout must be [B, T, N, H]')
+    dp, dv = torch.empty_like(probs), torch.empty_like(value)
+    rc = _lib.load().hgq_attn_combine_bwd(_ptr(dout), _ptr(probs), _ptr(value), _ptr(dp), _ptr(dv), B, T, S, N, H, _stream())
+    _lib.check(rc, 'hgq_attn_combine_bwd')
+    return dp, dv
+
+
+@attn_combine_bwd.register_fake
+def _(dout, probs, value):
+    return torch.empty_like(probs), torch.empty_like(value)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -658,6 +733,40 @@ class _ColMoments(torch.autograd.Function):
 def col_moments(x2d: Tensor):
     """``(mean(x, 0), mean(x * x, 0))`` of a [rows, N] matrix in one pass."""
     return _ColMoments.apply(x2d.contiguous())
+
+
+class _AttnScores(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, query, key):
+        ctx.save_for_backward(query, key)
+        return attn_scores_fwd(query, key)
+
+    @staticmethod
+    def backward(ctx, g):
+        query, key = ctx.saved_tensors
+        return attn_scores_bwd(g.contiguous(), query, key)
+
+
+class _AttnCombine(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, probs, value):
+        ctx.save_for_backward(probs, value)
+        return attn_combine_fwd(probs, value)
+
+    @staticmethod
+    def backward(ctx, g):
+        probs, value = ctx.saved_tensors
+        return attn_combine_bwd(g.contiguous(), probs, value)
+
+
+def attn_scores(query: Tensor, key: Tensor) -> Tensor:
+    """``einsum('aecd,abcd->acbe', key, query)``: query [B, T, N, H], key [B, S, N, H] -> [B, N, T, S]."""
+    return _AttnScores.apply(query.contiguous(), key.contiguous())
+
+
+def attn_combine(probs: Tensor, value: Tensor) -> Tensor:
+    """``einsum('acbe,aecd->abcd', probs, value)``: probs [B, N, T, S], value [B, S, N, H] -> [B, T, N, H]."""
+    return _AttnCombine.apply(probs.contiguous(), value.contiguous())
 
 
 class _SparseCE(torch.autograd.Function):

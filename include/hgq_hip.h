@@ -332,6 +332,23 @@ int hgq_col_moments_fwd(const float *x, int64_t rows, int N, float *mean, float 
 int hgq_col_moments_bwd(const float *x, const float *dmean, const float *dmeansq, int64_t rows, int N, float *dx,
                         void *stream);
 
+/*
+ * The two score contractions of QMultiHeadAttention._compute_attention for rank-3 inputs
+ * (src/hgq/layers/attn/mha.py:418-470; einsum strings built by Keras, imported at mha.py:10):
+ *     scores[b, n, t, s] = sum_h query[b, t, n, h] * key[b, s, n, h]        'aecd,abcd->acbe'
+ *     out[b, t, n, h]    = sum_s probs[b, n, t, s] * value[b, s, n, h]      'acbe,aecd->abcd'
+ * and their autograd, reading the projections in their own [B, seq, N, H] layout (the reference
+ * path permutes and copies around a batched library GEMM).  T, S, H <= 64.
+ *   query / dquery [B, T, N, H];  key, value / dkey, dvalue [B, S, N, H];  scores, probs and their
+ *   gradients [B, N, T, S];  out / dout [B, T, N, H].  Gradient outputs may be NULL to skip.
+ */
+int hgq_attn_scores_fwd(const float *query, const float *key, float *scores, int B, int T, int S, int N, int H, void *stream);
+int hgq_attn_scores_bwd(const float *dscores, const float *query, const float *key, float *dquery, float *dkey, int B, int T,
+                        int S, int N, int H, void *stream);
+int hgq_attn_combine_fwd(const float *probs, const float *value, float *out, int B, int T, int S, int N, int H, void *stream);
+int hgq_attn_combine_bwd(const float *dout, const float *probs, const float *value, float *dprobs, float *dvalue, int B, int T,
+                         int S, int N, int H, void *stream);
+
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
 

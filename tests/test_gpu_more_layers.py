@@ -215,3 +215,28 @@ def test_einsum_dense_many_tracker_slices(dev):
     _close(got, want, what='output')
     assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
     assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+
+
+@pytest.mark.parametrize('dims', [(8, 64, 64, 4, 16), (5, 12, 20, 2, 8), (3, 33, 7, 3, 40), (2, 64, 64, 1, 64)])
+def test_attention_contractions_match_einsum(dev, dims):
+    """hgq_attn_scores / hgq_attn_combine and their gradients against the einsum strings they replace (fp64)."""
+    from hgq2_amd import ops
+
+    B, T, S, N, H = dims
+    g = torch.Generator().manual_seed(B * 100 + T)
+    q, k, v = (torch.randn(B, L, N, H, generator=g) for L in (T, S, S))
+    p = torch.rand(B, N, T, S, generator=g)
+    refs = [t.double().requires_grad_(True) for t in (q, k, v, p)]
+    outs = [t.to(dev).requires_grad_(True) for t in (q, k, v, p)]
+    want_s = torch.einsum('aecd,abcd->acbe', refs[1], refs[0])
+    want_o = torch.einsum('acbe,aecd->abcd', refs[3], refs[2])
+    got_s = ops.attn_scores(outs[0], outs[1])
+    got_o = ops.attn_combine(outs[3], outs[2])
+    us, uo = torch.randn(want_s.shape, generator=g), torch.randn(want_o.shape, generator=g)
+    ((want_s * us.double()).sum() + (want_o * uo.double()).sum()).backward()
+    ((got_s * us.to(dev)).sum() + (got_o * uo.to(dev)).sum()).backward()
+    for name, a, b in [('scores', got_s, want_s), ('out', got_o, want_o)] + [
+            (f'grad {n}', o.grad, r.grad) for n, o, r in zip('qkvp', outs, refs)]:
+        scale = b.abs().max().item() + 1e-9
+        err = float((a.detach().cpu().double() - b.detach()).abs().max())
+        assert err <= 1e-5 * scale, f'{name}: {err:.3e} vs scale {scale:.3e}'
