@@ -18,29 +18,51 @@
 namespace hgq {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
-#define AT_LD 65
-typedef float AtTile[64][AT_LD];
+typedef float f32x4_a __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int at_acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
 
+// An operand tile in LDS: 64 rows of `ld` floats (ld odd, >= padded width + 1), zero padded.
+struct Tile {
+    float *p;
+    int ld;
+    __device__ __forceinline__ float at(int r, int c) const { return p[r * ld + c]; }
+};
+__host__ __device__ inline int tile_ld(int W) { return ((W + 3) & ~3) + 1; }
+
 // C block (rb, cb) of sum_k A(i, k) B(k, j), k < K2 (even); TA / TB read the LDS tile transposed.
 template <bool TA, bool TB>
-__device__ __forceinline__ floatx16 tile_mma(const AtTile &As, const AtTile &Bs, int K2, int rb, int cb, int lane) {
+__device__ __forceinline__ floatx16 tile_mma(const Tile &A, const Tile &B, int K2, int rb, int cb, int lane) {
     floatx16 acc = {0};
     const int i = rb * 32 + (lane & 31), j = cb * 32 + (lane & 31), kq = lane >> 5;
     for (int k = 0; k < K2; k += 2) {
-        const float a = TA ? As[k + kq][i] : As[i][k + kq];
-        const float b = TB ? Bs[j][k + kq] : Bs[k + kq][j];
+        const float a = TA ? A.at(k + kq, i) : A.at(i, k + kq);
+        const float b = TB ? B.at(j, k + kq) : B.at(k + kq, j);
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
     }
     return acc;
 }
 
-// Stage a [R, W] operand whose rows are `ld` floats apart into a zero-padded 64 x 64 tile.
-__device__ __forceinline__ void stage(AtTile &dst, const float *__restrict__ src, int R, int W, int64_t ld) {
-    for (int id = threadIdx.x; id < 64 * 64; id += 256) {
-        const int r = id >> 6, c = id & 63;
-        dst[r][c] = (r < R && c < W) ? src[(int64_t)r * ld + c] : 0.f;
+// Stage a [R, W] operand whose rows are `ld` floats apart into a tile, zero padded to 64 rows and
+// to a multiple of 4 columns; 128-bit loads when W is a multiple of 4 and the rows are aligned.
+__device__ __forceinline__ void stage(const Tile &t, const float *__restrict__ src, int R, int W, int64_t ld) {
+    const int W4 = (W + 3) >> 2;
+    const bool vec = (W & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)src & 15u) == 0;
+    for (int id = threadIdx.x; id < 64 * W4; id += 256) {
+        const int r = id / W4, c = (id - r * W4) << 2;
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (r < R) {
+            if (vec) {
+                const f32x4_a q = __builtin_nontemporal_load((const f32x4_a *)(src + (int64_t)r * ld + c));
+                v[0] = q.x, v[1] = q.y, v[2] = q.z, v[3] = q.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (c + e < W) v[e] = src[(int64_t)r * ld + c + e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t.p[r * t.ld + c + e] = v[e];
     }
 }
 
@@ -60,37 +82,36 @@ struct AttnDims {
     int B, T, S, N, H;
 };
 
+// One workgroup per (batch, head) pair; dynamic LDS holds the operand tiles back to back.
+#define AT_PROLOGUE                                                                             \
+    extern __shared__ float lds[];                                                              \
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, rb = wave & 1, cb = wave >> 1; \
+    const int64_t ld = (int64_t)d.N * d.H;                                                      \
+    const int64_t pair = blockIdx.x, b = pair / d.N, n = pair % d.N;                            \
+    const int ldh = tile_ld(d.H), lds_ = tile_ld(d.S);                                          \
+    (void)lds_, (void)ldh
+
 __global__ __launch_bounds__(256) void attn_scores_fwd_kernel(const float *__restrict__ q, const float *__restrict__ k,
                                                               float *__restrict__ scores, AttnDims d) {
-    __shared__ AtTile qs, ks;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, rb = wave & 1, cb = wave >> 1;
-    const int64_t ld = (int64_t)d.N * d.H;
-    for (int64_t pair = blockIdx.x; pair < (int64_t)d.B * d.N; pair += gridDim.x) {
-        const int64_t b = pair / d.N, n = pair % d.N;
-        __syncthreads();
-        stage(qs, q + (b * d.T * d.N + n) * d.H, d.T, d.H, ld);
-        stage(ks, k + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
-        __syncthreads();
-        const floatx16 acc = tile_mma<false, true>(qs, ks, (d.H + 1) & ~1, rb, cb, lane);
-        store_block(acc, scores + pair * d.T * d.S, d.T, d.S, d.S, rb, cb, lane);
-    }
+    AT_PROLOGUE;
+    const Tile qs = {lds, ldh}, ks = {lds + 64 * ldh, ldh};
+    stage(qs, q + (b * d.T * d.N + n) * d.H, d.T, d.H, ld);
+    stage(ks, k + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
+    __syncthreads();
+    const floatx16 acc = tile_mma<false, true>(qs, ks, (d.H + 1) & ~1, rb, cb, lane);
+    store_block(acc, scores + pair * d.T * d.S, d.T, d.S, d.S, rb, cb, lane);
 }
 
 __global__ __launch_bounds__(256) void attn_combine_fwd_kernel(const float *__restrict__ p, const float *__restrict__ v,
                                                                float *__restrict__ out, AttnDims d) {
-    __shared__ AtTile ps, vs;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, rb = wave & 1, cb = wave >> 1;
-    const int64_t ld = (int64_t)d.N * d.H;
-    for (int64_t pair = blockIdx.x; pair < (int64_t)d.B * d.N; pair += gridDim.x) {
-        const int64_t b = pair / d.N, n = pair % d.N;
-        __syncthreads();
-        stage(ps, p + pair * d.T * d.S, d.T, d.S, d.S);
-        stage(vs, v + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
-        __syncthreads();
-        if (cb * 32 < d.H) {
-            const floatx16 acc = tile_mma<false, false>(ps, vs, (d.S + 1) & ~1, rb, cb, lane);
-            store_block(acc, out + (b * d.T * d.N + n) * d.H, d.T, d.H, ld, rb, cb, lane);
-        }
+    AT_PROLOGUE;
+    const Tile ps = {lds, lds_}, vs = {lds + 64 * lds_, ldh};
+    stage(ps, p + pair * d.T * d.S, d.T, d.S, d.S);
+    stage(vs, v + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
+    __syncthreads();
+    if (cb * 32 < d.H) {
+        const floatx16 acc = tile_mma<false, false>(ps, vs, (d.S + 1) & ~1, rb, cb, lane);
+        store_block(acc, out + (b * d.T * d.N + n) * d.H, d.T, d.H, ld, rb, cb, lane);
     }
 }
 
@@ -98,24 +119,19 @@ __global__ __launch_bounds__(256) void attn_combine_fwd_kernel(const float *__re
 __global__ __launch_bounds__(256) void attn_combine_bwd_kernel(const float *__restrict__ dout, const float *__restrict__ p,
                                                                const float *__restrict__ v, float *__restrict__ dp,
                                                                float *__restrict__ dv, AttnDims d) {
-    __shared__ AtTile ps, vs, gs;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, rb = wave & 1, cb = wave >> 1;
-    const int64_t ld = (int64_t)d.N * d.H;
-    for (int64_t pair = blockIdx.x; pair < (int64_t)d.B * d.N; pair += gridDim.x) {
-        const int64_t b = pair / d.N, n = pair % d.N;
-        __syncthreads();
-        stage(ps, p + pair * d.T * d.S, d.T, d.S, d.S);
-        stage(vs, v + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
-        stage(gs, dout + (b * d.T * d.N + n) * d.H, d.T, d.H, ld);
-        __syncthreads();
-        if (dp) {
-            const floatx16 acc = tile_mma<false, true>(gs, vs, (d.H + 1) & ~1, rb, cb, lane);
-            store_block(acc, dp + pair * d.T * d.S, d.T, d.S, d.S, rb, cb, lane);
-        }
-        if (dv && cb * 32 < d.H) {
-            const floatx16 acc = tile_mma<true, false>(ps, gs, (d.T + 1) & ~1, rb, cb, lane);
-            store_block(acc, dv + (b * d.S * d.N + n) * d.H, d.S, d.H, ld, rb, cb, lane);
-        }
+    AT_PROLOGUE;
+    const Tile ps = {lds, lds_}, vs = {lds + 64 * lds_, ldh}, gs = {lds + 64 * lds_ + 64 * ldh, ldh};
+    stage(ps, p + pair * d.T * d.S, d.T, d.S, d.S);
+    stage(vs, v + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
+    stage(gs, dout + (b * d.T * d.N + n) * d.H, d.T, d.H, ld);
+    __syncthreads();
+    if (dp) {
+        const floatx16 acc = tile_mma<false, true>(gs, vs, (d.H + 1) & ~1, rb, cb, lane);
+        store_block(acc, dp + pair * d.T * d.S, d.T, d.S, d.S, rb, cb, lane);
+    }
+    if (dv && cb * 32 < d.H) {
+        const floatx16 acc = tile_mma<true, false>(ps, gs, (d.T + 1) & ~1, rb, cb, lane);
+        store_block(acc, dv + (b * d.S * d.N + n) * d.H, d.S, d.H, ld, rb, cb, lane);
     }
 }
 
@@ -123,38 +139,35 @@ __global__ __launch_bounds__(256) void attn_combine_bwd_kernel(const float *__re
 __global__ __launch_bounds__(256) void attn_scores_bwd_kernel(const float *__restrict__ ds, const float *__restrict__ q,
                                                               const float *__restrict__ k, float *__restrict__ dq,
                                                               float *__restrict__ dk, AttnDims d) {
-    __shared__ AtTile ss, qs, ks;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, rb = wave & 1, cb = wave >> 1;
-    const int64_t ld = (int64_t)d.N * d.H;
-    for (int64_t pair = blockIdx.x; pair < (int64_t)d.B * d.N; pair += gridDim.x) {
-        const int64_t b = pair / d.N, n = pair % d.N;
-        __syncthreads();
-        stage(ss, ds + pair * d.T * d.S, d.T, d.S, d.S);
-        stage(qs, q + (b * d.T * d.N + n) * d.H, d.T, d.H, ld);
-        stage(ks, k + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
-        __syncthreads();
-        if (cb * 32 < d.H) {
-            if (dq) {
-                const floatx16 acc = tile_mma<false, false>(ss, ks, (d.S + 1) & ~1, rb, cb, lane);
-                store_block(acc, dq + (b * d.T * d.N + n) * d.H, d.T, d.H, ld, rb, cb, lane);
-            }
-            if (dk) {
-                const floatx16 acc = tile_mma<true, false>(ss, qs, (d.T + 1) & ~1, rb, cb, lane);
-                store_block(acc, dk + (b * d.S * d.N + n) * d.H, d.S, d.H, ld, rb, cb, lane);
-            }
+    AT_PROLOGUE;
+    const Tile ss = {lds, lds_}, qs = {lds + 64 * lds_, ldh}, ks = {lds + 64 * lds_ + 64 * ldh, ldh};
+    stage(ss, ds + pair * d.T * d.S, d.T, d.S, d.S);
+    stage(qs, q + (b * d.T * d.N + n) * d.H, d.T, d.H, ld);
+    stage(ks, k + (b * d.S * d.N + n) * d.H, d.S, d.H, ld);
+    __syncthreads();
+    if (cb * 32 < d.H) {
+        if (dq) {
+            const floatx16 acc = tile_mma<false, false>(ss, ks, (d.S + 1) & ~1, rb, cb, lane);
+            store_block(acc, dq + (b * d.T * d.N + n) * d.H, d.T, d.H, ld, rb, cb, lane);
+        }
+        if (dk) {
+            const floatx16 acc = tile_mma<true, false>(ss, qs, (d.T + 1) & ~1, rb, cb, lane);
+            store_block(acc, dk + (b * d.S * d.N + n) * d.H, d.S, d.H, ld, rb, cb, lane);
         }
     }
 }
 
 static int check_dims(int B, int T, int S, int N, int H, const char *who, AttnDims &d) {
     if (B < 0 || T < 1 || S < 1 || N < 1 || H < 1) return fail(HGQ_ERR_ARG, "%s: bad sizes", who);
+    if ((int64_t)B * N >= (1ll << 31)) return fail(HGQ_ERR_UNSUPPORTED, "%s: too many (batch, head) pairs", who);
     if (T > 64 || S > 64 || H > 64)
         return fail(HGQ_ERR_UNSUPPORTED, "%s: sequence lengths and head size up to 64 are supported (T=%d S=%d H=%d)", who, T, S, H);
     d.B = B, d.T = T, d.S = S, d.N = N, d.H = H;
     return HGQ_OK;
 }
 
-static unsigned pair_grid(const AttnDims &d) { return (unsigned)persistent_grid((int64_t)d.B * d.N, 16); }
+static unsigned pair_grid(const AttnDims &d) { return (unsigned)((int64_t)d.B * d.N); }
+static size_t lds_bytes(int n_h, int n_s, const AttnDims &d) { return (size_t)64 * (n_h * tile_ld(d.H) + n_s * tile_ld(d.S)) * sizeof(float); }
 
 }  // namespace hgq
 
@@ -167,7 +180,7 @@ extern "C" int hgq_attn_scores_fwd(const float *query, const float *key, float *
     if (rc) return rc;
     if (B == 0) return HGQ_OK;
     if (!query || !key || !scores) return fail(HGQ_ERR_ARG, "hgq_attn_scores_fwd: null pointer");
-    hipLaunchKernelGGL(attn_scores_fwd_kernel, dim3(pair_grid(d)), dim3(256), 0, (hipStream_t)stream, query, key, scores, d);
+    hipLaunchKernelGGL(attn_scores_fwd_kernel, dim3(pair_grid(d)), dim3(256), lds_bytes(2, 0, d), (hipStream_t)stream, query, key, scores, d);
     return check_launch("hgq_attn_scores_fwd");
 }
 
@@ -178,7 +191,7 @@ extern "C" int hgq_attn_scores_bwd(const float *dscores, const float *query, con
     if (rc) return rc;
     if (B == 0) return HGQ_OK;
     if (!dscores || !query || !key) return fail(HGQ_ERR_ARG, "hgq_attn_scores_bwd: null pointer");
-    hipLaunchKernelGGL(attn_scores_bwd_kernel, dim3(pair_grid(d)), dim3(256), 0, (hipStream_t)stream, dscores, query, key, dquery, dkey, d);
+    hipLaunchKernelGGL(attn_scores_bwd_kernel, dim3(pair_grid(d)), dim3(256), lds_bytes(2, 1, d), (hipStream_t)stream, dscores, query, key, dquery, dkey, d);
     return check_launch("hgq_attn_scores_bwd");
 }
 
@@ -189,7 +202,7 @@ extern "C" int hgq_attn_combine_fwd(const float *probs, const float *value, floa
     if (rc) return rc;
     if (B == 0) return HGQ_OK;
     if (!probs || !value || !out) return fail(HGQ_ERR_ARG, "hgq_attn_combine_fwd: null pointer");
-    hipLaunchKernelGGL(attn_combine_fwd_kernel, dim3(pair_grid(d)), dim3(256), 0, (hipStream_t)stream, probs, value, out, d);
+    hipLaunchKernelGGL(attn_combine_fwd_kernel, dim3(pair_grid(d)), dim3(256), lds_bytes(1, 1, d), (hipStream_t)stream, probs, value, out, d);
     return check_launch("hgq_attn_combine_fwd");
 }
 
@@ -200,6 +213,6 @@ extern "C" int hgq_attn_combine_bwd(const float *dout, const float *probs, const
     if (rc) return rc;
     if (B == 0) return HGQ_OK;
     if (!dout || !probs || !value) return fail(HGQ_ERR_ARG, "hgq_attn_combine_bwd: null pointer");
-    hipLaunchKernelGGL(attn_combine_bwd_kernel, dim3(pair_grid(d)), dim3(256), 0, (hipStream_t)stream, dout, probs, value, dprobs, dvalue, d);
+    hipLaunchKernelGGL(attn_combine_bwd_kernel, dim3(pair_grid(d)), dim3(256), lds_bytes(2, 1, d), (hipStream_t)stream, dout, probs, value, dprobs, dvalue, d);
     return check_launch("hgq_attn_combine_bwd");
 }
