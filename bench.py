@@ -166,13 +166,13 @@ def softmax_roofline(iters=50, shape=(2048, 4, 64, 64), scaler=0.25):
 
 
 def config_step_time(name, steps=20, warmup=5, graph=False):
-    """One forward + backward pass of the configurations other than the headline one, at their full
+    """One training step (forward, backward, SGD update) of the configurations other than the headline one, at their full
     sizes: 'particle' (QEinsumDenseBatchnorm per-particle network, batch 4096 x 64 x 16), 'conv'
     (QConv2D stack on 28 x 28 x 1, batch 1024), 'mha' (QMultiHeadAttention, batch 2048 x 64 x 64)."""
     import torch
 
     from hgq2_amd import ops
-    from hgq2_amd.train import model_loss
+    from hgq2_amd.train import SGD, model_loss
     from hgq2_amd.utils import models
 
     dev = torch.device('cuda:0')
@@ -198,12 +198,17 @@ def config_step_time(name, steps=20, warmup=5, graph=False):
     else:
         raise ValueError(name)
 
+    model(x, training=True)  # build
+    opt = SGD(model.parameters(), lr=1e-3, fold_regularizers=True)
+
     def step():
-        for p in model.parameters():
-            p.grad = None
-        loss = model_loss(model, loss_fn(model(x, training=True)))
+        # forward, loss (+ EBOPs terms), backward, SGD update with the MonoL1 gradient and the
+        # bit-width constraints folded into the update kernel
+        opt.zero_grad()
+        loss = model_loss(model, loss_fn(model(x, training=True)), True)
         loss.backward()
-        return loss
+        opt.step()
+        return loss.detach()
 
     run = step
     if graph:
