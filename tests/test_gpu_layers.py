@@ -171,3 +171,41 @@ def test_fused_qdense_stack_step_matches_oracle(dev, batch, dims):
             _close(pl.kq.quantizer._i, rl.kq.quantizer._i, scale=rl.kq.quantizer._i.detach().abs() + 1e-3, what=f'kq._i {n}')
             _close(pl.bq.quantizer._b, rl.bq.quantizer._b, scale=rl.bq.quantizer._b.detach().abs() + 1e-3, what=f'bq._b {n}')
             _close(pl.bq.quantizer._i, rl.bq.quantizer._i, scale=rl.bq.quantizer._i.detach().abs() + 1e-3, what=f'bq._i {n}')
+
+
+def test_trace_minmax_matches_oracle(dev):
+    """The calibration pass (training='tracing') leaves the same integer bits, keep-negative flags
+    and EBOPs as the oracle, and inference after it is bit-identical."""
+    from hgq2_amd.utils import trace_minmax
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(8)
+    data = torch.randn(3000, 16, generator=g) * 1.5
+    oracle = ref.RefMLP(seed=2)
+    model = qdense_mlp(device=dev)
+    _copy_mlp(oracle, model, dev)
+    total = trace_minmax(model, data.numpy(), batch_size=1024)
+    for rl in oracle.layers:  # reset, then three calibration batches
+        q = rl.iq.quantizer
+        with torch.no_grad():
+            q._i.fill_(-1e9)
+            q._k.zero_()
+    from hgq2_amd.core import TrainingFlagWrapper
+
+    for s in range(0, 3000, 1024):  # the flag object is falsy and compares equal to 'tracing', as in the reference
+        oracle.forward(data[s:s + 1024], training=TrainingFlagWrapper('tracing'))
+    for rl, pl in zip(oracle.layers, model.layers):
+        assert torch.equal(pl.iq.quantizer._i.cpu(), rl.iq.quantizer._i.detach())
+        assert torch.equal(pl.iq.quantizer._k.cpu(), rl.iq.quantizer._k)
+        assert int(pl.ebops.cpu().view(torch.int32)) == int(rl.ebops_value)
+    assert total == sum(int(rl.ebops_value) for rl in oracle.layers)
+    with torch.no_grad():
+        got = model(data[:512].to(dev), training=False)
+        want = oracle.forward(data[:512], training=False)
+    _close(got, want, scale=want.abs() + 1.0, rtol=2e-5, what='logits after calibration')
+    # continuing without a reset only ever widens
+    before = [pl.iq.quantizer._i.clone() for pl in model.layers]
+    out = trace_minmax(model, (data[:100] * 4).numpy(), reset=False, return_results=True)
+    assert out.shape == (100, 5)
+    for b, pl in zip(before, model.layers):
+        assert torch.all(pl.iq.quantizer._i >= b)
