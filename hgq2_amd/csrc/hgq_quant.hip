@@ -114,12 +114,14 @@ __global__ __launch_bounds__(Q1D_BS) void quant_fwd_1d(const float *__restrict__
     KIF ps;
     if (SHARED) ps = resolve_kif(load_k(k, 0, m.k_u8), i[0], fb[0], m.kbi, m.round_params);
     uint32_t lmax = 0, lneg = 0;
+    const bool need_k = !(OM == HGQ_WRAP && m.training), need_i = need_k || m.kbi;
     for (int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * Q1D_BS) {
-        float xv[VEC], kv[VEC], iv[VEC], fv[VEC], yv[VEC];
+        float xv[VEC], kv[VEC] = {0.f}, iv[VEC] = {0.f}, fv[VEC], yv[VEC];
         VecIO<VEC>::load(x, v, xv);
         if (!SHARED) {
-            VecIO<VEC>::load_k(k, v, m.k_u8, kv);
-            VecIO<VEC>::load(i, v, iv);
+            // a WRAP quantizer in training mode only rounds: k (and i, unless f = b - i) are dead operands
+            if (need_k) VecIO<VEC>::load_k(k, v, m.k_u8, kv);
+            if (need_i) VecIO<VEC>::load(i, v, iv);
             VecIO<VEC>::load(fb, v, fv);
         }
         uint32_t ab[VEC], ng[VEC];
@@ -163,13 +165,14 @@ __global__ __launch_bounds__(Q1D_BS) void quant_bwd_1d(const float *__restrict__
     KIF ps;
     if (SHARED) ps = resolve_kif(load_k(k, 0, m.k_u8), i[0], fb[0], m.kbi, m.round_params);
     float si = 0.0f, sf = 0.0f;
+    const bool need_k = OM != HGQ_WRAP, need_i = need_k || m.kbi;  // the WRAP surrogate gradient only rounds
     for (int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * Q1D_BS) {
-        float gv[VEC], xv[VEC], kv[VEC], iv[VEC], fv[VEC], dxv[VEC], div[VEC], dfv[VEC];
+        float gv[VEC], xv[VEC], kv[VEC] = {0.f}, iv[VEC] = {0.f}, fv[VEC], dxv[VEC], div[VEC], dfv[VEC];
         VecIO<VEC>::load(dy, v, gv);
         VecIO<VEC>::load(x, v, xv);
         if (!SHARED) {
-            VecIO<VEC>::load_k(k, v, m.k_u8, kv);
-            VecIO<VEC>::load(i, v, iv);
+            if (need_k) VecIO<VEC>::load_k(k, v, m.k_u8, kv);
+            if (need_i) VecIO<VEC>::load(i, v, iv);
             VecIO<VEC>::load(fb, v, fv);
         }
 #pragma unroll

@@ -76,11 +76,12 @@ def _(x, k, i, fb, mode, bw_inner, track):
 
 
 @torch.library.custom_op('hgq::quantize_bwd', mutates_args=())
-def quantize_bwd(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int) -> tuple[Tensor, Tensor, Tensor]:
+def quantize_bwd(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, need_dx: bool,
+                 need_di: bool) -> tuple[Tensor, Tensor, Tensor]:
     _check_f32('dy', dy), _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
     _need(dy.numel() == x.numel(), 'dy and x differ in size')
-    dx = torch.empty_like(x)
-    di = torch.empty_like(i)
+    dx = torch.empty_like(x) if need_dx else x.new_empty(0)
+    di = torch.empty_like(i) if need_di else i.new_empty(0)
     dfb = torch.empty_like(fb)
     rc = _lib.load().hgq_quantize_bwd(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), _ptr(di), _ptr(dfb),
                                       x.numel(), i.numel(), bw_inner, _kmode(mode, k), _stream())
@@ -89,8 +90,9 @@ def quantize_bwd(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: 
 
 
 @quantize_bwd.register_fake
-def _(dy, x, k, i, fb, mode, bw_inner):
-    return torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+def _(dy, x, k, i, fb, mode, bw_inner, need_dx, need_di):
+    return (torch.empty_like(x) if need_dx else x.new_empty(0), torch.empty_like(i) if need_di else i.new_empty(0),
+            torch.empty_like(fb))
 
 
 @torch.library.custom_op('hgq::wrap_track_i', mutates_args=('i_var', 'k_var'))
@@ -522,7 +524,17 @@ class _Quantize(torch.autograd.Function):
         if not (ctx.mode & _lib.MODE_TRAINING):
             raise RuntimeError('hgq quantizer: gradients are defined for the training-mode forward only')
         x, k, i, fb = ctx.saved_tensors
-        dx, di, dfb = quantize_bwd(gy.contiguous(), x, k, i, fb, ctx.mode, ctx.bw_inner)
+        gy = gy.contiguous()
+        # a WRAP quantizer in training mode only rounds: the gradient passes straight through to x
+        # and (unless f = b - i) none reaches the integer bits, so the kernel writes neither
+        wrap = ((ctx.mode >> 4) & 0xf) == _lib.WRAP
+        need_dx = ctx.needs_input_grad[0] and not wrap
+        need_di = ctx.needs_input_grad[2] and (not wrap or bool(ctx.mode & _lib.MODE_KBI))
+        dx, di, dfb = quantize_bwd(gy, x, k, i, fb, ctx.mode, ctx.bw_inner, need_dx, need_di)
+        if ctx.needs_input_grad[0] and wrap:
+            dx = gy
+        if ctx.needs_input_grad[2] and not need_di:
+            di = torch.zeros_like(i)
         return (dx if ctx.needs_input_grad[0] else None, None, di if ctx.needs_input_grad[2] else None,
                 dfb if ctx.needs_input_grad[3] else None, None, None, None)
 
