@@ -128,3 +128,45 @@ def test_constraints_and_regularizers():
     assert Min(0)(w).tolist() == [0.0, 0.5, 30.0] and Max(1)(w).tolist() == [-30.0, 0.5, 1.0]
     assert Constant(2)(w).tolist() == [2.0, 2.0, 2.0]
     assert float(MonoL1(1e-2)(w)) == pytest.approx(0.005)
+
+
+def test_entry_points_validate_arguments_before_any_launch():
+    """Bad shapes and null pointers are rejected with the documented codes by host-side checks
+    (these calls return before the GPU is touched, so they run anywhere)."""
+    from hgq2_amd import _lib
+
+    lib = _lib.load()
+    OK, ARG, UNSUPPORTED = 0, -1, -3
+    none = ctypes.c_void_p(0)
+    # fixed-point quantizer
+    assert lib.hgq_quantize_fwd(none, none, none, none, none, none, none, 0, 1, 1, 1, none) == OK   # empty tensor
+    assert lib.hgq_quantize_fwd(none, none, none, none, none, none, none, 16, 1, 1, 1, none) == ARG  # null pointers
+    assert lib.hgq_quantize_fwd(none, none, none, none, none, none, none, 10, 4, 1, 1, none) == ARG  # 10 % 4 != 0
+    assert b'null' in lib.hgq_last_error() or b'multiple' in lib.hgq_last_error()
+    # table softmax: row length, table rows
+    assert lib.hgq_qsoftmax_bwd_workspace(1024, 64, 256, 1) > 0
+    assert lib.hgq_qsoftmax_bwd_workspace(1024, 300, 1, 0) == -1          # rows longer than 256
+    assert lib.hgq_qsoftmax_bwd_workspace(1024, 70, 1, 0) == -1           # > 64 and not a multiple of 4
+    assert lib.hgq_qsoftmax_bwd_workspace(1000, 64, 256, 1) == -1         # rows not a multiple of the table rows
+    assert lib.hgq_qsoftmax_fwd(none, none, 1024, 300, 1, 1.0, 1e-7, none, none, none, none, none, none, none, none, none) == UNSUPPORTED
+    assert lib.hgq_qsoftmax_fwd(none, none, 1024, 64, 1, 1.0, 1e-7, none, none, none, none, none, none, none, none, none) == ARG
+    assert lib.hgq_qsoftmax_fwd(none, none, 0, 64, 1, 1.0, 1e-7, none, none, none, none, none, none, none, none, none) == OK
+    # convolution geometry
+    good = _lib.ConvGeom(4, 8, 8, 3, 3, 3, 1, 1, 0, 0, 1, 1, 6, 6)
+    bad = _lib.ConvGeom(4, 8, 8, 3, 3, 3, 0, 1, 0, 0, 1, 1, 6, 6)  # stride 0
+    assert lib.hgq_conv2d_bwd_workspace(ctypes.addressof(good), 16) > 0
+    assert lib.hgq_conv2d_fwd_workspace(ctypes.addressof(good), 16) == 0
+    assert lib.hgq_conv2d_bwd_workspace(ctypes.addressof(bad), 16) == -1
+    assert lib.hgq_conv2d_fwd(none, none, none, none, none, ctypes.addressof(bad), 16, 0, none) == ARG
+    assert lib.hgq_conv2d_fwd(none, none, none, none, none, ctypes.addressof(good), 16, 7, none) == ARG  # unknown activation
+    assert lib.hgq_conv2d_fwd(none, none, none, none, none, ctypes.addressof(good), 16, 0, none) == ARG  # null pointers
+    wide = _lib.ConvGeom(8, 1, 1, 4096, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1)
+    assert lib.hgq_conv2d_fwd_workspace(ctypes.addressof(wide), 10) > 0   # long contraction, few rows: split along k
+    # attention contractions
+    assert lib.hgq_attn_scores_fwd(none, none, none, 4, 65, 64, 2, 16, none) == UNSUPPORTED
+    assert lib.hgq_attn_scores_fwd(none, none, none, 4, 64, 64, 2, 16, none) == ARG
+    assert lib.hgq_attn_combine_bwd(none, none, none, none, none, 0, 64, 64, 2, 16, none) == OK
+    # dense
+    assert lib.hgq_qdense_bwd(none, none, none, none, 0, none, none, none, none, none, none, 128, 80, 10, 0, 0, none) == UNSUPPORTED
+    assert lib.hgq_col_moments_workspace(1000, 64) > 0 and lib.hgq_col_moments_workspace(-1, 64) == -1
+    assert lib.hgq_col_moments_fwd(none, 0, 64, none, none, none, none) == ARG
