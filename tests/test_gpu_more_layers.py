@@ -295,3 +295,83 @@ def test_graph_replay_equals_eager_steps(dev, kind):
                 assert torch.allclose(pg, pe, rtol=2e-4, atol=2e-6), f'{kind}: {name}'
             else:
                 assert torch.equal(pg, pe), f'{kind}: {name}'
+
+
+@pytest.mark.parametrize('kind', ['particle', 'conv', 'mha'])
+def test_full_size_forward_matches_oracle(dev, kind):
+    """The per-particle, image and attention configurations at their full sizes: one training-mode
+    forward (quantized values, tracked integer bits, EBOPs) against the CPU oracle twins."""
+    from hgq2_amd.utils import models
+
+    g = torch.Generator().manual_seed(31)
+    torch.manual_seed(31)
+    if kind == 'particle':
+        x = torch.randn(4096, 64, 16, generator=g)
+        model = models.particle_mlp(device=dev)
+    elif kind == 'conv':
+        x = torch.rand(1024, 28, 28, 1, generator=g)
+        model = models.conv_stack(device=dev)
+    else:
+        x = torch.randn(2048, 64, 64, generator=g)
+        model = models.mha_block(device=dev)
+    with torch.no_grad():
+        model(x.to(dev), training=True)  # build, adapt the tracked bits
+    _perturb(model, g)
+    if kind == 'mha':
+        r = twin.ref_mha(model, tuple(x.shape))
+        with torch.no_grad():
+            got = model(x.to(dev), training=True)
+            want = r(x, training=True)
+        _close(got, want, rtol=2e-5, what='attention output')
+        assert int(model._ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+        assert torch.equal(model._softmax.oq.quantizer._i.cpu(), r.softmax.oq.quantizer._i.detach())
+        assert torch.equal(model._value_dense.iq.quantizer._i.cpu(), r.vd.iq.quantizer._i.detach())
+        return
+    # sequential models: walk the layers, twin each quantized one, pass the oracle's activations along
+    h_p, h_r = x.to(dev), x
+    with torch.no_grad():
+        for layer in model.layers:
+            if isinstance(layer, models.Lambda):
+                h_p, h_r = layer(h_p), layer.fn(h_r)
+                continue
+            if kind == 'conv' and layer.__class__.__name__ == 'QConv2D':
+                r = twin.ref_conv2d(layer)
+            elif layer.__class__.__name__ == 'QEinsumDenseBatchnorm':
+                r = twin.ref_einsum_dense_bn(layer, tuple(h_r.shape))
+            else:
+                r = twin.ref_dense(layer)
+            h_p, h_r = layer(h_p, training=True), r(h_r, training=True)
+            _close(h_p, h_r, rtol=5e-5, what=f'{kind}: output of {layer.name}')
+            assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach()), layer.name
+            assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value), layer.name
+            h_p = h_r.to(dev)  # continue from the oracle's activations so that layers are compared one by one
+
+
+def test_full_size_attention_step_matches_oracle(dev):
+    """QMultiHeadAttention at the full attention configuration (2048 x 64 x 64, 4 heads of 16): output,
+    loss terms and the gradients of inputs, kernels and bit-widths against the oracle twin."""
+    from hgq2_amd.utils import models
+
+    g = torch.Generator().manual_seed(41)
+    torch.manual_seed(41)
+    x = torch.randn(2048, 64, 64, generator=g)
+    layer = models.mha_block(device=dev)
+    with torch.no_grad():
+        layer(x.to(dev), training=True)
+    _perturb(layer, g)
+    r = twin.ref_mha(layer, tuple(x.shape))
+    xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
+    sm, rs = layer._softmax, r.softmax
+    named_p = [('x', xp), ('wq', layer._query_dense._kernel), ('wk', layer._key_dense._kernel),
+               ('wv', layer._value_dense._kernel), ('wo', layer._output_dense._kernel),
+               ('q_oq_f', layer._query_dense.oq.quantizer._f), ('sm_oq_f', sm.oq.quantizer._f),
+               ('v_iq_f', layer._value_dense.iq.quantizer._f), ('exp_iq_f', sm.exp_table.iq.quantizer._f),
+               ('exp_oq_b', sm.exp_table.oq.quantizer._b), ('inv_iq_f', sm.inv_table.iq.quantizer._f),
+               ('inv_oq_b', sm.inv_table.oq.quantizer._b)]
+    named_r = [('x', xr), ('wq', r.qd.kernel), ('wk', r.kd.kernel), ('wv', r.vd.kernel), ('wo', r.od.kernel),
+               ('q_oq_f', r.qd.oq.quantizer._f), ('sm_oq_f', rs.oq.quantizer._f), ('v_iq_f', r.vd.iq.quantizer._f),
+               ('exp_iq_f', rs.exp_table.iq.quantizer._f), ('exp_oq_b', rs.exp_table.oq.quantizer._b),
+               ('inv_iq_f', rs.inv_table.iq.quantizer._f), ('inv_oq_b', rs.inv_table.oq.quantizer._b)]
+    # sums over up to 33.5 M terms: fp32 accumulation order differs between the kernels and the CPU
+    _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=5e-4)
+    assert int(layer._ebops.cpu().view(torch.int32)) == int(r.ebops_value)
