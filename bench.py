@@ -169,7 +169,7 @@ def softmax_roofline(iters=50, shape=(2048, 4, 64, 64), scaler=0.25):
     return out
 
 
-def config_step_time(name, steps=20, warmup=5, graph=False):
+def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False):
     """One training step (forward, backward, SGD update) of the configurations other than the headline one, at their full
     sizes: 'particle' (QEinsumDenseBatchnorm per-particle network, batch 4096 x 64 x 16), 'conv'
     (QConv2D stack on 28 x 28 x 1, batch 1024), 'mha' (QMultiHeadAttention, batch 2048 x 64 x 64)."""
@@ -198,6 +198,7 @@ def config_step_time(name, steps=20, warmup=5, graph=False):
         batch = 2048
         x = torch.randn(batch, 64, 64, generator=g).to(dev)
         model = models.mha_block(device=dev)
+        labels = None
         loss_fn = lambda out: (out * out).mean()  # noqa: E731
     else:
         raise ValueError(name)
@@ -242,8 +243,68 @@ def config_step_time(name, steps=20, warmup=5, graph=False):
         loss = run()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / steps * 1e3
-    return {'workload': name, 'batch': batch, 'ms_per_step': ms, 'samples_per_s': batch / ms * 1e3, 'loss': float(loss),
-            'launch': 'hip-graph replay' if graph else 'eager'}
+    out = {'workload': name, 'batch': batch, 'ms_per_step': ms, 'samples_per_s': batch / ms * 1e3, 'loss': float(loss),
+           'launch': 'hip-graph replay' if graph else 'eager'}
+    if cpu:
+        out['cpu_baseline'] = _config_cpu_baseline(name, model, x, labels if name != 'mha' else None, batch)
+        out['gpu_over_cpu'] = out['samples_per_s'] / out['cpu_baseline']['value']
+    return out
+
+
+def _config_cpu_baseline(name, model, x, labels, batch, budget_s=15.0):
+    """The oracle's eager torch-CPU restatement of the same model (same weights and bit-widths) timed
+    on the host cores: forward, loss, backward (no optimizer), a bounded number of steps."""
+    import torch
+    import torch.nn.functional as F
+
+    from hgq2_amd.utils import models
+    from tests import twin
+
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    xc = x.cpu()
+    if name == 'mha':
+        r = twin.ref_mha(model, tuple(xc.shape))
+
+        def step():
+            out = r(xc, training=True)
+            ((out * out).mean() + r.extra_loss()).backward()
+    else:
+        twins = []
+        shape = tuple(xc.shape)
+        for layer in model.layers:
+            if isinstance(layer, models.Lambda):
+                twins.append(layer.fn)
+                shape = tuple(layer.fn(torch.zeros(shape)).shape)
+                continue
+            kind = layer.__class__.__name__
+            r = twin.ref_conv2d(layer) if kind == 'QConv2D' else (
+                twin.ref_einsum_dense_bn(layer, shape) if kind == 'QEinsumDenseBatchnorm' else twin.ref_dense(layer))
+            twins.append(r)
+            shape = (shape[0],) + tuple(layer.compute_output_shape(shape)[1:])
+        yc = labels.cpu()
+
+        def step():
+            h = xc
+            extra = 0.0
+            for t in twins:
+                if callable(t) and not hasattr(t, 'extra_loss'):
+                    h = t(h)
+                else:
+                    h = t(h, training=True)
+                    extra = extra + t.extra_loss()
+            (F.cross_entropy(h, yc) + extra).backward()
+
+    step()
+    n, t0 = 0, time.perf_counter()
+    while True:
+        step()
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 20:
+            break
+    return {'value': batch * n / el, 'unit': 'samples/s', 'cores': cores, 'kind': 'port',
+            'sample': f'{n} forward+backward passes of the same model at batch {batch} (eager torch-CPU restatement of the reference path)'}
 
 
 def cpu_baseline(budget_s=20.0):
@@ -282,6 +343,7 @@ def main():
                     help='run only the standalone quantizer kernels and a plain copy of known size (for counter runs)')
     ap.add_argument('--config-step', choices=('particle', 'conv', 'mha'), default=None,
                     help='time one forward + backward pass of another configuration at full size instead of the headline run')
+    ap.add_argument('--config-cpu', action='store_true', help='with --config-step: also time the CPU oracle of the same model')
     ap.add_argument('--graph', action='store_true', help='with --config-step: capture the step in a HIP graph and replay it')
     ap.add_argument('--softmax-only', action='store_true',
                     help='run only the one-pass table-softmax kernels at the attention configuration (for profiler runs)')
@@ -301,7 +363,7 @@ def main():
         return
     if args.config_step:
         torch.cuda.set_device(0)
-        print(json.dumps({'config_step': config_step_time(args.config_step, steps=args.steps if args.steps != 300 else 20, graph=args.graph)}))
+        print(json.dumps({'config_step': config_step_time(args.config_step, steps=args.steps if args.steps != 300 else 20, graph=args.graph, cpu=args.config_cpu)}))
         return
     if args.softmax_only:
         torch.cuda.set_device(0)
