@@ -274,8 +274,8 @@ def _config_cpu_baseline(name, model, x, labels, batch, budget_s=15.0):
         shape = tuple(xc.shape)
         for layer in model.layers:
             if isinstance(layer, models.Lambda):
-                twins.append(layer.fn)
-                shape = tuple(layer.fn(torch.zeros(shape)).shape)
+                twins.append(layer.host_fn)
+                shape = tuple(layer.host_fn(torch.zeros(shape)).shape)
                 continue
             kind = layer.__class__.__name__
             r = twin.ref_conv2d(layer) if kind == 'QConv2D' else (

@@ -60,6 +60,8 @@ SIGNATURES = {
     'hgq_attn_scores_bwd': (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_void_p]),
     'hgq_attn_combine_fwd': (c_int, [c_void_p] * 3 + [c_int] * 5 + [c_void_p]),
     'hgq_attn_combine_bwd': (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_void_p]),
+    'hgq_pool2d_fwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    'hgq_pool2d_bwd': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     'hgq_col_moments_workspace': (c_int64, [c_int64, c_int]),
     'hgq_col_moments_fwd': (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_col_moments_bwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p]),

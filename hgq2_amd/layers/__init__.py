@@ -4,7 +4,10 @@ from .attn import QMultiHeadAttention
 from .conv import QConv2D
 from .core import QDense, QEinsumDense, QLayerBase, QLayerBaseMultiInputs, QLayerBaseSingleInput
 from .einsum_dense_batchnorm import QEinsumDenseBatchnorm
+from .pooling import (QAveragePooling2D, QGlobalAveragePooling1D, QGlobalAveragePooling2D, QGlobalMaxPooling1D,
+                      QGlobalMaxPooling2D, QMaxPooling2D)
 from .softmax import QSoftmax
 
 __all__ = ['Quantizer', 'QDense', 'QEinsumDense', 'QEinsumDenseBatchnorm', 'QConv2D', 'QSoftmax', 'QUnaryFunctionLUT',
-           'QMultiHeadAttention', 'QLayerBase', 'QLayerBaseSingleInput', 'QLayerBaseMultiInputs']
+           'QMultiHeadAttention', 'QMaxPooling2D', 'QAveragePooling2D', 'QGlobalAveragePooling1D', 'QGlobalAveragePooling2D',
+           'QGlobalMaxPooling1D', 'QGlobalMaxPooling2D', 'QLayerBase', 'QLayerBaseSingleInput', 'QLayerBaseMultiInputs']

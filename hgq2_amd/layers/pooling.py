@@ -1,0 +1,114 @@
+"""Quantized pooling layers (reference src/hgq/layers/pooling.py:23-315): the input quantizer
+followed by the plain pooling; EBOPs ``sum(bits_in) * parallelization_factor / n_parallel``.
+The 2-D window poolings run in the channels-last pooling kernels (``hgq_pool2d_fwd / _bwd``); the
+global poolings are single reductions over the spatial axes."""
+
+from __future__ import annotations
+
+from math import prod
+
+import torch
+
+from .. import ops
+from ..quantizer import QuantizerConfig
+from .core.base import QLayerBaseSingleInput
+
+
+def _pair(v):
+    return (int(v), int(v)) if isinstance(v, int) else tuple(int(t) for t in v)
+
+
+class QBasePooling(QLayerBaseSingleInput):
+    def __init__(self, *args, parallelization_factor=-1, iq_conf: QuantizerConfig | None = None,
+                 oq_conf: QuantizerConfig | None = None, **kwargs):
+        self.parallelization_factor = parallelization_factor
+        super().__init__(*args, iq_conf=iq_conf, oq_conf=oq_conf, **kwargs)
+        self.data_format = 'channels_last'
+
+    def _compute_ebops(self, shape):
+        bw_inp = self.iq.bits_(shape)
+        return torch.sum(bw_inp) * self.parallelization_factor / self.n_parallel
+
+    def pool(self, inputs):
+        raise NotImplementedError
+
+    def call(self, inputs, training=None):
+        if self.enable_iq:
+            inputs = self.iq(inputs, training=training)
+        return self.pool(inputs)
+
+    def build(self, input_shape):
+        super().build(input_shape)
+        out_shape = self.compute_output_shape(input_shape)
+        self.n_parallel = None if None in out_shape[1:] else prod(out_shape[1:-1])
+        if self.parallelization_factor <= 0:
+            assert self.n_parallel is not None
+            self.parallelization_factor = self.n_parallel
+
+
+class _QWindowPooling2D(QBasePooling):
+    _mode = 'max'
+
+    def __init__(self, pool_size=(2, 2), strides=None, padding='valid', data_format=None, **kwargs):
+        if data_format not in (None, 'channels_last'):
+            raise NotImplementedError('pooling: channels_last only')
+        super().__init__(**kwargs)
+        self.pool_size = _pair(pool_size)
+        self.strides = _pair(strides) if strides is not None else self.pool_size
+        self.padding = padding.lower()
+        assert self.padding in ('valid', 'same')
+
+    def compute_output_shape(self, input_shape):
+        out = [input_shape[0]]
+        for n, p, s in zip(input_shape[1:3], self.pool_size, self.strides):
+            out.append(None if n is None else (-(-n // s) if self.padding == 'same' else (n - p) // s + 1))
+        return tuple(out) + (input_shape[3],)
+
+    def pool(self, inputs):
+        return ops.pool2d(inputs, self.pool_size, self.strides, self.padding, self._mode)
+
+
+class QMaxPooling2D(_QWindowPooling2D):
+    _mode = 'max'
+
+
+class QAveragePooling2D(_QWindowPooling2D):
+    _mode = 'avg'
+
+
+class _QGlobalPooling(QBasePooling):
+    _rank = 2
+    _mode = 'avg'
+
+    def __init__(self, data_format=None, keepdims=False, **kwargs):
+        if data_format not in (None, 'channels_last'):
+            raise NotImplementedError('pooling: channels_last only')
+        super().__init__(**kwargs)
+        self.keepdims = keepdims
+
+    def compute_output_shape(self, input_shape):
+        if self.keepdims:
+            return (input_shape[0],) + (1,) * self._rank + (input_shape[-1],)
+        return (input_shape[0], input_shape[-1])
+
+    def pool(self, inputs):
+        axes = tuple(range(1, 1 + self._rank))
+        if self._mode == 'avg':
+            return torch.mean(inputs, dim=axes, keepdim=self.keepdims)
+        return torch.amax(inputs, dim=axes, keepdim=self.keepdims)
+
+
+class QGlobalAveragePooling1D(_QGlobalPooling):
+    _rank, _mode = 1, 'avg'
+
+
+class QGlobalAveragePooling2D(_QGlobalPooling):
+    _rank, _mode = 2, 'avg'
+
+
+class QGlobalMaxPooling1D(_QGlobalPooling):
+    _rank, _mode = 1, 'max'
+
+
+class QGlobalMaxPooling2D(_QGlobalPooling):
+    _rank, _mode = 2, 'max'

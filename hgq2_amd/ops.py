@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d']
 
 
 def _ptr(t: Tensor | None):
@@ -504,6 +504,38 @@ def _(dout, probs, value):
     return torch.empty_like(probs), torch.empty_like(value)
 
 
+@torch.library.custom_op('hgq::pool2d_fwd', mutates_args=())
+def pool2d_fwd(x: Tensor, geom: Sequence[int], is_max: bool) -> Tensor:
+    _check_f32('x', x)
+    _need(len(geom) == 12 and x.numel() == geom[0] * geom[1] * geom[2] * geom[3], 'x must be [B, H, W, C] as in the geometry')
+    y = torch.empty((geom[0], geom[10], geom[11], geom[3]), dtype=torch.float32, device=x.device)
+    g = (ctypes.c_int * 12)(*[int(v) for v in geom])
+    rc = _lib.load().hgq_pool2d_fwd(_ptr(x), _ptr(y), g, int(is_max), _stream())
+    _lib.check(rc, 'hgq_pool2d_fwd')
+    return y
+
+
+@pool2d_fwd.register_fake
+def _(x, geom, is_max):
+    return x.new_empty((geom[0], geom[10], geom[11], geom[3]))
+
+
+@torch.library.custom_op('hgq::pool2d_bwd', mutates_args=())
+def pool2d_bwd(dy: Tensor, x: Tensor, geom: Sequence[int], is_max: bool) -> Tensor:
+    _check_f32('dy', dy), _check_f32('x', x)
+    _need(dy.numel() == geom[0] * geom[10] * geom[11] * geom[3], 'dy must be [B, OH, OW, C] as in the geometry')
+    dx = torch.empty_like(x)
+    g = (ctypes.c_int * 12)(*[int(v) for v in geom])
+    rc = _lib.load().hgq_pool2d_bwd(_ptr(dy), _ptr(x), _ptr(dx), g, int(is_max), _stream())
+    _lib.check(rc, 'hgq_pool2d_bwd')
+    return dx
+
+
+@pool2d_bwd.register_fake
+def _(dy, x, geom, is_max):
+    return torch.empty_like(x)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -779,6 +811,33 @@ def attn_scores(query: Tensor, key: Tensor) -> Tensor:
 def attn_combine(probs: Tensor, value: Tensor) -> Tensor:
     """``einsum('acbe,aecd->abcd', probs, value)``: probs [B, N, T, S], value [B, S, N, H] -> [B, T, N, H]."""
     return _AttnCombine.apply(probs.contiguous(), value.contiguous())
+
+
+class _Pool2D(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, geom, is_max):
+        ctx.save_for_backward(x)
+        ctx.geom, ctx.is_max = tuple(geom), is_max
+        return pool2d_fwd(x, list(geom), is_max)
+
+    @staticmethod
+    def backward(ctx, g):
+        (x,) = ctx.saved_tensors
+        return pool2d_bwd(g.contiguous(), x, list(ctx.geom), ctx.is_max), None, None
+
+
+def pool2d(x: Tensor, pool_size, strides=None, padding: str = 'valid', mode: str = 'max') -> Tensor:
+    """Max / average pooling of a channels-last [B, H, W, C] tensor; 'same' pads like Keras (odd pad after)."""
+    B, H, W, C = x.shape
+    ph, pw = pool_size
+    sy, sx = strides if strides is not None else pool_size
+    if padding == 'same':
+        OH, OW = -(-H // sy), -(-W // sx)
+        py, px = max((OH - 1) * sy + ph - H, 0) // 2, max((OW - 1) * sx + pw - W, 0) // 2
+    else:
+        OH, OW, py, px = (H - ph) // sy + 1, (W - pw) // sx + 1, 0, 0
+    _need(OH >= 1 and OW >= 1, 'the pooling window does not fit the input')
+    return _Pool2D.apply(x.contiguous(), (B, H, W, C, ph, pw, sy, sx, py, px, OH, OW), mode == 'max')
 
 
 class _SparseCE(torch.autograd.Function):

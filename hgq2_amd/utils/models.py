@@ -4,6 +4,7 @@ from __future__ import annotations
 
 from ..config import LayerConfigScope, QuantizerConfigScope
 from ..core import Sequential, set_default_device
+from .. import ops
 from ..core import Layer
 from ..layers import QConv2D, QDense, QEinsumDenseBatchnorm, QMultiHeadAttention
 
@@ -47,9 +48,10 @@ def qdense_mlp(dims=(16, 64, 32, 32, 5), beta0=1e-5, device=None, batch=None):
 class Lambda(Layer):
     """A parameter-free step between quantized layers (pooling, flatten, mean)."""
 
-    def __init__(self, fn, **kwargs):
+    def __init__(self, fn, host_fn=None, **kwargs):
         super().__init__(**kwargs)
         self.fn = fn
+        self.host_fn = host_fn or fn  # the same step on CPU tensors, for checking against the oracle
 
     def call(self, x, training=None):
         return self.fn(x)
@@ -77,16 +79,16 @@ def conv_stack(filters=32, n_out=10, beta0=1e-5, device=None):
     if device is not None:
         set_default_device(device)
 
-    def pool(t):  # NHWC max-pool 2x2, stride 2, 'valid'
-        b, h, w, c = t.shape
-        t = t[:, :h // 2 * 2, :w // 2 * 2, :].reshape(b, h // 2, 2, w // 2, 2, c)
-        return torch.amax(t, dim=(2, 4))
+    def pool(t):  # NHWC max-pool 2x2, stride 2, 'valid', in the pooling kernels
+        return ops.pool2d(t, (2, 2), (2, 2), 'valid', 'max')
+
+    def pool_host(t):
+        return F.max_pool2d(t.permute(0, 3, 1, 2), 2, 2).permute(0, 2, 3, 1)
 
     with _Scopes(beta0):
-        layers = [QConv2D(filters, (3, 3), activation='relu'), Lambda(pool, name='max_pool'),
+        layers = [QConv2D(filters, (3, 3), activation='relu'), Lambda(pool, pool_host, name='max_pool'),
                   QConv2D(filters, (3, 3), activation='relu'), Lambda(lambda t: t.reshape(t.shape[0], -1), name='flatten'),
                   QDense(n_out)]
-    del F
     return Sequential(layers)
 
 

@@ -349,6 +349,18 @@ int hgq_attn_combine_fwd(const float *probs, const float *value, float *out, int
 int hgq_attn_combine_bwd(const float *dout, const float *probs, const float *value, float *dprobs, float *dvalue, int B, int T,
                          int S, int N, int H, void *stream);
 
+/*
+ * 2-D max / average pooling on channels-last tensors, forward and backward.  Replaces the Keras
+ * MaxPooling2D / AveragePooling2D `call` that QMaxPooling2D / QAveragePooling2D apply to the
+ * quantized input (src/hgq/layers/pooling.py:23-47; the Keras torch backend transposes to
+ * channels-first around the library pooling) and its autograd.
+ *   geom = {B, H, W, C, pool_h, pool_w, stride_y, stride_x, pad_top, pad_left, OH, OW};
+ *   x, dx [B, H, W, C];  y, dy [B, OH, OW, C].  Max pooling sends the gradient to the first maximum
+ *   of a window in row-major order; average pooling divides by the number of in-range elements.
+ */
+int hgq_pool2d_fwd(const float *x, float *y, const int *geom, int is_max, void *stream);
+int hgq_pool2d_bwd(const float *dy, const float *x, float *dx, const int *geom, int is_max, void *stream);
+
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
 

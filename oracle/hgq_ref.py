@@ -753,6 +753,47 @@ class RefQConv2D(RefQLayer):
         return ebops
 
 
+class RefQPooling2D(RefQLayer):
+    """src/hgq/layers/pooling.py:23-47 on top of MaxPooling2D / AveragePooling2D (channels-last;
+    'same' pads like Keras: odd pad after, padding never wins a maximum and is not counted in a mean)."""
+
+    def __init__(self, mode, pool_size, strides, padding, iq, oq=None, beta0=1e-5, enable_ebops=True, parallelization_factor=-1,
+                 n_parallel=1):
+        self._init_common(beta0, enable_ebops and iq is not None)
+        self.mode, self.pool_size, self.strides, self.padding = mode, tuple(pool_size), tuple(strides), padding
+        self.iq, self.oq = iq, oq
+        self.n_parallel = n_parallel
+        self.parallelization_factor = parallelization_factor if parallelization_factor > 0 else n_parallel
+
+    def weights(self):
+        return []
+
+    def quantizers(self):
+        return [q for q in (self.iq, self.oq) if q is not None]
+
+    def call(self, x, training=None):
+        if self.iq is not None:
+            x = self.iq(x, training=training)
+        x = x.permute(0, 3, 1, 2)
+        pads = [0, 0, 0, 0]
+        if self.padding == 'same':
+            pads = []
+            for d in (1, 0):
+                n, k, st = x.shape[2 + d], self.pool_size[d], self.strides[d]
+                total = max((-(-n // st) - 1) * st + k - n, 0)
+                pads += [total // 2, total - total // 2]
+        if self.mode == 'max':
+            y = F.max_pool2d(F.pad(x, pads, value=float('-inf')), self.pool_size, self.strides)
+        else:
+            num = F.avg_pool2d(F.pad(x, pads), self.pool_size, self.strides, divisor_override=1)
+            cnt = F.avg_pool2d(F.pad(torch.ones_like(x[:1, :1]), pads), self.pool_size, self.strides, divisor_override=1)
+            y = num / cnt
+        return y.permute(0, 2, 3, 1)
+
+    def _compute_ebops(self, shape):
+        return torch.sum(self.iq.bits_(shape)) * self.parallelization_factor / self.n_parallel
+
+
 # --------------------------------------------------------------------------------------
 # the QDense-MLP training step (reference call stack: tests/base.py:302-321 and README.md:57-67)
 # --------------------------------------------------------------------------------------

@@ -104,3 +104,35 @@ def test_wide_dense_layer_matches_oracle(dev):
     _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=1e-4)
     assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
     assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+
+
+@pytest.mark.parametrize('mode', ['max', 'avg'])
+@pytest.mark.parametrize('case', [
+    # B, H, W, C, pool, strides, padding
+    (16, 26, 26, 32, (2, 2), None, 'valid'),     # the pooling of the image configuration
+    (5, 9, 11, 3, (3, 2), (2, 1), 'same'),       # overlapping windows, odd padding, scalar channel path
+    (4, 7, 7, 8, (3, 3), (3, 3), 'valid'),       # border pixels that no window covers
+    (3, 8, 6, 4, (2, 3), (1, 2), 'same'),
+])
+def test_pooling_layers_match_oracle(dev, mode, case):
+    """QMaxPooling2D / QAveragePooling2D: values, EBOPs, tracked bits and gradients (incl. where the
+    gradient of a tied maximum goes: quantized ReLU-like inputs tie often) against the oracle twin."""
+    from hgq2_amd.layers import QAveragePooling2D, QMaxPooling2D
+    from tests import twin
+    from tests.test_gpu_more_layers import _compare_step, _perturb, readme_scopes
+
+    B, H, W, C, pool, strides, padding = case
+    g = torch.Generator().manual_seed(B + H)
+    cls = QMaxPooling2D if mode == 'max' else QAveragePooling2D
+    with readme_scopes():
+        layer = cls(pool, strides=strides, padding=padding)
+    x = torch.relu(torch.randn(B, H, W, C, generator=g))  # many exact zeros after quantization: ties
+    layer(x.to(dev), training=True)
+    _perturb(layer, g)
+    r = twin.ref_pooling2d(layer)
+    xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
+    named_p = [('x', xp), ('iq_f', layer.iq.quantizer._f)]
+    named_r = [('x', xr), ('iq_f', r.iq.quantizer._f)]
+    _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=2e-5)
+    assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
+    assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)

@@ -332,7 +332,7 @@ def test_full_size_forward_matches_oracle(dev, kind):
     with torch.no_grad():
         for layer in model.layers:
             if isinstance(layer, models.Lambda):
-                h_p, h_r = layer(h_p), layer.fn(h_r)
+                h_p, h_r = layer(h_p), layer.host_fn(h_r)
                 continue
             if kind == 'conv' and layer.__class__.__name__ == 'QConv2D':
                 r = twin.ref_conv2d(layer)

@@ -130,3 +130,9 @@ def ref_conv2d(layer):
 
 def quantizer_pairs(ref_layer_quantizers, prod_quantizers):
     return list(zip(ref_layer_quantizers, prod_quantizers))
+
+
+def ref_pooling2d(layer):
+    return ref.RefQPooling2D(layer._mode, layer.pool_size, layer.strides, layer.padding, _iq(layer), oq=_oq(layer),
+                             beta0=_beta(layer), enable_ebops=layer.enable_ebops,
+                             parallelization_factor=layer.parallelization_factor, n_parallel=layer.n_parallel)
