@@ -65,6 +65,7 @@ SIGNATURES = {
     'hgq_col_moments_workspace': (c_int64, [c_int64, c_int]),
     'hgq_col_moments_fwd': (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_col_moments_bwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p]),
+    'hgq_conv2d_ebops': (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_conv2d_fwd_workspace': (c_int64, [c_void_p, c_int]),
     'hgq_conv2d_fwd': (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p]),
     'hgq_conv2d_bwd_workspace': (c_int64, [c_void_p, c_int]),

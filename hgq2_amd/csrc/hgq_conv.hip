@@ -457,6 +457,87 @@ static int fwd_ksplit(int64_t rows, int K, int F) {
     return s < 1 ? 1 : (int)s;
 }
 
+
+// EBOPs of a convolution: sum over all output pixels and filters of conv(bits_in, bits_ker), and
+// its gradient, without running the convolution:
+//     S[tap, c] = sum of bits_in over the input pixels that tap visits,   Wsum[tap, c] = sum_f bits_ker[tap, c, f]
+//     total = sum S * Wsum;   d total / d bits_ker[tap, c, f] = S[tap, c];
+//     d total / d bits_in[y, x, c] = sum over the taps that visit (y, x) of Wsum[tap, c]
+// One workgroup; every quantity is a sum of small integers, exact in fp32 in any order while below 2^24.
+#define CE_MAX 4096  // kh * kw * C
+__global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restrict__ bits_in, const float *__restrict__ bits_ker,
+                                                          hgq_conv_geom g, int F, float *total,
+                                                          float *__restrict__ g_in, float *__restrict__ g_ker) {
+    __shared__ float S[CE_MAX], Ws[CE_MAX];
+    __shared__ float red[1024];
+    const int t = threadIdx.x, taps = g.kh * g.kw, TC = taps * g.C;
+    for (int e = t; e < TC; e += 1024) S[e] = 0.f, Ws[e] = 0.f;
+    __syncthreads();
+    // S: flat sweep over (tap, output pixel, channel), channel fastest so reads coalesce
+    const int OP = g.OH * g.OW, n_s = taps * OP * g.C;
+    for (int e0 = 0; e0 < n_s; e0 += 4 * 1024) {
+        float v[4];
+        int dst[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e0 + u * 1024 + t;
+            v[u] = 0.f, dst[u] = -1;
+            if (e < n_s) {
+                const int c = e % g.C, r = e / g.C, op = r % OP, tap = r / OP;
+                const int oy = op / g.OW, ox = op - oy * g.OW, ky = tap / g.kw, kx = tap - ky * g.kw;
+                const int iy = oy * g.sy - g.py + ky * g.dly, ix = ox * g.sx - g.px + kx * g.dlx;
+                if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W)
+                    v[u] = bits_in[((int64_t)iy * g.W + ix) * g.C + c], dst[u] = tap * g.C + c;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (dst[u] >= 0) atomicAdd(&S[dst[u]], v[u]);
+    }
+    const int n_w = TC * F;
+    for (int e0 = 0; e0 < n_w; e0 += 4 * 1024) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e0 + u * 1024 + t;
+            v[u] = e < n_w ? bits_ker[e] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e0 + u * 1024 + t;
+            if (e < n_w) atomicAdd(&Ws[e / F], v[u]);
+        }
+    }
+    __syncthreads();
+    float part = 0.f;
+    for (int e = t; e < TC; e += 1024) part += S[e] * Ws[e];
+    red[t] = part;
+    __syncthreads();
+    for (int o = 512; o > 0; o >>= 1) {
+        if (t < o) red[t] += red[t + o];
+        __syncthreads();
+    }
+    if (t == 0) total[0] = red[0];
+    if (g_ker)
+        for (int e = t; e < n_w; e += 1024) g_ker[e] = S[e / F];
+    if (g_in) {
+        for (int e = t; e < g.H * g.W * g.C; e += 1024) {
+            const int c = e % g.C, pix = e / g.C, y = pix / g.W, x = pix - y * g.W;
+            float a = 0.f;
+            for (int ky = 0; ky < g.kh; ++ky) {
+                const int ty = y + g.py - ky * g.dly;
+                if (ty < 0 || ty % g.sy != 0 || ty / g.sy >= g.OH) continue;
+                for (int kx = 0; kx < g.kw; ++kx) {
+                    const int tx = x + g.px - kx * g.dlx;
+                    if (tx < 0 || tx % g.sx != 0 || tx / g.sx >= g.OW) continue;
+                    a += Ws[(ky * g.kw + kx) * g.C + c];
+                }
+            }
+            g_in[e] = a;
+        }
+    }
+}
+
 static int check_geom(const hgq_conv_geom *g, int F, const char *who) {
     if (!g) return fail(HGQ_ERR_ARG, "%s: null geometry", who);
     if (g->B < 0 || g->H < 1 || g->W < 1 || g->C < 1 || g->kh < 1 || g->kw < 1 || g->sy < 1 || g->sx < 1 || g->dly < 1 ||
@@ -597,4 +678,18 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
         if ((rc = reduce_parts(workspace, (int)splits, M, dqw, KF, dqb, (int64_t)F, nullptr, 0, s))) return rc;
     }
     return HGQ_OK;
+}
+
+extern "C" int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, const hgq_conv_geom *g, int F, float *total,
+                                float *g_bits_in, float *g_bits_ker, void *stream) {
+    int rc = check_geom(g, F, "hgq_conv2d_ebops");
+    if (rc) return rc;
+    if (!bits_in || !bits_ker || !total) return fail(HGQ_ERR_ARG, "hgq_conv2d_ebops: null pointer");
+    if ((int64_t)g->kh * g->kw * g->C > CE_MAX)
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: kh * kw * C = %lld exceeds %d", (long long)g->kh * g->kw * g->C, CE_MAX);
+    if ((int64_t)g->kh * g->kw * g->C * g->OH * g->OW >= (1ll << 31) || (int64_t)g->kh * g->kw * g->C * F >= (1ll << 31) ||
+        (int64_t)g->H * g->W * g->C >= (1ll << 31))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: geometry too large for 32-bit sweeps");
+    hipLaunchKernelGGL(conv_ebops_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, bits_in, bits_ker, *g, F, total, g_bits_in, g_bits_ker);
+    return check_launch("hgq_conv2d_ebops");
 }

@@ -36,7 +36,23 @@ __device__ __forceinline__ float entry_bits(const void *k, const float *i, const
 
 #define HGQ_EBOPS_MAXK 4096
 
-__global__ __launch_bounds__(256) void dense_ebops_kernel(const uint32_t *amax_part, int n_parts, float decay,
+#define HGQ_EBOPS_NT 1024
+
+__device__ __forceinline__ float block_sum_ebops(float v, float *scratch16) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if ((threadIdx.x & 63) == 0) scratch16[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < HGQ_EBOPS_NT / 64; ++w) s += scratch16[w];
+    __syncthreads();
+    return s;
+}
+
+// One workgroup of 1024 threads.  Bit-widths are integers, so the per-row / per-column sums are exact
+// in fp32 in any order and are accumulated with LDS atomics over flat, coalesced sweeps.
+__global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_t *amax_part, int n_parts, float decay,
                                                           const float *beta, float *loss_term,
                                                           const void *k_in, float *i_in, const float *f_in,
                                                           int64_t P, int K, int N, const void *k_ker,
@@ -44,22 +60,24 @@ __global__ __launch_bounds__(256) void dense_ebops_kernel(const uint32_t *amax_p
                                                           float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
                                                           float *ebops, uint32_t *ebops_u32, float *g_f_in,
                                                           float *g_b_ker, float *g_b_bias) {
+    constexpr int NT = HGQ_EBOPS_NT;
     __shared__ float colsum[HGQ_EBOPS_MAXK];  // sum_n bits_ker[k, n]
     __shared__ float insum[HGQ_EBOPS_MAXK];   // sum_p bits_in[p, k]
-    __shared__ float red[4];
+    __shared__ float red[NT / 64];
     const Mode mi(mode_in), mk(mode_ker), mb(mode_bias);
     const int t = threadIdx.x;
     // with beta the gradients are those of the loss term ebops * beta
     const float gscale = beta ? scale * beta[0] : scale;
+    const int64_t PK = P * K;
+    for (int k = t; k < K; k += NT) colsum[k] = 0.0f, insum[k] = 0.0f;
     if (amax_part) {
         // integer-bit tracking of the (KIF, WRAP, training) input quantizer, before its bits are read:
         // _i <- max(_i - decay, ceil(log2(max|x_q| + 2**-f)))
-        // 256 threads = `ne` entries x `ng` slice groups per pass, combined through LDS
-        __shared__ uint32_t tmax[256];
-        const int64_t PK = P * K;
+        // NT threads = `ne` entries x `ng` slice groups per pass, combined through LDS
+        __shared__ uint32_t tmax[NT];
         int ne = 1;
-        while (ne < 256 && ne < PK) ne <<= 1;
-        const int ng = 256 / ne, el = t % ne, grp = t / ne;
+        while (ne < NT && ne < PK) ne <<= 1;
+        const int ng = NT / ne, el = t % ne, grp = t / ne;
         const int per = (n_parts + ng - 1) / ng;
         for (int64_t e0 = 0; e0 < PK; e0 += ne) {
             const int64_t e = e0 + el;
@@ -89,33 +107,43 @@ __global__ __launch_bounds__(256) void dense_ebops_kernel(const uint32_t *amax_p
             __syncthreads();
         }
         __threadfence_block();
-        __syncthreads();
     }
-    for (int k = t; k < K; k += 256) {
-        float s = 0.0f, d;
-        for (int n = 0; n < N; ++n) s += entry_bits(k_ker, nullptr, b_ker, (int64_t)k * N + n, mk, d);
-        colsum[k] = s;
-        float a = 0.0f;
-        for (int64_t p = 0; p < P; ++p) {
-            const float b = entry_bits(k_in, i_in, f_in, p * K + k, mi, d);
-            a += b;
-            if (g_f_in) g_f_in[p * K + k] = d * s * gscale;
+    __syncthreads();
+    const int64_t KN = (int64_t)K * N;
+    for (int64_t e0 = 0; e0 < KN; e0 += 4 * NT) {
+        float b[4], d;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t e = e0 + u * NT + t;
+            b[u] = e < KN ? entry_bits(k_ker, nullptr, b_ker, e, mk, d) : 0.0f;
         }
-        insum[k] = a;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t e = e0 + u * NT + t;
+            if (e < KN) atomicAdd(&colsum[e / N], b[u]);
+        }
+    }
+    __syncthreads();
+    for (int64_t e = t; e < PK; e += NT) {
+        float d;
+        const int k = (int)(e % K);
+        const float b = entry_bits(k_in, i_in, f_in, e, mi, d);
+        atomicAdd(&insum[k], b);
+        if (g_f_in) g_f_in[e] = d * colsum[k] * gscale;
     }
     __syncthreads();
     float part = 0.0f;
-    for (int k = t; k < K; k += 256) part += insum[k] * colsum[k];
-    float total = block_sum_256(part, red);
+    for (int k = t; k < K; k += NT) part += insum[k] * colsum[k];
+    float total = block_sum_ebops(part, red);
     if (g_b_ker)
-        for (int64_t e = t; e < (int64_t)K * N; e += 256) g_b_ker[e] = insum[e / N] * gscale;
+        for (int64_t e = t; e < KN; e += NT) g_b_ker[e] = insum[e / N] * gscale;
     if (b_bias) {
         float bs = 0.0f, d;
-        for (int n = t; n < N; n += 256) {
+        for (int n = t; n < N; n += NT) {
             bs += entry_bits(k_bias, nullptr, b_bias, n, mb, d);
             if (g_b_bias) g_b_bias[n] = bias_size / (float)N * gscale;
         }
-        bs = block_sum_256(bs, red);
+        bs = block_sum_ebops(bs, red);
         total += bs / (float)N * bias_size;
     }
     if (t == 0) {
@@ -276,7 +304,7 @@ extern "C" int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float dec
     if (!(Mode(mode_ker).kbi) || (b_bias && !(Mode(mode_bias).kbi))) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops: kernel/bias bit-widths must use the KBI parametrisation");
     if (amax_part && (n_parts < 1 || Mode(mode_in).kbi || Mode(mode_in).overflow_mode != HGQ_WRAP))
         return fail(HGQ_ERR_ARG, "hgq_dense_ebops: fused tracking is for KIF WRAP input quantizers");
-    hipLaunchKernelGGL(dense_ebops_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, amax_part, n_parts, decay, beta, loss_term, k_in,
+    hipLaunchKernelGGL(dense_ebops_kernel, dim3(1), dim3(HGQ_EBOPS_NT), 0, (hipStream_t)stream, amax_part, n_parts, decay, beta, loss_term, k_in,
                        i_in, f_in, P, K, N, k_ker, b_ker,
                        k_bias, b_bias, scale, bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
     return check_launch("hgq_dense_ebops");

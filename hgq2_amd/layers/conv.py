@@ -113,7 +113,10 @@ class QConv2D(QLayerBaseSingleInput):
     def _compute_ebops(self, shape):
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self._kernel.shape)
-        ebops = torch.sum(self.convolution_op(bw_inp, bw_ker))
+        if prod(self.kernel_size) * bw_inp.shape[-1] <= ops.CONV_EBOPS_MAX and bw_inp.is_cuda:
+            ebops = ops.conv2d_ebops(bw_inp, bw_ker, self.strides, self.padding, self.dilation_rate)
+        else:
+            ebops = torch.sum(self.convolution_op(bw_inp, bw_ker))
         ebops = ebops * (self.parallelization_factor / self.n_parallel)
         if self.bq is not None:
             size = float(prod(shape[:-1]) * self.filters)

@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'CONV_EBOPS_MAX']
 
 
 def _ptr(t: Tensor | None):
@@ -536,6 +536,27 @@ def _(dy, x, geom, is_max):
     return torch.empty_like(x)
 
 
+CONV_EBOPS_MAX = 4096  # hgq_conv2d_ebops covers kh * kw * C up to this
+
+
+@torch.library.custom_op('hgq::conv2d_ebops', mutates_args=())
+def conv2d_ebops_op(bits_in: Tensor, bits_ker: Tensor, geom: Sequence[int]) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('bits_in', bits_in), _check_f32('bits_ker', bits_ker)
+    g = _geom(geom)
+    F = bits_ker.shape[-1]
+    _need(bits_in.numel() == g.H * g.W * g.C and bits_ker.numel() == g.kh * g.kw * g.C * F, 'bit-width tensors do not match the geometry')
+    total = torch.empty((), dtype=torch.float32, device=bits_in.device)
+    g_in, g_ker = torch.empty_like(bits_in), torch.empty_like(bits_ker)
+    rc = _lib.load().hgq_conv2d_ebops(_ptr(bits_in), _ptr(bits_ker), ctypes.addressof(g), F, _ptr(total), _ptr(g_in), _ptr(g_ker), _stream())
+    _lib.check(rc, 'hgq_conv2d_ebops')
+    return total, g_in, g_ker
+
+
+@conv2d_ebops_op.register_fake
+def _(bits_in, bits_ker, geom):
+    return bits_in.new_empty(()), torch.empty_like(bits_in), torch.empty_like(bits_ker)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -734,18 +755,8 @@ class _Conv2D(torch.autograd.Function):
 def conv2d(xq: Tensor, qw: Tensor, qb, strides=(1, 1), padding='valid', dilation=(1, 1), act: int = 0) -> Tensor:
     """``act(conv2d(xq, qw) + qb)`` for a channels-last input [B, H, W, C] and an HWIO kernel; 'same'
     padding puts the odd pad after the last row / column, as Keras / TensorFlow do."""
-    B, H, W, C = xq.shape
-    kh, kw, c2, F = qw.shape
-    _need(c2 == C, f'kernel has {c2} input channels, input has {C}')
-    (sy, sx), (dly, dlx) = strides, dilation
-    eh, ew = dly * (kh - 1) + 1, dlx * (kw - 1) + 1
-    if padding == 'same':
-        OH, OW = -(-H // sy), -(-W // sx)
-        py, px = max((OH - 1) * sy + eh - H, 0) // 2, max((OW - 1) * sx + ew - W, 0) // 2
-    else:
-        OH, OW, py, px = (H - eh) // sy + 1, (W - ew) // sx + 1, 0, 0
-    _need(OH >= 1 and OW >= 1, 'the kernel does not fit the input')
-    geom = (B, H, W, C, kh, kw, sy, sx, py, px, dly, dlx, OH, OW)
+    _need(qw.shape[2] == xq.shape[3], f'kernel has {qw.shape[2]} input channels, input has {xq.shape[3]}')
+    geom = conv_geometry(tuple(xq.shape), tuple(qw.shape), strides, padding, dilation)
     return _Conv2D.apply(xq.contiguous(), qw.contiguous(), qb.contiguous() if qb is not None else xq.new_empty(0), geom, act)
 
 
@@ -838,6 +849,40 @@ def pool2d(x: Tensor, pool_size, strides=None, padding: str = 'valid', mode: str
         OH, OW, py, px = (H - ph) // sy + 1, (W - pw) // sx + 1, 0, 0
     _need(OH >= 1 and OW >= 1, 'the pooling window does not fit the input')
     return _Pool2D.apply(x.contiguous(), (B, H, W, C, ph, pw, sy, sx, py, px, OH, OW), mode == 'max')
+
+
+class _Conv2DEbops(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, bits_in, bits_ker, geom):
+        total, g_in, g_ker = conv2d_ebops_op(bits_in, bits_ker, list(geom))
+        ctx.save_for_backward(g_in, g_ker)
+        return total
+
+    @staticmethod
+    def backward(ctx, g):
+        g_in, g_ker = ctx.saved_tensors
+        return g * g_in, g * g_ker, None
+
+
+def conv_geometry(in_shape, kernel_shape, strides=(1, 1), padding='valid', dilation=(1, 1)):
+    """The 14-entry geometry of a channels-last convolution; 'same' pads like Keras (odd pad after)."""
+    B, H, W, C = in_shape
+    kh, kw = kernel_shape[0], kernel_shape[1]
+    (sy, sx), (dly, dlx) = strides, dilation
+    eh, ew = dly * (kh - 1) + 1, dlx * (kw - 1) + 1
+    if padding == 'same':
+        OH, OW = -(-H // sy), -(-W // sx)
+        py, px = max((OH - 1) * sy + eh - H, 0) // 2, max((OW - 1) * sx + ew - W, 0) // 2
+    else:
+        OH, OW, py, px = (H - eh) // sy + 1, (W - ew) // sx + 1, 0, 0
+    _need(OH >= 1 and OW >= 1, 'the kernel does not fit the input')
+    return (B, H, W, C, kh, kw, sy, sx, py, px, dly, dlx, OH, OW)
+
+
+def conv2d_ebops(bits_in: Tensor, bits_ker: Tensor, strides=(1, 1), padding='valid', dilation=(1, 1)) -> Tensor:
+    """``sum(conv2d(bits_in, bits_ker))`` for bit-width tensors [1, H, W, C] and [kh, kw, C, F], differentiable."""
+    geom = conv_geometry(tuple(bits_in.shape), tuple(bits_ker.shape), strides, padding, dilation)
+    return _Conv2DEbops.apply(bits_in.contiguous(), bits_ker.contiguous(), geom)
 
 
 class _SparseCE(torch.autograd.Function):

@@ -361,6 +361,17 @@ int hgq_attn_combine_bwd(const float *dout, const float *probs, const float *val
 int hgq_pool2d_fwd(const float *x, float *y, const int *geom, int is_max, void *stream);
 int hgq_pool2d_bwd(const float *dy, const float *x, float *dx, const int *geom, int is_max, void *stream);
 
+/*
+ * EBOPs of a convolution and their gradient.  Replaces `ops.sum(self.convolution_op(bw_inp, bw_ker))`
+ * of QBaseConv._compute_ebops (src/hgq/layers/conv.py:91-102), evaluated on the bit-width tensors of
+ * one sample, by its closed form (no convolution is run): every kernel tap visits a rectangle of
+ * input pixels, so the sum factorises per (tap, channel).
+ *   bits_in [H, W, C];  bits_ker [kh, kw, C, F];  total [1];  g_bits_in [H, W, C], g_bits_ker
+ *   [kh, kw, C, F] = d total / d bits (either may be NULL).  g->B is ignored.  kh * kw * C <= 4096.
+ */
+int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, const hgq_conv_geom *g, int F, float *total,
+                     float *g_bits_in, float *g_bits_ker, void *stream);
+
 /* Fill kernel (graph-capture safe replacement for a memset). */
 int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream);
 

@@ -136,3 +136,26 @@ def test_pooling_layers_match_oracle(dev, mode, case):
     _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=2e-5)
     assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
     assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+
+
+@pytest.mark.parametrize('case', [(28, 28, 1, 3, 3, 32, (1, 1), 'valid', (1, 1)), (13, 13, 32, 3, 3, 32, (1, 1), 'valid', (1, 1)),
+                                  (10, 9, 3, 3, 3, 8, (2, 1), 'same', (1, 1)), (11, 11, 6, 3, 2, 10, (2, 3), 'same', (2, 1))])
+def test_conv_ebops_closed_form_is_exact(dev, case):
+    """hgq_conv2d_ebops against the definition it replaces (sum of the convolution of the bit-width
+    tensors, src/hgq/layers/conv.py:91-102), in integer arithmetic, and its gradients via autograd."""
+    from hgq2_amd import ops
+
+    H, W, C, kh, kw, Fo, strides, padding, dilation = case
+    g = torch.Generator().manual_seed(H * W)
+    bi = torch.randint(0, 13, (1, H, W, C), generator=g).float()
+    bk = torch.randint(0, 9, (kh, kw, C, Fo), generator=g).float()
+    bir, bkr = bi.clone().requires_grad_(True), bk.clone().requires_grad_(True)
+    want = _ref_conv(bir.double(), bkr.double(), None, strides, padding, dilation, False).sum()
+    want.backward()
+    bip, bkp = bi.to(dev).requires_grad_(True), bk.to(dev).requires_grad_(True)
+    got = ops.conv2d_ebops(bip, bkp, strides, padding, dilation)
+    (got * 3.0).backward()
+    # the total is one fp32 number: exact below 2**24, correctly rounded partial sums above
+    assert abs(float(got) - float(want)) <= (0 if float(want) < 2**24 else 1e-6 * float(want))
+    assert torch.equal(bip.grad.cpu().double(), 3.0 * bir.grad.double())
+    assert torch.equal(bkp.grad.cpu().double(), 3.0 * bkr.grad.double())
