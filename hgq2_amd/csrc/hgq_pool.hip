@@ -1,9 +1,10 @@
 // 2-D max / average pooling on channels-last tensors, forward and backward.
 //
 // One thread per (pixel, channel group): adjacent threads take adjacent channels, so every window
-// read is coalesced along the channel axis (128-bit when C is a multiple of 4).  The backward is
-// gather-style - a thread owns an INPUT element and visits the windows that contain it - so there
-// are no atomics and uncovered border pixels get an exact zero.  Max pooling routes the gradient
+// read is coalesced along the channel axis (128-bit when C is a multiple of 4).  The backward for
+// overlapping windows is gather-style - a thread owns an INPUT element and visits the windows that
+// contain it - and the one for disjoint windows owns a stride tile; neither uses atomics and
+// uncovered border pixels get an exact zero.  Max pooling routes the gradient
 // to the first maximum of a window in row-major order (what the library max-pool the reference
 // sits on does), recomputed from the forward input.
 #include "hgq_device.h"
@@ -128,6 +129,67 @@ __global__ __launch_bounds__(256) void pool2d_bwd_kernel(const float *__restrict
     }
 }
 
+// Backward for disjoint windows (stride >= pool size, the usual case): a thread owns one stride
+// tile of the INPUT - the window in its corner plus the pixels no window covers - so x and dy are
+// read once and dx is written once.
+template <int VEC, bool MAX>
+__global__ __launch_bounds__(256) void pool2d_bwd_tiles_kernel(const float *__restrict__ dy, const float *__restrict__ x,
+                                                               float *__restrict__ dx, PoolGeom g, int TH, int TW) {
+    const int cg = g.C / VEC;
+    const int64_t n = (int64_t)g.B * TH * TW * cg;
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < n; t += (int64_t)gridDim.x * 256) {
+        const int c = (int)(t % cg) * VEC;
+        int64_t r = t / cg;
+        const int tx = (int)(r % TW);
+        r /= TW;
+        const int ty = (int)(r % TH), b = (int)(r / TH);
+        const bool valid = ty < g.OH && tx < g.OW;
+        const int y0 = ty * g.sy - g.py, x0 = tx * g.sx - g.px;
+        PV<VEC> gv;
+        int first[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) gv.v[e] = 0.f, first[e] = -1;
+        if (valid) {
+            gv = pload<VEC>(dy + (((int64_t)b * g.OH + ty) * g.OW + tx) * g.C + c);
+            if (MAX) {
+                float best[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) best[e] = -INFINITY;
+                for (int wy = 0; wy < g.ph; ++wy) {
+                    const int iy = y0 + wy;
+                    if ((unsigned)iy >= (unsigned)g.H) continue;
+                    for (int wx = 0; wx < g.pw; ++wx) {
+                        const int ix = x0 + wx;
+                        if ((unsigned)ix >= (unsigned)g.W) continue;
+                        const PV<VEC> v = pload<VEC>(x + (((int64_t)b * g.H + iy) * g.W + ix) * g.C + c);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            if (v.v[e] > best[e] || first[e] < 0) best[e] = v.v[e], first[e] = wy * g.pw + wx;
+                    }
+                }
+            } else {
+                const int ya = max(0, y0), yb = min(g.H, y0 + g.ph), xa = max(0, x0), xb = min(g.W, x0 + g.pw);
+                const float inv = 1.0f / (float)((yb - ya) * (xb - xa));
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) gv.v[e] *= inv;
+            }
+        }
+        for (int ry = 0; ry < g.sy; ++ry) {
+            const int iy = y0 + ry;
+            if ((unsigned)iy >= (unsigned)g.H) continue;
+            for (int rx = 0; rx < g.sx; ++rx) {
+                const int ix = x0 + rx;
+                if ((unsigned)ix >= (unsigned)g.W) continue;
+                const bool in_win = valid && ry < g.ph && rx < g.pw;
+                PV<VEC> o;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o.v[e] = in_win && (!MAX || first[e] == ry * g.pw + rx) ? gv.v[e] : 0.f;
+                pstore<VEC>(dx + (((int64_t)b * g.H + iy) * g.W + ix) * g.C + c, o);
+            }
+        }
+    }
+}
+
 static int check_pool(const int *d, PoolGeom &g, const char *who) {
     g.B = d[0], g.H = d[1], g.W = d[2], g.C = d[3], g.ph = d[4], g.pw = d[5], g.sy = d[6], g.sx = d[7], g.py = d[8], g.px = d[9],
     g.OH = d[10], g.OW = d[11];
@@ -167,9 +229,19 @@ extern "C" int hgq_pool2d_bwd(const float *dy, const float *x, float *dx, const 
     if (g.B == 0) return HGQ_OK;
     if (!dy || !dx || (is_max && !x)) return fail(HGQ_ERR_ARG, "hgq_pool2d_bwd: null pointer");
     const bool vec = g.C % 4 == 0 && ((uintptr_t)dy & 15u) == 0 && ((uintptr_t)dx & 15u) == 0 && (!is_max || ((uintptr_t)x & 15u) == 0);
+    hipStream_t s = (hipStream_t)stream;
+    if (g.sy >= g.ph && g.sx >= g.pw) {
+        const int TH = (g.H + g.py + g.sy - 1) / g.sy, TW = (g.W + g.px + g.sx - 1) / g.sx;
+        const int64_t n = (int64_t)g.B * TH * TW * (vec ? g.C / 4 : g.C);
+        const dim3 grid((unsigned)persistent_grid((n + 255) / 256, 32));
+        if (vec && is_max) hipLaunchKernelGGL((pool2d_bwd_tiles_kernel<4, true>), grid, dim3(256), 0, s, dy, x, dx, g, TH, TW);
+        else if (vec) hipLaunchKernelGGL((pool2d_bwd_tiles_kernel<4, false>), grid, dim3(256), 0, s, dy, x, dx, g, TH, TW);
+        else if (is_max) hipLaunchKernelGGL((pool2d_bwd_tiles_kernel<1, true>), grid, dim3(256), 0, s, dy, x, dx, g, TH, TW);
+        else hipLaunchKernelGGL((pool2d_bwd_tiles_kernel<1, false>), grid, dim3(256), 0, s, dy, x, dx, g, TH, TW);
+        return check_launch("hgq_pool2d_bwd");
+    }
     const int64_t n = (int64_t)g.B * g.H * g.W * (vec ? g.C / 4 : g.C);
     const dim3 grid((unsigned)persistent_grid((n + 255) / 256, 32));
-    hipStream_t s = (hipStream_t)stream;
     if (vec && is_max) hipLaunchKernelGGL((pool2d_bwd_kernel<4, true>), grid, dim3(256), 0, s, dy, x, dx, g);
     else if (vec) hipLaunchKernelGGL((pool2d_bwd_kernel<4, false>), grid, dim3(256), 0, s, dy, x, dx, g);
     else if (is_max) hipLaunchKernelGGL((pool2d_bwd_kernel<1, true>), grid, dim3(256), 0, s, dy, x, dx, g);

@@ -113,6 +113,9 @@ def test_wide_dense_layer_matches_oracle(dev):
     (5, 9, 11, 3, (3, 2), (2, 1), 'same'),       # overlapping windows, odd padding, scalar channel path
     (4, 7, 7, 8, (3, 3), (3, 3), 'valid'),       # border pixels that no window covers
     (3, 8, 6, 4, (2, 3), (1, 2), 'same'),
+    (2, 7, 8, 4, (3, 3), (3, 3), 'same'),        # disjoint windows that start in the padding
+    (2, 9, 10, 1, (2, 2), (3, 3), 'valid'),      # stride larger than the window: gaps between windows
+    (3, 7, 9, 8, (2, 2), (2, 2), 'same'),
 ])
 def test_pooling_layers_match_oracle(dev, mode, case):
     """QMaxPooling2D / QAveragePooling2D: values, EBOPs, tracked bits and gradients (incl. where the
