@@ -166,6 +166,134 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
     }
 }
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+// Four consecutive k columns (same tap, channels ch .. ch + 3; the depth is a multiple of 4) of one row.
+template <int MODE>
+__device__ __forceinline__ void gather4(const float *__restrict__ src, const float *__restrict__ mask, const RowInfo &r,
+                                        const ColInfo &c, const hgq_conv_geom &g, int F, f32x4_t &v, f32x4_t &mk) {
+    v = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    mk = f32x4_t{1.f, 1.f, 1.f, 1.f};
+    if (r.base < 0 || !c.on) return;
+    if (MODE == 0) {
+        const int iy = r.y0 + c.ky * g.dly, ix = r.x0 + c.kx * g.dlx;
+        if ((unsigned)iy >= (unsigned)g.H || (unsigned)ix >= (unsigned)g.W) return;
+        v = *(const f32x4_t *)(src + ((int64_t)r.base + iy * g.W + ix) * g.C + c.ch);
+    } else {
+        const int ty = r.y0 - c.ky * g.dly, tx = r.x0 - c.kx * g.dlx;
+        if (ty < 0 || tx < 0) return;
+        const int oy = ty / g.sy, ox = tx / g.sx;
+        if (oy * g.sy != ty || ox * g.sx != tx || oy >= g.OH || ox >= g.OW) return;
+        const int64_t a = ((int64_t)r.base + oy * g.OW + ox) * F + c.ch;
+        v = *(const f32x4_t *)(src + a);
+        if (mask) mk = *(const f32x4_t *)(mask + a);
+    }
+}
+
+// The same contraction for a gathered depth (C forward, F data gradient) that is a multiple of 4
+// and 16-byte aligned operands.  A row's 32 k columns of a step are read as eight 128-bit loads
+// by eight adjacent lanes, the loads of step s + 1 are in flight while the matrix cores work on
+// step s (two LDS buffers, one barrier per step), and the A tile sits k-major in LDS with a row
+// stride of BM + 2 words: the transposing writes and the operand reads both spread evenly over
+// the banks.
+template <int MODE, int WN>
+__global__ __launch_bounds__(256) void igemm_vec_kernel(const float *__restrict__ src, const float *__restrict__ mask,
+                                                        const float *__restrict__ w, const float *__restrict__ bias,
+                                                        float *__restrict__ out, hgq_conv_geom g, int F, int64_t rows, int K,
+                                                        int N, int act, int kchunk) {
+    constexpr int WM = 4 / WN, BM = 32 * WM, BN = 32 * WN, AS = BM + 2, NP = BM / 32, NB = CV_BK * BN / 256;
+    const bool split = gridDim.z > 1;
+    const int k_begin = blockIdx.z * kchunk, k_end = min(K, k_begin + kchunk);
+    if (split) out += (int64_t)blockIdx.z * rows * N;
+    __shared__ float as[2][CV_BK][AS];
+    __shared__ float bs[2][CV_BK][BN + 1];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int n0 = blockIdx.y * BN;
+    const int64_t n_tiles = (rows + BM - 1) / BM;
+    const int q = tid & 7, rbase = tid >> 3;
+    const int n_steps = (k_end - k_begin + CV_BK - 1) / CV_BK;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t r0 = tile * BM;
+        RowInfo ri[NP];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) ri[p] = decode_row<MODE>(r0 + rbase + 32 * p, rows, g);
+        f32x4_t av[NP], am[NP];
+        float bv[NB];
+        auto fetch = [&](int k0) {
+            const ColInfo ci = decode_col<MODE>(k0 + 4 * q, k_end, g, F);
+#pragma unroll
+            for (int p = 0; p < NP; ++p) gather4<MODE>(src, mask, ri[p], ci, g, F, av[p], am[p]);
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const int id = tid + 256 * j;
+                int kk, nn;
+                if (MODE == 0) kk = id / BN, nn = id % BN;
+                else nn = id / CV_BK, kk = id % CV_BK;
+                const int k = k0 + kk, n = n0 + nn;
+                float v = 0.f;
+                if (k < k_end && n < N) {
+                    if (MODE == 0) {
+                        v = w[(int64_t)k * N + n];
+                    } else {
+                        const int tap = k / F, f = k - tap * F;
+                        v = w[((int64_t)tap * N + n) * F + f];
+                    }
+                }
+                bv[j] = v;
+            }
+        };
+        auto stash = [&](int buf) {
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float v = av[p][j];
+                    if (MODE == 1 && !(am[p][j] > 0.f)) v = 0.f;
+                    as[buf][4 * q + j][rbase + 32 * p] = v;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const int id = tid + 256 * j;
+                if (MODE == 0) bs[buf][id / BN][id % BN] = bv[j];
+                else bs[buf][id % CV_BK][id / CV_BK] = bv[j];
+            }
+        };
+        __syncthreads();  // the previous tile's last step may still be reading buffer (n_steps - 1) & 1
+        fetch(k_begin);
+        stash(0);
+        __syncthreads();
+        floatx16 acc = {0};
+        for (int st = 0; st < n_steps; ++st) {
+            const int buf = st & 1;
+            const bool more = st + 1 < n_steps;
+            if (more) fetch(k_begin + (st + 1) * CV_BK);
+            {
+                const int arow = wm * 32 + (lane & 31), kq = lane >> 5, bcol = wn * 32 + (lane & 31);
+#pragma unroll
+                for (int kk = 0; kk < CV_BK; kk += 2)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[buf][kk + kq][arow], bs[buf][kk + kq][bcol], acc, 0, 0, 0);
+            }
+            if (more) stash(buf ^ 1);
+            __syncthreads();
+        }
+        const int n = n0 + wn * 32 + (lane & 31);
+        if (n < N) {
+            const float bb = (MODE == 0 && bias && !split) ? bias[n] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = r0 + wm * 32 + cv_acc_row(r, lane);
+                if (m < rows) {
+                    float v = acc[r] + bb;
+                    if (MODE == 0 && act == HGQ_ACT_RELU && !split) v = v > 0.f ? v : 0.f;
+                    out[m * N + n] = v;
+                }
+            }
+        }
+    }
+}
+
 // y = act(sum of the k-split slices + bias), slices added in order.
 __global__ __launch_bounds__(256) void splitk_finish_kernel(const float *__restrict__ part, int n_parts, int64_t n,
                                                             const float *__restrict__ bias, int N, int act,
@@ -559,6 +687,17 @@ static int64_t wgrad_splits(int64_t rows, int n_tiles_kn) {
     return s < 1 ? 1 : s;
 }
 
+static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+template <int MODE>
+static void launch_igemm(bool vec, bool wide, dim3 grid, hipStream_t s, const float *src, const float *mask, const float *w,
+                         const float *bias, float *out, const hgq_conv_geom &g, int F, int64_t rows, int K, int N, int act, int kchunk) {
+    if (vec && wide) hipLaunchKernelGGL((igemm_vec_kernel<MODE, 2>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
+    else if (vec) hipLaunchKernelGGL((igemm_vec_kernel<MODE, 1>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
+    else if (wide) hipLaunchKernelGGL((igemm_kernel<MODE, 2>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
+    else hipLaunchKernelGGL((igemm_kernel<MODE, 1>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
+}
+
 }  // namespace hgq
 
 using namespace hgq;
@@ -586,12 +725,13 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
     kchunk = (kchunk + CV_BK - 1) / CV_BK * CV_BK;
     const int nz = (K + kchunk - 1) / kchunk;
     float *dst = nz > 1 ? workspace : y;
+    const bool vec = g->C % 4 == 0 && aligned16(xq);
     if (F <= 32) {
-        const dim3 grid((unsigned)persistent_grid((rows + 127) / 128, 8), 1, (unsigned)nz);
-        hipLaunchKernelGGL((igemm_kernel<0, 1>), grid, dim3(256), 0, s, xq, (const float *)nullptr, qw, qb, dst, *g, F, rows, K, F, act, kchunk);
+        const dim3 grid((unsigned)persistent_grid((rows + 127) / 128, vec ? 3 : 8), 1, (unsigned)nz);
+        launch_igemm<0>(vec, false, grid, s, xq, nullptr, qw, qb, dst, *g, F, rows, K, F, act, kchunk);
     } else {
-        const dim3 grid((unsigned)persistent_grid((rows + 63) / 64, 8), (unsigned)((F + 63) / 64), (unsigned)nz);
-        hipLaunchKernelGGL((igemm_kernel<0, 2>), grid, dim3(256), 0, s, xq, (const float *)nullptr, qw, qb, dst, *g, F, rows, K, F, act, kchunk);
+        const dim3 grid((unsigned)persistent_grid((rows + 63) / 64, vec ? 4 : 8), (unsigned)((F + 63) / 64), (unsigned)nz);
+        launch_igemm<0>(vec, true, grid, s, xq, nullptr, qw, qb, dst, *g, F, rows, K, F, act, kchunk);
     }
     if ((rc = check_launch("hgq_conv2d_fwd"))) return rc;
     if (nz > 1) {
@@ -650,12 +790,15 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
             else if (fp == 32) HGQ_DG(32);
             else HGQ_DG(64);
 #undef HGQ_DG
-        } else if (g->C <= 32) {
-            const dim3 grid((unsigned)persistent_grid((in_rows + 127) / 128, 8), 1);
-            hipLaunchKernelGGL((igemm_kernel<1, 1>), grid, dim3(256), 0, s, dy, mask, qw, (const float *)nullptr, dxq, *g, F, in_rows, Kt, g->C, act, Kt);
         } else {
-            const dim3 grid((unsigned)persistent_grid((in_rows + 63) / 64, 8), (unsigned)((g->C + 63) / 64));
-            hipLaunchKernelGGL((igemm_kernel<1, 2>), grid, dim3(256), 0, s, dy, mask, qw, (const float *)nullptr, dxq, *g, F, in_rows, Kt, g->C, act, Kt);
+            const bool vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask));
+            if (g->C <= 32) {
+                const dim3 grid((unsigned)persistent_grid((in_rows + 127) / 128, vec ? 3 : 8), 1);
+                launch_igemm<1>(vec, false, grid, s, dy, mask, qw, nullptr, dxq, *g, F, in_rows, Kt, g->C, act, Kt);
+            } else {
+                const dim3 grid((unsigned)persistent_grid((in_rows + 63) / 64, vec ? 4 : 8), (unsigned)((g->C + 63) / 64));
+                launch_igemm<1>(vec, true, grid, s, dy, mask, qw, nullptr, dxq, *g, F, in_rows, Kt, g->C, act, Kt);
+            }
         }
         if ((rc = check_launch("hgq_conv2d_bwd(data)"))) return rc;
     }

@@ -38,6 +38,9 @@ CASES = [
     (48, 1, 1, 3872, 1, 1, 10, (1, 1), 'valid', (1, 1), True, True),           # long contraction, few rows: split along k
     (300, 6, 6, 2, 3, 3, 24, (1, 1), 'valid', (1, 1), True, True),             # K = 18: row-split weight gradient
     (40, 8, 8, 5, 3, 3, 16, (1, 1), 'valid', (1, 1), False, True),             # K = 45: two k blocks, two row groups
+    (3, 10, 11, 8, 3, 2, 12, (2, 1), 'same', (1, 2), True, True),              # 128-bit gathers with stride, dilation, padding
+    (2, 9, 9, 36, 3, 3, 36, (2, 2), 'same', (1, 1), True, True),               # 128-bit gathers, 64-wide tiles both ways
+    (1024, 12, 12, 8, 3, 3, 8, (1, 1), 'valid', (1, 1), True, True),           # more row tiles than workgroups
 ]
 
 
