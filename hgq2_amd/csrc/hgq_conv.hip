@@ -561,6 +561,118 @@ __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ sr
     }
 }
 
+// The weight / bias gradient for C and F multiples of 4 and 16-byte aligned operands: 128-bit
+// gathers and dz loads, the loads of row step s + 1 in flight while the matrix cores work on
+// step s (two LDS buffers, one barrier per step).  Same tiling and slice layout as wgrad_kernel.
+template <int WK, int WN, int WS>
+__global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict__ src, const float *__restrict__ dy,
+                                                        const float *__restrict__ y, float *__restrict__ part, hgq_conv_geom g,
+                                                        int F, int64_t rows, int K, int64_t chunk, int act, int n_ktiles) {
+    constexpr int BKT = 32 * WK, BN = 32 * WN, BMS = 32 * WS;
+    constexpr int AQ = 8 * WK, AP = WS * WK, AR = 32 / WK;  // A: float4 per row, passes per thread, rows per pass
+    constexpr int ZQ = 8 * WN, ZP = WS * WN, ZR = 32 / WN;  // dz: the same
+    constexpr int AST = BKT + 4, ZST = BN + 4;
+    static_assert(WK * WN * WS == 4, "four wavefronts");
+    __shared__ float as[2][BMS][AST];
+    __shared__ float zs[2][BMS][ZST];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wsub = wave / (WK * WN), wk = (wave / WN) % WK, wn = wave % WN;
+    const int kt = blockIdx.x % n_ktiles, nt = blockIdx.x / n_ktiles;
+    const int k0 = kt * BKT, n0 = nt * BN;
+    const int64_t m_begin = (int64_t)blockIdx.y * chunk, m_end = min(rows, m_begin + chunk);
+    const int64_t KF = (int64_t)K * F;
+    float *my = part + (int64_t)blockIdx.y * (KF + F);
+    const int aq = tid % AQ, ar = tid / AQ, zq = tid % ZQ, zr = tid / ZQ;
+    const ColInfo ci = decode_col<0>(k0 + 4 * aq, K, g, F);
+    const bool z_on = n0 + 4 * zq < F, relu = act == HGQ_ACT_RELU;
+    floatx16 acc = {0};
+    f32x4_t bsum = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t av[AP], zv[ZP], zm[ZP];
+    auto fetch = [&](int64_t m0) {
+#pragma unroll
+        for (int p = 0; p < AP; ++p) {
+            const int64_t m = m0 + ar + AR * p;
+            const RowInfo ri = decode_row<0>(m < m_end ? m : rows, rows, g);
+            f32x4_t unused;
+            gather4<0>(src, nullptr, ri, ci, g, F, av[p], unused);
+        }
+#pragma unroll
+        for (int p = 0; p < ZP; ++p) {
+            const int64_t m = m0 + zr + ZR * p;
+            zv[p] = f32x4_t{0.f, 0.f, 0.f, 0.f}, zm[p] = f32x4_t{1.f, 1.f, 1.f, 1.f};
+            if (m < m_end && z_on) {
+                zv[p] = *(const f32x4_t *)(dy + m * F + n0 + 4 * zq);
+                if (relu) zm[p] = *(const f32x4_t *)(y + m * F + n0 + 4 * zq);
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < AP; ++p) *(f32x4_t *)&as[buf][ar + AR * p][4 * aq] = av[p];
+#pragma unroll
+        for (int p = 0; p < ZP; ++p) {
+            f32x4_t v = zv[p];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (!(zm[p][j] > 0.f)) v[j] = 0.f;
+            bsum += v;
+            *(f32x4_t *)&zs[buf][zr + ZR * p][4 * zq] = v;
+        }
+    };
+    const int64_t n_steps = m_end > m_begin ? (m_end - m_begin + BMS - 1) / BMS : 0;
+    if (n_steps > 0) {
+        fetch(m_begin);
+        stash(0);
+    }
+    __syncthreads();
+    for (int64_t st = 0; st < n_steps; ++st) {
+        const int buf = (int)(st & 1);
+        const bool more = st + 1 < n_steps;
+        if (more) fetch(m_begin + (st + 1) * BMS);
+        const int kq = lane >> 5, c32 = lane & 31, mb = wsub * 32;
+#pragma unroll
+        for (int mm = 0; mm < 32; mm += 2)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[buf][mb + mm + kq][wk * 32 + c32], zs[buf][mb + mm + kq][wn * 32 + c32], acc, 0, 0, 0);
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+    }
+    float *red = &as[0][0][0];  // 2 * BMS * AST >= 4096 floats whenever WS > 1
+    if (WS > 1) {
+        const int blk = wk * WN + wn;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[((blk * WS + wsub) * 32 + cv_acc_row(r, lane)) * 32 + (lane & 31)] = acc[r];
+        __syncthreads();
+        if (wsub == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = 0.f;
+                for (int u = 0; u < WS; ++u) v += red[((blk * WS + u) * 32 + cv_acc_row(r, lane)) * 32 + (lane & 31)];
+                acc[r] = v;
+            }
+        }
+        __syncthreads();
+    }
+    const int n = n0 + wn * 32 + (lane & 31);
+    if (wsub == 0 && n < F) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int k = k0 + wk * 32 + cv_acc_row(r, lane);
+            if (k < K) my[(int64_t)k * F + n] = acc[r];
+        }
+    }
+    if (kt == 0) {
+        // bias gradient: the threads that share four dz columns add up in a fixed order
+#pragma unroll
+        for (int j = 0; j < 4; ++j) red[tid * 4 + j] = bsum[j];
+        __syncthreads();
+        if (tid < BN && n0 + tid < F) {
+            float sacc = 0.f;
+            for (int u = 0; u < 256 / ZQ; ++u) sacc += red[(u * ZQ + tid / 4) * 4 + tid % 4];
+            my[KF + n0 + tid] = sacc;
+        }
+    }
+}
+
 struct WgradCfg {
     int wk, wn, ws;
     int n_kt, n_nt;
@@ -809,8 +921,12 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
         int64_t chunk = (rows + splits - 1) / splits;
         chunk = (chunk + 127) / 128 * 128;
         const dim3 grid((unsigned)(c.n_kt * c.n_nt), (unsigned)splits);
+        const bool vec = g->C % 4 == 0 && F % 4 == 0 && aligned16(xq) && aligned16(dy) && (!mask || aligned16(mask));
 #define HGQ_WGRAD(WK, WN, WS) \
-    hipLaunchKernelGGL((wgrad_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt)
+    do { \
+        if (vec) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+        else hipLaunchKernelGGL((wgrad_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+    } while (0)
         if (c.wk == 2 && c.wn == 2) HGQ_WGRAD(2, 2, 1);
         else if (c.wk == 1) HGQ_WGRAD(1, 1, 4);
         else if (c.wk == 2) HGQ_WGRAD(2, 1, 2);
