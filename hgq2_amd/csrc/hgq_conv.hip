@@ -474,6 +474,234 @@ __global__ __launch_bounds__(256) void dgrad_patch_kernel(const float *__restric
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Few input channels (C <= 4: the image itself), at most 32 filters, kernel size known at compile
+// time.  A matrix-core tile would be almost empty and the layer is bound by the HBM traffic of the
+// [.., F] tensor, so these kernels work on an 8 x 32 pixel tile per workgroup with lanes along
+// the filter axis: every access to the F-wide tensor is a coalesced 128-byte row, the small
+// operand sits in LDS and is read as a broadcast, the kernel entries of a lane sit in registers.
+// ---------------------------------------------------------------------------------------------
+#define SC_TH 8
+#define SC_TW 32
+
+template <int KH, int KW, int C>
+__global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                         const float *__restrict__ bias, float *__restrict__ out, hgq_conv_geom g,
+                                                         int F, int act, int tiles_x, int tiles_y) {
+    constexpr int KC = KH * KW * C;
+    extern __shared__ float lds[];  // input patch [XH][XW][C]
+    const int XH = (SC_TH - 1) * g.sy + (KH - 1) * g.dly + 1, XW = (SC_TW - 1) * g.sx + (KW - 1) * g.dlx + 1;
+    const int f = threadIdx.x & 31, slot = threadIdx.x >> 5;
+    const bool f_on = f < F;
+    float wreg[KC];
+#pragma unroll
+    for (int t = 0; t < KC; ++t) wreg[t] = f_on ? w[t * F + f] : 0.f;
+    const float bb = (bias && f_on) ? bias[f] : 0.f;
+    const int64_t n_tiles = (int64_t)g.B * tiles_y * tiles_x;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int b = (int)(tile / (tiles_y * tiles_x)), rem = (int)(tile - (int64_t)b * tiles_y * tiles_x);
+        const int oy0 = (rem / tiles_x) * SC_TH, ox0 = (rem % tiles_x) * SC_TW;
+        const int iy0 = oy0 * g.sy - g.py, ix0 = ox0 * g.sx - g.px;
+        __syncthreads();
+        for (int e = threadIdx.x; e < XH * XW * C; e += 256) {
+            const int r = e / (XW * C), q = e - r * XW * C, iy = iy0 + r, ix = ix0 + q / C;
+            float v = 0.f;
+            if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) v = x[(((int64_t)b * g.H + iy) * g.W + ix0) * C + q];
+            lds[e] = v;
+        }
+        __syncthreads();
+        const int oy = oy0 + slot;
+        if (oy < g.OH) {
+            const int n_x = min(SC_TW, g.OW - ox0);
+            float *orow = out + (((int64_t)b * g.OH + oy) * g.OW + ox0) * F + f;
+            for (int tx = 0; tx < n_x; ++tx) {
+                const float *xp = lds + (slot * g.sy * XW + tx * g.sx) * C;
+                float acc = bb;
+#pragma unroll
+                for (int t = 0; t < KC; ++t) {
+                    const int ky = t / (KW * C), kx = (t / C) % KW, c = t % C;
+                    acc += xp[(ky * g.dly * XW + kx * g.dlx) * C + c] * wreg[t];
+                }
+                if (act == HGQ_ACT_RELU) acc = acc > 0.f ? acc : 0.f;
+                if (f_on) orow[(int64_t)tx * F] = acc;
+            }
+        }
+    }
+}
+
+// Data, weight and bias gradient in one pass over dy (and the forward output for the ReLU mask),
+// for unit stride and dilation.  A workgroup takes an 8 x 32 tile of INPUT pixels, stages the
+// (8 + KH - 1) x (32 + KW - 1) patch of dz = dy * mask it touches (pixel stride F + 1 words) and
+// the matching input patch, then
+//   - thread = input pixel contracts the patch with the kernel (data gradient), and
+//   - lane = filter, 8 row slots: every OUTPUT pixel is owned by exactly one tile (the patch
+//     without its top / left halo; the first tile row / column also owns the pixels above / left
+//     of it that exist because of the padding); a lane accumulates dz * x for its KC kernel
+//     entries over the owned pixels in registers.
+// After its last tile the workgroup adds the 8 slots in slot order and writes slice blockIdx.x of
+// `part` ([KC * F | F]); a second kernel adds the slices in order.
+template <int KH, int KW, int C>
+__global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict__ dy, const float *__restrict__ mask,
+                                                         const float *__restrict__ x, const float *__restrict__ w,
+                                                         float *__restrict__ dx, float *__restrict__ part, hgq_conv_geom g, int F,
+                                                         int tiles_x, int tiles_y, int vec) {
+    constexpr int KC = KH * KW * C, PH = SC_TH + KH - 1, PW = SC_TW + KW - 1;
+    extern __shared__ float lds[];  // kernel [KC * F] | dz patch [PH * PW][F + 1] (reused for the final sum) | input patch
+    const int FS = F + 1, XH = PH + g.py, XW = PW + g.px;
+    float *wl = lds, *zp = lds + ((KC * F + 3) & ~3), *xp = zp + max(PH * PW * FS, SC_TH * (KC + 1) * 32);
+    const int tid = threadIdx.x, f = tid & 31, slot = tid >> 5;
+    const bool f_on = f < F;
+    for (int t = tid; t < KC * F; t += 256) wl[t] = w[t];
+    float wacc[KC], bacc = 0.f;
+#pragma unroll
+    for (int t = 0; t < KC; ++t) wacc[t] = 0.f;
+    const int64_t n_tiles = (int64_t)g.B * tiles_y * tiles_x;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int b = (int)(tile / (tiles_y * tiles_x)), rem = (int)(tile - (int64_t)b * tiles_y * tiles_x);
+        const int iy0 = (rem / tiles_x) * SC_TH, ix0 = (rem % tiles_x) * SC_TW;
+        const int oy0 = iy0 + g.py - (KH - 1), ox0 = ix0 + g.px - (KW - 1);
+        __syncthreads();
+        if (vec) {
+            // 128-bit loads, four units (dz and mask) in flight per thread
+            const int upr = PW * F / 4, n_u = PH * upr;
+            for (int e0 = 0; e0 < n_u; e0 += 4 * 256) {
+                f32x4_t v[4], m[4];
+                int dst[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int e = e0 + u * 256 + tid;
+                    v[u] = f32x4_t{0.f, 0.f, 0.f, 0.f}, m[u] = f32x4_t{1.f, 1.f, 1.f, 1.f}, dst[u] = -1;
+                    if (e < n_u) {
+                        const int pr = e / upr, q = (e - pr * upr) * 4, pc = q / F, f0 = q - pc * F;
+                        const int oy = oy0 + pr, ox = ox0 + pc;
+                        dst[u] = (pr * PW + pc) * FS + f0;
+                        if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) {
+                            const int64_t a = (((int64_t)b * g.OH + oy) * g.OW + ox) * F + f0;
+                            v[u] = *(const f32x4_t *)(dy + a);
+                            if (mask) m[u] = *(const f32x4_t *)(mask + a);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (dst[u] >= 0) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) zp[dst[u] + j] = m[u][j] > 0.f ? v[u][j] : 0.f;
+                    }
+                }
+            }
+        } else {
+            const int upr = PW * F, n_u = PH * upr;
+            for (int e0 = 0; e0 < n_u; e0 += 8 * 256) {
+                float v[8], m[8];
+                int dst[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int e = e0 + u * 256 + tid;
+                    v[u] = 0.f, m[u] = 1.f, dst[u] = -1;
+                    if (e < n_u) {
+                        const int pr = e / upr, q = e - pr * upr, pc = q / F, f0 = q - pc * F;
+                        const int oy = oy0 + pr, ox = ox0 + pc;
+                        dst[u] = (pr * PW + pc) * FS + f0;
+                        if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) {
+                            const int64_t a = (((int64_t)b * g.OH + oy) * g.OW + ox) * F + f0;
+                            v[u] = dy[a];
+                            if (mask) m[u] = mask[a];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (dst[u] >= 0) zp[dst[u]] = m[u] > 0.f ? v[u] : 0.f;
+            }
+        }
+        if (part) {
+            for (int e = tid; e < XH * XW * C; e += 256) {
+                const int r = e / (XW * C), q = e - r * XW * C, iy = iy0 - g.py + r, ix = ix0 - g.px + q / C;
+                float v = 0.f;
+                if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) v = x[(((int64_t)b * g.H + iy) * g.W + ix) * C + q % C];
+                xp[e] = v;
+            }
+        }
+        __syncthreads();
+        if (dx) {
+            const int tx = tid % SC_TW, ty = tid / SC_TW;
+            const int iy = iy0 + ty, ix = ix0 + tx;
+            if (iy < g.H && ix < g.W) {
+                float acc[C];
+#pragma unroll
+                for (int c = 0; c < C; ++c) acc[c] = 0.f;
+#pragma unroll
+                for (int ky = 0; ky < KH; ++ky) {
+#pragma unroll
+                    for (int kx = 0; kx < KW; ++kx) {
+                        // oy = iy + py - ky  ->  patch row ty + (KH - 1) - ky
+                        const float *pp = zp + ((ty + KH - 1 - ky) * PW + (tx + KW - 1 - kx)) * FS;
+                        const float *wt = wl + (ky * KW + kx) * C * F;
+                        int ff = 0;
+                        for (; ff + 8 <= F; ff += 8) {
+                            float v[8];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) v[u] = pp[ff + u];
+#pragma unroll
+                            for (int c = 0; c < C; ++c) {
+                                float wv[8];
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) wv[u] = wt[c * F + ff + u];
+#pragma unroll
+                                for (int u = 0; u < 8; ++u) acc[c] += v[u] * wv[u];
+                            }
+                        }
+                        for (; ff < F; ++ff) {
+                            const float v = pp[ff];
+#pragma unroll
+                            for (int c = 0; c < C; ++c) acc[c] += v * wt[c * F + ff];
+                        }
+                    }
+                }
+                const int64_t o = (((int64_t)b * g.H + iy) * g.W + ix) * C;
+#pragma unroll
+                for (int c = 0; c < C; ++c) dx[o + c] = acc[c];
+            }
+        }
+        if (part) {
+            for (int pr = slot; pr < PH; pr += SC_TH) {
+                const int oy = oy0 + pr;
+                if ((unsigned)oy >= (unsigned)g.OH || !(pr >= KH - 1 || iy0 == 0)) continue;
+                const int pc_lo = ix0 == 0 ? max(0, -ox0) : KW - 1, pc_hi = min(PW, g.OW - ox0);
+                for (int pc = pc_lo; pc < pc_hi; ++pc) {
+                    const float z = f_on ? zp[(pr * PW + pc) * FS + f] : 0.f;
+                    bacc += z;
+                    // input pixel of tap (ky, kx): patch-relative (pr + ky - (KH - 1) + py, pc + kx - (KW - 1) + px)
+                    const float *xq = xp + ((pr - (KH - 1) + g.py) * XW + (pc - (KW - 1) + g.px)) * C;
+#pragma unroll
+                    for (int t = 0; t < KC; ++t) {
+                        const int ky = t / (KW * C), kx = (t / C) % KW, c = t % C;
+                        wacc[t] += xq[(ky * XW + kx) * C + c] * z;
+                    }
+                }
+            }
+        }
+    }
+    if (part) {
+        __syncthreads();
+        float *red = zp;  // [slot][KC + 1][32]
+#pragma unroll
+        for (int t = 0; t < KC; ++t) red[(slot * (KC + 1) + t) * 32 + f] = wacc[t];
+        red[(slot * (KC + 1) + KC) * 32 + f] = bacc;
+        __syncthreads();
+        float *my = part + (int64_t)blockIdx.x * ((int64_t)KC * F + F);
+        for (int e = tid; e < (KC + 1) * 32; e += 256) {
+            const int t = e >> 5, ff = e & 31;
+            if (ff < F) {
+                float sacc = 0.f;
+                for (int u = 0; u < SC_TH; ++u) sacc += red[(u * (KC + 1) + t) * 32 + ff];
+                my[(int64_t)t * F + ff] = sacc;
+            }
+        }
+    }
+}
+
 // Weight / bias gradient.  Workgroup (kt, nt, split): k tile of 32 * WK columns of the im2col
 // matrix, n tile of 32 * WN filters, rows [split * chunk, (split + 1) * chunk) taken 32 * WS at
 // a step, WS wavefronts sharing one output block (combined through LDS at the end);
@@ -799,6 +1027,40 @@ static int64_t wgrad_splits(int64_t rows, int n_tiles_kn) {
     return s < 1 ? 1 : s;
 }
 
+// Launch plan of the few-channel kernels: which (kh, kw, C) are instantiated, LDS sizes, grid.
+static bool smallc_shape(const hgq_conv_geom &g, int F) {
+    const bool k33 = g.kh == 3 && g.kw == 3 && g.C >= 1 && g.C <= 4;
+    const bool k55 = g.kh == 5 && g.kw == 5 && g.C == 1;
+    return (k33 || k55) && F <= 32;
+}
+static size_t fwd_smallc_lds(const hgq_conv_geom &g) {
+    const size_t XH = (size_t)(SC_TH - 1) * g.sy + (size_t)(g.kh - 1) * g.dly + 1, XW = (size_t)(SC_TW - 1) * g.sx + (size_t)(g.kw - 1) * g.dlx + 1;
+    return XH * XW * g.C * sizeof(float);
+}
+static bool fwd_smallc_ok(const hgq_conv_geom &g, int F) { return smallc_shape(g, F) && fwd_smallc_lds(g) <= 48 * 1024; }
+static size_t bwd_smallc_lds(const hgq_conv_geom &g, int F) {
+    const size_t KC = (size_t)g.kh * g.kw * g.C, PH = SC_TH + g.kh - 1, PW = SC_TW + g.kw - 1;
+    size_t zp = PH * PW * (F + 1), red = SC_TH * (KC + 1) * 32;
+    if (red > zp) zp = red;
+    return (((KC * F + 3) & ~(size_t)3) + zp + (PH + g.py) * (PW + g.px) * g.C) * sizeof(float);
+}
+static bool bwd_smallc_ok(const hgq_conv_geom &g, int F) {
+    return smallc_shape(g, F) && g.sy == 1 && g.sx == 1 && g.dly == 1 && g.dlx == 1 && g.py < g.kh && g.px < g.kw &&
+           bwd_smallc_lds(g, F) <= 64 * 1024;
+}
+static int bwd_smallc_grid(const hgq_conv_geom &g) {
+    const int64_t tiles = (int64_t)g.B * ((g.H + SC_TH - 1) / SC_TH) * ((g.W + SC_TW - 1) / SC_TW);
+    return persistent_grid(tiles, 3);
+}
+#define HGQ_SMALLC_DISPATCH(CALL) \
+    do { \
+        if (g->kh == 5) CALL(5, 5, 1); \
+        else if (g->C == 1) CALL(3, 3, 1); \
+        else if (g->C == 2) CALL(3, 3, 2); \
+        else if (g->C == 3) CALL(3, 3, 3); \
+        else CALL(3, 3, 4); \
+    } while (0)
+
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 template <int MODE>
@@ -837,6 +1099,15 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
     kchunk = (kchunk + CV_BK - 1) / CV_BK * CV_BK;
     const int nz = (K + kchunk - 1) / kchunk;
     float *dst = nz > 1 ? workspace : y;
+    if (fwd_smallc_ok(*g, F)) {
+        const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
+        const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
+        const size_t lds = fwd_smallc_lds(*g);
+#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y)
+        HGQ_SMALLC_DISPATCH(HGQ_FWD_SC);
+#undef HGQ_FWD_SC
+        return check_launch("hgq_conv2d_fwd(few channels)");
+    }
     const bool vec = g->C % 4 == 0 && aligned16(xq);
     if (F <= 32) {
         const dim3 grid((unsigned)persistent_grid((rows + 127) / 128, vec ? 3 : 8), 1, (unsigned)nz);
@@ -860,7 +1131,9 @@ extern "C" int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F) {
     const int64_t rows = (int64_t)g->B * g->OH * g->OW;
     const int K = g->kh * g->kw * g->C;
     const WgradCfg c = wgrad_cfg(K, F);
-    return wgrad_splits(rows, c.n_kt * c.n_nt) * ((int64_t)K * F + F);
+    int64_t slices = wgrad_splits(rows, c.n_kt * c.n_nt);
+    if (bwd_smallc_ok(*g, F) && bwd_smallc_grid(*g) > slices) slices = bwd_smallc_grid(*g);
+    return slices * ((int64_t)K * F + F);
 }
 
 extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw,
@@ -881,6 +1154,21 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
     if (!dy || !qw || !xq) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null pointer");
     if (act == HGQ_ACT_RELU && !y) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: relu needs the forward output");
     const float *mask = act == HGQ_ACT_RELU ? y : nullptr;
+    if (bwd_smallc_ok(*g, F)) {
+        const bool want_w = dqw || dqb;
+        if (want_w && !workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null workspace");
+        const int tiles_x = (g->W + SC_TW - 1) / SC_TW, tiles_y = (g->H + SC_TH - 1) / SC_TH;
+        const int grid = bwd_smallc_grid(*g);
+        const size_t lds = bwd_smallc_lds(*g, F);
+        const int vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask));
+#define HGQ_BWD_SC(KH, KW, CC) \
+    hipLaunchKernelGGL((bwd_smallc_kernel<KH, KW, CC>), dim3((unsigned)grid), dim3(256), lds, s, dy, mask, xq, qw, dxq, want_w ? workspace : (float *)nullptr, *g, F, tiles_x, tiles_y, vec)
+        HGQ_SMALLC_DISPATCH(HGQ_BWD_SC);
+#undef HGQ_BWD_SC
+        if ((rc = check_launch("hgq_conv2d_bwd(few channels)"))) return rc;
+        if (want_w) return reduce_parts(workspace, grid, KF + F, dqw, KF, dqb, (int64_t)F, nullptr, 0, s);
+        return HGQ_OK;
+    }
     if (dxq) {
         const int Kt = g->kh * g->kw * F;  // contraction length of the data gradient
         const size_t patch_lds = ((size_t)g->kh * g->kw * g->C * F + (size_t)(DP_TH + g->kh - 1) * (DP_TW + g->kw - 1) * (F + 1)) * sizeof(float);

@@ -41,6 +41,11 @@ CASES = [
     (3, 10, 11, 8, 3, 2, 12, (2, 1), 'same', (1, 2), True, True),              # 128-bit gathers with stride, dilation, padding
     (2, 9, 9, 36, 3, 3, 36, (2, 2), 'same', (1, 1), True, True),               # 128-bit gathers, 64-wide tiles both ways
     (1024, 12, 12, 8, 3, 3, 8, (1, 1), 'valid', (1, 1), True, True),           # more row tiles than workgroups
+    (5, 40, 37, 3, 3, 3, 32, (1, 1), 'same', (1, 1), True, True),              # few channels: ragged pixel tiles both ways, padding
+    (3, 19, 70, 4, 3, 3, 16, (1, 1), 'valid', (1, 1), False, True),            # four channels
+    (4, 17, 33, 1, 5, 5, 7, (1, 1), 'same', (1, 1), True, False),              # 5 x 5 on one channel, scalar staging
+    (2, 20, 45, 1, 3, 3, 12, (2, 1), 'valid', (2, 3), True, True),             # few channels forward with stride and dilation
+    (900, 9, 34, 2, 3, 3, 8, (1, 1), 'same', (1, 1), True, True),              # more pixel tiles than workgroups
 ]
 
 
