@@ -931,37 +931,49 @@ static int fwd_ksplit(int64_t rows, int K, int F) {
 //     S[tap, c] = sum of bits_in over the input pixels that tap visits,   Wsum[tap, c] = sum_f bits_ker[tap, c, f]
 //     total = sum S * Wsum;   d total / d bits_ker[tap, c, f] = S[tap, c];
 //     d total / d bits_in[y, x, c] = sum over the taps that visit (y, x) of Wsum[tap, c]
+// The pixels a tap visits form a (strided) rectangle, so S is computed separably: column sums
+// R[ky][x][c] over the visited rows first, then sums of R over the visited columns.
 // One workgroup; every quantity is a sum of small integers, exact in fp32 in any order while below 2^24.
-#define CE_MAX 4096  // kh * kw * C
+#define CE_MAX 4096   // kh * kw * C
+#define CE_MAXR 8192  // kh * W * C
+#define CE_MAXV 2048  // H * kh and W * kw
 __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restrict__ bits_in, const float *__restrict__ bits_ker,
                                                           hgq_conv_geom g, int F, float *total,
                                                           float *__restrict__ g_in, float *__restrict__ g_ker) {
-    __shared__ float S[CE_MAX], Ws[CE_MAX];
+    __shared__ float S[CE_MAX], Ws[CE_MAX], R[CE_MAXR];
     __shared__ float red[1024];
-    const int t = threadIdx.x, taps = g.kh * g.kw, TC = taps * g.C;
-    for (int e = t; e < TC; e += 1024) S[e] = 0.f, Ws[e] = 0.f;
-    __syncthreads();
-    // S: flat sweep over (tap, output pixel, channel), channel fastest so reads coalesce
-    const int OP = g.OH * g.OW, n_s = taps * OP * g.C;
-    for (int e0 = 0; e0 < n_s; e0 += 4 * 1024) {
-        float v[4];
-        int dst[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int e = e0 + u * 1024 + t;
-            v[u] = 0.f, dst[u] = -1;
-            if (e < n_s) {
-                const int c = e % g.C, r = e / g.C, op = r % OP, tap = r / OP;
-                const int oy = op / g.OW, ox = op - oy * g.OW, ky = tap / g.kw, kx = tap - ky * g.kw;
-                const int iy = oy * g.sy - g.py + ky * g.dly, ix = ox * g.sx - g.px + kx * g.dlx;
-                if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W)
-                    v[u] = bits_in[((int64_t)iy * g.W + ix) * g.C + c], dst[u] = tap * g.C + c;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-            if (dst[u] >= 0) atomicAdd(&S[dst[u]], v[u]);
+    __shared__ unsigned char vy[CE_MAXV], vx[CE_MAXV];  // vy[y * kh + ky]: row y is visited by kernel row ky
+    const int t = threadIdx.x, taps = g.kh * g.kw, TC = taps * g.C, WC = g.W * g.C;
+    for (int e = t; e < TC; e += 1024) Ws[e] = 0.f;
+    for (int e = t; e < g.H * g.kh; e += 1024) {
+        const int y = e / g.kh, ky = e - y * g.kh, ty = y + g.py - ky * g.dly;
+        vy[e] = ty >= 0 && ty % g.sy == 0 && ty / g.sy < g.OH;
     }
+    for (int e = t; e < g.W * g.kw; e += 1024) {
+        const int x = e / g.kw, kx = e - x * g.kw, tx = x + g.px - kx * g.dlx;
+        vx[e] = tx >= 0 && tx % g.sx == 0 && tx / g.sx < g.OW;
+    }
+    // R[ky][x][c]: adjacent threads take adjacent (x, c), so every row read is coalesced
+    for (int e = t; e < g.kh * WC; e += 1024) {
+        const int ky = e / WC, xc = e - ky * WC;
+        float r = 0.f;
+        int oy = 0;
+        for (; oy + 4 <= g.OH; oy += 4) {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int iy = (oy + u) * g.sy - g.py + ky * g.dly;
+                v[u] = (unsigned)iy < (unsigned)g.H ? bits_in[(int64_t)iy * WC + xc] : 0.f;
+            }
+            r += (v[0] + v[1]) + (v[2] + v[3]);
+        }
+        for (; oy < g.OH; ++oy) {
+            const int iy = oy * g.sy - g.py + ky * g.dly;
+            if ((unsigned)iy < (unsigned)g.H) r += bits_in[(int64_t)iy * WC + xc];
+        }
+        R[e] = r;
+    }
+    __syncthreads();
     const int n_w = TC * F;
     for (int e0 = 0; e0 < n_w; e0 += 4 * 1024) {
         float v[4];
@@ -976,6 +988,15 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
             if (e < n_w) atomicAdd(&Ws[e / F], v[u]);
         }
     }
+    for (int e = t; e < TC; e += 1024) {
+        const int tap = e / g.C, c = e - tap * g.C, ky = tap / g.kw, kx = tap - ky * g.kw;
+        float sacc = 0.f;
+        for (int ox = 0; ox < g.OW; ++ox) {
+            const int ix = ox * g.sx - g.px + kx * g.dlx;
+            if ((unsigned)ix < (unsigned)g.W) sacc += R[ky * WC + ix * g.C + c];
+        }
+        S[e] = sacc;
+    }
     __syncthreads();
     float part = 0.f;
     for (int e = t; e < TC; e += 1024) part += S[e] * Ws[e];
@@ -989,17 +1010,13 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
     if (g_ker)
         for (int e = t; e < n_w; e += 1024) g_ker[e] = S[e / F];
     if (g_in) {
-        for (int e = t; e < g.H * g.W * g.C; e += 1024) {
-            const int c = e % g.C, pix = e / g.C, y = pix / g.W, x = pix - y * g.W;
+        for (int e = t; e < g.H * WC; e += 1024) {
+            const int y = e / WC, xc = e - y * WC, x = xc / g.C, c = xc - x * g.C;
             float a = 0.f;
             for (int ky = 0; ky < g.kh; ++ky) {
-                const int ty = y + g.py - ky * g.dly;
-                if (ty < 0 || ty % g.sy != 0 || ty / g.sy >= g.OH) continue;
-                for (int kx = 0; kx < g.kw; ++kx) {
-                    const int tx = x + g.px - kx * g.dlx;
-                    if (tx < 0 || tx % g.sx != 0 || tx / g.sx >= g.OW) continue;
-                    a += Ws[(ky * g.kw + kx) * g.C + c];
-                }
+                if (!vy[y * g.kh + ky]) continue;
+                for (int kx = 0; kx < g.kw; ++kx)
+                    if (vx[x * g.kw + kx]) a += Ws[(ky * g.kw + kx) * g.C + c];
             }
             g_in[e] = a;
         }
@@ -1232,8 +1249,10 @@ extern "C" int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, con
     int rc = check_geom(g, F, "hgq_conv2d_ebops");
     if (rc) return rc;
     if (!bits_in || !bits_ker || !total) return fail(HGQ_ERR_ARG, "hgq_conv2d_ebops: null pointer");
-    if ((int64_t)g->kh * g->kw * g->C > CE_MAX)
-        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: kh * kw * C = %lld exceeds %d", (long long)g->kh * g->kw * g->C, CE_MAX);
+    if ((int64_t)g->kh * g->kw * g->C > CE_MAX || (int64_t)g->kh * g->W * g->C > CE_MAXR || (int64_t)g->H * g->kh > CE_MAXV ||
+        (int64_t)g->W * g->kw > CE_MAXV)
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: needs kh * kw * C <= %d, kh * W * C <= %d, H * kh and W * kw <= %d", CE_MAX,
+                    CE_MAXR, CE_MAXV);
     if ((int64_t)g->kh * g->kw * g->C * g->OH * g->OW >= (1ll << 31) || (int64_t)g->kh * g->kw * g->C * F >= (1ll << 31) ||
         (int64_t)g->H * g->W * g->C >= (1ll << 31))
         return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: geometry too large for 32-bit sweeps");

@@ -304,6 +304,13 @@ extern "C" int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float dec
     if (!(Mode(mode_ker).kbi) || (b_bias && !(Mode(mode_bias).kbi))) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops: kernel/bias bit-widths must use the KBI parametrisation");
     if (amax_part && (n_parts < 1 || Mode(mode_in).kbi || Mode(mode_in).overflow_mode != HGQ_WRAP))
         return fail(HGQ_ERR_ARG, "hgq_dense_ebops: fused tracking is for KIF WRAP input quantizers");
+    if (amax_part && P * K * n_parts > 16384) {
+        // many tracker slices: combine them with one thread group per entry across the device first
+        int rc = hgq_wrap_track_i(amax_part, nullptr, n_parts, i_in, f_in, nullptr, P * K, decay, 0.0f, 0.0f,
+                                  mode_in & ~(HGQ_MODE_TRACING | HGQ_MODE_SYMMETRIC), stream);
+        if (rc) return rc;
+        amax_part = nullptr;
+    }
     hipLaunchKernelGGL(dense_ebops_kernel, dim3(1), dim3(HGQ_EBOPS_NT), 0, (hipStream_t)stream, amax_part, n_parts, decay, beta, loss_term, k_in,
                        i_in, f_in, P, K, N, k_ker, b_ker,
                        k_bias, b_bias, scale, bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);

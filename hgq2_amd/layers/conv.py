@@ -113,7 +113,7 @@ class QConv2D(QLayerBaseSingleInput):
     def _compute_ebops(self, shape):
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self._kernel.shape)
-        if prod(self.kernel_size) * bw_inp.shape[-1] <= ops.CONV_EBOPS_MAX and bw_inp.is_cuda:
+        if bw_inp.is_cuda and ops.conv2d_ebops_supported(tuple(bw_inp.shape), tuple(bw_ker.shape)):
             ebops = ops.conv2d_ebops(bw_inp, bw_ker, self.strides, self.padding, self.dilation_rate)
         else:
             ebops = torch.sum(self.convolution_op(bw_inp, bw_ker))

@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'CONV_EBOPS_MAX']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported']
 
 
 def _ptr(t: Tensor | None):
@@ -536,7 +536,11 @@ def _(dy, x, geom, is_max):
     return torch.empty_like(x)
 
 
-CONV_EBOPS_MAX = 4096  # hgq_conv2d_ebops covers kh * kw * C up to this
+def conv2d_ebops_supported(in_shape, kernel_shape) -> bool:
+    """Whether hgq_conv2d_ebops covers bit-width tensors [1, H, W, C] x [kh, kw, C, F] (its LDS tables bound the sizes)."""
+    _, H, W, C = in_shape
+    kh, kw = kernel_shape[0], kernel_shape[1]
+    return kh * kw * C <= 4096 and kh * W * C <= 8192 and H * kh <= 2048 and W * kw <= 2048
 
 
 @torch.library.custom_op('hgq::conv2d_ebops', mutates_args=())
