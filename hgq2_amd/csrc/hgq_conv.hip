@@ -166,7 +166,6 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
     }
 }
 
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // Four consecutive k columns (same tap, channels ch .. ch + 3; the depth is a multiple of 4) of one row.
 template <int MODE>

@@ -322,37 +322,44 @@ struct FastMap {
     }
 };
 
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ float4 ld4_or_zero(const float *p, bool ok) {
-    if (!ok) return make_float4(0.f, 0.f, 0.f, 0.f);
-    const f32x4_t t = __builtin_nontemporal_load((const f32x4_t *)p);
-    return make_float4(t.x, t.y, t.z, t.w);
-}
 __device__ __forceinline__ void st4(float *p, const float4 &v) {
     f32x4_t t;
     t.x = v.x, t.y = v.y, t.z = v.z, t.w = v.w;
-    __builtin_nontemporal_store(t, (f32x4_t *)p);
+    *(f32x4_t *)p = t;
 }
 
-template <int RM, bool QUANT>
+// Forward.  The kernel matrix never touches LDS: lane (j, h) of a wavefront keeps the 32 entries
+// W[2 s + h][column j] it multiplies by in registers for the whole launch.  The input tile sits
+// in LDS with its columns permuted (even k first, then odd k) so that the 32 operands of a lane,
+// x[row][2 s + h], s = 0 .. 31, are contiguous and are read four at a time; rows are 68 words
+// apart, which keeps those 128-bit reads free of bank conflicts.  The output tile goes back
+// through LDS so that it leaves as full 128-bit rows.
+#define FAST_XLD 68
+template <int RM, bool QUANT, int NS4>
 __global__ __launch_bounds__(256) void qdense_fwd_fast_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw,
                                                               const float *__restrict__ qb, float *__restrict__ y,
                                                               uint32_t *amax_part, int64_t rows, int K, int N, int act,
                                                               int mode) {
-    __shared__ float xs[2][FAST_BM][FAST_LD];
-    __shared__ float ws[64][FAST_LD];
+    __shared__ __attribute__((aligned(16))) float xs[2][FAST_BM + 1][FAST_XLD];  // row FAST_BM: sink of the idle staging slots
+    __shared__ __attribute__((aligned(16))) float ys[FAST_BM][FAST_XLD];
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rh = wave & 1, cb = wave >> 1;
     const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
-    for (int id = tid; id < 64 * 64; id += 256) {
-        const int kk = id >> 6, nn = id & 63;
-        ws[kk][nn] = (kk < K && nn < N) ? qw[(int64_t)kk * N + nn] : 0.f;
-        xs[0][kk][nn] = 0.f, xs[1][kk][nn] = 0.f;  // columns >= K stay zero
+    for (int id = tid; id < 2 * (FAST_BM + 1) * FAST_XLD; id += 256) (&xs[0][0][0])[id] = 0.f;  // columns >= K stay zero
+    const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
+    float wreg[4 * NS4];
+#pragma unroll
+    for (int sidx = 0; sidx < 4 * NS4; ++sidx) {
+        const int k = 2 * sidx + kq;
+        wreg[sidx] = (k < K && bcol < N) ? qw[(int64_t)k * N + bcol] : 0.f;
     }
-    FastMap mp;
+    const float bias = (qb && bcol < N) ? qb[bcol] : 0.f;
+    FastMap mp, mo;
     mp.init(K);
+    const bool vec_out = (N & 3) == 0 && ((uintptr_t)y & 15u) == 0;
+    mo.init(vec_out ? N : 4);
     int fi[FAST_NJ][4];
     uint32_t amx[FAST_NJ][4];
 #pragma unroll
@@ -365,58 +372,80 @@ __global__ __launch_bounds__(256) void qdense_fwd_fast_kernel(const float *__res
                 fi[j][e] = (int)(m.round_params ? rintf(f) : f);
             }
         }
-    float4 raw[FAST_NJ];
-    int64_t tile = blockIdx.x;
-    if (tile < n_tiles) {
+    f32x4_t raw[FAST_NJ];
+    uint32_t xoff[FAST_NJ];
 #pragma unroll
-        for (int j = 0; j < FAST_NJ; ++j) {
-            const int64_t gr = tile * FAST_BM + mp.row[j];
-            raw[j] = ld4_or_zero(x + gr * K + mp.col[j], mp.on[j] && gr < rows);
-        }
-    }
-    const int K2 = (K + 1) & ~1;
+    for (int j = 0; j < FAST_NJ; ++j) xoff[j] = mp.on[j] ? (uint32_t)(mp.row[j] * K + mp.col[j]) * 4u : BUF_OOB;
+    // the descriptor covers the valid rows of one tile: rows past the end read as zero
+    auto load_tile = [&](int64_t t) {
+        const int64_t r0 = t * FAST_BM, left = rows - r0;
+        const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K, (left < FAST_BM ? left : FAST_BM) * K * 4);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) raw[j] = buf_ld4(rs, xoff[j]);
+    };
+    int64_t tile = blockIdx.x;
+    if (tile < n_tiles) load_tile(tile);
+    __syncthreads();
+    // everything loaded so far (kernel entries, bit-widths) has arrived: no wait on them inside the loop
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     int buf = 0;
     for (; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
+        // no branch around a staging slot (a wait inside one would cover every load): idle slots
+        // hold zeros and write them to the sink row
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
-            if (mp.on[j]) {
-                float v[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+            float v[4] = {raw[j][0], raw[j][1], raw[j][2], raw[j][3]};
+            if (QUANT) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (QUANT) {
-                        v[e] = ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]);
-                        amx[j][e] = max(amx[j][e], abs_bits(v[e]));
-                    }
-                    xs[buf][mp.row[j]][mp.col[j] + e] = v[e];
+                    v[e] = ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]);
+                    amx[j][e] = max(amx[j][e], abs_bits(v[e]));
                 }
             }
+            // columns k0 .. k0 + 3 -> even ones at k0 / 2, odd ones at 32 + k0 / 2
+            float *dst = &xs[buf][mp.on[j] ? mp.row[j] : FAST_BM][mp.col[j] >> 1];
+            *(float2 *)dst = make_float2(v[0], v[2]);
+            *(float2 *)(dst + 32) = make_float2(v[1], v[3]);
         }
         __syncthreads();
         const int64_t next = tile + gridDim.x;
-        if (next < n_tiles) {
+        if (next < n_tiles) load_tile(next);
+        floatx16 acc = {0};
+        if (cb * 32 < N) {
+            const float *arow_p = &xs[buf][arow][kq * 32];
+            // NS4 groups of four k pairs cover K (columns past K are zero on both sides)
+            f32x4_t a4[NS4];
+#pragma unroll
+            for (int s4 = 0; s4 < NS4; ++s4) a4[s4] = *(const f32x4_t *)(arow_p + 4 * s4);
+#pragma unroll
+            for (int s4 = 0; s4 < NS4; ++s4)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[s4][e], wreg[4 * s4 + e], acc, 0, 0, 0);
+        }
+        const int64_t r0 = tile * FAST_BM;
+        if (vec_out) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = acc[r] + bias;
+                if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                ys[rh * 32 + acc_row(r, lane)][bcol] = v;
+            }
+            __syncthreads();
 #pragma unroll
             for (int j = 0; j < FAST_NJ; ++j) {
-                const int64_t gr = next * FAST_BM + mp.row[j];
-                raw[j] = ld4_or_zero(x + gr * K + mp.col[j], mp.on[j] && gr < rows);
+                const int64_t gr = r0 + mo.row[j];
+                if (mo.on[j] && gr < rows) {
+                    *(f32x4_t *)(y + gr * N + mo.col[j]) = *(const f32x4_t *)&ys[mo.row[j]][mo.col[j]];
+                }
             }
-        }
-        if (cb * 32 < N) {
-            floatx16 acc = {0};
-            const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
-            for (int kk = 0; kk < K2; kk += 2)
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[buf][arow][kk + kq], ws[kk + kq][bcol], acc, 0, 0, 0);
-            const int n = bcol;
-            if (n < N) {
-                const float bias = qb ? qb[n] : 0.f;
-                const int64_t r0 = tile * FAST_BM + rh * 32;
+        } else if (bcol < N) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int64_t gr = r0 + acc_row(r, lane);
-                    if (gr < rows) {
-                        float v = acc[r] + bias;
-                        if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
-                        y[gr * N + n] = v;
-                    }
+            for (int r = 0; r < 16; ++r) {
+                const int64_t gr = r0 + rh * 32 + acc_row(r, lane);
+                if (gr < rows) {
+                    float v = acc[r] + bias;
+                    if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                    y[gr * N + bcol] = v;
                 }
             }
         }
@@ -449,8 +478,8 @@ __global__ __launch_bounds__(256) void qdense_bwd_fast_kernel(const float *__res
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
                                                               float *part, int has_bias, int64_t rows, int K, int N, int act,
                                                               int mode) {
-    __shared__ float xs[FAST_BM][FAST_LD];
-    __shared__ float dzs[FAST_BM][FAST_LD];  // dz, then the dx tile
+    __shared__ float xs[FAST_BM + 1][FAST_LD];   // row FAST_BM: sink of the idle staging slots
+    __shared__ float dzs[FAST_BM + 1][FAST_LD];  // dz, then the dx tile
     __shared__ float ws[64][FAST_LD];
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -490,38 +519,49 @@ __global__ __launch_bounds__(256) void qdense_bwd_fast_kernel(const float *__res
     const int bn = tid & 63, bq = tid >> 6;
     const bool relu = act == HGQ_ACT_RELU;
 
-    float4 rx[FAST_NJ], rg[FAST_NJ], ry[FAST_NJ];
+    f32x4_t rx[FAST_NJ], rg[FAST_NJ], ry[FAST_NJ];
+    uint32_t xoff[FAST_NJ], zoff[FAST_NJ];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) {
+        xoff[j] = mx.on[j] ? (uint32_t)(mx.row[j] * K + mx.col[j]) * 4u : BUF_OOB;
+        zoff[j] = mz.on[j] ? (uint32_t)(mz.row[j] * N + mz.col[j]) * 4u : BUF_OOB;
+    }
     int64_t tile = blockIdx.x;
+    // descriptors cover the valid rows of one tile (rows past the end read as zero); without ReLU
+    // the mask descriptor is empty and is not consulted
     auto load_tile = [&](int64_t t) {
+        const int64_t r0 = t * FAST_BM, left = rows - r0, vr = left < FAST_BM ? left : FAST_BM;
+        const __amdgpu_buffer_rsrc_t sx = buf_rsrc(x + r0 * K, vr * K * 4), sg = buf_rsrc(dy + r0 * N, vr * N * 4);
+        const __amdgpu_buffer_rsrc_t sy = buf_rsrc(relu ? y + r0 * N : dy, relu ? vr * N * 4 : 0);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
-            const int64_t gx = t * FAST_BM + mx.row[j], gz = t * FAST_BM + mz.row[j];
-            rx[j] = ld4_or_zero(x + gx * K + mx.col[j], mx.on[j] && gx < rows);
-            rg[j] = ld4_or_zero(dy + gz * N + mz.col[j], mz.on[j] && gz < rows);
-            ry[j] = relu ? ld4_or_zero(y + gz * N + mz.col[j], mz.on[j] && gz < rows) : make_float4(1.f, 1.f, 1.f, 1.f);
+            rx[j] = buf_ld4(sx, xoff[j]);
+            rg[j] = buf_ld4(sg, zoff[j]);
+            ry[j] = buf_ld4(sy, zoff[j]);
         }
     };
     if (tile < n_tiles) load_tile(tile);
+    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing loaded before the loop is waited for inside it
     for (; tile < n_tiles; tile += gridDim.x) {
         float dlt[FAST_NJ][4];  // xq - x of the elements this thread stages
         __syncthreads();        // previous tile's dx has been read back
+        // no branch around a staging slot (a wait inside one would cover every load): idle slots
+        // hold zeros and write them to the sink row
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
-            if (mx.on[j]) {
-                const float v[4] = {rx[j].x, rx[j].y, rx[j].z, rx[j].w};
+            const float v[4] = {rx[j][0], rx[j][1], rx[j][2], rx[j][3]};
+            const int xr = mx.on[j] ? mx.row[j] : FAST_BM, zr = mz.on[j] ? mz.row[j] : FAST_BM;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float q = QUANT ? ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]) : v[e];
-                    dlt[j][e] = q - v[e];
-                    xs[mx.row[j]][mx.col[j] + e] = q;
-                }
+            for (int e = 0; e < 4; ++e) {
+                const float q = QUANT ? ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]) : v[e];
+                dlt[j][e] = q - v[e];
+                xs[xr][mx.col[j] + e] = q;
             }
-            if (mz.on[j]) {
-                const float g[4] = {rg[j].x, rg[j].y, rg[j].z, rg[j].w};
-                const float a[4] = {ry[j].x, ry[j].y, ry[j].z, ry[j].w};
+            const float g[4] = {rg[j][0], rg[j][1], rg[j][2], rg[j][3]};
+            const float a[4] = {ry[j][0], ry[j][1], ry[j][2], ry[j][3]};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) dzs[mz.row[j]][mz.col[j] + e] = a[e] > 0.f ? g[e] : 0.f;
-            }
+            for (int e = 0; e < 4; ++e) dzs[zr][mz.col[j] + e] = (!relu || a[e] > 0.f) ? g[e] : 0.f;
         }
         __syncthreads();
         const int64_t next = tile + gridDim.x;
@@ -695,10 +735,18 @@ extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_i
     if (fast) {
         const dim3 fgrid((unsigned)row_parts(rows, FWD_BM));
         const int P = quant ? (int)bw_rows : 1;
-        if (!quant) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_TRN, false>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, (uint32_t *)nullptr, rows, K, N, act, mode);
-        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_TRN, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode);
-        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_RND, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode);
-        else hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_RND_CONV, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode);
+#define HGQ_FWD_FAST(NS4V) \
+    do { \
+        if (!quant) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_TRN, false, NS4V>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, (uint32_t *)nullptr, rows, K, N, act, mode); \
+        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_TRN, true, NS4V>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode); \
+        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_RND, true, NS4V>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode); \
+        else hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_RND_CONV, true, NS4V>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode); \
+    } while (0)
+        if (K <= 8) HGQ_FWD_FAST(1);
+        else if (K <= 16) HGQ_FWD_FAST(2);
+        else if (K <= 32) HGQ_FWD_FAST(4);
+        else HGQ_FWD_FAST(8);
+#undef HGQ_FWD_FAST
         return check_launch("hgq_qdense_fwd");
     }
     const dim3 grid((unsigned)row_parts(rows, FWD_BM), (unsigned)((N + FWD_BN - 1) / FWD_BN));

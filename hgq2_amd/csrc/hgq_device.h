@@ -163,6 +163,26 @@ __device__ __forceinline__ float ceil_log2_exact(float v) {
     return (float)(mant == 0.5f ? e - 1 : e);
 }
 
+
+// ---- buffer loads ------------------------------------------------------------------------
+// The hardware returns 0 for an offset outside the descriptor's range, so a lane that must not
+// read passes BUF_OOB instead of branching around the load.  (A load inside a branch - and the
+// compiler turns `ok ? load : 0` into one - is waited for where it is issued, which serialises
+// the loads of a tile and defeats any prefetch.)  `base` must be wave-uniform; ranges are capped
+// at 2 GiB, so callers rebase the descriptor per tile for large tensors.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+#define BUF_OOB 0xfffffff0u
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buf_rsrc(const void *base, int64_t bytes) {
+    const int64_t cap = 0x7fffffff;
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes < 0 ? 0 : (bytes > cap ? cap : bytes)), 0x00020000);
+}
+__device__ __forceinline__ f32x4_t buf_ld4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+    return __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0));
+}
+__device__ __forceinline__ float buf_ld1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+}
+
 // ------------------------------------------------------------------------------------------
 // all-reduce over groups of SUB consecutive lanes (SUB = 16, 32 or 64): four DPP steps inside
 // each 16-lane row (xor 1, xor 2, half-row mirror, row mirror), then the row totals are read
