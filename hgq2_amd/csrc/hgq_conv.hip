@@ -167,25 +167,22 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
 }
 
 
-// Four consecutive k columns (same tap, channels ch .. ch + 3; the depth is a multiple of 4) of one row.
+// Byte offset of four consecutive k columns (same tap, channels ch .. ch + 3; the depth is a
+// multiple of 4) of one row in the gathered tensor, or BUF_OOB where the tap falls outside it:
+// the buffer load then returns zeros and no branch surrounds the load.
 template <int MODE>
-__device__ __forceinline__ void gather4(const float *__restrict__ src, const float *__restrict__ mask, const RowInfo &r,
-                                        const ColInfo &c, const hgq_conv_geom &g, int F, f32x4_t &v, f32x4_t &mk) {
-    v = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    mk = f32x4_t{1.f, 1.f, 1.f, 1.f};
-    if (r.base < 0 || !c.on) return;
+__device__ __forceinline__ uint32_t gather4_offset(const RowInfo &r, const ColInfo &c, const hgq_conv_geom &g, int F) {
+    if (r.base < 0 || !c.on) return BUF_OOB;
     if (MODE == 0) {
         const int iy = r.y0 + c.ky * g.dly, ix = r.x0 + c.kx * g.dlx;
-        if ((unsigned)iy >= (unsigned)g.H || (unsigned)ix >= (unsigned)g.W) return;
-        v = *(const f32x4_t *)(src + ((int64_t)r.base + iy * g.W + ix) * g.C + c.ch);
+        if ((unsigned)iy >= (unsigned)g.H || (unsigned)ix >= (unsigned)g.W) return BUF_OOB;
+        return (uint32_t)((r.base + iy * g.W + ix) * g.C + c.ch) * 4u;
     } else {
         const int ty = r.y0 - c.ky * g.dly, tx = r.x0 - c.kx * g.dlx;
-        if (ty < 0 || tx < 0) return;
+        if (ty < 0 || tx < 0) return BUF_OOB;
         const int oy = ty / g.sy, ox = tx / g.sx;
-        if (oy * g.sy != ty || ox * g.sx != tx || oy >= g.OH || ox >= g.OW) return;
-        const int64_t a = ((int64_t)r.base + oy * g.OW + ox) * F + c.ch;
-        v = *(const f32x4_t *)(src + a);
-        if (mask) mk = *(const f32x4_t *)(mask + a);
+        if (oy * g.sy != ty || ox * g.sx != tx || oy >= g.OH || ox >= g.OW) return BUF_OOB;
+        return (uint32_t)((r.base + oy * g.OW + ox) * F + c.ch) * 4u;
     }
 }
 
@@ -212,6 +209,10 @@ __global__ __launch_bounds__(256) void igemm_vec_kernel(const float *__restrict_
     const int64_t n_tiles = (rows + BM - 1) / BM;
     const int q = tid & 7, rbase = tid >> 3;
     const int n_steps = (k_end - k_begin + CV_BK - 1) / CV_BK;
+    // the gathered tensor (and the ReLU mask, same shape) as buffer descriptors: the launcher
+    // guarantees they are smaller than 2 GiB
+    const int64_t src_bytes = (MODE == 0 ? (int64_t)g.B * g.H * g.W * g.C : (int64_t)g.B * g.OH * g.OW * F) * 4;
+    const __amdgpu_buffer_rsrc_t rs_src = buf_rsrc(src, src_bytes), rs_mask = buf_rsrc(mask ? mask : src, mask ? src_bytes : 0);
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int64_t r0 = tile * BM;
         RowInfo ri[NP];
@@ -222,7 +223,11 @@ __global__ __launch_bounds__(256) void igemm_vec_kernel(const float *__restrict_
         auto fetch = [&](int k0) {
             const ColInfo ci = decode_col<MODE>(k0 + 4 * q, k_end, g, F);
 #pragma unroll
-            for (int p = 0; p < NP; ++p) gather4<MODE>(src, mask, ri[p], ci, g, F, av[p], am[p]);
+            for (int p = 0; p < NP; ++p) {
+                const uint32_t off = gather4_offset<MODE>(ri[p], ci, g, F);
+                av[p] = buf_ld4(rs_src, off);
+                if (MODE == 1) am[p] = buf_ld4(rs_mask, off);
+            }
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
                 const int id = tid + 256 * j;
@@ -248,7 +253,7 @@ __global__ __launch_bounds__(256) void igemm_vec_kernel(const float *__restrict_
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     float v = av[p][j];
-                    if (MODE == 1 && !(am[p][j] > 0.f)) v = 0.f;
+                    if (MODE == 1 && mask && !(am[p][j] > 0.f)) v = 0.f;
                     as[buf][4 * q + j][rbase + 32 * p] = v;
                 }
             }
@@ -496,6 +501,7 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
 #pragma unroll
     for (int t = 0; t < KC; ++t) wreg[t] = f_on ? w[t * F + f] : 0.f;
     const float bb = (bias && f_on) ? bias[f] : 0.f;
+    const __amdgpu_buffer_rsrc_t rs_x = buf_rsrc(x, (int64_t)g.B * g.H * g.W * C * 4);  // < 2 GiB (checked by the launcher)
     const int64_t n_tiles = (int64_t)g.B * tiles_y * tiles_x;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int b = (int)(tile / (tiles_y * tiles_x)), rem = (int)(tile - (int64_t)b * tiles_y * tiles_x);
@@ -504,9 +510,8 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
         __syncthreads();
         for (int e = threadIdx.x; e < XH * XW * C; e += 256) {
             const int r = e / (XW * C), q = e - r * XW * C, iy = iy0 + r, ix = ix0 + q / C;
-            float v = 0.f;
-            if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) v = x[(((int64_t)b * g.H + iy) * g.W + ix0) * C + q];
-            lds[e] = v;
+            const bool ok = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+            lds[e] = buf_ld1(rs_x, ok ? (uint32_t)(((b * g.H + iy) * g.W + ix0) * C + q) * 4u : BUF_OOB);
         }
         __syncthreads();
         const int oy = oy0 + slot;
@@ -551,6 +556,10 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
     const int tid = threadIdx.x, f = tid & 31, slot = tid >> 5;
     const bool f_on = f < F;
     for (int t = tid; t < KC * F; t += 256) wl[t] = w[t];
+    // whole-tensor buffer descriptors (the launcher guarantees they are smaller than 2 GiB)
+    const int64_t dy_bytes = (int64_t)g.B * g.OH * g.OW * F * 4;
+    const __amdgpu_buffer_rsrc_t rs_dy = buf_rsrc(dy, dy_bytes), rs_mask = buf_rsrc(mask ? mask : dy, mask ? dy_bytes : 0),
+                                 rs_x = buf_rsrc(x, (int64_t)g.B * g.H * g.W * C * 4);
     float wacc[KC], bacc = 0.f;
 #pragma unroll
     for (int t = 0; t < KC; ++t) wacc[t] = 0.f;
@@ -560,8 +569,8 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
         const int iy0 = (rem / tiles_x) * SC_TH, ix0 = (rem % tiles_x) * SC_TW;
         const int oy0 = iy0 + g.py - (KH - 1), ox0 = ix0 + g.px - (KW - 1);
         __syncthreads();
+        // buffer loads (zeros outside the tensor, no branch around a load): all units of a batch are in flight together
         if (vec) {
-            // 128-bit loads, four units (dz and mask) in flight per thread
             const int upr = PW * F / 4, n_u = PH * upr;
             for (int e0 = 0; e0 < n_u; e0 += 4 * 256) {
                 f32x4_t v[4], m[4];
@@ -569,23 +578,22 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int e = e0 + u * 256 + tid;
-                    v[u] = f32x4_t{0.f, 0.f, 0.f, 0.f}, m[u] = f32x4_t{1.f, 1.f, 1.f, 1.f}, dst[u] = -1;
+                    uint32_t off = BUF_OOB;
+                    dst[u] = -1;
                     if (e < n_u) {
                         const int pr = e / upr, q = (e - pr * upr) * 4, pc = q / F, f0 = q - pc * F;
                         const int oy = oy0 + pr, ox = ox0 + pc;
                         dst[u] = (pr * PW + pc) * FS + f0;
-                        if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) {
-                            const int64_t a = (((int64_t)b * g.OH + oy) * g.OW + ox) * F + f0;
-                            v[u] = *(const f32x4_t *)(dy + a);
-                            if (mask) m[u] = *(const f32x4_t *)(mask + a);
-                        }
+                        if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) off = (uint32_t)(((b * g.OH + oy) * g.OW + ox) * F + f0) * 4u;
                     }
+                    v[u] = buf_ld4(rs_dy, off);
+                    m[u] = buf_ld4(rs_mask, off);
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     if (dst[u] >= 0) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) zp[dst[u] + j] = m[u][j] > 0.f ? v[u][j] : 0.f;
+                        for (int j = 0; j < 4; ++j) zp[dst[u] + j] = (!mask || m[u][j] > 0.f) ? v[u][j] : 0.f;
                     }
                 }
             }
@@ -597,29 +605,27 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     const int e = e0 + u * 256 + tid;
-                    v[u] = 0.f, m[u] = 1.f, dst[u] = -1;
+                    uint32_t off = BUF_OOB;
+                    dst[u] = -1;
                     if (e < n_u) {
                         const int pr = e / upr, q = e - pr * upr, pc = q / F, f0 = q - pc * F;
                         const int oy = oy0 + pr, ox = ox0 + pc;
                         dst[u] = (pr * PW + pc) * FS + f0;
-                        if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) {
-                            const int64_t a = (((int64_t)b * g.OH + oy) * g.OW + ox) * F + f0;
-                            v[u] = dy[a];
-                            if (mask) m[u] = mask[a];
-                        }
+                        if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) off = (uint32_t)(((b * g.OH + oy) * g.OW + ox) * F + f0) * 4u;
                     }
+                    v[u] = buf_ld1(rs_dy, off);
+                    m[u] = buf_ld1(rs_mask, off);
                 }
 #pragma unroll
                 for (int u = 0; u < 8; ++u)
-                    if (dst[u] >= 0) zp[dst[u]] = m[u] > 0.f ? v[u] : 0.f;
+                    if (dst[u] >= 0) zp[dst[u]] = (!mask || m[u] > 0.f) ? v[u] : 0.f;
             }
         }
         if (part) {
             for (int e = tid; e < XH * XW * C; e += 256) {
                 const int r = e / (XW * C), q = e - r * XW * C, iy = iy0 - g.py + r, ix = ix0 - g.px + q / C;
-                float v = 0.f;
-                if ((unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W) v = x[(((int64_t)b * g.H + iy) * g.W + ix) * C + q % C];
-                xp[e] = v;
+                const bool ok = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
+                xp[e] = buf_ld1(rs_x, ok ? (uint32_t)(((b * g.H + iy) * g.W + ix) * C + q % C) * 4u : BUF_OOB);
             }
         }
         __syncthreads();
@@ -812,6 +818,9 @@ __global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict_
     const int aq = tid % AQ, ar = tid / AQ, zq = tid % ZQ, zr = tid / ZQ;
     const ColInfo ci = decode_col<0>(k0 + 4 * aq, K, g, F);
     const bool z_on = n0 + 4 * zq < F, relu = act == HGQ_ACT_RELU;
+    // whole-tensor buffer descriptors (the launcher guarantees they are smaller than 2 GiB)
+    const __amdgpu_buffer_rsrc_t rs_src = buf_rsrc(src, (int64_t)g.B * g.H * g.W * g.C * 4), rs_dy = buf_rsrc(dy, rows * F * 4),
+                                 rs_y = buf_rsrc(relu ? y : dy, relu ? rows * F * 4 : 0);
     floatx16 acc = {0};
     f32x4_t bsum = {0.f, 0.f, 0.f, 0.f};
     f32x4_t av[AP], zv[ZP], zm[ZP];
@@ -820,17 +829,14 @@ __global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict_
         for (int p = 0; p < AP; ++p) {
             const int64_t m = m0 + ar + AR * p;
             const RowInfo ri = decode_row<0>(m < m_end ? m : rows, rows, g);
-            f32x4_t unused;
-            gather4<0>(src, nullptr, ri, ci, g, F, av[p], unused);
+            av[p] = buf_ld4(rs_src, gather4_offset<0>(ri, ci, g, F));
         }
 #pragma unroll
         for (int p = 0; p < ZP; ++p) {
             const int64_t m = m0 + zr + ZR * p;
-            zv[p] = f32x4_t{0.f, 0.f, 0.f, 0.f}, zm[p] = f32x4_t{1.f, 1.f, 1.f, 1.f};
-            if (m < m_end && z_on) {
-                zv[p] = *(const f32x4_t *)(dy + m * F + n0 + 4 * zq);
-                if (relu) zm[p] = *(const f32x4_t *)(y + m * F + n0 + 4 * zq);
-            }
+            const uint32_t off = (m < m_end && z_on) ? (uint32_t)(m * F + n0 + 4 * zq) * 4u : BUF_OOB;
+            zv[p] = buf_ld4(rs_dy, off);
+            zm[p] = buf_ld4(rs_y, off);
         }
     };
     auto stash = [&](int buf) {
@@ -841,7 +847,7 @@ __global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict_
             f32x4_t v = zv[p];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                if (!(zm[p][j] > 0.f)) v[j] = 0.f;
+                if (relu && !(zm[p][j] > 0.f)) v[j] = 0.f;
             bsum += v;
             *(f32x4_t *)&zs[buf][zr + ZR * p][4 * zq] = v;
         }
@@ -1053,7 +1059,9 @@ static size_t fwd_smallc_lds(const hgq_conv_geom &g) {
     const size_t XH = (size_t)(SC_TH - 1) * g.sy + (size_t)(g.kh - 1) * g.dly + 1, XW = (size_t)(SC_TW - 1) * g.sx + (size_t)(g.kw - 1) * g.dlx + 1;
     return XH * XW * g.C * sizeof(float);
 }
-static bool fwd_smallc_ok(const hgq_conv_geom &g, int F) { return smallc_shape(g, F) && fwd_smallc_lds(g) <= 48 * 1024; }
+static bool fwd_smallc_ok(const hgq_conv_geom &g, int F) {
+    return smallc_shape(g, F) && fwd_smallc_lds(g) <= 48 * 1024 && (int64_t)g.B * g.H * g.W * g.C * 4 < (1ll << 31);
+}
 static size_t bwd_smallc_lds(const hgq_conv_geom &g, int F) {
     const size_t KC = (size_t)g.kh * g.kw * g.C, PH = SC_TH + g.kh - 1, PW = SC_TW + g.kw - 1;
     size_t zp = PH * PW * (F + 1), red = SC_TH * (KC + 1) * 32;
@@ -1062,7 +1070,8 @@ static size_t bwd_smallc_lds(const hgq_conv_geom &g, int F) {
 }
 static bool bwd_smallc_ok(const hgq_conv_geom &g, int F) {
     return smallc_shape(g, F) && g.sy == 1 && g.sx == 1 && g.dly == 1 && g.dlx == 1 && g.py < g.kh && g.px < g.kw &&
-           bwd_smallc_lds(g, F) <= 64 * 1024;
+           bwd_smallc_lds(g, F) <= 64 * 1024 && (int64_t)g.B * g.OH * g.OW * F * 4 < (1ll << 31) &&
+           (int64_t)g.B * g.H * g.W * g.C * 4 < (1ll << 31);
 }
 static int bwd_smallc_grid(const hgq_conv_geom &g) {
     const int64_t tiles = (int64_t)g.B * ((g.H + SC_TH - 1) / SC_TH) * ((g.W + SC_TW - 1) / SC_TW);
@@ -1124,7 +1133,7 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
 #undef HGQ_FWD_SC
         return check_launch("hgq_conv2d_fwd(few channels)");
     }
-    const bool vec = g->C % 4 == 0 && aligned16(xq);
+    const bool vec = g->C % 4 == 0 && aligned16(xq) && (int64_t)g->B * g->H * g->W * g->C * 4 < (1ll << 31);
     if (F <= 32) {
         const dim3 grid((unsigned)persistent_grid((rows + 127) / 128, vec ? 3 : 8), 1, (unsigned)nz);
         launch_igemm<0>(vec, false, grid, s, xq, nullptr, qw, qb, dst, *g, F, rows, K, F, act, kchunk);
@@ -1207,7 +1216,7 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
             else HGQ_DG(64);
 #undef HGQ_DG
         } else {
-            const bool vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask));
+            const bool vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask)) && rows * F * 4 < (1ll << 31);
             if (g->C <= 32) {
                 const dim3 grid((unsigned)persistent_grid((in_rows + 127) / 128, vec ? 3 : 8), 1);
                 launch_igemm<1>(vec, false, grid, s, dy, mask, qw, nullptr, dxq, *g, F, in_rows, Kt, g->C, act, Kt);
@@ -1225,7 +1234,8 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
         int64_t chunk = (rows + splits - 1) / splits;
         chunk = (chunk + 127) / 128 * 128;
         const dim3 grid((unsigned)(c.n_kt * c.n_nt), (unsigned)splits);
-        const bool vec = g->C % 4 == 0 && F % 4 == 0 && aligned16(xq) && aligned16(dy) && (!mask || aligned16(mask));
+        const bool vec = g->C % 4 == 0 && F % 4 == 0 && aligned16(xq) && aligned16(dy) && (!mask || aligned16(mask)) &&
+                         rows * F * 4 < (1ll << 31) && in_rows * g->C * 4 < (1ll << 31);
 #define HGQ_WGRAD(WK, WN, WS) \
     do { \
         if (vec) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
