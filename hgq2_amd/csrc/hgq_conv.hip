@@ -945,11 +945,12 @@ static int fwd_ksplit(int64_t rows, int K, int F) {
 __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restrict__ bits_in, const float *__restrict__ bits_ker,
                                                           hgq_conv_geom g, int F, float *total,
                                                           float *__restrict__ g_in, float *__restrict__ g_ker) {
-    __shared__ float S[CE_MAX], Ws[CE_MAX], R[CE_MAXR];
+    __shared__ float S[CE_MAX], R[CE_MAXR];
+    __shared__ int Ws[CE_MAX];  // integer sums: native LDS atomics
     __shared__ float red[1024];
     __shared__ unsigned char vy[CE_MAXV], vx[CE_MAXV];  // vy[y * kh + ky]: row y is visited by kernel row ky
     const int t = threadIdx.x, taps = g.kh * g.kw, TC = taps * g.C, WC = g.W * g.C;
-    for (int e = t; e < TC; e += 1024) Ws[e] = 0.f;
+    for (int e = t; e < TC; e += 1024) Ws[e] = 0;
     for (int e = t; e < g.H * g.kh; e += 1024) {
         const int y = e / g.kh, ky = e - y * g.kh, ty = y + g.py - ky * g.dly;
         vy[e] = ty >= 0 && ty % g.sy == 0 && ty / g.sy < g.OH;
@@ -990,7 +991,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int e = e0 + u * 1024 + t;
-            if (e < n_w) atomicAdd(&Ws[e / F], v[u]);
+            if (e < n_w) atomicAdd(&Ws[e / F], (int)v[u]);
         }
     }
     for (int e = t; e < TC; e += 1024) {
@@ -1004,7 +1005,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
     }
     __syncthreads();
     float part = 0.f;
-    for (int e = t; e < TC; e += 1024) part += S[e] * Ws[e];
+    for (int e = t; e < TC; e += 1024) part += S[e] * (float)Ws[e];
     red[t] = part;
     __syncthreads();
     for (int o = 512; o > 0; o >>= 1) {
@@ -1021,7 +1022,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
             for (int ky = 0; ky < g.kh; ++ky) {
                 if (!vy[y * g.kh + ky]) continue;
                 for (int kx = 0; kx < g.kw; ++kx)
-                    if (vx[x * g.kw + kx]) a += Ws[(ky * g.kw + kx) * g.C + c];
+                    if (vx[x * g.kw + kx]) a += (float)Ws[(ky * g.kw + kx) * g.C + c];
             }
             g_in[e] = a;
         }

@@ -50,8 +50,8 @@ __device__ __forceinline__ float block_sum_ebops(float v, float *scratch16) {
     return s;
 }
 
-// One workgroup of 1024 threads.  Bit-widths are integers, so the per-row / per-column sums are exact
-// in fp32 in any order and are accumulated with LDS atomics over flat, coalesced sweeps.
+// One workgroup of 1024 threads.  Bit-widths are integers, so the per-row / per-column sums are
+// accumulated with integer LDS atomics over flat, coalesced sweeps (exact in any order).
 __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_t *amax_part, int n_parts, float decay,
                                                           const float *beta, float *loss_term,
                                                           const void *k_in, float *i_in, const float *f_in,
@@ -61,15 +61,16 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_
                                                           float *ebops, uint32_t *ebops_u32, float *g_f_in,
                                                           float *g_b_ker, float *g_b_bias) {
     constexpr int NT = HGQ_EBOPS_NT;
-    __shared__ float colsum[HGQ_EBOPS_MAXK];  // sum_n bits_ker[k, n]
-    __shared__ float insum[HGQ_EBOPS_MAXK];   // sum_p bits_in[p, k]
+    // bit-widths are integers: the sums are accumulated with native integer LDS atomics
+    __shared__ int colsum[HGQ_EBOPS_MAXK];  // sum_n bits_ker[k, n]
+    __shared__ int insum[HGQ_EBOPS_MAXK];   // sum_p bits_in[p, k]
     __shared__ float red[NT / 64];
     const Mode mi(mode_in), mk(mode_ker), mb(mode_bias);
     const int t = threadIdx.x;
     // with beta the gradients are those of the loss term ebops * beta
     const float gscale = beta ? scale * beta[0] : scale;
     const int64_t PK = P * K;
-    for (int k = t; k < K; k += NT) colsum[k] = 0.0f, insum[k] = 0.0f;
+    for (int k = t; k < K; k += NT) colsum[k] = 0, insum[k] = 0;
     if (amax_part) {
         // integer-bit tracking of the (KIF, WRAP, training) input quantizer, before its bits are read:
         // _i <- max(_i - decay, ceil(log2(max|x_q| + 2**-f)))
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int64_t e = e0 + u * NT + t;
-            if (e < KN) atomicAdd(&colsum[e / N], b[u]);
+            if (e < KN) atomicAdd(&colsum[e / N], (int)b[u]);
         }
     }
     __syncthreads();
@@ -128,15 +129,15 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_
         float d;
         const int k = (int)(e % K);
         const float b = entry_bits(k_in, i_in, f_in, e, mi, d);
-        atomicAdd(&insum[k], b);
-        if (g_f_in) g_f_in[e] = d * colsum[k] * gscale;
+        atomicAdd(&insum[k], (int)b);
+        if (g_f_in) g_f_in[e] = d * (float)colsum[k] * gscale;
     }
     __syncthreads();
     float part = 0.0f;
-    for (int k = t; k < K; k += NT) part += insum[k] * colsum[k];
+    for (int k = t; k < K; k += NT) part += (float)insum[k] * (float)colsum[k];
     float total = block_sum_ebops(part, red);
     if (g_b_ker)
-        for (int64_t e = t; e < KN; e += NT) g_b_ker[e] = insum[e / N] * gscale;
+        for (int64_t e = t; e < KN; e += NT) g_b_ker[e] = (float)insum[e / N] * gscale;
     if (b_bias) {
         float bs = 0.0f, d;
         for (int n = t; n < N; n += NT) {
