@@ -1134,6 +1134,7 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
 #undef HGQ_FWD_SC
         return check_launch("hgq_conv2d_fwd(few channels)");
     }
+    if (nz == 1 && aligned16(xq) && conv_patch_ok(0, *g, F)) return conv_patch_launch(0, xq, nullptr, qw, qb, y, *g, F, act, s);
     const bool vec = g->C % 4 == 0 && aligned16(xq) && (int64_t)g->B * g->H * g->W * g->C * 4 < (1ll << 31);
     if (F <= 32) {
         const dim3 grid((unsigned)persistent_grid((rows + 127) / 128, vec ? 3 : 8), 1, (unsigned)nz);
@@ -1216,6 +1217,8 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
             else if (fp == 32) HGQ_DG(32);
             else HGQ_DG(64);
 #undef HGQ_DG
+        } else if (aligned16(dy) && (!mask || aligned16(mask)) && conv_patch_ok(1, *g, F)) {
+            if ((rc = conv_patch_launch(1, dy, mask, qw, nullptr, dxq, *g, F, act, s))) return rc;
         } else {
             const bool vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask)) && rows * F * 4 < (1ll << 31);
             if (g->C <= 32) {

@@ -490,10 +490,21 @@ __global__ __launch_bounds__(256) void qdense_bwd_fast_kernel(const float *__res
     float *my_dw = part + (int64_t)blockIdx.x * M;
     float *my_db = my_dw + (int64_t)K * N;
     float *my_df = my_db + N;
-    for (int id = tid; id < 64 * 64; id += 256) {
-        const int kk = id >> 6, nn = id & 63;
-        ws[kk][nn] = (kk < K && nn < N) ? qw[(int64_t)kk * N + nn] : 0.f;
-        xs[kk][nn] = 0.f, dzs[kk][nn] = 0.f;
+    {
+        // all 16 kernel-matrix loads of a thread in flight (one per loop trip would cost a memory latency each)
+        const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(qw, (int64_t)K * N * 4);
+        float wv[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
+            wv[u] = buf_ld1(rs_w, (kk < K && nn < N) ? (uint32_t)(kk * N + nn) * 4u : BUF_OOB);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
+            ws[kk][nn] = wv[u];
+            xs[kk][nn] = 0.f, dzs[kk][nn] = 0.f;
+        }
     }
     FastMap mx, mz;
     mx.init(K), mz.init(N);

@@ -49,4 +49,9 @@ inline int fill_f32(float *p, float v, int64_t n, hipStream_t s) {
 int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb, float *df,
                  int64_t n_df, hipStream_t s);
 
+// Convolution through LDS-resident operands (hgq_conv_patch.hip): mode 0 forward, 1 data gradient.
+bool conv_patch_ok(int mode, const hgq_conv_geom &g, int F);
+int conv_patch_launch(int mode, const float *src, const float *mask, const float *w, const float *bias, float *out,
+                      const hgq_conv_geom &g, int F, int act, hipStream_t s);
+
 }  // namespace hgq

@@ -46,6 +46,9 @@ CASES = [
     (4, 17, 33, 1, 5, 5, 7, (1, 1), 'same', (1, 1), True, False),              # 5 x 5 on one channel, scalar staging
     (2, 20, 45, 1, 3, 3, 12, (2, 1), 'valid', (2, 3), True, True),             # few channels forward with stride and dilation
     (900, 9, 34, 2, 3, 3, 8, (1, 1), 'same', (1, 1), True, True),              # more pixel tiles than workgroups
+    (3, 14, 9, 8, 3, 3, 16, (1, 1), 'same', (2, 1), True, True),               # LDS-resident operands: dilation and padding both ways
+    (2, 20, 70, 8, 3, 3, 12, (1, 1), 'same', (1, 1), True, True),              # ... several pixel tiles along x and y
+    (2, 40, 12, 16, 5, 2, 32, (2, 1), 'valid', (1, 1), False, True),           # ... stride in the forward, 5 x 2 kernel
 ]
 
 
