@@ -19,9 +19,38 @@ namespace hgq {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 #define MLP_BM 64
+#define MLP_NT 512  // eight wavefronts: two per SIMD, so the chains of one hide the latencies of the other
 #define MLP_LDZ 65
 
 __device__ __forceinline__ int acc_row_(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
+
+// acc += sum over 16 * n_batches contraction steps of A * B on the matrix cores, A at ap[k * sa],
+// B at bp[k * sb] (k even; the lane's k parity is already folded into ap / bp).  The sixteen LDS
+// operands of a batch of eight instructions are read together, and the next batch's reads are
+// issued before the current batch's instructions, so a workgroup that is alone on its CU pays one
+// LDS latency per chain instead of one per instruction.  n_batches <= 4 (contractions up to 64).
+__device__ __forceinline__ floatx16 mfma_chain(floatx16 acc, const float *ap, int sa, const float *bp, int sb, int n_batches) {
+    float a[8], b[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a[u] = ap[2 * u * sa], b[u] = bp[2 * u * sb];
+#pragma unroll
+    for (int bt = 0; bt < 4; ++bt) {
+        if (bt < n_batches) {
+            float an[8], bn[8];
+            if (bt + 1 < n_batches) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) an[u] = ap[(16 * (bt + 1) + 2 * u) * sa], bn[u] = bp[(16 * (bt + 1) + 2 * u) * sb];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+            if (bt + 1 < n_batches) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) a[u] = an[u], b[u] = bn[u];
+            }
+        }
+    }
+    return acc;
+}
 
 struct MlpLayerDev {
     hgq_mlp_layer h;
@@ -77,7 +106,7 @@ __global__ __launch_bounds__(256) void mlp_prep_kernel(MlpDev d, float *__restri
     img[e] = v;
 }
 
-__global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ img, const float *__restrict__ x,
+__global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ img, const float *__restrict__ x,
                                                           const int64_t *__restrict__ labels, int64_t rows,
                                                           float *part) {
     extern __shared__ float lds[];
@@ -91,9 +120,22 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
     const float inv_rows = 1.0f / (float)rows;
 
     // ---- prologue: fetch the quantized kernels / biases / rounded fractional bits (off_raw is a multiple of 4)
-    for (int id = tid * 4; id < d.off_raw; id += 4 * 256) *(float4 *)(lds + id) = *(const float4 *)(img + id);
-    for (int id = tid; id < MLP_BM * d.ld_rx; id += 256) rx[id] = 0.f;  // padding columns stay zero for good
-    for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += 256) dfs[id] = 0.f, amx[id] = 0u;
+    // (four 128-bit loads per thread in flight: one load per loop trip would cost a memory latency each)
+    for (int id0 = 0; id0 < d.off_raw; id0 += 4 * 4 * MLP_NT) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int id = id0 + (u * MLP_NT + tid) * 4;
+            v[u] = *(const float4 *)(img + (id < d.off_raw ? id : 0));
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int id = id0 + (u * MLP_NT + tid) * 4;
+            if (id < d.off_raw) *(float4 *)(lds + id) = v[u];
+        }
+    }
+    for (int id = tid; id < MLP_BM * d.ld_rx; id += MLP_NT) rx[id] = 0.f;  // padding columns stay zero for good
+    for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += MLP_NT) dfs[id] = 0.f, amx[id] = 0u;
     __syncthreads();
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -104,17 +146,31 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
             const MlpLayerDev &l0 = d.l[0];
             const int K0 = l0.h.K, rm = Mode(l0.h.mode_in).round_mode;
             const float *fl = lds + l0.off_f;
-            for (int id = tid; id < MLP_BM * K0; id += 256) {
-                const int row = id / K0, k = id - row * K0;
-                const int64_t gr = r0 + row;
-                float v = 0.f, q = 0.f;
-                if (gr < rows) {
-                    v = x[gr * K0 + k];
-                    q = fixed_round_dyn(v, fl[k], rm);
-                    atomicMax(&amx[k], abs_bits(q));
+            // the tile's rows are contiguous in x: buffer loads, zeros past the last row, four in flight
+            const int64_t left = rows - r0;
+            const int n_el = MLP_BM * K0;
+            const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K0, (left < MLP_BM ? left : MLP_BM) * K0 * 4);
+            for (int id0 = 0; id0 < n_el; id0 += 4 * MLP_NT) {
+                float v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int id = id0 + u * MLP_NT + tid;
+                    v[u] = buf_ld1(rs, id < n_el ? (uint32_t)id * 4u : BUF_OOB);
                 }
-                raw[row * d.ld_raw + l0.acol + k] = v;
-                rx[row * d.ld_rx + l0.acol + k] = q;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int id = id0 + u * MLP_NT + tid;
+                    if (id < n_el) {
+                        const int row = id / K0, k = id - row * K0;
+                        float q = 0.f;
+                        if (r0 + row < rows) {
+                            q = fixed_round_dyn(v[u], fl[k], rm);
+                            atomicMax(&amx[k], abs_bits(q));
+                        }
+                        raw[row * d.ld_raw + l0.acol + k] = v[u];
+                        rx[row * d.ld_rx + l0.acol + k] = q;
+                    }
+                }
             }
         }
         __syncthreads();
@@ -123,13 +179,12 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
             const MlpLayerDev &ly = d.l[l];
             const int N = ly.h.N;
             const int rh = wave & 1, cb = wave >> 1;
-            if (cb * 32 < ly.Np) {
+            if (wave < 4 && cb * 32 < ly.Np) {
                 floatx16 acc = {0};
                 const float *ws = lds + ly.off_w;
                 const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
-                const int ksteps = (ly.h.K + 1) & ~1;
-                for (int kk = 0; kk < ksteps; kk += 2)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(rx[arow * d.ld_rx + ly.acol + kk + kq], ws[(kk + kq) * ly.ldw + bcol], acc, 0, 0, 0);
+                // input columns and kernel rows are zero padded to a multiple of 32
+                acc = mfma_chain(acc, rx + arow * d.ld_rx + ly.acol + kq, 1, ws + kq * ly.ldw + bcol, ly.ldw, (ly.h.K + 15) >> 4);
                 if (bcol < N) {
                     const float bias = lds[ly.off_qb + bcol];
                     const bool last = l + 1 == L;
@@ -199,14 +254,14 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
             const int K = ly.h.K, N = ly.h.N;
             const int K32 = ly.Kp >> 5, N32 = ly.Np >> 5;
             const int nblk = K32 * N32;
-            // ---- kernel gradient: one 32 x 32 block per wave over the whole tile
-            if (wave < nblk) {
-                const int wkb = wave / N32, wnb = wave % N32;
+            // ---- kernel gradient: one 32 x 32 block per wave over the whole tile, on waves 4 .. 7
+            // (waves 0 .. 3 work on the input gradient at the same time)
+            if (wave >= 4 && wave - 4 < nblk) {
+                const int wkb = (wave - 4) / N32, wnb = (wave - 4) % N32;
                 floatx16 acc = {0};
                 const int kq = lane >> 5, c32 = lane & 31;
-                for (int rr = 0; rr < MLP_BM; rr += 2)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(rx[(rr + kq) * d.ld_rx + ly.acol + wkb * 32 + c32],
-                                                               cur[(rr + kq) * MLP_LDZ + wnb * 32 + c32], acc, 0, 0, 0);
+                acc = mfma_chain(acc, rx + kq * d.ld_rx + ly.acol + wkb * 32 + c32, d.ld_rx, cur + kq * MLP_LDZ + wnb * 32 + c32, MLP_LDZ,
+                                 MLP_BM / 16);
                 const int n = wnb * 32 + c32;
                 if (n < N) {
 #pragma unroll
@@ -220,7 +275,7 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
                 }
             }
             // ---- bias gradient: the last wave is free of kernel-gradient work unless all four blocks exist
-            if (ly.h.bias && wave == 3 && lane < N) {
+            if (ly.h.bias && wave == 7 && lane < N) {
                 float s0 = 0.f, s1 = 0.f;
 #pragma unroll 8
                 for (int r = 0; r < MLP_BM; r += 2) s0 += cur[r * MLP_LDZ + lane], s1 += cur[(r + 1) * MLP_LDZ + lane];
@@ -230,13 +285,12 @@ __global__ __launch_bounds__(256) void mlp_fwd_bwd_kernel(MlpDev d, const float 
             // ---- input gradient, the relu mask of the layer below, and this layer's fractional-bit gradient
             {
                 const int rh = wave & 1, kb = wave >> 1;
-                if (kb < K32) {
+                if (wave < 4 && kb < K32) {
                     floatx16 acc = {0};
                     const float *ws = lds + ly.off_w;
                     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
-                    const int nsteps = (N + 1) & ~1;
-                    for (int nn = 0; nn < nsteps; nn += 2)
-                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(cur[arow * MLP_LDZ + nn + kq], ws[wrow * ly.ldw + nn + kq], acc, 0, 0, 0);
+                    // gradient columns and kernel columns are zero padded to a multiple of 32
+                    acc = mfma_chain(acc, cur + arow * MLP_LDZ + kq, 1, ws + wrow * ly.ldw + kq, 1, (N + 15) >> 4);
                     const int kcol = kb * 32 + (lane & 31);
                     const bool mask_below = l > 0 && d.l[l - 1].h.act == HGQ_ACT_RELU;
                     float dfsum = 0.f;
@@ -509,7 +563,7 @@ extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, con
     img += (4 - ((uintptr_t)img / 4) % 4) % 4;  // 16-byte aligned
     hipLaunchKernelGGL(mlp_prep_kernel, dim3((d.off_raw + 255) / 256), dim3(256), 0, s, d, img);
     if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
-    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(256), lds_bytes, s, d, img, x, labels, rows, workspace);
+    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, workspace);
     if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
     hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(256), 0, s, d, workspace, parts, reduced, loss);
     if ((rc = check_launch("hgq_mlp_train_step(reduce)"))) return rc;
