@@ -329,12 +329,13 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
 // quantizer's integer bits in place, and leave for the update pass - which must not read variables
 // another workgroup is updating - the per-feature bit counts of the input quantizer and the
 // per-row sums of the kernel bit counts, all from the pre-update variables.
-__global__ __launch_bounds__(256) void mlp_reduce_kernel(MlpDev d, const float *__restrict__ part, int n_parts, float *out,
+#define MLP_RG 16  // slice groups per entry: 64 entries x 16 groups = 1024 threads, few loads per thread
+__global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_kernel(MlpDev d, const float *__restrict__ part, int n_parts, float *out,
                                                          float *loss) {
-    __shared__ float red[256];
+    __shared__ float red[64 * MLP_RG];
     const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int n_main = (d.M + 63) / 64;
-    const int per = (n_parts + 3) / 4;
+    const int per = (n_parts + MLP_RG - 1) / MLP_RG;
     const int g0 = grp * per, g1 = min(n_parts, g0 + per);
     if ((int)blockIdx.x < n_main) {
         const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
@@ -352,7 +353,10 @@ __global__ __launch_bounds__(256) void mlp_reduce_kernel(MlpDev d, const float *
         red[threadIdx.x] = s;
         __syncthreads();
         if (grp == 0 && e < d.M) {
-            const float v = (red[e_local] + red[e_local + 64]) + (red[e_local + 128] + red[e_local + 192]);
+            float v = 0.f;  // groups in order
+#pragma unroll
+            for (int w = 0; w < MLP_RG; w += 4)
+                v += (red[e_local + 64 * w] + red[e_local + 64 * (w + 1)]) + (red[e_local + 64 * (w + 2)] + red[e_local + 64 * (w + 3)]);
             out[e] = v;
             if (e == d.p_loss && loss) loss[0] = v;
         }
@@ -376,20 +380,20 @@ __global__ __launch_bounds__(256) void mlp_reduce_kernel(MlpDev d, const float *
             for (int u = 0; u < 8; ++u) mx = max(mx, v[u]);
         }
         for (; g < g1; ++g) mx = max(mx, pa[(int64_t)g * d.M]);
-        // this thread's quarter of row k of the kernel bit counts
-        const int nper = (N + 3) / 4, n0 = grp * nper, n1 = min(N, n0 + nper);
+        // this thread's share of row k of the kernel bit counts
+        const int nper = (N + MLP_RG - 1) / MLP_RG, n0 = grp * nper, n1 = min(N, n0 + nper);
         for (int n = n0; n < n1; ++n) {
             float bk = rintf(h.b_ker[k * N + n]);
             if (mk.overflow_mode == HGQ_SAT) bk += load_k(h.k_ker, k * N + n, mk.k_u8);
             cs += bk;
         }
     }
-    __shared__ uint32_t smx[256];
+    __shared__ uint32_t smx[64 * MLP_RG];
     smx[threadIdx.x] = mx;
     red[threadIdx.x] = cs;
     __syncthreads();
     if (grp == 0 && k < K) {
-        for (int w = 1; w < 4; ++w) mx = max(mx, smx[k + 64 * w]);
+        for (int w = 1; w < MLP_RG; ++w) mx = max(mx, smx[k + 64 * w]);
         const float f = rintf(h.f_in[k]);
         const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-f)));
         const float ni = fmaxf(__fsub_rn(h.i_in[k], h.decay), mi_);
@@ -398,7 +402,9 @@ __global__ __launch_bounds__(256) void mlp_reduce_kernel(MlpDev d, const float *
         float b = sfi > 0.f ? sfi : 0.f;
         if (mi.overflow_mode == HGQ_SAT) b += load_k(h.k_in, k, mi.k_u8);
         float *aux = out + d.M + l * MLP_AUX;
-        aux[k] = (red[k] + red[k + 64]) + (red[k + 128] + red[k + 192]);
+        float csum = 0.f;  // integers: exact in any order
+        for (int w = 0; w < MLP_RG; ++w) csum += red[k + 64 * w];
+        aux[k] = csum;
         aux[64 + k] = b;
         aux[128 + k] = sfi > 0.f ? 1.f : 0.f;
     }
@@ -565,7 +571,7 @@ extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, con
     if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
     hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, workspace);
     if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
-    hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(256), 0, s, d, workspace, parts, reduced, loss);
+    hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(64 * MLP_RG), 0, s, d, workspace, parts, reduced, loss);
     if ((rc = check_launch("hgq_mlp_train_step(reduce)"))) return rc;
     hipLaunchKernelGGL(mlp_update_kernel, dim3(n_layers, MLP_UPD_SPLIT), dim3(256), 0, s, d, reduced, lr, loss);
     return check_launch("hgq_mlp_train_step(update)");
