@@ -17,7 +17,6 @@
 
 namespace hgq {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f32x4_a __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ int at_acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }

@@ -20,7 +20,6 @@
 
 namespace hgq {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 #define CV_BK 32
 

@@ -21,7 +21,6 @@
 
 namespace hgq {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define PG_WS 33  // row stride of the kernel matrix in LDS
 
 __device__ __forceinline__ int pg_acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }

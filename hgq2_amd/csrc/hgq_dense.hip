@@ -18,7 +18,6 @@
 
 namespace hgq {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 #define FWD_BM 64
 #define FWD_BK 32
@@ -263,8 +262,7 @@ __global__ __launch_bounds__(256) void qdense_bwd_kernel(const float *__restrict
         {
             const int rbeg = sub * rows_per;
             const int kq = lane >> 5, c32 = lane & 31;
-            for (int rr = rbeg; rr < rbeg + rows_per; rr += 2)
-                accw = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[rr + kq][wkb * 32 + c32], dzs[rr + kq][wnb * 32 + c32], accw, 0, 0, 0);
+            accw = mfma_chain(accw, &xs[rbeg + kq][wkb * 32 + c32], BWD_LD, &dzs[rbeg + kq][wnb * 32 + c32], BWD_LD, rows_per / 16);
         }
         // ---- bias gradient partial sums
         if (has_bias) {
@@ -583,16 +581,13 @@ __global__ __launch_bounds__(256) void qdense_bwd_fast_kernel(const float *__res
         const int rh = wave & 1, kb = wave >> 1;
         if (kb < K32) {
             const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
-            const int nsteps = N32 * 32;
-            for (int nn = 0; nn < nsteps; nn += 2)
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(dzs[arow][nn + kq], ws[wrow][nn + kq], acc, 0, 0, 0);
+            acc = mfma_chain(acc, &dzs[arow][kq], 1, &ws[wrow][kq], 1, N32 * 2);
         }
         // ---- dW += xq^T @ dz : this wave's block, its slice of the tile's rows
         {
             const int rbeg = sub * rows_per;
             const int kq = lane >> 5, c32 = lane & 31;
-            for (int rr = rbeg; rr < rbeg + rows_per; rr += 2)
-                accw = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[rr + kq][wkb * 32 + c32], dzs[rr + kq][wnb * 32 + c32], accw, 0, 0, 0);
+            accw = mfma_chain(accw, &xs[rbeg + kq][wkb * 32 + c32], FAST_LD, &dzs[rbeg + kq][wnb * 32 + c32], FAST_LD, rows_per / 16);
         }
         if (has_bias) {
 #pragma unroll

@@ -218,6 +218,36 @@ __device__ __forceinline__ float row_reduce_sum(float v) { return sub_reduce<SUB
 template <int SUB>
 __device__ __forceinline__ float row_reduce_max(float v) { return sub_reduce<SUB, OpMax>(v); }
 
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// acc += sum over 16 * n_batches contraction steps of A * B on the matrix cores, A at ap[k * sa],
+// B at bp[k * sb] (k even; the lane's k parity is already folded into ap / bp).  The sixteen LDS
+// operands of a batch of eight instructions are read together, and the next batch's reads are
+// issued before the current batch's instructions, so a workgroup that is alone on its CU pays one
+// LDS latency per chain instead of one per instruction.  n_batches <= 4 (contractions up to 64); longer ones chain several calls.
+__device__ __forceinline__ floatx16 mfma_chain(floatx16 acc, const float *ap, int sa, const float *bp, int sb, int n_batches) {
+    float a[8], b[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a[u] = ap[2 * u * sa], b[u] = bp[2 * u * sb];
+#pragma unroll
+    for (int bt = 0; bt < 4; ++bt) {
+        if (bt < n_batches) {
+            float an[8], bn[8];
+            if (bt + 1 < n_batches) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) an[u] = ap[(16 * (bt + 1) + 2 * u) * sa], bn[u] = bp[(16 * (bt + 1) + 2 * u) * sb];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+            if (bt + 1 < n_batches) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) a[u] = an[u], b[u] = bn[u];
+            }
+        }
+    }
+    return acc;
+}
+
 }  // namespace hgq
 
 // dispatch a (round_mode, overflow_mode) pair to template arguments
