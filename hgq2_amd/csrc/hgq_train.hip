@@ -155,6 +155,53 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_
     }
 }
 
+// Mean squared error: per-workgroup partial sums (fixed order inside a workgroup), added in order
+// by one wavefront of a second launch: the loss does not depend on scheduling.
+#define MSE_PARTS 1024
+__global__ __launch_bounds__(256) void mse_partial_kernel(const float *__restrict__ pred, const float *__restrict__ target, int64_t n,
+                                                          float *__restrict__ part) {
+    __shared__ float red[4];
+    float acc = 0.f;
+    const int64_t n4 = n >> 2, stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
+        const f32x4_t p = ((const f32x4_t *)pred)[i];
+        const f32x4_t t = target ? ((const f32x4_t *)target)[i] : f32x4_t{0.f, 0.f, 0.f, 0.f};
+        const f32x4_t d = p - t;
+        acc += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (n4 << 2) + threadIdx.x;
+        const float d = pred[i] - (target ? target[i] : 0.f);
+        acc += d * d;
+    }
+    acc = block_sum_256(acc, red);
+    if (threadIdx.x == 0) part[blockIdx.x] = acc;
+}
+
+__global__ __launch_bounds__(64) void mse_finish_kernel(const float *__restrict__ part, int n_parts, float inv_n, float *loss) {
+    float acc = 0.f;
+    for (int i = threadIdx.x; i < n_parts; i += 64) acc += part[i];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (threadIdx.x == 0) loss[0] = acc * inv_n;
+}
+
+// dpred = g * 2 (pred - target) / n, g read from device memory
+__global__ __launch_bounds__(256) void mse_bwd_kernel(const float *__restrict__ pred, const float *__restrict__ target,
+                                                      const float *__restrict__ g, float two_over_n, int64_t n, float *__restrict__ dpred) {
+    const float c = g[0] * two_over_n;
+    const int64_t n4 = n >> 2, stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
+        const f32x4_t p = ((const f32x4_t *)pred)[i];
+        const f32x4_t t = target ? ((const f32x4_t *)target)[i] : f32x4_t{0.f, 0.f, 0.f, 0.f};
+        ((f32x4_t *)dpred)[i] = (p - t) * c;
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+        const int64_t i = (n4 << 2) + threadIdx.x;
+        dpred[i] = (pred[i] - (target ? target[i] : 0.f)) * c;
+    }
+}
+
 // one thread per row; C is small (class count)
 __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict__ logits,
                                                         const int64_t *__restrict__ labels, float *loss,
@@ -328,6 +375,32 @@ extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels,
     const int grid = persistent_grid((rows + 255) / 256, 4);
     hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C);
     return check_launch("hgq_sparse_ce_fwd_bwd");
+}
+
+extern "C" int64_t hgq_mse_workspace(void) { return MSE_PARTS; }
+
+extern "C" int hgq_mse_fwd(const float *pred, const float *target, float *loss, float *workspace, int64_t n, void *stream) {
+    if (n < 1) return fail(HGQ_ERR_ARG, "hgq_mse_fwd: bad size");
+    if (!pred || !loss || !workspace) return fail(HGQ_ERR_ARG, "hgq_mse_fwd: null pointer");
+    if (((uintptr_t)pred & 15u) || ((uintptr_t)target & 15u)) return fail(HGQ_ERR_ARG, "hgq_mse_fwd: operands must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    int grid = persistent_grid(((n >> 2) + 255) / 256, 4);
+    if (grid > MSE_PARTS) grid = MSE_PARTS;
+    hipLaunchKernelGGL(mse_partial_kernel, dim3(grid), dim3(256), 0, s, pred, target, n, workspace);
+    int rc = check_launch("hgq_mse_fwd");
+    if (rc) return rc;
+    hipLaunchKernelGGL(mse_finish_kernel, dim3(1), dim3(64), 0, s, workspace, grid, 1.0f / (float)n, loss);
+    return check_launch("hgq_mse_fwd(finish)");
+}
+
+extern "C" int hgq_mse_bwd(const float *pred, const float *target, const float *g, float *dpred, int64_t n, void *stream) {
+    if (n < 1) return fail(HGQ_ERR_ARG, "hgq_mse_bwd: bad size");
+    if (!pred || !g || !dpred) return fail(HGQ_ERR_ARG, "hgq_mse_bwd: null pointer");
+    if (((uintptr_t)pred & 15u) || ((uintptr_t)target & 15u) || ((uintptr_t)dpred & 15u))
+        return fail(HGQ_ERR_ARG, "hgq_mse_bwd: operands must be 16-byte aligned");
+    const int grid = persistent_grid(((n >> 2) + 255) / 256, 8);
+    hipLaunchKernelGGL(mse_bwd_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, pred, target, g, 2.0f / (float)n, n, dpred);
+    return check_launch("hgq_mse_bwd");
 }
 
 extern "C" int hgq_sgd_update(float *w, const float *g, int64_t n, float lr, float l1, float lo, float hi, void *stream) {

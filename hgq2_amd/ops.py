@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse']
 
 
 def _ptr(t: Tensor | None):
@@ -561,6 +561,37 @@ def _(bits_in, bits_ker, geom):
     return bits_in.new_empty(()), torch.empty_like(bits_in), torch.empty_like(bits_ker)
 
 
+@torch.library.custom_op('hgq::mse_fwd', mutates_args=())
+def mse_fwd_op(pred: Tensor, target: Tensor) -> Tensor:
+    _check_f32('pred', pred)
+    if target.numel():
+        _check_f32('target', target)
+        _need(target.numel() == pred.numel(), 'target size mismatch')
+    lib = _lib.load()
+    loss = torch.empty((), dtype=torch.float32, device=pred.device)
+    ws = torch.empty(lib.hgq_mse_workspace(), dtype=torch.float32, device=pred.device)
+    _lib.check(lib.hgq_mse_fwd(_ptr(pred), _ptr(target), _ptr(loss), _ptr(ws), pred.numel(), _stream()), 'hgq_mse_fwd')
+    return loss
+
+
+@mse_fwd_op.register_fake
+def _(pred, target):
+    return pred.new_empty(())
+
+
+@torch.library.custom_op('hgq::mse_bwd', mutates_args=())
+def mse_bwd_op(pred: Tensor, target: Tensor, g: Tensor) -> Tensor:
+    _check_f32('pred', pred), _check_f32('g', g)
+    dpred = torch.empty_like(pred)
+    _lib.check(_lib.load().hgq_mse_bwd(_ptr(pred), _ptr(target), _ptr(g), _ptr(dpred), pred.numel(), _stream()), 'hgq_mse_bwd')
+    return dpred
+
+
+@mse_bwd_op.register_fake
+def _(pred, target, g):
+    return torch.empty_like(pred)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -900,6 +931,26 @@ class _SparseCE(torch.autograd.Function):
     def backward(ctx, g):
         (dlogits,) = ctx.saved_tensors
         return g * dlogits, None
+
+
+class _MSE(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, pred, target):
+        ctx.save_for_backward(pred, target)
+        return mse_fwd_op(pred, target)
+
+    @staticmethod
+    def backward(ctx, g):
+        pred, target = ctx.saved_tensors
+        return mse_bwd_op(pred, target, g.contiguous()), None
+
+
+def mse(pred: Tensor, target: Tensor | None = None) -> Tensor:
+    """Mean squared error ``mean((pred - target) ** 2)``; ``target=None`` means zeros."""
+    pred = pred.contiguous()
+    if pred.numel() == 0:
+        raise ValueError('mse of an empty tensor')
+    return _MSE.apply(pred, target.contiguous() if target is not None else pred.new_empty(0))
 
 
 def sparse_ce(logits: Tensor, labels: Tensor) -> Tensor:

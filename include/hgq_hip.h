@@ -162,6 +162,18 @@ int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const f
                     uint32_t *ebops_u32, float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream);
 
 /*
+ * Mean squared error, the regression loss HGQ models are trained with through Keras
+ * (`loss='mse'`; the reference has no loss code of its own).  target may be NULL (zeros).
+ *   loss [1] = mean((pred - target)^2) over n elements, summed in a fixed order;
+ *   workspace: hgq_mse_workspace() floats.
+ *   hgq_mse_bwd: dpred = g[0] * 2 (pred - target) / n with the upstream gradient g read on the device.
+ * Operands must be 16-byte aligned.
+ */
+int64_t hgq_mse_workspace(void);
+int hgq_mse_fwd(const float *pred, const float *target, float *loss, float *workspace, int64_t n, void *stream);
+int hgq_mse_bwd(const float *pred, const float *target, const float *g, float *dpred, int64_t n, void *stream);
+
+/*
  * Mean sparse categorical cross-entropy from logits, forward and gradient in one pass.
  *   logits [rows, C]; labels [rows] int64;  loss [1] = mean_r(-log softmax(logits_r)[label_r]);
  *   dlogits [rows, C] = (softmax - onehot) / rows.

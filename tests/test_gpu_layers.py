@@ -209,3 +209,26 @@ def test_trace_minmax_matches_oracle(dev):
     assert out.shape == (100, 5)
     for b, pl in zip(before, model.layers):
         assert torch.all(pl.iq.quantizer._i >= b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('n,with_target', [(1, False), (7, True), (4096 * 33 + 3, True), (2048 * 64 * 64, False)])
+def test_mse_loss_and_gradient(n, with_target):
+    """ops.mse against the fp64 definition mean((pred - target)^2) and its gradient 2 (pred - target) / n
+    scaled by the upstream gradient; run twice: the fixed summation order gives the same bits."""
+    from hgq2_amd import ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(n % 1000)
+    pred = torch.randn(n, generator=g)
+    target = torch.randn(n, generator=g) if with_target else None
+    ref_d = pred.double() - (target.double() if with_target else 0.0)
+    want = float((ref_d * ref_d).mean())
+    p = pred.to(dev).requires_grad_(True)
+    t = target.to(dev) if with_target else None
+    loss = ops.mse(p, t)
+    (loss * 3.0).backward()
+    assert abs(float(loss) - want) <= 2e-6 * abs(want) + 1e-12
+    want_g = 3.0 * 2.0 * ref_d / n
+    assert float((p.grad.cpu().double() - want_g).abs().max()) <= 2e-6 * float(want_g.abs().max())
+    assert float(ops.mse(p.detach(), t)) == float(loss)
