@@ -334,7 +334,7 @@ __device__ __forceinline__ void st4(float *p, const float4 &v) {
 // through LDS so that it leaves as full 128-bit rows.
 #define FAST_XLD 68
 template <int RM, bool QUANT, int NS4>
-__global__ __launch_bounds__(256) void qdense_fwd_fast_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
+__global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw,
                                                               const float *__restrict__ qb, float *__restrict__ y,
                                                               uint32_t *amax_part, int64_t rows, int K, int N, int act,
@@ -471,7 +471,7 @@ __global__ __launch_bounds__(256) void qdense_fwd_fast_kernel(const float *__res
 // meets the rounding residue (xq - x) of the staging thread for the fractional-bit gradient.
 // Slice blockIdx.x of `part` is [K * N | N | P * K].
 template <int RM, bool QUANT>
-__global__ __launch_bounds__(256) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
+__global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
                                                               float *part, int has_bias, int64_t rows, int K, int N, int act,
