@@ -209,11 +209,26 @@ __global__ __launch_bounds__(Q1D_BS) void quant_bwd_1d(const float *__restrict__
 // 2-D kernels: x = [rows, M], one bit-width entry per column
 // thread (tx, ty): tx walks column groups of VEC, ty walks rows; TX is a power of two <= 64
 // ------------------------------------------------------------------------------------------
+// Row batches of the per-column kernels: a thread has QC_U rows of its column group in flight
+// (buffer loads; rows past the end of the workgroup's chunk read as zero, which is neutral for
+// every reduction below), and a workgroup walks a contiguous chunk of rows so that a column sees
+// few workgroups - and few atomics - at the end.
+#define QC_U 8
+template <int VEC>
+__device__ __forceinline__ void qc_load(const __amdgpu_buffer_rsrc_t rs, uint32_t off, float *o) {
+    if (VEC == 4) {
+        const f32x4_t t = buf_ld4(rs, off);
+        o[0] = t[0], o[1 % VEC] = t[1], o[2 % VEC] = t[2], o[3 % VEC] = t[3];
+    } else {
+        o[0] = buf_ld1(rs, off);
+    }
+}
+
 template <int RM, int OM, int VEC>
 __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ x, const void *__restrict__ k,
                                                       const float *__restrict__ i, const float *__restrict__ fb,
                                                       float *__restrict__ y, uint32_t *amax, uint32_t *anyneg,
-                                                      int64_t rows, int64_t M, int TX, int mode) {
+                                                      int64_t rows, int64_t M, int TX, int64_t rows_per_wg, int mode) {
     const Mode m(mode);
     const int TY = 256 / TX;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
@@ -222,6 +237,8 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
     const bool active = c < cg;
     KIF p[VEC];
     uint32_t lmax[VEC], lneg[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) p[e] = KIF{0.f, 0.f, 0.f}, lmax[e] = 0, lneg[e] = 0;
     if (active) {
         float kv[VEC], iv[VEC], fv[VEC];
         VecIO<VEC>::load_k(k, c, m.k_u8, kv);
@@ -230,21 +247,30 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
 #pragma unroll
         for (int e = 0; e < VEC; ++e) p[e] = resolve_kif(kv[e], iv[e], fv[e], m.kbi, m.round_params);
     }
+    const int64_t row0 = (int64_t)blockIdx.y * rows_per_wg;
+    const int64_t n_rows = min(rows - row0, rows_per_wg);
+    const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + row0 * M, n_rows * M * 4);
+    float *yb = y + row0 * M;
+    for (int64_t rb = 0; rb < n_rows; rb += (int64_t)TY * QC_U) {
+        float xv[QC_U][VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) lmax[e] = 0, lneg[e] = 0;
-    if (active) {
-        for (int64_t r = (int64_t)blockIdx.y * TY + ty; r < rows; r += (int64_t)gridDim.y * TY) {
-            float xv[VEC], yv[VEC];
-            VecIO<VEC>::load(x, r * cg + c, xv);
+        for (int u = 0; u < QC_U; ++u) {
+            const int64_t r = rb + ty + (int64_t)TY * u;
+            qc_load<VEC>(rs, (active && r < n_rows) ? (uint32_t)((r * cg + c) * VEC) * 4u : BUF_OOB, xv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < QC_U; ++u) {
+            const int64_t r = rb + ty + (int64_t)TY * u;
+            float yv[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                yv[e] = quantize<RM, OM>(xv[e], p[e], m.training);
-                const float tv = m.track_input ? xv[e] : yv[e];
+                yv[e] = quantize<RM, OM>(xv[u][e], p[e], m.training);
+                const float tv = m.track_input ? xv[u][e] : yv[e];
                 const uint32_t ab = abs_bits(tv);
                 lmax[e] = ab > lmax[e] ? ab : lmax[e];
                 lneg[e] |= tv < 0.0f ? 1u : 0u;
             }
-            VecIO<VEC>::store(y, r * cg + c, yv);
+            if (active && r < n_rows) VecIO<VEC>::store(yb, r * cg + c, yv);
         }
     }
     if (amax || anyneg) {
@@ -278,7 +304,7 @@ template <int RM, int OM, int VEC>
 __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ dy, const float *__restrict__ x,
                                                       const void *__restrict__ k, const float *__restrict__ i,
                                                       const float *__restrict__ fb, float *__restrict__ dx, float *di,
-                                                      float *dfb, int64_t rows, int64_t M, int TX, int mode) {
+                                                      float *dfb, int64_t rows, int64_t M, int TX, int64_t rows_per_wg, int mode) {
     const Mode m(mode);
     const int TY = 256 / TX;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
@@ -288,7 +314,7 @@ __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ 
     KIF p[VEC];
     float si[VEC], sf[VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) si[e] = 0.0f, sf[e] = 0.0f;
+    for (int e = 0; e < VEC; ++e) p[e] = KIF{0.f, 0.f, 0.f}, si[e] = 0.0f, sf[e] = 0.0f;
     if (active) {
         float kv[VEC], iv[VEC], fv[VEC];
         VecIO<VEC>::load_k(k, c, m.k_u8, kv);
@@ -296,18 +322,33 @@ __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ 
         VecIO<VEC>::load(fb, c, fv);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) p[e] = resolve_kif(kv[e], iv[e], fv[e], m.kbi, m.round_params);
-        for (int64_t r = (int64_t)blockIdx.y * TY + ty; r < rows; r += (int64_t)gridDim.y * TY) {
-            float gv[VEC], xv[VEC], dxv[VEC];
-            VecIO<VEC>::load(dy, r * cg + c, gv);
-            VecIO<VEC>::load(x, r * cg + c, xv);
+    }
+    const int64_t row0 = (int64_t)blockIdx.y * rows_per_wg;
+    const int64_t n_rows = min(rows - row0, rows_per_wg);
+    const __amdgpu_buffer_rsrc_t rs_g = buf_rsrc(dy + row0 * M, n_rows * M * 4), rs_x = buf_rsrc(x + row0 * M, n_rows * M * 4);
+    float *dxb = dx ? dx + row0 * M : nullptr;
+    constexpr int U = QC_U / 2;  // two operands per row
+    for (int64_t rb = 0; rb < n_rows; rb += (int64_t)TY * U) {
+        float gv[U][VEC], xv[U][VEC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t r = rb + ty + (int64_t)TY * u;
+            const uint32_t off = (active && r < n_rows) ? (uint32_t)((r * cg + c) * VEC) * 4u : BUF_OOB;
+            qc_load<VEC>(rs_g, off, gv[u]);
+            qc_load<VEC>(rs_x, off, xv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t r = rb + ty + (int64_t)TY * u;
+            float dxv[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 float gi, gf;
-                quantize_grad<RM, OM>(xv[e], gv[e], p[e], dxv[e], gi, gf);
+                quantize_grad<RM, OM>(xv[u][e], gv[u][e], p[e], dxv[e], gi, gf);
                 if (m.kbi) gi -= gf;
                 si[e] += gi, sf[e] += gf;
             }
-            if (dx) VecIO<VEC>::store(dx, r * cg + c, dxv);
+            if (dxb && active && r < n_rows) VecIO<VEC>::store(dxb, r * cg + c, dxv);
         }
     }
     __shared__ float ssi[256 * VEC], ssf[256 * VEC];
@@ -464,6 +505,23 @@ extern "C" int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream
     return fill_u32(p, value, n, (hipStream_t)stream);
 }
 
+// Row split of the per-column kernels: about four workgroups per CU in total, every workgroup a
+// whole number of row batches, and a chunk below 2 GiB (one buffer descriptor per workgroup).
+static bool cols_grid(int64_t rows, int64_t M, int batch_rows, int64_t gx, int64_t &gy, int64_t &rows_per_wg) {
+    const int64_t n_batches = (rows + batch_rows - 1) / batch_rows;
+    int64_t want = (int64_t)persistent_grid(1 << 30, 4) / gx;
+    if (want < 1) want = 1;
+    gy = n_batches < want ? n_batches : want;
+    if (gy < 1) gy = 1;
+    int64_t bpw = (n_batches + gy - 1) / gy;                         // batches per workgroup
+    const int64_t max_rows = ((1ll << 31) - 1) / (M * 4);             // rows in one descriptor
+    if (max_rows < batch_rows) return false;  // absurdly wide rows: the generic kernel takes them
+    if (bpw * batch_rows > max_rows) bpw = max_rows / batch_rows;
+    rows_per_wg = bpw * batch_rows;
+    gy = (rows + rows_per_wg - 1) / rows_per_wg;
+    return true;
+}
+
 extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, const float *fb, float *y,
                                 uint32_t *amax, uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner,
                                 int mode, void *stream) {
@@ -508,21 +566,20 @@ extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, c
         });
         return check_launch("hgq_quantize_fwd");
     }
-    if (bw_inner == 1) {
+    if (bw_inner == 1 && bw_size * 4 * 256 * QC_U < (1ll << 31)) {
         const int64_t M = bw_size, rows = n / M;
         const bool vec = (M % 4 == 0) && aligned16(x) && aligned16(y) && aligned16(i) && aligned16(fb) &&
                          ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0;
         const int64_t cg = vec ? M / 4 : M;
         const int TX = pow2_floor_le64(cg), TY = 256 / TX;
         const int64_t gx = (cg + TX - 1) / TX;
-        int64_t gy = (rows + TY - 1) / TY;
-        const int64_t cap = (int64_t)persistent_grid(1 << 30, 8) / gx;
-        if (gy > cap) gy = cap < 1 ? 1 : cap;
+        int64_t gy, rows_per_wg;
+        cols_grid(rows, M, TY * QC_U, gx, gy, rows_per_wg);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (vec)
-                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, mode);
+                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode);
             else
-                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, mode);
+                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode);
         });
         return check_launch("hgq_quantize_fwd");
     }
@@ -578,21 +635,20 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
         });
         return check_launch("hgq_quantize_bwd");
     }
-    if (bw_inner == 1) {
+    if (bw_inner == 1 && bw_size * 4 * 256 * QC_U < (1ll << 31)) {
         const int64_t M = bw_size, rows = n / M;
         const bool vec = (M % 4 == 0) && aligned16(x) && aligned16(dy) && (!dx || aligned16(dx)) && aligned16(i) &&
                          aligned16(fb) && ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0;
         const int64_t cg = vec ? M / 4 : M;
         const int TX = pow2_floor_le64(cg), TY = 256 / TX;
         const int64_t gx = (cg + TX - 1) / TX;
-        int64_t gy = (rows + TY - 1) / TY;
-        const int64_t cap = (int64_t)persistent_grid(1 << 30, 8) / gx;
-        if (gy > cap) gy = cap < 1 ? 1 : cap;
+        int64_t gy, rows_per_wg;
+        cols_grid(rows, M, TY * (QC_U / 2), gx, gy, rows_per_wg);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (vec)
-                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, mode);
+                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode);
             else
-                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, mode);
+                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode);
         });
         return check_launch("hgq_quantize_bwd");
     }
