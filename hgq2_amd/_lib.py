@@ -53,6 +53,7 @@ SIGNATURES = {
     'hgq_sgd_update_multi': (c_int, [c_void_p, c_int, c_float, c_void_p]),
     'hgq_mlp_workspace': (c_int64, [c_void_p, c_int, c_int64]),
     'hgq_mlp_train_step': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p]),
+    'hgq_mlp_train_step_cached': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_float, c_void_p, c_void_p, c_int, c_void_p]),
     'hgq_fill_u32': (c_int, [c_void_p, ctypes.c_uint32, c_int64, c_void_p]),
     'hgq_qsoftmax_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int64, c_float, c_float] + [c_void_p] * 5
                          + [c_void_p] * 3 + [c_void_p]),

@@ -390,7 +390,7 @@ __device__ __forceinline__ float sgd_clip(float w, float g, float lr, float l1, 
 // Grid (layers, MLP_UPD_SPLIT).  Each workgroup updates its share of the layer's kernel entries;
 // the first one of a layer also owns EBOPs, the bias and the input quantizer's fractional bits.
 // Everything a workgroup needs about variables it does not own comes from the reduce pass.
-__global__ __launch_bounds__(256) void mlp_update_kernel(MlpDev d, const float *__restrict__ g, float lr, float *loss) {
+__global__ __launch_bounds__(256) void mlp_update_kernel(MlpDev d, const float *__restrict__ g, float lr, float *loss, float *img) {
     __shared__ float colsum[64];   // sum_n bits_ker[k, n]
     __shared__ float bits_in[64];  // relu(round(i) + round(f)) with the tracked i
     __shared__ float dbits_in[64];
@@ -432,10 +432,14 @@ __global__ __launch_bounds__(256) void mlp_update_kernel(MlpDev d, const float *
             reg += h.b_bias_l1 * h.b_bias[tid] + (h.train_i_bias ? h.i_bias_l1 * h.i_bias[tid] : 0.f);
             h.b_bias[tid] = sgd_clip(h.b_bias[tid], db + h.bias_size / (float)N * gs, lr, h.b_bias_l1, h.b_bias_lo, h.b_bias_hi);
             if (h.train_i_bias) h.i_bias[tid] = sgd_clip(h.i_bias[tid], di, lr, h.i_bias_l1, h.i_bias_lo, h.i_bias_hi);
+            // the next step's image entry, from the updated variables (what mlp_prep_kernel would compute)
+            img[ly.off_qb + tid] = quantize_dyn(h.bias[tid], kbi_entry(h.k_bias, h.i_bias, h.b_bias, tid, h.mode_bias), mb.round_mode,
+                                                mb.overflow_mode, true);
         }
         if (tid < K) {
             reg += h.f_in_l1 * h.f_in[tid];
             h.f_in[tid] = sgd_clip(h.f_in[tid], g[ly.p_df + tid] + dbits_in[tid] * colsum[tid] * gs, lr, h.f_in_l1, h.f_in_lo, h.f_in_hi);
+            img[ly.off_f + tid] = rintf(h.f_in[tid]);
         }
     }
     // quantizer backward of this workgroup's kernel entries, SGD + constraints
@@ -449,6 +453,8 @@ __global__ __launch_bounds__(256) void mlp_update_kernel(MlpDev d, const float *
         reg += h.b_ker_l1 * h.b_ker[e] + (h.train_i_ker ? h.i_ker_l1 * h.i_ker[e] : 0.f);
         h.b_ker[e] = sgd_clip(h.b_ker[e], db + bits_in[k] * gs, lr, h.b_ker_l1, h.b_ker_lo, h.b_ker_hi);
         if (h.train_i_ker) h.i_ker[e] = sgd_clip(h.i_ker[e], di, lr, h.i_ker_l1, h.i_ker_lo, h.i_ker_hi);
+        img[ly.off_w + k * ly.ldw + (e - k * N)] = quantize_dyn(h.w[e], kbi_entry(h.k_ker, h.i_ker, h.b_ker, e, h.mode_ker), mk.round_mode,
+                                                                mk.overflow_mode, true);
     }
     if (loss) {
 #pragma unroll
@@ -520,14 +526,15 @@ extern "C" int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, 
     return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX + d.off_raw + 4;
 }
 
-extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
-                                  int64_t rows, float lr, float *loss, float *workspace, void *stream) {
+extern "C" int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
+                                         int64_t rows, float lr, float *loss, float *workspace, int image_current, void *stream) {
     hipStream_t s = (hipStream_t)stream;
     MlpDev d;
     size_t lds_bytes;
     int rc = mlp_plan(layers, n_layers, d, lds_bytes);
     if (rc) return rc;
     if (rows < 1 || !x || !labels || !workspace) return fail(HGQ_ERR_ARG, "hgq_mlp_train_step: bad arguments");
+    if ((uintptr_t)workspace & 15u) return fail(HGQ_ERR_ARG, "hgq_mlp_train_step: the workspace must be 16-byte aligned");
     static bool raised = false;
     if (!raised) {
         hipError_t e = hipFuncSetAttribute((const void *)mlp_fwd_bwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 512);
@@ -535,15 +542,24 @@ extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, con
         raised = true;
     }
     const int parts = mlp_parts(rows);
-    float *reduced = workspace + (int64_t)parts * d.M;
-    float *img = reduced + d.M + (int64_t)n_layers * MLP_AUX;
-    img += (4 - ((uintptr_t)img / 4) % 4) % 4;  // 16-byte aligned
-    hipLaunchKernelGGL(mlp_prep_kernel, dim3((d.off_raw + 255) / 256), dim3(256), 0, s, d, img);
-    if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
-    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, workspace);
+    // workspace: [image | per-workgroup slices | reduced sums + per-layer aux]; the image comes first so
+    // that its place does not depend on the batch size
+    float *img = workspace;
+    float *slices = workspace + ((d.off_raw + 3) & ~3);
+    float *reduced = slices + (int64_t)parts * d.M;
+    if (!image_current) {
+        hipLaunchKernelGGL(mlp_prep_kernel, dim3((d.off_raw + 255) / 256), dim3(256), 0, s, d, img);
+        if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
+    }
+    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, slices);
     if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
-    hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(64 * MLP_RG), 0, s, d, workspace, parts, reduced, loss);
+    hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(64 * MLP_RG), 0, s, d, slices, parts, reduced, loss);
     if ((rc = check_launch("hgq_mlp_train_step(reduce)"))) return rc;
-    hipLaunchKernelGGL(mlp_update_kernel, dim3(n_layers, MLP_UPD_SPLIT), dim3(256), 0, s, d, reduced, lr, loss);
+    hipLaunchKernelGGL(mlp_update_kernel, dim3(n_layers, MLP_UPD_SPLIT), dim3(256), 0, s, d, reduced, lr, loss, img);
     return check_launch("hgq_mlp_train_step(update)");
+}
+
+extern "C" int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
+                                  int64_t rows, float lr, float *loss, float *workspace, void *stream) {
+    return hgq_mlp_train_step_cached(layers, n_layers, x, labels, rows, lr, loss, workspace, 0, stream);
 }

@@ -115,7 +115,8 @@ class GraphedTrainStep:
 
 class FusedQDenseStack:
     """One SGD training step of a stack of :class:`QDense` layers with mean sparse categorical
-    cross-entropy, executed by the whole-step kernels (three launches, see ``hgq_mlp_train_step``).
+    cross-entropy, executed by the whole-step kernels (three launches once the quantized weight image of
+    the previous step can be reused, see ``hgq_mlp_train_step_cached``).
 
     It updates exactly the variables the layer-by-layer path updates (kernels, biases, every
     bit-width variable, the tracked integer bits, ``ebops``) with the same arithmetic; it exists
@@ -189,8 +190,20 @@ class FusedQDenseStack:
                 it.train_i_bias = int(qb._i.requires_grad)
         self._arr = arr
         self._ws = None
+        # every variable the step reads: an in-place change from outside (seen through the tensors'
+        # version counters, which the kernels do not touch) invalidates the cached weight image
+        self._vars = [t for layer in layers for t in self._layer_vars(layer)]
+        self._versions = None
         self.device = layers[0]._kernel.device
         self.loss = torch.zeros((), dtype=torch.float32, device=self.device)
+
+    @staticmethod
+    def _layer_vars(layer):
+        qs = [layer.iq.quantizer, layer.kq.quantizer] + ([layer.bq.quantizer] if layer.bq is not None else [])
+        out = [layer._kernel] + ([layer.bias] if layer.bias is not None else [])
+        for q in qs:
+            out += [v for v in (getattr(q, '_k', None), getattr(q, '_i', None), getattr(q, '_f', None), getattr(q, '_b', None)) if v is not None]
+        return out
 
     def step(self, x, labels):
         """Run one training step in place; returns the loss tensor (cross-entropy + sum of EBOPs * beta
@@ -204,10 +217,14 @@ class FusedQDenseStack:
         need = lib.hgq_mlp_workspace(self._arr, len(self.layers), rows)
         if need < 0:
             self._lib.check(-3, 'hgq_mlp_workspace')
+        versions = [t._version for t in self._vars]
+        current = self._versions == versions
         if self._ws is None or self._ws.numel() < need:
             self._ws = torch.empty(need, dtype=torch.float32, device=self.device)
-        rc = lib.hgq_mlp_train_step(self._arr, len(self.layers), ct.c_void_p(x.data_ptr()), ct.c_void_p(labels.data_ptr()), rows,
-                                    self.lr, ct.c_void_p(self.loss.data_ptr()), ct.c_void_p(self._ws.data_ptr()),
-                                    ct.c_void_p(torch.cuda.current_stream().cuda_stream))
-        self._lib.check(rc, 'hgq_mlp_train_step')
+            current = False
+        rc = lib.hgq_mlp_train_step_cached(self._arr, len(self.layers), ct.c_void_p(x.data_ptr()), ct.c_void_p(labels.data_ptr()), rows,
+                                           self.lr, ct.c_void_p(self.loss.data_ptr()), ct.c_void_p(self._ws.data_ptr()), int(current),
+                                           ct.c_void_p(torch.cuda.current_stream().cuda_stream))
+        self._lib.check(rc, 'hgq_mlp_train_step_cached')
+        self._versions = versions
         return self.loss

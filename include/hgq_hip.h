@@ -243,6 +243,16 @@ typedef struct {
 int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, int64_t rows);
 int hgq_mlp_train_step(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
                        int64_t rows, float lr, float *loss, float *workspace, void *stream);
+/*
+ * The same step for a caller that owns the variables between steps.  The update pass leaves the
+ * quantized kernels / biases / rounded fractional bits of the UPDATED variables at the start of the
+ * workspace (the image the next step's forward reads); with image_current != 0 the step uses it
+ * instead of quantizing the variables again.  Pass 0 on the first step, after any change to a
+ * variable from outside, and whenever the workspace or the layer descriptors differ from the previous
+ * call's.  workspace must be 16-byte aligned.
+ */
+int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
+                              int64_t rows, float lr, float *loss, float *workspace, int image_current, void *stream);
 
 /*
  * Table-driven softmax, forward.  Replaces QSoftmax.call for the stable form without a mask

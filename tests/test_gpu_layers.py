@@ -173,6 +173,34 @@ def test_fused_qdense_stack_step_matches_oracle(dev, batch, dims):
             _close(pl.bq.quantizer._i, rl.bq.quantizer._i, scale=rl.bq.quantizer._i.detach().abs() + 1e-3, what=f'bq._i {n}')
 
 
+def test_fused_step_reuses_its_weight_image_only_while_it_owns_the_variables(dev):
+    """Steps that reuse the quantized weight image left by the previous update are bit-identical to
+    steps that quantize the variables again, across a change of batch size, and an in-place change
+    of a variable from outside (seen through the tensor's version counter) is picked up."""
+    from hgq2_amd.train import FusedQDenseStack
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(11)
+    xs = [torch.randn(n, 16, generator=g).to(dev) for n in (700, 700, 256, 700, 700)]
+    ys = [torch.randint(0, 5, (x.shape[0],), generator=g).to(dev) for x in xs]
+    oracle = ref.RefMLP(seed=5)
+    models = [qdense_mlp(device=dev) for _ in range(2)]
+    for m in models:
+        _copy_mlp(oracle, m, dev)
+    cached, fresh = (FusedQDenseStack(m, lr=0.05) for m in models)
+    for step, (x, y) in enumerate(zip(xs, ys)):
+        if step == 3:  # an outside change of a kernel entry, on both models
+            for m in models:
+                with torch.no_grad():
+                    m.layers[1]._kernel[3, 4] += 0.25
+        fresh._versions = None  # always quantize again
+        la, lb = cached.step(x, y), fresh.step(x, y)
+        # the reported loss adds its regularisation terms with atomics: equal up to the order of those adds
+        assert abs(float(la) - float(lb)) <= 1e-6 * abs(float(lb)), f'loss step {step}'
+        for pa, pb in zip(models[0].parameters(), models[1].parameters()):
+            assert torch.equal(pa, pb), f'step {step}'
+
+
 def test_trace_minmax_matches_oracle(dev):
     """The calibration pass (training='tracing') leaves the same integer bits, keep-negative flags
     and EBOPs as the oracle, and inference after it is bit-identical."""
