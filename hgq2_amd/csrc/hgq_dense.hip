@@ -659,15 +659,16 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 }
 
 // out[e] = sum over slices of part[g][e], in slice order.  256 threads = 64 elements x 4 slice groups.
-__global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restrict__ part, int n_parts, int64_t M,
-                                                           float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb,
-                                                           float *df, int64_t n_df) {
-    __shared__ float red[256];
+#define RP_G 16  // slice groups per entry: 64 entries x 16 groups = 1024 threads, few dependent load batches per thread
+__global__ __launch_bounds__(64 * RP_G) void reduce_parts_kernel(const float *__restrict__ part, int n_parts, int64_t M,
+                                                                 float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb,
+                                                                 float *df, int64_t n_df) {
+    __shared__ float red[64 * RP_G];
     const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
     float s = 0.f;
     if (e < M) {
-        const int per = (n_parts + 3) / 4;
+        const int per = (n_parts + RP_G - 1) / RP_G;
         const int g0 = grp * per, g1 = min(n_parts, g0 + per);
         // eight independent loads in flight per thread: the loop is latency-bound otherwise
         int g = g0;
@@ -682,7 +683,10 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restri
     red[threadIdx.x] = s;
     __syncthreads();
     if (grp == 0 && e < M) {
-        const float v = (red[e_local] + red[e_local + 64]) + (red[e_local + 128] + red[e_local + 192]);
+        float v = 0.f;  // groups in order
+#pragma unroll
+        for (int w = 0; w < RP_G; w += 4)
+            v += (red[e_local + 64 * w] + red[e_local + 64 * (w + 1)]) + (red[e_local + 64 * (w + 2)] + red[e_local + 64 * (w + 3)]);
         if (e < n_dqw) {
             if (dqw) dqw[e] = v;
         } else if (e < n_dqw + n_dqb) {
@@ -695,7 +699,7 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(const float *__restri
 
 int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb, float *df,
                  int64_t n_df, hipStream_t s) {
-    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(256), 0, s, part, n_parts, M, dqw, n_dqw, dqb, n_dqb, df, n_df);
+    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(64 * RP_G), 0, s, part, n_parts, M, dqw, n_dqw, dqb, n_dqb, df, n_df);
     return check_launch("reduce_parts");
 }
 
@@ -840,7 +844,7 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
                        act, mode, df_lds);
     int rc = check_launch("hgq_qdense_bwd");
     if (rc) return rc;
-    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(256), 0, s, workspace, parts, M, dqw, (int64_t)K * N, dqb,
+    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(64 * RP_G), 0, s, workspace, parts, M, dqw, (int64_t)K * N, dqb,
                        (int64_t)N, quant ? df_in : (float *)nullptr, PK);
     return check_launch("hgq_qdense_bwd(reduce)");
 }

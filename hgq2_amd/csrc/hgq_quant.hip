@@ -415,19 +415,20 @@ __global__ __launch_bounds__(256) void quant_bwd_generic(const float *__restrict
 // ------------------------------------------------------------------------------------------
 // integer-bit tracking
 // ------------------------------------------------------------------------------------------
-// 256 threads = 64 entries x 4 slice groups: the abs-max / any-negative trackers arrive as
+// 1024 threads = 64 entries x 16 slice groups: the abs-max / any-negative trackers arrive as
 // `n_parts` slices of [n] (one per producing workgroup) and are combined here.
-__global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__restrict__ amax,
-                                                           const uint32_t *__restrict__ anyneg, int n_parts,
-                                                           float *i_var, const float *__restrict__ fb, uint8_t *k_var,
-                                                           int64_t n, float decay, float c_lo, float c_hi, int mode) {
-    __shared__ uint32_t smax[256], sneg[256];
+#define WT_G 16
+__global__ __launch_bounds__(64 * WT_G) void wrap_track_i_kernel(const uint32_t *__restrict__ amax,
+                                                                 const uint32_t *__restrict__ anyneg, int n_parts,
+                                                                 float *i_var, const float *__restrict__ fb, uint8_t *k_var,
+                                                                 int64_t n, float decay, float c_lo, float c_hi, int mode) {
+    __shared__ uint32_t smax[64 * WT_G], sneg[64 * WT_G];
     const Mode m(mode);
     const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int64_t t = (int64_t)blockIdx.x * 64 + e_local;
     uint32_t mx = 0, ng = 0;
     if (t < n) {
-        const int per = (n_parts + 3) / 4;
+        const int per = (n_parts + WT_G - 1) / WT_G;
         const int g0 = grp * per, g1 = min(n_parts, g0 + per);
         int g = g0;
         for (; g + 8 <= g1; g += 8) {  // independent loads in flight
@@ -450,7 +451,7 @@ __global__ __launch_bounds__(256) void wrap_track_i_kernel(const uint32_t *__res
     smax[threadIdx.x] = mx, sneg[threadIdx.x] = ng;
     __syncthreads();
     if (grp != 0 || t >= n) return;
-    for (int w = 1; w < 4; ++w) {
+    for (int w = 1; w < WT_G; ++w) {
         const uint32_t a = smax[e_local + 64 * w];
         mx = a > mx ? a : mx;
         ng |= sneg[e_local + 64 * w];
@@ -664,7 +665,7 @@ extern "C" int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, in
     if (m < 0 || n_parts < 1) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i: bad size");
     if (m == 0) return HGQ_OK;
     if (!amax || !i_var || !fb) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i: null pointer");
-    hipLaunchKernelGGL(wrap_track_i_kernel, dim3((unsigned)((m + 63) / 64)), dim3(256), 0, (hipStream_t)stream, amax, anyneg, n_parts,
+    hipLaunchKernelGGL(wrap_track_i_kernel, dim3((unsigned)((m + 63) / 64)), dim3(64 * WT_G), 0, (hipStream_t)stream, amax, anyneg, n_parts,
                        i_var, fb, k_var, m, decay, c_lo, c_hi, mode);
     return check_launch("hgq_wrap_track_i");
 }
