@@ -466,11 +466,94 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
     }
 }
 
+// Column statistics of the contraction without writing it: sum_r z and sum_r z^2 of z = x W per
+// output column, for the batch statistics of QEinsumDenseBatchnorm.  Same tiling as the forward
+// above; a lane keeps the sums of its column over its 16 accumulator rows in registers across
+// tiles.  Slice blockIdx.x of `part` is [N sums | N sums of squares].
+template <int NS4>
+__global__ __launch_bounds__(256, 2) void dense_moments_fast_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                                   float *__restrict__ part, int64_t rows, int K, int N) {
+    __shared__ __attribute__((aligned(16))) float xs[2][FAST_BM + 1][FAST_XLD];
+    __shared__ float red[4][64][2];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rh = wave & 1, cb = wave >> 1;
+    const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
+    for (int id = tid; id < 2 * (FAST_BM + 1) * FAST_XLD; id += 256) (&xs[0][0][0])[id] = 0.f;
+    const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
+    float wreg[4 * NS4];
+#pragma unroll
+    for (int sidx = 0; sidx < 4 * NS4; ++sidx) {
+        const int k = 2 * sidx + kq;
+        wreg[sidx] = (k < K && bcol < N) ? w[(int64_t)k * N + bcol] : 0.f;
+    }
+    FastMap mp;
+    mp.init(K);
+    f32x4_t raw[FAST_NJ];
+    uint32_t xoff[FAST_NJ];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) xoff[j] = mp.on[j] ? (uint32_t)(mp.row[j] * K + mp.col[j]) * 4u : BUF_OOB;
+    auto load_tile = [&](int64_t t) {
+        const int64_t r0 = t * FAST_BM, left = rows - r0;
+        const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K, (left < FAST_BM ? left : FAST_BM) * K * 4);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) raw[j] = buf_ld4(rs, xoff[j]);
+    };
+    int64_t tile = blockIdx.x;
+    if (tile < n_tiles) load_tile(tile);
+    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    float s1 = 0.f, s2 = 0.f;
+    int buf = 0;
+    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            float *dst = &xs[buf][mp.on[j] ? mp.row[j] : FAST_BM][mp.col[j] >> 1];
+            *(float2 *)dst = make_float2(raw[j][0], raw[j][2]);
+            *(float2 *)(dst + 32) = make_float2(raw[j][1], raw[j][3]);
+        }
+        __syncthreads();
+        const int64_t next = tile + gridDim.x;
+        if (next < n_tiles) load_tile(next);
+        if (cb * 32 < N) {
+            floatx16 acc = {0};
+            const float *arow_p = &xs[buf][arow][kq * 32];
+            f32x4_t a4[NS4];
+#pragma unroll
+            for (int s4 = 0; s4 < NS4; ++s4) a4[s4] = *(const f32x4_t *)(arow_p + 4 * s4);
+#pragma unroll
+            for (int s4 = 0; s4 < NS4; ++s4)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[s4][e], wreg[4 * s4 + e], acc, 0, 0, 0);
+            // rows past the end were staged as zeros: z = 0 there, which adds nothing
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s1 += acc[r], s2 += acc[r] * acc[r];
+        }
+    }
+    // a column's sums sit in two lanes (row groups) of two wavefronts (row halves): add them in a fixed order
+    red[wave][lane][0] = s1, red[wave][lane][1] = s2;
+    __syncthreads();
+    if (tid < 2 * N) {
+        const int c = tid % N, which = tid / N, wcb = c >> 5, l = c & 31;
+        float v = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) v += red[wcb * 2 + h][l][which] + red[wcb * 2 + h][l + 32][which];
+        part[(int64_t)blockIdx.x * 2 * N + which * N + c] = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void moments_scale_kernel(float *mean, float *meansq, int N, float inv_rows) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t < N) mean[t] *= inv_rows, meansq[t] *= inv_rows;
+}
+
 // Backward.  Per tile: stage dz = dy (masked by y for ReLU) and the quantized input; dx = dz W^T
 // and dW += xq^T dz on MFMA; dx goes back through LDS so that it is stored with 128-bit writes and
 // meets the rounding residue (xq - x) of the staging thread for the fractional-bit gradient.
 // Slice blockIdx.x of `part` is [K * N | N | P * K].
-template <int RM, bool QUANT>
+// STATS: the gradient at the pre-activation is not read but computed in the tile from the upstream
+// gradients of the column statistics: dz[r, c] = (gm[c] + 2 z[r, c] gs[c]) / rows with z = x W
+// recomputed on the matrix cores (dy = gm, y = gs, both [N]); no activation, no bias, no quantizer.
+template <int RM, bool QUANT, bool STATS = false>
 __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
@@ -540,15 +623,19 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     // the mask descriptor is empty and is not consulted
     auto load_tile = [&](int64_t t) {
         const int64_t r0 = t * FAST_BM, left = rows - r0, vr = left < FAST_BM ? left : FAST_BM;
-        const __amdgpu_buffer_rsrc_t sx = buf_rsrc(x + r0 * K, vr * K * 4), sg = buf_rsrc(dy + r0 * N, vr * N * 4);
-        const __amdgpu_buffer_rsrc_t sy = buf_rsrc(relu ? y + r0 * N : dy, relu ? vr * N * 4 : 0);
+        const __amdgpu_buffer_rsrc_t sx = buf_rsrc(x + r0 * K, vr * K * 4);
+        const __amdgpu_buffer_rsrc_t sg = buf_rsrc(STATS ? x : dy + r0 * N, STATS ? 0 : vr * N * 4);
+        const __amdgpu_buffer_rsrc_t sy = buf_rsrc((relu && !STATS) ? y + r0 * N : x, (relu && !STATS) ? vr * N * 4 : 0);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
             rx[j] = buf_ld4(sx, xoff[j]);
-            rg[j] = buf_ld4(sg, zoff[j]);
-            ry[j] = buf_ld4(sy, zoff[j]);
+            if (!STATS) {
+                rg[j] = buf_ld4(sg, zoff[j]);
+                ry[j] = buf_ld4(sy, zoff[j]);
+            }
         }
     };
+    const float inv_rows = 1.0f / (float)rows;
     if (tile < n_tiles) load_tile(tile);
     __syncthreads();
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing loaded before the loop is waited for inside it
@@ -567,12 +654,31 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                 dlt[j][e] = q - v[e];
                 xs[xr][mx.col[j] + e] = q;
             }
-            const float g[4] = {rg[j][0], rg[j][1], rg[j][2], rg[j][3]};
-            const float a[4] = {ry[j][0], ry[j][1], ry[j][2], ry[j][3]};
+            if (!STATS) {
+                const float g[4] = {rg[j][0], rg[j][1], rg[j][2], rg[j][3]};
+                const float a[4] = {ry[j][0], ry[j][1], ry[j][2], ry[j][3]};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) dzs[zr][mz.col[j] + e] = (!relu || a[e] > 0.f) ? g[e] : 0.f;
+                for (int e = 0; e < 4; ++e) dzs[zr][mz.col[j] + e] = (!relu || a[e] > 0.f) ? g[e] : 0.f;
+            }
         }
         __syncthreads();
+        if (STATS) {
+            // z block (row half, column block) of this wave, then dz into the gradient tile
+            const int zrh = wave & 1, zcb = wave >> 1;
+            if (zcb < N32) {
+                floatx16 z = {0};
+                const int arow = zrh * 32 + (lane & 31), kq = lane >> 5, bcol = zcb * 32 + (lane & 31);
+                z = mfma_chain(z, &xs[arow][kq], 1, &ws[kq][bcol], FAST_LD, K32 * 2);
+                const float gm = bcol < N ? dy[bcol] : 0.f, gs = bcol < N ? y[bcol] : 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = zrh * 32 + acc_row(r, lane);
+                    const bool live = tile * FAST_BM + row < rows && bcol < N;
+                    dzs[row][bcol] = live ? (gm + 2.0f * z[r] * gs) * inv_rows : 0.f;
+                }
+            }
+            __syncthreads();
+        }
         const int64_t next = tile + gridDim.x;
         const int64_t r0 = tile * FAST_BM;
         if (next < n_tiles) load_tile(next);
@@ -770,6 +876,52 @@ extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_i
         });
     }
     return check_launch("hgq_qdense_fwd");
+}
+
+extern "C" int64_t hgq_dense_moments_workspace(int64_t rows, int K, int N) {
+    if (rows < 0 || K < 1 || N < 1) return -1;
+    const int64_t parts = rows > 0 ? row_parts(rows, FAST_BM) : 1;
+    const int64_t fwd = parts * 2 * N, bwd = parts * ((int64_t)K * N + N);
+    return fwd > bwd ? fwd : bwd;
+}
+
+static int moments_check(const char *who, int64_t rows, int K, int N, const void *x) {
+    if (rows < 1 || K < 1 || N < 1) return fail(HGQ_ERR_ARG, "%s: bad sizes", who);
+    if (K > 64 || N > 64 || K % 4 != 0 || N % 4 != 0 || !aligned16(x))
+        return fail(HGQ_ERR_UNSUPPORTED, "%s: needs K, N <= 64, multiples of 4, and a 16-byte aligned input (K=%d N=%d)", who, K, N);
+    return HGQ_OK;
+}
+
+extern "C" int hgq_dense_moments_fwd(const float *x, const float *w, float *mean, float *meansq, float *workspace, int64_t rows,
+                                     int K, int N, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    int rc = moments_check("hgq_dense_moments_fwd", rows, K, N, x);
+    if (rc) return rc;
+    if (!x || !w || !mean || !meansq || !workspace) return fail(HGQ_ERR_ARG, "hgq_dense_moments_fwd: null pointer");
+    const int parts = row_parts(rows, FAST_BM);
+    const dim3 grid((unsigned)parts);
+    if (K <= 8) hipLaunchKernelGGL((dense_moments_fast_kernel<1>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
+    else if (K <= 16) hipLaunchKernelGGL((dense_moments_fast_kernel<2>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
+    else if (K <= 32) hipLaunchKernelGGL((dense_moments_fast_kernel<4>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
+    else hipLaunchKernelGGL((dense_moments_fast_kernel<8>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
+    if ((rc = check_launch("hgq_dense_moments_fwd"))) return rc;
+    if ((rc = reduce_parts(workspace, parts, 2 * (int64_t)N, mean, (int64_t)N, meansq, (int64_t)N, nullptr, 0, s))) return rc;
+    hipLaunchKernelGGL(moments_scale_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, mean, meansq, N, 1.0f / (float)rows);
+    return check_launch("hgq_dense_moments_fwd(scale)");
+}
+
+extern "C" int hgq_dense_moments_bwd(const float *x, const float *w, const float *dmean, const float *dmeansq, float *dx, float *dw,
+                                     float *workspace, int64_t rows, int K, int N, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    int rc = moments_check("hgq_dense_moments_bwd", rows, K, N, x);
+    if (rc) return rc;
+    if (!x || !w || !dmean || !dmeansq || !dx || !dw || !workspace) return fail(HGQ_ERR_ARG, "hgq_dense_moments_bwd: null pointer");
+    if (!aligned16(dx)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_moments_bwd: dx must be 16-byte aligned");
+    const int parts = row_parts(rows, BWD_BM);
+    hipLaunchKernelGGL((qdense_bwd_fast_kernel<HGQ_TRN, false, true>), dim3((unsigned)parts), dim3(256), 0, s, dmean, dmeansq, x,
+                       (const float *)nullptr, 1, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, 0);
+    if ((rc = check_launch("hgq_dense_moments_bwd"))) return rc;
+    return reduce_parts(workspace, parts, (int64_t)K * N + N, dw, (int64_t)K * N, nullptr, (int64_t)N, nullptr, 0, s);
 }
 
 extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,

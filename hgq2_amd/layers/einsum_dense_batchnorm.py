@@ -95,11 +95,15 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         if trailing and qinputs.is_cuda:
             x2d = qinputs.reshape(-1, self._K)
             w2d = self._kernel.reshape(self._K, self._N)
-            if self._K <= ops.FUSED_BWD_MAX and self._N <= ops.FUSED_BWD_MAX:
-                pre, _ = ops.qdense(x2d.contiguous(), None, None, None, w2d, None, _lib.ACT_NONE, 0, 0, False)
+            x2d = x2d.contiguous()
+            if ops.dense_moments_supported(x2d, w2d):
+                mean, meansq = ops.dense_moments(x2d, w2d)  # one pass over x, the pre-activation is never written
             else:
-                pre = ops.matmul_bias_act(x2d, w2d, None, _lib.ACT_NONE)
-            mean, meansq = ops.col_moments(pre)
+                if self._K <= ops.FUSED_BWD_MAX and self._N <= ops.FUSED_BWD_MAX:
+                    pre, _ = ops.qdense(x2d, None, None, None, w2d, None, _lib.ACT_NONE, 0, 0, False)
+                else:
+                    pre = ops.matmul_bias_act(x2d, w2d, None, _lib.ACT_NONE)
+                mean, meansq = ops.col_moments(pre)
             shape = tuple(self.full_output_shape[n_out - self._gemm[1]:])
             mean, meansq = mean.view(shape), meansq.view(shape)
             return mean, meansq - torch.square(mean)

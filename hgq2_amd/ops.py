@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported']
 
 
 def _ptr(t: Tensor | None):
@@ -592,6 +592,48 @@ def _(pred, target, g):
     return torch.empty_like(pred)
 
 
+def dense_moments_supported(x2d: Tensor, w2d: Tensor) -> bool:
+    """Whether hgq_dense_moments_* covers this contraction (K, N <= 64, multiples of 4, aligned input)."""
+    K, N = w2d.shape
+    return x2d.is_cuda and x2d.shape[0] > 0 and K <= 64 and N <= 64 and K % 4 == 0 and N % 4 == 0 and x2d.data_ptr() % 16 == 0
+
+
+@torch.library.custom_op('hgq::dense_moments_fwd', mutates_args=())
+def dense_moments_fwd(x: Tensor, w: Tensor) -> tuple[Tensor, Tensor]:
+    _check_f32('x', x), _check_f32('w', w)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[0], 'shape mismatch')
+    rows, K = x.shape
+    N = w.shape[1]
+    lib = _lib.load()
+    mean, meansq = (torch.empty(N, dtype=torch.float32, device=x.device) for _ in range(2))
+    ws = torch.empty(max(lib.hgq_dense_moments_workspace(rows, K, N), 1), dtype=torch.float32, device=x.device)
+    _lib.check(lib.hgq_dense_moments_fwd(_ptr(x), _ptr(w), _ptr(mean), _ptr(meansq), _ptr(ws), rows, K, N, _stream()), 'hgq_dense_moments_fwd')
+    return mean, meansq
+
+
+@dense_moments_fwd.register_fake
+def _(x, w):
+    return x.new_empty(w.shape[1]), x.new_empty(w.shape[1])
+
+
+@torch.library.custom_op('hgq::dense_moments_bwd', mutates_args=())
+def dense_moments_bwd(x: Tensor, w: Tensor, dmean: Tensor, dmeansq: Tensor) -> tuple[Tensor, Tensor]:
+    _check_f32('x', x), _check_f32('w', w), _check_f32('dmean', dmean), _check_f32('dmeansq', dmeansq)
+    rows, K = x.shape
+    N = w.shape[1]
+    lib = _lib.load()
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    ws = torch.empty(max(lib.hgq_dense_moments_workspace(rows, K, N), 1), dtype=torch.float32, device=x.device)
+    _lib.check(lib.hgq_dense_moments_bwd(_ptr(x), _ptr(w), _ptr(dmean), _ptr(dmeansq), _ptr(dx), _ptr(dw), _ptr(ws), rows, K, N, _stream()),
+               'hgq_dense_moments_bwd')
+    return dx, dw
+
+
+@dense_moments_bwd.register_fake
+def _(x, w, dmean, dmeansq):
+    return torch.empty_like(x), torch.empty_like(w)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -823,6 +865,25 @@ class _ColMoments(torch.autograd.Function):
 def col_moments(x2d: Tensor):
     """``(mean(x, 0), mean(x * x, 0))`` of a [rows, N] matrix in one pass."""
     return _ColMoments.apply(x2d.contiguous())
+
+
+class _DenseMoments(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return dense_moments_fwd(x, w)
+
+    @staticmethod
+    def backward(ctx, gm, gs):
+        x, w = ctx.saved_tensors
+        gm = torch.zeros(w.shape[1], device=x.device) if gm is None else gm.contiguous()
+        gs = torch.zeros(w.shape[1], device=x.device) if gs is None else gs.contiguous()
+        return dense_moments_bwd(x, w, gm, gs)
+
+
+def dense_moments(x2d: Tensor, w2d: Tensor):
+    """``(mean(z, 0), mean(z * z, 0))`` of ``z = x2d @ w2d`` without materialising ``z``."""
+    return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous())
 
 
 class _AttnScores(torch.autograd.Function):

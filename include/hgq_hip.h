@@ -342,6 +342,22 @@ int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float
                    float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
 
 /*
+ * Batch statistics of the un-quantized pre-activation z = x W of QEinsumDenseBatchnorm.call
+ * (src/hgq/layers/einsum_dense_batchnorm.py:99-124) WITHOUT materialising z: the contraction and the
+ * column sums run in one pass over x, and the backward recomputes z tile by tile.
+ *   x [rows, K];  w [K, N] (the un-quantized kernel);  mean, meansq [N] = mean_r z, mean_r z^2;
+ *   backward: with dz[r, c] = (dmean[c] + 2 z[r, c] dmeansq[c]) / rows,  dx = dz W^T,  dw = x^T dz.
+ *   workspace: hgq_dense_moments_workspace(rows, K, N) floats (per-workgroup slices, fixed-order sum).
+ * K, N <= 64 and multiples of 4; x (and dx) 16-byte aligned; otherwise HGQ_ERR_UNSUPPORTED and the
+ * caller uses hgq_qdense_fwd + hgq_col_moments_fwd.
+ */
+int64_t hgq_dense_moments_workspace(int64_t rows, int K, int N);
+int hgq_dense_moments_fwd(const float *x, const float *w, float *mean, float *meansq, float *workspace, int64_t rows, int K,
+                          int N, void *stream);
+int hgq_dense_moments_bwd(const float *x, const float *w, const float *dmean, const float *dmeansq, float *dx, float *dw,
+                          float *workspace, int64_t rows, int K, int N, void *stream);
+
+/*
  * Per-column mean and mean of squares of a [rows, N] matrix, and the gradient of both.  Replaces
  * `ops.mean(x, axis)` / `ops.mean(ops.square(x), axis)` and their autograd in
  * QEinsumDenseBatchnorm.call (src/hgq/layers/einsum_dense_batchnorm.py:99-124, the batch

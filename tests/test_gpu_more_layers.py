@@ -375,3 +375,29 @@ def test_full_size_attention_step_matches_oracle(dev):
     # sums over up to 33.5 M terms: fp32 accumulation order differs between the kernels and the CPU
     _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=5e-4)
     assert int(layer._ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('rows,K,N', [(1000, 16, 64), (64 * 3 + 5, 64, 32), (7, 4, 4), (70000, 64, 64), (513, 20, 12)])
+def test_dense_moments_without_materialising_the_contraction(rows, K, N):
+    """ops.dense_moments = (mean(z), mean(z^2)) of z = x @ w and its gradients against fp64
+    (reference: the batch statistics of QEinsumDenseBatchnorm.call, einsum_dense_batchnorm.py:99-124)."""
+    from hgq2_amd import ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(rows + K)
+    x = torch.randn(rows, K, generator=g)
+    w = torch.randn(K, N, generator=g) * 0.4
+    um, us = torch.randn(N, generator=g), torch.randn(N, generator=g)
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    z = xr @ wr
+    mean_r, msq_r = z.mean(0), (z * z).mean(0)
+    ((mean_r * um.double()).sum() + (msq_r * us.double()).sum()).backward()
+    xd, wd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    assert ops.dense_moments_supported(xd, wd)
+    mean, msq = ops.dense_moments(xd, wd)
+    ((mean * um.to(dev)).sum() + (msq * us.to(dev)).sum()).backward()
+    for name, got, want in (('mean', mean, mean_r), ('meansq', msq, msq_r), ('dx', xd.grad, xr.grad), ('dw', wd.grad, wr.grad)):
+        scale = float(want.abs().max()) + 1e-12
+        err = float((got.detach().cpu().double() - want.detach()).abs().max())
+        assert err <= 2e-5 * scale, f'{name}: {err:.3e} vs scale {scale:.3e}'
