@@ -202,6 +202,71 @@ __global__ __launch_bounds__(256) void mse_bwd_kernel(const float *__restrict__ 
     }
 }
 
+// Batch-norm folding of QEinsumDenseBatchnorm for a [K, N] kernel normalised over its N outputs:
+//     var = second - mean^2 (second = mean of squares) or var = second;  scaler = gamma / sqrt(var + eps)
+//     fused_w[k, n] = w[k, n] * scaler[n];   fused_b[n] = bias[n] + (-mean[n] * scaler[n])
+// and, when moving statistics are given, their momentum update.  One thread per kernel entry; the
+// first K-row also writes the per-column results.  IEEE division and square root, reference order.
+__device__ __forceinline__ float bn_var(float mean, float second, int is_meansq) {
+    return is_meansq ? __fsub_rn(second, __fmul_rn(mean, mean)) : second;
+}
+
+__global__ __launch_bounds__(256) void bn_fold_fwd_kernel(const float *__restrict__ w, const float *__restrict__ bias,
+                                                          const float *__restrict__ gamma, const float *__restrict__ mean,
+                                                          const float *__restrict__ second, int is_meansq, float eps,
+                                                          float *__restrict__ fused_w, float *__restrict__ fused_b, float *moving_mean,
+                                                          float *moving_var, float momentum, float one_minus_momentum, int K, int N) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (int64_t)K * N) return;
+    const int n = (int)(e % N);
+    const float var = bn_var(mean[n], second[n], is_meansq);
+    const float scaler = __fdiv_rn(gamma ? gamma[n] : 1.0f, __fsqrt_rn(__fadd_rn(var, eps)));
+    fused_w[e] = __fmul_rn(w[e], scaler);
+    if (e < N) {
+        fused_b[n] = __fadd_rn(bias[n], __fmul_rn(-mean[n], scaler));
+        if (moving_mean) moving_mean[n] = __fadd_rn(__fmul_rn(moving_mean[n], momentum), __fmul_rn(mean[n], one_minus_momentum));
+        if (moving_var) moving_var[n] = __fadd_rn(__fmul_rn(moving_var[n], momentum), __fmul_rn(var, one_minus_momentum));
+    }
+}
+
+// Gradients of the folding.  One thread per output column n walks the K kernel rows (coalesced
+// across columns):  dw = d_fw * scaler;  dscaler = sum_k d_fw * w - d_fb * mean;  dbias = d_fb;
+// dgamma = dscaler / sqrt(var + eps);  dvar = -dscaler * gamma / (2 (var + eps)^(3/2));
+// dmean = -d_fb * scaler (- 2 mean dvar when var comes from the mean of squares);  dsecond = dvar.
+__global__ __launch_bounds__(64) void bn_fold_bwd_kernel(const float *__restrict__ w, const float *__restrict__ gamma,
+                                                         const float *__restrict__ mean, const float *__restrict__ second,
+                                                         int is_meansq, float eps, const float *__restrict__ d_fw,
+                                                         const float *__restrict__ d_fb, float *__restrict__ dw, float *dbias,
+                                                         float *dgamma, float *dmean, float *dsecond, int K, int N) {
+    const int n = blockIdx.x * 64 + threadIdx.x;
+    if (n >= N) return;
+    const float g = gamma ? gamma[n] : 1.0f, m = mean[n];
+    const float ve = bn_var(m, second[n], is_meansq) + eps, sd = __fsqrt_rn(ve);
+    const float scaler = __fdiv_rn(g, sd);
+    float ds = 0.f;
+    for (int k0 = 0; k0 < K; k0 += 8) {
+        float gv[8], wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const bool on = k0 + u < K;
+            gv[u] = on ? d_fw[(int64_t)(k0 + u) * N + n] : 0.f;
+            wv[u] = on ? w[(int64_t)(k0 + u) * N + n] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            ds += gv[u] * wv[u];
+            if (k0 + u < K) dw[(int64_t)(k0 + u) * N + n] = gv[u] * scaler;
+        }
+    }
+    const float gb = d_fb[n];
+    ds -= gb * m;
+    const float dvar = -ds * g / (2.0f * ve * sd);
+    if (dbias) dbias[n] = gb;
+    if (dgamma) dgamma[n] = ds / sd;
+    if (dsecond) dsecond[n] = dvar;
+    if (dmean) dmean[n] = -gb * scaler - (is_meansq ? 2.0f * m * dvar : 0.f);
+}
+
 // one thread per row; C is small (class count)
 __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict__ logits,
                                                         const int64_t *__restrict__ labels, float *loss,
@@ -375,6 +440,27 @@ extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels,
     const int grid = persistent_grid((rows + 255) / 256, 4);
     hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C);
     return check_launch("hgq_sparse_ce_fwd_bwd");
+}
+
+extern "C" int hgq_bn_fold_fwd(const float *w, const float *bias, const float *gamma, const float *mean, const float *second,
+                               int is_meansq, float eps, float *fused_w, float *fused_b, float *moving_mean, float *moving_var,
+                               float momentum, float one_minus_momentum, int K, int N, void *stream) {
+    if (K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_bn_fold_fwd: bad sizes");
+    if (!w || !bias || !mean || !second || !fused_w || !fused_b) return fail(HGQ_ERR_ARG, "hgq_bn_fold_fwd: null pointer");
+    const int64_t n = (int64_t)K * N;
+    hipLaunchKernelGGL(bn_fold_fwd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, w, bias, gamma, mean, second,
+                       is_meansq, eps, fused_w, fused_b, moving_mean, moving_var, momentum, one_minus_momentum, K, N);
+    return check_launch("hgq_bn_fold_fwd");
+}
+
+extern "C" int hgq_bn_fold_bwd(const float *w, const float *gamma, const float *mean, const float *second, int is_meansq, float eps,
+                               const float *d_fw, const float *d_fb, float *dw, float *dbias, float *dgamma, float *dmean,
+                               float *dsecond, int K, int N, void *stream) {
+    if (K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_bn_fold_bwd: bad sizes");
+    if (!w || !mean || !second || !d_fw || !d_fb || !dw) return fail(HGQ_ERR_ARG, "hgq_bn_fold_bwd: null pointer");
+    hipLaunchKernelGGL(bn_fold_bwd_kernel, dim3((unsigned)((N + 63) / 64)), dim3(64), 0, (hipStream_t)stream, w, gamma, mean, second,
+                       is_meansq, eps, d_fw, d_fb, dw, dbias, dgamma, dmean, dsecond, K, N);
+    return check_launch("hgq_bn_fold_bwd");
 }
 
 extern "C" int64_t hgq_mse_workspace(void) { return MSE_PARTS; }

@@ -86,12 +86,18 @@ class QEinsumDenseBatchnorm(QEinsumDense):
     def qbias(self):
         return self.get_fused_qkernel_and_qbias(False, self.moving_mean, self.moving_variance)[1]
 
-    def _batch_moments(self, qinputs):
-        """Mean and variance of the un-quantized-kernel pre-activation over the non-normalised axes
-        (reference :108-112).  GEMM-shaped equations whose normalised axes are all the new output axes
-        run through the dense and column-moment kernels; others through the library einsum."""
+    def _trailing_gemm(self):
+        """GEMM-shaped equation whose normalised axes are exactly the new output axes."""
         n_out = len(self.full_output_shape)
-        trailing = self._gemm is not None and self._reduction_axes == tuple(range(n_out - self._gemm[1]))
+        return self._gemm is not None and self._reduction_axes == tuple(range(n_out - self._gemm[1]))
+
+    def _batch_moments(self, qinputs, raw=False):
+        """Mean and variance (``raw``: mean of squares, flat) of the un-quantized-kernel pre-activation
+        over the non-normalised axes (reference :108-112).  GEMM-shaped equations whose normalised axes
+        are all the new output axes run through the dense and column-moment kernels; others through the
+        library einsum."""
+        n_out = len(self.full_output_shape)
+        trailing = self._trailing_gemm()
         if trailing and qinputs.is_cuda:
             x2d = qinputs.reshape(-1, self._K)
             w2d = self._kernel.reshape(self._K, self._N)
@@ -104,6 +110,8 @@ class QEinsumDenseBatchnorm(QEinsumDense):
                 else:
                     pre = ops.matmul_bias_act(x2d, w2d, None, _lib.ACT_NONE)
                 mean, meansq = ops.col_moments(pre)
+            if raw:
+                return mean, meansq
             shape = tuple(self.full_output_shape[n_out - self._gemm[1]:])
             mean, meansq = mean.view(shape), meansq.view(shape)
             return mean, meansq - torch.square(mean)
@@ -114,14 +122,24 @@ class QEinsumDenseBatchnorm(QEinsumDense):
     def call(self, inputs, training=None):
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
-        if training and self.trainable:
-            mean, var = self._batch_moments(inputs)
-            with torch.no_grad():
-                self.moving_mean.copy_(self.moving_mean * self.momentum + mean * (1.0 - self.momentum))
-                self.moving_variance.copy_(self.moving_variance * self.momentum + var * (1.0 - self.momentum))
+        if training and self.trainable and inputs.is_cuda and self._trailing_gemm() and self.bias.numel() == self._N:
+            # statistics, folding and the moving-average update in three launches (the folding algebra and its
+            # gradient would otherwise be some forty elementwise launches on [N] vectors)
+            mean, meansq = self._batch_moments(inputs, raw=True)
+            fused_kernel, fused_bias = ops.bn_fold(self._kernel.reshape(self._K, self._N), self.bias.reshape(-1),
+                                                   self.bn_gamma.reshape(-1) if self.scale else None, mean, meansq, True, epsilon(),
+                                                   self.moving_mean.view(-1), self.moving_variance.view(-1), self.momentum)
+            qkernel = self.kq(fused_kernel.view(self._kernel.shape), training=training)
+            qbias = self.bq(fused_bias.view(self.bias.shape), training=training)
         else:
-            var, mean = self.moving_variance, self.moving_mean
-        qkernel, qbias = self.get_fused_qkernel_and_qbias(training, mean, var)
+            if training and self.trainable:
+                mean, var = self._batch_moments(inputs)
+                with torch.no_grad():
+                    self.moving_mean.copy_(self.moving_mean * self.momentum + mean * (1.0 - self.momentum))
+                    self.moving_variance.copy_(self.moving_variance * self.momentum + var * (1.0 - self.momentum))
+            else:
+                var, mean = self.moving_variance, self.moving_mean
+            qkernel, qbias = self.get_fused_qkernel_and_qbias(training, mean, var)
         # the input is already quantized: contract without the fused input quantizer
         enable_iq, self._enable_iq = self._enable_iq, False
         try:

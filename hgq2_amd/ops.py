@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold']
 
 
 def _ptr(t: Tensor | None):
@@ -634,6 +634,46 @@ def _(x, w, dmean, dmeansq):
     return torch.empty_like(x), torch.empty_like(w)
 
 
+@torch.library.custom_op('hgq::bn_fold_fwd', mutates_args=('moving_mean', 'moving_var'))
+def bn_fold_fwd(w: Tensor, bias: Tensor, gamma: Tensor, mean: Tensor, second: Tensor, is_meansq: bool, eps: float,
+                moving_mean: Tensor, moving_var: Tensor, momentum: float) -> tuple[Tensor, Tensor]:
+    for name, t in (('w', w), ('bias', bias), ('mean', mean), ('second', second)):
+        _check_f32(name, t)
+    K, N = w.shape
+    _need(bias.numel() == N and mean.numel() == N and second.numel() == N and gamma.numel() in (0, N), 'per-column operands must have N entries')
+    _need(moving_mean.numel() in (0, N) and moving_var.numel() in (0, N), 'moving statistics must have N entries')
+    fw, fb = torch.empty_like(w), torch.empty_like(bias)
+    rc = _lib.load().hgq_bn_fold_fwd(_ptr(w), _ptr(bias), _ptr(gamma), _ptr(mean), _ptr(second), int(is_meansq), eps, _ptr(fw), _ptr(fb),
+                                     _ptr(moving_mean), _ptr(moving_var), momentum, 1.0 - momentum, K, N, _stream())
+    _lib.check(rc, 'hgq_bn_fold_fwd')
+    return fw, fb
+
+
+@bn_fold_fwd.register_fake
+def _(w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum):
+    return torch.empty_like(w), torch.empty_like(bias)
+
+
+@torch.library.custom_op('hgq::bn_fold_bwd', mutates_args=())
+def bn_fold_bwd(w: Tensor, gamma: Tensor, mean: Tensor, second: Tensor, is_meansq: bool, eps: float, d_fw: Tensor,
+                d_fb: Tensor) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
+    _check_f32('d_fw', d_fw), _check_f32('d_fb', d_fb)
+    K, N = w.shape
+    dw = torch.empty_like(w)
+    dbias, dmean, dsecond = (torch.empty(N, dtype=torch.float32, device=w.device) for _ in range(3))
+    dgamma = torch.empty(N if gamma.numel() else 0, dtype=torch.float32, device=w.device)
+    rc = _lib.load().hgq_bn_fold_bwd(_ptr(w), _ptr(gamma), _ptr(mean), _ptr(second), int(is_meansq), eps, _ptr(d_fw), _ptr(d_fb), _ptr(dw),
+                                     _ptr(dbias), _ptr(dgamma), _ptr(dmean), _ptr(dsecond), K, N, _stream())
+    _lib.check(rc, 'hgq_bn_fold_bwd')
+    return dw, dbias, dgamma, dmean, dsecond
+
+
+@bn_fold_bwd.register_fake
+def _(w, gamma, mean, second, is_meansq, eps, d_fw, d_fb):
+    n = w.shape[1]
+    return torch.empty_like(w), w.new_empty(n), w.new_empty(n if gamma.numel() else 0), w.new_empty(n), w.new_empty(n)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -884,6 +924,32 @@ class _DenseMoments(torch.autograd.Function):
 def dense_moments(x2d: Tensor, w2d: Tensor):
     """``(mean(z, 0), mean(z * z, 0))`` of ``z = x2d @ w2d`` without materialising ``z``."""
     return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous())
+
+
+class _BnFold(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum):
+        ctx.save_for_backward(w, gamma, mean, second)
+        ctx.cfg = (is_meansq, eps)
+        return bn_fold_fwd(w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum)
+
+    @staticmethod
+    def backward(ctx, d_fw, d_fb):
+        w, gamma, mean, second = ctx.saved_tensors
+        is_meansq, eps = ctx.cfg
+        dw, dbias, dgamma, dmean, dsecond = bn_fold_bwd(w, gamma, mean, second, is_meansq, eps, d_fw.contiguous(), d_fb.contiguous())
+        return dw, dbias, (dgamma if gamma.numel() else None), dmean, dsecond, None, None, None, None, None
+
+
+def bn_fold(w2d: Tensor, bias: Tensor, gamma, mean: Tensor, second: Tensor, is_meansq: bool, eps: float, moving_mean=None,
+            moving_var=None, momentum: float = 0.0):
+    """Batch-norm folding ``(w * s, bias - mean * s)`` with ``s = gamma / sqrt(var + eps)`` for a ``[K, N]`` kernel
+    normalised over its outputs; ``second`` is the mean of squares (``is_meansq``) or the variance.  Moving statistics,
+    when given, are updated in place with ``momentum``."""
+    empty = w2d.new_empty(0)
+    return _BnFold.apply(w2d.contiguous(), bias.contiguous(), gamma.contiguous() if gamma is not None else empty, mean.contiguous(),
+                         second.contiguous(), bool(is_meansq), float(eps), moving_mean if moving_mean is not None else empty,
+                         moving_var if moving_var is not None else empty, float(momentum))
 
 
 class _AttnScores(torch.autograd.Function):

@@ -342,6 +342,24 @@ int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float
                    float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
 
 /*
+ * Batch-norm folding of QEinsumDenseBatchnorm.get_fused_qkernel_and_qbias
+ * (src/hgq/layers/einsum_dense_batchnorm.py:160-172) for a [K, N] kernel normalised over its N
+ * outputs, before the kernel / bias quantizers:
+ *     var = second - mean^2 if is_meansq else second;   scaler = gamma / sqrt(var + eps)   (gamma NULL = 1)
+ *     fused_w[k, n] = w[k, n] * scaler[n];   fused_b[n] = bias[n] - mean[n] * scaler[n]
+ * With moving_mean / moving_var (each may be NULL) the forward also applies the momentum update of
+ * QEinsumDenseBatchnorm.call (:113-117): m <- m * momentum + batch * one_minus_momentum.
+ * The backward returns the gradients w.r.t. w, bias, gamma, mean and `second` (any of dbias, dgamma,
+ * dmean, dsecond may be NULL).
+ */
+int hgq_bn_fold_fwd(const float *w, const float *bias, const float *gamma, const float *mean, const float *second, int is_meansq,
+                    float eps, float *fused_w, float *fused_b, float *moving_mean, float *moving_var, float momentum,
+                    float one_minus_momentum, int K, int N, void *stream);
+int hgq_bn_fold_bwd(const float *w, const float *gamma, const float *mean, const float *second, int is_meansq, float eps,
+                    const float *d_fw, const float *d_fb, float *dw, float *dbias, float *dgamma, float *dmean, float *dsecond,
+                    int K, int N, void *stream);
+
+/*
  * Batch statistics of the un-quantized pre-activation z = x W of QEinsumDenseBatchnorm.call
  * (src/hgq/layers/einsum_dense_batchnorm.py:99-124) WITHOUT materialising z: the contraction and the
  * column sums run in one pass over x, and the backward recomputes z tile by tile.

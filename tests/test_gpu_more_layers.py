@@ -401,3 +401,47 @@ def test_dense_moments_without_materialising_the_contraction(rows, K, N):
         scale = float(want.abs().max()) + 1e-12
         err = float((got.detach().cpu().double() - want.detach()).abs().max())
         assert err <= 2e-5 * scale, f'{name}: {err:.3e} vs scale {scale:.3e}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('K,N,with_gamma,is_meansq', [(16, 64, True, True), (64, 32, False, True), (5, 7, True, False), (300, 130, True, True)])
+def test_bn_fold_matches_the_reference_formula(K, N, with_gamma, is_meansq):
+    """ops.bn_fold against get_fused_qkernel_and_qbias' algebra (einsum_dense_batchnorm.py:160-172) and
+    the momentum update of call (:113-117): values against the fp32 formula, gradients against fp64 autograd."""
+    from hgq2_amd import ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(K * N)
+    w, bias = torch.randn(K, N, generator=g), torch.randn(N, generator=g)
+    gamma = torch.rand(N, generator=g) + 0.5 if with_gamma else None
+    mean = torch.randn(N, generator=g)
+    spread = torch.rand(N, generator=g) + 0.1
+    second = spread + mean * mean if is_meansq else spread
+    mm, mv = torch.randn(N, generator=g), torch.rand(N, generator=g)
+    eps, mom = 1e-7, 0.9
+    up_w, up_b = torch.randn(K, N, generator=g), torch.randn(N, generator=g)
+    # fp32 restatement in the reference's operation order
+    var32 = second - mean * mean if is_meansq else second
+    s32 = (gamma if with_gamma else 1) / torch.sqrt(var32 + eps)
+    want_w, want_b = w * s32, bias + (-mean * s32)
+    want_mm, want_mv = mm * mom + mean * (1.0 - mom), mv * mom + var32 * (1.0 - mom)
+    # fp64 autograd for the gradients
+    leaves = [t.double().requires_grad_(True) for t in (w, bias, mean, second)] + ([gamma.double().requires_grad_(True)] if with_gamma else [])
+    wd, bd, md, sd = leaves[:4]
+    var = sd - md * md if is_meansq else sd
+    sc = (leaves[4] if with_gamma else 1.0) / torch.sqrt(var + eps)
+    ((wd * sc * up_w.double()).sum() + ((bd - md * sc) * up_b.double()).sum()).backward()
+    dev_leaves = [t.to(dev).requires_grad_(True) for t in (w, bias, mean, second)] + ([gamma.to(dev).requires_grad_(True)] if with_gamma else [])
+    mmd, mvd = mm.to(dev), mv.to(dev)
+    fw, fb = ops.bn_fold(dev_leaves[0], dev_leaves[1], dev_leaves[4] if with_gamma else None, dev_leaves[2], dev_leaves[3], is_meansq, eps,
+                         mmd, mvd, mom)
+    ((fw * up_w.to(dev)).sum() + (fb * up_b.to(dev)).sum()).backward()
+    # sqrt and division differ by an ulp between numpy, torch-CPU and torch-GPU themselves: a few ulp here
+    for name, got, want in (('fused_w', fw, want_w), ('fused_b', fb, want_b), ('moving_mean', mmd, want_mm), ('moving_var', mvd, want_mv)):
+        err = float((got.detach().cpu() - want).abs().max())
+        assert err <= 6e-7 * (float(want.abs().max()) + 1e-12), f'{name}: {err:.3e}'
+    assert torch.equal(mmd.cpu(), want_mm)  # no sqrt / division involved
+    for name, got, ref_leaf in zip(('dw', 'dbias', 'dmean', 'dsecond', 'dgamma'), dev_leaves, leaves):
+        scale = float(ref_leaf.grad.abs().max()) + 1e-12
+        err = float((got.grad.cpu().double() - ref_leaf.grad).abs().max())
+        assert err <= 3e-5 * scale, f'{name}: {err:.3e} vs scale {scale:.3e}'
