@@ -267,6 +267,41 @@ __global__ __launch_bounds__(64) void bn_fold_bwd_kernel(const float *__restrict
     if (dmean) dmean[n] = -gb * scaler - (is_meansq ? 2.0f * m * dvar : 0.f);
 }
 
+// Bit-widths of a quantizer from its raw variables, in one launch each way (the host formula is a
+// chain of round / add / relu / cast launches per quantizer and step):
+//   KIF:  b = relu(rint(i) + rint(f));   KBI:  b = rint(fb)
+//   add_mode 0: b;  1: b + k (SAT `bits`, non-WRAP `fbits`);  2: b + k * (b > 0) (WRAP `fbits`)
+// Straight-through rounding: d b / d i = d b / d f = [rint(i) + rint(f) > 0] (KIF), d b / d fb = 1 (KBI).
+__global__ __launch_bounds__(256) void qbits_fwd_kernel(const uint8_t *__restrict__ k, const float *__restrict__ i,
+                                                        const float *__restrict__ fb, int64_t n, int kbi, int add_mode,
+                                                        float *__restrict__ out) {
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+        float b;
+        if (kbi) {
+            b = rintf(fb[e]);
+        } else {
+            const float sum = __fadd_rn(rintf(i[e]), rintf(fb[e]));
+            b = sum > 0.f ? sum : 0.f;
+        }
+        if (add_mode == 1) b = __fadd_rn(b, (float)k[e]);
+        else if (add_mode == 2) b = __fadd_rn(b, (float)k[e] * (b > 0.f ? 1.f : 0.f));
+        out[e] = b;
+    }
+}
+
+__global__ __launch_bounds__(256) void qbits_bwd_kernel(const float *__restrict__ g, const float *__restrict__ i,
+                                                        const float *__restrict__ fb, int64_t n, int kbi, float *__restrict__ di,
+                                                        float *__restrict__ dfb) {
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
+        if (kbi) {
+            dfb[e] = g[e];
+        } else {
+            const float v = __fadd_rn(rintf(i[e]), rintf(fb[e])) > 0.f ? g[e] : 0.f;
+            di[e] = v, dfb[e] = v;
+        }
+    }
+}
+
 // one thread per row; C is small (class count)
 __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict__ logits,
                                                         const int64_t *__restrict__ labels, float *loss,
@@ -440,6 +475,25 @@ extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels,
     const int grid = persistent_grid((rows + 255) / 256, 4);
     hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C);
     return check_launch("hgq_sparse_ce_fwd_bwd");
+}
+
+extern "C" int hgq_qbits_fwd(const uint8_t *k, const float *i, const float *fb, int64_t n, int kbi, int add_mode, float *out,
+                             void *stream) {
+    if (n < 0 || add_mode < 0 || add_mode > 2) return fail(HGQ_ERR_ARG, "hgq_qbits_fwd: bad arguments");
+    if (n == 0) return HGQ_OK;
+    if (!fb || !out || (!kbi && !i) || (add_mode && !k)) return fail(HGQ_ERR_ARG, "hgq_qbits_fwd: null pointer");
+    hipLaunchKernelGGL(qbits_fwd_kernel, dim3((unsigned)persistent_grid((n + 255) / 256, 8)), dim3(256), 0, (hipStream_t)stream, k, i, fb, n, kbi,
+                       add_mode, out);
+    return check_launch("hgq_qbits_fwd");
+}
+
+extern "C" int hgq_qbits_bwd(const float *g, const float *i, const float *fb, int64_t n, int kbi, float *di, float *dfb, void *stream) {
+    if (n < 0) return fail(HGQ_ERR_ARG, "hgq_qbits_bwd: bad size");
+    if (n == 0) return HGQ_OK;
+    if (!g || !dfb || (!kbi && (!i || !fb || !di))) return fail(HGQ_ERR_ARG, "hgq_qbits_bwd: null pointer");
+    hipLaunchKernelGGL(qbits_bwd_kernel, dim3((unsigned)persistent_grid((n + 255) / 256, 8)), dim3(256), 0, (hipStream_t)stream, g, i, fb, n, kbi,
+                       di, dfb);
+    return check_launch("hgq_qbits_bwd");
 }
 
 extern "C" int hgq_bn_fold_fwd(const float *w, const float *bias, const float *gamma, const float *mean, const float *second,

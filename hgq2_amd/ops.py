@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits']
 
 
 def _ptr(t: Tensor | None):
@@ -674,6 +674,39 @@ def _(w, gamma, mean, second, is_meansq, eps, d_fw, d_fb):
     return torch.empty_like(w), w.new_empty(n), w.new_empty(n if gamma.numel() else 0), w.new_empty(n), w.new_empty(n)
 
 
+@torch.library.custom_op('hgq::qbits_fwd', mutates_args=())
+def qbits_fwd(k: Tensor, i: Tensor, fb: Tensor, kbi: bool, add_mode: int) -> Tensor:
+    _check_f32('fb', fb)
+    n = fb.numel()
+    if not kbi:
+        _check_f32('i', i)
+        _need(i.numel() == n, 'i / f size mismatch')
+    if add_mode:
+        _need(k.dtype == torch.uint8 and k.is_cuda and k.is_contiguous() and k.numel() == n, 'k must be a contiguous uint8 GPU tensor of the same size')
+    out = torch.empty_like(fb)
+    _lib.check(_lib.load().hgq_qbits_fwd(_ptr(k), _ptr(i), _ptr(fb), n, int(kbi), add_mode, _ptr(out), _stream()), 'hgq_qbits_fwd')
+    return out
+
+
+@qbits_fwd.register_fake
+def _(k, i, fb, kbi, add_mode):
+    return torch.empty_like(fb)
+
+
+@torch.library.custom_op('hgq::qbits_bwd', mutates_args=())
+def qbits_bwd(g: Tensor, i: Tensor, fb: Tensor, kbi: bool) -> tuple[Tensor, Tensor]:
+    _check_f32('g', g)
+    dfb = torch.empty_like(fb)
+    di = torch.empty_like(fb) if not kbi else fb.new_empty(0)
+    _lib.check(_lib.load().hgq_qbits_bwd(_ptr(g), _ptr(i), _ptr(fb), fb.numel(), int(kbi), _ptr(di), _ptr(dfb), _stream()), 'hgq_qbits_bwd')
+    return di, dfb
+
+
+@qbits_bwd.register_fake
+def _(g, i, fb, kbi):
+    return (torch.empty_like(fb) if not kbi else fb.new_empty(0)), torch.empty_like(fb)
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -950,6 +983,27 @@ def bn_fold(w2d: Tensor, bias: Tensor, gamma, mean: Tensor, second: Tensor, is_m
     return _BnFold.apply(w2d.contiguous(), bias.contiguous(), gamma.contiguous() if gamma is not None else empty, mean.contiguous(),
                          second.contiguous(), bool(is_meansq), float(eps), moving_mean if moving_mean is not None else empty,
                          moving_var if moving_var is not None else empty, float(momentum))
+
+
+class _QBits(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, k, i, fb, kbi, add_mode):
+        ctx.save_for_backward(i, fb)
+        ctx.kbi = kbi
+        return qbits_fwd(k, i, fb, kbi, add_mode)
+
+    @staticmethod
+    def backward(ctx, g):
+        i, fb = ctx.saved_tensors
+        di, dfb = qbits_bwd(g.contiguous(), i, fb, ctx.kbi)
+        return None, (None if ctx.kbi else di), dfb, None, None
+
+
+def qbits(k: Tensor, i, fb: Tensor, kbi: bool, add_mode: int = 0) -> Tensor:
+    """Bit-widths ``relu(round(i) + round(f))`` (KIF) or ``round(b)`` (KBI) of raw quantizer variables, plus ``k``
+    (``add_mode`` 1) or ``k * (b > 0)`` (``add_mode`` 2), with straight-through rounding; shaped like ``fb``."""
+    empty = fb.new_empty(0)
+    return _QBits.apply(k if add_mode else empty, i if not kbi else empty, fb, bool(kbi), int(add_mode))
 
 
 class _AttnScores(torch.autograd.Function):

@@ -63,15 +63,31 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
     def i_decay_speed(self):
         return self._i_decay_speed
 
-    # ---- bit-width views (torch ops on the small bit-width tensors, differentiable)
+    # ---- bit-width views (differentiable).  On the GPU one launch each way (`ops.qbits`); the torch
+    # formula below is the same arithmetic as a chain of round / add / relu / cast launches.
+    def _fused_bits(self, add_mode: int):
+        kbi = not hasattr(self, '_f')
+        fb = self._b if kbi else self._f
+        if not (fb.is_cuda and fb.is_contiguous() and self._k.is_contiguous() and (kbi or self._i.is_contiguous())):
+            return None
+        from ... import ops
+
+        return ops.qbits(self._k, None if kbi else self._i, fb, kbi, add_mode)
+
     @property
     def bits(self):
+        fused = self._fused_bits(1 if self.overflow_mode == 'SAT' else 0)
+        if fused is not None:
+            return fused
         if self.overflow_mode != 'SAT':
             return self.b
         return self.b + self.k
 
     @property
     def fbits(self):
+        fused = self._fused_bits(2 if self.overflow_mode == 'WRAP' else 1)
+        if fused is not None:
+            return fused
         b = self.b
         if self.overflow_mode == 'WRAP':
             return b + self.k * (b > 0).to(b.dtype)

@@ -342,6 +342,17 @@ int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float
                    float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
 
 /*
+ * Bit-widths of a quantizer from its raw variables: the `b`, `bits` and `fbits` properties of
+ * FixedPointQuantizerKIF / KBI (src/hgq/quantizer/internal/fixed_point_quantizer.py:60-79,
+ * :206-215, :311-320) in one launch, with the straight-through gradient of round_conv.
+ *   KIF (kbi = 0): b = relu(rint(i) + rint(fb));   KBI (kbi = 1): b = rint(fb) (i unused)
+ *   add_mode 0: b;  1: b + k;  2: b + k * (b > 0).   k is the uint8 keep-negative variable.
+ *   backward: KIF di = dfb = g * [rint(i) + rint(fb) > 0];  KBI dfb = g (di untouched).
+ */
+int hgq_qbits_fwd(const uint8_t *k, const float *i, const float *fb, int64_t n, int kbi, int add_mode, float *out, void *stream);
+int hgq_qbits_bwd(const float *g, const float *i, const float *fb, int64_t n, int kbi, float *di, float *dfb, void *stream);
+
+/*
  * Batch-norm folding of QEinsumDenseBatchnorm.get_fused_qkernel_and_qbias
  * (src/hgq/layers/einsum_dense_batchnorm.py:160-172) for a [K, N] kernel normalised over its N
  * outputs, before the kernel / bias quantizers:
