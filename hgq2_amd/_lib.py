@@ -45,6 +45,8 @@ SIGNATURES = {
         [c_void_p, c_int, c_float, c_void_p, c_void_p] + [c_void_p] * 3 + [c_int64, c_int, c_int] + [c_void_p] * 4
         + [c_float, c_float, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p],
     ),
+    'hgq_ebops_finish_fwd': (c_int, [c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
+    'hgq_ebops_finish_bwd': (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_void_p]),
     'hgq_qbits_fwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     'hgq_qbits_bwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p]),
     'hgq_bn_fold_fwd': (c_int, [c_void_p] * 5 + [c_int, c_float] + [c_void_p] * 4 + [c_float, c_float, c_int, c_int, c_void_p]),

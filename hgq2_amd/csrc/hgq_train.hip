@@ -302,6 +302,17 @@ __global__ __launch_bounds__(256) void qbits_bwd_kernel(const float *__restrict_
     }
 }
 
+// The tail of QLayerBase's call wrapper on a scalar: ebops <- ebops * factor, the uint32 variable,
+// and the loss term ebops * beta, in one launch (and its gradient in another).
+__global__ void ebops_finish_fwd_kernel(const float *ebops, float factor, const float *beta, uint32_t *ebops_u32, float *out) {
+    const float e = __fmul_rn(ebops[0], factor);
+    if (ebops_u32) ebops_u32[0] = (uint32_t)(int64_t)e;
+    out[0] = __fmul_rn(e, beta[0]);
+}
+__global__ void ebops_finish_bwd_kernel(const float *g, const float *beta, float factor, float *d_ebops) {
+    d_ebops[0] = __fmul_rn(__fmul_rn(g[0], beta[0]), factor);
+}
+
 // one thread per row; C is small (class count)
 __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict__ logits,
                                                         const int64_t *__restrict__ labels, float *loss,
@@ -475,6 +486,18 @@ extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels,
     const int grid = persistent_grid((rows + 255) / 256, 4);
     hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C);
     return check_launch("hgq_sparse_ce_fwd_bwd");
+}
+
+extern "C" int hgq_ebops_finish_fwd(const float *ebops, float factor, const float *beta, uint32_t *ebops_u32, float *out, void *stream) {
+    if (!ebops || !beta || !out) return fail(HGQ_ERR_ARG, "hgq_ebops_finish_fwd: null pointer");
+    hipLaunchKernelGGL(ebops_finish_fwd_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, ebops, factor, beta, ebops_u32, out);
+    return check_launch("hgq_ebops_finish_fwd");
+}
+
+extern "C" int hgq_ebops_finish_bwd(const float *g, const float *beta, float factor, float *d_ebops, void *stream) {
+    if (!g || !beta || !d_ebops) return fail(HGQ_ERR_ARG, "hgq_ebops_finish_bwd: null pointer");
+    hipLaunchKernelGGL(ebops_finish_bwd_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, g, beta, factor, d_ebops);
+    return check_launch("hgq_ebops_finish_bwd");
 }
 
 extern "C" int hgq_qbits_fwd(const uint8_t *k, const float *i, const float *fb, int64_t n, int kbi, int add_mode, float *out,

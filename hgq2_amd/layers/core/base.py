@@ -93,7 +93,12 @@ class QLayerBase(Layer):
     def _ebops_loss_term(self, *shapes):
         """``ebops = _compute_ebops(...) * ebops_factor; _ebops.assign(cast(ebops, uint32))``; returns
         the loss term ``ebops * beta`` (reference :101-104).  Layers with a fused kernel override this."""
-        ebops = self._compute_ebops(*shapes) * self.ebops_factor
+        ebops = self._compute_ebops(*shapes)
+        if ebops.is_cuda and ebops.dtype == torch.float32 and ebops.numel() == 1 and self._beta.dtype == torch.float32:
+            from ... import ops
+
+            return ops.ebops_finish(ebops, self.ebops_factor, self._beta, self._ebops)  # one launch instead of five
+        ebops = ebops * self.ebops_factor
         with torch.no_grad():
             self._ebops.view(torch.int32).copy_(ebops.detach().to(torch.int64).to(torch.int32))
         return ebops * self._beta

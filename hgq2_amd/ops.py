@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits', 'ebops_finish']
 
 
 def _ptr(t: Tensor | None):
@@ -707,6 +707,33 @@ def _(g, i, fb, kbi):
     return (torch.empty_like(fb) if not kbi else fb.new_empty(0)), torch.empty_like(fb)
 
 
+@torch.library.custom_op('hgq::ebops_finish_fwd', mutates_args=('ebops_var',))
+def ebops_finish_fwd(ebops: Tensor, factor: float, beta: Tensor, ebops_var: Tensor) -> Tensor:
+    _check_f32('ebops', ebops), _check_f32('beta', beta)
+    _need(ebops.numel() == 1 and beta.numel() == 1 and ebops_var.numel() == 1 and ebops_var.element_size() == 4, 'scalars expected')
+    out = torch.empty((), dtype=torch.float32, device=ebops.device)
+    _lib.check(_lib.load().hgq_ebops_finish_fwd(_ptr(ebops), factor, _ptr(beta), _ptr(ebops_var), _ptr(out), _stream()), 'hgq_ebops_finish_fwd')
+    return out
+
+
+@ebops_finish_fwd.register_fake
+def _(ebops, factor, beta, ebops_var):
+    return ebops.new_empty(())
+
+
+@torch.library.custom_op('hgq::ebops_finish_bwd', mutates_args=())
+def ebops_finish_bwd(g: Tensor, beta: Tensor, factor: float) -> Tensor:
+    _check_f32('g', g)
+    d = torch.empty((), dtype=torch.float32, device=g.device)
+    _lib.check(_lib.load().hgq_ebops_finish_bwd(_ptr(g), _ptr(beta), factor, _ptr(d), _stream()), 'hgq_ebops_finish_bwd')
+    return d
+
+
+@ebops_finish_bwd.register_fake
+def _(g, beta, factor):
+    return g.new_empty(())
+
+
 # ======================================================================================
 # autograd pairing
 # ======================================================================================
@@ -1004,6 +1031,24 @@ def qbits(k: Tensor, i, fb: Tensor, kbi: bool, add_mode: int = 0) -> Tensor:
     (``add_mode`` 1) or ``k * (b > 0)`` (``add_mode`` 2), with straight-through rounding; shaped like ``fb``."""
     empty = fb.new_empty(0)
     return _QBits.apply(k if add_mode else empty, i if not kbi else empty, fb, bool(kbi), int(add_mode))
+
+
+class _EbopsFinish(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, ebops, factor, beta, ebops_var):
+        ctx.save_for_backward(beta)
+        ctx.factor, ctx.shape = factor, ebops.shape
+        return ebops_finish_fwd(ebops, factor, beta, ebops_var)
+
+    @staticmethod
+    def backward(ctx, g):
+        (beta,) = ctx.saved_tensors
+        return ebops_finish_bwd(g.contiguous(), beta, ctx.factor).view(ctx.shape), None, None, None
+
+
+def ebops_finish(ebops: Tensor, factor: float, beta: Tensor, ebops_var: Tensor) -> Tensor:
+    """``ebops * factor`` stored into the uint32 variable and returned times ``beta`` (the loss term)."""
+    return _EbopsFinish.apply(ebops.contiguous(), float(factor), beta, ebops_var)
 
 
 class _AttnScores(torch.autograd.Function):

@@ -342,6 +342,14 @@ int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float
                    float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
 
 /*
+ * The scalar tail of QLayerBase.call (src/hgq/layers/core/base.py:101-104):
+ *     ebops = ebops * ebops_factor;  self._ebops.assign(cast(ebops, uint32));  loss term = ebops * beta
+ * forward writes the uint32 variable (may be NULL) and out [1]; backward: d_ebops = (g * beta) * factor.
+ */
+int hgq_ebops_finish_fwd(const float *ebops, float factor, const float *beta, uint32_t *ebops_u32, float *out, void *stream);
+int hgq_ebops_finish_bwd(const float *g, const float *beta, float factor, float *d_ebops, void *stream);
+
+/*
  * Bit-widths of a quantizer from its raw variables: the `b`, `bits` and `fbits` properties of
  * FixedPointQuantizerKIF / KBI (src/hgq/quantizer/internal/fixed_point_quantizer.py:60-79,
  * :206-215, :311-320) in one launch, with the straight-through gradient of round_conv.

@@ -260,3 +260,21 @@ def test_mse_loss_and_gradient(n, with_target):
     want_g = 3.0 * 2.0 * ref_d / n
     assert float((p.grad.cpu().double() - want_g).abs().max()) <= 2e-6 * float(want_g.abs().max())
     assert float(ops.mse(p.detach(), t)) == float(loss)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('value', [0.0, 1234.75, 3.0e9, 5.0e9])
+def test_ebops_finish_scalar_tail(dev, value):
+    """ebops * factor -> uint32 variable and loss term ebops * beta (reference src/hgq/layers/core/base.py:101-104);
+    5e9 wraps modulo 2**32 like the reference's cast chain."""
+    from hgq2_amd import ops
+
+    e = torch.tensor(value, device=dev, requires_grad=True)
+    beta = torch.tensor(3.5e-6, device=dev)
+    var = torch.zeros((), dtype=torch.uint32, device=dev)
+    out = ops.ebops_finish(e, 0.5, beta, var)
+    out.backward(torch.tensor(2.0, device=dev))
+    ef = np.float32(value) * np.float32(0.5)
+    assert out.item() == float(ef * np.float32(3.5e-6))
+    assert int(var.view(torch.int32).item()) & 0xFFFFFFFF == int(ef) & 0xFFFFFFFF
+    assert e.grad.item() == float(np.float32(2.0) * np.float32(3.5e-6) * np.float32(0.5))
