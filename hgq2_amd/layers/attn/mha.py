@@ -22,6 +22,8 @@ _OUT_EQ, _OUT_BIAS = 'abcd,cde->abe', 'e'
 _DOT_EQ = 'aecd,abcd->acbe'      # key [B,S,N,H], query [B,T,N,H] -> scores [B,N,T,S]
 _COMBINE_EQ = 'acbe,aecd->abcd'  # scores [B,N,T,S], value [B,S,N,H] -> [B,T,N,H]
 
+FUSED = True  # module switch: False composes scores, softmax and combine from their own kernels (cross-check)
+
 
 class QMultiHeadAttention(QLayerBase):
     __output_quantizer_handled__ = True
@@ -171,7 +173,7 @@ class QMultiHeadAttention(QLayerBase):
         q = self._query_dense(query)
         k = self._key_dense(key)
         v = self._value_dense(value)
-        out, scores = self._compute_attention(q, k, v, attention_mask, training)
+        out, scores = self._compute_attention(q, k, v, attention_mask, training, need_scores=return_attention_scores)
         out = self._output_dense(out)
         if self.enable_oq:
             out = self.oq(out, training=training)
@@ -179,9 +181,13 @@ class QMultiHeadAttention(QLayerBase):
             return out, scores
         return out
 
-    def _compute_attention(self, query, key, value, attention_mask=None, training=None):
+    def _compute_attention(self, query, key, value, attention_mask=None, training=None, need_scores=True):
         if self._inverse_sqrt_key_dim != 1.0:  # 1 after build: the scale lives in the softmax's exp table
             query = query * self._inverse_sqrt_key_dim
+        if FUSED and not need_scores and attention_mask is None and not (self._dropout and training):
+            stand_in = self._softmax.attention_plan(query, key, value, training)
+            if stand_in is not None:  # one kernel each way; scores and probabilities are never written
+                return self._softmax(stand_in, attention=(query, key, value)), None
         own = query.is_cuda and max(query.shape[1], key.shape[1], query.shape[3], value.shape[3]) <= ops.ATTN_MAX
         scores = ops.attn_scores(query, key) if own else torch.einsum(_DOT_EQ, key, query)
         mask = None

@@ -136,11 +136,15 @@ class QSoftmax(QLayerBaseSingleInput):
             return None  # a row layout outside the kernel family
         return qs
 
-    def _call_fused(self, x, training, qs):
+    def _call_fused(self, x, training, qs, attention=None):
         e, v = self.exp_table, self.inv_table
         owners = (e.iq, e.oq, v.iq, v.oq, self.oq if self.enable_oq else None)
         track_mask = sum(bit for bit, q in zip((1, 0, 2, 0, 4), qs) if q is not None and q[4])
-        y, a1, a3, ao = ops.qsoftmax(x, [None if q is None else q[:4] for q in qs], self.input_scaler, epsilon(), track_mask)
+        descs = [None if q is None else q[:4] for q in qs]
+        if attention is not None:  # scores and probabilities stay inside the kernel; y is the combined output
+            y, a1, a3, ao = ops.qattention(*attention, descs, self.input_scaler, epsilon(), track_mask)
+        else:
+            y, a1, a3, ao = ops.qsoftmax(x, descs, self.input_scaler, epsilon(), track_mask)
         for amax, n in ((a1, 0), (a3, 2), (ao, 4)):
             if amax.numel():
                 owners[n].quantizer._track(amax, True)
@@ -152,7 +156,25 @@ class QSoftmax(QLayerBaseSingleInput):
                 table.add_loss(table._ebops_loss_term((1,) + shape[1:]))
         return y
 
-    def call(self, inputs, training=None, mask=None):
+    def attention_plan(self, query, key, value, training):
+        """Whether ``self(stand_in, attention=(query, key, value))`` can run scores, softmax and combine as one kernel;
+        returns the shape-only stand-in for the scores, or ``None``."""
+        if self.enable_iq or not query.is_cuda or query.dim() != 4:
+            return None
+        B, T, N, _ = query.shape
+        stand_in = query.new_empty(()).expand(B, N, T, key.shape[1])
+        qs = self._fused_plan(stand_in, training, None)
+        if qs is None:
+            return None
+        entries = qs[4][1].numel() if qs[4] is not None else 0
+        inner = self.oq.quantizer if qs[4] is not None else None
+        saturates = inner is not None and (inner.overflow_mode != 'WRAP' or isinstance(inner, FixedPointQuantizerKBI))
+        return stand_in if ops.qattention_supported(query, key, value, entries, saturates) else None
+
+    def call(self, inputs, training=None, mask=None, attention=None):
+        if attention is not None:  # `inputs` carries the shape of the scores only (see attention_plan)
+            self._oq_applied_in_call = self.enable_oq
+            return self._call_fused(inputs, training, self._fused_plan(inputs, training, None), attention)
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
         qs = self._fused_plan(inputs, training, mask)

@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits', 'ebops_finish']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits', 'ebops_finish', 'qattention', 'qattention_supported']
 
 
 def _ptr(t: Tensor | None):
@@ -337,6 +337,92 @@ def qsoftmax_bwd(dy: Tensor, x: Tensor, ks: Sequence[Tensor], is_: Sequence[Tens
 def _(dy, x, ks, is_, fbs, modes, input_scaler, eps):
     n_o = is_[4].numel()
     return torch.empty_like(x), x.new_empty(8), x.new_empty(n_o), x.new_empty(n_o)
+
+
+def _qattn_dims(q: Tensor, k: Tensor, v: Tensor):
+    _check_f32('query', q), _check_f32('key', k), _check_f32('value', v)
+    _need(q.dim() == 4 and k.dim() == 4 and v.shape == k.shape and q.shape[0] == k.shape[0] and q.shape[2:] == k.shape[2:],
+          'query [B, T, N, H] and key / value [B, S, N, H] are expected')
+    B, T, N, H = q.shape
+    return B, T, k.shape[1], N, H
+
+
+def _attn_bw_rows(S: int, oq_i: Tensor) -> int:
+    if oq_i.numel() == 0:
+        return 1
+    _need(oq_i.numel() % S == 0, 'the output quantizer table must be [bw_rows, S]')
+    return oq_i.numel() // S
+
+
+def qattention_supported(q: Tensor, k: Tensor, v: Tensor, oq_entries: int, oq_saturates: bool) -> bool:
+    """Whether ``qattention`` takes these operands (else compose attn_scores, qsoftmax, attn_combine)."""
+    if not (q.is_cuda and q.dtype == torch.float32 and q.dim() == 4 and k.dim() == 4 and v.shape == k.shape) or oq_saturates:
+        return False
+    B, T, N, H = q.shape
+    S = k.shape[1]
+    if k.shape[0] != B or tuple(k.shape[2:]) != (N, H) or (oq_entries and oq_entries % S):
+        return False
+    return _lib.load().hgq_qattention_bwd_workspace(B, T, S, N, H, max(oq_entries // S, 1), int(oq_entries > 0)) >= 0
+
+
+@torch.library.custom_op('hgq::qattention_fwd', mutates_args=())
+def qattention_fwd(q: Tensor, k: Tensor, v: Tensor, ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor],
+                   modes: Sequence[int], input_scaler: float, eps: float, track_mask: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    B, T, S, N, H = _qattn_dims(q, k, v)
+    descs = _qdescs(ks, is_, fbs, modes)
+    bw_rows = _attn_bw_rows(S, is_[4])
+    out = torch.empty_like(q)
+    i32 = dict(dtype=torch.int32, device=q.device)
+    a1 = torch.empty(1 if track_mask & 1 else 0, **i32)
+    a3 = torch.empty(1 if track_mask & 2 else 0, **i32)
+    ao = torch.empty(bw_rows * S if track_mask & 4 else 0, **i32)
+    lib = _lib.load()
+    n_ws = lib.hgq_qattention_fwd_workspace(B, T, S, N, H, bw_rows, int(bool(track_mask & 4)))
+    _need(n_ws >= 0, 'hgq_qattention_fwd_workspace rejected the shape')
+    ws = torch.empty(int(n_ws), **i32)
+    rc = lib.hgq_qattention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), B, T, S, N, H, bw_rows, input_scaler, eps,
+                                *[ctypes.addressof(d) for d in descs], _ptr(a1), _ptr(a3), _ptr(ao), _ptr(ws), _stream())
+    _lib.check(rc, 'hgq_qattention_fwd')
+    return out, a1, a3, ao
+
+
+@qattention_fwd.register_fake
+def _(q, k, v, ks, is_, fbs, modes, input_scaler, eps, track_mask):
+    n_o = is_[4].numel() if track_mask & 4 else 0
+    return (torch.empty_like(q), q.new_empty(1 if track_mask & 1 else 0, dtype=torch.int32),
+            q.new_empty(1 if track_mask & 2 else 0, dtype=torch.int32), q.new_empty(n_o, dtype=torch.int32))
+
+
+@torch.library.custom_op('hgq::qattention_bwd', mutates_args=())
+def qattention_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, ks: Sequence[Tensor], is_: Sequence[Tensor],
+                   fbs: Sequence[Tensor], modes: Sequence[int], input_scaler: float,
+                   eps: float) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
+    B, T, S, N, H = _qattn_dims(q, k, v)
+    _check_f32('dout', dout)
+    _need(dout.shape == q.shape, 'dout and query differ in shape')
+    descs = _qdescs(ks, is_, fbs, modes)
+    has_oq = is_[4].numel() > 0
+    bw_rows = _attn_bw_rows(S, is_[4])
+    lib = _lib.load()
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    f32 = dict(dtype=torch.float32, device=q.device)
+    g_shared = torch.empty(8, **f32)
+    g_oi = torch.empty(bw_rows * S if has_oq else 0, **f32)
+    g_of = torch.empty(bw_rows * S if has_oq else 0, **f32)
+    n_ws = lib.hgq_qattention_bwd_workspace(B, T, S, N, H, bw_rows, int(has_oq))
+    _need(n_ws >= 0, 'hgq_qattention_bwd_workspace rejected the shape')
+    ws = torch.empty(max(int(n_ws), 1), **f32)
+    rc = lib.hgq_qattention_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(dq), _ptr(dk), _ptr(dv), B, T, S, N, H, bw_rows,
+                                input_scaler, eps, *[ctypes.addressof(d) for d in descs], _ptr(g_shared), _ptr(g_oi), _ptr(g_of),
+                                _ptr(ws), _stream())
+    _lib.check(rc, 'hgq_qattention_bwd')
+    return dq, dk, dv, g_shared, g_oi, g_of
+
+
+@qattention_bwd.register_fake
+def _(dout, q, k, v, ks, is_, fbs, modes, input_scaler, eps):
+    n_o = is_[4].numel()
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), q.new_empty(8), q.new_empty(n_o), q.new_empty(n_o)
 
 
 def _geom(g: Sequence[int]):
@@ -912,6 +998,59 @@ def qsoftmax(x: Tensor, quantizers, input_scaler: float, eps: float, track_mask:
             flat += [k.contiguous(), i.contiguous(), fb.contiguous()]
             modes.append(int(mode))
     return _QSoftmax.apply(x.contiguous(), tuple(modes), float(input_scaler), float(eps), int(track_mask), *flat)
+
+
+class _QAttention(torch.autograd.Function):
+    """Arguments after the scalars: k, i, fb of exp_iq, exp_oq, inv_iq, inv_oq, oq (15 tensors, empty = absent)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, modes, input_scaler, eps, track_mask, *qvars):
+        ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
+        out, a1, a3, ao = qattention_fwd(q, k, v, ks, is_, fbs, list(modes), input_scaler, eps, track_mask)
+        ctx.save_for_backward(q, k, v, *qvars)
+        ctx.modes, ctx.input_scaler, ctx.eps = tuple(modes), input_scaler, eps
+        ctx.mark_non_differentiable(a1, a3, ao)
+        ctx.set_materialize_grads(False)
+        return out, a1, a3, ao
+
+    @staticmethod
+    def backward(ctx, gout, *_unused):
+        n_in = 7 + 15
+        if gout is None:
+            return (None,) * n_in
+        q, k, v, *qvars = ctx.saved_tensors
+        ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
+        dq, dk, dv, g_shared, g_oi, g_of = qattention_bwd(gout.contiguous(), q, k, v, ks, is_, fbs, list(ctx.modes),
+                                                          ctx.input_scaler, ctx.eps)
+        need = ctx.needs_input_grad
+        grads = [dq if need[0] else None, dk if need[1] else None, dv if need[2] else None, None, None, None, None]
+        for n in range(5):
+            gi = g_shared[2 * n] if n < 4 else g_oi
+            gf = g_shared[2 * n + 1] if n < 4 else g_of
+            present = ks[n].numel() > 0
+            base = 7 + 3 * n
+            grads.append(None)
+            grads.append(gi.view(is_[n].shape) if present and need[base + 1] else None)
+            grads.append(gf.view(fbs[n].shape) if present and need[base + 2] else None)
+        return tuple(grads)
+
+
+def qattention(q: Tensor, k: Tensor, v: Tensor, quantizers, input_scaler: float, eps: float, track_mask: int = 0):
+    """``combine(qsoftmax(scores(q, k)), v)`` without materialising scores or probabilities.  ``quantizers`` as for
+    ``qsoftmax``.  Returns ``(out, amax_exp_iq, amax_inv_iq, amax_oq)``."""
+    e_f = q.new_empty(0)
+    e_k = torch.empty(0, dtype=torch.uint8, device=q.device)
+    flat, modes = [], []
+    for qz in quantizers:
+        if qz is None:
+            flat += [e_k, e_f, e_f]
+            modes.append(0)
+        else:
+            kk, i, fb, mode = qz
+            flat += [kk.contiguous(), i.contiguous(), fb.contiguous()]
+            modes.append(int(mode))
+    return _QAttention.apply(q.contiguous(), k.contiguous(), v.contiguous(), tuple(modes), float(input_scaler), float(eps),
+                             int(track_mask), *flat)
 
 
 class _Conv2D(torch.autograd.Function):

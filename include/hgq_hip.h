@@ -425,6 +425,32 @@ int hgq_attn_combine_bwd(const float *dout, const float *probs, const float *val
                          int S, int N, int H, void *stream);
 
 /*
+ * The attention core of QMultiHeadAttention._compute_attention (src/hgq/layers/attn/mha.py:418-470) with
+ * the table softmax of QSoftmax.call (src/hgq/layers/softmax.py:121-141) in one pass each way:
+ *     out = combine(qsoftmax(scores(query, key)), value)
+ * scores and probabilities are never written: the backward pass recomputes them from query / key /
+ * value.  Quantizer descriptors, trackers, g_shared / g_oq_i / g_oq_fb and bw_rows (rows of the output
+ * quantizer's [bw_rows, S] table; row (n * T + t) % bw_rows serves head n, query position t; must
+ * divide N * T) are those of hgq_qsoftmax_fwd / _bwd.  Supported: T = S = 32 or 64, H = 8, 16 or 32
+ * (query / key and value alike), N * T / 32 <= 8, N * H <= 64, an output quantizer that does not
+ * saturate and is not of the (k, b, i) kind in the backward pass; anything else returns
+ * HGQ_ERR_UNSUPPORTED (the workspace queries return -1) and the caller composes hgq_attn_scores_*,
+ * hgq_qsoftmax_* and hgq_attn_combine_*.  Operands and workspaces 16-byte aligned.  The forward
+ * workspace (needed with amax_oq only) holds one abs-max slice per workgroup: entries are combined by a
+ * second launch, not by atomics.
+ */
+int hgq_qattention_fwd(const float *query, const float *key, const float *value, float *out, int B, int T, int S, int N, int H,
+                       int64_t bw_rows, float input_scaler, float eps, const hgq_qdesc *exp_iq, const hgq_qdesc *exp_oq,
+                       const hgq_qdesc *inv_iq, const hgq_qdesc *inv_oq, const hgq_qdesc *oq, uint32_t *amax_exp_iq,
+                       uint32_t *amax_inv_iq, uint32_t *amax_oq, void *workspace, void *stream);
+int64_t hgq_qattention_fwd_workspace(int B, int T, int S, int N, int H, int64_t bw_rows, int track_oq); /* 4-byte words */
+int64_t hgq_qattention_bwd_workspace(int B, int T, int S, int N, int H, int64_t bw_rows, int has_oq);
+int hgq_qattention_bwd(const float *dout, const float *query, const float *key, const float *value, float *dquery, float *dkey,
+                       float *dvalue, int B, int T, int S, int N, int H, int64_t bw_rows, float input_scaler, float eps,
+                       const hgq_qdesc *exp_iq, const hgq_qdesc *exp_oq, const hgq_qdesc *inv_iq, const hgq_qdesc *inv_oq,
+                       const hgq_qdesc *oq, float *g_shared, float *g_oq_i, float *g_oq_fb, float *workspace, void *stream);
+
+/*
  * 2-D max / average pooling on channels-last tensors, forward and backward.  Replaces the Keras
  * MaxPooling2D / AveragePooling2D `call` that QMaxPooling2D / QAveragePooling2D apply to the
  * quantized input (src/hgq/layers/pooling.py:23-47; the Keras torch backend transposes to

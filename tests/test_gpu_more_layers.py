@@ -445,3 +445,60 @@ def test_bn_fold_matches_the_reference_formula(K, N, with_gamma, is_meansq):
         scale = float(ref_leaf.grad.abs().max()) + 1e-12
         err = float((got.grad.cpu().double() - ref_leaf.grad).abs().max())
         assert err <= 3e-5 * scale, f'{name}: {err:.3e} vs scale {scale:.3e}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('batch,seq,heads,key_dim', [(2048, 64, 4, 16), (300, 32, 2, 8), (37, 32, 2, 32), (5, 64, 1, 8)])
+def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim):
+    """scores -> table softmax -> combine as one kernel each way (hgq_qattention_fwd / _bwd) against the same
+    layer composing hgq_attn_scores_*, hgq_qsoftmax_* and hgq_attn_combine_*: outputs, tracked integer
+    bits and loss terms bit-identical, gradients within fp32 summation noise."""
+    import hgq2_amd.layers.attn.mha as mha
+    from hgq2_amd.layers import QMultiHeadAttention
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(batch + seq)
+    torch.manual_seed(batch)
+    with readme_scopes():
+        layer = QMultiHeadAttention(num_heads=heads, key_dim=key_dim)
+    x = torch.randn(batch, seq, heads * key_dim, generator=g)
+    with torch.no_grad():
+        layer(x.to(dev), training=True)
+    _perturb(layer, g)
+    state = {n: p.detach().clone() for n, p in layer.state_dict().items()}
+    w = torch.randn(batch, seq, heads * key_dim, generator=g).to(dev)
+    sm = layer._softmax
+    params = lambda: [layer._query_dense._kernel, layer._key_dense._kernel, layer._value_dense._kernel,  # noqa: E731
+                      layer._query_dense.oq.quantizer._f, layer._key_dense.oq.quantizer._f, layer._value_dense.oq.quantizer._f,
+                      sm.oq.quantizer._f, sm.exp_table.iq.quantizer._f, sm.exp_table.iq.quantizer._i, sm.exp_table.oq.quantizer._b,
+                      sm.exp_table.oq.quantizer._i, sm.inv_table.iq.quantizer._f, sm.inv_table.oq.quantizer._b,
+                      sm.inv_table.oq.quantizer._i]
+    results = []
+    for fused in (True, False):
+        layer.load_state_dict(state)
+        mha.FUSED = fused
+        try:
+            xp = x.to(dev).requires_grad_(True)
+            y = layer(xp, training=True)
+            (y * w).sum().backward()
+        finally:
+            mha.FUSED = True
+        grads = [xp.grad.detach().clone()] + [None if p.grad is None else p.grad.detach().clone() for p in params()]
+        for p in params():
+            p.grad = None
+        i_vars = [q.quantizer._i.detach().clone() for q in (sm.exp_table.iq, sm.inv_table.iq, sm.oq)]
+        results.append((y.detach(), grads, i_vars, [float(t.detach()) for t in layer.losses]))
+    (y1, g1, i1, l1), (y2, g2, i2, l2) = results
+    assert torch.equal(y1, y2), f'outputs differ by {float((y1 - y2).abs().max()):.3e}'
+    for a, b in zip(i1, i2):
+        assert torch.equal(a, b)
+    assert l1 == l2
+    names = ['x', 'wq', 'wk', 'wv', 'q_oq_f', 'k_oq_f', 'v_oq_f', 'sm_oq_f', 'exp_iq_f', 'exp_iq_i', 'exp_oq_b', 'exp_oq_i',
+             'inv_iq_f', 'inv_oq_b', 'inv_oq_i']
+    for n, a, b in zip(names, g1, g2):
+        assert (a is None) == (b is None), n
+        if a is None:
+            continue
+        scale = b.abs().max().item() + 1e-12
+        tol = (2e-5 if n in ('x', 'sm_oq_f') else 3e-4) * scale
+        assert float((a - b).abs().max()) <= tol, f'grad {n}: {float((a - b).abs().max()):.3e} vs scale {scale:.3e}'
