@@ -112,7 +112,8 @@ __device__ __forceinline__ floatx16 contract_keys(const float *tile, int col0, i
     return o;
 }
 
-// D[h][s] = sum_t tile[t][col0 + h] * buf[t][s0 + s], t < 32 * TH (buf rows are QA_LD words apart).
+// D[h][s] = sum_t tile[t][col0 + h] * buf[t][s0 + s], t < 32 * TH (buf rows are QA_LD words apart).  A step pairs
+// rows t and t + 8: 8 * QA_LD = 32 (mod 64) words, so the two half-wavefronts read disjoint banks.
 template <int TH>
 __device__ __forceinline__ floatx16 contract_queries(const float *tile, int col0, const float *buf, int s0, int t_l, int hf) {
     floatx16 o = {0};
@@ -121,7 +122,7 @@ __device__ __forceinline__ floatx16 contract_queries(const float *tile, int col0
         float a[16], b[16];
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-            const int t = 2 * (j0 + j) + hf;
+            const int t = 2 * j0 + (j >> 3) * 16 + (j & 7) + 8 * hf;
             a[j] = tile[t * QA_LD + col0 + t_l];
             b[j] = buf[t * QA_LD + s0 + t_l];
         }
@@ -143,6 +144,16 @@ __device__ __forceinline__ void store_rows(const floatx16 &o, float *__restrict_
             v.x = o[4 * g], v.y = o[4 * g + 1], v.z = o[4 * g + 2], v.w = o[4 * g + 3];
             *(f32x4_t *)(dst + (int64_t)pos * pos_stride + d0) = v;
         }
+    }
+}
+
+// One accumulator tile of a wavefront into its [32 positions][S] block of buf (row = lane % 32).
+__device__ __forceinline__ void spill_tile(float *buf, int st, const floatx16 &acc, int t_l, int hf) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        f32x4_t v;
+        v.x = acc[4 * g], v.y = acc[4 * g + 1], v.z = acc[4 * g + 2], v.w = acc[4 * g + 3];
+        *(f32x4_t *)(buf + t_l * QA_LD + st * 32 + 8 * g + 4 * hf) = v;
     }
 }
 
@@ -251,6 +262,38 @@ __device__ __forceinline__ void exp_tile(const float *tab, int stride, const Exp
     }
 }
 
+// The output quantizer's operands of this lane's entries (row `row` of the [P, S] table, key positions
+// qa_row(st, r, hf)), packed as LaneQ::load packs them.  Four consecutive entries per 128-bit load, and every
+// load is issued before the first value is used: entry-by-entry loads would cost a memory round trip each.
+template <int ST>
+__device__ __forceinline__ void load_oq_entries(const hgq_qdesc &d, int64_t row, int S, int hf, int (&pk)[ST][16]) {
+    const Mode m(d.mode);
+    f32x4_t iv[ST][4], fv[ST][4], kf[ST][4];
+    uint32_t kb[ST][4];
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int64_t off = row * S + st * 32 + 8 * g + 4 * hf;
+            iv[st][g] = *(const f32x4_t *)(d.i + off);
+            fv[st][g] = *(const f32x4_t *)(d.fb + off);
+            if (m.k_u8)
+                kb[st][g] = *(const uint32_t *)((const uint8_t *)d.k + off);
+            else
+                kf[st][g] = *(const f32x4_t *)((const float *)d.k + off);
+        }
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float kk = m.k_u8 ? (float)((kb[st][g] >> (8 * c)) & 0xff) : kf[st][g][c];
+                const KIF p = resolve_kif(kk, iv[st][g][c], fv[st][g][c], m.kbi, m.round_params);
+                pk[st][4 * g + c] = (LaneQ::clamp8(p.f) & 0xff) | ((LaneQ::clamp8(p.i) & 0xff) << 8) | (p.k != 0.f ? 1 << 16 : 0);
+            }
+}
+
 // OQ_PLAIN: training mode and an output quantizer that only rounds (or none): its fractional bits are
 // packed four to a register; otherwise (k, i, f) take a register per element.
 template <int HD, int TH, int ST, bool TRAIN, bool OQ_PLAIN>
@@ -278,19 +321,23 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
     qo.init(dq);
     int po[ST][NPO];
     uint32_t mo[ST][16];
+    {
+        int pk_[ST][16];
 #pragma unroll
-    for (int st = 0; st < ST; ++st) {
+        for (int st = 0; st < ST; ++st)
 #pragma unroll
-        for (int j = 0; j < NPO; ++j) po[st][j] = 0;
+            for (int r = 0; r < 16; ++r) pk_[st][r] = 0, mo[st][r] = 0;
+        if (qo.present && active) load_oq_entries<ST>(dq, table_row, S, hf, pk_);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            mo[st][r] = 0;
-            if (qo.present && active) {
-                const int pk_ = qo.load(dq, (int64_t)table_row * S + qa_row(st, r, hf));
+        for (int st = 0; st < ST; ++st) {
+#pragma unroll
+            for (int j = 0; j < NPO; ++j) po[st][j] = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
                 if (OQ_PLAIN)
-                    po[st][r >> 2] |= (LaneQ::f_of(pk_) & 0xff) << (8 * (r & 3));
+                    po[st][r >> 2] |= (LaneQ::f_of(pk_[st][r]) & 0xff) << (8 * (r & 3));
                 else
-                    po[st][r % NPO] = pk_;
+                    po[st][r % NPO] = pk_[st][r];
             }
         }
     }
@@ -309,6 +356,8 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
     Stage sq_, sk_, sv_;
     sq_.init(q, pl.B, T, RL), sk_.init(k, pl.B, S, RL), sv_.init(v, pl.B, S, RL);
     f32x4_t pq[2], pk[2], pv[2];
+    floatx16 o_prev = {0};
+    int b_prev = -1;
     int b = blockIdx.x;
     sq_.fetch(pq, b, b < pl.B), sk_.fetch(pk, b, b < pl.B), sv_.fetch(pv, b, b < pl.B);
     for (; b < pl.B; b += pl.n_wg) {
@@ -318,6 +367,9 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
         sq_.fetch(pq, nb, nb < pl.B), sk_.fetch(pk, nb, nb < pl.B), sv_.fetch(pv, nb, nb < pl.B);
         __syncthreads();
         if (!active) continue;
+        // the previous element's output leaves here, a whole element ahead of the wait at the top of the walk
+        // (that wait covers every outstanding memory operation, stores included)
+        if (b_prev >= 0) store_rows<HD>(o_prev, out + ((int64_t)b_prev * T * pl.N + h) * HD, (int64_t)pl.N * HD, t0 + t_l, hf);
         // the packed operands stay packed: without this the unpacking is hoisted out of the walk and
         // every element's fractional bits (and their negation) take a register for the whole kernel
 #pragma unroll
@@ -357,23 +409,49 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
         const float sq = q3.fwd<TRAIN>(s);
         const float rr = q4.fwd<TRAIN>(__fdiv_rn(1.0f, __fadd_rn(sq, eps)));
         m3 = max(m3, abs_bits(sq));
+        // the output quantizer of an element, then its step of out = probs value: the MFMA of one element runs
+        // while the next one is quantized (the presence test is hoisted: no branch between the elements)
+        floatx16 o = {0};
+        if (qo.present) {
 #pragma unroll
-        for (int st = 0; st < ST; ++st)
+            for (int st = 0; st < ST; ++st) {
+                float a[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float y = __fmul_rn(acc[st][r], rr);
-                if (OQ_PLAIN) {
-                    if (qo.present) y = qo.round_at(y, (int)(int8_t)((po[st][r >> 2] >> (8 * (r & 3))) & 0xff));
-                } else {
-                    if (qo.present) y = qo.fwd<TRAIN>(y, po[st][r % NPO]);
-                    if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                for (int r = 0; r < 16; ++r) a[r] = Vs[qa_row(st, r, hf) * QA_LD + col0 + t_l];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float y = __fmul_rn(acc[st][r], rr);
+                    if (OQ_PLAIN)
+                        y = qo.round_at(y, (int)(int8_t)((po[st][r >> 2] >> (8 * (r & 3))) & 0xff));
+                    else
+                        y = qo.fwd<TRAIN>(y, po[st][r % NPO]);
+                    mo[st][r] = max(mo[st][r], abs_bits(y));
+                    o = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r], y, o, 0, 0, 0);
+                    if (OQ_PLAIN) {
+                        __builtin_amdgcn_sched_group_barrier(0x002, 11, 0);  // VALU of this element
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // its MFMA
+                    } else if ((r & 3) == 3) {
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
-                mo[st][r] = max(mo[st][r], abs_bits(y));
-                acc[st][r] = y;
             }
-        const floatx16 o = contract_keys<ST>(Vs, col0, t_l, hf, acc);
-        store_rows<HD>(o, out + ((int64_t)b * T * pl.N + h) * HD, (int64_t)pl.N * HD, t0 + t_l, hf);
+        } else {
+#pragma unroll
+            for (int st = 0; st < ST; ++st) {
+                float a[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) a[r] = Vs[qa_row(st, r, hf) * QA_LD + col0 + t_l];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float y = __fmul_rn(acc[st][r], rr);
+                    mo[st][r] = max(mo[st][r], abs_bits(y));
+                    o = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r], y, o, 0, 0, 0);
+                }
+            }
+        }
+        o_prev = o, b_prev = b;
     }
+    if (active && b_prev >= 0) store_rows<HD>(o_prev, out + ((int64_t)b_prev * T * pl.N + h) * HD, (int64_t)pl.N * HD, t0 + t_l, hf);
     m1 = max(m1, abs_bits(ldexpf(cmax, -ec.fi)));
     if (amax1 || amax3) {
         m1 = wave_max_bits(m1), m3 = wave_max_bits(m3);
@@ -439,6 +517,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
     float *Qs = lds, *Ks = Qs + (T + 1) * QA_LD, *Vs = Ks + (S + 1) * QA_LD, *Gs = Vs + (S + 1) * QA_LD;
     float *Pm = Gs + (T + 1) * QA_LD + QA_PAD;                           // [NW][32][QA_LD]: probs, then dscores
     ExpTable::Entry *tabp = (ExpTable::Entry *)(Pm + NW * 32 * QA_LD);  // [SM_TABLE]
+    float *tab_e = (float *)(tabp + SM_TABLE);                          // [SM_TABLE]: e alone, one bank per code
     __shared__ float part[NW][8];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, t_l = lane & 31, hf = lane >> 5;
@@ -455,18 +534,22 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
     qo.init(dq);
     int pf[ST][4];  // fractional bits of the output quantizer, element r of a tile in byte r % 4 of pf[st][r / 4]
     float gof[ST][16];
+    {
+        int pk_[ST][16];
 #pragma unroll
-    for (int st = 0; st < ST; ++st)
+        for (int st = 0; st < ST; ++st)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            pf[st][g] = 0;
+            for (int r = 0; r < 16; ++r) pk_[st][r] = 0, gof[st][r] = 0.f;
+        if (qo.present && active) load_oq_entries<ST>(dq, table_row, S, hf, pk_);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                gof[st][4 * g + c] = 0.f;
-                if (qo.present && active)
-                    pf[st][g] |= (LaneQ::f_of(qo.load(dq, (int64_t)table_row * S + qa_row(st, 4 * g + c, hf))) & 0xff) << (8 * c);
+        for (int st = 0; st < ST; ++st)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                pf[st][g] = 0;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) pf[st][g] |= (LaneQ::f_of(pk_[st][4 * g + c]) & 0xff) << (8 * c);
             }
-        }
+    }
     float gs[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) gs[j] = 0.f;
@@ -477,20 +560,29 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
         ExpTable tab;
         tab.build_bwd(tabp, q1, q2, scale);
         ec.init(q1, tab);
+        if (tab.on) {
+            for (int n = threadIdx.x; n < SM_TABLE; n += QA_NT) tab_e[n] = tabp[n].e;
+            __syncthreads();
+        }
     }
-    const float *tab_e = &tabp[0].e;  // e of code n at tab_e[4 n]
 
     Stage sq_, sk_, sv_, sg_;
     sq_.init(q, pl.B, T, RL), sk_.init(k, pl.B, S, RL), sv_.init(v, pl.B, S, RL), sg_.init(dout, pl.B, T, RL);
     f32x4_t pq[2], pk[2], pv[2], pg[2];
+    floatx16 dk_prev = {0};
+    int b_prev = -1;
     int b = blockIdx.x;
     sq_.fetch(pq, b, b < pl.B), sk_.fetch(pk, b, b < pl.B), sv_.fetch(pv, b, b < pl.B), sg_.fetch(pg, b, b < pl.B);
     for (; b < pl.B; b += pl.n_wg) {
         __syncthreads();  // the previous element's tiles and buffers are no longer read
         sq_.stash(Qs, T, pq), sk_.stash(Ks, S, pk), sv_.stash(Vs, S, pv), sg_.stash(Gs, T, pg);
-        const int nb = b + pl.n_wg;
-        sq_.fetch(pq, nb, nb < pl.B), sk_.fetch(pk, nb, nb < pl.B), sv_.fetch(pv, nb, nb < pl.B), sg_.fetch(pg, nb, nb < pl.B);
         __syncthreads();
+        // the previous element's dkey leaves here, well ahead of the wait at the top of the walk
+        if (active && b_prev >= 0) {
+#pragma unroll
+            for (int st = 0; st < ST; ++st)
+                if (st % TH == th) store_rows<HD>(dk_prev, dk_ + ((int64_t)b_prev * S * pl.N + h) * HD, (int64_t)pl.N * HD, st * 32 + t_l, hf);
+        }
         floatx16 xs[ST], ga[ST];
         float mx = 0.f, rr = 0.f, ds = 0.f;
         // the packed fractional bits stay packed (see the forward kernel)
@@ -509,16 +601,16 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
                 for (int r = 0; r < 16; ++r) mx = fmaxf(mx, xs[st][r]);
             mx = fmaxf(mx, xor32(mx));
             float s = 0.f;
-            floatx16 ev[ST];
             {
                 float cmax = 0.f;
                 uint32_t m1 = 0;
 #pragma unroll
                 for (int st = 0; st < ST; ++st) {
-                    ev[st] = xs[st];
-                    exp_tile(tab_e, 4, ec, d1, d2, scale, mx, ev[st], cmax, m1);
+                    floatx16 ev = xs[st];
+                    exp_tile(tab_e, 1, ec, d1, d2, scale, mx, ev, cmax, m1);
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) s += ev[st][r];
+                    for (int r = 0; r < 16; ++r) s += ev[r];
+                    spill_tile(my_buf, st, ev, t_l, hf);  // e waits in the buffer where its prob will go
                 }
             }
             s += xor32(s);
@@ -531,20 +623,22 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
             for (int st = 0; st < ST; ++st)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
+                    float *slot = my_buf + t_l * QA_LD + st * 32 + 8 * g + 4 * hf;
+                    const f32x4_t e4 = *(const f32x4_t *)slot;
                     f32x4_t p4;
 #pragma unroll
                     for (int c = 0; c < 4; ++c) {
                         const int r = 4 * g + c;
-                        const float y0 = __fmul_rn(ev[st][r], rr);
+                        const float y0 = __fmul_rn(e4[c], rr);
                         float p = y0;
                         if (qo.present) {
                             p = qo.round_at(y0, (int)(int8_t)((pf[st][g] >> (8 * c)) & 0xff));
                             gof[st][r] += -HGQ_LN2 * (p - y0) * ga[st][r];
                         }
                         p4[c] = p;
-                        drr += ga[st][r] * ev[st][r];
+                        drr += ga[st][r] * e4[c];
                     }
-                    *(f32x4_t *)(my_buf + t_l * QA_LD + st * 32 + 8 * g + 4 * hf) = p4;
+                    *(f32x4_t *)slot = p4;
                 }
             drr += xor32(drr);
             float dr0, gi4, gf4, gi3, gf3;
@@ -606,6 +700,13 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
             for (int st = 0; st < ST; ++st)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) ga[st][r] = (xs[st][r] == mx) ? share - ga[st][r] : -ga[st][r];
+        }
+        {
+            // the next element's operands: issued here, after the register-hungry stages, some eighty MFMAs ahead of their use
+            const int nb = b + pl.n_wg;
+            sq_.fetch(pq, nb, nb < pl.B), sk_.fetch(pk, nb, nb < pl.B), sv_.fetch(pv, nb, nb < pl.B), sg_.fetch(pg, nb, nb < pl.B);
+        }
+        if (active) {
             // dquery[t][h] = sum_s dscores[t][s] key[s][h]
             const floatx16 o = contract_keys<ST>(Ks, col0, t_l, hf, ga);
             store_rows<HD>(o, dq_ + ((int64_t)b * T * pl.N + h) * HD, (int64_t)pl.N * HD, t0 + t_l, hf);
@@ -617,11 +718,14 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
             // dkey[s][h] = sum_t dscores[t][s] query[t][h]
 #pragma unroll
             for (int st = 0; st < ST; ++st)
-                if (st % TH == th) {
-                    const floatx16 o = contract_queries<TH>(Qs, col0, head_buf, st * 32, t_l, hf);
-                    store_rows<HD>(o, dk_ + ((int64_t)b * S * pl.N + h) * HD, (int64_t)pl.N * HD, st * 32 + t_l, hf);
-                }
+                if (st % TH == th) dk_prev = contract_queries<TH>(Qs, col0, head_buf, st * 32, t_l, hf);
+            b_prev = b;
         }
+    }
+    if (active && b_prev >= 0) {
+#pragma unroll
+        for (int st = 0; st < ST; ++st)
+            if (st % TH == th) store_rows<HD>(dk_prev, dk_ + ((int64_t)b_prev * S * pl.N + h) * HD, (int64_t)pl.N * HD, st * 32 + t_l, hf);
     }
     // shared-quantizer gradients: wavefront sums, then the workgroup's in a fixed order
 #pragma unroll
@@ -651,7 +755,7 @@ static size_t qattn_lds_bytes(int T, int S, bool bwd) {
     size_t words = (size_t)(T + 1 + 2 * (S + 1)) * QA_LD + QA_PAD;
     if (!bwd) return (words + SM_TABLE) * sizeof(float);
     words += (size_t)(T + 1) * QA_LD + (size_t)(QA_NT / 64) * 32 * QA_LD;
-    return words * sizeof(float) + SM_TABLE * sizeof(ExpTable::Entry);
+    return words * sizeof(float) + SM_TABLE * (sizeof(ExpTable::Entry) + sizeof(float));
 }
 
 // Shapes the kernels take: sequence lengths 32 or 64 (both the same number of tiles), head size 8, 16 or
@@ -720,6 +824,8 @@ extern "C" int hgq_qattention_fwd(const float *query, const float *key, const fl
     if (!softmax_desc_ok(exp_iq) || !softmax_desc_ok(exp_oq) || !softmax_desc_ok(inv_iq) || !softmax_desc_ok(inv_oq) || !softmax_desc_ok(oq))
         return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: a quantizer descriptor has k but not i / fb");
     if (amax_oq && !has_oq) return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: amax_oq without an output quantizer");
+    if (has_oq && !(aligned16(oq->i) && aligned16(oq->fb) && ((uintptr_t)oq->k & 3u) == 0))
+        return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: the output quantizer's i / fb must be 16-byte aligned, k 4-byte aligned");
     if (amax_oq && !workspace && B > 0) return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: amax_oq needs the workspace");
     if ((rc = softmax_clear_trackers(amax_exp_iq, 1, amax_inv_iq, 1, B == 0 ? amax_oq : nullptr, pl.P_table * S, s))) return rc;
     if (B == 0) return HGQ_OK;
@@ -785,6 +891,8 @@ extern "C" int hgq_qattention_bwd(const float *dout, const float *query, const f
     for (const hgq_qdesc *d : all)
         if (d && d->k && !(d->mode & HGQ_MODE_TRAINING))
             return fail(HGQ_ERR_ARG, "hgq_qattention_bwd: the surrogate gradient is defined for training mode only");
+    if (has_oq && !(aligned16(oq->i) && aligned16(oq->fb) && ((uintptr_t)oq->k & 3u) == 0))
+        return fail(HGQ_ERR_ARG, "hgq_qattention_bwd: the output quantizer's i / fb must be 16-byte aligned, k 4-byte aligned");
     if (has_oq && (((oq->mode >> 4) & 0xf) != HGQ_WRAP || (oq->mode & HGQ_MODE_KBI)))
         return fail(HGQ_ERR_UNSUPPORTED, "hgq_qattention_bwd: a saturating or (k, b, i) output quantizer takes the separate softmax kernels");
     if (B == 0) {
