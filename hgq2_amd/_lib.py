@@ -47,6 +47,9 @@ SIGNATURES = {
     ),
     'hgq_ebops_finish_fwd': (c_int, [c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_ebops_finish_bwd': (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_void_p]),
+    'hgq_lut_ebops': (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
+    'hgq_softmax_ebops': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
+    'hgq_mha_ebops': (c_int, [c_void_p] * 4 + [c_int] * 5 + [c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_qbits_fwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     'hgq_qbits_bwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p]),
     'hgq_bn_fold_fwd': (c_int, [c_void_p] * 5 + [c_int, c_float] + [c_void_p] * 4 + [c_float, c_float, c_int, c_int, c_void_p]),
@@ -103,6 +106,13 @@ class QDesc(ctypes.Structure):
 
     _fields_ = [('k', c_void_p), ('i', c_void_p), ('fb', c_void_p), ('mode', c_int)]
 
+
+
+class BitsDesc(ctypes.Structure):
+    """``hgq_bits_desc`` of include/hgq_hip.h: a quantizer's bit-width view and where its gradients go."""
+
+    _fields_ = [('k', c_void_p), ('i', c_void_p), ('fb', c_void_p), ('size', c_int64), ('inner', c_int64), ('kbi', c_int),
+                ('add_mode', c_int), ('g_i', c_void_p), ('g_fb', c_void_p)]
 
 
 class MlpLayer(ctypes.Structure):

@@ -47,6 +47,19 @@ class QUnaryFunctionLUT(QLayerBaseSingleInput):
             inputs = self.iq(inputs, training=training)
         return self.activation(inputs)
 
+    def _ebops_loss_term(self, shape):
+        # value, uint32 variable, loss term and the bit-width gradients in one launch where the quantizers allow it
+        if self.enable_iq and self.enable_oq and self._beta is not None and self._beta.is_cuda:
+            operands = [self.iq.bits_operand(shape), self.oq.bits_operand(shape)]
+            n_cells = 1
+            for s in shape:
+                n_cells *= int(s)
+            if all(op is not None for op in operands) and 0 < n_cells < 2**31:
+                from .. import ops
+
+                return ops.bits_ebops('lut', operands, (n_cells, 1e-4, float(self.ebops_factor)), self._beta, self._ebops)
+        return super()._ebops_loss_term(shape)
+
     def _compute_ebops(self, shape):
         bw_inp = self.iq.bits_(shape)
         bw_out = self.oq.bits_(shape)

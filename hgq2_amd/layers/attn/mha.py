@@ -138,6 +138,17 @@ class QMultiHeadAttention(QLayerBase):
         k = args[2] if len(args) > 2 and args[2] is not None else None
         self.build(tuple(q.shape), tuple(v.shape) if v is not None else None, tuple(k.shape) if k is not None else None)
 
+    def _ebops_loss_term(self, query_shape, value_shape=None, key_shape=None):
+        # both score contractions' EBOPs from the marginal sums of the four bit-width tensors, in one launch
+        if self._beta is not None and self._beta.is_cuda and self._softmax.enable_oq:
+            (_, T, N, H), (_, S, _, Hv) = self._q_shape, self._v_shape
+            operands = [self._query_dense.oq.bits_operand(self._q_shape), self._key_dense.oq.bits_operand(self._k_shape),
+                        self._value_dense.oq.bits_operand(self._v_shape), self._softmax.oq.bits_operand((1, N, T, S))]
+            if all(op is not None for op in operands) and N * H <= 1024 and N * S <= 4096:
+                pf = float(self.parallelization_factor) if self.parallelization_factor > 0 else 1.0
+                return ops.bits_ebops('mha', operands, (T, S, N, H, Hv, pf, float(self.ebops_factor)), self._beta, self._ebops)
+        return super()._ebops_loss_term(query_shape, value_shape, key_shape)
+
     def _compute_ebops(self, query_shape, value_shape=None, key_shape=None):
         value_shape = query_shape if value_shape is None else value_shape
         attn_shape = (1, self._num_heads, query_shape[1], value_shape[1])

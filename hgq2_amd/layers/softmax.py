@@ -193,6 +193,20 @@ class QSoftmax(QLayerBaseSingleInput):
         divisor = self.inv_table(sums, training=training)
         return exp_inp * divisor
 
+    def _ebops_loss_term(self, shape):
+        # the stable form over the last axis: one launch for value, uint32 variable, loss term and gradients
+        shape = tuple(shape)
+        if self.stable and self.axes == (len(shape) - 1,) and self._beta is not None and self._beta.is_cuda:
+            rows, L = prod(shape[:-1]), shape[-1]
+            sub = self.iq if self.enable_iq else self.exp_table.iq
+            operands = [sub.bits_operand(shape), self.exp_table.oq.bits_operand(shape),
+                        self.inv_table.oq.bits_operand(shape[:-1] + (1,))]
+            if all(op is not None for op in operands) and 0 < rows <= 4096 and rows * L < 2**31:
+                n_instance = self.parallelization_factor if self.parallelization_factor > 0 else rows
+                return ops.bits_ebops('softmax', operands, (rows, L, n_instance / rows, float(self.ebops_factor)), self._beta,
+                                      self._ebops)
+        return super()._ebops_loss_term(shape)
+
     def _compute_ebops(self, shape):
         accum_shape = tuple(1 if i in self.axes else s for i, s in enumerate(shape))
         max_instance = prod(accum_shape)

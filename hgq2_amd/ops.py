@@ -17,7 +17,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits', 'ebops_finish', 'qattention', 'qattention_supported']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits', 'ebops_finish', 'qattention', 'qattention_supported', 'bits_ebops']
 
 
 def _ptr(t: Tensor | None):
@@ -1188,6 +1188,83 @@ class _EbopsFinish(torch.autograd.Function):
 def ebops_finish(ebops: Tensor, factor: float, beta: Tensor, ebops_var: Tensor) -> Tensor:
     """``ebops * factor`` stored into the uint32 variable and returned times ``beta`` (the loss term)."""
     return _EbopsFinish.apply(ebops.contiguous(), float(factor), beta, ebops_var)
+
+
+class _BitsEbops(torch.autograd.Function):
+    """EBOPs that are algebra on bit-width tensors (``hgq_lut_ebops`` / ``hgq_softmax_ebops`` / ``hgq_mha_ebops``).
+    ``layouts[n]`` = ``(size, inner, kbi, add_mode)`` of operand n or ``None``; ``qvars`` = k, i, fb per operand
+    (empty tensors where absent).  The kernel leaves the gradients for a unit upstream gradient; backward scales them."""
+
+    @staticmethod
+    def forward(ctx, kind, params, beta, ebops_var, layouts, *qvars):
+        lib = _lib.load()
+        ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
+        total = sum(2 * fb.numel() for fb, lay in zip(fbs, layouts) if lay is not None)
+        buf = torch.empty(max(total, 1), dtype=torch.float32, device=beta.device)
+        descs, slots, off = [], [], 0
+        for k, i, fb, lay in zip(ks, is_, fbs, layouts):
+            if lay is None:
+                descs.append(None), slots.append(None)
+                continue
+            size, inner, kbi, add_mode = lay
+            _check_f32('fb', fb)
+            _need(fb.numel() == size and (kbi or i.numel() == size) and (not add_mode or k.numel() == size), 'operand sizes differ')
+            n = fb.numel()
+            g_i, g_fb = buf[off:off + n], buf[off + n:off + 2 * n]
+            off += 2 * n
+            slots.append((g_i, g_fb))
+            descs.append(_lib.BitsDesc(k.data_ptr() if add_mode else None, None if kbi else i.data_ptr(), fb.data_ptr(), size, inner,
+                                       int(kbi), int(add_mode), None if kbi else g_i.data_ptr(), g_fb.data_ptr()))
+        out = torch.empty((), dtype=torch.float32, device=beta.device)
+        ptrs = [ctypes.addressof(d) if d is not None else None for d in descs]
+        if kind == 'lut':
+            n_cells, scale, factor = params
+            rc = lib.hgq_lut_ebops(ptrs[0], ptrs[1], n_cells, scale, factor, _ptr(beta), _ptr(ebops_var), _ptr(out), _stream())
+        elif kind == 'softmax':
+            rows, L, f1, f2 = params
+            rc = lib.hgq_softmax_ebops(ptrs[0], ptrs[1], ptrs[2], rows, L, f1, f2, _ptr(beta), _ptr(ebops_var), _ptr(out), _stream())
+        else:
+            T, S, N, H, Hv, f1, f2 = params
+            rc = lib.hgq_mha_ebops(ptrs[0], ptrs[1], ptrs[2], ptrs[3], T, S, N, H, Hv, f1, f2, _ptr(beta), _ptr(ebops_var), _ptr(out),
+                                   _stream())
+        _lib.check(rc, f'hgq_{kind}_ebops')
+        ctx.save_for_backward(buf)
+        ctx.slots = [None if s is None else (s[0].storage_offset(), s[1].storage_offset(), s[1].numel()) for s in slots]
+        ctx.kbis = [None if lay is None else lay[2] for lay in layouts]
+        ctx.shapes = [(i.shape, fb.shape) for i, fb in zip(is_, fbs)]
+        ctx.mark_non_differentiable(ebops_var)
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        (buf,) = ctx.saved_tensors
+        scaled = buf * g  # one launch for every operand
+        grads = [None, None, None, None, None]
+        for slot, kbi, (i_shape, fb_shape) in zip(ctx.slots, ctx.kbis, ctx.shapes):
+            if slot is None:
+                grads += [None, None, None]
+                continue
+            oi, of, n = slot
+            grads += [None, None if kbi else scaled[oi:oi + n].view(i_shape), scaled[of:of + n].view(fb_shape)]
+        return tuple(grads)
+
+
+def bits_ebops(kind: str, operands, params, beta: Tensor, ebops_var: Tensor) -> Tensor:
+    """Loss term ``ebops * beta`` of a layer whose EBOPs are algebra on bit-width tensors, in one launch; also assigns
+    the uint32 variable.  ``operands``: per operand ``None`` or ``(k, i, fb, size, inner, kbi, add_mode)`` (``i`` is
+    ``None`` for the (k, b, i) kind); ``params`` as the C entry point of ``kind`` ('lut', 'softmax', 'mha') takes them."""
+    e_f = beta.new_empty(0)
+    e_k = torch.empty(0, dtype=torch.uint8, device=beta.device)
+    flat, layouts = [], []
+    for op in operands:
+        if op is None:
+            flat += [e_k, e_f, e_f]
+            layouts.append(None)
+            continue
+        k, i, fb, size, inner, kbi, add_mode = op
+        flat += [k if add_mode else e_k, e_f if kbi else i, fb]
+        layouts.append((int(size), int(inner), bool(kbi), int(add_mode)))
+    return _BitsEbops.apply(kind, tuple(params), beta, ebops_var, tuple(layouts), *flat)
 
 
 class _AttnScores(torch.autograd.Function):

@@ -74,6 +74,25 @@ class Quantizer(Layer):
     def __repr__(self):
         return f'{self.__class__.__name__}(q_type={self.config.q_type}, name={self.name}, built={self.built})'
 
+    def bits_operand(self, shape):
+        """``bits_(shape)`` as the operand of a fused EBOPs kernel (``ops.bits_ebops``): the raw variables and the
+        broadcast rule ``(k, i, fb, size, inner, kbi, add_mode)``, or ``None`` when that form does not apply."""
+        from .internal import FixedPointQuantizerKBI, FixedPointQuantizerKIF
+        from .internal.base import bw_layout
+
+        inner = self.quantizer
+        if not isinstance(inner, (FixedPointQuantizerKIF, FixedPointQuantizerKBI)) or not inner.built:
+            return None
+        kbi = isinstance(inner, FixedPointQuantizerKBI)
+        fb = inner._third()
+        tensors = (inner._k, fb) if kbi else (inner._k, inner._i, fb)
+        if not all(t.is_cuda and t.is_contiguous() for t in tensors) or fb.dtype != torch.float32:
+            return None
+        layout = bw_layout(fb.shape, tuple(shape))
+        if layout is None:
+            return None
+        return (inner._k, None if kbi else inner._i, fb, layout[0], layout[1], kbi, 1 if inner.overflow_mode == 'SAT' else 0)
+
     def _bw_to_x(self, t, shape):
         t = torch.as_tensor(t)
         return self.quantizer.bw_mapper.bw_to_x(t, shape)

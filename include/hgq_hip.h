@@ -342,6 +342,43 @@ int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float
                    float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
 
 /*
+ * One quantizer's bit-width view for the EBOPs entry points below: `bits` / `fbits` as hgq_qbits_fwd forms
+ * them from the raw variables, broadcast to a tensor of n cells by the rule entry = (cell / inner) % size.
+ * g_i / g_fb [size] receive the gradient of the LOSS TERM (ebops * beta, unit upstream gradient) with
+ * respect to the variables, through the straight-through rounding of hgq_qbits_bwd (g_i unused for kbi).
+ */
+typedef struct hgq_bits_desc {
+    const uint8_t *k; /* uint8 keep-negative flags; may be NULL when add_mode == 0 */
+    const float *i;   /* NULL for the (k, b, i) kind */
+    const float *fb;
+    int64_t size, inner;
+    int kbi, add_mode;
+    float *g_i, *g_fb;
+} hgq_bits_desc;
+
+/*
+ * EBOPs of layers whose estimate is algebra on bit-width tensors, one launch each: value * factors ->
+ * uint32 variable (may be NULL), loss_term[0] = ebops * beta, gradients into the descriptors.
+ *   hgq_lut_ebops      QUnaryFunctionLUT._compute_ebops (src/hgq/layers/activation.py:101-104):
+ *                      sum over n_cells of 2**bits_in * bits_out, times `scale` (1e-4), times ebops_factor.
+ *   hgq_softmax_ebops  QSoftmax._compute_ebops, stable form (src/hgq/layers/softmax.py:177-206) for a softmax over
+ *                      the last axis of [rows, L]: sum(bits_sub) + sum(bits_exp) - sum_rows min_l bits_exp +
+ *                      sum(bits_exp * bits_inv[row]), times instance_factor, times ebops_factor; bits_inv is
+ *                      laid out over the rows; bits_sub may be NULL.  rows <= 4096.
+ *   hgq_mha_ebops      QMultiHeadAttention._compute_ebops (src/hgq/layers/attn/mha.py:507-524) for rank-3 inputs:
+ *                      sum bits_q[t,n,h] bits_k[s,n,h] + sum bits_attn[n,t,s] bits_v[s,n,h]; cells of q / k / v in
+ *                      [seq, N, H] order, of attn in [N, T, S] order.  N * H <= 1024, N * S <= 4096.
+ * Every sum is formed in a fixed order; values are exact while they stay below 2**53.
+ */
+int hgq_lut_ebops(const hgq_bits_desc *bits_in, const hgq_bits_desc *bits_out, int64_t n_cells, float scale, float ebops_factor,
+                  const float *beta, uint32_t *ebops_u32, float *loss_term, void *stream);
+int hgq_softmax_ebops(const hgq_bits_desc *bits_sub, const hgq_bits_desc *bits_exp, const hgq_bits_desc *bits_inv, int64_t rows, int L,
+                      float instance_factor, float ebops_factor, const float *beta, uint32_t *ebops_u32, float *loss_term, void *stream);
+int hgq_mha_ebops(const hgq_bits_desc *bits_q, const hgq_bits_desc *bits_k, const hgq_bits_desc *bits_v, const hgq_bits_desc *bits_attn, int T,
+                  int S, int N, int H, int Hv, float parallel_factor, float ebops_factor, const float *beta, uint32_t *ebops_u32,
+                  float *loss_term, void *stream);
+
+/*
  * The scalar tail of QLayerBase.call (src/hgq/layers/core/base.py:101-104):
  *     ebops = ebops * ebops_factor;  self._ebops.assign(cast(ebops, uint32));  loss term = ebops * beta
  * forward writes the uint32 variable (may be NULL) and out [1]; backward: d_ebops = (g * beta) * factor.

@@ -502,3 +502,57 @@ def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim):
         scale = b.abs().max().item() + 1e-12
         tol = (2e-5 if n in ('x', 'sm_oq_f') else 3e-4) * scale
         assert float((a - b).abs().max()) <= tol, f'grad {n}: {float((a - b).abs().max()):.3e} vs scale {scale:.3e}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('oq_hom', [None, (0, 1)])
+def test_bit_width_algebra_ebops_kernels_match_the_layer_formulas(oq_hom):
+    """hgq_lut_ebops / hgq_softmax_ebops / hgq_mha_ebops against the layers' own formulas evaluated with library
+    ops (QUnaryFunctionLUT / QSoftmax / QMultiHeadAttention._compute_ebops, reference activation.py:101-104,
+    softmax.py:177-206, mha.py:507-524): value and uint32 variable exactly, loss term and bit-width gradients to rounding."""
+    from hgq2_amd.config import QuantizerConfig
+    from hgq2_amd.layers import QMultiHeadAttention
+    from hgq2_amd.quantizer.quantizer import Quantizer
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(17)
+    kw = {}
+    if oq_hom is not None:
+        kw['softmax_oq_conf'] = QuantizerConfig(place='datalane', homogeneous_axis=oq_hom)
+    with readme_scopes():
+        layer = QMultiHeadAttention(num_heads=3, key_dim=8, parallelization_factor=5 if oq_hom else -1, **kw)
+    x = torch.randn(6, 20, 24, generator=g)
+    with torch.no_grad():
+        layer(x.to(dev), training=True)
+    _perturb(layer, g)
+    sm = layer._softmax
+    cases = [(layer, [(1, 20, 24)]), (sm, [(1, 3, 20, 20)]), (sm.exp_table, [(1, 3, 20, 20)]), (sm.inv_table, [(1, 3, 20, 1)])]
+    fused_operand = Quantizer.bits_operand
+    for obj, shapes in cases:
+        params = [p for p in layer.parameters() if p.requires_grad]
+        results = []
+        for fused in (True, False):
+            Quantizer.bits_operand = fused_operand if fused else (lambda self, shape: None)
+            try:
+                with torch.no_grad():
+                    obj._ebops.zero_()
+                term = obj._ebops_loss_term(*shapes)
+                (term * 3.0).backward()
+            finally:
+                Quantizer.bits_operand = fused_operand
+            results.append((float(term.detach()), int(obj._ebops.cpu().view(torch.int32)),
+                            [None if p.grad is None else p.grad.detach().clone() for p in params]))
+            for p in params:
+                p.grad = None
+        (t1, e1, g1), (t2, e2, g2) = results
+        name = type(obj).__name__
+        assert e1 == e2 and e1 > 0, (name, e1, e2)
+        assert abs(t1 - t2) <= 1e-6 * abs(t2), (name, t1, t2)
+        touched = 0
+        for a, b in zip(g1, g2):
+            assert (a is None) == (b is None) or (a is None and float(b.abs().max()) == 0.0) or (b is None and float(a.abs().max()) == 0.0), name
+            if a is None or b is None:
+                continue
+            touched += 1
+            assert float((a - b).abs().max()) <= 1e-6 * float(b.abs().max()) + 1e-12, (name, float((a - b).abs().max()))
+        assert touched > 0, name
