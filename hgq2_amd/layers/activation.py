@@ -54,7 +54,7 @@ class QUnaryFunctionLUT(QLayerBaseSingleInput):
             n_cells = 1
             for s in shape:
                 n_cells *= int(s)
-            if all(op is not None for op in operands) and 0 < n_cells < 2**31:
+            if all(op is not None for op in operands) and 0 < n_cells < 2**31 and sum(op[3] for op in operands) <= 30720:
                 from .. import ops
 
                 return ops.bits_ebops('lut', operands, (n_cells, 1e-4, float(self.ebops_factor)), self._beta, self._ebops)

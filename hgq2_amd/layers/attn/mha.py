@@ -144,7 +144,7 @@ class QMultiHeadAttention(QLayerBase):
             (_, T, N, H), (_, S, _, Hv) = self._q_shape, self._v_shape
             operands = [self._query_dense.oq.bits_operand(self._q_shape), self._key_dense.oq.bits_operand(self._k_shape),
                         self._value_dense.oq.bits_operand(self._v_shape), self._softmax.oq.bits_operand((1, N, T, S))]
-            if all(op is not None for op in operands) and N * H <= 1024 and N * S <= 4096:
+            if all(op is not None for op in operands) and N * H <= 1024 and N * S <= 2048 and sum(op[3] for op in operands) <= 30720:
                 pf = float(self.parallelization_factor) if self.parallelization_factor > 0 else 1.0
                 return ops.bits_ebops('mha', operands, (T, S, N, H, Hv, pf, float(self.ebops_factor)), self._beta, self._ebops)
         return super()._ebops_loss_term(query_shape, value_shape, key_shape)

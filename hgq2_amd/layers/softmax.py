@@ -201,7 +201,7 @@ class QSoftmax(QLayerBaseSingleInput):
             sub = self.iq if self.enable_iq else self.exp_table.iq
             operands = [sub.bits_operand(shape), self.exp_table.oq.bits_operand(shape),
                         self.inv_table.oq.bits_operand(shape[:-1] + (1,))]
-            if all(op is not None for op in operands) and 0 < rows <= 4096 and rows * L < 2**31:
+            if all(op is not None for op in operands) and 0 < rows <= 2048 and rows * L < 2**31 and sum(op[3] for op in operands) <= 30720:
                 n_instance = self.parallelization_factor if self.parallelization_factor > 0 else rows
                 return ops.bits_ebops('softmax', operands, (rows, L, n_instance / rows, float(self.ebops_factor)), self._beta,
                                       self._ebops)

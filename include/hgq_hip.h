@@ -364,11 +364,12 @@ typedef struct hgq_bits_desc {
  *   hgq_softmax_ebops  QSoftmax._compute_ebops, stable form (src/hgq/layers/softmax.py:177-206) for a softmax over
  *                      the last axis of [rows, L]: sum(bits_sub) + sum(bits_exp) - sum_rows min_l bits_exp +
  *                      sum(bits_exp * bits_inv[row]), times instance_factor, times ebops_factor; bits_inv is
- *                      laid out over the rows; bits_sub may be NULL.  rows <= 4096.
+ *                      laid out over the rows; bits_sub may be NULL.  rows <= 2048.
  *   hgq_mha_ebops      QMultiHeadAttention._compute_ebops (src/hgq/layers/attn/mha.py:507-524) for rank-3 inputs:
  *                      sum bits_q[t,n,h] bits_k[s,n,h] + sum bits_attn[n,t,s] bits_v[s,n,h]; cells of q / k / v in
- *                      [seq, N, H] order, of attn in [N, T, S] order.  N * H <= 1024, N * S <= 4096.
- * Every sum is formed in a fixed order; values are exact while they stay below 2**53.
+ *                      [seq, N, H] order, of attn in [N, T, S] order.  N * H <= 1024, N * S <= 2048.
+ * Every sum is formed in a fixed order; values are exact while they stay below 2**53.  The operands' entries are
+ * staged in LDS: at most 30720 over all operands of a call (HGQ_ERR_UNSUPPORTED beyond, as for the other limits).
  */
 int hgq_lut_ebops(const hgq_bits_desc *bits_in, const hgq_bits_desc *bits_out, int64_t n_cells, float scale, float ebops_factor,
                   const float *beta, uint32_t *ebops_u32, float *loss_term, void *stream);

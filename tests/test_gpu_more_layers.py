@@ -505,8 +505,8 @@ def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('oq_hom', [None, (0, 1)])
-def test_bit_width_algebra_ebops_kernels_match_the_layer_formulas(oq_hom):
+@pytest.mark.parametrize('oq_hom,het_table', [(None, False), ((0, 1), False), (None, True)])
+def test_bit_width_algebra_ebops_kernels_match_the_layer_formulas(oq_hom, het_table):
     """hgq_lut_ebops / hgq_softmax_ebops / hgq_mha_ebops against the layers' own formulas evaluated with library
     ops (QUnaryFunctionLUT / QSoftmax / QMultiHeadAttention._compute_ebops, reference activation.py:101-104,
     softmax.py:177-206, mha.py:507-524): value and uint32 variable exactly, loss term and bit-width gradients to rounding."""
@@ -520,7 +520,8 @@ def test_bit_width_algebra_ebops_kernels_match_the_layer_formulas(oq_hom):
     if oq_hom is not None:
         kw['softmax_oq_conf'] = QuantizerConfig(place='datalane', homogeneous_axis=oq_hom)
     with readme_scopes():
-        layer = QMultiHeadAttention(num_heads=3, key_dim=8, parallelization_factor=5 if oq_hom else -1, **kw)
+        layer = QMultiHeadAttention(num_heads=3, key_dim=8, parallelization_factor=5 if oq_hom else -1,
+                                    softmax_allow_heterogeneous_table=het_table, **kw)
     x = torch.randn(6, 20, 24, generator=g)
     with torch.no_grad():
         layer(x.to(dev), training=True)
