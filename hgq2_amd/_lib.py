@@ -34,6 +34,8 @@ SIGNATURES = {
     'hgq_version': (c_int, []),
     'hgq_last_error': (c_char_p, []),
     'hgq_quantize_fwd': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    'hgq_quantize_tracker_slices': (c_int64, [c_int64, c_int64, c_int64]),
+    'hgq_quantize_fwd_sliced': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_bwd': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_wrap_track_i': (c_int, [c_void_p] * 2 + [c_int] + [c_void_p] * 3 + [c_int64, c_float, c_float, c_float, c_int, c_void_p]),
     'hgq_qdense_fwd_parts': (c_int, [c_int64]),

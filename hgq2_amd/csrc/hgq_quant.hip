@@ -228,7 +228,7 @@ template <int RM, int OM, int VEC>
 __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ x, const void *__restrict__ k,
                                                       const float *__restrict__ i, const float *__restrict__ fb,
                                                       float *__restrict__ y, uint32_t *amax, uint32_t *anyneg,
-                                                      int64_t rows, int64_t M, int TX, int64_t rows_per_wg, int mode) {
+                                                      int64_t rows, int64_t M, int TX, int64_t rows_per_wg, int mode, int sliced) {
     const Mode m(mode);
     const int TY = 256 / TX;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
@@ -239,6 +239,18 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
     uint32_t lmax[VEC], lneg[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) p[e] = KIF{0.f, 0.f, 0.f}, lmax[e] = 0, lneg[e] = 0;
+    const int64_t row0 = (int64_t)blockIdx.y * rows_per_wg;
+    const int64_t n_rows = min(rows - row0, rows_per_wg);
+    const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + row0 * M, n_rows * M * 4);
+    float *yb = y + row0 * M;
+    // the first rows are requested before the bit-width operands: a workgroup is short-lived (often a single
+    // trip), and operands first would put two memory round trips end to end
+    float xv[QC_U][VEC];
+#pragma unroll
+    for (int u = 0; u < QC_U; ++u) {
+        const int64_t r = ty + (int64_t)TY * u;
+        qc_load<VEC>(rs, (active && r < n_rows) ? (uint32_t)((r * cg + c) * VEC) * 4u : BUF_OOB, xv[u]);
+    }
     if (active) {
         float kv[VEC], iv[VEC], fv[VEC];
         VecIO<VEC>::load_k(k, c, m.k_u8, kv);
@@ -247,15 +259,16 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
 #pragma unroll
         for (int e = 0; e < VEC; ++e) p[e] = resolve_kif(kv[e], iv[e], fv[e], m.kbi, m.round_params);
     }
-    const int64_t row0 = (int64_t)blockIdx.y * rows_per_wg;
-    const int64_t n_rows = min(rows - row0, rows_per_wg);
-    const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + row0 * M, n_rows * M * 4);
-    float *yb = y + row0 * M;
     for (int64_t rb = 0; rb < n_rows; rb += (int64_t)TY * QC_U) {
-        float xv[QC_U][VEC];
+        float cur[QC_U][VEC];
+#pragma unroll
+        for (int u = 0; u < QC_U; ++u)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) cur[u][e] = xv[u][e];
+        // next trip's rows in flight while this one is quantized
 #pragma unroll
         for (int u = 0; u < QC_U; ++u) {
-            const int64_t r = rb + ty + (int64_t)TY * u;
+            const int64_t r = rb + (int64_t)TY * QC_U + ty + (int64_t)TY * u;
             qc_load<VEC>(rs, (active && r < n_rows) ? (uint32_t)((r * cg + c) * VEC) * 4u : BUF_OOB, xv[u]);
         }
 #pragma unroll
@@ -264,8 +277,8 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
             float yv[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                yv[e] = quantize<RM, OM>(xv[u][e], p[e], m.training);
-                const float tv = m.track_input ? xv[u][e] : yv[e];
+                yv[e] = quantize<RM, OM>(cur[u][e], p[e], m.training);
+                const float tv = m.track_input ? cur[u][e] : yv[e];
                 const uint32_t ab = abs_bits(tv);
                 lmax[e] = ab > lmax[e] ? ab : lmax[e];
                 lneg[e] |= tv < 0.0f ? 1u : 0u;
@@ -291,10 +304,21 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
             __syncthreads();
         }
         if (ty == 0 && active) {
+            if (sliced) {
+                // one tracker slice per row chunk, written whole: nothing to clear beforehand, no atomics; the
+                // integer-bit update combines the slices
+                const int64_t base = (int64_t)blockIdx.y * M + c * VEC;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                if (amax) atomicMax(&amax[c * VEC + e], smax[tx * VEC + e]);
-                if (anyneg && sneg[tx * VEC + e]) atomicOr(&anyneg[c * VEC + e], 1u);
+                for (int e = 0; e < VEC; ++e) {
+                    if (amax) amax[base + e] = smax[tx * VEC + e];
+                    if (anyneg) anyneg[base + e] = sneg[tx * VEC + e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    if (amax) atomicMax(&amax[c * VEC + e], smax[tx * VEC + e]);
+                    if (anyneg && sneg[tx * VEC + e]) atomicOr(&anyneg[c * VEC + e], 1u);
+                }
             }
         }
     }
@@ -578,9 +602,9 @@ extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, c
         cols_grid(rows, M, TY * QC_U, gx, gy, rows_per_wg);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (vec)
-                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode);
+                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 0);
             else
-                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode);
+                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 0);
         });
         return check_launch("hgq_quantize_fwd");
     }
@@ -589,6 +613,46 @@ extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, c
         hipLaunchKernelGGL((quant_fwd_generic<RM, OM>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n, bw_size, bw_inner, mode);
     });
     return check_launch("hgq_quantize_fwd");
+}
+
+// Geometry of the per-column kernels for the sliced tracker form (16-byte aligned operands when bw_size is a multiple of 4).
+static bool sliced_geometry(int64_t n, int64_t bw_size, int64_t bw_inner, bool &vec, int &TX, int64_t &gx, int64_t &gy, int64_t &rows_per_wg) {
+    if (n < 1 || bw_size < 1 || bw_inner != 1 || bw_size >= n || n % bw_size != 0 || bw_size * 4 * 256 * QC_U >= (1ll << 31)) return false;
+    vec = bw_size % 4 == 0;
+    const int64_t cg = vec ? bw_size / 4 : bw_size;
+    TX = pow2_floor_le64(cg);
+    gx = (cg + TX - 1) / TX;
+    return cols_grid(n / bw_size, bw_size, (256 / TX) * QC_U, gx, gy, rows_per_wg);
+}
+
+extern "C" int64_t hgq_quantize_tracker_slices(int64_t n, int64_t bw_size, int64_t bw_inner) {
+    bool vec;
+    int TX;
+    int64_t gx, gy, rows_per_wg;
+    return sliced_geometry(n, bw_size, bw_inner, vec, TX, gx, gy, rows_per_wg) ? gy : 0;
+}
+
+extern "C" int hgq_quantize_fwd_sliced(const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax,
+                                       uint32_t *anyneg, int64_t n_slices, int64_t n, int64_t bw_size, int64_t bw_inner, int mode,
+                                       void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    bool vec;
+    int TX;
+    int64_t gx, gy, rows_per_wg;
+    if (!sliced_geometry(n, bw_size, bw_inner, vec, TX, gx, gy, rows_per_wg) || gy != n_slices)
+        return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_sliced: n_slices must be hgq_quantize_tracker_slices(n, bw_size, bw_inner) > 0");
+    if (!x || !k || !i || !fb || !y) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_sliced: null pointer");
+    const Mode m(mode);
+    if (vec && !(aligned16(x) && aligned16(y) && aligned16(i) && aligned16(fb) && ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0))
+        return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_sliced: operands must be 16-byte aligned when bw_size is a multiple of 4");
+    const int64_t M = bw_size, rows = n / M;
+    HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+        if (vec)
+            hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 1);
+        else
+            hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 1);
+    });
+    return check_launch("hgq_quantize_fwd_sliced");
 }
 
 extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,

@@ -61,10 +61,20 @@ def quantize_fwd(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inne
     _need(bw_size >= 1 and bw_inner >= 1 and (n == 0 or n % (bw_size * bw_inner) == 0),
           f'x has {n} elements, not a multiple of bw_size*bw_inner = {bw_size}*{bw_inner}')
     y = torch.empty_like(x)
+    lib = _lib.load()
+    slices = lib.hgq_quantize_tracker_slices(n, bw_size, bw_inner) if track and n else 0
+    if slices and all(t.data_ptr() % 16 == 0 for t in (x, y, k, i, fb)):
+        # trackers as one slice per row chunk ([slices, bw_size]): no clearing launch, no atomics
+        amax = torch.empty(slices * bw_size, dtype=torch.int32, device=x.device)
+        neg = torch.empty(slices * bw_size, dtype=torch.int32, device=x.device)
+        rc = lib.hgq_quantize_fwd_sliced(_ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(y), _ptr(amax), _ptr(neg), slices, n, bw_size,
+                                         bw_inner, _kmode(mode, k), _stream())
+        _lib.check(rc, 'hgq_quantize_fwd_sliced')
+        return y, amax, neg
     amax = torch.empty(bw_size if track else 0, dtype=torch.int32, device=x.device)
     neg = torch.empty(bw_size if track else 0, dtype=torch.int32, device=x.device)
-    rc = _lib.load().hgq_quantize_fwd(_ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(y), _ptr(amax), _ptr(neg), n, bw_size,
-                                      bw_inner, _kmode(mode, k), _stream())
+    rc = lib.hgq_quantize_fwd(_ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(y), _ptr(amax), _ptr(neg), n, bw_size,
+                              bw_inner, _kmode(mode, k), _stream())
     _lib.check(rc, 'hgq_quantize_fwd')
     return y, amax, neg
 
@@ -72,6 +82,8 @@ def quantize_fwd(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inne
 @quantize_fwd.register_fake
 def _(x, k, i, fb, mode, bw_inner, track):
     m = i.numel() if track else 0
+    if m and x.numel():
+        m *= max(int(_lib.load().hgq_quantize_tracker_slices(x.numel(), i.numel(), bw_inner)), 1)
     return torch.empty_like(x), x.new_empty(m, dtype=torch.int32), x.new_empty(m, dtype=torch.int32)
 
 

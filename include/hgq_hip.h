@@ -79,6 +79,17 @@ int hgq_quantize_fwd(const float *x, const void *k, const float *i, const float 
                      int mode, void *stream);
 
 /*
+ * hgq_quantize_fwd with the trackers as slices: when bit-widths are shared along the leading axis only
+ * (bw_inner == 1, bw_size < n) the kernel can leave one abs-max / any-negative slice per row chunk instead of
+ * combining them with atomics; hgq_wrap_track_i takes the slices as they are (n_parts = n_slices), nothing has
+ * to be cleared first.  hgq_quantize_tracker_slices returns the slice count for a shape (0: use hgq_quantize_fwd).
+ *   amax / anyneg [n_slices, bw_size] (either may be NULL).  Operands 16-byte aligned when bw_size % 4 == 0.
+ */
+int64_t hgq_quantize_tracker_slices(int64_t n, int64_t bw_size, int64_t bw_inner);
+int hgq_quantize_fwd_sliced(const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax, uint32_t *anyneg,
+                            int64_t n_slices, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
+
+/*
  * Fixed-point quantizer, surrogate backward (training mode only).  Replaces the custom
  * gradients of the same third-party callable plus autograd through broadcast_to (the sum over
  * the homogeneous axes) and through `f = b - i` for the KBI parametrisation

@@ -121,6 +121,9 @@ def test_quantize_broadcast_bitwidths(dev, shape, bw_shape, overflow_mode):
     hom = tuple(a for a in range(len(shape)) if not len(bw_shape) or bw_shape[a] == 1)
     want_amax = torch.amax(y.detach().abs(), dim=hom).reshape(-1)
     want_neg = torch.amax((y.detach() < 0).int(), dim=hom).reshape(-1)
+    # the trackers come as one entry per bit-width entry, or as slices [n_slices, bw_size] that the
+    # integer-bit update combines (non-negative floats order like their bit patterns)
+    amax, neg = amax.view(-1, bw_size).amax(0), neg.view(-1, bw_size).amax(0)
     assert torch.equal(amax.view(torch.float32).cpu(), want_amax)
     assert torch.equal(neg.cpu(), want_neg.int())
     yd.backward(gy.to(dev))
