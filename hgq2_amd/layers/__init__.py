@@ -1,6 +1,7 @@
 from ..quantizer import Quantizer
 from .activation import QUnaryFunctionLUT
 from .attn import QMultiHeadAttention
+from .batch_normalization import QBatchNormalization
 from .conv import QConv2D
 from .core import QDense, QEinsumDense, QLayerBase, QLayerBaseMultiInputs, QLayerBaseSingleInput
 from .einsum_dense_batchnorm import QEinsumDenseBatchnorm
@@ -8,6 +9,6 @@ from .pooling import (QAveragePooling2D, QGlobalAveragePooling1D, QGlobalAverage
                       QGlobalMaxPooling2D, QMaxPooling2D)
 from .softmax import QSoftmax
 
-__all__ = ['Quantizer', 'QDense', 'QEinsumDense', 'QEinsumDenseBatchnorm', 'QConv2D', 'QSoftmax', 'QUnaryFunctionLUT',
+__all__ = ['Quantizer', 'QDense', 'QEinsumDense', 'QEinsumDenseBatchnorm', 'QBatchNormalization', 'QConv2D', 'QSoftmax', 'QUnaryFunctionLUT',
            'QMultiHeadAttention', 'QMaxPooling2D', 'QAveragePooling2D', 'QGlobalAveragePooling1D', 'QGlobalAveragePooling2D',
            'QGlobalMaxPooling1D', 'QGlobalMaxPooling2D', 'QLayerBase', 'QLayerBaseSingleInput', 'QLayerBaseMultiInputs']

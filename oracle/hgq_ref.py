@@ -561,6 +561,61 @@ class RefQEinsumDenseBatchnorm(RefQEinsumDense):
         return y
 
 
+class RefQBatchNormalization(RefQLayer):
+    """src/hgq/layers/batch_normalization.py:10-206 on top of Keras' BatchNormalization: moments are mean and
+    mean(x**2) - mean**2 over all axes but ``axis`` (the torch backend's ``moments``); the layer's own epsilon;
+    ``center=False`` puts 1 in the place of ``bn_beta`` (:117-120, :145-148)."""
+
+    def __init__(self, axis, gamma, beta_bn, moving_mean, moving_variance, iq, kq, bq, momentum=0.99, epsilon=1e-3, beta0=1e-5,
+                 enable_ebops=True):
+        self._init_common(beta0, enable_ebops)
+        self.axis, self.momentum, self.epsilon = axis, momentum, epsilon
+        self.gamma = None if gamma is None else gamma.detach().clone().requires_grad_(True)
+        self.bn_beta = None if beta_bn is None else beta_bn.detach().clone().requires_grad_(True)
+        self.moving_mean, self.moving_variance = moving_mean.detach().clone(), moving_variance.detach().clone()
+        self.iq, self.kq, self.bq = iq, kq, bq
+
+    def weights(self):
+        return [w for w in (self.gamma, self.bn_beta) if w is not None]
+
+    def quantizers(self):
+        return [q for q in (self.iq, self.kq, self.bq) if q is not None]
+
+    def _bshape(self, x):
+        shape = [1] * x.dim()
+        shape[self.axis] = x.shape[self.axis]
+        return shape
+
+    def call(self, x, training=None):
+        if self.iq is not None:
+            x = self.iq(x, training=training)
+        if training:
+            axes = tuple(a for a in range(x.dim()) if a != self.axis % x.dim())
+            mean = torch.mean(x, dim=axes)
+            var = torch.mean(torch.square(x), dim=axes) - torch.square(mean)
+            with torch.no_grad():
+                self.moving_mean.copy_(self.moving_mean * self.momentum + mean * (1.0 - self.momentum))
+                self.moving_variance.copy_(self.moving_variance * self.momentum + var * (1.0 - self.momentum))
+        else:
+            mean, var = self.moving_mean, self.moving_variance
+        gamma = self.gamma if self.gamma is not None else 1
+        bn_beta = self.bn_beta if self.bn_beta is not None else 1
+        scale = gamma / torch.sqrt(var + self.epsilon)
+        offset = bn_beta - mean * scale
+        qscale = torch.reshape(self.kq(scale, training=training), self._bshape(x))
+        qoffset = torch.reshape(self.bq(offset, training=training), self._bshape(x))
+        return x * qscale + qoffset
+
+    def _compute_ebops(self, shape):
+        bshape = [1] * len(shape)
+        bshape[self.axis] = shape[self.axis]
+        bw_inp = self.iq.bits_(shape)
+        bw_ker = torch.reshape(self.kq.bits_(self.moving_mean.shape), bshape)
+        bw_bias = torch.reshape(self.bq.bits_(self.moving_mean.shape), bshape)
+        size = float(np.prod(shape))
+        return torch.sum(bw_inp * bw_ker) + torch.mean(bw_bias) * size
+
+
 class RefQUnaryFunctionLUT(RefQLayer):
     """src/hgq/layers/activation.py:18-67."""
 

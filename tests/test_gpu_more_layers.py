@@ -557,3 +557,44 @@ def test_bit_width_algebra_ebops_kernels_match_the_layer_formulas(oq_hom, het_ta
             touched += 1
             assert float((a - b).abs().max()) <= 1e-6 * float(b.abs().max()) + 1e-12, (name, float((a - b).abs().max()))
         assert touched > 0, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('shape,axis,center,scale', [((64, 12, 16), -1, True, True), ((32, 6, 8), 1, True, True),
+                                                       ((128, 10), -1, False, True), ((40, 5, 7, 12), 3, True, False)])
+def test_batch_normalization_layer(shape, axis, center, scale):
+    """QBatchNormalization (reference src/hgq/layers/batch_normalization.py) against the oracle twin: output, moving
+    statistics, loss terms, EBOPs and the gradients of input, gamma / beta and bit-widths."""
+    from hgq2_amd.layers import QBatchNormalization
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(len(shape) * 10 + axis % len(shape))
+    with readme_scopes():
+        layer = QBatchNormalization(axis=axis, center=center, scale=scale, momentum=0.9)
+    x = torch.randn(shape, generator=g) * 1.5 + 0.3
+    layer(x.to(dev), training=True)
+    _perturb(layer, g)
+    with torch.no_grad():
+        if scale:
+            layer.bn_gamma.copy_(torch.rand(layer.bn_gamma.shape, generator=g) + 0.5)
+        if center:
+            layer.bn_beta.copy_(torch.randn(layer.bn_beta.shape, generator=g) * 0.3)
+    r = twin.ref_batchnorm(layer)
+    xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
+    named_p = [('x', xp), ('iq_f', layer.iq.quantizer._f), ('kq_b', layer.kq.quantizer._b), ('kq_i', layer.kq.quantizer._i),
+               ('bq_b', layer.bq.quantizer._b)]
+    named_r = [('x', xr), ('iq_f', r.iq.quantizer._f), ('kq_b', r.kq.quantizer._b), ('kq_i', r.kq.quantizer._i),
+               ('bq_b', r.bq.quantizer._b)]
+    if scale:
+        named_p.append(('gamma', layer.bn_gamma)), named_r.append(('gamma', r.gamma))
+    if center:
+        named_p.append(('beta', layer.bn_beta)), named_r.append(('beta', r.bn_beta))
+    _compare_step(layer, r, lambda t: layer(xp, training=t), lambda t: r(xr, training=t), named_p, named_r, grad_rtol=1e-4)
+    _close(layer.moving_mean, r.moving_mean, what='moving mean')
+    _close(layer.moving_variance, r.moving_variance, what='moving variance')
+    assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach())
+    assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+    y_p, y_r = layer(xp, training=False), r(xr, training=False)
+    _close(y_p, y_r, what='inference output')
+    qs, qo = layer.qscaler_and_qoffset
+    assert qs.shape == layer.moving_mean.shape and qo.shape == layer.moving_mean.shape

@@ -187,3 +187,27 @@ def test_kif_wrap_training_state_machine():
     # col0: max .203125 -> ceil(log2(.21875)) = -2 -> max(1.99,-2)=1.99 ; col1: 7.984375+2^-6 = 8 -> 3 ; col2: 100 -> 7
     assert torch.allclose(q.quantizer._i, torch.tensor([[1.99, 3.0, 7.0]]))
     assert q.quantizer.bits.tolist() == [[8.0, 9.0, 13.0]]
+
+
+def test_dummy_quantizers_reduce_qbatchnorm_to_batch_normalisation():
+    """The oracle's QBatchNormalization with dummy quantizers is the textbook batch normalisation: training output
+    (x - mean) / sqrt(var + eps) * gamma + beta with the biased batch variance, and with momentum 0 the inference
+    output repeats it (the check the reference makes at tests/test_batchnorm.py:44-59)."""
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(6, 8, 5, generator=g) * 2 + 1
+    gamma, beta = torch.rand(5, generator=g) + 0.5, torch.randn(5, generator=g)
+    q = lambda: ref.RefQuantizer(ref.RefDummyQuantizer(), None, None, None)  # noqa: E731
+    bn = ref.RefQBatchNormalization(2, gamma, beta, torch.randn(5, generator=g), torch.rand(5, generator=g) * 8, q(), q(), q(),
+                                    momentum=0.0, epsilon=1e-3, enable_ebops=False)
+    mean = x.double().mean(dim=(0, 1))
+    var = ((x.double() - mean) ** 2).mean(dim=(0, 1))
+    want = ((x.double() - mean) / torch.sqrt(var + 1e-3) * gamma.double() + beta.double()).float()
+    y_train = bn(x, training=True)
+    assert torch.allclose(y_train, want, atol=2e-6), float((y_train - want).abs().max())
+    assert torch.allclose(bn.moving_mean, mean.float(), atol=1e-6) and torch.allclose(bn.moving_variance, var.float(), atol=1e-5)
+    y_test = bn(x, training=False)
+    assert torch.allclose(y_test, want, atol=2e-6)
+    # a dropped term shows: without centring the reference puts 1 in beta's place, without scaling gamma is 1
+    bn2 = ref.RefQBatchNormalization(2, None, None, torch.zeros(5), torch.ones(5), q(), q(), q(), momentum=0.0, enable_ebops=False)
+    y2 = bn2(x, training=True)
+    assert torch.allclose(y2, ((x.double() - mean) / torch.sqrt(var + 1e-3) + 1.0).float(), atol=2e-6)

@@ -92,6 +92,14 @@ def ref_einsum_dense_bn(layer, input_shape):
                             momentum=layer.momentum)
 
 
+def ref_batchnorm(layer):
+    return ref.RefQBatchNormalization(layer.axis, layer.bn_gamma.detach().cpu() if layer.scale else None,
+                                      layer.bn_beta.detach().cpu() if layer.center else None, layer.moving_mean.detach().cpu(),
+                                      layer.moving_variance.detach().cpu(), _iq(layer), ref_quantizer(layer.kq), ref_quantizer(layer.bq),
+                                      momentum=layer.momentum, epsilon=layer.epsilon, beta0=_beta(layer),
+                                      enable_ebops=layer.enable_ebops)
+
+
 def ref_lut(layer, fn):
     return ref.RefQUnaryFunctionLUT(fn, _iq(layer), _oq(layer), beta0=_beta(layer), enable_ebops=layer.enable_ebops)
 
