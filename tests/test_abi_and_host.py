@@ -170,3 +170,47 @@ def test_entry_points_validate_arguments_before_any_launch():
     assert lib.hgq_qdense_bwd(none, none, none, none, 0, none, none, none, none, none, none, 128, 80, 10, 0, 0, none) == UNSUPPORTED
     assert lib.hgq_col_moments_workspace(1000, 64) > 0 and lib.hgq_col_moments_workspace(-1, 64) == -1
     assert lib.hgq_col_moments_fwd(none, 0, 64, none, none, none, none) == ARG
+
+
+def test_beta_controllers_and_ebops_logging():
+    """Host-side hooks of reference src/hgq/utils/sugar/{ebops,beta_scheduler,beta_pid}.py on layers built on the CPU
+    (no kernel is launched: the hooks only read `_ebops` and assign `_beta`)."""
+    from math import log10
+
+    from hgq2_amd.core import Sequential
+    from hgq2_amd.layers import QDense
+    from hgq2_amd.utils.sugar import PID, BetaPID, BetaScheduler, FreeEBOPs, PieceWiseSchedule, fit
+
+    sched = PieceWiseSchedule([(10, 1e-5, 'log'), (0, 0.0, 'linear'), (20, 1e-3, 'constant')])
+    assert sched(0) == 0.0 and abs(sched(5) - 5e-6) < 1e-12 and abs(sched(10) - 1e-5) < 1e-12
+    assert abs(sched(15) - 1e-4) < 1e-9 and sched(20) == 1e-3 and sched(300) == 1e-3
+    pid = PID(2.0, 0.5, 0.25, neg=False)
+    assert pid(1.0, 0.0) == 2.0 + 0.5 + 0.25 and pid(1.0, 0.5) == 1.0 + 0.75 - 0.125
+    layers = [QDense(8), QDense(4)]
+    model = Sequential(layers)
+    shape = (None, 16)
+    for layer in layers:
+        layer.build(shape)
+        shape = (None, layer.units)
+    counters = iter([(1000, 3000), (800, 2400), (500, 1000), (100, 300)])
+
+    def step(_):
+        a, b = next(counters)
+        with torch.no_grad():
+            layers[0]._ebops.view(torch.int32).fill_(a), layers[1]._ebops.view(torch.int32).fill_(b)
+        return 1.5
+
+    history = fit(model, step, lambda epoch: [0], 4, [BetaScheduler(sched), FreeEBOPs()])
+    assert [h['ebops'] for h in history] == [4000, 3200, 1500, 400]
+    assert [h['beta'] for h in history] == [sched(e) for e in range(4)] and history[0]['loss'] == 1.5
+    assert float(layers[1]._beta) == pytest.approx(sched(3))
+    # the PID controller: idle during warm-up, then its first output repeats the beta in force (integral initialisation),
+    # and a model above its EBOPs target gets a larger beta the next epoch
+    counters = iter([(1000, 3000)] * 6)
+    ctl = BetaPID(target_ebops=2000.0, init_beta=1e-6, p=1.0, i=0.1, warmup=2, log=True)
+    history = fit(model, step, lambda epoch: [0], 5, [ctl])
+    assert float(layers[0]._beta) == pytest.approx(history[-1]['beta'])
+    assert history[0]['beta'] == pytest.approx(1e-6) and history[2]['beta'] == pytest.approx(1e-6, rel=1e-6)
+    err = log10(4000 / 2000)
+    assert history[3]['beta'] == pytest.approx(10 ** (log10(1e-6) + 0.1 * err), rel=1e-6) and history[4]['beta'] > history[3]['beta']
+    assert all(h['ebops'] == 4000 for h in history)
