@@ -448,19 +448,24 @@ def test_bn_fold_matches_the_reference_formula(K, N, with_gamma, is_meansq):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('batch,seq,heads,key_dim', [(2048, 64, 4, 16), (300, 32, 2, 8), (37, 32, 2, 32), (5, 64, 1, 8)])
-def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim):
+@pytest.mark.parametrize('batch,seq,heads,key_dim,oq_hom', [(2048, 64, 4, 16, None), (300, 32, 2, 8, None), (37, 32, 2, 32, None),
+                                                            (5, 64, 1, 8, None), (70, 64, 2, 16, (0, 1)), (33, 32, 4, 16, (0, 1, 2))])
+def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim, oq_hom):
     """scores -> table softmax -> combine as one kernel each way (hgq_qattention_fwd / _bwd) against the same
     layer composing hgq_attn_scores_*, hgq_qsoftmax_* and hgq_attn_combine_*: outputs, tracked integer
     bits and loss terms bit-identical, gradients within fp32 summation noise."""
     import hgq2_amd.layers.attn.mha as mha
+    from hgq2_amd.config import QuantizerConfig
     from hgq2_amd.layers import QMultiHeadAttention
 
     dev = torch.device('cuda:0')
     g = torch.Generator().manual_seed(batch + seq)
     torch.manual_seed(batch)
+    kw = {}
+    if oq_hom is not None:  # output quantizer entries shared by heads (and query positions): table rows are reused
+        kw['softmax_oq_conf'] = QuantizerConfig(place='datalane', homogeneous_axis=oq_hom)
     with readme_scopes():
-        layer = QMultiHeadAttention(num_heads=heads, key_dim=key_dim)
+        layer = QMultiHeadAttention(num_heads=heads, key_dim=key_dim, **kw)
     x = torch.randn(batch, seq, heads * key_dim, generator=g)
     with torch.no_grad():
         layer(x.to(dev), training=True)
@@ -487,9 +492,17 @@ def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim):
         for p in params():
             p.grad = None
         i_vars = [q.quantizer._i.detach().clone() for q in (sm.exp_table.iq, sm.inv_table.iq, sm.oq)]
-        results.append((y.detach(), grads, i_vars, [float(t.detach()) for t in layer.losses]))
-    (y1, g1, i1, l1), (y2, g2, i2, l2) = results
+        losses = [float(t.detach()) for t in layer.losses]
+        mha.FUSED = fused
+        try:
+            with torch.no_grad():
+                y_inf = layer(x.to(dev), training=False)  # inference mode: wrapping quantizers wrap, empty words are zeroed
+        finally:
+            mha.FUSED = True
+        results.append((y.detach(), grads, i_vars, losses, y_inf))
+    (y1, g1, i1, l1, f1), (y2, g2, i2, l2, f2) = results
     assert torch.equal(y1, y2), f'outputs differ by {float((y1 - y2).abs().max()):.3e}'
+    assert torch.equal(f1, f2), f'inference outputs differ by {float((f1 - f2).abs().max()):.3e}'
     for a, b in zip(i1, i2):
         assert torch.equal(a, b)
     assert l1 == l2
