@@ -488,7 +488,20 @@ __global__ __launch_bounds__(1024) void qattn_amax_reduce_kernel(const uint32_t 
     uint32_t m = 0;
     if (e < M) {
         const int64_t p = e / S, s = e - p * S;
-        for (int64_t it = grp; it < (int64_t)n_slices * fold; it += 16) {
+        // eight loads in flight per thread
+        const int64_t n_it = (int64_t)n_slices * fold;
+        int64_t it = grp;
+        for (; it + 7 * 16 < n_it; it += 8 * 16) {
+            uint32_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int64_t iu = it + u * 16, sl = iu / fold, r = p + (iu - sl * fold) * P;
+                v[u] = slices[(sl * rows + r) * S + s];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) m = max(m, v[u]);
+        }
+        for (; it < n_it; it += 16) {
             const int64_t sl = it / fold, r = p + (it - sl * fold) * P;
             m = max(m, slices[(sl * rows + r) * S + s]);
         }

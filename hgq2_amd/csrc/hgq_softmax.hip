@@ -383,7 +383,20 @@ __global__ __launch_bounds__(1024) void qsoftmax_reduce_kernel(const float *__re
     const float *wf = ws + nblk * 8, *wi = wf + pl.n_chunks * PL;
     float si = 0.f, sf = 0.f;
     if (e < M) {
-        for (int64_t sl = grp; sl < n_slices; sl += 16) {
+        // eight loads in flight per thread; the order of the additions is fixed
+        int64_t sl = grp;
+        for (; sl + 7 * 16 < n_slices; sl += 8 * 16) {
+            float vf[8], vi[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int64_t su = sl + u * 16, o = (su / fold) * PL + (su % fold) * M + e;
+                vf[u] = wf[o];
+                vi[u] = oq_gi ? wi[o] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) sf += vf[u], si += vi[u];
+        }
+        for (; sl < n_slices; sl += 16) {
             const int64_t o = (sl / fold) * PL + (sl % fold) * M + e;
             sf += wf[o];
             if (oq_gi) si += wi[o];
