@@ -470,9 +470,12 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
 // output column, for the batch statistics of QEinsumDenseBatchnorm.  Same tiling as the forward
 // above; a lane keeps the sums of its column over its 16 accumulator rows in registers across
 // tiles.  Slice blockIdx.x of `part` is [N sums | N sums of squares].
-template <int NS4>
-__global__ __launch_bounds__(256, 2) void dense_moments_fast_kernel(const float *__restrict__ x, const float *__restrict__ w,
-                                                                   float *__restrict__ part, int64_t rows, int K, int N) {
+// QUANT: x is the raw input of a training-mode WRAP quantizer (round only) with a [P, K] table of fractional bits,
+// quantized while it is staged exactly as the forward kernel does.
+template <int RM, bool QUANT, int NS4>
+__global__ __launch_bounds__(256, 2) void dense_moments_fast_kernel(const float *__restrict__ x, const float *__restrict__ f_in, int P,
+                                                                   const float *__restrict__ w, float *__restrict__ part,
+                                                                   int64_t rows, int K, int N, int mode) {
     __shared__ __attribute__((aligned(16))) float xs[2][FAST_BM + 1][FAST_XLD];
     __shared__ float red[4][64][2];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -488,6 +491,17 @@ __global__ __launch_bounds__(256, 2) void dense_moments_fast_kernel(const float 
     }
     FastMap mp;
     mp.init(K);
+    int fi[FAST_NJ][4];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            fi[j][e] = 0;
+            if (QUANT && mp.on[j]) {
+                const float f = f_in[(mp.row[j] % P) * K + mp.col[j] + e];
+                fi[j][e] = (int)(Mode(mode).round_params ? rintf(f) : f);
+            }
+        }
     f32x4_t raw[FAST_NJ];
     uint32_t xoff[FAST_NJ];
 #pragma unroll
@@ -507,9 +521,14 @@ __global__ __launch_bounds__(256, 2) void dense_moments_fast_kernel(const float 
     for (; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
+            float v[4] = {raw[j][0], raw[j][1], raw[j][2], raw[j][3]};
+            if (QUANT) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]);
+            }
             float *dst = &xs[buf][mp.on[j] ? mp.row[j] : FAST_BM][mp.col[j] >> 1];
-            *(float2 *)dst = make_float2(raw[j][0], raw[j][2]);
-            *(float2 *)(dst + 32) = make_float2(raw[j][1], raw[j][3]);
+            *(float2 *)dst = make_float2(v[0], v[2]);
+            *(float2 *)(dst + 32) = make_float2(v[1], v[3]);
         }
         __syncthreads();
         const int64_t next = tile + gridDim.x;
@@ -878,50 +897,93 @@ extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_i
     return check_launch("hgq_qdense_fwd");
 }
 
-extern "C" int64_t hgq_dense_moments_workspace(int64_t rows, int K, int N) {
-    if (rows < 0 || K < 1 || N < 1) return -1;
+extern "C" int64_t hgq_qdense_moments_workspace(int64_t rows, int K, int N, int64_t bw_rows) {
+    if (rows < 0 || K < 1 || N < 1 || bw_rows < 0) return -1;
     const int64_t parts = rows > 0 ? row_parts(rows, FAST_BM) : 1;
-    const int64_t fwd = parts * 2 * N, bwd = parts * ((int64_t)K * N + N);
+    const int64_t fwd = parts * 2 * N, bwd = parts * ((int64_t)K * N + N + bw_rows * K);
     return fwd > bwd ? fwd : bwd;
 }
 
-static int moments_check(const char *who, int64_t rows, int K, int N, const void *x) {
-    if (rows < 1 || K < 1 || N < 1) return fail(HGQ_ERR_ARG, "%s: bad sizes", who);
+extern "C" int64_t hgq_dense_moments_workspace(int64_t rows, int K, int N) { return hgq_qdense_moments_workspace(rows, K, N, 0); }
+
+static int moments_check(const char *who, int64_t rows, int K, int N, const void *x, const float *f_in, int64_t bw_rows, int mode) {
+    if (rows < 1 || K < 1 || N < 1 || bw_rows < 0) return fail(HGQ_ERR_ARG, "%s: bad sizes", who);
     if (K > 64 || N > 64 || K % 4 != 0 || N % 4 != 0 || !aligned16(x))
         return fail(HGQ_ERR_UNSUPPORTED, "%s: needs K, N <= 64, multiples of 4, and a 16-byte aligned input (K=%d N=%d)", who, K, N);
+    if (bw_rows > 0) {
+        const Mode m(mode);
+        if (!f_in) return fail(HGQ_ERR_ARG, "%s: null bit-width pointer", who);
+        if (!(m.overflow_mode == HGQ_WRAP && m.training && !m.kbi))
+            return fail(HGQ_ERR_UNSUPPORTED, "%s: the fused input quantizer must be a training-mode WRAP (k, i, f) quantizer", who);
+        if (bw_rows > 64 || 64 % bw_rows != 0 || rows % bw_rows != 0)
+            return fail(HGQ_ERR_UNSUPPORTED, "%s: bw_rows=%lld must divide 64 and rows", who, (long long)bw_rows);
+        if (m.round_mode != HGQ_TRN && m.round_mode != HGQ_RND && m.round_mode != HGQ_RND_CONV) return fail(HGQ_ERR_ARG, "%s: unknown round mode", who);
+    }
     return HGQ_OK;
+}
+
+extern "C" int hgq_qdense_moments_fwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, float *mean,
+                                      float *meansq, float *workspace, int64_t rows, int K, int N, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    int rc = moments_check("hgq_qdense_moments_fwd", rows, K, N, x, f_in, bw_rows, mode);
+    if (rc) return rc;
+    if (!x || !w || !mean || !meansq || !workspace) return fail(HGQ_ERR_ARG, "hgq_qdense_moments_fwd: null pointer");
+    const int parts = row_parts(rows, FAST_BM);
+    const dim3 grid((unsigned)parts);
+    const bool quant = bw_rows > 0;
+    const int P = quant ? (int)bw_rows : 1;
+    const int rm = Mode(mode).round_mode;
+#define HGQ_MOM_FAST(NS4V) \
+    do { \
+        if (!quant) hipLaunchKernelGGL((dense_moments_fast_kernel<HGQ_TRN, false, NS4V>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+        else if (rm == HGQ_TRN) hipLaunchKernelGGL((dense_moments_fast_kernel<HGQ_TRN, true, NS4V>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+        else if (rm == HGQ_RND) hipLaunchKernelGGL((dense_moments_fast_kernel<HGQ_RND, true, NS4V>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+        else hipLaunchKernelGGL((dense_moments_fast_kernel<HGQ_RND_CONV, true, NS4V>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+    } while (0)
+    if (K <= 8) HGQ_MOM_FAST(1);
+    else if (K <= 16) HGQ_MOM_FAST(2);
+    else if (K <= 32) HGQ_MOM_FAST(4);
+    else HGQ_MOM_FAST(8);
+#undef HGQ_MOM_FAST
+    if ((rc = check_launch("hgq_qdense_moments_fwd"))) return rc;
+    if ((rc = reduce_parts(workspace, parts, 2 * (int64_t)N, mean, (int64_t)N, meansq, (int64_t)N, nullptr, 0, s))) return rc;
+    hipLaunchKernelGGL(moments_scale_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, mean, meansq, N, 1.0f / (float)rows);
+    return check_launch("hgq_qdense_moments_fwd(scale)");
 }
 
 extern "C" int hgq_dense_moments_fwd(const float *x, const float *w, float *mean, float *meansq, float *workspace, int64_t rows,
                                      int K, int N, void *stream) {
+    return hgq_qdense_moments_fwd(x, nullptr, 0, 0, w, mean, meansq, workspace, rows, K, N, stream);
+}
+
+extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, const float *dmean,
+                                      const float *dmeansq, float *dx, float *dw, float *df_in, float *workspace, int64_t rows, int K,
+                                      int N, void *stream) {
     hipStream_t s = (hipStream_t)stream;
-    int rc = moments_check("hgq_dense_moments_fwd", rows, K, N, x);
+    int rc = moments_check("hgq_qdense_moments_bwd", rows, K, N, x, f_in, bw_rows, mode);
     if (rc) return rc;
-    if (!x || !w || !mean || !meansq || !workspace) return fail(HGQ_ERR_ARG, "hgq_dense_moments_fwd: null pointer");
-    const int parts = row_parts(rows, FAST_BM);
+    if (!x || !w || !dmean || !dmeansq || !dx || !dw || !workspace) return fail(HGQ_ERR_ARG, "hgq_qdense_moments_bwd: null pointer");
+    if (!aligned16(dx)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_moments_bwd: dx must be 16-byte aligned");
+    const int parts = row_parts(rows, BWD_BM);
+    const bool quant = bw_rows > 0;
+    const int P = quant ? (int)bw_rows : 1;
+    const int rm = Mode(mode).round_mode;
     const dim3 grid((unsigned)parts);
-    if (K <= 8) hipLaunchKernelGGL((dense_moments_fast_kernel<1>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
-    else if (K <= 16) hipLaunchKernelGGL((dense_moments_fast_kernel<2>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
-    else if (K <= 32) hipLaunchKernelGGL((dense_moments_fast_kernel<4>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
-    else hipLaunchKernelGGL((dense_moments_fast_kernel<8>), grid, dim3(256), 0, s, x, w, workspace, rows, K, N);
-    if ((rc = check_launch("hgq_dense_moments_fwd"))) return rc;
-    if ((rc = reduce_parts(workspace, parts, 2 * (int64_t)N, mean, (int64_t)N, meansq, (int64_t)N, nullptr, 0, s))) return rc;
-    hipLaunchKernelGGL(moments_scale_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, mean, meansq, N, 1.0f / (float)rows);
-    return check_launch("hgq_dense_moments_fwd(scale)");
+#define HGQ_MOM_BWD(RMV, QV) \
+    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode)
+    if (!quant) HGQ_MOM_BWD(HGQ_TRN, false);
+    else if (rm == HGQ_TRN) HGQ_MOM_BWD(HGQ_TRN, true);
+    else if (rm == HGQ_RND) HGQ_MOM_BWD(HGQ_RND, true);
+    else HGQ_MOM_BWD(HGQ_RND_CONV, true);
+#undef HGQ_MOM_BWD
+    if ((rc = check_launch("hgq_qdense_moments_bwd"))) return rc;
+    const int64_t PK = bw_rows * (int64_t)K;
+    return reduce_parts(workspace, parts, (int64_t)K * N + N + PK, dw, (int64_t)K * N, nullptr, (int64_t)N, quant ? df_in : (float *)nullptr, PK, s);
 }
 
 extern "C" int hgq_dense_moments_bwd(const float *x, const float *w, const float *dmean, const float *dmeansq, float *dx, float *dw,
                                      float *workspace, int64_t rows, int K, int N, void *stream) {
-    hipStream_t s = (hipStream_t)stream;
-    int rc = moments_check("hgq_dense_moments_bwd", rows, K, N, x);
-    if (rc) return rc;
-    if (!x || !w || !dmean || !dmeansq || !dx || !dw || !workspace) return fail(HGQ_ERR_ARG, "hgq_dense_moments_bwd: null pointer");
-    if (!aligned16(dx)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_moments_bwd: dx must be 16-byte aligned");
-    const int parts = row_parts(rows, BWD_BM);
-    hipLaunchKernelGGL((qdense_bwd_fast_kernel<HGQ_TRN, false, true>), dim3((unsigned)parts), dim3(256), 0, s, dmean, dmeansq, x,
-                       (const float *)nullptr, 1, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, 0);
-    if ((rc = check_launch("hgq_dense_moments_bwd"))) return rc;
-    return reduce_parts(workspace, parts, (int64_t)K * N + N, dw, (int64_t)K * N, nullptr, (int64_t)N, nullptr, 0, s);
+    return hgq_qdense_moments_bwd(x, nullptr, 0, 0, w, dmean, dmeansq, dx, dw, nullptr, workspace, rows, K, N, stream);
 }
 
 extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,

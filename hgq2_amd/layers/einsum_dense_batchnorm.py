@@ -10,6 +10,7 @@ import torch
 
 from .. import _lib, ops
 from ..core import epsilon, get_initializer
+from .core._contraction import fused_iq_rows
 from .core.einsum_dense import QEinsumDense, analyze_einsum_string
 
 
@@ -91,7 +92,7 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         n_out = len(self.full_output_shape)
         return self._gemm is not None and self._reduction_axes == tuple(range(n_out - self._gemm[1]))
 
-    def _batch_moments(self, qinputs, raw=False):
+    def _batch_moments(self, qinputs, raw=False, quant=None):
         """Mean and variance (``raw``: mean of squares, flat) of the un-quantized-kernel pre-activation
         over the non-normalised axes (reference :108-112).  GEMM-shaped equations whose normalised axes
         are all the new output axes run through the dense and column-moment kernels; others through the
@@ -103,7 +104,7 @@ class QEinsumDenseBatchnorm(QEinsumDense):
             w2d = self._kernel.reshape(self._K, self._N)
             x2d = x2d.contiguous()
             if ops.dense_moments_supported(x2d, w2d):
-                mean, meansq = ops.dense_moments(x2d, w2d)  # one pass over x, the pre-activation is never written
+                mean, meansq = ops.dense_moments(x2d, w2d, quant)  # one pass over x, the pre-activation is never written
             else:
                 if self._K <= ops.FUSED_BWD_MAX and self._N <= ops.FUSED_BWD_MAX:
                     pre, _ = ops.qdense(x2d, None, None, None, w2d, None, _lib.ACT_NONE, 0, 0, False)
@@ -119,13 +120,28 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         mean = torch.mean(x, dim=self._reduction_axes)
         return mean, torch.mean(torch.square(x), dim=self._reduction_axes) - torch.square(mean)
 
+    def _fused_iq(self, inputs, training):
+        """``(f_in, bw_rows, mode)`` if the input quantizer can run inside both contractions (statistics and output) while
+        they stage their operand - the quantized input is then never written - else ``None``."""
+        if not (self.enable_iq and training is True and self.trainable and inputs.is_cuda and self._trailing_gemm()):
+            return None
+        if self.bias.numel() != self._N or self._K > ops.FUSED_BWD_MAX or self._N > ops.FUSED_BWD_MAX:
+            return None
+        bw_rows = fused_iq_rows(self.iq, tuple(inputs.shape), self._K, training)
+        x2d = inputs.reshape(-1, self._K)
+        if not bw_rows or 64 % bw_rows or not x2d.is_contiguous() or not ops.dense_moments_supported(x2d, self._kernel.reshape(self._K, self._N)):
+            return None
+        q = self.iq.quantizer
+        return q._f.view(-1), bw_rows, q._mode(True)
+
     def call(self, inputs, training=None):
-        if self.enable_iq:
+        quant = self._fused_iq(inputs, training)
+        if quant is None and self.enable_iq:
             inputs = self.iq(inputs, training=training)
         if training and self.trainable and inputs.is_cuda and self._trailing_gemm() and self.bias.numel() == self._N:
             # statistics, folding and the moving-average update in three launches (the folding algebra and its
             # gradient would otherwise be some forty elementwise launches on [N] vectors)
-            mean, meansq = self._batch_moments(inputs, raw=True)
+            mean, meansq = self._batch_moments(inputs, raw=True, quant=quant)
             fused_kernel, fused_bias = ops.bn_fold(self._kernel.reshape(self._K, self._N), self.bias.reshape(-1),
                                                    self.bn_gamma.reshape(-1) if self.scale else None, mean, meansq, True, epsilon(),
                                                    self.moving_mean.view(-1), self.moving_variance.view(-1), self.momentum)
@@ -140,8 +156,9 @@ class QEinsumDenseBatchnorm(QEinsumDense):
             else:
                 var, mean = self.moving_variance, self.moving_mean
             qkernel, qbias = self.get_fused_qkernel_and_qbias(training, mean, var)
-        # the input is already quantized: contract without the fused input quantizer
-        enable_iq, self._enable_iq = self._enable_iq, False
+        # an input quantized above is contracted as it is; otherwise the contraction quantizes it while staging
+        # (and leaves the abs-max slices for the integer-bit update, as QEinsumDense does)
+        enable_iq, self._enable_iq = self._enable_iq, quant is not None
         try:
             y, act_done = self._contract(inputs, qkernel, qbias, training)
         finally:

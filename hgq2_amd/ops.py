@@ -697,39 +697,45 @@ def dense_moments_supported(x2d: Tensor, w2d: Tensor) -> bool:
 
 
 @torch.library.custom_op('hgq::dense_moments_fwd', mutates_args=())
-def dense_moments_fwd(x: Tensor, w: Tensor) -> tuple[Tensor, Tensor]:
+def dense_moments_fwd(x: Tensor, w: Tensor, f_in: Tensor, bw_rows: int, mode: int) -> tuple[Tensor, Tensor]:
     _check_f32('x', x), _check_f32('w', w)
     _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[0], 'shape mismatch')
     rows, K = x.shape
     N = w.shape[1]
+    if bw_rows:
+        _check_f32('f_in', f_in)
+        _need(f_in.numel() == bw_rows * K, 'f_in must be a [bw_rows, K] table')
     lib = _lib.load()
     mean, meansq = (torch.empty(N, dtype=torch.float32, device=x.device) for _ in range(2))
-    ws = torch.empty(max(lib.hgq_dense_moments_workspace(rows, K, N), 1), dtype=torch.float32, device=x.device)
-    _lib.check(lib.hgq_dense_moments_fwd(_ptr(x), _ptr(w), _ptr(mean), _ptr(meansq), _ptr(ws), rows, K, N, _stream()), 'hgq_dense_moments_fwd')
+    ws = torch.empty(max(lib.hgq_qdense_moments_workspace(rows, K, N, bw_rows), 1), dtype=torch.float32, device=x.device)
+    _lib.check(lib.hgq_qdense_moments_fwd(_ptr(x), _ptr(f_in), bw_rows, mode, _ptr(w), _ptr(mean), _ptr(meansq), _ptr(ws), rows, K, N,
+                                          _stream()), 'hgq_qdense_moments_fwd')
     return mean, meansq
 
 
 @dense_moments_fwd.register_fake
-def _(x, w):
+def _(x, w, f_in, bw_rows, mode):
     return x.new_empty(w.shape[1]), x.new_empty(w.shape[1])
 
 
 @torch.library.custom_op('hgq::dense_moments_bwd', mutates_args=())
-def dense_moments_bwd(x: Tensor, w: Tensor, dmean: Tensor, dmeansq: Tensor) -> tuple[Tensor, Tensor]:
+def dense_moments_bwd(x: Tensor, w: Tensor, f_in: Tensor, bw_rows: int, mode: int, dmean: Tensor,
+                      dmeansq: Tensor) -> tuple[Tensor, Tensor, Tensor]:
     _check_f32('x', x), _check_f32('w', w), _check_f32('dmean', dmean), _check_f32('dmeansq', dmeansq)
     rows, K = x.shape
     N = w.shape[1]
     lib = _lib.load()
     dx, dw = torch.empty_like(x), torch.empty_like(w)
-    ws = torch.empty(max(lib.hgq_dense_moments_workspace(rows, K, N), 1), dtype=torch.float32, device=x.device)
-    _lib.check(lib.hgq_dense_moments_bwd(_ptr(x), _ptr(w), _ptr(dmean), _ptr(dmeansq), _ptr(dx), _ptr(dw), _ptr(ws), rows, K, N, _stream()),
-               'hgq_dense_moments_bwd')
-    return dx, dw
+    df = torch.empty(bw_rows * K, dtype=torch.float32, device=x.device)
+    ws = torch.empty(max(lib.hgq_qdense_moments_workspace(rows, K, N, bw_rows), 1), dtype=torch.float32, device=x.device)
+    _lib.check(lib.hgq_qdense_moments_bwd(_ptr(x), _ptr(f_in), bw_rows, mode, _ptr(w), _ptr(dmean), _ptr(dmeansq), _ptr(dx), _ptr(dw),
+                                          _ptr(df), _ptr(ws), rows, K, N, _stream()), 'hgq_qdense_moments_bwd')
+    return dx, dw, df
 
 
 @dense_moments_bwd.register_fake
-def _(x, w, dmean, dmeansq):
-    return torch.empty_like(x), torch.empty_like(w)
+def _(x, w, f_in, bw_rows, mode, dmean, dmeansq):
+    return torch.empty_like(x), torch.empty_like(w), x.new_empty(bw_rows * x.shape[1])
 
 
 @torch.library.custom_op('hgq::bn_fold_fwd', mutates_args=('moving_mean', 'moving_var'))
@@ -1120,21 +1126,29 @@ def col_moments(x2d: Tensor):
 
 class _DenseMoments(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w):
-        ctx.save_for_backward(x, w)
-        return dense_moments_fwd(x, w)
+    def forward(ctx, x, w, f_in, bw_rows, mode):
+        ctx.save_for_backward(x, w, f_in)
+        ctx.quant = (bw_rows, mode)
+        return dense_moments_fwd(x, w, f_in, bw_rows, mode)
 
     @staticmethod
-    def backward(ctx, gm, gs):
-        x, w = ctx.saved_tensors
-        gm = torch.zeros(w.shape[1], device=x.device) if gm is None else gm.contiguous()
-        gs = torch.zeros(w.shape[1], device=x.device) if gs is None else gs.contiguous()
-        return dense_moments_bwd(x, w, gm, gs)
+    def backward(ctx, dmean, dmeansq):
+        x, w, f_in = ctx.saved_tensors
+        bw_rows, mode = ctx.quant
+        zero = x.new_zeros(w.shape[1])
+        dx, dw, df = dense_moments_bwd(x, w, f_in, bw_rows, mode, dmean.contiguous() if dmean is not None else zero,
+                                       dmeansq.contiguous() if dmeansq is not None else zero)
+        return dx, dw, (df.view(f_in.shape) if bw_rows else None), None, None
 
 
-def dense_moments(x2d: Tensor, w2d: Tensor):
-    """``(mean(z, 0), mean(z * z, 0))`` of ``z = x2d @ w2d`` without materialising ``z``."""
-    return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous())
+def dense_moments(x2d: Tensor, w2d: Tensor, quant=None):
+    """``(mean(z, 0), mean(z * z, 0))`` of ``z = q(x2d) @ w2d`` without materialising ``z`` (nor ``q(x2d)``).
+    ``quant`` = ``(f_in, bw_rows, mode)``: the raw fractional bits of a training-mode WRAP input quantizer laid out as
+    a ``[bw_rows, K]`` table; ``None``: ``x2d`` is contracted as it is."""
+    if quant is None:
+        return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous(), x2d.new_empty(0), 0, 0)
+    f_in, bw_rows, mode = quant
+    return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous(), f_in.contiguous(), int(bw_rows), int(mode))
 
 
 class _BnFold(torch.autograd.Function):

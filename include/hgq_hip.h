@@ -444,6 +444,21 @@ int hgq_dense_moments_bwd(const float *x, const float *w, const float *dmean, co
                           float *workspace, int64_t rows, int K, int N, void *stream);
 
 /*
+ * The same with the layer's input quantizer applied while x is staged (QEinsumDenseBatchnorm.call quantizes its
+ * input once, :101-102, and contracts it twice): x is the RAW input, f_in the raw fractional-bit variable of a
+ * training-mode WRAP (k, i, f) quantizer laid out as a [bw_rows, K] table (row r of x uses table row r % bw_rows,
+ * bw_rows divides 64), mode its HGQ_MODE(...) bits.  The quantized input is never written; the backward returns dx
+ * with respect to the raw input (straight-through) and df_in [bw_rows * K], this contraction's share of the
+ * fractional-bit gradient.  bw_rows == 0: no quantizer (the entry points above).
+ */
+int64_t hgq_qdense_moments_workspace(int64_t rows, int K, int N, int64_t bw_rows);
+int hgq_qdense_moments_fwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, float *mean, float *meansq,
+                           float *workspace, int64_t rows, int K, int N, void *stream);
+int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, const float *dmean,
+                           const float *dmeansq, float *dx, float *dw, float *df_in, float *workspace, int64_t rows, int K, int N,
+                           void *stream);
+
+/*
  * Per-column mean and mean of squares of a [rows, N] matrix, and the gradient of both.  Replaces
  * `ops.mean(x, axis)` / `ops.mean(ops.square(x), axis)` and their autograd in
  * QEinsumDenseBatchnorm.call (src/hgq/layers/einsum_dense_batchnorm.py:99-124, the batch
