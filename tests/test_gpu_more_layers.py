@@ -611,3 +611,35 @@ def test_batch_normalization_layer(shape, axis, center, scale):
     _close(y_p, y_r, what='inference output')
     qs, qo = layer.qscaler_and_qoffset
     assert qs.shape == layer.moving_mean.shape and qo.shape == layer.moving_mean.shape
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('rows,K,N,bw_rows', [(4096, 16, 64, 64), (640, 64, 32, 16), (70 * 64, 64, 64, 1)])
+def test_dense_moments_with_the_input_quantizer_inside(rows, K, N, bw_rows):
+    """ops.dense_moments(x, w, quant): column moments of q(x) @ w with q a training-mode WRAP quantizer applied while
+    the operand is staged, against fp64 on the separately quantized input: moments, dx (straight-through), dw and the
+    fractional-bit gradient sum(-ln2 (q(x) - x) dq) of this contraction."""
+    from hgq2_amd import _lib, ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(rows + K + bw_rows)
+    x = torch.randn(rows, K, generator=g) * 2
+    w = torch.randn(K, N, generator=g) * 0.4
+    f = torch.randint(2, 7, (bw_rows, K), generator=g).float()
+    um, us = torch.randn(N, generator=g), torch.randn(N, generator=g)
+    fr = f.repeat(rows // bw_rows, 1)
+    xq = torch.floor(x * 2.0**fr + 0.5) / 2.0**fr  # RND, exact in fp32
+    xr, wr = xq.double().requires_grad_(True), w.double().requires_grad_(True)
+    z = xr @ wr
+    mean_r, msq_r = z.mean(0), (z * z).mean(0)
+    ((mean_r * um.double()).sum() + (msq_r * us.double()).sum()).backward()
+    df_r = (-0.6931471805599453 * (xq.double() - x.double()) * xr.grad).view(rows // bw_rows, bw_rows, K).sum(0)
+    xd, wd, fd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True), f.to(dev).requires_grad_(True)
+    mode = _lib.mode_bits('RND', 'WRAP', training=True, round_params=True)
+    mean, msq = ops.dense_moments(xd, wd, (fd.view(-1), bw_rows, mode))
+    ((mean * um.to(dev)).sum() + (msq * us.to(dev)).sum()).backward()
+    for name, got, want in (('mean', mean, mean_r), ('meansq', msq, msq_r), ('dx', xd.grad, xr.grad), ('dw', wd.grad, wr.grad),
+                            ('df', fd.grad, df_r)):
+        want = want.detach().float()
+        err = float((got.detach().cpu() - want).abs().max())
+        assert err <= 2e-5 * float(want.abs().max()) + 1e-7, f'{name}: {err:.3e}'
