@@ -111,18 +111,38 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_
     }
     __syncthreads();
     const int64_t KN = (int64_t)K * N;
-    for (int64_t e0 = 0; e0 < KN; e0 += 4 * NT) {
+    // kernel entries in blocks of 4 * NT: loaded with consecutive lanes on consecutive entries, handed over through
+    // LDS so that a thread adds a contiguous run of four before it touches a row's sum - one LDS atomic per (thread,
+    // row) instead of one per entry (up to 64 lanes on one address serialise)
+    __shared__ int sbits[4 * NT];
+    for (int64_t blk = 0; blk < KN; blk += 4 * NT) {
         float b[4], d;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int64_t e = e0 + u * NT + t;
-            b[u] = e < KN ? entry_bits(k_ker, nullptr, b_ker, e, mk, d) : 0.0f;
+            const int64_t e = blk + u * NT + t;
+            b[u] = entry_bits(k_ker, nullptr, b_ker, e < KN ? e : 0, mk, d);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t e = e0 + u * NT + t;
-            if (e < KN) atomicAdd(&colsum[e / N], (int)b[u]);
+        for (int u = 0; u < 4; ++u) sbits[u * NT + t] = (int)b[u];
+        __syncthreads();
+        const int64_t e0 = blk + 4 * (int64_t)t;
+        if (e0 < KN) {
+            const int4 v = *(const int4 *)&sbits[4 * t];
+            const int vals[4] = {v.x, v.y, v.z, v.w};
+            int k = (int)(e0 / N), rem = (int)(e0 - (int64_t)k * N), acc = 0;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (e0 + u < KN) {
+                    acc += vals[u];
+                    if (++rem == N) {
+                        atomicAdd(&colsum[k], acc);
+                        acc = 0, rem = 0, ++k;
+                    }
+                }
+            }
+            if (acc) atomicAdd(&colsum[k], acc);
         }
+        __syncthreads();
     }
     __syncthreads();
     for (int64_t e = t; e < PK; e += NT) {

@@ -57,7 +57,7 @@ def test_conv2d_matches_fp64_reference(dev, case):
     from hgq2_amd import _lib, ops
 
     B, H, W, C, kh, kw, Fo, strides, padding, dilation, relu, bias = case
-    g = torch.Generator().manual_seed(hash(case) % 1000)
+    g = torch.Generator().manual_seed(CASES.index(case))
     x = torch.randn(B, H, W, C, generator=g)
     w = torch.randn(kh, kw, C, Fo, generator=g) * 0.3
     b = torch.randn(Fo, generator=g) if bias else None
@@ -73,6 +73,11 @@ def test_conv2d_matches_fp64_reference(dev, case):
     scale = want.abs().max().item() + 1e-9
     assert float((got.detach().cpu().double() - want.detach()).abs().max()) <= 1e-5 * scale
     up = torch.randn(want.shape, generator=g)
+    if relu:
+        # An output within fp32 rounding of the kink has no agreed derivative: fp32 and fp64 may
+        # land on opposite sides of zero there, so such outputs get no upstream gradient.
+        pre = _ref_conv(x, w, b, strides, padding, dilation, False)
+        up = up * (pre.abs() > 1e-5 * scale)
     (want * up.double()).sum().backward()
     (got * up.to(dev)).sum().backward()
     for name, p, r in (('x', xp, xr), ('w', wp, wr)) + ((('b', bp, br),) if bias else ()):
