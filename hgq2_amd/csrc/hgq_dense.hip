@@ -308,17 +308,39 @@ __global__ __launch_bounds__(256) void qdense_bwd_kernel(const float *__restrict
 struct FastMap {
     int row[FAST_NJ], col[FAST_NJ];
     bool on[FAST_NJ];
-    __device__ __forceinline__ void init(int W) {  // W = row width in floats, a multiple of 4
+    __device__ __forceinline__ void init(int W) {  // W = row width in floats, a multiple of 4, at most 64
         const int w4 = W >> 2;
+        // id / w4 for id < 1024, w4 <= 16 by a 16-bit reciprocal (exact: id * (ceil(2^16 / w4) - 2^16 / w4) < 2^16 / w4)
+        const uint32_t rcp = (65536u + (uint32_t)w4 - 1u) / (uint32_t)w4;
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
             const int id = threadIdx.x + 256 * j;
             on[j] = id < FAST_BM * w4;
-            row[j] = on[j] ? id / w4 : 0;
+            row[j] = on[j] ? (int)(((uint32_t)id * rcp) >> 16) : 0;
             col[j] = on[j] ? (id - row[j] * w4) << 2 : 0;
         }
     }
 };
+
+// Fractional bits of the elements a thread stages, fi[j][e], from the [P, K] table (P a power of two); tix[j] is the
+// table entry of slot j's first element.  Every load is issued before any is waited for (a load inside a branch is
+// waited for where it is issued, one memory latency per element).
+template <bool QUANT>
+__device__ __forceinline__ void fast_frac_bits(const float *f_in, int P, int K, const FastMap &mp, bool round_params,
+                                               int (&fi)[FAST_NJ][4], int (&tix)[FAST_NJ]) {
+    const __amdgpu_buffer_rsrc_t rs_f = buf_rsrc(f_in, QUANT ? (int64_t)P * K * 4 : 0);
+    float fv[FAST_NJ][4];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) {
+        tix[j] = (mp.row[j] & (P - 1)) * K + mp.col[j];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) fv[j][e] = QUANT ? buf_ld1(rs_f, mp.on[j] ? (uint32_t)(tix[j] + e) * 4u : BUF_OOB) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) fi[j][e] = (int)(round_params ? rintf(fv[j][e]) : fv[j][e]);
+}
 
 __device__ __forceinline__ void st4(float *p, const float4 &v) {
     f32x4_t t;
@@ -358,18 +380,13 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
     mp.init(K);
     const bool vec_out = (N & 3) == 0 && ((uintptr_t)y & 15u) == 0;
     mo.init(vec_out ? N : 4);
-    int fi[FAST_NJ][4];
+    int fi[FAST_NJ][4], tix[FAST_NJ];
     uint32_t amx[FAST_NJ][4];
+    fast_frac_bits<QUANT>(f_in, P, K, mp, m.round_params, fi, tix);
 #pragma unroll
     for (int j = 0; j < FAST_NJ; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            amx[j][e] = 0, fi[j][e] = 0;
-            if (QUANT && mp.on[j]) {
-                const float f = f_in[(mp.row[j] % P) * K + mp.col[j] + e];
-                fi[j][e] = (int)(m.round_params ? rintf(f) : f);
-            }
-        }
+        for (int e = 0; e < 4; ++e) amx[j][e] = 0;
     f32x4_t raw[FAST_NJ];
     uint32_t xoff[FAST_NJ];
 #pragma unroll
@@ -415,6 +432,8 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
             f32x4_t a4[NS4];
 #pragma unroll
             for (int s4 = 0; s4 < NS4; ++s4) a4[s4] = *(const f32x4_t *)(arow_p + 4 * s4);
+            // the reads stay ahead of the chain (rescheduled, they would share registers and wait for the instructions in between)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int s4 = 0; s4 < NS4; ++s4)
 #pragma unroll
@@ -459,7 +478,7 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
         for (int j = 0; j < FAST_NJ; ++j)
             if (mp.on[j])
 #pragma unroll
-                for (int e = 0; e < 4; ++e) atomicMax(&tab[(mp.row[j] % P) * K + mp.col[j] + e], amx[j][e]);
+                for (int e = 0; e < 4; ++e) atomicMax(&tab[tix[j] + e], amx[j][e]);
         __syncthreads();
         uint32_t *my = amax_part + (int64_t)blockIdx.x * PK;
         for (int t = tid; t < PK; t += 256) my[t] = tab[t];
@@ -491,17 +510,8 @@ __global__ __launch_bounds__(256, 2) void dense_moments_fast_kernel(const float 
     }
     FastMap mp;
     mp.init(K);
-    int fi[FAST_NJ][4];
-#pragma unroll
-    for (int j = 0; j < FAST_NJ; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            fi[j][e] = 0;
-            if (QUANT && mp.on[j]) {
-                const float f = f_in[(mp.row[j] % P) * K + mp.col[j] + e];
-                fi[j][e] = (int)(Mode(mode).round_params ? rintf(f) : f);
-            }
-        }
+    int fi[FAST_NJ][4], tix[FAST_NJ];
+    fast_frac_bits<QUANT>(f_in, P, K, mp, Mode(mode).round_params, fi, tix);
     f32x4_t raw[FAST_NJ];
     uint32_t xoff[FAST_NJ];
 #pragma unroll
@@ -608,18 +618,13 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     }
     FastMap mx, mz;
     mx.init(K), mz.init(N);
-    int fi[FAST_NJ][4];
+    int fi[FAST_NJ][4], tix[FAST_NJ];
     float gf[FAST_NJ][4];
+    fast_frac_bits<QUANT>(f_in, P, K, mx, m.round_params, fi, tix);
 #pragma unroll
     for (int j = 0; j < FAST_NJ; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            gf[j][e] = 0.f, fi[j][e] = 0;
-            if (QUANT && mx.on[j]) {
-                const float f = f_in[(mx.row[j] % P) * K + mx.col[j] + e];
-                fi[j][e] = (int)(m.round_params ? rintf(f) : f);
-            }
-        }
+        for (int e = 0; e < 4; ++e) gf[j][e] = 0.f;
     // kernel-gradient block owned by this wave
     const int nblk = K32 * N32, wpb = 4 / nblk;
     const int blk = wave / wpb, sub = wave % wpb;
@@ -757,7 +762,10 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         }
         __syncthreads();
     }
-    for (int id = tid; id < K * N; id += 256) my_dw[id] = comb[(id / N) * FAST_LD + (id % N)];
+    for (int id = tid; id < K * 64; id += 256) {
+        const int kk = id >> 6, nn = id & 63;
+        if (nn < N) my_dw[kk * N + nn] = comb[kk * FAST_LD + nn];
+    }
     float *bred = &ws[0][0];
     __syncthreads();
     bred[tid] = accb;
@@ -774,11 +782,13 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 #pragma unroll
                 for (int e = 0; e < 4; ++e) gt[mx.row[j] * FAST_LD + mx.col[j] + e] = gf[j][e];
         __syncthreads();
-        for (int t = tid; t < PK; t += 256) {
-            const int p = t / K, c = t - p * K;
-            float s = 0.f;
-            for (int r = p; r < FAST_BM; r += P) s += gt[r * FAST_LD + c];
-            my_df[t] = s;
+        for (int id = tid; id < P * 64; id += 256) {
+            const int p = id >> 6, c = id & 63;
+            if (c < K) {
+                float s = 0.f;
+                for (int r = p; r < FAST_BM; r += P) s += gt[r * FAST_LD + c];
+                my_df[p * K + c] = s;
+            }
         }
     }
 }
