@@ -594,6 +594,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5;
+    const bool split_n = K32 == 1 && N32 == 2;
     const int PK = QUANT ? P * K : 0;
     const int64_t M = (int64_t)K * N + N + PK;
     const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
@@ -709,7 +710,11 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         // ---- dx = dz @ qW^T : blocks (row half, k block), kept in registers until dz is no longer needed
         floatx16 acc = {0};
         const int rh = wave & 1, kb = wave >> 1;
-        if (kb < K32) {
+        if (split_n) {
+            // one k block, two column blocks: the two wavefronts of a row half take one half of the contraction each
+            const int arow = rh * 32 + (lane & 31), kq = lane >> 5, n0 = kb * 32;
+            acc = mfma_chain(acc, &dzs[arow][n0 + kq], 1, &ws[lane & 31][n0 + kq], 1, 2);
+        } else if (kb < K32) {
             const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
             acc = mfma_chain(acc, &dzs[arow][kq], 1, &ws[wrow][kq], 1, N32 * 2);
         }
@@ -723,8 +728,12 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 #pragma unroll
             for (int j = 0; j < FAST_BM / 4; ++j) accb += dzs[bq * (FAST_BM / 4) + j][bn];
         }
-        __syncthreads();  // dz consumed: the dx tile takes its place
-        if (kb < K32) {
+        __syncthreads();  // dz and xq consumed: the dx tile takes the place of dz (its second partial sum that of xq)
+        if (split_n) {
+            float(*dst)[FAST_LD] = kb ? xs : dzs;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dst[rh * 32 + acc_row(r, lane)][lane & 31] = acc[r];
+        } else if (kb < K32) {
             const int kcol = kb * 32 + (lane & 31);
 #pragma unroll
             for (int r = 0; r < 16; ++r) dzs[rh * 32 + acc_row(r, lane)][kcol] = acc[r];
@@ -737,6 +746,10 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                 float4 o;
                 o.x = dzs[mx.row[j]][mx.col[j]], o.y = dzs[mx.row[j]][mx.col[j] + 1];
                 o.z = dzs[mx.row[j]][mx.col[j] + 2], o.w = dzs[mx.row[j]][mx.col[j] + 3];
+                if (split_n) {
+                    o.x += xs[mx.row[j]][mx.col[j]], o.y += xs[mx.row[j]][mx.col[j] + 1];
+                    o.z += xs[mx.row[j]][mx.col[j] + 2], o.w += xs[mx.row[j]][mx.col[j] + 3];
+                }
                 if (gr < rows) {
                     st4(dx + gr * K + mx.col[j], o);
                     if (QUANT) {
@@ -762,6 +775,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         }
         __syncthreads();
     }
+#pragma unroll 4
     for (int id = tid; id < K * 64; id += 256) {
         const int kk = id >> 6, nn = id & 63;
         if (nn < N) my_dw[kk * N + nn] = comb[kk * FAST_LD + nn];
@@ -782,6 +796,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 #pragma unroll
                 for (int e = 0; e < 4; ++e) gt[mx.row[j] * FAST_LD + mx.col[j] + e] = gf[j][e];
         __syncthreads();
+#pragma unroll 4
         for (int id = tid; id < P * 64; id += 256) {
             const int p = id >> 6, c = id & 63;
             if (c < K) {
