@@ -58,7 +58,7 @@ SIGNATURES = {
     'hgq_bn_fold_bwd': (c_int, [c_void_p] * 4 + [c_int, c_float] + [c_void_p] * 7 + [c_int, c_int, c_void_p]),
     'hgq_qdense_moments_workspace': (c_int64, [c_int64, c_int, c_int, c_int64]),
     'hgq_qdense_moments_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
-    'hgq_qdense_moments_bwd': (c_int, [c_void_p, c_void_p, c_int64, c_int] + [c_void_p] * 7 + [c_int64, c_int, c_int, c_void_p]),
+    'hgq_qdense_moments_bwd': (c_int, [c_void_p, c_void_p, c_int64, c_int] + [c_void_p] * 8 + [c_int64, c_int, c_int, c_void_p]),
     'hgq_dense_moments_workspace': (c_int64, [c_int64, c_int, c_int]),
     'hgq_dense_moments_fwd': (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_void_p]),
     'hgq_dense_moments_bwd': (c_int, [c_void_p] * 7 + [c_int64, c_int, c_int, c_void_p]),

@@ -587,10 +587,12 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
                                                               float *part, int has_bias, int64_t rows, int K, int N, int act,
-                                                              int mode) {
+                                                              int mode, const float *__restrict__ dx_add) {
     __shared__ float xs[FAST_BM + 1][FAST_LD];   // row FAST_BM: sink of the idle staging slots
     __shared__ float dzs[FAST_BM + 1][FAST_LD];  // dz, then the dx tile
     __shared__ float ws[64][FAST_LD];
+    __shared__ float adds[STATS ? FAST_BM + 1 : 1][STATS ? FAST_LD : 1];  // STATS: the tile of dx_add, staged with x
+    const bool has_add = STATS && dx_add != nullptr;
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5;
@@ -649,7 +651,8 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     auto load_tile = [&](int64_t t) {
         const int64_t r0 = t * FAST_BM, left = rows - r0, vr = left < FAST_BM ? left : FAST_BM;
         const __amdgpu_buffer_rsrc_t sx = buf_rsrc(x + r0 * K, vr * K * 4);
-        const __amdgpu_buffer_rsrc_t sg = buf_rsrc(STATS ? x : dy + r0 * N, STATS ? 0 : vr * N * 4);
+        const __amdgpu_buffer_rsrc_t sg = STATS ? buf_rsrc(has_add ? dx_add + r0 * K : x, has_add ? vr * K * 4 : 0)
+                                                : buf_rsrc(dy + r0 * N, vr * N * 4);
         const __amdgpu_buffer_rsrc_t sy = buf_rsrc((relu && !STATS) ? y + r0 * N : x, (relu && !STATS) ? vr * N * 4 : 0);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
@@ -657,6 +660,8 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
             if (!STATS) {
                 rg[j] = buf_ld4(sg, zoff[j]);
                 ry[j] = buf_ld4(sy, zoff[j]);
+            } else {
+                rg[j] = buf_ld4(sg, xoff[j]);  // the other gradient of x, laid out like x (zeros without one)
             }
         }
     };
@@ -679,7 +684,12 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                 dlt[j][e] = q - v[e];
                 xs[xr][mx.col[j] + e] = q;
             }
-            if (!STATS) {
+            if (STATS) {
+                if (has_add) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) adds[xr][mx.col[j] + e] = rg[j][e];
+                }
+            } else {
                 const float g[4] = {rg[j][0], rg[j][1], rg[j][2], rg[j][3]};
                 const float a[4] = {ry[j][0], ry[j][1], ry[j][2], ry[j][3]};
 #pragma unroll
@@ -750,11 +760,16 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                     o.x += xs[mx.row[j]][mx.col[j]], o.y += xs[mx.row[j]][mx.col[j] + 1];
                     o.z += xs[mx.row[j]][mx.col[j] + 2], o.w += xs[mx.row[j]][mx.col[j] + 3];
                 }
+                float4 og = o;  // this contraction's own gradient: the one the rounding residue meets
+                if (has_add) {
+                    o.x += adds[mx.row[j]][mx.col[j]], o.y += adds[mx.row[j]][mx.col[j] + 1];
+                    o.z += adds[mx.row[j]][mx.col[j] + 2], o.w += adds[mx.row[j]][mx.col[j] + 3];
+                }
                 if (gr < rows) {
                     st4(dx + gr * K + mx.col[j], o);
                     if (QUANT) {
-                        gf[j][0] += -HGQ_LN2 * dlt[j][0] * o.x, gf[j][1] += -HGQ_LN2 * dlt[j][1] * o.y;
-                        gf[j][2] += -HGQ_LN2 * dlt[j][2] * o.z, gf[j][3] += -HGQ_LN2 * dlt[j][3] * o.w;
+                        gf[j][0] += -HGQ_LN2 * dlt[j][0] * og.x, gf[j][1] += -HGQ_LN2 * dlt[j][1] * og.y;
+                        gf[j][2] += -HGQ_LN2 * dlt[j][2] * og.z, gf[j][3] += -HGQ_LN2 * dlt[j][3] * og.w;
                     }
                 }
             }
@@ -982,20 +997,20 @@ extern "C" int hgq_dense_moments_fwd(const float *x, const float *w, float *mean
 }
 
 extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, const float *dmean,
-                                      const float *dmeansq, float *dx, float *dw, float *df_in, float *workspace, int64_t rows, int K,
-                                      int N, void *stream) {
+                                      const float *dmeansq, const float *dx_add, float *dx, float *dw, float *df_in, float *workspace,
+                                      int64_t rows, int K, int N, void *stream) {
     hipStream_t s = (hipStream_t)stream;
     int rc = moments_check("hgq_qdense_moments_bwd", rows, K, N, x, f_in, bw_rows, mode);
     if (rc) return rc;
     if (!x || !w || !dmean || !dmeansq || !dx || !dw || !workspace) return fail(HGQ_ERR_ARG, "hgq_qdense_moments_bwd: null pointer");
-    if (!aligned16(dx)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_moments_bwd: dx must be 16-byte aligned");
+    if (!aligned16(dx) || !aligned16(dx_add)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_moments_bwd: dx and dx_add must be 16-byte aligned");
     const int parts = row_parts(rows, BWD_BM);
     const bool quant = bw_rows > 0;
     const int P = quant ? (int)bw_rows : 1;
     const int rm = Mode(mode).round_mode;
     const dim3 grid((unsigned)parts);
 #define HGQ_MOM_BWD(RMV, QV) \
-    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode)
+    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode, dx_add)
     if (!quant) HGQ_MOM_BWD(HGQ_TRN, false);
     else if (rm == HGQ_TRN) HGQ_MOM_BWD(HGQ_TRN, true);
     else if (rm == HGQ_RND) HGQ_MOM_BWD(HGQ_RND, true);
@@ -1008,7 +1023,7 @@ extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t
 
 extern "C" int hgq_dense_moments_bwd(const float *x, const float *w, const float *dmean, const float *dmeansq, float *dx, float *dw,
                                      float *workspace, int64_t rows, int K, int N, void *stream) {
-    return hgq_qdense_moments_bwd(x, nullptr, 0, 0, w, dmean, dmeansq, dx, dw, nullptr, workspace, rows, K, N, stream);
+    return hgq_qdense_moments_bwd(x, nullptr, 0, 0, w, dmean, dmeansq, nullptr, dx, dw, nullptr, workspace, rows, K, N, stream);
 }
 
 extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
@@ -1042,7 +1057,7 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
         const int P = quant ? (int)bw_rows : 1;
         const dim3 fgrid((unsigned)parts);
 #define HGQ_BWD_FAST(RMV, QV) \
-    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, dqb ? 1 : 0, rows, K, N, act, mode)
+    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr)
         if (!quant) HGQ_BWD_FAST(HGQ_TRN, false);
         else if (m.round_mode == HGQ_TRN) HGQ_BWD_FAST(HGQ_TRN, true);
         else if (m.round_mode == HGQ_RND) HGQ_BWD_FAST(HGQ_RND, true);

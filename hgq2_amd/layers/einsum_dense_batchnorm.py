@@ -92,19 +92,27 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         n_out = len(self.full_output_shape)
         return self._gemm is not None and self._reduction_axes == tuple(range(n_out - self._gemm[1]))
 
-    def _batch_moments(self, qinputs, raw=False, quant=None):
+    def _batch_moments(self, qinputs, raw=False, quant=None, chain=False):
         """Mean and variance (``raw``: mean of squares, flat) of the un-quantized-kernel pre-activation
         over the non-normalised axes (reference :108-112).  GEMM-shaped equations whose normalised axes
         are all the new output axes run through the dense and column-moment kernels; others through the
-        library einsum."""
+        library einsum.  ``chain`` (with ``raw``): a third result, the input to hand to the output contraction
+        - the same values, routed so that its gradient is added inside the statistics' backward kernel -
+        or ``None`` where the path taken has no such kernel."""
         n_out = len(self.full_output_shape)
         trailing = self._trailing_gemm()
         if trailing and qinputs.is_cuda:
             x2d = qinputs.reshape(-1, self._K)
             w2d = self._kernel.reshape(self._K, self._N)
             x2d = x2d.contiguous()
+            alias = None
             if ops.dense_moments_supported(x2d, w2d):
-                mean, meansq = ops.dense_moments(x2d, w2d, quant)  # one pass over x, the pre-activation is never written
+                # one pass over x, the pre-activation is never written
+                if chain and raw:
+                    mean, meansq, alias = ops.dense_moments(x2d, w2d, quant, chain=True)
+                    alias = alias.view(qinputs.shape)
+                else:
+                    mean, meansq = ops.dense_moments(x2d, w2d, quant)
             else:
                 if self._K <= ops.FUSED_BWD_MAX and self._N <= ops.FUSED_BWD_MAX:
                     pre, _ = ops.qdense(x2d, None, None, None, w2d, None, _lib.ACT_NONE, 0, 0, False)
@@ -112,7 +120,7 @@ class QEinsumDenseBatchnorm(QEinsumDense):
                     pre = ops.matmul_bias_act(x2d, w2d, None, _lib.ACT_NONE)
                 mean, meansq = ops.col_moments(pre)
             if raw:
-                return mean, meansq
+                return (mean, meansq, alias) if chain else (mean, meansq)
             shape = tuple(self.full_output_shape[n_out - self._gemm[1]:])
             mean, meansq = mean.view(shape), meansq.view(shape)
             return mean, meansq - torch.square(mean)
@@ -141,7 +149,9 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         if training and self.trainable and inputs.is_cuda and self._trailing_gemm() and self.bias.numel() == self._N:
             # statistics, folding and the moving-average update in three launches (the folding algebra and its
             # gradient would otherwise be some forty elementwise launches on [N] vectors)
-            mean, meansq = self._batch_moments(inputs, raw=True, quant=quant)
+            mean, meansq, chained = self._batch_moments(inputs, raw=True, quant=quant, chain=True)
+            if chained is not None:
+                inputs = chained
             fused_kernel, fused_bias = ops.bn_fold(self._kernel.reshape(self._K, self._N), self.bias.reshape(-1),
                                                    self.bn_gamma.reshape(-1) if self.scale else None, mean, meansq, True, epsilon(),
                                                    self.moving_mean.view(-1), self.moving_variance.view(-1), self.momentum)

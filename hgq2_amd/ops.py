@@ -720,21 +720,24 @@ def _(x, w, f_in, bw_rows, mode):
 
 @torch.library.custom_op('hgq::dense_moments_bwd', mutates_args=())
 def dense_moments_bwd(x: Tensor, w: Tensor, f_in: Tensor, bw_rows: int, mode: int, dmean: Tensor,
-                      dmeansq: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+                      dmeansq: Tensor, dx_add: Tensor) -> tuple[Tensor, Tensor, Tensor]:
     _check_f32('x', x), _check_f32('w', w), _check_f32('dmean', dmean), _check_f32('dmeansq', dmeansq)
+    if dx_add.numel():
+        _check_f32('dx_add', dx_add)
+        _need(dx_add.shape == x.shape, 'dx_add must have the shape of x')
     rows, K = x.shape
     N = w.shape[1]
     lib = _lib.load()
     dx, dw = torch.empty_like(x), torch.empty_like(w)
     df = torch.empty(bw_rows * K, dtype=torch.float32, device=x.device)
     ws = torch.empty(max(lib.hgq_qdense_moments_workspace(rows, K, N, bw_rows), 1), dtype=torch.float32, device=x.device)
-    _lib.check(lib.hgq_qdense_moments_bwd(_ptr(x), _ptr(f_in), bw_rows, mode, _ptr(w), _ptr(dmean), _ptr(dmeansq), _ptr(dx), _ptr(dw),
-                                          _ptr(df), _ptr(ws), rows, K, N, _stream()), 'hgq_qdense_moments_bwd')
+    _lib.check(lib.hgq_qdense_moments_bwd(_ptr(x), _ptr(f_in), bw_rows, mode, _ptr(w), _ptr(dmean), _ptr(dmeansq), _ptr(dx_add), _ptr(dx),
+                                          _ptr(dw), _ptr(df), _ptr(ws), rows, K, N, _stream()), 'hgq_qdense_moments_bwd')
     return dx, dw, df
 
 
 @dense_moments_bwd.register_fake
-def _(x, w, f_in, bw_rows, mode, dmean, dmeansq):
+def _(x, w, f_in, bw_rows, mode, dmean, dmeansq, dx_add):
     return torch.empty_like(x), torch.empty_like(w), x.new_empty(bw_rows * x.shape[1])
 
 
@@ -1125,30 +1128,38 @@ def col_moments(x2d: Tensor):
 
 
 class _DenseMoments(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, x, w, f_in, bw_rows, mode):
-        ctx.save_for_backward(x, w, f_in)
-        ctx.quant = (bw_rows, mode)
-        return dense_moments_fwd(x, w, f_in, bw_rows, mode)
+    """``chain``: the input is also returned, as the third output, for its other consumer (the output contraction of
+    the same layer); the gradient that comes back through it is added while this backward writes dx, instead of in an
+    accumulation pass of its own."""
 
     @staticmethod
-    def backward(ctx, dmean, dmeansq):
+    def forward(ctx, x, w, f_in, bw_rows, mode, chain):
+        ctx.save_for_backward(x, w, f_in)
+        ctx.quant = (bw_rows, mode)
+        mean, meansq = dense_moments_fwd(x, w, f_in, bw_rows, mode)
+        return (mean, meansq, x) if chain else (mean, meansq)
+
+    @staticmethod
+    def backward(ctx, dmean, dmeansq, dx_chain=None):
         x, w, f_in = ctx.saved_tensors
         bw_rows, mode = ctx.quant
         zero = x.new_zeros(w.shape[1])
+        # without a consumer of dx (an input that needs no gradient) the chained gradient is not read either
+        dx_add = x.new_empty(0) if dx_chain is None or not ctx.needs_input_grad[0] else dx_chain.contiguous()
         dx, dw, df = dense_moments_bwd(x, w, f_in, bw_rows, mode, dmean.contiguous() if dmean is not None else zero,
-                                       dmeansq.contiguous() if dmeansq is not None else zero)
-        return dx, dw, (df.view(f_in.shape) if bw_rows else None), None, None
+                                       dmeansq.contiguous() if dmeansq is not None else zero, dx_add)
+        return dx, dw, (df.view(f_in.shape) if bw_rows else None), None, None, None
 
 
-def dense_moments(x2d: Tensor, w2d: Tensor, quant=None):
+def dense_moments(x2d: Tensor, w2d: Tensor, quant=None, chain=False):
     """``(mean(z, 0), mean(z * z, 0))`` of ``z = q(x2d) @ w2d`` without materialising ``z`` (nor ``q(x2d)``).
     ``quant`` = ``(f_in, bw_rows, mode)``: the raw fractional bits of a training-mode WRAP input quantizer laid out as
-    a ``[bw_rows, K]`` table; ``None``: ``x2d`` is contracted as it is."""
+    a ``[bw_rows, K]`` table; ``None``: ``x2d`` is contracted as it is.  ``chain``: a third result, ``x2d`` again, to be
+    used by the caller instead of ``x2d`` from here on (see ``_DenseMoments``)."""
     if quant is None:
-        return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous(), x2d.new_empty(0), 0, 0)
+        return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous(), x2d.new_empty(0), 0, 0, chain)
     f_in, bw_rows, mode = quant
-    return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous(), f_in.contiguous(), int(bw_rows), int(mode))
+    return _DenseMoments.apply(x2d.contiguous(), w2d.contiguous(), f_in.contiguous(), int(bw_rows), int(mode), chain)
 
 
 class _BnFold(torch.autograd.Function):

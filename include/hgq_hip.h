@@ -450,13 +450,15 @@ int hgq_dense_moments_bwd(const float *x, const float *w, const float *dmean, co
  * bw_rows divides 64), mode its HGQ_MODE(...) bits.  The quantized input is never written; the backward returns dx
  * with respect to the raw input (straight-through) and df_in [bw_rows * K], this contraction's share of the
  * fractional-bit gradient.  bw_rows == 0: no quantizer (the entry points above).
+ * dx_add (may be null): [rows, K], 16-byte aligned, added to dx while it is written - the gradient x receives from its
+ * other use, the output contraction, so that the two need no separate accumulation pass; it does not enter df_in.
  */
 int64_t hgq_qdense_moments_workspace(int64_t rows, int K, int N, int64_t bw_rows);
 int hgq_qdense_moments_fwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, float *mean, float *meansq,
                            float *workspace, int64_t rows, int K, int N, void *stream);
 int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, const float *dmean,
-                           const float *dmeansq, float *dx, float *dw, float *df_in, float *workspace, int64_t rows, int K, int N,
-                           void *stream);
+                           const float *dmeansq, const float *dx_add, float *dx, float *dw, float *df_in, float *workspace,
+                           int64_t rows, int K, int N, void *stream);
 
 /*
  * Per-column mean and mean of squares of a [rows, N] matrix, and the gradient of both.  Replaces

@@ -643,3 +643,40 @@ def test_dense_moments_with_the_input_quantizer_inside(rows, K, N, bw_rows):
         want = want.detach().float()
         err = float((got.detach().cpu() - want).abs().max())
         assert err <= 2e-5 * float(want.abs().max()) + 1e-7, f'{name}: {err:.3e}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('rows,K,N,bw_rows', [(640, 16, 64, 64), (200, 64, 32, 0), (131, 20, 12, 1)])
+def test_dense_moments_chained_input_gradient(rows, K, N, bw_rows):
+    """``chain=True``: the third result stands for x in a second consumer, whose gradient is added while the
+    statistics' backward writes dx - equal to the unchained gradient plus that of the second consumer; the
+    fractional-bit gradient of the statistics does not see it."""
+    from hgq2_amd import _lib, ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(rows + K)
+    x = (torch.randn(rows, K, generator=g) * 2).to(dev)
+    w = (torch.randn(K, N, generator=g) * 0.4).to(dev)
+    um, us, u2 = torch.randn(N, generator=g).to(dev), torch.randn(N, generator=g).to(dev), torch.randn(rows, K, generator=g).to(dev)
+    quant = None
+    if bw_rows:
+        f = torch.randint(2, 7, (bw_rows, K), generator=g).float().to(dev)
+        mode = _lib.mode_bits('RND', 'WRAP', training=True, round_params=True)
+    res = []
+    for chain in (False, True):
+        xd, wd = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        fd = f.clone().requires_grad_(True) if bw_rows else None
+        quant = (fd.view(-1), bw_rows, mode) if bw_rows else None
+        out = ops.dense_moments(xd, wd, quant, chain=chain)
+        second = out[2] if chain else xd
+        if chain:
+            assert torch.equal(second, xd)
+        ((out[0] * um).sum() + (out[1] * us).sum() + (second * second * u2).sum()).backward()
+        res.append((out[0].detach(), out[1].detach(), xd.grad, wd.grad, fd.grad if bw_rows else None))
+    for name, a, b in zip(('mean', 'meansq', 'dx', 'dw', 'df'), *res):
+        if a is None:
+            continue
+        if name == 'dx':  # the sum is formed in a different order
+            assert float((a - b).abs().max()) <= 1e-6 * float(a.abs().max()), name
+        else:
+            assert torch.equal(a, b), name
