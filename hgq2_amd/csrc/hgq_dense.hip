@@ -467,7 +467,17 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
             }
         }
     }
-    if (QUANT && amax_part) {
+    if (QUANT && amax_part && P == FAST_BM && ((uintptr_t)amax_part & 15u) == 0) {
+        // one table row per tile row: every entry of this workgroup's slice has exactly one owner thread
+        uint32_t *my = amax_part + (int64_t)blockIdx.x * (P * K);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j)
+            if (mp.on[j]) {
+                uint4 v;
+                v.x = amx[j][0], v.y = amx[j][1], v.z = amx[j][2], v.w = amx[j][3];
+                *(uint4 *)(my + tix[j]) = v;
+            }
+    } else if (QUANT && amax_part) {
         // this workgroup's slice: combine the registers of all threads through an LDS table
         const int PK = P * K;
         uint32_t *tab = (uint32_t *)&xs[0][0][0];
