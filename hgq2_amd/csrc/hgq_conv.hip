@@ -491,6 +491,7 @@ template <int KH, int KW, int C>
 __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                          const float *__restrict__ bias, float *__restrict__ out, hgq_conv_geom g,
                                                          int F, int act, int tiles_x, int tiles_y) {
+#pragma clang fp contract(fast)  // multiply-adds of the convolution sum may fuse (see bwd_smallc_kernel)
     constexpr int KC = KH * KW * C;
     extern __shared__ float lds[];  // input patch [XH][XW][C]
     const int XH = (SC_TH - 1) * g.sy + (KH - 1) * g.dly + 1, XW = (SC_TW - 1) * g.sx + (KW - 1) * g.dlx + 1;
@@ -507,8 +508,9 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
         const int oy0 = (rem / tiles_x) * SC_TH, ox0 = (rem % tiles_x) * SC_TW;
         const int iy0 = oy0 * g.sy - g.py, ix0 = ox0 * g.sx - g.px;
         __syncthreads();
+        const FastDiv d_xw((uint32_t)(XW * C));
         for (int e = threadIdx.x; e < XH * XW * C; e += 256) {
-            const int r = e / (XW * C), q = e - r * XW * C, iy = iy0 + r, ix = ix0 + q / C;
+            const int r = (int)d_xw.div((uint32_t)e), q = e - r * XW * C, iy = iy0 + r, ix = ix0 + q / C;
             const bool ok = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
             lds[e] = buf_ld1(rs_x, ok ? (uint32_t)(((b * g.H + iy) * g.W + ix0) * C + q) * 4u : BUF_OOB);
         }
@@ -548,13 +550,15 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                                                          const float *__restrict__ x, const float *__restrict__ w,
                                                          float *__restrict__ dx, float *__restrict__ part, hgq_conv_geom g, int F,
                                                          int tiles_x, int tiles_y, int vec) {
+    // the multiply-adds of the two contractions below may fuse (the file is built without contraction for the quantizer
+    // arithmetic; a convolution sum has no such contract, and unfused it costs two vector instructions per term)
+#pragma clang fp contract(fast)
     constexpr int KC = KH * KW * C, PH = SC_TH + KH - 1, PW = SC_TW + KW - 1;
     extern __shared__ float lds[];  // kernel [KC * F] | dz patch [PH * PW][F + 1] (reused for the final sum) | input patch
     const int FS = F + 1, XH = PH + g.py, XW = PW + g.px;
-    float *wl = lds, *zp = lds + ((KC * F + 3) & ~3), *xp = zp + max(PH * PW * FS, SC_TH * (KC + 1) * 32);
+    float *zp = lds + ((KC * F + 3) & ~3), *xp = zp + max(PH * PW * FS, SC_TH * (KC + 1) * 32);
     const int tid = threadIdx.x, f = tid & 31, slot = tid >> 5;
     const bool f_on = f < F;
-    for (int t = tid; t < KC * F; t += 256) wl[t] = w[t];
     // whole-tensor buffer descriptors (the launcher guarantees they are smaller than 2 GiB)
     const int64_t dy_bytes = (int64_t)g.B * g.OH * g.OW * F * 4;
     const __amdgpu_buffer_rsrc_t rs_dy = buf_rsrc(dy, dy_bytes), rs_mask = buf_rsrc(mask ? mask : dy, mask ? dy_bytes : 0),
@@ -571,6 +575,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
         // buffer loads (zeros outside the tensor, no branch around a load): all units of a batch are in flight together
         if (vec) {
             const int upr = PW * F / 4, n_u = PH * upr;
+            const FastDiv d_upr((uint32_t)upr), d_f((uint32_t)F);  // no integer division per unit
             for (int e0 = 0; e0 < n_u; e0 += 4 * 256) {
                 f32x4_t v[4], m[4];
                 int dst[4];
@@ -580,7 +585,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                     uint32_t off = BUF_OOB;
                     dst[u] = -1;
                     if (e < n_u) {
-                        const int pr = e / upr, q = (e - pr * upr) * 4, pc = q / F, f0 = q - pc * F;
+                        const int pr = (int)d_upr.div((uint32_t)e), q = (e - pr * upr) * 4, pc = (int)d_f.div((uint32_t)q), f0 = q - pc * F;
                         const int oy = oy0 + pr, ox = ox0 + pc;
                         dst[u] = (pr * PW + pc) * FS + f0;
                         if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) off = (uint32_t)(((b * g.OH + oy) * g.OW + ox) * F + f0) * 4u;
@@ -598,6 +603,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
             }
         } else {
             const int upr = PW * F, n_u = PH * upr;
+            const FastDiv d_upr((uint32_t)upr), d_f((uint32_t)F);
             for (int e0 = 0; e0 < n_u; e0 += 8 * 256) {
                 float v[8], m[8];
                 int dst[8];
@@ -607,7 +613,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                     uint32_t off = BUF_OOB;
                     dst[u] = -1;
                     if (e < n_u) {
-                        const int pr = e / upr, q = e - pr * upr, pc = q / F, f0 = q - pc * F;
+                        const int pr = (int)d_upr.div((uint32_t)e), q = e - pr * upr, pc = (int)d_f.div((uint32_t)q), f0 = q - pc * F;
                         const int oy = oy0 + pr, ox = ox0 + pc;
                         dst[u] = (pr * PW + pc) * FS + f0;
                         if ((unsigned)oy < (unsigned)g.OH && (unsigned)ox < (unsigned)g.OW) off = (uint32_t)(((b * g.OH + oy) * g.OW + ox) * F + f0) * 4u;
@@ -621,8 +627,9 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
             }
         }
         if (part) {
+            const FastDiv d_xw((uint32_t)(XW * C));
             for (int e = tid; e < XH * XW * C; e += 256) {
-                const int r = e / (XW * C), q = e - r * XW * C, iy = iy0 - g.py + r, ix = ix0 - g.px + q / C;
+                const int r = (int)d_xw.div((uint32_t)e), q = e - r * XW * C, iy = iy0 - g.py + r, ix = ix0 - g.px + q / C;
                 const bool ok = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
                 xp[e] = buf_ld1(rs_x, ok ? (uint32_t)(((b * g.H + iy) * g.W + ix) * C + q % C) * 4u : BUF_OOB);
             }
@@ -641,7 +648,9 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                     for (int kx = 0; kx < KW; ++kx) {
                         // oy = iy + py - ky  ->  patch row ty + (KH - 1) - ky
                         const float *pp = zp + ((ty + KH - 1 - ky) * PW + (tx + KW - 1 - kx)) * FS;
-                        const float *wt = wl + (ky * KW + kx) * C * F;
+                        // kernel entries straight from memory: the address is the same in every lane, so they arrive
+                        // through the scalar cache and enter the multiply-adds as scalar operands (no LDS reads for them)
+                        const float *wt = w + (ky * KW + kx) * C * F;
                         int ff = 0;
                         for (; ff + 8 <= F; ff += 8) {
                             float v[8];

@@ -183,6 +183,16 @@ __device__ __forceinline__ float buf_ld1(__amdgpu_buffer_rsrc_t r, uint32_t byte
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
 }
 
+// c / d for c < 2**21 through the float reciprocal: (c + 0.5) / d is at least 0.5 / d away from an integer, more than the
+// rounding error of the two float operations below that bound.
+struct FastDiv {
+    uint32_t d;
+    float inv;
+    __device__ __forceinline__ explicit FastDiv(uint32_t d_) : d(d_), inv(1.0f / (float)d_) {}
+    __device__ __forceinline__ uint32_t div(uint32_t c) const { return (uint32_t)(((float)c + 0.5f) * inv); }
+    __device__ __forceinline__ uint32_t mod(uint32_t c) const { return c - div(c) * d; }
+};
+
 // ------------------------------------------------------------------------------------------
 // all-reduce over groups of SUB consecutive lanes (SUB = 16, 32 or 64): four DPP steps inside
 // each 16-lane row (xor 1, xor 2, half-row mirror, row mirror), then the row totals are read

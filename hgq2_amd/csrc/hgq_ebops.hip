@@ -112,16 +112,6 @@ struct Bits {
     }
 };
 
-// c / d for c < 2**21 through the float reciprocal: (c + 0.5) / d is at least 0.5 / d away from an integer, more than the
-// rounding error of the two float operations below that bound.
-struct FastDiv {
-    uint32_t d;
-    float inv;
-    __device__ __forceinline__ explicit FastDiv(uint32_t d_) : d(d_), inv(1.0f / (float)d_) {}
-    __device__ __forceinline__ uint32_t div(uint32_t c) const { return (uint32_t)(((float)c + 0.5f) * inv); }
-    __device__ __forceinline__ uint32_t mod(uint32_t c) const { return c - div(c) * d; }
-};
-
 // Fixed-order sum over the workgroup (double: exact for integer-valued terms far beyond 2**24).
 __device__ __forceinline__ double block_sum(double v, double *red) {
     const int t = threadIdx.x;
