@@ -472,6 +472,31 @@ extern "C" int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float 
     return HGQ_OK;
 }
 
+struct SumBatch {
+    const float *term[HGQ_SUM_BATCH];
+};
+
+// one thread: the terms are added in list order, exactly as a chain of scalar additions would
+__global__ void sum_scalars_kernel(SumBatch b, int count, float *out) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        float v = b.term[0][0];
+        for (int t = 1; t < count; ++t) v = __fadd_rn(v, b.term[t][0]);
+        out[0] = v;
+    }
+}
+
+extern "C" int hgq_sum_scalars(const float *const *terms, int count, float *out, void *stream) {
+    if (!terms || !out || count < 1 || count > HGQ_SUM_BATCH) return fail(HGQ_ERR_ARG, "hgq_sum_scalars: 1 <= count <= %d terms expected", HGQ_SUM_BATCH);
+    SumBatch b;
+    for (int t = 0; t < count; ++t) {
+        if (!terms[t]) return fail(HGQ_ERR_ARG, "hgq_sum_scalars: null term %d", t);
+        b.term[t] = terms[t];
+    }
+    for (int t = count; t < HGQ_SUM_BATCH; ++t) b.term[t] = nullptr;
+    hipLaunchKernelGGL(sum_scalars_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, b, count, out);
+    return check_launch("hgq_sum_scalars");
+}
+
 extern "C" int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const float *beta, float *loss_term,
                                const void *k_in, float *i_in, const float *f_in, int64_t P, int K, int N,
                                const void *k_ker, const float *b_ker, const void *k_bias, const float *b_bias,

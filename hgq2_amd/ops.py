@@ -267,6 +267,51 @@ def sgd_update_multi_op(ws: Sequence[Tensor], gs: Sequence[Tensor], l1: Sequence
     _lib.check(rc, 'hgq_sgd_update_multi')
 
 
+SUM_BATCH = 64
+
+
+@torch.library.custom_op('hgq::sum_scalars', mutates_args=())
+def sum_scalars_op(terms: Sequence[Tensor]) -> Tensor:
+    n = len(terms)
+    _need(1 <= n <= SUM_BATCH, f'1 to {SUM_BATCH} terms are expected')
+    ptrs = (ctypes.c_void_p * n)()
+    for t, term in enumerate(terms):
+        _check_f32('term', term)
+        _need(term.numel() == 1, 'every term must hold one element')
+        ptrs[t] = term.data_ptr()
+    out = torch.empty((), dtype=torch.float32, device=terms[0].device)
+    rc = _lib.load().hgq_sum_scalars(ptrs, n, _ptr(out), _stream())
+    _lib.check(rc, 'hgq_sum_scalars')
+    return out
+
+
+@sum_scalars_op.register_fake
+def _(terms):
+    return terms[0].new_empty(())
+
+
+class _SumScalars(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, *terms):
+        ctx.shapes = [t.shape for t in terms]
+        return sum_scalars_op([t.detach() for t in terms])
+
+    @staticmethod
+    def backward(ctx, g):
+        # every term receives the same upstream gradient: views of it, no launches
+        return tuple(g.reshape(s) if ctx.needs_input_grad[t] else None for t, s in enumerate(ctx.shapes))
+
+
+def sum_scalars(terms: Sequence[Tensor]) -> Tensor:
+    """``((terms[0] + terms[1]) + terms[2]) + ...`` of one-element GPU tensors, in that order, in one launch
+    (chunks of ``SUM_BATCH``); differentiable."""
+    terms = list(terms)
+    while len(terms) > 1:
+        head, terms = terms[:SUM_BATCH], terms[SUM_BATCH:]
+        terms.insert(0, _SumScalars.apply(*head))
+    return terms[0]
+
+
 def _qdescs(ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor], modes: Sequence[int]):
     """Five ``hgq_qdesc`` structures (exp_iq, exp_oq, inv_iq, inv_oq, oq); an empty ``k`` means absent."""
     _need(len(ks) == 5 and len(is_) == 5 and len(fbs) == 5 and len(modes) == 5, 'five quantizer descriptors are expected')

@@ -18,17 +18,22 @@ def model_loss(model, base_loss, fold_regularizers: bool = False):
     """``base_loss + sum(add_loss terms) (+ variable regularizers)``.  With ``fold_regularizers``
     the MonoL1 terms are left out of the autograd graph: their constant gradient ``l1`` is added by
     :class:`SGD` inside the update kernel instead (same update, one launch less per variable)."""
-    loss = base_loss
+    terms = [base_loss]
     for m in model.modules():
-        for term in getattr(m, '_losses', ()):
-            loss = loss + term
+        terms.extend(getattr(m, '_losses', ()))
     for p in model.parameters():
         r = getattr(p, 'regularizer', None)
         if r is None or not p.requires_grad:  # Keras regularises trainable variables only
             continue
         if fold_regularizers and isinstance(r, MonoL1):
             continue
-        loss = loss + r(p)
+        terms.append(r(p))
+    if len(terms) > 1 and all(torch.is_tensor(t) and t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 for t in terms):
+        # the same additions in the same order, one launch
+        return ops.sum_scalars(terms).reshape(torch.broadcast_shapes(*[t.shape for t in terms]))
+    loss = base_loss
+    for term in terms[1:]:
+        loss = loss + term
     return loss
 
 

@@ -214,6 +214,15 @@ typedef struct {
 int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *stream);
 
 /*
+ * out[0] = ((terms[0][0] + terms[1][0]) + terms[2][0]) + ... : the scalar loss terms of a step (user loss, one
+ * `add_loss` term per layer - src/hgq/layers/core/base.py:102-110 - and the variable regularizers) added in list
+ * order, as Keras adds them one at a time, in one launch.  `terms` is a HOST array of `count` device pointers
+ * (1 <= count <= HGQ_SUM_BATCH); they travel as launch arguments, so the call is safe under HIP graph capture.
+ */
+#define HGQ_SUM_BATCH 64
+int hgq_sum_scalars(const float *const *terms, int count, float *out, void *stream);
+
+/*
  * One training step (forward, mean sparse categorical cross-entropy from logits, backward, SGD)
  * of a stack of QDense layers in three launches.  It performs, in the same order and with the
  * same arithmetic, what the per-layer entry points above do when the reference's call stack

@@ -278,3 +278,27 @@ def test_ebops_finish_scalar_tail(dev, value):
     assert out.item() == float(ef * np.float32(3.5e-6))
     assert int(var.view(torch.int32).item()) & 0xFFFFFFFF == int(ef) & 0xFFFFFFFF
     assert e.grad.item() == float(np.float32(2.0) * np.float32(3.5e-6) * np.float32(0.5))
+
+
+@pytest.mark.gpu
+def test_scalar_loss_terms_summed_in_one_launch():
+    """ops.sum_scalars == the chain of additions it stands for, bit for bit, and hands the upstream gradient to
+    every term; train.model_loss takes that route for GPU scalars."""
+    from hgq2_amd import ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(5)
+    vals = (torch.randn(70, generator=g) * torch.logspace(-6, 3, 70)).to(dev)
+    terms = [vals[t].clone().requires_grad_(t % 3 != 1) for t in range(70)]
+    terms[4] = terms[4].detach().reshape(1, 1).requires_grad_(True)
+    want = terms[0]
+    for t in terms[1:]:
+        want = want + t.reshape(())
+    got = ops.sum_scalars(terms)
+    assert torch.equal(got.reshape(()), want.detach().reshape(()))
+    (got * 3.0).backward()
+    for t, term in enumerate(terms):
+        if term.requires_grad:
+            assert term.grad.shape == term.shape and float(term.grad.reshape(())) == 3.0
+        else:
+            assert term.grad is None
