@@ -193,6 +193,15 @@ struct FastDiv {
     __device__ __forceinline__ uint32_t mod(uint32_t c) const { return c - div(c) * d; }
 };
 
+// Stores through a descriptor: a store at BUF_OOB (or anywhere past the descriptor's range) is dropped.
+typedef unsigned int u32x4_raw_t __attribute__((__vector_size__(16)));
+__device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, f32x4_t v) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_raw_t, v), r, byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st1(__amdgpu_buffer_rsrc_t r, uint32_t byte_off, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), r, byte_off, 0, 0);
+}
+
 // ------------------------------------------------------------------------------------------
 // all-reduce over groups of SUB consecutive lanes (SUB = 16, 32 or 64): four DPP steps inside
 // each 16-lane row (xor 1, xor 2, half-row mirror, row mirror), then the row totals are read

@@ -224,7 +224,21 @@ __device__ __forceinline__ void qc_load(const __amdgpu_buffer_rsrc_t rs, uint32_
     }
 }
 
-template <int RM, int OM, int VEC>
+template <int VEC>
+__device__ __forceinline__ void qc_store(const __amdgpu_buffer_rsrc_t rs, uint32_t off, const float *v) {
+    if (VEC == 4) {
+        f32x4_t t;
+        t[0] = v[0], t[1] = v[1 % VEC], t[2] = v[2 % VEC], t[3] = v[3 % VEC];
+        buf_st4(rs, off, t);
+    } else {
+        buf_st1(rs, off, v[0]);
+    }
+}
+
+// TRAIN: the quantizer's training flag as a template argument (the WRAP training branch is decided once, not per element).
+// A workgroup's chunk is below 2 GiB, so all index arithmetic inside it is 32-bit and a load and the store of the same
+// row share one byte offset; rows past the end of the chunk are dropped by the descriptors' range check.
+template <int RM, int OM, int VEC, bool TRAIN>
 __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ x, const void *__restrict__ k,
                                                       const float *__restrict__ i, const float *__restrict__ fb,
                                                       float *__restrict__ y, uint32_t *amax, uint32_t *anyneg,
@@ -232,24 +246,29 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
     const Mode m(mode);
     const int TY = 256 / TX;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
-    const int64_t cg = M / VEC;
-    const int64_t c = (int64_t)blockIdx.x * TX + tx;
+    const int cg = (int)(M / VEC);
+    const int c = (int)blockIdx.x * TX + tx;
     const bool active = c < cg;
     KIF p[VEC];
-    uint32_t lmax[VEC], lneg[VEC];
+    uint32_t lmax[VEC];
+    float lmin[VEC];  // a negative minimum <=> some tracked value was negative (-0 and NaN are not)
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) p[e] = KIF{0.f, 0.f, 0.f}, lmax[e] = 0, lneg[e] = 0;
+    for (int e = 0; e < VEC; ++e) p[e] = KIF{0.f, 0.f, 0.f}, lmax[e] = 0, lmin[e] = 0.f;
     const int64_t row0 = (int64_t)blockIdx.y * rows_per_wg;
-    const int64_t n_rows = min(rows - row0, rows_per_wg);
-    const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + row0 * M, n_rows * M * 4);
-    float *yb = y + row0 * M;
+    const int n_rows = (int)min(rows - row0, rows_per_wg);
+    const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + row0 * M, (int64_t)n_rows * M * 4);
+    const __amdgpu_buffer_rsrc_t rs_y = buf_rsrc(y + row0 * M, (int64_t)n_rows * M * 4);
+    const uint32_t row_bytes = (uint32_t)cg * VEC * 4u, trip_rows = (uint32_t)TY * QC_U;
+    // byte offset of this thread's element(s) in row `r` of the chunk
+    auto offset = [&](int r) { return (active && r < n_rows) ? (uint32_t)r * row_bytes + (uint32_t)c * (VEC * 4u) : BUF_OOB; };
     // the first rows are requested before the bit-width operands: a workgroup is short-lived (often a single
     // trip), and operands first would put two memory round trips end to end
     float xv[QC_U][VEC];
+    uint32_t off[QC_U];
 #pragma unroll
     for (int u = 0; u < QC_U; ++u) {
-        const int64_t r = ty + (int64_t)TY * u;
-        qc_load<VEC>(rs, (active && r < n_rows) ? (uint32_t)((r * cg + c) * VEC) * 4u : BUF_OOB, xv[u]);
+        off[u] = offset(ty + TY * u);
+        qc_load<VEC>(rs, off[u], xv[u]);
     }
     if (active) {
         float kv[VEC], iv[VEC], fv[VEC];
@@ -259,37 +278,40 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
 #pragma unroll
         for (int e = 0; e < VEC; ++e) p[e] = resolve_kif(kv[e], iv[e], fv[e], m.kbi, m.round_params);
     }
-    for (int64_t rb = 0; rb < n_rows; rb += (int64_t)TY * QC_U) {
+    const bool track_input = m.track_input;
+    for (int rb = 0; rb < n_rows; rb += (int)trip_rows) {
         float cur[QC_U][VEC];
+        uint32_t cur_off[QC_U];
 #pragma unroll
-        for (int u = 0; u < QC_U; ++u)
+        for (int u = 0; u < QC_U; ++u) {
+            cur_off[u] = off[u];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) cur[u][e] = xv[u][e];
+        }
         // next trip's rows in flight while this one is quantized
 #pragma unroll
         for (int u = 0; u < QC_U; ++u) {
-            const int64_t r = rb + (int64_t)TY * QC_U + ty + (int64_t)TY * u;
-            qc_load<VEC>(rs, (active && r < n_rows) ? (uint32_t)((r * cg + c) * VEC) * 4u : BUF_OOB, xv[u]);
+            off[u] = offset(rb + (int)trip_rows + ty + TY * u);
+            qc_load<VEC>(rs, off[u], xv[u]);
         }
 #pragma unroll
         for (int u = 0; u < QC_U; ++u) {
-            const int64_t r = rb + ty + (int64_t)TY * u;
             float yv[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                yv[e] = quantize<RM, OM>(cur[u][e], p[e], m.training);
-                const float tv = m.track_input ? cur[u][e] : yv[e];
+                yv[e] = quantize<RM, OM>(cur[u][e], p[e], TRAIN);
+                const float tv = track_input ? cur[u][e] : yv[e];
                 const uint32_t ab = abs_bits(tv);
                 lmax[e] = ab > lmax[e] ? ab : lmax[e];
-                lneg[e] |= tv < 0.0f ? 1u : 0u;
+                lmin[e] = fminf(lmin[e], tv);
             }
-            if (active && r < n_rows) VecIO<VEC>::store(yb, r * cg + c, yv);
+            qc_store<VEC>(rs_y, cur_off[u], yv);
         }
     }
     if (amax || anyneg) {
         __shared__ uint32_t smax[256 * VEC], sneg[256 * VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) smax[threadIdx.x * VEC + e] = lmax[e], sneg[threadIdx.x * VEC + e] = lneg[e];
+        for (int e = 0; e < VEC; ++e) smax[threadIdx.x * VEC + e] = lmax[e], sneg[threadIdx.x * VEC + e] = lmin[e] < 0.0f ? 1u : 0u;
         __syncthreads();
         for (int s = TY / 2; s > 0; s >>= 1) {
             if (ty < s) {
@@ -307,7 +329,7 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
             if (sliced) {
                 // one tracker slice per row chunk, written whole: nothing to clear beforehand, no atomics; the
                 // integer-bit update combines the slices
-                const int64_t base = (int64_t)blockIdx.y * M + c * VEC;
+                const int64_t base = (int64_t)blockIdx.y * M + (int64_t)c * VEC;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     if (amax) amax[base + e] = smax[tx * VEC + e];
@@ -547,6 +569,18 @@ static bool cols_grid(int64_t rows, int64_t M, int batch_rows, int64_t gx, int64
     return true;
 }
 
+// launch of the per-column forward kernel: vector width and training flag as template arguments
+#define HGQ_FWD_COLS_1(VECV, TRAINV, SLICED)                                                                                       \
+    hipLaunchKernelGGL((quant_fwd_cols<RM, OM, VECV, TRAINV>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, \
+                       amax, anyneg, rows, M, TX, rows_per_wg, mode, SLICED)
+#define HGQ_FWD_COLS(SLICED)                                  \
+    do {                                                      \
+        if (vec && m.training) HGQ_FWD_COLS_1(4, true, SLICED);       \
+        else if (vec) HGQ_FWD_COLS_1(4, false, SLICED);               \
+        else if (m.training) HGQ_FWD_COLS_1(1, true, SLICED);         \
+        else HGQ_FWD_COLS_1(1, false, SLICED);                        \
+    } while (0)
+
 extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, const float *fb, float *y,
                                 uint32_t *amax, uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner,
                                 int mode, void *stream) {
@@ -601,10 +635,7 @@ extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, c
         int64_t gy, rows_per_wg;
         cols_grid(rows, M, TY * QC_U, gx, gy, rows_per_wg);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
-            if (vec)
-                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 0);
-            else
-                hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 0);
+            HGQ_FWD_COLS(0);
         });
         return check_launch("hgq_quantize_fwd");
     }
@@ -647,10 +678,7 @@ extern "C" int hgq_quantize_fwd_sliced(const float *x, const void *k, const floa
         return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_sliced: operands must be 16-byte aligned when bw_size is a multiple of 4");
     const int64_t M = bw_size, rows = n / M;
     HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
-        if (vec)
-            hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 1);
-        else
-            hipLaunchKernelGGL((quant_fwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, rows, M, TX, rows_per_wg, mode, 1);
+        HGQ_FWD_COLS(1);
     });
     return check_launch("hgq_quantize_fwd_sliced");
 }
