@@ -350,7 +350,8 @@ template <int RM, int OM, int VEC>
 __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ dy, const float *__restrict__ x,
                                                       const void *__restrict__ k, const float *__restrict__ i,
                                                       const float *__restrict__ fb, float *__restrict__ dx, float *di,
-                                                      float *dfb, int64_t rows, int64_t M, int TX, int64_t rows_per_wg, int mode) {
+                                                      float *dfb, int64_t rows, int64_t M, int TX, int64_t rows_per_wg, int mode,
+                                                      float *part) {
     const Mode m(mode);
     const int TY = 256 / TX;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
@@ -412,10 +413,21 @@ __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ 
         __syncthreads();
     }
     if (ty == 0 && active) {
+        if (part) {
+            // slice blockIdx.y of `part`, [df (M) | di (M, only when wanted)], written whole: nothing to clear, no atomics,
+            // and the sum over the slices that follows has a fixed order
+            float *my = part + (int64_t)blockIdx.y * (di ? 2 * M : M) + c * VEC;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            if (di) atomicAdd(&di[c * VEC + e], ssi[tx * VEC + e]);
-            if (dfb) atomicAdd(&dfb[c * VEC + e], ssf[tx * VEC + e]);
+            for (int e = 0; e < VEC; ++e) {
+                my[e] = ssf[tx * VEC + e];
+                if (di) my[M + e] = ssi[tx * VEC + e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if (di) atomicAdd(&di[c * VEC + e], ssi[tx * VEC + e]);
+                if (dfb) atomicAdd(&dfb[c * VEC + e], ssf[tx * VEC + e]);
+            }
         }
     }
 }
@@ -683,6 +695,50 @@ extern "C" int hgq_quantize_fwd_sliced(const float *x, const void *k, const floa
     return check_launch("hgq_quantize_fwd_sliced");
 }
 
+// Geometry of the per-column backward for the sliced form of the bit-width gradients.
+static bool sliced_bwd_geometry(int64_t n, int64_t bw_size, int64_t bw_inner, bool &vec, int &TX, int64_t &gx, int64_t &gy, int64_t &rows_per_wg) {
+    if (n < 1 || bw_size < 2 || bw_inner != 1 || bw_size >= n || n % bw_size != 0 || bw_size * 4 * 256 * QC_U >= (1ll << 31)) return false;
+    vec = bw_size % 4 == 0;
+    const int64_t cg = vec ? bw_size / 4 : bw_size;
+    TX = pow2_floor_le64(cg);
+    gx = (cg + TX - 1) / TX;
+    return cols_grid(n / bw_size, bw_size, (256 / TX) * (QC_U / 2), gx, gy, rows_per_wg);
+}
+
+extern "C" int64_t hgq_quantize_bwd_workspace(int64_t n, int64_t bw_size, int64_t bw_inner) {
+    bool vec;
+    int TX;
+    int64_t gx, gy, rows_per_wg;
+    return sliced_bwd_geometry(n, bw_size, bw_inner, vec, TX, gx, gy, rows_per_wg) ? gy * 2 * bw_size : 0;
+}
+
+extern "C" int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx,
+                                       float *di, float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner,
+                                       int mode, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    bool vec;
+    int TX;
+    int64_t gx, gy, rows_per_wg;
+    if (!sliced_bwd_geometry(n, bw_size, bw_inner, vec, TX, gx, gy, rows_per_wg))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_quantize_bwd_sliced: shape outside the per-column kernels (hgq_quantize_bwd_workspace returns 0 for it)");
+    if (!dy || !x || !k || !i || !fb || !dfb || !workspace) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_sliced: null pointer");
+    const Mode m(mode);
+    if (!m.training) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_sliced: the surrogate gradient is defined for training mode only");
+    if (vec && !(aligned16(x) && aligned16(dy) && (!dx || aligned16(dx)) && aligned16(i) && aligned16(fb) &&
+                 ((uintptr_t)k & (m.k_u8 ? 3u : 15u)) == 0))
+        return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_sliced: operands must be 16-byte aligned when bw_size is a multiple of 4");
+    const int64_t M = bw_size, rows = n / M;
+    HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+        if (vec)
+            hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode, workspace);
+        else
+            hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode, workspace);
+    });
+    int rc = check_launch("hgq_quantize_bwd_sliced");
+    if (rc) return rc;
+    return reduce_parts(workspace, (int)gy, di ? 2 * M : M, dfb, M, di, di ? M : 0, nullptr, 0, s);
+}
+
 extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,
                                 float *dx, float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner,
                                 int mode, void *stream) {
@@ -739,9 +795,9 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
         cols_grid(rows, M, TY * (QC_U / 2), gx, gy, rows_per_wg);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (vec)
-                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode);
+                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode, (float *)nullptr);
             else
-                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode);
+                hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode, (float *)nullptr);
         });
         return check_launch("hgq_quantize_bwd");
     }

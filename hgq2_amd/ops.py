@@ -95,8 +95,17 @@ def quantize_bwd(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: 
     dx = torch.empty_like(x) if need_dx else x.new_empty(0)
     di = torch.empty_like(i) if need_di else i.new_empty(0)
     dfb = torch.empty_like(fb)
-    rc = _lib.load().hgq_quantize_bwd(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), _ptr(di), _ptr(dfb),
-                                      x.numel(), i.numel(), bw_inner, _kmode(mode, k), _stream())
+    lib = _lib.load()
+    n_ws = lib.hgq_quantize_bwd_workspace(x.numel(), i.numel(), bw_inner)
+    if n_ws and all(t.data_ptr() % 16 == 0 for t in (dy, x, k, i, fb, dx)):
+        # bit-width gradients as one slice per row chunk, added in a fixed order: no clearing launch, no atomics
+        ws = torch.empty(n_ws, dtype=torch.float32, device=x.device)
+        rc = lib.hgq_quantize_bwd_sliced(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), _ptr(di), _ptr(dfb), _ptr(ws),
+                                         x.numel(), i.numel(), bw_inner, _kmode(mode, k), _stream())
+        _lib.check(rc, 'hgq_quantize_bwd_sliced')
+        return dx, di, dfb
+    rc = lib.hgq_quantize_bwd(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), _ptr(di), _ptr(dfb),
+                              x.numel(), i.numel(), bw_inner, _kmode(mode, k), _stream())
     _lib.check(rc, 'hgq_quantize_bwd')
     return dx, di, dfb
 

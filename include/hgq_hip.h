@@ -98,6 +98,16 @@ int hgq_quantize_fwd_sliced(const float *x, const void *k, const float *i, const
  *   dx  [n];  di, dfb [bw_size]  (either may be NULL to skip).  With HGQ_MODE_KBI `dfb` is the
  *   gradient w.r.t. b and `di` the total gradient w.r.t. i (direct - via f).
  */
+/*
+ * hgq_quantize_bwd with the bit-width gradients summed in a fixed order: when bit-widths are shared along the leading
+ * axis only (bw_inner == 1, 1 < bw_size < n) every row chunk leaves a slice of partial sums in `workspace`
+ * (hgq_quantize_bwd_workspace floats; 0: the shape is not handled here, use hgq_quantize_bwd) and a second launch adds
+ * the slices in order - no atomics, nothing to clear, the same bits on every run.  dfb is required, di and dx optional.
+ */
+int64_t hgq_quantize_bwd_workspace(int64_t n, int64_t bw_size, int64_t bw_inner);
+int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
+                            float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
+
 int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,
                      float *dx, float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner,
                      int mode, void *stream);

@@ -315,3 +315,25 @@ def test_sparse_ce_and_sgd(dev):
     ops.sgd_update_multi_(wds, gds, [1e-8] * n, [-1.0] * n, [float('inf')] * n, 0.05)
     for wd_, w_, g_ in zip(wds, ws, gs):
         assert torch.equal(wd_.cpu(), torch.clamp(w_ - 0.05 * (g_ + 1e-8), min=-1.0))
+
+
+@pytest.mark.parametrize('rows,M', [(4096, 16), (2048, 4096), (1000, 7)])
+def test_per_column_bit_width_gradients_have_a_fixed_order(dev, rows, M):
+    """Bit-widths shared along the leading axis: the reduced gradients come from per-chunk slices added in a fixed
+    order (hgq_quantize_bwd_sliced), so two runs give the same bits; the value is that of fp64 within fp32 rounding."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(rows + M)
+    x = (torch.randn(rows, M, generator=g) * 3).to(dev)
+    dy = torch.randn(rows, M, generator=g).to(dev)
+    k = torch.ones(M, dtype=torch.uint8).to(dev)
+    i = torch.randint(1, 4, (M,), generator=g).float().to(dev)
+    f = torch.randint(1, 6, (M,), generator=g).float().to(dev)
+    mode = _lib.mode_bits('RND', 'WRAP', training=True)
+    assert _lib.load().hgq_quantize_bwd_workspace(rows * M, M, 1) > 0
+    runs = [ops.quantize_bwd(dy, x, k, i, f, mode, 1, True, False) for _ in range(2)]
+    assert torch.equal(runs[0][2], runs[1][2]) and torch.equal(runs[0][0], runs[1][0])
+    xq = torch.floor(x.double() * 2.0**f.double() + 0.5) / 2.0**f.double()
+    want = (-0.6931471805599453 * (xq - x.double()) * dy.double()).sum(0)
+    err = float((runs[0][2].double() - want).abs().max())
+    assert err <= 1e-5 * float(want.abs().max()) + 1e-6
+    assert torch.equal(runs[0][0], dy)  # straight-through
