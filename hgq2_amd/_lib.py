@@ -70,6 +70,8 @@ SIGNATURES = {
     'hgq_sgd_update_multi': (c_int, [c_void_p, c_int, c_float, c_void_p]),
     'hgq_quantize_bwd_workspace': (c_int64, [c_int64, c_int64, c_int64]),
     'hgq_quantize_bwd_sliced': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    'hgq_quantize_fwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
+    'hgq_quantize_bwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_sum_scalars': (c_int, [c_void_p, c_int, c_void_p, c_void_p]),
     'hgq_mlp_workspace': (c_int64, [c_void_p, c_int, c_int64]),
     'hgq_mlp_train_step': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p]),

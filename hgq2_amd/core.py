@@ -138,6 +138,10 @@ def _auto_name(cls_name: str) -> str:
     return base if n == 0 else f'{base}_{n}'
 
 
+# Top-level training calls run all kernel / bias quantizers of the model in one launch first (quantizer/prefetch.py).
+PREFETCH_WEIGHT_QUANTIZERS = True
+
+
 class Layer(nn.Module):
     """Keras-like layer on top of ``torch.nn.Module``."""
 
@@ -231,6 +235,10 @@ class Layer(nn.Module):
         top = getattr(_ctx, 'depth', 0) == 0
         if top:
             self._clear_losses()
+            if training is True and self.built and PREFETCH_WEIGHT_QUANTIZERS:
+                from .quantizer.prefetch import prefetch_weight_quantizers
+
+                prefetch_weight_quantizers(self)
         else:
             self._losses = []
         _ctx.training = training

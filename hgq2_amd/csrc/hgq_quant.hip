@@ -471,6 +471,41 @@ __global__ __launch_bounds__(256) void quant_bwd_generic(const float *__restrict
 }
 
 // ------------------------------------------------------------------------------------------
+// many small quantizers with per-element bit-widths in one launch (the kernel / bias quantizers of a model: a few
+// thousand elements each, every launch of its own costs more than its work)
+// ------------------------------------------------------------------------------------------
+struct QuantBatch {
+    hgq_quant_item item[HGQ_QUANT_BATCH];
+};
+struct QuantGradBatch {
+    hgq_quant_grad_item item[HGQ_QUANT_BATCH];
+};
+
+// grid.y = quantizer, grid.x strides over its elements; round and overflow modes are read per item
+__global__ __launch_bounds__(256) void quant_fwd_multi_kernel(QuantBatch b) {
+    const hgq_quant_item it = b.item[blockIdx.y];
+    const Mode m(it.mode);
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < it.n; t += (int64_t)gridDim.x * 256) {
+        const KIF p = resolve_kif(load_k(it.k, t, m.k_u8), it.i[t], it.fb[t], m.kbi, m.round_params);
+        it.y[t] = quantize_dyn(it.x[t], p, m.round_mode, m.overflow_mode, m.training);
+    }
+}
+
+__global__ __launch_bounds__(256) void quant_bwd_multi_kernel(QuantGradBatch b) {
+    const hgq_quant_grad_item it = b.item[blockIdx.y];
+    const Mode m(it.mode);
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < it.n; t += (int64_t)gridDim.x * 256) {
+        const KIF p = resolve_kif(load_k(it.k, t, m.k_u8), it.i[t], it.fb[t], m.kbi, m.round_params);
+        float gx, gi, gf;
+        quantize_grad_dyn(it.x[t], it.dy ? it.dy[t] : 0.0f, p, m.round_mode, m.overflow_mode, gx, gi, gf);
+        if (m.kbi) gi -= gf;
+        if (it.dx) it.dx[t] = gx;
+        if (it.di) it.di[t] = gi;
+        if (it.dfb) it.dfb[t] = gf;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // integer-bit tracking
 // ------------------------------------------------------------------------------------------
 // 1024 threads = 64 entries x 16 slice groups: the abs-max / any-negative trackers arrive as
@@ -693,6 +728,55 @@ extern "C" int hgq_quantize_fwd_sliced(const float *x, const void *k, const floa
         HGQ_FWD_COLS(1);
     });
     return check_launch("hgq_quantize_fwd_sliced");
+}
+
+static unsigned multi_grid_x(int64_t max_n) {
+    int64_t gx = (max_n + 1023) / 1024;
+    return (unsigned)(gx < 1 ? 1 : (gx > 256 ? 256 : gx));
+}
+
+extern "C" int hgq_quantize_fwd_multi(const hgq_quant_item *items, int count, void *stream) {
+    if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_multi: bad arguments");
+    for (int base = 0; base < count; base += HGQ_QUANT_BATCH) {
+        QuantBatch b;
+        const int nb = count - base < HGQ_QUANT_BATCH ? count - base : HGQ_QUANT_BATCH;
+        int64_t max_n = 0;
+        for (int t = 0; t < nb; ++t) {
+            b.item[t] = items[base + t];
+            const hgq_quant_item &it = b.item[t];
+            if (it.n < 0 || (it.n > 0 && (!it.x || !it.k || !it.i || !it.fb || !it.y)))
+                return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_multi: bad item %d", base + t);
+            if (it.n > max_n) max_n = it.n;
+        }
+        if (max_n == 0) continue;
+        hipLaunchKernelGGL(quant_fwd_multi_kernel, dim3(multi_grid_x(max_n), (unsigned)nb), dim3(256), 0, (hipStream_t)stream, b);
+        int rc = check_launch("hgq_quantize_fwd_multi");
+        if (rc) return rc;
+    }
+    return HGQ_OK;
+}
+
+extern "C" int hgq_quantize_bwd_multi(const hgq_quant_grad_item *items, int count, void *stream) {
+    if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_multi: bad arguments");
+    for (int base = 0; base < count; base += HGQ_QUANT_BATCH) {
+        QuantGradBatch b;
+        const int nb = count - base < HGQ_QUANT_BATCH ? count - base : HGQ_QUANT_BATCH;
+        int64_t max_n = 0;
+        for (int t = 0; t < nb; ++t) {
+            b.item[t] = items[base + t];
+            const hgq_quant_grad_item &it = b.item[t];
+            if (it.n < 0 || (it.n > 0 && (!it.x || !it.k || !it.i || !it.fb)))
+                return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_multi: bad item %d", base + t);
+            if (!Mode(it.mode).training)
+                return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_multi: item %d: the surrogate gradient is defined for training mode only", base + t);
+            if (it.n > max_n) max_n = it.n;
+        }
+        if (max_n == 0) continue;
+        hipLaunchKernelGGL(quant_bwd_multi_kernel, dim3(multi_grid_x(max_n), (unsigned)nb), dim3(256), 0, (hipStream_t)stream, b);
+        int rc = check_launch("hgq_quantize_bwd_multi");
+        if (rc) return rc;
+    }
+    return HGQ_OK;
 }
 
 // Geometry of the per-column backward for the sliced form of the bit-width gradients.

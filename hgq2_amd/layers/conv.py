@@ -124,6 +124,14 @@ class QConv2D(QLayerBaseSingleInput):
             ebops = ebops + torch.mean(bw_bias) * size
         return ebops
 
+    def _weight_quantizer_inputs(self):
+        """(quantizer, variable) pairs this layer's call quantizes as they are: candidates for the batched launch
+        ahead of the forward pass (quantizer/prefetch.py)."""
+        pairs = [(self.kq, self._kernel)]
+        if self.bias is not None and self.bq is not None:
+            pairs.append((self.bq, self.bias))
+        return pairs
+
     @property
     def qkernel(self):
         return self.kq(self._kernel)

@@ -87,6 +87,9 @@ class QEinsumDenseBatchnorm(QEinsumDense):
     def qbias(self):
         return self.get_fused_qkernel_and_qbias(False, self.moving_mean, self.moving_variance)[1]
 
+    def _weight_quantizer_inputs(self):
+        return []  # kernel and bias are quantized after folding the batch statistics in: they depend on the input
+
     def _trailing_gemm(self):
         """GEMM-shaped equation whose normalised axes are exactly the new output axes."""
         n_out = len(self.full_output_shape)

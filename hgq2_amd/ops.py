@@ -930,6 +930,100 @@ class _Quantize(torch.autograd.Function):
                 dfb if ctx.needs_input_grad[3] else None, None, None, None)
 
 
+class _QuantItem(ctypes.Structure):
+    _fields_ = [('x', ctypes.c_void_p), ('k', ctypes.c_void_p), ('i', ctypes.c_void_p), ('fb', ctypes.c_void_p),
+                ('y', ctypes.c_void_p), ('n', ctypes.c_int64), ('mode', ctypes.c_int)]
+
+
+class _QuantGradItem(ctypes.Structure):
+    _fields_ = [('dy', ctypes.c_void_p), ('x', ctypes.c_void_p), ('k', ctypes.c_void_p), ('i', ctypes.c_void_p),
+                ('fb', ctypes.c_void_p), ('dx', ctypes.c_void_p), ('di', ctypes.c_void_p), ('dfb', ctypes.c_void_p),
+                ('n', ctypes.c_int64), ('mode', ctypes.c_int)]
+
+
+def _check_multi(xs, ks, is_, fbs, modes):
+    n = len(xs)
+    _need(len(ks) == n and len(is_) == n and len(fbs) == n and len(modes) == n, 'per-quantizer lists differ in length')
+    for x, k, i, fb in zip(xs, ks, is_, fbs):
+        _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
+        _need(k.numel() == x.numel() and i.numel() == x.numel() and fb.numel() == x.numel(),
+              'the batched quantizer takes per-element bit-widths (k, i, f of the size of x)')
+
+
+@torch.library.custom_op('hgq::quantize_fwd_multi', mutates_args=())
+def quantize_fwd_multi(xs: Sequence[Tensor], ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor],
+                       modes: Sequence[int]) -> list[Tensor]:
+    _check_multi(xs, ks, is_, fbs, modes)
+    n = len(xs)
+    ys = [torch.empty_like(x) for x in xs]
+    items = (_QuantItem * max(n, 1))()
+    for t in range(n):
+        items[t] = _QuantItem(xs[t].data_ptr(), ks[t].data_ptr(), is_[t].data_ptr(), fbs[t].data_ptr(), ys[t].data_ptr(),
+                              xs[t].numel(), _kmode(modes[t], ks[t]))
+    _lib.check(_lib.load().hgq_quantize_fwd_multi(items, n, _stream()), 'hgq_quantize_fwd_multi')
+    return ys
+
+
+@quantize_fwd_multi.register_fake
+def _(xs, ks, is_, fbs, modes):
+    return [torch.empty_like(x) for x in xs]
+
+
+@torch.library.custom_op('hgq::quantize_bwd_multi', mutates_args=())
+def quantize_bwd_multi(dys: Sequence[Tensor], xs: Sequence[Tensor], ks: Sequence[Tensor], is_: Sequence[Tensor],
+                       fbs: Sequence[Tensor], modes: Sequence[int]) -> list[Tensor]:
+    """``dys[t]`` empty: zero upstream gradient.  Returns ``dx_0 .. dx_{n-1}, di_0 .., dfb_0 ..``."""
+    _check_multi(xs, ks, is_, fbs, modes)
+    n = len(xs)
+    _need(len(dys) == n, 'one upstream gradient per quantizer (an empty tensor for none)')
+    dxs, dis, dfs = [torch.empty_like(x) for x in xs], [torch.empty_like(i) for i in is_], [torch.empty_like(f) for f in fbs]
+    items = (_QuantGradItem * max(n, 1))()
+    for t in range(n):
+        if dys[t].numel():
+            _check_f32('dy', dys[t])
+            _need(dys[t].numel() == xs[t].numel(), 'dy and x differ in size')
+        items[t] = _QuantGradItem(dys[t].data_ptr() if dys[t].numel() else 0, xs[t].data_ptr(), ks[t].data_ptr(), is_[t].data_ptr(),
+                                  fbs[t].data_ptr(), dxs[t].data_ptr(), dis[t].data_ptr(), dfs[t].data_ptr(), xs[t].numel(),
+                                  _kmode(modes[t], ks[t]))
+    _lib.check(_lib.load().hgq_quantize_bwd_multi(items, n, _stream()), 'hgq_quantize_bwd_multi')
+    return dxs + dis + dfs
+
+
+@quantize_bwd_multi.register_fake
+def _(dys, xs, ks, is_, fbs, modes):
+    return [torch.empty_like(x) for x in xs] + [torch.empty_like(i) for i in is_] + [torch.empty_like(f) for f in fbs]
+
+
+class _QuantizeMulti(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, n, modes, *tensors):
+        xs, ks, is_, fbs = tensors[:n], tensors[n:2 * n], tensors[2 * n:3 * n], tensors[3 * n:]
+        ctx.save_for_backward(*tensors)
+        ctx.n, ctx.modes = n, modes
+        ctx.set_materialize_grads(False)
+        return tuple(quantize_fwd_multi(list(xs), list(ks), list(is_), list(fbs), list(modes)))
+
+    @staticmethod
+    def backward(ctx, *gys):
+        n, t = ctx.n, ctx.saved_tensors
+        xs, ks, is_, fbs = t[:n], t[n:2 * n], t[2 * n:3 * n], t[3 * n:]
+        for mode in ctx.modes:
+            if not (mode & _lib.MODE_TRAINING):
+                raise RuntimeError('hgq quantizer: gradients are defined for the training-mode forward only')
+        dys = [x.new_empty(0) if g is None else g.contiguous() for g, x in zip(gys, xs)]
+        out = quantize_bwd_multi(dys, list(xs), list(ks), list(is_), list(fbs), list(ctx.modes))
+        need = ctx.needs_input_grad[2:]
+        grads = list(out[:n]) + [None] * n + list(out[n:])
+        return (None, None) + tuple(g if need[j] else None for j, g in enumerate(grads))
+
+
+def quantize_multi(xs, ks, is_, fbs, modes):
+    """Several quantizers with per-element bit-widths in one launch each way; returns the quantized tensors."""
+    n = len(xs)
+    flat = [t.contiguous() for group in (xs, ks, is_, fbs) for t in group]
+    return _QuantizeMulti.apply(n, tuple(int(m) for m in modes), *flat)
+
+
 def quantize(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int = 1, track: bool = False):
     """Fixed-point quantizer.  Returns ``(y, amax_bits, anyneg)``; the last two are empty unless ``track``."""
     return _Quantize.apply(x.contiguous(), k.contiguous(), i.contiguous(), fb.contiguous(), mode, bw_inner, track)

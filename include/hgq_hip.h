@@ -108,6 +108,34 @@ int64_t hgq_quantize_bwd_workspace(int64_t n, int64_t bw_size, int64_t bw_inner)
 int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
                             float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
 
+/*
+ * Many quantizers with per-element bit-widths (bw_size == n, no trackers) in one launch each way: the kernel and bias
+ * quantizers of a model (src/hgq/layers/core/dense.py:72-79 `self.kq(self._kernel)`, `self.bq(self.bias)` and the same
+ * in the other layers) depend on the variables only, so all of them can run before the first layer and their gradients
+ * after the last.  Per item the arithmetic is that of hgq_quantize_fwd / hgq_quantize_bwd with bw_size == n; each item
+ * carries its own HGQ_MODE(...) bits.  Descriptors are read on the host and travel as launch arguments (safe under HIP
+ * graph capture).  Backward: dy NULL = zero upstream gradient; dx, di, dfb may each be NULL.
+ */
+#define HGQ_QUANT_BATCH 32
+typedef struct {
+    const float *x;
+    const void *k;
+    const float *i, *fb;
+    float *y;
+    int64_t n;
+    int mode;
+} hgq_quant_item;
+typedef struct {
+    const float *dy, *x;
+    const void *k;
+    const float *i, *fb;
+    float *dx, *di, *dfb;
+    int64_t n;
+    int mode;
+} hgq_quant_grad_item;
+int hgq_quantize_fwd_multi(const hgq_quant_item *items, int count, void *stream);
+int hgq_quantize_bwd_multi(const hgq_quant_grad_item *items, int count, void *stream);
+
 int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,
                      float *dx, float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner,
                      int mode, void *stream);

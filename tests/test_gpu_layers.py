@@ -302,3 +302,68 @@ def test_scalar_loss_terms_summed_in_one_launch():
             assert term.grad.shape == term.shape and float(term.grad.reshape(())) == 3.0
         else:
             assert term.grad is None
+
+
+@pytest.mark.gpu
+def test_weight_quantizers_in_one_launch_change_nothing():
+    """With the kernel / bias quantizers of a model batched ahead of the forward pass (quantizer/prefetch.py) a
+    training step gives the same loss and the same gradients, bit for bit, as with one launch per quantizer."""
+    import hgq2_amd.core as core
+    from hgq2_amd import ops, train
+    from hgq2_amd.quantizer.prefetch import prefetch_weight_quantizers
+    from hgq2_amd.utils import models
+
+    dev = torch.device('cuda:0')
+    results = []
+    for flag in (True, False):
+        torch.manual_seed(3)
+        model = models.mha_block(device=dev)
+        x = torch.randn(8, 64, 64, generator=torch.Generator().manual_seed(1)).to(dev)
+        with torch.no_grad():
+            model(x, training=True)  # build
+        core.PREFETCH_WEIGHT_QUANTIZERS = flag
+        try:
+            y = model(x, training=True)
+            loss = train.model_loss(model, (y * y).mean())
+            loss.backward()
+        finally:
+            core.PREFETCH_WEIGHT_QUANTIZERS = True
+        results.append((loss.detach().clone(), {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}))
+        if flag:
+            assert prefetch_weight_quantizers(model) >= 4  # at least the kernels of the q, k, v and output projections
+    (l1, g1), (l0, g0) = results
+    assert torch.equal(l1, l0) and g1.keys() == g0.keys()
+    for n in g1:
+        assert torch.equal(g1[n], g0[n]), n
+
+
+@pytest.mark.gpu
+def test_batched_quantizer_matches_single_launches():
+    from hgq2_amd import _lib, ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(9)
+    cases = [(4096, 'RND', 'SAT_SYM', True), (64, 'TRN', 'SAT', False), (33, 'RND_CONV', 'SAT', True), (700, 'RND', 'WRAP', False)]
+    xs, ks, is_, fs, modes, singles = [], [], [], [], [], []
+    for n, rm, om, kbi in cases:
+        x = (torch.randn(n, generator=g) * 3).to(dev).requires_grad_(True)
+        k = torch.randint(0, 2, (n,), generator=g).to(torch.uint8).to(dev)
+        i = torch.randint(-1, 3, (n,), generator=g).float().to(dev).requires_grad_(True)
+        f = (torch.randint(1, 6, (n,), generator=g).float() + (i.detach().cpu() if kbi else 0)).to(dev).requires_grad_(True)
+        mode = _lib.mode_bits(rm, om, training=True, kbi=kbi, round_params=True)
+        xs.append(x), ks.append(k), is_.append(i), fs.append(f), modes.append(mode)
+    ups = [torch.randn(x.shape, generator=g).to(dev) for x in xs]
+    ys = ops.quantize_multi(xs, ks, is_, fs, modes)
+    sum((y * u).sum() for y, u in zip(ys[:-1], ups)).backward()  # the last output stays unused: zero gradients
+    got = [(y.detach(), x.grad, i.grad, f.grad) for y, x, i, f in zip(ys, xs, is_, fs)]
+    for t, (x, k, i, f, mode, u) in enumerate(zip(xs, ks, is_, fs, modes, ups)):
+        x1, i1, f1 = (v.detach().clone().requires_grad_(True) for v in (x, i, f))
+        y1, _, _ = ops.quantize(x1, k, i1, f1, mode)
+        assert torch.equal(got[t][0], y1.detach())
+        if t < len(xs) - 1:
+            (y1 * u).sum().backward()
+            for a, b in zip(got[t][1:], (x1.grad, i1.grad, f1.grad)):
+                assert torch.equal(a, b)
+        else:
+            for a in got[t][1:]:
+                assert a is None or not a.any()
