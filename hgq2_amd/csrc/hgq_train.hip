@@ -472,6 +472,7 @@ extern "C" int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float 
     return HGQ_OK;
 }
 
+namespace hgq {
 struct SumBatch {
     const float *term[HGQ_SUM_BATCH];
 };
@@ -484,6 +485,7 @@ __global__ void sum_scalars_kernel(SumBatch b, int count, float *out) {
         out[0] = v;
     }
 }
+}  // namespace hgq
 
 extern "C" int hgq_sum_scalars(const float *const *terms, int count, float *out, void *stream) {
     if (!terms || !out || count < 1 || count > HGQ_SUM_BATCH) return fail(HGQ_ERR_ARG, "hgq_sum_scalars: 1 <= count <= %d terms expected", HGQ_SUM_BATCH);
