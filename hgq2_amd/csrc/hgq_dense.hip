@@ -592,7 +592,7 @@ __global__ __launch_bounds__(256) void moments_scale_kernel(float *mean, float *
 // STATS: the gradient at the pre-activation is not read but computed in the tile from the upstream
 // gradients of the column statistics: dz[r, c] = (gm[c] + 2 z[r, c] gs[c]) / rows with z = x W
 // recomputed on the matrix cores (dy = gm, y = gs, both [N]); no activation, no bias, no quantizer.
-template <int RM, bool QUANT, bool STATS = false>
+template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true>
 __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
@@ -630,7 +630,9 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         }
     }
     FastMap mx, mz;
-    mx.init(K), mz.init(N);
+    // !ZVEC - N not a multiple of 4, or unaligned gradient rows: the gradient tile is staged in groups of four columns
+    // of the width rounded up, each element with a load of its own (columns past N read as zero)
+    mx.init(K), mz.init((N + 3) & ~3);
     int fi[FAST_NJ][4], tix[FAST_NJ];
     float gf[FAST_NJ][4];
     fast_frac_bits<QUANT>(f_in, P, K, mx, m.round_params, fi, tix);
@@ -668,8 +670,17 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         for (int j = 0; j < FAST_NJ; ++j) {
             rx[j] = buf_ld4(sx, xoff[j]);
             if (!STATS) {
-                rg[j] = buf_ld4(sg, zoff[j]);
-                ry[j] = buf_ld4(sy, zoff[j]);
+                if (ZVEC) {
+                    rg[j] = buf_ld4(sg, zoff[j]);
+                    ry[j] = buf_ld4(sy, zoff[j]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t off = (mz.on[j] && mz.col[j] + e < N) ? zoff[j] + 4u * e : BUF_OOB;
+                        rg[j][e] = buf_ld1(sg, off);
+                        ry[j][e] = buf_ld1(sy, off);
+                    }
+                }
             } else {
                 rg[j] = buf_ld4(sg, xoff[j]);  // the other gradient of x, laid out like x (zeros without one)
             }
@@ -1060,14 +1071,21 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
         if (df_in && (rc = fill_f32(df_in, 0.f, PK, s))) return rc;
         return HGQ_OK;
     }
-    const bool fast = K % 4 == 0 && N % 4 == 0 && aligned16(x) && aligned16(dy) && aligned16(dx) && (act != HGQ_ACT_RELU || aligned16(y)) &&
-                      (!quant || (bw_rows <= 64 && 64 % bw_rows == 0));
+    const bool fast = K % 4 == 0 && aligned16(x) && aligned16(dx) && (!quant || (bw_rows <= 64 && 64 % bw_rows == 0));
     if (fast) {
         const int parts = row_parts(rows, BWD_BM);
         const int P = quant ? (int)bw_rows : 1;
         const dim3 fgrid((unsigned)parts);
-#define HGQ_BWD_FAST(RMV, QV) \
-    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr)
+        const bool zvec = N % 4 == 0 && aligned16(dy) && (act != HGQ_ACT_RELU || aligned16(y));
+#define HGQ_BWD_FAST(RMV, QV)                                                                                                          \
+    do {                                                                                                                               \
+        if (zvec)                                                                                                                      \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
+                               dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
+        else                                                                                                                           \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, false>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
+                               dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
+    } while (0)
         if (!quant) HGQ_BWD_FAST(HGQ_TRN, false);
         else if (m.round_mode == HGQ_TRN) HGQ_BWD_FAST(HGQ_TRN, true);
         else if (m.round_mode == HGQ_RND) HGQ_BWD_FAST(HGQ_RND, true);
