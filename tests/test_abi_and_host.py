@@ -214,3 +214,20 @@ def test_beta_controllers_and_ebops_logging():
     err = log10(4000 / 2000)
     assert history[3]['beta'] == pytest.approx(10 ** (log10(1e-6) + 0.1 * err), rel=1e-6) and history[4]['beta'] > history[3]['beta']
     assert all(h['ebops'] == 4000 for h in history)
+
+
+def test_reciprocal_index_arithmetic_is_exact_on_the_ranges_the_kernels_use():
+    """The staging maps of the fused dense kernels divide by a 16-bit reciprocal (ids below 1024, divisors up to 16);
+    the staging loops of the small-channel convolution and the EBOPs kernels by a float reciprocal (values below
+    2**21).  Both claim to equal integer division on those ranges."""
+    import numpy as np
+
+    for w4 in range(1, 17):
+        rcp = (65536 + w4 - 1) // w4
+        ids = np.arange(1024, dtype=np.uint64)
+        assert np.array_equal((ids * rcp) >> 16, ids // w4), w4
+    c = np.arange(1 << 21, dtype=np.uint32)
+    for d in (1, 2, 3, 5, 7, 12, 31, 32, 33, 68, 272, 340, 1088, 3872, 30719):
+        inv = np.float32(1.0) / np.float32(d)
+        q = ((c.astype(np.float32) + np.float32(0.5)) * inv).astype(np.uint32)
+        assert np.array_equal(q, c // d), d
