@@ -173,7 +173,7 @@ __device__ __forceinline__ float finish(double raw, float f1, float f2, const fl
     const float e = __fmul_rn(__fmul_rn((float)raw, f1), f2);
     if (threadIdx.x == 0) {
         if (ebops_u32) ebops_u32[0] = (uint32_t)(int64_t)e;
-        loss_term[0] = __fmul_rn(e, beta[0]);
+        if (loss_term) loss_term[0] = __fmul_rn(e, beta[0]);
     }
     return __fmul_rn(__fmul_rn(beta[0], f2), f1);
 }
@@ -262,6 +262,8 @@ __global__ __launch_bounds__(EB_NT) void softmax_ebops_kernel(hgq_bits_desc d_su
 
 // QMultiHeadAttention: sum_{t,s,n,h} bq[t,n,h] bk[s,n,h] + sum_{n,t,s,h} ba[n,t,s] bv[s,n,h], through the marginal sums
 //   Q[n,h] = sum_t bq, K[n,h] = sum_s bk, A[n,s] = sum_t ba, V[s,n] = sum_h bv.
+// Four workgroups: each forms the marginal sums and the total (the same bits in each), then writes the gradients of one
+// of the four operands; the first also writes the value.
 template <bool GENERIC>
 __global__ __launch_bounds__(EB_NT) void mha_ebops_kernel(hgq_bits_desc d_q, hgq_bits_desc d_k, hgq_bits_desc d_v, hgq_bits_desc d_a, uint32_t T,
                                                           uint32_t S, uint32_t N, uint32_t H, uint32_t Hv, float f1, float f2,
@@ -298,18 +300,22 @@ __global__ __launch_bounds__(EB_NT) void mha_ebops_kernel(hgq_bits_desc d_q, hgq
         const uint32_t n = e / S, s = e - n * S;
         part += (double)Am[e] * (double)Vm[s * N + n];
     }
-    const float gs = finish(block_sum(part, red), f1, f2, beta, ebops_u32, loss_term);
+    const bool lead = blockIdx.x == 0;
+    const float gs = finish(block_sum(part, red), f1, f2, beta, lead ? ebops_u32 : nullptr, lead ? loss_term : nullptr);
     const FastDiv by_nh(NH), by_nhv(N * Hv), by_hv(Hv), by_n(N), by_ts(T * S), by_s(S);
-    entry_grads(bq, T * NH, gs, [&](uint32_t c) { return Km[by_nh.mod(c)]; }, red);
-    entry_grads(bk, S * NH, gs, [&](uint32_t c) { return Qm[by_nh.mod(c)]; }, red);
-    entry_grads(bv, S * N * Hv, gs, [&](uint32_t c) {
-        const uint32_t s = by_nhv.div(c), n = by_n.mod(by_hv.div(c));
-        return Am[n * S + s];
-    }, red);
-    entry_grads(ba, N * T * S, gs, [&](uint32_t c) {
-        const uint32_t n = by_ts.div(c), s = by_s.mod(c);
-        return Vm[s * N + n];
-    }, red);
+    const uint32_t which = blockIdx.x, all = gridDim.x == 1;
+    if (all || which == 0) entry_grads(bq, T * NH, gs, [&](uint32_t c) { return Km[by_nh.mod(c)]; }, red);
+    if (all || which == 1) entry_grads(bk, S * NH, gs, [&](uint32_t c) { return Qm[by_nh.mod(c)]; }, red);
+    if (all || which == 2)
+        entry_grads(bv, S * N * Hv, gs, [&](uint32_t c) {
+            const uint32_t s = by_nhv.div(c), n = by_n.mod(by_hv.div(c));
+            return Am[n * S + s];
+        }, red);
+    if (all || which == 3)
+        entry_grads(ba, N * T * S, gs, [&](uint32_t c) {
+            const uint32_t n = by_ts.div(c), s = by_s.mod(c);
+            return Vm[s * N + n];
+        }, red);
 }
 
 static int pool_bytes(int64_t entries, const char *who, size_t &bytes) {
@@ -404,7 +410,7 @@ extern "C" int hgq_mha_ebops(const hgq_bits_desc *bits_q, const hgq_bits_desc *b
         return rc;
     const bool generic = !(simple_layout(bits_q, (int64_t)T * N * H) && simple_layout(bits_k, (int64_t)S * N * H) &&
                            simple_layout(bits_v, (int64_t)S * N * Hv) && simple_layout(bits_attn, (int64_t)N * T * S));
-    hipLaunchKernelGGL(generic ? mha_ebops_kernel<true> : mha_ebops_kernel<false>, dim3(1), dim3(EB_NT), lds, (hipStream_t)stream, *bits_q, *bits_k, *bits_v, *bits_attn, (uint32_t)T, (uint32_t)S,
+    hipLaunchKernelGGL(generic ? mha_ebops_kernel<true> : mha_ebops_kernel<false>, dim3(4), dim3(EB_NT), lds, (hipStream_t)stream, *bits_q, *bits_k, *bits_v, *bits_attn, (uint32_t)T, (uint32_t)S,
                        (uint32_t)N, (uint32_t)H, (uint32_t)Hv, parallel_factor, ebops_factor, beta, ebops_u32, loss_term);
     return check_launch(who);
 }
