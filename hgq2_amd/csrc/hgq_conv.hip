@@ -958,6 +958,8 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
     __shared__ float red[1024];
     __shared__ unsigned char vy[CE_MAXV], vx[CE_MAXV];  // vy[y * kh + ky]: row y is visited by kernel row ky
     const int t = threadIdx.x, taps = g.kh * g.kw, TC = taps * g.C, WC = g.W * g.C;
+    // flat sweeps decode their index with float reciprocals (every swept range is below 2**21: checked by the launcher)
+    const FastDiv by_wc((uint32_t)WC), by_f((uint32_t)F), by_c((uint32_t)g.C), by_kw((uint32_t)g.kw);
     for (int e = t; e < TC; e += 1024) Ws[e] = 0;
     for (int e = t; e < g.H * g.kh; e += 1024) {
         const int y = e / g.kh, ky = e - y * g.kh, ty = y + g.py - ky * g.dly;
@@ -969,7 +971,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
     }
     // R[ky][x][c]: adjacent threads take adjacent (x, c), so every row read is coalesced
     for (int e = t; e < g.kh * WC; e += 1024) {
-        const int ky = e / WC, xc = e - ky * WC;
+        const int ky = (int)by_wc.div((uint32_t)e), xc = e - ky * WC;
         float r = 0.f;
         int oy = 0;
         for (; oy + 4 <= g.OH; oy += 4) {
@@ -999,11 +1001,11 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int e = e0 + u * 1024 + t;
-            if (e < n_w) atomicAdd(&Ws[e / F], (int)v[u]);
+            if (e < n_w) atomicAdd(&Ws[by_f.div((uint32_t)e)], (int)v[u]);
         }
     }
     for (int e = t; e < TC; e += 1024) {
-        const int tap = e / g.C, c = e - tap * g.C, ky = tap / g.kw, kx = tap - ky * g.kw;
+        const int tap = (int)by_c.div((uint32_t)e), c = e - tap * g.C, ky = (int)by_kw.div((uint32_t)tap), kx = tap - ky * g.kw;
         float sacc = 0.f;
         for (int ox = 0; ox < g.OW; ++ox) {
             const int ix = ox * g.sx - g.px + kx * g.dlx;
@@ -1022,10 +1024,10 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
     }
     if (t == 0) total[0] = red[0];
     if (g_ker)
-        for (int e = t; e < n_w; e += 1024) g_ker[e] = S[e / F];
+        for (int e = t; e < n_w; e += 1024) g_ker[e] = S[by_f.div((uint32_t)e)];
     if (g_in) {
         for (int e = t; e < g.H * WC; e += 1024) {
-            const int y = e / WC, xc = e - y * WC, x = xc / g.C, c = xc - x * g.C;
+            const int y = (int)by_wc.div((uint32_t)e), xc = e - y * WC, x = (int)by_c.div((uint32_t)xc), c = xc - x * g.C;
             float a = 0.f;
             for (int ky = 0; ky < g.kh; ++ky) {
                 if (!vy[y * g.kh + ky]) continue;
@@ -1274,9 +1276,9 @@ extern "C" int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, con
         (int64_t)g->W * g->kw > CE_MAXV)
         return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: needs kh * kw * C <= %d, kh * W * C <= %d, H * kh and W * kw <= %d", CE_MAX,
                     CE_MAXR, CE_MAXV);
-    if ((int64_t)g->kh * g->kw * g->C * g->OH * g->OW >= (1ll << 31) || (int64_t)g->kh * g->kw * g->C * F >= (1ll << 31) ||
-        (int64_t)g->H * g->W * g->C >= (1ll << 31))
-        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: geometry too large for 32-bit sweeps");
+    if ((int64_t)g->kh * g->kw * g->C * g->OH * g->OW >= (1ll << 31) || (int64_t)g->kh * g->kw * g->C * F >= (1ll << 21) ||
+        (int64_t)g->H * g->W * g->C >= (1ll << 21))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: needs kh * kw * C * F and H * W * C below 2**21 (flat sweeps of one workgroup)");
     hipLaunchKernelGGL(conv_ebops_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, bits_in, bits_ker, *g, F, total, g_bits_in, g_bits_ker);
     return check_launch("hgq_conv2d_ebops");
 }

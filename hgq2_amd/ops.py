@@ -691,8 +691,9 @@ def _(dy, x, geom, is_max):
 def conv2d_ebops_supported(in_shape, kernel_shape) -> bool:
     """Whether hgq_conv2d_ebops covers bit-width tensors [1, H, W, C] x [kh, kw, C, F] (its LDS tables bound the sizes)."""
     _, H, W, C = in_shape
-    kh, kw = kernel_shape[0], kernel_shape[1]
-    return kh * kw * C <= 4096 and kh * W * C <= 8192 and H * kh <= 2048 and W * kw <= 2048
+    kh, kw, F = kernel_shape[0], kernel_shape[1], kernel_shape[3]
+    return (kh * kw * C <= 4096 and kh * W * C <= 8192 and H * kh <= 2048 and W * kw <= 2048 and kh * kw * C * F < 2**21
+            and H * W * C < 2**21)
 
 
 @torch.library.custom_op('hgq::conv2d_ebops', mutates_args=())

@@ -582,7 +582,8 @@ int hgq_pool2d_bwd(const float *dy, const float *x, float *dx, const int *geom, 
  * input pixels, so the sum factorises per (tap, channel).
  *   bits_in [H, W, C];  bits_ker [kh, kw, C, F];  total [1];  g_bits_in [H, W, C], g_bits_ker
  *   [kh, kw, C, F] = d total / d bits (either may be NULL).  g->B is ignored.  Needs kh * kw * C <= 4096,
- *   kh * W * C <= 8192, H * kh <= 2048 and W * kw <= 2048 (HGQ_ERR_UNSUPPORTED otherwise).
+ *   kh * W * C <= 8192, H * kh <= 2048, W * kw <= 2048, kh * kw * C * F < 2**21 and H * W * C < 2**21
+ *   (HGQ_ERR_UNSUPPORTED otherwise).
  */
 int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, const hgq_conv_geom *g, int F, float *total,
                      float *g_bits_in, float *g_bits_ker, void *stream);
