@@ -300,7 +300,10 @@ __global__ __launch_bounds__(256) void quant_fwd_cols(const float *__restrict__ 
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 yv[e] = quantize<RM, OM>(cur[u][e], p[e], TRAIN);
-                const float tv = track_input ? cur[u][e] : yv[e];
+                float tv = track_input ? cur[u][e] : yv[e];
+                // rows past the end read as zero; a saturating quantizer whose range excludes zero maps that to a bound,
+                // which must not reach the trackers (WRAP keeps zero at zero)
+                if (OM != HGQ_WRAP) tv = cur_off[u] != BUF_OOB ? tv : 0.0f;
                 const uint32_t ab = abs_bits(tv);
                 lmax[e] = ab > lmax[e] ? ab : lmax[e];
                 lmin[e] = fminf(lmin[e], tv);

@@ -337,3 +337,25 @@ def test_per_column_bit_width_gradients_have_a_fixed_order(dev, rows, M):
     err = float((runs[0][2].double() - want).abs().max())
     assert err <= 1e-5 * float(want.abs().max()) + 1e-6
     assert torch.equal(runs[0][0], dy)  # straight-through
+
+
+@pytest.mark.parametrize('shape', [(5, 64), (2, 1024), (2, 63), (300, 7)])
+def test_trackers_ignore_the_padding_of_a_row_chunk(dev, shape):
+    """A saturating quantizer whose range excludes zero (2**i < 2**-f) maps the zeros that pad a workgroup's row
+    chunk to its upper bound; those must not show up in the abs-max / any-negative trackers."""
+    _lib, ops = _ops()
+    rows, M = shape
+    g = torch.Generator().manual_seed(rows)
+    x = torch.rand(shape, generator=g) * 0.01  # everything saturates at the (negative) upper bound or at zero
+    k = torch.zeros(M)
+    k[::2] = 1.0
+    i = torch.full((M,), -2.0)
+    f = torch.zeros(M)
+    for om in ('SAT', 'SAT_SYM'):
+        want = ofp.get_fixed_quantizer('RND', om)(x, *(torch.broadcast_to(t, shape) for t in (k, i, f)), True, None)
+        mode = _lib.mode_bits('RND', om, training=True)
+        y, amax, neg = ops.quantize(x.to(dev), k.to(dev), i.to(dev), f.to(dev), mode, bw_inner=1, track=True)
+        assert torch.equal(y.cpu(), want)
+        amax, neg = amax.view(-1, M).amax(0), neg.view(-1, M).amax(0)
+        assert torch.equal(amax.view(torch.float32).cpu(), want.abs().amax(0))
+        assert torch.equal(neg.cpu(), (want < 0).int().amax(0))
