@@ -359,3 +359,65 @@ def test_trackers_ignore_the_padding_of_a_row_chunk(dev, shape):
         amax, neg = amax.view(-1, M).amax(0), neg.view(-1, M).amax(0)
         assert torch.equal(amax.view(torch.float32).cpu(), want.abs().amax(0))
         assert torch.equal(neg.cpu(), (want < 0).int().amax(0))
+
+
+def _dense_sweep_cases(n, seed=0):
+    import random
+
+    rnd = random.Random(seed)
+    cases = []
+    for _ in range(n):
+        K = rnd.choice([4, 8, 12, 16, 20, 32, 36, 48, 64])
+        N = rnd.choice([1, 3, 4, 5, 8, 10, 16, 24, 31, 32, 33, 40, 64])
+        P = rnd.choice([0, 1, 2, 4, 8, 16, 32, 64])
+        rows = rnd.choice([1, 7, 63, 64, 65, 200, 640, 1000]) * (P or 1)
+        cases.append((rows, K, N, P, rnd.choice([0, 1]), rnd.choice([True, False]), rnd.choice(ROUND)))
+    return cases
+
+
+@pytest.mark.parametrize('rows,K,N,P,act,has_bias,round_mode', _dense_sweep_cases(40))
+def test_qdense_sweep_against_fp64(dev, rows, K, N, P, act, has_bias, round_mode):
+    """ops.qdense over widths that are and are not multiples of 4 / 32, table heights 0 (no input quantizer) to 64, ragged
+    last tiles: output, abs-max slices, dx, dW, db and the fractional-bit gradient against an fp64 statement."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(rows * 131 + K * 7 + N)
+    x = torch.randn(rows, K, generator=g) * 2
+    w = torch.randn(K, N, generator=g) * 0.4
+    b = torch.randn(N, generator=g) if has_bias else None
+    up = torch.randn(rows, N, generator=g)
+    if P:
+        f = torch.randint(1, 6, (P, K), generator=g).float()
+        fr = f.repeat(rows // P, 1)
+        t = x * 2.0**fr
+        xq = (torch.floor(t + 0.5) if round_mode == 'RND' else torch.floor(t) if round_mode == 'TRN' else torch.round(t)) / 2.0**fr
+    else:
+        xq = x
+    xr, wr = xq.double().requires_grad_(True), w.double().requires_grad_(True)
+    br = b.double().requires_grad_(True) if has_bias else None
+    z = xr @ wr + (br if has_bias else 0)
+    if act:  # no upstream gradient where fp32 and fp64 may disagree on the side of the kink
+        up = up * (z.detach().abs() > 1e-5 * float(z.detach().abs().max())).float()
+    y_r = torch.relu(z) if act else z
+    (y_r * up.double()).sum().backward()
+    xd, wd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    bd = b.to(dev).requires_grad_(True) if has_bias else None
+    if P:
+        fd = f.to(dev).requires_grad_(True)
+        mode = _lib.mode_bits(round_mode, 'WRAP', training=True, round_params=True)
+        kk, ii = torch.ones(P * K, dtype=torch.uint8, device=dev), torch.full((P * K,), 3.0, device=dev)
+        y, amax = ops.qdense(xd, kk, ii, fd.view(-1), wd, bd, act, mode, P, True)
+        am = amax.view(-1, P * K).amax(0).view(torch.float32).cpu().view(P, K)
+        assert torch.equal(am, xq.abs().view(rows // P, P, K).amax(0))
+    else:
+        y, _ = ops.qdense(xd, None, None, None, wd, bd, act, 0, 0, False)
+    (y * up.to(dev)).sum().backward()
+    checks = [('y', y.detach(), y_r.detach()), ('dx', xd.grad, xr.grad), ('dw', wd.grad, wr.grad)]
+    if has_bias:
+        checks.append(('db', bd.grad, br.grad))
+    if P:
+        df_r = (-np.log(2) * (xq.double() - x.double()) * xr.grad).view(rows // P, P, K).sum(0)
+        checks.append(('df', fd.grad.view(P, K), df_r))
+    for name, got, want in checks:
+        want = want.float()
+        err = float((got.cpu() - want).abs().max())
+        assert err <= 3e-5 * (float(want.abs().max()) + 1e-6), f'{name}: {err:.3e}'
