@@ -358,8 +358,8 @@ __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ 
     const Mode m(mode);
     const int TY = 256 / TX;
     const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
-    const int64_t cg = M / VEC;
-    const int64_t c = (int64_t)blockIdx.x * TX + tx;
+    const int cg = (int)(M / VEC);
+    const int c = (int)blockIdx.x * TX + tx;
     const bool active = c < cg;
     KIF p[VEC];
     float si[VEC], sf[VEC];
@@ -374,22 +374,26 @@ __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ 
         for (int e = 0; e < VEC; ++e) p[e] = resolve_kif(kv[e], iv[e], fv[e], m.kbi, m.round_params);
     }
     const int64_t row0 = (int64_t)blockIdx.y * rows_per_wg;
-    const int64_t n_rows = min(rows - row0, rows_per_wg);
-    const __amdgpu_buffer_rsrc_t rs_g = buf_rsrc(dy + row0 * M, n_rows * M * 4), rs_x = buf_rsrc(x + row0 * M, n_rows * M * 4);
-    float *dxb = dx ? dx + row0 * M : nullptr;
+    const int n_rows = (int)min(rows - row0, rows_per_wg);
+    // a chunk is below 2 GiB: 32-bit index arithmetic, one byte offset for a row's two loads and its store (rows past
+    // the end are dropped by the descriptors' range check)
+    const int64_t chunk_bytes = (int64_t)n_rows * M * 4;
+    const __amdgpu_buffer_rsrc_t rs_g = buf_rsrc(dy + row0 * M, chunk_bytes), rs_x = buf_rsrc(x + row0 * M, chunk_bytes);
+    const __amdgpu_buffer_rsrc_t rs_dx = buf_rsrc(dx ? dx + row0 * M : const_cast<float *>(x), dx ? chunk_bytes : 0);
+    const uint32_t row_bytes = (uint32_t)cg * VEC * 4u;
     constexpr int U = QC_U / 2;  // two operands per row
-    for (int64_t rb = 0; rb < n_rows; rb += (int64_t)TY * U) {
+    for (int rb = 0; rb < n_rows; rb += TY * U) {
         float gv[U][VEC], xv[U][VEC];
+        uint32_t off[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int64_t r = rb + ty + (int64_t)TY * u;
-            const uint32_t off = (active && r < n_rows) ? (uint32_t)((r * cg + c) * VEC) * 4u : BUF_OOB;
-            qc_load<VEC>(rs_g, off, gv[u]);
-            qc_load<VEC>(rs_x, off, xv[u]);
+            const int r = rb + ty + TY * u;
+            off[u] = (active && r < n_rows) ? (uint32_t)r * row_bytes + (uint32_t)c * (VEC * 4u) : BUF_OOB;
+            qc_load<VEC>(rs_g, off[u], gv[u]);
+            qc_load<VEC>(rs_x, off[u], xv[u]);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int64_t r = rb + ty + (int64_t)TY * u;
             float dxv[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
@@ -398,7 +402,7 @@ __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ 
                 if (m.kbi) gi -= gf;
                 si[e] += gi, sf[e] += gf;
             }
-            if (dxb && active && r < n_rows) VecIO<VEC>::store(dxb, r * cg + c, dxv);
+            if (dx) qc_store<VEC>(rs_dx, off[u], dxv);  // nothing is issued when the data gradient is not wanted
         }
     }
     __shared__ float ssi[256 * VEC], ssf[256 * VEC];
