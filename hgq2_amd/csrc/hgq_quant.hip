@@ -214,6 +214,7 @@ __global__ __launch_bounds__(Q1D_BS) void quant_bwd_1d(const float *__restrict__
 // every reduction below), and a workgroup walks a contiguous chunk of rows so that a column sees
 // few workgroups - and few atomics - at the end.
 #define QC_U 8
+#define QC_BWD_U 8
 template <int VEC>
 __device__ __forceinline__ void qc_load(const __amdgpu_buffer_rsrc_t rs, uint32_t off, float *o) {
     if (VEC == 4) {
@@ -381,7 +382,7 @@ __global__ __launch_bounds__(256) void quant_bwd_cols(const float *__restrict__ 
     const __amdgpu_buffer_rsrc_t rs_g = buf_rsrc(dy + row0 * M, chunk_bytes), rs_x = buf_rsrc(x + row0 * M, chunk_bytes);
     const __amdgpu_buffer_rsrc_t rs_dx = buf_rsrc(dx ? dx + row0 * M : const_cast<float *>(x), dx ? chunk_bytes : 0);
     const uint32_t row_bytes = (uint32_t)cg * VEC * 4u;
-    constexpr int U = QC_U / 2;  // two operands per row
+    constexpr int U = QC_BWD_U;  // rows in flight per thread (two operands each)
     for (int rb = 0; rb < n_rows; rb += TY * U) {
         float gv[U][VEC], xv[U][VEC];
         uint32_t off[U];
@@ -793,7 +794,7 @@ static bool sliced_bwd_geometry(int64_t n, int64_t bw_size, int64_t bw_inner, bo
     const int64_t cg = vec ? bw_size / 4 : bw_size;
     TX = pow2_floor_le64(cg);
     gx = (cg + TX - 1) / TX;
-    return cols_grid(n / bw_size, bw_size, (256 / TX) * (QC_U / 2), gx, gy, rows_per_wg);
+    return cols_grid(n / bw_size, bw_size, (256 / TX) * QC_BWD_U, gx, gy, rows_per_wg);
 }
 
 extern "C" int64_t hgq_quantize_bwd_workspace(int64_t n, int64_t bw_size, int64_t bw_inner) {
@@ -883,7 +884,7 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
         const int TX = pow2_floor_le64(cg), TY = 256 / TX;
         const int64_t gx = (cg + TX - 1) / TX;
         int64_t gy, rows_per_wg;
-        cols_grid(rows, M, TY * (QC_U / 2), gx, gy, rows_per_wg);
+        cols_grid(rows, M, TY * QC_BWD_U, gx, gy, rows_per_wg);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (vec)
                 hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode, (float *)nullptr);
