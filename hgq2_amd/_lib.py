@@ -72,6 +72,8 @@ SIGNATURES = {
     'hgq_quantize_bwd_sliced': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_fwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_quantize_bwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
+    'hgq_mean_mid_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    'hgq_mean_mid_bwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     'hgq_sum_scalars': (c_int, [c_void_p, c_int, c_void_p, c_void_p]),
     'hgq_mlp_workspace': (c_int64, [c_void_p, c_int, c_int64]),
     'hgq_mlp_train_step': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p]),

@@ -199,9 +199,116 @@ static int check_pool(const int *d, PoolGeom &g, const char *who) {
     return HGQ_OK;
 }
 
+// ------------------------------------------------------------------------------------------
+// mean over the middle axis of [B, P, N] (global average pooling of a channels-last tensor; the mean over the
+// particles of the per-particle configuration)
+// ------------------------------------------------------------------------------------------
+// One workgroup per batch element: thread (c, ty) owns VEC columns and walks rows ty, ty + TY, ... with eight loads
+// in flight; the TY partial sums of a column group are added in row-group order through LDS.
+template <int VEC>
+__global__ __launch_bounds__(256) void mean_mid_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, int P, int N, int TX,
+                                                           float inv) {
+    __shared__ float red[256 * VEC];
+    const int cg = N / VEC, TY = 256 / TX, c0 = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t b = blockIdx.x;
+    const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + b * P * N, (int64_t)P * N * 4);
+    for (int cb = 0; cb < cg; cb += TX) {
+        const int c = cb + c0;
+        const bool on = c < cg;
+        float s[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) s[e] = 0.f;
+        for (int p0 = ty; p0 < P; p0 += 8 * TY) {
+            float v[8][VEC];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int p = p0 + u * TY;
+                const uint32_t off = (on && p < P) ? (uint32_t)(p * N + c * VEC) * 4u : BUF_OOB;
+                if (VEC == 4) {
+                    const f32x4_t t = buf_ld4(rs, off);
+                    v[u][0] = t[0], v[u][1 % VEC] = t[1], v[u][2 % VEC] = t[2], v[u][3 % VEC] = t[3];
+                } else {
+                    v[u][0] = buf_ld1(rs, off);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) s[e] += v[u][e];
+        }
+        __syncthreads();  // the previous column block's sums have been read
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) red[threadIdx.x * VEC + e] = s[e];
+        __syncthreads();
+        if (ty == 0 && on) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float t = 0.f;
+                for (int g = 0; g < TY; ++g) t += red[(g * TX + c0) * VEC + e];
+                y[b * N + c * VEC + e] = t * inv;
+            }
+        }
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void mean_mid_bwd_kernel(const float *__restrict__ dy, float *__restrict__ dx, int P, int N, int TX,
+                                                           float inv) {
+    const int cg = N / VEC, TY = 256 / TX, c0 = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t b = blockIdx.x;
+    const __amdgpu_buffer_rsrc_t rs = buf_rsrc(dx + b * P * N, (int64_t)P * N * 4);
+    for (int cb = 0; cb < cg; cb += TX) {
+        const int c = cb + c0;
+        if (c >= cg) continue;
+        float g[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) g[e] = dy[b * N + c * VEC + e] * inv;
+        for (int p = ty; p < P; p += TY) {
+            const uint32_t off = (uint32_t)(p * N + c * VEC) * 4u;
+            if (VEC == 4) {
+                f32x4_t t;
+                t[0] = g[0], t[1] = g[1 % VEC], t[2] = g[2 % VEC], t[3] = g[3 % VEC];
+                buf_st4(rs, off, t);
+            } else {
+                buf_st1(rs, off, g[0]);
+            }
+        }
+    }
+}
+
 }  // namespace hgq
 
 using namespace hgq;
+
+extern "C" int hgq_mean_mid_fwd(const float *x, float *y, int64_t B, int64_t P, int64_t N, void *stream) {
+    if (B < 0 || P < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_mean_mid_fwd: bad sizes");
+    if (B == 0) return HGQ_OK;
+    if (!x || !y) return fail(HGQ_ERR_ARG, "hgq_mean_mid_fwd: null pointer");
+    if (P * N * 4 >= (1ll << 31) || B >= (1ll << 31)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_mean_mid_fwd: one batch element must stay below 2 GiB");
+    const bool vec = N % 4 == 0 && ((uintptr_t)x & 15u) == 0;
+    const int64_t cg = vec ? N / 4 : N;
+    int TX = 1;
+    while (TX < cg && TX < 256) TX <<= 1;
+    const float inv = 1.0f / (float)P;
+    if (vec) hipLaunchKernelGGL(mean_mid_fwd_kernel<4>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, x, y, (int)P, (int)N, TX, inv);
+    else hipLaunchKernelGGL(mean_mid_fwd_kernel<1>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, x, y, (int)P, (int)N, TX, inv);
+    return check_launch("hgq_mean_mid_fwd");
+}
+
+extern "C" int hgq_mean_mid_bwd(const float *dy, float *dx, int64_t B, int64_t P, int64_t N, void *stream) {
+    if (B < 0 || P < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_mean_mid_bwd: bad sizes");
+    if (B == 0) return HGQ_OK;
+    if (!dy || !dx) return fail(HGQ_ERR_ARG, "hgq_mean_mid_bwd: null pointer");
+    if (P * N * 4 >= (1ll << 31) || B >= (1ll << 31)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_mean_mid_bwd: one batch element must stay below 2 GiB");
+    const bool vec = N % 4 == 0 && ((uintptr_t)dx & 15u) == 0;
+    const int64_t cg = vec ? N / 4 : N;
+    int TX = 1;
+    while (TX < cg && TX < 256) TX <<= 1;
+    const float inv = 1.0f / (float)P;
+    if (vec) hipLaunchKernelGGL(mean_mid_bwd_kernel<4>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dy, dx, (int)P, (int)N, TX, inv);
+    else hipLaunchKernelGGL(mean_mid_bwd_kernel<1>, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, dy, dx, (int)P, (int)N, TX, inv);
+    return check_launch("hgq_mean_mid_bwd");
+}
 
 extern "C" int hgq_pool2d_fwd(const float *x, float *y, const int *geom, int is_max, void *stream) {
     PoolGeom g;

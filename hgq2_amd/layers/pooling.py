@@ -94,6 +94,10 @@ class _QGlobalPooling(QBasePooling):
     def pool(self, inputs):
         axes = tuple(range(1, 1 + self._rank))
         if self._mode == 'avg':
+            if inputs.is_cuda and inputs.dtype == torch.float32 and inputs.dim() == self._rank + 2 and inputs.numel():
+                # channels-last: the pooled axes are the middle ones and collapse into one
+                y = ops.mean_mid(inputs.reshape(inputs.shape[0], -1, inputs.shape[-1]))
+                return y.reshape(self.compute_output_shape(tuple(inputs.shape))) if self.keepdims else y
             return torch.mean(inputs, dim=axes, keepdim=self.keepdims)
         return torch.amax(inputs, dim=axes, keepdim=self.keepdims)
 

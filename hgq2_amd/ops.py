@@ -688,6 +688,51 @@ def _(dy, x, geom, is_max):
     return torch.empty_like(x)
 
 
+@torch.library.custom_op('hgq::mean_mid_fwd', mutates_args=())
+def mean_mid_fwd(x: Tensor) -> Tensor:
+    _check_f32('x', x)
+    _need(x.dim() == 3, 'x must be [B, P, N]')
+    B, P, N = x.shape
+    y = torch.empty((B, N), dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().hgq_mean_mid_fwd(_ptr(x), _ptr(y), B, P, N, _stream()), 'hgq_mean_mid_fwd')
+    return y
+
+
+@mean_mid_fwd.register_fake
+def _(x):
+    return x.new_empty((x.shape[0], x.shape[2]))
+
+
+@torch.library.custom_op('hgq::mean_mid_bwd', mutates_args=())
+def mean_mid_bwd(dy: Tensor, P: int) -> Tensor:
+    _check_f32('dy', dy)
+    B, N = dy.shape
+    dx = torch.empty((B, P, N), dtype=torch.float32, device=dy.device)
+    _lib.check(_lib.load().hgq_mean_mid_bwd(_ptr(dy), _ptr(dx), B, P, N, _stream()), 'hgq_mean_mid_bwd')
+    return dx
+
+
+@mean_mid_bwd.register_fake
+def _(dy, P):
+    return dy.new_empty((dy.shape[0], P, dy.shape[1]))
+
+
+class _MeanMid(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        ctx.P = x.shape[1]
+        return mean_mid_fwd(x)
+
+    @staticmethod
+    def backward(ctx, g):
+        return mean_mid_bwd(g.contiguous(), ctx.P)
+
+
+def mean_mid(x: Tensor) -> Tensor:
+    """``x.mean(1)`` of a ``[B, P, N]`` GPU tensor (one pass each way, rows added in a fixed order)."""
+    return _MeanMid.apply(x.contiguous())
+
+
 def conv2d_ebops_supported(in_shape, kernel_shape) -> bool:
     """Whether hgq_conv2d_ebops covers bit-width tensors [1, H, W, C] x [kh, kw, C, F] (its LDS tables bound the sizes)."""
     _, H, W, C = in_shape

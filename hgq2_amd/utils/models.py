@@ -66,7 +66,8 @@ def particle_mlp(n_particles=64, n_features=16, hidden=(64, 32), n_out=5, beta0=
         set_default_device(device)
     with _Scopes(beta0):
         layers = [QEinsumDenseBatchnorm('bpf,fh->bph', (n_particles, h), bias_axes='h', activation='relu') for h in hidden]
-        layers.append(Lambda(lambda t: torch.mean(t, dim=1), name='mean_over_particles'))
+        layers.append(Lambda(lambda t: ops.mean_mid(t) if t.is_cuda else torch.mean(t, dim=1), lambda t: torch.mean(t, dim=1),
+                             name='mean_over_particles'))
         layers.append(QDense(n_out))
     return Sequential(layers)
 

@@ -576,6 +576,16 @@ int hgq_pool2d_fwd(const float *x, float *y, const int *geom, int is_max, void *
 int hgq_pool2d_bwd(const float *dy, const float *x, float *dx, const int *geom, int is_max, void *stream);
 
 /*
+ * Mean over the middle axis: y[b, n] = mean_p x[b, p, n] and its gradient dx[b, p, n] = dy[b, n] / P.  Replaces
+ * `ops.mean(x, axis)` of the global average pooling layers on channels-last tensors
+ * (src/hgq/layers/pooling.py:23-47 wrap keras.layers.GlobalAveragePooling1D / 2D; the spatial axes are the middle
+ * ones and collapse into P) and the mean over the particles of the per-particle configuration.  A row's partial sums
+ * are added in a fixed order.  One batch element (P * N floats) must be smaller than 2 GiB.
+ */
+int hgq_mean_mid_fwd(const float *x, float *y, int64_t B, int64_t P, int64_t N, void *stream);
+int hgq_mean_mid_bwd(const float *dy, float *dx, int64_t B, int64_t P, int64_t N, void *stream);
+
+/*
  * EBOPs of a convolution and their gradient.  Replaces `ops.sum(self.convolution_op(bw_inp, bw_ker))`
  * of QBaseConv._compute_ebops (src/hgq/layers/conv.py:91-102), evaluated on the bit-width tensors of
  * one sample, by its closed form (no convolution is run): every kernel tap visits a rectangle of

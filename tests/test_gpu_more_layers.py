@@ -680,3 +680,43 @@ def test_dense_moments_chained_input_gradient(rows, K, N, bw_rows):
             assert float((a - b).abs().max()) <= 1e-6 * float(a.abs().max()), name
         else:
             assert torch.equal(a, b), name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('shape', [(4096, 64, 32), (3, 1, 5), (17, 100, 7), (2, 300, 1028), (5, 9, 260), (0, 4, 8)])
+def test_mean_over_the_middle_axis(shape):
+    """ops.mean_mid == x.mean(1) and its gradient (fp64 reference), the form the global average pooling layers and the
+    mean over the particles take on the GPU."""
+    from hgq2_amd import ops
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(sum(shape))
+    x = torch.randn(shape, generator=g)
+    up = torch.randn(shape[0], shape[2], generator=g)
+    xd = x.to(dev).requires_grad_(True)
+    y = ops.mean_mid(xd)
+    assert tuple(y.shape) == (shape[0], shape[2])
+    if shape[0] == 0:
+        return
+    want = x.double().mean(1)
+    assert float((y.detach().cpu().double() - want).abs().max()) <= 1e-6 * (float(want.abs().max()) + 1e-6)
+    (y * up.to(dev)).sum().backward()
+    want_dx = (up.double() / shape[1]).unsqueeze(1).expand(shape)
+    assert float((xd.grad.cpu().double() - want_dx).abs().max()) <= 1e-6 * float(want_dx.abs().max())
+
+
+@pytest.mark.gpu
+def test_global_average_pooling_layers_use_it_and_match_the_library_mean():
+    from hgq2_amd.config import QuantizerConfigScope
+    from hgq2_amd.layers import QGlobalAveragePooling1D, QGlobalAveragePooling2D
+
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(8)
+    with QuantizerConfigScope(default_q_type='dummy'):
+        for layer, shape in ((QGlobalAveragePooling1D(enable_ebops=False), (6, 10, 12)),
+                             (QGlobalAveragePooling2D(enable_ebops=False, keepdims=True), (3, 5, 7, 8))):
+            x = torch.randn(shape, generator=g)
+            y = layer(x.to(dev), training=False)
+            want = x.mean(dim=tuple(range(1, len(shape) - 1)), keepdim=layer.keepdims)
+            assert y.shape == want.shape
+            assert torch.allclose(y.cpu(), want, rtol=1e-6, atol=1e-6)
