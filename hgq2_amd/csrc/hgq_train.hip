@@ -249,35 +249,46 @@ __global__ __launch_bounds__(256) void bn_fold_fwd_kernel(const float *__restric
     }
 }
 
-// Gradients of the folding.  One thread per output column n walks the K kernel rows (coalesced
-// across columns):  dw = d_fw * scaler;  dscaler = sum_k d_fw * w - d_fb * mean;  dbias = d_fb;
-// dgamma = dscaler / sqrt(var + eps);  dvar = -dscaler * gamma / (2 (var + eps)^(3/2));
-// dmean = -d_fb * scaler (- 2 mean dvar when var comes from the mean of squares);  dsecond = dvar.
-__global__ __launch_bounds__(64) void bn_fold_bwd_kernel(const float *__restrict__ w, const float *__restrict__ gamma,
-                                                         const float *__restrict__ mean, const float *__restrict__ second,
-                                                         int is_meansq, float eps, const float *__restrict__ d_fw,
-                                                         const float *__restrict__ d_fb, float *__restrict__ dw, float *dbias,
-                                                         float *dgamma, float *dmean, float *dsecond, int K, int N) {
-    const int n = blockIdx.x * 64 + threadIdx.x;
-    if (n >= N) return;
-    const float g = gamma ? gamma[n] : 1.0f, m = mean[n];
-    const float ve = bn_var(m, second[n], is_meansq) + eps, sd = __fsqrt_rn(ve);
+// Gradients of the folding.  Thread (column n, row group r of 4) walks kernel rows r, r + 4, ... with all its loads in
+// flight (coalesced across columns); the four partial sums of a column meet in LDS in group order:
+//   dw = d_fw * scaler;  dscaler = sum_k d_fw * w - d_fb * mean;  dbias = d_fb;
+//   dgamma = dscaler / sqrt(var + eps);  dvar = -dscaler * gamma / (2 (var + eps)^(3/2));
+//   dmean = -d_fb * scaler (- 2 mean dvar when var comes from the mean of squares);  dsecond = dvar.
+#define BNF_ROWS 16  // rows per thread and trip
+__global__ __launch_bounds__(256) void bn_fold_bwd_kernel(const float *__restrict__ w, const float *__restrict__ gamma,
+                                                          const float *__restrict__ mean, const float *__restrict__ second,
+                                                          int is_meansq, float eps, const float *__restrict__ d_fw,
+                                                          const float *__restrict__ d_fb, float *__restrict__ dw, float *dbias,
+                                                          float *dgamma, float *dmean, float *dsecond, int K, int N) {
+    __shared__ float part[4][64];
+    const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6, n = blockIdx.x * 64 + nl;
+    const bool col = n < N;
+    const float g = (gamma && col) ? gamma[n] : 1.0f, m = col ? mean[n] : 0.f;
+    const float ve = bn_var(m, col ? second[n] : 1.0f, is_meansq) + eps, sd = __fsqrt_rn(ve);
     const float scaler = __fdiv_rn(g, sd);
+    const int64_t bytes = (int64_t)K * N * 4;
+    const __amdgpu_buffer_rsrc_t rs_g = buf_rsrc(d_fw, bytes), rs_w = buf_rsrc(w, bytes), rs_dw = buf_rsrc(dw, bytes);
     float ds = 0.f;
-    for (int k0 = 0; k0 < K; k0 += 8) {
-        float gv[8], wv[8];
+    for (int k0 = grp; k0 < K; k0 += 4 * BNF_ROWS) {
+        float gv[BNF_ROWS], wv[BNF_ROWS];
+        uint32_t off[BNF_ROWS];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const bool on = k0 + u < K;
-            gv[u] = on ? d_fw[(int64_t)(k0 + u) * N + n] : 0.f;
-            wv[u] = on ? w[(int64_t)(k0 + u) * N + n] : 0.f;
+        for (int u = 0; u < BNF_ROWS; ++u) {
+            const int k = k0 + 4 * u;
+            off[u] = (col && k < K) ? (uint32_t)(k * N + n) * 4u : BUF_OOB;  // rows / columns past the end read as zero
+            gv[u] = buf_ld1(rs_g, off[u]);
+            wv[u] = buf_ld1(rs_w, off[u]);
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < BNF_ROWS; ++u) {
             ds += gv[u] * wv[u];
-            if (k0 + u < K) dw[(int64_t)(k0 + u) * N + n] = gv[u] * scaler;
+            buf_st1(rs_dw, off[u], gv[u] * scaler);
         }
     }
+    part[grp][nl] = ds;
+    __syncthreads();
+    if (grp != 0 || !col) return;
+    ds = ((part[0][nl] + part[1][nl]) + part[2][nl]) + part[3][nl];
     const float gb = d_fb[n];
     ds -= gb * m;
     const float dvar = -ds * g / (2.0f * ve * sd);
@@ -582,7 +593,8 @@ extern "C" int hgq_bn_fold_bwd(const float *w, const float *gamma, const float *
                                float *dsecond, int K, int N, void *stream) {
     if (K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_bn_fold_bwd: bad sizes");
     if (!w || !mean || !second || !d_fw || !d_fb || !dw) return fail(HGQ_ERR_ARG, "hgq_bn_fold_bwd: null pointer");
-    hipLaunchKernelGGL(bn_fold_bwd_kernel, dim3((unsigned)((N + 63) / 64)), dim3(64), 0, (hipStream_t)stream, w, gamma, mean, second,
+    if ((int64_t)K * N * 4 >= (1ll << 31)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_bn_fold_bwd: the kernel matrix must be smaller than 2 GiB");
+    hipLaunchKernelGGL(bn_fold_bwd_kernel, dim3((unsigned)((N + 63) / 64)), dim3(256), 0, (hipStream_t)stream, w, gamma, mean, second,
                        is_meansq, eps, d_fw, d_fb, dw, dbias, dgamma, dmean, dsecond, K, N);
     return check_launch("hgq_bn_fold_bwd");
 }
