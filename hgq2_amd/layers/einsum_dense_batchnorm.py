@@ -10,6 +10,7 @@ import torch
 
 from .. import _lib, ops
 from ..core import epsilon, get_initializer
+from ..quantizer.prefetch import quantize_together
 from .core._contraction import fused_iq_rows
 from .core.einsum_dense import QEinsumDense, analyze_einsum_string
 
@@ -158,8 +159,9 @@ class QEinsumDenseBatchnorm(QEinsumDense):
             fused_kernel, fused_bias = ops.bn_fold(self._kernel.reshape(self._K, self._N), self.bias.reshape(-1),
                                                    self.bn_gamma.reshape(-1) if self.scale else None, mean, meansq, True, epsilon(),
                                                    self.moving_mean.view(-1), self.moving_variance.view(-1), self.momentum)
-            qkernel = self.kq(fused_kernel.view(self._kernel.shape), training=training)
-            qbias = self.bq(fused_bias.view(self.bias.shape), training=training)
+            # kernel and bias quantizers in one launch each way (they are a few thousand elements together)
+            qkernel, qbias = quantize_together([(self.kq, fused_kernel.view(self._kernel.shape)),
+                                                (self.bq, fused_bias.view(self.bias.shape))], training)
         else:
             if training and self.trainable:
                 mean, var = self._batch_moments(inputs)

@@ -27,6 +27,18 @@ def _eligible(q, p):
     return fq
 
 
+def quantize_together(pairs, training):
+    """``[q(x) for q, x in pairs]`` for quantizer wrappers ``q`` and tensors ``x`` (not necessarily variables): one
+    launch each way when every pair is a plain per-element saturating quantizer in training mode, else one by one."""
+    if training is True and len(pairs) > 1:
+        fqs = [_eligible(q, x) for q, x in pairs]
+        if all(fq is not None for fq in fqs):
+            ys = ops.quantize_multi([x for _, x in pairs], [fq._k.view(-1) for fq in fqs], [fq._i.view(-1) for fq in fqs],
+                                    [fq._third().view(-1) for fq in fqs], [fq._mode(True) for fq in fqs])
+            return list(ys)
+    return [q(x, training=training) for q, x in pairs]
+
+
 def prefetch_weight_quantizers(root) -> int:
     """Quantize the kernels and biases of every layer under ``root`` that declares them (``_weight_quantizer_inputs``)
     in one launch and leave each result with its quantizer for the layer's own call to pick up.  Returns the number
