@@ -18,6 +18,7 @@ import torch
 from .. import ops
 from ..core import get_initializer
 from ..quantizer import Quantizer, QuantizerConfig
+from ..quantizer.prefetch import quantize_together
 from .core.base import QLayerBaseSingleInput
 
 
@@ -104,8 +105,8 @@ class QBatchNormalization(QLayerBaseSingleInput):
         else:
             mean, variance = self.moving_mean, self.moving_variance
         scale, offset = self._scale_offset(mean, variance)
-        qscale = self.kq(scale, training=training).reshape(self._shape)
-        qoffset = self.bq(offset, training=training).reshape(self._shape)
+        qscale, qoffset = quantize_together([(self.kq, scale.contiguous()), (self.bq, offset.contiguous())], training)
+        qscale, qoffset = qscale.reshape(self._shape), qoffset.reshape(self._shape)
         return inputs * qscale + qoffset
 
     def _compute_ebops(self, shape):
