@@ -38,7 +38,9 @@ What pins what
       clip: d/dx = 1 inside, 0 outside; the active bound receives the upstream
             gradient, and the bounds are differentiable functions of i and f:
             d max/d i = ln2*2**i, d max/d f = +ln2*2**-f, min = -k*2**i or -k*max.
-  The clip part is additionally checked against finite differences of the bounds.
+  The clip part is additionally checked against finite differences of the bounds, and the
+  rounding part against a numerical derivative of the stated error model
+  (delta(f+h) = delta(f) * 2**-h); that the package uses this model stays unverifiable here.
 * ``i`` is not clamped against ``-f`` inside the callable (any such clamp in the
   third-party package is unpinned; it can only matter where k+i+f <= 0, which the
   reference zeroes at inference, fixed_point_quantizer.py:148-149).

@@ -730,7 +730,7 @@ class RefQMultiHeadAttention(RefQLayer):
     def __call__(self, x, training=None, mask=None):
         self.losses = []
         r = self.call(x, training=training, mask=mask)
-        if training and self.enable_ebops:
+        if (training or training == 'tracing') and self.enable_ebops:
             ebops = self._compute_ebops()
             self.ebops_value = ebops.detach().to(torch.int64)
             self.losses.append(ebops * self.beta)
