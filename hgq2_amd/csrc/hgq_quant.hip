@@ -568,7 +568,7 @@ __global__ __launch_bounds__(64 * WT_G) void wrap_track_i_kernel(const uint32_t 
         const float eps = 1e-7f;
         const float num = __fadd_rn(xr, eps);
         const float den = __fadd_rn(__fsub_rn(1.0f, pow2(-b)), eps);
-        mi = ceilf(log2f(__fdiv_rn(num, den)));
+        mi = ceil_log2_exact(__fdiv_rn(num, den));  // exact: log2f is only faithfully rounded
         if (!m.symmetric && !(b > 0.0f)) mi = 32.0f;
     }
     float ni;

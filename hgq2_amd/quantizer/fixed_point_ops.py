@@ -34,15 +34,22 @@ class FixedQuantizer:
         _lib.mode_bits(self.round_mode, self.overflow_mode)  # validates
 
     def _run(self, x, k, i, f, training, overflow_mode):
-        shape = x.shape
-        k, i, f = (torch.broadcast_to(t, shape) if t.shape != shape else t for t in (k, i, f))
-        kc, ic, fc = _compact(k), _compact(i), _compact(f)
-        layout = bw_layout(ic.shape, shape) if kc.shape == ic.shape == fc.shape else None
-        if layout is None:
-            kc, ic, fc = k.contiguous(), i.contiguous(), f.contiguous()
-            layout = (x.numel(), 1)
+        shape = tuple(x.shape)
+        small = []
+        for t in (k, i, f):
+            t = torch.as_tensor(t, dtype=x.dtype, device=x.device)
+            if tuple(t.shape) != shape:
+                t = torch.broadcast_to(t, shape)
+            small.append(_compact(t))
+        # the three operands may broadcast along different axes (``round`` passes constants for k and i): the
+        # bit-width block is the smallest shape that holds all of them
+        bw_shape = tuple(max(dims) for dims in zip(*(t.shape for t in small))) if shape else ()
+        layout = bw_layout(bw_shape, shape)
+        if layout is None:  # a broadcast pattern the kernels do not index: per-element operands
+            bw_shape, layout = shape, (x.numel(), 1)
+        kc, ic, fc = (t.expand(bw_shape).contiguous() for t in small)
         mode = _lib.mode_bits(self.round_mode, overflow_mode, training=bool(training))
-        y, _, _ = ops.quantize(x, kc.contiguous(), ic.contiguous(), fc.contiguous(), mode, bw_inner=layout[1])
+        y, _, _ = ops.quantize(x.contiguous(), kc, ic, fc, mode, bw_inner=layout[1])
         return y
 
     def __call__(self, x, k, i, f, training=False, seed_gen=None):
@@ -55,8 +62,9 @@ class FixedQuantizer:
     def round(self, x, f, stochastic=False, seed_gen=None):
         if stochastic:
             raise NotImplementedError('stochastic rounding is not part of this build')
-        one = torch.ones((), dtype=x.dtype, device=x.device).expand(x.shape)
-        zero = torch.zeros((), dtype=x.dtype, device=x.device).expand(x.shape)
+        # rounding only = the WRAP training branch; k and i are not read there (0-dim constants, nothing expanded)
+        one = torch.ones((), dtype=x.dtype, device=x.device)
+        zero = torch.zeros((), dtype=x.dtype, device=x.device)
         return self._run(x, one, zero, f, True, 'WRAP')
 
 

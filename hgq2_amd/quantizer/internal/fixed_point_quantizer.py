@@ -260,7 +260,9 @@ class FixedPointQuantizerKBI(FixedPointQuantizerBase):
                 y, _, neg = self._quantize(inputs, self._mode(True), track=not is_training)
                 if not is_training:
                     with torch.no_grad():
-                        new_k = neg.view(self._k.shape).bool() & (torch.round(self._b) > 0)
+                        # the tracker arrives as one entry per bit-width entry or as [slices, entries]
+                        seen = neg.view(-1, self._k.numel()).ne(0).any(0).view(self._k.shape)
+                        new_k = seen & (torch.round(self._b) > 0)
                         self._k.copy_((self._k.bool() | new_k).to(torch.uint8))
                 return y
             if self._is_weight and self.round_mode == 'RND':

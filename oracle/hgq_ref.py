@@ -27,6 +27,21 @@ from .fixed_point import get_fixed_quantizer, round_conv
 
 EPSILON = 1e-7  # keras.backend.epsilon() default
 
+# Checker precision.  False: every op in fp32, as the reference executes (this is what ``cpu_baseline`` times).
+# True: the contractions (matmul / einsum / convolution) and everything downstream of them are evaluated in float64,
+# while every quantizer still sees and produces fp32 values; a parity test that compares sums over 10^5..10^7 terms
+# sets it so that its tolerance measures the kernel under test and not the fp32 summation order of this file.
+ACC64 = False
+
+
+def _acc(t):
+    return t.double() if ACC64 else t
+
+
+def _f32(t):
+    """Operand of a quantizer: always fp32 (a float64 intermediate is rounded once, like the fp32 op would)."""
+    return t.float() if t.dtype == torch.float64 else t
+
 
 # --------------------------------------------------------------------------------------
 # fpq.py:16-31
@@ -436,7 +451,7 @@ class RefQDense(RefQLayer):
         if self.iq is not None:
             x = self.iq(x, training=training)
         qkernel = self.kq(self.kernel, training=training)
-        y = torch.matmul(x, qkernel)
+        y = torch.matmul(_acc(x), _acc(qkernel))
         if self.bias is not None:
             y = y + self.bq(self.bias, training=training)
         if self.activation == 'relu':
@@ -493,7 +508,7 @@ class RefQEinsumDense(RefQLayer):
         qkernel = self.kq(self.kernel, training=training)
         if self.iq is not None:
             x = self.iq(x, training=training)
-        y = torch.einsum(self.equation, x, qkernel)
+        y = torch.einsum(self.equation, _acc(x), _acc(qkernel))
         if self.bias is not None:
             y = y + self.bq(self.bias, training=training)
         if self.activation == 'relu':
@@ -536,17 +551,17 @@ class RefQEinsumDenseBatchnorm(RefQEinsumDense):
     def fused(self, training, mean, var):
         gamma = self.gamma if self.gamma is not None else 1
         scaler = gamma / torch.sqrt(var + EPSILON)
-        fused_kernel = torch.einsum(self.fused_kernel_equation, self.kernel, scaler)
-        qkernel = self.kq(fused_kernel, training=training)
+        fused_kernel = torch.einsum(self.fused_kernel_equation, _acc(self.kernel), scaler)
+        qkernel = self.kq(_f32(fused_kernel), training=training)
         offset = torch.reshape(-mean * scaler, self.bias.shape)
-        qbias = self.bq(self.bias + offset, training=training)
+        qbias = self.bq(_f32(self.bias + offset), training=training)
         return qkernel, qbias
 
     def call(self, x, training=None):
         if self.iq is not None:
             x = self.iq(x, training=training)
         if training:
-            z = torch.einsum(self.equation, x, self.kernel)
+            z = torch.einsum(self.equation, _acc(x), _acc(self.kernel))
             mean = torch.mean(z, dim=self.reduction_axes)
             var = torch.mean(torch.square(z), dim=self.reduction_axes) - torch.square(mean)
             with torch.no_grad():
@@ -555,7 +570,7 @@ class RefQEinsumDenseBatchnorm(RefQEinsumDense):
         else:
             var, mean = self.moving_variance, self.moving_mean
         qkernel, qbias = self.fused(training, mean, var)
-        y = torch.einsum(self.equation, x, qkernel) + qbias
+        y = torch.einsum(self.equation, _acc(x), _acc(qkernel)) + qbias
         if self.activation == 'relu':
             y = torch.relu(y)
         return y
@@ -791,7 +806,7 @@ class RefQConv2D(RefQLayer):
     def call(self, x, training=None):
         if self.iq is not None:
             x = self.iq(x, training=training)
-        y = self.conv(x, self.kq(self.kernel, training=training))
+        y = self.conv(_acc(x), _acc(self.kq(self.kernel, training=training)))
         if self.bias is not None:
             y = y + self.bq(self.bias, training=training).reshape(1, 1, 1, -1)
         if self.activation == 'relu':

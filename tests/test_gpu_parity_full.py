@@ -1,0 +1,350 @@
+"""GPU parity at the full sizes of the benchmark configurations, and of the seams and branches the smaller tests do
+not reach: the standalone quantizer at 4 Mi elements, the stateless callable driven the way the reference drives it,
+the KBI WRAP state machine (training and calibration) with batch-shared bit-widths, the ``Quantizer`` wrapper with
+scaler / noise blend / affine map, and the backward pass of the per-particle and image configurations.
+
+Bars: quantized values, tracked integer bits, keep-negative flags and EBOPs bit-exact; everything that is a sum in
+fp32 within 1e-5 of the sum of the absolute values of its terms (the oracle evaluates its contractions in float64 for
+these tests, ``oracle.hgq_ref.ACC64``, so the bound measures the kernel and not the oracle's own summation order)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import fixed_point as ofp
+from oracle import hgq_ref as ref
+from tests import twin
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+@pytest.fixture
+def acc64():
+    ref.ACC64 = True
+    yield
+    ref.ACC64 = False
+
+
+def _close_scaled(got, want, scale, what, rtol=RTOL):
+    got, want, scale = got.detach().double().cpu(), want.detach().double(), scale.detach().double()
+    err = (got.reshape(want.shape) - want).abs()
+    tol = rtol * scale.reshape(want.shape) + 1e-30
+    ratio = (err / tol).reshape(-1)
+    at = int(ratio.argmax())
+    assert float(ratio[at]) <= 1.0, (f'{what}: error is {float(ratio[at]):.2f} x the bound at element {at}: got '
+                                     f'{float(got.reshape(-1)[at]):.6e}, want {float(want.reshape(-1)[at]):.6e}, sum of |terms| '
+                                     f'{float(scale.reshape(-1)[at]):.3e} (max err anywhere {float(err.max()):.3e})')
+
+
+def _close_tensor(got, want, what, rtol=RTOL):
+    """Per element within rtol * (|want| + max|want|): for gradients that are not a plain sum of products."""
+    want = want.detach().double()
+    _close_scaled(got, want, want.abs() + want.abs().max() + 1e-12, what, rtol)
+
+
+# --------------------------------------------------------------------------------------------------------------
+# configuration 1: the standalone quantizer at its full size
+# --------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('overflow_mode', ['WRAP', 'SAT', 'SAT_SYM'])
+@pytest.mark.parametrize('training', [True, False])
+def test_standalone_quantizer_at_4Mi(dev, overflow_mode, training):
+    """4 Mi fp32 elements, x ~ N(0, 4), per-element k = 1, i ~ U{0..4}, f ~ U{0..8}, RND: values bit-exact in
+    training and inference mode, dx / di / df (training) within 1e-5 per element (no sums are involved)."""
+    from hgq2_amd import _lib, ops
+
+    n = 4 * 1024 * 1024
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(n, generator=g) * 2.0).requires_grad_(training)
+    k = torch.ones(n)
+    i = torch.randint(0, 5, (n,), generator=g).float().requires_grad_(training)
+    f = torch.randint(0, 9, (n,), generator=g).float().requires_grad_(training)
+    gy = torch.randn(n, generator=g)
+    q = ofp.get_fixed_quantizer('RND', overflow_mode)
+    want = q(x, k, i, f, training, None)
+    if not training:
+        want = torch.where(k + i + f > 0, want, torch.zeros_like(want))
+    mode = _lib.mode_bits('RND', overflow_mode, training=training)
+    xd, idv, fd = (t.detach().to(dev).requires_grad_(training) for t in (x, i, f))
+    y, _, _ = ops.quantize(xd, k.to(dev), idv, fd, mode)
+    assert torch.equal(y.detach().cpu(), want.detach())
+    if not training:
+        return
+    want.backward(gy)
+    y.backward(gy.to(dev))
+    for got, ref_g, name in ((xd.grad, x.grad, 'dx'), (idv.grad, i.grad, 'di'), (fd.grad, f.grad, 'df')):
+        ref_g = torch.zeros(n) if ref_g is None else ref_g
+        got = torch.zeros(n) if got is None else got.cpu()
+        np.testing.assert_allclose(got.numpy(), ref_g.numpy(), rtol=RTOL, atol=1e-30, err_msg=f'{overflow_mode} {name}')
+
+
+# --------------------------------------------------------------------------------------------------------------
+# the stateless callable, driven as the reference drives it
+# --------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('x_shape,bw_shape', [((3000, 24), (1, 24)), ((700, 6, 10), (1, 6, 10)), ((513, 33), (1, 1)),
+                                              ((64, 8, 16), (1, 8, 1)), ((40, 50), (40, 50))])
+@pytest.mark.parametrize('overflow_mode', ['WRAP', 'SAT', 'SAT_SYM'])
+def test_fixed_quantizer_callable_as_the_reference_calls_it(dev, x_shape, bw_shape, overflow_mode):
+    """Reference src/hgq/quantizer/internal/fixed_point_quantizer.py:142-150: k, i, f are ``broadcast_to`` the
+    input's shape, then ``q(x, k, i, f, training, None)``; :288,:405: ``q.round(x, f, False, None)``.  The callable of
+    ``hgq2_amd.quantizer.fixed_point_ops`` must give the oracle's values bit for bit and its gradients to x and to the
+    small bit-width tensors (autograd sums the broadcast back)."""
+    from hgq2_amd.quantizer.fixed_point_ops import get_fixed_quantizer
+
+    g = torch.Generator().manual_seed(sum(x_shape))
+    x = torch.randn(x_shape, generator=g) * 3
+    k = torch.randint(0, 2, bw_shape, generator=g).float()
+    i = torch.randint(-1, 4, bw_shape, generator=g).float()
+    f = torch.randint(0, 7, bw_shape, generator=g).float()
+    gy = torch.randn(x_shape, generator=g)
+    q_ref, q_dev = ofp.get_fixed_quantizer('RND', overflow_mode), get_fixed_quantizer('RND', overflow_mode)
+    assert q_dev.round_mode == 'RND' and q_dev.stochastic is False
+
+    def run(q, device, training, rounding_only):
+        xs = x.clone().to(device).requires_grad_(True)
+        ks = k.to(device)
+        is_, fs = i.clone().to(device).requires_grad_(True), f.clone().to(device).requires_grad_(True)
+        kb, ib, fb = (torch.broadcast_to(t, x_shape) for t in (ks, is_, fs))
+        y = q.round(xs, fb, False, None) if rounding_only else q(xs, kb, ib, fb, training, None)
+        if training:
+            y.backward(gy.to(device))
+        return y.detach().cpu(), xs.grad, is_.grad, fs.grad
+
+    for training, rounding_only in ((True, False), (False, False), (True, True)):
+        want = run(q_ref, 'cpu', training, rounding_only)
+        got = run(q_dev, dev, training, rounding_only)
+        want_y = want[0]
+        if not training:
+            kb, ib, fb = (torch.broadcast_to(t, x_shape) for t in (k, i, f))
+            want_y = torch.where(kb + ib + fb > 0, want_y, torch.zeros_like(want_y))  # the reference applies this around the call
+        assert torch.equal(got[0], want_y), f'values training={training} round={rounding_only}'
+        if not training:
+            continue
+        np.testing.assert_allclose(got[1].cpu().numpy(), want[1].numpy(), rtol=RTOL, atol=1e-30)
+        hom = tuple(a for a in range(len(x_shape)) if bw_shape[a] == 1 and x_shape[a] != 1)
+        for gg, wg, name in ((got[2], want[2], 'di'), (got[3], want[3], 'df')):
+            wg = torch.zeros(bw_shape) if wg is None else wg
+            gg = torch.zeros(bw_shape) if gg is None else gg.cpu()
+            # a sum over the broadcast axes: bound by the sum of |terms|, which is at most sum |gy| * max coefficient
+            scale = gy.abs().sum(dim=hom, keepdim=True) * (math.log(2) * 2.0 ** i.clamp(min=0) + 1.0) if hom else wg.abs() + 1e-6
+            _close_scaled(gg, wg, scale.expand(bw_shape) if hom else scale, f'{name} training={training} round={rounding_only}')
+
+
+# --------------------------------------------------------------------------------------------------------------
+# KBI WRAP with batch-shared bit-widths: training and calibration
+# --------------------------------------------------------------------------------------------------------------
+def _kbi_wrap_pair(dev, F, g):
+    from hgq2_amd.config import QuantizerConfig
+    from hgq2_amd.quantizer import Quantizer
+
+    q = Quantizer(QuantizerConfig('kbi', 'datalane', overflow_mode='WRAP', round_mode='RND'))
+    q(torch.zeros(4, F, device=dev), training=False)  # build on the device
+    with torch.no_grad():
+        q.quantizer._b.copy_(torch.randint(0, 9, (1, F), generator=g).float().to(dev))
+        q.quantizer._i.copy_((torch.randint(-2, 3, (1, F), generator=g).float() + 0.3).to(dev))
+    return q, twin.ref_quantizer(q)
+
+
+def test_kbi_wrap_training_matches_oracle_with_many_row_chunks(dev):
+    """Reference fixed_point_quantizer.py:277-288.  2000 rows of a [1, F] quantizer span several row chunks of the
+    per-column kernels; integer bits exact over three steps, values exact, d/db within the sum bound."""
+    g = torch.Generator().manual_seed(21)
+    F = 16
+    q, r = _kbi_wrap_pair(dev, F, g)
+    assert tuple(q.quantizer._b.shape) == (1, F) and q.quantizer.overflow_mode == 'WRAP'
+    x = torch.randn(2000, F, generator=g) * torch.logspace(-2, 2, F)
+    x[:, 3] = 0.0
+    x[:, 4:7] = x[:, 4:7].clamp(-0.25, 0.25)
+    x[0, 4], x[1, 5], x[2, 6] = 1.0, -0.5, 4.0  # exact powers of two as column maxima (they stay so when halved)
+    for step in range(3):
+        xs = x * (0.5 ** step)
+        xp, xr = xs.to(dev).requires_grad_(True), xs.clone().requires_grad_(True)
+        gy = torch.randn(xs.shape, generator=g)
+        yp, yr = q(xp, training=True), r(xr, training=True)
+        assert torch.equal(q.quantizer._i.cpu(), r.quantizer._i.detach()), f'_i step {step}'
+        assert torch.equal(yp.detach().cpu(), yr.detach()), f'values step {step}'
+        q.quantizer._b.grad = r.quantizer._b.grad = None
+        yp.backward(gy.to(dev))
+        yr.backward(gy)
+        np.testing.assert_allclose(xp.grad.cpu().numpy(), xr.grad.numpy(), rtol=RTOL, atol=1e-30)
+        delta = (yr.detach() - xs).double()
+        scale = (math.log(2) * delta.abs() * gy.double().abs()).sum(0, keepdim=True) + 1e-12
+        _close_scaled(q.quantizer._b.grad, r.quantizer._b.grad, scale, f'd/db step {step}')
+    assert torch.equal(q.quantizer._k.cpu(), r.quantizer._k)
+
+
+def test_kbi_wrap_tracing_matches_oracle_with_many_row_chunks(dev):
+    """Reference fixed_point_quantizer.py:289-300 through the calibration flag: integer bits only grow, rounding uses
+    the new integer bits, the keep-negative flag collects negatives of the rounded values where b > 0."""
+    from hgq2_amd.core import TrainingFlagWrapper
+
+    g = torch.Generator().manual_seed(22)
+    F = 16
+    q, r = _kbi_wrap_pair(dev, F, g)
+    with torch.no_grad():
+        for inner in (q.quantizer, r.quantizer):
+            inner._i.fill_(-1e9)
+            inner._k.zero_()
+    flag = TrainingFlagWrapper('tracing')
+    base = torch.randn(1500, F, generator=g) * torch.logspace(-2, 1.5, F)
+    base[:, 2] = base[:, 2].abs()            # a lane that never goes negative
+    base[:, 7] = -base[:, 7].abs() * 1e-4    # negatives that round to zero for small f
+    for scale in (0.25, 1.0, 0.5):
+        xs = base * scale
+        yp, yr = q(xs.to(dev), training=flag), r(xs, training=flag)
+        assert torch.equal(yp.cpu(), yr), f'values at scale {scale}'
+        assert torch.equal(q.quantizer._i.cpu(), r.quantizer._i.detach()), f'_i at scale {scale}'
+        assert torch.equal(q.quantizer._k.cpu(), r.quantizer._k), f'_k at scale {scale}'
+    assert int(r.quantizer._k.sum()) not in (0, F)  # both outcomes occur
+
+
+# --------------------------------------------------------------------------------------------------------------
+# the Quantizer wrapper with its optional stages
+# --------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('extras', [dict(scaler=4.0), dict(qnoise_factor=0.3), dict(affine=(0.5, -2.0)),
+                                    dict(scaler=0.125, qnoise_factor=0.75, affine=(3.0, 1.0))])
+@pytest.mark.parametrize('overflow_mode', ['WRAP', 'SAT'])
+def test_quantizer_wrapper_scaler_qnoise_affine(dev, extras, overflow_mode):
+    """Reference src/hgq/quantizer/quantizer.py:49-60 against the oracle twin: the inner quantizer's values are exact,
+    the elementwise stages around it are fp32 ops in the same order, so the outputs are compared bit for bit in
+    inference and at 1e-6 in training (noise blend: one fused multiply-add may differ)."""
+    from hgq2_amd.config import QuantizerConfig
+    from hgq2_amd.quantizer import Quantizer
+
+    g = torch.Generator().manual_seed(23)
+    q = Quantizer(QuantizerConfig('kif', 'datalane', overflow_mode=overflow_mode, **extras))
+    x = torch.randn(3000, 12, generator=g) * 3
+    q(x.to(dev), training=False)
+    with torch.no_grad():
+        q.quantizer._f.copy_(torch.randint(1, 6, (1, 12), generator=g).float().to(dev))
+        q.quantizer._i.copy_(torch.randint(0, 3, (1, 12), generator=g).float().to(dev))
+    r = twin.ref_quantizer(q)
+    with torch.no_grad():
+        assert torch.equal(q(x.to(dev), training=False).cpu(), r(x, training=False))
+    xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
+    gy = torch.randn(x.shape, generator=g)
+    yp, yr = q(xp, training=True), r(xr, training=True)
+    np.testing.assert_allclose(yp.detach().cpu().numpy(), yr.detach().numpy(), rtol=1e-6, atol=1e-6)
+    assert torch.equal(q.quantizer._i.cpu(), r.quantizer._i.detach())
+    yp.backward(gy.to(dev))
+    yr.backward(gy)
+    np.testing.assert_allclose(xp.grad.cpu().numpy(), xr.grad.numpy(), rtol=RTOL, atol=1e-7)
+    scale = gy.abs().sum(0, keepdim=True) * 64.0  # sum of |gy| x the largest coefficient any stage can contribute
+    _close_scaled(q.quantizer._f.grad, r.quantizer._f.grad, scale, 'd/df')
+    if overflow_mode == 'SAT':  # the integer bits are trainable unless the overflow mode is WRAP
+        _close_scaled(q.quantizer._i.grad, r.quantizer._i.grad, scale, 'd/di')
+
+
+# --------------------------------------------------------------------------------------------------------------
+# configurations 3 and 4: backward at full size
+# --------------------------------------------------------------------------------------------------------------
+def _abs_sum_scales(contract, x_q, w_q, dz):
+    """Sum of |terms| of the three gradients of a bilinear contraction y = contract(x, w): autograd of the same
+    contraction on absolute operands, in float64."""
+    xa = x_q.detach().double().abs().requires_grad_(True)
+    wa = w_q.detach().double().abs().requires_grad_(True)
+    contract(xa, wa).backward(dz.detach().double().abs())
+    return xa.grad, wa.grad
+
+
+def _layer_backward_check(dev, layer, r, x, g, contract, what, second_path=False):
+    """One training forward + backward of a product layer and its oracle twin from the same input and upstream
+    gradient; every gradient compared."""
+    from hgq2_amd.train import model_loss
+
+    xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
+    yp = layer(xp, training=True)
+    yr = r(xr, training=True)
+    gy = torch.randn(yr.shape, generator=g)
+    model_loss(layer, (yp * gy.to(dev)).sum()).backward()
+    ((yr * gy.double()).sum() + r.extra_loss()).backward()
+    assert torch.equal(layer.iq.quantizer._i.cpu(), r.iq.quantizer._i.detach()), f'{what}: tracked integer bits'
+    assert int(layer.ebops.cpu().view(torch.int32)) == int(r.ebops_value), f'{what}: EBOPs'
+    # forward: each output is a sum over the contraction
+    with torch.no_grad():  # the operands of the contraction, for the sum-of-|terms| scales
+        xq = ofp.fixed_round(x, torch.broadcast_to(r.iq.quantizer.f.detach(), x.shape), r.iq.quantizer.round_mode, False)
+        wq = r.kq.last
+        y_scale = contract(xq.double().abs(), wq.double().abs()) + 1e-6
+    _close_scaled(yp, yr, y_scale, f'{what}: output')
+    dz = gy.double() * (yr.detach() > 0) if r.activation == 'relu' else gy.double()
+    sx, sw = _abs_sum_scales(contract, xq, wq, dz)
+    if second_path:
+        # batch-norm folding: x also reaches the loss through the batch statistics, a path the sum above does not see
+        # (it alone carries the gradient of a row whose outputs are all inactive); its terms are bounded through the result
+        sx = sx + xr.grad.detach().double().abs() + xr.grad.detach().double().abs().mean()
+    _close_scaled(xp.grad, xr.grad, sx + 1e-9, f'{what}: dx')
+    return dz, sw, yr.detach().float()
+
+
+class _TapQuantizer(ref.RefQuantizer):
+    """Keeps the last result (the quantized kernel that entered the contraction)."""
+
+    def __call__(self, x, training=None):
+        out = super().__call__(x, training=training)
+        self.last = out.detach()
+        return out
+
+
+@pytest.mark.parametrize('kind', ['particle', 'conv'])
+def test_full_size_backward_matches_oracle(dev, acc64, kind):
+    """The per-particle network (4096 x 64 x 16 -> 64 -> 32 -> mean -> 5) and the image network (1024 x 28 x 28 x 1,
+    two 3x3x32 convolutions, 10 outputs) at full size, layer by layer from the oracle's activations: output, dx and
+    the gradients of kernel, bias, batch-norm scale and every bit-width variable."""
+    import torch.nn.functional as F
+
+    from hgq2_amd.utils import models
+
+    g = torch.Generator().manual_seed(51)
+    torch.manual_seed(51)
+    if kind == 'particle':
+        x = torch.randn(4096, 64, 16, generator=g)
+        model = models.particle_mlp(device=dev)
+    else:
+        x = torch.rand(1024, 28, 28, 1, generator=g)
+        model = models.conv_stack(device=dev)
+    with torch.no_grad():
+        model(x.to(dev), training=True)  # build, adapt the tracked bits
+    from tests.test_gpu_more_layers import _perturb
+
+    _perturb(model, g)
+    h = x
+    for layer in model.layers:
+        if isinstance(layer, models.Lambda):
+            h = layer.host_fn(h)
+            continue
+        name = layer.__class__.__name__
+        for p in layer.parameters():
+            p.grad = None
+        if name == 'QConv2D':
+            r = twin.ref_conv2d(layer)
+            contract = lambda a, w: F.conv2d(a.permute(0, 3, 1, 2), w.permute(3, 2, 0, 1)).permute(0, 2, 3, 1)  # noqa: E731
+        elif name == 'QEinsumDenseBatchnorm':
+            r = twin.ref_einsum_dense_bn(layer, tuple(h.shape))
+            contract = lambda a, w: torch.einsum('bpf,fh->bph', a, w)  # noqa: E731
+        else:
+            r = twin.ref_dense(layer)
+            contract = lambda a, w: a @ w  # noqa: E731
+        r.kq.__class__ = _TapQuantizer
+        what = f'{kind}/{layer.name}'
+        dz, sw, h_next = _layer_backward_check(dev, layer, r, h, g, contract, what, second_path=name == 'QEinsumDenseBatchnorm')
+        # kernel: the straight-through gradient of the quantized kernel is the contraction's weight gradient
+        named = [('kernel', layer._kernel, r.kernel), ('bias', layer.bias, r.bias), ('iq._f', layer.iq.quantizer._f, r.iq.quantizer._f),
+                 ('kq._b', layer.kq.quantizer._b, r.kq.quantizer._b), ('kq._i', layer.kq.quantizer._i, r.kq.quantizer._i),
+                 ('bq._b', layer.bq.quantizer._b, r.bq.quantizer._b), ('bq._i', layer.bq.quantizer._i, r.bq.quantizer._i)]
+        if name == 'QEinsumDenseBatchnorm':
+            named.append(('gamma', layer.bn_gamma, r.gamma))
+        for vname, p, rv in named:
+            if rv.grad is None:
+                assert p.grad is None or float(p.grad.abs().max()) == 0.0, f'{what}: {vname} should have no gradient'
+                continue
+            assert p.grad is not None, f'{what}: {vname} has no gradient'
+            if vname == 'kernel' and name != 'QEinsumDenseBatchnorm':
+                _close_scaled(p.grad, rv.grad, sw + 1e-9, f'{what}: d{vname}')
+            elif vname == 'bias' and name != 'QEinsumDenseBatchnorm':
+                red = tuple(range(dz.dim() - 1))
+                _close_scaled(p.grad, rv.grad, dz.abs().sum(dim=red) + 1e-9, f'{what}: d{vname}')
+            else:
+                _close_tensor(p.grad, rv.grad, f'{what}: d{vname}')
+        h = h_next  # continue from the oracle's activations
