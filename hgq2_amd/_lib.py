@@ -28,6 +28,8 @@ ROUND_MODES = {'TRN': TRN, 'RND': RND, 'RND_CONV': RND_CONV}
 OVERFLOW_MODES = {'WRAP': WRAP, 'SAT': SAT, 'SAT_SYM': SAT_SYM}
 
 ERRORS = {-1: 'HGQ_ERR_ARG', -2: 'HGQ_ERR_LAUNCH', -3: 'HGQ_ERR_UNSUPPORTED'}
+ERR_ARG, ERR_LAUNCH, ERR_UNSUPPORTED = -1, -2, -3
+STATIC_SCRATCH_FLOATS = 1 << 18  # HGQ_STATIC_SCRATCH_FLOATS of include/hgq_hip.h
 
 # name -> (restype, argtypes); exactly the declarations of include/hgq_hip.h
 SIGNATURES = {
@@ -70,6 +72,7 @@ SIGNATURES = {
     'hgq_sgd_update_multi': (c_int, [c_void_p, c_int, c_float, c_void_p]),
     'hgq_quantize_bwd_workspace': (c_int64, [c_int64, c_int64, c_int64]),
     'hgq_quantize_bwd_sliced': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    'hgq_quantize_bwd_static': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_fwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_quantize_bwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_mean_mid_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),

@@ -11,6 +11,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "hgq_device.h"
 #include "hgq_host.h"
 
@@ -829,6 +831,49 @@ extern "C" int hgq_quantize_bwd_sliced(const float *dy, const float *x, const vo
     int rc = check_launch("hgq_quantize_bwd_sliced");
     if (rc) return rc;
     return reduce_parts(workspace, (int)gy, di ? 2 * M : M, dfb, M, di, di ? M : 0, nullptr, 0, s);
+}
+
+// ------------------------------------------------------------------------------------------
+// hgq_quantize_bwd_sliced for callers that cannot allocate: the slices live in a file-scope device array.
+// Every GPU the library runs on holds its own copy of the array (HGQ_STATIC_SCRATCH_FLOATS * 4 bytes) until the
+// process ends.  In host code the array's NAME is only a handle for hipGetSymbolAddress: the device address is looked
+// up once per device and only that pointer is ever handed to a kernel.
+// ------------------------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[HGQ_STATIC_SCRATCH_FLOATS];
+
+#define HGQ_MAX_DEVICES 64
+static std::mutex g_scratch_mutex;
+static float *g_scratch_ptr[HGQ_MAX_DEVICES];  // per device: each GPU has the array at its own address
+
+static int static_scratch(float **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(HGQ_ERR_LAUNCH, "hgq_quantize_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= HGQ_MAX_DEVICES) return fail(HGQ_ERR_UNSUPPORTED, "hgq_quantize_bwd_static: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // with device `dev` current: its copy of the array
+        if (e != hipSuccess || !p) return fail(HGQ_ERR_LAUNCH, "hgq_quantize_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = (float *)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return HGQ_OK;
+}
+
+extern "C" int hgq_quantize_bwd_static(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx,
+                                       float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream) {
+    const int64_t need = hgq_quantize_bwd_workspace(n, bw_size, bw_inner);
+    if (need <= 0)
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_quantize_bwd_static: shape outside the per-column kernels (hgq_quantize_bwd_workspace returns 0 for it)");
+    if (need > (int64_t)HGQ_STATIC_SCRATCH_FLOATS)
+        return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_static: %lld floats of slices needed, the static scratch holds %lld; use hgq_quantize_bwd_sliced with a caller workspace",
+                    (long long)need, (long long)HGQ_STATIC_SCRATCH_FLOATS);
+    float *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc) return rc;
+    // every slice entry that the reduction reads is written whole by the kernel before: nothing to clear between calls
+    return hgq_quantize_bwd_sliced(dy, x, k, i, fb, dx, di, dfb, ws, n, bw_size, bw_inner, mode, stream);
 }
 
 extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,

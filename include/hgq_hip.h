@@ -109,6 +109,20 @@ int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, cons
                             float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
 
 /*
+ * hgq_quantize_bwd_sliced without a workspace argument.  This entry point has no counterpart in the reference.  It is
+ * for callers that cannot allocate device memory around the call: code running under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  The slices go to a device array that is part of the library's code object
+ * (HGQ_STATIC_SCRATCH_FLOATS floats = 1 MiB, held on every GPU the library runs on until the process ends); the call
+ * allocates and frees nothing.  Same arguments, results (bit for bit) and errors as hgq_quantize_bwd_sliced, plus
+ * HGQ_ERR_ARG when hgq_quantize_bwd_workspace(n, bw_size, bw_inner) exceeds HGQ_STATIC_SCRATCH_FLOATS.
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams or threads) race;
+ * calls on one stream are ordered.  Nothing needs clearing between calls: every slice entry read is written first.
+ */
+#define HGQ_STATIC_SCRATCH_FLOATS (1 << 18)
+int hgq_quantize_bwd_static(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
+                            float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
+
+/*
  * Many quantizers with per-element bit-widths (bw_size == n, no trackers) in one launch each way: the kernel and bias
  * quantizers of a model (src/hgq/layers/core/dense.py:72-79 `self.kq(self._kernel)`, `self.bq(self.bias)` and the same
  * in the other layers) depend on the variables only, so all of them can run before the first layer and their gradients
