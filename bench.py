@@ -22,12 +22,23 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of the 4 Mi-element quantizer kernels from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# counters, each scaled by what the same counter reads for a 16 MiB device copy (FETCH_SIZE x 1.997,
-# WRITE_SIZE x 1.000); summary and commands in profiles/quantizer_4Mi_hbm_counters.md
-TRAFFIC_BYTES = {'quant_fwd_1d': 50.3e6, 'quant_bwd_1d': 100.6e6}
+# counters, each scaled by what the same counter reads for the plain streaming kernel of known size
+# (hgq_stream_probe); summary and commands in profiles/quantizer_4Mi_hbm_counters.md
+TRAFFIC_BYTES = {'quant_fwd': 50.34e6, 'quant_bwd': 100.67e6, 'quant_fwd_sat': 83.89e6, 'quant_bwd_sat': 134.22e6}
 BATCH = 16384
 DIMS = (16, 64, 32, 32, 5)
 QN = 4 * 1024 * 1024  # standalone quantizer case: 4 Mi fp32 elements
+
+
+def _cpu_threads():
+    """Threads the CPU baseline runs on: the cores this process may use (its affinity mask; a GPU box hands a
+    one-GPU job a share of the host, and OMP_NUM_THREADS names that share), not every core the host has."""
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = os.cpu_count() or 1
+    share = int(os.environ.get('OMP_NUM_THREADS', '0') or 0)
+    return max(1, min(allowed, share) if share > 0 else allowed)
 
 
 def _events_ms(fn, iters):
@@ -43,10 +54,12 @@ def _events_ms(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
-def quantizer_roofline(iters=200, with_copy=False):
-    """Standalone KIF quantizer, RND/WRAP, per-element k, i, f, training forward + surrogate
-    backward, launched straight through the C ABI on torch's current stream and timed with HIP
-    events on that stream."""
+def quantizer_roofline(iters=200):
+    """Standalone KIF quantizer, RND rounding, per-element k, i, f, training forward + surrogate backward at 4 Mi
+    elements, launched straight through the C ABI on torch's current stream and timed with HIP events on that stream.
+    Two overflow modes: WRAP (the benchmark configuration; its training branch only rounds, so k and i never cross HBM)
+    and SAT (every operand is live).  Next to them a plain streaming kernel (``hgq_stream_probe``) with the same number
+    of bytes and a comparable read / write mix: what this memory system gives a kernel that does nothing else."""
     import torch
 
     from hgq2_amd import _lib
@@ -54,7 +67,7 @@ def quantizer_roofline(iters=200, with_copy=False):
     lib = _lib.load()
     dev = torch.device('cuda:0')
     g = torch.Generator().manual_seed(0)
-    # The MI355X has a 256 MB memory-side cache; one launch touches 80-128 MB, so re-running on
+    # The MI355X has a 256 MB memory-side cache; one launch touches 50-134 MB, so re-running on
     # one buffer set would be served from that cache.  Rotate over enough distinct sets (> 1 GB in
     # total) that every launch streams from HBM.
     n_sets = 10
@@ -66,44 +79,43 @@ def quantizer_roofline(iters=200, with_copy=False):
         f = torch.randint(0, 9, (QN,), generator=g).float().to(dev)
         dy = torch.randn(QN, generator=g).to(dev)
         sets.append((x, k, i, f, dy) + tuple(torch.empty(QN, device=dev) for _ in range(4)))
-    mode = _lib.mode_bits('RND', 'WRAP', training=True)
     s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
     state = {'n': 0}
-    # argument tuples are built once per buffer set: a launch is then one foreign call, so the host
-    # keeps ahead of a 10-20 us kernel and the event-to-event time is kernel time
-    fwd_calls = [(p(x), p(k), p(i), p(f), p(y), None, None, QN, QN, 1, mode, s) for x, k, i, f, dy, y, dx, di, df in sets]
-    bwd_calls = [(p(dy), p(x), p(k), p(i), p(f), p(dx), p(di), p(df), QN, QN, 1, mode, s) for x, k, i, f, dy, y, dx, di, df in sets]
-    q_fwd, q_bwd = lib.hgq_quantize_fwd, lib.hgq_quantize_bwd
 
-    def fwd():
-        state['n'] += 1
-        if q_fwd(*fwd_calls[state['n'] % n_sets]):
-            raise RuntimeError('hgq_quantize_fwd failed')
-
-    def bwd():
-        state['n'] += 1
-        if q_bwd(*bwd_calls[state['n'] % n_sets]):
-            raise RuntimeError('hgq_quantize_bwd failed')
-
-    for _ in range(10):
-        fwd(), bwd()
-    t_fwd = _events_ms(fwd, iters)
-    t_bwd = _events_ms(bwd, iters)
-    out = {}
-    if with_copy:
-        # calibration for hardware counters: a plain device copy of known size (16 MiB read + 16 MiB written)
-        def cp():
-            x, k, i, f, dy, y, dx, di, df = sets[state['n'] % n_sets]
+    def timed(fn, calls):
+        # argument tuples are built once per buffer set: a launch is then one foreign call, so the host
+        # keeps ahead of a 10-20 us kernel and the event-to-event time is kernel time
+        def one():
             state['n'] += 1
-            y.copy_(x)
+            if fn(*calls[state['n'] % n_sets]):
+                raise RuntimeError(lib.hgq_last_error().decode())
 
-        t_cp = _events_ms(cp, iters)
-        out['copy_4Mi_f32'] = {'ms': t_cp, 'bytes': 8 * QN, 'GBps': 8 * QN / (t_cp * 1e-3) / 1e9, 'frac': 8 * QN / (t_cp * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    for name, ms, bpe in (('quant_fwd_1d', t_fwd, 20), ('quant_bwd_1d', t_bwd, 32)):
-        gbs = bpe * QN / (ms * 1e-3) / 1e9
-        out[name] = {'ms': ms, 'bytes': bpe * QN, 'GBps': gbs, 'frac': gbs / HBM_PEAK_GBS, 'traffic': TRAFFIC_BYTES[name],
-                     'traffic_GBps': TRAFFIC_BYTES[name] / (ms * 1e-3) / 1e9}
+        for _ in range(10):
+            one()
+        return _events_ms(one, iters)
+
+    out = {}
+    for om in ('WRAP', 'SAT'):
+        mode = _lib.mode_bits('RND', om, training=True)
+        fwd_calls = [(p(x), p(k), p(i), p(f), p(y), None, None, QN, QN, 1, mode, s) for x, k, i, f, dy, y, dx, di, df in sets]
+        bwd_calls = [(p(dy), p(x), p(k), p(i), p(f), p(dx), p(di), p(df), QN, QN, 1, mode, s) for x, k, i, f, dy, y, dx, di, df in sets]
+        t_fwd = timed(lib.hgq_quantize_fwd, fwd_calls)
+        t_bwd = timed(lib.hgq_quantize_bwd, bwd_calls)
+        suffix = '' if om == 'WRAP' else '_sat'
+        for name, ms, bpe in (('quant_fwd' + suffix, t_fwd, 20), ('quant_bwd' + suffix, t_bwd, 32)):
+            traffic = TRAFFIC_BYTES[name]
+            out[name] = {'ms': ms, 'operand_bytes': bpe * QN, 'operand_GBps': bpe * QN / (ms * 1e-3) / 1e9,
+                         'traffic': traffic, 'GBps': traffic / (ms * 1e-3) / 1e9, 'frac': traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                         'frac_operands': bpe * QN / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    # plain streaming kernels: 2 arrays read + 1 written (the bytes of the WRAP forward), 3 + 3 (the WRAP backward)
+    for name, nr, nw in (('stream_2r1w', 2, 1), ('stream_3r3w', 3, 3), ('stream_1r1w', 1, 1)):
+        calls = [(p(x), p(f), p(dy), p(y), p(dx), p(df), nr, nw, QN, s) for x, k, i, f, dy, y, dx, di, df in sets]
+        ms = timed(lib.hgq_stream_probe, calls)
+        nbytes = 4 * (nr + nw) * QN
+        out[name] = {'ms': ms, 'traffic': nbytes, 'GBps': nbytes / (ms * 1e-3) / 1e9, 'frac': nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    out['quant_fwd']['of_plain_stream'] = out['stream_2r1w']['ms'] / out['quant_fwd']['ms']
+    out['quant_bwd']['of_plain_stream'] = out['stream_3r3w']['ms'] / out['quant_bwd']['ms']
     return out
 
 
@@ -169,7 +181,7 @@ def softmax_roofline(iters=50, shape=(2048, 4, 64, 64), scaler=0.25):
     return out
 
 
-def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False):
+def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False, cpu_budget_s=15.0):
     """One training step (forward, backward, SGD update) of the configurations other than the headline one, at their full
     sizes: 'particle' (QEinsumDenseBatchnorm per-particle network, batch 4096 x 64 x 16), 'conv'
     (QConv2D stack on 28 x 28 x 1, batch 1024), 'mha' (QMultiHeadAttention, batch 2048 x 64 x 64)."""
@@ -246,7 +258,7 @@ def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False):
     out = {'workload': name, 'batch': batch, 'ms_per_step': ms, 'samples_per_s': batch / ms * 1e3, 'loss': float(loss),
            'launch': 'hip-graph replay' if graph else 'eager'}
     if cpu:
-        out['cpu_baseline'] = _config_cpu_baseline(name, model, x, labels if name != 'mha' else None, batch)
+        out['cpu_baseline'] = _config_cpu_baseline(name, model, x, labels if name != 'mha' else None, batch, budget_s=cpu_budget_s)
         out['gpu_over_cpu'] = out['samples_per_s'] / out['cpu_baseline']['value']
     return out
 
@@ -258,9 +270,9 @@ def _config_cpu_baseline(name, model, x, labels, batch, budget_s=15.0):
     import torch.nn.functional as F
 
     from hgq2_amd.utils import models
-    from tests import twin
+    from oracle import twin
 
-    cores = min(os.cpu_count() or 1, 16)
+    cores = _cpu_threads()
     torch.set_num_threads(cores)
     xc = x.cpu()
     if name == 'mha':
@@ -303,7 +315,7 @@ def _config_cpu_baseline(name, model, x, labels, batch, budget_s=15.0):
         el = time.perf_counter() - t0
         if el > budget_s or n >= 20:
             break
-    return {'value': batch * n / el, 'unit': 'samples/s', 'cores': cores, 'kind': 'port',
+    return {'value': batch * n / el, 'unit': 'samples/s', 'cores': cores, 'host_cores': os.cpu_count(), 'kind': 'port',
             'sample': f'{n} forward+backward passes of the same model at batch {batch} (eager torch-CPU restatement of the reference path)'}
 
 
@@ -313,8 +325,7 @@ def cpu_baseline(budget_s=20.0):
 
     from oracle import hgq_ref as ref
 
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
+    cores = _cpu_threads()
     torch.set_num_threads(cores)
     g = torch.Generator().manual_seed(0)
     x = torch.randn(BATCH, DIMS[0], generator=g)
@@ -329,7 +340,7 @@ def cpu_baseline(budget_s=20.0):
         el = time.perf_counter() - t0
         if el > budget_s or n >= 200:
             break
-    return {'value': BATCH * n / el, 'unit': 'samples/s', 'cores': cores, 'kind': 'port',
+    return {'value': BATCH * n / el, 'unit': 'samples/s', 'cores': cores, 'host_cores': os.cpu_count(), 'kind': 'port',
             'sample': f'{n} training steps of the same MLP at batch {BATCH} (eager torch-CPU restatement of the reference path)'}
 
 
@@ -339,6 +350,7 @@ def main():
     ap.add_argument('--steps', type=int, default=300)
     ap.add_argument('--warmup', type=int, default=30)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-extras', action='store_true', help='headline and roofline only: skip the per-path and per-configuration timings')
     ap.add_argument('--roofline-only', action='store_true',
                     help='run only the standalone quantizer kernels and a plain copy of known size (for counter runs)')
     ap.add_argument('--config-step', choices=('particle', 'conv', 'mha'), default=None,
@@ -359,7 +371,7 @@ def main():
 
     if args.roofline_only:
         torch.cuda.set_device(0)
-        print(json.dumps({'quantizer_kernels': quantizer_roofline(iters=20, with_copy=True)}))
+        print(json.dumps({'quantizer_kernels': quantizer_roofline(iters=50)}))
         return
     if args.config_step:
         torch.cuda.set_device(0)
@@ -379,75 +391,108 @@ def main():
     g = torch.Generator().manual_seed(0)
     x = torch.randn(BATCH, DIMS[0], generator=g).to(dev)
     labels = torch.randint(0, DIMS[-1], (BATCH,), generator=g).to(dev)
-    torch.manual_seed(1)
-    model = qdense_mlp(DIMS, beta0=1e-5, device=dev)
-    opt = SGD(model.parameters(), lr=0.01, fold_regularizers=True)
 
-    if args.path == 'layers-eager':
-        def step():
-            opt.zero_grad()
-            loss = model_loss(model, ops.sparse_ce(model(x, training=True), labels), True)
-            loss.backward()
-            opt.step()
-            return loss
-    elif args.path == 'layers-graph':
-        step = GraphedTrainStep(model, ops.sparse_ce, opt, x, labels, warmup=3)
-    else:
+    def make_step(path):
+        """A fresh model (same seed) and one training step of it along `path`."""
+        torch.manual_seed(1)
+        model = qdense_mlp(DIMS, beta0=1e-5, device=dev)
+        opt = SGD(model.parameters(), lr=0.01, fold_regularizers=True)
+        if path == 'layers-eager':
+            def step():
+                opt.zero_grad()
+                loss = model_loss(model, ops.sparse_ce(model(x, training=True), labels), True)
+                loss.backward()
+                opt.step()
+                return loss
+            return step
+        if path == 'layers-graph':
+            return GraphedTrainStep(model, ops.sparse_ce, opt, x, labels, warmup=3)
         fused = FusedQDenseStack(model, lr=0.01)
-        if args.path == 'fused':
-            def step():
-                return fused.step(x, labels)
-        else:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                for _ in range(3):
-                    fused.step(x, labels)
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+        if path == 'fused':
+            return lambda: fused.step(x, labels)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
                 fused.step(x, labels)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fused.step(x, labels)
 
-            def step():
-                graph.replay()
-                return fused.loss
+        def step():
+            graph.replay()
+            return fused.loss
+        return step
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = step()
-    torch.cuda.synchronize()
-    el = time.perf_counter() - t0
+    def time_steps(step, steps, warmup):
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss = step()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, loss
+
+    # the headline: exactly `steps` timed steps after `warmup` untimed ones
+    step = make_step(args.path)
+    el, loss = time_steps(step, args.steps, args.warmup)
     ms_per_step = el / args.steps * 1e3
     value = BATCH * args.steps / el
 
-    qr = quantizer_roofline()
-    dom = qr['quant_bwd_1d']
-    roofline = {'bound': 'hbm', 'kernel': 'quant_bwd_1d', 'achieved': dom['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': dom['frac'], 'traffic': dom['traffic'], 'traffic_frac': dom['traffic_GBps'] / HBM_PEAK_GBS,
-                'workload': 'standalone kif quantizer RND/WRAP, 4 Mi fp32 elements, per-element k/i/f: backward, 32 B/elem '
-                            'algorithmic (dy, x, k, i, f in; dx, di, df out); the WRAP training branch needs neither k nor i, '
-                            'so 24 B/elem cross HBM (traffic)'}
+    labels_of = {'fused': 'whole-step kernels of a QDense stack with sparse CE and SGD, 3 launches (a special-case trainer)',
+                 'fused-graph': 'the same whole-step kernels replayed from a HIP graph',
+                 'layers-graph': 'the layer API: per-layer operators + autograd, the step replayed from a HIP graph',
+                 'layers-eager': 'the layer API: per-layer operators + autograd, eager launches (host-bound)'}
     out = {
         'metric': 'QDense MLP train samples/s @bs16384; quantizer HBM GB/s vs peak',
         'value': value, 'unit': 'samples/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': ms_per_step, 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32',
         'data': 'synthetic',
         'config': {'workload': 'QDense MLP 16-64-32-32-5 (ReLU hidden, linear out), batch 16384, kbi SAT_SYM weights, '
-                               'kif WRAP datalanes, EBOPs beta0=1e-5, sparse CE, one fwd+bwd+SGD step'
-                               + {'fused': ' (whole-step kernels, 3 launches)', 'fused-graph': ' (whole-step kernels, HIP-graph replay)',
-                                  'layers-graph': ' (per-layer operators + autograd, HIP-graph replay)',
-                                  'layers-eager': ' (per-layer operators + autograd, eager launches)'}[args.path]},
+                               'kif WRAP datalanes, EBOPs beta0=1e-5, sparse CE, one fwd+bwd+SGD step; path = ' + args.path
+                               + ': ' + labels_of[args.path]},
         'final_loss': float(loss),
-        'roofline': roofline,
-        'quantizer_kernels': qr,
     }
+    if not args.no_extras:
+        # every way the same step can be driven, each on a fresh model, over a few hundred steps
+        paths = {}
+        for path in ('fused', 'layers-graph', 'layers-eager'):
+            n_steps = max(args.steps, 300 if path != 'layers-eager' else 100)
+            el_p, _ = time_steps(make_step(path), n_steps, max(args.warmup, 10))
+            paths[path.replace('-', '_')] = {'samples_per_s': BATCH * n_steps / el_p, 'ms_per_step': el_p / n_steps * 1e3, 'steps': n_steps,
+                                             'what': labels_of[path]}
+        out['paths'] = paths
+
+    qr = quantizer_roofline()
+    dom = qr['quant_bwd']
+    out['roofline'] = {
+        'bound': 'hbm', 'kernel': 'quant_bwd_pe<RND, WRAP>', 'achieved': dom['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+        'frac': dom['frac'], 'traffic': dom['traffic'], 'frac_operands': dom['frac_operands'],
+        'of_plain_stream': dom['of_plain_stream'],
+        'workload': 'standalone kif quantizer RND/WRAP, 4 Mi fp32 elements, per-element k/i/f: backward.  achieved = HBM bytes '
+                    'per launch by the traffic counters (24 B/elem: dy, x, f in; dx, di, df out - the WRAP training branch '
+                    'reads neither k nor i) / HIP-event time; frac_operands prices the same time at all 32 B/elem of operands; '
+                    'of_plain_stream = time of a plain 3-read 3-write streaming kernel of the same bytes / this kernel\'s time'}
+    sat = qr['quant_bwd_sat']
+    out['roofline_all_operands_live'] = {
+        'bound': 'hbm', 'kernel': 'quant_bwd_pe<RND, SAT>', 'achieved': sat['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+        'frac': sat['frac'], 'traffic': sat['traffic'],
+        'workload': 'the same quantizer with overflow mode SAT: every operand is live, 32 B/elem cross HBM (forward: 20 B/elem, '
+                    'see quantizer_kernels.quant_fwd_sat)'}
+    out['quantizer_kernels'] = qr
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()
         out['gpu_over_cpu'] = value / out['cpu_baseline']['value']
+        if 'paths' in out:
+            for v in out['paths'].values():
+                v['gpu_over_cpu'] = v['samples_per_s'] / out['cpu_baseline']['value']
+    if not args.no_extras:
+        # one training step of the other configurations at full size (HIP-graph replay), each with its CPU baseline
+        out['config_steps'] = {name: config_step_time(name, steps=20, graph=True, cpu=not args.no_cpu_baseline, cpu_budget_s=6.0)
+                               for name in ('particle', 'conv', 'mha')}
     print(json.dumps(out))
 
 

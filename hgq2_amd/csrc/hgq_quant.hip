@@ -208,6 +208,69 @@ __global__ __launch_bounds__(Q1D_BS) void quant_bwd_1d(const float *__restrict__
 }
 
 // ------------------------------------------------------------------------------------------
+// Per-element bit-widths, fp32 k, no trackers: the standalone-quantizer case.  One 128-bit vector per operand
+// per thread and nothing else: the training flag and the set of live operands are template arguments, the
+// raw variables are always rounded (the identity on integer-valued ones), KIF / KBI is a select - no branch
+// sits between the loads.  With one vector per thread the waves of a launch run in step (all load, all
+// compute, all store), so every vector instruction saved here is time saved: at 4 Mi elements the kernel runs
+// two such rounds and ~100 instructions cost about a microsecond of a ten-microsecond launch.
+// LIVE bit 0: `i` is read; bit 1: `k` is read.  A WRAP quantizer in training mode only rounds, so k is dead
+// there, and i as well unless f = b - i.
+// ------------------------------------------------------------------------------------------
+template <int LIVE>
+__device__ __forceinline__ KIF pe_kif(const f32x4 &kv, const f32x4 &iv, const f32x4 &fv, int c, bool kbi) {
+    KIF p;
+    p.k = (LIVE & 2) ? kv[c] : 1.0f;
+    p.i = (LIVE & 1) ? rintf(iv[c]) : 0.0f;
+    const float fb = rintf(fv[c]);
+    p.f = kbi ? __fsub_rn(fb, p.i) : fb;
+    return p;
+}
+
+template <int RM, int OM, bool TRAIN, int LIVE>
+__global__ __launch_bounds__(Q1D_BS) void quant_fwd_pe(const f32x4 *__restrict__ x, const f32x4 *__restrict__ k,
+                                                       const f32x4 *__restrict__ i, const f32x4 *__restrict__ fb,
+                                                       f32x4 *__restrict__ y, int64_t nvec, int kbi) {
+    const int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x;
+    if (v >= nvec) return;
+    const f32x4 xv = __builtin_nontemporal_load(x + v);
+    const f32x4 fv = __builtin_nontemporal_load(fb + v);
+    f32x4 iv = {0.f, 0.f, 0.f, 0.f}, kv = {0.f, 0.f, 0.f, 0.f};
+    if (LIVE & 1) iv = __builtin_nontemporal_load(i + v);
+    if (LIVE & 2) kv = __builtin_nontemporal_load(k + v);
+    f32x4 yv;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) yv[c] = quantize<RM, OM>(xv[c], pe_kif<LIVE>(kv, iv, fv, c, kbi != 0), TRAIN);
+    __builtin_nontemporal_store(yv, y + v);
+}
+
+template <int RM, int OM, int LIVE>
+__global__ __launch_bounds__(Q1D_BS) void quant_bwd_pe(const f32x4 *__restrict__ dy, const f32x4 *__restrict__ x,
+                                                       const f32x4 *__restrict__ k, const f32x4 *__restrict__ i,
+                                                       const f32x4 *__restrict__ fb, f32x4 *__restrict__ dx,
+                                                       f32x4 *__restrict__ di, f32x4 *__restrict__ dfb, int64_t nvec, int kbi) {
+    const int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x;
+    if (v >= nvec) return;
+    const f32x4 gv = __builtin_nontemporal_load(dy + v);
+    const f32x4 xv = __builtin_nontemporal_load(x + v);
+    const f32x4 fv = __builtin_nontemporal_load(fb + v);
+    f32x4 iv = {0.f, 0.f, 0.f, 0.f}, kv = {0.f, 0.f, 0.f, 0.f};
+    if (LIVE & 1) iv = __builtin_nontemporal_load(i + v);
+    if (LIVE & 2) kv = __builtin_nontemporal_load(k + v);
+    f32x4 gx, gi, gf;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float a, b, d;
+        quantize_grad<RM, OM>(xv[c], gv[c], pe_kif<LIVE>(kv, iv, fv, c, kbi != 0), a, b, d);
+        if (kbi) b -= d;  // f = b - i
+        gx[c] = a, gi[c] = b, gf[c] = d;
+    }
+    if (dx) __builtin_nontemporal_store(gx, dx + v);
+    if (di) __builtin_nontemporal_store(gi, di + v);
+    if (dfb) __builtin_nontemporal_store(gf, dfb + v);
+}
+
+// ------------------------------------------------------------------------------------------
 // 2-D kernels: x = [rows, M], one bit-width entry per column
 // thread (tx, ty): tx walks column groups of VEC, ty walks rows; TX is a power of two <= 64
 // ------------------------------------------------------------------------------------------
@@ -516,6 +579,26 @@ __global__ __launch_bounds__(256) void quant_bwd_multi_kernel(QuantGradBatch b) 
 }
 
 // ------------------------------------------------------------------------------------------
+// Measurement aid: a plain streaming kernel with a chosen mix of read and written arrays (one 128-bit
+// non-temporal access per array per thread, like the per-element quantizer kernels, and no arithmetic to speak
+// of).  It calibrates the hardware traffic counters (known bytes) and gives the bandwidth this memory system
+// yields for a given read / write mix and size, which is the ceiling the quantizer kernels are measured against.
+// ------------------------------------------------------------------------------------------
+template <int NR, int NW>
+__global__ __launch_bounds__(Q1D_BS) void stream_probe_kernel(const f32x4 *__restrict__ a, const f32x4 *__restrict__ b,
+                                                              const f32x4 *__restrict__ c, f32x4 *__restrict__ o0,
+                                                              f32x4 *__restrict__ o1, f32x4 *__restrict__ o2, int64_t nvec) {
+    const int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x;
+    if (v >= nvec) return;
+    f32x4 t = __builtin_nontemporal_load(a + v);
+    if (NR > 1) t += __builtin_nontemporal_load(b + v);
+    if (NR > 2) t += __builtin_nontemporal_load(c + v);
+    __builtin_nontemporal_store(t, o0 + v);
+    if (NW > 1) __builtin_nontemporal_store(t * 2.0f, o1 + v);
+    if (NW > 2) __builtin_nontemporal_store(t * 3.0f, o2 + v);
+}
+
+// ------------------------------------------------------------------------------------------
 // integer-bit tracking
 // ------------------------------------------------------------------------------------------
 // 1024 threads = 64 entries x 16 slice groups: the abs-max / any-negative trackers arrive as
@@ -604,6 +687,36 @@ using namespace hgq;
 extern "C" int hgq_version(void) { return 1; }
 extern "C" const char *hgq_last_error(void) { return g_err; }
 
+extern "C" int hgq_stream_probe(const float *a, const float *b, const float *c, float *o0, float *o1, float *o2, int n_read,
+                                int n_write, int64_t n, void *stream) {
+    if (n < 4 || n % 4 != 0 || n_read < 1 || n_read > 3 || n_write < 1 || n_write > 3)
+        return fail(HGQ_ERR_ARG, "hgq_stream_probe: n must be a positive multiple of 4, 1..3 arrays each way");
+    const float *in[3] = {a, b, c};
+    float *out[3] = {o0, o1, o2};
+    for (int t = 0; t < 3; ++t)
+        if ((t < n_read && (!in[t] || !aligned16(in[t]))) || (t < n_write && (!out[t] || !aligned16(out[t]))))
+            return fail(HGQ_ERR_ARG, "hgq_stream_probe: arrays must be non-null and 16-byte aligned");
+    const int64_t nvec = n / 4, grid = (nvec + Q1D_BS - 1) / Q1D_BS;
+    if (grid >= (1ll << 31)) return fail(HGQ_ERR_ARG, "hgq_stream_probe: n too large");
+    hipStream_t s = (hipStream_t)stream;
+#define HGQ_PROBE(NRV, NWV)                                                                                                    \
+    hipLaunchKernelGGL((stream_probe_kernel<NRV, NWV>), dim3((unsigned)grid), dim3(Q1D_BS), 0, s, (const f32x4 *)a, (const f32x4 *)b, \
+                       (const f32x4 *)c, (f32x4 *)o0, (f32x4 *)o1, (f32x4 *)o2, nvec)
+    switch (n_read * 4 + n_write) {
+        case 1 * 4 + 1: HGQ_PROBE(1, 1); break;
+        case 1 * 4 + 2: HGQ_PROBE(1, 2); break;
+        case 1 * 4 + 3: HGQ_PROBE(1, 3); break;
+        case 2 * 4 + 1: HGQ_PROBE(2, 1); break;
+        case 2 * 4 + 2: HGQ_PROBE(2, 2); break;
+        case 2 * 4 + 3: HGQ_PROBE(2, 3); break;
+        case 3 * 4 + 1: HGQ_PROBE(3, 1); break;
+        case 3 * 4 + 2: HGQ_PROBE(3, 2); break;
+        default: HGQ_PROBE(3, 3); break;
+    }
+#undef HGQ_PROBE
+    return check_launch("hgq_stream_probe");
+}
+
 extern "C" int hgq_fill_u32(uint32_t *p, uint32_t value, int64_t n, void *stream) {
     if (n < 0 || (n > 0 && !p)) return fail(HGQ_ERR_ARG, "hgq_fill_u32: bad arguments");
     return fill_u32(p, value, n, (hipStream_t)stream);
@@ -625,6 +738,14 @@ static bool cols_grid(int64_t rows, int64_t M, int batch_rows, int64_t gx, int64
     gy = (rows + rows_per_wg - 1) / rows_per_wg;
     return true;
 }
+
+// launches of the lean per-element kernels (inside HGQ_DISPATCH_RM_OM: RM, OM, and the locals of the entry point)
+#define HGQ_FWD_PE(TRAINV, LIVEV)                                                                                                     \
+    hipLaunchKernelGGL((quant_fwd_pe<RM, OM, TRAINV, LIVEV>), dim3((unsigned)pe_grid), dim3(Q1D_BS), 0, s, (const f32x4 *)x, (const f32x4 *)k, \
+                       (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)y, n4, (int)m.kbi)
+#define HGQ_BWD_PE(LIVEV)                                                                                                              \
+    hipLaunchKernelGGL((quant_bwd_pe<RM, OM, LIVEV>), dim3((unsigned)pe_grid), dim3(Q1D_BS), 0, s, (const f32x4 *)dy, (const f32x4 *)x,      \
+                       (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)dx, (f32x4 *)di, (f32x4 *)dfb, n4, (int)m.kbi)
 
 // launch of the per-column forward kernel: vector width and training flag as template arguments
 #define HGQ_FWD_COLS_1(VECV, TRAINV, SLICED)                                                                                       \
@@ -661,8 +782,21 @@ extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, c
                            (!amax || aligned16(amax)) && (!anyneg || aligned16(anyneg));
         const int64_t n4 = vec ? (n / 4) : 0;
         const int64_t tail0 = n4 * 4, tail = n - tail0;
+        // the lean per-element kernel: no trackers, and k either dead or stored as fp32
+        const bool k_dead = m.overflow_mode == HGQ_WRAP && m.training;
+        const int64_t pe_grid = (n4 + Q1D_BS - 1) / Q1D_BS;
+        const bool lean = !shared && n4 > 0 && !amax && !anyneg && !m.track_input && (k_dead || !m.k_u8) && pe_grid < (1ll << 31);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
-            if (n4 > 0) {
+            if (lean) {
+                if (OM == HGQ_WRAP && m.training) {
+                    if (m.kbi) HGQ_FWD_PE(true, 1);
+                    else HGQ_FWD_PE(true, 0);
+                } else if (m.training) {
+                    HGQ_FWD_PE(true, 3);
+                } else {
+                    HGQ_FWD_PE(false, 3);
+                }
+            } else if (n4 > 0) {
                 const int grid = persistent_grid((n4 + Q1D_BS - 1) / Q1D_BS, 16);
                 if (shared)
                     hipLaunchKernelGGL((quant_fwd_1d<RM, OM, 4, true>), dim3(grid), dim3(Q1D_BS), 0, s, x, k, i, fb, y, amax, anyneg, n4, mode);
@@ -899,8 +1033,18 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
                            (!di || aligned16(di)) && (!dfb || aligned16(dfb));
         const int64_t n4 = vec ? (n / 4) : 0;
         const int64_t tail0 = n4 * 4, tail = n - tail0;
+        const bool k_dead = m.overflow_mode == HGQ_WRAP;  // the WRAP surrogate gradient only rounds
+        const int64_t pe_grid = (n4 + Q1D_BS - 1) / Q1D_BS;
+        const bool lean = !shared && n4 > 0 && (k_dead || !m.k_u8) && pe_grid < (1ll << 31);
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
-            if (n4 > 0) {
+            if (lean) {
+                if (OM == HGQ_WRAP) {
+                    if (m.kbi) HGQ_BWD_PE(1);
+                    else HGQ_BWD_PE(0);
+                } else {
+                    HGQ_BWD_PE(3);
+                }
+            } else if (n4 > 0) {
                 const int grid = persistent_grid((n4 + Q1D_BS - 1) / Q1D_BS, 16);
                 if (shared)
                     hipLaunchKernelGGL((quant_bwd_1d<RM, OM, 4, true>), dim3(grid), dim3(Q1D_BS), 0, s, dy, x, k, i, fb, dx, di, dfb, n4, mode);

@@ -109,6 +109,15 @@ int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, cons
                             float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
 
 /*
+ * Measurement aid (no counterpart in the reference): o_j[e] = (j + 1) * (a[e] (+ b[e]) (+ c[e])) for the first n_write
+ * outputs and n_read inputs, one 128-bit non-temporal access per array per thread.  4 * (n_read + n_write) * n bytes
+ * cross HBM per launch and nothing else: used to scale the hardware traffic counters and as the bandwidth a plain
+ * streaming kernel of a given read / write mix reaches at a given size.  n a multiple of 4, arrays 16-byte aligned.
+ */
+int hgq_stream_probe(const float *a, const float *b, const float *c, float *o0, float *o1, float *o2, int n_read, int n_write,
+                     int64_t n, void *stream);
+
+/*
  * hgq_quantize_bwd_sliced without a workspace argument.  This entry point has no counterpart in the reference.  It is
  * for callers that cannot allocate device memory around the call: code running under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  The slices go to a device array that is part of the library's code object

@@ -16,4 +16,6 @@ Modules
                   only to pin ``fixed_point`` (it shares no code with it).
 ``hgq_ref``       eager torch-CPU restatement of the reference's own Python
                   (quantizer classes, QDense, QEinsumDense, ..., EBOPs), autograd backward.
+``twin``          builds the ``hgq_ref`` twin of a product layer (same configuration, same variable
+                  values) for the parity tests and the ``cpu_baseline`` timings.
 """

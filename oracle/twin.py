@@ -2,7 +2,7 @@
 
 import torch
 
-from oracle import hgq_ref as ref
+from . import hgq_ref as ref
 
 
 def _constraint(c):

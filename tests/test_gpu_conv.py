@@ -102,7 +102,7 @@ def test_wide_dense_layer_matches_oracle(dev):
     """QDense 3872 -> 10 (the classifier of the image configuration): beyond the fused dense
     kernels, so the contraction runs in the 1 x 1 implicit-GEMM kernels."""
     from hgq2_amd.layers import QDense
-    from tests import twin
+    from oracle import twin
     from tests.test_gpu_more_layers import _compare_step, _perturb, readme_scopes
 
     g = torch.Generator().manual_seed(9)
@@ -137,7 +137,7 @@ def test_pooling_layers_match_oracle(dev, mode, case):
     """QMaxPooling2D / QAveragePooling2D: values, EBOPs, tracked bits and gradients (incl. where the
     gradient of a tied maximum goes: quantized ReLU-like inputs tie often) against the oracle twin."""
     from hgq2_amd.layers import QAveragePooling2D, QMaxPooling2D
-    from tests import twin
+    from oracle import twin
     from tests.test_gpu_more_layers import _compare_step, _perturb, readme_scopes
 
     B, H, W, C, pool, strides, padding = case

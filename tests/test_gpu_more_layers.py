@@ -5,7 +5,7 @@ forward values, the loss terms, state updates, and the gradients of every traina
 import pytest
 import torch
 
-from tests import twin
+from oracle import twin
 
 pytestmark = pytest.mark.gpu
 RTOL = 1e-5

@@ -15,7 +15,7 @@ import torch
 
 from oracle import fixed_point as ofp
 from oracle import hgq_ref as ref
-from tests import twin
+from oracle import twin
 
 pytestmark = pytest.mark.gpu
 RTOL = 1e-5

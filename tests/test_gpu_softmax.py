@@ -10,7 +10,7 @@
 import pytest
 import torch
 
-from tests import twin
+from oracle import twin
 from tests.test_gpu_more_layers import _close, _compare_step, readme_scopes
 
 pytestmark = pytest.mark.gpu
