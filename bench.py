@@ -223,7 +223,7 @@ def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False, cpu_budge
         # bit-width constraints folded into the update kernel
         opt.zero_grad()
         loss = model_loss(model, loss_fn(model(x, training=True)), True)
-        loss.backward()
+        opt.backward(loss)
         opt.step()
         return loss.detach()
 
@@ -401,7 +401,7 @@ def main():
             def step():
                 opt.zero_grad()
                 loss = model_loss(model, ops.sparse_ce(model(x, training=True), labels), True)
-                loss.backward()
+                opt.backward(loss)
                 opt.step()
                 return loss
             return step

@@ -385,8 +385,15 @@ struct SgdBatch {
 // grid.y = variable, grid.x strides over its elements; the descriptors travel as a kernel argument
 __global__ __launch_bounds__(256) void sgd_multi_kernel(SgdBatch b, float lr) {
     const hgq_sgd_item it = b.item[blockIdx.y];
+    float sc[HGQ_SGD_SIDES];
+#pragma unroll
+    for (int s = 0; s < HGQ_SGD_SIDES; ++s) sc[s] = (it.side[s] && it.side_scale[s]) ? it.side_scale[s][0] : 1.0f;
     for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < it.n; t += (int64_t)gridDim.x * 256) {
-        const float v = __fsub_rn(it.w[t], __fmul_rn(lr, __fadd_rn(it.g[t], it.l1)));
+        float g = it.g ? it.g[t] : 0.0f;
+#pragma unroll
+        for (int s = 0; s < HGQ_SGD_SIDES; ++s)
+            if (it.side[s]) g = __fadd_rn(g, __fmul_rn(sc[s], it.side[s][t]));
+        const float v = __fsub_rn(it.w[t], __fmul_rn(lr, __fadd_rn(g, it.l1)));
         it.w[t] = fminf(fmaxf(v, it.lo), it.hi);
     }
 }
@@ -469,7 +476,9 @@ extern "C" int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float 
         int64_t max_n = 0;
         for (int t = 0; t < nb; ++t) {
             b.item[t] = items[base + t];
-            if (b.item[t].n < 0 || (b.item[t].n > 0 && (!b.item[t].w || !b.item[t].g)))
+            bool any = b.item[t].g != nullptr;
+            for (int sd = 0; sd < HGQ_SGD_SIDES; ++sd) any = any || b.item[t].side[sd] != nullptr;
+            if (b.item[t].n < 0 || (b.item[t].n > 0 && (!b.item[t].w || !any)))
                 return fail(HGQ_ERR_ARG, "hgq_sgd_update_multi: bad item %d", base + t);
             if (b.item[t].n > max_n) max_n = b.item[t].n;
         }

@@ -124,5 +124,6 @@ def dense_ebops_term(layer, iq, kq, bq, K, N, scale, bias_size, deferred):
         qi._k.view(-1), qi._i.view(-1), qi._third().view(-1), qk._k.view(-1), qk._b.view(-1),
         qb._k.view(-1) if qb is not None else None, qb._b.view(-1) if qb is not None else None, P, K, N,
         scale * layer.ebops_factor, bias_size, qi._mode(True), qk._mode(True), qb._mode(True) if qb is not None else 0,
-        amax=amax, decay=decay, beta=layer._beta, ebops_var=layer._ebops.view(torch.int32))
+        amax=amax, decay=decay, beta=layer._beta, ebops_var=layer._ebops.view(torch.int32),
+        owners=(qi._i, qi._third(), qk._b, qb._b if qb is not None else None))
     return term

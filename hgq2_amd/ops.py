@@ -257,21 +257,40 @@ def sgd_update_op(w: Tensor, g: Tensor, lr: float, l1: float, lo: float, hi: flo
     _lib.check(rc, 'hgq_sgd_update')
 
 
+SGD_SIDES = 3
+
+
 class _SgdItem(ctypes.Structure):
     _fields_ = [('w', ctypes.c_void_p), ('g', ctypes.c_void_p), ('n', ctypes.c_int64), ('l1', ctypes.c_float),
-                ('lo', ctypes.c_float), ('hi', ctypes.c_float)]
+                ('lo', ctypes.c_float), ('hi', ctypes.c_float), ('side', ctypes.c_void_p * SGD_SIDES),
+                ('side_scale', ctypes.c_void_p * SGD_SIDES)]
 
 
 @torch.library.custom_op('hgq::sgd_update_multi', mutates_args=('ws',))
 def sgd_update_multi_op(ws: Sequence[Tensor], gs: Sequence[Tensor], l1: Sequence[float], lo: Sequence[float],
-                        hi: Sequence[float], lr: float) -> None:
+                        hi: Sequence[float], lr: float, sides: Sequence[Tensor], side_scales: Sequence[Tensor]) -> None:
+    """``gs[t]`` empty: no plain gradient.  ``sides`` / ``side_scales``: SGD_SIDES entries per variable (empty = absent;
+    an absent scale means 1)."""
     n = len(ws)
     _need(len(gs) == n and len(l1) == n and len(lo) == n and len(hi) == n, 'per-variable lists differ in length')
+    _need(len(sides) == SGD_SIDES * n and len(side_scales) == SGD_SIDES * n, 'side-gradient lists must hold SGD_SIDES entries per variable')
     items = (_SgdItem * n)()
     for t, (w, g) in enumerate(zip(ws, gs)):
-        _check_f32('w', w), _check_f32('g', g)
-        _need(w.numel() == g.numel(), 'gradient size mismatch')
-        items[t] = _SgdItem(w.data_ptr(), g.data_ptr(), w.numel(), l1[t], lo[t], hi[t])
+        _check_f32('w', w)
+        if g.numel():
+            _check_f32('g', g)
+            _need(w.numel() == g.numel(), 'gradient size mismatch')
+        it = _SgdItem(w.data_ptr(), g.data_ptr() if g.numel() else None, w.numel(), l1[t], lo[t], hi[t])
+        for s in range(SGD_SIDES):
+            sd, sc = sides[SGD_SIDES * t + s], side_scales[SGD_SIDES * t + s]
+            if sd.numel():
+                _check_f32('side gradient', sd)
+                _need(sd.numel() == w.numel(), 'side gradient size mismatch')
+                it.side[s] = sd.data_ptr()
+                if sc.numel():
+                    _need(sc.is_cuda and sc.dtype == torch.float32 and sc.numel() == 1, 'a side-gradient scale is one float32 on the GPU')
+                    it.side_scale[s] = sc.data_ptr()
+        items[t] = it
     rc = _lib.load().hgq_sgd_update_multi(items, n, lr, _stream())
     _lib.check(rc, 'hgq_sgd_update_multi')
 
@@ -1119,7 +1138,8 @@ def qdense(x2d, k_in, i_in, f_in, qw, qb, act: int, mode: int, bw_rows: int, tra
 class _DenseEbops(torch.autograd.Function):
     @staticmethod
     def forward(ctx, i_in, f_in, b_ker, b_bias, amax, decay, beta, k_in, k_ker, k_bias, ebops_var, P, K, N, scale, bias_size,
-                mode_in, mode_ker, mode_bias):
+                mode_in, mode_ker, mode_bias, owners):
+        ctx.owners = owners
         op = dense_ebops_track_op if amax.numel() else dense_ebops_op
         ebops, term, g = op(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N,
                                         scale, bias_size, mode_in, mode_ker, mode_bias)
@@ -1140,21 +1160,35 @@ class _DenseEbops(torch.autograd.Function):
         (g,) = ctx.saved_tensors
         up = g_term if ctx.has_beta else g_ebops
         if up is None:
-            return (None,) * 19
-        grads = up * g
+            return (None,) * 20
         n_f, n_k, n_b = ctx.sizes
         s_i, s_f, s_k, s_b = ctx.shapes
+        want_i = ctx.needs_input_grad[0] and not ctx.kbi_in
+        if _SINK['open'] and ctx.owners is not None:
+            # the pieces stay as the kernel left them (for a unit upstream gradient) and go to the optimizer with `up`
+            o_i, o_f, o_k, o_b = ctx.owners
+            pieces = [(o_f, g[:n_f]), (o_k, g[n_f:n_f + n_k])]
+            if want_i:
+                pieces.append((o_i, g[:n_f]))
+            if n_b:
+                pieces.append((o_b, g[n_f + n_k:]))
+            if all(o is not None for o, _ in pieces):
+                for o, piece in pieces:
+                    _stash_side(o, up, piece)
+                return (None,) * 20
+        grads = g if _is_unit(up) else up * g
         gf = grads[:n_f]
-        gi = gf.view(s_i) if (ctx.needs_input_grad[0] and not ctx.kbi_in) else None
-        return (gi, gf.view(s_f), grads[n_f:n_f + n_k].view(s_k), grads[n_f + n_k:].view(s_b) if n_b else None) + (None,) * 15
+        gi = gf.view(s_i) if want_i else None
+        return (gi, gf.view(s_f), grads[n_f:n_f + n_k].view(s_k), grads[n_f + n_k:].view(s_b) if n_b else None) + (None,) * 16
 
 
 def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, bias_size, mode_in, mode_ker, mode_bias,
-                amax=None, decay=0.0, beta=None, ebops_var=None):
+                amax=None, decay=0.0, beta=None, ebops_var=None, owners=None):
     """EBOPs of a dense contraction.  Returns ``(ebops, ebops * beta)``: with ``beta`` the second
     carries the gradient (and the first is a plain value), without it the first does.  With
     ``amax`` the input quantizer's integer bits are tracked in place first; with ``ebops_var`` the
-    uint32 variable is assigned."""
+    uint32 variable is assigned.  ``owners`` = the variables behind ``(i_in, f_in, b_ker, b_bias)``: with the gradient
+    sink open their gradient pieces are left on them instead of going back through autograd."""
     dev = f_in.device
     e_f = torch.empty(0, dtype=torch.float32, device=dev)
     e_i = torch.empty(0, dtype=torch.int32, device=dev)
@@ -1162,7 +1196,7 @@ def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, 
     return _DenseEbops.apply(i_in, f_in, b_ker, b_bias if b_bias is not None else e_f, amax if amax is not None else e_i,
                              float(decay), beta if beta is not None else e_f, k_in, k_ker,
                              k_bias if k_bias is not None else e_k, ebops_var if ebops_var is not None else e_i, P, K, N,
-                             float(scale), float(bias_size), mode_in, mode_ker, mode_bias)
+                             float(scale), float(bias_size), mode_in, mode_ker, mode_bias, owners)
 
 
 class _QSoftmax(torch.autograd.Function):
@@ -1427,7 +1461,8 @@ class _BitsEbops(torch.autograd.Function):
     (empty tensors where absent).  The kernel leaves the gradients for a unit upstream gradient; backward scales them."""
 
     @staticmethod
-    def forward(ctx, kind, params, beta, ebops_var, layouts, *qvars):
+    def forward(ctx, kind, params, beta, ebops_var, layouts, owners, *qvars):
+        ctx.owners = owners
         lib = _lib.load()
         ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
         total = sum(2 * fb.numel() for fb, lay in zip(fbs, layouts) if lay is not None)
@@ -1469,8 +1504,23 @@ class _BitsEbops(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         (buf,) = ctx.saved_tensors
-        scaled = buf * g  # one launch for every operand
-        grads = [None, None, None, None, None]
+        n_args = 6 + 3 * len(ctx.slots)
+        if _SINK['open'] and ctx.owners is not None:
+            pieces = []
+            for slot, kbi, own in zip(ctx.slots, ctx.kbis, ctx.owners):
+                if slot is None:
+                    continue
+                oi, of, n = slot
+                o_i, o_fb = own if own is not None else (None, None)
+                pieces.append((o_fb, buf[of:of + n]))
+                if not kbi and (o_i is None or o_i.requires_grad):  # an unknown owner makes the whole call fall back
+                    pieces.append((o_i, buf[oi:oi + n]))
+            if all(o is not None for o, _ in pieces):
+                for o, piece in pieces:
+                    _stash_side(o, g, piece)
+                return (None,) * n_args
+        scaled = buf if _is_unit(g) else buf * g  # one launch for every operand
+        grads = [None, None, None, None, None, None]
         for slot, kbi, (i_shape, fb_shape) in zip(ctx.slots, ctx.kbis, ctx.shapes):
             if slot is None:
                 grads += [None, None, None]
@@ -1480,12 +1530,16 @@ class _BitsEbops(torch.autograd.Function):
         return tuple(grads)
 
 
-def bits_ebops(kind: str, operands, params, beta: Tensor, ebops_var: Tensor) -> Tensor:
+def bits_ebops(kind: str, operands, params, beta: Tensor, ebops_var: Tensor, owners=None) -> Tensor:
     """Loss term ``ebops * beta`` of a layer whose EBOPs are algebra on bit-width tensors, in one launch; also assigns
     the uint32 variable.  ``operands``: per operand ``None`` or ``(k, i, fb, size, inner, kbi, add_mode)`` (``i`` is
-    ``None`` for the (k, b, i) kind); ``params`` as the C entry point of ``kind`` ('lut', 'softmax', 'mha') takes them."""
+    ``None`` for the (k, b, i) kind); ``params`` as the C entry point of ``kind`` ('lut', 'softmax', 'mha') takes them;
+    ``owners``: per operand ``None`` or the variables ``(i, fb)`` behind it (see :class:`side_gradients`)."""
     e_f = beta.new_empty(0)
     e_k = torch.empty(0, dtype=torch.uint8, device=beta.device)
+    if owners is None:  # operands that are the variables themselves own their gradient pieces
+        as_var = lambda t: t if isinstance(t, torch.nn.Parameter) else None  # noqa: E731
+        owners = [None if op is None else (as_var(op[1]), as_var(op[2])) for op in operands]
     flat, layouts = [], []
     for op in operands:
         if op is None:
@@ -1495,7 +1549,7 @@ def bits_ebops(kind: str, operands, params, beta: Tensor, ebops_var: Tensor) -> 
         k, i, fb, size, inner, kbi, add_mode = op
         flat += [k if add_mode else e_k, e_f if kbi else i, fb]
         layouts.append((int(size), int(inner), bool(kbi), int(add_mode)))
-    return _BitsEbops.apply(kind, tuple(params), beta, ebops_var, tuple(layouts), *flat)
+    return _BitsEbops.apply(kind, tuple(params), beta, ebops_var, tuple(layouts), tuple(owners) if owners is not None else None, *flat)
 
 
 class _AttnScores(torch.autograd.Function):
@@ -1603,7 +1657,7 @@ class _SparseCE(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         (dlogits,) = ctx.saved_tensors
-        return g * dlogits, None
+        return (dlogits if _is_unit(g) else g * dlogits), None
 
 
 class _MSE(torch.autograd.Function):
@@ -1635,6 +1689,61 @@ def sgd_update_(w, g, lr, l1=0.0, lo=float('-inf'), hi=float('inf')):
     sgd_update_op(w, g.contiguous(), float(lr), float(l1), float(lo), float(hi))
 
 
-def sgd_update_multi_(ws, gs, l1, lo, hi, lr):
-    sgd_update_multi_op(list(ws), [g.contiguous() for g in gs], [float(v) for v in l1], [float(v) for v in lo],
-                        [float(v) for v in hi], float(lr))
+def sgd_update_multi_(ws, gs, l1, lo, hi, lr, sides=None):
+    """``gs[t]`` may be ``None``; ``sides[t]`` is a list of up to ``SGD_SIDES`` ``(scale or None, gradient)`` pairs."""
+    n = len(ws)
+    dev = ws[0].device
+    empty = torch.empty(0, dtype=torch.float32, device=dev)
+    flat_s, flat_c = [], []
+    for t in range(n):
+        pairs = list(sides[t]) if sides is not None else []
+        if len(pairs) > SGD_SIDES:
+            raise ValueError(f'at most {SGD_SIDES} side gradients per variable')
+        for sc, sd in pairs:
+            flat_s.append(sd.contiguous())
+            flat_c.append(sc if sc is not None else empty)
+        for _ in range(SGD_SIDES - len(pairs)):
+            flat_s.append(empty), flat_c.append(empty)
+    sgd_update_multi_op(list(ws), [g.contiguous() if g is not None else empty for g in gs], [float(v) for v in l1],
+                        [float(v) for v in lo], [float(v) for v in hi], float(lr), flat_s, flat_c)
+
+
+# ======================================================================================
+# gradient pieces that bypass autograd's accumulation
+# ======================================================================================
+# With the sink open, an EBOPs operator does not hand the gradients of the bit-width variables back to autograd (where
+# each would cost a multiplication by the upstream gradient and an addition to the variable's other gradient, one
+# library launch each): it leaves ``(upstream gradient, unit-upstream gradient)`` on the variable, and the optimizer's
+# update kernel adds the pieces while it reads them.  Only an optimizer that consumes ``_hgq_side`` may open the sink.
+_SINK = {'open': False, 'unit_ptr': 0}
+
+
+class side_gradients:
+    """Context manager around ``loss.backward(root)``: opens the sink; ``root`` is the gradient the caller seeds the
+    backward pass with when that gradient is exactly one (its address identifies "the upstream gradient is 1")."""
+
+    def __init__(self, unit_root: Tensor | None = None):
+        self.unit_ptr = unit_root.data_ptr() if unit_root is not None else 0
+
+    def __enter__(self):
+        self.prev = dict(_SINK)
+        _SINK['open'], _SINK['unit_ptr'] = True, self.unit_ptr
+        return self
+
+    def __exit__(self, *exc):
+        _SINK.update(self.prev)
+
+
+def _is_unit(g: Tensor) -> bool:
+    """The tensor is (a view of) the seed gradient that the caller declared to be one."""
+    return _SINK['unit_ptr'] != 0 and g.numel() == 1 and g.data_ptr() == _SINK['unit_ptr']
+
+
+def _stash_side(owner, up: Tensor, piece: Tensor) -> bool:
+    """Leave ``up * piece`` on ``owner`` for the optimizer; False when the sink is closed or the owner is unknown."""
+    if not _SINK['open'] or owner is None or not getattr(owner, 'requires_grad', False):
+        return False
+    if not hasattr(owner, '_hgq_side') or owner._hgq_side is None:
+        owner._hgq_side = []
+    owner._hgq_side.append((None if _is_unit(up) else up.reshape(1), piece.reshape(-1)))
+    return True

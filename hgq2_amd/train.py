@@ -45,20 +45,39 @@ class SGD:
         self.params = [p for p in params if p.requires_grad]
         self.lr = float(lr)
         self.fold_regularizers = fold_regularizers
+        self._unit = None
 
     def zero_grad(self, set_to_none: bool = True):
         for p in self.params:
+            p._hgq_side = None
             if set_to_none:
                 p.grad = None
             elif p.grad is not None:
                 p.grad.zero_()
 
+    def backward(self, loss):
+        """``loss.backward()`` with the gradient sink of :class:`hgq2_amd.ops.side_gradients` open: the EBOPs terms leave
+        their bit-width gradients on the variables as ``(upstream gradient, piece)`` pairs instead of sending them through
+        autograd, and :meth:`step` adds the pieces inside the update kernel.  Same update as ``loss.backward()`` followed by
+        :meth:`step`; about four launches fewer per quantized layer."""
+        if loss.numel() != 1:
+            raise ValueError('backward(loss) expects a scalar loss')
+        if self._unit is None or self._unit.device != loss.device or self._unit.shape != loss.shape:
+            self._unit = torch.ones_like(loss)  # the seed gradient: allocated once, also outside a captured graph
+        with ops.side_gradients(self._unit):
+            loss.backward(self._unit)
+
     @torch.no_grad()
     def step(self):
-        ws, gs, l1s, los, his, post = [], [], [], [], [], []
+        ws, gs, l1s, los, his, sides, post = [], [], [], [], [], [], []
         for p in self.params:
-            if p.grad is None:
+            side = list(getattr(p, '_hgq_side', None) or ())
+            g = p.grad
+            if g is None and not side:
                 continue
+            while len(side) > ops.SGD_SIDES:  # more pieces than the kernel takes: fold the surplus into one
+                (s1, d1), (s2, d2) = side.pop(), side.pop()
+                side.append((None, (d1 if s1 is None else s1 * d1) + (d2 if s2 is None else s2 * d2)))
             c = getattr(p, 'constraint', None)
             r = getattr(p, 'regularizer', None)
             bounds = c.bounds() if c is not None else (float('-inf'), float('inf'))
@@ -66,12 +85,13 @@ class SGD:
                 bounds = (float('-inf'), float('inf'))
                 post.append((p, c))
             ws.append(p.data)
-            gs.append(p.grad)
+            gs.append(g)
+            sides.append(side)
             l1s.append(r.l1 if (self.fold_regularizers and isinstance(r, MonoL1)) else 0.0)
             los.append(bounds[0])
             his.append(bounds[1])
         if ws:
-            ops.sgd_update_multi_(ws, gs, l1s, los, his, self.lr)
+            ops.sgd_update_multi_(ws, gs, l1s, los, his, self.lr, sides)
         for p, c in post:
             p.copy_(c(p))
 
@@ -105,7 +125,7 @@ class GraphedTrainStep:
         self.opt.zero_grad(set_to_none=True)
         out = self.model(self.x, training=True)
         loss = model_loss(self.model, self.loss_fn(out, self.y), self.opt.fold_regularizers)
-        loss.backward()
+        self.opt.backward(loss)
         self.opt.step()
         return loss.detach()
 

@@ -264,13 +264,23 @@ int hgq_sgd_update(float *w, const float *g, int64_t n, float lr, float l1, floa
 /*
  * The same update for many variables in one launch (descriptors are read on the host and travel
  * to the kernel as launch arguments, so the call is safe under HIP graph capture).
+ *
+ * A variable's gradient may arrive in several pieces: `g` (NULL = none) plus up to HGQ_SGD_SIDES further contributions
+ * `side[s]` of the same length, each multiplied by the device scalar `side_scale[s][0]` (NULL = 1):
+ *     grad = g + sum_s side_scale[s] * side[s];   w <- clip(w - lr * (grad + l1), lo, hi)
+ * In the reference a bit-width variable collects its gradient from its quantizer's backward and from every EBOPs term
+ * it enters (src/hgq/layers/core/base.py:100-104), and autograd adds the pieces one launch at a time; here the
+ * pieces are added where they are consumed.
  */
-#define HGQ_SGD_BATCH 48
+#define HGQ_SGD_BATCH 32
+#define HGQ_SGD_SIDES 3
 typedef struct {
     float *w;
     const float *g;
     int64_t n;
     float l1, lo, hi;
+    const float *side[HGQ_SGD_SIDES];
+    const float *side_scale[HGQ_SGD_SIDES];
 } hgq_sgd_item;
 int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *stream);
 

@@ -367,3 +367,57 @@ def test_batched_quantizer_matches_single_launches():
         else:
             for a in got[t][1:]:
                 assert a is None or not a.any()
+
+
+@pytest.mark.parametrize('kind', ['mlp', 'particle', 'conv', 'mha'])
+def test_gradient_sink_gives_the_autograd_update(dev, kind):
+    """``opt.backward(loss)`` leaves the EBOPs gradients of the bit-width variables on the variables and the update
+    kernel adds them; the result must be the update of plain ``loss.backward()``.  Where a variable has one piece from
+    autograd and one from an EBOPs term the two paths add the same two numbers: bit-identical."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, model_loss
+    from hgq2_amd.utils import models
+
+    g = torch.Generator().manual_seed(61)
+    if kind == 'mlp':
+        x, y = torch.randn(4096, 16, generator=g), torch.randint(0, 5, (4096,), generator=g)
+        build = lambda: models.qdense_mlp(device=dev)  # noqa: E731
+        loss_fn = lambda out: ops.sparse_ce(out, y.to(dev))  # noqa: E731
+    elif kind == 'particle':
+        x, y = torch.randn(256, 16, 16, generator=g), torch.randint(0, 5, (256,), generator=g)
+        build = lambda: models.particle_mlp(n_particles=16, device=dev)  # noqa: E731
+        loss_fn = lambda out: ops.sparse_ce(out, y.to(dev))  # noqa: E731
+    elif kind == 'conv':
+        x, y = torch.rand(64, 28, 28, 1, generator=g), torch.randint(0, 10, (64,), generator=g)
+        build = lambda: models.conv_stack(device=dev)  # noqa: E731
+        loss_fn = lambda out: ops.sparse_ce(out, y.to(dev))  # noqa: E731
+    else:
+        x = torch.randn(64, 64, 64, generator=g)
+        build = lambda: models.mha_block(device=dev)  # noqa: E731
+        loss_fn = lambda out: ops.mse(out)  # noqa: E731
+    xd = x.to(dev)
+    torch.manual_seed(7)
+    a = build()
+    a(xd, training=True)
+    torch.manual_seed(7)
+    b = build()
+    b(xd, training=True)
+    b.load_state_dict(a.state_dict())
+    opt_a, opt_b = SGD(a.parameters(), lr=0.05, fold_regularizers=True), SGD(b.parameters(), lr=0.05, fold_regularizers=True)
+    for step in range(2):
+        opt_a.zero_grad()
+        la = model_loss(a, loss_fn(a(xd, training=True)), True)
+        la.backward()
+        opt_a.step()
+        opt_b.zero_grad()
+        lb = model_loss(b, loss_fn(b(xd, training=True)), True)
+        opt_b.backward(lb)
+        n_pieces = sum(len(getattr(p, '_hgq_side', None) or ()) for p in b.parameters())
+        assert n_pieces > 0, 'no EBOPs gradient took the side channel'
+        opt_b.step()
+        assert abs(float(la) - float(lb)) <= 1e-6 * abs(float(la))  # the loss value is summed with atomics
+        for (name, pa), (_, pb) in zip(a.named_parameters(), b.named_parameters()):
+            if kind == 'mlp':
+                assert torch.equal(pa, pb), f'{name} step {step}'
+            else:
+                assert torch.allclose(pa, pb, rtol=1e-6, atol=1e-9), f'{name} step {step}: {float((pa - pb).abs().max()):.3e}'
