@@ -243,12 +243,21 @@ class Layer(nn.Module):
             self._losses = []
         _ctx.training = training
         _ctx.depth = getattr(_ctx, 'depth', 0) + 1
+        if top:
+            from . import ops
+
+            ops.begin_deferred()  # single-workgroup launches that nothing in the forward waits for go out together at the end
+        ok = False
         try:
             self._maybe_build(args)
-            return self._wrapped_call(*args, training=training, **kwargs)
+            out = self._wrapped_call(*args, training=training, **kwargs)
+            ok = True
+            return out
         finally:
             _ctx.depth -= 1
             _ctx.training = outer
+            if top:
+                ops.end_deferred(discard=not ok)
 
     def _wrapped_call(self, *args, training=None, **kwargs):
         return self.call(*args, training=training, **kwargs)

@@ -52,14 +52,14 @@ __device__ __forceinline__ float block_sum_ebops(float v, float *scratch16) {
 
 // One workgroup of 1024 threads.  Bit-widths are integers, so the per-row / per-column sums are
 // accumulated with integer LDS atomics over flat, coalesced sweeps (exact in any order).
-__global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_t *amax_part, int n_parts, float decay,
-                                                          const float *beta, float *loss_term,
-                                                          const void *k_in, float *i_in, const float *f_in,
-                                                          int64_t P, int K, int N, const void *k_ker,
-                                                          const float *b_ker, const void *k_bias, const float *b_bias,
-                                                          float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
-                                                          float *ebops, uint32_t *ebops_u32, float *g_f_in,
-                                                          float *g_b_ker, float *g_b_bias) {
+__device__ __forceinline__ void dense_ebops_body(const uint32_t *amax_part, int n_parts, float decay,
+                                                 const float *beta, float *loss_term,
+                                                 const void *k_in, float *i_in, const float *f_in,
+                                                 int64_t P, int K, int N, const void *k_ker,
+                                                 const float *b_ker, const void *k_bias, const float *b_bias,
+                                                 float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
+                                                 float *ebops, uint32_t *ebops_u32, float *g_f_in,
+                                                 float *g_b_ker, float *g_b_bias) {
     constexpr int NT = HGQ_EBOPS_NT;
     // bit-widths are integers: the sums are accumulated with native integer LDS atomics
     __shared__ int colsum[HGQ_EBOPS_MAXK];  // sum_n bits_ker[k, n]
@@ -173,6 +173,30 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_
         if (ebops_u32) ebops_u32[0] = (uint32_t)e;
         if (loss_term && beta) loss_term[0] = e * beta[0];
     }
+}
+
+__global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_t *amax_part, int n_parts, float decay,
+                                                          const float *beta, float *loss_term,
+                                                          const void *k_in, float *i_in, const float *f_in,
+                                                          int64_t P, int K, int N, const void *k_ker,
+                                                          const float *b_ker, const void *k_bias, const float *b_bias,
+                                                          float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
+                                                          float *ebops, uint32_t *ebops_u32, float *g_f_in,
+                                                          float *g_b_ker, float *g_b_bias) {
+    dense_ebops_body(amax_part, n_parts, decay, beta, loss_term, k_in, i_in, f_in, P, K, N, k_ker, b_ker, k_bias, b_bias, scale, bias_size,
+                     mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
+}
+
+// the layers of a model, one workgroup each: the estimates depend on the bit-width variables only, so they can all be
+// computed at the end of the forward pass in one launch instead of one single-workgroup launch per layer
+struct DenseEbopsBatch {
+    hgq_dense_ebops_item item[HGQ_EBOPS_BATCH];
+};
+__global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_multi_kernel(DenseEbopsBatch b) {
+    const hgq_dense_ebops_item &it = b.item[blockIdx.x];
+    dense_ebops_body(it.amax_part, it.n_parts, it.decay, it.beta, it.loss_term, it.k_in, it.i_in, it.f_in, it.P, it.K, it.N, it.k_ker,
+                     it.b_ker, it.k_bias, it.b_bias, it.scale, it.bias_size, it.mode_in, it.mode_ker, it.mode_bias, it.ebops, it.ebops_u32,
+                     it.g_f_in, it.g_b_ker, it.g_b_bias);
 }
 
 // Mean squared error: per-workgroup partial sums (fixed order inside a workgroup), added in order
@@ -541,6 +565,37 @@ extern "C" int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float dec
                        i_in, f_in, P, K, N, k_ker, b_ker,
                        k_bias, b_bias, scale, bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
     return check_launch("hgq_dense_ebops");
+}
+
+extern "C" int hgq_dense_ebops_multi(const hgq_dense_ebops_item *items, int count, void *stream) {
+    if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: bad arguments");
+    for (int base = 0; base < count; base += HGQ_EBOPS_BATCH) {
+        DenseEbopsBatch b;
+        const int nb = count - base < HGQ_EBOPS_BATCH ? count - base : HGQ_EBOPS_BATCH;
+        for (int t = 0; t < nb; ++t) {
+            const hgq_dense_ebops_item &it = items[base + t];
+            if (it.P < 1 || it.K < 1 || it.N < 1) return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: bad sizes in item %d", base + t);
+            if (!it.i_in || !it.f_in || !it.b_ker || !it.ebops || !it.k_in || !it.k_ker)
+                return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: null pointer in item %d", base + t);
+            if (it.K > HGQ_EBOPS_MAXK) return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops_multi: K=%d > %d", it.K, HGQ_EBOPS_MAXK);
+            if (!(Mode(it.mode_ker).kbi) || (it.b_bias && !(Mode(it.mode_bias).kbi)))
+                return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops_multi: kernel/bias bit-widths must use the KBI parametrisation");
+            if (it.amax_part && (it.n_parts < 1 || Mode(it.mode_in).kbi || Mode(it.mode_in).overflow_mode != HGQ_WRAP))
+                return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: fused tracking is for KIF WRAP input quantizers");
+            b.item[t] = it;
+            if (it.amax_part && it.P * it.K * it.n_parts > 16384) {
+                // many tracker slices: combine them with one thread group per entry across the device first
+                int rc = hgq_wrap_track_i(it.amax_part, nullptr, it.n_parts, it.i_in, it.f_in, nullptr, it.P * it.K, it.decay, 0.0f, 0.0f,
+                                          it.mode_in & ~(HGQ_MODE_TRACING | HGQ_MODE_SYMMETRIC), stream);
+                if (rc) return rc;
+                b.item[t].amax_part = nullptr;
+            }
+        }
+        hipLaunchKernelGGL(dense_ebops_multi_kernel, dim3((unsigned)nb), dim3(HGQ_EBOPS_NT), 0, (hipStream_t)stream, b);
+        int rc = check_launch("hgq_dense_ebops_multi");
+        if (rc) return rc;
+    }
+    return HGQ_OK;
 }
 
 extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *loss, float *dlogits,

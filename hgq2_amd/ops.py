@@ -190,11 +190,8 @@ def _(dy, y, x, f_in, qw, has_bias, act, mode, bw_rows):
             x.new_empty(bw_rows * x.shape[1]))
 
 
-def _dense_ebops_impl(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor,
-                   b_ker: Tensor, k_bias: Tensor, b_bias: Tensor, ebops_var: Tensor, P: int, K: int, N: int, scale: float,
-                   bias_size: float, mode_in: int, mode_ker: int, mode_bias: int) -> tuple[Tensor, Tensor, Tensor]:
-    """Returns (ebops, ebops*beta, [g_f_in | g_b_ker | g_b_bias] in one buffer); with ``beta`` the
-    gradient buffer holds d(ebops*beta)/d variable, else d ebops / d variable."""
+def _dense_ebops_check(amax, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N, mode_in, mode_ker, mode_bias):
+    """Validates one dense-EBOPs call; returns ``(n_parts, has_bias, mode_in, mode_ker, mode_bias)`` with the k-storage flags set."""
     _check_k('k_in', k_in), _check_f32('i_in', i_in), _check_f32('f_in', f_in), _check_k('k_ker', k_ker), _check_f32('b_ker', b_ker)
     _need(i_in.numel() == P * K and f_in.numel() == P * K and k_in.numel() == P * K, 'input bit-width size mismatch')
     _need(b_ker.numel() == K * N and k_ker.numel() == K * N, 'kernel bit-width size mismatch')
@@ -211,6 +208,16 @@ def _dense_ebops_impl(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_
         _need(ebops_var.is_cuda and ebops_var.element_size() == 4, 'the ebops variable must be a 4-byte GPU scalar')
     if beta.numel():
         _check_f32('beta', beta)
+    return n_parts, has_bias, _kmode(mode_in, k_in), _kmode(mode_ker, k_ker), mode_bias
+
+
+def _dense_ebops_impl(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor,
+                   b_ker: Tensor, k_bias: Tensor, b_bias: Tensor, ebops_var: Tensor, P: int, K: int, N: int, scale: float,
+                   bias_size: float, mode_in: int, mode_ker: int, mode_bias: int) -> tuple[Tensor, Tensor, Tensor]:
+    """Returns (ebops, ebops*beta, [g_f_in | g_b_ker | g_b_bias] in one buffer); with ``beta`` the
+    gradient buffer holds d(ebops*beta)/d variable, else d ebops / d variable."""
+    n_parts, has_bias, m_in, m_ker, m_bias = _dense_ebops_check(amax, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var,
+                                                               P, K, N, mode_in, mode_ker, mode_bias)
     dev = f_in.device
     ebops = torch.empty((), dtype=torch.float32, device=dev)
     term = torch.empty((), dtype=torch.float32, device=dev)
@@ -219,9 +226,96 @@ def _dense_ebops_impl(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_
     g_f, g_bk, g_bb = g[:P * K], g[P * K:P * K + K * N], g[P * K + K * N:]
     rc = _lib.load().hgq_dense_ebops(_ptr(amax), n_parts, decay, _ptr(beta), _ptr(term), _ptr(k_in), _ptr(i_in), _ptr(f_in),
                                      P, K, N, _ptr(k_ker), _ptr(b_ker), _ptr(k_bias), _ptr(b_bias), scale, bias_size,
-                                     _kmode(mode_in, k_in), _kmode(mode_ker, k_ker), mode_bias, _ptr(ebops), _ptr(ebops_var),
+                                     m_in, m_ker, m_bias, _ptr(ebops), _ptr(ebops_var),
                                      _ptr(g_f), _ptr(g_bk), _ptr(g_bb), _stream())
     _lib.check(rc, 'hgq_dense_ebops')
+    return ebops, term, g
+
+
+class _DenseEbopsItem(ctypes.Structure):
+    _fields_ = [('amax_part', ctypes.c_void_p), ('n_parts', ctypes.c_int), ('decay', ctypes.c_float), ('beta', ctypes.c_void_p),
+                ('loss_term', ctypes.c_void_p), ('k_in', ctypes.c_void_p), ('i_in', ctypes.c_void_p), ('f_in', ctypes.c_void_p),
+                ('P', ctypes.c_int64), ('K', ctypes.c_int), ('N', ctypes.c_int), ('k_ker', ctypes.c_void_p), ('b_ker', ctypes.c_void_p),
+                ('k_bias', ctypes.c_void_p), ('b_bias', ctypes.c_void_p), ('scale', ctypes.c_float), ('bias_size', ctypes.c_float),
+                ('mode_in', ctypes.c_int), ('mode_ker', ctypes.c_int), ('mode_bias', ctypes.c_int), ('ebops', ctypes.c_void_p),
+                ('ebops_u32', ctypes.c_void_p), ('g_f_in', ctypes.c_void_p), ('g_b_ker', ctypes.c_void_p), ('g_b_bias', ctypes.c_void_p)]
+
+
+@torch.library.custom_op('hgq::dense_ebops_multi', mutates_args=('i_ins', 'ebops_vars', 'ebops_outs', 'terms', 'gs'))
+def dense_ebops_multi_op(amaxs: Sequence[Tensor], betas: Sequence[Tensor], k_ins: Sequence[Tensor], i_ins: Sequence[Tensor],
+                         f_ins: Sequence[Tensor], k_kers: Sequence[Tensor], b_kers: Sequence[Tensor], k_biases: Sequence[Tensor],
+                         b_biases: Sequence[Tensor], ebops_vars: Sequence[Tensor], ebops_outs: Sequence[Tensor], terms: Sequence[Tensor],
+                         gs: Sequence[Tensor], decays: Sequence[float], dims: Sequence[int], scales: Sequence[float],
+                         bias_sizes: Sequence[float], modes: Sequence[int]) -> None:
+    """The dense-EBOPs launch of several layers at once; outputs are preallocated (``ebops_outs``, ``terms``, ``gs`` as
+    ``_dense_ebops_impl`` returns them).  ``dims`` = P, K, N per item, ``modes`` = mode_in, mode_ker, mode_bias per item."""
+    n = len(f_ins)
+    items = (_DenseEbopsItem * n)()
+    for t in range(n):
+        P, K, N = dims[3 * t:3 * t + 3]
+        n_parts, has_bias, m_in, m_ker, m_bias = _dense_ebops_check(
+            amaxs[t], betas[t], k_ins[t], i_ins[t], f_ins[t], k_kers[t], b_kers[t], k_biases[t], b_biases[t], ebops_vars[t], P, K, N,
+            modes[3 * t], modes[3 * t + 1], modes[3 * t + 2])
+        g = gs[t]
+        _need(g.numel() == P * K + K * N + (N if has_bias else 0) and g.is_contiguous(), 'gradient buffer size mismatch')
+        g_f, g_bk, g_bb = g[:P * K], g[P * K:P * K + K * N], g[P * K + K * N:]
+        p = lambda x: x.data_ptr() if x.numel() else None  # noqa: E731
+        items[t] = _DenseEbopsItem(p(amaxs[t]), n_parts, decays[t], p(betas[t]), p(terms[t]), p(k_ins[t]), p(i_ins[t]), p(f_ins[t]), P, K, N,
+                                   p(k_kers[t]), p(b_kers[t]), p(k_biases[t]), p(b_biases[t]), scales[t], bias_sizes[t], m_in, m_ker, m_bias,
+                                   p(ebops_outs[t]), p(ebops_vars[t]), p(g_f), p(g_bk), p(g_bb))
+    rc = _lib.load().hgq_dense_ebops_multi(items, n, _stream())
+    _lib.check(rc, 'hgq_dense_ebops_multi')
+
+
+# ---- launches deferred to the end of the outermost layer call
+# The EBOPs estimate of a dense layer (and the integer-bit update fused into it) reads bit-width variables and the
+# abs-max slices its own forward left; nothing later in the forward pass reads what it writes.  While a model call is
+# open the calls are queued - outputs allocated, nothing launched - and go out as one launch when the call returns.
+_DEFER = {'depth': 0, 'dense_ebops': []}
+
+
+def begin_deferred():
+    _DEFER['depth'] += 1
+
+
+def end_deferred(discard: bool = False):
+    _DEFER['depth'] -= 1
+    if _DEFER['depth'] == 0:
+        if discard:
+            _DEFER['dense_ebops'] = []
+        else:
+            flush_deferred()
+
+
+def flush_deferred():
+    q, _DEFER['dense_ebops'] = _DEFER['dense_ebops'], []
+    if not q:
+        return
+    cols = list(zip(*q))
+    (amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims, scales,
+     bias_sizes, modes) = cols
+    with torch.no_grad():
+        _flush_dense_ebops(amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims,
+                           scales, bias_sizes, modes)
+
+
+def _flush_dense_ebops(amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims,
+                       scales, bias_sizes, modes):
+    dense_ebops_multi_op(list(amaxs), list(betas), list(k_ins), list(i_ins), list(f_ins), list(k_kers), list(b_kers), list(k_biases),
+                         list(b_biases), list(ebops_vars), list(outs), list(terms), list(gs), [float(d) for d in decays],
+                         [int(v) for d in dims for v in d], [float(v) for v in scales], [float(v) for v in bias_sizes],
+                         [int(v) for m in modes for v in m])
+
+
+def _dense_ebops_queue(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N, scale, bias_size,
+                       mode_in, mode_ker, mode_bias):
+    dev = f_in.device
+    ebops = torch.empty((), dtype=torch.float32, device=dev)
+    term = torch.empty((), dtype=torch.float32, device=dev)
+    g = torch.empty(P * K + K * N + (N if b_bias.numel() else 0), dtype=torch.float32, device=dev)
+    # `.data`: the update of the integer bits is a state assignment, not an operation autograd should see
+    _DEFER['dense_ebops'].append((amax, beta, k_in, i_in.data, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, ebops, term, g, decay, (P, K, N),
+                                  scale, bias_size, (mode_in, mode_ker, mode_bias)))
     return ebops, term, g
 
 
@@ -1140,10 +1234,13 @@ class _DenseEbops(torch.autograd.Function):
     def forward(ctx, i_in, f_in, b_ker, b_bias, amax, decay, beta, k_in, k_ker, k_bias, ebops_var, P, K, N, scale, bias_size,
                 mode_in, mode_ker, mode_bias, owners):
         ctx.owners = owners
-        op = dense_ebops_track_op if amax.numel() else dense_ebops_op
+        if _DEFER['depth'] > 0:  # inside a model call: queued, launched with the other layers' when the call returns
+            op = _dense_ebops_queue
+        else:
+            op = dense_ebops_track_op if amax.numel() else dense_ebops_op
         ebops, term, g = op(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N,
                                         scale, bias_size, mode_in, mode_ker, mode_bias)
-        ctx.save_for_backward(g)
+        ctx.g = g  # kept as a plain attribute: a queued call fills it after this function has returned
         ctx.has_beta = beta.numel() > 0
         ctx.sizes = (P * K, K * N, b_bias.numel())
         ctx.kbi_in = bool(mode_in & _lib.MODE_KBI)
@@ -1157,7 +1254,7 @@ class _DenseEbops(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_ebops, g_term):
-        (g,) = ctx.saved_tensors
+        g = ctx.g
         up = g_term if ctx.has_beta else g_ebops
         if up is None:
             return (None,) * 20

@@ -234,6 +234,36 @@ int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const f
                     uint32_t *ebops_u32, float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream);
 
 /*
+ * hgq_dense_ebops for several layers in one launch (one workgroup per item; argument meaning as above).  The estimate of a
+ * layer depends on bit-width variables only (src/hgq/layers/core/base.py:100: shapes (1,) + shape[1:]), so the layers of
+ * a model can be served together once the forward pass has produced every input quantizer's abs-max slices.
+ * Descriptors are read on the host and travel as launch arguments (safe under HIP graph capture).
+ */
+#define HGQ_EBOPS_BATCH 16
+typedef struct {
+    const uint32_t *amax_part;
+    int n_parts;
+    float decay;
+    const float *beta;
+    float *loss_term;
+    const void *k_in;
+    float *i_in;
+    const float *f_in;
+    int64_t P;
+    int K, N;
+    const void *k_ker;
+    const float *b_ker;
+    const void *k_bias;
+    const float *b_bias;
+    float scale, bias_size;
+    int mode_in, mode_ker, mode_bias;
+    float *ebops;
+    uint32_t *ebops_u32;
+    float *g_f_in, *g_b_ker, *g_b_bias;
+} hgq_dense_ebops_item;
+int hgq_dense_ebops_multi(const hgq_dense_ebops_item *items, int count, void *stream);
+
+/*
  * Mean squared error, the regression loss HGQ models are trained with through Keras
  * (`loss='mse'`; the reference has no loss code of its own).  target may be NULL (zeros).
  *   loss [1] = mean((pred - target)^2) over n elements, summed in a fixed order;
