@@ -351,7 +351,7 @@ def sgd_update_op(w: Tensor, g: Tensor, lr: float, l1: float, lo: float, hi: flo
     _lib.check(rc, 'hgq_sgd_update')
 
 
-SGD_SIDES = 3
+SGD_SIDES = 4
 
 
 class _SgdItem(ctypes.Structure):
@@ -1205,6 +1205,7 @@ class _QDense(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track):
         y, amax = qdense_fwd(x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track)
+        ctx.f_owner = _owner(f_in)
         ctx.save_for_backward(x, f_in, qw, y)
         ctx.has_bias = qb.numel() > 0
         ctx.act, ctx.mode, ctx.bw_rows, ctx.f_shape = act, mode, bw_rows, f_in.shape
@@ -1218,7 +1219,8 @@ class _QDense(torch.autograd.Function):
             return (None,) * 10
         x, f_in, qw, y = ctx.saved_tensors
         dx, dqw, dqb, df = qdense_bwd(gy.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows)
-        return (dx, None, None, df.view(ctx.f_shape) if ctx.bw_rows > 0 else None, dqw, dqb if ctx.has_bias else None,
+        df = _route(ctx.f_owner, df) if ctx.bw_rows > 0 else None
+        return (dx, None, None, df.view(ctx.f_shape) if df is not None else None, dqw, dqb if ctx.has_bias else None,
                 None, None, None, None)
 
 
@@ -1461,6 +1463,7 @@ class _DenseMoments(torch.autograd.Function):
     def forward(ctx, x, w, f_in, bw_rows, mode, chain):
         ctx.save_for_backward(x, w, f_in)
         ctx.quant = (bw_rows, mode)
+        ctx.owners = (_owner(w), _owner(f_in))
         mean, meansq = dense_moments_fwd(x, w, f_in, bw_rows, mode)
         return (mean, meansq, x) if chain else (mean, meansq)
 
@@ -1468,12 +1471,15 @@ class _DenseMoments(torch.autograd.Function):
     def backward(ctx, dmean, dmeansq, dx_chain=None):
         x, w, f_in = ctx.saved_tensors
         bw_rows, mode = ctx.quant
-        zero = x.new_zeros(w.shape[1])
+        zero = x.new_zeros(w.shape[1]) if (dmean is None or dmeansq is None) else None
         # without a consumer of dx (an input that needs no gradient) the chained gradient is not read either
         dx_add = x.new_empty(0) if dx_chain is None or not ctx.needs_input_grad[0] else dx_chain.contiguous()
         dx, dw, df = dense_moments_bwd(x, w, f_in, bw_rows, mode, dmean.contiguous() if dmean is not None else zero,
                                        dmeansq.contiguous() if dmeansq is not None else zero, dx_add)
-        return dx, dw, (df.view(f_in.shape) if bw_rows else None), None, None, None
+        o_w, o_f = ctx.owners
+        dw = _route(o_w, dw)
+        df = _route(o_f, df) if bw_rows else None
+        return dx, dw, (df.view(f_in.shape) if df is not None else None), None, None, None
 
 
 def dense_moments(x2d: Tensor, w2d: Tensor, quant=None, chain=False):
@@ -1492,6 +1498,7 @@ class _BnFold(torch.autograd.Function):
     def forward(ctx, w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum):
         ctx.save_for_backward(w, gamma, mean, second)
         ctx.cfg = (is_meansq, eps)
+        ctx.w_owner = _owner(w)
         return bn_fold_fwd(w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum)
 
     @staticmethod
@@ -1499,7 +1506,7 @@ class _BnFold(torch.autograd.Function):
         w, gamma, mean, second = ctx.saved_tensors
         is_meansq, eps = ctx.cfg
         dw, dbias, dgamma, dmean, dsecond = bn_fold_bwd(w, gamma, mean, second, is_meansq, eps, d_fw.contiguous(), d_fb.contiguous())
-        return dw, dbias, (dgamma if gamma.numel() else None), dmean, dsecond, None, None, None, None, None
+        return _route(ctx.w_owner, dw), dbias, (dgamma if gamma.numel() else None), dmean, dsecond, None, None, None, None, None
 
 
 def bn_fold(w2d: Tensor, bias: Tensor, gamma, mean: Tensor, second: Tensor, is_meansq: bool, eps: float, moving_mean=None,
@@ -1836,11 +1843,31 @@ def _is_unit(g: Tensor) -> bool:
     return _SINK['unit_ptr'] != 0 and g.numel() == 1 and g.data_ptr() == _SINK['unit_ptr']
 
 
-def _stash_side(owner, up: Tensor, piece: Tensor) -> bool:
-    """Leave ``up * piece`` on ``owner`` for the optimizer; False when the sink is closed or the owner is unknown."""
+def _stash_side(owner, up, piece: Tensor) -> bool:
+    """Leave ``up * piece`` (``up`` None: the piece as it is) on ``owner`` for the optimizer; False when the sink is
+    closed or the owner is unknown."""
     if not _SINK['open'] or owner is None or not getattr(owner, 'requires_grad', False):
         return False
     if not hasattr(owner, '_hgq_side') or owner._hgq_side is None:
         owner._hgq_side = []
-    owner._hgq_side.append((None if _is_unit(up) else up.reshape(1), piece.reshape(-1)))
+    owner._hgq_side.append((None if (up is None or _is_unit(up)) else up.reshape(1), piece.reshape(-1)))
     return True
+
+
+def _owner(t):
+    """The variable a kernel operand is (a view of), or None."""
+    if isinstance(t, torch.nn.Parameter):
+        return t
+    base = getattr(t, '_base', None)
+    return base if isinstance(base, torch.nn.Parameter) else None
+
+
+def _route(owner, grad):
+    """A finished gradient of a variable that also receives gradient from elsewhere: with the sink open it is left on
+    the variable (returns None, so autograd has nothing to accumulate), otherwise handed back."""
+    if grad is None or owner is None or not _SINK['open'] or not owner.requires_grad or grad.numel() != owner.numel():
+        return grad
+    if len(getattr(owner, '_hgq_side', None) or ()) >= SGD_SIDES:
+        return grad  # no room left in the update kernel's descriptor: autograd accumulates this one
+    _stash_side(owner, None, grad.contiguous())
+    return None

@@ -302,8 +302,8 @@ int hgq_sgd_update(float *w, const float *g, int64_t n, float lr, float l1, floa
  * it enters (src/hgq/layers/core/base.py:100-104), and autograd adds the pieces one launch at a time; here the
  * pieces are added where they are consumed.
  */
-#define HGQ_SGD_BATCH 32
-#define HGQ_SGD_SIDES 3
+#define HGQ_SGD_BATCH 28
+#define HGQ_SGD_SIDES 4
 typedef struct {
     float *w;
     const float *g;
