@@ -267,6 +267,15 @@ def dense_ebops_multi_op(amaxs: Sequence[Tensor], betas: Sequence[Tensor], k_ins
     _lib.check(rc, 'hgq_dense_ebops_multi')
 
 
+# ---- state epoch: bumped by everything in this package that writes variables through `.data` or from a kernel (writes
+# the tensors' version counters do not see); a cache keyed on variable versions also keys on it
+STATE_EPOCH = [0]
+
+
+def touch_state():
+    STATE_EPOCH[0] += 1
+
+
 # ---- launches deferred to the end of the outermost layer call
 # The EBOPs estimate of a dense layer (and the integer-bit update fused into it) reads bit-width variables and the
 # abs-max slices its own forward left; nothing later in the forward pass reads what it writes.  While a model call is
@@ -294,6 +303,7 @@ def flush_deferred():
     cols = list(zip(*q))
     (amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims, scales,
      bias_sizes, modes) = cols
+    touch_state()  # the fused integer-bit update writes `_i`
     with torch.no_grad():
         _flush_dense_ebops(amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims,
                            scales, bias_sizes, modes)
@@ -1192,6 +1202,7 @@ def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('
     """In-place integer-bit tracking; ``amax`` is [m] or [n_parts, m]."""
     m = i_var.numel()
     n_parts = amax.numel() // m
+    touch_state()
     empty_i = amax.new_empty(0)
     empty_k = torch.empty(0, dtype=torch.uint8, device=amax.device)
     wrap_track_i_op(amax, anyneg if anyneg is not None else empty_i, n_parts, i_var, fb,

@@ -51,7 +51,9 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
         if self.overflow_mode == 'WRAP':
             init = self._i_decay_speed0
             self._i_decay_speed = self.add_weight(name='i_decay_speed', shape=(), initializer=init, trainable=False)
-            self._decay_host = float(init.value) if isinstance(init, ConstantInit) else float(self._i_decay_speed)
+            # host copy of the variable for the launch arguments, refreshed when the variable is written
+            self._decay_value = float(init.value) if isinstance(init, ConstantInit) else float(self._i_decay_speed)
+            self._decay_version = self._i_decay_speed._version
         self._symmetric = self.overflow_mode.endswith('SYM')
         self.built = True
 
@@ -62,6 +64,15 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
     @property
     def i_decay_speed(self):
         return self._i_decay_speed
+
+    @property
+    def _decay_host(self) -> float:
+        """``i_decay_speed`` as a host float (kernels take it as a launch argument): read back from the device only after
+        the variable has been written (``assign``-style in-place writes and ``load_state_dict`` bump its version)."""
+        v = self._i_decay_speed._version
+        if v != self._decay_version:
+            self._decay_value, self._decay_version = float(self._i_decay_speed), v
+        return self._decay_value
 
     # ---- bit-width views (differentiable).  On the GPU one launch each way (`ops.qbits`); the torch
     # formula below is the same arithmetic as a chain of round / add / relu / cast launches.

@@ -91,6 +91,7 @@ class SGD:
             los.append(bounds[0])
             his.append(bounds[1])
         if ws:
+            ops.touch_state()  # written through `.data`: the version counters do not move
             ops.sgd_update_multi_(ws, gs, l1s, los, his, self.lr, sides)
         for p, c in post:
             p.copy_(c(p))
@@ -134,6 +135,7 @@ class GraphedTrainStep:
             self.x.copy_(x)
         if y is not None:
             self.y.copy_(y)
+        ops.touch_state()  # the replayed kernels update the variables
         self.graph.replay()
         return self.loss
 
@@ -222,6 +224,11 @@ class FusedQDenseStack:
         self.device = layers[0]._kernel.device
         self.loss = torch.zeros((), dtype=torch.float32, device=self.device)
 
+    def invalidate(self):
+        """Forget the cached quantized-weight image (after writing the variables in a way neither version counters nor
+        this package's own updaters see, e.g. through a raw pointer)."""
+        self._versions = None
+
     @staticmethod
     def _layer_vars(layer):
         qs = [layer.iq.quantizer, layer.kq.quantizer] + ([layer.bq.quantizer] if layer.bq is not None else [])
@@ -242,7 +249,10 @@ class FusedQDenseStack:
         need = lib.hgq_mlp_workspace(self._arr, len(self.layers), rows)
         if need < 0:
             self._lib.check(-3, 'hgq_mlp_workspace')
-        versions = [t._version for t in self._vars]
+        for it, layer in zip(self._arr, self.layers):
+            it.decay = layer.iq.quantizer._decay_host  # follows the variable
+        # the kernels of this class do not move version counters or the state epoch: both unchanged = nobody else wrote
+        versions = [t._version for t in self._vars] + [ops.STATE_EPOCH[0]]
         current = self._versions == versions
         if self._ws is None or self._ws.numel() < need:
             self._ws = torch.empty(need, dtype=torch.float32, device=self.device)

@@ -421,3 +421,114 @@ def test_gradient_sink_gives_the_autograd_update(dev, kind):
                 assert torch.equal(pa, pb), f'{name} step {step}'
             else:
                 assert torch.allclose(pa, pb, rtol=1e-6, atol=1e-9), f'{name} step {step}: {float((pa - pb).abs().max()):.3e}'
+
+
+def test_fused_stack_sees_updates_made_by_the_per_layer_optimizer(dev):
+    """Alternating the whole-step kernels with the per-layer path: the fused trainer must not reuse the quantized
+    weight image of its previous step after ``SGD.step`` (which writes through ``.data``) changed the variables."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, FusedQDenseStack, model_loss
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(71)
+    x, y = torch.randn(2048, 16, generator=g).to(dev), torch.randint(0, 5, (2048,), generator=g).to(dev)
+    src = ref.RefMLP(seed=9)
+    models = [qdense_mlp(device=dev) for _ in range(2)]
+    for m in models:
+        _copy_mlp(src, m, dev)
+    fused = [FusedQDenseStack(m, lr=0.01) for m in models]
+    opts = [SGD(m.parameters(), lr=0.5, fold_regularizers=True) for m in models]
+    for f in fused:
+        f.step(x, y)
+    for step in range(3):
+        for m, opt in zip(models, opts):  # a large per-layer update in between
+            opt.zero_grad()
+            opt.backward(model_loss(m, ops.sparse_ce(m(x, training=True), y), True))
+            opt.step()
+        fused[1].invalidate()  # the second one quantizes again whatever it believes
+        la, lb = fused[0].step(x, y), fused[1].step(x, y)
+        assert abs(float(la) - float(lb)) <= 1e-6 * abs(float(lb)), f'loss step {step}'
+        for pa, pb in zip(models[0].parameters(), models[1].parameters()):
+            assert torch.equal(pa, pb), f'step {step}'
+
+
+def test_beta_written_by_the_controllers_reaches_the_device_loss_term(dev):
+    """``BetaScheduler`` / ``BetaPID`` assign the layers' ``beta`` between steps (reference
+    src/hgq/utils/sugar/beta_scheduler.py:21-27, beta_pid.py:49-60).  The kernels read beta through the variable's
+    device address: the EBOPs * beta term of the loss and the bit-width gradients must follow on the per-layer path, in
+    a HIP graph recorded before the change, and in the whole-step kernels."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, FusedQDenseStack, GraphedTrainStep, model_loss
+    from hgq2_amd.utils.models import qdense_mlp
+    from hgq2_amd.utils.sugar import BetaPID, BetaScheduler, FreeEBOPs, PieceWiseSchedule
+
+    g = torch.Generator().manual_seed(72)
+    x, y = torch.randn(2048, 16, generator=g).to(dev), torch.randint(0, 5, (2048,), generator=g).to(dev)
+    src = ref.RefMLP(seed=10)
+    eager, graphed, whole = (qdense_mlp(device=dev) for _ in range(3))
+    for m in (eager, graphed, whole):
+        _copy_mlp(src, m, dev)
+    warm = 2
+    opt = SGD(eager.parameters(), lr=0.01, fold_regularizers=True)
+    fused = FusedQDenseStack(whole, lr=0.01)
+
+    def eager_step():
+        opt.zero_grad()
+        loss = model_loss(eager, ops.sparse_ce(eager(x, training=True), y), True)
+        loss.backward()
+        opt.step()
+        return loss.detach()
+
+    for _ in range(warm):  # the capture below trains `warm` steps on its example batch: same history everywhere
+        eager_step()
+        fused.step(x, y)
+    gstep = GraphedTrainStep(graphed, ops.sparse_ce, SGD(graphed.parameters(), lr=0.01, fold_regularizers=True), x, y, warmup=warm)
+    gstep()
+    eager_step()
+    fused.step(x, y)
+
+    schedule = PieceWiseSchedule([(0, 1e-6, 'log'), (2, 1e-2, 'constant')])
+    cbs = [BetaScheduler(schedule) for _ in range(3)]
+    logger = FreeEBOPs()
+    logger.set_model(eager)
+    for cb, m in zip(cbs, (eager, graphed, whole)):
+        cb.set_model(m)
+    terms = []
+    for epoch in range(4):
+        for cb in cbs:
+            cb.on_epoch_begin(epoch, {})
+        beta = schedule(epoch)
+        assert all(abs(float(layer._beta) - beta) <= 1e-7 * beta for layer in graphed.layers)
+        # the whole-step kernels report the full loss; the other two fold the MonoL1 terms into the update and leave
+        # them out of the reported value
+        with torch.no_grad():
+            reg = float(sum(p.regularizer(p) for p in eager.parameters() if getattr(p, 'regularizer', None) is not None and p.requires_grad))
+        le, lg, lw = eager_step(), gstep(), fused.step(x, y)
+        torch.cuda.synchronize()
+        lw = lw - reg
+        assert abs(float(lg) - float(le)) <= 2e-6 * abs(float(le)), f'graph replay, epoch {epoch}: {float(lg)} vs {float(le)}'
+        assert abs(float(lw) - float(le)) <= 2e-5 * abs(float(le)), f'whole-step kernels, epoch {epoch}: {float(lw)} vs {float(le)}'
+        logs = {}
+        logger.on_epoch_end(epoch, logs)
+        # the loss holds sum(ebops) * beta: compare with the counters the logger reads (state after the update, so loosely)
+        with torch.no_grad():
+            ce = float(ops.sparse_ce(eager(x, training=False), y))
+        terms.append((beta, logs['ebops'], float(le)))
+        for (_, pe), (name, pg) in zip(eager.named_parameters(), graphed.named_parameters()):
+            assert torch.allclose(pe, pg, rtol=1e-5, atol=1e-7), f'{name} epoch {epoch}'
+    # beta rose by four orders of magnitude: the regularisation part of the loss must have risen with it
+    reg_first, reg_last = terms[0][0] * terms[0][1], terms[-1][0] * terms[-1][1]
+    assert reg_last > 1e3 * reg_first
+    assert terms[-1][2] - terms[0][2] > 0.5 * (reg_last - reg_first)
+    # a PID controller reads the device counters and writes beta
+    pid = BetaPID(target_ebops=0.5 * terms[-1][1], init_beta=1e-5, warmup=0, p=1.0, i=0.1)
+    pid.set_model(graphed)
+    pid.on_train_begin({})
+    pid.on_epoch_begin(0, {})
+    before = float(graphed.layers[0]._beta)
+    pid.on_epoch_end(0, {})
+    pid.on_epoch_begin(1, {})
+    after = float(graphed.layers[0]._beta)
+    assert after > before > 0  # above the target: beta is pushed up
+    l1 = gstep()
+    assert torch.isfinite(l1)
