@@ -285,7 +285,7 @@ def _config_cpu_baseline(name, model, x, labels, batch, budget_s=15.0):
         twins = []
         shape = tuple(xc.shape)
         for layer in model.layers:
-            if isinstance(layer, models.Lambda):
+            if isinstance(layer, models.PARAMETER_FREE):
                 twins.append(layer.host_fn)
                 shape = tuple(layer.host_fn(torch.zeros(shape)).shape)
                 continue

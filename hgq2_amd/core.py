@@ -71,10 +71,16 @@ class Constant(Initializer):
     def clone(self):
         return Constant(self.value)
 
+    def get_config(self):
+        return {'value': self.value}
+
 
 class GlorotUniform(Initializer):
     def __init__(self, seed=None):
         self.seed = seed
+
+    def get_config(self):
+        return {'seed': self.seed}
 
     def __call__(self, shape, dtype, device, generator=None):
         shape = tuple(shape)
@@ -131,8 +137,13 @@ def default_device():
 _name_counts: dict[str, int] = {}
 
 
+def base_name(cls_name: str) -> str:
+    """``QDense`` -> ``q_dense``: the stem of a layer's automatic name."""
+    return ''.join('_' + c.lower() if c.isupper() and i else c.lower() for i, c in enumerate(cls_name))
+
+
 def _auto_name(cls_name: str) -> str:
-    base = ''.join('_' + c.lower() if c.isupper() and i else c.lower() for i, c in enumerate(cls_name))
+    base = base_name(cls_name)
     n = _name_counts.get(base, 0)
     _name_counts[base] = n + 1
     return base if n == 0 else f'{base}_{n}'
@@ -249,6 +260,8 @@ class Layer(nn.Module):
             ops.begin_deferred()  # single-workgroup launches that nothing in the forward waits for go out together at the end
         ok = False
         try:
+            if top and args and isinstance(args[0], torch.Tensor):
+                self._last_input_shape = (None,) + tuple(args[0].shape[1:])
             self._maybe_build(args)
             out = self._wrapped_call(*args, training=training, **kwargs)
             ok = True
@@ -268,6 +281,13 @@ class Layer(nn.Module):
     def forward(self, *args, **kwargs):  # nn.Module API
         return self(*args, **kwargs)
 
+    def get_config(self):
+        return {'name': self.name}
+
+    @classmethod
+    def from_config(cls, config):
+        return cls(**config)
+
     def extra_repr(self):
         return f'name={self.name}'
 
@@ -279,6 +299,9 @@ class Sequential(Layer):
 
     def add(self, layer):
         self.layers.append(layer)
+
+    def get_config(self):
+        return {'name': self.name, 'layers': list(self.layers)}
 
     def build(self, input_shape=None):
         self.built = True

@@ -39,6 +39,29 @@ class _Pooling2D(Layer):
     def call(self, x, training=None):
         return ops.pool2d(x, self.pool_size, self.strides, self.padding, self._mode)
 
+    def get_config(self):
+        return {'name': self.name, 'pool_size': self.pool_size, 'strides': self.strides, 'padding': self.padding}
+
+    def host_fn(self, x):
+        """The same pooling on a CPU tensor with library routines (for checks against a CPU model)."""
+        import torch.nn.functional as F
+
+        t = x.permute(0, 3, 1, 2)
+        pads = [0, 0, 0, 0]
+        if self.padding == 'same':
+            pads = []
+            for d in (1, 0):
+                n, k, st = t.shape[2 + d], self.pool_size[d], self.strides[d]
+                total = max((-(-n // st) - 1) * st + k - n, 0)
+                pads += [total // 2, total - total // 2]
+        if self._mode == 'max':
+            y = F.max_pool2d(F.pad(t, pads, value=float('-inf')), self.pool_size, self.strides)
+        else:
+            num = F.avg_pool2d(F.pad(t, pads), self.pool_size, self.strides, divisor_override=1)
+            cnt = F.avg_pool2d(F.pad(torch.ones_like(t[:1, :1]), pads), self.pool_size, self.strides, divisor_override=1)
+            y = num / cnt
+        return y.permute(0, 2, 3, 1)
+
 
 class MaxPooling2D(_Pooling2D):
     _mode = 'max'
@@ -58,6 +81,8 @@ class Flatten(Layer):
     def call(self, x, training=None):
         return x.reshape(x.shape[0], -1)
 
+    host_fn = staticmethod(lambda x: x.reshape(x.shape[0], -1))
+
 
 class GlobalAveragePooling1D(Layer):
     """Mean over the middle axis of a [batch, steps, channels] tensor."""
@@ -69,6 +94,8 @@ class GlobalAveragePooling1D(Layer):
         if x.is_cuda and x.dtype == torch.float32 and x.numel():
             return ops.mean_mid(x)
         return torch.mean(x, dim=1)
+
+    host_fn = staticmethod(lambda x: torch.mean(x, dim=1))
 
 
 layers = SimpleNamespace(MaxPooling2D=MaxPooling2D, AveragePooling2D=AveragePooling2D, Flatten=Flatten,

@@ -67,6 +67,7 @@ class QUnaryFunctionLUT(QLayerBaseSingleInput):
 
     def get_config(self):
         config = super().get_config()
+        config['activation'] = self._act_name  # a named activation; a callable has to be passed again on loading
         config['allow_heterogeneous_table'] = self._allow_heterogeneous_table
         config['allow_heterogeneous_input'] = self._allow_heterogeneous_input
         return config

@@ -57,6 +57,21 @@ class QMultiHeadAttention(QLayerBase):
         self._fuse = fuse.lower()
         self._inverse_sqrt_key_dim = 1.0 / math.sqrt(float(key_dim))
 
+    def get_config(self):
+        config = super().get_config()
+        config.pop('oq_conf', None)
+        config.update({'num_heads': self._num_heads, 'key_dim': self._key_dim, 'value_dim': self._value_dim, 'dropout': self._dropout,
+                       'use_bias': self._use_bias, 'output_shape': self._output_shape, 'kernel_initializer': self._kernel_initializer,
+                       'bias_initializer': self._bias_initializer, 'fuse': self._fuse, 'qkvo_iq_conf': self._qkvo_iq_conf,
+                       'qkvo_kq_conf': self._qkvo_kq_conf, 'qkvo_bq_conf': self._qkvo_bq_conf, 'qkvo_oq_conf': self._qkvo_oq_conf,
+                       'softmax_iq_conf': self._softmax_iq_conf, 'softmax_exp_iq_conf': self._softmax_exp_iq_conf,
+                       'softmax_exp_oq_conf': self._softmax_exp_oq_conf, 'softmax_inv_iq_conf': self._softmax_inv_iq_conf,
+                       'softmax_inv_oq_conf': self._softmax_inv_oq_conf, 'softmax_oq_conf': self._softmax_oq_conf,
+                       'stable_softmax': self._stable_softmax,
+                       'softmax_allow_heterogeneous_table': self._softmax_allow_heterogeneous_table,
+                       'parallelization_factor': self.parallelization_factor})
+        return config
+
     def _sub_kwargs(self):
         return dict(kernel_initializer=self._kernel_initializer, bias_initializer=self._bias_initializer,
                     iq_conf=self._qkvo_iq_conf.copy(), kq_conf=self._qkvo_kq_conf.copy(), bq_conf=self._qkvo_bq_conf.copy(),
@@ -109,7 +124,7 @@ class QMultiHeadAttention(QLayerBase):
             exp_iq_conf=self._softmax_exp_iq_conf, exp_oq_conf=self._softmax_exp_oq_conf,
             inv_iq_conf=self._softmax_inv_iq_conf, inv_oq_conf=self._softmax_inv_oq_conf, oq_conf=self._softmax_oq_conf,
             allow_heterogeneous_table=self._softmax_allow_heterogeneous_table, input_scaler=self._inverse_sqrt_key_dim,
-            enable_ebops=self.enable_ebops)
+            enable_ebops=self.enable_ebops, name=f'{self.name}_softmax')  # a fixed name: variable paths must be reproducible
         self._inverse_sqrt_key_dim = 1.0  # the scale now lives in the softmax's exp table
         self._build_sub(self._softmax, (query_shape[0], N, T, S))
 

@@ -124,6 +124,15 @@ class QConv2D(QLayerBaseSingleInput):
             ebops = ebops + torch.mean(bw_bias) * size
         return ebops
 
+    def get_config(self):
+        config = super().get_config()
+        config.update({'filters': self.filters, 'kernel_size': self.kernel_size, 'strides': self.strides, 'padding': self.padding,
+                       'dilation_rate': self.dilation_rate, 'activation': self._act_name, 'use_bias': self.use_bias,
+                       'kernel_initializer': self.kernel_initializer, 'bias_initializer': self.bias_initializer,
+                       'kq_conf': self.kq.config, 'bq_conf': self.bq.config if self.bq is not None else None,
+                       'parallelization_factor': self.parallelization_factor})
+        return config
+
     def _weight_quantizer_inputs(self):
         """(quantizer, variable) pairs this layer's call quantizes as they are: candidates for the batched launch
         ahead of the forward pass (quantizer/prefetch.py)."""

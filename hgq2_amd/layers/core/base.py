@@ -123,6 +123,7 @@ class QLayerBase(Layer):
 
     def get_config(self):
         return {
+            'name': self.name,
             'enable_ebops': self.enable_ebops,
             'ebops_factor': self.ebops_factor,
             'beta0': self._beta0,

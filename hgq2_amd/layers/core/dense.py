@@ -106,7 +106,8 @@ class QDense(QLayerBaseSingleInput):
         config = super().get_config()
         config.update({'units': self.units, 'activation': self._act_name, 'use_bias': self.use_bias,
                        'kq_conf': self.kq.config, 'bq_conf': self.bq.config if self.bq is not None else None,
-                       'parallelization_factor': self.parallelization_factor})
+                       'parallelization_factor': self.parallelization_factor,
+                       'kernel_initializer': self.kernel_initializer, 'bias_initializer': self.bias_initializer})
         return config
 
     def _weight_quantizer_inputs(self):

@@ -138,6 +138,10 @@ class QEinsumDense(QLayerBaseSingleInput):
             # the bias rides in the GEMM epilogue only when it is exactly one value per output column
             self._bias_in_gemm = bias_shape is not None and prod(bias_shape) == self._N and \
                 tuple(s for s in bias_shape if s != 1) == tuple(s for s in kernel_shape[nc:] if s != 1)
+        if self.enable_oq and not self.oq.built:
+            # the output shape is known only now (the reference's parent class sets it before the base class builds the
+            # output quantizer, src/hgq/layers/core/base.py:183-186)
+            self.try_build_output_quantizer(input_shape)
 
     def compute_output_shape(self, input_shape):
         return (input_shape[0],) + tuple(self.full_output_shape[1:])
@@ -201,7 +205,8 @@ class QEinsumDense(QLayerBaseSingleInput):
         config.update({'equation': self.equation, 'output_shape': self.partial_output_shape, 'bias_axes': self.bias_axes,
                        'activation': self._act_name, 'kq_conf': self.kq.config,
                        'bq_conf': self.bq.config if self.bq is not None else None,
-                       'parallelization_factor': self.parallelization_factor})
+                       'parallelization_factor': self.parallelization_factor,
+                       'kernel_initializer': self.kernel_initializer, 'bias_initializer': self.bias_initializer})
         return config
 
     def _weight_quantizer_inputs(self):

@@ -36,6 +36,14 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         self.normalize_axes = normalize_axes
         self._check_normalize_axes()
 
+    def get_config(self):
+        config = super().get_config()
+        config.update({'normalize_axes': self.normalize_axes, 'momentum': self.momentum, 'epsilon': self.epsilon, 'center': self.center,
+                       'scale': self.scale, 'gamma_initializer': self.gamma_initializer,
+                       'moving_mean_initializer': self.moving_mean_initializer,
+                       'moving_variance_initializer': self.moving_variance_initializer, 'synchronized': self.synchronized})
+        return config
+
     def _check_normalize_axes(self):
         kernel_axes, output_axes = self.equation.split(',')[1].split('->')
         for c in self.normalize_axes:

@@ -67,6 +67,12 @@ class _QWindowPooling2D(QBasePooling):
     def pool(self, inputs):
         return ops.pool2d(inputs, self.pool_size, self.strides, self.padding, self._mode)
 
+    def get_config(self):
+        config = super().get_config()
+        config.update({'pool_size': self.pool_size, 'strides': self.strides, 'padding': self.padding,
+                       'parallelization_factor': self.parallelization_factor})
+        return config
+
 
 class QMaxPooling2D(_QWindowPooling2D):
     _mode = 'max'
@@ -85,6 +91,11 @@ class _QGlobalPooling(QBasePooling):
             raise NotImplementedError('pooling: channels_last only')
         super().__init__(**kwargs)
         self.keepdims = keepdims
+
+    def get_config(self):
+        config = super().get_config()
+        config.update({'keepdims': self.keepdims, 'parallelization_factor': self.parallelization_factor})
+        return config
 
     def compute_output_shape(self, input_shape):
         if self.keepdims:

@@ -75,6 +75,15 @@ class QSoftmax(QLayerBaseSingleInput):
             name=f'{self.name}_exp_table', enable_ebops=self.enable_ebops and stable, beta0=self._beta0.clone())
         self.supports_masking = True
 
+    def get_config(self):
+        config = super().get_config()
+        config.update({'axes': tuple(self.axes), 'stable': self.stable, 'exp_oq_conf': self.exp_table.oq.config,
+                       'exp_iq_conf': self.exp_table.iq.config if self.stable else None,
+                       'inv_oq_conf': self.inv_table.oq.config, 'inv_iq_conf': self.inv_table.iq.config,
+                       'allow_heterogeneous_table': self._allow_heterogeneous_table, 'input_scaler': self.input_scaler,
+                       'parallelization_factor': self.parallelization_factor})
+        return config
+
     def build(self, input_shape):
         self.exp_table._build_device = self._build_device
         self.exp_table.build(tuple(input_shape))

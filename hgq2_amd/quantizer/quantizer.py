@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from ..core import Layer
+from ..core import Layer, base_name
 from .config import QuantizerConfig, all_quantizer_keys
 
 
@@ -21,6 +21,9 @@ class Quantizer(Layer):
         self.scaler = config.scaler
         self.affine = config.affine
         self.quantizer = config.get_quantizer()
+        # the one inner quantizer is named after its class alone: variable paths must not depend on how many
+        # quantizers the process has created before
+        self.quantizer.name = base_name(type(self.quantizer).__name__)
 
     def build(self, input_shape):
         if not self.quantizer.built:
@@ -57,7 +60,7 @@ class Quantizer(Layer):
         return self.scaler is None and self.qnoise_factor is None and self.affine is None
 
     def get_config(self):
-        return {'config': self.config}
+        return {'name': self.name, 'config': self.config}
 
     @property
     def bits(self):

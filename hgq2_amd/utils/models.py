@@ -4,7 +4,7 @@ from __future__ import annotations
 
 from ..config import LayerConfigScope, QuantizerConfigScope
 from ..core import Sequential, set_default_device
-from .. import ops
+from .. import host, ops
 from ..core import Layer
 from ..layers import QConv2D, QDense, QEinsumDenseBatchnorm, QMultiHeadAttention
 
@@ -57,39 +57,29 @@ class Lambda(Layer):
         return self.fn(x)
 
 
+# layers without variables between the quantized ones; each has ``host_fn``, the same step on CPU tensors
+PARAMETER_FREE = (Lambda, host.MaxPooling2D, host.AveragePooling2D, host.Flatten, host.GlobalAveragePooling1D)
+
+
 def particle_mlp(n_particles=64, n_features=16, hidden=(64, 32), n_out=5, beta0=1e-5, device=None):
     """Per-particle network: QEinsumDenseBatchnorm('bpf,fh->bph') x len(hidden) with ReLU, mean over the
     particles, QDense(n_out)."""
-    import torch
-
     if device is not None:
         set_default_device(device)
     with _Scopes(beta0):
         layers = [QEinsumDenseBatchnorm('bpf,fh->bph', (n_particles, h), bias_axes='h', activation='relu') for h in hidden]
-        layers.append(Lambda(lambda t: ops.mean_mid(t) if t.is_cuda else torch.mean(t, dim=1), lambda t: torch.mean(t, dim=1),
-                             name='mean_over_particles'))
+        layers.append(host.GlobalAveragePooling1D(name='mean_over_particles'))
         layers.append(QDense(n_out))
     return Sequential(layers)
 
 
 def conv_stack(filters=32, n_out=10, beta0=1e-5, device=None):
     """QConv2D 3x3 ReLU -> MaxPool 2x2 -> QConv2D 3x3 ReLU -> Flatten -> QDense(n_out), channels-last."""
-    import torch
-    import torch.nn.functional as F
-
     if device is not None:
         set_default_device(device)
-
-    def pool(t):  # NHWC max-pool 2x2, stride 2, 'valid', in the pooling kernels
-        return ops.pool2d(t, (2, 2), (2, 2), 'valid', 'max')
-
-    def pool_host(t):
-        return F.max_pool2d(t.permute(0, 3, 1, 2), 2, 2).permute(0, 2, 3, 1)
-
     with _Scopes(beta0):
-        layers = [QConv2D(filters, (3, 3), activation='relu'), Lambda(pool, pool_host, name='max_pool'),
-                  QConv2D(filters, (3, 3), activation='relu'), Lambda(lambda t: t.reshape(t.shape[0], -1), name='flatten'),
-                  QDense(n_out)]
+        layers = [QConv2D(filters, (3, 3), activation='relu'), host.MaxPooling2D((2, 2), name='max_pool'),
+                  QConv2D(filters, (3, 3), activation='relu'), host.Flatten(name='flatten'), QDense(n_out)]
     return Sequential(layers)
 
 

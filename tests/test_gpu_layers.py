@@ -532,3 +532,50 @@ def test_beta_written_by_the_controllers_reaches_the_device_loss_term(dev):
     assert after > before > 0  # above the target: beta is pushed up
     l1 = gstep()
     assert torch.isfinite(l1)
+
+
+@pytest.mark.parametrize('kind', ['mlp', 'particle', 'conv', 'mha'])
+def test_saved_and_loaded_model_gives_equal_outputs(dev, kind, tmp_path):
+    """The reference's serialization test (tests/base.py:184-201): train a little, calibrate, save, load into a model
+    rebuilt from the saved configuration, compare the inference outputs for equality.  Container: ``.npz`` keyed by
+    variable path (``hgq2_amd.saving``); the load must also restore what a checkpoint is for - continuing to train gives
+    the same next step."""
+    from hgq2_amd import ops, saving
+    from hgq2_amd.train import SGD, model_loss
+    from hgq2_amd.utils import models
+
+    g = torch.Generator().manual_seed(81)
+    torch.manual_seed(81)
+    if kind == 'mlp':
+        x, model = torch.randn(512, 16, generator=g), models.qdense_mlp(device=dev)
+    elif kind == 'particle':
+        x, model = torch.randn(128, 16, 16, generator=g), models.particle_mlp(n_particles=16, device=dev)
+    elif kind == 'conv':
+        x, model = torch.rand(32, 28, 28, 1, generator=g), models.conv_stack(device=dev)
+    else:
+        x, model = torch.randn(32, 64, 64, generator=g), models.mha_block(device=dev)
+    xd = x.to(dev)
+
+    def train_step(m):
+        opt = SGD(m.parameters(), lr=0.05, fold_regularizers=True)
+        opt.zero_grad()
+        out = m(xd, training=True)
+        opt.backward(model_loss(m, ops.mse(out), True))
+        opt.step()
+
+    for _ in range(2):
+        train_step(model)
+    file = tmp_path / f'{kind}.npz'
+    saving.save_model(model, file)
+    clone = saving.load_model(file, device=dev)
+    with torch.no_grad():
+        want, got = model(xd, training=False), clone(xd, training=False)
+    assert torch.equal(got, want)
+    for (na, ta), (nb, tb) in zip(saving.variable_paths(model).items(), saving.variable_paths(clone).items()):
+        assert na == nb and ta.dtype == tb.dtype
+        assert torch.equal(ta.view(torch.int32) if ta.dtype == torch.uint32 else ta, tb.view(torch.int32) if tb.dtype == torch.uint32 else tb), na
+    train_step(model)
+    train_step(clone)
+    for (na, ta), (_, tb) in zip(saving.variable_paths(model).items(), saving.variable_paths(clone).items()):
+        if ta.dtype == torch.float32:
+            assert torch.allclose(ta, tb, rtol=1e-6, atol=1e-9), f'{na} after one more step'
