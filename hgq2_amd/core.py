@@ -206,9 +206,13 @@ class Layer(nn.Module):
         return out
 
     def _clear_losses(self):
-        for m in self.modules():
-            if isinstance(m, Layer):
-                m._losses = []
+        layers = self.__dict__.get('_hgq_layer_list')
+        n = sum(1 for _ in self.modules())
+        if layers is None or layers[0] != n:
+            layers = (n, [m for m in self.modules() if isinstance(m, Layer)])
+            object.__setattr__(self, '_hgq_layer_list', layers)
+        for m in layers[1]:
+            m.__dict__['_losses'] = []
 
     def apply_constraints(self):
         """What a Keras optimizer does after each update."""

@@ -1039,6 +1039,125 @@ __global__ __launch_bounds__(1024) void conv_ebops_kernel(const float *__restric
     }
 }
 
+// The same estimate straight from the quantizers' raw variables, as one launch for the whole `_compute_ebops` of a
+// convolution layer: bits are formed on the fly (hgq_qbits_fwd's rule), the bias term, the scale factors, the uint32
+// variable, the loss term ebops * beta and the gradients of that term with respect to the variables (straight-through
+// rounding, hgq_qbits_bwd's rule) all come out of it.  Every operand must have one bit-width entry per cell.
+__device__ __forceinline__ float ce_bits(const hgq_bits_desc &d, uint32_t j, bool &open) {
+    float b;
+    open = true;
+    if (d.kbi) {
+        b = rintf(d.fb[j]);
+    } else {
+        const float sum = __fadd_rn(rintf(d.i[j]), rintf(d.fb[j]));
+        open = sum > 0.f;
+        b = open ? sum : 0.f;
+    }
+    if (d.add_mode == 1) b = __fadd_rn(b, (float)d.k[j]);
+    else if (d.add_mode == 2) b = __fadd_rn(b, (float)d.k[j] * (b > 0.f ? 1.f : 0.f));
+    return b;
+}
+__device__ __forceinline__ void ce_put(const hgq_bits_desc &d, uint32_t j, bool open, float g) {
+    if (d.kbi) {
+        d.g_fb[j] = g;
+    } else {
+        d.g_i[j] = open ? g : 0.f, d.g_fb[j] = open ? g : 0.f;
+    }
+}
+
+__global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, hgq_bits_desc dker, hgq_bits_desc dbias, int has_bias,
+                                                            hgq_conv_geom g, int F, float conv_scale, float bias_size, float factor,
+                                                            const float *beta, uint32_t *ebops_u32, float *loss_term) {
+    __shared__ float S[CE_MAX], R[CE_MAXR];
+    __shared__ int Ws[CE_MAX];
+    __shared__ float red[1024];
+    __shared__ unsigned char vy[CE_MAXV], vx[CE_MAXV];
+    const int t = threadIdx.x, taps = g.kh * g.kw, TC = taps * g.C, WC = g.W * g.C;
+    const FastDiv by_wc((uint32_t)WC), by_f((uint32_t)F), by_c((uint32_t)g.C), by_kw((uint32_t)g.kw);
+    for (int e = t; e < TC; e += 1024) Ws[e] = 0;
+    for (int e = t; e < g.H * g.kh; e += 1024) {
+        const int y = e / g.kh, ky = e - y * g.kh, ty = y + g.py - ky * g.dly;
+        vy[e] = ty >= 0 && ty % g.sy == 0 && ty / g.sy < g.OH;
+    }
+    for (int e = t; e < g.W * g.kw; e += 1024) {
+        const int x = e / g.kw, kx = e - x * g.kw, tx = x + g.px - kx * g.dlx;
+        vx[e] = tx >= 0 && tx % g.sx == 0 && tx / g.sx < g.OW;
+    }
+    for (int e = t; e < g.kh * WC; e += 1024) {
+        const int ky = (int)by_wc.div((uint32_t)e), xc = e - ky * WC;
+        float r = 0.f;
+        for (int oy = 0; oy < g.OH; ++oy) {
+            const int iy = oy * g.sy - g.py + ky * g.dly;
+            bool open;
+            if ((unsigned)iy < (unsigned)g.H) r += ce_bits(din, (uint32_t)(iy * WC + xc), open);
+        }
+        R[e] = r;
+    }
+    __syncthreads();
+    const int n_w = TC * F;
+    for (int e = t; e < n_w; e += 1024) {
+        bool open;
+        atomicAdd(&Ws[by_f.div((uint32_t)e)], (int)ce_bits(dker, (uint32_t)e, open));
+    }
+    for (int e = t; e < TC; e += 1024) {
+        const int tap = (int)by_c.div((uint32_t)e), c = e - tap * g.C, ky = (int)by_kw.div((uint32_t)tap), kx = tap - ky * g.kw;
+        float sacc = 0.f;
+        for (int ox = 0; ox < g.OW; ++ox) {
+            const int ix = ox * g.sx - g.px + kx * g.dlx;
+            if ((unsigned)ix < (unsigned)g.W) sacc += R[ky * WC + ix * g.C + c];
+        }
+        S[e] = sacc;
+    }
+    __syncthreads();
+    float part = 0.f;
+    for (int e = t; e < TC; e += 1024) part += S[e] * (float)Ws[e];
+    red[t] = part;
+    __syncthreads();
+    for (int o = 512; o > 0; o >>= 1) {
+        if (t < o) red[t] += red[t + o];
+        __syncthreads();
+    }
+    const float conv_total = red[0];
+    __syncthreads();
+    float bias_sum = 0.f;
+    if (has_bias) {
+        float bs = 0.f;
+        for (int n = t; n < F; n += 1024) {
+            bool open;
+            bs += ce_bits(dbias, (uint32_t)n, open);
+        }
+        red[t] = bs;
+        __syncthreads();
+        for (int o = 512; o > 0; o >>= 1) {
+            if (t < o) red[t] += red[t + o];
+            __syncthreads();
+        }
+        bias_sum = red[0];
+    }
+    // the reference's order: sum(conv) * (pf / n_parallel) + mean(bits_bias) * size, then * ebops_factor
+    const float ebops = __fmul_rn(__fadd_rn(__fmul_rn(conv_total, conv_scale), has_bias ? __fmul_rn(__fdiv_rn(bias_sum, (float)F), bias_size) : 0.f), factor);
+    const float gs = beta[0] * factor;  // gradients are those of the loss term ebops * beta
+    if (t == 0) {
+        if (ebops_u32) ebops_u32[0] = (uint32_t)ebops;
+        loss_term[0] = ebops * beta[0];
+    }
+    for (int e = t; e < n_w; e += 1024) ce_put(dker, (uint32_t)e, true, S[by_f.div((uint32_t)e)] * conv_scale * gs);
+    for (int e = t; e < g.H * WC; e += 1024) {
+        const int y = (int)by_wc.div((uint32_t)e), xc = e - y * WC, x = (int)by_c.div((uint32_t)xc), c = xc - x * g.C;
+        float a = 0.f;
+        for (int ky = 0; ky < g.kh; ++ky) {
+            if (!vy[y * g.kh + ky]) continue;
+            for (int kx = 0; kx < g.kw; ++kx)
+                if (vx[x * g.kw + kx]) a += (float)Ws[(ky * g.kw + kx) * g.C + c];
+        }
+        bool open;
+        (void)ce_bits(din, (uint32_t)e, open);
+        ce_put(din, (uint32_t)e, open, a * conv_scale * gs);
+    }
+    if (has_bias)
+        for (int n = t; n < F; n += 1024) ce_put(dbias, (uint32_t)n, true, bias_size / (float)F * gs);
+}
+
 static int check_geom(const hgq_conv_geom *g, int F, const char *who) {
     if (!g) return fail(HGQ_ERR_ARG, "%s: null geometry", who);
     if (g->B < 0 || g->H < 1 || g->W < 1 || g->C < 1 || g->kh < 1 || g->kw < 1 || g->sy < 1 || g->sx < 1 || g->dly < 1 ||
@@ -1281,4 +1400,32 @@ extern "C" int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, con
         return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops: needs kh * kw * C * F and H * W * C below 2**21 (flat sweeps of one workgroup)");
     hipLaunchKernelGGL(conv_ebops_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, bits_in, bits_ker, *g, F, total, g_bits_in, g_bits_ker);
     return check_launch("hgq_conv2d_ebops");
+}
+
+extern "C" int hgq_conv2d_ebops_q(const hgq_bits_desc *bits_in, const hgq_bits_desc *bits_ker, const hgq_bits_desc *bits_bias,
+                                  const hgq_conv_geom *g, int F, float conv_scale, float bias_size, float ebops_factor, const float *beta,
+                                  uint32_t *ebops_u32, float *loss_term, void *stream) {
+    int rc = check_geom(g, F, "hgq_conv2d_ebops_q");
+    if (rc) return rc;
+    if (!bits_in || !bits_ker || !beta || !loss_term) return fail(HGQ_ERR_ARG, "hgq_conv2d_ebops_q: null pointer");
+    if ((int64_t)g->kh * g->kw * g->C > CE_MAX || (int64_t)g->kh * g->W * g->C > CE_MAXR || (int64_t)g->H * g->kh > CE_MAXV ||
+        (int64_t)g->W * g->kw > CE_MAXV)
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops_q: needs kh * kw * C <= %d, kh * W * C <= %d, H * kh and W * kw <= %d", CE_MAX,
+                    CE_MAXR, CE_MAXV);
+    const int64_t n_in = (int64_t)g->H * g->W * g->C, n_w = (int64_t)g->kh * g->kw * g->C * F;
+    if ((int64_t)g->kh * g->kw * g->C * g->OH * g->OW >= (1ll << 31) || n_w >= (1ll << 21) || n_in >= (1ll << 21))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops_q: needs kh * kw * C * F and H * W * C below 2**21 (flat sweeps of one workgroup)");
+    const hgq_bits_desc *ds[3] = {bits_in, bits_ker, bits_bias};
+    const int64_t cells[3] = {n_in, n_w, (int64_t)F};
+    for (int t = 0; t < 3; ++t) {
+        if (!ds[t]) continue;
+        if (ds[t]->size != cells[t] || ds[t]->inner != 1)
+            return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_ebops_q: operand %d must have one bit-width entry per cell", t);
+        if (!ds[t]->fb || !ds[t]->g_fb || (!ds[t]->kbi && (!ds[t]->i || !ds[t]->g_i)) || (ds[t]->add_mode && !ds[t]->k))
+            return fail(HGQ_ERR_ARG, "hgq_conv2d_ebops_q: null pointer in operand %d", t);
+    }
+    hgq_bits_desc none = *bits_ker;
+    hipLaunchKernelGGL(conv_ebops_q_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, *bits_in, *bits_ker, bits_bias ? *bits_bias : none,
+                       bits_bias ? 1 : 0, *g, F, conv_scale, bias_size, ebops_factor, beta, ebops_u32, loss_term);
+    return check_launch("hgq_conv2d_ebops_q");
 }

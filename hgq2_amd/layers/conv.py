@@ -110,6 +110,22 @@ class QConv2D(QLayerBaseSingleInput):
             outputs = self.activation(outputs)
         return outputs
 
+    def _ebops_loss_term(self, shape):
+        # the whole estimate, the uint32 variable, the loss term and the bit-width gradients in one launch where every
+        # quantizer has one bit-width entry per cell
+        if self.enable_iq and self._beta is not None and self._beta.is_cuda:
+            operands = [self.iq.bits_operand(shape), self.kq.bits_operand(tuple(self._kernel.shape)),
+                        self.bq.bits_operand((self.filters,)) if self.bq is not None else None]
+            cells = [prod(shape), self._kernel.numel(), self.filters]
+            ok = all(op is None or (op[3] == n and op[4] == 1) for op, n in zip(operands, cells)) and operands[0] is not None \
+                and operands[1] is not None and (self.bq is None or operands[2] is not None)
+            if ok and ops.conv2d_ebops_supported(tuple(shape), tuple(self._kernel.shape)):
+                geom = ops.conv_geometry(tuple(shape), tuple(self._kernel.shape), self.strides, self.padding, self.dilation_rate)
+                size = float(prod(shape[:-1]) * self.filters)
+                return ops.bits_ebops('conv', operands, (tuple(geom), self.filters, self.parallelization_factor / self.n_parallel, size,
+                                                         float(self.ebops_factor)), self._beta, self._ebops)
+        return super()._ebops_loss_term(shape)
+
     def _compute_ebops(self, shape):
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self._kernel.shape)

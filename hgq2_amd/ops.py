@@ -1604,6 +1604,10 @@ class _BitsEbops(torch.autograd.Function):
         elif kind == 'softmax':
             rows, L, f1, f2 = params
             rc = lib.hgq_softmax_ebops(ptrs[0], ptrs[1], ptrs[2], rows, L, f1, f2, _ptr(beta), _ptr(ebops_var), _ptr(out), _stream())
+        elif kind == 'conv':
+            geom, F, conv_scale, bias_size, factor = params
+            rc = lib.hgq_conv2d_ebops_q(ptrs[0], ptrs[1], ptrs[2], ctypes.byref(_geom(geom)), F, conv_scale, bias_size, factor, _ptr(beta),
+                                        _ptr(ebops_var), _ptr(out), _stream())
         else:
             T, S, N, H, Hv, f1, f2 = params
             rc = lib.hgq_mha_ebops(ptrs[0], ptrs[1], ptrs[2], ptrs[3], T, S, N, H, Hv, f1, f2, _ptr(beta), _ptr(ebops_var), _ptr(out),
@@ -1648,7 +1652,7 @@ class _BitsEbops(torch.autograd.Function):
 def bits_ebops(kind: str, operands, params, beta: Tensor, ebops_var: Tensor, owners=None) -> Tensor:
     """Loss term ``ebops * beta`` of a layer whose EBOPs are algebra on bit-width tensors, in one launch; also assigns
     the uint32 variable.  ``operands``: per operand ``None`` or ``(k, i, fb, size, inner, kbi, add_mode)`` (``i`` is
-    ``None`` for the (k, b, i) kind); ``params`` as the C entry point of ``kind`` ('lut', 'softmax', 'mha') takes them;
+    ``None`` for the (k, b, i) kind); ``params`` as the C entry point of ``kind`` ('lut', 'softmax', 'mha', 'conv') takes them;
     ``owners``: per operand ``None`` or the variables ``(i, fb)`` behind it (see :class:`side_gradients`)."""
     e_f = beta.new_empty(0)
     e_k = torch.empty(0, dtype=torch.uint8, device=beta.device)
@@ -1882,3 +1886,38 @@ def _route(owner, grad):
         return grad  # no room left in the update kernel's descriptor: autograd accumulates this one
     _stash_side(owner, None, grad.contiguous())
     return None
+
+
+# ======================================================================================
+# eager fast path
+# ======================================================================================
+# Every ``hgq::*`` operator above is registered with the dispatcher (fake tensors, tracing and ``torch.ops.hgq.*`` see
+# it).  A call through the dispatcher costs the host some tens of microseconds - schema matching, the autograd and
+# in-place bookkeeping layers the registration adds - which is several times the launch it wraps.  Inside this module the
+# operators are only ever called from ``torch.autograd.Function`` bodies (no gradient mode, arguments already validated
+# by the implementation itself), so when no dispatch mode is active the registered implementation is called directly.
+def _direct(op):
+    impl = op._init_fn
+
+    def call(*args, **kwargs):
+        if torch._C._len_torch_dispatch_stack() or torch.compiler.is_compiling():
+            return op(*args, **kwargs)
+        return impl(*args, **kwargs)
+
+    call.__name__ = getattr(impl, '__name__', 'op')
+    call.__doc__ = impl.__doc__
+    call.op = op  # the dispatcher-registered operator
+    call.register_fake = op.register_fake
+    return call
+
+
+def _install_direct_calls():
+    from torch._library.custom_ops import CustomOpDef
+
+    g = globals()
+    for name, obj in list(g.items()):
+        if isinstance(obj, CustomOpDef):
+            g[name] = _direct(obj)
+
+
+_install_direct_calls()

@@ -39,16 +39,27 @@ def quantize_together(pairs, training):
     return [q(x, training=training) for q, x in pairs]
 
 
+def _plan(root):
+    """The layers under ``root`` that declare kernel / bias quantizers; cached on ``root`` until its module tree changes
+    (the set of modules and their built flags)."""
+    mods = list(root.modules())
+    key = (len(mods), sum(1 for m in mods if getattr(m, 'built', False)))
+    cached = getattr(root, '_hgq_prefetch_plan', None)
+    if cached is None or cached[0] != key:
+        cached = (key, [m for m in mods if hasattr(m, '_weight_quantizer_inputs')])
+        object.__setattr__(root, '_hgq_prefetch_plan', cached)
+    return cached[1]
+
+
 def prefetch_weight_quantizers(root) -> int:
     """Quantize the kernels and biases of every layer under ``root`` that declares them (``_weight_quantizer_inputs``)
     in one launch and leave each result with its quantizer for the layer's own call to pick up.  Returns the number
     of quantizers served (0: fewer than two were eligible, nothing was done)."""
     pairs = []
-    for m in root.modules():
-        fn = getattr(m, '_weight_quantizer_inputs', None)
-        if fn is None or not getattr(m, 'built', False):
+    for m in _plan(root):
+        if not getattr(m, 'built', False):
             continue
-        for q, p in fn():
+        for q, p in m._weight_quantizer_inputs():
             fq = _eligible(q, p)
             if fq is not None:
                 fq._prefetched = None

@@ -501,6 +501,18 @@ int hgq_mha_ebops(const hgq_bits_desc *bits_q, const hgq_bits_desc *bits_k, cons
                   float *loss_term, void *stream);
 
 /*
+ * The whole QBaseConv._compute_ebops (src/hgq/layers/conv.py:91-102) and the scalar tail of the call wrapper
+ * (src/hgq/layers/core/base.py:101-104) from the quantizers' raw variables, in one launch:
+ *     ebops = (sum(conv(bits_in, bits_ker)) * conv_scale + mean(bits_bias) * bias_size) * ebops_factor
+ * by the closed form of hgq_conv2d_ebops; uint32 variable (may be NULL), loss_term[0] = ebops * beta, gradients of the
+ * loss term into the descriptors.  Every operand needs one bit-width entry per cell (size = cells, inner = 1):
+ * bits_in over [H, W, C], bits_ker over [kh, kw, C, F], bits_bias (may be NULL) over [F]; limits as hgq_conv2d_ebops.
+ */
+int hgq_conv2d_ebops_q(const hgq_bits_desc *bits_in, const hgq_bits_desc *bits_ker, const hgq_bits_desc *bits_bias,
+                       const hgq_conv_geom *g, int F, float conv_scale, float bias_size, float ebops_factor, const float *beta,
+                       uint32_t *ebops_u32, float *loss_term, void *stream);
+
+/*
  * The scalar tail of QLayerBase.call (src/hgq/layers/core/base.py:101-104):
  *     ebops = ebops * ebops_factor;  self._ebops.assign(cast(ebops, uint32));  loss term = ebops * beta
  * forward writes the uint32 variable (may be NULL) and out [1]; backward: d_ebops = (g * beta) * factor.

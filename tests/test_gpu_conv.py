@@ -178,3 +178,44 @@ def test_conv_ebops_closed_form_is_exact(dev, case):
     assert abs(float(got) - float(want)) <= (0 if float(want) < 2**24 else 1e-6 * float(want))
     assert torch.equal(bip.grad.cpu().double(), 3.0 * bir.grad.double())
     assert torch.equal(bkp.grad.cpu().double(), 3.0 * bkr.grad.double())
+
+
+@pytest.mark.parametrize('case', [(12, 10, 3, (3, 3), 6, (1, 1), 'valid', 'SAT'), (9, 9, 4, (3, 2), 5, (2, 1), 'same', 'WRAP'),
+                                  (8, 11, 2, (2, 3), 4, (2, 3), 'same', 'SAT_SYM')])
+def test_one_launch_conv_ebops_term_equals_the_composed_path(dev, case):
+    """The loss term ebops * beta of a QConv2D from the raw quantizer variables in one launch (``hgq_conv2d_ebops_q``)
+    against the same layer's generic path (bit-width views, closed-form convolution sum, library algebra for the bias
+    term and the factors, autograd): value, uint32 variable, and the gradient of every bit-width variable."""
+    from hgq2_amd.config import QuantizerConfig
+    from hgq2_amd.layers import QConv2D
+    from hgq2_amd.layers.core.base import QLayerBase
+    from tests.test_gpu_more_layers import _perturb, readme_scopes
+
+    H, W, C, ksize, Fo, strides, padding, iq_over = case
+    g = torch.Generator().manual_seed(H * W + C)
+    with readme_scopes(beta0=3e-4):
+        layer = QConv2D(Fo, ksize, strides=strides, padding=padding, parallelization_factor=3,
+                        iq_conf=QuantizerConfig('kif', 'datalane', overflow_mode=iq_over))
+    layer.ebops_factor = 1.5
+    x = torch.randn(4, H, W, C, generator=g).to(dev)
+    layer(x, training=True)
+    _perturb(layer, g)
+    with torch.no_grad():  # closed straight-through gates and empty words among the entries
+        layer.iq.quantizer._f.view(-1)[::5] = -9.0
+        layer.kq.quantizer._b.view(-1)[::7] = 0.0
+    variables = [layer.iq.quantizer._f, layer.kq.quantizer._b, layer.bq.quantizer._b]
+    if layer.iq.quantizer._i.requires_grad:
+        variables.append(layer.iq.quantizer._i)
+    shape = (1, H, W, C)
+    results = []
+    for fused in (True, False):
+        for v in variables:
+            v.grad = None
+        term = layer._ebops_loss_term(shape) if fused else QLayerBase._ebops_loss_term(layer, shape)
+        (term * 2.0).backward()
+        results.append((float(term), int(layer._ebops.cpu().view(torch.int32)), [v.grad.clone() for v in variables]))
+    (t1, e1, g1), (t0, e0, g0) = results
+    assert e1 == e0 and e0 > 0
+    assert abs(t1 - t0) <= 1e-6 * abs(t0)
+    for a, b, v in zip(g1, g0, variables):
+        assert torch.allclose(a, b, rtol=1e-6, atol=1e-12), float((a - b).abs().max())
