@@ -74,6 +74,8 @@ SIGNATURES = {
     'hgq_quantize_bwd_sliced': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_conv2d_ebops_q': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_dense_ebops_multi': (c_int, [c_void_p, c_int, c_void_p]),
+    'hgq_qdense_bwd_slices': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 3 + [c_int, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_reduce_slices_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_stream_probe': (c_int, [c_void_p] * 6 + [c_int, c_int, c_int64, c_void_p]),
     'hgq_quantize_bwd_static': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_fwd_multi': (c_int, [c_void_p, c_int, c_void_p]),

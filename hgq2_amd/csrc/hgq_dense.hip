@@ -889,6 +889,79 @@ int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t 
     return check_launch("reduce_parts");
 }
 
+// The same reduction for several independent slice sets in one launch: block b serves the set whose block range holds b.
+struct ReduceBatch {
+    hgq_reduce_item item[HGQ_REDUCE_BATCH];
+    int first_block[HGQ_REDUCE_BATCH + 1];
+    int count;
+};
+
+__global__ __launch_bounds__(64 * RP_G) void reduce_parts_multi_kernel(const ReduceBatch b) {
+    __shared__ float red[64 * RP_G];
+    int t = 0;
+    while (t + 1 < b.count && (int)blockIdx.x >= b.first_block[t + 1]) ++t;
+    const hgq_reduce_item &it = b.item[t];
+    const float *__restrict__ part = it.slices;
+    const int n_parts = it.n_slices;
+    const int64_t M = it.width;
+    const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int64_t e = (int64_t)((int)blockIdx.x - b.first_block[t]) * 64 + e_local;
+    float s = 0.f;
+    if (e < M) {
+        const int per = (n_parts + RP_G - 1) / RP_G;
+        const int g0 = grp * per, g1 = min(n_parts, g0 + per);
+        int g = g0;
+        for (; g + 8 <= g1; g += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = part[(int64_t)(g + u) * M + e];
+            s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+        }
+        for (; g < g1; ++g) s += part[(int64_t)g * M + e];
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    if (grp == 0 && e < M) {
+        float v = 0.f;  // groups in order: the same association as reduce_parts_kernel
+#pragma unroll
+        for (int w = 0; w < RP_G; w += 4)
+            v += (red[e_local + 64 * w] + red[e_local + 64 * (w + 1)]) + (red[e_local + 64 * (w + 2)] + red[e_local + 64 * (w + 3)]);
+        int64_t off = e;
+#pragma unroll
+        for (int o = 0; o < 3; ++o) {
+            if (off < it.n_out[o]) {
+                if (it.out[o]) it.out[o][off] = v;
+                break;
+            }
+            off -= it.n_out[o];
+        }
+    }
+}
+
+extern "C" int hgq_reduce_slices_multi(const hgq_reduce_item *items, int count, void *stream) {
+    if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_reduce_slices_multi: bad arguments");
+    for (int base = 0; base < count; base += HGQ_REDUCE_BATCH) {
+        ReduceBatch b;
+        b.count = count - base < HGQ_REDUCE_BATCH ? count - base : HGQ_REDUCE_BATCH;
+        int64_t blocks = 0;
+        for (int t = 0; t < b.count; ++t) {
+            const hgq_reduce_item &it = items[base + t];
+            if (it.n_slices < 1 || it.width < 1 || !it.slices) return fail(HGQ_ERR_ARG, "hgq_reduce_slices_multi: bad sizes in item %d", base + t);
+            if (it.n_out[0] < 0 || it.n_out[1] < 0 || it.n_out[2] < 0 || it.n_out[0] + it.n_out[1] + it.n_out[2] != it.width)
+                return fail(HGQ_ERR_ARG, "hgq_reduce_slices_multi: item %d: output lengths do not add up to the slice width", base + t);
+            b.item[t] = it;
+            b.first_block[t] = (int)blocks;
+            blocks += (it.width + 63) / 64;
+            if (blocks > (1 << 24)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_reduce_slices_multi: too many columns");
+        }
+        for (int t = b.count; t <= HGQ_REDUCE_BATCH; ++t) b.first_block[t] = (int)blocks;
+        hipLaunchKernelGGL(reduce_parts_multi_kernel, dim3((unsigned)blocks), dim3(64 * RP_G), 0, (hipStream_t)stream, b);
+        int rc = check_launch("hgq_reduce_slices_multi");
+        if (rc) return rc;
+    }
+    return HGQ_OK;
+}
+
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
 static inline int row_parts(int64_t rows, int bm) {
@@ -1047,9 +1120,10 @@ extern "C" int hgq_dense_moments_bwd(const float *x, const float *w, const float
     return hgq_qdense_moments_bwd(x, nullptr, 0, 0, w, dmean, dmeansq, nullptr, dx, dw, nullptr, workspace, rows, K, N, stream);
 }
 
-extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
-                              const float *qw, float *dx, float *dqw, float *dqb, float *df_in, float *workspace,
-                              int64_t rows, int K, int N, int act, int mode, void *stream) {
+// Launches the backward kernel; the slices are reduced here (reduce == true) or left in the workspace for the caller.
+static int qdense_bwd_impl(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows, const float *qw, float *dx,
+                           float *dqw, float *dqb, float *df_in, float *workspace, int64_t rows, int K, int N, int act, int mode,
+                           void *stream, bool reduce) {
     hipStream_t s = (hipStream_t)stream;
     if (rows < 0 || K < 1 || N < 1 || bw_rows < 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: bad sizes");
     if (K > 64 || N > 64) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_bwd: K=%d N=%d exceed the fused kernel's 64 x 64", K, N);
@@ -1066,6 +1140,7 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
     const int64_t M = (int64_t)K * N + N + PK;
     if (rows == 0) {
         int rc;
+        if (!reduce) return fill_f32(workspace, 0.f, M, s);  // one slice of zeros
         if (dqw && (rc = fill_f32(dqw, 0.f, (int64_t)K * N, s))) return rc;
         if (dqb && (rc = fill_f32(dqb, 0.f, N, s))) return rc;
         if (df_in && (rc = fill_f32(df_in, 0.f, PK, s))) return rc;
@@ -1092,7 +1167,7 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
         else HGQ_BWD_FAST(HGQ_RND_CONV, true);
 #undef HGQ_BWD_FAST
         int rc = check_launch("hgq_qdense_bwd");
-        if (rc) return rc;
+        if (rc || !reduce) return rc;
         return reduce_parts(workspace, parts, M, dqw, (int64_t)K * N, dqb, (int64_t)N, quant ? df_in : (float *)nullptr, PK, s);
     }
     const int df_lds = (quant && PK <= DF_LDS_MAX) ? 1 : 0;
@@ -1125,8 +1200,22 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
     hipLaunchKernelGGL(fn, grid, dim3(256), dyn, s, dy, y, x, f_in, quant ? bw_rows : (int64_t)1, qw, dx, workspace, dqb ? 1 : 0, rows, K, N,
                        act, mode, df_lds);
     int rc = check_launch("hgq_qdense_bwd");
-    if (rc) return rc;
+    if (rc || !reduce) return rc;
     hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(64 * RP_G), 0, s, workspace, parts, M, dqw, (int64_t)K * N, dqb,
                        (int64_t)N, quant ? df_in : (float *)nullptr, PK);
     return check_launch("hgq_qdense_bwd(reduce)");
+}
+
+extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
+                              const float *qw, float *dx, float *dqw, float *dqb, float *df_in, float *workspace,
+                              int64_t rows, int K, int N, int act, int mode, void *stream) {
+    return qdense_bwd_impl(dy, y, x, f_in, bw_rows, qw, dx, dqw, dqb, df_in, workspace, rows, K, N, act, mode, stream, true);
+}
+
+extern "C" int hgq_qdense_bwd_slices(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
+                                     const float *qw, float *dx, float *workspace, int has_bias, int64_t rows, int K, int N, int act,
+                                     int mode, void *stream) {
+    // the kernels only test the bias pointer for "is there a bias": any non-null value stands for it
+    return qdense_bwd_impl(dy, y, x, f_in, bw_rows, qw, dx, nullptr, has_bias ? workspace : nullptr, nullptr, workspace, rows, K, N, act, mode,
+                           stream, false);
 }

@@ -153,7 +153,12 @@ class QEinsumDense(QLayerBaseSingleInput):
             x = inputs  # the contracted axes are trailing and contiguous: a [rows, K] view of the same memory
             b1d = qbias.reshape(-1) if (qbias is not None and self._bias_in_gemm) else None
             fuse_act = self._act_name if (qbias is None or self._bias_in_gemm) else None
-            y, act_done, self._deferred = dense_contraction(x, iq, qkernel.reshape(self._K, self._N), b1d, fuse_act, training)
+            w2d = qkernel.reshape(self._K, self._N)
+            # a view's gradient goes back through the view unread: the "one reader" mark of a prefetched operand holds for it
+            for view, base in ((w2d, qkernel), (b1d, qbias)):
+                if view is not None and view is not base and getattr(base, '_hgq_single_use', False) and view._base is base:
+                    view._hgq_single_use = True
+            y, act_done, self._deferred = dense_contraction(x, iq, w2d, b1d, fuse_act, training)
             y = y.view(inputs.shape[0], *self.full_output_shape[1:])
             if qbias is not None and not self._bias_in_gemm:
                 y = y + qbias

@@ -190,6 +190,73 @@ def _(dy, y, x, f_in, qw, has_bias, act, mode, bw_rows):
             x.new_empty(bw_rows * x.shape[1]))
 
 
+@torch.library.custom_op('hgq::qdense_bwd_slices', mutates_args=())
+def qdense_bwd_slices(dy: Tensor, y: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_bias: bool, act: int, mode: int,
+                      bw_rows: int) -> tuple[Tensor, Tensor]:
+    """The dense backward without its slice reduction: ``(dx, slices [n, K*N + N + bw_rows*K])``."""
+    _check_f32('dy', dy), _check_f32('x', x), _check_f32('qw', qw), _check_f32('y', y)
+    rows, K = x.shape
+    N = qw.shape[1]
+    _need(tuple(dy.shape) == (rows, N), 'dy shape mismatch')
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    width = K * N + N + bw_rows * K
+    ws = torch.empty((lib.hgq_qdense_bwd_workspace(rows, K, N, bw_rows) // width, width), dtype=torch.float32, device=x.device)
+    rc = lib.hgq_qdense_bwd_slices(_ptr(dy), _ptr(y), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(ws), int(has_bias), rows, K, N,
+                                   act, mode, _stream())
+    _lib.check(rc, 'hgq_qdense_bwd_slices')
+    return dx, ws
+
+
+@qdense_bwd_slices.register_fake
+def _(dy, y, x, f_in, qw, has_bias, act, mode, bw_rows):
+    K, N = x.shape[1], qw.shape[1]
+    return torch.empty_like(x), x.new_empty((max(1, -(-x.shape[0] // 64)), K * N + N + bw_rows * K))
+
+
+class _ReduceItem(ctypes.Structure):
+    _fields_ = [('slices', ctypes.c_void_p), ('n_slices', ctypes.c_int32), ('width', ctypes.c_int64), ('out', ctypes.c_void_p * 3),
+                ('n_out', ctypes.c_int64 * 3)]
+
+
+@torch.library.custom_op('hgq::reduce_slices_multi', mutates_args=('outs',))
+def reduce_slices_multi_op(slices: Sequence[Tensor], outs: Sequence[Tensor], skip: Sequence[bool]) -> None:
+    """``outs[3t .. 3t+2]`` (concatenated) = column sums of ``slices[t]`` [n, width], fixed order, all sets in one launch; a
+    segment with ``skip`` set has its length in ``outs`` but is not written."""
+    n = len(slices)
+    _need(len(outs) == 3 * n and len(skip) == 3 * n, 'three outputs per slice set')
+    items = (_ReduceItem * n)()
+    for t in range(n):
+        sl = slices[t]
+        _check_f32('slices', sl)
+        _need(sl.dim() == 2 and sl.shape[0] >= 1, 'slices must be [n, width]')
+        o = outs[3 * t:3 * t + 3]
+        for v in o:
+            _check_f32('out', v)
+        _need(sum(v.numel() for v in o) == sl.shape[1], 'outputs do not add up to the slice width')
+        items[t].slices, items[t].n_slices, items[t].width = sl.data_ptr(), sl.shape[0], sl.shape[1]
+        for j in range(3):
+            items[t].out[j] = o[j].data_ptr() if (o[j].numel() and not skip[3 * t + j]) else None
+            items[t].n_out[j] = o[j].numel()
+    rc = _lib.load().hgq_reduce_slices_multi(items, n, _stream())
+    _lib.check(rc, 'hgq_reduce_slices_multi')
+
+
+# ---- slice reductions whose results nothing reads before the kernel / bias quantizers' backward or the optimizer:
+# queued while the gradient sink is open, run as one launch by ``flush_reductions``
+_PENDING_REDUCE: list = []
+
+
+def flush_reductions():
+    if not _PENDING_REDUCE:
+        return
+    sl, outs, skip = [], [], []
+    for s_, o_, k_ in _PENDING_REDUCE:
+        sl.append(s_), outs.extend(o_), skip.extend(k_)
+    _PENDING_REDUCE.clear()
+    reduce_slices_multi_op(sl, outs, skip)
+
+
 def _dense_ebops_check(amax, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N, mode_in, mode_ker, mode_bias):
     """Validates one dense-EBOPs call; returns ``(n_parts, has_bias, mode_in, mode_ker, mode_bias)`` with the k-storage flags set."""
     _check_k('k_in', k_in), _check_f32('i_in', i_in), _check_f32('f_in', f_in), _check_k('k_ker', k_ker), _check_f32('b_ker', b_ker)
@@ -1174,6 +1241,7 @@ class _QuantizeMulti(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, *gys):
+        flush_reductions()
         n, t = ctx.n, ctx.saved_tensors
         xs, ks, is_, fbs = t[:n], t[n:2 * n], t[2 * n:3 * n], t[3 * n:]
         for mode in ctx.modes:
@@ -1219,6 +1287,8 @@ class _QDense(torch.autograd.Function):
         ctx.f_owner = _owner(f_in)
         ctx.save_for_backward(x, f_in, qw, y)
         ctx.has_bias = qb.numel() > 0
+        # both operands were handed out once by the model-wide weight-quantizer launch: their only reader is its backward
+        ctx.defer = getattr(qw, '_hgq_single_use', False) and (qb.numel() == 0 or getattr(qb, '_hgq_single_use', False))
         ctx.act, ctx.mode, ctx.bw_rows, ctx.f_shape = act, mode, bw_rows, f_in.shape
         ctx.mark_non_differentiable(amax)
         ctx.set_materialize_grads(False)
@@ -1229,7 +1299,15 @@ class _QDense(torch.autograd.Function):
         if gy is None:
             return (None,) * 10
         x, f_in, qw, y = ctx.saved_tensors
-        dx, dqw, dqb, df = qdense_bwd(gy.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows)
+        if ctx.defer and _SINK['open'] and (ctx.bw_rows == 0 or _can_route(ctx.f_owner, ctx.bw_rows * x.shape[1])):
+            # the kernel / bias gradients are first read by the backward of the prefetched quantizers and the bit-width
+            # gradient by the optimizer: their slice reduction joins those of the other layers
+            dx, ws = qdense_bwd_slices(gy.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows)
+            K, N = qw.shape
+            dqw, dqb, df = torch.empty_like(qw), x.new_empty(N), x.new_empty(ctx.bw_rows * K)
+            _PENDING_REDUCE.append((ws, (dqw, dqb, df), (False, not ctx.has_bias, False)))
+        else:
+            dx, dqw, dqb, df = qdense_bwd(gy.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows)
         df = _route(ctx.f_owner, df) if ctx.bw_rows > 0 else None
         return (dx, None, None, df.view(ctx.f_shape) if df is not None else None, dqw, dqb if ctx.has_bias else None,
                 None, None, None, None)
@@ -1850,6 +1928,10 @@ class side_gradients:
         return self
 
     def __exit__(self, *exc):
+        if exc[0] is None:
+            flush_reductions()
+        else:
+            _PENDING_REDUCE.clear()
         _SINK.update(self.prev)
 
 
@@ -1875,6 +1957,12 @@ def _owner(t):
         return t
     base = getattr(t, '_base', None)
     return base if isinstance(base, torch.nn.Parameter) else None
+
+
+def _can_route(owner, numel) -> bool:
+    """``_route`` would leave a gradient of ``numel`` elements on ``owner`` rather than hand it back."""
+    return (owner is not None and _SINK['open'] and owner.requires_grad and numel == owner.numel()
+            and len(getattr(owner, '_hgq_side', None) or ()) < SGD_SIDES)
 
 
 def _route(owner, grad):

@@ -69,5 +69,6 @@ def prefetch_weight_quantizers(root) -> int:
     ys = ops.quantize_multi([p for _, p in pairs], [fq._k.view(-1) for fq, _ in pairs], [fq._i.view(-1) for fq, _ in pairs],
                             [fq._third().view(-1) for fq, _ in pairs], [fq._mode(True) for fq, _ in pairs])
     for (fq, p), y in zip(pairs, ys):
+        y._hgq_single_use = True  # handed out once, to the layer's own call: the only other reader of its gradient is this launch's backward
         fq._prefetched = (p, y)
     return len(pairs)

@@ -212,6 +212,30 @@ int hgq_qdense_bwd(const float *dy, const float *y, const float *x, const float 
                    int64_t rows, int K, int N, int act, int mode, void *stream);
 
 /*
+ * The same backward in two halves, for a caller that reduces the slices of several layers in one launch: the kernel
+ * gradient of a layer is first read by the backward of its kernel quantizer, which in a training step runs after the
+ * backward of every layer (the quantizers depend on the variables only: src/hgq/layers/core/dense.py:72-79).
+ *   hgq_qdense_bwd_slices: writes dx and leaves n = hgq_qdense_bwd_workspace(...) / width slices of
+ *   width = K*N + N + bw_rows*K floats in `workspace`: [dqw | dqb | df_in] partial sums per workgroup
+ *   (the dqb segment is undefined when has_bias == 0).
+ *   hgq_reduce_slices_multi: out[0] | out[1] | out[2] (lengths n_out[0..2], summing to `width`; a NULL pointer skips
+ *   that segment) = sum over the slices, in slice order and with the association hgq_qdense_bwd uses, so both routes
+ *   give the same bits.  Up to HGQ_REDUCE_BATCH sets per launch, more are split over launches.
+ */
+#define HGQ_REDUCE_BATCH 16
+typedef struct {
+    const float *slices; /* [n_slices, width] */
+    int32_t n_slices;
+    int64_t width;
+    float *out[3];
+    int64_t n_out[3];
+} hgq_reduce_item;
+int hgq_qdense_bwd_slices(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,
+                          const float *qw, float *dx, float *workspace, int has_bias, int64_t rows, int K, int N, int act,
+                          int mode, void *stream);
+int hgq_reduce_slices_multi(const hgq_reduce_item *items, int count, void *stream);
+
+/*
  * EBOPs of a dense contraction and its gradient.  Replaces QDense._compute_ebops
  * (src/hgq/layers/core/dense.py:70-80) / QEinsumDense._compute_ebops for GEMM-shaped equations
  * (einsum_dense.py:85-93) evaluated on bit-width tensors, i.e.

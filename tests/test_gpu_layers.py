@@ -370,7 +370,7 @@ def test_batched_quantizer_matches_single_launches():
 
 
 @pytest.mark.parametrize('kind', ['mlp', 'particle', 'conv', 'mha'])
-def test_gradient_sink_gives_the_autograd_update(dev, kind):
+def test_gradient_sink_gives_the_autograd_update(dev, kind, monkeypatch):
     """``opt.backward(loss)`` leaves the EBOPs gradients of the bit-width variables on the variables and the update
     kernel adds them; the result must be the update of plain ``loss.backward()``.  Where a variable has one piece from
     autograd and one from an EBOPs term the two paths add the same two numbers: bit-identical."""
@@ -404,6 +404,9 @@ def test_gradient_sink_gives_the_autograd_update(dev, kind):
     b(xd, training=True)
     b.load_state_dict(a.state_dict())
     opt_a, opt_b = SGD(a.parameters(), lr=0.05, fold_regularizers=True), SGD(b.parameters(), lr=0.05, fold_regularizers=True)
+    joined = []  # slice sets per joint reduction launch
+    plain_reduce = ops.reduce_slices_multi_op
+    monkeypatch.setattr(ops, 'reduce_slices_multi_op', lambda sl, outs, skip: (joined.append(len(sl)), plain_reduce(sl, outs, skip))[1])
     for step in range(2):
         opt_a.zero_grad()
         la = model_loss(a, loss_fn(a(xd, training=True)), True)
@@ -421,6 +424,42 @@ def test_gradient_sink_gives_the_autograd_update(dev, kind):
                 assert torch.equal(pa, pb), f'{name} step {step}'
             else:
                 assert torch.allclose(pa, pb, rtol=1e-6, atol=1e-9), f'{name} step {step}: {float((pa - pb).abs().max()):.3e}'
+    if kind in ('mlp', 'mha'):  # the dense backward of every layer left its slices for one joint reduction per step
+        assert joined == [4, 4], joined
+
+
+def test_dense_backward_in_two_halves_gives_the_same_bits(dev):
+    """``qdense_bwd_slices`` + ``reduce_slices_multi`` (several sets per launch, a skipped bias segment, widths that are
+    not multiples of 64) against ``qdense_bwd``: identical bits."""
+    from hgq2_amd import _lib, ops
+
+    g = torch.Generator().manual_seed(5)
+    cases = [(1000, 16, 64, 1, True), (4096, 64, 32, 2, True), (333, 32, 5, 0, False), (64, 8, 4, 1, True)]
+    mode = _lib.RND | (_lib.WRAP << 4) | _lib.MODE_TRAINING | _lib.MODE_ROUND_PARAMS
+    want, slices, outs, skip = [], [], [], []
+    for rows, K, N, bw_rows, has_bias in cases:
+        rows -= rows % max(bw_rows, 1)
+        x = (torch.randn(rows, K, generator=g) * 3).to(dev)
+        qw = (torch.randint(-8, 9, (K, N), generator=g) / 4.0).to(dev)
+        y = torch.randn(rows, N, generator=g).to(dev)
+        dy = torch.randn(rows, N, generator=g).to(dev)
+        f_in = torch.randint(0, 5, (bw_rows * K,), generator=g).float().to(dev)
+        act = _lib.ACT_RELU if N > 4 else _lib.ACT_NONE
+        m = mode if bw_rows else 0
+        want.append(ops.qdense_bwd(dy, y, x, f_in, qw, has_bias, act, m, bw_rows))
+        dx, ws = ops.qdense_bwd_slices(dy, y, x, f_in, qw, has_bias, act, m, bw_rows)
+        assert torch.equal(dx, want[-1][0])
+        slices.append(ws)
+        outs += [torch.full((K, N), 7.0, device=dev), torch.full((N,), 7.0, device=dev), torch.full((bw_rows * K,), 7.0, device=dev)]
+        skip += [False, not has_bias, False]
+    ops.reduce_slices_multi_op(slices, outs, skip)
+    for t, (rows, K, N, bw_rows, has_bias) in enumerate(cases):
+        dqw, dqb, df = outs[3 * t:3 * t + 3]
+        assert torch.equal(dqw, want[t][1]), t
+        assert torch.equal(dqb, want[t][2]) if has_bias else bool((dqb == 7.0).all()), t  # a skipped segment is left alone
+        assert torch.equal(df, want[t][3]), t
+    with pytest.raises(ValueError):
+        ops.reduce_slices_multi_op(slices[:1], outs[:2] + [outs[5]], skip[:3])  # lengths do not add up to the width
 
 
 def test_fused_stack_sees_updates_made_by_the_per_layer_optimizer(dev):
