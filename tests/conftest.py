@@ -28,3 +28,13 @@ def dev():
     if not torch.cuda.is_available():
         pytest.skip('no GPU')
     return torch.device('cuda:0')
+
+
+@pytest.fixture
+def acc64():
+    """The oracle's contractions in float64 (its quantizers stay fp32) for the duration of a test."""
+    from oracle import hgq_ref
+
+    hgq_ref.ACC64 = True
+    yield
+    hgq_ref.ACC64 = False

@@ -21,13 +21,6 @@ pytestmark = pytest.mark.gpu
 RTOL = 1e-5
 
 
-@pytest.fixture
-def acc64():
-    ref.ACC64 = True
-    yield
-    ref.ACC64 = False
-
-
 def _close_scaled(got, want, scale, what, rtol=RTOL):
     got, want, scale = got.detach().double().cpu(), want.detach().double(), scale.detach().double()
     err = (got.reshape(want.shape) - want).abs()
