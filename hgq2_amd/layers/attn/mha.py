@@ -1,7 +1,10 @@
-"""QMultiHeadAttention (reference src/hgq/layers/attn/mha.py:27-537) for rank-3 inputs
-``[batch, sequence, features]``: four QEinsumDense projections (query / key / value with output
-quantizers, attention_output), scaled dot-product scores, the table softmax, and the EBOPs of
-the two score contractions.  The einsum strings are those Keras builds for rank-3 inputs."""
+"""QMultiHeadAttention (reference src/hgq/layers/attn/mha.py:27-537): four QEinsumDense projections (query / key /
+value with output quantizers, attention_output), scaled dot-product scores, the table softmax, and the EBOPs of the
+two score contractions, for inputs ``[batch, seq..., features]`` of any rank attending over all sequence axes.
+
+Rank-3 inputs ``[batch, sequence, features]`` take the one-pass attention kernels.  With more sequence axes the
+projections run on the same dense kernels, the two score contractions on the attention contraction kernels over the
+flattened sequence axes, and the softmax over its trailing axes stage by stage."""
 
 from __future__ import annotations
 
@@ -16,11 +19,10 @@ from ...quantizer.config import QuantizerConfig
 from ..core.base import QLayerBase
 from ..core.einsum_dense import QEinsumDense
 from ..softmax import QSoftmax
+from ._equations import attention_equations, proj_equation, projected_shape
 
-_PROJ_EQ, _PROJ_BIAS = 'abc,cde->abde', 'de'
-_OUT_EQ, _OUT_BIAS = 'abcd,cde->abe', 'e'
-_DOT_EQ = 'aecd,abcd->acbe'      # key [B,S,N,H], query [B,T,N,H] -> scores [B,N,T,S]
-_COMBINE_EQ = 'acbe,aecd->abcd'  # scores [B,N,T,S], value [B,S,N,H] -> [B,T,N,H]
+# with the sequence axes flattened: key [B,S,N,H], query [B,T,N,H] -> scores [B,N,T,S] -> [B,T,N,H]
+_DOT_EQ, _COMBINE_EQ = 'aecd,abcd->acbe', 'acbe,aecd->abcd'
 
 FUSED = True  # module switch: False composes scores, softmax and combine from their own kernels (cross-check)
 
@@ -35,8 +37,8 @@ class QMultiHeadAttention(QLayerBase):
                  softmax_inv_oq_conf=None, softmax_oq_conf=None, stable_softmax=True,
                  softmax_allow_heterogeneous_table: bool = False, parallelization_factor=-1, **kwargs):
         super().__init__(**kwargs)
-        if attention_axes is not None:
-            raise NotImplementedError('only attention over the sequence axis of rank-3 inputs is supported')
+        self._attention_axes = None if attention_axes is None else tuple(
+            attention_axes if isinstance(attention_axes, (tuple, list)) else (attention_axes,))
         self._num_heads, self._key_dim = int(num_heads), int(key_dim)
         self._value_dim = int(value_dim) if value_dim else int(key_dim)
         self._dropout, self._use_bias, self._output_shape = float(dropout), use_bias, output_shape
@@ -61,6 +63,7 @@ class QMultiHeadAttention(QLayerBase):
         config = super().get_config()
         config.pop('oq_conf', None)
         config.update({'num_heads': self._num_heads, 'key_dim': self._key_dim, 'value_dim': self._value_dim, 'dropout': self._dropout,
+                       'attention_axes': self._attention_axes,
                        'use_bias': self._use_bias, 'output_shape': self._output_shape, 'kernel_initializer': self._kernel_initializer,
                        'bias_initializer': self._bias_initializer, 'fuse': self._fuse, 'qkvo_iq_conf': self._qkvo_iq_conf,
                        'qkvo_kq_conf': self._qkvo_kq_conf, 'qkvo_bq_conf': self._qkvo_bq_conf, 'qkvo_oq_conf': self._qkvo_oq_conf,
@@ -91,24 +94,26 @@ class QMultiHeadAttention(QLayerBase):
             key_shape = shapes[2] if len(shapes) > 2 else None
         value_shape = query_shape if value_shape is None else value_shape
         key_shape = value_shape if key_shape is None else key_shape
-        if len(query_shape) != 3:
-            raise NotImplementedError('QMultiHeadAttention: rank-3 inputs [batch, sequence, features] only')
+        if len(query_shape) < 3 or len(value_shape) != len(query_shape) or len(key_shape) != len(query_shape):
+            raise ValueError('QMultiHeadAttention: query, value and key must be [batch, seq..., features] of one rank')
         if self._fuse == 'qkv':
             assert query_shape == value_shape == key_shape, 'For fuse=qkv, query, key and value must have the same shape'
         if self._fuse == 'kv':
             assert value_shape == key_shape, 'For fuse=kv, key and value must have the same shape'
         if tuple(value_shape[1:-1]) != tuple(key_shape[1:-1]):
             raise ValueError('All dimensions of `value` and `key`, except the last one, must be equal.')
-        T, S = query_shape[1], value_shape[1]
+        rank = len(query_shape)
         N = self._num_heads
-        bias = _PROJ_BIAS if self._use_bias else None
-        self._query_dense = QEinsumDense(_PROJ_EQ, output_shape=[T, N, self._key_dim], bias_axes=bias, name='query',
-                                         enable_iq=self.enable_iq and not self._fuse == 'qkv', enable_oq=True, **self._sub_kwargs())
-        self._key_dense = QEinsumDense(_PROJ_EQ, output_shape=[S, N, self._key_dim], bias_axes=None, name='key',
-                                       enable_iq=self.enable_iq and self._fuse not in ('qkv', 'kv'), enable_oq=True,
-                                       **self._sub_kwargs())
-        self._value_dense = QEinsumDense(_PROJ_EQ, output_shape=[S, N, self._value_dim], bias_axes=bias, name='value',
-                                         enable_iq=self.enable_iq, enable_oq=True, **self._sub_kwargs())
+        eq, bias_axes, out_rank = proj_equation(rank - 1, 1, 2)
+        bias = bias_axes if self._use_bias else None
+        self._query_dense = QEinsumDense(eq, output_shape=projected_shape(out_rank - 1, [N, self._key_dim], query_shape),
+                                         bias_axes=bias, name='query', enable_iq=self.enable_iq and not self._fuse == 'qkv',
+                                         enable_oq=True, **self._sub_kwargs())
+        self._key_dense = QEinsumDense(eq, output_shape=projected_shape(out_rank - 1, [N, self._key_dim], key_shape),
+                                       bias_axes=None, name='key', enable_iq=self.enable_iq and self._fuse not in ('qkv', 'kv'),
+                                       enable_oq=True, **self._sub_kwargs())
+        self._value_dense = QEinsumDense(eq, output_shape=projected_shape(out_rank - 1, [N, self._value_dim], value_shape),
+                                         bias_axes=bias, name='value', enable_iq=self.enable_iq, enable_oq=True, **self._sub_kwargs())
         self._build_sub(self._value_dense, value_shape)
         if self._fuse == 'qkv' and self.enable_iq:
             self._query_dense._iq = self._value_dense._iq
@@ -119,29 +124,43 @@ class QMultiHeadAttention(QLayerBase):
         self._build_sub(self._query_dense, query_shape)
         self._build_sub(self._key_dense, key_shape)
 
+        # the reference sizes the softmax as [batch, heads, query seq..., key seq...] (mha.py:352-355), which is the
+        # layout of the scores only when every sequence axis is attended: that is the case built here
+        all_axes = tuple(range(1, out_rank - 2))
+        if self._attention_axes is None:
+            self._attention_axes = all_axes
+        if tuple(a % out_rank for a in self._attention_axes) != all_axes:
+            raise NotImplementedError('QMultiHeadAttention: attention over a subset of the sequence axes is not supported')
+        self._dot_eq, self._combine_eq, scores_rank = attention_equations(out_rank, self._attention_axes)
+        q_seq, k_seq = tuple(query_shape[1:-1]), tuple(value_shape[1:-1])
+        self._n_seq = len(q_seq)
+        self._T, self._S = math.prod(q_seq), math.prod(k_seq)
+        norm_axes = tuple(range(scores_rank - len(self._attention_axes), scores_rank))
         self._softmax = QSoftmax(
-            enable_oq=True, axis=(3,), stable=self._stable_softmax, iq_conf=self._softmax_iq_conf,
+            enable_oq=True, axis=norm_axes, stable=self._stable_softmax, iq_conf=self._softmax_iq_conf,
             exp_iq_conf=self._softmax_exp_iq_conf, exp_oq_conf=self._softmax_exp_oq_conf,
             inv_iq_conf=self._softmax_inv_iq_conf, inv_oq_conf=self._softmax_inv_oq_conf, oq_conf=self._softmax_oq_conf,
             allow_heterogeneous_table=self._softmax_allow_heterogeneous_table, input_scaler=self._inverse_sqrt_key_dim,
             enable_ebops=self.enable_ebops, name=f'{self.name}_softmax')  # a fixed name: variable paths must be reproducible
         self._inverse_sqrt_key_dim = 1.0  # the scale now lives in the softmax's exp table
-        self._build_sub(self._softmax, (query_shape[0], N, T, S))
+        self._scores_shape = (query_shape[0], N) + q_seq + k_seq
+        self._build_sub(self._softmax, self._scores_shape)
 
-        out_dim = self._output_shape if self._output_shape else query_shape[-1]
-        if isinstance(out_dim, (tuple, list)):
-            (out_dim,) = out_dim
-        self._output_dense = QEinsumDense(_OUT_EQ, output_shape=[T, out_dim], bias_axes=_OUT_BIAS if self._use_bias else None,
-                                          name='attention_output', enable_iq=True, enable_oq=self.enable_oq,
-                                          **self._sub_kwargs())
-        self._build_sub(self._output_dense, (query_shape[0], T, N, self._value_dim))
+        out_shape = self._output_shape if self._output_shape else [query_shape[-1]]
+        if not isinstance(out_shape, (tuple, list)):
+            out_shape = [out_shape]
+        o_eq, o_bias, o_rank = proj_equation(rank - 1, 2, len(out_shape))
+        self._output_dense = QEinsumDense(o_eq, output_shape=projected_shape(o_rank - 1, out_shape, query_shape),
+                                          bias_axes=o_bias if self._use_bias else None, name='attention_output', enable_iq=True,
+                                          enable_oq=self.enable_oq, **self._sub_kwargs())
+        self._build_sub(self._output_dense, (query_shape[0],) + q_seq + (N, self._value_dim))
 
         if self.enable_ebops:
             self._beta = self.add_weight(name='beta', shape=(), initializer=self._beta0, trainable=False)
             self._ebops = self.add_weight(name='ebops', shape=(), initializer=Constant(0.0), trainable=False, dtype='uint32')
-        self._q_shape = (1, T, N, self._key_dim)
-        self._k_shape = (1, S, N, self._key_dim)
-        self._v_shape = (1, S, N, self._value_dim)
+        self._q_shape = (1,) + q_seq + (N, self._key_dim)
+        self._k_shape = (1,) + k_seq + (N, self._key_dim)
+        self._v_shape = (1,) + k_seq + (N, self._value_dim)
         self.built = True
 
     def _maybe_build(self, args):
@@ -155,7 +174,7 @@ class QMultiHeadAttention(QLayerBase):
 
     def _ebops_loss_term(self, query_shape, value_shape=None, key_shape=None):
         # both score contractions' EBOPs from the marginal sums of the four bit-width tensors, in one launch
-        if self._beta is not None and self._beta.is_cuda and self._softmax.enable_oq:
+        if self._beta is not None and self._beta.is_cuda and self._softmax.enable_oq and self._n_seq == 1:
             (_, T, N, H), (_, S, _, Hv) = self._q_shape, self._v_shape
             operands = [self._query_dense.oq.bits_operand(self._q_shape), self._key_dense.oq.bits_operand(self._k_shape),
                         self._value_dense.oq.bits_operand(self._v_shape), self._softmax.oq.bits_operand((1, N, T, S))]
@@ -165,14 +184,13 @@ class QMultiHeadAttention(QLayerBase):
         return super()._ebops_loss_term(query_shape, value_shape, key_shape)
 
     def _compute_ebops(self, query_shape, value_shape=None, key_shape=None):
-        value_shape = query_shape if value_shape is None else value_shape
-        attn_shape = (1, self._num_heads, query_shape[1], value_shape[1])
+        attn_shape = (1,) + tuple(self._scores_shape[1:])
         bw_q = self._query_dense.oq.bits_(self._q_shape)
         bw_k = self._key_dense.oq.bits_(self._k_shape)
         bw_v = self._value_dense.oq.bits_(self._v_shape)
         bw_attn = self._softmax.oq.bits_(attn_shape)
-        ebops_qk = torch.einsum(_DOT_EQ.split('->')[0] + '->', bw_k, bw_q)
-        ebops_av = torch.einsum(_COMBINE_EQ.split('->')[0] + '->', bw_attn, bw_v)
+        ebops_qk = torch.einsum(self._dot_eq.split('->')[0] + '->', bw_k, bw_q)
+        ebops_av = torch.einsum(self._combine_eq.split('->')[0] + '->', bw_attn, bw_v)
         ebops = ebops_qk + ebops_av
         if self.parallelization_factor > 0:
             return ebops * self.parallelization_factor
@@ -193,6 +211,8 @@ class QMultiHeadAttention(QLayerBase):
         if key is None:
             key = value
         if use_causal_mask:
+            if self._n_seq != 1:
+                raise NotImplementedError('use_causal_mask needs a single sequence axis')
             T, S = query.shape[1], value.shape[1]
             causal = torch.tril(torch.ones((1, T, S), dtype=torch.bool, device=query.device))
             attention_mask = causal if attention_mask is None else (attention_mask.bool() & causal)
@@ -210,15 +230,26 @@ class QMultiHeadAttention(QLayerBase):
     def _compute_attention(self, query, key, value, attention_mask=None, training=None, need_scores=True):
         if self._inverse_sqrt_key_dim != 1.0:  # 1 after build: the scale lives in the softmax's exp table
             query = query * self._inverse_sqrt_key_dim
-        if FUSED and not need_scores and attention_mask is None and not (self._dropout and training):
+        flat = self._n_seq == 1
+        if FUSED and flat and not need_scores and attention_mask is None and not (self._dropout and training):
             stand_in = self._softmax.attention_plan(query, key, value, training)
             if stand_in is not None:  # one kernel each way; scores and probabilities are never written
                 return self._softmax(stand_in, attention=(query, key, value)), None
-        own = query.is_cuda and max(query.shape[1], key.shape[1], query.shape[3], value.shape[3]) <= ops.ATTN_MAX
-        scores = ops.attn_scores(query, key) if own else torch.einsum(_DOT_EQ, key, query)
+        # several sequence axes, all attended: the contractions see them as one axis (same memory), the softmax and its
+        # quantizers see [batch, heads, query seq..., key seq...] as the reference builds them
+        B, N = query.shape[0], self._num_heads
+        q_seq, k_seq = tuple(query.shape[1:-2]), tuple(key.shape[1:-2])
+        q4, k4, v4 = (t.reshape(B, -1, N, t.shape[-1]) for t in (query, key, value))
+        own = q4.is_cuda and max(q4.shape[1], k4.shape[1], q4.shape[3], v4.shape[3]) <= ops.ATTN_MAX
+        scores = ops.attn_scores(q4, k4) if own else torch.einsum(_DOT_EQ, k4, q4)
+        scores = scores.view((B, N) + q_seq + k_seq)
         mask = None
         if attention_mask is not None:
-            mask = attention_mask.unsqueeze(1)  # broadcast over heads
+            mask = attention_mask
+            while mask.dim() < scores.dim():  # broadcast over the heads (and any other axis ahead of the attended ones)
+                mask = mask.unsqueeze(-2 * self._n_seq - 1)
         scores = self._softmax(scores, mask=mask)
         final = torch.nn.functional.dropout(scores, self._dropout) if (self._dropout and training) else scores
-        return (ops.attn_combine(final, value) if own else torch.einsum(_COMBINE_EQ, final, value)), scores
+        f4 = final.reshape(B, N, q4.shape[1], k4.shape[1])
+        out = ops.attn_combine(f4, v4) if own else torch.einsum(_COMBINE_EQ, f4, v4)
+        return out.view((B,) + q_seq + (N, v4.shape[3])), scores

@@ -707,8 +707,28 @@ class RefQSoftmax(RefQLayer):
         return (sub + accum + mult) * factor
 
 
+def keras_attention_equations(rank, attn_axes):
+    """The einsum strings Keras' multi-head attention builds for projected tensors of ``rank`` axes
+    [batch, seq..., heads, channels] (the reference imports the builder at src/hgq/layers/attn/mha.py:10 and uses its
+    result at :315-319): query axes are lettered a, b, c, ...; the key / value side reuses the query's letter on every
+    axis that is not attended and on the last axis, and takes the next unused letters on the attended ones; scores are
+    [kept axes..., attended query axes..., attended key axes...]."""
+    letters = 'abcdefghijklmnopqrstuvwxyz'
+    target = letters[:rank]
+    kept = tuple(i for i in range(rank) if i not in tuple(attn_axes) + (rank - 1,))
+    nxt, source = rank, ''
+    for i in range(rank):
+        if i in kept or i == rank - 1:
+            source += target[i]
+        else:
+            source += letters[nxt]
+            nxt += 1
+    product = ''.join([target[i] for i in kept] + [target[i] for i in attn_axes] + [source[i] for i in attn_axes])
+    return '%s,%s->%s' % (source, target, product), '%s,%s->%s' % (product, source, target)
+
+
 class RefQMultiHeadAttention(RefQLayer):
-    """src/hgq/layers/attn/mha.py:27-537 for rank-3 inputs; einsum strings as Keras builds them."""
+    """src/hgq/layers/attn/mha.py:27-537 for inputs [batch, seq..., features] attending over all sequence axes."""
 
     def __init__(self, query_dense, key_dense, value_dense, output_dense, softmax, beta0=1e-5, enable_ebops=True,
                  parallelization_factor=-1):
@@ -731,20 +751,28 @@ class RefQMultiHeadAttention(RefQLayer):
                     out.append(q)
         return out
 
-    def call(self, x, training=None, mask=None):
+    def call(self, x, value=None, key=None, training=None, mask=None):
+        value = x if value is None else value  # mha.py:452-455
+        key = value if key is None else key
         q = self.qd(x, training=training)
-        k = self.kd(x, training=training)
-        v = self.vd(x, training=training)
-        scores = torch.einsum('aecd,abcd->acbe', k, q * 1.0)
-        m = None if mask is None else mask.unsqueeze(1)
+        k = self.kd(key, training=training)
+        v = self.vd(value, training=training)
+        rank = q.dim()
+        attn_axes = tuple(range(1, rank - 2))  # mha.py:312-313
+        self._dot_eq, self._combine_eq = keras_attention_equations(rank, attn_axes)
+        scores = torch.einsum(self._dot_eq, k, q * 1.0)  # mha.py:521-525 (the 1/sqrt(d) factor sits in the softmax)
+        m = mask
+        if m is not None:  # Keras' _masked_softmax: new axes ahead of the attended ones until the ranks agree
+            while m.dim() < scores.dim():
+                m = m.unsqueeze(-2 * len(attn_axes) - 1)
         scores = self.softmax(scores, training=training, mask=m)
-        out = torch.einsum('acbe,aecd->abcd', scores, v)
+        out = torch.einsum(self._combine_eq, scores, v)  # mha.py:536
         self._shapes = (q.shape, k.shape, v.shape, scores.shape)
         return self.od(out, training=training)
 
-    def __call__(self, x, training=None, mask=None):
+    def __call__(self, x, value=None, key=None, training=None, mask=None):
         self.losses = []
-        r = self.call(x, training=training, mask=mask)
+        r = self.call(x, value, key, training=training, mask=mask)
         if (training or training == 'tracing') and self.enable_ebops:
             ebops = self._compute_ebops()
             self.ebops_value = ebops.detach().to(torch.int64)
@@ -766,7 +794,9 @@ class RefQMultiHeadAttention(RefQLayer):
         qs, ks, vs, ss = ((1,) + tuple(s[1:]) for s in self._shapes)
         bw_q, bw_k, bw_v = self.qd.oq.bits_(qs), self.kd.oq.bits_(ks), self.vd.oq.bits_(vs)
         bw_attn = self.softmax.oq.bits_(ss)
-        ebops = torch.einsum('aecd,abcd->', bw_k, bw_q) + torch.einsum('acbe,aecd->', bw_attn, bw_v)
+        # mha.py:386-416 with the strings of :246-247
+        dot_eq, combine_eq = keras_attention_equations(len(qs), tuple(range(1, len(qs) - 2)))
+        ebops = torch.einsum(dot_eq.split('->')[0] + '->', bw_k, bw_q) + torch.einsum(combine_eq.split('->')[0] + '->', bw_attn, bw_v)
         if self.parallelization_factor > 0:
             return ebops * self.parallelization_factor
         return ebops

@@ -112,13 +112,14 @@ def ref_softmax(layer):
                            enable_ebops=layer.enable_ebops, parallelization_factor=layer.parallelization_factor)
 
 
-def ref_mha(layer, query_shape):
-    B, T, D = query_shape
+def ref_mha(layer, query_shape, value_shape=None, key_shape=None):
+    value_shape = query_shape if value_shape is None else value_shape
+    key_shape = value_shape if key_shape is None else key_shape
     N = layer._num_heads
     qd = ref_einsum_dense(layer._query_dense, query_shape)
-    kd = ref_einsum_dense(layer._key_dense, query_shape)
-    vd = ref_einsum_dense(layer._value_dense, query_shape)
-    od = ref_einsum_dense(layer._output_dense, (B, T, N, layer._value_dim))
+    kd = ref_einsum_dense(layer._key_dense, key_shape)
+    vd = ref_einsum_dense(layer._value_dense, value_shape)
+    od = ref_einsum_dense(layer._output_dense, tuple(query_shape[:-1]) + (N, layer._value_dim))
     # fused input quantizers are one shared object in the product; share the twin as well
     if layer._query_dense.enable_iq and layer._query_dense._iq is layer._value_dense._iq:
         qd.iq = vd.iq

@@ -178,6 +178,40 @@ def test_multi_head_attention(dev):
         assert int(layer._ebops.cpu().view(torch.int32)) == int(r.ebops_value), fuse
 
 
+@pytest.mark.parametrize('fuse,shapes,causal', [('none', ((2, 4, 8), (2, 4, 9), (2, 4, 10)), False), ('kv', ((2, 4, 3), (2, 4, 5)), False),
+                                                ('none', ((3, 2, 8), (2, 5, 6)), False), ('qkv', ((9, 8),), True)])
+@pytest.mark.parametrize('num_heads', [1, 2])
+def test_multi_head_attention_shapes_of_the_reference_tests(dev, fuse, shapes, causal, num_heads):
+    """The input shapes reference tests/test_mha.py:29-37 runs: two sequence axes with separate query / value / key
+    inputs of different widths, fused key-value input, and one sequence axis with the causal mask."""
+    from hgq2_amd.layers import QMultiHeadAttention
+
+    g = torch.Generator().manual_seed(5 + num_heads)
+    B = 48
+    with readme_scopes():
+        layer = QMultiHeadAttention(num_heads=num_heads, key_dim=8, fuse=fuse)
+    xs = [torch.randn((B,) + sh, generator=g).clamp(-1, 1) for sh in shapes]
+    kw = {'use_causal_mask': True} if causal else {}
+    layer(*[x.to(dev) for x in xs], training=True, **kw)
+    _perturb(layer, g)
+    r = twin.ref_mha(layer, *[tuple(x.shape) for x in xs])
+    xp = [x.to(dev).requires_grad_(True) for x in xs]
+    xr = [x.clone().requires_grad_(True) for x in xs]
+    mask = torch.tril(torch.ones(1, shapes[0][0], shapes[0][0], dtype=torch.bool)) if causal else None
+    named_p = [(f'x{j}', t) for j, t in enumerate(xp)] + [
+        ('wq', layer._query_dense._kernel), ('wk', layer._key_dense._kernel), ('wv', layer._value_dense._kernel),
+        ('wo', layer._output_dense._kernel), ('q_oq_f', layer._query_dense.oq.quantizer._f), ('k_oq_f', layer._key_dense.oq.quantizer._f),
+        ('sm_oq_f', layer._softmax.oq.quantizer._f), ('v_iq_f', layer._value_dense.iq.quantizer._f)]
+    named_r = [(f'x{j}', t) for j, t in enumerate(xr)] + [
+        ('wq', r.qd.kernel), ('wk', r.kd.kernel), ('wv', r.vd.kernel), ('wo', r.od.kernel), ('q_oq_f', r.qd.oq.quantizer._f),
+        ('k_oq_f', r.kd.oq.quantizer._f), ('sm_oq_f', r.softmax.oq.quantizer._f), ('v_iq_f', r.vd.iq.quantizer._f)]
+    _compare_step(layer, r, lambda t: layer(*xp, training=t, **kw), lambda t: r(*xr, training=t, mask=mask), named_p, named_r)
+    assert int(layer._ebops.cpu().view(torch.int32)) == int(r.ebops_value)
+    assert torch.equal(layer._softmax.oq.quantizer._i.cpu(), r.softmax.oq.quantizer._i.detach())
+    with torch.no_grad():
+        _close(layer(*[x.to(dev) for x in xs], training=False, **kw), r(*xs, training=False, mask=mask), what='inference output')
+
+
 def test_conv2d_stack_layer(dev):
     from hgq2_amd.layers import QConv2D
 
