@@ -1141,7 +1141,11 @@ __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, h
         if (ebops_u32) ebops_u32[0] = (uint32_t)ebops;
         loss_term[0] = ebops * beta[0];
     }
-    for (int e = t; e < n_w; e += 1024) ce_put(dker, (uint32_t)e, true, S[by_f.div((uint32_t)e)] * conv_scale * gs);
+    for (int e = t; e < n_w; e += 1024) {
+        bool open;  // a KIF kernel quantizer's width relu(i + f) is flat where i + f <= 0
+        (void)ce_bits(dker, (uint32_t)e, open);
+        ce_put(dker, (uint32_t)e, open, S[by_f.div((uint32_t)e)] * conv_scale * gs);
+    }
     for (int e = t; e < g.H * WC; e += 1024) {
         const int y = (int)by_wc.div((uint32_t)e), xc = e - y * WC, x = (int)by_c.div((uint32_t)xc), c = xc - x * g.C;
         float a = 0.f;
@@ -1155,7 +1159,11 @@ __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, h
         ce_put(din, (uint32_t)e, open, a * conv_scale * gs);
     }
     if (has_bias)
-        for (int n = t; n < F; n += 1024) ce_put(dbias, (uint32_t)n, true, bias_size / (float)F * gs);
+        for (int n = t; n < F; n += 1024) {
+            bool open;
+            (void)ce_bits(dbias, (uint32_t)n, open);
+            ce_put(dbias, (uint32_t)n, open, bias_size / (float)F * gs);
+        }
 }
 
 static int check_geom(const hgq_conv_geom *g, int F, const char *who) {

@@ -32,6 +32,10 @@ EPSILON = 1e-7  # keras.backend.epsilon() default
 # while every quantizer still sees and produces fp32 values; a parity test that compares sums over 10^5..10^7 terms
 # sets it so that its tolerance measures the kernel under test and not the fp32 summation order of this file.
 ACC64 = False
+# True: every quantizer call keeps its result (with ``retain_grad``) in ``quantizer.taps``, so that a test can bound the
+# sum of |terms| behind a bit-width gradient (|term| <= ln2 * 2^-f * |upstream gradient|) and state its tolerance
+# relative to that sum instead of to the cancelled total.
+TAP_GRADS = False
 
 
 def _acc(t):
@@ -361,6 +365,9 @@ class RefQuantizer:
         if self.scaler is not None:
             inputs = inputs / self.scaler
         out = self.quantizer.call(inputs, training=training)
+        if TAP_GRADS and out.requires_grad:  # a test wants the upstream gradient of every quantizer call afterwards
+            out.retain_grad()
+            self.quantizer.taps = getattr(self.quantizer, 'taps', []) + [out]
         if self.scaler is not None:
             out = out * self.scaler
         if self.qnoise_factor is not None and training:
@@ -656,11 +663,13 @@ class RefQUnaryFunctionLUT(RefQLayer):
 
 
 class RefQSoftmax(RefQLayer):
-    """src/hgq/layers/softmax.py:13-161 (stable form)."""
+    """src/hgq/layers/softmax.py:13-161.  ``stable`` False is the form without the max subtraction (:116-120): the
+    exp table then has no input quantizer and no EBOPs of its own (:87-96) and its function is exp(+x * scaler) (:49-53)."""
 
     def __init__(self, axes, exp_table, inv_table, oq, iq=None, input_scaler=1.0, beta0=1e-5, enable_ebops=True,
-                 parallelization_factor=-1):
+                 parallelization_factor=-1, stable=True):
         self._init_common(beta0, enable_ebops)
+        self.stable = stable
         self.axes = tuple(axes)
         self.exp_table, self.inv_table, self.oq, self.iq = exp_table, inv_table, oq, iq
         self.input_scaler = input_scaler
@@ -680,13 +689,13 @@ class RefQSoftmax(RefQLayer):
         mask = self._mask
         if self.iq is not None:
             x = self.iq(x, training=training)
-        if mask is not None:
-            mask = mask.to(x.dtype)
-            x = mask * x - (1 - mask) * 1e9
-        x = torch.amax(x, dim=self.axes, keepdim=True) - x
+        if self.stable:
+            if mask is not None:
+                x = mask.to(x.dtype) * x - (1 - mask.to(x.dtype)) * 1e9
+            x = torch.amax(x, dim=self.axes, keepdim=True) - x
         e = self.exp_table(x, training=training)
         if mask is not None:
-            e = mask * e
+            e = mask.to(x.dtype) * e
         s = torch.sum(e, dim=self.axes, keepdim=True)
         return e * self.inv_table(s, training=training)
 
@@ -701,10 +710,16 @@ class RefQSoftmax(RefQLayer):
         inp_bits = self.iq.bits_(shape) if self.iq is not None else 0
         exp_bits = self.exp_table.oq.bits_(shape)
         inv_bits = self.inv_table.oq.bits_(accum_shape)
-        sub = torch.sum(inp_bits) if self.iq is not None else torch.sum(self.exp_table.iq.bits_(shape))
+        if self.stable:
+            sub = torch.sum(inp_bits) if self.iq is not None else torch.sum(self.exp_table.iq.bits_(shape))
+        else:
+            sub = 0.0
         accum = torch.sum(exp_bits) - torch.sum(torch.amin(exp_bits, dim=self.axes))
         mult = torch.sum(exp_bits * inv_bits)
-        return (sub + accum + mult) * factor
+        ebops = sub + accum + mult
+        if not self.stable:  # the exp table has no input quantizer of its own: its size is counted here (:150-152)
+            ebops = ebops + torch.sum((2.0**inp_bits) * exp_bits) * 1e-4
+        return ebops * factor
 
 
 def keras_attention_equations(rank, attn_axes):
@@ -823,7 +838,7 @@ class RefQConv2D(RefQLayer):
 
     def conv(self, x, w):
         x = x.permute(0, 3, 1, 2)
-        w = w.permute(3, 2, 0, 1)
+        w = w.permute(3, 2, 0, 1).contiguous()  # (a permuted one-filter kernel trips torch's CPU convolution backward)
         if self.padding == 'same':
             pads = []
             for d in (1, 0):

@@ -25,6 +25,9 @@ def _reg(r):
     return None if r is None else r.l1
 
 
+PAIRS = []  # (product internal quantizer, oracle internal quantizer) of every twin built since the list was cleared
+
+
 def ref_quantizer(q):
     """hgq2_amd.quantizer.Quantizer -> oracle RefQuantizer with copied variables."""
     if q is None:
@@ -52,6 +55,7 @@ def ref_quantizer(q):
             r._f.copy_(inner._f.detach().cpu())
         else:
             r._b.copy_(inner._b.detach().cpu())
+    PAIRS.append((inner, r))
     return ref.RefQuantizer(r, q.scaler, q.affine, q.qnoise_factor)
 
 
@@ -106,10 +110,12 @@ def ref_lut(layer, fn):
 
 def ref_softmax(layer):
     scaler = layer.input_scaler
-    exp = ref_lut(layer.exp_table, lambda x: torch.exp(-x * scaler))
+    sign = -1.0 if layer.stable else 1.0
+    exp = ref_lut(layer.exp_table, lambda x: torch.exp(sign * x * scaler))
     inv = ref_lut(layer.inv_table, lambda x: 1.0 / (x + ref.EPSILON))
     return ref.RefQSoftmax(layer.axes, exp, inv, _oq(layer), iq=_iq(layer), input_scaler=scaler, beta0=_beta(layer),
-                           enable_ebops=layer.enable_ebops, parallelization_factor=layer.parallelization_factor)
+                           enable_ebops=layer.enable_ebops, parallelization_factor=layer.parallelization_factor,
+                           stable=layer.stable)
 
 
 def ref_mha(layer, query_shape, value_shape=None, key_shape=None):
