@@ -464,6 +464,32 @@ def test_ebops_softmax_bruteforce(with_iq, pf):
     assert float(sm._compute_ebops(shape)) == pytest.approx(float(want), rel=1e-6)
 
 
+def test_unstable_softmax_form_is_softmax_and_counts_its_exp_table_itself():
+    """``stable=False`` (reference src/hgq/layers/softmax.py:49-53,87-96,116-120,150-152): no maximum is subtracted and the
+    exp table evaluates exp(+x * scaler) without an input quantizer, so with dummy quantizers the layer is still softmax;
+    in the EBOPs the subtraction drops out and the table size sum(2^input bits * exp bits) * 1e-4 is counted here."""
+    g = torch.Generator().manual_seed(27)
+    x = torch.randn(6, 3, 4, generator=g)
+    exp = ref.RefQUnaryFunctionLUT(lambda t: torch.exp(t * 0.5), None, dummy(), enable_ebops=False)
+    inv = ref.RefQUnaryFunctionLUT(lambda t: 1.0 / (t + ref.EPSILON), dummy(), dummy(), enable_ebops=False)
+    sm = ref.RefQSoftmax((2,), exp, inv, dummy(), iq=None, input_scaler=0.5, enable_ebops=False, stable=False)
+    assert torch.allclose(sm(x, training=False).double(), torch.softmax(x.double() * 0.5, dim=2), atol=1e-6)
+
+    A, S = 3, 4
+    shape = (1, A, S)
+    exp_oq = _q('table', (None, A, S), 'kbi', 'SAT', g, homogeneous_axis=(0,), k=0)
+    inv_iq = _q('datalane', (None, A, 1), 'kif', 'WRAP', g, heterogeneous_axis=())
+    inv_oq = _q('table', (None, A, 1), 'kbi', 'SAT', g, homogeneous_axis=(0,), k=0)
+    iq = _q('datalane', (None, A, S), 'kif', 'WRAP', g)
+    sm = ref.RefQSoftmax((2,), ref.RefQUnaryFunctionLUT(None, None, exp_oq, enable_ebops=False), ref.RefQUnaryFunctionLUT(None, inv_iq, inv_oq),
+                         None, iq=iq, stable=False)
+    be, bv, bi = int_bits(exp_oq, shape), int_bits(inv_oq, (1, A, 1)), int_bits(iq, shape)
+    accum = sum(sum(be[0][a]) - min(be[0][a]) for a in range(A))
+    mult = sum(be[0][a][s] * bv[0][a][0] for a in range(A) for s in range(S))
+    table = sum(Fraction(2) ** bi[0][a][s] * be[0][a][s] for a in range(A) for s in range(S)) / 10000
+    assert float(sm._compute_ebops(shape)) == pytest.approx(float(accum + mult + table), rel=1e-6)
+
+
 def test_ebops_mha_bruteforce():
     """Reference src/hgq/layers/attn/mha.py:386-416: every (query position, key position, head, channel) product of
     the two attention contractions, by nested loops over Python ints."""
