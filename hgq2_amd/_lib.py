@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, 'libhgq_hip.so')
 
 # mode bits, mirrored from include/hgq_hip.h
 TRN, RND, RND_CONV = 0, 1, 2
+S_RND, S_RND_CONV = 3, 4  # stochastic in training (hgq_quantize_*_stochastic), RND / RND_CONV otherwise
 WRAP, SAT, SAT_SYM = 0, 1, 2
 MODE_TRAINING = 1 << 8
 MODE_KBI = 1 << 9
@@ -39,6 +40,8 @@ SIGNATURES = {
     'hgq_quantize_tracker_slices': (c_int64, [c_int64, c_int64, c_int64]),
     'hgq_quantize_fwd_sliced': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_bwd': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    'hgq_quantize_fwd_stochastic': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int, ctypes.c_uint64, ctypes.c_uint64, c_void_p]),
+    'hgq_quantize_bwd_stochastic': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, ctypes.c_uint64, ctypes.c_uint64, c_void_p]),
     'hgq_wrap_track_i': (c_int, [c_void_p] * 2 + [c_int] + [c_void_p] * 3 + [c_int64, c_float, c_float, c_float, c_int, c_void_p]),
     'hgq_qdense_fwd_parts': (c_int, [c_int64]),
     'hgq_qdense_bwd_workspace': (c_int64, [c_int64, c_int, c_int, c_int64]),

@@ -108,6 +108,8 @@ class QSoftmax(QLayerBaseSingleInput):
             return None
         if shared and inner._i.numel() != 1:
             return None
+        if inner.stochastic and training is True:
+            return None  # stochastic rounding draws in its own kernel
         track = False
         if inner.overflow_mode == 'WRAP' and inner.trainable:
             if training == 'tracing' or (training and not isinstance(inner, FixedPointQuantizerKIF)):

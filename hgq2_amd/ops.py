@@ -1166,6 +1166,75 @@ class _Quantize(torch.autograd.Function):
                 dfb if ctx.needs_input_grad[3] else None, None, None, None)
 
 
+@torch.library.custom_op('hgq::quantize_fwd_stochastic', mutates_args=())
+def quantize_fwd_stochastic(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, track: bool, seed: int,
+                            offset: int) -> tuple[Tensor, Tensor, Tensor]:
+    """Training-mode quantizer with stochastic rounding: floor(x * 2^f + u), u a pure function of (seed, offset, element)."""
+    _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
+    bw = i.numel()
+    _need(k.numel() == bw and fb.numel() == bw and bw >= 1 and bw_inner >= 1, 'bit-width operands must have equal sizes')
+    y = torch.empty_like(x)
+    amax = torch.empty(bw if track else 0, dtype=torch.int32, device=x.device)
+    neg = torch.empty(bw if track else 0, dtype=torch.int32, device=x.device)
+    m = (_kmode(mode, k) & ~0xf) | _lib.S_RND
+    rc = _lib.load().hgq_quantize_fwd_stochastic(_ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(y), _ptr(amax) if track else None,
+                                                 _ptr(neg) if track else None, x.numel(), bw, bw_inner, m, seed, offset, _stream())
+    _lib.check(rc, 'hgq_quantize_fwd_stochastic')
+    return y, amax, neg
+
+
+@quantize_fwd_stochastic.register_fake
+def _(x, k, i, fb, mode, bw_inner, track, seed, offset):
+    n = i.numel() if track else 0
+    return torch.empty_like(x), x.new_empty(n, dtype=torch.int32), x.new_empty(n, dtype=torch.int32)
+
+
+@torch.library.custom_op('hgq::quantize_bwd_stochastic', mutates_args=())
+def quantize_bwd_stochastic(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, seed: int,
+                            offset: int) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('dy', dy), _check_f32('x', x)
+    _need(dy.shape == x.shape, 'dy shape mismatch')
+    dx, di, dfb = torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+    m = (_kmode(mode, k) & ~0xf) | _lib.S_RND
+    rc = _lib.load().hgq_quantize_bwd_stochastic(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), _ptr(di), _ptr(dfb), x.numel(),
+                                                 i.numel(), bw_inner, m, seed, offset, _stream())
+    _lib.check(rc, 'hgq_quantize_bwd_stochastic')
+    return dx, di, dfb
+
+
+@quantize_bwd_stochastic.register_fake
+def _(dy, x, k, i, fb, mode, bw_inner, seed, offset):
+    return torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+
+
+class _QuantizeStochastic(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, k, i, fb, mode, bw_inner, track, seed, offset):
+        y, amax, neg = quantize_fwd_stochastic(x, k, i, fb, mode, bw_inner, track, seed, offset)
+        ctx.save_for_backward(x, k, i, fb)
+        ctx.mode, ctx.bw_inner, ctx.draw = mode, bw_inner, (seed, offset)
+        ctx.mark_non_differentiable(amax, neg)
+        ctx.set_materialize_grads(False)
+        return y, amax, neg
+
+    @staticmethod
+    def backward(ctx, gy, _ga, _gn):
+        if gy is None:
+            return (None,) * 9
+        x, k, i, fb = ctx.saved_tensors
+        dx, di, dfb = quantize_bwd_stochastic(gy.contiguous(), x, k, i, fb, ctx.mode, ctx.bw_inner, *ctx.draw)
+        return (dx if ctx.needs_input_grad[0] else None, None, di if ctx.needs_input_grad[2] else None,
+                dfb if ctx.needs_input_grad[3] else None, None, None, None, None, None)
+
+
+def quantize_stochastic(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, seed: int, offset: int, bw_inner: int = 1,
+                        track: bool = False):
+    """The training-mode quantizer of round modes S_RND / S_RND_CONV; ``(seed, offset)`` names the draw."""
+    _need(bool(mode & _lib.MODE_TRAINING), 'stochastic rounding applies to the training-mode forward only')
+    return _QuantizeStochastic.apply(x.contiguous(), k.contiguous(), i.contiguous(), fb.contiguous(), mode, bw_inner, track,
+                                     int(seed), int(offset))
+
+
 class _QuantItem(ctypes.Structure):
     _fields_ = [('x', ctypes.c_void_p), ('k', ctypes.c_void_p), ('i', ctypes.c_void_p), ('fb', ctypes.c_void_p),
                 ('y', ctypes.c_void_p), ('n', ctypes.c_int64), ('mode', ctypes.c_int)]

@@ -25,6 +25,31 @@ def _compact(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+class SeedGenerator:
+    """Stands in for ``keras.random.SeedGenerator`` (reference :56-57): a seed and a counter that advances with every
+    draw.  ``next()`` names one call's draw as ``(seed, offset)``; the kernels derive every element's uniform number from
+    that pair, so the backward pass recomputes it.  Keras' own stream is backend-specific and is not reproduced."""
+
+    def __init__(self, seed: int | None = None):
+        self.seed = int(seed if seed is not None else torch.seed()) & (2**63 - 1)
+        self.offset = 0
+
+    def next(self):
+        if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+            # the pair travels as a launch argument: a captured launch would repeat the same draw on every replay
+            raise RuntimeError('stochastic rounding cannot be captured into a HIP graph: its draw would be the same on every replay')
+        self.offset += 1
+        return self.seed, self.offset
+
+
+def _draw(seed_gen):
+    if isinstance(seed_gen, SeedGenerator):
+        return seed_gen.next()
+    if isinstance(seed_gen, (tuple, list)) and len(seed_gen) == 2:
+        return int(seed_gen[0]), int(seed_gen[1])
+    raise TypeError('stochastic rounding needs seed_gen: a SeedGenerator or a (seed, offset) pair')
+
+
 class FixedQuantizer:
     def __init__(self, round_mode: str = 'TRN', overflow_mode: str = 'WRAP'):
         round_mode = round_mode.upper()
@@ -33,7 +58,7 @@ class FixedQuantizer:
         self.overflow_mode = overflow_mode.upper()
         _lib.mode_bits(self.round_mode, self.overflow_mode)  # validates
 
-    def _run(self, x, k, i, f, training, overflow_mode):
+    def _run(self, x, k, i, f, training, overflow_mode, draw=None):
         shape = tuple(x.shape)
         small = []
         for t in (k, i, f):
@@ -49,23 +74,24 @@ class FixedQuantizer:
             bw_shape, layout = shape, (x.numel(), 1)
         kc, ic, fc = (t.expand(bw_shape).contiguous() for t in small)
         mode = _lib.mode_bits(self.round_mode, overflow_mode, training=bool(training))
-        y, _, _ = ops.quantize(x.contiguous(), kc, ic, fc, mode, bw_inner=layout[1])
+        if draw is not None:
+            y, _, _ = ops.quantize_stochastic(x.contiguous(), kc, ic, fc, mode, draw[0], draw[1], bw_inner=layout[1])
+        else:
+            y, _, _ = ops.quantize(x.contiguous(), kc, ic, fc, mode, bw_inner=layout[1])
         return y
 
     def __call__(self, x, k, i, f, training=False, seed_gen=None):
-        if self.stochastic and training:
-            raise NotImplementedError('stochastic rounding is not part of this build')
+        # stochastic modes draw in training and are their deterministic counterparts otherwise.
         # inference mode: entries with k+i+f <= 0 (empty words) come out as zero, which is what
         # the reference applies around the callable (fixed_point_quantizer.py:148-149)
-        return self._run(x, k, i, f, training, self.overflow_mode)
+        draw = _draw(seed_gen) if (self.stochastic and training) else None
+        return self._run(x, k, i, f, training, self.overflow_mode, draw)
 
     def round(self, x, f, stochastic=False, seed_gen=None):
-        if stochastic:
-            raise NotImplementedError('stochastic rounding is not part of this build')
         # rounding only = the WRAP training branch; k and i are not read there (0-dim constants, nothing expanded)
         one = torch.ones((), dtype=x.dtype, device=x.device)
         zero = torch.zeros((), dtype=x.dtype, device=x.device)
-        return self._run(x, one, zero, f, True, 'WRAP')
+        return self._run(x, one, zero, f, True, 'WRAP', _draw(seed_gen) if stochastic else None)
 
 
 def get_fixed_quantizer(round_mode: str = 'TRN', overflow_mode: str = 'WRAP') -> FixedQuantizer:

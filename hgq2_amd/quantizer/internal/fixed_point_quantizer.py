@@ -42,11 +42,13 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
         return self._seed_gen
 
     def build(self, input_shape):
-        if self.round_mode.startswith('S_'):
-            raise NotImplementedError('stochastic rounding modes are not part of this build')
         if self.overflow_mode not in _lib.OVERFLOW_MODES:
             raise ValueError(f'unsupported overflow mode {self.overflow_mode}')
-        if self.round_mode not in _lib.ROUND_MODES:
+        if self.round_mode.startswith('S_'):  # reference :56-57
+            from ..fixed_point_ops import SeedGenerator
+
+            self._seed_gen = SeedGenerator(self._seed)
+        if (self.round_mode[2:] if self.round_mode.startswith('S_') else self.round_mode) not in _lib.ROUND_MODES:
             raise ValueError(f'unsupported round mode {self.round_mode}')
         if self.overflow_mode == 'WRAP':
             init = self._i_decay_speed0
@@ -151,8 +153,16 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
         t = torch.broadcast_to(self._third(), shape).contiguous()
         return k, i, t, (x.numel(), 1)
 
-    def _quantize(self, x, mode: int, track: bool = False):
+    @property
+    def stochastic(self) -> bool:
+        return self._seed_gen is not None
+
+    def _quantize(self, x, mode: int, track: bool = False, stochastic: bool = False):
+        """``stochastic``: this call is one of those the reference hands ``seed_gen`` to with training on (:147,:279,:404)."""
         k, i, t, (_, inner) = self._operands(x)
+        if stochastic and self.stochastic and (mode & _lib.MODE_TRAINING):
+            seed, offset = self._seed_gen.next()
+            return ops.quantize_stochastic(x, k, i, t, mode, seed, offset, bw_inner=inner, track=track)
         return ops.quantize(x, k, i, t, mode, bw_inner=inner, track=track)
 
     def _constraint_bounds(self):
@@ -186,7 +196,7 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
         pf, self._prefetched = self._prefetched, None
         if pf is not None and training and pf[0] is inputs:
             return pf[1]
-        y, _, _ = self._quantize(inputs, self._mode(training))
+        y, _, _ = self._quantize(inputs, self._mode(training), stochastic=training)
         return y
 
     def call(self, inputs, training=None):
@@ -268,7 +278,7 @@ class FixedPointQuantizerKBI(FixedPointQuantizerBase):
                 track_mode = self._mode(True) | _lib.MODE_TRACK_INPUT
                 _, amax, _ = self._quantize(inputs.detach(), track_mode, track=True)
                 self._track(amax, is_training, clip=True)
-                y, _, neg = self._quantize(inputs, self._mode(True), track=not is_training)
+                y, _, neg = self._quantize(inputs, self._mode(True), track=not is_training, stochastic=training is True)
                 if not is_training:
                     with torch.no_grad():
                         # the tracker arrives as one entry per bit-width entry or as [slices, entries]
@@ -323,13 +333,13 @@ class FixedPointQuantizerKIF(FixedPointQuantizerBase):
     def wrap_training_fusable(self, training) -> bool:
         """True when the call reduces to "round with f, track max|.|" (reference :401-413), the
         form the dense kernel fuses into its operand load."""
-        return self.overflow_mode == 'WRAP' and self.trainable and training is True
+        return self.overflow_mode == 'WRAP' and self.trainable and training is True and not self.stochastic
 
     def call(self, inputs, training=None):
         if self.overflow_mode == 'WRAP' and self.trainable:
             if training or training == 'tracing':
                 is_training = bool(training)
-                y, amax, neg = self._quantize(inputs, self._mode(True), track=True)
+                y, amax, neg = self._quantize(inputs, self._mode(True), track=True, stochastic=training is True)
                 # training: the reference applies the constraint to a dead value (:411-412), so the
                 # assigned value is unclipped; tracing clips before the max (:416-418)
                 self._track(amax, is_training, anyneg=neg)

@@ -18,7 +18,7 @@ def _eligible(q, p):
     if q is None or p is None or not getattr(q, 'built', False) or not q.plain:
         return None
     fq = q.quantizer
-    if not isinstance(fq, FixedPointQuantizerBase) or fq.overflow_mode == 'WRAP':
+    if not isinstance(fq, FixedPointQuantizerBase) or fq.overflow_mode == 'WRAP' or fq.stochastic:
         return None
     if not (p.is_cuda and p.dtype == torch.float32 and p.is_contiguous()):
         return None

@@ -188,6 +188,7 @@ class FusedQDenseStack:
                   and layer.kq.plain and isinstance(qk, FixedPointQuantizerKBI) and qk.overflow_mode != 'WRAP'
                   and (qb is None or (layer.bq.plain and isinstance(qb, FixedPointQuantizerKBI) and qb.overflow_mode != 'WRAP'))
                   and layer._act_name in ('relu', 'linear') and not layer.enable_oq
+                  and not any(q is not None and q.stochastic for q in (qi, qk, qb))
                   and all(getattr(p, 'regularizer', None) is None and getattr(p, 'constraint', None) is None
                           for p in (layer._kernel, layer.bias) if p is not None))
             if not ok:

@@ -40,6 +40,8 @@ extern "C" {
 #define HGQ_TRN 0
 #define HGQ_RND 1
 #define HGQ_RND_CONV 2
+#define HGQ_S_RND 3      /* stochastic in training (hgq_quantize_*_stochastic); RND otherwise */
+#define HGQ_S_RND_CONV 4 /* stochastic in training; RND_CONV otherwise */
 /* overflow modes (second nibble of `mode`) */
 #define HGQ_WRAP 0
 #define HGQ_SAT 1
@@ -107,6 +109,23 @@ int hgq_quantize_fwd_sliced(const float *x, const void *k, const float *i, const
 int64_t hgq_quantize_bwd_workspace(int64_t n, int64_t bw_size, int64_t bw_inner);
 int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
                             float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
+
+/*
+ * Stochastic rounding: the training-mode forward and surrogate backward of round modes S_RND / S_RND_CONV
+ * (src/hgq/quantizer/internal/fixed_point_quantizer.py:56-57,279,288,404-405: `q(..., seed_gen)`,
+ * `q.round(x, f, stochastic, seed_gen)`): R(t) = floor(t + u) with u uniform in [0, 1), then the overflow mode.
+ * The reference's draws come from a Keras SeedGenerator, whose stream is backend-specific; here element e of a call
+ * draws u = (word e % 4 of Philox4x32-10(counter = (e / 4, offset), key = seed) >> 8) * 2^-24, so a call is a pure
+ * function of (seed, offset): pass the same pair to the backward, and a new offset to every forward call.
+ * Outside training these round modes are the deterministic RND / RND_CONV: call hgq_quantize_fwd with that mode.
+ *   amax / anyneg [bw_size] optional trackers as in hgq_quantize_fwd.  di / dfb [bw_size]: with shared bit-widths the
+ *   sums are accumulated with float atomics (the last bits depend on the order of arrival).
+ */
+int hgq_quantize_fwd_stochastic(const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax, uint32_t *anyneg,
+                                int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset, void *stream);
+int hgq_quantize_bwd_stochastic(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
+                                float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset,
+                                void *stream);
 
 /*
  * Measurement aid (no counterpart in the reference): o_j[e] = (j + 1) * (a[e] (+ b[e]) (+ c[e])) for the first n_write

@@ -44,8 +44,12 @@ What pins what
 * ``i`` is not clamped against ``-f`` inside the callable (any such clamp in the
   third-party package is unpinned; it can only matter where k+i+f <= 0, which the
   reference zeroes at inference, fixed_point_quantizer.py:148-149).
-* stochastic modes (``S_RND``, ``S_RND_CONV``): only the deterministic branch
-  (``stochastic=False`` or ``training=False``) is restated.
+* stochastic modes (``S_RND``, ``S_RND_CONV``): the rule floor(x * 2^f + u), u uniform in [0, 1), in training and the
+  deterministic counterpart otherwise is what the name and the call sites (fpq.py:279,404) fix; the package's own
+  random stream (keras.random, backend-specific) cannot be matched, so the draw is this build's definition
+  (``stochastic_uniform``: Philox4x32-10 keyed by the seed, counter = element block and call offset), pinned by the
+  generator's published known-answer vectors and by the properties of stochastic rounding (neighbour values only,
+  unbiased mean, reproducible per (seed, offset)).
 """
 
 from __future__ import annotations
@@ -94,25 +98,71 @@ def round_conv(x: torch.Tensor) -> torch.Tensor:
     return _RoundConv.apply(x)
 
 
+def philox4x32_10(counter, key):
+    """Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11) on numpy uint64
+    arrays holding 32-bit words: ``counter`` four arrays, ``key`` two; returns the four output words.  Pinned by the
+    known-answer vectors of the authors' Random123 library (tests/test_oracle_pins.py)."""
+    import numpy as np
+
+    mask = np.uint64(0xFFFFFFFF)
+    c = [np.asarray(v, dtype=np.uint64) & mask for v in counter]
+    k = [np.asarray(v, dtype=np.uint64) & mask for v in key]
+    for _ in range(10):
+        p0, p1 = np.uint64(0xD2511F53) * c[0], np.uint64(0xCD9E8D57) * c[2]  # 32 x 32 -> 64 bits: no overflow in uint64
+        c = [(p1 >> np.uint64(32)) ^ c[1] ^ k[0], p1 & mask, (p0 >> np.uint64(32)) ^ c[3] ^ k[1], p0 & mask]
+        k = [(k[0] + np.uint64(0x9E3779B9)) & mask, (k[1] + np.uint64(0xBB67AE85)) & mask]
+    return c
+
+
+def stochastic_uniform(n: int, seed: int, offset: int) -> torch.Tensor:
+    """The n uniform numbers in [0, 1) of one stochastic-rounding call: element e takes word e % 4 of the block with
+    counter (e // 4, offset) under key ``seed``, top 24 bits.  (The draw this build defines; the reference's comes from
+    keras.random and differs per backend.)"""
+    import numpy as np
+
+    blocks = np.arange((n + 3) // 4, dtype=np.uint64)
+    off = np.full_like(blocks, offset)
+    words = philox4x32_10([blocks, blocks >> np.uint64(32), off, off >> np.uint64(32)],
+                          [np.uint64(seed), np.uint64(seed) >> np.uint64(32)])
+    flat = np.stack(words, axis=1).reshape(-1)[:n]
+    return torch.from_numpy(((flat >> np.uint64(8)).astype(np.float64) * 2.0**-24).astype(np.float32))
+
+
+class SeedGenerator:
+    """A seed and a call counter; ``next()`` names one call's draw."""
+
+    def __init__(self, seed):
+        self.seed, self.offset = int(seed), 0
+
+    def next(self):
+        self.offset += 1
+        return self.seed, self.offset
+
+
+def _draw(seed_gen):
+    return seed_gen.next() if hasattr(seed_gen, 'next') else (int(seed_gen[0]), int(seed_gen[1]))
+
+
 class _RoundF(torch.autograd.Function):
-    """Rounding to ``f`` fractional bits with the surrogate gradient (training)."""
+    """Rounding to ``f`` fractional bits with the surrogate gradient (training); with ``u`` the stochastic form
+    floor(x * 2^f + u)."""
 
     @staticmethod
-    def forward(ctx, x, f, round_mode):
+    def forward(ctx, x, f, round_mode, u=None):
         scale = _pow2(f)
-        xq = _round_scaled(x * scale, round_mode) / scale
+        xq = (torch.floor(x * scale + u) if u is not None else _round_scaled(x * scale, round_mode)) / scale
         ctx.save_for_backward(xq - x)
         return xq
 
     @staticmethod
     def backward(ctx, g):
         (delta,) = ctx.saved_tensors
-        return g, -LN2 * delta * g, None
+        return g, -LN2 * delta * g, None, None
 
 
-def fixed_round(x, f, round_mode: str, training: bool):
+def fixed_round(x, f, round_mode: str, training: bool, u=None):
     if training:
-        return _RoundF.apply(x, f, round_mode)
+        return _RoundF.apply(x, f, round_mode, u)
     scale = _pow2(f)
     return _round_scaled(x * scale, round_mode) / scale
 
@@ -164,15 +214,17 @@ class FixedQuantizer:
         self.overflow_mode = overflow_mode.upper()
         assert self.overflow_mode in OVERFLOW_MODES, overflow_mode
 
+    def _uniform(self, x, seed_gen):
+        seed, offset = _draw(seed_gen)
+        return stochastic_uniform(x.numel(), seed, offset).view(x.shape)  # element order = row-major order of x
+
     def round(self, x, f, stochastic=False, seed_gen=None, training=True):
-        if stochastic:
-            raise NotImplementedError('stochastic rounding is not restated by the oracle')
-        return fixed_round(x, f, self.round_mode, training)
+        return fixed_round(x, f, self.round_mode, training, self._uniform(x, seed_gen) if stochastic else None)
 
     def __call__(self, x, k, i, f, training=False, seed_gen=None):
-        if self.stochastic and training:
-            raise NotImplementedError('stochastic rounding is not restated by the oracle')
-        xq = fixed_round(x, f, self.round_mode, bool(training))
+        # a stochastic mode draws in training and is its deterministic counterpart otherwise
+        u = self._uniform(x, seed_gen) if (self.stochastic and training) else None
+        xq = fixed_round(x, f, self.round_mode, bool(training), u)
         return _overflow(xq, k, i, f, self.overflow_mode, bool(training))
 
 

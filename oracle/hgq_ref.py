@@ -23,7 +23,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from .fixed_point import get_fixed_quantizer, round_conv
+from .fixed_point import SeedGenerator, get_fixed_quantizer, round_conv
 
 EPSILON = 1e-7  # keras.backend.epsilon() default
 
@@ -153,6 +153,7 @@ class RefFixedPointQuantizer:
         heterogeneous_axis=None,
         is_weight=False,
         trainable=True,
+        seed=0,
     ):
         self.q_type = q_type
         self.round_mode = round_mode.upper()
@@ -162,6 +163,7 @@ class RefFixedPointQuantizer:
         self.trainable = trainable
         self.bw_mapper = BitwidthMapper(heterogeneous_axis, homogeneous_axis)
         self.q = get_fixed_quantizer(self.round_mode, self.overflow_mode)
+        self.seed_gen = SeedGenerator(seed) if self.q.stochastic else None  # fpq.py:56-57
         shape = self.bw_mapper.inference_weight_shape(tuple(input_shape))
         self._k = torch.full(shape, int(k0), dtype=torch.uint8)
         i_trainable = self.overflow_mode != 'WRAP'
@@ -262,7 +264,7 @@ class RefFixedPointQuantizer:
         k = self.bw_mapper.bw_to_x(k, x.shape)
         i = self.bw_mapper.bw_to_x(i, x.shape)
         f = self.bw_mapper.bw_to_x(f, x.shape)
-        ret = self.q(x, k, i, f, training is True, None)
+        ret = self.q(x, k, i, f, training is True, self.seed_gen)
         if not training:
             ret = torch.where(k + i + f > 0, ret, torch.zeros_like(ret))
         return ret
@@ -276,7 +278,8 @@ class RefFixedPointQuantizer:
     def _call_kif(self, x, training):
         if self.overflow_mode == 'WRAP' and self.trainable:
             f = self.bw_mapper.bw_to_x(self.f, x.shape)
-            rx = self.q.round(x, f, False, None)
+            stochastic = self.q.stochastic and training is True  # fpq.py:404
+            rx = self.q.round(x, f, stochastic, self.seed_gen)
             if training or training == 'tracing':
                 xr = self.bw_mapper.x_to_bw_absmax(rx.detach())
                 _new_i = minimal_i_given_xf(xr, self.f.detach(), self.symmetric)
@@ -308,7 +311,7 @@ class RefFixedPointQuantizer:
                         new_i = _clip_constraint(self.i_constraint, new_i)
                         self._i.copy_(new_i)
                     f = self.bw_mapper.bw_to_x(self.f, x.shape)
-                    return self.q.round(x, f, False, None)
+                    return self.q.round(x, f, self.q.stochastic, self.seed_gen)  # fpq.py:279,288
                 with torch.no_grad():
                     new_i = torch.maximum(self.i.detach(), new_i)
                     new_i = _clip_constraint(self.i_constraint, new_i)

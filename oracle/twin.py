@@ -39,7 +39,7 @@ def ref_quantizer(q):
     shape = tuple(inner._i.shape)
     kw = dict(round_mode=inner.round_mode, overflow_mode=inner.overflow_mode, ic=_constraint(cfg.get('ic')),
               ir=_reg(cfg.get('ir')), i_decay_speed=cfg['i_decay_speed'], heterogeneous_axis=tuple(range(len(shape))),
-              is_weight=cfg['is_weight'], trainable=cfg['trainable'])
+              is_weight=cfg['is_weight'], trainable=cfg['trainable'], seed=getattr(inner, '_seed', 0))
     if q.config.q_type == 'kif':
         kw.update(fc=_constraint(cfg.get('fc')), fr=_reg(cfg.get('fr')))
     else:
@@ -55,6 +55,8 @@ def ref_quantizer(q):
             r._f.copy_(inner._f.detach().cpu())
         else:
             r._b.copy_(inner._b.detach().cpu())
+    if r.seed_gen is not None:  # both sides continue from the same position of the same stream
+        r.seed_gen.seed, r.seed_gen.offset = inner._seed_gen.seed, inner._seed_gen.offset
     PAIRS.append((inner, r))
     return ref.RefQuantizer(r, q.scaler, q.affine, q.qnoise_factor)
 

@@ -341,3 +341,102 @@ def test_full_size_backward_matches_oracle(dev, acc64, kind):
             else:
                 _close_tensor(p.grad, rv.grad, f'{what}: d{vname}')
         h = h_next  # continue from the oracle's activations
+
+
+# ---- stochastic rounding (round modes S_RND / S_RND_CONV)
+@pytest.mark.parametrize('overflow_mode', ['WRAP', 'SAT', 'SAT_SYM'])
+@pytest.mark.parametrize('bw_shape', [None, (1, 37), ()])
+def test_stochastic_rounding_kernels_match_oracle(dev, overflow_mode, bw_shape):
+    """The training-mode forward and surrogate backward with the draw named by (seed, offset): values bit-exact against
+    the oracle's restatement of the same generator, gradients to 1e-5, for per-element, per-column and scalar bit-widths."""
+    from hgq2_amd import _lib, ops
+
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(301, 37, generator=g) * 3
+    shape = tuple(x.shape) if bw_shape is None else bw_shape
+    k = torch.randint(0, 2, shape, generator=g).float()
+    i = torch.randint(-1, 3, shape, generator=g).float()
+    f = torch.randint(0, 6, shape, generator=g).float()
+    seed, offset = 2**40 + 12345, 2**33 + 9
+    q = ofp.get_fixed_quantizer("S_RND", overflow_mode)
+    xr, ir, fr = x.clone().requires_grad_(True), i.clone().requires_grad_(True), f.clone().requires_grad_(True)
+    want = q(xr, k.expand(x.shape), ir.expand(x.shape), fr.expand(x.shape), True, (seed, offset))
+    up = torch.randn(x.shape, generator=g)
+    (want * up).sum().backward()
+    from hgq2_amd.quantizer.internal.base import bw_layout
+
+    inner = bw_layout(shape, tuple(x.shape))[1]
+    xd = x.to(dev).requires_grad_(True)
+    idv, fd = i.reshape(-1).to(dev).requires_grad_(True), f.reshape(-1).to(dev).requires_grad_(True)
+    mode = _lib.mode_bits('S_RND', overflow_mode, training=True)
+    got, _, _ = ops.quantize_stochastic(xd, k.reshape(-1).to(dev), idv, fd, mode, seed, offset, bw_inner=inner)
+    assert torch.equal(got.detach().cpu(), want.detach()), float((got.detach().cpu() - want.detach()).abs().max())
+    (got * up.to(dev)).sum().backward()
+    assert torch.equal(xd.grad.cpu(), xr.grad)
+    for name, a, b in (('di', idv.grad, ir.grad), ('df', fd.grad, fr.grad)):
+        if b is None:  # WRAP in training is rounding only: nothing reaches the integer bits
+            assert a is None or float(a.abs().max()) == 0.0, name
+            continue
+        b = b.reshape(-1)
+        scale = float(b.abs().max()) + 1e-30
+        terms = math.log(2.0) * float(up.abs().sum()) / max(b.numel(), 1) if bw_shape is not None else 0.0  # sum of |terms| per entry, about
+        assert float((a.cpu() - b).abs().max()) <= 1e-5 * (scale + terms), name
+    # another offset is another draw; the same pair repeats it
+    again, _, _ = ops.quantize_stochastic(xd.detach(), k.reshape(-1).to(dev), idv.detach(), fd.detach(), mode, seed, offset, bw_inner=inner)
+    other, _, _ = ops.quantize_stochastic(xd.detach(), k.reshape(-1).to(dev), idv.detach(), fd.detach(), mode, seed, offset + 1, bw_inner=inner)
+    assert torch.equal(again, got.detach()) and not torch.equal(other, got.detach())
+
+
+@pytest.mark.parametrize('q_type,overflow_mode,round_mode', [('kif', 'WRAP', 'S_RND'), ('kif', 'SAT', 'S_RND_CONV'), ('kbi', 'WRAP', 'S_RND'),
+                                                             ('kbi', 'SAT_SYM', 'S_RND')])
+def test_stochastic_quantizer_classes_follow_the_oracle(dev, q_type, overflow_mode, round_mode):
+    """KIF / KBI quantizer layers with a stochastic round mode: two training calls (the generator advances), the tracked
+    integer bits, the gradients, a tracing call and inference (both deterministic) against the oracle twin."""
+    from hgq2_amd.quantizer import Quantizer, QuantizerConfig
+
+    g = torch.Generator().manual_seed(78)
+    x = torch.randn(700, 24, generator=g) * 2
+    conf = QuantizerConfig(q_type, 'datalane', overflow_mode=overflow_mode, round_mode=round_mode)
+    q = Quantizer(conf)
+    q.quantizer._seed = 4242  # (drawn at random at construction, like the reference's; fixed here before the build uses it)
+    q(x.to(dev), training=True)  # build
+    r = twin.ref_quantizer(q)
+    assert q.quantizer.stochastic and r.quantizer.seed_gen is not None
+    for step in range(2):
+        xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
+        yp, yr = q(xp, training=True), r(xr, training=True)
+        assert torch.equal(yp.detach().cpu(), yr.detach()), f'step {step}'
+        assert torch.equal(q.quantizer._i.detach().cpu(), r.quantizer._i.detach()), f'step {step}'
+        up = torch.randn(x.shape, generator=g)
+        for v in (q.quantizer._i, q.quantizer._third(), r.quantizer._i, r.quantizer._f if q_type == 'kif' else r.quantizer._b):
+            v.grad = None
+        (yp * up.to(dev)).sum().backward()
+        (yr * up).sum().backward()
+        assert torch.equal(xp.grad.cpu(), xr.grad)
+        want = (r.quantizer._f if q_type == 'kif' else r.quantizer._b).grad
+        got = q.quantizer._third().grad
+        bound = 1e-5 * (float(want.abs().max()) + math.log(2.0) * float(up.abs().sum()) / want.numel())
+        assert float((got.cpu() - want).abs().max()) <= bound, f'step {step}'
+    assert q.quantizer._seed_gen.offset == r.quantizer.seed_gen.offset == 3
+    from hgq2_amd.core import TrainingFlagWrapper
+
+    with torch.no_grad():
+        assert torch.equal(q(x.to(dev), training=TrainingFlagWrapper('tracing')).cpu(), r(x, training=TrainingFlagWrapper('tracing')))
+        assert torch.equal(q(x.to(dev), training=False).cpu(), r(x, training=False))
+    assert q.quantizer._seed_gen.offset == 3  # no draw outside training
+
+
+def test_stochastic_rounding_refuses_graph_capture(dev):
+    from hgq2_amd.quantizer.fixed_point_ops import SeedGenerator
+
+    gen = SeedGenerator(1)
+    graph = torch.cuda.CUDAGraph()
+    x = torch.zeros(8, device=dev)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        with pytest.raises(RuntimeError, match='HIP graph'):
+            with torch.cuda.graph(graph, stream=s):
+                x.add_(1.0)
+                gen.next()
+    torch.cuda.current_stream().wait_stream(s)

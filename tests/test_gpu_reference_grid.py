@@ -279,3 +279,18 @@ def test_qbatch_normalization(dev, grid):
         return twin.ref_batchnorm(layer)
 
     _run_case(dev, make, (6, 8), make_twin, grid, 107)
+
+
+# ---- stochastic round modes (the reference lists S_RND / S_RND_CONV beside the deterministic ones,
+# src/hgq/quantizer/internal/fixed_point_quantizer.py:166,323; its tests do not run them)
+@pytest.mark.parametrize('round_mode', ['S_RND', 'S_RND_CONV'])
+@pytest.mark.parametrize('overflow_mode', ['WRAP', 'SAT'])
+@pytest.mark.parametrize('parallel_io', [True, False], ids=['elem', 'tensor'])
+def test_layers_with_stochastic_rounding(dev, round_mode, overflow_mode, parallel_io):
+    """Every quantizer of a QDense and a QConv2D layer (kif weights, bias and data) rounds stochastically in training:
+    the twin continues each quantizer's generator from the same position, so outputs are compared exactly as above."""
+    from hgq2_amd.layers import QConv2D, QDense
+
+    grid = (parallel_io, 'kif', overflow_mode, round_mode)
+    _run_case(dev, lambda: QDense(8, activation='relu'), (8, 8), lambda layer, s: twin.ref_dense(layer), grid, 108)
+    _run_case(dev, lambda: QConv2D(4, kernel_size=(3, 3), padding='same'), (6, 6, 2), lambda layer, s: twin.ref_conv2d(layer), grid, 109)

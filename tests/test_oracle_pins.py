@@ -3,6 +3,7 @@
 differences, textbook routines)."""
 
 import itertools
+import math
 from fractions import Fraction
 
 import numpy as np
@@ -211,3 +212,57 @@ def test_dummy_quantizers_reduce_qbatchnorm_to_batch_normalisation():
     bn2 = ref.RefQBatchNormalization(2, None, None, torch.zeros(5), torch.ones(5), q(), q(), q(), momentum=0.0, enable_ebops=False)
     y2 = bn2(x, training=True)
     assert torch.allclose(y2, ((x.double() - mean) / torch.sqrt(var + 1e-3) + 1.0).float(), atol=2e-6)
+
+
+def test_philox4x32_10_known_answers():
+    """The three known-answer vectors of the Random123 library (kat_vectors, philox4x32 with 10 rounds)."""
+    import numpy as np
+
+    from oracle.fixed_point import philox4x32_10
+
+    cases = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+             ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+             ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0), (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in cases:
+        got = philox4x32_10([np.array([c], dtype=np.uint64) for c in ctr], [np.uint64(k) for k in key])
+        assert tuple(int(w[0]) for w in got) == want
+    # vectorised: the blocks of an array are the blocks of its elements
+    ctrs = np.arange(5, dtype=np.uint64)
+    many = philox4x32_10([ctrs, ctrs * 0, ctrs * 0 + np.uint64(7), ctrs * 0], [np.uint64(3), np.uint64(0)])
+    for j in range(5):
+        one = philox4x32_10([np.array([j], dtype=np.uint64), np.zeros(1, np.uint64), np.full(1, 7, np.uint64), np.zeros(1, np.uint64)],
+                            [np.uint64(3), np.uint64(0)])
+        assert [int(w[j]) for w in many] == [int(w[0]) for w in one]
+
+
+def test_stochastic_rounding_is_floor_or_ceil_unbiased_and_reproducible():
+    """S_RND in training: every value is one of the two neighbours on the 2^-f grid, the mean over many draws is the
+    input (the defining property of stochastic rounding), a draw is a function of (seed, offset) only, grid points are
+    fixed points, and outside training the mode is plain RND."""
+    from oracle.fixed_point import SeedGenerator, get_fixed_quantizer, stochastic_uniform
+
+    u = stochastic_uniform(100001, 12345, 1)
+    assert float(u.min()) >= 0.0 and float(u.max()) < 1.0 and abs(float(u.double().mean()) - 0.5) < 5e-3
+    assert torch.equal(u[:4097], stochastic_uniform(4097, 12345, 1))  # a prefix does not depend on the length
+    assert not torch.equal(u[:64], stochastic_uniform(64, 12345, 2)[:64])
+
+    q = get_fixed_quantizer('S_RND', 'WRAP')
+    assert q.stochastic and q.round_mode == 'RND'
+    x = torch.tensor([0.3, -1.26, 2.0, 0.125]).repeat(20000, 1)
+    f = torch.full_like(x, 2.0)
+    gen = SeedGenerator(7)
+    y = q.round(x, f, True, gen)
+    lo = torch.floor(x * 4) / 4
+    assert bool(((y == lo) | (y == lo + 0.25)).all())
+    assert bool((y[:, 2] == 2.0).all())  # already on the grid
+    assert torch.allclose(y.double().mean(0), x[0].double(), atol=4e-3)
+    assert torch.equal(q.round(x, f, True, (7, 1)), y) and gen.offset == 1
+    assert not torch.equal(q.round(x, f, True, gen), y)  # the generator has moved on
+    k, i = torch.ones_like(x), torch.full_like(x, 3.0)
+    assert torch.equal(q(x, k, i, f, False, gen), get_fixed_quantizer('RND', 'WRAP')(x, k, i, f, False, None))
+    # surrogate gradient of the draw that was made: d/df = -ln2 * (y - x), d/dx = 1
+    xg, fg = x[:8].clone().requires_grad_(True), f[:8].clone().requires_grad_(True)
+    yy = q.round(xg, fg, True, (7, 1))
+    yy.sum().backward()
+    assert torch.equal(xg.grad, torch.ones_like(xg))
+    assert torch.allclose(fg.grad, -math.log(2.0) * (yy.detach() - xg.detach()), rtol=1e-6, atol=0)
