@@ -77,6 +77,7 @@ SIGNATURES = {
     'hgq_quantize_bwd_sliced': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_conv2d_ebops_q': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_dense_ebops_multi': (c_int, [c_void_p, c_int, c_void_p]),
+    'hgq_wrap_track_i_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_qdense_bwd_slices': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 3 + [c_int, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     'hgq_reduce_slices_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_stream_probe': (c_int, [c_void_p] * 6 + [c_int, c_int, c_int64, c_void_p]),

@@ -604,14 +604,13 @@ __global__ __launch_bounds__(Q1D_BS) void stream_probe_kernel(const f32x4 *__res
 // 1024 threads = 64 entries x 16 slice groups: the abs-max / any-negative trackers arrive as
 // `n_parts` slices of [n] (one per producing workgroup) and are combined here.
 #define WT_G 16
-__global__ __launch_bounds__(64 * WT_G) void wrap_track_i_kernel(const uint32_t *__restrict__ amax,
-                                                                 const uint32_t *__restrict__ anyneg, int n_parts,
-                                                                 float *i_var, const float *__restrict__ fb, uint8_t *k_var,
-                                                                 int64_t n, float decay, float c_lo, float c_hi, int mode) {
+__device__ __forceinline__ void wrap_track_body(const uint32_t *__restrict__ amax, const uint32_t *__restrict__ anyneg, int n_parts,
+                                                float *i_var, const float *__restrict__ fb, uint8_t *k_var, int64_t n, float decay,
+                                                float c_lo, float c_hi, int mode, int64_t block) {
     __shared__ uint32_t smax[64 * WT_G], sneg[64 * WT_G];
     const Mode m(mode);
     const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const int64_t t = (int64_t)blockIdx.x * 64 + e_local;
+    const int64_t t = block * 64 + e_local;
     uint32_t mx = 0, ng = 0;
     if (t < n) {
         const int per = (n_parts + WT_G - 1) / WT_G;
@@ -670,6 +669,28 @@ __global__ __launch_bounds__(64 * WT_G) void wrap_track_i_kernel(const uint32_t 
         if (k_var && anyneg && ng) k_var[t] = 1;
     }
     i_var[t] = ni;
+}
+
+__global__ __launch_bounds__(64 * WT_G) void wrap_track_i_kernel(const uint32_t *__restrict__ amax,
+                                                                 const uint32_t *__restrict__ anyneg, int n_parts,
+                                                                 float *i_var, const float *__restrict__ fb, uint8_t *k_var,
+                                                                 int64_t n, float decay, float c_lo, float c_hi, int mode) {
+    wrap_track_body(amax, anyneg, n_parts, i_var, fb, k_var, n, decay, c_lo, c_hi, mode, blockIdx.x);
+}
+
+// The same update for several quantizers in one launch: block b serves the item whose block range holds b.
+struct TrackBatch {
+    hgq_track_item item[HGQ_TRACK_BATCH];
+    int first_block[HGQ_TRACK_BATCH + 1];
+    int count;
+};
+
+__global__ __launch_bounds__(64 * WT_G) void wrap_track_i_multi_kernel(const TrackBatch b) {
+    int t = 0;
+    while (t + 1 < b.count && (int)blockIdx.x >= b.first_block[t + 1]) ++t;
+    const hgq_track_item &it = b.item[t];
+    wrap_track_body(it.amax, it.anyneg, it.n_parts, it.i_var, it.fb, it.k_var, it.m, it.decay, it.c_lo, it.c_hi, it.mode,
+                    (int)blockIdx.x - b.first_block[t]);
 }
 
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
@@ -1097,4 +1118,30 @@ extern "C" int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, in
     hipLaunchKernelGGL(wrap_track_i_kernel, dim3((unsigned)((m + 63) / 64)), dim3(64 * WT_G), 0, (hipStream_t)stream, amax, anyneg, n_parts,
                        i_var, fb, k_var, m, decay, c_lo, c_hi, mode);
     return check_launch("hgq_wrap_track_i");
+}
+
+extern "C" int hgq_wrap_track_i_multi(const hgq_track_item *items, int count, void *stream) {
+    if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i_multi: bad arguments");
+    for (int base = 0; base < count; base += HGQ_TRACK_BATCH) {
+        TrackBatch b;
+        b.count = 0;
+        int64_t blocks = 0;
+        const int nb = count - base < HGQ_TRACK_BATCH ? count - base : HGQ_TRACK_BATCH;
+        for (int t = 0; t < nb; ++t) {
+            const hgq_track_item &it = items[base + t];
+            if (it.m < 0 || it.n_parts < 1) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i_multi: bad size in item %d", base + t);
+            if (it.m == 0) continue;
+            if (!it.amax || !it.i_var || !it.fb) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i_multi: null pointer in item %d", base + t);
+            b.item[b.count] = it;
+            b.first_block[b.count++] = (int)blocks;
+            blocks += (it.m + 63) / 64;
+            if (blocks > (1 << 24)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_wrap_track_i_multi: too many entries");
+        }
+        if (b.count == 0) continue;
+        for (int t = b.count; t <= HGQ_TRACK_BATCH; ++t) b.first_block[t] = (int)blocks;
+        hipLaunchKernelGGL(wrap_track_i_multi_kernel, dim3((unsigned)blocks), dim3(64 * WT_G), 0, (hipStream_t)stream, b);
+        int rc = check_launch("hgq_wrap_track_i_multi");
+        if (rc) return rc;
+    }
+    return HGQ_OK;
 }

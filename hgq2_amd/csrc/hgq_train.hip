@@ -571,6 +571,8 @@ extern "C" int hgq_dense_ebops_multi(const hgq_dense_ebops_item *items, int coun
     if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: bad arguments");
     for (int base = 0; base < count; base += HGQ_EBOPS_BATCH) {
         DenseEbopsBatch b;
+        hgq_track_item tracks[HGQ_EBOPS_BATCH];
+        int n_tracks = 0;
         const int nb = count - base < HGQ_EBOPS_BATCH ? count - base : HGQ_EBOPS_BATCH;
         for (int t = 0; t < nb; ++t) {
             const hgq_dense_ebops_item &it = items[base + t];
@@ -584,12 +586,18 @@ extern "C" int hgq_dense_ebops_multi(const hgq_dense_ebops_item *items, int coun
                 return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: fused tracking is for KIF WRAP input quantizers");
             b.item[t] = it;
             if (it.amax_part && it.P * it.K * it.n_parts > 16384) {
-                // many tracker slices: combine them with one thread group per entry across the device first
-                int rc = hgq_wrap_track_i(it.amax_part, nullptr, it.n_parts, it.i_in, it.f_in, nullptr, it.P * it.K, it.decay, 0.0f, 0.0f,
-                                          it.mode_in & ~(HGQ_MODE_TRACING | HGQ_MODE_SYMMETRIC), stream);
-                if (rc) return rc;
+                // many tracker slices: combine them with one thread group per entry across the device first (all such
+                // layers in one launch)
+                hgq_track_item &tr = tracks[n_tracks++];
+                tr.amax = it.amax_part, tr.anyneg = nullptr, tr.n_parts = it.n_parts, tr.i_var = it.i_in, tr.fb = it.f_in, tr.k_var = nullptr;
+                tr.m = it.P * it.K, tr.decay = it.decay, tr.c_lo = 0.0f, tr.c_hi = 0.0f;
+                tr.mode = it.mode_in & ~(HGQ_MODE_TRACING | HGQ_MODE_SYMMETRIC);
                 b.item[t].amax_part = nullptr;
             }
+        }
+        if (n_tracks) {
+            int rc = hgq_wrap_track_i_multi(tracks, n_tracks, stream);
+            if (rc) return rc;
         }
         hipLaunchKernelGGL(dense_ebops_multi_kernel, dim3((unsigned)nb), dim3(HGQ_EBOPS_NT), 0, (hipStream_t)stream, b);
         int rc = check_launch("hgq_dense_ebops_multi");

@@ -132,6 +132,30 @@ def wrap_track_i_op(amax: Tensor, anyneg: Tensor, n_parts: int, i_var: Tensor, f
     _lib.check(rc, 'hgq_wrap_track_i')
 
 
+class _TrackItem(ctypes.Structure):
+    _fields_ = [('amax', ctypes.c_void_p), ('anyneg', ctypes.c_void_p), ('n_parts', ctypes.c_int32), ('i_var', ctypes.c_void_p),
+                ('fb', ctypes.c_void_p), ('k_var', ctypes.c_void_p), ('m', ctypes.c_int64), ('decay', ctypes.c_float),
+                ('c_lo', ctypes.c_float), ('c_hi', ctypes.c_float), ('mode', ctypes.c_int32)]
+
+
+@torch.library.custom_op('hgq::wrap_track_i_multi', mutates_args=('i_vars',))
+def wrap_track_i_multi_op(amaxs: Sequence[Tensor], i_vars: Sequence[Tensor], fbs: Sequence[Tensor], decays: Sequence[float],
+                          modes: Sequence[int]) -> None:
+    """The training-mode integer-bit update of several quantizers (no sign tracker, no constraint) in one launch."""
+    n = len(i_vars)
+    items = (_TrackItem * n)()
+    for t in range(n):
+        _check_f32('i_var', i_vars[t]), _check_f32('fb', fbs[t])
+        m = i_vars[t].numel()
+        _need(m > 0 and amaxs[t].numel() % m == 0 and amaxs[t].numel() >= m and amaxs[t].dtype == torch.int32 and amaxs[t].is_cuda,
+              'amax must be an int32 GPU tensor of whole slices matching i_var')
+        _need(fbs[t].numel() == m, 'fb must match i_var')
+        items[t] = _TrackItem(amaxs[t].data_ptr(), None, amaxs[t].numel() // m, i_vars[t].data_ptr(), fbs[t].data_ptr(), None, m,
+                              decays[t], 0.0, 0.0, modes[t])
+    rc = _lib.load().hgq_wrap_track_i_multi(items, n, _stream())
+    _lib.check(rc, 'hgq_wrap_track_i_multi')
+
+
 @torch.library.custom_op('hgq::qdense_fwd', mutates_args=())
 def qdense_fwd(x: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, qw: Tensor, qb: Tensor, act: int, mode: int,
                bw_rows: int, track: bool) -> tuple[Tensor, Tensor]:
@@ -347,7 +371,7 @@ def touch_state():
 # The EBOPs estimate of a dense layer (and the integer-bit update fused into it) reads bit-width variables and the
 # abs-max slices its own forward left; nothing later in the forward pass reads what it writes.  While a model call is
 # open the calls are queued - outputs allocated, nothing launched - and go out as one launch when the call returns.
-_DEFER = {'depth': 0, 'dense_ebops': []}
+_DEFER = {'depth': 0, 'dense_ebops': [], 'tracks': []}
 
 
 def begin_deferred():
@@ -358,12 +382,25 @@ def end_deferred(discard: bool = False):
     _DEFER['depth'] -= 1
     if _DEFER['depth'] == 0:
         if discard:
-            _DEFER['dense_ebops'] = []
+            _DEFER['dense_ebops'], _DEFER['tracks'] = [], []
         else:
             flush_deferred()
 
 
+def flush_tracks():
+    """Run the queued integer-bit updates (one launch).  Everything that reads integer bits of a WRAP quantizer inside a
+    model call - the EBOPs launches, the bit-width views - calls this first."""
+    q, _DEFER['tracks'] = _DEFER['tracks'], []
+    if not q:
+        return
+    touch_state()
+    amaxs, i_vars, fbs, decays, modes = (list(c) for c in zip(*q))
+    with torch.no_grad():
+        wrap_track_i_multi_op(amaxs, i_vars, fbs, [float(d) for d in decays], [int(m) for m in modes])
+
+
 def flush_deferred():
+    flush_tracks()
     q, _DEFER['dense_ebops'] = _DEFER['dense_ebops'], []
     if not q:
         return
@@ -1339,6 +1376,12 @@ def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('
     """In-place integer-bit tracking; ``amax`` is [m] or [n_parts, m]."""
     m = i_var.numel()
     n_parts = amax.numel() // m
+    if (_DEFER['depth'] > 0 and anyneg is None and k_var is None and not (mode & (_lib.MODE_KBI | _lib.MODE_TRACING))
+            and c_lo == float('-inf') and c_hi == float('inf')):
+        # a KIF quantizer's training-mode update (its own forward does not read the integer bits): joins the other
+        # quantizers' updates of this model call in one launch, ahead of the first reader
+        _DEFER['tracks'].append((amax, i_var, fb, decay, mode))
+        return
     touch_state()
     empty_i = amax.new_empty(0)
     empty_k = torch.empty(0, dtype=torch.uint8, device=amax.device)
@@ -1696,6 +1739,7 @@ def qbits(k: Tensor, i, fb: Tensor, kbi: bool, add_mode: int = 0) -> Tensor:
     """Bit-widths ``relu(round(i) + round(f))`` (KIF) or ``round(b)`` (KBI) of raw quantizer variables, plus ``k``
     (``add_mode`` 1) or ``k * (b > 0)`` (``add_mode`` 2), with straight-through rounding; shaped like ``fb``."""
     empty = fb.new_empty(0)
+    flush_tracks()
     return _QBits.apply(k if add_mode else empty, i if not kbi else empty, fb, bool(kbi), int(add_mode))
 
 
@@ -1725,6 +1769,7 @@ class _BitsEbops(torch.autograd.Function):
     @staticmethod
     def forward(ctx, kind, params, beta, ebops_var, layouts, owners, *qvars):
         ctx.owners = owners
+        flush_tracks()  # the bit-widths read here include integer bits whose update may still be queued
         lib = _lib.load()
         ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
         total = sum(2 * fb.numel() for fb, lay in zip(fbs, layouts) if lay is not None)

@@ -359,6 +359,7 @@ class FixedPointQuantizerKIF(FixedPointQuantizerBase):
 
     @property
     def i(self):
+        ops.flush_tracks()  # an integer-bit update of this model call may still be queued
         return round_conv(self._i)
 
     @property

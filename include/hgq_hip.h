@@ -197,6 +197,25 @@ int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, int n_parts, 
                      uint8_t *k_var, int64_t m, float decay, float c_lo, float c_hi, int mode, void *stream);
 
 /*
+ * The same update for several quantizers in one launch.  In a training step each WRAP quantizer of a model updates
+ * its integer bits right after its own forward (fixed_point_quantizer.py:406-413); the updates are independent of
+ * each other and nothing in the forward pass reads them before the EBOPs estimates do, so a caller may collect them.
+ * Items with the fields of hgq_wrap_track_i; up to HGQ_TRACK_BATCH per launch, more are split over launches.
+ */
+#define HGQ_TRACK_BATCH 16
+typedef struct {
+    const uint32_t *amax, *anyneg;
+    int32_t n_parts;
+    float *i_var;
+    const float *fb;
+    uint8_t *k_var;
+    int64_t m;
+    float decay, c_lo, c_hi;
+    int32_t mode;
+} hgq_track_item;
+int hgq_wrap_track_i_multi(const hgq_track_item *items, int count, void *stream);
+
+/*
  * QDense / QEinsumDense contraction, forward, with the input quantizer fused into the operand
  * load.  Replaces `ops.matmul(self.iq(inputs), self.qkernel) + self.qbias` and the activation
  * (src/hgq/layers/core/dense.py:60-68; einsum_dense.py:72-83 for equations that reshape to a
