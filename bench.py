@@ -360,7 +360,7 @@ def main():
     ap.add_argument('--softmax-only', action='store_true',
                     help='run only the one-pass table-softmax kernels at the attention configuration (for profiler runs)')
     ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused',
-                    help='fused: whole-step kernels (3 launches); layers: per-layer torch.library operators with autograd; '
+                    help='fused: whole-step kernels (2 launches); layers: per-layer torch.library operators with autograd; '
                          '-graph: the step is captured once in a HIP graph and replayed')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -442,7 +442,7 @@ def main():
     ms_per_step = el / args.steps * 1e3
     value = BATCH * args.steps / el
 
-    labels_of = {'fused': 'whole-step kernels of a QDense stack with sparse CE and SGD, 3 launches (a special-case trainer)',
+    labels_of = {'fused': 'whole-step kernels of a QDense stack with sparse CE and SGD, 2 launches (a special-case trainer)',
                  'fused-graph': 'the same whole-step kernels replayed from a HIP graph',
                  'layers-graph': 'the layer API: per-layer operators + autograd, the step replayed from a HIP graph',
                  'layers-eager': 'the layer API: per-layer operators + autograd, eager launches (host-bound)'}

@@ -1,4 +1,5 @@
-// One training step of a stack of QDense layers in four launches.
+// One training step of a stack of QDense layers in two launches (three when the quantized weight image has to be
+// rebuilt first).
 //
 // At the layer sizes HGQ targets (tens of units per layer) a training step built from per-layer
 // kernels is bound by launch latency, not by HBM or MFMA.  Here the whole data path - every
@@ -6,9 +7,10 @@
 // full backward pass - runs in ONE kernel: the quantized weights of all layers sit in LDS
 // (a few tens of KB), a workgroup takes a tile of 64 samples through forward and backward without
 // touching HBM in between, and writes its partial gradient sums to a private slice.  A second
-// kernel adds the slices in a fixed order; a third applies, per layer, the integer-bit tracking,
+// kernel adds the slices in a fixed order and applies, per variable entry, the integer-bit tracking,
 // EBOPs (value, variable and gradient), the weight / bias quantizer backward and the SGD update
-// with the MonoL1 gradient and the clip constraints folded in.
+// with the MonoL1 gradient and the clip constraints folded in; it also leaves the quantized weight
+// image of the updated variables for the next step.
 //
 // HBM traffic per step is the input batch, the labels and the partial slices.
 #include "hgq_device.h"
@@ -77,11 +79,61 @@ __global__ __launch_bounds__(256) void mlp_prep_kernel(MlpDev d, float *__restri
     img[e] = v;
 }
 
+#define MLP_AUX 192  // per layer, after the slices: colsum[64], i_in[64], round(f_in)[64] of the variables BEFORE this step's update
+
+// Snapshot the update pass needs of variables it overwrites: taken by the main kernel (which runs to completion before
+// the update pass starts), so that an update workgroup never reads a variable another one is writing.  Row (l, k) is
+// computed by one wavefront: colsum = sum_n bits_ker[k, n].
+struct MlpSnapRow {
+    int l, k;      // layer and row (l < 0: none)
+    float cs, i, f;
+};
+
+// Row `row` of the snapshot, first half: the loads (one kernel-row entry per lane) are issued and nothing waits for them.
+__device__ __forceinline__ MlpSnapRow mlp_snapshot_begin(const MlpDev &d, int row, int lane) {
+    MlpSnapRow r;
+    r.l = -1, r.k = 0, r.cs = 0.f, r.i = 0.f, r.f = 0.f;
+    int base = 0;
+    for (int l = 0; l < d.n_layers; ++l) {  // (the layer index stays a loop counter: indexing the kernel-argument
+        const hgq_mlp_layer &h = d.l[l].h;  //  structure with a computed value would move it to scratch memory)
+        const int k = row - base;
+        if (k >= 0 && k < h.K) {
+            const Mode mk(h.mode_ker);
+            r.l = l, r.k = k;
+            if (lane < h.N) {
+                r.cs = rintf(h.b_ker[k * h.N + lane]);
+                if (mk.overflow_mode == HGQ_SAT) r.cs += load_k(h.k_ker, k * h.N + lane, mk.k_u8);
+            }
+            r.i = h.i_in[k], r.f = h.f_in[k];
+        }
+        base += h.K;
+    }
+    return r;
+}
+
+// Second half: the row sum over the lanes (integers: exact in any order) and the three stores.
+__device__ __forceinline__ void mlp_snapshot_end(MlpSnapRow r, float *aux, int lane) {
+    if (r.l < 0) return;
+    float cs = r.cs;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) cs += __shfl_xor(cs, o, 64);
+    if (lane == 0) {
+        float *a = aux + r.l * MLP_AUX;
+        a[r.k] = cs, a[64 + r.k] = r.i, a[128 + r.k] = rintf(r.f);
+    }
+}
+
 __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ img, const float *__restrict__ x,
                                                           const int64_t *__restrict__ labels, int64_t rows,
-                                                          float *part) {
+                                                          float *part, float *aux, float *loss) {
     extern __shared__ float lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // snapshot for the update pass: workgroup w's last wavefront takes row w; its loads travel with the image fetch below
+    const bool snap_wave = __builtin_amdgcn_readfirstlane(wave) == MLP_NT / 64 - 1;
+    MlpSnapRow snap;
+    snap.l = -1;
+    if (snap_wave) snap = mlp_snapshot_begin(d, (int)blockIdx.x, lane);
+    if (blockIdx.x == 0 && tid == 0 && loss) loss[0] = 0.f;  // the update pass accumulates into it
     const int L = d.n_layers;
     float *raw = lds + d.off_raw, *rx = lds + d.off_rx;
     float *dfs = lds + d.off_red;                                 // [L][64] fractional-bit gradient sums
@@ -108,6 +160,13 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
     for (int id = tid; id < MLP_BM * d.ld_rx; id += MLP_NT) rx[id] = 0.f;  // padding columns stay zero for good
     for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += MLP_NT) dfs[id] = 0.f, amx[id] = 0u;
     __syncthreads();
+    if (snap_wave) {
+        mlp_snapshot_end(snap, aux, lane);
+        // fewer workgroups than rows (small batches): the remaining rows, one after the other
+        int total = 0;
+        for (int l = 0; l < L; ++l) total += d.l[l].h.K;
+        for (int row = (int)blockIdx.x + (int)gridDim.x; row < total; row += (int)gridDim.x) mlp_snapshot_end(mlp_snapshot_begin(d, row, lane), aux, lane);
+    }
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const bool first = tile == blockIdx.x;
@@ -293,173 +352,192 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
     }
 }
 
-#define MLP_AUX 192  // per layer, after the M reduced sums: colsum[64], bits_in[64], dbits_in[64]
-
-// Blocks [0, ceil(M/64)): out[e] = sum over slices of part[g][e] (the abs-max sections are skipped
-// here).  Blocks beyond that, one per layer: reduce the layer's abs-max section, track the input
-// quantizer's integer bits in place, and leave for the update pass - which must not read variables
-// another workgroup is updating - the per-feature bit counts of the input quantizer and the
-// per-row sums of the kernel bit counts, all from the pre-update variables.
-#define MLP_RG 16  // slice groups per entry: 64 entries x 16 groups = 1024 threads, few loads per thread
-__global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_kernel(MlpDev d, const float *__restrict__ part, int n_parts, float *out,
-                                                         float *loss) {
-    __shared__ float red[64 * MLP_RG];
-    const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const int n_main = (d.M + 63) / 64;
-    const int per = (n_parts + MLP_RG - 1) / MLP_RG;
-    const int g0 = grp * per, g1 = min(n_parts, g0 + per);
-    if ((int)blockIdx.x < n_main) {
-        const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
-        float s = 0.f;
-        if (e < d.M) {
-            int g = g0;
-            for (; g + 8 <= g1; g += 8) {
-                float v[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = part[(int64_t)(g + u) * d.M + e];
-                s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
-            }
-            for (; g < g1; ++g) s += part[(int64_t)g * d.M + e];
-        }
-        red[threadIdx.x] = s;
-        __syncthreads();
-        if (grp == 0 && e < d.M) {
-            float v = 0.f;  // groups in order
-#pragma unroll
-            for (int w = 0; w < MLP_RG; w += 4)
-                v += (red[e_local + 64 * w] + red[e_local + 64 * (w + 1)]) + (red[e_local + 64 * (w + 2)] + red[e_local + 64 * (w + 3)]);
-            out[e] = v;
-            if (e == d.p_loss && loss) loss[0] = v;
-        }
-        return;
-    }
-    const int l = blockIdx.x - n_main;
-    const MlpLayerDev &ly = d.l[l];
-    const hgq_mlp_layer &h = ly.h;
-    const int k = e_local, K = h.K, N = h.N;
-    const Mode mk(h.mode_ker), mi(h.mode_in);
-    uint32_t mx = 0;
-    float cs = 0.f;
-    if (k < K) {
-        const uint32_t *pa = (const uint32_t *)part + ly.p_amax + k;
-        int g = g0;
-        for (; g + 8 <= g1; g += 8) {
-            uint32_t v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = pa[(int64_t)(g + u) * d.M];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) mx = max(mx, v[u]);
-        }
-        for (; g < g1; ++g) mx = max(mx, pa[(int64_t)g * d.M]);
-        // this thread's share of row k of the kernel bit counts
-        const int nper = (N + MLP_RG - 1) / MLP_RG, n0 = grp * nper, n1 = min(N, n0 + nper);
-        for (int n = n0; n < n1; ++n) {
-            float bk = rintf(h.b_ker[k * N + n]);
-            if (mk.overflow_mode == HGQ_SAT) bk += load_k(h.k_ker, k * N + n, mk.k_u8);
-            cs += bk;
-        }
-    }
-    __shared__ uint32_t smx[64 * MLP_RG];
-    smx[threadIdx.x] = mx;
-    red[threadIdx.x] = cs;
-    __syncthreads();
-    if (grp == 0 && k < K) {
-        for (int w = 1; w < MLP_RG; ++w) mx = max(mx, smx[k + 64 * w]);
-        const float f = rintf(h.f_in[k]);
-        const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-f)));
-        const float ni = fmaxf(__fsub_rn(h.i_in[k], h.decay), mi_);
-        h.i_in[k] = ni;
-        const float sfi = __fadd_rn(rintf(ni), f);
-        float b = sfi > 0.f ? sfi : 0.f;
-        if (mi.overflow_mode == HGQ_SAT) b += load_k(h.k_in, k, mi.k_u8);
-        float *aux = out + d.M + l * MLP_AUX;
-        float csum = 0.f;  // integers: exact in any order
-        for (int w = 0; w < MLP_RG; ++w) csum += red[k + 64 * w];
-        aux[k] = csum;
-        aux[64 + k] = b;
-        aux[128 + k] = sfi > 0.f ? 1.f : 0.f;
-    }
-}
-
 __device__ __forceinline__ float sgd_clip(float w, float g, float lr, float l1, float lo, float hi) {
     return fminf(fmaxf(__fsub_rn(w, __fmul_rn(lr, __fadd_rn(g, l1))), lo), hi);
 }
 
-#define MLP_UPD_SPLIT 8
-
-// Grid (layers, MLP_UPD_SPLIT).  Each workgroup updates its share of the layer's kernel entries;
-// the first one of a layer also owns EBOPs, the bias and the input quantizer's fractional bits.
-// Everything a workgroup needs about variables it does not own comes from the reduce pass.
-__global__ __launch_bounds__(256) void mlp_update_kernel(MlpDev d, const float *__restrict__ g, float lr, float *loss, float *img) {
-    __shared__ float colsum[64];   // sum_n bits_ker[k, n]
-    __shared__ float bits_in[64];  // relu(round(i) + round(f)) with the tracked i
-    __shared__ float dbits_in[64];
-    const MlpLayerDev &ly = d.l[blockIdx.x];
+// Second and last launch of a step.  A workgroup is 64 entries x 16 slice groups; its role, from its block index:
+//   role 0 (ceil(K N / 64) per layer): 64 kernel entries - their gradient sums over the slices, quantizer backward,
+//           SGD + constraints, the next step's image entries;
+//   role 1 (one per layer): the bias entries likewise, and the layer's EBOPs (value, variable, loss term);
+//   role 2 (one per layer): the input quantizer's fractional bits, and the assignment of its tracked integer bits;
+//   last block: the cross-entropy loss slot.
+// Every workgroup of a layer also reduces the layer's abs-max section, so each knows the tracked integer bits (hence the
+// input bit counts the EBOPs gradients need) without waiting for another workgroup; pre-update values of variables it
+// does not own come from the main kernel's snapshot.
+#define MLP_RG 16
+__global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d, const float *__restrict__ part, int n_parts,
+                                                                        const float *__restrict__ aux, float lr, float *loss, float *img) {
+    __shared__ float red[64 * MLP_RG];
+    __shared__ uint32_t smx[64 * MLP_RG];
+    __shared__ float val[64], bits_in[64], dbits_in[64], new_i[64];
+    const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int per = (n_parts + MLP_RG - 1) / MLP_RG;
+    const int g0 = grp * per, g1 = min(n_parts, g0 + per);
+    // ---- role
+    int l = 0, role = 3, j = 0;
+    {
+        int b = blockIdx.x;
+        for (; l < d.n_layers; ++l) {
+            const int na = (d.l[l].h.K * d.l[l].h.N + 63) / 64;
+            if (b < na + 2) {
+                role = b < na ? 0 : (b == na ? 1 : 2);
+                j = b;
+                break;
+            }
+            b -= na + 2;
+        }
+    }
+    const bool loss_block = role == 3;
+    if (loss_block) l = 0;
+    const MlpLayerDev &ly = d.l[l];
     const hgq_mlp_layer &h = ly.h;
-    const int tid = threadIdx.x, K = h.K, N = h.N;
-    const bool owner = blockIdx.y == 0;
+    const int K = h.K, N = h.N;
+    // ---- this workgroup's 64 gradient sums
+    int n_mine, p0;
+    if (role == 0) p0 = ly.p_dw + 64 * j, n_mine = min(64, K * N - 64 * j);
+    else if (role == 1) p0 = ly.p_db, n_mine = h.bias ? N : 0;
+    else if (role == 2) p0 = ly.p_df, n_mine = K;
+    else p0 = d.p_loss, n_mine = 1;
+    // the variables of the entry this thread will update, requested before the slices (the updates are applied by the
+    // first wavefront only; the loads are in flight while all sixteen reduce)
+    const int t = e_local;
+    const bool mine = grp == 0 && t < n_mine && !loss_block;
+    float v_w = 0.f, v_k = 0.f, v_i = 0.f, v_b = 0.f;
     const Mode mk(h.mode_ker), mb(h.mode_bias);
-    if (tid < 64) {
-        const float *aux = g + d.M + blockIdx.x * MLP_AUX;
-        colsum[tid] = aux[tid], bits_in[tid] = aux[64 + tid], dbits_in[tid] = aux[128 + tid];
+    if (mine) {
+        if (role == 0) {
+            const int e = 64 * j + t;
+            v_w = h.w[e], v_k = load_k(h.k_ker, e, mk.k_u8), v_i = h.i_ker[e], v_b = h.b_ker[e];
+        } else if (role == 1) {
+            v_w = h.bias[t], v_k = load_k(h.k_bias, t, mb.k_u8), v_i = h.i_bias[t], v_b = h.b_bias[t];
+        } else {
+            v_w = h.f_in[t];
+        }
+    }
+    // both reductions of a thread (its entry's sums, its feature's abs-max) with all loads of a 16-slice run in flight
+    {
+        float s = 0.f;
+        uint32_t mx = 0;
+        const bool have_e = e_local < n_mine, have_a = !loss_block && e_local < K;
+        const float *pe = part + p0 + (have_e ? e_local : 0);
+        const uint32_t *pa = (const uint32_t *)part + ly.p_amax + (have_a ? e_local : 0);
+        for (int g = g0; g < g1; g += 16) {
+            float v[16];
+            uint32_t a[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int64_t row = (int64_t)min(g + u, g1 - 1) * d.M;
+                v[u] = pe[row], a[u] = pa[row];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (g + u >= g1) v[u] = 0.f, a[u] = 0u;
+            s += (((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]))) +
+                 (((v[8] + v[9]) + (v[10] + v[11])) + ((v[12] + v[13]) + (v[14] + v[15])));
+#pragma unroll
+            for (int u = 0; u < 16; ++u) mx = max(mx, a[u]);
+        }
+        red[threadIdx.x] = have_e ? s : 0.f;
+        smx[threadIdx.x] = have_a ? mx : 0u;
     }
     __syncthreads();
+    if (grp != 0) return;  // one wavefront applies the 64 updates
+    {
+        float v = 0.f;  // groups in order
+#pragma unroll
+        for (int w = 0; w < MLP_RG; w += 4)
+            v += (red[e_local + 64 * w] + red[e_local + 64 * (w + 1)]) + (red[e_local + 64 * (w + 2)] + red[e_local + 64 * (w + 3)]);
+        val[e_local] = v;
+        if (!loss_block && e_local < K) {
+            const float *a = aux + l * MLP_AUX;
+            uint32_t mx = smx[e_local];
+            for (int w = 1; w < MLP_RG; ++w) mx = max(mx, smx[e_local + 64 * w]);
+            const float f = a[128 + e_local];
+            const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-f)));
+            const float ni = fmaxf(__fsub_rn(a[64 + e_local], h.decay), mi_);
+            const float sfi = __fadd_rn(rintf(ni), f);
+            float b = sfi > 0.f ? sfi : 0.f;
+            const Mode mi(h.mode_in);
+            if (mi.overflow_mode == HGQ_SAT) b += load_k(h.k_in, e_local, mi.k_u8);
+            new_i[e_local] = ni, bits_in[e_local] = b, dbits_in[e_local] = sfi > 0.f ? 1.f : 0.f;
+        } else {
+            new_i[e_local] = 0.f, bits_in[e_local] = 0.f, dbits_in[e_local] = 0.f;
+        }
+    }
+    // (one wavefront from here on: its LDS writes above are ordered before its reads below)
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    if (loss_block) {
+        if (t == 0 && loss) atomicAdd(loss, val[0]);
+        return;
+    }
+    const float *colsum = aux + l * MLP_AUX;
     const float beta = h.beta ? h.beta[0] : 0.f;
     const float gs = h.ebops_scale * beta;  // d(ebops * beta) / d bits
     float reg = 0.f;  // MonoL1 regularisation loss of the trainable bit-width variables (pre-update values)
-    if (owner) {
-        float part = tid < K ? bits_in[tid] * colsum[tid] : 0.f;
+    if (role == 0) {
+        const int e = 64 * j + t;
+        if (t < n_mine) {
+            const int k = e / N;
+            const KIF p = resolve_kif(v_k, v_i, v_b, true, true);
+            float dw, di, db;
+            quantize_grad_dyn(v_w, val[t], p, mk.round_mode, mk.overflow_mode, dw, di, db);
+            di -= db;  // f = b - i
+            const float w_new = __fsub_rn(v_w, __fmul_rn(lr, dw));
+            h.w[e] = w_new;
+            reg += h.b_ker_l1 * v_b + (h.train_i_ker ? h.i_ker_l1 * v_i : 0.f);
+            const float b_new = sgd_clip(v_b, db + bits_in[k] * gs, lr, h.b_ker_l1, h.b_ker_lo, h.b_ker_hi);
+            h.b_ker[e] = b_new;
+            float i_new = v_i;
+            if (h.train_i_ker) h.i_ker[e] = i_new = sgd_clip(v_i, di, lr, h.i_ker_l1, h.i_ker_lo, h.i_ker_hi);
+            // the next step's image entry, from the updated variables (what mlp_prep_kernel would compute)
+            img[ly.off_w + k * ly.ldw + (e - k * N)] = quantize_dyn(w_new, resolve_kif(v_k, i_new, b_new, true, true), mk.round_mode,
+                                                                    mk.overflow_mode, true);
+        }
+    } else if (role == 1) {
+        float part_e = t < K ? bits_in[t] * colsum[t] : 0.f;
         float bsum = 0.f;
-        if (h.bias && tid < N) {
-            bsum = rintf(h.b_bias[tid]);
-            if (mb.overflow_mode == HGQ_SAT) bsum += load_k(h.k_bias, tid, mb.k_u8);
+        if (h.bias && t < N) {
+            bsum = rintf(v_b);
+            if (mb.overflow_mode == HGQ_SAT) bsum += v_k;
         }
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64), bsum += __shfl_xor(bsum, o, 64);
-        if (tid == 0) {  // K, N <= 64: wave 0 holds every non-zero term
-            float total = part;
+        for (int o = 32; o > 0; o >>= 1) part_e += __shfl_xor(part_e, o, 64), bsum += __shfl_xor(bsum, o, 64);
+        if (t == 0) {
+            float total = part_e;
             if (h.bias) total += bsum / (float)N * h.bias_size;
             const float e = total * h.ebops_scale;
             if (h.ebops) h.ebops[0] = (uint32_t)e;
             if (loss) atomicAdd(loss, e * beta);
         }
-        if (h.bias && tid < N) {
-            const KIF p = kbi_entry(h.k_bias, h.i_bias, h.b_bias, tid, h.mode_bias);
+        if (h.bias && t < N) {
+            const KIF p = resolve_kif(v_k, v_i, v_b, true, true);
             float dw, di, db;
-            quantize_grad_dyn(h.bias[tid], g[ly.p_db + tid], p, mb.round_mode, mb.overflow_mode, dw, di, db);
+            quantize_grad_dyn(v_w, val[t], p, mb.round_mode, mb.overflow_mode, dw, di, db);
             di -= db;
-            h.bias[tid] = __fsub_rn(h.bias[tid], __fmul_rn(lr, dw));
-            reg += h.b_bias_l1 * h.b_bias[tid] + (h.train_i_bias ? h.i_bias_l1 * h.i_bias[tid] : 0.f);
-            h.b_bias[tid] = sgd_clip(h.b_bias[tid], db + h.bias_size / (float)N * gs, lr, h.b_bias_l1, h.b_bias_lo, h.b_bias_hi);
-            if (h.train_i_bias) h.i_bias[tid] = sgd_clip(h.i_bias[tid], di, lr, h.i_bias_l1, h.i_bias_lo, h.i_bias_hi);
-            // the next step's image entry, from the updated variables (what mlp_prep_kernel would compute)
-            img[ly.off_qb + tid] = quantize_dyn(h.bias[tid], kbi_entry(h.k_bias, h.i_bias, h.b_bias, tid, h.mode_bias), mb.round_mode,
-                                                mb.overflow_mode, true);
+            const float w_new = __fsub_rn(v_w, __fmul_rn(lr, dw));
+            h.bias[t] = w_new;
+            reg += h.b_bias_l1 * v_b + (h.train_i_bias ? h.i_bias_l1 * v_i : 0.f);
+            const float b_new = sgd_clip(v_b, db + h.bias_size / (float)N * gs, lr, h.b_bias_l1, h.b_bias_lo, h.b_bias_hi);
+            h.b_bias[t] = b_new;
+            float i_new = v_i;
+            if (h.train_i_bias) h.i_bias[t] = i_new = sgd_clip(v_i, di, lr, h.i_bias_l1, h.i_bias_lo, h.i_bias_hi);
+            img[ly.off_qb + t] = quantize_dyn(w_new, resolve_kif(v_k, i_new, b_new, true, true), mb.round_mode, mb.overflow_mode, true);
         }
-        if (tid < K) {
-            reg += h.f_in_l1 * h.f_in[tid];
-            h.f_in[tid] = sgd_clip(h.f_in[tid], g[ly.p_df + tid] + dbits_in[tid] * colsum[tid] * gs, lr, h.f_in_l1, h.f_in_lo, h.f_in_hi);
-            img[ly.off_f + tid] = rintf(h.f_in[tid]);
+    } else {
+        if (t < K) {
+            h.i_in[t] = new_i[t];
+            reg += h.f_in_l1 * v_w;
+            const float f_new = sgd_clip(v_w, val[t] + dbits_in[t] * colsum[t] * gs, lr, h.f_in_l1, h.f_in_lo, h.f_in_hi);
+            h.f_in[t] = f_new;
+            img[ly.off_f + t] = rintf(f_new);
         }
-    }
-    // quantizer backward of this workgroup's kernel entries, SGD + constraints
-    for (int e = blockIdx.y * 256 + tid; e < K * N; e += MLP_UPD_SPLIT * 256) {
-        const int k = e / N;
-        const KIF p = kbi_entry(h.k_ker, h.i_ker, h.b_ker, e, h.mode_ker);
-        float dw, di, db;
-        quantize_grad_dyn(h.w[e], g[ly.p_dw + e], p, mk.round_mode, mk.overflow_mode, dw, di, db);
-        di -= db;  // f = b - i
-        h.w[e] = __fsub_rn(h.w[e], __fmul_rn(lr, dw));
-        reg += h.b_ker_l1 * h.b_ker[e] + (h.train_i_ker ? h.i_ker_l1 * h.i_ker[e] : 0.f);
-        h.b_ker[e] = sgd_clip(h.b_ker[e], db + bits_in[k] * gs, lr, h.b_ker_l1, h.b_ker_lo, h.b_ker_hi);
-        if (h.train_i_ker) h.i_ker[e] = sgd_clip(h.i_ker[e], di, lr, h.i_ker_l1, h.i_ker_lo, h.i_ker_hi);
-        img[ly.off_w + k * ly.ldw + (e - k * N)] = quantize_dyn(h.w[e], kbi_entry(h.k_ker, h.i_ker, h.b_ker, e, h.mode_ker), mk.round_mode,
-                                                                mk.overflow_mode, true);
     }
     if (loss) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) reg += __shfl_xor(reg, o, 64);
-        if ((tid & 63) == 0 && reg != 0.f) atomicAdd(loss, reg);
+        if (t == 0 && reg != 0.f) atomicAdd(loss, reg);
     }
 }
 
@@ -542,7 +620,7 @@ extern "C" int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_laye
         raised = true;
     }
     const int parts = mlp_parts(rows);
-    // workspace: [image | per-workgroup slices | reduced sums + per-layer aux]; the image comes first so
+    // workspace: [image | per-workgroup slices | per-layer snapshot of pre-update variables]; the image comes first so
     // that its place does not depend on the batch size
     float *img = workspace;
     float *slices = workspace + ((d.off_raw + 3) & ~3);
@@ -551,11 +629,11 @@ extern "C" int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_laye
         hipLaunchKernelGGL(mlp_prep_kernel, dim3((d.off_raw + 255) / 256), dim3(256), 0, s, d, img);
         if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
     }
-    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, slices);
+    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, slices, reduced, loss);
     if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
-    hipLaunchKernelGGL(mlp_reduce_kernel, dim3((d.M + 63) / 64 + n_layers), dim3(64 * MLP_RG), 0, s, d, slices, parts, reduced, loss);
-    if ((rc = check_launch("hgq_mlp_train_step(reduce)"))) return rc;
-    hipLaunchKernelGGL(mlp_update_kernel, dim3(n_layers, MLP_UPD_SPLIT), dim3(256), 0, s, d, reduced, lr, loss, img);
+    int blocks = 1;
+    for (int l = 0; l < n_layers; ++l) blocks += (layers[l].K * layers[l].N + 63) / 64 + 2;
+    hipLaunchKernelGGL(mlp_reduce_update_kernel, dim3(blocks), dim3(64 * MLP_RG), 0, s, d, slices, parts, reduced, lr, loss, img);
     return check_launch("hgq_mlp_train_step(update)");
 }
 

@@ -142,7 +142,7 @@ class GraphedTrainStep:
 
 class FusedQDenseStack:
     """One SGD training step of a stack of :class:`QDense` layers with mean sparse categorical
-    cross-entropy, executed by the whole-step kernels (three launches once the quantized weight image of
+    cross-entropy, executed by the whole-step kernels (two launches once the quantized weight image of
     the previous step can be reused, see ``hgq_mlp_train_step_cached``).
 
     It updates exactly the variables the layer-by-layer path updates (kernels, biases, every

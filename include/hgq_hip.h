@@ -387,7 +387,7 @@ int hgq_sum_scalars(const float *const *terms, int count, float *out, void *stre
 
 /*
  * One training step (forward, mean sparse categorical cross-entropy from logits, backward, SGD)
- * of a stack of QDense layers in three launches.  It performs, in the same order and with the
+ * of a stack of QDense layers in two launches (three when the quantized weight image is rebuilt).  It performs, in the same order and with the
  * same arithmetic, what the per-layer entry points above do when the reference's call stack
  * (src/hgq/layers/core/base.py:88-110 around src/hgq/layers/core/dense.py:60-80, then the
  * optimizer and the constraints) is followed layer by layer: input quantizer (KIF, WRAP,

@@ -195,8 +195,9 @@ def test_fused_step_reuses_its_weight_image_only_while_it_owns_the_variables(dev
                     m.layers[1]._kernel[3, 4] += 0.25
         fresh._versions = None  # always quantize again
         la, lb = cached.step(x, y), fresh.step(x, y)
-        # the reported loss adds its regularisation terms with atomics: equal up to the order of those adds
-        assert abs(float(la) - float(lb)) <= 1e-6 * abs(float(lb)), f'loss step {step}'
+        # the reported loss is the sum of some eighty terms (cross-entropy, EBOPs and regularisation terms of every update
+        # workgroup) added with atomics: equal up to the order of those fp32 adds
+        assert abs(float(la) - float(lb)) <= 5e-6 * abs(float(lb)), f'loss step {step}'
         for pa, pb in zip(models[0].parameters(), models[1].parameters()):
             assert torch.equal(pa, pb), f'step {step}'
 
@@ -486,7 +487,8 @@ def test_fused_stack_sees_updates_made_by_the_per_layer_optimizer(dev):
             opt.step()
         fused[1].invalidate()  # the second one quantizes again whatever it believes
         la, lb = fused[0].step(x, y), fused[1].step(x, y)
-        assert abs(float(la) - float(lb)) <= 1e-6 * abs(float(lb)), f'loss step {step}'
+        # (the reported loss is a sum of some eighty terms added with atomics: equal up to the order of those fp32 adds)
+        assert abs(float(la) - float(lb)) <= 5e-6 * abs(float(lb)), f'loss step {step}'
         for pa, pb in zip(models[0].parameters(), models[1].parameters()):
             assert torch.equal(pa, pb), f'step {step}'
 
