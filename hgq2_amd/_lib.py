@@ -50,7 +50,7 @@ SIGNATURES = {
     'hgq_dense_ebops': (
         c_int,
         [c_void_p, c_int, c_float, c_void_p, c_void_p] + [c_void_p] * 3 + [c_int64, c_int, c_int] + [c_void_p] * 4
-        + [c_float, c_float, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p],
+        + [c_float, c_float, c_float, c_float, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p],
     ),
     'hgq_ebops_finish_fwd': (c_int, [c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_ebops_finish_bwd': (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_void_p]),
@@ -145,7 +145,7 @@ class MlpLayer(ctypes.Structure):
     _fields_ = (
         [(n, c_int) for n in ('K', 'N', 'act', 'mode_in', 'mode_ker', 'mode_bias')]
         + [(n, c_void_p) for n in ('w', 'bias', 'k_in', 'i_in', 'f_in', 'k_ker', 'b_ker', 'i_ker', 'k_bias', 'b_bias', 'i_bias')]
-        + [('decay', c_float), ('beta', c_void_p), ('ebops', c_void_p), ('ebops_scale', c_float), ('bias_size', c_float)]
+        + [('decay', c_float), ('beta', c_void_p), ('ebops', c_void_p), ('par_factor', c_float), ('n_parallel', c_float), ('ebops_factor', c_float), ('bias_size', c_float)]
         + [(n, c_float) for n in ('f_in_l1', 'f_in_lo', 'f_in_hi', 'b_ker_l1', 'b_ker_lo', 'b_ker_hi', 'i_ker_l1', 'i_ker_lo',
                                   'i_ker_hi', 'b_bias_l1', 'b_bias_lo', 'b_bias_hi', 'i_bias_l1', 'i_bias_lo', 'i_bias_hi')]
         + [('train_i_ker', c_int), ('train_i_bias', c_int)]

@@ -474,7 +474,8 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
     }
     const float *colsum = aux + l * MLP_AUX;
     const float beta = h.beta ? h.beta[0] : 0.f;
-    const float gs = h.ebops_scale * beta;  // d(ebops * beta) / d bits
+    // d(ebops * beta) / d bits: the chain rule through ((total * par_factor) / n_parallel) * ebops_factor * beta
+    const float gs = __fmul_rn(__fdiv_rn(__fmul_rn(beta, h.ebops_factor), h.n_parallel), h.par_factor);
     float reg = 0.f;  // MonoL1 regularisation loss of the trainable bit-width variables (pre-update values)
     if (role == 0) {
         const int e = 64 * j + t;
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
         if (t == 0) {
             float total = part_e;
             if (h.bias) total += bsum / (float)N * h.bias_size;
-            const float e = total * h.ebops_scale;
+            const float e = __fmul_rn(__fdiv_rn(__fmul_rn(total, h.par_factor), h.n_parallel), h.ebops_factor);
             if (h.ebops) h.ebops[0] = (uint32_t)e;
             if (loss) atomicAdd(loss, e * beta);
         }

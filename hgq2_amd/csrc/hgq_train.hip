@@ -57,7 +57,7 @@ __device__ __forceinline__ void dense_ebops_body(const uint32_t *amax_part, int 
                                                  const void *k_in, float *i_in, const float *f_in,
                                                  int64_t P, int K, int N, const void *k_ker,
                                                  const float *b_ker, const void *k_bias, const float *b_bias,
-                                                 float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
+                                                 float par_factor, float n_parallel, float ebops_factor, float bias_size, int mode_in, int mode_ker, int mode_bias,
                                                  float *ebops, uint32_t *ebops_u32, float *g_f_in,
                                                  float *g_b_ker, float *g_b_bias) {
     constexpr int NT = HGQ_EBOPS_NT;
@@ -68,7 +68,8 @@ __device__ __forceinline__ void dense_ebops_body(const uint32_t *amax_part, int 
     const Mode mi(mode_in), mk(mode_ker), mb(mode_bias);
     const int t = threadIdx.x;
     // with beta the gradients are those of the loss term ebops * beta
-    const float gscale = beta ? scale * beta[0] : scale;
+    // the chain rule walks ((total * par_factor) / n_parallel) * ebops_factor (* beta) back one operation at a time
+    const float gscale = __fmul_rn(__fdiv_rn(__fmul_rn(beta ? beta[0] : 1.0f, ebops_factor), n_parallel), par_factor);
     const int64_t PK = P * K;
     for (int k = t; k < K; k += NT) colsum[k] = 0, insum[k] = 0;
     if (amax_part) {
@@ -168,7 +169,7 @@ __device__ __forceinline__ void dense_ebops_body(const uint32_t *amax_part, int 
         total += bs / (float)N * bias_size;
     }
     if (t == 0) {
-        const float e = total * scale;
+        const float e = __fmul_rn(__fdiv_rn(__fmul_rn(total, par_factor), n_parallel), ebops_factor);
         ebops[0] = e;
         if (ebops_u32) ebops_u32[0] = (uint32_t)e;
         if (loss_term && beta) loss_term[0] = e * beta[0];
@@ -180,11 +181,11 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_kernel(const uint32_
                                                           const void *k_in, float *i_in, const float *f_in,
                                                           int64_t P, int K, int N, const void *k_ker,
                                                           const float *b_ker, const void *k_bias, const float *b_bias,
-                                                          float scale, float bias_size, int mode_in, int mode_ker, int mode_bias,
+                                                          float par_factor, float n_parallel, float ebops_factor, float bias_size, int mode_in, int mode_ker, int mode_bias,
                                                           float *ebops, uint32_t *ebops_u32, float *g_f_in,
                                                           float *g_b_ker, float *g_b_bias) {
-    dense_ebops_body(amax_part, n_parts, decay, beta, loss_term, k_in, i_in, f_in, P, K, N, k_ker, b_ker, k_bias, b_bias, scale, bias_size,
-                     mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
+    dense_ebops_body(amax_part, n_parts, decay, beta, loss_term, k_in, i_in, f_in, P, K, N, k_ker, b_ker, k_bias, b_bias, par_factor, n_parallel, ebops_factor,
+                     bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
 }
 
 // the layers of a model, one workgroup each: the estimates depend on the bit-width variables only, so they can all be
@@ -195,7 +196,7 @@ struct DenseEbopsBatch {
 __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_multi_kernel(DenseEbopsBatch b) {
     const hgq_dense_ebops_item &it = b.item[blockIdx.x];
     dense_ebops_body(it.amax_part, it.n_parts, it.decay, it.beta, it.loss_term, it.k_in, it.i_in, it.f_in, it.P, it.K, it.N, it.k_ker,
-                     it.b_ker, it.k_bias, it.b_bias, it.scale, it.bias_size, it.mode_in, it.mode_ker, it.mode_bias, it.ebops, it.ebops_u32,
+                     it.b_ker, it.k_bias, it.b_bias, it.par_factor, it.n_parallel, it.ebops_factor, it.bias_size, it.mode_in, it.mode_ker, it.mode_bias, it.ebops, it.ebops_u32,
                      it.g_f_in, it.g_b_ker, it.g_b_bias);
 }
 
@@ -546,7 +547,7 @@ extern "C" int hgq_sum_scalars(const float *const *terms, int count, float *out,
 extern "C" int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const float *beta, float *loss_term,
                                const void *k_in, float *i_in, const float *f_in, int64_t P, int K, int N,
                                const void *k_ker, const float *b_ker, const void *k_bias, const float *b_bias,
-                               float scale, float bias_size, int mode_in, int mode_ker, int mode_bias, float *ebops,
+                               float par_factor, float n_parallel, float ebops_factor, float bias_size, int mode_in, int mode_ker, int mode_bias, float *ebops,
                                uint32_t *ebops_u32, float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream) {
     if (P < 1 || K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_dense_ebops: bad sizes");
     if (!i_in || !f_in || !b_ker || !ebops || !k_in || !k_ker) return fail(HGQ_ERR_ARG, "hgq_dense_ebops: null pointer");
@@ -563,7 +564,8 @@ extern "C" int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float dec
     }
     hipLaunchKernelGGL(dense_ebops_kernel, dim3(1), dim3(HGQ_EBOPS_NT), 0, (hipStream_t)stream, amax_part, n_parts, decay, beta, loss_term, k_in,
                        i_in, f_in, P, K, N, k_ker, b_ker,
-                       k_bias, b_bias, scale, bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker, g_b_bias);
+                       k_bias, b_bias, par_factor, n_parallel, ebops_factor, bias_size, mode_in, mode_ker, mode_bias, ebops, ebops_u32, g_f_in, g_b_ker,
+                       g_b_bias);
     return check_launch("hgq_dense_ebops");
 }
 

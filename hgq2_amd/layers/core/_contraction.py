@@ -98,7 +98,7 @@ def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training):
     return y, act_code != _lib.ACT_NONE, None
 
 
-def dense_ebops_term(layer, iq, kq, bq, K, N, scale, bias_size, deferred):
+def dense_ebops_term(layer, iq, kq, bq, K, N, bias_size, deferred):
     """``ebops * beta`` through the fused kernel (which also assigns the layer's ``_ebops`` and, when
     ``deferred`` tracking is pending and small enough, updates the input quantizer's ``_i`` first).
     Returns ``None`` when the quantizers are not the fixed-point kinds the kernel covers."""
@@ -123,7 +123,7 @@ def dense_ebops_term(layer, iq, kq, bq, K, N, scale, bias_size, deferred):
     _, term = ops.dense_ebops(
         qi._k.view(-1), qi._i.view(-1), qi._third().view(-1), qk._k.view(-1), qk._b.view(-1),
         qb._k.view(-1) if qb is not None else None, qb._b.view(-1) if qb is not None else None, P, K, N,
-        scale * layer.ebops_factor, bias_size, qi._mode(True), qk._mode(True), qb._mode(True) if qb is not None else 0,
+        layer.parallelization_factor, layer.n_parallel, layer.ebops_factor, bias_size, qi._mode(True), qk._mode(True), qb._mode(True) if qb is not None else 0,
         amax=amax, decay=decay, beta=layer._beta, ebops_var=layer._ebops.view(torch.int32),
         owners=(qi._i, qi._third(), qk._b, qb._b if qb is not None else None))
     return term

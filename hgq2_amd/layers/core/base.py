@@ -18,6 +18,17 @@ from ...core import Constant, Initializer, Layer
 from ...quantizer import Quantizer, QuantizerConfig
 
 
+def scale_ebops(ebops: torch.Tensor, parallelization_factor, n_parallel) -> torch.Tensor:
+    """``ebops * parallelization_factor / n_parallel`` as the reference evaluates it (src/hgq/layers/core/dense.py:80,
+    pooling.py:30): a product, then a correctly rounded fp32 division.  On the GPU torch divides by a Python number with a
+    reciprocal multiply, which can land one ulp low - and the uint32 cast of the estimate one count low - so the divisor
+    goes in as a tensor."""
+    ebops = ebops * float(parallelization_factor)
+    if float(n_parallel) == 1.0:
+        return ebops
+    return ebops / torch.full((), float(n_parallel), dtype=ebops.dtype, device=ebops.device)
+
+
 class QLayerBase(Layer):
     """Handles the input / output quantizers, the ``beta`` and ``ebops`` variables and the
     EBOPs loss term.  Subclasses implement ``call`` and ``_compute_ebops(*input_shapes)``."""

@@ -10,7 +10,7 @@ from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
 from ._contraction import dense_contraction, dense_ebops_term, get_activation
-from .base import QLayerBaseSingleInput
+from .base import QLayerBaseSingleInput, scale_ebops
 
 
 class QDense(QLayerBaseSingleInput):
@@ -83,8 +83,7 @@ class QDense(QLayerBaseSingleInput):
 
     def _ebops_loss_term(self, shape):
         out_size = float(prod(shape[:-1]) * self.units)
-        scale = self.parallelization_factor / self.n_parallel
-        term = dense_ebops_term(self, self.iq, self.kq, self.bq, shape[-1], self.units, scale, out_size,
+        term = dense_ebops_term(self, self.iq, self.kq, self.bq, shape[-1], self.units, out_size,
                                 getattr(self, '_deferred', None))
         if term is not None:
             return term
@@ -93,14 +92,13 @@ class QDense(QLayerBaseSingleInput):
 
     def _compute_ebops(self, shape):
         out_size = float(prod(shape[:-1]) * self.units)
-        scale = self.parallelization_factor / self.n_parallel
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self._kernel.shape).to(bw_inp.device)
         ebops = torch.sum(torch.matmul(bw_inp, bw_ker))
         if self.bq is not None:
             bw_bias = self.bq.bits_(self.bias.shape)
             ebops = ebops + torch.mean(bw_bias) * out_size
-        return ebops * scale
+        return scale_ebops(ebops, self.parallelization_factor, self.n_parallel)
 
     def get_config(self):
         config = super().get_config()

@@ -17,7 +17,7 @@ from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
 from ._contraction import dense_contraction, dense_ebops_term, get_activation
-from .base import QLayerBaseSingleInput
+from .base import QLayerBaseSingleInput, scale_ebops
 
 
 def _einsum_free0_size(equation: str, input_shape) -> int:
@@ -184,10 +184,9 @@ class QEinsumDense(QLayerBaseSingleInput):
             d.flush()
 
     def _ebops_loss_term(self, shape):
-        scale = self.parallelization_factor / self.n_parallel
         out_size = float(prod(self.full_output_shape[1:]))
         if self._gemm is not None and (self.bq is None or self._bias_in_gemm):
-            term = dense_ebops_term(self, self.iq, self.kq, self.bq, self._K, self._N, scale, out_size,
+            term = dense_ebops_term(self, self.iq, self.kq, self.bq, self._K, self._N, out_size,
                                     getattr(self, '_deferred', None))
             if term is not None:
                 return term
@@ -195,7 +194,6 @@ class QEinsumDense(QLayerBaseSingleInput):
         return super()._ebops_loss_term(shape)
 
     def _compute_ebops(self, shape):
-        scale = self.parallelization_factor / self.n_parallel
         out_size = float(prod(self.full_output_shape[1:]))
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self._kernel.shape)
@@ -203,7 +201,7 @@ class QEinsumDense(QLayerBaseSingleInput):
         if self.bq is not None:
             bw_bias = self.bq.bits_(self.bias.shape)
             ebops = ebops + torch.mean(bw_bias) * out_size
-        return ebops * scale
+        return scale_ebops(ebops, self.parallelization_factor, self.n_parallel)
 
     def get_config(self):
         config = super().get_config()

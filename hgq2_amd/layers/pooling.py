@@ -11,7 +11,7 @@ import torch
 
 from .. import ops
 from ..quantizer import QuantizerConfig
-from .core.base import QLayerBaseSingleInput
+from .core.base import QLayerBaseSingleInput, scale_ebops
 
 
 def _pair(v):
@@ -27,7 +27,7 @@ class QBasePooling(QLayerBaseSingleInput):
 
     def _compute_ebops(self, shape):
         bw_inp = self.iq.bits_(shape)
-        return torch.sum(bw_inp) * self.parallelization_factor / self.n_parallel
+        return scale_ebops(torch.sum(bw_inp), self.parallelization_factor, self.n_parallel)
 
     def pool(self, inputs):
         raise NotImplementedError

@@ -303,8 +303,8 @@ def _dense_ebops_check(amax, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bia
 
 
 def _dense_ebops_impl(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_in: Tensor, f_in: Tensor, k_ker: Tensor,
-                   b_ker: Tensor, k_bias: Tensor, b_bias: Tensor, ebops_var: Tensor, P: int, K: int, N: int, scale: float,
-                   bias_size: float, mode_in: int, mode_ker: int, mode_bias: int) -> tuple[Tensor, Tensor, Tensor]:
+                   b_ker: Tensor, k_bias: Tensor, b_bias: Tensor, ebops_var: Tensor, P: int, K: int, N: int, par_factor: float,
+                   n_parallel: float, ebops_factor: float, bias_size: float, mode_in: int, mode_ker: int, mode_bias: int) -> tuple[Tensor, Tensor, Tensor]:
     """Returns (ebops, ebops*beta, [g_f_in | g_b_ker | g_b_bias] in one buffer); with ``beta`` the
     gradient buffer holds d(ebops*beta)/d variable, else d ebops / d variable."""
     n_parts, has_bias, m_in, m_ker, m_bias = _dense_ebops_check(amax, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var,
@@ -316,7 +316,7 @@ def _dense_ebops_impl(amax: Tensor, decay: float, beta: Tensor, k_in: Tensor, i_
     g = torch.empty(P * K + K * N + nb, dtype=torch.float32, device=dev)
     g_f, g_bk, g_bb = g[:P * K], g[P * K:P * K + K * N], g[P * K + K * N:]
     rc = _lib.load().hgq_dense_ebops(_ptr(amax), n_parts, decay, _ptr(beta), _ptr(term), _ptr(k_in), _ptr(i_in), _ptr(f_in),
-                                     P, K, N, _ptr(k_ker), _ptr(b_ker), _ptr(k_bias), _ptr(b_bias), scale, bias_size,
+                                     P, K, N, _ptr(k_ker), _ptr(b_ker), _ptr(k_bias), _ptr(b_bias), par_factor, n_parallel, ebops_factor, bias_size,
                                      m_in, m_ker, m_bias, _ptr(ebops), _ptr(ebops_var),
                                      _ptr(g_f), _ptr(g_bk), _ptr(g_bb), _stream())
     _lib.check(rc, 'hgq_dense_ebops')
@@ -327,7 +327,8 @@ class _DenseEbopsItem(ctypes.Structure):
     _fields_ = [('amax_part', ctypes.c_void_p), ('n_parts', ctypes.c_int), ('decay', ctypes.c_float), ('beta', ctypes.c_void_p),
                 ('loss_term', ctypes.c_void_p), ('k_in', ctypes.c_void_p), ('i_in', ctypes.c_void_p), ('f_in', ctypes.c_void_p),
                 ('P', ctypes.c_int64), ('K', ctypes.c_int), ('N', ctypes.c_int), ('k_ker', ctypes.c_void_p), ('b_ker', ctypes.c_void_p),
-                ('k_bias', ctypes.c_void_p), ('b_bias', ctypes.c_void_p), ('scale', ctypes.c_float), ('bias_size', ctypes.c_float),
+                ('k_bias', ctypes.c_void_p), ('b_bias', ctypes.c_void_p), ('par_factor', ctypes.c_float), ('n_parallel', ctypes.c_float), ('ebops_factor', ctypes.c_float),
+                ('bias_size', ctypes.c_float),
                 ('mode_in', ctypes.c_int), ('mode_ker', ctypes.c_int), ('mode_bias', ctypes.c_int), ('ebops', ctypes.c_void_p),
                 ('ebops_u32', ctypes.c_void_p), ('g_f_in', ctypes.c_void_p), ('g_b_ker', ctypes.c_void_p), ('g_b_bias', ctypes.c_void_p)]
 
@@ -339,7 +340,8 @@ def dense_ebops_multi_op(amaxs: Sequence[Tensor], betas: Sequence[Tensor], k_ins
                          gs: Sequence[Tensor], decays: Sequence[float], dims: Sequence[int], scales: Sequence[float],
                          bias_sizes: Sequence[float], modes: Sequence[int]) -> None:
     """The dense-EBOPs launch of several layers at once; outputs are preallocated (``ebops_outs``, ``terms``, ``gs`` as
-    ``_dense_ebops_impl`` returns them).  ``dims`` = P, K, N per item, ``modes`` = mode_in, mode_ker, mode_bias per item."""
+    ``_dense_ebops_impl`` returns them).  ``dims`` = P, K, N per item, ``scales`` = par_factor, n_parallel, ebops_factor per item,
+    ``modes`` = mode_in, mode_ker, mode_bias per item."""
     n = len(f_ins)
     items = (_DenseEbopsItem * n)()
     for t in range(n):
@@ -352,7 +354,7 @@ def dense_ebops_multi_op(amaxs: Sequence[Tensor], betas: Sequence[Tensor], k_ins
         g_f, g_bk, g_bb = g[:P * K], g[P * K:P * K + K * N], g[P * K + K * N:]
         p = lambda x: x.data_ptr() if x.numel() else None  # noqa: E731
         items[t] = _DenseEbopsItem(p(amaxs[t]), n_parts, decays[t], p(betas[t]), p(terms[t]), p(k_ins[t]), p(i_ins[t]), p(f_ins[t]), P, K, N,
-                                   p(k_kers[t]), p(b_kers[t]), p(k_biases[t]), p(b_biases[t]), scales[t], bias_sizes[t], m_in, m_ker, m_bias,
+                                   p(k_kers[t]), p(b_kers[t]), p(k_biases[t]), p(b_biases[t]), scales[3 * t], scales[3 * t + 1], scales[3 * t + 2], bias_sizes[t], m_in, m_ker, m_bias,
                                    p(ebops_outs[t]), p(ebops_vars[t]), p(g_f), p(g_bk), p(g_bb))
     rc = _lib.load().hgq_dense_ebops_multi(items, n, _stream())
     _lib.check(rc, 'hgq_dense_ebops_multi')
@@ -417,11 +419,12 @@ def _flush_dense_ebops(amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_bias
                        scales, bias_sizes, modes):
     dense_ebops_multi_op(list(amaxs), list(betas), list(k_ins), list(i_ins), list(f_ins), list(k_kers), list(b_kers), list(k_biases),
                          list(b_biases), list(ebops_vars), list(outs), list(terms), list(gs), [float(d) for d in decays],
-                         [int(v) for d in dims for v in d], [float(v) for v in scales], [float(v) for v in bias_sizes],
+                         [int(v) for d in dims for v in d], [float(v) for s in scales for v in s], [float(v) for v in bias_sizes],
                          [int(v) for m in modes for v in m])
 
 
-def _dense_ebops_queue(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N, scale, bias_size,
+def _dense_ebops_queue(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N, par_factor, n_parallel,
+                       ebops_factor, bias_size,
                        mode_in, mode_ker, mode_bias):
     dev = f_in.device
     ebops = torch.empty((), dtype=torch.float32, device=dev)
@@ -429,7 +432,7 @@ def _dense_ebops_queue(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias
     g = torch.empty(P * K + K * N + (N if b_bias.numel() else 0), dtype=torch.float32, device=dev)
     # `.data`: the update of the integer bits is a state assignment, not an operation autograd should see
     _DEFER['dense_ebops'].append((amax, beta, k_in, i_in.data, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, ebops, term, g, decay, (P, K, N),
-                                  scale, bias_size, (mode_in, mode_ker, mode_bias)))
+                                  (par_factor, n_parallel, ebops_factor), bias_size, (mode_in, mode_ker, mode_bias)))
     return ebops, term, g
 
 
@@ -1435,14 +1438,14 @@ def qdense(x2d, k_in, i_in, f_in, qw, qb, act: int, mode: int, bw_rows: int, tra
 class _DenseEbops(torch.autograd.Function):
     @staticmethod
     def forward(ctx, i_in, f_in, b_ker, b_bias, amax, decay, beta, k_in, k_ker, k_bias, ebops_var, P, K, N, scale, bias_size,
-                mode_in, mode_ker, mode_bias, owners):
+                mode_in, mode_ker, mode_bias, owners):  # scale = (par_factor, n_parallel, ebops_factor)
         ctx.owners = owners
         if _DEFER['depth'] > 0:  # inside a model call: queued, launched with the other layers' when the call returns
             op = _dense_ebops_queue
         else:
             op = dense_ebops_track_op if amax.numel() else dense_ebops_op
         ebops, term, g = op(amax, decay, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N,
-                                        scale, bias_size, mode_in, mode_ker, mode_bias)
+                                        *scale, bias_size, mode_in, mode_ker, mode_bias)
         ctx.g = g  # kept as a plain attribute: a queued call fills it after this function has returned
         ctx.has_beta = beta.numel() > 0
         ctx.sizes = (P * K, K * N, b_bias.numel())
@@ -1482,9 +1485,10 @@ class _DenseEbops(torch.autograd.Function):
         return (gi, gf.view(s_f), grads[n_f:n_f + n_k].view(s_k), grads[n_f + n_k:].view(s_b) if n_b else None) + (None,) * 16
 
 
-def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, bias_size, mode_in, mode_ker, mode_bias,
-                amax=None, decay=0.0, beta=None, ebops_var=None, owners=None):
-    """EBOPs of a dense contraction.  Returns ``(ebops, ebops * beta)``: with ``beta`` the second
+def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, par_factor, n_parallel, ebops_factor, bias_size, mode_in,
+                mode_ker, mode_bias, amax=None, decay=0.0, beta=None, ebops_var=None, owners=None):
+    """EBOPs of a dense contraction, scaled as ``sum * par_factor / n_parallel * ebops_factor`` left to right in fp32
+    (reference src/hgq/layers/core/dense.py:80, base.py:102).  Returns ``(ebops, ebops * beta)``: with ``beta`` the second
     carries the gradient (and the first is a plain value), without it the first does.  With
     ``amax`` the input quantizer's integer bits are tracked in place first; with ``ebops_var`` the
     uint32 variable is assigned.  ``owners`` = the variables behind ``(i_in, f_in, b_ker, b_bias)``: with the gradient
@@ -1496,7 +1500,8 @@ def dense_ebops(k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, P, K, N, scale, 
     return _DenseEbops.apply(i_in, f_in, b_ker, b_bias if b_bias is not None else e_f, amax if amax is not None else e_i,
                              float(decay), beta if beta is not None else e_f, k_in, k_ker,
                              k_bias if k_bias is not None else e_k, ebops_var if ebops_var is not None else e_i, P, K, N,
-                             float(scale), float(bias_size), mode_in, mode_ker, mode_bias, owners)
+                             (float(par_factor), float(n_parallel), float(ebops_factor)), float(bias_size), mode_in, mode_ker,
+                             mode_bias, owners)
 
 
 class _QSoftmax(torch.autograd.Function):

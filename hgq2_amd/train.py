@@ -206,7 +206,8 @@ class FusedQDenseStack:
             it.decay = qi._decay_host
             if layer.enable_ebops:
                 it.beta, it.ebops = ptr(layer._beta), ptr(layer._ebops)
-            it.ebops_scale = layer.parallelization_factor / layer.n_parallel * layer.ebops_factor
+            it.par_factor, it.n_parallel = float(layer.parallelization_factor), float(layer.n_parallel)
+            it.ebops_factor = float(layer.ebops_factor)
             it.bias_size = float(layer.units)
             it.f_in_l1, it.f_in_lo, it.f_in_hi = var_params(qi._f)
             it.b_ker_l1, it.b_ker_lo, it.b_ker_hi = var_params(qk._b)

@@ -277,7 +277,12 @@ int hgq_reduce_slices_multi(const hgq_reduce_item *items, int count, void *strea
  * EBOPs of a dense contraction and its gradient.  Replaces QDense._compute_ebops
  * (src/hgq/layers/core/dense.py:70-80) / QEinsumDense._compute_ebops for GEMM-shaped equations
  * (einsum_dense.py:85-93) evaluated on bit-width tensors, i.e.
- *     ebops = (sum_p sum_k bits_in[p,k] * sum_n bits_ker[k,n] + mean(bits_bias) * bias_size) * scale
+ *     ebops = (sum_p sum_k bits_in[p,k] * sum_n bits_ker[k,n] + mean(bits_bias) * bias_size)
+ *             * par_factor / n_parallel * ebops_factor
+ * evaluated left to right in fp32 with a correctly rounded division, as the reference's
+ * `ebops * self.parallelization_factor / self.n_parallel` (dense.py:80) followed by `* self.ebops_factor`
+ * (base.py:102) is: a single precomputed factor can land one ulp away, and the cast to uint32 then one count away.
+ * The gradients are scaled in the order the chain rule walks those operations back.
  * with bits_in = relu(round(i_in)+round(f_in)) (+k for SAT), bits_ker / bits_bias = round(b) (+k for SAT).
  *
  *   ebops [1] fp32;  ebops_u32 [1] optional: the value cast to uint32 (the `_ebops` variable,
@@ -292,7 +297,8 @@ int hgq_reduce_slices_multi(const hgq_reduce_item *items, int count, void *strea
 int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const float *beta, float *loss_term,
                     const void *k_in, float *i_in, const float *f_in, int64_t P, int K, int N,
                     const void *k_ker, const float *b_ker, const void *k_bias, const float *b_bias,
-                    float scale, float bias_size, int mode_in, int mode_ker, int mode_bias, float *ebops,
+                    float par_factor, float n_parallel, float ebops_factor, float bias_size, int mode_in, int mode_ker,
+                    int mode_bias, float *ebops,
                     uint32_t *ebops_u32, float *g_f_in, float *g_b_ker, float *g_b_bias, void *stream);
 
 /*
@@ -317,7 +323,7 @@ typedef struct {
     const float *b_ker;
     const void *k_bias;
     const float *b_bias;
-    float scale, bias_size;
+    float par_factor, n_parallel, ebops_factor, bias_size;
     int mode_in, mode_ker, mode_bias;
     float *ebops;
     uint32_t *ebops_u32;
@@ -415,7 +421,7 @@ typedef struct {
     float decay;                      /* i_decay_speed of the input quantizer */
     const float *beta;                /* the layer's beta variable [1] */
     uint32_t *ebops;                  /* the layer's ebops variable [1] */
-    float ebops_scale;                /* parallelization_factor / n_parallel * ebops_factor */
+    float par_factor, n_parallel, ebops_factor; /* ebops = sum * par_factor / n_parallel * ebops_factor, left to right */
     float bias_size;                  /* number of bias additions: prod(shape[:-1]) * N for shape (1, ..., K) */
     /* MonoL1 coefficient and clip bounds of each trainable bit-width variable (-inf / +inf for none) */
     float f_in_l1, f_in_lo, f_in_hi;
