@@ -263,7 +263,12 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                     const int lab = (int)labels[gr];
                     lrow = logf(se) - (z[lab] - mx);
                     const float inv = 1.0f / se;
-                    for (int c = 0; c < C; ++c) dz[c] = (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows;
+                    // a relu on the output layer: its mask (z holds the values after the activation)
+                    const bool mask_out = d.l[L - 1].h.act == HGQ_ACT_RELU;
+                    for (int c = 0; c < C; ++c) {
+                        const float gz = (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows;
+                        dz[c] = (!mask_out || z[c] > 0.f) ? gz : 0.f;
+                    }
                     for (int c = C; c < Cp; ++c) dz[c] = 0.f;
                 } else {
                     for (int c = 0; c < Cp; ++c) dz[c] = 0.f;

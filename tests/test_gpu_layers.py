@@ -173,6 +173,59 @@ def test_fused_qdense_stack_step_matches_oracle(dev, acc64, batch, dims):
             _close(pl.bq.quantizer._i, rl.bq.quantizer._i, scale=rl.bq.quantizer._i.detach().abs() + 1e-3, what=f'bq._i {n}')
 
 
+def test_fused_stack_with_an_activation_on_the_output_layer(dev, acc64):
+    """QDense applies its activation whatever follows it (reference src/hgq/layers/core/dense.py:66-67): with relu on the
+    last layer the cross-entropy gradient passes the relu mask before it reaches that layer's kernel."""
+    import torch.nn.functional as F
+
+    from hgq2_amd.config import LayerConfigScope, QuantizerConfigScope
+    from hgq2_amd.core import Sequential
+    from hgq2_amd.layers import QDense
+    from hgq2_amd.train import FusedQDenseStack
+    from oracle import twin
+
+    g = torch.Generator().manual_seed(11)
+    torch.manual_seed(11)
+    x = torch.randn(500, 9, generator=g)
+    labels = torch.randint(0, 6, (500,), generator=g)
+    with QuantizerConfigScope(place='all', default_q_type='kbi', overflow_mode='SAT_SYM'), \
+            QuantizerConfigScope(place='datalane', default_q_type='kif', overflow_mode='WRAP'), \
+            LayerConfigScope(enable_ebops=True, beta0=1e-5):
+        layers = [QDense(20, activation='relu'), QDense(6, activation='relu')]
+    model = Sequential(layers)
+    xd, yd = x.to(dev), labels.to(dev)
+    model(xd, training=True)
+    refs = [twin.ref_dense(layer) for layer in layers]
+    fused = FusedQDenseStack(model, lr=0.05)
+    for step in range(3):
+        variables = [v for r in refs for v in r.trainable_variables()]
+        for v in variables:
+            v.grad = None
+        h = x
+        for r in refs:
+            h = r(h, training=True)
+        assert bool((h == 0).any()), 'the case needs clipped outputs'
+        want_loss = F.cross_entropy(h.float(), labels)
+        for r in refs:
+            want_loss = want_loss + r.extra_loss()
+        want_loss.backward()
+        with torch.no_grad():
+            for v in variables:
+                if v.grad is not None:
+                    v.sub_(0.05 * v.grad)
+        for r in refs:
+            r.apply_constraints()
+        loss = fused.step(xd, yd)
+        assert abs(loss.item() - want_loss.item()) <= 1e-5 * abs(want_loss.item()), f'loss step {step}'
+        for n, (rl, pl) in enumerate(zip(refs, layers)):
+            assert torch.equal(pl.iq.quantizer._i.cpu(), rl.iq.quantizer._i.detach()), f'layer {n} _i step {step}'
+            assert int(pl.ebops.cpu().view(torch.int32)) == int(rl.ebops_value), f'layer {n} ebops step {step}'
+            _close(pl._kernel, rl.kernel, scale=rl.kernel.detach().abs() + 1e-3, what=f'kernel {n} step {step}')
+            _close(pl.bias, rl.bias, scale=rl.bias.detach().abs() + 1e-3, what=f'bias {n} step {step}')
+            _close(pl.iq.quantizer._f, rl.iq.quantizer._f, scale=rl.iq.quantizer._f.detach().abs() + 1e-3, what=f'iq._f {n}')
+            _close(pl.kq.quantizer._b, rl.kq.quantizer._b, scale=rl.kq.quantizer._b.detach().abs() + 1e-3, what=f'kq._b {n}')
+
+
 def test_fused_step_reuses_its_weight_image_only_while_it_owns_the_variables(dev):
     """Steps that reuse the quantized weight image left by the previous update are bit-identical to
     steps that quantize the variables again, across a change of batch size, and an in-place change
