@@ -1132,6 +1132,10 @@ extern "C" int hgq_wrap_track_i_multi(const hgq_track_item *items, int count, vo
             if (it.m < 0 || it.n_parts < 1) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i_multi: bad size in item %d", base + t);
             if (it.m == 0) continue;
             if (!it.amax || !it.i_var || !it.fb) return fail(HGQ_ERR_ARG, "hgq_wrap_track_i_multi: null pointer in item %d", base + t);
+            // the items of one launch run concurrently: two updates of one variable would race
+            for (int u = 0; u < b.count; ++u)
+                if (b.item[u].i_var == it.i_var)
+                    return fail(HGQ_ERR_ARG, "hgq_wrap_track_i_multi: items %d and an earlier one update the same variable; pass them in separate calls", base + t);
             b.item[b.count] = it;
             b.first_block[b.count++] = (int)blocks;
             blocks += (it.m + 63) / 64;

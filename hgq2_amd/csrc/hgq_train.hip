@@ -586,6 +586,10 @@ extern "C" int hgq_dense_ebops_multi(const hgq_dense_ebops_item *items, int coun
                 return fail(HGQ_ERR_UNSUPPORTED, "hgq_dense_ebops_multi: kernel/bias bit-widths must use the KBI parametrisation");
             if (it.amax_part && (it.n_parts < 1 || Mode(it.mode_in).kbi || Mode(it.mode_in).overflow_mode != HGQ_WRAP))
                 return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: fused tracking is for KIF WRAP input quantizers");
+            // the items of one launch run concurrently: an update of integer bits another item reads or updates would race
+            for (int u = 0; u < t; ++u)
+                if (b.item[u].i_in == it.i_in && (it.amax_part || items[base + u].amax_part))
+                    return fail(HGQ_ERR_ARG, "hgq_dense_ebops_multi: items %d and %d share integer bits one of them updates; pass them in separate calls", base + u, base + t);
             b.item[t] = it;
             if (it.amax_part && it.P * it.K * it.n_parts > 16384) {
                 // many tracker slices: combine them with one thread group per entry across the device first (all such

@@ -389,16 +389,33 @@ def end_deferred(discard: bool = False):
             flush_deferred()
 
 
+def _rounds(keys):
+    """Split queue positions into launches: entries of one launch run concurrently, so entries with the same key (the
+    address of the integer-bit variable they update or read) go to successive launches, in queue order.  A quantizer
+    shared by several layers (the fused inputs of an attention layer, reference src/hgq/layers/attn/mha.py:205-210) is
+    updated once per call of each layer, one after the other."""
+    rounds, seen = [], {}
+    for n, key in enumerate(keys):
+        r = seen.get(key, 0)
+        seen[key] = r + 1
+        if r == len(rounds):
+            rounds.append([])
+        rounds[r].append(n)
+    return rounds
+
+
 def flush_tracks():
-    """Run the queued integer-bit updates (one launch).  Everything that reads integer bits of a WRAP quantizer inside a
-    model call - the EBOPs launches, the bit-width views - calls this first."""
+    """Run the queued integer-bit updates (one launch; one more for every repeated update of the same variable).  Everything
+    that reads integer bits of a WRAP quantizer inside a model call - the EBOPs launches, the bit-width views - calls
+    this first."""
     q, _DEFER['tracks'] = _DEFER['tracks'], []
     if not q:
         return
     touch_state()
-    amaxs, i_vars, fbs, decays, modes = (list(c) for c in zip(*q))
     with torch.no_grad():
-        wrap_track_i_multi_op(amaxs, i_vars, fbs, [float(d) for d in decays], [int(m) for m in modes])
+        for members in _rounds([item[1].data_ptr() for item in q]):
+            amaxs, i_vars, fbs, decays, modes = (list(c) for c in zip(*[q[n] for n in members]))
+            wrap_track_i_multi_op(amaxs, i_vars, fbs, [float(d) for d in decays], [int(m) for m in modes])
 
 
 def flush_deferred():
@@ -406,13 +423,11 @@ def flush_deferred():
     q, _DEFER['dense_ebops'] = _DEFER['dense_ebops'], []
     if not q:
         return
-    cols = list(zip(*q))
-    (amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims, scales,
-     bias_sizes, modes) = cols
     touch_state()  # the fused integer-bit update writes `_i`
     with torch.no_grad():
-        _flush_dense_ebops(amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims,
-                           scales, bias_sizes, modes)
+        # layers that share an input quantizer update and read its integer bits one after the other
+        for members in _rounds([item[3].data_ptr() for item in q]):
+            _flush_dense_ebops(*zip(*[q[n] for n in members]))
 
 
 def _flush_dense_ebops(amaxs, betas, k_ins, i_ins, f_ins, k_kers, b_kers, k_biases, b_biases, ebops_vars, outs, terms, gs, decays, dims,
@@ -1379,6 +1394,8 @@ def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('
     """In-place integer-bit tracking; ``amax`` is [m] or [n_parts, m]."""
     m = i_var.numel()
     n_parts = amax.numel() // m
+    if _DEFER['dense_ebops'] and any(item[3].data_ptr() == i_var.data_ptr() for item in _DEFER['dense_ebops']):
+        flush_deferred()  # a queued EBOPs estimate reads these integer bits as they stand now
     if (_DEFER['depth'] > 0 and anyneg is None and k_var is None and not (mode & (_lib.MODE_KBI | _lib.MODE_TRACING))
             and c_lo == float('-inf') and c_hi == float('inf')):
         # a KIF quantizer's training-mode update (its own forward does not read the integer bits): joins the other

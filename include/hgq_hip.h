@@ -201,6 +201,8 @@ int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, int n_parts, 
  * its integer bits right after its own forward (fixed_point_quantizer.py:406-413); the updates are independent of
  * each other and nothing in the forward pass reads them before the EBOPs estimates do, so a caller may collect them.
  * Items with the fields of hgq_wrap_track_i; up to HGQ_TRACK_BATCH per launch, more are split over launches.
+ * The items of a launch run concurrently: two items of one launch that name the same i_var are refused (HGQ_ERR_ARG) - the
+ * repeated updates of a quantizer that several layers share go into successive calls.
  */
 #define HGQ_TRACK_BATCH 16
 typedef struct {
@@ -306,6 +308,9 @@ int hgq_dense_ebops(const uint32_t *amax_part, int n_parts, float decay, const f
  * layer depends on bit-width variables only (src/hgq/layers/core/base.py:100: shapes (1,) + shape[1:]), so the layers of
  * a model can be served together once the forward pass has produced every input quantizer's abs-max slices.
  * Descriptors are read on the host and travel as launch arguments (safe under HIP graph capture).
+ * The items of a launch (HGQ_EBOPS_BATCH consecutive items) run concurrently: two of them may share `i_in` only if neither
+ * tracks (amax_part NULL in both), else HGQ_ERR_ARG - a quantizer shared by several layers is updated by each layer's
+ * call in turn (src/hgq/layers/attn/mha.py:205-210), so such layers go into successive calls.
  */
 #define HGQ_EBOPS_BATCH 16
 typedef struct {

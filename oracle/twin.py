@@ -129,10 +129,11 @@ def ref_mha(layer, query_shape, value_shape=None, key_shape=None):
     vd = ref_einsum_dense(layer._value_dense, value_shape)
     od = ref_einsum_dense(layer._output_dense, tuple(query_shape[:-1]) + (N, layer._value_dim))
     # fused input quantizers are one shared object in the product; share the twin as well
-    if layer._query_dense.enable_iq and layer._query_dense._iq is layer._value_dense._iq:
-        qd.iq = vd.iq
-    if layer._key_dense.enable_iq and layer._key_dense._iq is layer._value_dense._iq:
-        kd.iq = vd.iq
+    for d, own in ((qd, layer._query_dense), (kd, layer._key_dense)):
+        if own.enable_iq and own._iq is layer._value_dense._iq:
+            orphan = d.iq.quantizer
+            d.iq = vd.iq
+            PAIRS[:] = [pair for pair in PAIRS if pair[1] is not orphan]  # the twin that was built for it is never called
     return ref.RefQMultiHeadAttention(qd, kd, vd, od, ref_softmax(layer._softmax), beta0=_beta(layer),
                                       enable_ebops=layer.enable_ebops, parallelization_factor=layer.parallelization_factor)
 

@@ -322,6 +322,42 @@ def test_ebops_scaling_is_a_product_then_a_correctly_rounded_division(dev):
         assert torch.equal(b_k.grad, torch.full_like(b_k, float(g))) and torch.equal(f_in.grad, torch.full_like(f_in, float(g * np.float32(N))))
 
 
+def test_queued_updates_of_one_quantizer_run_in_turn(dev):
+    """Integer-bit updates queued during a model call go out together; the updates of a quantizer that several layers
+    share (reference src/hgq/layers/attn/mha.py:205-210) must still be applied one after the other, each from the value the
+    previous one left, and the library refuses a launch in which two items update the same variable."""
+    import ctypes
+
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(23)
+    m = 200
+    mode = _lib.mode_bits('RND', 'WRAP', training=True)
+    fb = torch.randint(0, 5, (m,), generator=g).float().to(dev)
+    amaxs = [(torch.rand(3, m, generator=g) * s).view(torch.int32).to(dev) for s in (0.5, 8.0, 2.0)]  # bit patterns of |x|
+    other_i, other_amax = torch.zeros(m, device=dev), (torch.rand(1, m, generator=g) * 4).view(torch.int32).to(dev)
+    start = torch.randint(-2, 6, (m,), generator=g).float().to(dev)
+    want = start.clone()
+    for a in amaxs:
+        ops.wrap_track_i_(a, want, fb, 0.75, mode)
+    want_other = other_i.clone()
+    ops.wrap_track_i_(other_amax, want_other, fb, 0.75, mode)
+    got = start.clone()
+    ops.begin_deferred()
+    ops.wrap_track_i_(amaxs[0], got, fb, 0.75, mode)
+    ops.wrap_track_i_(other_amax, other_i, fb, 0.75, mode)
+    ops.wrap_track_i_(amaxs[1], got, fb, 0.75, mode)
+    ops.wrap_track_i_(amaxs[2], got, fb, 0.75, mode)
+    assert torch.equal(got, start), 'queued, not yet applied'
+    ops.end_deferred()
+    assert torch.equal(got, want) and torch.equal(other_i, want_other)
+    assert not torch.equal(want, start)
+    items = (ops._TrackItem * 2)()
+    for t in range(2):
+        items[t] = ops._TrackItem(amaxs[t].data_ptr(), None, 3, got.data_ptr(), fb.data_ptr(), None, m, 0.75, 0.0, 0.0, mode)
+    assert _lib.load().hgq_wrap_track_i_multi(items, 2, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) != 0
+    assert torch.equal(got, want), 'a refused call changes nothing'
+
+
 def test_sparse_ce_and_sgd(dev):
     _lib, ops = _ops()
     g = torch.Generator().manual_seed(17)
