@@ -19,7 +19,7 @@ from .. import ops
 from ..core import get_initializer
 from ..quantizer import Quantizer, QuantizerConfig
 from ..quantizer.prefetch import quantize_together
-from .core.base import QLayerBaseSingleInput
+from .core.base import QLayerBaseSingleInput, mean_bits
 
 
 class QBatchNormalization(QLayerBaseSingleInput):
@@ -113,7 +113,7 @@ class QBatchNormalization(QLayerBaseSingleInput):
         bw_inp = self.iq.bits_(shape)
         bw_ker = self.kq.bits_(self.moving_mean.shape).reshape(self._shape)
         bw_bias = self.bq.bits_(self.moving_mean.shape).reshape(self._shape)
-        return torch.sum(bw_inp * bw_ker) + torch.mean(bw_bias) * float(prod(shape))
+        return torch.sum(bw_inp * bw_ker) + mean_bits(bw_bias) * float(prod(shape))
 
     def compute_output_shape(self, input_shape):
         return input_shape

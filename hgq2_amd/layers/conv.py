@@ -16,7 +16,7 @@ from ..core import get_initializer
 from ..quantizer import Quantizer
 from ..quantizer.config import QuantizerConfig
 from .core._contraction import get_activation
-from .core.base import QLayerBaseSingleInput
+from .core.base import QLayerBaseSingleInput, mean_bits
 
 
 def _pair(v):
@@ -137,7 +137,7 @@ class QConv2D(QLayerBaseSingleInput):
         if self.bq is not None:
             size = float(prod(shape[:-1]) * self.filters)
             bw_bias = self.bq.bits_(self.bias.shape)
-            ebops = ebops + torch.mean(bw_bias) * size
+            ebops = ebops + mean_bits(bw_bias) * size
         return ebops
 
     def get_config(self):

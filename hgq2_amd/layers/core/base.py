@@ -29,6 +29,11 @@ def scale_ebops(ebops: torch.Tensor, parallelization_factor, n_parallel) -> torc
     return ebops / torch.full((), float(n_parallel), dtype=ebops.dtype, device=ebops.device)
 
 
+def mean_bits(bits: torch.Tensor) -> torch.Tensor:
+    """``mean(bits)`` as a sum and one correctly rounded division (the library's GPU mean multiplies by a rounded 1 / n)."""
+    return torch.sum(bits) / torch.full((), float(bits.numel()), dtype=bits.dtype, device=bits.device)
+
+
 class QLayerBase(Layer):
     """Handles the input / output quantizers, the ``beta`` and ``ebops`` variables and the
     EBOPs loss term.  Subclasses implement ``call`` and ``_compute_ebops(*input_shapes)``."""

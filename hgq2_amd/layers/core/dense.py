@@ -10,7 +10,7 @@ from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
 from ._contraction import dense_contraction, dense_ebops_term, get_activation
-from .base import QLayerBaseSingleInput, scale_ebops
+from .base import QLayerBaseSingleInput, mean_bits, scale_ebops
 
 
 class QDense(QLayerBaseSingleInput):
@@ -97,7 +97,7 @@ class QDense(QLayerBaseSingleInput):
         ebops = torch.sum(torch.matmul(bw_inp, bw_ker))
         if self.bq is not None:
             bw_bias = self.bq.bits_(self.bias.shape)
-            ebops = ebops + torch.mean(bw_bias) * out_size
+            ebops = ebops + mean_bits(bw_bias) * out_size
         return scale_ebops(ebops, self.parallelization_factor, self.n_parallel)
 
     def get_config(self):

@@ -17,7 +17,7 @@ from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
 from ._contraction import dense_contraction, dense_ebops_term, get_activation
-from .base import QLayerBaseSingleInput, scale_ebops
+from .base import QLayerBaseSingleInput, mean_bits, scale_ebops
 
 
 def _einsum_free0_size(equation: str, input_shape) -> int:
@@ -200,7 +200,7 @@ class QEinsumDense(QLayerBaseSingleInput):
         ebops = torch.einsum(self.ebops_equation, bw_inp, bw_ker)
         if self.bq is not None:
             bw_bias = self.bq.bits_(self.bias.shape)
-            ebops = ebops + torch.mean(bw_bias) * out_size
+            ebops = ebops + mean_bits(bw_bias) * out_size
         return scale_ebops(ebops, self.parallelization_factor, self.n_parallel)
 
     def get_config(self):

@@ -44,7 +44,14 @@ class Quantizer(Layer):
 
     def call(self, inputs, training=None):
         if self.scaler is not None:
-            inputs = inputs / self.scaler
+            # the divisor goes in as a tensor: on the GPU torch divides by a Python number with a multiplication by its
+            # rounded reciprocal, one ulp away from the quotient for some inputs (and one quantization step after rounding)
+            key = (inputs.device, inputs.dtype)
+            cached = getattr(self, '_scaler_tensor', None)
+            if cached is None or cached[0] != key:
+                cached = (key, torch.full((), float(self.scaler), dtype=inputs.dtype, device=inputs.device))
+                object.__setattr__(self, '_scaler_tensor', cached)
+            inputs = inputs / cached[1]
         outputs = self.quantizer(inputs, training=training)
         if self.scaler is not None:
             outputs = outputs * self.scaler

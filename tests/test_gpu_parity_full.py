@@ -426,6 +426,25 @@ def test_stochastic_quantizer_classes_follow_the_oracle(dev, q_type, overflow_mo
     assert q.quantizer._seed_gen.offset == 3  # no draw outside training
 
 
+def test_scaler_division_is_correctly_rounded(dev):
+    """``inputs / scaler`` (reference src/hgq/quantizer/quantizer.py:50-51) with a scaler that is no power of two: the quotient
+    has to be the correctly rounded one - a multiplication by 1 / scaler is an ulp off for about one value in eight, which
+    stochastic rounding turns into a different quantized value for some of them."""
+    from hgq2_amd.quantizer import Quantizer, QuantizerConfig
+
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(20000, 24, generator=g) * 30
+    q = Quantizer(QuantizerConfig('kif', 'datalane', overflow_mode='SAT', round_mode='S_RND', scaler=3.0))
+    q.quantizer._seed = 99
+    q(x.to(dev), training=True)
+    r = twin.ref_quantizer(q)
+    want_in = x / 3.0
+    assert not torch.equal(want_in, x * torch.tensor(1.0 / 3.0)), 'the data must tell the two apart'
+    for step in range(2):
+        yp, yr = q(x.to(dev), training=True), r(x, training=True)
+        assert torch.equal(yp.cpu(), yr), f'step {step}: {int((yp.cpu() != yr).sum())} values differ'
+
+
 def test_stochastic_rounding_refuses_graph_capture(dev):
     from hgq2_amd.quantizer.fixed_point_ops import SeedGenerator
 
