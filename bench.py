@@ -10,6 +10,7 @@ Prints one JSON line.  Everything is synthetic (seeded) data with inputs residen
 from __future__ import annotations
 
 import argparse
+import contextlib
 import ctypes
 import json
 import os
@@ -221,10 +222,11 @@ def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False, cpu_budge
     def step():
         # forward, loss (+ EBOPs terms), backward, SGD update with the MonoL1 gradient and the
         # bit-width constraints folded into the update kernel
-        opt.zero_grad()
-        loss = model_loss(model, loss_fn(model(x, training=True)), True)
-        opt.backward(loss)
-        opt.step()
+        with ops.overlap_ebops() if OVERLAP else contextlib.nullcontext():
+            opt.zero_grad()
+            loss = model_loss(model, loss_fn(model(x, training=True)), True)
+            opt.backward(loss)
+            opt.step()
         return loss.detach()
 
     run = step
@@ -240,7 +242,7 @@ def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False, cpu_budge
         for p in model.parameters():
             p.grad = None
         g_ = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g_):
+        with torch.cuda.graph(g_, stream=side):  # the stream of the warm-up steps: per-stream scratch made there is reused
             static_loss = step()
 
         def run():
@@ -344,6 +346,9 @@ def cpu_baseline(budget_s=20.0):
             'sample': f'{n} training steps of the same MLP at batch {BATCH} (eager torch-CPU restatement of the reference path)'}
 
 
+OVERLAP = True  # EBOPs launches of the per-layer steps on a second stream (see hgq2_amd.ops.overlap_ebops)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -356,6 +361,7 @@ def main():
     ap.add_argument('--config-step', choices=('particle', 'conv', 'mha'), default=None,
                     help='time one forward + backward pass of another configuration at full size instead of the headline run')
     ap.add_argument('--config-cpu', action='store_true', help='with --config-step: also time the CPU oracle of the same model')
+    ap.add_argument('--no-overlap', action='store_true', help='keep the EBOPs launches of the per-layer steps on the main stream')
     ap.add_argument('--graph', action='store_true', help='with --config-step: capture the step in a HIP graph and replay it')
     ap.add_argument('--softmax-only', action='store_true',
                     help='run only the one-pass table-softmax kernels at the attention configuration (for profiler runs)')
@@ -363,6 +369,8 @@ def main():
                     help='fused: whole-step kernels (2 launches); layers: per-layer torch.library operators with autograd; '
                          '-graph: the step is captured once in a HIP graph and replayed')
     args = ap.parse_args()
+    global OVERLAP
+    OVERLAP = not args.no_overlap
     if args.gpus != 1:
         print(f'bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported', file=sys.stderr)
         sys.exit(2)

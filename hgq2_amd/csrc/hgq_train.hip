@@ -370,9 +370,10 @@ __global__ void ebops_finish_bwd_kernel(const float *g, const float *beta, float
 }
 
 // one thread per row; C is small (class count)
+// `state` = {running sum (float), finished workgroups}: both zero at the start and left zero at the end
 __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict__ logits,
                                                         const int64_t *__restrict__ labels, float *loss,
-                                                        float *__restrict__ dlogits, int64_t rows, int C) {
+                                                        float *__restrict__ dlogits, int64_t rows, int C, uint32_t *state) {
     __shared__ float red[4];
     const float inv_rows = 1.0f / (float)rows;
     float acc = 0.0f;
@@ -392,7 +393,20 @@ __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict_
         }
     }
     acc = block_sum_256(acc, red);
-    if (threadIdx.x == 0) atomicAdd(loss, acc * inv_rows);
+    if (threadIdx.x == 0) {
+        if (!state) {
+            atomicAdd(loss, acc * inv_rows);
+            return;
+        }
+        // both words are only ever touched by device-scope atomics, which are performed at the memory side: the wait
+        // between the two makes this workgroup's part arrive before it counts as finished (no cache write-back needed)
+        atomicAdd((float *)state, acc * inv_rows);
+        __threadfence_block();
+        if (atomicAdd(state + 1, 1u) == gridDim.x - 1) {
+            loss[0] = __uint_as_float(atomicExch(state, 0u));  // every other workgroup has added its part
+            atomicExch(state + 1, 0u);
+        }
+    }
 }
 
 __global__ __launch_bounds__(256) void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, int64_t n,
@@ -613,14 +627,16 @@ extern "C" int hgq_dense_ebops_multi(const hgq_dense_ebops_item *items, int coun
 }
 
 extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *loss, float *dlogits,
-                                     int64_t rows, int C, void *stream) {
+                                     int64_t rows, int C, uint32_t *state, void *stream) {
     if (rows < 1 || C < 1) return fail(HGQ_ERR_ARG, "hgq_sparse_ce_fwd_bwd: bad sizes");
     if (!logits || !labels || !loss) return fail(HGQ_ERR_ARG, "hgq_sparse_ce_fwd_bwd: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    int rc = fill_f32(loss, 0.0f, 1, s);
-    if (rc) return rc;
+    if (!state) {
+        int rc = fill_f32(loss, 0.0f, 1, s);
+        if (rc) return rc;
+    }
     const int grid = persistent_grid((rows + 255) / 256, 4);
-    hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C);
+    hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C, state);
     return check_launch("hgq_sparse_ce_fwd_bwd");
 }
 

@@ -107,7 +107,7 @@ class QBatchNormalization(QLayerBaseSingleInput):
         scale, offset = self._scale_offset(mean, variance)
         qscale, qoffset = quantize_together([(self.kq, scale.contiguous()), (self.bq, offset.contiguous())], training)
         qscale, qoffset = qscale.reshape(self._shape), qoffset.reshape(self._shape)
-        return inputs * qscale + qoffset
+        return ops.affine_rows(inputs, qscale, qoffset)
 
     def _compute_ebops(self, shape):
         bw_inp = self.iq.bits_(shape)

@@ -13,6 +13,7 @@ from math import prod
 
 import torch
 
+from ... import ops
 from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
@@ -161,13 +162,13 @@ class QEinsumDense(QLayerBaseSingleInput):
             y, act_done, self._deferred = dense_contraction(x, iq, w2d, b1d, fuse_act, training)
             y = y.view(inputs.shape[0], *self.full_output_shape[1:])
             if qbias is not None and not self._bias_in_gemm:
-                y = y + qbias
+                y = ops.bias_add_rows(y, qbias)
             return y, act_done
         if iq is not None:
             inputs = iq(inputs, training=training)
         y = torch.einsum(self.equation, inputs, qkernel)
         if qbias is not None:
-            y = y + qbias
+            y = ops.bias_add_rows(y, qbias)
         return y, False
 
     def call(self, inputs, training=None):

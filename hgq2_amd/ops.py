@@ -369,11 +369,79 @@ def touch_state():
     STATE_EPOCH[0] += 1
 
 
+# ---- launches on a second stream
+# The EBOPs estimates read bit-width variables (and the abs-max slices a quantizer left); what they write - the loss
+# term, the uint32 variable, gradient pieces - is read again only when the loss is summed and when the optimizer
+# steps.  They are single-workgroup, latency-bound launches.  Inside ``overlap_ebops()`` they go to a second stream
+# (default priority) that forks from the current one where they are issued and is joined where their results are read,
+# so they run beside the layers' data kernels; in a captured step the fork and join become edges of the graph.
+_OVERLAP = {'depth': 0, 'streams': {}, 'pending': [], 'keep': [], 'finish': []}
+
+
+class overlap_ebops:
+    """Context manager around a training step (forward, loss, backward, update): EBOPs launches inside it run on a
+    second stream.  Whoever opens it must leave it before the captured graph ends or before results are read from
+    another thread or stream; leaving it joins the second stream."""
+
+    def __enter__(self):
+        _OVERLAP['depth'] += 1
+        return self
+
+    def __exit__(self, *exc):
+        _OVERLAP['depth'] -= 1
+        if _OVERLAP['depth'] == 0:
+            join_side()
+        return False
+
+
+class side_branch:
+    """The launches inside go to the second stream when ``overlap_ebops`` is open (else nothing changes)."""
+
+    def __enter__(self):
+        self.ctx = None
+        if _OVERLAP['depth'] and torch.cuda.is_available():
+            cur = torch.cuda.current_stream()
+            side = _OVERLAP['streams'].get(cur.device)
+            if side is None:
+                side = _OVERLAP['streams'][cur.device] = torch.cuda.Stream(device=cur.device)
+            if side != cur:
+                side.wait_stream(cur)  # everything issued so far is visible to the branch
+                if not any(s is side for _, s in _OVERLAP['pending']):
+                    _OVERLAP['pending'].append((cur, side))
+                self.ctx = torch.cuda.stream(side)
+                self.ctx.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+
+def join_side():
+    """The current stream waits for the second stream's work (no-op when there is none)."""
+    pending, _OVERLAP['pending'] = _OVERLAP['pending'], []
+    for cur, side in pending:
+        torch.cuda.current_stream(cur.device).wait_stream(side)
+    finish, _OVERLAP['finish'] = _OVERLAP['finish'], []
+    for launch in finish:  # work that needed both streams' results (the sum of the loss terms)
+        launch()
+    _OVERLAP['keep'] = []
+
+
+def _keep(tensors):
+    """Short-lived inputs of a launch that may be on the second stream (tracker slices written by the data kernels) stay
+    referenced until the streams are joined: the allocator would otherwise hand their memory to a later launch of the
+    first stream while the second still reads it."""
+    if _OVERLAP['depth']:
+        _OVERLAP['keep'].extend(t for t in tensors if t is not None)
+
+
 # ---- launches deferred to the end of the outermost layer call
 # The EBOPs estimate of a dense layer (and the integer-bit update fused into it) reads bit-width variables and the
 # abs-max slices its own forward left; nothing later in the forward pass reads what it writes.  While a model call is
 # open the calls are queued - outputs allocated, nothing launched - and go out as one launch when the call returns.
-_DEFER = {'depth': 0, 'dense_ebops': [], 'tracks': []}
+_DEFER = {'depth': 0, 'dense_ebops': [], 'tracks': [], 'late': []}
 
 
 def begin_deferred():
@@ -384,7 +452,10 @@ def end_deferred(discard: bool = False):
     _DEFER['depth'] -= 1
     if _DEFER['depth'] == 0:
         if discard:
-            _DEFER['dense_ebops'], _DEFER['tracks'] = [], []
+            _DEFER['dense_ebops'], _DEFER['tracks'], _DEFER['late'] = [], [], []
+        elif _OVERLAP['depth'] and _worth_a_branch():
+            with side_branch():
+                flush_deferred()
         else:
             flush_deferred()
 
@@ -404,6 +475,15 @@ def _rounds(keys):
     return rounds
 
 
+def _order_after_side():
+    """A flush issued on the first stream while the second still has work of this step: the second goes first (its
+    launches were queued earlier and may touch the same variables)."""
+    if _OVERLAP['pending']:
+        cur = torch.cuda.current_stream()
+        if not any(cur == side for _, side in _OVERLAP['pending']):
+            join_side()
+
+
 def flush_tracks():
     """Run the queued integer-bit updates (one launch; one more for every repeated update of the same variable).  Everything
     that reads integer bits of a WRAP quantizer inside a model call - the EBOPs launches, the bit-width views - calls
@@ -411,20 +491,50 @@ def flush_tracks():
     q, _DEFER['tracks'] = _DEFER['tracks'], []
     if not q:
         return
+    _order_after_side()
     touch_state()
     with torch.no_grad():
+        _keep(item[0] for item in q)
         for members in _rounds([item[1].data_ptr() for item in q]):
             amaxs, i_vars, fbs, decays, modes = (list(c) for c in zip(*[q[n] for n in members]))
             wrap_track_i_multi_op(amaxs, i_vars, fbs, [float(d) for d in decays], [int(m) for m in modes])
 
 
+def _reads_queued(i_var) -> bool:
+    """Is a queued EBOPs launch going to read this integer-bit variable?"""
+    ptr = i_var.data_ptr()
+    return (any(item[3].data_ptr() == ptr for item in _DEFER['dense_ebops'])
+            or any(ptr in reads for reads, _ in _DEFER['late']))
+
+
+def _worth_a_branch() -> bool:
+    """A fork and a join between two streams cost a replayed graph about 15 us of idle time on this platform, a queued
+    single-workgroup launch hides 5 - 30 us: the branch pays from about three launches on, or one long one (the EBOPs of
+    a contraction with a few thousand input channels)."""
+    n = len(_DEFER['late']) + (1 if _DEFER['tracks'] else 0) + (1 if _DEFER['dense_ebops'] else 0)
+    big = any(item[14][1] * item[14][2] >= 16384 for item in _DEFER['dense_ebops'])
+    return n >= 3 or (big and n >= 2)
+
+
 def flush_deferred():
     flush_tracks()
+    if _DEFER['late'] or _DEFER['dense_ebops']:
+        _order_after_side()
+    late, _DEFER['late'] = _DEFER['late'], []
+    _flush_dense_queue()
+    for _, launch in late:
+        launch()
+
+
+def _flush_dense_queue():
     q, _DEFER['dense_ebops'] = _DEFER['dense_ebops'], []
     if not q:
         return
     touch_state()  # the fused integer-bit update writes `_i`
     with torch.no_grad():
+        # inputs and outputs alike: an output nobody holds on to (the plain EBOPs value beside the loss term) would be
+        # handed to the next allocation of the first stream and then overwritten from the second
+        _keep(t for item in q for t in item if torch.is_tensor(t))
         # layers that share an input quantizer update and read its integer bits one after the other
         for members in _rounds([item[3].data_ptr() for item in q]):
             _flush_dense_ebops(*zip(*[q[n] for n in members]))
@@ -457,6 +567,9 @@ dense_ebops_track_op = torch.library.custom_op('hgq::dense_ebops_track', _dense_
 dense_ebops_op = torch.library.custom_op('hgq::dense_ebops', _dense_ebops_impl, mutates_args=('ebops_var',))
 
 
+_CE_STATE = {}
+
+
 @torch.library.custom_op('hgq::sparse_ce', mutates_args=())
 def sparse_ce_op(logits: Tensor, labels: Tensor) -> tuple[Tensor, Tensor]:
     _check_f32('logits', logits)
@@ -464,8 +577,14 @@ def sparse_ce_op(logits: Tensor, labels: Tensor) -> tuple[Tensor, Tensor]:
     _need(labels.dtype == torch.int64 and labels.is_cuda and labels.is_contiguous(), 'labels must be a contiguous int64 GPU tensor')
     loss = torch.empty((), dtype=torch.float32, device=logits.device)
     dlogits = torch.empty_like(logits)
+    # two words per (device, stream), zeroed once: the kernel leaves them zero, so no call clears anything
+    stream = _stream()
+    key = (logits.device, stream.value if hasattr(stream, 'value') else stream)
+    state = _CE_STATE.get(key)
+    if state is None:
+        state = _CE_STATE[key] = torch.zeros(2, dtype=torch.int32, device=logits.device)
     rc = _lib.load().hgq_sparse_ce_fwd_bwd(_ptr(logits), _ptr(labels), _ptr(loss), _ptr(dlogits), logits.shape[0],
-                                           logits.shape[1], _stream())
+                                           logits.shape[1], _ptr(state), stream)
     _lib.check(rc, 'hgq_sparse_ce_fwd_bwd')
     return loss, dlogits
 
@@ -554,6 +673,22 @@ class _SumScalars(torch.autograd.Function):
     def backward(ctx, g):
         # every term receives the same upstream gradient: views of it, no launches
         return tuple(g.reshape(s) if ctx.needs_input_grad[t] else None for t, s in enumerate(ctx.shapes))
+
+
+def sum_scalars_into(terms: Sequence[Tensor], out: Tensor) -> None:
+    """``out <- ((terms[0] + terms[1]) + ...)`` (values only) on the current stream; ``out`` is a one-element fp32 GPU tensor."""
+    terms = [t.detach() for t in terms]
+    while len(terms) > SUM_BATCH:
+        terms = [sum_scalars_op(terms[:SUM_BATCH])] + terms[SUM_BATCH:]
+    n = len(terms)
+    ptrs = (ctypes.c_void_p * n)()
+    for t, term in enumerate(terms):
+        _check_f32('term', term)
+        _need(term.numel() == 1, 'every term must hold one element')
+        ptrs[t] = term.data_ptr()
+    _check_f32('out', out)
+    rc = _lib.load().hgq_sum_scalars(ptrs, n, _ptr(out), _stream())
+    _lib.check(rc, 'hgq_sum_scalars')
 
 
 def sum_scalars(terms: Sequence[Tensor]) -> Tensor:
@@ -1394,7 +1529,7 @@ def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('
     """In-place integer-bit tracking; ``amax`` is [m] or [n_parts, m]."""
     m = i_var.numel()
     n_parts = amax.numel() // m
-    if _DEFER['dense_ebops'] and any(item[3].data_ptr() == i_var.data_ptr() for item in _DEFER['dense_ebops']):
+    if (_DEFER['dense_ebops'] or _DEFER['late']) and _reads_queued(i_var):
         flush_deferred()  # a queued EBOPs estimate reads these integer bits as they stand now
     if (_DEFER['depth'] > 0 and anyneg is None and k_var is None and not (mode & (_lib.MODE_KBI | _lib.MODE_TRACING))
             and c_lo == float('-inf') and c_hi == float('inf')):
@@ -1403,6 +1538,7 @@ def wrap_track_i_(amax, i_var, fb, decay, mode, c_lo=float('-inf'), c_hi=float('
         _DEFER['tracks'].append((amax, i_var, fb, decay, mode))
         return
     touch_state()
+    _keep((amax, anyneg))
     empty_i = amax.new_empty(0)
     empty_k = torch.empty(0, dtype=torch.uint8, device=amax.device)
     wrap_track_i_op(amax, anyneg if anyneg is not None else empty_i, n_parts, i_var, fb,
@@ -1457,6 +1593,7 @@ class _DenseEbops(torch.autograd.Function):
     def forward(ctx, i_in, f_in, b_ker, b_bias, amax, decay, beta, k_in, k_ker, k_bias, ebops_var, P, K, N, scale, bias_size,
                 mode_in, mode_ker, mode_bias, owners):  # scale = (par_factor, n_parallel, ebops_factor)
         ctx.owners = owners
+        _keep((amax,))
         if _DEFER['depth'] > 0:  # inside a model call: queued, launched with the other layers' when the call returns
             op = _dense_ebops_queue
         else:
@@ -1496,6 +1633,7 @@ class _DenseEbops(torch.autograd.Function):
                 for o, piece in pieces:
                     _stash_side(o, up, piece)
                 return (None,) * 20
+        join_side()  # the kernel that fills `g` may have run on the second stream
         grads = g if _is_unit(up) else up * g
         gf = grads[:n_f]
         gi = gf.view(s_i) if want_i else None
@@ -1791,8 +1929,6 @@ class _BitsEbops(torch.autograd.Function):
     @staticmethod
     def forward(ctx, kind, params, beta, ebops_var, layouts, owners, *qvars):
         ctx.owners = owners
-        flush_tracks()  # the bit-widths read here include integer bits whose update may still be queued
-        lib = _lib.load()
         ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
         total = sum(2 * fb.numel() for fb, lay in zip(fbs, layouts) if lay is not None)
         buf = torch.empty(max(total, 1), dtype=torch.float32, device=beta.device)
@@ -1811,6 +1947,25 @@ class _BitsEbops(torch.autograd.Function):
             descs.append(_lib.BitsDesc(k.data_ptr() if add_mode else None, None if kbi else i.data_ptr(), fb.data_ptr(), size, inner,
                                        int(kbi), int(add_mode), None if kbi else g_i.data_ptr(), g_fb.data_ptr()))
         out = torch.empty((), dtype=torch.float32, device=beta.device)
+        if _DEFER['depth'] > 0 and _OVERLAP['depth'] > 0:
+            # a step that runs its EBOPs launches beside the data kernels: this one goes out with the others when the
+            # model call returns (outputs exist already; the integer bits it reads are guarded by `_reads_queued`)
+            reads = {i.data_ptr() for i, lay in zip(is_, layouts) if lay is not None and not lay[2]}
+            _keep(qvars + (out, buf))  # operands may be temporaries, outputs may be dropped: all outlive the launch on the second stream
+            _DEFER['late'].append((reads, lambda: _BitsEbops._launch(kind, params, beta, ebops_var, descs, out)))
+        else:
+            flush_tracks()  # the bit-widths read here include integer bits whose update may still be queued
+            _BitsEbops._launch(kind, params, beta, ebops_var, descs, out)
+        ctx.save_for_backward(buf)
+        ctx.slots = [None if s is None else (s[0].storage_offset(), s[1].storage_offset(), s[1].numel()) for s in slots]
+        ctx.kbis = [None if lay is None else lay[2] for lay in layouts]
+        ctx.shapes = [(i.shape, fb.shape) for i, fb in zip(is_, fbs)]
+        ctx.mark_non_differentiable(ebops_var)
+        return out
+
+    @staticmethod
+    def _launch(kind, params, beta, ebops_var, descs, out):
+        lib = _lib.load()
         ptrs = [ctypes.addressof(d) if d is not None else None for d in descs]
         if kind == 'lut':
             n_cells, scale, factor = params
@@ -1827,12 +1982,6 @@ class _BitsEbops(torch.autograd.Function):
             rc = lib.hgq_mha_ebops(ptrs[0], ptrs[1], ptrs[2], ptrs[3], T, S, N, H, Hv, f1, f2, _ptr(beta), _ptr(ebops_var), _ptr(out),
                                    _stream())
         _lib.check(rc, f'hgq_{kind}_ebops')
-        ctx.save_for_backward(buf)
-        ctx.slots = [None if s is None else (s[0].storage_offset(), s[1].storage_offset(), s[1].numel()) for s in slots]
-        ctx.kbis = [None if lay is None else lay[2] for lay in layouts]
-        ctx.shapes = [(i.shape, fb.shape) for i, fb in zip(is_, fbs)]
-        ctx.mark_non_differentiable(ebops_var)
-        return out
 
     @staticmethod
     def backward(ctx, g):
@@ -1852,6 +2001,7 @@ class _BitsEbops(torch.autograd.Function):
                 for o, piece in pieces:
                     _stash_side(o, g, piece)
                 return (None,) * n_args
+        join_side()  # the kernel that fills `buf` may have run on the second stream
         scaled = buf if _is_unit(g) else buf * g  # one launch for every operand
         grads = [None, None, None, None, None, None]
         for slot, kbi, (i_shape, fb_shape) in zip(ctx.slots, ctx.kbis, ctx.shapes):
@@ -1861,6 +2011,81 @@ class _BitsEbops(torch.autograd.Function):
             oi, of, n = slot
             grads += [None, None if kbi else scaled[oi:oi + n].view(i_shape), scaled[of:of + n].view(fb_shape)]
         return tuple(grads)
+
+
+class _BiasAddRows(torch.autograd.Function):
+    """``y + b`` for a bias that spans (a broadcast of) one batch element.  The bias gradient, a sum over the batch, is
+    taken by the library's fixed-order slice reduction: a framework reduction over many workgroups records a memory-clearing
+    node when the step is captured in a graph, and such nodes have replayed wrongly on this platform."""
+
+    @staticmethod
+    def forward(ctx, y, b):
+        ctx.b_shape = b.shape
+        return y + b
+
+    @staticmethod
+    def backward(ctx, g):
+        db = None
+        if ctx.needs_input_grad[1]:
+            g2 = g.contiguous().view(g.shape[0], -1)
+            full = torch.empty(g2.shape[1], dtype=torch.float32, device=g.device)
+            e = full.new_empty(0)
+            reduce_slices_multi_op([g2], [full, e, e], [False, False, False])
+            db = full.view(g.shape[1:]).sum_to_size(ctx.b_shape)  # over the bias' own broadcast axes, if any (small)
+        return g, db
+
+
+class _AffineRows(torch.autograd.Function):
+    """``x * s + o`` with ``s``, ``o`` of one value per trailing channel (a multiplication, then an addition, as the
+    reference's ``inputs * qscale + qoffset``, src/hgq/layers/batch_normalization.py:184).  The gradients of ``s`` and
+    ``o`` - sums over all rows - are taken by the library's fixed-order slice reduction, both in one launch."""
+
+    @staticmethod
+    def forward(ctx, x, s, o):
+        ctx.save_for_backward(x, s)
+        ctx.shapes = (s.shape, o.shape)
+        return x * s + o
+
+    @staticmethod
+    def backward(ctx, g):
+        x, s = ctx.saved_tensors
+        g = g.contiguous()
+        C = x.shape[-1]
+        dx = g * s if ctx.needs_input_grad[0] else None
+        ds = do = None
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            e = g.new_empty(0)
+            sets, outs = [], []
+            if ctx.needs_input_grad[1]:
+                ds = torch.empty(C, dtype=torch.float32, device=g.device)
+                sets.append((g * x).view(-1, C)), outs.extend([ds, e, e])
+            if ctx.needs_input_grad[2]:
+                do = torch.empty(C, dtype=torch.float32, device=g.device)
+                sets.append(g.view(-1, C)), outs.extend([do, e, e])
+            reduce_slices_multi_op(sets, outs, [False] * len(outs))
+            ds = ds.view(ctx.shapes[0]) if ds is not None else None
+            do = do.view(ctx.shapes[1]) if do is not None else None
+        return dx, ds, do
+
+
+def affine_rows(x: Tensor, s: Tensor, o: Tensor) -> Tensor:
+    """``x * s + o`` for per-channel ``s`` and ``o`` along the last axis of ``x`` (any other layout: plain tensor operations)."""
+    C = x.shape[-1] if x.dim() else 0
+    if (x.is_cuda and x.dtype == torch.float32 and x.dim() >= 2 and x.numel() > 0 and s.numel() == C and o.numel() == C
+            and s.shape[-1:] == (C,) and o.shape[-1:] == (C,) and s.dtype == torch.float32 and o.dtype == torch.float32):
+        return _AffineRows.apply(x.contiguous(), s, o)
+    return x * s + o
+
+
+def bias_add_rows(y: Tensor, b: Tensor) -> Tensor:
+    """``y + b`` with ``b`` broadcast over the leading (batch) axis of ``y`` only or also over trailing axes of size one."""
+    bs = tuple(b.shape)
+    if len(bs) == y.dim() and bs[0] == 1:
+        bs = bs[1:]
+    if (y.is_cuda and y.dtype == torch.float32 and b.dtype == torch.float32 and y.dim() >= 2 and y.shape[0] >= 1 and y.numel() > 0
+            and len(bs) <= y.dim() - 1 and all(s in (1, t) for s, t in zip(reversed(bs), reversed(tuple(y.shape[1:]))))):
+        return _BiasAddRows.apply(y, b)
+    return y + b
 
 
 def bits_ebops(kind: str, operands, params, beta: Tensor, ebops_var: Tensor, owners=None) -> Tensor:

@@ -28,6 +28,17 @@ def model_loss(model, base_loss, fold_regularizers: bool = False):
         if fold_regularizers and isinstance(r, MonoL1):
             continue
         terms.append(r(p))
+    if ops._OVERLAP['pending'] and len(terms) > 1 and all(
+            torch.is_tensor(t) and t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 for t in terms):
+        # EBOPs launches of this step are running on the second stream: the total (nothing but the caller's print-out
+        # reads it) is summed when the streams are joined, and the backward pass starts from the terms themselves -
+        # d total / d term = 1 - so the first stream does not wait for the second before the update
+        total = torch.empty(torch.broadcast_shapes(*[t.shape for t in terms]), dtype=torch.float32, device=terms[0].device)
+        held = list(terms)
+        ops._OVERLAP['finish'].append(lambda: ops.sum_scalars_into(held, total))
+        total._hgq_terms = [t for t in terms if t.requires_grad]
+        return total
+    ops.join_side()  # EBOPs terms issued on the second stream
     if len(terms) > 1 and all(torch.is_tensor(t) and t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 for t in terms):
         # the same additions in the same order, one launch
         return ops.sum_scalars(terms).reshape(torch.broadcast_shapes(*[t.shape for t in terms]))
@@ -64,11 +75,16 @@ class SGD:
             raise ValueError('backward(loss) expects a scalar loss')
         if self._unit is None or self._unit.device != loss.device or self._unit.shape != loss.shape:
             self._unit = torch.ones_like(loss)  # the seed gradient: allocated once, also outside a captured graph
+        terms = getattr(loss, '_hgq_terms', None)
         with ops.side_gradients(self._unit):
-            loss.backward(self._unit)
+            if terms is not None:  # `model_loss` inside `ops.overlap_ebops()`: the sum is a plain value, its terms carry the graph
+                torch.autograd.backward(terms, [self._unit.reshape(t.shape) for t in terms])
+            else:
+                loss.backward(self._unit)
 
     @torch.no_grad()
     def step(self):
+        ops.join_side()
         ws, gs, l1s, los, his, sides, post = [], [], [], [], [], [], []
         for p in self.params:
             side = list(getattr(p, '_hgq_side', None) or ())
@@ -105,8 +121,9 @@ class GraphedTrainStep:
     static buffers before each replay.  ``loss_fn(outputs, labels)`` must be built from capturable
     operations (``hgq2_amd.ops.sparse_ce`` is)."""
 
-    def __init__(self, model, loss_fn, optimizer: SGD, example_x, example_y, warmup: int = 3):
+    def __init__(self, model, loss_fn, optimizer: SGD, example_x, example_y, warmup: int = 3, overlap: bool = True):
         self.model, self.loss_fn, self.opt = model, loss_fn, optimizer
+        self.overlap = overlap  # EBOPs launches and the loss sum on a second branch of the graph, beside loss and backward
         self.x = example_x.clone()
         self.y = example_y.clone()
         self.loss = None
@@ -119,15 +136,20 @@ class GraphedTrainStep:
         torch.cuda.synchronize()
         self.opt.zero_grad(set_to_none=True)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
+        # captured on the stream the warm-up ran on: scratch that operators keep per stream (allocated and cleared once,
+        # during the warm-up) is found again instead of being created, and cleared, inside the graph
+        with torch.cuda.graph(self.graph, stream=side):
             self.loss = self._step()
 
     def _step(self):
-        self.opt.zero_grad(set_to_none=True)
-        out = self.model(self.x, training=True)
-        loss = model_loss(self.model, self.loss_fn(out, self.y), self.opt.fold_regularizers)
-        self.opt.backward(loss)
-        self.opt.step()
+        import contextlib
+
+        with ops.overlap_ebops() if self.overlap else contextlib.nullcontext():
+            self.opt.zero_grad(set_to_none=True)
+            out = self.model(self.x, training=True)
+            loss = model_loss(self.model, self.loss_fn(out, self.y), self.opt.fold_regularizers)
+            self.opt.backward(loss)
+            self.opt.step()
         return loss.detach()
 
     def __call__(self, x=None, y=None):

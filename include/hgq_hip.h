@@ -352,9 +352,12 @@ int hgq_mse_bwd(const float *pred, const float *target, const float *g, float *d
  * Mean sparse categorical cross-entropy from logits, forward and gradient in one pass.
  *   logits [rows, C]; labels [rows] int64;  loss [1] = mean_r(-log softmax(logits_r)[label_r]);
  *   dlogits [rows, C] = (softmax - onehot) / rows.
+ *   state: NULL, or two 32-bit words that are zero when the call starts; the kernel leaves them zero again (the
+ *   workgroup that finishes last takes the sum out and clears them), so one allocation zeroed once serves every later
+ *   call and the launch that would clear `loss` is saved.  Calls that overlap in time need separate words.
  */
 int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *loss, float *dlogits, int64_t rows,
-                          int C, void *stream);
+                          int C, uint32_t *state, void *stream);
 
 /*
  * Plain SGD update with the reference's post-update constraint and MonoL1 regulariser folded in.
