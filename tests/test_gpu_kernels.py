@@ -358,6 +358,39 @@ def test_queued_updates_of_one_quantizer_run_in_turn(dev):
     assert torch.equal(got, want), 'a refused call changes nothing'
 
 
+def test_bias_and_affine_gradients_without_framework_reductions(dev):
+    """``bias_add_rows`` / ``affine_rows``: values are the plain tensor expressions; the gradients of the small operands are
+    column sums taken by the library's fixed-order reduction (a framework reduction inside a captured step records a
+    memory-clearing node, which replays wrongly on this platform)."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(41)
+    y = torch.randn(1000, 16, 64, generator=g).to(dev)
+    up = torch.randn(1000, 16, 64, generator=g).to(dev)
+    for b_shape in ((16, 64), (1, 64), (16, 1), (64,)):
+        b1 = torch.randn(b_shape, generator=g).to(dev).requires_grad_(True)
+        b2 = b1.detach().clone().requires_grad_(True)
+        y1, y2 = y.clone().requires_grad_(True), y.clone().requires_grad_(True)
+        out = ops.bias_add_rows(y1, b1)
+        assert torch.equal(out, y2 + b2)
+        (out * up).sum().backward()
+        ((y2 + b2).double() * up.double()).sum().backward()
+        assert torch.equal(y1.grad, y2.grad)
+        scale = up.abs().double().sum(0).sum_to_size(b_shape)
+        assert torch.all((b1.grad.double() - b2.grad.double()).abs() <= 1e-6 * scale + 1e-30), b_shape
+    x = torch.randn(300, 7, 24, generator=g).to(dev)
+    up = torch.randn(300, 7, 24, generator=g).to(dev)
+    s1, o1 = torch.randn(1, 1, 24, generator=g).to(dev).requires_grad_(True), torch.randn(1, 1, 24, generator=g).to(dev).requires_grad_(True)
+    s2, o2 = s1.detach().double().requires_grad_(True), o1.detach().double().requires_grad_(True)
+    x1, x2 = x.clone().requires_grad_(True), x.double().requires_grad_(True)
+    out = ops.affine_rows(x1, s1, o1)
+    assert torch.equal(out, x * s1.detach() + o1.detach())
+    (out * up).sum().backward()
+    ((x2 * s2 + o2) * up.double()).sum().backward()
+    assert torch.allclose(x1.grad.double(), x2.grad, rtol=1e-6, atol=1e-7)
+    assert torch.all((s1.grad.double() - s2.grad).abs() <= 1e-6 * (up.double() * x.double()).abs().sum((0, 1), keepdim=True))
+    assert torch.all((o1.grad.double() - o2.grad).abs() <= 1e-6 * up.double().abs().sum((0, 1), keepdim=True))
+
+
 def test_sparse_ce_and_sgd(dev):
     _lib, ops = _ops()
     g = torch.Generator().manual_seed(17)

@@ -338,6 +338,98 @@ def test_graph_replay_equals_eager_steps(dev, kind):
                 assert torch.equal(pg, pe), f'{kind}: {name}'
 
 
+def test_graph_replays_with_row_broadcast_parameters(dev):
+    """A bias with one value per (position, channel) and the scale / offset of QBatchNormalization get their gradients from
+    sums over the batch.  Taken by framework reductions these were right in the first replay of a captured step and wrong
+    in later ones (memory-clearing nodes); taken by the library's slice reduction every replay follows the eager step."""
+    from hgq2_amd import ops
+    from hgq2_amd.core import Sequential
+    from hgq2_amd.layers import QBatchNormalization, QEinsumDense
+    from hgq2_amd.train import SGD, GraphedTrainStep, model_loss
+
+    g = torch.Generator().manual_seed(22116)
+    x = (torch.round(torch.randn(1000, 16, 8, generator=g).clamp(-5, 5) * 256) / 256).to(dev)
+
+    def make():
+        torch.manual_seed(5)
+        with readme_scopes(beta0=1e-4):
+            return Sequential([QEinsumDense('bpf,fh->bph', (16, 64), bias_axes='ph'), QBatchNormalization()])
+
+    eager, graphed = make(), make()
+    eager(x, training=True), graphed(x, training=True)
+    graphed.load_state_dict(eager.state_dict())
+    opt = SGD(eager.parameters(), lr=0.02, fold_regularizers=True)
+    gopt = SGD(graphed.parameters(), lr=0.02, fold_regularizers=True)
+
+    def eager_step():
+        opt.zero_grad()
+        loss = model_loss(eager, ops.mse(eager(x, training=True)), True)
+        opt.backward(loss)
+        opt.step()
+        return loss.detach()
+
+    for _ in range(3):
+        eager_step()
+    step = GraphedTrainStep(graphed, lambda out, y: ops.mse(out), gopt, x, x[:1], warmup=3)
+    for replay in range(4):
+        le, lg = eager_step(), step()
+        torch.cuda.synchronize()
+        assert abs(lg.item() - le.item()) <= 2e-5 * abs(le.item()) + 1e-9, f'replay {replay}'
+        for (name, pe), (_, pg) in zip(eager.state_dict().items(), graphed.state_dict().items()):
+            if pe.dtype.is_floating_point:
+                assert torch.allclose(pg, pe, rtol=2e-5, atol=1e-7), f'replay {replay}: {name}'
+            else:
+                assert torch.equal(pg, pe), f'replay {replay}: {name}'
+
+
+@pytest.mark.parametrize('kind', ['conv', 'mha', 'particle'])
+def test_ebops_on_a_second_stream_change_nothing(dev, kind):
+    """Inside ``ops.overlap_ebops()`` the EBOPs launches of a step (and the sum of the loss terms) run on a second stream
+    when there are enough of them: same loss, same update, bit for bit, as the single-stream step."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, model_loss
+    from hgq2_amd.utils import models
+
+    g = torch.Generator().manual_seed(33)
+    if kind == 'conv':
+        make = lambda: models.conv_stack(filters=8, n_out=10, device=dev)  # noqa: E731
+        x, y = torch.rand(64, 12, 12, 1, generator=g).to(dev), torch.randint(0, 10, (64,), generator=g).to(dev)
+        loss_fn = lambda out: ops.sparse_ce(out, y)  # noqa: E731
+    elif kind == 'particle':
+        make = lambda: models.particle_mlp(n_particles=8, n_features=16, hidden=(32, 16), device=dev)  # noqa: E731
+        x, y = torch.randn(64, 8, 16, generator=g).to(dev), torch.randint(0, 5, (64,), generator=g).to(dev)
+        loss_fn = lambda out: ops.sparse_ce(out, y)  # noqa: E731
+    else:
+        make = lambda: models.mha_block(num_heads=2, key_dim=8, device=dev)  # noqa: E731
+        x = torch.randn(32, 12, 16, generator=g).to(dev)
+        loss_fn = lambda out: ops.mse(out)  # noqa: E731
+    torch.manual_seed(3)
+    a = make()
+    a(x, training=True)
+    torch.manual_seed(3)
+    b = make()
+    b(x, training=True)
+    b.load_state_dict(a.state_dict())
+    oa, ob = SGD(a.parameters(), lr=0.02, fold_regularizers=True), SGD(b.parameters(), lr=0.02, fold_regularizers=True)
+    branched = 0
+    for step in range(3):
+        oa.zero_grad()
+        la = model_loss(a, loss_fn(a(x, training=True)), True)
+        oa.backward(la)
+        oa.step()
+        with ops.overlap_ebops():
+            ob.zero_grad()
+            lb = model_loss(b, loss_fn(b(x, training=True)), True)
+            branched += bool(ops._OVERLAP['pending'])
+            ob.backward(lb)
+            ob.step()
+        assert not ops._OVERLAP['pending'] and not ops._OVERLAP['keep'], 'joined when the context is left'
+        assert float(la) == float(lb), f'loss step {step}'
+        for (name, pa), (_, pb) in zip(a.state_dict().items(), b.state_dict().items()):
+            assert torch.equal(pa, pb), f'{name} step {step}'
+    assert (branched == 3) == (kind != 'particle'), 'the attention and image models have enough EBOPs launches to branch, the per-particle one does not'
+
+
 @pytest.mark.parametrize('kind', ['particle', 'conv', 'mha'])
 def test_full_size_forward_matches_oracle(dev, acc64, kind):
     """The per-particle, image and attention configurations at their full sizes: one training-mode
