@@ -153,8 +153,47 @@ def _auto_name(cls_name: str) -> str:
 PREFETCH_WEIGHT_QUANTIZERS = True
 
 
+# Walking a module tree costs the host tens of microseconds per layer; a training step needs the walk three times
+# (clearing the loss lists, collecting the weight quantizers, collecting loss terms and regularised variables).  The
+# results are cached per root and keyed on this counter, which every change of a tree bumps: a layer gaining a
+# sub-module or a variable, or being built.
+TREE_EPOCH = [0]
+
+
+class TreeCache:
+    __slots__ = ('key', 'layers', 'quantized', 'regularised')
+
+
+def tree_cache(root) -> TreeCache:
+    """Lists of a module tree that a training step needs: its layers, the layers that declare kernel / bias quantizers,
+    the trainable variables with a regularizer."""
+    key = (TREE_EPOCH[0], len(root._modules))
+    c = root.__dict__.get('_hgq_tree_cache')
+    if c is None or c.key != key:
+        c = TreeCache()
+        c.key = key
+        mods = list(root.modules())
+        c.layers = [m for m in mods if isinstance(m, Layer)]
+        c.quantized = [m for m in mods if hasattr(m, '_weight_quantizer_inputs')]
+        c.regularised = [p for p in root.parameters() if getattr(p, 'regularizer', None) is not None]
+        object.__setattr__(root, '_hgq_tree_cache', c)
+    return c
+
+
 class Layer(nn.Module):
     """Keras-like layer on top of ``torch.nn.Module``."""
+
+    def __setattr__(self, name, value):
+        if isinstance(value, (nn.Module, torch.Tensor)) or name == 'built':
+            if isinstance(value, (nn.Module, nn.Parameter)) or name == 'built':
+                TREE_EPOCH[0] += 1
+            super().__setattr__(name, value)
+            return
+        d = self.__dict__
+        if name in d.get('_parameters', ()) or name in d.get('_buffers', ()) or name in d.get('_modules', ()):
+            super().__setattr__(name, value)  # e.g. `self.bias = None` for a registered parameter
+            return
+        object.__setattr__(self, name, value)  # plain per-call state (flags, shapes, pending work): no registration logic
 
     def __init__(self, name: str | None = None, trainable: bool = True, dtype: Any = None, **kwargs):
         super().__init__()
@@ -183,6 +222,7 @@ class Layer(nn.Module):
             p.regularizer = regularizer
             p.var_name = name
             self.register_parameter(attr, p)
+            TREE_EPOCH[0] += 1
             return p
         self.register_buffer(attr, value)
         return getattr(self, attr)
@@ -206,12 +246,7 @@ class Layer(nn.Module):
         return out
 
     def _clear_losses(self):
-        layers = self.__dict__.get('_hgq_layer_list')
-        n = sum(1 for _ in self.modules())
-        if layers is None or layers[0] != n:
-            layers = (n, [m for m in self.modules() if isinstance(m, Layer)])
-            object.__setattr__(self, '_hgq_layer_list', layers)
-        for m in layers[1]:
+        for m in tree_cache(self).layers:
             m.__dict__['_losses'] = []
 
     def apply_constraints(self):
@@ -303,6 +338,7 @@ class Sequential(Layer):
 
     def add(self, layer):
         self.layers.append(layer)
+        TREE_EPOCH[0] += 1
 
     def get_config(self):
         return {'name': self.name, 'layers': list(self.layers)}

@@ -33,13 +33,21 @@ def _need(cond: bool, msg: str):
         raise ValueError(msg)
 
 
+_F32 = torch.float32
+
+
 def _check_f32(name: str, t: Tensor):
+    # (the messages are built only on failure: these checks run a hundred times per training step)
+    if t.is_cuda and t.dtype is _F32 and t.is_contiguous():
+        return
     _need(t.is_cuda, f'{name} must be a GPU tensor (there is no CPU implementation), got device {t.device}')
     _need(t.dtype == torch.float32, f'{name} must be float32, got {t.dtype}')
     _need(t.is_contiguous(), f'{name} must be contiguous')
 
 
 def _check_k(name: str, t: Tensor):
+    if t.is_cuda and (t.dtype is _F32 or t.dtype is torch.uint8) and t.is_contiguous():
+        return
     _need(t.is_cuda, f'{name} must be a GPU tensor')
     _need(t.dtype in (torch.float32, torch.uint8), f'{name} must be float32 or uint8, got {t.dtype}')
     _need(t.is_contiguous(), f'{name} must be contiguous')

@@ -42,13 +42,9 @@ def quantize_together(pairs, training):
 def _plan(root):
     """The layers under ``root`` that declare kernel / bias quantizers; cached on ``root`` until its module tree changes
     (the set of modules and their built flags)."""
-    mods = list(root.modules())
-    key = (len(mods), sum(1 for m in mods if getattr(m, 'built', False)))
-    cached = getattr(root, '_hgq_prefetch_plan', None)
-    if cached is None or cached[0] != key:
-        cached = (key, [m for m in mods if hasattr(m, '_weight_quantizer_inputs')])
-        object.__setattr__(root, '_hgq_prefetch_plan', cached)
-    return cached[1]
+    from ..core import tree_cache
+
+    return tree_cache(root).quantized
 
 
 def prefetch_weight_quantizers(root) -> int:

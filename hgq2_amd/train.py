@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from . import ops
+from .core import Layer, tree_cache
 from .regularizers import MonoL1
 
 
@@ -19,9 +20,10 @@ def model_loss(model, base_loss, fold_regularizers: bool = False):
     the MonoL1 terms are left out of the autograd graph: their constant gradient ``l1`` is added by
     :class:`SGD` inside the update kernel instead (same update, one launch less per variable)."""
     terms = [base_loss]
-    for m in model.modules():
+    cache = tree_cache(model) if isinstance(model, Layer) else None
+    for m in (cache.layers if cache is not None else model.modules()):
         terms.extend(getattr(m, '_losses', ()))
-    for p in model.parameters():
+    for p in (cache.regularised if cache is not None else model.parameters()):
         r = getattr(p, 'regularizer', None)
         if r is None or not p.requires_grad:  # Keras regularises trainable variables only
             continue
