@@ -961,9 +961,34 @@ extern "C" int64_t hgq_quantize_bwd_workspace(int64_t n, int64_t bw_size, int64_
     return sliced_bwd_geometry(n, bw_size, bw_inner, vec, TX, gx, gy, rows_per_wg) ? gy * 2 * bw_size : 0;
 }
 
+extern "C" int64_t hgq_quantize_bwd_slice_count(int64_t n, int64_t bw_size, int64_t bw_inner) {
+    bool vec;
+    int TX;
+    int64_t gx, gy, rows_per_wg;
+    return sliced_bwd_geometry(n, bw_size, bw_inner, vec, TX, gx, gy, rows_per_wg) ? gy : 0;
+}
+
+static int quantize_bwd_sliced_impl(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx,
+                                    float *di, float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner,
+                                    int mode, void *stream, bool reduce);
+
 extern "C" int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx,
                                        float *di, float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner,
                                        int mode, void *stream) {
+    return quantize_bwd_sliced_impl(dy, x, k, i, fb, dx, di, dfb, workspace, n, bw_size, bw_inner, mode, stream, true);
+}
+
+extern "C" int hgq_quantize_bwd_slices(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx,
+                                       int want_di, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode,
+                                       void *stream) {
+    // the kernel takes the two gradient pointers only as "wanted" flags when it writes slices
+    return quantize_bwd_sliced_impl(dy, x, k, i, fb, dx, want_di ? workspace : nullptr, workspace, workspace, n, bw_size, bw_inner, mode,
+                                    stream, false);
+}
+
+static int quantize_bwd_sliced_impl(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx,
+                                    float *di, float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner,
+                                    int mode, void *stream, bool reduce) {
     hipStream_t s = (hipStream_t)stream;
     bool vec;
     int TX;
@@ -984,7 +1009,7 @@ extern "C" int hgq_quantize_bwd_sliced(const float *dy, const float *x, const vo
             hipLaunchKernelGGL((quant_bwd_cols<RM, OM, 1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, rows, M, TX, rows_per_wg, mode, workspace);
     });
     int rc = check_launch("hgq_quantize_bwd_sliced");
-    if (rc) return rc;
+    if (rc || !reduce) return rc;
     return reduce_parts(workspace, (int)gy, di ? 2 * M : M, dfb, M, di, di ? M : 0, nullptr, 0, s);
 }
 

@@ -118,6 +118,35 @@ def quantize_bwd(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: 
     return dx, di, dfb
 
 
+@torch.library.custom_op('hgq::quantize_bwd_slices', mutates_args=())
+def quantize_bwd_slices(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, need_dx: bool,
+                        need_di: bool) -> tuple[Tensor, Tensor]:
+    """The data gradient and the slices ``[n_slices, bw (fb) + bw (i, with need_di)]`` of the bit-width gradients, left for
+    a joint reduction; only for shapes ``quantize_bwd_slices_supported`` accepts."""
+    _check_f32('dy', dy), _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
+    _need(dy.numel() == x.numel(), 'dy and x differ in size')
+    lib = _lib.load()
+    n_sl = lib.hgq_quantize_bwd_slice_count(x.numel(), i.numel(), bw_inner)
+    _need(n_sl > 0, 'shape outside the sliced backward')
+    dx = torch.empty_like(x) if need_dx else x.new_empty(0)
+    ws = torch.empty((n_sl, i.numel() * (2 if need_di else 1)), dtype=torch.float32, device=x.device)
+    rc = lib.hgq_quantize_bwd_slices(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), int(need_di), _ptr(ws), x.numel(), i.numel(),
+                                     bw_inner, _kmode(mode, k), _stream())
+    _lib.check(rc, 'hgq_quantize_bwd_slices')
+    return dx, ws
+
+
+@quantize_bwd_slices.register_fake
+def _(dy, x, k, i, fb, mode, bw_inner, need_dx, need_di):
+    n_sl = max(int(_lib.load().hgq_quantize_bwd_slice_count(x.numel(), i.numel(), bw_inner)), 1)
+    return (torch.empty_like(x) if need_dx else x.new_empty(0), x.new_empty((n_sl, i.numel() * (2 if need_di else 1))))
+
+
+def quantize_bwd_slices_supported(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, bw_inner: int) -> bool:
+    return (x.numel() > 0 and all(t.data_ptr() % 16 == 0 for t in (dy, x, k, i, fb))
+            and _lib.load().hgq_quantize_bwd_slice_count(x.numel(), i.numel(), bw_inner) > 0)
+
+
 @quantize_bwd.register_fake
 def _(dy, x, k, i, fb, mode, bw_inner, need_dx, need_di):
     return (torch.empty_like(x) if need_dx else x.new_empty(0), torch.empty_like(i) if need_di else i.new_empty(0),
@@ -1338,6 +1367,7 @@ class _Quantize(torch.autograd.Function):
         y, amax, neg = quantize_fwd(x, k, i, fb, mode, bw_inner, track)
         ctx.save_for_backward(x, k, i, fb)
         ctx.mode, ctx.bw_inner = mode, bw_inner
+        ctx.owners = (_owner(i), _owner(fb))
         ctx.mark_non_differentiable(amax, neg)
         ctx.set_materialize_grads(False)
         return y, amax, neg
@@ -1355,6 +1385,18 @@ class _Quantize(torch.autograd.Function):
         wrap = ((ctx.mode >> 4) & 0xf) == _lib.WRAP
         need_dx = ctx.needs_input_grad[0] and not wrap
         need_di = ctx.needs_input_grad[2] and (not wrap or bool(ctx.mode & _lib.MODE_KBI))
+        o_i, o_fb = ctx.owners
+        if (_SINK['open'] and ctx.needs_input_grad[3] and _can_route(o_fb, fb.numel()) and (not need_di or _can_route(o_i, i.numel()))
+                and (need_di or not ctx.needs_input_grad[2]) and quantize_bwd_slices_supported(gy, x, k, i, fb, ctx.bw_inner)):
+            # the bit-width gradients go to the optimizer and nowhere else: their slices join the pass's one reduction launch
+            dx, ws = quantize_bwd_slices(gy, x, k, i, fb, ctx.mode, ctx.bw_inner, need_dx, need_di)
+            dfb, di = torch.empty_like(fb), (torch.empty_like(i) if need_di else None)
+            e = fb.new_empty(0)
+            _PENDING_REDUCE.append((ws, (dfb.view(-1), di.view(-1) if need_di else e, e), (False, not need_di, True)))
+            _route(o_fb, dfb)
+            if need_di:
+                _route(o_i, di)
+            return (gy if wrap else dx) if ctx.needs_input_grad[0] else None, None, None, None, None, None, None
         dx, di, dfb = quantize_bwd(gy, x, k, i, fb, ctx.mode, ctx.bw_inner, need_dx, need_di)
         if ctx.needs_input_grad[0] and wrap:
             dx = gy

@@ -109,6 +109,14 @@ int hgq_quantize_fwd_sliced(const float *x, const void *k, const float *i, const
 int64_t hgq_quantize_bwd_workspace(int64_t n, int64_t bw_size, int64_t bw_inner);
 int hgq_quantize_bwd_sliced(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
                             float *dfb, float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
+/*
+ * The first launch of hgq_quantize_bwd_sliced alone: `workspace` keeps hgq_quantize_bwd_slice_count() slices, each
+ * [dfb (bw_size) | di (bw_size, only with want_di)], for a caller that adds the slice sets of several quantizers of a
+ * backward pass in one launch (hgq_reduce_slices_multi) - their sums are first read by the optimizer.
+ */
+int64_t hgq_quantize_bwd_slice_count(int64_t n, int64_t bw_size, int64_t bw_inner);
+int hgq_quantize_bwd_slices(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, int want_di,
+                            float *workspace, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
 
 /*
  * Stochastic rounding: the training-mode forward and surrogate backward of round modes S_RND / S_RND_CONV

@@ -478,8 +478,10 @@ def test_gradient_sink_gives_the_autograd_update(dev, kind, monkeypatch):
                 assert torch.equal(pa, pb), f'{name} step {step}'
             else:
                 assert torch.allclose(pa, pb, rtol=1e-6, atol=1e-9), f'{name} step {step}: {float((pa - pb).abs().max()):.3e}'
-    if kind in ('mlp', 'mha'):  # the dense backward of every layer left its slices for one joint reduction per step
-        assert joined == [4, 4], joined
+    if kind in ('mlp', 'mha'):
+        # the dense backward of every layer left its slices for one joint reduction per step; in the attention model the
+        # output quantizers of the three input projections (bit-widths shared along the batch) add theirs
+        assert joined == ([4, 4] if kind == 'mlp' else [7, 7]), joined
 
 
 def test_dense_backward_in_two_halves_gives_the_same_bits(dev):
