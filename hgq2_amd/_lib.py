@@ -76,6 +76,7 @@ SIGNATURES = {
     'hgq_quantize_bwd_workspace': (c_int64, [c_int64, c_int64, c_int64]),
     'hgq_quantize_bwd_sliced': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_bwd_slice_count': (c_int64, [c_int64, c_int64, c_int64]),
+    'hgq_dense_use_bf16_parts': (c_int, [c_int]),
     'hgq_quantize_bwd_slices': (c_int, [c_void_p] * 6 + [c_int, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_conv2d_ebops_q': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_dense_ebops_multi': (c_int, [c_void_p, c_int, c_void_p]),

@@ -495,6 +495,234 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// The same contraction on the bf16 matrix cores, exactly.  An fp32 number is the sum of three numbers
+// of eight significant bits each - its leading bits, the leading bits of what is left, and the rest -
+// and each of them is a bf16 number (same exponent range as fp32).  A product of two such parts is
+// exact in fp32, so  x W = sum over part pairs  x_p W_q  accumulated in fp32 is the contraction itself,
+// with only the accumulation rounded, as in the fp32 matrix instruction.  v_mfma_f32_32x32x16_bf16 does
+// sixteen times the work of v_mfma_f32_32x32x2_f32 per cycle, so even all nine pairs cost about half of
+// the fp32 chain - and quantized operands rarely need more than one part (eight bits) or two (sixteen):
+// the staging threads note which parts of a tile are non-zero, a wavefront notes it for its kernel
+// columns, and only those pairs are issued.
+// Operand layout of the 32x32x16 instruction (64 lanes, eight bf16 per lane and operand):
+// A[i][k]: i = lane % 32, k = 8 (lane / 32) + e;  B[k][j]: k = 8 (lane / 32) + e, j = lane % 32;  D as for 32x32x2.
+// ------------------------------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+#define BF_LD 72  // bf16 per LDS row: rows 144 bytes apart keep the 128-bit operand reads of 16 consecutive rows on different banks
+
+// the three parts of v as fp32 bit patterns whose low halves are zero (a part that is not needed is zero)
+__device__ __forceinline__ void bf16_parts(float v, uint32_t &h, uint32_t &m, uint32_t &l) {
+    h = __float_as_uint(v) & 0xffff0000u;
+    const float r1 = __fsub_rn(v, __uint_as_float(h));  // exact: the low 16 bits of the significand
+    m = __float_as_uint(r1) & 0xffff0000u;
+    l = __float_as_uint(__fsub_rn(r1, __uint_as_float(m)));  // exact, at most eight significant bits
+}
+// two parts (bit patterns with zero low halves) as one register of two bf16: `a` first
+__device__ __forceinline__ uint32_t bf16_pair(uint32_t a, uint32_t b) { return (a >> 16) | b; }
+
+__device__ __forceinline__ floatx16 mfma_bf16(const u32x4_t &a, const u32x4_t &b, floatx16 acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+}
+
+// NS = steps of sixteen k that cover K.
+template <int RM, bool QUANT, int NS>
+__global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
+                                                              int P, const float *__restrict__ qw,
+                                                              const float *__restrict__ qb, float *__restrict__ y,
+                                                              uint32_t *amax_part, int64_t rows, int K, int N, int act,
+                                                              int mode) {
+    // [buffer][part][row][k]; row FAST_BM: sink of the idle staging slots
+    __shared__ __attribute__((aligned(16))) uint16_t xp[2][3][FAST_BM + 1][BF_LD];
+    __shared__ __attribute__((aligned(16))) float ys[FAST_BM][FAST_XLD];
+    __shared__ uint32_t need[2];  // bit 0 / 1: the staged tile has a non-zero second / third part
+    const Mode m(mode);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rh = wave & 1, cb = wave >> 1;
+    const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
+    for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;  // columns >= K stay zero
+    if (tid < 2) need[tid] = 0u;
+    const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
+    // this lane's kernel column in parts: wp[part][step] holds k = 16 step + 8 kq + 0 .. 7
+    u32x4_t wp[3][NS];
+    uint32_t wnz1 = 0u, wnz2 = 0u;
+    {
+        float wv[NS][8];
+#pragma unroll
+        for (int st = 0; st < NS; ++st)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int k = 16 * st + 8 * kq + e;
+                wv[st][e] = (k < K && bcol < N) ? qw[(int64_t)k * N + bcol] : 0.f;
+            }
+#pragma unroll
+        for (int st = 0; st < NS; ++st)
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                uint32_t h0, m0, l0, h1, m1, l1;
+                bf16_parts(wv[st][e], h0, m0, l0), bf16_parts(wv[st][e + 1], h1, m1, l1);
+                wp[0][st][e >> 1] = bf16_pair(h0, h1), wp[1][st][e >> 1] = bf16_pair(m0, m1), wp[2][st][e >> 1] = bf16_pair(l0, l1);
+                wnz1 |= m0 | m1, wnz2 |= l0 | l1;
+            }
+    }
+    // parts of the kernel this wavefront has to multiply by (uniform over the wavefront)
+    const int PW = __any(wnz2 != 0u) ? 3 : (__any(wnz1 != 0u) ? 2 : 1);
+    const float bias = (qb && bcol < N) ? qb[bcol] : 0.f;
+    FastMap mp, mo;
+    mp.init(K);
+    const bool vec_out = (N & 3) == 0 && ((uintptr_t)y & 15u) == 0;
+    mo.init(vec_out ? N : 4);
+    int fi[FAST_NJ][4], tix[FAST_NJ];
+    uint32_t amx[FAST_NJ][4];
+    fast_frac_bits<QUANT>(f_in, P, K, mp, m.round_params, fi, tix);
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) amx[j][e] = 0;
+    f32x4_t raw[FAST_NJ];
+    uint32_t xoff[FAST_NJ];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) xoff[j] = mp.on[j] ? (uint32_t)(mp.row[j] * K + mp.col[j]) * 4u : BUF_OOB;
+    auto load_tile = [&](int64_t t) {
+        const int64_t r0 = t * FAST_BM, left = rows - r0;
+        const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K, (left < FAST_BM ? left : FAST_BM) * K * 4);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) raw[j] = buf_ld4(rs, xoff[j]);
+    };
+    int64_t tile = blockIdx.x;
+    if (tile < n_tiles) load_tile(tile);
+    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    int buf = 0;
+    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
+        float v[FAST_NJ][4];
+        uint32_t low = 0u;
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[j][e] = raw[j][e];
+                if (QUANT) {
+                    v[j][e] = ldexpf(round_scaled<RM>(ldexpf(v[j][e], fi[j][e])), -fi[j][e]);
+                    amx[j][e] = max(amx[j][e], abs_bits(v[j][e]));
+                }
+                low |= __float_as_uint(v[j][e]);
+            }
+            // leading parts: the high halves of the four words
+            const int r = mp.on[j] ? mp.row[j] : FAST_BM;
+            *(uint2 *)&xp[buf][0][r][mp.col[j]] =
+                make_uint2(__builtin_amdgcn_perm(__float_as_uint(v[j][1]), __float_as_uint(v[j][0]), 0x07060302u),
+                           __builtin_amdgcn_perm(__float_as_uint(v[j][3]), __float_as_uint(v[j][2]), 0x07060302u));
+        }
+        // the other parts only where a wavefront staged a value of more than eight significant bits (uniform branch);
+        // all three planes are written either way: every wavefront reads every staging wavefront's rows
+        if (__any((low & 0xffffu) != 0u)) {
+            uint32_t nz2 = 0u;
+#pragma unroll
+            for (int j = 0; j < FAST_NJ; ++j) {
+                uint32_t h[4], md[4], lo[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    bf16_parts(v[j][e], h[e], md[e], lo[e]);
+                    nz2 |= lo[e];
+                }
+                const int r = mp.on[j] ? mp.row[j] : FAST_BM;
+                *(uint2 *)&xp[buf][1][r][mp.col[j]] = make_uint2(bf16_pair(md[0], md[1]), bf16_pair(md[2], md[3]));
+                *(uint2 *)&xp[buf][2][r][mp.col[j]] = make_uint2(bf16_pair(lo[0], lo[1]), bf16_pair(lo[2], lo[3]));
+            }
+            const bool third = __any(nz2 != 0u);
+            if (lane == 0) atomicOr(&need[buf], third ? 3u : 1u);
+        } else {
+#pragma unroll
+            for (int j = 0; j < FAST_NJ; ++j) {
+                const int r = mp.on[j] ? mp.row[j] : FAST_BM;
+                *(uint2 *)&xp[buf][1][r][mp.col[j]] = make_uint2(0u, 0u);
+                *(uint2 *)&xp[buf][2][r][mp.col[j]] = make_uint2(0u, 0u);
+            }
+        }
+        __syncthreads();
+        if (tid == 0) need[buf ^ 1] = 0u;  // read by every wavefront before it reached the barrier above; written again after the next one
+        const int64_t next = tile + gridDim.x;
+        if (next < n_tiles) load_tile(next);
+        floatx16 acc = {0};
+        if (cb * 32 < N) {
+            const uint32_t nd = need[buf];
+            const int PX = (nd & 2u) ? 3 : ((nd & 1u) ? 2 : 1);
+            // leading parts first; the branches are uniform over the wavefront
+#pragma unroll
+            for (int px = 0; px < 3; ++px) {
+                if (px < PX) {
+                    u32x4_t a[NS];
+#pragma unroll
+                    for (int st = 0; st < NS; ++st) a[st] = *(const u32x4_t *)&xp[buf][px][arow][16 * st + 8 * kq];
+#pragma unroll
+                    for (int pw = 0; pw < 3; ++pw) {
+                        if (pw < PW) {
+#pragma unroll
+                            for (int st = 0; st < NS; ++st) acc = mfma_bf16(a[st], wp[pw][st], acc);
+                        }
+                    }
+                }
+            }
+        }
+        const int64_t r0 = tile * FAST_BM;
+        if (vec_out) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = acc[r] + bias;
+                if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                ys[rh * 32 + acc_row(r, lane)][bcol] = v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < FAST_NJ; ++j) {
+                const int64_t gr = r0 + mo.row[j];
+                if (mo.on[j] && gr < rows) {
+                    *(f32x4_t *)(y + gr * N + mo.col[j]) = *(const f32x4_t *)&ys[mo.row[j]][mo.col[j]];
+                }
+            }
+        } else {
+            if (bcol < N) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t gr = r0 + rh * 32 + acc_row(r, lane);
+                    if (gr < rows) {
+                        float v = acc[r] + bias;
+                        if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                        y[gr * N + bcol] = v;
+                    }
+                }
+            }
+            __syncthreads();  // the flags of the other buffer are cleared before they are set again
+        }
+    }
+    if (QUANT && amax_part && P == FAST_BM && ((uintptr_t)amax_part & 15u) == 0) {
+        uint32_t *my = amax_part + (int64_t)blockIdx.x * (P * K);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j)
+            if (mp.on[j]) {
+                uint4 v;
+                v.x = amx[j][0], v.y = amx[j][1], v.z = amx[j][2], v.w = amx[j][3];
+                *(uint4 *)(my + tix[j]) = v;
+            }
+    } else if (QUANT && amax_part) {
+        const int PK = P * K;
+        uint32_t *tab = (uint32_t *)&ys[0][0];
+        __syncthreads();
+        for (int t = tid; t < PK; t += 256) tab[t] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j)
+            if (mp.on[j])
+#pragma unroll
+                for (int e = 0; e < 4; ++e) atomicMax(&tab[tix[j] + e], amx[j][e]);
+        __syncthreads();
+        uint32_t *my = amax_part + (int64_t)blockIdx.x * PK;
+        for (int t = tid; t < PK; t += 256) my[t] = tab[t];
+    }
+}
+
 // Column statistics of the contraction without writing it: sum_r z and sum_r z^2 of z = x W per
 // output column, for the batch statistics of QEinsumDenseBatchnorm.  Same tiling as the forward
 // above; a lane keeps the sums of its column over its 16 accumulator rows in registers across
@@ -975,6 +1203,14 @@ static inline int row_parts(int64_t rows, int bm) {
 
 using namespace hgq;
 
+// 1: the streaming dense kernels contract on the bf16 matrix cores by exact splitting; 0: on the fp32 ones
+static int g_dense_bf16 = 1;
+extern "C" int hgq_dense_use_bf16_parts(int on) {
+    const int was = g_dense_bf16;
+    if (on >= 0) g_dense_bf16 = on ? 1 : 0;
+    return was;
+}
+
 extern "C" int hgq_qdense_fwd_parts(int64_t rows) { return rows > 0 ? row_parts(rows, FWD_BM) : 1; }
 
 extern "C" int64_t hgq_qdense_bwd_workspace(int64_t rows, int K, int N, int64_t bw_rows) {
@@ -1004,6 +1240,21 @@ extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_i
     if (fast) {
         const dim3 fgrid((unsigned)row_parts(rows, FWD_BM));
         const int P = quant ? (int)bw_rows : 1;
+#define HGQ_FWD_BF16(NSV) \
+    do { \
+        if (!quant) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, false, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, (uint32_t *)nullptr, rows, K, N, act, mode); \
+        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode); \
+        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode); \
+        else hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND_CONV, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode); \
+    } while (0)
+        if (g_dense_bf16) {
+            if (K <= 16) HGQ_FWD_BF16(1);
+            else if (K <= 32) HGQ_FWD_BF16(2);
+            else if (K <= 48) HGQ_FWD_BF16(3);
+            else HGQ_FWD_BF16(4);
+            return check_launch("hgq_qdense_fwd");
+        }
+#undef HGQ_FWD_BF16
 #define HGQ_FWD_FAST(NS4V) \
     do { \
         if (!quant) hipLaunchKernelGGL((qdense_fwd_fast_kernel<HGQ_TRN, false, NS4V>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, (uint32_t *)nullptr, rows, K, N, act, mode); \

@@ -241,6 +241,15 @@ int hgq_wrap_track_i_multi(const hgq_track_item *items, int count, void *stream)
  *   act is HGQ_ACT_*.
  */
 int hgq_qdense_fwd_parts(int64_t rows);
+/*
+ * The streaming kernels (K, N <= 64) contract on the bf16 matrix cores: every fp32 operand is split exactly into up to
+ * three bf16 parts (8 + 8 + 8 significant bits), the products of parts are exact in fp32 and are accumulated in fp32,
+ * and only the non-zero parts are multiplied - quantized operands of up to 8 bits need one part, up to 16 bits two.
+ * Same values as the fp32 matrix instruction up to the order of the fp32 accumulation.  `on` = 0 selects the fp32
+ * instruction instead, 1 the bf16 parts (default), a negative value changes nothing; returns the previous setting.
+ * Process-wide, not synchronised with launches in flight on other threads.
+ */
+int hgq_dense_use_bf16_parts(int on);
 int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_in, const float *f_in, int64_t bw_rows,
                    const float *qw, const float *qb, float *y, uint32_t *amax_part, int64_t rows, int K, int N,
                    int act, int mode, void *stream);
