@@ -508,22 +508,108 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
 // Operand layout of the 32x32x16 instruction (64 lanes, eight bf16 per lane and operand):
 // A[i][k]: i = lane % 32, k = 8 (lane / 32) + e;  B[k][j]: k = 8 (lane / 32) + e, j = lane % 32;  D as for 32x32x2.
 // ------------------------------------------------------------------------------------------
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 #define BF_LD 72  // bf16 per LDS row: rows 144 bytes apart keep the 128-bit operand reads of 16 consecutive rows on different banks
 
-// the three parts of v as fp32 bit patterns whose low halves are zero (a part that is not needed is zero)
-__device__ __forceinline__ void bf16_parts(float v, uint32_t &h, uint32_t &m, uint32_t &l) {
-    h = __float_as_uint(v) & 0xffff0000u;
-    const float r1 = __fsub_rn(v, __uint_as_float(h));  // exact: the low 16 bits of the significand
-    m = __float_as_uint(r1) & 0xffff0000u;
-    l = __float_as_uint(__fsub_rn(r1, __uint_as_float(m)));  // exact, at most eight significant bits
-}
-// two parts (bit patterns with zero low halves) as one register of two bf16: `a` first
-__device__ __forceinline__ uint32_t bf16_pair(uint32_t a, uint32_t b) { return (a >> 16) | b; }
+typedef uint16_t (*bf16_planes_t)[FAST_BM + 1][BF_LD];  // [part][row][k] of one staged tile
 
-__device__ __forceinline__ floatx16 mfma_bf16(const u32x4_t &a, const u32x4_t &b, floatx16 acc) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+// Stages the four 128-bit slots of a thread (quantized first when QUANT) as bf16 parts and records in `need` which of
+// the second / third parts of the tile are non-zero (bit 0 / 1).  TRACK: the abs-max of the staged values.
+template <int RM, bool QUANT, bool TRACK>
+__device__ __forceinline__ void bf16_stage(const f32x4_t (&raw)[FAST_NJ], const int (&fi)[FAST_NJ][4], const FastMap &mp, bf16_planes_t xp,
+                                           uint32_t *need, uint32_t (&amx)[FAST_NJ][4], float (*dlt)[4] = nullptr) {
+    float v[FAST_NJ][4];
+    uint32_t low = 0u;
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[j][e] = raw[j][e];
+            if (QUANT) {
+                v[j][e] = ldexpf(round_scaled<RM>(ldexpf(v[j][e], fi[j][e])), -fi[j][e]);
+                if (TRACK) amx[j][e] = max(amx[j][e], abs_bits(v[j][e]));
+            }
+            if (dlt) dlt[j][e] = v[j][e] - raw[j][e];
+            low |= __float_as_uint(v[j][e]);
+        }
+        // leading parts: the high halves of the four words
+        const int r = mp.on[j] ? mp.row[j] : FAST_BM;
+        *(uint2 *)&xp[0][r][mp.col[j]] = make_uint2(__builtin_amdgcn_perm(__float_as_uint(v[j][1]), __float_as_uint(v[j][0]), 0x07060302u),
+                                                   __builtin_amdgcn_perm(__float_as_uint(v[j][3]), __float_as_uint(v[j][2]), 0x07060302u));
+    }
+    // the other parts only where a wavefront staged a value of more than eight significant bits (uniform branch);
+    // all three planes are written either way: every wavefront reads every staging wavefront's rows
+    if (__any((low & 0xffffu) != 0u)) {
+        uint32_t nz2 = 0u;
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            uint32_t h[4], md[4], lo[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                bf16_parts(v[j][e], h[e], md[e], lo[e]);
+                nz2 |= lo[e];
+            }
+            const int r = mp.on[j] ? mp.row[j] : FAST_BM;
+            *(uint2 *)&xp[1][r][mp.col[j]] = make_uint2(bf16_pair(md[0], md[1]), bf16_pair(md[2], md[3]));
+            *(uint2 *)&xp[2][r][mp.col[j]] = make_uint2(bf16_pair(lo[0], lo[1]), bf16_pair(lo[2], lo[3]));
+        }
+        const bool third = __any(nz2 != 0u);
+        if ((threadIdx.x & 63) == 0) atomicOr(need, third ? 3u : 1u);
+    } else {
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            const int r = mp.on[j] ? mp.row[j] : FAST_BM;
+            *(uint2 *)&xp[1][r][mp.col[j]] = make_uint2(0u, 0u);
+            *(uint2 *)&xp[2][r][mp.col[j]] = make_uint2(0u, 0u);
+        }
+    }
+}
+
+// A lane's kernel column (B operand of x W) in parts: wp[part][step] holds k = 16 step + 8 kq + 0 .. 7 of column `col`;
+// returns the number of parts the wavefront has to multiply by.
+template <int NS>
+__device__ __forceinline__ int bf16_kernel_column(const float *__restrict__ qw, int K, int N, int col, int kq, u32x4_t (&wp)[3][NS]) {
+    float wv[NS][8];
+#pragma unroll
+    for (int st = 0; st < NS; ++st)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int k = 16 * st + 8 * kq + e;
+            wv[st][e] = (k < K && col < N) ? qw[(int64_t)k * N + col] : 0.f;
+        }
+    uint32_t wnz1 = 0u, wnz2 = 0u;
+#pragma unroll
+    for (int st = 0; st < NS; ++st)
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            uint32_t h0, m0, l0, h1, m1, l1;
+            bf16_parts(wv[st][e], h0, m0, l0), bf16_parts(wv[st][e + 1], h1, m1, l1);
+            wp[0][st][e >> 1] = bf16_pair(h0, h1), wp[1][st][e >> 1] = bf16_pair(m0, m1), wp[2][st][e >> 1] = bf16_pair(l0, l1);
+            wnz1 |= m0 | m1, wnz2 |= l0 | l1;
+        }
+    return __any(wnz2 != 0u) ? 3 : (__any(wnz1 != 0u) ? 2 : 1);
+}
+
+// acc += x W for this wavefront's 32 x 32 block: row `arow` of the staged tile against the lane's kernel column, over the
+// parts that are non-zero on either side, leading parts first (uniform branches).
+template <int NS>
+__device__ __forceinline__ floatx16 bf16_chain(floatx16 acc, bf16_planes_t xp, int arow, int kq, uint32_t nd, const u32x4_t (&wp)[3][NS], int PW) {
+    const int PX = (nd & 2u) ? 3 : ((nd & 1u) ? 2 : 1);
+#pragma unroll
+    for (int px = 0; px < 3; ++px) {
+        if (px < PX) {
+            u32x4_t a[NS];
+#pragma unroll
+            for (int st = 0; st < NS; ++st) a[st] = *(const u32x4_t *)&xp[px][arow][16 * st + 8 * kq];
+#pragma unroll
+            for (int pw = 0; pw < 3; ++pw) {
+                if (pw < PW) {
+#pragma unroll
+                    for (int st = 0; st < NS; ++st) acc = mfma_bf16(a[st], wp[pw][st], acc);
+                }
+            }
+        }
+    }
+    return acc;
 }
 
 // NS = steps of sixteen k that cover K.
@@ -536,38 +622,18 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     // [buffer][part][row][k]; row FAST_BM: sink of the idle staging slots
     __shared__ __attribute__((aligned(16))) uint16_t xp[2][3][FAST_BM + 1][BF_LD];
     __shared__ __attribute__((aligned(16))) float ys[FAST_BM][FAST_XLD];
-    __shared__ uint32_t need[2];  // bit 0 / 1: the staged tile has a non-zero second / third part
+    // bit 0 / 1: the staged tile has a non-zero second / third part.  Three slots in rotation: the slot of the tile after
+    // next is cleared behind this tile's barrier - its last readers passed that barrier, its next writers come after the next one
+    __shared__ uint32_t need[3];
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rh = wave & 1, cb = wave >> 1;
     const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
     for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;  // columns >= K stay zero
-    if (tid < 2) need[tid] = 0u;
+    if (tid < 3) need[tid] = 0u;
     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
-    // this lane's kernel column in parts: wp[part][step] holds k = 16 step + 8 kq + 0 .. 7
     u32x4_t wp[3][NS];
-    uint32_t wnz1 = 0u, wnz2 = 0u;
-    {
-        float wv[NS][8];
-#pragma unroll
-        for (int st = 0; st < NS; ++st)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int k = 16 * st + 8 * kq + e;
-                wv[st][e] = (k < K && bcol < N) ? qw[(int64_t)k * N + bcol] : 0.f;
-            }
-#pragma unroll
-        for (int st = 0; st < NS; ++st)
-#pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                uint32_t h0, m0, l0, h1, m1, l1;
-                bf16_parts(wv[st][e], h0, m0, l0), bf16_parts(wv[st][e + 1], h1, m1, l1);
-                wp[0][st][e >> 1] = bf16_pair(h0, h1), wp[1][st][e >> 1] = bf16_pair(m0, m1), wp[2][st][e >> 1] = bf16_pair(l0, l1);
-                wnz1 |= m0 | m1, wnz2 |= l0 | l1;
-            }
-    }
-    // parts of the kernel this wavefront has to multiply by (uniform over the wavefront)
-    const int PW = __any(wnz2 != 0u) ? 3 : (__any(wnz1 != 0u) ? 2 : 1);
+    const int PW = bf16_kernel_column<NS>(qw, K, N, bcol, kq, wp);  // parts of the kernel this wavefront multiplies by
     const float bias = (qb && bcol < N) ? qb[bcol] : 0.f;
     FastMap mp, mo;
     mp.init(K);
@@ -594,77 +660,16 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     if (tile < n_tiles) load_tile(tile);
     __syncthreads();
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    int buf = 0;
-    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
-        float v[FAST_NJ][4];
-        uint32_t low = 0u;
-#pragma unroll
-        for (int j = 0; j < FAST_NJ; ++j) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[j][e] = raw[j][e];
-                if (QUANT) {
-                    v[j][e] = ldexpf(round_scaled<RM>(ldexpf(v[j][e], fi[j][e])), -fi[j][e]);
-                    amx[j][e] = max(amx[j][e], abs_bits(v[j][e]));
-                }
-                low |= __float_as_uint(v[j][e]);
-            }
-            // leading parts: the high halves of the four words
-            const int r = mp.on[j] ? mp.row[j] : FAST_BM;
-            *(uint2 *)&xp[buf][0][r][mp.col[j]] =
-                make_uint2(__builtin_amdgcn_perm(__float_as_uint(v[j][1]), __float_as_uint(v[j][0]), 0x07060302u),
-                           __builtin_amdgcn_perm(__float_as_uint(v[j][3]), __float_as_uint(v[j][2]), 0x07060302u));
-        }
-        // the other parts only where a wavefront staged a value of more than eight significant bits (uniform branch);
-        // all three planes are written either way: every wavefront reads every staging wavefront's rows
-        if (__any((low & 0xffffu) != 0u)) {
-            uint32_t nz2 = 0u;
-#pragma unroll
-            for (int j = 0; j < FAST_NJ; ++j) {
-                uint32_t h[4], md[4], lo[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    bf16_parts(v[j][e], h[e], md[e], lo[e]);
-                    nz2 |= lo[e];
-                }
-                const int r = mp.on[j] ? mp.row[j] : FAST_BM;
-                *(uint2 *)&xp[buf][1][r][mp.col[j]] = make_uint2(bf16_pair(md[0], md[1]), bf16_pair(md[2], md[3]));
-                *(uint2 *)&xp[buf][2][r][mp.col[j]] = make_uint2(bf16_pair(lo[0], lo[1]), bf16_pair(lo[2], lo[3]));
-            }
-            const bool third = __any(nz2 != 0u);
-            if (lane == 0) atomicOr(&need[buf], third ? 3u : 1u);
-        } else {
-#pragma unroll
-            for (int j = 0; j < FAST_NJ; ++j) {
-                const int r = mp.on[j] ? mp.row[j] : FAST_BM;
-                *(uint2 *)&xp[buf][1][r][mp.col[j]] = make_uint2(0u, 0u);
-                *(uint2 *)&xp[buf][2][r][mp.col[j]] = make_uint2(0u, 0u);
-            }
-        }
+    int buf = 0, slot = 0;
+    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1, slot = slot == 2 ? 0 : slot + 1) {
+        bf16_stage<RM, QUANT, QUANT>(raw, fi, mp, xp[buf], &need[slot], amx);
         __syncthreads();
-        if (tid == 0) need[buf ^ 1] = 0u;  // read by every wavefront before it reached the barrier above; written again after the next one
+        if (tid == 0) need[slot == 0 ? 2 : slot - 1] = 0u;  // (slot + 2) % 3
         const int64_t next = tile + gridDim.x;
         if (next < n_tiles) load_tile(next);
         floatx16 acc = {0};
         if (cb * 32 < N) {
-            const uint32_t nd = need[buf];
-            const int PX = (nd & 2u) ? 3 : ((nd & 1u) ? 2 : 1);
-            // leading parts first; the branches are uniform over the wavefront
-#pragma unroll
-            for (int px = 0; px < 3; ++px) {
-                if (px < PX) {
-                    u32x4_t a[NS];
-#pragma unroll
-                    for (int st = 0; st < NS; ++st) a[st] = *(const u32x4_t *)&xp[buf][px][arow][16 * st + 8 * kq];
-#pragma unroll
-                    for (int pw = 0; pw < 3; ++pw) {
-                        if (pw < PW) {
-#pragma unroll
-                            for (int st = 0; st < NS; ++st) acc = mfma_bf16(a[st], wp[pw][st], acc);
-                        }
-                    }
-                }
-            }
+            acc = bf16_chain<NS>(acc, xp[buf], arow, kq, need[slot], wp, PW);
         }
         const int64_t r0 = tile * FAST_BM;
         if (vec_out) {
@@ -694,7 +699,6 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
                     }
                 }
             }
-            __syncthreads();  // the flags of the other buffer are cleared before they are set again
         }
     }
     if (QUANT && amax_part && P == FAST_BM && ((uintptr_t)amax_part & 15u) == 0) {
@@ -808,6 +812,69 @@ __global__ __launch_bounds__(256, 2) void dense_moments_fast_kernel(const float 
     }
 }
 
+// The column statistics on the bf16 matrix cores (exact splitting, see qdense_fwd_bf16_kernel).
+template <int RM, bool QUANT, int NS>
+__global__ __launch_bounds__(256, 2) void dense_moments_bf16_kernel(const float *__restrict__ x, const float *__restrict__ f_in, int P,
+                                                                   const float *__restrict__ w, float *__restrict__ part,
+                                                                   int64_t rows, int K, int N, int mode) {
+    __shared__ __attribute__((aligned(16))) uint16_t xp[2][3][FAST_BM + 1][BF_LD];
+    __shared__ float red[4][64][2];
+    __shared__ uint32_t need[3];  // three slots in rotation, as in the forward kernel
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rh = wave & 1, cb = wave >> 1;
+    const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
+    for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;
+    if (tid < 3) need[tid] = 0u;
+    const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
+    u32x4_t wp[3][NS];
+    const int PW = bf16_kernel_column<NS>(w, K, N, bcol, kq, wp);
+    FastMap mp;
+    mp.init(K);
+    int fi[FAST_NJ][4], tix[FAST_NJ];
+    uint32_t amx[FAST_NJ][4];  // not tracked here
+    fast_frac_bits<QUANT>(f_in, P, K, mp, Mode(mode).round_params, fi, tix);
+    f32x4_t raw[FAST_NJ];
+    uint32_t xoff[FAST_NJ];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) xoff[j] = mp.on[j] ? (uint32_t)(mp.row[j] * K + mp.col[j]) * 4u : BUF_OOB;
+    auto load_tile = [&](int64_t t) {
+        const int64_t r0 = t * FAST_BM, left = rows - r0;
+        const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K, (left < FAST_BM ? left : FAST_BM) * K * 4);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) raw[j] = buf_ld4(rs, xoff[j]);
+    };
+    int64_t tile = blockIdx.x;
+    if (tile < n_tiles) load_tile(tile);
+    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    float s1 = 0.f, s2 = 0.f;
+    int buf = 0, slot = 0;
+    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1, slot = slot == 2 ? 0 : slot + 1) {
+        bf16_stage<RM, QUANT, false>(raw, fi, mp, xp[buf], &need[slot], amx);
+        __syncthreads();
+        if (tid == 0) need[slot == 0 ? 2 : slot - 1] = 0u;
+        const uint32_t nd = need[slot];
+        const int64_t next = tile + gridDim.x;
+        if (next < n_tiles) load_tile(next);
+        if (cb * 32 < N) {
+            floatx16 acc = {0};
+            acc = bf16_chain<NS>(acc, xp[buf], arow, kq, nd, wp, PW);
+            // rows past the end were staged as zeros: z = 0 there, which adds nothing
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s1 += acc[r], s2 += acc[r] * acc[r];
+        }
+    }
+    red[wave][lane][0] = s1, red[wave][lane][1] = s2;
+    __syncthreads();
+    if (tid < 2 * N) {
+        const int c = tid % N, which = tid / N, wcb = c >> 5, l = c & 31;
+        float v = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) v += red[wcb * 2 + h][l][which] + red[wcb * 2 + h][l + 32][which];
+        part[(int64_t)blockIdx.x * 2 * N + which * N + c] = v;
+    }
+}
+
 __global__ __launch_bounds__(256) void moments_scale_kernel(float *mean, float *meansq, int N, float inv_rows) {
     const int t = blockIdx.x * 256 + threadIdx.x;
     if (t < N) mean[t] *= inv_rows, meansq[t] *= inv_rows;
@@ -820,7 +887,9 @@ __global__ __launch_bounds__(256) void moments_scale_kernel(float *mean, float *
 // STATS: the gradient at the pre-activation is not read but computed in the tile from the upstream
 // gradients of the column statistics: dz[r, c] = (gm[c] + 2 z[r, c] gs[c]) / rows with z = x W
 // recomputed on the matrix cores (dy = gm, y = gs, both [N]); no activation, no bias, no quantizer.
-template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true>
+// BF: the three contractions run on the bf16 matrix cores by exact splitting (mfma_chain_bf16); the gradient operand is
+// taken in all three parts without looking, the quantized input and the kernel in as many as they need.
+template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true, bool BF = false>
 __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
@@ -952,7 +1021,8 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
             if (zcb < N32) {
                 floatx16 z = {0};
                 const int arow = zrh * 32 + (lane & 31), kq = lane >> 5, bcol = zcb * 32 + (lane & 31);
-                z = mfma_chain(z, &xs[arow][kq], 1, &ws[kq][bcol], FAST_LD, K32 * 2);
+                z = BF ? mfma_chain_bf16<false, false>(z, &xs[arow][kq], 1, &ws[kq][bcol], FAST_LD, K32 * 2)
+                       : mfma_chain(z, &xs[arow][kq], 1, &ws[kq][bcol], FAST_LD, K32 * 2);
                 const float gm = bcol < N ? dy[bcol] : 0.f, gs = bcol < N ? y[bcol] : 0.f;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -972,16 +1042,19 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         if (split_n) {
             // one k block, two column blocks: the two wavefronts of a row half take one half of the contraction each
             const int arow = rh * 32 + (lane & 31), kq = lane >> 5, n0 = kb * 32;
-            acc = mfma_chain(acc, &dzs[arow][n0 + kq], 1, &ws[lane & 31][n0 + kq], 1, 2);
+            acc = BF ? mfma_chain_bf16<true, false>(acc, &dzs[arow][n0 + kq], 1, &ws[lane & 31][n0 + kq], 1, 2)
+                     : mfma_chain(acc, &dzs[arow][n0 + kq], 1, &ws[lane & 31][n0 + kq], 1, 2);
         } else if (kb < K32) {
             const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
-            acc = mfma_chain(acc, &dzs[arow][kq], 1, &ws[wrow][kq], 1, N32 * 2);
+            acc = BF ? mfma_chain_bf16<true, false>(acc, &dzs[arow][kq], 1, &ws[wrow][kq], 1, N32 * 2)
+                     : mfma_chain(acc, &dzs[arow][kq], 1, &ws[wrow][kq], 1, N32 * 2);
         }
         // ---- dW += xq^T @ dz : this wave's block, its slice of the tile's rows
         {
             const int rbeg = sub * rows_per;
             const int kq = lane >> 5, c32 = lane & 31;
-            accw = mfma_chain(accw, &xs[rbeg + kq][wkb * 32 + c32], FAST_LD, &dzs[rbeg + kq][wnb * 32 + c32], FAST_LD, rows_per / 16);
+            accw = BF ? mfma_chain_bf16<false, true>(accw, &xs[rbeg + kq][wkb * 32 + c32], FAST_LD, &dzs[rbeg + kq][wnb * 32 + c32], FAST_LD, rows_per / 16)
+                      : mfma_chain(accw, &xs[rbeg + kq][wkb * 32 + c32], FAST_LD, &dzs[rbeg + kq][wnb * 32 + c32], FAST_LD, rows_per / 16);
         }
         if (has_bias) {
 #pragma unroll
@@ -1318,6 +1391,13 @@ extern "C" int hgq_qdense_moments_fwd(const float *x, const float *f_in, int64_t
     const bool quant = bw_rows > 0;
     const int P = quant ? (int)bw_rows : 1;
     const int rm = Mode(mode).round_mode;
+#define HGQ_MOM_BF16(NSV) \
+    do { \
+        if (!quant) hipLaunchKernelGGL((dense_moments_bf16_kernel<HGQ_TRN, false, NSV>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+        else if (rm == HGQ_TRN) hipLaunchKernelGGL((dense_moments_bf16_kernel<HGQ_TRN, true, NSV>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+        else if (rm == HGQ_RND) hipLaunchKernelGGL((dense_moments_bf16_kernel<HGQ_RND, true, NSV>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+        else hipLaunchKernelGGL((dense_moments_bf16_kernel<HGQ_RND_CONV, true, NSV>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
+    } while (0)
 #define HGQ_MOM_FAST(NS4V) \
     do { \
         if (!quant) hipLaunchKernelGGL((dense_moments_fast_kernel<HGQ_TRN, false, NS4V>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
@@ -1325,11 +1405,17 @@ extern "C" int hgq_qdense_moments_fwd(const float *x, const float *f_in, int64_t
         else if (rm == HGQ_RND) hipLaunchKernelGGL((dense_moments_fast_kernel<HGQ_RND, true, NS4V>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
         else hipLaunchKernelGGL((dense_moments_fast_kernel<HGQ_RND_CONV, true, NS4V>), grid, dim3(256), 0, s, x, f_in, P, w, workspace, rows, K, N, mode); \
     } while (0)
-    if (K <= 8) HGQ_MOM_FAST(1);
+    if (g_dense_bf16) {
+        if (K <= 16) HGQ_MOM_BF16(1);
+        else if (K <= 32) HGQ_MOM_BF16(2);
+        else if (K <= 48) HGQ_MOM_BF16(3);
+        else HGQ_MOM_BF16(4);
+    } else if (K <= 8) HGQ_MOM_FAST(1);
     else if (K <= 16) HGQ_MOM_FAST(2);
     else if (K <= 32) HGQ_MOM_FAST(4);
     else HGQ_MOM_FAST(8);
 #undef HGQ_MOM_FAST
+#undef HGQ_MOM_BF16
     if ((rc = check_launch("hgq_qdense_moments_fwd"))) return rc;
     if ((rc = reduce_parts(workspace, parts, 2 * (int64_t)N, mean, (int64_t)N, meansq, (int64_t)N, nullptr, 0, s))) return rc;
     hipLaunchKernelGGL(moments_scale_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, mean, meansq, N, 1.0f / (float)rows);
@@ -1355,7 +1441,10 @@ extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t
     const int rm = Mode(mode).round_mode;
     const dim3 grid((unsigned)parts);
 #define HGQ_MOM_BWD(RMV, QV) \
-    hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode, dx_add)
+    do { \
+        if (g_dense_bf16) hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true, true, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode, dx_add); \
+        else hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode, dx_add); \
+    } while (0)
     if (!quant) HGQ_MOM_BWD(HGQ_TRN, false);
     else if (rm == HGQ_TRN) HGQ_MOM_BWD(HGQ_TRN, true);
     else if (rm == HGQ_RND) HGQ_MOM_BWD(HGQ_RND, true);
@@ -1405,8 +1494,14 @@ static int qdense_bwd_impl(const float *dy, const float *y, const float *x, cons
         const bool zvec = N % 4 == 0 && aligned16(dy) && (act != HGQ_ACT_RELU || aligned16(y));
 #define HGQ_BWD_FAST(RMV, QV)                                                                                                          \
     do {                                                                                                                               \
-        if (zvec)                                                                                                                      \
+        if (zvec && g_dense_bf16)                                                                                                      \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
+                               dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
+        else if (zvec)                                                                                                                 \
             hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
+                               dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
+        else if (g_dense_bf16)                                                                                                         \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, false, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
                                dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
         else                                                                                                                           \
             hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, false>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \

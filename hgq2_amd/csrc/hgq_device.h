@@ -267,6 +267,106 @@ __device__ __forceinline__ floatx16 mfma_chain(floatx16 acc, const float *ap, in
     return acc;
 }
 
+// ------------------------------------------------------------------------------------------
+// The same chain on the bf16 matrix cores, exactly.  An fp32 number is the sum of three numbers of eight significant
+// bits each - its leading bits, the leading bits of what is left, and the rest - and each is a bf16 number (same
+// exponent range).  A product of two parts is exact in fp32, so the sum over part pairs of A_p B_q, accumulated in fp32,
+// is the contraction with only the accumulation rounded, as in the fp32 instruction.  v_mfma_f32_32x32x16_bf16 takes the
+// sixteen contraction steps of a batch in one instruction of half the issue time of ONE fp32 instruction: one to nine
+// instructions replace eight.  Quantized operands rarely need more than one part (eight bits) or two (sixteen): a
+// wavefront looks at the operands it has just read and multiplies the non-zero parts only (uniform branches).
+// Operand layout (64 lanes, eight bf16 per lane): A[i][k]: i = lane % 32, k = 8 (lane / 32) + e; B[k][j] likewise; the
+// sum does not depend on which contraction step sits where, so element e of lane half h is step 2 e + h of the batch -
+// the LDS reads are those of the fp32 chain.
+// ------------------------------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// the three parts of v as fp32 bit patterns whose low halves are zero (a part that is not needed is zero)
+__device__ __forceinline__ void bf16_parts(float v, uint32_t &h, uint32_t &m, uint32_t &l) {
+    h = __float_as_uint(v) & 0xffff0000u;
+    const float r1 = __fsub_rn(v, __uint_as_float(h));  // exact: the low 16 bits of the significand
+    m = __float_as_uint(r1) & 0xffff0000u;
+    l = __float_as_uint(__fsub_rn(r1, __uint_as_float(m)));  // exact, at most eight significant bits
+}
+// two parts (bit patterns with zero low halves) as one register of two bf16: `a` first
+__device__ __forceinline__ uint32_t bf16_pair(uint32_t a, uint32_t b) { return (a >> 16) | b; }
+
+__device__ __forceinline__ floatx16 mfma_bf16(const u32x4_t &a, const u32x4_t &b, floatx16 acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+}
+
+// The leading parts of eight fp32 operands of a lane (the high halves of the words) and whether that is all of them for
+// every lane of the wavefront.
+__device__ __forceinline__ bool bf16_lead8(const float (&v)[8], u32x4_t &p0) {
+    uint32_t low = 0u;
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+        p0[e >> 1] = __builtin_amdgcn_perm(__float_as_uint(v[e + 1]), __float_as_uint(v[e]), 0x07060302u);
+        low |= __float_as_uint(v[e]) | __float_as_uint(v[e + 1]);
+    }
+    return !__any((low & 0xffffu) != 0u);
+}
+// The second and third parts; returns whether the third is non-zero anywhere in the wavefront.
+__device__ __forceinline__ bool bf16_rest8(const float (&v)[8], u32x4_t &p1, u32x4_t &p2) {
+    uint32_t nz2 = 0u;
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+        uint32_t h0, m0, l0, h1, m1, l1;
+        bf16_parts(v[e], h0, m0, l0), bf16_parts(v[e + 1], h1, m1, l1);
+        p1[e >> 1] = bf16_pair(m0, m1), p2[e >> 1] = bf16_pair(l0, l1);
+        nz2 |= l0 | l1;
+    }
+    return __any(nz2 != 0u);
+}
+
+// Same arguments and LDS reads as mfma_chain.  FULL_A / FULL_B: that operand is a gradient - arbitrary fp32, all three
+// parts taken without looking.  A batch whose part pairs would cost more than the eight fp32 instructions they replace
+// (splitting included) is issued as those eight instructions: the chain is never slower than mfma_chain by more than
+// the look at the operands.
+template <bool FULL_A, bool FULL_B>
+__device__ __forceinline__ floatx16 mfma_chain_bf16(floatx16 acc, const float *ap, int sa, const float *bp, int sb, int n_batches) {
+    static_assert(!(FULL_A && FULL_B), "one operand of a chain is a quantized tensor");
+    // (the next batch's operands are not requested ahead as in mfma_chain: the registers that takes spill in the kernels
+    // that use this chain, and a batch is a few instructions, not eight, so the other wavefronts cover the LDS latency)
+#pragma unroll
+    for (int bt = 0; bt < 4; ++bt) {
+        if (bt < n_batches) {
+            float a[8], b[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a[u] = ap[(16 * bt + 2 * u) * sa], b[u] = bp[(16 * bt + 2 * u) * sb];
+            u32x4_t pa0, pb0;
+            const bool one_a = bf16_lead8(a, pa0), one_b = bf16_lead8(b, pb0);
+            if (FULL_A || FULL_B) {
+                if (FULL_A ? one_b : one_a) {
+                    // three instructions: the quantized operand's single part against the gradient's three
+                    u32x4_t p1, p2;
+                    bf16_rest8(FULL_A ? a : b, p1, p2);
+                    acc = FULL_A ? mfma_bf16(pa0, pb0, acc) : mfma_bf16(pa0, pb0, acc);
+                    acc = FULL_A ? mfma_bf16(p1, pb0, acc) : mfma_bf16(pa0, p1, acc);
+                    acc = FULL_A ? mfma_bf16(p2, pb0, acc) : mfma_bf16(pa0, p2, acc);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+                }
+            } else if (one_a && one_b) {
+                acc = mfma_bf16(pa0, pb0, acc);
+            } else if (one_a || one_b) {
+                // one side has a single part: up to three instructions
+                u32x4_t p1, p2;
+                const bool third = bf16_rest8(one_a ? b : a, p1, p2);
+                acc = mfma_bf16(pa0, pb0, acc);
+                acc = one_a ? mfma_bf16(pa0, p1, acc) : mfma_bf16(p1, pb0, acc);
+                if (third) acc = one_a ? mfma_bf16(pa0, p2, acc) : mfma_bf16(p2, pb0, acc);
+            } else {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+            }
+        }
+    }
+    return acc;
+}
+
 }  // namespace hgq
 
 // dispatch a (round_mode, overflow_mode) pair to template arguments

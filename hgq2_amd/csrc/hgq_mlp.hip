@@ -20,6 +20,15 @@ namespace hgq {
 
 
 #define MLP_BM 64
+// the matrix-core chains: by exact bf16 parts (1) or with the fp32 instruction (0)
+#ifndef MLP_BF16
+#define MLP_BF16 1
+#endif
+#if MLP_BF16
+#define MLP_CHAIN(FA, FB) mfma_chain_bf16<FA, FB>
+#else
+#define MLP_CHAIN(FA, FB) mfma_chain
+#endif
 #define MLP_NT 512  // eight wavefronts: two per SIMD, so the chains of one hide the latencies of the other
 #define MLP_LDZ 65
 
@@ -214,7 +223,7 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                 const float *ws = lds + ly.off_w;
                 const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
                 // input columns and kernel rows are zero padded to a multiple of 32
-                acc = mfma_chain(acc, rx + arow * d.ld_rx + ly.acol + kq, 1, ws + kq * ly.ldw + bcol, ly.ldw, (ly.h.K + 15) >> 4);
+                acc = MLP_CHAIN(false, false)(acc, rx + arow * d.ld_rx + ly.acol + kq, 1, ws + kq * ly.ldw + bcol, ly.ldw, (ly.h.K + 15) >> 4);
                 if (bcol < N) {
                     const float bias = lds[ly.off_qb + bcol];
                     const bool last = l + 1 == L;
@@ -295,8 +304,8 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                 const int wkb = (wave - 4) / N32, wnb = (wave - 4) % N32;
                 floatx16 acc = {0};
                 const int kq = lane >> 5, c32 = lane & 31;
-                acc = mfma_chain(acc, rx + kq * d.ld_rx + ly.acol + wkb * 32 + c32, d.ld_rx, cur + kq * MLP_LDZ + wnb * 32 + c32, MLP_LDZ,
-                                 MLP_BM / 16);
+                acc = MLP_CHAIN(false, true)(acc, rx + kq * d.ld_rx + ly.acol + wkb * 32 + c32, d.ld_rx, cur + kq * MLP_LDZ + wnb * 32 + c32, MLP_LDZ,
+                                             MLP_BM / 16);
                 const int n = wnb * 32 + c32;
                 if (n < N) {
 #pragma unroll
@@ -325,7 +334,7 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                     const float *ws = lds + ly.off_w;
                     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
                     // gradient columns and kernel columns are zero padded to a multiple of 32
-                    acc = mfma_chain(acc, cur + arow * MLP_LDZ + kq, 1, ws + wrow * ly.ldw + kq, 1, (N + 15) >> 4);
+                    acc = MLP_CHAIN(true, false)(acc, cur + arow * MLP_LDZ + kq, 1, ws + wrow * ly.ldw + kq, 1, (N + 15) >> 4);
                     const int kcol = kb * 32 + (lane & 31);
                     const bool mask_below = l > 0 && d.l[l - 1].h.act == HGQ_ACT_RELU;
                     float dfsum = 0.f;
