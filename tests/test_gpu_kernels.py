@@ -391,6 +391,44 @@ def test_bias_and_affine_gradients_without_framework_reductions(dev):
     assert torch.all((o1.grad.double() - o2.grad).abs() <= 1e-6 * up.double().abs().sum((0, 1), keepdim=True))
 
 
+@pytest.mark.parametrize('rows,K,N,bits_x,bits_w,act', [(4096, 64, 64, 6, 6, 1), (1000, 64, 32, 12, 5, 0), (513, 48, 33, 12, 12, 1),
+                                                        (2000, 16, 64, 22, 22, 0), (70, 4, 4, 5, 5, 0), (3000, 20, 12, 8, 16, 1)])
+def test_dense_on_bf16_parts_is_the_fp32_contraction(dev, rows, K, N, bits_x, bits_w, act):
+    """The streaming dense kernels contract on the bf16 matrix cores after splitting every fp32 operand exactly into up to
+    three bf16 parts (8 + 8 + 8 significant bits).  Products of parts are exact and the accumulation is fp32, so the
+    result is the fp32 contraction up to the order of the accumulation: against float64 both instructions sit within
+    1e-6 of the sum of |terms|, and where every partial sum is exactly representable (few-bit operands) they agree bit
+    for bit.  Operands of 5 to 22 bits exercise one, two and three parts on either side."""
+    _lib, ops = _ops()
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(rows + K)
+    x = (torch.round(torch.randn(rows, K, generator=g) * 2 ** (bits_x - 3)) / 2 ** (bits_x - 3)).to(dev)
+    w = (torch.round(torch.randn(K, N, generator=g) * 2 ** (bits_w - 2)) / 2 ** bits_w).to(dev)
+    b = (torch.round(torch.randn(N, generator=g) * 16) / 16).to(dev)
+    dy, e = torch.randn(rows, N, generator=g).to(dev), x.new_empty(0)
+    want = x.double() @ w.double() + b.double()
+    mask = (want > 0).double() if act else torch.ones_like(want)
+    want = want * mask
+    dz = dy.double() * mask
+    refs = (want, dz @ w.double().T, x.double().T @ dz, dz.sum(0))
+    scales = (x.double().abs() @ w.double().abs() + b.double().abs(), dz.abs() @ w.double().abs().T, x.double().abs().T @ dz.abs(), dz.abs().sum(0))
+    was = lib.hgq_dense_use_bf16_parts(-1)
+    got = {}
+    try:
+        for on in (0, 1):
+            lib.hgq_dense_use_bf16_parts(on)
+            y, _ = ops.qdense_fwd(x, e, e, e, w, b, act, 0, 0, False)
+            dx, dqw, dqb, _ = ops.qdense_bwd(dy, y, x, e, w, True, act, 0, 0)
+            got[on] = (y, dx, dqw, dqb)
+            for name, t, want_t, sc in zip(('y', 'dx', 'dW', 'db'), got[on], refs, scales):
+                err = ((t.double() - want_t).abs() / (sc + 1e-30)).max().item()
+                assert err <= 1e-6, f'{name} with bf16 parts = {on}: {err:.2e} of the sum of |terms|'
+    finally:
+        lib.hgq_dense_use_bf16_parts(was)
+    if bits_x + bits_w + 7 <= 24:  # every partial sum of x W is exact in fp32: no accumulation order to differ in
+        assert torch.equal(got[0][0], got[1][0])
+
+
 def test_sparse_ce_and_sgd(dev):
     _lib, ops = _ops()
     g = torch.Generator().manual_seed(17)
