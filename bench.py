@@ -182,6 +182,55 @@ def softmax_roofline(iters=50, shape=(2048, 4, 64, 64), scaler=0.25):
     return out
 
 
+def dense_streaming(iters=20, rows=131072, K=64, N=64):
+    """The streaming dense kernels (the contraction of QDense / QEinsumDense with the batch as rows) at rows x K x N with
+    cold operands: six operand sets are rotated inside one captured HIP graph, timed with HIP events around its
+    replays.  Run once per matrix instruction (fp32 `32x32x2`, and bf16 `32x32x16` on exact bf16 parts of the fp32
+    operands) and per operand width (6 bits: one part; 12: two; 22: three).  Algorithmic bytes: forward
+    4 (rows K + rows N) B; backward 4 (2 rows N + 2 rows K) B (dy, y, x in; dx out) plus the slices."""
+    import torch
+
+    from hgq2_amd import _lib, ops
+
+    lib = _lib.load()
+    dev = torch.device('cuda:0')
+    g = torch.Generator().manual_seed(0)
+    e = torch.empty(0, device=dev)
+    n_sets = 6
+    out = {}
+    was = lib.hgq_dense_use_bf16_parts(-1)
+    for bits in (6, 12, 22):
+        xs = [(torch.round(torch.randn(rows, K, generator=g) * 2 ** (bits - 3)) / 2 ** (bits - 3)).to(dev) for _ in range(n_sets)]
+        w = (torch.round(torch.randn(K, N, generator=g) * 2 ** (bits - 2)) / 2 ** bits).to(dev)
+        b = torch.zeros(N, device=dev)
+        dys = [torch.randn(rows, N, generator=g).to(dev) for _ in range(n_sets)]
+        ys = [ops.qdense_fwd(x, e, e, e, w, b, 1, 0, 0, False)[0] for x in xs]
+        for on, name in ((0, 'fp32'), (1, 'bf16_parts')):
+            lib.hgq_dense_use_bf16_parts(on)
+            for what, nbytes in (('fwd', 4 * rows * (K + N)), ('bwd', 8 * rows * (K + N))):
+                def launches():
+                    for x, dy, y in zip(xs, dys, ys):
+                        if what == 'fwd':
+                            ops.qdense_fwd(x, e, e, e, w, b, 1, 0, 0, False)
+                        else:
+                            ops.qdense_bwd(dy, y, x, e, w, True, 1, 0, 0)
+
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    launches()
+                torch.cuda.current_stream().wait_stream(side)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    launches()
+                graph.replay()
+                ms = _events_ms(graph.replay, iters) / n_sets
+                gbs = nbytes / (ms * 1e-3) / 1e9
+                out[f'{what}_{name}_{bits}bit'] = {'ms': ms, 'bytes': nbytes, 'GBps': gbs, 'frac': gbs / HBM_PEAK_GBS}
+    lib.hgq_dense_use_bf16_parts(was)
+    return out
+
+
 def config_step_time(name, steps=20, warmup=5, graph=False, cpu=False, cpu_budget_s=15.0):
     """One training step (forward, backward, SGD update) of the configurations other than the headline one, at their full
     sizes: 'particle' (QEinsumDenseBatchnorm per-particle network, batch 4096 x 64 x 16), 'conv'
@@ -365,6 +414,8 @@ def main():
     ap.add_argument('--graph', action='store_true', help='with --config-step: capture the step in a HIP graph and replay it')
     ap.add_argument('--softmax-only', action='store_true',
                     help='run only the one-pass table-softmax kernels at the attention configuration (for profiler runs)')
+    ap.add_argument('--dense-only', action='store_true',
+                    help='run only the streaming dense kernels at 131072 x 64 x 64 with either matrix instruction (for profiler runs)')
     ap.add_argument('--path', choices=('fused', 'fused-graph', 'layers-graph', 'layers-eager'), default='fused',
                     help='fused: whole-step kernels (2 launches); layers: per-layer torch.library operators with autograd; '
                          '-graph: the step is captured once in a HIP graph and replayed')
@@ -388,6 +439,11 @@ def main():
     if args.softmax_only:
         torch.cuda.set_device(0)
         print(json.dumps({'softmax_kernels': softmax_roofline(iters=20)}))
+        return
+
+    if args.dense_only:
+        torch.cuda.set_device(0)
+        print(json.dumps({'dense_kernels': dense_streaming()}))
         return
 
     from hgq2_amd import ops
