@@ -289,3 +289,52 @@ class FusedQDenseStack:
         self._lib.check(rc, 'hgq_mlp_train_step_cached')
         self._versions = versions
         return self.loss
+
+
+class _FusedStep:
+    """The whole-step kernels behind the call signature of :class:`GraphedTrainStep`."""
+
+    path = 'fused'
+
+    def __init__(self, stack: FusedQDenseStack):
+        self.stack = stack
+
+    def __call__(self, x, y):
+        return self.stack.step(x, y)
+
+
+def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 'sparse_ce', fused: bool | None = None):
+    """A callable ``step(x, y) -> loss`` that runs one SGD training step of ``model`` on the fastest path that covers it.
+
+    A built stack of :class:`QDense` layers trained with mean sparse categorical cross-entropy and within what
+    :class:`FusedQDenseStack` checks (widths up to 64, the default quantizer kinds, an LDS plan that fits) runs on the
+    whole-step kernels; every other model, and ``loss='mse'``, runs the per-layer operators replayed from a HIP graph
+    (:class:`GraphedTrainStep` with :class:`SGD`, regularizers folded into the update).  Both paths update the same
+    variables with the same arithmetic (the whole-step kernels restate the per-layer sequence), so the choice changes
+    the time per step and nothing else.  ``fused=False`` forces the per-layer path, ``fused=True`` raises where the
+    whole-step path does not apply.  The returned object's ``path`` is ``'fused'`` or ``'layers_graph'``."""
+    if loss not in ('sparse_ce', 'mse'):
+        raise ValueError(f"loss must be 'sparse_ce' or 'mse', got {loss!r}")
+    if not model.built:
+        model(example_x, training=True)
+    if fused is not False and loss == 'sparse_ce':
+        try:
+            stack = FusedQDenseStack(model, lr=lr)
+            if example_x.dim() != 2 or example_x.shape[1] != stack._arr[0].K:
+                raise ValueError('the fused QDense step takes [rows, features] inputs')
+            from . import _lib
+
+            lib = _lib.load()
+            if lib.hgq_mlp_workspace(stack._arr, len(stack.layers), example_x.shape[0]) < 0:
+                raise ValueError('the fused QDense step does not cover this stack: ' + (lib.hgq_last_error() or b'').decode())
+            return _FusedStep(stack)
+        except ValueError:
+            if fused:
+                raise
+    elif fused:
+        raise ValueError('the fused QDense step computes sparse categorical cross-entropy only')
+    loss_fn = ops.sparse_ce if loss == 'sparse_ce' else ops.mse
+    step = GraphedTrainStep(model, loss_fn, SGD(model.parameters(), lr=lr, fold_regularizers=True), example_x, example_y)
+    step.path = 'layers_graph'
+    return step
+

@@ -675,3 +675,57 @@ def test_saved_and_loaded_model_gives_equal_outputs(dev, kind, tmp_path):
     for (na, ta), (_, tb) in zip(saving.variable_paths(model).items(), saving.variable_paths(clone).items()):
         if ta.dtype == torch.float32:
             assert torch.allclose(ta, tb, rtol=1e-6, atol=1e-9), f'{na} after one more step'
+
+
+def test_train_step_for_picks_the_path_and_both_paths_agree(dev):
+    """`train_step_for` runs a plain QDense stack with cross-entropy on the whole-step kernels and everything else on the
+    per-layer operators replayed from a HIP graph; the two paths restate the same sequence, so from the same start state
+    they reach the same variables (tracked integer bits and EBOPs exactly, trained variables to the order of fp32
+    sums)."""
+    import io
+
+    from hgq2_amd import saving
+    from hgq2_amd.config import LayerConfigScope, QuantizerConfigScope
+    from hgq2_amd.core import Sequential
+    from hgq2_amd.layers import QDense
+    from hgq2_amd.train import train_step_for
+
+    g = torch.Generator().manual_seed(5)
+    torch.manual_seed(5)
+    x = torch.randn(1000, 12, generator=g).to(dev)
+    labels = torch.randint(0, 4, (1000,), generator=g).to(dev)
+
+    def stack(widths, **kw):
+        with QuantizerConfigScope(place='all', default_q_type='kbi', overflow_mode='SAT_SYM'), \
+                QuantizerConfigScope(place='datalane', default_q_type='kif', overflow_mode='WRAP'), \
+                LayerConfigScope(enable_ebops=True, beta0=1e-5):
+            model = Sequential([QDense(w, activation='relu' if n + 1 < len(widths) else None, **kw) for n, w in enumerate(widths)])
+        model(x, training=True)
+        return model
+
+    model = stack([24, 16, 4])
+    buf = io.BytesIO()
+    saving.save_model(model, buf)
+    buf.seek(0)
+    clone = saving.load_model(buf, device=dev)
+    fused = train_step_for(model, x, labels, lr=0.05)
+    layered = train_step_for(clone, x, labels, lr=0.05, fused=False)
+    assert fused.path == 'fused' and layered.path == 'layers_graph'
+    buf.seek(0)
+    saving.load_weights(clone, buf)  # the capture's warm-up steps moved the clone: back to the common start
+    for step in range(4):
+        fused(x, labels), layered(x, labels)  # (the loss values differ by the regularizer terms the per-layer update folds in)
+        for a, b in zip(model.layers, clone.layers):
+            assert torch.equal(a.iq.quantizer._i, b.iq.quantizer._i)
+            assert int(a._ebops.view(torch.int32)) == int(b._ebops.view(torch.int32))
+        for (name, pa), (_, pb) in zip(model.named_parameters(), clone.named_parameters()):
+            err = (pa.detach().double() - pb.detach().double()).abs().max().item()
+            assert err <= 2e-5 * (pb.detach().abs().max().item() + 1e-6), (step, name, err)
+
+    # outside the whole-step kernels' cover: a layer wider than 64, an output quantizer, another loss
+    assert train_step_for(stack([80, 4]), x, labels).path == 'layers_graph'
+    assert train_step_for(stack([16, 4], enable_oq=True), x, labels).path == 'layers_graph'
+    target = torch.randn(1000, 4, generator=g).to(dev)
+    assert train_step_for(stack([16, 4]), x, target, loss='mse').path == 'layers_graph'
+    with pytest.raises(ValueError):
+        train_step_for(stack([80, 4]), x, labels, fused=True)
