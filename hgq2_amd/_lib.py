@@ -46,6 +46,9 @@ SIGNATURES = {
     'hgq_qdense_fwd_parts': (c_int, [c_int64]),
     'hgq_qdense_bwd_workspace': (c_int64, [c_int64, c_int, c_int, c_int64]),
     'hgq_qdense_fwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 4 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_qdense_fwd_oq_supported': (c_int, [c_int64, c_int, c_int, c_int64, c_int64, c_int, c_int]),
+    'hgq_qdense_fwd_oq': (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64] + [c_void_p] * 4
+                          + [c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     'hgq_qdense_bwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 6 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     'hgq_dense_ebops': (
         c_int,

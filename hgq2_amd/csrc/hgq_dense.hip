@@ -514,6 +514,15 @@ typedef uint16_t (*bf16_planes_t)[FAST_BM + 1][BF_LD];  // [part][row][k] of one
 
 // Stages the four 128-bit slots of a thread (quantized first when QUANT) as bf16 parts and records in `need` which of
 // the second / third parts of the tile are non-zero (bit 0 / 1).  TRACK: the abs-max of the staged values.
+// Four small integers (fractional bits: clamped to a signed byte) in one register.
+__device__ __forceinline__ int pack_i8x4(const int (&v)[4]) {
+    int r = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r |= (max(-128, min(127, v[e])) & 0xff) << (8 * e);
+    return r;
+}
+__device__ __forceinline__ int unpack_i8(int packed, int e) { return (int)(int8_t)((packed >> (8 * e)) & 0xff); }
+
 template <int RM, bool QUANT, bool TRACK>
 __device__ __forceinline__ void bf16_stage(const f32x4_t (&raw)[FAST_NJ], const int (&fi)[FAST_NJ][4], const FastMap &mp, bf16_planes_t xp,
                                            uint32_t *need, uint32_t (&amx)[FAST_NJ][4], float (*dlt)[4] = nullptr) {
@@ -613,12 +622,17 @@ __device__ __forceinline__ floatx16 bf16_chain(floatx16 acc, bf16_planes_t xp, i
 }
 
 // NS = steps of sixteen k that cover K.
-template <int RM, bool QUANT, int NS>
+// OQ: the layer's output quantizer (training-mode WRAP: round only, [Po, N] table of fractional bits, same round mode)
+// runs on the output tile as it leaves: `y` gets the contraction, `yq` its quantized values, slice blockIdx.x of
+// `oamax_part` the abs-max of the quantized values per table entry.
+template <int RM, bool QUANT, int NS, bool OQ = false>
 __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw,
                                                               const float *__restrict__ qb, float *__restrict__ y,
                                                               uint32_t *amax_part, int64_t rows, int K, int N, int act,
-                                                              int mode) {
+                                                              int mode, const float *__restrict__ f_out = nullptr, int Po = 1,
+                                                              int mode_out = 0, float *__restrict__ yq = nullptr,
+                                                              uint32_t *oamax_part = nullptr) {
     // [buffer][part][row][k]; row FAST_BM: sink of the idle staging slots
     __shared__ __attribute__((aligned(16))) uint16_t xp[2][3][FAST_BM + 1][BF_LD];
     __shared__ __attribute__((aligned(16))) float ys[FAST_BM][FAST_XLD];
@@ -639,13 +653,35 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     mp.init(K);
     const bool vec_out = (N & 3) == 0 && ((uintptr_t)y & 15u) == 0;
     mo.init(vec_out ? N : 4);
-    int fi[FAST_NJ][4], tix[FAST_NJ];
+    // fractional bits of the staged elements, four to a register (unpacked per tile: sixteen values and their negations
+    // would otherwise each hold a register for the whole launch)
+    int fip[FAST_NJ], tix[FAST_NJ];
     uint32_t amx[FAST_NJ][4];
-    fast_frac_bits<QUANT>(f_in, P, K, mp, m.round_params, fi, tix);
+    {
+        int fi[FAST_NJ][4];
+        fast_frac_bits<QUANT>(f_in, P, K, mp, m.round_params, fi, tix);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) fip[j] = pack_i8x4(fi[j]);
+    }
 #pragma unroll
     for (int j = 0; j < FAST_NJ; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e) amx[j][e] = 0;
+    // OQ: fractional bits of the output elements this thread stores, four to a register, and their trackers
+    int fo[OQ ? FAST_NJ : 1], otix[OQ ? FAST_NJ : 1];
+    uint32_t oamx[OQ ? FAST_NJ : 1][4];
+    if (OQ) {
+        int fo4[FAST_NJ][4], ot[FAST_NJ];
+        fast_frac_bits<true>(f_out, Po, N, mo, Mode(mode_out).round_params, fo4, ot);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            const int jj = OQ ? j : 0;
+            otix[jj] = ot[j];
+                        fo[jj] = pack_i8x4(fo4[j]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) oamx[jj][e] = 0;
+        }
+    }
     f32x4_t raw[FAST_NJ];
     uint32_t xoff[FAST_NJ];
 #pragma unroll
@@ -662,6 +698,13 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     int buf = 0, slot = 0;
     for (; tile < n_tiles; tile += gridDim.x, buf ^= 1, slot = slot == 2 ? 0 : slot + 1) {
+        int fi[FAST_NJ][4];
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            asm volatile("" : "+v"(fip[j]));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) fi[j][e] = unpack_i8(fip[j], e);
+        }
         bf16_stage<RM, QUANT, QUANT>(raw, fi, mp, xp[buf], &need[slot], amx);
         __syncthreads();
         if (tid == 0) need[slot == 0 ? 2 : slot - 1] = 0u;  // (slot + 2) % 3
@@ -684,7 +727,20 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
             for (int j = 0; j < FAST_NJ; ++j) {
                 const int64_t gr = r0 + mo.row[j];
                 if (mo.on[j] && gr < rows) {
-                    *(f32x4_t *)(y + gr * N + mo.col[j]) = *(const f32x4_t *)&ys[mo.row[j]][mo.col[j]];
+                    const f32x4_t v4 = *(const f32x4_t *)&ys[mo.row[j]][mo.col[j]];
+                    *(f32x4_t *)(y + gr * N + mo.col[j]) = v4;
+                    if (OQ) {
+                        const int jj = OQ ? j : 0;
+                        asm volatile("" : "+v"(fo[jj]));
+                        f32x4_t q4;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int f = unpack_i8(fo[jj], e);
+                            q4[e] = ldexpf(round_scaled<RM>(ldexpf(v4[e], f)), -f);
+                            oamx[jj][e] = max(oamx[jj][e], abs_bits(q4[e]));
+                        }
+                        *(f32x4_t *)(yq + gr * N + mo.col[j]) = q4;
+                    }
                 }
             }
         } else {
@@ -724,6 +780,32 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         __syncthreads();
         uint32_t *my = amax_part + (int64_t)blockIdx.x * PK;
         for (int t = tid; t < PK; t += 256) my[t] = tab[t];
+    }
+    if (OQ) {  // (launched with 128-bit output rows only)
+        const int PN = Po * N;
+        uint32_t *my = oamax_part + (int64_t)blockIdx.x * PN;
+        if (Po == FAST_BM) {
+#pragma unroll
+            for (int j = 0; j < FAST_NJ; ++j)
+                if (mo.on[j]) {
+                    const int jj = OQ ? j : 0;
+                    uint4 v;
+                    v.x = oamx[jj][0], v.y = oamx[jj][1], v.z = oamx[jj][2], v.w = oamx[jj][3];
+                    *(uint4 *)(my + otix[jj]) = v;
+                }
+        } else {
+            uint32_t *tab = (uint32_t *)&ys[0][0];
+            __syncthreads();
+            for (int t = tid; t < PN; t += 256) tab[t] = 0;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < FAST_NJ; ++j)
+                if (mo.on[j])
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) atomicMax(&tab[otix[OQ ? j : 0] + e], oamx[OQ ? j : 0][e]);
+            __syncthreads();
+            for (int t = tid; t < PN; t += 256) my[t] = tab[t];
+        }
     }
 }
 
@@ -930,9 +1012,16 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     // !ZVEC - N not a multiple of 4, or unaligned gradient rows: the gradient tile is staged in groups of four columns
     // of the width rounded up, each element with a load of its own (columns past N read as zero)
     mx.init(K), mz.init((N + 3) & ~3);
-    int fi[FAST_NJ][4], tix[FAST_NJ];
+    // fractional bits of the staged elements, four to a register (unpacked per tile: sixteen values and their negations
+    // would otherwise each hold a register for the whole launch)
+    int fip[FAST_NJ];
     float gf[FAST_NJ][4];
-    fast_frac_bits<QUANT>(f_in, P, K, mx, m.round_params, fi, tix);
+    {
+        int fi[FAST_NJ][4], tix[FAST_NJ];
+        fast_frac_bits<QUANT>(f_in, P, K, mx, m.round_params, fi, tix);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) fip[j] = pack_i8x4(fi[j]);
+    }
 #pragma unroll
     for (int j = 0; j < FAST_NJ; ++j)
 #pragma unroll
@@ -996,9 +1085,11 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         for (int j = 0; j < FAST_NJ; ++j) {
             const float v[4] = {rx[j][0], rx[j][1], rx[j][2], rx[j][3]};
             const int xr = mx.on[j] ? mx.row[j] : FAST_BM, zr = mz.on[j] ? mz.row[j] : FAST_BM;
+            asm volatile("" : "+v"(fip[j]));
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float q = QUANT ? ldexpf(round_scaled<RM>(ldexpf(v[e], fi[j][e])), -fi[j][e]) : v[e];
+                const int f = unpack_i8(fip[j], e);
+                const float q = QUANT ? ldexpf(round_scaled<RM>(ldexpf(v[e], f)), -f) : v[e];
                 dlt[j][e] = q - v[e];
                 xs[xr][mx.col[j] + e] = q;
             }
@@ -1353,6 +1444,45 @@ extern "C" int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_i
         });
     }
     return check_launch("hgq_qdense_fwd");
+}
+
+// 1 if hgq_qdense_fwd_oq covers the shape and modes
+extern "C" int hgq_qdense_fwd_oq_supported(int64_t rows, int K, int N, int64_t bw_rows, int64_t bw_rows_out, int mode, int mode_out) {
+    const Mode m(mode), mo(mode_out);
+    const bool wrap_in = m.overflow_mode == HGQ_WRAP && m.training && !m.kbi;
+    const bool wrap_out = mo.overflow_mode == HGQ_WRAP && mo.training && !mo.kbi;
+    return g_dense_bf16 && rows > 0 && K >= 1 && N >= 1 && K <= 64 && N <= 64 && K % 4 == 0 && N % 4 == 0 && wrap_in && wrap_out &&
+           m.round_mode == mo.round_mode && (m.round_mode == HGQ_TRN || m.round_mode == HGQ_RND || m.round_mode == HGQ_RND_CONV) &&
+           bw_rows > 0 && bw_rows <= 64 && 64 % bw_rows == 0 && rows % bw_rows == 0 &&
+           bw_rows_out > 0 && bw_rows_out <= 64 && 64 % bw_rows_out == 0 && rows % bw_rows_out == 0;
+}
+
+extern "C" int hgq_qdense_fwd_oq(const float *x, const float *f_in, int64_t bw_rows, const float *qw, const float *qb, const float *f_out,
+                                 int64_t bw_rows_out, float *y, float *yq, uint32_t *amax_part, uint32_t *oamax_part, int64_t rows,
+                                 int K, int N, int act, int mode, int mode_out, void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (rows == 0) return HGQ_OK;
+    if (!hgq_qdense_fwd_oq_supported(rows, K, N, bw_rows, bw_rows_out, mode, mode_out))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_fwd_oq: shape or modes outside the fused output quantizer (see hgq_qdense_fwd_oq_supported)");
+    if (!x || !f_in || !qw || !f_out || !y || !yq || !oamax_part) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_oq: null pointer");
+    if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_oq: unknown activation %d", act);
+    if (!aligned16(x) || !aligned16(y) || !aligned16(yq) || !aligned16(oamax_part))
+        return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_oq: x, y, yq and the tracker slices must be 16-byte aligned");
+    const Mode m(mode);
+    const dim3 fgrid((unsigned)row_parts(rows, FWD_BM));
+    const int P = (int)bw_rows, Po = (int)bw_rows_out;
+#define HGQ_FWD_OQ(NSV) \
+    do { \
+        if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, true, NSV, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, f_out, Po, mode_out, yq, oamax_part); \
+        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND, true, NSV, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, f_out, Po, mode_out, yq, oamax_part); \
+        else hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND_CONV, true, NSV, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, f_out, Po, mode_out, yq, oamax_part); \
+    } while (0)
+    if (K <= 16) HGQ_FWD_OQ(1);
+    else if (K <= 32) HGQ_FWD_OQ(2);
+    else if (K <= 48) HGQ_FWD_OQ(3);
+    else HGQ_FWD_OQ(4);
+#undef HGQ_FWD_OQ
+    return check_launch("hgq_qdense_fwd_oq");
 }
 
 extern "C" int64_t hgq_qdense_moments_workspace(int64_t rows, int K, int N, int64_t bw_rows) {

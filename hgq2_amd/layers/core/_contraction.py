@@ -72,8 +72,13 @@ class DeferredTracking:
 FUSED_TRACK_MAX = 65536  # slices * entries the single-workgroup EBOPs kernel is allowed to walk
 
 
-def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training):
-    """x [..., K] -> [rows, N].  Returns ``(y, activation applied, DeferredTracking or None)``."""
+def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training, oq=None, out_shape=None):
+    """x [..., K] -> [rows, N].  Returns ``(y, activation applied, DeferredTracking or None, output quantizer applied)``.
+
+    ``oq`` / ``out_shape``: the layer's output quantizer and the shape it sees.  When it is of the kind the input
+    quantizer fusion takes (plain KIF on its WRAP training branch, a table over the trailing axes) and nothing but a relu
+    stands between the contraction and it, the contraction kernel applies it to the tile it stores and leaves its abs-max
+    trackers as slices; its integer bits are then updated here as its own call would."""
     K, N = qkernel2d.shape
     x2d = x.reshape(-1, K)
     if not x2d.is_contiguous():
@@ -83,19 +88,28 @@ def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training):
     fused_bwd = K <= ops.FUSED_BWD_MAX and N <= ops.FUSED_BWD_MAX
     if bw_rows and fused_bwd:
         q = iq.quantizer
+        po = 0
+        if oq is not None and out_shape is not None and act_name in (None, 'linear', 'relu'):
+            po = fused_iq_rows(oq, tuple(out_shape), N, training)
+        if po and _lib.load().hgq_qdense_fwd_oq_supported(x2d.shape[0], K, N, bw_rows, po, q._mode(True), oq.quantizer._mode(True)):
+            qo = oq.quantizer
+            yq, amax, oamax = ops.qdense_oq(x2d, q._k.view(-1), q._f.view(-1), qkernel2d, qbias1d, qo._k.view(-1), qo._i.view(-1),
+                                            qo._f.view(-1), act_code, q._mode(True), qo._mode(True), bw_rows, po)
+            qo._track(oamax, True)
+            return yq, act_code != _lib.ACT_NONE, DeferredTracking(q, amax), True
         y, amax = ops.qdense(x2d, q._k.view(-1), q._i.view(-1), q._f.view(-1), qkernel2d, qbias1d, act_code,
                              q._mode(True), bw_rows, True)
-        return y, act_code != _lib.ACT_NONE, DeferredTracking(q, amax)
+        return y, act_code != _lib.ACT_NONE, DeferredTracking(q, amax), False
     if iq is not None:
         x2d = iq(x, training=training).reshape(-1, K)
         if not x2d.is_contiguous():
             x2d = x2d.contiguous()
     if fused_bwd:
         y, _ = ops.qdense(x2d, None, None, None, qkernel2d, qbias1d, act_code, 0, 0, False)
-        return y, act_code != _lib.ACT_NONE, None
+        return y, act_code != _lib.ACT_NONE, None, False
     # shapes beyond the fused backward kernel: the implicit-GEMM kernels in their 1 x 1 form
     y = ops.matmul_bias_act(x2d, qkernel2d, qbias1d, act_code)
-    return y, act_code != _lib.ACT_NONE, None
+    return y, act_code != _lib.ACT_NONE, None, False
 
 
 def dense_ebops_term(layer, iq, kq, bq, K, N, bias_size, deferred):

@@ -70,7 +70,9 @@ class QDense(QLayerBaseSingleInput):
 
     def call(self, inputs, training=None):
         iq = self.iq if self.enable_iq else None
-        y, act_done, self._deferred = dense_contraction(inputs, iq, self.qkernel, self.qbias, self._act_name, training)
+        oq = self.oq if (self.enable_oq and not self.__output_quantizer_handled__) else None
+        y, act_done, self._deferred, self._oq_applied_in_call = dense_contraction(
+            inputs, iq, self.qkernel, self.qbias, self._act_name, training, oq, tuple(inputs.shape[:-1]) + (self.units,))
         y = y.view(*inputs.shape[:-1], self.units)
         if self.activation is not None and not act_done:
             y = self.activation(y)

@@ -147,7 +147,7 @@ class QEinsumDense(QLayerBaseSingleInput):
     def compute_output_shape(self, input_shape):
         return (input_shape[0],) + tuple(self.full_output_shape[1:])
 
-    def _contract(self, inputs, qkernel, qbias, training):
+    def _contract(self, inputs, qkernel, qbias, training, oq_ok=False):
         iq = self.iq if self.enable_iq else None
         if self._gemm is not None:
             nc, _ = self._gemm
@@ -159,7 +159,14 @@ class QEinsumDense(QLayerBaseSingleInput):
             for view, base in ((w2d, qkernel), (b1d, qbias)):
                 if view is not None and view is not base and getattr(base, '_hgq_single_use', False) and view._base is base:
                     view._hgq_single_use = True
-            y, act_done, self._deferred = dense_contraction(x, iq, w2d, b1d, fuse_act, training)
+            # the output quantizer can join the kernel when nothing but the fused activation follows the contraction
+            oq = None
+            if oq_ok and self.enable_oq and not self.__output_quantizer_handled__ and (qbias is None or self._bias_in_gemm):
+                oq = self.oq
+            y, act_done, self._deferred, oq_done = dense_contraction(x, iq, w2d, b1d, fuse_act, training, oq,
+                                                                     (inputs.shape[0],) + tuple(self.full_output_shape[1:]))
+            if oq_done:
+                self._oq_applied_in_call = True
             y = y.view(inputs.shape[0], *self.full_output_shape[1:])
             if qbias is not None and not self._bias_in_gemm:
                 y = ops.bias_add_rows(y, qbias)
@@ -174,7 +181,7 @@ class QEinsumDense(QLayerBaseSingleInput):
     def call(self, inputs, training=None):
         qkernel = self.kq(self._kernel, training=training)
         qbias = self.bq(self.bias, training=training) if self.bias is not None else None
-        y, act_done = self._contract(inputs, qkernel, qbias, training)
+        y, act_done = self._contract(inputs, qkernel, qbias, training, oq_ok=True)
         if self.activation is not None and not act_done:
             y = self.activation(y)
         return y

@@ -226,6 +226,38 @@ def _(x, k_in, i_in, f_in, qw, qb, act, mode, bw_rows, track):
     return x.new_empty((x.shape[0], qw.shape[1])), x.new_empty((0, 0), dtype=torch.int32)
 
 
+@torch.library.custom_op('hgq::qdense_fwd_oq', mutates_args=())
+def qdense_fwd_oq(x: Tensor, k_in: Tensor, f_in: Tensor, qw: Tensor, qb: Tensor, k_out: Tensor, f_out: Tensor, act: int,
+                  mode: int, mode_out: int, bw_rows: int, bw_rows_out: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """``qdense_fwd`` with the output quantizer on the tile as it leaves: ``(y, q_out(y), amax slices of the input
+    quantizer, amax slices of the output quantizer)``."""
+    _check_f32('x', x), _check_f32('qw', qw), _check_f32('f_in', f_in), _check_f32('f_out', f_out)
+    _need(x.dim() == 2 and qw.dim() == 2 and x.shape[1] == qw.shape[0], f'shape mismatch {tuple(x.shape)} @ {tuple(qw.shape)}')
+    rows, K = x.shape
+    N = qw.shape[1]
+    if qb.numel():
+        _check_f32('qb', qb)
+        _need(qb.numel() == N, 'bias size mismatch')
+    _need(f_in.numel() == bw_rows * K and f_out.numel() == bw_rows_out * N, 'fractional-bit tables must be [bw_rows, K] and [bw_rows_out, N]')
+    mode, mode_out = _kmode(mode, k_in), _kmode(mode_out, k_out)
+    lib = _lib.load()
+    y, yq = torch.empty((rows, N), dtype=torch.float32, device=x.device), torch.empty((rows, N), dtype=torch.float32, device=x.device)
+    parts = lib.hgq_qdense_fwd_parts(rows)
+    amax = torch.empty((parts, bw_rows * K), dtype=torch.int32, device=x.device)
+    oamax = torch.empty((parts, bw_rows_out * N), dtype=torch.int32, device=x.device)
+    rc = lib.hgq_qdense_fwd_oq(_ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(qb), _ptr(f_out), bw_rows_out, _ptr(y), _ptr(yq), _ptr(amax),
+                               _ptr(oamax), rows, K, N, act, mode, mode_out, _stream())
+    _lib.check(rc, 'hgq_qdense_fwd_oq')
+    return y, yq, amax, oamax
+
+
+@qdense_fwd_oq.register_fake
+def _(x, k_in, f_in, qw, qb, k_out, f_out, act, mode, mode_out, bw_rows, bw_rows_out):
+    rows, N = x.shape[0], qw.shape[1]
+    return (x.new_empty((rows, N)), x.new_empty((rows, N)), x.new_empty((1, f_in.numel()), dtype=torch.int32),
+            x.new_empty((1, f_out.numel()), dtype=torch.int32))
+
+
 @torch.library.custom_op('hgq::qdense_bwd', mutates_args=())
 def qdense_bwd(dy: Tensor, y: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_bias: bool, act: int, mode: int,
                bw_rows: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
@@ -1376,34 +1408,40 @@ class _Quantize(torch.autograd.Function):
     def backward(ctx, gy, _ga, _gn):
         if gy is None:
             return (None,) * 7
-        if not (ctx.mode & _lib.MODE_TRAINING):
-            raise RuntimeError('hgq quantizer: gradients are defined for the training-mode forward only')
-        x, k, i, fb = ctx.saved_tensors
-        gy = gy.contiguous()
-        # a WRAP quantizer in training mode only rounds: the gradient passes straight through to x
-        # and (unless f = b - i) none reaches the integer bits, so the kernel writes neither
-        wrap = ((ctx.mode >> 4) & 0xf) == _lib.WRAP
-        need_dx = ctx.needs_input_grad[0] and not wrap
-        need_di = ctx.needs_input_grad[2] and (not wrap or bool(ctx.mode & _lib.MODE_KBI))
-        o_i, o_fb = ctx.owners
-        if (_SINK['open'] and ctx.needs_input_grad[3] and _can_route(o_fb, fb.numel()) and (not need_di or _can_route(o_i, i.numel()))
-                and (need_di or not ctx.needs_input_grad[2]) and quantize_bwd_slices_supported(gy, x, k, i, fb, ctx.bw_inner)):
-            # the bit-width gradients go to the optimizer and nowhere else: their slices join the pass's one reduction launch
-            dx, ws = quantize_bwd_slices(gy, x, k, i, fb, ctx.mode, ctx.bw_inner, need_dx, need_di)
-            dfb, di = torch.empty_like(fb), (torch.empty_like(i) if need_di else None)
-            e = fb.new_empty(0)
-            _PENDING_REDUCE.append((ws, (dfb.view(-1), di.view(-1) if need_di else e, e), (False, not need_di, True)))
-            _route(o_fb, dfb)
-            if need_di:
-                _route(o_i, di)
-            return (gy if wrap else dx) if ctx.needs_input_grad[0] else None, None, None, None, None, None, None
-        dx, di, dfb = quantize_bwd(gy, x, k, i, fb, ctx.mode, ctx.bw_inner, need_dx, need_di)
-        if ctx.needs_input_grad[0] and wrap:
-            dx = gy
-        if ctx.needs_input_grad[2] and not need_di:
-            di = torch.zeros_like(i)
-        return (dx if ctx.needs_input_grad[0] else None, None, di if ctx.needs_input_grad[2] else None,
-                dfb if ctx.needs_input_grad[3] else None, None, None, None)
+        return _quantize_backward(ctx, gy, ctx.needs_input_grad[0], ctx.needs_input_grad[2], ctx.needs_input_grad[3])
+
+
+def _quantize_backward(ctx, gy, want_x, want_i, want_fb):
+    """Backward of a training-mode quantizer call; ``ctx`` holds (x, k, i, fb), mode, bw_inner and the owners of i, fb.
+    Returns the 7-tuple of ``_Quantize``'s inputs."""
+    if not (ctx.mode & _lib.MODE_TRAINING):
+        raise RuntimeError('hgq quantizer: gradients are defined for the training-mode forward only')
+    x, k, i, fb = ctx.saved_tensors
+    gy = gy.contiguous()
+    # a WRAP quantizer in training mode only rounds: the gradient passes straight through to x
+    # and (unless f = b - i) none reaches the integer bits, so the kernel writes neither
+    wrap = ((ctx.mode >> 4) & 0xf) == _lib.WRAP
+    need_dx = want_x and not wrap
+    need_di = want_i and (not wrap or bool(ctx.mode & _lib.MODE_KBI))
+    o_i, o_fb = ctx.owners
+    if (_SINK['open'] and want_fb and _can_route(o_fb, fb.numel()) and (not need_di or _can_route(o_i, i.numel()))
+            and (need_di or not want_i) and quantize_bwd_slices_supported(gy, x, k, i, fb, ctx.bw_inner)):
+        # the bit-width gradients go to the optimizer and nowhere else: their slices join the pass's one reduction launch
+        dx, ws = quantize_bwd_slices(gy, x, k, i, fb, ctx.mode, ctx.bw_inner, need_dx, need_di)
+        dfb, di = torch.empty_like(fb), (torch.empty_like(i) if need_di else None)
+        e = fb.new_empty(0)
+        _PENDING_REDUCE.append((ws, (dfb.view(-1), di.view(-1) if need_di else e, e), (False, not need_di, True)))
+        _route(o_fb, dfb)
+        if need_di:
+            _route(o_i, di)
+        return (gy if wrap else dx) if want_x else None, None, None, None, None, None, None
+    dx, di, dfb = quantize_bwd(gy, x, k, i, fb, ctx.mode, ctx.bw_inner, need_dx, need_di)
+    if want_x and wrap:
+        dx = gy
+    if want_i and not need_di:
+        di = torch.zeros_like(i)
+    return (dx if want_x else None, None, di if want_i else None,
+            dfb if want_fb else None, None, None, None)
 
 
 @torch.library.custom_op('hgq::quantize_fwd_stochastic', mutates_args=())
@@ -1636,6 +1674,62 @@ def qdense(x2d, k_in, i_in, f_in, qw, qb, act: int, mode: int, bw_rows: int, tra
     empty = x2d.new_empty(0)
     return _QDense.apply(x2d, k_in if k_in is not None else empty, i_in if i_in is not None else empty,
                          f_in if f_in is not None else empty, qw, qb if qb is not None else empty, act, mode, bw_rows, track)
+
+
+class _QDenseOQ(torch.autograd.Function):
+    """``_QDense`` whose forward kernel also runs the layer's output quantizer: returns ``(y, yq, amax, oamax)`` with the
+    gradient of ``_QDense`` on ``y``; ``yq`` carries no gradient here - ``_QuantizeGiven`` ties it to ``y``."""
+
+    @staticmethod
+    def forward(ctx, x, k_in, f_in, qw, qb, k_out, f_out, act, mode, mode_out, bw_rows, bw_rows_out):
+        y, yq, amax, oamax = qdense_fwd_oq(x, k_in, f_in, qw, qb, k_out, f_out, act, mode, mode_out, bw_rows, bw_rows_out)
+        ctx.f_owner = _owner(f_in)
+        ctx.save_for_backward(x, f_in, qw, y)
+        ctx.has_bias = qb.numel() > 0
+        ctx.defer = getattr(qw, '_hgq_single_use', False) and (qb.numel() == 0 or getattr(qb, '_hgq_single_use', False))
+        ctx.act, ctx.mode, ctx.bw_rows, ctx.f_shape = act, _kmode(mode, k_in), bw_rows, f_in.shape
+        ctx.mark_non_differentiable(yq, amax, oamax)
+        ctx.set_materialize_grads(False)
+        return y, yq, amax, oamax
+
+    @staticmethod
+    def backward(ctx, gy, _gq, _ga, _go):
+        if gy is None:
+            return (None,) * 12
+        dx, _, _, df, dqw, dqb, _, _, _, _ = _QDense.backward(ctx, gy, None)
+        return dx, None, df, dqw, dqb, None, None, None, None, None, None, None
+
+
+class _QuantizeGiven(torch.autograd.Function):
+    """A quantizer call whose forward another kernel has already run (``yq`` = the quantized ``x``): hands ``yq`` on with
+    the backward of ``_Quantize``."""
+
+    @staticmethod
+    def forward(ctx, x, yq, k, i, fb, mode, bw_inner):
+        ctx.save_for_backward(x, k, i, fb)
+        ctx.mode, ctx.bw_inner = mode, bw_inner
+        ctx.owners = (_owner(i), _owner(fb))
+        ctx.set_materialize_grads(False)
+        return yq.view_as(yq)
+
+    @staticmethod
+    def backward(ctx, gy):
+        if gy is None:
+            return (None,) * 7
+        dx, _, di, dfb, _, _, _ = _quantize_backward(ctx, gy, ctx.needs_input_grad[0], ctx.needs_input_grad[3], ctx.needs_input_grad[4])
+        return dx, None, None, di, dfb, None, None
+
+
+def qdense_oq(x2d, k_in, f_in, qw, qb, k_out, i_out, f_out, act: int, mode: int, mode_out: int, bw_rows: int, bw_rows_out: int):
+    """``q_out(act(q_in(x) @ qw + qb))`` on a [rows, K] view with both quantizers (KIF, WRAP, training mode: they only
+    round) inside the contraction kernel; returns ``(yq, amax slices of the input quantizer, amax slices of the output
+    quantizer)``.  The backward is the output quantizer's own (its fractional-bit gradient from the stored ``y``; the data
+    gradient passes unchanged) followed by the contraction's."""
+    empty = x2d.new_empty(0)
+    y, yq, amax, oamax = _QDenseOQ.apply(x2d, k_in, f_in, qw, qb if qb is not None else empty, k_out, f_out, act, mode, mode_out,
+                                         bw_rows, bw_rows_out)
+    yq = _QuantizeGiven.apply(y, yq, k_out, i_out, f_out, _kmode(mode_out, k_out), 1)
+    return yq, amax, oamax
 
 
 class _DenseEbops(torch.autograd.Function):

@@ -250,6 +250,21 @@ int hgq_qdense_fwd_parts(int64_t rows);
  * Process-wide, not synchronised with launches in flight on other threads.
  */
 int hgq_dense_use_bf16_parts(int on);
+/*
+ * hgq_qdense_fwd with the layer's output quantizer run on the output tile as it leaves (reference
+ * src/hgq/layers/core/base.py:106-116: `return self.oq(r, training=training)` after the layer's call): `y` gets
+ * act(q_in(x) W + b), `yq` its quantized values, slice w of `oamax_part` ([hgq_qdense_fwd_parts(rows)][bw_rows_out * N]
+ * words, every slice written whole) the abs-max bit patterns of the quantized values per table entry, for
+ * hgq_wrap_track_i.  Covers what hgq_qdense_fwd_oq_supported says: both quantizers KIF on their WRAP training branch
+ * (round only) with the same round mode, fractional-bit tables [bw_rows, K] and [bw_rows_out, N] whose row counts divide
+ * 64 and the rows, K and N multiples of 4 up to 64, the bf16-part kernels selected; HGQ_ERR_UNSUPPORTED otherwise
+ * (run hgq_qdense_fwd and hgq_quantize_fwd then).  The gradient is the two separate ones: hgq_quantize_bwd* on (dyq, y),
+ * which passes dyq through unchanged, then hgq_qdense_bwd.
+ */
+int hgq_qdense_fwd_oq_supported(int64_t rows, int K, int N, int64_t bw_rows, int64_t bw_rows_out, int mode, int mode_out);
+int hgq_qdense_fwd_oq(const float *x, const float *f_in, int64_t bw_rows, const float *qw, const float *qb, const float *f_out,
+                      int64_t bw_rows_out, float *y, float *yq, uint32_t *amax_part, uint32_t *oamax_part, int64_t rows, int K,
+                      int N, int act, int mode, int mode_out, void *stream);
 int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_in, const float *f_in, int64_t bw_rows,
                    const float *qw, const float *qb, float *y, uint32_t *amax_part, int64_t rows, int K, int N,
                    int act, int mode, void *stream);

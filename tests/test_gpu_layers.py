@@ -729,3 +729,106 @@ def test_train_step_for_picks_the_path_and_both_paths_agree(dev):
     assert train_step_for(stack([16, 4]), x, target, loss='mse').path == 'layers_graph'
     with pytest.raises(ValueError):
         train_step_for(stack([80, 4]), x, labels, fused=True)
+
+
+@pytest.mark.parametrize('kind', ['dense_relu', 'einsum', 'einsum_small_table'])
+def test_output_quantizer_inside_the_dense_kernel(dev, kind):
+    """A layer's output quantizer of the fusable kind (plain KIF, WRAP, training) runs inside the contraction kernel.
+    The same layer with the bf16-part kernels switched off takes the separate launches: outputs, tracked integer bits of
+    both quantizers and EBOPs agree bit for bit (operands of a few bits: the contraction is exact either way), gradients
+    to the order of fp32 sums."""
+    import io
+
+    from hgq2_amd import _lib, ops, saving
+    from hgq2_amd.config import LayerConfigScope, QuantizerConfigScope
+    from hgq2_amd.core import Sequential
+    from hgq2_amd.layers import QDense, QEinsumDense
+    from hgq2_amd.train import SGD, model_loss
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(3)
+    torch.manual_seed(3)
+    with QuantizerConfigScope(place='all', default_q_type='kbi', overflow_mode='SAT_SYM'), \
+            QuantizerConfigScope(place='datalane', default_q_type='kif', overflow_mode='WRAP'), \
+            LayerConfigScope(enable_ebops=True, beta0=1e-5):
+        if kind == 'dense_relu':
+            x = torch.randn(300, 24, generator=g)
+            layers = [QDense(32, activation='relu', enable_oq=True), QDense(8, enable_oq=True)]
+        elif kind == 'einsum':
+            x = torch.randn(70, 64, 16, generator=g)
+            layers = [QEinsumDense('bpf,fnh->bpnh', (64, 4, 8), bias_axes='nh', enable_oq=True)]
+        else:
+            x = torch.randn(130, 16, 20, generator=g)
+            layers = [QEinsumDense('bpf,fh->bph', (16, 12), bias_axes='h', activation='relu', enable_oq=True)]
+    model = Sequential(layers)
+    x = x.to(dev)
+    model(x, training=True)
+    with torch.no_grad():
+        for layer in layers:
+            f = layer.oq.quantizer._f
+            f.add_(torch.randint(-2, 3, f.shape, generator=g).float().to(dev))
+    buf = io.BytesIO()
+    saving.save_model(model, buf)
+    buf.seek(0)
+    clone = saving.load_model(buf, device=dev)
+    up = torch.randn(model(x, training=False).shape, generator=g).to(dev)
+    buf.seek(0)
+    saving.load_weights(model, buf)
+
+    def run(m, steps=2):
+        opt = SGD(m.parameters(), lr=0.05, fold_regularizers=True)
+        outs = []
+        for _ in range(steps):
+            opt.zero_grad()
+            y = m(x, training=True)
+            outs.append(y.detach().clone())
+            loss = model_loss(m, ops.mse(y * up), True)
+            opt.backward(loss)
+            opt.step()
+        return outs
+
+    launches = []
+    real = ops.qdense_fwd_oq
+
+    def spy(*a, **k):
+        launches.append(1)
+        return real(*a, **k)
+
+    ops.qdense_fwd_oq = spy
+    try:
+        fused = run(model)
+        n_fused = len(launches)
+        was = lib.hgq_dense_use_bf16_parts(0)
+        try:
+            plain = run(clone)
+        finally:
+            lib.hgq_dense_use_bf16_parts(was)
+    finally:
+        ops.qdense_fwd_oq = real
+    assert n_fused == 2 * len(layers) and len(launches) == n_fused, 'the fused kernel runs exactly where it is switched on'
+    for a, b in zip(fused, plain):
+        assert torch.equal(a, b)
+    for la, lb in zip(model.layers, clone.layers):
+        assert torch.equal(la.oq.quantizer._i, lb.oq.quantizer._i) and torch.equal(la.iq.quantizer._i, lb.iq.quantizer._i)
+        assert int(la._ebops.view(torch.int32)) == int(lb._ebops.view(torch.int32))
+    for (name, pa), (_, pb) in zip(model.named_parameters(), clone.named_parameters()):
+        err = (pa.detach().double() - pb.detach().double()).abs().max().item()
+        assert err <= 2e-5 * (pb.detach().abs().max().item() + 1e-6), (name, err)
+
+    # plain autograd (no gradient sink): the one-pass backward reduces its own slices and hands every gradient back
+    def grads(m):
+        for p_ in m.parameters():
+            p_.grad = None
+        model_loss(m, ops.mse(m(x, training=True) * up)).backward()
+        return {n: p_.grad.detach().clone() for n, p_ in m.named_parameters() if p_.grad is not None}
+
+    ga = grads(model)
+    was = lib.hgq_dense_use_bf16_parts(0)
+    try:
+        gb = grads(clone)
+    finally:
+        lib.hgq_dense_use_bf16_parts(was)
+    assert ga.keys() == gb.keys() and any('oq' in n and n.endswith('_f') for n in ga)
+    for n in ga:
+        err = (ga[n].double() - gb[n].double()).abs().max().item()
+        assert err <= 2e-5 * (gb[n].abs().max().item() + 1e-6), (n, err)
