@@ -1300,8 +1300,19 @@ extern "C" int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F) {
     return slices * ((int64_t)K * F + F);
 }
 
-extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw,
-                              float *dqb, float *workspace, const hgq_conv_geom *g, int F, int act, void *stream) {
+extern "C" int64_t hgq_conv2d_bwd_slice_count(const hgq_conv_geom *g, int F) {
+    if (check_geom(g, F, "hgq_conv2d_bwd_slice_count")) return -1;
+    const int64_t rows = (int64_t)g->B * g->OH * g->OW;
+    if (rows == 0) return 1;
+    if (bwd_smallc_ok(*g, F)) return bwd_smallc_grid(*g);
+    const WgradCfg c = wgrad_cfg(g->kh * g->kw * g->C, F);
+    return wgrad_splits(rows, c.n_kt * c.n_nt);
+}
+
+// reduce: the slices of the kernel / bias gradient are summed into dqw / dqb; otherwise they stay in `workspace`
+// ([hgq_conv2d_bwd_slice_count][kh kw C F + F]) and dqw / dqb only say whether the gradient is wanted
+static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
+                           float *workspace, const hgq_conv_geom *g, int F, int act, void *stream, bool reduce) {
     int rc = check_geom(g, F, "hgq_conv2d_bwd");
     if (rc) return rc;
     if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: unknown activation %d", act);
@@ -1330,7 +1341,7 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
         HGQ_SMALLC_DISPATCH(HGQ_BWD_SC);
 #undef HGQ_BWD_SC
         if ((rc = check_launch("hgq_conv2d_bwd(few channels)"))) return rc;
-        if (want_w) return reduce_parts(workspace, grid, KF + F, dqw, KF, dqb, (int64_t)F, nullptr, 0, s);
+        if (want_w && reduce) return reduce_parts(workspace, grid, KF + F, dqw, KF, dqb, (int64_t)F, nullptr, 0, s);
         return HGQ_OK;
     }
     if (dxq) {
@@ -1389,9 +1400,25 @@ extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, 
 #undef HGQ_WGRAD
         if ((rc = check_launch("hgq_conv2d_bwd(weights)"))) return rc;
         const int64_t M = KF + F;
-        if ((rc = reduce_parts(workspace, (int)splits, M, dqw, KF, dqb, (int64_t)F, nullptr, 0, s))) return rc;
+        if (reduce && (rc = reduce_parts(workspace, (int)splits, M, dqw, KF, dqb, (int64_t)F, nullptr, 0, s))) return rc;
     }
     return HGQ_OK;
+}
+
+extern "C" int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw,
+                              float *dqb, float *workspace, const hgq_conv_geom *g, int F, int act, void *stream) {
+    return conv2d_bwd_impl(dy, y, xq, qw, dxq, dqw, dqb, workspace, g, F, act, stream, true);
+}
+
+extern "C" int hgq_conv2d_bwd_slices(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *workspace,
+                                     const hgq_conv_geom *g, int F, int act, void *stream) {
+    if (!workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd_slices: null workspace");
+    if (g && (int64_t)g->B * g->OH * g->OW == 0) {  // nothing to add up: one slice of zeros
+        const int rc = check_geom(g, F, "hgq_conv2d_bwd_slices");
+        return rc ? rc : fill_f32(workspace, 0.f, hgq_conv2d_bwd_slice_count(g, F) * ((int64_t)g->kh * g->kw * g->C * F + F), (hipStream_t)stream);
+    }
+    // the kernels only test the gradient pointers for "is it wanted": any non-null value stands for it
+    return conv2d_bwd_impl(dy, y, xq, qw, dxq, workspace, workspace, workspace, g, F, act, stream, false);
 }
 
 extern "C" int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, const hgq_conv_geom *g, int F, float *total,

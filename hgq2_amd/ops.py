@@ -995,6 +995,29 @@ def _(dy, y, xq, qw, geom, act, need_dx, has_bias):
     return (xq.new_empty(xq.shape if need_dx else (0,)), torch.empty_like(qw), xq.new_empty(qw.shape[-1] if has_bias else 0))
 
 
+@torch.library.custom_op('hgq::conv2d_bwd_slices', mutates_args=())
+def conv2d_bwd_slices(dy: Tensor, y: Tensor, xq: Tensor, qw: Tensor, geom: Sequence[int], act: int, need_dx: bool) -> tuple[Tensor, Tensor]:
+    """The convolution backward without the sum over its slices: ``(dx, slices [n, kh kw C F + F])``."""
+    _check_f32('dy', dy), _check_f32('y', y), _check_f32('xq', xq), _check_f32('qw', qw)
+    g = _geom(geom)
+    F = qw.shape[-1]
+    _need(dy.numel() == g.B * g.OH * g.OW * F and y.numel() == dy.numel(), 'dy / y must be [B, OH, OW, F]')
+    lib = _lib.load()
+    dx = torch.empty(xq.shape if need_dx else (0,), dtype=torch.float32, device=xq.device)
+    n = lib.hgq_conv2d_bwd_slice_count(ctypes.addressof(g), F)
+    _need(n >= 1, 'hgq_conv2d_bwd_slice_count rejected the geometry')
+    ws = torch.empty((int(n), qw.numel() + F), dtype=torch.float32, device=xq.device)
+    rc = lib.hgq_conv2d_bwd_slices(_ptr(dy), _ptr(y), _ptr(xq), _ptr(qw), _ptr(dx) if need_dx else None, _ptr(ws), ctypes.addressof(g), F,
+                                   act, _stream())
+    _lib.check(rc, 'hgq_conv2d_bwd_slices')
+    return dx, ws
+
+
+@conv2d_bwd_slices.register_fake
+def _(dy, y, xq, qw, geom, act, need_dx):
+    return xq.new_empty(xq.shape if need_dx else (0,)), xq.new_empty((1, qw.numel() + qw.shape[-1]))
+
+
 @torch.library.custom_op('hgq::col_moments_fwd', mutates_args=())
 def col_moments_fwd(x: Tensor) -> tuple[Tensor, Tensor]:
     _check_f32('x', x)
@@ -1912,12 +1935,21 @@ class _Conv2D(torch.autograd.Function):
         y = conv2d_fwd(xq, qw, qb, list(geom), act)
         ctx.save_for_backward(xq, qw, y)
         ctx.geom, ctx.act, ctx.has_bias = tuple(geom), act, qb.numel() > 0
+        # both operands were handed out once by the model-wide weight-quantizer launch: their only reader is its backward
+        ctx.defer = getattr(qw, '_hgq_single_use', False) and (qb.numel() == 0 or getattr(qb, '_hgq_single_use', False))
         return y
 
     @staticmethod
     def backward(ctx, gy):
         xq, qw, y = ctx.saved_tensors
-        dx, dqw, dqb = conv2d_bwd(gy.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, ctx.needs_input_grad[0], ctx.has_bias)
+        if ctx.defer and _SINK['open']:
+            # kernel and bias gradient are first read by the backward of the prefetched quantizers: their slices join the
+            # pass's one reduction launch
+            dx, ws = conv2d_bwd_slices(gy.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, ctx.needs_input_grad[0])
+            dqw, dqb = torch.empty_like(qw), xq.new_empty(qw.shape[-1])
+            _PENDING_REDUCE.append((ws, (dqw.view(-1), dqb, xq.new_empty(0)), (False, not ctx.has_bias, True)))
+        else:
+            dx, dqw, dqb = conv2d_bwd(gy.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, ctx.needs_input_grad[0], ctx.has_bias)
         return (dx if ctx.needs_input_grad[0] else None, dqw, dqb if ctx.has_bias else None, None, None)
 
 
@@ -1934,8 +1966,10 @@ def matmul_bias_act(x2d: Tensor, qw: Tensor, qb, act: int = 0) -> Tensor:
     rows, K = x2d.shape
     N = qw.shape[1]
     geom = (rows, 1, 1, K, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1)
-    y = _Conv2D.apply(x2d.contiguous(), qw.contiguous().view(1, 1, K, N), qb.contiguous() if qb is not None else x2d.new_empty(0),
-                      geom, act)
+    w4 = qw.contiguous().view(1, 1, K, N)
+    if getattr(qw, '_hgq_single_use', False) and w4._base is qw:
+        w4._hgq_single_use = True  # a view's gradient goes back through the view unread: the one-reader mark holds for it
+    y = _Conv2D.apply(x2d.contiguous(), w4, qb.contiguous() if qb is not None else x2d.new_empty(0), geom, act)
     return y.view(rows, N)
 
 

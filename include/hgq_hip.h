@@ -569,6 +569,14 @@ int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb, float *y, 
 int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F);
 int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
                    float *workspace, const hgq_conv_geom *g, int F, int act, void *stream);
+/*
+ * hgq_conv2d_bwd without the sum over the slices: dxq is written, the kernel / bias gradient stays in `workspace` as
+ * hgq_conv2d_bwd_slice_count(g, F) slices of [kh kw C F | F] floats (every slice written whole), for a caller that adds the
+ * slices of several layers in one launch (hgq_reduce_slices_multi).  Same reference lines as hgq_conv2d_bwd.
+ */
+int64_t hgq_conv2d_bwd_slice_count(const hgq_conv_geom *g, int F);
+int hgq_conv2d_bwd_slices(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *workspace,
+                          const hgq_conv_geom *g, int F, int act, void *stream);
 
 /*
  * One quantizer's bit-width view for the EBOPs entry points below: `bits` / `fbits` as hgq_qbits_fwd forms
