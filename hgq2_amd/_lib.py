@@ -63,6 +63,8 @@ SIGNATURES = {
     'hgq_qbits_fwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     'hgq_qbits_bwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p]),
     'hgq_bn_fold_fwd': (c_int, [c_void_p] * 5 + [c_int, c_float] + [c_void_p] * 4 + [c_float, c_float, c_int, c_int, c_void_p]),
+    'hgq_bn_fold_quant_fwd': (c_int, [c_void_p] * 5 + [c_int, c_float] + [c_void_p] * 6 + [c_float, c_float, c_int, c_int, c_void_p]),
+    'hgq_bn_fold_quant_bwd': (c_int, [c_void_p] * 5 + [c_int, c_float] + [c_void_p] * 13 + [c_int, c_int, c_void_p]),
     'hgq_bn_fold_bwd': (c_int, [c_void_p] * 4 + [c_int, c_float] + [c_void_p] * 7 + [c_int, c_int, c_void_p]),
     'hgq_qdense_moments_workspace': (c_int64, [c_int64, c_int, c_int, c_int64]),
     'hgq_qdense_moments_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),

@@ -957,11 +957,6 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bf16_kernel(const float 
     }
 }
 
-__global__ __launch_bounds__(256) void moments_scale_kernel(float *mean, float *meansq, int N, float inv_rows) {
-    const int t = blockIdx.x * 256 + threadIdx.x;
-    if (t < N) mean[t] *= inv_rows, meansq[t] *= inv_rows;
-}
-
 // Backward.  Per tile: stage dz = dy (masked by y for ReLU) and the quantized input; dx = dz W^T
 // and dW += xq^T dz on MFMA; dx goes back through LDS so that it is stored with 128-bit writes and
 // meets the rounding residue (xq - x) of the staging thread for the fractional-bit gradient.
@@ -1240,7 +1235,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 #define RP_G 16  // slice groups per entry: 64 entries x 16 groups = 1024 threads, few dependent load batches per thread
 __global__ __launch_bounds__(64 * RP_G) void reduce_parts_kernel(const float *__restrict__ part, int n_parts, int64_t M,
                                                                  float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb,
-                                                                 float *df, int64_t n_df) {
+                                                                 float *df, int64_t n_df, float scale) {
     __shared__ float red[64 * RP_G];
     const int e_local = threadIdx.x & 63, grp = threadIdx.x >> 6;
     const int64_t e = (int64_t)blockIdx.x * 64 + e_local;
@@ -1265,6 +1260,7 @@ __global__ __launch_bounds__(64 * RP_G) void reduce_parts_kernel(const float *__
 #pragma unroll
         for (int w = 0; w < RP_G; w += 4)
             v += (red[e_local + 64 * w] + red[e_local + 64 * (w + 1)]) + (red[e_local + 64 * (w + 2)] + red[e_local + 64 * (w + 3)]);
+        v *= scale;
         if (e < n_dqw) {
             if (dqw) dqw[e] = v;
         } else if (e < n_dqw + n_dqb) {
@@ -1276,8 +1272,8 @@ __global__ __launch_bounds__(64 * RP_G) void reduce_parts_kernel(const float *__
 }
 
 int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb, float *df,
-                 int64_t n_df, hipStream_t s) {
-    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(64 * RP_G), 0, s, part, n_parts, M, dqw, n_dqw, dqb, n_dqb, df, n_df);
+                 int64_t n_df, hipStream_t s, float scale) {
+    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(64 * RP_G), 0, s, part, n_parts, M, dqw, n_dqw, dqb, n_dqb, df, n_df, scale);
     return check_launch("reduce_parts");
 }
 
@@ -1547,9 +1543,8 @@ extern "C" int hgq_qdense_moments_fwd(const float *x, const float *f_in, int64_t
 #undef HGQ_MOM_FAST
 #undef HGQ_MOM_BF16
     if ((rc = check_launch("hgq_qdense_moments_fwd"))) return rc;
-    if ((rc = reduce_parts(workspace, parts, 2 * (int64_t)N, mean, (int64_t)N, meansq, (int64_t)N, nullptr, 0, s))) return rc;
-    hipLaunchKernelGGL(moments_scale_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, mean, meansq, N, 1.0f / (float)rows);
-    return check_launch("hgq_qdense_moments_fwd(scale)");
+    // the sums leave the reduction scaled by 1 / rows: mean and mean of squares
+    return reduce_parts(workspace, parts, 2 * (int64_t)N, mean, (int64_t)N, meansq, (int64_t)N, nullptr, 0, s, 1.0f / (float)rows);
 }
 
 extern "C" int hgq_dense_moments_fwd(const float *x, const float *w, float *mean, float *meansq, float *workspace, int64_t rows,
@@ -1678,7 +1673,7 @@ static int qdense_bwd_impl(const float *dy, const float *y, const float *x, cons
     int rc = check_launch("hgq_qdense_bwd");
     if (rc || !reduce) return rc;
     hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((M + 63) / 64)), dim3(64 * RP_G), 0, s, workspace, parts, M, dqw, (int64_t)K * N, dqb,
-                       (int64_t)N, quant ? df_in : (float *)nullptr, PK);
+                       (int64_t)N, quant ? df_in : (float *)nullptr, PK, 1.0f);
     return check_launch("hgq_qdense_bwd(reduce)");
 }
 

@@ -46,8 +46,9 @@ inline int fill_f32(float *p, float v, int64_t n, hipStream_t s) {
 
 // out[e] = sum over the n_parts slices of part[slice][e] (slice length M), in a fixed order; the
 // first n_dqw entries go to dqw, the next n_dqb to dqb, the remaining n_df to df (null = skip).
+// Every sum is multiplied by `scale` as it is stored (1: stored as it is).
 int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t n_dqw, float *dqb, int64_t n_dqb, float *df,
-                 int64_t n_df, hipStream_t s);
+                 int64_t n_df, hipStream_t s, float scale = 1.0f);
 
 // Convolution through LDS-resident operands (hgq_conv_patch.hip): mode 0 forward, 1 data gradient.
 bool conv_patch_ok(int mode, const hgq_conv_geom &g, int F);

@@ -256,19 +256,35 @@ __device__ __forceinline__ float bn_var(float mean, float second, int is_meansq)
     return is_meansq ? __fsub_rn(second, __fmul_rn(mean, mean)) : second;
 }
 
+// QUANT: the kernel and bias quantizers (per-element bit-widths, no trackers) follow in the same thread: fused_w / fused_b
+// then receive the QUANTIZED values (the folded ones are products the backward pass forms again, bit for bit).
+template <bool QUANT>
 __global__ __launch_bounds__(256) void bn_fold_fwd_kernel(const float *__restrict__ w, const float *__restrict__ bias,
                                                           const float *__restrict__ gamma, const float *__restrict__ mean,
                                                           const float *__restrict__ second, int is_meansq, float eps,
                                                           float *__restrict__ fused_w, float *__restrict__ fused_b, float *moving_mean,
-                                                          float *moving_var, float momentum, float one_minus_momentum, int K, int N) {
+                                                          float *moving_var, float momentum, float one_minus_momentum, int K, int N,
+                                                          hgq_qdesc qk, hgq_qdesc qb) {
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (e >= (int64_t)K * N) return;
     const int n = (int)(e % N);
     const float var = bn_var(mean[n], second[n], is_meansq);
     const float scaler = __fdiv_rn(gamma ? gamma[n] : 1.0f, __fsqrt_rn(__fadd_rn(var, eps)));
-    fused_w[e] = __fmul_rn(w[e], scaler);
+    float fw = __fmul_rn(w[e], scaler);
+    if (QUANT) {
+        const Mode mk(qk.mode);
+        fw = quantize_dyn(fw, resolve_kif(load_k(qk.k, e, mk.k_u8), qk.i[e], qk.fb[e], mk.kbi, mk.round_params), mk.round_mode,
+                          mk.overflow_mode, mk.training);
+    }
+    fused_w[e] = fw;
     if (e < N) {
-        fused_b[n] = __fadd_rn(bias[n], __fmul_rn(-mean[n], scaler));
+        float fb = __fadd_rn(bias[n], __fmul_rn(-mean[n], scaler));
+        if (QUANT) {
+            const Mode mb(qb.mode);
+            fb = quantize_dyn(fb, resolve_kif(load_k(qb.k, n, mb.k_u8), qb.i[n], qb.fb[n], mb.kbi, mb.round_params), mb.round_mode,
+                              mb.overflow_mode, mb.training);
+        }
+        fused_b[n] = fb;
         if (moving_mean) moving_mean[n] = __fadd_rn(__fmul_rn(moving_mean[n], momentum), __fmul_rn(mean[n], one_minus_momentum));
         if (moving_var) moving_var[n] = __fadd_rn(__fmul_rn(moving_var[n], momentum), __fmul_rn(var, one_minus_momentum));
     }
@@ -279,14 +295,22 @@ __global__ __launch_bounds__(256) void bn_fold_fwd_kernel(const float *__restric
 //   dw = d_fw * scaler;  dscaler = sum_k d_fw * w - d_fb * mean;  dbias = d_fb;
 //   dgamma = dscaler / sqrt(var + eps);  dvar = -dscaler * gamma / (2 (var + eps)^(3/2));
 //   dmean = -d_fb * scaler (- 2 mean dvar when var comes from the mean of squares);  dsecond = dvar.
-#define BNF_ROWS 16  // rows per thread and trip
+// QUANT: d_fw / d_fb are the gradients at the QUANTIZED folded kernel / bias; each passes its quantizer's surrogate
+// gradient first (the folded value is formed again from w and the scaler), whose bit-width parts go to dik / dfk [K, N]
+// and dib / dfbb [N].
+// CB columns per workgroup, 256 / CB row groups: the quantizer form takes 16 columns per workgroup (its work per element is
+// an order of magnitude more than the folding's, and a kernel of 64 columns would otherwise run on one CU).
+template <bool QUANT, int CB>
 __global__ __launch_bounds__(256) void bn_fold_bwd_kernel(const float *__restrict__ w, const float *__restrict__ gamma,
                                                           const float *__restrict__ mean, const float *__restrict__ second,
                                                           int is_meansq, float eps, const float *__restrict__ d_fw,
                                                           const float *__restrict__ d_fb, float *__restrict__ dw, float *dbias,
-                                                          float *dgamma, float *dmean, float *dsecond, int K, int N) {
-    __shared__ float part[4][64];
-    const int nl = threadIdx.x & 63, grp = threadIdx.x >> 6, n = blockIdx.x * 64 + nl;
+                                                          float *dgamma, float *dmean, float *dsecond, int K, int N,
+                                                          const float *__restrict__ bias, hgq_qdesc qk, hgq_qdesc qb,
+                                                          float *__restrict__ dik, float *__restrict__ dfk, float *dib, float *dfbb) {
+    constexpr int RG = 256 / CB, BNF_ROWS = 64 / RG;  // row groups; rows per thread and trip (64 rows per trip)
+    __shared__ float part[RG][CB];
+    const int nl = threadIdx.x % CB, grp = threadIdx.x / CB, n = blockIdx.x * CB + nl;
     const bool col = n < N;
     const float g = (gamma && col) ? gamma[n] : 1.0f, m = col ? mean[n] : 0.f;
     const float ve = bn_var(m, col ? second[n] : 1.0f, is_meansq) + eps, sd = __fsqrt_rn(ve);
@@ -294,15 +318,41 @@ __global__ __launch_bounds__(256) void bn_fold_bwd_kernel(const float *__restric
     const int64_t bytes = (int64_t)K * N * 4;
     const __amdgpu_buffer_rsrc_t rs_g = buf_rsrc(d_fw, bytes), rs_w = buf_rsrc(w, bytes), rs_dw = buf_rsrc(dw, bytes);
     float ds = 0.f;
-    for (int k0 = grp; k0 < K; k0 += 4 * BNF_ROWS) {
+    for (int k0 = grp; k0 < K; k0 += RG * BNF_ROWS) {
         float gv[BNF_ROWS], wv[BNF_ROWS];
         uint32_t off[BNF_ROWS];
 #pragma unroll
         for (int u = 0; u < BNF_ROWS; ++u) {
-            const int k = k0 + 4 * u;
+            const int k = k0 + RG * u;
             off[u] = (col && k < K) ? (uint32_t)(k * N + n) * 4u : BUF_OOB;  // rows / columns past the end read as zero
             gv[u] = buf_ld1(rs_g, off[u]);
             wv[u] = buf_ld1(rs_w, off[u]);
+        }
+        if (QUANT) {
+            const Mode mk(qk.mode);
+            const __amdgpu_buffer_rsrc_t rs_i = buf_rsrc(qk.i, bytes), rs_f = buf_rsrc(qk.fb, bytes);
+            const __amdgpu_buffer_rsrc_t rs_di = buf_rsrc(dik, bytes), rs_df = buf_rsrc(dfk, bytes);
+            // every operand of the trip is requested before the first is used (a load behind a branch is waited for on the spot)
+            const __amdgpu_buffer_rsrc_t rs_k = buf_rsrc(qk.k, mk.k_u8 ? bytes / 4 : bytes);
+            float iv[BNF_ROWS], fv[BNF_ROWS], kv[BNF_ROWS];
+#pragma unroll
+            for (int u = 0; u < BNF_ROWS; ++u) {
+                iv[u] = buf_ld1(rs_i, off[u]), fv[u] = buf_ld1(rs_f, off[u]);
+                if (mk.k_u8) kv[u] = (float)__builtin_amdgcn_raw_buffer_load_b8(rs_k, off[u] == BUF_OOB ? BUF_OOB : off[u] >> 2, 0, 0);
+                else kv[u] = buf_ld1(rs_k, off[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < BNF_ROWS; ++u) {
+                const int k = k0 + RG * u;
+                if (col && k < K) {
+                    const KIF p = resolve_kif(kv[u], iv[u], fv[u], mk.kbi, mk.round_params);
+                    float gx, gi, gf;
+                    quantize_grad_dyn(__fmul_rn(wv[u], scaler), gv[u], p, mk.round_mode, mk.overflow_mode, gx, gi, gf);
+                    if (mk.kbi) gi -= gf;
+                    buf_st1(rs_di, off[u], gi), buf_st1(rs_df, off[u], gf);
+                    gv[u] = gx;
+                }
+            }
         }
 #pragma unroll
         for (int u = 0; u < BNF_ROWS; ++u) {
@@ -313,8 +363,19 @@ __global__ __launch_bounds__(256) void bn_fold_bwd_kernel(const float *__restric
     part[grp][nl] = ds;
     __syncthreads();
     if (grp != 0 || !col) return;
-    ds = ((part[0][nl] + part[1][nl]) + part[2][nl]) + part[3][nl];
-    const float gb = d_fb[n];
+    ds = part[0][nl];
+#pragma unroll
+    for (int r = 1; r < RG; ++r) ds += part[r][nl];  // groups in order
+    float gb = d_fb[n];
+    if (QUANT) {
+        const Mode mb(qb.mode);
+        const KIF p = resolve_kif(load_k(qb.k, n, mb.k_u8), qb.i[n], qb.fb[n], mb.kbi, mb.round_params);
+        float gx, gi, gf;
+        quantize_grad_dyn(__fadd_rn(bias[n], __fmul_rn(-m, scaler)), gb, p, mb.round_mode, mb.overflow_mode, gx, gi, gf);
+        if (mb.kbi) gi -= gf;
+        dib[n] = gi, dfbb[n] = gf;
+        gb = gx;
+    }
     ds -= gb * m;
     const float dvar = -ds * g / (2.0f * ve * sd);
     if (dbias) dbias[n] = gb;
@@ -486,11 +547,6 @@ __global__ __launch_bounds__(256) void col_moments_kernel(const float *__restric
 #pragma unroll
         for (int e = 0; e < VEC; ++e) my[c * VEC + e] = s1[tx * VEC + e], my[N + c * VEC + e] = s2[tx * VEC + e];
     }
-}
-
-__global__ __launch_bounds__(256) void col_moments_scale_kernel(float *mean, float *meansq, int N, float inv_rows) {
-    const int t = blockIdx.x * 256 + threadIdx.x;
-    if (t < N) mean[t] *= inv_rows, meansq[t] *= inv_rows;
 }
 
 // dx[r, c] = (dmean[c] + 2 x[r, c] dmeansq[c]) / rows
@@ -677,9 +733,34 @@ extern "C" int hgq_bn_fold_fwd(const float *w, const float *bias, const float *g
     if (K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_bn_fold_fwd: bad sizes");
     if (!w || !bias || !mean || !second || !fused_w || !fused_b) return fail(HGQ_ERR_ARG, "hgq_bn_fold_fwd: null pointer");
     const int64_t n = (int64_t)K * N;
-    hipLaunchKernelGGL(bn_fold_fwd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, w, bias, gamma, mean, second,
-                       is_meansq, eps, fused_w, fused_b, moving_mean, moving_var, momentum, one_minus_momentum, K, N);
+    hipLaunchKernelGGL(bn_fold_fwd_kernel<false>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, w, bias, gamma, mean,
+                       second, is_meansq, eps, fused_w, fused_b, moving_mean, moving_var, momentum, one_minus_momentum, K, N, hgq_qdesc{},
+                       hgq_qdesc{});
     return check_launch("hgq_bn_fold_fwd");
+}
+
+static int fold_quant_check(const hgq_qdesc *qk, const hgq_qdesc *qb, const char *who) {
+    if (!qk || !qb || !qk->k || !qk->i || !qk->fb || !qb->k || !qb->i || !qb->fb) return fail(HGQ_ERR_ARG, "%s: null quantizer operand", who);
+    for (const hgq_qdesc *q : {qk, qb}) {
+        const Mode m(q->mode);
+        if (!m.training) return fail(HGQ_ERR_ARG, "%s: training-mode quantizers only", who);
+        if (m.overflow_mode == HGQ_WRAP) return fail(HGQ_ERR_UNSUPPORTED, "%s: WRAP quantizers track their integer bits per call and are not fused", who);
+    }
+    return HGQ_OK;
+}
+
+extern "C" int hgq_bn_fold_quant_fwd(const float *w, const float *bias, const float *gamma, const float *mean, const float *second,
+                                     int is_meansq, float eps, const hgq_qdesc *qk, const hgq_qdesc *qb, float *qw, float *qbias,
+                                     float *moving_mean, float *moving_var, float momentum, float one_minus_momentum, int K, int N,
+                                     void *stream) {
+    if (K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_bn_fold_quant_fwd: bad sizes");
+    if (!w || !bias || !mean || !second || !qw || !qbias) return fail(HGQ_ERR_ARG, "hgq_bn_fold_quant_fwd: null pointer");
+    const int rc = fold_quant_check(qk, qb, "hgq_bn_fold_quant_fwd");
+    if (rc) return rc;
+    const int64_t n = (int64_t)K * N;
+    hipLaunchKernelGGL(bn_fold_fwd_kernel<true>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, w, bias, gamma, mean,
+                       second, is_meansq, eps, qw, qbias, moving_mean, moving_var, momentum, one_minus_momentum, K, N, *qk, *qb);
+    return check_launch("hgq_bn_fold_quant_fwd");
 }
 
 extern "C" int hgq_bn_fold_bwd(const float *w, const float *gamma, const float *mean, const float *second, int is_meansq, float eps,
@@ -688,9 +769,25 @@ extern "C" int hgq_bn_fold_bwd(const float *w, const float *gamma, const float *
     if (K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_bn_fold_bwd: bad sizes");
     if (!w || !mean || !second || !d_fw || !d_fb || !dw) return fail(HGQ_ERR_ARG, "hgq_bn_fold_bwd: null pointer");
     if ((int64_t)K * N * 4 >= (1ll << 31)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_bn_fold_bwd: the kernel matrix must be smaller than 2 GiB");
-    hipLaunchKernelGGL(bn_fold_bwd_kernel, dim3((unsigned)((N + 63) / 64)), dim3(256), 0, (hipStream_t)stream, w, gamma, mean, second,
-                       is_meansq, eps, d_fw, d_fb, dw, dbias, dgamma, dmean, dsecond, K, N);
+    hipLaunchKernelGGL((bn_fold_bwd_kernel<false, 64>), dim3((unsigned)((N + 63) / 64)), dim3(256), 0, (hipStream_t)stream, w, gamma, mean, second,
+                       is_meansq, eps, d_fw, d_fb, dw, dbias, dgamma, dmean, dsecond, K, N, (const float *)nullptr, hgq_qdesc{}, hgq_qdesc{},
+                       (float *)nullptr, (float *)nullptr, (float *)nullptr, (float *)nullptr);
     return check_launch("hgq_bn_fold_bwd");
+}
+
+extern "C" int hgq_bn_fold_quant_bwd(const float *w, const float *bias, const float *gamma, const float *mean, const float *second,
+                                     int is_meansq, float eps, const hgq_qdesc *qk, const hgq_qdesc *qb, const float *d_qw,
+                                     const float *d_qb, float *dw, float *dbias, float *dgamma, float *dmean, float *dsecond, float *di_k,
+                                     float *dfb_k, float *di_b, float *dfb_b, int K, int N, void *stream) {
+    if (K < 1 || N < 1) return fail(HGQ_ERR_ARG, "hgq_bn_fold_quant_bwd: bad sizes");
+    if (!w || !bias || !mean || !second || !d_qw || !d_qb || !dw || !di_k || !dfb_k || !di_b || !dfb_b)
+        return fail(HGQ_ERR_ARG, "hgq_bn_fold_quant_bwd: null pointer");
+    if ((int64_t)K * N * 4 >= (1ll << 31)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_bn_fold_quant_bwd: the kernel matrix must be smaller than 2 GiB");
+    const int rc = fold_quant_check(qk, qb, "hgq_bn_fold_quant_bwd");
+    if (rc) return rc;
+    hipLaunchKernelGGL((bn_fold_bwd_kernel<true, 16>), dim3((unsigned)((N + 15) / 16)), dim3(256), 0, (hipStream_t)stream, w, gamma, mean, second,
+                       is_meansq, eps, d_qw, d_qb, dw, dbias, dgamma, dmean, dsecond, K, N, bias, *qk, *qb, di_k, dfb_k, di_b, dfb_b);
+    return check_launch("hgq_bn_fold_quant_bwd");
 }
 
 extern "C" int64_t hgq_mse_workspace(void) { return MSE_PARTS; }
@@ -765,9 +862,7 @@ extern "C" int hgq_col_moments_fwd(const float *x, int64_t rows, int N, float *m
         hipLaunchKernelGGL((col_moments_kernel<1>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, x, rows, N, TX, workspace);
     int rc = check_launch("hgq_col_moments_fwd");
     if (rc) return rc;
-    if ((rc = reduce_parts(workspace, (int)gy, 2 * (int64_t)N, mean, N, meansq, N, nullptr, 0, s))) return rc;
-    hipLaunchKernelGGL(col_moments_scale_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, s, mean, meansq, N, 1.0f / (float)rows);
-    return check_launch("hgq_col_moments_fwd(scale)");
+    return reduce_parts(workspace, (int)gy, 2 * (int64_t)N, mean, N, meansq, N, nullptr, 0, s, 1.0f / (float)rows);
 }
 
 extern "C" int hgq_col_moments_bwd(const float *x, const float *dmean, const float *dmeansq, int64_t rows, int N, float *dx,

@@ -10,7 +10,7 @@ import torch
 
 from .. import _lib, ops
 from ..core import epsilon, get_initializer
-from ..quantizer.prefetch import quantize_together
+from ..quantizer.prefetch import _eligible, quantize_together
 from .core._contraction import fused_iq_rows
 from .core.einsum_dense import QEinsumDense, analyze_einsum_string
 
@@ -164,12 +164,18 @@ class QEinsumDenseBatchnorm(QEinsumDense):
             mean, meansq, chained = self._batch_moments(inputs, raw=True, quant=quant, chain=True)
             if chained is not None:
                 inputs = chained
-            fused_kernel, fused_bias = ops.bn_fold(self._kernel.reshape(self._K, self._N), self.bias.reshape(-1),
-                                                   self.bn_gamma.reshape(-1) if self.scale else None, mean, meansq, True, epsilon(),
-                                                   self.moving_mean.view(-1), self.moving_variance.view(-1), self.momentum)
-            # kernel and bias quantizers in one launch each way (they are a few thousand elements together)
-            qkernel, qbias = quantize_together([(self.kq, fused_kernel.view(self._kernel.shape)),
-                                                (self.bq, fused_bias.view(self.bias.shape))], training)
+            fold = (self._kernel.reshape(self._K, self._N), self.bias.reshape(-1), self.bn_gamma.reshape(-1) if self.scale else None,
+                    mean, meansq, True, epsilon(), self.moving_mean.view(-1), self.moving_variance.view(-1), self.momentum)
+            fk, fb = (_eligible(self.kq, self._kernel), _eligible(self.bq, self.bias)) if training is True else (None, None)
+            if fk is not None and fb is not None:
+                # folding and both quantizers in one launch each way
+                qkernel, qbias = ops.bn_fold_quant(*fold, *((f._k.view(-1), f._i.view(-1), f._third().view(-1), f._mode(True)) for f in (fk, fb)))
+                qkernel, qbias = qkernel.view(self._kernel.shape), qbias.view(self.bias.shape)
+            else:
+                fused_kernel, fused_bias = ops.bn_fold(*fold)
+                # kernel and bias quantizers in one launch each way (they are a few thousand elements together)
+                qkernel, qbias = quantize_together([(self.kq, fused_kernel.view(self._kernel.shape)),
+                                                    (self.bq, fused_bias.view(self.bias.shape))], training)
         else:
             if training and self.trainable:
                 mean, var = self._batch_moments(inputs)

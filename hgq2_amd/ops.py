@@ -1353,6 +1353,62 @@ def _(w, gamma, mean, second, is_meansq, eps, d_fw, d_fb):
     return torch.empty_like(w), w.new_empty(n), w.new_empty(n if gamma.numel() else 0), w.new_empty(n), w.new_empty(n)
 
 
+def _qdesc(k: Tensor, i: Tensor, fb: Tensor, mode: int):
+    return _lib.QDesc(k.data_ptr(), i.data_ptr(), fb.data_ptr(), _kmode(mode, k))
+
+
+@torch.library.custom_op('hgq::bn_fold_quant_fwd', mutates_args=('moving_mean', 'moving_var'))
+def bn_fold_quant_fwd(w: Tensor, bias: Tensor, gamma: Tensor, mean: Tensor, second: Tensor, is_meansq: bool, eps: float,
+                      moving_mean: Tensor, moving_var: Tensor, momentum: float, qk: Sequence[Tensor], qb: Sequence[Tensor],
+                      modes: Sequence[int]) -> tuple[Tensor, Tensor]:
+    """``bn_fold_fwd`` followed, in the same launch, by the kernel and bias quantizers ``qk`` / ``qb`` = ``(k, i, fb)``:
+    returns the quantized folded kernel and bias."""
+    for name, t in (('w', w), ('bias', bias), ('mean', mean), ('second', second)):
+        _check_f32(name, t)
+    K, N = w.shape
+    _need(bias.numel() == N and mean.numel() == N and second.numel() == N and gamma.numel() in (0, N), 'per-column operands must have N entries')
+    _need(moving_mean.numel() in (0, N) and moving_var.numel() in (0, N), 'moving statistics must have N entries')
+    _need(all(t.numel() == K * N for t in qk) and all(t.numel() == N for t in qb), 'quantizer operands must match the kernel and the bias')
+    dk, db = _qdesc(*qk, modes[0]), _qdesc(*qb, modes[1])
+    qw, qbias = torch.empty_like(w), torch.empty_like(bias)
+    rc = _lib.load().hgq_bn_fold_quant_fwd(_ptr(w), _ptr(bias), _ptr(gamma), _ptr(mean), _ptr(second), int(is_meansq), eps,
+                                           ctypes.addressof(dk), ctypes.addressof(db), _ptr(qw), _ptr(qbias), _ptr(moving_mean),
+                                           _ptr(moving_var), momentum, 1.0 - momentum, K, N, _stream())
+    _lib.check(rc, 'hgq_bn_fold_quant_fwd')
+    return qw, qbias
+
+
+@bn_fold_quant_fwd.register_fake
+def _(w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum, qk, qb, modes):
+    return torch.empty_like(w), torch.empty_like(bias)
+
+
+@torch.library.custom_op('hgq::bn_fold_quant_bwd', mutates_args=())
+def bn_fold_quant_bwd(w: Tensor, bias: Tensor, gamma: Tensor, mean: Tensor, second: Tensor, is_meansq: bool, eps: float, d_qw: Tensor,
+                      d_qb: Tensor, qk: Sequence[Tensor], qb: Sequence[Tensor], modes: Sequence[int]) -> list[Tensor]:
+    """Backward of ``bn_fold_quant_fwd``: ``[dw, dbias, dgamma, dmean, dsecond, di_k, dfb_k, di_b, dfb_b]``."""
+    _check_f32('d_qw', d_qw), _check_f32('d_qb', d_qb)
+    K, N = w.shape
+    dev = w.device
+    dw, di_k, dfb_k = torch.empty_like(w), torch.empty_like(w), torch.empty_like(w)
+    dbias, dmean, dsecond, di_b, dfb_b = (torch.empty(N, dtype=torch.float32, device=dev) for _ in range(5))
+    dgamma = torch.empty(N if gamma.numel() else 0, dtype=torch.float32, device=dev)
+    dk, db = _qdesc(*qk, modes[0]), _qdesc(*qb, modes[1])
+    rc = _lib.load().hgq_bn_fold_quant_bwd(_ptr(w), _ptr(bias), _ptr(gamma), _ptr(mean), _ptr(second), int(is_meansq), eps,
+                                           ctypes.addressof(dk), ctypes.addressof(db), _ptr(d_qw), _ptr(d_qb), _ptr(dw), _ptr(dbias),
+                                           _ptr(dgamma), _ptr(dmean), _ptr(dsecond), _ptr(di_k), _ptr(dfb_k), _ptr(di_b), _ptr(dfb_b), K, N,
+                                           _stream())
+    _lib.check(rc, 'hgq_bn_fold_quant_bwd')
+    return [dw, dbias, dgamma, dmean, dsecond, di_k, dfb_k, di_b, dfb_b]
+
+
+@bn_fold_quant_bwd.register_fake
+def _(w, bias, gamma, mean, second, is_meansq, eps, d_qw, d_qb, qk, qb, modes):
+    n = w.shape[1]
+    return ([torch.empty_like(w), w.new_empty(n), w.new_empty(n if gamma.numel() else 0), w.new_empty(n), w.new_empty(n),
+             torch.empty_like(w), torch.empty_like(w), w.new_empty(n), w.new_empty(n)])
+
+
 @torch.library.custom_op('hgq::qbits_fwd', mutates_args=())
 def qbits_fwd(k: Tensor, i: Tensor, fb: Tensor, kbi: bool, add_mode: int) -> Tensor:
     _check_f32('fb', fb)
@@ -2046,6 +2102,45 @@ class _BnFold(torch.autograd.Function):
         is_meansq, eps = ctx.cfg
         dw, dbias, dgamma, dmean, dsecond = bn_fold_bwd(w, gamma, mean, second, is_meansq, eps, d_fw.contiguous(), d_fb.contiguous())
         return _route(ctx.w_owner, dw), dbias, (dgamma if gamma.numel() else None), dmean, dsecond, None, None, None, None, None
+
+
+class _BnFoldQuant(torch.autograd.Function):
+    """``_BnFold`` and the kernel / bias quantizers behind it, one launch each way."""
+
+    @staticmethod
+    def forward(ctx, w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum, modes, k_k, i_k, fb_k, k_b, i_b, fb_b):
+        ctx.save_for_backward(w, bias, gamma, mean, second, k_k, i_k, fb_k, k_b, i_b, fb_b)
+        ctx.cfg = (is_meansq, eps, modes)
+        ctx.w_owner = _owner(w)
+        ctx.set_materialize_grads(False)
+        return bn_fold_quant_fwd(w, bias, gamma, mean, second, is_meansq, eps, moving_mean, moving_var, momentum, [k_k, i_k, fb_k],
+                                 [k_b, i_b, fb_b], list(modes))
+
+    @staticmethod
+    def backward(ctx, d_qw, d_qb):
+        flush_reductions()  # the kernel / bias gradient may still be slices of the contraction's backward
+        w, bias, gamma, mean, second, k_k, i_k, fb_k, k_b, i_b, fb_b = ctx.saved_tensors
+        is_meansq, eps, modes = ctx.cfg
+        d_qw = torch.zeros_like(w) if d_qw is None else d_qw.contiguous()
+        d_qb = torch.zeros_like(bias) if d_qb is None else d_qb.contiguous()
+        dw, dbias, dgamma, dmean, dsecond, di_k, dfb_k, di_b, dfb_b = bn_fold_quant_bwd(
+            w, bias, gamma, mean, second, is_meansq, eps, d_qw.view(w.shape), d_qb.view(bias.shape), [k_k, i_k, fb_k], [k_b, i_b, fb_b],
+            list(modes))
+        need = ctx.needs_input_grad
+        return (_route(ctx.w_owner, dw), dbias, (dgamma if gamma.numel() else None), dmean, dsecond, None, None, None, None, None, None,
+                None, di_k.view(i_k.shape) if need[12] else None, dfb_k.view(fb_k.shape) if need[13] else None,
+                None, di_b.view(i_b.shape) if need[15] else None, dfb_b.view(fb_b.shape) if need[16] else None)
+
+
+def bn_fold_quant(w2d: Tensor, bias: Tensor, gamma, mean: Tensor, second: Tensor, is_meansq: bool, eps: float, moving_mean, moving_var,
+                  momentum: float, qk, qb):
+    """``(q_k(w s), q_b(bias - mean s))``: :func:`bn_fold` and the two quantizers ``qk`` / ``qb`` = ``(k, i, fb, mode)`` (flat
+    raw variables of training-mode quantizers with per-element bit-widths and no trackers) in one launch each way."""
+    empty = w2d.new_empty(0)
+    return _BnFoldQuant.apply(w2d.contiguous(), bias.contiguous(), gamma.contiguous() if gamma is not None else empty, mean.contiguous(),
+                              second.contiguous(), bool(is_meansq), float(eps), moving_mean if moving_mean is not None else empty,
+                              moving_var if moving_var is not None else empty, float(momentum), (int(qk[3]), int(qb[3])),
+                              qk[0], qk[1], qk[2], qb[0], qb[1], qb[2])
 
 
 def bn_fold(w2d: Tensor, bias: Tensor, gamma, mean: Tensor, second: Tensor, is_meansq: bool, eps: float, moving_mean=None,

@@ -664,6 +664,22 @@ int hgq_bn_fold_fwd(const float *w, const float *bias, const float *gamma, const
 int hgq_bn_fold_bwd(const float *w, const float *gamma, const float *mean, const float *second, int is_meansq, float eps,
                     const float *d_fw, const float *d_fb, float *dw, float *dbias, float *dgamma, float *dmean, float *dsecond,
                     int K, int N, void *stream);
+/*
+ * The folding with the kernel and bias quantizers behind it in the same launch each way (reference
+ * src/hgq/layers/einsum_dense_batchnorm.py:158-211, get_fused_qkernel_and_qbias: fold, then `self.kq(...)`, `self.bq(...)`).
+ * qk / qb: training-mode quantizers with per-element bit-widths ([K, N] and [N]) and no trackers (SAT / SAT_SYM).
+ * Forward: qw = q_k(w s), qbias = q_b(bias - mean s), moving statistics updated as by hgq_bn_fold_fwd.  Backward: d_qw /
+ * d_qb are the gradients at the quantized values; each passes its quantizer's surrogate gradient (bit-width parts to
+ * di_k / dfb_k [K, N] and di_b / dfb_b [N], the folded values formed again from w, bias and the statistics), then the
+ * folding's own gradient as in hgq_bn_fold_bwd.  Values and gradients equal the two separate launches'.
+ */
+int hgq_bn_fold_quant_fwd(const float *w, const float *bias, const float *gamma, const float *mean, const float *second, int is_meansq,
+                          float eps, const hgq_qdesc *qk, const hgq_qdesc *qb, float *qw, float *qbias, float *moving_mean,
+                          float *moving_var, float momentum, float one_minus_momentum, int K, int N, void *stream);
+int hgq_bn_fold_quant_bwd(const float *w, const float *bias, const float *gamma, const float *mean, const float *second, int is_meansq,
+                          float eps, const hgq_qdesc *qk, const hgq_qdesc *qb, const float *d_qw, const float *d_qb, float *dw,
+                          float *dbias, float *dgamma, float *dmean, float *dsecond, float *di_k, float *dfb_k, float *di_b,
+                          float *dfb_b, int K, int N, void *stream);
 
 /*
  * Batch statistics of the un-quantized pre-activation z = x W of QEinsumDenseBatchnorm.call

@@ -560,3 +560,42 @@ def test_qdense_sweep_against_fp64(dev, rows, K, N, P, act, has_bias, round_mode
         want = want.float()
         err = float((got.cpu() - want).abs().max())
         assert err <= 3e-5 * (float(want.abs().max()) + 1e-6), f'{name}: {err:.3e}'
+
+
+@pytest.mark.parametrize('K,N,overflow', [(16, 64, 'SAT_SYM'), (64, 32, 'SAT'), (5, 7, 'SAT_SYM'), (130, 20, 'SAT')])
+def test_bn_fold_with_its_quantizers_in_one_launch(dev, K, N, overflow):
+    """`bn_fold_quant` = `bn_fold` followed by the kernel and bias quantizers (reference
+    src/hgq/layers/einsum_dense_batchnorm.py:158-211): the quantized values and the moving statistics equal the separate
+    launches' bit for bit (the same arithmetic per element), every gradient to the order of the column sums."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(K * N)
+    mode = _lib.mode_bits('RND', overflow, training=True, kbi=True, round_params=True)
+    mk = lambda *s, scale=1.0: (torch.randn(*s, generator=g) * scale).to(dev)  # noqa: E731
+    w, bias, gamma, mean = mk(K, N, scale=0.5), mk(N), mk(N).abs() + 0.5, mk(N, scale=0.3)
+    meansq = mean * mean + mk(N).abs() * 0.5 + 0.01
+    qk = (torch.ones(K * N, dtype=torch.uint8, device=dev), torch.randint(0, 3, (K * N,), generator=g).float().to(dev),
+          (torch.randint(2, 9, (K * N,), generator=g).float() + torch.rand(K * N, generator=g) * 0.4).to(dev))
+    qb = (torch.ones(N, dtype=torch.uint8, device=dev), torch.randint(0, 3, (N,), generator=g).float().to(dev),
+          (torch.randint(2, 9, (N,), generator=g).float() + torch.rand(N, generator=g) * 0.4).to(dev))
+    up_w, up_b = mk(K, N), mk(N)
+
+    def run(fused):
+        leaves = [t.clone().requires_grad_(True) for t in (w, bias, gamma, mean, meansq, qk[1], qk[2], qb[1], qb[2])]
+        lw, lb, lg, lm, ls, ik, fk, ib, fb = leaves
+        mm, mv = torch.zeros(N, device=dev), torch.ones(N, device=dev)
+        if fused:
+            qw, qbias = ops.bn_fold_quant(lw, lb, lg, lm, ls, True, 1e-3, mm, mv, 0.9, (qk[0], ik, fk, mode), (qb[0], ib, fb, mode))
+        else:
+            fw, fbias = ops.bn_fold(lw, lb, lg, lm, ls, True, 1e-3, mm, mv, 0.9)
+            qw, qbias = ops.quantize_multi([fw, fbias], [qk[0], qb[0]], [ik, ib], [fk, fb], [mode, mode])
+        ((qw * up_w).sum() + (qbias * up_b).sum()).backward()
+        return (qw.detach(), qbias.detach(), mm, mv), [t.grad for t in leaves]
+
+    (vals_a, grads_a), (vals_b, grads_b) = run(True), run(False)
+    for a, b in zip(vals_a, vals_b):
+        assert torch.equal(a, b)
+    for name, a, b in zip(('w', 'bias', 'gamma', 'mean', 'meansq', 'i_k', 'b_k', 'i_b', 'b_b'), grads_a, grads_b):
+        assert (a is None) == (b is None), name
+        if a is not None:
+            err = (a.double() - b.double()).abs().max().item()
+            assert err <= 1e-5 * (b.abs().max().item() + 1e-6), (name, err)
