@@ -1558,7 +1558,7 @@ extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t
     hipStream_t s = (hipStream_t)stream;
     int rc = moments_check("hgq_qdense_moments_bwd", rows, K, N, x, f_in, bw_rows, mode);
     if (rc) return rc;
-    if (!x || !w || !dmean || !dmeansq || !dx || !dw || !workspace) return fail(HGQ_ERR_ARG, "hgq_qdense_moments_bwd: null pointer");
+    if (!x || !w || !dmean || !dmeansq || !dx || !workspace) return fail(HGQ_ERR_ARG, "hgq_qdense_moments_bwd: null pointer");
     if (!aligned16(dx) || !aligned16(dx_add)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_moments_bwd: dx and dx_add must be 16-byte aligned");
     const int parts = row_parts(rows, BWD_BM);
     const bool quant = bw_rows > 0;
@@ -1576,6 +1576,7 @@ extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t
     else HGQ_MOM_BWD(HGQ_RND_CONV, true);
 #undef HGQ_MOM_BWD
     if ((rc = check_launch("hgq_qdense_moments_bwd"))) return rc;
+    if (!dw) return HGQ_OK;  // the slices stay in the workspace for the caller's own reduction
     const int64_t PK = bw_rows * (int64_t)K;
     return reduce_parts(workspace, parts, (int64_t)K * N + N + PK, dw, (int64_t)K * N, nullptr, (int64_t)N, quant ? df_in : (float *)nullptr, PK, s);
 }

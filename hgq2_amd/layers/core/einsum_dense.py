@@ -157,8 +157,9 @@ class QEinsumDense(QLayerBaseSingleInput):
             w2d = qkernel.reshape(self._K, self._N)
             # a view's gradient goes back through the view unread: the "one reader" mark of a prefetched operand holds for it
             for view, base in ((w2d, qkernel), (b1d, qbias)):
-                if view is not None and view is not base and getattr(base, '_hgq_single_use', False) and view._base is base:
-                    view._hgq_single_use = True
+                if (view is not None and view is not base and getattr(base, '_hgq_single_use', False)
+                        and view._base is not None and view.data_ptr() == base.data_ptr() and view.numel() == base.numel()):
+                    view._hgq_single_use = True  # the same elements under another shape
             # the output quantizer can join the kernel when nothing but the fused activation follows the contraction
             oq = None
             if oq_ok and self.enable_oq and not self.__output_quantizer_handled__ and (qbias is None or self._bias_in_gemm):

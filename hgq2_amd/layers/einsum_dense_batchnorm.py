@@ -171,6 +171,9 @@ class QEinsumDenseBatchnorm(QEinsumDense):
                 # folding and both quantizers in one launch each way
                 qkernel, qbias = ops.bn_fold_quant(*fold, *((f._k.view(-1), f._i.view(-1), f._third().view(-1), f._mode(True)) for f in (fk, fb)))
                 qkernel, qbias = qkernel.view(self._kernel.shape), qbias.view(self.bias.shape)
+                # their gradients are read by the folding's backward and by nothing else, and it sums pending slices first:
+                # the contraction may leave its kernel / bias gradient as slices for that launch
+                qkernel._hgq_single_use = qbias._hgq_single_use = True
             else:
                 fused_kernel, fused_bias = ops.bn_fold(*fold)
                 # kernel and bias quantizers in one launch each way (they are a few thousand elements together)

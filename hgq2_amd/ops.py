@@ -1313,6 +1313,31 @@ def _(x, w, f_in, bw_rows, mode, dmean, dmeansq, dx_add):
     return torch.empty_like(x), torch.empty_like(w), x.new_empty(bw_rows * x.shape[1])
 
 
+@torch.library.custom_op('hgq::dense_moments_bwd_slices', mutates_args=())
+def dense_moments_bwd_slices(x: Tensor, w: Tensor, f_in: Tensor, bw_rows: int, mode: int, dmean: Tensor, dmeansq: Tensor,
+                             dx_add: Tensor) -> tuple[Tensor, Tensor]:
+    """``dense_moments_bwd`` without the sum over its slices: ``(dx, slices [n, K*N + N + bw_rows*K])`` (the N section unused)."""
+    _check_f32('x', x), _check_f32('w', w), _check_f32('dmean', dmean), _check_f32('dmeansq', dmeansq)
+    if dx_add.numel():
+        _check_f32('dx_add', dx_add)
+        _need(dx_add.shape == x.shape, 'dx_add must have the shape of x')
+    rows, K = x.shape
+    N = w.shape[1]
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    width = K * N + N + bw_rows * K
+    ws = torch.empty((lib.hgq_qdense_bwd_workspace(rows, K, N, bw_rows) // width, width), dtype=torch.float32, device=x.device)
+    _lib.check(lib.hgq_qdense_moments_bwd(_ptr(x), _ptr(f_in), bw_rows, mode, _ptr(w), _ptr(dmean), _ptr(dmeansq), _ptr(dx_add), _ptr(dx),
+                                          None, None, _ptr(ws), rows, K, N, _stream()), 'hgq_qdense_moments_bwd')
+    return dx, ws
+
+
+@dense_moments_bwd_slices.register_fake
+def _(x, w, f_in, bw_rows, mode, dmean, dmeansq, dx_add):
+    K, N = w.shape
+    return torch.empty_like(x), x.new_empty((1, K * N + N + bw_rows * K))
+
+
 @torch.library.custom_op('hgq::bn_fold_fwd', mutates_args=('moving_mean', 'moving_var'))
 def bn_fold_fwd(w: Tensor, bias: Tensor, gamma: Tensor, mean: Tensor, second: Tensor, is_meansq: bool, eps: float,
                 moving_mean: Tensor, moving_var: Tensor, momentum: float) -> tuple[Tensor, Tensor]:
@@ -2069,9 +2094,15 @@ class _DenseMoments(torch.autograd.Function):
         zero = x.new_zeros(w.shape[1]) if (dmean is None or dmeansq is None) else None
         # without a consumer of dx (an input that needs no gradient) the chained gradient is not read either
         dx_add = x.new_empty(0) if dx_chain is None or not ctx.needs_input_grad[0] else dx_chain.contiguous()
-        dx, dw, df = dense_moments_bwd(x, w, f_in, bw_rows, mode, dmean.contiguous() if dmean is not None else zero,
-                                       dmeansq.contiguous() if dmeansq is not None else zero, dx_add)
         o_w, o_f = ctx.owners
+        gm, gs = dmean.contiguous() if dmean is not None else zero, dmeansq.contiguous() if dmeansq is not None else zero
+        if _SINK['open'] and _can_route(o_w, w.numel()) and (not bw_rows or _can_route(o_f, f_in.numel())):
+            # kernel and fractional-bit gradient go to the optimizer and nowhere else: their slices join the pass's one reduction
+            dx, ws = dense_moments_bwd_slices(x, w, f_in, bw_rows, mode, gm, gs, dx_add)
+            dw, df = torch.empty_like(w), x.new_empty(bw_rows * x.shape[1])
+            _PENDING_REDUCE.append((ws, (dw.view(-1), x.new_empty(w.shape[1]), df), (False, True, not bw_rows)))
+        else:
+            dx, dw, df = dense_moments_bwd(x, w, f_in, bw_rows, mode, gm, gs, dx_add)
         dw = _route(o_w, dw)
         df = _route(o_f, df) if bw_rows else None
         return dx, dw, (df.view(f_in.shape) if df is not None else None), None, None, None

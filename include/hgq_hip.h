@@ -706,6 +706,9 @@ int hgq_dense_moments_bwd(const float *x, const float *w, const float *dmean, co
  * fractional-bit gradient.  bw_rows == 0: no quantizer (the entry points above).
  * dx_add (may be null): [rows, K], 16-byte aligned, added to dx while it is written - the gradient x receives from its
  * other use, the output contraction, so that the two need no separate accumulation pass; it does not enter df_in.
+ * dw == NULL in the backward: the kernel / fractional-bit gradient is left in `workspace` as hgq_qdense_bwd_workspace(rows,
+ * K, N, bw_rows) / (K N + N + bw_rows K) slices of [K N | N (unused) | bw_rows K] floats for the caller's own reduction
+ * (hgq_reduce_slices_multi).
  */
 int64_t hgq_qdense_moments_workspace(int64_t rows, int K, int N, int64_t bw_rows);
 int hgq_qdense_moments_fwd(const float *x, const float *f_in, int64_t bw_rows, int mode, const float *w, float *mean, float *meansq,
