@@ -557,6 +557,9 @@ def main():
         # one training step of the other configurations at full size (HIP-graph replay), each with its CPU baseline
         out['config_steps'] = {name: config_step_time(name, steps=20, graph=True, cpu=not args.no_cpu_baseline, cpu_budget_s=6.0)
                                for name in ('particle', 'conv', 'mha')}
+        # the streaming dense kernels alone, 131072 x 64 x 64 with cold operands, either matrix instruction
+        out['dense_kernels'] = {k: {'ms': round(v['ms'], 5), 'GBps': round(v['GBps'], 1), 'frac': round(v['frac'], 4)}
+                                for k, v in dense_streaming(iters=10).items()}
     print(json.dumps(out))
 
 
