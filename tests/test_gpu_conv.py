@@ -219,3 +219,29 @@ def test_one_launch_conv_ebops_term_equals_the_composed_path(dev, case):
     assert abs(t1 - t0) <= 1e-6 * abs(t0)
     for a, b, v in zip(g1, g0, variables):
         assert torch.allclose(a, b, rtol=1e-6, atol=1e-12), float((a - b).abs().max())
+
+
+@pytest.mark.parametrize('case', [CASES[0], CASES[1], CASES[4], CASES[7], CASES[9], CASES[10], CASES[15]])
+def test_conv2d_backward_slices_sum_to_the_reduced_gradient(dev, case):
+    """`hgq_conv2d_bwd_slices` leaves what `hgq_conv2d_bwd` adds up: same data gradient, and the slices, added in slice
+    order as the joint reduction adds them, are its kernel and bias gradient."""
+    from hgq2_amd import _lib, ops
+
+    B, H, W, C, kh, kw, Fo, strides, padding, dilation, relu, bias = case
+    g = torch.Generator().manual_seed(100 + CASES.index(case))
+    x = torch.randn(B, H, W, C, generator=g).to(dev)
+    w = (torch.randn(kh, kw, C, Fo, generator=g) * 0.3).to(dev)
+    b = torch.randn(Fo, generator=g).to(dev) if bias else x.new_empty(0)
+    act = _lib.ACT_RELU if relu else _lib.ACT_NONE
+    geom = ops.conv_geometry(tuple(x.shape), tuple(w.shape), strides, padding, dilation)
+    y = ops.conv2d_fwd(x, w, b, list(geom), act)
+    dy = torch.randn(y.shape, generator=g).to(dev) if y.numel() else torch.empty_like(y)
+    dx, dqw, dqb = ops.conv2d_bwd(dy, y, x, w, list(geom), act, True, bias)
+    dx2, slices = ops.conv2d_bwd_slices(dy, y, x, w, list(geom), act, True)
+    assert torch.equal(dx, dx2)
+    assert slices.shape[1] == w.numel() + Fo
+    outs = [torch.empty(w.numel(), device=dev), torch.empty(Fo, device=dev), x.new_empty(0)]
+    ops.reduce_slices_multi_op([slices], outs, [False, False, True])
+    assert torch.equal(outs[0].view(w.shape), dqw)
+    if bias:
+        assert torch.equal(outs[1], dqb)
