@@ -301,7 +301,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
                                                           const float *__restrict__ v, float *__restrict__ out, QAttnPlan pl,
                                                           float scale, float eps, hgq_qdesc d1, hgq_qdesc d2, hgq_qdesc d3,
                                                           hgq_qdesc d4, hgq_qdesc dq, uint32_t *amax1, uint32_t *amax3,
-                                                          uint32_t *__restrict__ amax_slices) {
+                                                          uint32_t *__restrict__ amax_slices, uint32_t *__restrict__ pair_slices) {
     static_assert(TRAIN || !OQ_PLAIN, "the packed form is for training mode");
     extern __shared__ __align__(16) float lds[];
     constexpr int T = 32 * TH, S = 32 * ST, NPO = OQ_PLAIN ? 4 : 16;
@@ -460,8 +460,13 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
         if (threadIdx.x < 2) {
             uint32_t m = 0;
             for (int w = 0; w < QA_NT / 64; ++w) m = max(m, lds_m13[w][threadIdx.x]);
-            uint32_t *dst = threadIdx.x == 0 ? amax1 : amax3;
-            if (dst) atomicMax(dst, m);
+            if (pair_slices) {
+                // one pair per workgroup behind the output quantizer's slices; the reduction launch folds them (nothing to clear)
+                pair_slices[2 * blockIdx.x + threadIdx.x] = m;
+            } else {
+                uint32_t *dst = threadIdx.x == 0 ? amax1 : amax3;
+                if (dst) atomicMax(dst, m);
+            }
         }
     }
     if (amax_slices && active) {
@@ -480,10 +485,21 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
 
 // amax_o[p * S + s] = max over the workgroups' slices and over the walked rows r = p (mod P) of slices[wg][r][s];
 // a block takes 64 entries, its 16 thread groups share the (slice, row) pairs.
+// pairs (may be null): [n_slices][2] maxima of the two scalar trackers, folded into amax1 / amax3 by the first workgroup
 __global__ __launch_bounds__(1024) void qattn_amax_reduce_kernel(const uint32_t *__restrict__ slices, int n_slices, int64_t rows,
-                                                                 int S, int64_t P, uint32_t *__restrict__ amax_o) {
+                                                                 int S, int64_t P, uint32_t *__restrict__ amax_o,
+                                                                 const uint32_t *__restrict__ pairs, uint32_t *amax1, uint32_t *amax3) {
     __shared__ uint32_t red[1024];
     const int t = threadIdx.x, e_local = t & 63, grp = t >> 6;
+    if (pairs && blockIdx.x == 0 && t < 128) {
+        // wavefront 0 takes the first tracker, wavefront 1 the second
+        const int which = t >> 6;
+        uint32_t pm = 0;
+        for (int i = t & 63; i < n_slices; i += 64) pm = max(pm, pairs[2 * i + which]);
+        pm = wave_max_bits(pm);
+        uint32_t *dst = which == 0 ? amax1 : amax3;
+        if ((t & 63) == 0 && dst) dst[0] = pm;
+    }
     const int64_t e = (int64_t)blockIdx.x * 64 + e_local, M = P * S, fold = rows / P;
     uint32_t m = 0;
     if (e < M) {
@@ -840,9 +856,12 @@ extern "C" int hgq_qattention_fwd(const float *query, const float *key, const fl
     if (has_oq && !(aligned16(oq->i) && aligned16(oq->fb) && ((uintptr_t)oq->k & 3u) == 0))
         return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: the output quantizer's i / fb must be 16-byte aligned, k 4-byte aligned");
     if (amax_oq && !workspace && B > 0) return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: amax_oq needs the workspace");
-    if ((rc = softmax_clear_trackers(amax_exp_iq, 1, amax_inv_iq, 1, B == 0 ? amax_oq : nullptr, pl.P_table * S, s))) return rc;
+    uint32_t *slices = (amax_oq && B > 0) ? (uint32_t *)workspace : nullptr;
+    // with the output quantizer's slices there is a reduction launch anyway: it also folds the scalar trackers' per-workgroup
+    // maxima, so nothing needs clearing; otherwise the scalar trackers are cleared and updated by atomics
+    uint32_t *pairs = slices ? slices + (int64_t)pl.n_wg * N * T * S : nullptr;
+    if (!pairs && (rc = softmax_clear_trackers(amax_exp_iq, 1, amax_inv_iq, 1, B == 0 ? amax_oq : nullptr, pl.P_table * S, s))) return rc;
     if (B == 0) return HGQ_OK;
-    uint32_t *slices = amax_oq ? (uint32_t *)workspace : nullptr;
     if (!query || !key || !value || !out) return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: null pointer");
     if (!(aligned16(query) && aligned16(key) && aligned16(value) && aligned16(out)))
         return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: operands must be 16-byte aligned");
@@ -859,7 +878,7 @@ extern "C" int hgq_qattention_fwd(const float *query, const float *key, const fl
         raised = true;                                                                                                          \
         hipLaunchKernelGGL(kern, dim3(pl.n_wg), dim3(QA_NT), lds, s, query, key, value, out, pl, input_scaler, eps,             \
                            softmax_desc_or_none(exp_iq), softmax_desc_or_none(exp_oq), softmax_desc_or_none(inv_iq),            \
-                           softmax_desc_or_none(inv_oq), softmax_desc_or_none(oq), amax_exp_iq, amax_inv_iq, slices);           \
+                           softmax_desc_or_none(inv_oq), softmax_desc_or_none(oq), amax_exp_iq, amax_inv_iq, slices, pairs);    \
     })
     if (train && (!has_oq || ((oq->mode >> 4) & 0xf) == HGQ_WRAP))
         QA_FWD(true, true);
@@ -872,14 +891,14 @@ extern "C" int hgq_qattention_fwd(const float *query, const float *key, const fl
     if (!slices) return HGQ_OK;
     const int64_t entries = pl.P_table * S;
     hipLaunchKernelGGL(qattn_amax_reduce_kernel, dim3((unsigned)((entries + 63) / 64)), dim3(1024), 0, s, slices, pl.n_wg, (int64_t)N * T, S,
-                       pl.P_table, amax_oq);
+                       pl.P_table, amax_oq, (const uint32_t *)pairs, amax_exp_iq, amax_inv_iq);
     return check_launch("hgq_qattention_fwd(trackers)");
 }
 
 extern "C" int64_t hgq_qattention_fwd_workspace(int B, int T, int S, int N, int H, int64_t bw_rows, int track_oq) {
     QAttnPlan pl;
     if (plan_qattn(B, T, S, N, H, bw_rows, track_oq != 0, pl, "hgq_qattention_fwd_workspace")) return -1;
-    return track_oq ? (int64_t)pl.n_wg * N * T * S : 0;
+    return track_oq ? (int64_t)pl.n_wg * N * T * S + 2 * (int64_t)pl.n_wg : 0;  // slices + a pair of scalar trackers per workgroup
 }
 
 extern "C" int64_t hgq_qattention_bwd_workspace(int B, int T, int S, int N, int H, int64_t bw_rows, int has_oq) {
