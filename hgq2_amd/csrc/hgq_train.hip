@@ -203,8 +203,10 @@ __global__ __launch_bounds__(HGQ_EBOPS_NT) void dense_ebops_multi_kernel(DenseEb
 // Mean squared error: per-workgroup partial sums (fixed order inside a workgroup), added in order
 // by one wavefront of a second launch: the loss does not depend on scheduling.
 #define MSE_PARTS 1024
+// dpred (may be null): also receives the gradient for a unit upstream gradient, (pred - target) * two_over_n, the value
+// mse_bwd_kernel gives for g = 1
 __global__ __launch_bounds__(256) void mse_partial_kernel(const float *__restrict__ pred, const float *__restrict__ target, int64_t n,
-                                                          float *__restrict__ part) {
+                                                          float *__restrict__ part, float *__restrict__ dpred, float two_over_n) {
     __shared__ float red[4];
     float acc = 0.f;
     const int64_t n4 = n >> 2, stride = (int64_t)gridDim.x * 256;
@@ -213,11 +215,13 @@ __global__ __launch_bounds__(256) void mse_partial_kernel(const float *__restric
         const f32x4_t t = target ? ((const f32x4_t *)target)[i] : f32x4_t{0.f, 0.f, 0.f, 0.f};
         const f32x4_t d = p - t;
         acc += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+        if (dpred) ((f32x4_t *)dpred)[i] = d * two_over_n;
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
         const int64_t i = (n4 << 2) + threadIdx.x;
         const float d = pred[i] - (target ? target[i] : 0.f);
         acc += d * d;
+        if (dpred) dpred[i] = d * two_over_n;
     }
     acc = block_sum_256(acc, red);
     if (threadIdx.x == 0) part[blockIdx.x] = acc;
@@ -799,11 +803,26 @@ extern "C" int hgq_mse_fwd(const float *pred, const float *target, float *loss, 
     hipStream_t s = (hipStream_t)stream;
     int grid = persistent_grid(((n >> 2) + 255) / 256, 4);
     if (grid > MSE_PARTS) grid = MSE_PARTS;
-    hipLaunchKernelGGL(mse_partial_kernel, dim3(grid), dim3(256), 0, s, pred, target, n, workspace);
+    hipLaunchKernelGGL(mse_partial_kernel, dim3(grid), dim3(256), 0, s, pred, target, n, workspace, (float *)nullptr, 0.f);
     int rc = check_launch("hgq_mse_fwd");
     if (rc) return rc;
     hipLaunchKernelGGL(mse_finish_kernel, dim3(1), dim3(64), 0, s, workspace, grid, 1.0f / (float)n, loss);
     return check_launch("hgq_mse_fwd(finish)");
+}
+
+extern "C" int hgq_mse_fwd_bwd(const float *pred, const float *target, float *loss, float *dpred, float *workspace, int64_t n, void *stream) {
+    if (n < 1) return fail(HGQ_ERR_ARG, "hgq_mse_fwd_bwd: bad size");
+    if (!pred || !loss || !dpred || !workspace) return fail(HGQ_ERR_ARG, "hgq_mse_fwd_bwd: null pointer");
+    if (((uintptr_t)pred & 15u) || ((uintptr_t)target & 15u) || ((uintptr_t)dpred & 15u))
+        return fail(HGQ_ERR_ARG, "hgq_mse_fwd_bwd: operands must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    int grid = persistent_grid(((n >> 2) + 255) / 256, 4);
+    if (grid > MSE_PARTS) grid = MSE_PARTS;
+    hipLaunchKernelGGL(mse_partial_kernel, dim3(grid), dim3(256), 0, s, pred, target, n, workspace, dpred, 2.0f / (float)n);
+    int rc = check_launch("hgq_mse_fwd_bwd");
+    if (rc) return rc;
+    hipLaunchKernelGGL(mse_finish_kernel, dim3(1), dim3(64), 0, s, workspace, grid, 1.0f / (float)n, loss);
+    return check_launch("hgq_mse_fwd_bwd(finish)");
 }
 
 extern "C" int hgq_mse_bwd(const float *pred, const float *target, const float *g, float *dpred, int64_t n, void *stream) {

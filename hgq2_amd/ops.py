@@ -1249,17 +1249,24 @@ def _(pred, target):
     return pred.new_empty(())
 
 
-@torch.library.custom_op('hgq::mse_bwd', mutates_args=())
-def mse_bwd_op(pred: Tensor, target: Tensor, g: Tensor) -> Tensor:
-    _check_f32('pred', pred), _check_f32('g', g)
+@torch.library.custom_op('hgq::mse_fwd_bwd', mutates_args=())
+def mse_fwd_bwd_op(pred: Tensor, target: Tensor) -> tuple[Tensor, Tensor]:
+    """``(loss, dpred for a unit upstream gradient)`` in one pass over the operands."""
+    _check_f32('pred', pred)
+    if target.numel():
+        _check_f32('target', target)
+        _need(target.numel() == pred.numel(), 'target size mismatch')
+    lib = _lib.load()
+    loss = torch.empty((), dtype=torch.float32, device=pred.device)
     dpred = torch.empty_like(pred)
-    _lib.check(_lib.load().hgq_mse_bwd(_ptr(pred), _ptr(target), _ptr(g), _ptr(dpred), pred.numel(), _stream()), 'hgq_mse_bwd')
-    return dpred
+    ws = torch.empty(lib.hgq_mse_workspace(), dtype=torch.float32, device=pred.device)
+    _lib.check(lib.hgq_mse_fwd_bwd(_ptr(pred), _ptr(target), _ptr(loss), _ptr(dpred), _ptr(ws), pred.numel(), _stream()), 'hgq_mse_fwd_bwd')
+    return loss, dpred
 
 
-@mse_bwd_op.register_fake
-def _(pred, target, g):
-    return torch.empty_like(pred)
+@mse_fwd_bwd_op.register_fake
+def _(pred, target):
+    return pred.new_empty(()), torch.empty_like(pred)
 
 
 def dense_moments_supported(x2d: Tensor, w2d: Tensor) -> bool:
@@ -2523,15 +2530,22 @@ class _SparseCE(torch.autograd.Function):
 
 
 class _MSE(torch.autograd.Function):
+    """With a gradient to come (``pred`` requires one), the forward pass also writes the gradient for a unit upstream
+    gradient - one pass over the operands instead of two; another upstream gradient scales it."""
+
     @staticmethod
     def forward(ctx, pred, target):
-        ctx.save_for_backward(pred, target)
+        if pred.requires_grad:
+            loss, dpred = mse_fwd_bwd_op(pred, target)
+            ctx.save_for_backward(dpred)
+            return loss
+        ctx.save_for_backward()
         return mse_fwd_op(pred, target)
 
     @staticmethod
     def backward(ctx, g):
-        pred, target = ctx.saved_tensors
-        return mse_bwd_op(pred, target, g.contiguous()), None
+        (dpred,) = ctx.saved_tensors
+        return (dpred if _is_unit(g) else g * dpred), None
 
 
 def mse(pred: Tensor, target: Tensor | None = None) -> Tensor:

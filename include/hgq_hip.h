@@ -379,6 +379,9 @@ int hgq_dense_ebops_multi(const hgq_dense_ebops_item *items, int count, void *st
 int64_t hgq_mse_workspace(void);
 int hgq_mse_fwd(const float *pred, const float *target, float *loss, float *workspace, int64_t n, void *stream);
 int hgq_mse_bwd(const float *pred, const float *target, const float *g, float *dpred, int64_t n, void *stream);
+/* Loss and, in the same pass over pred / target, the gradient for a unit upstream gradient: dpred = 2 (pred - target) / n
+ * (what hgq_mse_bwd gives for g = 1); a caller with another upstream gradient scales it. */
+int hgq_mse_fwd_bwd(const float *pred, const float *target, float *loss, float *dpred, float *workspace, int64_t n, void *stream);
 
 /*
  * Mean sparse categorical cross-entropy from logits, forward and gradient in one pass.
