@@ -92,7 +92,7 @@ __device__ __forceinline__ float gather(const float *__restrict__ src, const flo
 
 // Forward (MODE 0, N = F) and data gradient (MODE 1, N = C).  WN = wavefronts along n (1 or 2):
 // the workgroup's tile is (128 / WN) x (32 * WN).
-template <int MODE, int WN>
+template <int MODE, int WN, bool BF = false>
 __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ src, const float *__restrict__ mask,
                                                     const float *__restrict__ w, const float *__restrict__ bias,
                                                     float *__restrict__ out, hgq_conv_geom g, int F, int64_t rows, int K,
@@ -143,9 +143,13 @@ __global__ __launch_bounds__(256) void igemm_kernel(const float *__restrict__ sr
             __syncthreads();
             {
                 const int arow = wm * 32 + (lane & 31), kq = lane >> 5, bcol = wn * 32 + (lane & 31);
+                if (BF) {
+                    acc = mfma_chain_bf16<MODE == 1, false>(acc, &as[arow][kq], 1, &bs[kq][bcol], BN + 1, CV_BK / 16);
+                } else {
 #pragma unroll
-                for (int kk = 0; kk < CV_BK; kk += 2)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[arow][kk + kq], bs[kk + kq][bcol], acc, 0, 0, 0);
+                    for (int kk = 0; kk < CV_BK; kk += 2)
+                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[arow][kk + kq], bs[kk + kq][bcol], acc, 0, 0, 0);
+                }
             }
             __syncthreads();
         }
@@ -191,7 +195,7 @@ __device__ __forceinline__ uint32_t gather4_offset(const RowInfo &r, const ColIn
 // step s (two LDS buffers, one barrier per step), and the A tile sits k-major in LDS with a row
 // stride of BM + 2 words: the transposing writes and the operand reads both spread evenly over
 // the banks.
-template <int MODE, int WN>
+template <int MODE, int WN, bool BF = false>
 __global__ __launch_bounds__(256) void igemm_vec_kernel(const float *__restrict__ src, const float *__restrict__ mask,
                                                         const float *__restrict__ w, const float *__restrict__ bias,
                                                         float *__restrict__ out, hgq_conv_geom g, int F, int64_t rows, int K,
@@ -274,9 +278,13 @@ __global__ __launch_bounds__(256) void igemm_vec_kernel(const float *__restrict_
             if (more) fetch(k_begin + (st + 1) * CV_BK);
             {
                 const int arow = wm * 32 + (lane & 31), kq = lane >> 5, bcol = wn * 32 + (lane & 31);
+                if (BF) {
+                    acc = mfma_chain_bf16<MODE == 1, false>(acc, &as[buf][kq][arow], AS, &bs[buf][kq][bcol], BN + 1, CV_BK / 16);
+                } else {
 #pragma unroll
-                for (int kk = 0; kk < CV_BK; kk += 2)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[buf][kk + kq][arow], bs[buf][kk + kq][bcol], acc, 0, 0, 0);
+                    for (int kk = 0; kk < CV_BK; kk += 2)
+                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[buf][kk + kq][arow], bs[buf][kk + kq][bcol], acc, 0, 0, 0);
+                }
             }
             if (more) stash(buf ^ 1);
             __syncthreads();
@@ -719,7 +727,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
 // matrix, n tile of 32 * WN filters, rows [split * chunk, (split + 1) * chunk) taken 32 * WS at
 // a step, WS wavefronts sharing one output block (combined through LDS at the end);
 // WK * WN * WS = 4.  Slice `split` of `part` is [K * F | F].
-template <int WK, int WN, int WS>
+template <int WK, int WN, int WS, bool BF = false>
 __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ src, const float *__restrict__ dy,
                                                     const float *__restrict__ y, float *__restrict__ part, hgq_conv_geom g,
                                                     int F, int64_t rows, int K, int64_t chunk, int act, int n_ktiles) {
@@ -760,9 +768,13 @@ __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ sr
         }
         __syncthreads();
         const int kq = lane >> 5, c32 = lane & 31, mb = wsub * 32;
+        if (BF) {
+            acc = mfma_chain_bf16<false, true>(acc, &as[mb + kq][wk * 32 + c32], BKT + 1, &zs[mb + kq][wn * 32 + c32], BN + 1, 2);
+        } else {
 #pragma unroll
-        for (int mm = 0; mm < 32; mm += 2)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[mb + mm + kq][wk * 32 + c32], zs[mb + mm + kq][wn * 32 + c32], acc, 0, 0, 0);
+            for (int mm = 0; mm < 32; mm += 2)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[mb + mm + kq][wk * 32 + c32], zs[mb + mm + kq][wn * 32 + c32], acc, 0, 0, 0);
+        }
     }
     __syncthreads();
     float *red = &as[0][0];  // BMS * (BKT + 1) >= 4096 floats whenever WS > 1
@@ -805,7 +817,8 @@ __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ sr
 // The weight / bias gradient for C and F multiples of 4 and 16-byte aligned operands: 128-bit
 // gathers and dz loads, the loads of row step s + 1 in flight while the matrix cores work on
 // step s (two LDS buffers, one barrier per step).  Same tiling and slice layout as wgrad_kernel.
-template <int WK, int WN, int WS>
+// BF: the contraction on the bf16 matrix instruction over exact bf16 parts (mfma_chain_bf16; dz is an arbitrary fp32 tensor).
+template <int WK, int WN, int WS, bool BF = false>
 __global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict__ src, const float *__restrict__ dy,
                                                         const float *__restrict__ y, float *__restrict__ part, hgq_conv_geom g,
                                                         int F, int64_t rows, int K, int64_t chunk, int act, int n_ktiles) {
@@ -871,9 +884,13 @@ __global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict_
         const bool more = st + 1 < n_steps;
         if (more) fetch(m_begin + (st + 1) * BMS);
         const int kq = lane >> 5, c32 = lane & 31, mb = wsub * 32;
+        if (BF) {
+            acc = mfma_chain_bf16<false, true>(acc, &as[buf][mb + kq][wk * 32 + c32], AST, &zs[buf][mb + kq][wn * 32 + c32], ZST, 2);
+        } else {
 #pragma unroll
-        for (int mm = 0; mm < 32; mm += 2)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[buf][mb + mm + kq][wk * 32 + c32], zs[buf][mb + mm + kq][wn * 32 + c32], acc, 0, 0, 0);
+            for (int mm = 0; mm < 32; mm += 2)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as[buf][mb + mm + kq][wk * 32 + c32], zs[buf][mb + mm + kq][wn * 32 + c32], acc, 0, 0, 0);
+        }
         if (more) stash(buf ^ 1);
         __syncthreads();
     }
@@ -1229,10 +1246,17 @@ static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; 
 template <int MODE>
 static void launch_igemm(bool vec, bool wide, dim3 grid, hipStream_t s, const float *src, const float *mask, const float *w,
                          const float *bias, float *out, const hgq_conv_geom &g, int F, int64_t rows, int K, int N, int act, int kchunk) {
-    if (vec && wide) hipLaunchKernelGGL((igemm_vec_kernel<MODE, 2>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
-    else if (vec) hipLaunchKernelGGL((igemm_vec_kernel<MODE, 1>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
-    else if (wide) hipLaunchKernelGGL((igemm_kernel<MODE, 2>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
-    else hipLaunchKernelGGL((igemm_kernel<MODE, 1>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk);
+#define HGQ_IGEMM(BFV) \
+    do { \
+        if (vec && wide) hipLaunchKernelGGL((igemm_vec_kernel<MODE, 2, BFV>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk); \
+        else if (vec) hipLaunchKernelGGL((igemm_vec_kernel<MODE, 1, BFV>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk); \
+        else if (wide) hipLaunchKernelGGL((igemm_kernel<MODE, 2, BFV>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk); \
+        else hipLaunchKernelGGL((igemm_kernel<MODE, 1, BFV>), grid, dim3(256), 0, s, src, mask, w, bias, out, g, F, rows, K, N, act, kchunk); \
+    } while (0)
+    // the process-wide choice of matrix instruction (hgq_dense_use_bf16_parts)
+    if (hgq_dense_use_bf16_parts(-1)) HGQ_IGEMM(true);
+    else HGQ_IGEMM(false);
+#undef HGQ_IGEMM
 }
 
 }  // namespace hgq
@@ -1388,9 +1412,12 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
         const dim3 grid((unsigned)(c.n_kt * c.n_nt), (unsigned)splits);
         const bool vec = g->C % 4 == 0 && F % 4 == 0 && aligned16(xq) && aligned16(dy) && (!mask || aligned16(mask)) &&
                          rows * F * 4 < (1ll << 31) && in_rows * g->C * 4 < (1ll << 31);
+        const bool bf = hgq_dense_use_bf16_parts(-1) != 0;
 #define HGQ_WGRAD(WK, WN, WS) \
     do { \
-        if (vec) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+        if (vec && bf) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS, true>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+        else if (vec) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+        else if (bf) hipLaunchKernelGGL((wgrad_kernel<WK, WN, WS, true>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
         else hipLaunchKernelGGL((wgrad_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
     } while (0)
         if (c.wk == 2 && c.wn == 2) HGQ_WGRAD(2, 2, 1);

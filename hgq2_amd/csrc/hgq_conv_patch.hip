@@ -110,7 +110,9 @@ __device__ __forceinline__ int tile_pos_advance(int pos, int by, int TW) {  // b
 }
 
 // MODE 0: forward; MODE 1: data gradient.  NW wavefronts, each owning 32 rows of the tile.
-template <int MODE, int NW>
+// BF: the contraction runs on the bf16 matrix instruction over exact bf16 parts of the fp32 operands (mfma_chain_bf16: same
+// LDS reads, the same values up to the order of the fp32 additions); the source of the data gradient is an arbitrary fp32 tensor.
+template <int MODE, int NW, bool BF = false>
 __global__ __launch_bounds__(NW * 64) void pgemm_kernel(const float *__restrict__ src, const float *__restrict__ mask,
                                                        const float *__restrict__ w, const float *__restrict__ bias,
                                                        float *__restrict__ out, hgq_conv_geom g, int F, int act, PatchPlan p) {
@@ -215,6 +217,9 @@ __global__ __launch_bounds__(NW * 64) void pgemm_kernel(const float *__restrict_
                 const float *bp = wl + (tap * p.D + kq) * PG_WS + n;
                 // eight depth steps at a time, operands read ahead of the matrix instructions (D is a multiple of 4)
                 int d = 0;
+                if (BF) {
+                    for (; d + 16 <= p.D; d += 16) acc = mfma_chain_bf16<MODE == 1, false>(acc, ap + d, 1, bp + d * PG_WS, PG_WS, 1);
+                }
                 for (; d + 16 <= p.D; d += 16) {
                     float a[8], bq[8];
 #pragma unroll
@@ -293,17 +298,24 @@ int conv_patch_launch(int mode, const float *src, const float *mask, const float
     // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
     static bool allowed = false;
     if (!allowed) {
-        const void *kernels[4] = {(const void *)pgemm_kernel<0, 4>, (const void *)pgemm_kernel<0, 8>, (const void *)pgemm_kernel<1, 4>,
-                                  (const void *)pgemm_kernel<1, 8>};
+        const void *kernels[8] = {(const void *)pgemm_kernel<0, 4>, (const void *)pgemm_kernel<0, 8>, (const void *)pgemm_kernel<1, 4>,
+                                  (const void *)pgemm_kernel<1, 8>, (const void *)pgemm_kernel<0, 4, true>, (const void *)pgemm_kernel<0, 8, true>,
+                                  (const void *)pgemm_kernel<1, 4, true>, (const void *)pgemm_kernel<1, 8, true>};
         for (const void *k : kernels)
             if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, PG_MAX_LDS) != hipSuccess)
                 return fail(HGQ_ERR_LAUNCH, "conv_patch_launch: cannot raise the dynamic LDS limit");
         allowed = true;
     }
-    if (mode == 0 && wide) hipLaunchKernelGGL((pgemm_kernel<0, 8>), grid, dim3(512), lds, s, src, mask, w, bias, out, g, F, act, p);
-    else if (mode == 0) hipLaunchKernelGGL((pgemm_kernel<0, 4>), grid, dim3(256), lds, s, src, mask, w, bias, out, g, F, act, p);
-    else if (wide) hipLaunchKernelGGL((pgemm_kernel<1, 8>), grid, dim3(512), lds, s, src, mask, w, bias, out, g, F, act, p);
-    else hipLaunchKernelGGL((pgemm_kernel<1, 4>), grid, dim3(256), lds, s, src, mask, w, bias, out, g, F, act, p);
+#define PG_LAUNCH(BFV) \
+    do { \
+        if (mode == 0 && wide) hipLaunchKernelGGL((pgemm_kernel<0, 8, BFV>), grid, dim3(512), lds, s, src, mask, w, bias, out, g, F, act, p); \
+        else if (mode == 0) hipLaunchKernelGGL((pgemm_kernel<0, 4, BFV>), grid, dim3(256), lds, s, src, mask, w, bias, out, g, F, act, p); \
+        else if (wide) hipLaunchKernelGGL((pgemm_kernel<1, 8, BFV>), grid, dim3(512), lds, s, src, mask, w, bias, out, g, F, act, p); \
+        else hipLaunchKernelGGL((pgemm_kernel<1, 4, BFV>), grid, dim3(256), lds, s, src, mask, w, bias, out, g, F, act, p); \
+    } while (0)
+    if (hgq_dense_use_bf16_parts(-1)) PG_LAUNCH(true);
+    else PG_LAUNCH(false);
+#undef PG_LAUNCH
     return check_launch("conv_patch_launch");
 }
 
