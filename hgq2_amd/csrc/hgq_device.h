@@ -297,18 +297,18 @@ __device__ __forceinline__ floatx16 mfma_bf16(const u32x4_t &a, const u32x4_t &b
 }
 
 // The leading parts of eight fp32 operands of a lane (the high halves of the words) and whether that is all of them for
-// every lane of the wavefront.
-__device__ __forceinline__ bool bf16_lead8(const float (&v)[8], u32x4_t &p0) {
+// every lane of the wavefront that counts (`counts` = false: a lane that feeds padding rows, whatever it read).
+__device__ __forceinline__ bool bf16_lead8(const float (&v)[8], u32x4_t &p0, bool counts = true) {
     uint32_t low = 0u;
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
         p0[e >> 1] = __builtin_amdgcn_perm(__float_as_uint(v[e + 1]), __float_as_uint(v[e]), 0x07060302u);
         low |= __float_as_uint(v[e]) | __float_as_uint(v[e + 1]);
     }
-    return !__any((low & 0xffffu) != 0u);
+    return !__any(counts && (low & 0xffffu) != 0u);
 }
-// The second and third parts; returns whether the third is non-zero anywhere in the wavefront.
-__device__ __forceinline__ bool bf16_rest8(const float (&v)[8], u32x4_t &p1, u32x4_t &p2) {
+// The second and third parts; returns whether the third is non-zero in a lane that counts.
+__device__ __forceinline__ bool bf16_rest8(const float (&v)[8], u32x4_t &p1, u32x4_t &p2, bool counts = true) {
     uint32_t nz2 = 0u;
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
@@ -317,16 +317,52 @@ __device__ __forceinline__ bool bf16_rest8(const float (&v)[8], u32x4_t &p1, u32
         p1[e >> 1] = bf16_pair(m0, m1), p2[e >> 1] = bf16_pair(l0, l1);
         nz2 |= l0 | l1;
     }
-    return __any(nz2 != 0u);
+    return __any(counts && nz2 != 0u);
 }
 
-// Same arguments and LDS reads as mfma_chain.  FULL_A / FULL_B: that operand is a gradient - arbitrary fp32, all three
+// One batch of sixteen contraction steps: a[u], b[u] are the operands lane (column / row, half h) would hand to the u-th
+// of eight `32x32x2` instructions (step 2 u + h).  FULL_A / FULL_B: that operand is a gradient - arbitrary fp32, all three
 // parts taken without looking.  A batch whose part pairs would cost more than the eight fp32 instructions they replace
-// (splitting included) is issued as those eight instructions: the chain is never slower than mfma_chain by more than
-// the look at the operands.
+// (splitting included) is issued as those eight instructions.  a_counts = false: this lane's `a` feeds result rows that are
+// never read (padding of a short operand): its values take no part in the choice of the parts, so the choice - and with it
+// the order of the additions - depends on the operands alone.
+template <bool FULL_A, bool FULL_B>
+__device__ __forceinline__ floatx16 mfma_batch_bf16(floatx16 acc, const float (&a)[8], const float (&b)[8], bool a_counts = true) {
+    static_assert(!(FULL_A && FULL_B), "one operand of a chain is a quantized tensor");
+    u32x4_t pa0, pb0;
+    const bool one_a = bf16_lead8(a, pa0, a_counts), one_b = bf16_lead8(b, pb0);
+    if (FULL_A || FULL_B) {
+        if (FULL_A ? one_b : one_a) {
+            // three instructions: the quantized operand's single part against the gradient's three
+            u32x4_t p1, p2;
+            bf16_rest8(FULL_A ? a : b, p1, p2);
+            acc = mfma_bf16(pa0, pb0, acc);
+            acc = FULL_A ? mfma_bf16(p1, pb0, acc) : mfma_bf16(pa0, p1, acc);
+            acc = FULL_A ? mfma_bf16(p2, pb0, acc) : mfma_bf16(pa0, p2, acc);
+        } else {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+        }
+    } else if (one_a && one_b) {
+        acc = mfma_bf16(pa0, pb0, acc);
+    } else if (one_a || one_b) {
+        // one side has a single part: up to three instructions
+        u32x4_t p1, p2;
+        const bool third = bf16_rest8(one_a ? b : a, p1, p2, one_a || a_counts);
+        acc = mfma_bf16(pa0, pb0, acc);
+        acc = one_a ? mfma_bf16(pa0, p1, acc) : mfma_bf16(p1, pb0, acc);
+        if (third) acc = one_a ? mfma_bf16(pa0, p2, acc) : mfma_bf16(p2, pb0, acc);
+    } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+    }
+    return acc;
+}
+
+// Same arguments and LDS reads as mfma_chain, every batch through mfma_batch_bf16: never slower than mfma_chain by more
+// than the look at the operands.
 template <bool FULL_A, bool FULL_B>
 __device__ __forceinline__ floatx16 mfma_chain_bf16(floatx16 acc, const float *ap, int sa, const float *bp, int sb, int n_batches) {
-    static_assert(!(FULL_A && FULL_B), "one operand of a chain is a quantized tensor");
     // (the next batch's operands are not requested ahead as in mfma_chain: the registers that takes spill in the kernels
     // that use this chain, and a batch is a few instructions, not eight, so the other wavefronts cover the LDS latency)
 #pragma unroll
@@ -335,33 +371,7 @@ __device__ __forceinline__ floatx16 mfma_chain_bf16(floatx16 acc, const float *a
             float a[8], b[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) a[u] = ap[(16 * bt + 2 * u) * sa], b[u] = bp[(16 * bt + 2 * u) * sb];
-            u32x4_t pa0, pb0;
-            const bool one_a = bf16_lead8(a, pa0), one_b = bf16_lead8(b, pb0);
-            if (FULL_A || FULL_B) {
-                if (FULL_A ? one_b : one_a) {
-                    // three instructions: the quantized operand's single part against the gradient's three
-                    u32x4_t p1, p2;
-                    bf16_rest8(FULL_A ? a : b, p1, p2);
-                    acc = FULL_A ? mfma_bf16(pa0, pb0, acc) : mfma_bf16(pa0, pb0, acc);
-                    acc = FULL_A ? mfma_bf16(p1, pb0, acc) : mfma_bf16(pa0, p1, acc);
-                    acc = FULL_A ? mfma_bf16(p2, pb0, acc) : mfma_bf16(pa0, p2, acc);
-                } else {
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
-                }
-            } else if (one_a && one_b) {
-                acc = mfma_bf16(pa0, pb0, acc);
-            } else if (one_a || one_b) {
-                // one side has a single part: up to three instructions
-                u32x4_t p1, p2;
-                const bool third = bf16_rest8(one_a ? b : a, p1, p2);
-                acc = mfma_bf16(pa0, pb0, acc);
-                acc = one_a ? mfma_bf16(pa0, p1, acc) : mfma_bf16(p1, pb0, acc);
-                if (third) acc = one_a ? mfma_bf16(pa0, p2, acc) : mfma_bf16(p2, pb0, acc);
-            } else {
-#pragma unroll
-                for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
-            }
+            acc = mfma_batch_bf16<FULL_A, FULL_B>(acc, a, b);
         }
     }
     return acc;

@@ -36,6 +36,7 @@ struct QAttnPlan {
     int B, T, S, N;
     int n_wg;         // workgroup w takes batch elements w, w + n_wg, ...
     int64_t P_table;  // rows of the output quantizer's [P_table, S] table; row (n * T + t) % P_table serves (n, t)
+    int bf;           // contractions on the bf16 matrix instruction over exact bf16 parts (mfma_batch_bf16), batch by batch
 };
 
 // One operand array of a batch element in flight: up to two 128-bit words per thread.
@@ -73,8 +74,10 @@ __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32); }
 __device__ __forceinline__ int qa_row(int st, int r, int hf) { return st * 32 + (r >> 2) * 8 + hf * 4 + (r & 3); }
 
 // Transposed score tile of one head: acc[st][r] = sum_h key[s][h] query[t][h], s = qa_row(st, r, hf), t = t0 + lane % 32.
-template <int HD, int ST>
-__device__ __forceinline__ void score_tiles(const float *a_tile, const float *b_tile, int t0, int col0, int t_l, int hf, floatx16 (&acc)[ST]) {
+// bf: sixteen contraction steps at a time through mfma_batch_bf16 (FULL_B: b_tile holds a gradient).
+template <int HD, int ST, bool FULL_B = false>
+__device__ __forceinline__ void score_tiles(const float *a_tile, const float *b_tile, int t0, int col0, int t_l, int hf, floatx16 (&acc)[ST],
+                                            bool bf = false) {
     constexpr int HH = HD / 2;
     float b[HH];
 #pragma unroll
@@ -91,31 +94,55 @@ __device__ __forceinline__ void score_tiles(const float *a_tile, const float *b_
             a[4 * g] = v.x, a[4 * g + 1] = v.y, a[4 * g + 2] = v.z, a[4 * g + 3] = v.w;
         }
         floatx16 c = {0};
+        if (HH % 8 == 0 && bf) {
 #pragma unroll
-        for (int j = 0; j < HH; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], c, 0, 0, 0);
+            for (int j0 = 0; j0 < HH; j0 += 8) {
+                float a8[8], b8[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a8[j] = a[(j0 + j) % HH], b8[j] = b[(j0 + j) % HH];
+                c = mfma_batch_bf16<false, FULL_B>(c, a8, b8);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < HH; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], c, 0, 0, 0);
+        }
         acc[st] = c;
     }
 }
 
 // D[h][t] = sum_s tile[s][col0 + h] * acc[s][t]: the accumulator registers are the B operand as they stand.
-template <int ST>
-__device__ __forceinline__ floatx16 contract_keys(const float *tile, int col0, int t_l, int hf, const floatx16 (&acc)[ST]) {
+// bf: sixteen contraction steps at a time through mfma_batch_bf16 (FULL_B: the accumulators hold a gradient).
+template <int ST, bool FULL_B = false>
+__device__ __forceinline__ floatx16 contract_keys(const float *tile, int col0, int t_l, int hf, const floatx16 (&acc)[ST], bool bf = false,
+                                                  int hd = 32) {
     floatx16 o = {0};
 #pragma unroll
     for (int st = 0; st < ST; ++st) {
         float a[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) a[r] = tile[qa_row(st, r, hf) * QA_LD + col0 + t_l];
+        if (bf) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r], acc[st][r], o, 0, 0, 0);
+            for (int r0 = 0; r0 < 16; r0 += 8) {
+                float a8[8], b8[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a8[j] = a[r0 + j], b8[j] = acc[st][r0 + j];
+                o = mfma_batch_bf16<false, FULL_B>(o, a8, b8, t_l < hd);  // lanes past the head size feed rows nobody reads
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o = __builtin_amdgcn_mfma_f32_32x32x2f32(a[r], acc[st][r], o, 0, 0, 0);
+        }
     }
     return o;
 }
 
 // D[h][s] = sum_t tile[t][col0 + h] * buf[t][s0 + s], t < 32 * TH (buf rows are QA_LD words apart).  A step pairs
 // rows t and t + 8: 8 * QA_LD = 32 (mod 64) words, so the two half-wavefronts read disjoint banks.
-template <int TH>
-__device__ __forceinline__ floatx16 contract_queries(const float *tile, int col0, const float *buf, int s0, int t_l, int hf) {
+// bf: sixteen contraction steps at a time through mfma_batch_bf16 (FULL_A / FULL_B: tile / buf holds a gradient).
+template <int TH, bool FULL_A = false, bool FULL_B = false>
+__device__ __forceinline__ floatx16 contract_queries(const float *tile, int col0, const float *buf, int s0, int t_l, int hf, bool bf = false,
+                                                     int hd = 32) {
     floatx16 o = {0};
 #pragma unroll
     for (int j0 = 0; j0 < 16 * TH; j0 += 16) {
@@ -126,8 +153,18 @@ __device__ __forceinline__ floatx16 contract_queries(const float *tile, int col0
             a[j] = tile[t * QA_LD + col0 + t_l];
             b[j] = buf[t * QA_LD + s0 + t_l];
         }
+        if (bf) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) o = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], o, 0, 0, 0);
+            for (int h0 = 0; h0 < 16; h0 += 8) {
+                float a8[8], b8[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a8[j] = a[h0 + j], b8[j] = b[h0 + j];
+                o = mfma_batch_bf16<FULL_A, FULL_B>(o, a8, b8, t_l < hd);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) o = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[j], o, 0, 0, 0);
+        }
     }
     return o;
 }
@@ -377,7 +414,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
 #pragma unroll
             for (int j = 0; j < NPO; ++j) asm volatile("" : "+v"(po[st][j]));
         floatx16 acc[ST];
-        score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, acc);
+        score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, acc, pl.bf != 0);
         float mx = acc[0][0];
 #pragma unroll
         for (int st = 0; st < ST; ++st)
@@ -412,7 +449,31 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
         // the output quantizer of an element, then its step of out = probs value: the MFMA of one element runs
         // while the next one is quantized (the presence test is hoisted: no branch between the elements)
         floatx16 o = {0};
-        if (qo.present) {
+        if (qo.present && pl.bf) {
+            // eight quantized probabilities at a time, then their sixteen contraction steps as one batch
+#pragma unroll
+            for (int st = 0; st < ST; ++st) {
+                float a[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) a[r] = Vs[qa_row(st, r, hf) * QA_LD + col0 + t_l];
+#pragma unroll
+                for (int r0 = 0; r0 < 16; r0 += 8) {
+                    float a8[8], y8[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int r = r0 + j;
+                        float y = __fmul_rn(acc[st][r], rr);
+                        if (OQ_PLAIN)
+                            y = qo.round_at(y, (int)(int8_t)((po[st][r >> 2] >> (8 * (r & 3))) & 0xff));
+                        else
+                            y = qo.fwd<TRAIN>(y, po[st][r % NPO]);
+                        mo[st][r] = max(mo[st][r], abs_bits(y));
+                        a8[j] = a[r], y8[j] = y;
+                    }
+                    o = mfma_batch_bf16<false, false>(o, a8, y8, t_l < HD);  // lanes past the head size feed rows nobody reads
+                }
+            }
+        } else if (qo.present) {
 #pragma unroll
             for (int st = 0; st < ST; ++st) {
                 float a[16];
@@ -620,8 +681,8 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
             for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(pf[st][g]));
         if (active) {
-            score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, xs);  // scores, transposed
-            score_tiles<HD, ST>(Vs, Gs, t0, col0, t_l, hf, ga);  // d probs = dout value^T, transposed
+            score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, xs, pl.bf != 0);        // scores, transposed
+            score_tiles<HD, ST, true>(Vs, Gs, t0, col0, t_l, hf, ga, pl.bf != 0);  // d probs = dout value^T, transposed
             // ---- forward chain: e of every element (kept in the wavefront's buffer), row sum, inverse stage
             mx = xs[0][0];
 #pragma unroll
@@ -681,7 +742,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
             for (int st = 0; st < ST; ++st)
                 if (st % TH == th) {
-                    const floatx16 o = contract_queries<TH>(Gs, col0, head_buf, st * 32, t_l, hf);
+                    const floatx16 o = contract_queries<TH, true, false>(Gs, col0, head_buf, st * 32, t_l, hf, pl.bf != 0, HD);
                     store_rows<HD>(o, dv_ + ((int64_t)b * S * pl.N + h) * HD, (int64_t)pl.N * HD, st * 32 + t_l, hf);
                 }
             // ---- exp stage and the maximum
@@ -737,7 +798,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
         }
         if (active) {
             // dquery[t][h] = sum_s dscores[t][s] key[s][h]
-            const floatx16 o = contract_keys<ST>(Ks, col0, t_l, hf, ga);
+            const floatx16 o = contract_keys<ST, true>(Ks, col0, t_l, hf, ga, pl.bf != 0, HD);
             store_rows<HD>(o, dq_ + ((int64_t)b * T * pl.N + h) * HD, (int64_t)pl.N * HD, t0 + t_l, hf);
         }
         __syncthreads();  // dvalue has read the probs
@@ -747,7 +808,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
             // dkey[s][h] = sum_t dscores[t][s] query[t][h]
 #pragma unroll
             for (int st = 0; st < ST; ++st)
-                if (st % TH == th) dk_prev = contract_queries<TH>(Qs, col0, head_buf, st * 32, t_l, hf);
+                if (st % TH == th) dk_prev = contract_queries<TH, false, true>(Qs, col0, head_buf, st * 32, t_l, hf, pl.bf != 0, HD);
             b_prev = b;
         }
     }
@@ -802,6 +863,7 @@ static int plan_qattn(int B, int T, int S, int N, int H, int64_t bw_rows, bool h
         return fail(HGQ_ERR_ARG, "%s: bw_rows=%lld does not divide N * T=%d", who, (long long)P, N * T);
     pl.B = B, pl.T = T, pl.S = S, pl.N = N, pl.P_table = P;
     pl.n_wg = persistent_grid(B > 0 ? B : 1, 1);
+    pl.bf = hgq_dense_use_bf16_parts(-1);
     return HGQ_OK;
 }
 

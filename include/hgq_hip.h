@@ -245,6 +245,8 @@ int hgq_qdense_fwd_parts(int64_t rows);
  * The streaming kernels (K, N <= 64) contract on the bf16 matrix cores: every fp32 operand is split exactly into up to
  * three bf16 parts (8 + 8 + 8 significant bits), the products of parts are exact in fp32 and are accumulated in fp32,
  * and only the non-zero parts are multiplied - quantized operands of up to 8 bits need one part, up to 16 bits two.
+ * The convolution and attention kernels take the same choice (sixteen contraction steps at a time: one bf16 instruction
+ * where both operands have one part, three where one of them is a gradient, the eight fp32 instructions otherwise).
  * Same values as the fp32 matrix instruction up to the order of the fp32 accumulation.  `on` = 0 selects the fp32
  * instruction instead, 1 the bf16 parts (default), a negative value changes nothing; returns the previous setting.
  * Process-wide, not synchronised with launches in flight on other threads.
