@@ -185,6 +185,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.restype = restype
         fn.argtypes = argtypes
+    if os.environ.get('HGQ_MATRIX_INSTRUCTION', '').lower() == 'fp32':
+        lib.hgq_dense_use_bf16_parts(0)  # contractions on the fp32 matrix instruction instead of bf16 parts
     _lib = lib
     return lib
 

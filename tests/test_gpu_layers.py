@@ -795,15 +795,14 @@ def test_output_quantizer_inside_the_dense_kernel(dev, kind):
         return real(*a, **k)
 
     ops.qdense_fwd_oq = spy
+    was = lib.hgq_dense_use_bf16_parts(1)  # (the process may have been started on the fp32 matrix instruction)
     try:
         fused = run(model)
         n_fused = len(launches)
-        was = lib.hgq_dense_use_bf16_parts(0)
-        try:
-            plain = run(clone)
-        finally:
-            lib.hgq_dense_use_bf16_parts(was)
+        lib.hgq_dense_use_bf16_parts(0)
+        plain = run(clone)
     finally:
+        lib.hgq_dense_use_bf16_parts(was)
         ops.qdense_fwd_oq = real
     assert n_fused == 2 * len(layers) and len(launches) == n_fused, 'the fused kernel runs exactly where it is switched on'
     for a, b in zip(fused, plain):
@@ -822,9 +821,10 @@ def test_output_quantizer_inside_the_dense_kernel(dev, kind):
         model_loss(m, ops.mse(m(x, training=True) * up)).backward()
         return {n: p_.grad.detach().clone() for n, p_ in m.named_parameters() if p_.grad is not None}
 
-    ga = grads(model)
-    was = lib.hgq_dense_use_bf16_parts(0)
+    was = lib.hgq_dense_use_bf16_parts(1)
     try:
+        ga = grads(model)
+        lib.hgq_dense_use_bf16_parts(0)
         gb = grads(clone)
     finally:
         lib.hgq_dense_use_bf16_parts(was)
