@@ -289,8 +289,8 @@ __device__ __forceinline__ void bf16_parts(float v, uint32_t &h, uint32_t &m, ui
     m = __float_as_uint(r1) & 0xffff0000u;
     l = __float_as_uint(__fsub_rn(r1, __uint_as_float(m)));  // exact, at most eight significant bits
 }
-// two parts (bit patterns with zero low halves) as one register of two bf16: `a` first
-__device__ __forceinline__ uint32_t bf16_pair(uint32_t a, uint32_t b) { return (a >> 16) | b; }
+// the high halves of two words as one register of two bf16, `a` first (one byte-permute instruction)
+__device__ __forceinline__ uint32_t bf16_pair(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 
 __device__ __forceinline__ floatx16 mfma_bf16(const u32x4_t &a, const u32x4_t &b, floatx16 acc) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
