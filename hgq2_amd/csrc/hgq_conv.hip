@@ -818,7 +818,9 @@ __global__ __launch_bounds__(256) void wgrad_kernel(const float *__restrict__ sr
 // gathers and dz loads, the loads of row step s + 1 in flight while the matrix cores work on
 // step s (two LDS buffers, one barrier per step).  Same tiling and slice layout as wgrad_kernel.
 // BF: the contraction on the bf16 matrix instruction over exact bf16 parts (mfma_chain_bf16; dz is an arbitrary fp32 tensor).
-template <int WK, int WN, int WS, bool BF = false>
+// ZS: the filter count is not a multiple of 4 (or dy is not 16-byte aligned): dz and the mask are loaded element by element,
+// columns past F as zeros; the gathers of the source stay 128 bits wide.
+template <int WK, int WN, int WS, bool BF = false, bool ZS = false>
 __global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict__ src, const float *__restrict__ dy,
                                                         const float *__restrict__ y, float *__restrict__ part, hgq_conv_geom g,
                                                         int F, int64_t rows, int K, int64_t chunk, int act, int n_ktiles) {
@@ -855,9 +857,18 @@ __global__ __launch_bounds__(256) void wgrad_vec_kernel(const float *__restrict_
 #pragma unroll
         for (int p = 0; p < ZP; ++p) {
             const int64_t m = m0 + zr + ZR * p;
-            const uint32_t off = (m < m_end && z_on) ? (uint32_t)(m * F + n0 + 4 * zq) * 4u : BUF_OOB;
-            zv[p] = buf_ld4(rs_dy, off);
-            zm[p] = buf_ld4(rs_y, off);
+            if (ZS) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t off = (m < m_end && n0 + 4 * zq + j < F) ? (uint32_t)(m * F + n0 + 4 * zq + j) * 4u : BUF_OOB;
+                    zv[p][j] = buf_ld1(rs_dy, off);
+                    zm[p][j] = buf_ld1(rs_y, off);
+                }
+            } else {
+                const uint32_t off = (m < m_end && z_on) ? (uint32_t)(m * F + n0 + 4 * zq) * 4u : BUF_OOB;
+                zv[p] = buf_ld4(rs_dy, off);
+                zm[p] = buf_ld4(rs_y, off);
+            }
         }
     };
     auto stash = [&](int buf) {
@@ -1410,12 +1421,15 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
         int64_t chunk = (rows + splits - 1) / splits;
         chunk = (chunk + 127) / 128 * 128;
         const dim3 grid((unsigned)(c.n_kt * c.n_nt), (unsigned)splits);
-        const bool vec = g->C % 4 == 0 && F % 4 == 0 && aligned16(xq) && aligned16(dy) && (!mask || aligned16(mask)) &&
-                         rows * F * 4 < (1ll << 31) && in_rows * g->C * 4 < (1ll << 31);
+        const bool src_vec = g->C % 4 == 0 && aligned16(xq) && rows * F * 4 < (1ll << 31) && in_rows * g->C * 4 < (1ll << 31);
+        const bool z_vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask));
+        const bool vec = src_vec && z_vec;
         const bool bf = hgq_dense_use_bf16_parts(-1) != 0;
 #define HGQ_WGRAD(WK, WN, WS) \
     do { \
-        if (vec && bf) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS, true>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+        if (src_vec && !z_vec && bf) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS, true, true>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+        else if (src_vec && !z_vec) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS, false, true>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
+        else if (vec && bf) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS, true>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
         else if (vec) hipLaunchKernelGGL((wgrad_vec_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
         else if (bf) hipLaunchKernelGGL((wgrad_kernel<WK, WN, WS, true>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
         else hipLaunchKernelGGL((wgrad_kernel<WK, WN, WS>), grid, dim3(256), 0, s, xq, dy, mask, workspace, *g, F, rows, K, chunk, act, c.n_kt); \
