@@ -231,3 +231,21 @@ def test_reciprocal_index_arithmetic_is_exact_on_the_ranges_the_kernels_use():
         inv = np.float32(1.0) / np.float32(d)
         q = ((c.astype(np.float32) + np.float32(0.5)) * inv).astype(np.uint32)
         assert np.array_equal(q, c // d), d
+
+
+def test_matrix_instruction_choice_from_the_environment():
+    """`HGQ_MATRIX_INSTRUCTION=fp32` starts the package with the contractions on the fp32 matrix instruction; without it the
+    bf16-part kernels are the default (`hgq_dense_use_bf16_parts`: a negative argument only reads the setting)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = 'from hgq2_amd import _lib; print(_lib.load().hgq_dense_use_bf16_parts(-1))'
+    for value, want in ((None, '1'), ('fp32', '0'), ('bf16', '1')):
+        env = {k: v for k, v in os.environ.items() if k != 'HGQ_MATRIX_INSTRUCTION'}
+        if value is not None:
+            env['HGQ_MATRIX_INSTRUCTION'] = value
+        out = subprocess.run([sys.executable, '-c', code], cwd=root, env=env, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert out.stdout.strip().splitlines()[-1] == want, (value, out.stdout)
