@@ -79,6 +79,7 @@ SIGNATURES = {
     'hgq_sparse_ce_fwd_bwd': (c_int, [c_void_p] * 4 + [c_int64, c_int, c_void_p, c_void_p]),
     'hgq_sgd_update': (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_float, c_void_p]),
     'hgq_sgd_update_multi': (c_int, [c_void_p, c_int, c_float, c_void_p]),
+    'hgq_sgd_update_multi_sum': (c_int, [c_void_p, c_int, c_float, c_void_p, c_int, c_void_p, c_void_p]),
     'hgq_quantize_bwd_workspace': (c_int64, [c_int64, c_int64, c_int64]),
     'hgq_quantize_bwd_sliced': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_bwd_slice_count': (c_int64, [c_int64, c_int64, c_int64]),

@@ -485,9 +485,19 @@ __global__ __launch_bounds__(256) void sgd_kernel(float *__restrict__ w, const f
 struct SgdBatch {
     hgq_sgd_item item[HGQ_SGD_BATCH];
 };
+struct SumBatch {
+    const float *term[HGQ_SUM_BATCH];
+};
 
 // grid.y = variable, grid.x strides over its elements; the descriptors travel as a kernel argument
-__global__ __launch_bounds__(256) void sgd_multi_kernel(SgdBatch b, float lr) {
+// n_sum > 0: the first thread of the launch also adds the scalars of `sums` in list order into sum_out (the step's loss
+// terms: the update does not read them, they only ride along instead of taking a launch of their own)
+__global__ __launch_bounds__(256) void sgd_multi_kernel(SgdBatch b, float lr, SumBatch sums, int n_sum, float *sum_out) {
+    if (n_sum > 0 && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        float v = sums.term[0][0];
+        for (int t = 1; t < n_sum; ++t) v = __fadd_rn(v, sums.term[t][0]);
+        sum_out[0] = v;
+    }
     const hgq_sgd_item it = b.item[blockIdx.y];
     float sc[HGQ_SGD_SIDES];
 #pragma unroll
@@ -567,8 +577,12 @@ __global__ __launch_bounds__(256) void col_moments_bwd_kernel(const float *__res
 
 using namespace hgq;
 
-extern "C" int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *stream) {
+static int sgd_update_multi_impl(const hgq_sgd_item *items, int count, float lr, const float *const *terms, int n_terms, float *sum_out,
+                                 void *stream) {
     if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_sgd_update_multi: bad arguments");
+    SumBatch sums;
+    for (int t = 0; t < HGQ_SUM_BATCH; ++t) sums.term[t] = t < n_terms ? terms[t] : nullptr;
+    bool summed = n_terms == 0;
     for (int base = 0; base < count; base += HGQ_SGD_BATCH) {
         SgdBatch b;
         const int nb = count - base < HGQ_SGD_BATCH ? count - base : HGQ_SGD_BATCH;
@@ -584,18 +598,30 @@ extern "C" int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float 
         if (max_n == 0) continue;
         int64_t gx = (max_n + 1023) / 1024;
         if (gx > 512) gx = 512;
-        hipLaunchKernelGGL(sgd_multi_kernel, dim3((unsigned)gx, (unsigned)nb), dim3(256), 0, (hipStream_t)stream, b, lr);
+        hipLaunchKernelGGL(sgd_multi_kernel, dim3((unsigned)gx, (unsigned)nb), dim3(256), 0, (hipStream_t)stream, b, lr, sums, summed ? 0 : n_terms,
+                           sum_out);
+        summed = true;
         int rc = check_launch("hgq_sgd_update_multi");
         if (rc) return rc;
     }
+    if (!summed) return hgq_sum_scalars(terms, n_terms, sum_out, stream);  // nothing to update: the sum alone
     return HGQ_OK;
 }
 
-namespace hgq {
-struct SumBatch {
-    const float *term[HGQ_SUM_BATCH];
-};
+extern "C" int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *stream) {
+    return sgd_update_multi_impl(items, count, lr, nullptr, 0, nullptr, stream);
+}
 
+extern "C" int hgq_sgd_update_multi_sum(const hgq_sgd_item *items, int count, float lr, const float *const *terms, int n_terms,
+                                        float *sum_out, void *stream) {
+    if (n_terms < 1 || n_terms > HGQ_SUM_BATCH || !terms || !sum_out)
+        return fail(HGQ_ERR_ARG, "hgq_sgd_update_multi_sum: 1 <= n_terms <= %d terms and an output are expected", HGQ_SUM_BATCH);
+    for (int t = 0; t < n_terms; ++t)
+        if (!terms[t]) return fail(HGQ_ERR_ARG, "hgq_sgd_update_multi_sum: null term %d", t);
+    return sgd_update_multi_impl(items, count, lr, terms, n_terms, sum_out, stream);
+}
+
+namespace hgq {
 // one thread: the terms are added in list order, exactly as a chain of scalar additions would
 __global__ void sum_scalars_kernel(SumBatch b, int count, float *out) {
     if (threadIdx.x == 0 && blockIdx.x == 0) {

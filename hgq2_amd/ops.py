@@ -450,7 +450,9 @@ _OVERLAP = {'depth': 0, 'streams': {}, 'pending': [], 'keep': [], 'finish': []}
 class overlap_ebops:
     """Context manager around a training step (forward, loss, backward, update): EBOPs launches inside it run on a
     second stream.  Whoever opens it must leave it before the captured graph ends or before results are read from
-    another thread or stream; leaving it joins the second stream."""
+    another thread or stream; leaving it joins the second stream.  ``hgq2_amd.train.model_loss`` called inside it
+    returns a total without an autograd graph whose value is there once the context is left (the terms carry the
+    graph: ``SGD.backward`` starts from them)."""
 
     def __enter__(self):
         _OVERLAP['depth'] += 1
@@ -487,15 +489,25 @@ class side_branch:
         return False
 
 
-def join_side():
-    """The current stream waits for the second stream's work (no-op when there is none)."""
+def join_side(hand_over_sums: bool = False, sums_later: bool = False):
+    """The current stream waits for the second stream's work (no-op when there is none).  Work that needed both streams'
+    results - the sums of loss terms, ``(terms, out)`` pairs - runs now, or is returned to a caller that folds it into a
+    launch of its own (``hand_over_sums``; sums of more than ``SUM_BATCH`` terms run here either way), or stays queued
+    for the next join (``sums_later``: a join in the middle of a step; the one that ends the step finds them)."""
     pending, _OVERLAP['pending'] = _OVERLAP['pending'], []
     for cur, side in pending:
         torch.cuda.current_stream(cur.device).wait_stream(side)
+    if sums_later:
+        return []
     finish, _OVERLAP['finish'] = _OVERLAP['finish'], []
-    for launch in finish:  # work that needed both streams' results (the sum of the loss terms)
-        launch()
+    handed = []
+    for terms, out in finish:
+        if hand_over_sums and len(terms) <= SUM_BATCH:
+            handed.append((terms, out))
+        else:
+            sum_scalars_into(terms, out)
     _OVERLAP['keep'] = []
+    return handed
 
 
 def _keep(tensors):
@@ -550,7 +562,7 @@ def _order_after_side():
     if _OVERLAP['pending']:
         cur = torch.cuda.current_stream()
         if not any(cur == side for _, side in _OVERLAP['pending']):
-            join_side()
+            join_side(sums_later=True)
 
 
 def flush_tracks():
@@ -680,11 +692,13 @@ class _SgdItem(ctypes.Structure):
                 ('side_scale', ctypes.c_void_p * SGD_SIDES)]
 
 
-@torch.library.custom_op('hgq::sgd_update_multi', mutates_args=('ws',))
+@torch.library.custom_op('hgq::sgd_update_multi', mutates_args=('ws', 'sum_out'))
 def sgd_update_multi_op(ws: Sequence[Tensor], gs: Sequence[Tensor], l1: Sequence[float], lo: Sequence[float],
-                        hi: Sequence[float], lr: float, sides: Sequence[Tensor], side_scales: Sequence[Tensor]) -> None:
+                        hi: Sequence[float], lr: float, sides: Sequence[Tensor], side_scales: Sequence[Tensor],
+                        sum_terms: Sequence[Tensor], sum_out: Tensor) -> None:
     """``gs[t]`` empty: no plain gradient.  ``sides`` / ``side_scales``: SGD_SIDES entries per variable (empty = absent;
-    an absent scale means 1)."""
+    an absent scale means 1).  ``sum_terms`` (1 to SUM_BATCH one-element tensors, or none): added in list order into
+    ``sum_out`` by the same launch - the step's loss terms, which the update does not read."""
     n = len(ws)
     _need(len(gs) == n and len(l1) == n and len(lo) == n and len(hi) == n, 'per-variable lists differ in length')
     _need(len(sides) == SGD_SIDES * n and len(side_scales) == SGD_SIDES * n, 'side-gradient lists must hold SGD_SIDES entries per variable')
@@ -705,6 +719,17 @@ def sgd_update_multi_op(ws: Sequence[Tensor], gs: Sequence[Tensor], l1: Sequence
                     _need(sc.is_cuda and sc.dtype == torch.float32 and sc.numel() == 1, 'a side-gradient scale is one float32 on the GPU')
                     it.side_scale[s] = sc.data_ptr()
         items[t] = it
+    if len(sum_terms):
+        _need(len(sum_terms) <= SUM_BATCH, f'at most {SUM_BATCH} terms ride along with the update')
+        ptrs = (ctypes.c_void_p * len(sum_terms))()
+        for t, term in enumerate(sum_terms):
+            _check_f32('term', term)
+            _need(term.numel() == 1, 'every term must hold one element')
+            ptrs[t] = term.data_ptr()
+        _check_f32('sum_out', sum_out)
+        rc = _lib.load().hgq_sgd_update_multi_sum(items, n, lr, ptrs, len(sum_terms), _ptr(sum_out), _stream())
+        _lib.check(rc, 'hgq_sgd_update_multi_sum')
+        return
     rc = _lib.load().hgq_sgd_update_multi(items, n, lr, _stream())
     _lib.check(rc, 'hgq_sgd_update_multi')
 
@@ -2565,8 +2590,9 @@ def sgd_update_(w, g, lr, l1=0.0, lo=float('-inf'), hi=float('inf')):
     sgd_update_op(w, g.contiguous(), float(lr), float(l1), float(lo), float(hi))
 
 
-def sgd_update_multi_(ws, gs, l1, lo, hi, lr, sides=None):
-    """``gs[t]`` may be ``None``; ``sides[t]`` is a list of up to ``SGD_SIDES`` ``(scale or None, gradient)`` pairs."""
+def sgd_update_multi_(ws, gs, l1, lo, hi, lr, sides=None, sum_terms=None, sum_out=None):
+    """``gs[t]`` may be ``None``; ``sides[t]`` is a list of up to ``SGD_SIDES`` ``(scale or None, gradient)`` pairs.
+    ``sum_terms`` / ``sum_out``: scalars added up in list order into ``sum_out`` by the update's launch."""
     n = len(ws)
     dev = ws[0].device
     empty = torch.empty(0, dtype=torch.float32, device=dev)
@@ -2581,7 +2607,8 @@ def sgd_update_multi_(ws, gs, l1, lo, hi, lr, sides=None):
         for _ in range(SGD_SIDES - len(pairs)):
             flat_s.append(empty), flat_c.append(empty)
     sgd_update_multi_op(list(ws), [g.contiguous() if g is not None else empty for g in gs], [float(v) for v in l1],
-                        [float(v) for v in lo], [float(v) for v in hi], float(lr), flat_s, flat_c)
+                        [float(v) for v in lo], [float(v) for v in hi], float(lr), flat_s, flat_c,
+                        [t.detach() for t in sum_terms] if sum_terms else [], sum_out if sum_terms else empty)
 
 
 # ======================================================================================

@@ -30,14 +30,15 @@ def model_loss(model, base_loss, fold_regularizers: bool = False):
         if fold_regularizers and isinstance(r, MonoL1):
             continue
         terms.append(r(p))
-    if ops._OVERLAP['pending'] and len(terms) > 1 and all(
+    if ops._OVERLAP['depth'] and len(terms) > 1 and all(
             torch.is_tensor(t) and t.is_cuda and t.dtype == torch.float32 and t.numel() == 1 for t in terms):
-        # EBOPs launches of this step are running on the second stream: the total (nothing but the caller's print-out
-        # reads it) is summed when the streams are joined, and the backward pass starts from the terms themselves -
+        # inside `ops.overlap_ebops()` (EBOPs launches of this step may be running on the second stream): the total -
+        # nothing but the caller's print-out reads it - is summed when the streams are joined for the last time, inside
+        # the update's launch when :class:`SGD` makes it, and the backward pass starts from the terms themselves -
         # d total / d term = 1 - so the first stream does not wait for the second before the update
         total = torch.empty(torch.broadcast_shapes(*[t.shape for t in terms]), dtype=torch.float32, device=terms[0].device)
         held = list(terms)
-        ops._OVERLAP['finish'].append(lambda: ops.sum_scalars_into(held, total))
+        ops._OVERLAP['finish'].append((held, total))
         total._hgq_terms = [t for t in terms if t.requires_grad]
         return total
     ops.join_side()  # EBOPs terms issued on the second stream
@@ -86,7 +87,7 @@ class SGD:
 
     @torch.no_grad()
     def step(self):
-        ops.join_side()
+        sums = ops.join_side(hand_over_sums=True)  # the loss terms' sum rides along with the update launch
         ws, gs, l1s, los, his, sides, post = [], [], [], [], [], [], []
         for p in self.params:
             side = list(getattr(p, '_hgq_side', None) or ())
@@ -108,9 +109,12 @@ class SGD:
             l1s.append(r.l1 if (self.fold_regularizers and isinstance(r, MonoL1)) else 0.0)
             los.append(bounds[0])
             his.append(bounds[1])
+        ride = sums.pop(0) if (ws and sums) else (None, None)
+        for terms, out in sums:
+            ops.sum_scalars_into(terms, out)
         if ws:
             ops.touch_state()  # written through `.data`: the version counters do not move
-            ops.sgd_update_multi_(ws, gs, l1s, los, his, self.lr, sides)
+            ops.sgd_update_multi_(ws, gs, l1s, los, his, self.lr, sides, sum_terms=ride[0], sum_out=ride[1])
         for p, c in post:
             p.copy_(c(p))
 

@@ -435,6 +435,10 @@ int hgq_sgd_update_multi(const hgq_sgd_item *items, int count, float lr, void *s
  */
 #define HGQ_SUM_BATCH 64
 int hgq_sum_scalars(const float *const *terms, int count, float *out, void *stream);
+/* hgq_sgd_update_multi with hgq_sum_scalars riding along in its (first) launch: a training step's loss terms, which the
+ * update does not read, are added up for the caller's report without a launch of their own. */
+int hgq_sgd_update_multi_sum(const hgq_sgd_item *items, int count, float lr, const float *const *terms, int n_terms, float *sum_out,
+                             void *stream);
 
 /*
  * One training step (forward, mean sparse categorical cross-entropy from logits, backward, SGD)

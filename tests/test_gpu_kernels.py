@@ -454,6 +454,16 @@ def test_sparse_ce_and_sgd(dev):
     ops.sgd_update_multi_(wds, gds, [1e-8] * n, [-1.0] * n, [float('inf')] * n, 0.05)
     for wd_, w_, g_ in zip(wds, ws, gs):
         assert torch.equal(wd_.cpu(), torch.clamp(w_ - 0.05 * (g_ + 1e-8), min=-1.0))
+    # loss terms riding along with the update: the same additions in the same order as the launch of their own,
+    # the update unchanged
+    terms = [(torch.randn((), generator=g) * 10.0 ** (t % 5)).to(dev) for t in range(ops.SUM_BATCH)]
+    for n_terms in (1, 3, ops.SUM_BATCH):
+        wds2, out = [t.to(dev) for t in ws], torch.full((), float('nan'), device=dev)
+        ops.sgd_update_multi_(wds2, gds, [1e-8] * n, [-1.0] * n, [float('inf')] * n, 0.05, sum_terms=terms[:n_terms], sum_out=out)
+        assert torch.equal(out, ops.sum_scalars([t.clone() for t in terms[:n_terms]]).reshape(()))
+        assert all(torch.equal(a, b) for a, b in zip(wds2, wds))
+    with pytest.raises(ValueError):
+        ops.sgd_update_multi_(wds2, gds, [0.0] * n, [-1.0] * n, [1.0] * n, 0.05, sum_terms=terms + terms[:1], sum_out=out)
 
 
 @pytest.mark.parametrize('rows,M', [(4096, 16), (2048, 4096), (1000, 7)])
