@@ -347,6 +347,16 @@ class Sequential(Layer):
         self.built = True
 
     def call(self, x, training=None):
-        for layer in self.layers:
+        layers, k = list(self.layers), 0
+        while k < len(layers):
+            layer = layers[k]
+            nxt = layers[k + 1] if k + 1 < len(layers) else None
+            absorbs = getattr(layer, 'absorbs', None)
+            if nxt is not None and absorbs is not None and isinstance(layer, Layer) and absorbs(nxt, x):
+                # the two layers as one call: nothing else can read what passes between them here
+                x = layer(x, training=training, then=nxt)
+                k += 2
+                continue
             x = layer(x) if not isinstance(layer, Layer) else layer(x, training=training)
+            k += 1
         return x

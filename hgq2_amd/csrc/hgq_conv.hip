@@ -553,11 +553,15 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
 //     entries over the owned pixels in registers.
 // After its last tile the workgroup adds the 8 slots in slot order and writes slice blockIdx.x of
 // `part` ([KC * F | F]); a second kernel adds the slices in order.
+// `dyp` (with `mask` = the forward output): the gradient arrives behind a 2 x 2 maximum pooling of stride 2 without
+// padding, as [B, PHo, PWo, F]; dz is built from it while the patch is staged (the pooling layer's backward pass - one
+// more read of the forward output and a write and a read of a gradient four times the size - does not run).
 template <int KH, int KW, int C>
 __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict__ dy, const float *__restrict__ mask,
                                                          const float *__restrict__ x, const float *__restrict__ w,
                                                          float *__restrict__ dx, float *__restrict__ part, hgq_conv_geom g, int F,
-                                                         int tiles_x, int tiles_y, int vec) {
+                                                         int tiles_x, int tiles_y, int vec, const float *__restrict__ dyp, int PHo,
+                                                         int PWo, int relu) {
     // the multiply-adds of the two contractions below may fuse (the file is built without contraction for the quantizer
     // arithmetic; a convolution sum has no such contract, and unfused it costs two vector instructions per term)
 #pragma clang fp contract(fast)
@@ -570,7 +574,8 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
     // whole-tensor buffer descriptors (the launcher guarantees they are smaller than 2 GiB)
     const int64_t dy_bytes = (int64_t)g.B * g.OH * g.OW * F * 4;
     const __amdgpu_buffer_rsrc_t rs_dy = buf_rsrc(dy, dy_bytes), rs_mask = buf_rsrc(mask ? mask : dy, mask ? dy_bytes : 0),
-                                 rs_x = buf_rsrc(x, (int64_t)g.B * g.H * g.W * C * 4);
+                                 rs_x = buf_rsrc(x, (int64_t)g.B * g.H * g.W * C * 4),
+                                 rs_dyp = buf_rsrc(dyp ? dyp : mask, dyp ? (int64_t)g.B * PHo * PWo * F * 4 : 0);
     float wacc[KC], bacc = 0.f;
 #pragma unroll
     for (int t = 0; t < KC; ++t) wacc[t] = 0.f;
@@ -581,7 +586,51 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
         const int oy0 = iy0 + g.py - (KH - 1), ox0 = ix0 + g.px - (KW - 1);
         __syncthreads();
         // buffer loads (zeros outside the tensor, no branch around a load): all units of a batch are in flight together
-        if (vec) {
+        if (dyp) {
+            // unit = one pooling window x four filters (the patch starts on a window boundary and holds whole windows:
+            // the launcher checks it).  An output pixel takes its window's gradient where it holds the window's first
+            // maximum in row-major order - what the pooling kernels do - and, behind a ReLU, is positive.
+            const int f4 = F / 4, wpr = PW / 2, n_u = (PH / 2) * wpr * f4;
+            const FastDiv d_f4((uint32_t)f4), d_wpr((uint32_t)wpr);
+            for (int e0 = 0; e0 < n_u; e0 += 2 * 256) {
+                f32x4_t yv[2][4], gv[2];
+                int dst[2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int e = e0 + u * 256 + tid;
+                    uint32_t off_g = BUF_OOB, off_y = BUF_OOB;
+                    dst[u] = -1;
+                    if (e < n_u) {
+                        const int wi = (int)d_f4.div((uint32_t)e), f0 = (e - wi * f4) * 4, wr = (int)d_wpr.div((uint32_t)wi), wc = wi - wr * wpr;
+                        const int oy = oy0 + 2 * wr, ox = ox0 + 2 * wc;
+                        dst[u] = (2 * wr * PW + 2 * wc) * FS + f0;
+                        if ((unsigned)oy < (unsigned)(2 * PHo) && (unsigned)ox < (unsigned)(2 * PWo)) {
+                            off_g = (uint32_t)(((b * PHo + (oy >> 1)) * PWo + (ox >> 1)) * F + f0) * 4u;
+                            off_y = (uint32_t)(((b * g.OH + oy) * g.OW + ox) * F + f0) * 4u;
+                        }
+                    }
+                    gv[u] = buf_ld4(rs_dyp, off_g);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        yv[u][j] = buf_ld4(rs_mask, off_y == BUF_OOB ? BUF_OOB : off_y + (uint32_t)(((j >> 1) * g.OW + (j & 1)) * F) * 4u);
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    if (dst[u] < 0) continue;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float best = yv[u][0][c];
+                        int first = 0;
+#pragma unroll
+                        for (int j = 1; j < 4; ++j)
+                            if (yv[u][j][c] > best) best = yv[u][j][c], first = j;
+                        const float gz = (!relu || best > 0.f) ? gv[u][c] : 0.f;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) zp[dst[u] + ((j >> 1) * PW + (j & 1)) * FS + c] = first == j ? gz : 0.f;
+                    }
+                }
+            }
+        } else if (vec) {
             const int upr = PW * F / 4, n_u = PH * upr;
             const FastDiv d_upr((uint32_t)upr), d_f((uint32_t)F);  // no integer division per unit
             for (int e0 = 0; e0 < n_u; e0 += 4 * 256) {
@@ -1335,6 +1384,14 @@ extern "C" int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F) {
     return slices * ((int64_t)K * F + F);
 }
 
+extern "C" int hgq_conv2d_maxpool_bwd_supported(const hgq_conv_geom *g, int F) {
+    if (!g || F < 1) return 0;
+    // the kernel's patch of output pixels starts at (8 ty + py - (kh - 1), 32 tx + px - (kw - 1)) and is (8 + kh - 1) x
+    // (32 + kw - 1): whole windows when both offsets and both sizes are even
+    return bwd_smallc_ok(*g, F) && F % 4 == 0 && g->OH >= 2 && g->OW >= 2 && (g->kh - 1 - g->py) % 2 == 0 &&
+           (g->kw - 1 - g->px) % 2 == 0 && (g->kh & 1) && (g->kw & 1) && (int64_t)g->B * g->OH * g->OW > 0;
+}
+
 extern "C" int64_t hgq_conv2d_bwd_slice_count(const hgq_conv_geom *g, int F) {
     if (check_geom(g, F, "hgq_conv2d_bwd_slice_count")) return -1;
     const int64_t rows = (int64_t)g->B * g->OH * g->OW;
@@ -1346,8 +1403,10 @@ extern "C" int64_t hgq_conv2d_bwd_slice_count(const hgq_conv_geom *g, int F) {
 
 // reduce: the slices of the kernel / bias gradient are summed into dqw / dqb; otherwise they stay in `workspace`
 // ([hgq_conv2d_bwd_slice_count][kh kw C F + F]) and dqw / dqb only say whether the gradient is wanted
+// dyp: the gradient behind a 2 x 2 / stride 2 / unpadded maximum pooling of the output ([B, OH / 2, OW / 2, F]) instead of dy
 static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
-                           float *workspace, const hgq_conv_geom *g, int F, int act, void *stream, bool reduce) {
+                           float *workspace, const hgq_conv_geom *g, int F, int act, void *stream, bool reduce,
+                           const float *dyp = nullptr) {
     int rc = check_geom(g, F, "hgq_conv2d_bwd");
     if (rc) return rc;
     if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: unknown activation %d", act);
@@ -1361,9 +1420,11 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
         if (dxq && (rc = fill_f32(dxq, 0.f, in_rows * g->C, s))) return rc;
         return HGQ_OK;
     }
-    if (!dy || !qw || !xq) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null pointer");
-    if (act == HGQ_ACT_RELU && !y) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: relu needs the forward output");
-    const float *mask = act == HGQ_ACT_RELU ? y : nullptr;
+    if ((!dy && !dyp) || !qw || !xq) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null pointer");
+    if ((act == HGQ_ACT_RELU || dyp) && !y) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: relu / pooling need the forward output");
+    const float *mask = (act == HGQ_ACT_RELU || dyp) ? y : nullptr;
+    if (dyp && !(hgq_conv2d_maxpool_bwd_supported(g, F) && aligned16(dyp) && aligned16(y)))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_maxpool_bwd: shape or alignment not supported (ask hgq_conv2d_maxpool_bwd_supported)");
     if (bwd_smallc_ok(*g, F)) {
         const bool want_w = dqw || dqb;
         if (want_w && !workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null workspace");
@@ -1372,7 +1433,7 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
         const size_t lds = bwd_smallc_lds(*g, F);
         const int vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask));
 #define HGQ_BWD_SC(KH, KW, CC) \
-    hipLaunchKernelGGL((bwd_smallc_kernel<KH, KW, CC>), dim3((unsigned)grid), dim3(256), lds, s, dy, mask, xq, qw, dxq, want_w ? workspace : (float *)nullptr, *g, F, tiles_x, tiles_y, vec)
+    hipLaunchKernelGGL((bwd_smallc_kernel<KH, KW, CC>), dim3((unsigned)grid), dim3(256), lds, s, dy, mask, xq, qw, dxq, want_w ? workspace : (float *)nullptr, *g, F, tiles_x, tiles_y, vec, dyp, g->OH / 2, g->OW / 2, act == HGQ_ACT_RELU)
         HGQ_SMALLC_DISPATCH(HGQ_BWD_SC);
 #undef HGQ_BWD_SC
         if ((rc = check_launch("hgq_conv2d_bwd(few channels)"))) return rc;
@@ -1460,6 +1521,14 @@ extern "C" int hgq_conv2d_bwd_slices(const float *dy, const float *y, const floa
     }
     // the kernels only test the gradient pointers for "is it wanted": any non-null value stands for it
     return conv2d_bwd_impl(dy, y, xq, qw, dxq, workspace, workspace, workspace, g, F, act, stream, false);
+}
+
+extern "C" int hgq_conv2d_maxpool_bwd(const float *dyp, const float *y, const float *xq, const float *qw, float *dxq, float *dqw,
+                                      float *dqb, float *workspace, const hgq_conv_geom *g, int F, int act, int reduce, void *stream) {
+    if (!dyp) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_bwd: null pointer");
+    if (!reduce && !workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_bwd: null workspace");
+    if (reduce) return conv2d_bwd_impl(nullptr, y, xq, qw, dxq, dqw, dqb, workspace, g, F, act, stream, true, dyp);
+    return conv2d_bwd_impl(nullptr, y, xq, qw, dxq, workspace, workspace, workspace, g, F, act, stream, false, dyp);
 }
 
 extern "C" int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, const hgq_conv_geom *g, int F, float *total,

@@ -97,14 +97,29 @@ class QConv2D(QLayerBaseSingleInput):
             assert self.n_parallel is not None
             self.parallelization_factor = self.n_parallel
 
-    def convolution_op(self, x_nhwc, kernel_hwio, bias=None, act_code=_lib.ACT_NONE):
+    def convolution_op(self, x_nhwc, kernel_hwio, bias=None, act_code=_lib.ACT_NONE, maxpool2=False):
         """``act(conv(x, kernel) + bias)`` on channels-last tensors through the implicit-GEMM kernels."""
-        return ops.conv2d(x_nhwc, kernel_hwio, bias, self.strides, self.padding, self.dilation_rate, act_code)
+        return ops.conv2d(x_nhwc, kernel_hwio, bias, self.strides, self.padding, self.dilation_rate, act_code, maxpool2)
 
-    def call(self, inputs, training=None):
+    def absorbs(self, nxt, x) -> bool:
+        """Whether a call may take the layer that follows in a :class:`Sequential` with it (``call(..., then=nxt)``): a plain
+        2 x 2 maximum pooling of stride 2 behind a linear or ReLU convolution without output quantizer, on a shape the
+        kernels take.  The unpooled output then never leaves the layer, and its backward pass starts from the pooled gradient."""
+        from ..host import MaxPooling2D
+
+        if type(nxt) is not MaxPooling2D or nxt.pool_size != (2, 2) or nxt.strides != (2, 2) or nxt.padding != 'valid':
+            return False
+        if self.enable_oq or self._act_name not in (None, 'linear', 'relu') or not torch.is_tensor(x) or not x.is_cuda or x.dim() != 4:
+            return False
+        geom = ops.conv_geometry(tuple(x.shape), self.kernel_size + (x.shape[-1], self.filters), self.strides, self.padding, self.dilation_rate)
+        return geom[0] > 0 and ops.conv2d_maxpool_supported(geom, self.filters)
+
+    def call(self, inputs, training=None, then=None):
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
         fused_act = _lib.ACT_RELU if self._act_name == 'relu' else _lib.ACT_NONE
+        if then is not None:
+            return self.convolution_op(inputs, self.qkernel, self.qbias if self.use_bias else None, fused_act, True)
         outputs = self.convolution_op(inputs, self.qkernel, self.qbias if self.use_bias else None, fused_act)
         if self.activation is not None and fused_act == _lib.ACT_NONE:
             outputs = self.activation(outputs)

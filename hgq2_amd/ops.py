@@ -1043,6 +1043,40 @@ def _(dy, y, xq, qw, geom, act, need_dx):
     return xq.new_empty(xq.shape if need_dx else (0,)), xq.new_empty((1, qw.numel() + qw.shape[-1]))
 
 
+@torch.library.custom_op('hgq::conv2d_maxpool_bwd', mutates_args=())
+def conv2d_maxpool_bwd(dyp: Tensor, y: Tensor, xq: Tensor, qw: Tensor, geom: Sequence[int], act: int, need_dx: bool,
+                       reduce: bool) -> tuple[Tensor, Tensor]:
+    """Backward of a convolution behind a 2 x 2 / stride 2 / unpadded maximum pooling from the pooled gradient ``dyp``:
+    ``(dx, slices [n, kh kw C F + F])``, or with ``reduce`` ``(dx, [kh kw C F + F])`` (kernel gradient, then bias gradient)."""
+    _check_f32('dyp', dyp), _check_f32('y', y), _check_f32('xq', xq), _check_f32('qw', qw)
+    g = _geom(geom)
+    F = qw.shape[-1]
+    _need(y.numel() == g.B * g.OH * g.OW * F, 'y must be [B, OH, OW, F]')
+    _need(dyp.numel() == g.B * (g.OH // 2) * (g.OW // 2) * F, 'dyp must be [B, OH // 2, OW // 2, F]')
+    lib = _lib.load()
+    dx = torch.empty(xq.shape if need_dx else (0,), dtype=torch.float32, device=xq.device)
+    n = lib.hgq_conv2d_bwd_slice_count(ctypes.addressof(g), F)
+    _need(n >= 1, 'hgq_conv2d_bwd_slice_count rejected the geometry')
+    ws = torch.empty((int(n), qw.numel() + F), dtype=torch.float32, device=xq.device)
+    out = torch.empty(qw.numel() + F, dtype=torch.float32, device=xq.device) if reduce else ws
+    rc = lib.hgq_conv2d_maxpool_bwd(_ptr(dyp), _ptr(y), _ptr(xq), _ptr(qw), _ptr(dx) if need_dx else None, _ptr(out),
+                                    out.data_ptr() + 4 * qw.numel() if reduce else None, _ptr(ws), ctypes.addressof(g), F, act,
+                                    int(reduce), _stream())
+    _lib.check(rc, 'hgq_conv2d_maxpool_bwd')
+    return dx, out
+
+
+@conv2d_maxpool_bwd.register_fake
+def _(dyp, y, xq, qw, geom, act, need_dx, reduce):
+    n = qw.numel() + qw.shape[-1]
+    return xq.new_empty(xq.shape if need_dx else (0,)), xq.new_empty((n,) if reduce else (1, n))
+
+
+def conv2d_maxpool_supported(geom, F: int) -> bool:
+    g = _geom(geom)
+    return bool(_lib.load().hgq_conv2d_maxpool_bwd_supported(ctypes.addressof(g), int(F)))
+
+
 @torch.library.custom_op('hgq::col_moments_fwd', mutates_args=())
 def col_moments_fwd(x: Tensor) -> tuple[Tensor, Tensor]:
     _check_f32('x', x)
@@ -2066,11 +2100,43 @@ class _Conv2D(torch.autograd.Function):
         return (dx if ctx.needs_input_grad[0] else None, dqw, dqb if ctx.has_bias else None, None, None)
 
 
-def conv2d(xq: Tensor, qw: Tensor, qb, strides=(1, 1), padding='valid', dilation=(1, 1), act: int = 0) -> Tensor:
+class _Conv2DMaxPool(torch.autograd.Function):
+    """Convolution and the 2 x 2 maximum pooling that is its only reader as one node: the unpooled output stays inside
+    (saved for the backward pass, which forms its gradient from the pooled one while it stages its tiles)."""
+
+    @staticmethod
+    def forward(ctx, xq, qw, qb, geom, act):
+        y = conv2d_fwd(xq, qw, qb, list(geom), act)
+        B, OH, OW, F = geom[0], geom[12], geom[13], qw.shape[-1]
+        yp = pool2d_fwd(y, [B, OH, OW, F, 2, 2, 2, 2, 0, 0, OH // 2, OW // 2], True)
+        ctx.save_for_backward(xq, qw, y)
+        ctx.geom, ctx.act, ctx.has_bias = tuple(geom), act, qb.numel() > 0
+        ctx.defer = getattr(qw, '_hgq_single_use', False) and (qb.numel() == 0 or getattr(qb, '_hgq_single_use', False))
+        return yp
+
+    @staticmethod
+    def backward(ctx, gyp):
+        xq, qw, y = ctx.saved_tensors
+        need_dx = ctx.needs_input_grad[0]
+        if ctx.defer and _SINK['open']:  # as in _Conv2D: the slices join the pass's one reduction launch
+            dx, ws = conv2d_maxpool_bwd(gyp.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, need_dx, False)
+            dqw, dqb = torch.empty_like(qw), xq.new_empty(qw.shape[-1])
+            _PENDING_REDUCE.append((ws, (dqw.view(-1), dqb, xq.new_empty(0)), (False, not ctx.has_bias, True)))
+        else:
+            dx, flat = conv2d_maxpool_bwd(gyp.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, need_dx, True)
+            dqw, dqb = flat[:qw.numel()].view(qw.shape), flat[qw.numel():]
+        return (dx if need_dx else None, dqw, dqb if ctx.has_bias else None, None, None)
+
+
+def conv2d(xq: Tensor, qw: Tensor, qb, strides=(1, 1), padding='valid', dilation=(1, 1), act: int = 0, maxpool2: bool = False) -> Tensor:
     """``act(conv2d(xq, qw) + qb)`` for a channels-last input [B, H, W, C] and an HWIO kernel; 'same'
-    padding puts the odd pad after the last row / column, as Keras / TensorFlow do."""
+    padding puts the odd pad after the last row / column, as Keras / TensorFlow do.  ``maxpool2``: followed by a 2 x 2
+    maximum pooling of stride 2 without padding, for shapes ``conv2d_maxpool_supported`` accepts."""
     _need(qw.shape[2] == xq.shape[3], f'kernel has {qw.shape[2]} input channels, input has {xq.shape[3]}')
     geom = conv_geometry(tuple(xq.shape), tuple(qw.shape), strides, padding, dilation)
+    if maxpool2:
+        _need(conv2d_maxpool_supported(geom, qw.shape[-1]), 'convolution + pooling in one node: shape not supported')
+        return _Conv2DMaxPool.apply(xq.contiguous(), qw.contiguous(), qb.contiguous() if qb is not None else xq.new_empty(0), geom, act)
     return _Conv2D.apply(xq.contiguous(), qw.contiguous(), qb.contiguous() if qb is not None else xq.new_empty(0), geom, act)
 
 

@@ -586,6 +586,21 @@ int hgq_conv2d_bwd(const float *dy, const float *y, const float *xq, const float
 int64_t hgq_conv2d_bwd_slice_count(const hgq_conv_geom *g, int F);
 int hgq_conv2d_bwd_slices(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *workspace,
                           const hgq_conv_geom *g, int F, int act, void *stream);
+/*
+ * hgq_conv2d_bwd for a convolution whose output is read by a 2 x 2 maximum pooling of stride 2 without padding and by
+ * nothing else (QConv2D followed by MaxPooling2D - the Keras layer the reference's models put behind it, e.g.
+ * /root/reference/tests/test_layers/test_pool.py:16-40 for the pooling semantics): `dyp` is the gradient of the POOLED
+ * output, [B, OH / 2, OW / 2, F]; the gradient of the convolution's output - dyp where a pixel holds its window's first
+ * maximum in row-major order (what hgq_pool2d_bwd does), zero elsewhere and in a trailing odd row / column - is formed
+ * while the kernel stages its tiles, so the pooling's own backward pass does not run.  `y` (the convolution's output) is
+ * always read.  reduce = 0: the kernel / bias gradient stays in `workspace` as slices (hgq_conv2d_bwd_slices), else it is
+ * summed into dqw / dqb.  hgq_conv2d_maxpool_bwd_supported: 1 where the few-input-channel kernel takes the shape with F a
+ * multiple of 4 (kernels of odd size; 'valid', or a 'same' padding that keeps the tiles on window boundaries);
+ * HGQ_ERR_UNSUPPORTED otherwise, and for dyp / y not aligned to 16 bytes.
+ */
+int hgq_conv2d_maxpool_bwd_supported(const hgq_conv_geom *g, int F);
+int hgq_conv2d_maxpool_bwd(const float *dyp, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
+                           float *workspace, const hgq_conv_geom *g, int F, int act, int reduce, void *stream);
 
 /*
  * One quantizer's bit-width view for the EBOPs entry points below: `bits` / `fbits` as hgq_qbits_fwd forms

@@ -245,3 +245,98 @@ def test_conv2d_backward_slices_sum_to_the_reduced_gradient(dev, case):
     assert torch.equal(outs[0].view(w.shape), dqw)
     if bias:
         assert torch.equal(outs[1], dqb)
+
+
+@pytest.mark.parametrize('shape', [
+    # B, H, W, C, k, F, padding, relu, bias, quantized (ties inside the windows)
+    (3, 28, 28, 1, 3, 32, 'valid', True, True, False),   # the image configuration's first layer
+    (2, 13, 17, 3, 3, 8, 'valid', False, True, True),    # odd output sizes: a trailing row and column without a window
+    (2, 12, 40, 1, 5, 16, 'same', True, False, True),    # 5 x 5 'same' keeps the tiles on window boundaries
+    (1, 9, 70, 4, 3, 4, 'valid', True, True, False),     # several tiles across
+])
+def test_convolution_backward_from_the_pooled_gradient(dev, shape):
+    """`hgq_conv2d_maxpool_bwd` (the convolution and the 2 x 2 maximum pooling behind it as one autograd node) gives the
+    bits of the two nodes one after the other: the same pooled output, data / kernel / bias gradient."""
+    from hgq2_amd import _lib, ops
+
+    B, H, W, C, k, Fo, padding, relu, bias, quantized = shape
+    g = torch.Generator().manual_seed(B * H + W + Fo)
+    x = torch.randn(B, H, W, C, generator=g)
+    w = torch.randn(k, k, C, Fo, generator=g) * 0.3
+    b = torch.randn(Fo, generator=g) if bias else None
+    if quantized:  # few distinct values: equal maxima inside a window
+        x, w = torch.round(x * 2) / 2, torch.round(w * 4) / 4
+        b = torch.round(b) if bias else None
+    act = _lib.ACT_RELU if relu else _lib.ACT_NONE
+    geom = ops.conv_geometry((B, H, W, C), (k, k, C, Fo), (1, 1), padding, (1, 1))
+    assert ops.conv2d_maxpool_supported(geom, Fo)
+    got = []
+    for fused in (False, True):
+        xs, ws = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+        bs = b.to(dev).requires_grad_(True) if bias else None
+        if fused:
+            yp = ops.conv2d(xs, ws, bs, (1, 1), padding, (1, 1), act, maxpool2=True)
+        else:
+            yp = ops.pool2d(ops.conv2d(xs, ws, bs, (1, 1), padding, (1, 1), act), (2, 2), (2, 2), 'valid', 'max')
+        dyp = torch.randn(yp.shape, generator=torch.Generator().manual_seed(5)).to(dev)
+        yp.backward(dyp)
+        got.append((yp.detach(), xs.grad, ws.grad, bs.grad if bias else None))
+    for name, a, f in zip(('pooled output', 'dx', 'dw', 'db'), got[0], got[1]):
+        if a is not None:
+            assert torch.equal(a, f), f'{name}: {float((a - f).abs().max())}'
+    # and against torch's own kernels in fp64 on the CPU
+    xd, wd = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    pad = (k - 1) // 2 if padding == 'same' else 0
+    yd = torch.nn.functional.conv2d(xd.permute(0, 3, 1, 2), wd.permute(3, 2, 0, 1), b.double() if bias else None, padding=pad)
+    ypd = torch.nn.functional.max_pool2d(torch.relu(yd) if relu else yd, 2).permute(0, 2, 3, 1)
+    assert float((got[1][0].cpu().double() - ypd.detach()).abs().max()) <= 1e-5 * float(ypd.detach().abs().max())
+    if not quantized:  # with ties torch may pick another of the equal maxima
+        ypd.backward(torch.randn(ypd.shape, generator=torch.Generator().manual_seed(5)).double())
+        for name, f, r in (('dx', got[1][1], xd.grad), ('dw', got[1][2], wd.grad)):
+            assert float((f.cpu().double() - r).abs().max()) <= 1e-5 * float(r.abs().max()) + 1e-6, name
+
+
+def test_unsupported_shapes_of_the_pooled_backward_are_refused(dev):
+    from hgq2_amd import ops
+
+    for geom_args, Fo in ((((2, 12, 12, 1), (3, 3, 1, 8), (1, 1), 'same', (1, 1)), 8),    # 3 x 3 'same': tiles off the windows
+                          (((2, 12, 12, 1), (3, 3, 1, 6), (1, 1), 'valid', (1, 1)), 6),   # filters not a multiple of 4
+                          (((2, 12, 12, 16), (3, 3, 16, 8), (1, 1), 'valid', (1, 1)), 8),  # many input channels
+                          (((2, 12, 12, 1), (3, 3, 1, 8), (2, 2), 'valid', (1, 1)), 8)):   # strided
+        geom = ops.conv_geometry(*geom_args)
+        assert not ops.conv2d_maxpool_supported(geom, Fo)
+    x = torch.randn(2, 12, 12, 1, device=dev)
+    w = torch.randn(3, 3, 1, 8, device=dev)
+    with pytest.raises(ValueError):
+        ops.conv2d(x, w, None, (1, 1), 'same', (1, 1), 0, maxpool2=True)
+
+
+def test_sequential_takes_the_pooling_into_the_convolution(dev):
+    """A QConv2D followed by MaxPooling2D((2, 2)) inside a Sequential runs as one node; outputs, losses and every gradient
+    equal those of the layers called one by one."""
+    import copy
+
+    from hgq2_amd import host, ops
+    from hgq2_amd.utils import models
+
+    model = models.conv_stack(filters=8, device=dev)
+    x = torch.rand(4, 28, 28, 1, generator=torch.Generator().manual_seed(3)).to(dev)
+    labels = torch.tensor([1, 0, 7, 3], device=dev)
+    twin = models.conv_stack(filters=8, device=dev)
+    model(x, training=False), twin(x, training=False)  # build
+    twin.load_state_dict(copy.deepcopy(model.state_dict()))
+    assert type(model.layers[1]) is host.MaxPooling2D and model.layers[0].absorbs(model.layers[1], x)
+
+    def by_hand(m, inp):
+        for layer in m.layers:
+            inp = layer(inp, training=True)
+        return inp
+
+    out_a = model(x, training=True)
+    out_b = by_hand(twin, x)
+    assert torch.equal(out_a, out_b)
+    ops.sparse_ce(out_a, labels).backward()
+    ops.sparse_ce(out_b, labels).backward()
+    for (name, pa), (_, pb) in zip(model.named_parameters(), twin.named_parameters()):
+        if pa.grad is not None or pb.grad is not None:
+            assert torch.equal(pa.grad, pb.grad), name
