@@ -129,6 +129,7 @@ SIGNATURES = {
     'hgq_conv2d_bwd_slice_count': (c_int64, [c_void_p, c_int]),
     'hgq_conv2d_bwd_slices': (c_int, [c_void_p] * 7 + [c_int, c_int, c_void_p]),
     'hgq_conv2d_maxpool_bwd_supported': (c_int, [c_void_p, c_int]),
+    'hgq_conv2d_maxpool_fwd': (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p]),
     'hgq_conv2d_maxpool_bwd': (c_int, [c_void_p] * 9 + [c_int, c_int, c_int, c_void_p]),
 }
 

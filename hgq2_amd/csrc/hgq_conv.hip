@@ -498,7 +498,7 @@ __global__ __launch_bounds__(256) void dgrad_patch_kernel(const float *__restric
 template <int KH, int KW, int C>
 __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                          const float *__restrict__ bias, float *__restrict__ out, hgq_conv_geom g,
-                                                         int F, int act, int tiles_x, int tiles_y) {
+                                                         int F, int act, int tiles_x, int tiles_y, float *__restrict__ pooled) {
 #pragma clang fp contract(fast)  // multiply-adds of the convolution sum may fuse (see bwd_smallc_kernel)
     constexpr int KC = KH * KW * C;
     extern __shared__ float lds[];  // input patch [XH][XW][C]
@@ -527,6 +527,12 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
         if (oy < g.OH) {
             const int n_x = min(SC_TW, g.OW - ox0);
             float *orow = out + (((int64_t)b * g.OH + oy) * g.OW + ox0) * F + f;
+            // `pooled`: also the 2 x 2 / stride 2 maxima, [B, OH / 2, OW / 2, F].  Tiles start on even rows and columns; a
+            // window's two rows are the two halves of one wavefront (slots 2 w and 2 w + 1), its columns two trips of the loop
+            const int PHo = g.OH >> 1, PWo = g.OW >> 1;
+            float *prow = pooled ? pooled + (((int64_t)b * PHo + (oy >> 1)) * PWo + (ox0 >> 1)) * F + f : nullptr;
+            const bool p_row = pooled && (oy >> 1) < PHo;  // both rows of the window exist: both halves are in this loop
+            float left = 0.f;
             for (int tx = 0; tx < n_x; ++tx) {
                 const float *xp = lds + (slot * g.sy * XW + tx * g.sx) * C;
                 float acc = bb;
@@ -537,6 +543,15 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
                 }
                 if (act == HGQ_ACT_RELU) acc = acc > 0.f ? acc : 0.f;
                 if (f_on) orow[(int64_t)tx * F] = acc;
+                if (p_row) {
+                    if (tx & 1) {
+                        float m = fmaxf(left, acc);
+                        m = fmaxf(m, __shfl_xor(m, 32));
+                        if (!(slot & 1) && f_on && ((ox0 + tx) >> 1) < PWo) prow[(int64_t)(tx >> 1) * F] = m;
+                    } else {
+                        left = acc;
+                    }
+                }
             }
         }
     }
@@ -1350,7 +1365,7 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
         const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
         const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
         const size_t lds = fwd_smallc_lds(*g);
-#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y)
+#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, (float *)nullptr)
         HGQ_SMALLC_DISPATCH(HGQ_FWD_SC);
 #undef HGQ_FWD_SC
         return check_launch("hgq_conv2d_fwd(few channels)");
@@ -1521,6 +1536,24 @@ extern "C" int hgq_conv2d_bwd_slices(const float *dy, const float *y, const floa
     }
     // the kernels only test the gradient pointers for "is it wanted": any non-null value stands for it
     return conv2d_bwd_impl(dy, y, xq, qw, dxq, workspace, workspace, workspace, g, F, act, stream, false);
+}
+
+extern "C" int hgq_conv2d_maxpool_fwd(const float *xq, const float *qw, const float *qb, float *y, float *yp, const hgq_conv_geom *g,
+                                      int F, int act, void *stream) {
+    int rc = check_geom(g, F, "hgq_conv2d_maxpool_fwd");
+    if (rc) return rc;
+    if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_fwd: unknown activation %d", act);
+    if (!hgq_conv2d_maxpool_bwd_supported(g, F) || !fwd_smallc_ok(*g, F))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_maxpool_fwd: shape not supported (ask hgq_conv2d_maxpool_bwd_supported)");
+    if (!xq || !qw || !y || !yp) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_fwd: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
+    const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
+    const size_t lds = fwd_smallc_lds(*g);
+#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, yp)
+    HGQ_SMALLC_DISPATCH(HGQ_FWD_SC);
+#undef HGQ_FWD_SC
+    return check_launch("hgq_conv2d_maxpool_fwd");
 }
 
 extern "C" int hgq_conv2d_maxpool_bwd(const float *dyp, const float *y, const float *xq, const float *qw, float *dxq, float *dqw,

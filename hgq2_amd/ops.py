@@ -1043,6 +1043,28 @@ def _(dy, y, xq, qw, geom, act, need_dx):
     return xq.new_empty(xq.shape if need_dx else (0,)), xq.new_empty((1, qw.numel() + qw.shape[-1]))
 
 
+@torch.library.custom_op('hgq::conv2d_maxpool_fwd', mutates_args=())
+def conv2d_maxpool_fwd(xq: Tensor, qw: Tensor, qb: Tensor, geom: Sequence[int], act: int) -> tuple[Tensor, Tensor]:
+    """``(y, maxpool2x2(y))`` with ``y = act(conv2d(xq, qw) + qb)`` in one launch (``qb`` empty: no bias)."""
+    _check_f32('xq', xq), _check_f32('qw', qw), _check_f32('qb', qb)
+    g = _geom(geom)
+    F = qw.shape[-1]
+    _need(xq.numel() == g.B * g.H * g.W * g.C and tuple(qw.shape) == (g.kh, g.kw, g.C, F), 'xq / qw do not match the geometry')
+    _need(qb.numel() in (0, F), 'qb must hold one entry per filter')
+    y = torch.empty((g.B, g.OH, g.OW, F), dtype=torch.float32, device=xq.device)
+    yp = torch.empty((g.B, g.OH // 2, g.OW // 2, F), dtype=torch.float32, device=xq.device)
+    rc = _lib.load().hgq_conv2d_maxpool_fwd(_ptr(xq), _ptr(qw), _ptr(qb) if qb.numel() else None, _ptr(y), _ptr(yp), ctypes.addressof(g),
+                                            F, act, _stream())
+    _lib.check(rc, 'hgq_conv2d_maxpool_fwd')
+    return y, yp
+
+
+@conv2d_maxpool_fwd.register_fake
+def _(xq, qw, qb, geom, act):
+    F = qw.shape[-1]
+    return xq.new_empty((geom[0], geom[12], geom[13], F)), xq.new_empty((geom[0], geom[12] // 2, geom[13] // 2, F))
+
+
 @torch.library.custom_op('hgq::conv2d_maxpool_bwd', mutates_args=())
 def conv2d_maxpool_bwd(dyp: Tensor, y: Tensor, xq: Tensor, qw: Tensor, geom: Sequence[int], act: int, need_dx: bool,
                        reduce: bool) -> tuple[Tensor, Tensor]:
@@ -2106,9 +2128,7 @@ class _Conv2DMaxPool(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, xq, qw, qb, geom, act):
-        y = conv2d_fwd(xq, qw, qb, list(geom), act)
-        B, OH, OW, F = geom[0], geom[12], geom[13], qw.shape[-1]
-        yp = pool2d_fwd(y, [B, OH, OW, F, 2, 2, 2, 2, 0, 0, OH // 2, OW // 2], True)
+        y, yp = conv2d_maxpool_fwd(xq, qw, qb, list(geom), act)
         ctx.save_for_backward(xq, qw, y)
         ctx.geom, ctx.act, ctx.has_bias = tuple(geom), act, qb.numel() > 0
         ctx.defer = getattr(qw, '_hgq_single_use', False) and (qb.numel() == 0 or getattr(qb, '_hgq_single_use', False))

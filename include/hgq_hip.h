@@ -597,8 +597,12 @@ int hgq_conv2d_bwd_slices(const float *dy, const float *y, const float *xq, cons
  * summed into dqw / dqb.  hgq_conv2d_maxpool_bwd_supported: 1 where the few-input-channel kernel takes the shape with F a
  * multiple of 4 (kernels of odd size; 'valid', or a 'same' padding that keeps the tiles on window boundaries);
  * HGQ_ERR_UNSUPPORTED otherwise, and for dyp / y not aligned to 16 bytes.
+ * hgq_conv2d_maxpool_fwd (same shapes): hgq_conv2d_fwd that also writes the pooled output yp [B, OH / 2, OW / 2, F] from
+ * the values it has in registers (hgq_pool2d_fwd's result without its pass over y).
  */
 int hgq_conv2d_maxpool_bwd_supported(const hgq_conv_geom *g, int F);
+int hgq_conv2d_maxpool_fwd(const float *xq, const float *qw, const float *qb, float *y, float *yp, const hgq_conv_geom *g, int F,
+                           int act, void *stream);
 int hgq_conv2d_maxpool_bwd(const float *dyp, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
                            float *workspace, const hgq_conv_geom *g, int F, int act, int reduce, void *stream);
 
