@@ -594,6 +594,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
     float wacc[KC], bacc = 0.f;
 #pragma unroll
     for (int t = 0; t < KC; ++t) wacc[t] = 0.f;
+    const bool two_step = KC <= F;  // the KC sums of a pixel fit into its dz row
     const int64_t n_tiles = (int64_t)g.B * tiles_y * tiles_x;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int b = (int)(tile / (tiles_y * tiles_x)), rem = (int)(tile - (int64_t)b * tiles_y * tiles_x);
@@ -707,7 +708,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
             }
         }
         __syncthreads();
-        if (dx) {
+        if (dx && !two_step) {
             const int tx = tid % SC_TW, ty = tid / SC_TW;
             const int iy = iy0 + ty, ix = ix0 + tx;
             if (iy < g.H && ix < g.W) {
@@ -754,17 +755,82 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                 const int oy = oy0 + pr;
                 if ((unsigned)oy >= (unsigned)g.OH || !(pr >= KH - 1 || iy0 == 0)) continue;
                 const int pc_lo = ix0 == 0 ? max(0, -ox0) : KW - 1, pc_hi = min(PW, g.OW - ox0);
-                for (int pc = pc_lo; pc < pc_hi; ++pc) {
+                // input pixel of tap (ky, kx): patch-relative (pr + ky - (KH - 1) + py, pc + kx - (KW - 1) + px).  The KH x KW
+                // window of a pixel shares all but one column with its left neighbour's: it lives in registers and takes KH * C
+                // new entries per pixel (LDS broadcasts) instead of KC
+                const float *xq = xp + ((pr - (KH - 1) + g.py) * XW + (pc_lo - (KW - 1) + g.px)) * C;
+                float xw[KH][KW * C];
+#pragma unroll
+                for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+                    for (int j = 0; j < (KW - 1) * C; ++j) xw[ky][j + C] = xq[ky * XW * C + j];
+                for (int pc = pc_lo; pc < pc_hi; ++pc, xq += C) {
                     const float z = f_on ? zp[(pr * PW + pc) * FS + f] : 0.f;
                     bacc += z;
-                    // input pixel of tap (ky, kx): patch-relative (pr + ky - (KH - 1) + py, pc + kx - (KW - 1) + px)
-                    const float *xq = xp + ((pr - (KH - 1) + g.py) * XW + (pc - (KW - 1) + g.px)) * C;
+#pragma unroll
+                    for (int ky = 0; ky < KH; ++ky) {
+#pragma unroll
+                        for (int j = 0; j < (KW - 1) * C; ++j) xw[ky][j] = xw[ky][j + C];
+#pragma unroll
+                        for (int c = 0; c < C; ++c) xw[ky][(KW - 1) * C + c] = xq[(ky * XW + KW - 1) * C + c];
+                    }
+#pragma unroll
+                    for (int t = 0; t < KC; ++t) wacc[t] += xw[t / (KW * C)][t % (KW * C)] * z;
+                }
+            }
+        }
+        if (dx && two_step) {
+            // data gradient in two steps, after the weight gradient has read dz: (1) thread = OUTPUT pixel of the patch
+            // contracts its F entries of dz with the kernel - KC sums u[tap] - and writes them over the start of its own dz
+            // row (nobody else touches that row); (2) thread = input pixel adds the KH * KW * C sums that meet in it.  One LDS
+            // read of dz feeds KC multiply-adds instead of one.
+            __syncthreads();
+            for (int p = tid; p < PH * PW; p += 256) {
+                float *row = zp + p * FS;
+                float u[KC];
+#pragma unroll
+                for (int t = 0; t < KC; ++t) u[t] = 0.f;
+                int ff = 0;
+                for (; ff + 8 <= F; ff += 8) {
+                    float v[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = row[ff + j];
 #pragma unroll
                     for (int t = 0; t < KC; ++t) {
-                        const int ky = t / (KW * C), kx = (t / C) % KW, c = t % C;
-                        wacc[t] += xq[(ky * XW + kx) * C + c] * z;
+                        float wv[8];  // the same address in every lane: scalar loads
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) wv[j] = w[t * F + ff + j];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) u[t] += v[j] * wv[j];
                     }
                 }
+                for (; ff < F; ++ff) {
+                    const float v = row[ff];
+#pragma unroll
+                    for (int t = 0; t < KC; ++t) u[t] += v * w[t * F + ff];
+                }
+#pragma unroll
+                for (int t = 0; t < KC; ++t) row[t] = u[t];
+            }
+            __syncthreads();
+            const int tx = tid % SC_TW, ty = tid / SC_TW;
+            const int iy = iy0 + ty, ix = ix0 + tx;
+            if (iy < g.H && ix < g.W) {
+                float acc[C];
+#pragma unroll
+                for (int c = 0; c < C; ++c) acc[c] = 0.f;
+#pragma unroll
+                for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+                    for (int kx = 0; kx < KW; ++kx) {
+                        // oy = iy + py - ky  ->  patch row ty + (KH - 1) - ky
+                        const float *up = zp + ((ty + KH - 1 - ky) * PW + (tx + KW - 1 - kx)) * FS + (ky * KW + kx) * C;
+#pragma unroll
+                        for (int c = 0; c < C; ++c) acc[c] += up[c];
+                    }
+                const int64_t o = (((int64_t)b * g.H + iy) * g.W + ix) * C;
+#pragma unroll
+                for (int c = 0; c < C; ++c) dx[o + c] = acc[c];
             }
         }
     }
