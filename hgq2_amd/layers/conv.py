@@ -109,6 +109,8 @@ class QConv2D(QLayerBaseSingleInput):
 
         if type(nxt) is not MaxPooling2D or nxt.pool_size != (2, 2) or nxt.strides != (2, 2) or nxt.padding != 'valid':
             return False
+        if type(self).call is not QConv2D.call or type(self).convolution_op is not QConv2D.convolution_op:
+            return False  # a subclass with its own call: it does not know the `then` argument
         if self.enable_oq or self._act_name not in (None, 'linear', 'relu') or not torch.is_tensor(x) or not x.is_cuda or x.dim() != 4:
             return False
         geom = ops.conv_geometry(tuple(x.shape), self.kernel_size + (x.shape[-1], self.filters), self.strides, self.padding, self.dilation_rate)
