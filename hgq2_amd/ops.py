@@ -451,8 +451,7 @@ class overlap_ebops:
     """Context manager around a training step (forward, loss, backward, update): EBOPs launches inside it run on a
     second stream.  Whoever opens it must leave it before the captured graph ends or before results are read from
     another thread or stream; leaving it joins the second stream.  ``hgq2_amd.train.model_loss`` called inside it
-    returns a total without an autograd graph whose value is there once the context is left (the terms carry the
-    graph: ``SGD.backward`` starts from them)."""
+    returns a total whose value is there once the context is left (its gradient does not need the value)."""
 
     def __enter__(self):
         _OVERLAP['depth'] += 1

@@ -15,6 +15,20 @@ from .core import Layer, tree_cache
 from .regularizers import MonoL1
 
 
+class _SumLater(torch.autograd.Function):
+    """The sum of one-element terms whose VALUE is written later (by the launch that joins the streams, or by the update);
+    its gradient - the upstream gradient to every term - needs no value, so ``loss.backward()`` works on the result."""
+
+    @staticmethod
+    def forward(ctx, shape, *terms):
+        ctx.shapes = [t.shape for t in terms]
+        return terms[0].new_empty(shape)
+
+    @staticmethod
+    def backward(ctx, g):
+        return (None,) + tuple(g.reshape(s) if ctx.needs_input_grad[1 + t] else None for t, s in enumerate(ctx.shapes))
+
+
 def model_loss(model, base_loss, fold_regularizers: bool = False):
     """``base_loss + sum(add_loss terms) (+ variable regularizers)``.  With ``fold_regularizers``
     the MonoL1 terms are left out of the autograd graph: their constant gradient ``l1`` is added by
@@ -36,9 +50,9 @@ def model_loss(model, base_loss, fold_regularizers: bool = False):
         # nothing but the caller's print-out reads it - is summed when the streams are joined for the last time, inside
         # the update's launch when :class:`SGD` makes it, and the backward pass starts from the terms themselves -
         # d total / d term = 1 - so the first stream does not wait for the second before the update
-        total = torch.empty(torch.broadcast_shapes(*[t.shape for t in terms]), dtype=torch.float32, device=terms[0].device)
+        total = _SumLater.apply(torch.broadcast_shapes(*[t.shape for t in terms]), *terms)
         held = list(terms)
-        ops._OVERLAP['finish'].append((held, total))
+        ops._OVERLAP['finish'].append((held, total.detach()))
         total._hgq_terms = [t for t in terms if t.requires_grad]
         return total
     ops.join_side()  # EBOPs terms issued on the second stream

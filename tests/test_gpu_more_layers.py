@@ -854,3 +854,43 @@ def test_global_average_pooling_layers_use_it_and_match_the_library_mean():
             want = x.mean(dim=tuple(range(1, len(shape) - 1)), keepdim=layer.keepdims)
             assert y.shape == want.shape
             assert torch.allclose(y.cpu(), want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize('kind', ['conv', 'particle'])
+def test_plain_backward_inside_the_overlap_context(dev, kind):
+    """``model_loss`` inside ``ops.overlap_ebops()`` returns a total whose value is written later; ``loss.backward()`` -
+    without the optimizer's gradient sink - still gives the gradients of the step outside the context, and the value is
+    there when the context is left."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, model_loss
+    from hgq2_amd.utils import models
+
+    g = torch.Generator().manual_seed(34)
+    if kind == 'conv':
+        make = lambda: models.conv_stack(filters=8, n_out=10, device=dev)  # noqa: E731
+        x, y = torch.rand(64, 12, 12, 1, generator=g).to(dev), torch.randint(0, 10, (64,), generator=g).to(dev)
+    else:
+        make = lambda: models.particle_mlp(n_particles=8, n_features=16, hidden=(32, 16), device=dev)  # noqa: E731
+        x, y = torch.randn(64, 8, 16, generator=g).to(dev), torch.randint(0, 5, (64,), generator=g).to(dev)
+    torch.manual_seed(4)
+    a = make()
+    a(x, training=True)
+    torch.manual_seed(4)
+    b = make()
+    b(x, training=True)
+    b.load_state_dict(a.state_dict())
+    oa, ob = SGD(a.parameters(), lr=0.02), SGD(b.parameters(), lr=0.02)
+    for step in range(2):
+        oa.zero_grad()
+        la = model_loss(a, ops.sparse_ce(a(x, training=True), y))
+        la.backward()
+        oa.step()
+        with ops.overlap_ebops():
+            ob.zero_grad()
+            lb = model_loss(b, ops.sparse_ce(b(x, training=True), y))
+            assert lb.requires_grad
+            lb.backward()
+            ob.step()
+        assert float(la) == float(lb), f'loss step {step}'
+        for (name, pa), (_, pb) in zip(a.state_dict().items(), b.state_dict().items()):
+            assert torch.equal(pa, pb), f'{name} step {step}'
