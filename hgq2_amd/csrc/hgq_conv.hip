@@ -1400,6 +1400,60 @@ static void launch_igemm(bool vec, bool wide, dim3 grid, hipStream_t s, const fl
 #undef HGQ_IGEMM
 }
 
+// A long contraction onto a handful of filters for few rows (the classifier behind a flattened feature map: 1024 x 3872
+// onto 10): an implicit-GEMM tile would be mostly padding and needs a split along k plus a finishing launch.  Here a
+// wavefront takes one row and a quarter of k - lanes along k, so the row is read in 256-byte pieces and a lane reads the
+// F kernel entries of its k - adds up across its lanes, and the four quarters meet in LDS in a fixed order.  (Measured on
+// 1024 x 3872 x 10: 14.8 us; two rows x eight parts of k per workgroup 17.1 us; the kernel matrix read as flat 256-byte
+// pieces with the row entries gathered to match 24.4 us; implicit GEMM with split + finishing launch 12.2 + 8.3 us.)
+#define SK_ROWS 4
+#define SK_SPLIT 4
+template <int F>
+__global__ __launch_bounds__(1024) void skinny_fwd_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                          const float *__restrict__ bias, float *__restrict__ y, int64_t rows, int K,
+                                                          int act) {
+#pragma clang fp contract(fast)  // a contraction sum: multiply-adds may fuse, as in the other contraction kernels
+    __shared__ float red[SK_ROWS][SK_SPLIT][F];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = wave / SK_SPLIT, sp = wave % SK_SPLIT;
+    const int64_t row = (int64_t)blockIdx.x * SK_ROWS + r;
+    const int kchunk = (K + SK_SPLIT * 64 - 1) / (SK_SPLIT * 64) * 64;
+    const int k_begin = sp * kchunk, k_end = min(K, k_begin + kchunk);
+    float acc[F];
+#pragma unroll
+    for (int n = 0; n < F; ++n) acc[n] = 0.f;
+    if (row < rows) {
+        const float *xr = x + row * K;
+#pragma unroll 4
+        for (int k = k_begin + lane; k < k_end; k += 64) {
+            const float xv = xr[k];
+            const float *wr = w + (int64_t)k * F;
+#pragma unroll
+            for (int n = 0; n < F; ++n) acc[n] += xv * wr[n];
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < F; ++n) {
+        float v = acc[n];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        if (lane == 0) red[r][sp][n] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < SK_ROWS * F) {
+        const int rr = threadIdx.x / F, n = threadIdx.x % F;
+        const int64_t orow = (int64_t)blockIdx.x * SK_ROWS + rr;
+        if (orow < rows) {
+            float v = red[rr][0][n];
+#pragma unroll
+            for (int q = 1; q < SK_SPLIT; ++q) v += red[rr][q][n];
+            if (bias) v += bias[n];
+            if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+            y[orow * F + n] = v;
+        }
+    }
+}
+
 }  // namespace hgq
 
 using namespace hgq;
@@ -1427,6 +1481,18 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
     kchunk = (kchunk + CV_BK - 1) / CV_BK * CV_BK;
     const int nz = (K + kchunk - 1) / kchunk;
     float *dst = nz > 1 ? workspace : y;
+    if (g->kh == 1 && g->kw == 1 && g->sy == 1 && g->sx == 1 && g->py == 0 && g->px == 0 && g->OH == g->H && g->OW == g->W && F <= 16 &&
+        K >= 1024 && rows <= 16384) {
+        const dim3 grid((unsigned)((rows + SK_ROWS - 1) / SK_ROWS));
+#define HGQ_SKINNY(FV) \
+    case FV: hipLaunchKernelGGL((skinny_fwd_kernel<FV>), grid, dim3(1024), 0, s, xq, qw, qb, y, rows, K, act); break
+        switch (F) {
+            HGQ_SKINNY(1); HGQ_SKINNY(2); HGQ_SKINNY(3); HGQ_SKINNY(4); HGQ_SKINNY(5); HGQ_SKINNY(6); HGQ_SKINNY(7); HGQ_SKINNY(8);
+            HGQ_SKINNY(9); HGQ_SKINNY(10); HGQ_SKINNY(11); HGQ_SKINNY(12); HGQ_SKINNY(13); HGQ_SKINNY(14); HGQ_SKINNY(15); HGQ_SKINNY(16);
+        }
+#undef HGQ_SKINNY
+        return check_launch("hgq_conv2d_fwd(few filters, long contraction)");
+    }
     if (fwd_smallc_ok(*g, F)) {
         const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
         const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));

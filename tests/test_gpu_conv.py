@@ -340,3 +340,26 @@ def test_sequential_takes_the_pooling_into_the_convolution(dev):
     for (name, pa), (_, pb) in zip(model.named_parameters(), twin.named_parameters()):
         if pa.grad is not None or pb.grad is not None:
             assert torch.equal(pa.grad, pb.grad), name
+
+
+@pytest.mark.parametrize('rows,K,N,relu,bias', [(1024, 3872, 10, False, True), (7, 1500, 16, True, True), (33, 1024, 1, False, False),
+                                               (5, 2049, 3, True, False), (4097, 1100, 5, False, True)])
+def test_few_filters_behind_a_long_contraction(dev, rows, K, N, relu, bias):
+    """A classifier behind a flattened feature map (few rows, K in the thousands, a handful of outputs) has a kernel of
+    its own in `hgq_conv2d_fwd`; values against fp64 within 1e-5 of the sum of the terms' magnitudes, the same bits on
+    every run."""
+    from hgq2_amd import _lib, ops
+
+    g = torch.Generator().manual_seed(rows + K + N)
+    x = torch.randn(rows, K, generator=g)
+    w = torch.randn(K, N, generator=g) * 0.1
+    b = torch.randn(N, generator=g) if bias else None
+    act = _lib.ACT_RELU if relu else _lib.ACT_NONE
+    runs = [ops.matmul_bias_act(x.to(dev), w.to(dev), b.to(dev) if bias else None, act) for _ in range(2)]
+    assert torch.equal(runs[0], runs[1])
+    want = x.double() @ w.double() + (b.double() if bias else 0.0)
+    scale = x.double().abs() @ w.double().abs() + (b.double().abs() if bias else 0.0)
+    if relu:
+        want = torch.relu(want)
+    err = ((runs[0].cpu().double() - want).abs() / scale).max()
+    assert float(err) <= 1e-5, float(err)
