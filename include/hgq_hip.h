@@ -555,6 +555,8 @@ int hgq_qsoftmax_bwd(const float *dy, const float *x, float *dx, int64_t rows, i
  *   positions outside the input contribute zero ('same' padding: py, px = the top / left pad);
  *   workspace: hgq_conv2d_fwd_workspace(g, F) floats (0 for most shapes; a long contraction with few
  *   output tiles is split along k and the slices are added by a second kernel), may be NULL if 0.
+ *   A 1 x 1 geometry with at most 16384 rows, a contraction of 1024 or more and at most 16 filters (a classifier behind a
+ *   flattened feature map) runs in one launch that does not touch the workspace.
  */
 typedef struct {
     int B, H, W, C;   /* input: batch, height, width, channels */
