@@ -25,7 +25,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of the 4 Mi-element quantizer kernels from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # counters, each scaled by what the same counter reads for the plain streaming kernel of known size
 # (hgq_stream_probe); summary and commands in profiles/quantizer_4Mi_hbm_counters.md
-TRAFFIC_BYTES = {'quant_fwd': 50.34e6, 'quant_bwd': 100.67e6, 'quant_fwd_sat': 83.89e6, 'quant_bwd_sat': 134.22e6}
+TRAFFIC_BYTES = {'quant_fwd': 50.34e6, 'quant_bwd': 100.67e6, 'quant_fwd_sat': 83.89e6, 'quant_bwd_sat': 134.22e6,
+                 'quant_fwd_bwd': 117.44e6, 'quant_fwd_bwd_sat': 150.99e6}
 BATCH = 16384
 DIMS = (16, 64, 32, 32, 5)
 QN = 4 * 1024 * 1024  # standalone quantizer case: 4 Mi fp32 elements
@@ -101,20 +102,26 @@ def quantizer_roofline(iters=200):
         mode = _lib.mode_bits('RND', om, training=True)
         fwd_calls = [(p(x), p(k), p(i), p(f), p(y), None, None, QN, QN, 1, mode, s) for x, k, i, f, dy, y, dx, di, df in sets]
         bwd_calls = [(p(dy), p(x), p(k), p(i), p(f), p(dx), p(di), p(df), QN, QN, 1, mode, s) for x, k, i, f, dy, y, dx, di, df in sets]
+        both_calls = [(p(x), p(k), p(i), p(f), p(dy), p(y), p(dx), p(di), p(df), QN, QN, 1, mode, s) for x, k, i, f, dy, y, dx, di, df in sets]
         t_fwd = timed(lib.hgq_quantize_fwd, fwd_calls)
         t_bwd = timed(lib.hgq_quantize_bwd, bwd_calls)
+        t_both = timed(lib.hgq_quantize_fwd_bwd, both_calls)
         suffix = '' if om == 'WRAP' else '_sat'
-        for name, ms, bpe in (('quant_fwd' + suffix, t_fwd, 20), ('quant_bwd' + suffix, t_bwd, 32)):
+        # operand bytes per element: forward x, k, i, f in, y out; backward dy, x, k, i, f in, dx, di, df out; both in one
+        # launch x, k, i, f, dy in, y, dx, di, df out
+        for name, ms, bpe in (('quant_fwd' + suffix, t_fwd, 20), ('quant_bwd' + suffix, t_bwd, 32), ('quant_fwd_bwd' + suffix, t_both, 36)):
             traffic = TRAFFIC_BYTES[name]
             out[name] = {'ms': ms, 'operand_bytes': bpe * QN, 'operand_GBps': bpe * QN / (ms * 1e-3) / 1e9,
                          'traffic': traffic, 'GBps': traffic / (ms * 1e-3) / 1e9, 'frac': traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                          'frac_operands': bpe * QN / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    # plain streaming kernels: 2 arrays read + 1 written (the bytes of the WRAP forward), 3 + 3 (the WRAP backward)
-    for name, nr, nw in (('stream_2r1w', 2, 1), ('stream_3r3w', 3, 3), ('stream_1r1w', 1, 1)):
-        calls = [(p(x), p(f), p(dy), p(y), p(dx), p(df), nr, nw, QN, s) for x, k, i, f, dy, y, dx, di, df in sets]
+        out['quant_fwd_bwd' + suffix]['two_launches_ms'] = t_fwd + t_bwd
+    # plain streaming kernels: 2 arrays read + 1 written (the bytes of the WRAP forward), 3 + 3 (the WRAP backward), 3 + 4 (both in one)
+    for name, nr, nw in (('stream_2r1w', 2, 1), ('stream_3r3w', 3, 3), ('stream_3r4w', 3, 4), ('stream_1r1w', 1, 1)):
+        calls = [(p(x), p(f), p(dy), p(y), p(dx), p(df), p(di), nr, nw, QN, s) for x, k, i, f, dy, y, dx, di, df in sets]
         ms = timed(lib.hgq_stream_probe, calls)
         nbytes = 4 * (nr + nw) * QN
         out[name] = {'ms': ms, 'traffic': nbytes, 'GBps': nbytes / (ms * 1e-3) / 1e9, 'frac': nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    out['quant_fwd_bwd']['of_plain_stream'] = out['stream_3r4w']['ms'] / out['quant_fwd_bwd']['ms']
     out['quant_fwd']['of_plain_stream'] = out['stream_2r1w']['ms'] / out['quant_fwd']['ms']
     out['quant_bwd']['of_plain_stream'] = out['stream_3r3w']['ms'] / out['quant_bwd']['ms']
     return out
@@ -531,21 +538,23 @@ def main():
         out['paths'] = paths
 
     qr = quantizer_roofline()
-    dom = qr['quant_bwd']
+    dom = qr['quant_fwd_bwd']
     out['roofline'] = {
-        'bound': 'hbm', 'kernel': 'quant_bwd_pe<RND, WRAP>', 'achieved': dom['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+        'bound': 'hbm', 'kernel': 'quant_fwd_bwd_pe<RND, WRAP>', 'achieved': dom['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
         'frac': dom['frac'], 'traffic': dom['traffic'], 'frac_operands': dom['frac_operands'],
-        'of_plain_stream': dom['of_plain_stream'],
-        'workload': 'standalone kif quantizer RND/WRAP, 4 Mi fp32 elements, per-element k/i/f: backward.  achieved = HBM bytes '
-                    'per launch by the traffic counters (24 B/elem: dy, x, f in; dx, di, df out - the WRAP training branch '
-                    'reads neither k nor i) / HIP-event time; frac_operands prices the same time at all 32 B/elem of operands; '
-                    'of_plain_stream = time of a plain 3-read 3-write streaming kernel of the same bytes / this kernel\'s time'}
-    sat = qr['quant_bwd_sat']
+        'of_plain_stream': dom['of_plain_stream'], 'two_launches_ms': dom['two_launches_ms'], 'ms': dom['ms'],
+        'workload': 'standalone kif quantizer RND/WRAP, 4 Mi fp32 elements, per-element k/i/f: training forward + surrogate backward '
+                    'in ONE launch (hgq_quantize_fwd_bwd).  achieved = HBM bytes per launch by the traffic counters (28 B/elem: x, f, '
+                    'dy in; y, dx, di, df out - the WRAP training branch reads neither k nor i) / HIP-event time; frac_operands '
+                    'prices the same time at all 36 B/elem of operands; of_plain_stream = time of a plain 3-read 4-write streaming '
+                    'kernel of the same bytes / this kernel\'s time; two_launches_ms = hgq_quantize_fwd + hgq_quantize_bwd '
+                    '(quantizer_kernels.quant_fwd / quant_bwd: the separate kernels priced the same way)'}
+    sat = qr['quant_fwd_bwd_sat']
     out['roofline_all_operands_live'] = {
-        'bound': 'hbm', 'kernel': 'quant_bwd_pe<RND, SAT>', 'achieved': sat['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-        'frac': sat['frac'], 'traffic': sat['traffic'],
-        'workload': 'the same quantizer with overflow mode SAT: every operand is live, 32 B/elem cross HBM (forward: 20 B/elem, '
-                    'see quantizer_kernels.quant_fwd_sat)'}
+        'bound': 'hbm', 'kernel': 'quant_fwd_bwd_pe<RND, SAT>', 'achieved': sat['GBps'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+        'frac': sat['frac'], 'traffic': sat['traffic'], 'two_launches_ms': sat['two_launches_ms'], 'ms': sat['ms'],
+        'workload': 'the same quantizer with overflow mode SAT: every operand is live, 36 B/elem cross HBM in the one-launch form '
+                    '(separate launches: forward 20 B/elem, backward 32 B/elem, see quantizer_kernels.quant_fwd_sat / quant_bwd_sat)'}
     out['quantizer_kernels'] = qr
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline()

@@ -90,8 +90,9 @@ SIGNATURES = {
     'hgq_wrap_track_i_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_qdense_bwd_slices': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 3 + [c_int, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     'hgq_reduce_slices_multi': (c_int, [c_void_p, c_int, c_void_p]),
-    'hgq_stream_probe': (c_int, [c_void_p] * 6 + [c_int, c_int, c_int64, c_void_p]),
+    'hgq_stream_probe': (c_int, [c_void_p] * 7 + [c_int, c_int, c_int64, c_void_p]),
     'hgq_quantize_bwd_static': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    'hgq_quantize_fwd_bwd': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_fwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_quantize_bwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_mean_mid_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),

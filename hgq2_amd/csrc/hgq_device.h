@@ -123,6 +123,35 @@ __device__ __forceinline__ void quantize_grad(float x, float dy, const KIF &p, f
     }
 }
 
+// Training-mode forward and surrogate backward of one element from one rounding: y is what quantize<RM, OM>(x, p, true)
+// returns and dx / di / df what quantize_grad<RM, OM> returns, bit for bit (same operations in the same order).
+template <int RM, int OM>
+__device__ __forceinline__ float quantize_with_grad(float x, float dy, const KIF &p, float &dx, float &di, float &df) {
+    const float xq = fixed_round<RM>(x, p.f);
+    int st = 0;
+    float y = xq;
+    if (OM != HGQ_WRAP) y = overflow<OM>(xq, p, true, st);
+    if (st == 0) {
+        dx = dy;
+        di = 0.0f;
+        df = -HGQ_LN2 * (xq - x) * dy;
+    } else {
+        dx = 0.0f;
+        const float gi = HGQ_LN2 * pow2(p.i) * dy;
+        const float gf = HGQ_LN2 * pow2(-p.f) * dy;
+        di = 0.0f, df = 0.0f;
+        if (st & 1) {
+            di += gi;
+            df += gf;
+        }
+        if (st & 2) {
+            di += -p.k * gi;
+            if (OM == HGQ_SAT_SYM) df += -p.k * gf;
+        }
+    }
+    return y;
+}
+
 // Bit pattern of |v| as an unsigned integer: monotone for non-negative floats, so an integer
 // atomic max is a float max.  NaN payloads compare above every finite value and propagate.
 __device__ __forceinline__ uint32_t abs_bits(float v) { return __float_as_uint(v) & 0x7fffffffu; }

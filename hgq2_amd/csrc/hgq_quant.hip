@@ -208,14 +208,17 @@ __global__ __launch_bounds__(Q1D_BS) void quant_bwd_1d(const float *__restrict__
 }
 
 // ------------------------------------------------------------------------------------------
-// Per-element bit-widths, fp32 k, no trackers: the standalone-quantizer case.  One 128-bit vector per operand
-// per thread and nothing else: the training flag and the set of live operands are template arguments, the
-// raw variables are always rounded (the identity on integer-valued ones), KIF / KBI is a select - no branch
-// sits between the loads.  With one vector per thread the waves of a launch run in step (all load, all
-// compute, all store), so every vector instruction saved here is time saved: at 4 Mi elements the kernel runs
-// two such rounds and ~100 instructions cost about a microsecond of a ten-microsecond launch.
-// LIVE bit 0: `i` is read; bit 1: `k` is read.  A WRAP quantizer in training mode only rounds, so k is dead
-// there, and i as well unless f = b - i.
+// Per-element bit-widths, fp32 k, no trackers: the standalone-quantizer case.  Nothing but the streams: the training
+// flag and the set of live operands are template arguments, the raw variables are always rounded (the identity on
+// integer-valued ones), KIF / KBI is a select - no branch sits between the loads.  LIVE bit 0: `i` is read; bit 1: `k`
+// is read.  A WRAP quantizer in training mode only rounds, so k is dead there, and i as well unless f = b - i.
+//
+// U = vectors (128 bits) per lane and array.  U = 1: thread t of the launch takes vector v_begin + t (checked against
+// v_end): the form for small inputs and for the remainder behind whole tiles.  U = 2: a wavefront owns 2 KB of every
+// array (lane l takes vectors l and l + 64 of the wavefront's tile) and requests them one after the other (see
+// HGQ_PE_WAIT below); the launch covers whole tiles only, so no load sits behind a bounds check.  At 4 Mi elements U = 2 puts the whole problem on the device in ONE round of workgroups (1024 workgroups of
+// 512 threads = what 256 CUs hold) instead of two rounds that run in step - all load, all store, all retire, all
+// start again - and pay the store-acknowledge + launch + first-load latency once more in the middle.
 // ------------------------------------------------------------------------------------------
 template <int LIVE>
 __device__ __forceinline__ KIF pe_kif(const f32x4 &kv, const f32x4 &iv, const f32x4 &fv, int c, bool kbi) {
@@ -227,47 +230,112 @@ __device__ __forceinline__ KIF pe_kif(const f32x4 &kv, const f32x4 &iv, const f3
     return p;
 }
 
-template <int RM, int OM, bool TRAIN, int LIVE>
-__global__ __launch_bounds__(Q1D_BS) void quant_fwd_pe(const f32x4 *__restrict__ x, const f32x4 *__restrict__ k,
-                                                       const f32x4 *__restrict__ i, const f32x4 *__restrict__ fb,
-                                                       f32x4 *__restrict__ y, int64_t nvec, int kbi) {
-    const int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x;
-    if (v >= nvec) return;
-    const f32x4 xv = __builtin_nontemporal_load(x + v);
-    const f32x4 fv = __builtin_nontemporal_load(fb + v);
-    f32x4 iv = {0.f, 0.f, 0.f, 0.f}, kv = {0.f, 0.f, 0.f, 0.f};
-    if (LIVE & 1) iv = __builtin_nontemporal_load(i + v);
-    if (LIVE & 2) kv = __builtin_nontemporal_load(k + v);
-    f32x4 yv;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) yv[c] = quantize<RM, OM>(xv[c], pe_kif<LIVE>(kv, iv, fv, c, kbi != 0), TRAIN);
-    __builtin_nontemporal_store(yv, y + v);
+template <int U>
+__device__ __forceinline__ int64_t pe_first_vector(int64_t v_begin) {
+    if (U == 1) return v_begin + (int64_t)blockIdx.x * Q1D_BS + threadIdx.x;
+    return v_begin + ((int64_t)blockIdx.x * (Q1D_BS / 64) + (threadIdx.x >> 6)) * (64 * U) + (threadIdx.x & 63);
 }
 
-template <int RM, int OM, int LIVE>
+// In the two-vector form every load is waited for before the next one is issued, and every array's pair of stores before
+// the next array's: ONE request in flight per wavefront.  The 32 wavefronts of a CU still keep 8 MB in flight across
+// the device, which covers the memory latency; more only queues up in front of the memory channels, and the queues cost
+// bandwidth - measured on the 3-read 4-write stream at 4 Mi elements: all six loads in flight 22.3 us, pairs 21.3 us,
+// one at a time 19.2 us, and 18.8 us with the store pairs waited for as well.  The waits also keep the device in step:
+// all wavefronts read the same array at the same time, then the next one, then all write.
+#define HGQ_PE_WAIT() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+#define HGQ_PE_LOAD(dst, src)                                                 \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                           \
+        dst[u] = __builtin_nontemporal_load(src + v0 + 64 * u);               \
+        if (U > 1) HGQ_PE_WAIT();                                             \
+    }
+#define HGQ_PE_STORE(src, dst)                                                \
+    do {                                                                      \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) __builtin_nontemporal_store(src[u], dst + v0 + 64 * u); \
+        if (U > 1) HGQ_PE_WAIT();                                             \
+    } while (0)
+
+template <int RM, int OM, bool TRAIN, int LIVE, int U>
+__global__ __launch_bounds__(Q1D_BS) void quant_fwd_pe(const f32x4 *__restrict__ x, const f32x4 *__restrict__ k,
+                                                       const f32x4 *__restrict__ i, const f32x4 *__restrict__ fb,
+                                                       f32x4 *__restrict__ y, int64_t v_begin, int64_t v_end, int kbi) {
+    const int64_t v0 = pe_first_vector<U>(v_begin);
+    if (U == 1 && v0 >= v_end) return;
+    f32x4 xv[U], fv[U], iv[U], kv[U], yv[U];
+    HGQ_PE_LOAD(xv, x);
+    HGQ_PE_LOAD(fv, fb);
+    if (LIVE & 1) HGQ_PE_LOAD(iv, i);
+    if (LIVE & 2) HGQ_PE_LOAD(kv, k);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) yv[u][c] = quantize<RM, OM>(xv[u][c], pe_kif<LIVE>(kv[u], iv[u], fv[u], c, kbi != 0), TRAIN);
+    }
+    HGQ_PE_STORE(yv, y);
+}
+
+template <int RM, int OM, int LIVE, int U>
 __global__ __launch_bounds__(Q1D_BS) void quant_bwd_pe(const f32x4 *__restrict__ dy, const f32x4 *__restrict__ x,
                                                        const f32x4 *__restrict__ k, const f32x4 *__restrict__ i,
                                                        const f32x4 *__restrict__ fb, f32x4 *__restrict__ dx,
-                                                       f32x4 *__restrict__ di, f32x4 *__restrict__ dfb, int64_t nvec, int kbi) {
-    const int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x;
-    if (v >= nvec) return;
-    const f32x4 gv = __builtin_nontemporal_load(dy + v);
-    const f32x4 xv = __builtin_nontemporal_load(x + v);
-    const f32x4 fv = __builtin_nontemporal_load(fb + v);
-    f32x4 iv = {0.f, 0.f, 0.f, 0.f}, kv = {0.f, 0.f, 0.f, 0.f};
-    if (LIVE & 1) iv = __builtin_nontemporal_load(i + v);
-    if (LIVE & 2) kv = __builtin_nontemporal_load(k + v);
-    f32x4 gx, gi, gf;
+                                                       f32x4 *__restrict__ di, f32x4 *__restrict__ dfb, int64_t v_begin,
+                                                       int64_t v_end, int kbi) {
+    const int64_t v0 = pe_first_vector<U>(v_begin);
+    if (U == 1 && v0 >= v_end) return;
+    f32x4 gv[U], xv[U], fv[U], iv[U], kv[U];
+    HGQ_PE_LOAD(gv, dy);
+    HGQ_PE_LOAD(xv, x);
+    HGQ_PE_LOAD(fv, fb);
+    if (LIVE & 1) HGQ_PE_LOAD(iv, i);
+    if (LIVE & 2) HGQ_PE_LOAD(kv, k);
+    f32x4 gx[U], gi[U], gf[U];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        float a, b, d;
-        quantize_grad<RM, OM>(xv[c], gv[c], pe_kif<LIVE>(kv, iv, fv, c, kbi != 0), a, b, d);
-        if (kbi) b -= d;  // f = b - i
-        gx[c] = a, gi[c] = b, gf[c] = d;
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float a, b, d;
+            quantize_grad<RM, OM>(xv[u][c], gv[u][c], pe_kif<LIVE>(kv[u], iv[u], fv[u], c, kbi != 0), a, b, d);
+            if (kbi) b -= d;  // f = b - i
+            gx[u][c] = a, gi[u][c] = b, gf[u][c] = d;
+        }
     }
-    if (dx) __builtin_nontemporal_store(gx, dx + v);
-    if (di) __builtin_nontemporal_store(gi, di + v);
-    if (dfb) __builtin_nontemporal_store(gf, dfb + v);
+    if (dx) HGQ_PE_STORE(gx, dx);
+    if (di) HGQ_PE_STORE(gi, di);
+    if (dfb) HGQ_PE_STORE(gf, dfb);
+}
+
+// Forward and surrogate backward of a training step in ONE pass: x (and k, i where live), f and the upstream gradient
+// in; y, dx, di, df out.  The value is rounded once and every operand crosses HBM once: 28 B/elem in WRAP training
+// (x, f, dy read; four arrays written) against 12 + 24 for the two separate launches, 36 B/elem with every operand
+// live against 20 + 32, and one launch ramp instead of two.
+template <int RM, int OM, int LIVE, int U>
+__global__ __launch_bounds__(Q1D_BS) void quant_fwd_bwd_pe(const f32x4 *__restrict__ x, const f32x4 *__restrict__ k,
+                                                           const f32x4 *__restrict__ i, const f32x4 *__restrict__ fb,
+                                                           const f32x4 *__restrict__ dy, f32x4 *__restrict__ y,
+                                                           f32x4 *__restrict__ dx, f32x4 *__restrict__ di,
+                                                           f32x4 *__restrict__ dfb, int64_t v_begin, int64_t v_end, int kbi) {
+    const int64_t v0 = pe_first_vector<U>(v_begin);
+    if (U == 1 && v0 >= v_end) return;
+    f32x4 xv[U], fv[U], gv[U], iv[U], kv[U];
+    HGQ_PE_LOAD(xv, x);
+    HGQ_PE_LOAD(fv, fb);
+    HGQ_PE_LOAD(gv, dy);
+    if (LIVE & 1) HGQ_PE_LOAD(iv, i);
+    if (LIVE & 2) HGQ_PE_LOAD(kv, k);
+    f32x4 yv[U], gx[U], gi[U], gf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float a, b, d;
+            yv[u][c] = quantize_with_grad<RM, OM>(xv[u][c], gv[u][c], pe_kif<LIVE>(kv[u], iv[u], fv[u], c, kbi != 0), a, b, d);
+            if (kbi) b -= d;  // f = b - i
+            gx[u][c] = a, gi[u][c] = b, gf[u][c] = d;
+        }
+    }
+    HGQ_PE_STORE(yv, y);
+    if (dx) HGQ_PE_STORE(gx, dx);
+    if (di) HGQ_PE_STORE(gi, di);
+    if (dfb) HGQ_PE_STORE(gf, dfb);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -587,7 +655,8 @@ __global__ __launch_bounds__(256) void quant_bwd_multi_kernel(QuantGradBatch b) 
 template <int NR, int NW>
 __global__ __launch_bounds__(Q1D_BS) void stream_probe_kernel(const f32x4 *__restrict__ a, const f32x4 *__restrict__ b,
                                                               const f32x4 *__restrict__ c, f32x4 *__restrict__ o0,
-                                                              f32x4 *__restrict__ o1, f32x4 *__restrict__ o2, int64_t nvec) {
+                                                              f32x4 *__restrict__ o1, f32x4 *__restrict__ o2,
+                                                              f32x4 *__restrict__ o3, int64_t nvec) {
     const int64_t v = (int64_t)blockIdx.x * Q1D_BS + threadIdx.x;
     if (v >= nvec) return;
     f32x4 t = __builtin_nontemporal_load(a + v);
@@ -596,6 +665,7 @@ __global__ __launch_bounds__(Q1D_BS) void stream_probe_kernel(const f32x4 *__res
     __builtin_nontemporal_store(t, o0 + v);
     if (NW > 1) __builtin_nontemporal_store(t * 2.0f, o1 + v);
     if (NW > 2) __builtin_nontemporal_store(t * 3.0f, o2 + v);
+    if (NW > 3) __builtin_nontemporal_store(t * 4.0f, o3 + v);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -708,13 +778,13 @@ using namespace hgq;
 extern "C" int hgq_version(void) { return 1; }
 extern "C" const char *hgq_last_error(void) { return g_err; }
 
-extern "C" int hgq_stream_probe(const float *a, const float *b, const float *c, float *o0, float *o1, float *o2, int n_read,
-                                int n_write, int64_t n, void *stream) {
-    if (n < 4 || n % 4 != 0 || n_read < 1 || n_read > 3 || n_write < 1 || n_write > 3)
-        return fail(HGQ_ERR_ARG, "hgq_stream_probe: n must be a positive multiple of 4, 1..3 arrays each way");
+extern "C" int hgq_stream_probe(const float *a, const float *b, const float *c, float *o0, float *o1, float *o2, float *o3,
+                                int n_read, int n_write, int64_t n, void *stream) {
+    if (n < 4 || n % 4 != 0 || n_read < 1 || n_read > 3 || n_write < 1 || n_write > 4)
+        return fail(HGQ_ERR_ARG, "hgq_stream_probe: n must be a positive multiple of 4, 1..3 arrays read, 1..4 written");
     const float *in[3] = {a, b, c};
-    float *out[3] = {o0, o1, o2};
-    for (int t = 0; t < 3; ++t)
+    float *out[4] = {o0, o1, o2, o3};
+    for (int t = 0; t < 4; ++t)
         if ((t < n_read && (!in[t] || !aligned16(in[t]))) || (t < n_write && (!out[t] || !aligned16(out[t]))))
             return fail(HGQ_ERR_ARG, "hgq_stream_probe: arrays must be non-null and 16-byte aligned");
     const int64_t nvec = n / 4, grid = (nvec + Q1D_BS - 1) / Q1D_BS;
@@ -722,17 +792,20 @@ extern "C" int hgq_stream_probe(const float *a, const float *b, const float *c, 
     hipStream_t s = (hipStream_t)stream;
 #define HGQ_PROBE(NRV, NWV)                                                                                                    \
     hipLaunchKernelGGL((stream_probe_kernel<NRV, NWV>), dim3((unsigned)grid), dim3(Q1D_BS), 0, s, (const f32x4 *)a, (const f32x4 *)b, \
-                       (const f32x4 *)c, (f32x4 *)o0, (f32x4 *)o1, (f32x4 *)o2, nvec)
-    switch (n_read * 4 + n_write) {
-        case 1 * 4 + 1: HGQ_PROBE(1, 1); break;
-        case 1 * 4 + 2: HGQ_PROBE(1, 2); break;
-        case 1 * 4 + 3: HGQ_PROBE(1, 3); break;
-        case 2 * 4 + 1: HGQ_PROBE(2, 1); break;
-        case 2 * 4 + 2: HGQ_PROBE(2, 2); break;
-        case 2 * 4 + 3: HGQ_PROBE(2, 3); break;
-        case 3 * 4 + 1: HGQ_PROBE(3, 1); break;
-        case 3 * 4 + 2: HGQ_PROBE(3, 2); break;
-        default: HGQ_PROBE(3, 3); break;
+                       (const f32x4 *)c, (f32x4 *)o0, (f32x4 *)o1, (f32x4 *)o2, (f32x4 *)o3, nvec)
+    switch (n_read * 8 + n_write) {
+        case 1 * 8 + 1: HGQ_PROBE(1, 1); break;
+        case 1 * 8 + 2: HGQ_PROBE(1, 2); break;
+        case 1 * 8 + 3: HGQ_PROBE(1, 3); break;
+        case 1 * 8 + 4: HGQ_PROBE(1, 4); break;
+        case 2 * 8 + 1: HGQ_PROBE(2, 1); break;
+        case 2 * 8 + 2: HGQ_PROBE(2, 2); break;
+        case 2 * 8 + 3: HGQ_PROBE(2, 3); break;
+        case 2 * 8 + 4: HGQ_PROBE(2, 4); break;
+        case 3 * 8 + 1: HGQ_PROBE(3, 1); break;
+        case 3 * 8 + 2: HGQ_PROBE(3, 2); break;
+        case 3 * 8 + 3: HGQ_PROBE(3, 3); break;
+        default: HGQ_PROBE(3, 4); break;
     }
 #undef HGQ_PROBE
     return check_launch("hgq_stream_probe");
@@ -760,13 +833,57 @@ static bool cols_grid(int64_t rows, int64_t M, int batch_rows, int64_t gx, int64
     return true;
 }
 
-// launches of the lean per-element kernels (inside HGQ_DISPATCH_RM_OM: RM, OM, and the locals of the entry point)
-#define HGQ_FWD_PE(TRAINV, LIVEV)                                                                                                     \
-    hipLaunchKernelGGL((quant_fwd_pe<RM, OM, TRAINV, LIVEV>), dim3((unsigned)pe_grid), dim3(Q1D_BS), 0, s, (const f32x4 *)x, (const f32x4 *)k, \
-                       (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)y, n4, (int)m.kbi)
-#define HGQ_BWD_PE(LIVEV)                                                                                                              \
-    hipLaunchKernelGGL((quant_bwd_pe<RM, OM, LIVEV>), dim3((unsigned)pe_grid), dim3(Q1D_BS), 0, s, (const f32x4 *)dy, (const f32x4 *)x,      \
-                       (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)dx, (f32x4 *)di, (f32x4 *)dfb, n4, (int)m.kbi)
+// Launches of the lean per-element kernels over n4 vectors (inside HGQ_DISPATCH_RM_OM: RM, OM, and the locals of the
+// entry point).  Whole tiles of two vectors per lane first where that form pays (pe_two_vectors), then the remaining
+// vectors - all of them for small inputs - one per thread.
+#define HGQ_PE_SPLIT(TWO)                                                                                   \
+    const int64_t pe_tiles = (TWO) ? n4 / (2 * Q1D_BS) : 0, pe_main = pe_tiles * 2 * Q1D_BS, pe_rest = n4 - pe_main, \
+                  pe_rest_grid = (pe_rest + Q1D_BS - 1) / Q1D_BS
+#define HGQ_FWD_PE(TRAINV, LIVEV)                                                                                                    \
+    do {                                                                                                                              \
+        if (pe_tiles > 0)                                                                                                             \
+            hipLaunchKernelGGL((quant_fwd_pe<RM, OM, TRAINV, LIVEV, 2>), dim3((unsigned)pe_tiles), dim3(Q1D_BS), 0, s, (const f32x4 *)x, \
+                               (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)y, (int64_t)0, pe_main, (int)m.kbi);   \
+        if (pe_rest > 0)                                                                                                              \
+            hipLaunchKernelGGL((quant_fwd_pe<RM, OM, TRAINV, LIVEV, 1>), dim3((unsigned)pe_rest_grid), dim3(Q1D_BS), 0, s,            \
+                               (const f32x4 *)x, (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)y, pe_main, n4,      \
+                               (int)m.kbi);                                                                                           \
+    } while (0)
+#define HGQ_BWD_PE(LIVEV)                                                                                                             \
+    do {                                                                                                                              \
+        if (pe_tiles > 0)                                                                                                             \
+            hipLaunchKernelGGL((quant_bwd_pe<RM, OM, LIVEV, 2>), dim3((unsigned)pe_tiles), dim3(Q1D_BS), 0, s, (const f32x4 *)dy,     \
+                               (const f32x4 *)x, (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)dx, (f32x4 *)di,     \
+                               (f32x4 *)dfb, (int64_t)0, pe_main, (int)m.kbi);                                                        \
+        if (pe_rest > 0)                                                                                                              \
+            hipLaunchKernelGGL((quant_bwd_pe<RM, OM, LIVEV, 1>), dim3((unsigned)pe_rest_grid), dim3(Q1D_BS), 0, s, (const f32x4 *)dy, \
+                               (const f32x4 *)x, (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (f32x4 *)dx, (f32x4 *)di,     \
+                               (f32x4 *)dfb, pe_main, n4, (int)m.kbi);                                                                \
+    } while (0)
+#define HGQ_FWD_BWD_PE(LIVEV)                                                                                                         \
+    do {                                                                                                                              \
+        if (pe_tiles > 0)                                                                                                             \
+            hipLaunchKernelGGL((quant_fwd_bwd_pe<RM, OM, LIVEV, 2>), dim3((unsigned)pe_tiles), dim3(Q1D_BS), 0, s, (const f32x4 *)x,  \
+                               (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (const f32x4 *)dy, (f32x4 *)y, (f32x4 *)dx,     \
+                               (f32x4 *)di, (f32x4 *)dfb, (int64_t)0, pe_main, (int)m.kbi);                                           \
+        if (pe_rest > 0)                                                                                                              \
+            hipLaunchKernelGGL((quant_fwd_bwd_pe<RM, OM, LIVEV, 1>), dim3((unsigned)pe_rest_grid), dim3(Q1D_BS), 0, s,                \
+                               (const f32x4 *)x, (const f32x4 *)k, (const f32x4 *)i, (const f32x4 *)fb, (const f32x4 *)dy,            \
+                               (f32x4 *)y, (f32x4 *)dx, (f32x4 *)di, (f32x4 *)dfb, pe_main, n4, (int)m.kbi);                          \
+    } while (0)
+
+// Two vectors per lane pay where they put the whole input on the device in one round of workgroups, or nearly so, and one
+// vector per thread would take two to three rounds: measured per size with both forms, the two-vector form is 10 - 17 %
+// faster from one to two rounds' worth of vectors (2 Mi - 4 Mi elements on 256 CUs), within +-2 % up to three rounds, and
+// 1 - 3 % slower beyond, where the rounds of the one-vector form no longer run in step anyway.  The forward alone has few
+// streams and gains only from one and a half rounds on.
+static bool pe_two_vectors(int64_t n4, bool many_streams) {
+#ifdef HGQ_PE_FORCE_VECTORS
+    return HGQ_PE_FORCE_VECTORS == 2;  // measurement builds only
+#endif
+    const int64_t one_round = (int64_t)persistent_grid(1ll << 40, 1) * 2048;  // threads the device holds at once
+    return (many_streams ? n4 >= one_round : 2 * n4 >= 3 * one_round) && n4 <= 3 * one_round;
+}
 
 // launch of the per-column forward kernel: vector width and training flag as template arguments
 #define HGQ_FWD_COLS_1(VECV, TRAINV, SLICED)                                                                                       \
@@ -805,8 +922,8 @@ extern "C" int hgq_quantize_fwd(const float *x, const void *k, const float *i, c
         const int64_t tail0 = n4 * 4, tail = n - tail0;
         // the lean per-element kernel: no trackers, and k either dead or stored as fp32
         const bool k_dead = m.overflow_mode == HGQ_WRAP && m.training;
-        const int64_t pe_grid = (n4 + Q1D_BS - 1) / Q1D_BS;
-        const bool lean = !shared && n4 > 0 && !amax && !anyneg && !m.track_input && (k_dead || !m.k_u8) && pe_grid < (1ll << 31);
+        const bool lean = !shared && n4 > 0 && !amax && !anyneg && !m.track_input && (k_dead || !m.k_u8) && n4 / Q1D_BS < (1ll << 30);
+        HGQ_PE_SPLIT(lean && pe_two_vectors(n4, false));
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (lean) {
                 if (OM == HGQ_WRAP && m.training) {
@@ -1080,8 +1197,8 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
         const int64_t n4 = vec ? (n / 4) : 0;
         const int64_t tail0 = n4 * 4, tail = n - tail0;
         const bool k_dead = m.overflow_mode == HGQ_WRAP;  // the WRAP surrogate gradient only rounds
-        const int64_t pe_grid = (n4 + Q1D_BS - 1) / Q1D_BS;
-        const bool lean = !shared && n4 > 0 && (k_dead || !m.k_u8) && pe_grid < (1ll << 31);
+        const bool lean = !shared && n4 > 0 && (k_dead || !m.k_u8) && n4 / Q1D_BS < (1ll << 30);
+        HGQ_PE_SPLIT(lean && pe_two_vectors(n4, true));
         HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
             if (lean) {
                 if (OM == HGQ_WRAP) {
@@ -1133,6 +1250,47 @@ extern "C" int hgq_quantize_bwd(const float *dy, const float *x, const void *k, 
         hipLaunchKernelGGL((quant_bwd_generic<RM, OM>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n, bw_size, bw_inner, mode);
     });
     return check_launch("hgq_quantize_bwd");
+}
+
+extern "C" int hgq_quantize_fwd_bwd(const float *x, const void *k, const float *i, const float *fb, const float *dy, float *y,
+                                    float *dx, float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode,
+                                    void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (n < 0 || bw_size < 1 || bw_inner < 1) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_bwd: bad sizes");
+    if (n == 0) return HGQ_OK;
+    if (!x || !k || !i || !fb || !dy || !y) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_bwd: null pointer");
+    if (bw_size * bw_inner > n || n % (bw_size * bw_inner) != 0)
+        return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_bwd: n=%lld is not a multiple of bw_size*bw_inner", (long long)n);
+    const Mode m(mode);
+    if (!m.training) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_bwd: the surrogate gradient is defined for training mode only");
+    if (m.track_input) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_bwd: no trackers here; HGQ_MODE_TRACK_INPUT has no meaning");
+    const bool k_dead = m.overflow_mode == HGQ_WRAP;  // a WRAP quantizer in training mode only rounds
+    const bool all16 = aligned16(x) && aligned16(i) && aligned16(fb) && aligned16(dy) && aligned16(y) && (!dx || aligned16(dx)) &&
+                       (!di || aligned16(di)) && (!dfb || aligned16(dfb)) && (k_dead || (!m.k_u8 && aligned16(k)));
+    const int64_t n4 = n / 4;
+    if (bw_size == n && n4 > 0 && all16 && n4 / Q1D_BS < (1ll << 30)) {
+        const int64_t tail0 = n4 * 4, tail = n - tail0;
+        HGQ_PE_SPLIT(pe_two_vectors(n4, true));
+        HGQ_DISPATCH_RM_OM(m.round_mode, m.overflow_mode, {
+            if (OM == HGQ_WRAP) {
+                if (m.kbi) HGQ_FWD_BWD_PE(1);
+                else HGQ_FWD_BWD_PE(0);
+            } else {
+                HGQ_FWD_BWD_PE(3);
+            }
+        });
+        int rc = check_launch("hgq_quantize_fwd_bwd");
+        if (rc || tail == 0) return rc;
+        // up to three trailing elements: the general kernels, one workgroup each
+        const void *kt = m.k_u8 ? (const void *)((const uint8_t *)k + tail0) : (const void *)((const float *)k + tail0);
+        if ((rc = hgq_quantize_fwd(x + tail0, kt, i + tail0, fb + tail0, y + tail0, nullptr, nullptr, tail, tail, 1, mode, stream))) return rc;
+        return hgq_quantize_bwd(dy + tail0, x + tail0, kt, i + tail0, fb + tail0, dx ? dx + tail0 : nullptr, di ? di + tail0 : nullptr,
+                                dfb ? dfb + tail0 : nullptr, tail, tail, 1, mode, stream);
+    }
+    // shared or per-column bit-widths, uint8 k with a live k, unaligned operands: the two separate passes
+    int rc = hgq_quantize_fwd(x, k, i, fb, y, nullptr, nullptr, n, bw_size, bw_inner, mode, stream);
+    if (rc) return rc;
+    return hgq_quantize_bwd(dy, x, k, i, fb, dx, di, dfb, n, bw_size, bw_inner, mode, stream);
 }
 
 extern "C" int hgq_wrap_track_i(const uint32_t *amax, const uint32_t *anyneg, int n_parts, float *i_var, const float *fb,

@@ -118,6 +118,29 @@ def quantize_bwd(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: 
     return dx, di, dfb
 
 
+@torch.library.custom_op('hgq::quantize_fwd_bwd', mutates_args=())
+def quantize_fwd_bwd(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, dy: Tensor, mode: int, bw_inner: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Training-mode forward and surrogate backward in one launch: ``(y, dx, di, dfb)`` for a caller that holds the upstream
+    gradient ``dy`` when it quantizes.  ``mode`` must carry MODE_TRAINING."""
+    _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb), _check_f32('dy', dy)
+    bw_size = i.numel()
+    _need(k.numel() == bw_size and fb.numel() == bw_size, 'k, i, f must have the same number of elements')
+    _need(dy.numel() == x.numel(), 'dy and x differ in size')
+    n = x.numel()
+    _need(bw_size >= 1 and bw_inner >= 1 and (n == 0 or n % (bw_size * bw_inner) == 0),
+          f'x has {n} elements, not a multiple of bw_size*bw_inner = {bw_size}*{bw_inner}')
+    y, dx, di, dfb = torch.empty_like(x), torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+    rc = _lib.load().hgq_quantize_fwd_bwd(_ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dy), _ptr(y), _ptr(dx), _ptr(di), _ptr(dfb), n,
+                                          bw_size, bw_inner, _kmode(mode, k), _stream())
+    _lib.check(rc, 'hgq_quantize_fwd_bwd')
+    return y, dx, di, dfb
+
+
+@quantize_fwd_bwd.register_fake
+def _(x, k, i, fb, dy, mode, bw_inner):
+    return torch.empty_like(x), torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+
+
 @torch.library.custom_op('hgq::quantize_bwd_slices', mutates_args=())
 def quantize_bwd_slices(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, need_dx: bool,
                         need_di: bool) -> tuple[Tensor, Tensor]:

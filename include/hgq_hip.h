@@ -137,12 +137,12 @@ int hgq_quantize_bwd_stochastic(const float *dy, const float *x, const void *k, 
 
 /*
  * Measurement aid (no counterpart in the reference): o_j[e] = (j + 1) * (a[e] (+ b[e]) (+ c[e])) for the first n_write
- * outputs and n_read inputs, one 128-bit non-temporal access per array per thread.  4 * (n_read + n_write) * n bytes
- * cross HBM per launch and nothing else: used to scale the hardware traffic counters and as the bandwidth a plain
+ * (1..4) outputs and n_read (1..3) inputs, one 128-bit non-temporal access per array per thread.  4 * (n_read + n_write) * n
+ * bytes cross HBM per launch and nothing else: used to scale the hardware traffic counters and as the bandwidth a plain
  * streaming kernel of a given read / write mix reaches at a given size.  n a multiple of 4, arrays 16-byte aligned.
  */
-int hgq_stream_probe(const float *a, const float *b, const float *c, float *o0, float *o1, float *o2, int n_read, int n_write,
-                     int64_t n, void *stream);
+int hgq_stream_probe(const float *a, const float *b, const float *c, float *o0, float *o1, float *o2, float *o3, int n_read,
+                     int n_write, int64_t n, void *stream);
 
 /*
  * hgq_quantize_bwd_sliced without a workspace argument.  This entry point has no counterpart in the reference.  It is
@@ -189,6 +189,19 @@ int hgq_quantize_bwd_multi(const hgq_quant_grad_item *items, int count, void *st
 int hgq_quantize_bwd(const float *dy, const float *x, const void *k, const float *i, const float *fb,
                      float *dx, float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner,
                      int mode, void *stream);
+
+/*
+ * Training-mode forward and surrogate backward of the fixed-point quantizer in one launch, for callers that hold the
+ * upstream gradient when they quantize (the standalone quantizer step: `y = q(x, k, i, f, training=True)` followed by
+ * the custom gradients of the same callable, src/hgq/quantizer/internal/fixed_point_quantizer.py:142-150,401-429).
+ * Results are those of hgq_quantize_fwd (HGQ_MODE_TRAINING, no trackers) and hgq_quantize_bwd on the same operands,
+ * bit for bit.  With per-element bit-widths (bw_size == n), 16-byte aligned operands and an fp32 or dead k every
+ * operand crosses HBM once: x, f, dy read and y, dx, di, dfb written (28 B per element) for a WRAP quantizer, whose
+ * training branch reads neither k nor i; 36 B per element with every operand live.  Other layouts run the two passes.
+ *   y [n] required; dx [n], di, dfb [bw_size] may each be NULL.  HGQ_MODE_TRAINING must be set.
+ */
+int hgq_quantize_fwd_bwd(const float *x, const void *k, const float *i, const float *fb, const float *dy, float *y, float *dx,
+                         float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, void *stream);
 
 /*
  * Integer-bit tracking of WRAP quantizers.  Replaces minimal_i_given_xf / minimal_i_given_xb

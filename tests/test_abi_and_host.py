@@ -143,6 +143,14 @@ def test_entry_points_validate_arguments_before_any_launch():
     assert lib.hgq_quantize_fwd(none, none, none, none, none, none, none, 16, 1, 1, 1, none) == ARG  # null pointers
     assert lib.hgq_quantize_fwd(none, none, none, none, none, none, none, 10, 4, 1, 1, none) == ARG  # 10 % 4 != 0
     assert b'null' in lib.hgq_last_error() or b'multiple' in lib.hgq_last_error()
+    # forward + backward in one launch: same checks, and training mode is required
+    TRAIN = _lib.MODE_TRAINING | 1
+    args9 = [none] * 9
+    assert lib.hgq_quantize_fwd_bwd(*args9, 0, 1, 1, TRAIN, none) == OK
+    assert lib.hgq_quantize_fwd_bwd(*args9, 16, 16, 1, TRAIN, none) == ARG and b'null' in lib.hgq_last_error()
+    one = ctypes.c_void_p(256)  # never dereferenced: the mode check comes before any launch
+    assert lib.hgq_quantize_fwd_bwd(*([one] * 9), 16, 16, 1, 1, none) == ARG and b'training' in lib.hgq_last_error()
+    assert lib.hgq_quantize_fwd_bwd(*([one] * 9), 10, 4, 1, TRAIN, none) == ARG
     # table softmax: row length, table rows
     assert lib.hgq_qsoftmax_bwd_workspace(1024, 64, 256, 1) > 0
     assert lib.hgq_qsoftmax_bwd_workspace(1024, 300, 1, 0) == -1          # rows longer than 256

@@ -73,6 +73,71 @@ def test_standalone_quantizer_at_4Mi(dev, overflow_mode, training):
         np.testing.assert_allclose(got.numpy(), ref_g.numpy(), rtol=RTOL, atol=1e-30, err_msg=f'{overflow_mode} {name}')
 
 
+@pytest.mark.parametrize('overflow_mode', ['WRAP', 'SAT', 'SAT_SYM'])
+@pytest.mark.parametrize('kbi', [False, True])
+def test_standalone_quantizer_fwd_bwd_in_one_launch_at_4Mi(dev, overflow_mode, kbi):
+    """``hgq_quantize_fwd_bwd`` on the configuration's operands (4 Mi elements, per-element bit-widths, RND, training):
+    y bit-exact, dx / di / df within 1e-5 per element of the oracle's callable and its custom gradients
+    (reference fixed_point_quantizer.py:142-150; KBI: f = b - i, :256-265), and bit-equal to the two separate
+    launches.  i reaches below -f here, so SAT words with i + f < 0 are part of the case."""
+    from hgq2_amd import _lib, ops
+
+    n = 4 * 1024 * 1024
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(n, generator=g) * 2.0).requires_grad_(True)
+    k = torch.randint(0, 2, (n,), generator=g).float() if overflow_mode != 'WRAP' else torch.ones(n)
+    i = torch.randint(-2, 5, (n,), generator=g).float().requires_grad_(True)
+    fb = torch.randint(0, 9, (n,), generator=g).float().requires_grad_(True)  # f, or b with kbi
+    gy = torch.randn(n, generator=g)
+    q = ofp.get_fixed_quantizer('RND', overflow_mode)
+    want = q(x, k, i, fb - i if kbi else fb, True, None)
+    want.backward(gy)
+    mode = _lib.mode_bits('RND', overflow_mode, training=True, kbi=kbi)
+    xd, kd, idv, fd, gd = (t.detach().to(dev) for t in (x, k, i, fb, gy))
+    y, dx, di, dfb = ops.quantize_fwd_bwd(xd, kd, idv, fd, gd, mode, 1)
+    assert torch.equal(y.cpu(), want.detach())
+    for got, ref_g, name in ((dx, x.grad, 'dx'), (di, i.grad, 'di'), (dfb, fb.grad, 'df')):
+        ref_g = torch.zeros(n) if ref_g is None else ref_g
+        np.testing.assert_allclose(got.cpu().numpy(), ref_g.numpy(), rtol=RTOL, atol=1e-30, err_msg=f'{overflow_mode} kbi={kbi} {name}')
+    y2, _, _ = ops.quantize_fwd(xd, kd, idv, fd, mode, 1, False)
+    dx2, di2, dfb2 = ops.quantize_bwd(gd, xd, kd, idv, fd, mode, 1, True, True)
+    for a, b in ((y, y2), (dx, dx2), (di, di2), (dfb, dfb2)):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize('n,bw_shape,x_shape', [(4 * 1000 + 3, None, None), (7, None, None), (2, None, None),
+                                               (None, (1, 24), (300, 24)), (None, (1, 1), (37, 5)), (None, (1, 6, 1), (9, 6, 10))])
+@pytest.mark.parametrize('round_mode,overflow_mode', [('RND', 'WRAP'), ('TRN', 'SAT'), ('RND_CONV', 'SAT_SYM')])
+def test_quantizer_fwd_bwd_in_one_launch_ragged_and_shared(dev, n, bw_shape, x_shape, round_mode, overflow_mode):
+    """Sizes that are not a multiple of four, tiny inputs, a uint8 k, and bit-widths shared over axes (where the
+    entry point runs the two passes): the same results as the separate forward and backward operators."""
+    from hgq2_amd import _lib, ops
+
+    g = torch.Generator().manual_seed(7)
+    if x_shape is None:
+        x_shape = bw_shape = (n,)
+    x = (torch.randn(x_shape, generator=g) * 3).to(dev)
+    gy = torch.randn(x_shape, generator=g).to(dev)
+    k = torch.randint(0, 2, bw_shape, generator=g).to(torch.uint8).to(dev)
+    i = torch.randint(-1, 4, bw_shape, generator=g).float().to(dev)
+    f = torch.randint(0, 7, bw_shape, generator=g).float().to(dev)
+    inner = 1
+    for a in range(len(x_shape) - 1, -1, -1):
+        if bw_shape[a] != 1:
+            break
+        inner *= x_shape[a]
+    mode = _lib.mode_bits(round_mode, overflow_mode, training=True)
+    y, dx, di, df = ops.quantize_fwd_bwd(x, k, i, f, gy, mode, inner)
+    y2, _, _ = ops.quantize_fwd(x, k, i, f, mode, inner, False)
+    dx2, di2, df2 = ops.quantize_bwd(gy, x, k, i, f, mode, inner, True, True)
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
+    if i.numel() == x.numel():
+        assert torch.equal(di, di2) and torch.equal(df, df2)
+    else:  # sums over the shared axes: the separate operator may add them in another (fixed) order
+        scale = gy.abs().sum() * (math.log(2) * 8.0 + 1.0)
+        assert float((di - di2).abs().max()) <= RTOL * float(scale) and float((df - df2).abs().max()) <= RTOL * float(scale)
+
+
 # --------------------------------------------------------------------------------------------------------------
 # the stateless callable, driven as the reference drives it
 # --------------------------------------------------------------------------------------------------------------
