@@ -25,8 +25,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of the 4 Mi-element quantizer kernels from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # counters, each scaled by what the same counter reads for the plain streaming kernel of known size
 # (hgq_stream_probe); summary and commands in profiles/quantizer_4Mi_hbm_counters.md
-TRAFFIC_BYTES = {'quant_fwd': 50.34e6, 'quant_bwd': 100.67e6, 'quant_fwd_sat': 83.89e6, 'quant_bwd_sat': 134.22e6,
-                 'quant_fwd_bwd': 117.44e6, 'quant_fwd_bwd_sat': 150.99e6}
+TRAFFIC_BYTES = {'quant_fwd': 50.36e6, 'quant_bwd': 100.72e6, 'quant_fwd_sat': 83.88e6, 'quant_bwd_sat': 134.28e6,
+                 'quant_fwd_bwd': 117.53e6, 'quant_fwd_bwd_sat': 151.07e6}
 BATCH = 16384
 DIMS = (16, 64, 32, 32, 5)
 QN = 4 * 1024 * 1024  # standalone quantizer case: 4 Mi fp32 elements
