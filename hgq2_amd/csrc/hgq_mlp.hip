@@ -134,7 +134,7 @@ __device__ __forceinline__ void mlp_snapshot_end(MlpSnapRow r, float *aux, int l
 
 __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ img, const float *__restrict__ x,
                                                           const int64_t *__restrict__ labels, int64_t rows,
-                                                          float *part, float *aux, float *loss) {
+                                                          float *part, float *aux, uint32_t *ticket) {
     extern __shared__ float lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // snapshot for the update pass: workgroup w's last wavefront takes row w; its loads travel with the image fetch below
@@ -142,11 +142,13 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
     MlpSnapRow snap;
     snap.l = -1;
     if (snap_wave) snap = mlp_snapshot_begin(d, (int)blockIdx.x, lane);
-    if (blockIdx.x == 0 && tid == 0 && loss) loss[0] = 0.f;  // the update pass accumulates into it
+    if (blockIdx.x == 0 && tid == 0) ticket[0] = 0u;  // the update pass counts its finished workgroups here
     const int L = d.n_layers;
     float *raw = lds + d.off_raw, *rx = lds + d.off_rx;
-    float *dfs = lds + d.off_red;                                 // [L][64] fractional-bit gradient sums
-    uint32_t *amx = (uint32_t *)(lds + d.off_red) + 64 * HGQ_MLP_MAX_LAYERS;  // [L][64] abs-max of each layer's quantized input
+    // [2][L][64] fractional-bit gradient sums: one set per row half of the tile, each entry owned by one wavefront for the
+    // whole launch (no atomics: the two halves are added in a fixed order at the end)
+    float *dfs = lds + d.off_red;
+    uint32_t *amx = (uint32_t *)(lds + d.off_red) + 2 * 64 * HGQ_MLP_MAX_LAYERS;  // [L][64] abs-max of each layer's quantized input
     float *my = part + (int64_t)blockIdx.x * d.M;
     const int64_t n_tiles = (rows + MLP_BM - 1) / MLP_BM;
     const float inv_rows = 1.0f / (float)rows;
@@ -167,7 +169,7 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
         }
     }
     for (int id = tid; id < MLP_BM * d.ld_rx; id += MLP_NT) rx[id] = 0.f;  // padding columns stay zero for good
-    for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += MLP_NT) dfs[id] = 0.f, amx[id] = 0u;
+    for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += MLP_NT) dfs[id] = 0.f, dfs[64 * HGQ_MLP_MAX_LAYERS + id] = 0.f, amx[id] = 0u;
     __syncthreads();
     if (snap_wave) {
         mlp_snapshot_end(snap, aux, lane);
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                         nxt[row * MLP_LDZ + kcol] = (kcol < K && (!mask_below || a > 0.f)) ? acc[r] : 0.f;
                     }
                     dfsum += __shfl_xor(dfsum, 32, 64);
-                    if (lane < 32 && kcol < K) atomicAdd(&dfs[l * 64 + kcol], dfsum);
+                    if (lane < 32 && kcol < K) dfs[(rh * HGQ_MLP_MAX_LAYERS + l) * 64 + kcol] += dfsum;  // this wavefront's own entry
                 }
             }
             __syncthreads();
@@ -360,7 +362,7 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
     for (int l = 0; l < L; ++l) {
         const MlpLayerDev &ly = d.l[l];
         if (tid < ly.h.K) {
-            my[ly.p_df + tid] = dfs[l * 64 + tid];
+            my[ly.p_df + tid] = dfs[l * 64 + tid] + dfs[(HGQ_MLP_MAX_LAYERS + l) * 64 + tid];
             ((uint32_t *)(my + ly.p_amax))[tid] = amx[l * 64 + tid];
         }
     }
@@ -380,8 +382,30 @@ __device__ __forceinline__ float sgd_clip(float w, float g, float lr, float l1, 
 // input bit counts the EBOPs gradients need) without waiting for another workgroup; pre-update values of variables it
 // does not own come from the main kernel's snapshot.
 #define MLP_RG 16
+// The loss is the sum of one piece per workgroup (cross-entropy, a layer's ebops * beta, MonoL1 terms).  Every workgroup
+// leaves its piece in its own slot and draws a ticket; the one that draws the last ticket adds the slots in block order.
+// Slots and ticket are only touched by device-scope atomics (performed where all workgroups meet, no cache write-back),
+// and the ticket's operand depends on the value the slot's exchange returns, so a piece is in place before its
+// workgroup counts as finished.  The main kernel cleared the ticket.
+__device__ __forceinline__ void mlp_loss_piece(float piece, float *slots, uint32_t *ticket, float *loss, int lane) {
+    int last = 0;
+    if (lane == 0) {
+        const float before = __uint_as_float(atomicExch((uint32_t *)slots + blockIdx.x, __float_as_uint(piece)));
+        uint32_t one = 1u;
+        asm volatile("" : "+v"(one) : "v"(before));
+        last = atomicAdd(ticket, one) == gridDim.x - 1;
+    }
+    if (!__builtin_amdgcn_readfirstlane(last)) return;
+    float v = 0.f;  // lane j adds slots j, j + 64, ... in order; then the lanes in a fixed tree
+    for (int b = lane; b < (int)gridDim.x; b += 64) v += __uint_as_float(atomicOr((uint32_t *)slots + b, 0u));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if (lane == 0) loss[0] = v;
+}
+
 __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d, const float *__restrict__ part, int n_parts,
-                                                                        const float *__restrict__ aux, float lr, float *loss, float *img) {
+                                                                        const float *__restrict__ aux, float lr, float *loss, float *img,
+                                                                        float *loss_slots, uint32_t *ticket) {
     __shared__ float red[64 * MLP_RG];
     __shared__ uint32_t smx[64 * MLP_RG];
     __shared__ float val[64], bits_in[64], dbits_in[64], new_i[64];
@@ -483,7 +507,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     __builtin_amdgcn_wave_barrier();
     if (loss_block) {
-        if (t == 0 && loss) atomicAdd(loss, val[0]);
+        if (loss) mlp_loss_piece(val[0], loss_slots, ticket, loss, t);
         return;
     }
     const float *colsum = aux + l * MLP_AUX;
@@ -491,6 +515,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
     // d(ebops * beta) / d bits: the chain rule through ((total * par_factor) / n_parallel) * ebops_factor * beta
     const float gs = __fmul_rn(__fdiv_rn(__fmul_rn(beta, h.ebops_factor), h.n_parallel), h.par_factor);
     float reg = 0.f;  // MonoL1 regularisation loss of the trainable bit-width variables (pre-update values)
+    float ebops_term = 0.f;  // role 1, lane 0: the layer's ebops * beta
     if (role == 0) {
         const int e = 64 * j + t;
         if (t < n_mine) {
@@ -524,7 +549,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
             if (h.bias) total += bsum / (float)N * h.bias_size;
             const float e = __fmul_rn(__fdiv_rn(__fmul_rn(total, h.par_factor), h.n_parallel), h.ebops_factor);
             if (h.ebops) h.ebops[0] = (uint32_t)e;
-            if (loss) atomicAdd(loss, e * beta);
+            ebops_term = e * beta;
         }
         if (h.bias && t < N) {
             const KIF p = resolve_kif(v_k, v_i, v_b, true, true);
@@ -552,7 +577,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
     if (loss) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) reg += __shfl_xor(reg, o, 64);
-        if (t == 0 && reg != 0.f) atomicAdd(loss, reg);
+        mlp_loss_piece(ebops_term + reg, loss_slots, ticket, loss, t);
     }
 }
 
@@ -597,7 +622,7 @@ static int mlp_plan(const hgq_mlp_layer *layers, int n_layers, MlpDev &d, size_t
     d.off_rx = off, off += MLP_BM * d.ld_rx;
     d.off_dz0 = off, off += MLP_BM * MLP_LDZ;
     d.off_dz1 = off, off += MLP_BM * MLP_LDZ;
-    d.off_red = off, off += 2 * 64 * HGQ_MLP_MAX_LAYERS;  // fractional-bit sums and abs-max, [layers][64] each
+    d.off_red = off, off += 3 * 64 * HGQ_MLP_MAX_LAYERS;  // fractional-bit sums (two sets) and abs-max, [layers][64] each
     lds_bytes = (size_t)off * 4;
     if (lds_bytes > 160 * 1024 - 512) return fail(HGQ_ERR_UNSUPPORTED, "hgq_mlp: the stack needs %zu bytes of LDS", lds_bytes);
     return HGQ_OK;
@@ -616,7 +641,7 @@ extern "C" int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, 
     MlpDev d;
     size_t lds_bytes;
     if (mlp_plan(layers, n_layers, d, lds_bytes)) return -1;
-    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX + d.off_raw + 4;
+    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX + d.off_raw + 4 + 64;  // (+ 64: slots of tiny stacks)
 }
 
 extern "C" int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
@@ -644,11 +669,15 @@ extern "C" int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_laye
         hipLaunchKernelGGL(mlp_prep_kernel, dim3((d.off_raw + 255) / 256), dim3(256), 0, s, d, img);
         if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
     }
-    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, slices, reduced, loss);
-    if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
+    // behind the snapshot: one loss slot per workgroup of the update pass and their ticket
+    float *loss_slots = reduced + (int64_t)n_layers * MLP_AUX;
     int blocks = 1;
     for (int l = 0; l < n_layers; ++l) blocks += (layers[l].K * layers[l].N + 63) / 64 + 2;
-    hipLaunchKernelGGL(mlp_reduce_update_kernel, dim3(blocks), dim3(64 * MLP_RG), 0, s, d, slices, parts, reduced, lr, loss, img);
+    uint32_t *ticket = (uint32_t *)(loss_slots + blocks);
+    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, slices, reduced, ticket);
+    if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
+    hipLaunchKernelGGL(mlp_reduce_update_kernel, dim3(blocks), dim3(64 * MLP_RG), 0, s, d, slices, parts, reduced, lr, loss, img, loss_slots,
+                       ticket);
     return check_launch("hgq_mlp_train_step(update)");
 }
 

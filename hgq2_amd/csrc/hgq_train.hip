@@ -450,11 +450,13 @@ __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict_
         for (int c = 0; c < C; ++c) se += expf(z[c] - mx);
         const float lse = logf(se);
         const int64_t lab = labels[r];
-        acc += lse - (z[lab] - mx);
+        // a label outside [0, C) (an ignore index, 1-based labels) reads nothing: the loss becomes NaN, the row's gradient zero
+        const bool lab_ok = (uint64_t)lab < (uint64_t)C;
+        acc += lab_ok ? lse - (z[lab_ok ? lab : 0] - mx) : NAN;
         if (dlogits) {
             float *d = dlogits + r * C;
             const float inv = 1.0f / se;
-            for (int c = 0; c < C; ++c) d[c] = (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows;
+            for (int c = 0; c < C; ++c) d[c] = lab_ok ? (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows : 0.0f;
         }
     }
     acc = block_sum_256(acc, red);
@@ -463,11 +465,15 @@ __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict_
             atomicAdd(loss, acc * inv_rows);
             return;
         }
-        // both words are only ever touched by device-scope atomics, which are performed at the memory side: the wait
-        // between the two makes this workgroup's part arrive before it counts as finished (no cache write-back needed)
-        atomicAdd((float *)state, acc * inv_rows);
-        __threadfence_block();
-        if (atomicAdd(state + 1, 1u) == gridDim.x - 1) {
+        // Both words are only ever touched by device-scope atomics, which are performed where all workgroups meet (not
+        // in a cache that would need a write-back).  The ticket is drawn with an operand that depends on the value the
+        // first atomic RETURNS, so it cannot leave this wavefront before this workgroup's part has been added: whoever
+        // draws the last ticket finds every part in the sum.  (A fence of workgroup scope between two non-returning
+        // atomics orders nothing for other workgroups; one of device scope costs a cache write-back, ~2 us here.)
+        const float before = atomicAdd((float *)state, acc * inv_rows);
+        uint32_t one = 1u;
+        asm volatile("" : "+v"(one) : "v"(before));
+        if (atomicAdd(state + 1, one) == gridDim.x - 1) {
             loss[0] = __uint_as_float(atomicExch(state, 0u));  // every other workgroup has added its part
             atomicExch(state + 1, 0u);
         }

@@ -138,6 +138,45 @@ def test_quantizer_fwd_bwd_in_one_launch_ragged_and_shared(dev, n, bw_shape, x_s
         assert float((di - di2).abs().max()) <= RTOL * float(scale) and float((df - df2).abs().max()) <= RTOL * float(scale)
 
 
+@pytest.mark.parametrize('overflow_mode', ['SAT', 'SAT_SYM'])
+@pytest.mark.parametrize('bw_shape', [(600, 24), (1, 24), (1, 1)])
+def test_saturating_training_where_the_word_has_no_bits(dev, overflow_mode, bw_shape):
+    """SAT / SAT_SYM in training with i + f < 0 on most entries (i in -6..0, f in 0..3): this build's definition of the
+    case - the reference's bound formulas applied as they stand, upper bound first, every violated bound taking gradient
+    (tests/test_oracle_pins.py::test_saturating_words_with_negative_total_width_are_defined_by_the_bounds) - values bit
+    for bit and gradients to 1e-5 of the summed |terms|, with bit-widths per element, per column and shared."""
+    from hgq2_amd import _lib, ops
+
+    shape = (600, 24)
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(shape, generator=g) * 0.5)
+    k = torch.randint(0, 2, bw_shape, generator=g).float()
+    i = torch.randint(-6, 1, bw_shape, generator=g).float()
+    f = torch.randint(0, 4, bw_shape, generator=g).float()
+    if i.numel() == 1:
+        i, f = torch.full(bw_shape, -2.0), torch.full(bw_shape, 1.0)
+    assert float(((i + f) < 0).float().mean()) > 0.4
+    gy = torch.randn(shape, generator=g)
+    q = ofp.get_fixed_quantizer('RND', overflow_mode)
+    xs = x.clone().requires_grad_(True)
+    ie, fe = (t.expand(shape).clone().requires_grad_(True) for t in (i, f))   # per-element terms of the oracle
+    want = q(xs, k.expand(shape), ie, fe, True, None)
+    want.backward(gy)
+    hom = tuple(a for a in range(2) if bw_shape[a] == 1)
+    mode = _lib.mode_bits('RND', overflow_mode, training=True)
+    xd = x.to(dev).requires_grad_(True)
+    idv, fd = (t.reshape(-1).to(dev).requires_grad_(True) for t in (i, f))
+    y, _, _ = ops.quantize(xd, k.reshape(-1).to(dev), idv, fd, mode, bw_inner=1)
+    assert torch.equal(y.detach().cpu(), want.detach())
+    y.backward(gy.to(dev))
+    assert torch.equal(xd.grad.cpu(), xs.grad)
+    for got, terms, name in ((idv.grad, ie.grad, 'di'), (fd.grad, fe.grad, 'df')):
+        t64 = terms.double()
+        want_g = t64.sum(dim=hom).reshape(-1) if hom else t64.reshape(-1)
+        scale = t64.abs().sum(dim=hom).reshape(-1) if hom else t64.abs().reshape(-1)
+        _close_scaled(got, want_g, scale, f'{overflow_mode} {bw_shape} {name}')
+
+
 # --------------------------------------------------------------------------------------------------------------
 # the stateless callable, driven as the reference drives it
 # --------------------------------------------------------------------------------------------------------------

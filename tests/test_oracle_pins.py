@@ -144,6 +144,47 @@ def test_clip_bound_gradients_match_finite_differences(overflow_mode):
         assert np.isclose(float(f.grad[n]), df, rtol=1e-5, atol=1e-7)
 
 
+def test_saturating_words_with_negative_total_width_are_defined_by_the_bounds():
+    """SAT / SAT_SYM in training where i + f < 0 (the word has no bits left): whether the third-party callable clamps i
+    against -f cannot be read from the reference tree, so this build DEFINES the case by the reference's own range
+    formulas (fixed_point_quantizer.py:107-116) applied as they stand: hi = 2^i - 2^-f may lie below lo, the upper bound
+    wins the forward value, and every violated bound hands the upstream gradient to its own i / f derivative.  Hand-worked
+    with k = 1, i = -3, f = 2: 2^i = 0.125, 2^-f = 0.25, hi = -0.125; SAT lo = -0.125; SAT_SYM lo = +0.125 (above hi)."""
+    ln2 = math.log(2.0)
+    x = torch.tensor([0.3, -1.0, 0.0, -0.125], requires_grad=True)   # rounds (RND, f = 2) to 0.25, -1, 0, 0
+    g = torch.tensor([1.0, 2.0, -3.0, 0.5])
+
+    def run(mode, k):
+        xs = x.detach().clone().requires_grad_(True)
+        i = torch.full((4,), -3.0, requires_grad=True)
+        f = torch.full((4,), 2.0, requires_grad=True)
+        y = fp.get_fixed_quantizer('RND', mode)(xs, torch.full((4,), float(k)), i, f, True, None)
+        y.backward(g)
+        return y.detach().tolist(), xs.grad.tolist(), i.grad.tolist(), f.grad.tolist()
+
+    # SAT, k = 1: hi = lo = -0.125.  0.25 and 0 are above hi (upper bound, d/di = ln2 2^i, d/df = ln2 2^-f); -1 is below
+    # lo (lower bound -2^i: d/di = -ln2 2^i, d/df = 0); nothing passes, so d/dx = 0 everywhere
+    y, dx, di, df = run('SAT', 1)
+    assert y == [-0.125] * 4 and dx == [0.0] * 4
+    assert di == pytest.approx([ln2 * 0.125 * 1.0, -ln2 * 0.125 * 2.0, ln2 * 0.125 * -3.0, ln2 * 0.125 * 0.5], rel=1e-6)
+    assert df == pytest.approx([ln2 * 0.25 * 1.0, 0.0, ln2 * 0.25 * -3.0, ln2 * 0.25 * 0.5], rel=1e-6)
+    # SAT, k = 0: lo = 0.  -1 is below lo and not above hi: value 0, no bit-width gradient (lo does not depend on i, f)
+    y, dx, di, df = run('SAT', 0)
+    assert y == [-0.125, 0.0, -0.125, -0.125] and dx == [0.0] * 4
+    assert di == pytest.approx([ln2 * 0.125, 0.0, ln2 * 0.125 * -3.0, ln2 * 0.125 * 0.5], rel=1e-6)
+    # SAT_SYM, k = 1: lo = -hi = +0.125 > hi.  0.25 is above hi only; -1 below lo only (value lo = +0.125, d lo = -d hi);
+    # 0 violates both: the upper bound wins the value and the two bound gradients cancel exactly
+    y, dx, di, df = run('SAT_SYM', 1)
+    assert y == [-0.125, 0.125, -0.125, -0.125] and dx == [0.0] * 4
+    assert di == pytest.approx([ln2 * 0.125, -ln2 * 0.125 * 2.0, 0.0, 0.0], abs=1e-9)
+    assert df == pytest.approx([ln2 * 0.25, -ln2 * 0.25 * 2.0, 0.0, 0.0], abs=1e-9)
+    # bit-widths shared by the four elements: autograd of the broadcast adds the per-element terms
+    i1, f1 = torch.tensor([-3.0], requires_grad=True), torch.tensor([2.0], requires_grad=True)
+    fp.get_fixed_quantizer('RND', 'SAT')(x.detach(), torch.ones(4), i1.expand(4), f1.expand(4), True, None).backward(g)
+    assert float(i1.grad) == pytest.approx(ln2 * 0.125 * (1.0 - 2.0 - 3.0 + 0.5), rel=1e-6)
+    assert float(f1.grad) == pytest.approx(ln2 * 0.25 * (1.0 - 3.0 + 0.5), rel=1e-6)
+
+
 def test_ebops_known_answers_at_construction():
     """Closed form dense.py:70-80 with the default bit-widths (8 everywhere):
     in*out*64 + 8*out for the four layers of the 16-64-32-32-5 MLP."""
