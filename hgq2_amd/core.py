@@ -164,6 +164,23 @@ class TreeCache:
     __slots__ = ('key', 'layers', 'quantized', 'regularised')
 
 
+def _structure_changed(*_):
+    TREE_EPOCH[0] += 1
+
+
+# any module or parameter registered anywhere (an `nn.ModuleList.append` inside a custom layer, `register_parameter`)
+# ends the validity of the cached lists; what these hooks cannot see - a regularizer attached to an existing parameter
+# after the first step - needs `invalidate_tree_caches()`
+torch.nn.modules.module.register_module_module_registration_hook(_structure_changed)
+torch.nn.modules.module.register_module_parameter_registration_hook(_structure_changed)
+
+
+def invalidate_tree_caches():
+    """Call after changing a model in a way no registration shows: attaching or removing ``regularizer`` / ``constraint``
+    attributes of existing parameters."""
+    TREE_EPOCH[0] += 1
+
+
 def tree_cache(root) -> TreeCache:
     """Lists of a module tree that a training step needs: its layers, the layers that declare kernel / bias quantizers,
     the trainable variables with a regularizer."""

@@ -10,6 +10,7 @@ raises.
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import Sequence
 
 import torch
@@ -34,6 +35,28 @@ def _need(cond: bool, msg: str):
 
 
 _F32 = torch.float32
+
+
+# The queues and flags further down (deferred launches, the second stream's branch, the gradient sink) belong to the
+# ONE training step that is running: they are process-wide on purpose, because the backward functions that read them run
+# on the autograd engine's device thread, not on the thread that opened them.  Two Python threads driving model calls at
+# the same time would mix their queues, so the second one is refused loudly.
+_STEP_OWNER = {'thread': None, 'depth': 0}
+
+
+def _claim_step(what: str):
+    me = threading.get_ident()
+    if _STEP_OWNER['depth'] and _STEP_OWNER['thread'] != me:
+        raise RuntimeError(f'{what}: another thread is inside a model call or training step of this package; its launch queues '
+                           'are process-wide (the autograd engine reads them from its own thread), so steps must not overlap')
+    _STEP_OWNER['thread'] = me
+    _STEP_OWNER['depth'] += 1
+
+
+def _release_step():
+    _STEP_OWNER['depth'] -= 1
+    if _STEP_OWNER['depth'] <= 0:
+        _STEP_OWNER['depth'], _STEP_OWNER['thread'] = 0, None
 
 
 def _check_f32(name: str, t: Tensor):
@@ -477,13 +500,17 @@ class overlap_ebops:
     returns a total whose value is there once the context is left (its gradient does not need the value)."""
 
     def __enter__(self):
+        _claim_step('overlap_ebops')
         _OVERLAP['depth'] += 1
         return self
 
     def __exit__(self, *exc):
         _OVERLAP['depth'] -= 1
-        if _OVERLAP['depth'] == 0:
-            join_side()
+        try:
+            if _OVERLAP['depth'] == 0:
+                join_side()
+        finally:
+            _release_step()
         return False
 
 
@@ -548,19 +575,23 @@ _DEFER = {'depth': 0, 'dense_ebops': [], 'tracks': [], 'late': []}
 
 
 def begin_deferred():
+    _claim_step('model call')
     _DEFER['depth'] += 1
 
 
 def end_deferred(discard: bool = False):
     _DEFER['depth'] -= 1
-    if _DEFER['depth'] == 0:
-        if discard:
-            _DEFER['dense_ebops'], _DEFER['tracks'], _DEFER['late'] = [], [], []
-        elif _OVERLAP['depth'] and _worth_a_branch():
-            with side_branch():
+    try:
+        if _DEFER['depth'] == 0:
+            if discard:
+                _DEFER['dense_ebops'], _DEFER['tracks'], _DEFER['late'] = [], [], []
+            elif _OVERLAP['depth'] and _worth_a_branch():
+                with side_branch():
+                    flush_deferred()
+            else:
                 flush_deferred()
-        else:
-            flush_deferred()
+    finally:
+        _release_step()
 
 
 def _rounds(keys):
@@ -1987,7 +2018,7 @@ class _DenseEbops(torch.autograd.Function):
                 pieces.append((o_i, g[:n_f]))
             if n_b:
                 pieces.append((o_b, g[n_f + n_k:]))
-            if all(o is not None for o, _ in pieces):
+            if all(_parkable(o) for o, _ in pieces):
                 for o, piece in pieces:
                     _stash_side(o, up, piece)
                 return (None,) * 20
@@ -2441,7 +2472,7 @@ class _BitsEbops(torch.autograd.Function):
                 pieces.append((o_fb, buf[of:of + n]))
                 if not kbi and (o_i is None or o_i.requires_grad):  # an unknown owner makes the whole call fall back
                     pieces.append((o_i, buf[oi:oi + n]))
-            if all(o is not None for o, _ in pieces):
+            if all(_parkable(o) for o, _ in pieces):
                 for o, piece in pieces:
                     _stash_side(o, g, piece)
                 return (None,) * n_args
@@ -2726,27 +2757,49 @@ def sgd_update_multi_(ws, gs, l1, lo, hi, lr, sides=None, sum_terms=None, sum_ou
 # each would cost a multiplication by the upstream gradient and an addition to the variable's other gradient, one
 # library launch each): it leaves ``(upstream gradient, unit-upstream gradient)`` on the variable, and the optimizer's
 # update kernel adds the pieces while it reads them.  Only an optimizer that consumes ``_hgq_side`` may open the sink.
-_SINK = {'open': False, 'unit_ptr': 0}
+_SINK = {'open': False, 'unit_ptr': 0, 'owners': None}
 
 
 class side_gradients:
     """Context manager around ``loss.backward(root)``: opens the sink; ``root`` is the gradient the caller seeds the
-    backward pass with when that gradient is exactly one (its address identifies "the upstream gradient is 1")."""
+    backward pass with when that gradient is exactly one (its address identifies "the upstream gradient is 1").
+    ``owners``: the variables whose pieces the opening optimizer will consume (``id`` values); a piece for any other
+    variable - one that another optimizer steps, or none - goes back to autograd instead of being parked where nobody
+    reads it.  ``None`` accepts every variable."""
 
-    def __init__(self, unit_root: Tensor | None = None):
+    def __init__(self, unit_root: Tensor | None = None, owners=None):
         self.unit_ptr = unit_root.data_ptr() if unit_root is not None else 0
+        self.owners = owners
 
     def __enter__(self):
+        _claim_step('side_gradients')
         self.prev = dict(_SINK)
-        _SINK['open'], _SINK['unit_ptr'] = True, self.unit_ptr
+        _SINK['open'], _SINK['unit_ptr'], _SINK['owners'] = True, self.unit_ptr, self.owners
         return self
 
     def __exit__(self, *exc):
-        if exc[0] is None:
-            flush_reductions()
-        else:
-            _PENDING_REDUCE.clear()
-        _SINK.update(self.prev)
+        try:
+            if exc[0] is None:
+                flush_reductions()
+            else:
+                _PENDING_REDUCE.clear()
+        finally:
+            _SINK.update(self.prev)
+            _release_step()
+
+
+def _parkable(owner) -> bool:
+    """A gradient piece for ``owner`` may be left with :func:`_stash_side`: the open sink's optimizer consumes it, or the
+    variable is frozen and needs none.  (A trainable variable of another optimizer makes the caller fall back to autograd.)"""
+    return owner is not None and (_sink_takes(owner) or not getattr(owner, 'requires_grad', False))
+
+
+def _sink_takes(owner) -> bool:
+    """The sink is open and ``owner`` is a trainable variable of the optimizer that opened it."""
+    if owner is None or not _SINK['open'] or not getattr(owner, 'requires_grad', False):
+        return False
+    owners = _SINK['owners']
+    return owners is None or id(owner) in owners
 
 
 def _is_unit(g: Tensor) -> bool:
@@ -2757,7 +2810,7 @@ def _is_unit(g: Tensor) -> bool:
 def _stash_side(owner, up, piece: Tensor) -> bool:
     """Leave ``up * piece`` (``up`` None: the piece as it is) on ``owner`` for the optimizer; False when the sink is
     closed or the owner is unknown."""
-    if not _SINK['open'] or owner is None or not getattr(owner, 'requires_grad', False):
+    if not _sink_takes(owner):
         return False
     if not hasattr(owner, '_hgq_side') or owner._hgq_side is None:
         owner._hgq_side = []
@@ -2775,14 +2828,13 @@ def _owner(t):
 
 def _can_route(owner, numel) -> bool:
     """``_route`` would leave a gradient of ``numel`` elements on ``owner`` rather than hand it back."""
-    return (owner is not None and _SINK['open'] and owner.requires_grad and numel == owner.numel()
-            and len(getattr(owner, '_hgq_side', None) or ()) < SGD_SIDES)
+    return _sink_takes(owner) and numel == owner.numel() and len(getattr(owner, '_hgq_side', None) or ()) < SGD_SIDES
 
 
 def _route(owner, grad):
     """A finished gradient of a variable that also receives gradient from elsewhere: with the sink open it is left on
     the variable (returns None, so autograd has nothing to accumulate), otherwise handed back."""
-    if grad is None or owner is None or not _SINK['open'] or not owner.requires_grad or grad.numel() != owner.numel():
+    if grad is None or not _sink_takes(owner) or grad.numel() != owner.numel():
         return grad
     if len(getattr(owner, '_hgq_side', None) or ()) >= SGD_SIDES:
         return grad  # no room left in the update kernel's descriptor: autograd accumulates this one

@@ -46,7 +46,7 @@ class Quantizer(Layer):
         if self.scaler is not None:
             # the divisor goes in as a tensor: on the GPU torch divides by a Python number with a multiplication by its
             # rounded reciprocal, one ulp away from the quotient for some inputs (and one quantization step after rounding)
-            key = (inputs.device, inputs.dtype)
+            key = (inputs.device, inputs.dtype, float(self.scaler))
             cached = getattr(self, '_scaler_tensor', None)
             if cached is None or cached[0] != key:
                 cached = (key, torch.full((), float(self.scaler), dtype=inputs.dtype, device=inputs.device))

@@ -71,6 +71,7 @@ class SGD:
 
     def __init__(self, params, lr: float = 0.01, fold_regularizers: bool = False):
         self.params = [p for p in params if p.requires_grad]
+        self._owner_ids = frozenset(id(p) for p in self.params)  # the variables whose parked gradient pieces `step` consumes
         self.lr = float(lr)
         self.fold_regularizers = fold_regularizers
         self._unit = None
@@ -93,7 +94,7 @@ class SGD:
         if self._unit is None or self._unit.device != loss.device or self._unit.shape != loss.shape:
             self._unit = torch.ones_like(loss)  # the seed gradient: allocated once, also outside a captured graph
         terms = getattr(loss, '_hgq_terms', None)
-        with ops.side_gradients(self._unit):
+        with ops.side_gradients(self._unit, self._owner_ids):
             if terms is not None:  # `model_loss` inside `ops.overlap_ebops()`: the sum is a plain value, its terms carry the graph
                 torch.autograd.backward(terms, [self._unit.reshape(t.shape) for t in terms])
             else:

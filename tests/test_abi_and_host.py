@@ -180,6 +180,35 @@ def test_entry_points_validate_arguments_before_any_launch():
     assert lib.hgq_col_moments_fwd(none, 0, 64, none, none, none, none) == ARG
 
 
+def test_a_second_thread_inside_a_training_step_is_refused():
+    """The launch queues of a step are process-wide (the autograd engine's thread reads them): a second Python thread that
+    opens a step while one is open gets an error instead of another step's queue."""
+    import threading
+
+    from hgq2_amd import ops
+
+    seen = []
+
+    def other():
+        try:
+            with ops.side_gradients(None):
+                seen.append('entered')
+        except RuntimeError as e:
+            seen.append(str(e))
+
+    with ops.side_gradients(None):
+        t = threading.Thread(target=other)
+        t.start()
+        t.join()
+        with ops.side_gradients(None):  # the same thread may nest
+            pass
+    assert len(seen) == 1 and 'another thread' in seen[0]
+    t = threading.Thread(target=other)  # and once the step is over another thread may run one
+    t.start()
+    t.join()
+    assert seen[1] == 'entered'
+
+
 def test_beta_controllers_and_ebops_logging():
     """Host-side hooks of reference src/hgq/utils/sugar/{ebops,beta_scheduler,beta_pid}.py on layers built on the CPU
     (no kernel is launched: the hooks only read `_ebops` and assign `_beta`)."""

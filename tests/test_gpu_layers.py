@@ -177,6 +177,44 @@ def test_fused_qdense_stack_step_matches_oracle(dev, acc64, batch, dims):
             _close(pl.bq.quantizer._i, rl.bq.quantizer._i, scale=rl.bq.quantizer._i.detach().abs() + 1e-3, what=f'bq._i {n}')
 
 
+def test_gradient_pieces_of_variables_the_optimizer_does_not_own_go_through_autograd(dev):
+    """``SGD.backward`` parks EBOPs gradient pieces on the variables for its own update kernel.  A variable that this
+    optimizer does not step (here: every bit-width variable) must get its whole gradient in ``.grad`` instead - the same
+    values a plain ``loss.backward()`` gives."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, model_loss
+    from hgq2_amd.utils.models import qdense_mlp
+
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(512, 16, generator=g).to(dev)
+    y = torch.randint(0, 5, (512,), generator=g).to(dev)
+    model = qdense_mlp(device=dev)
+    _copy_mlp(ref.RefMLP(seed=6), model, dev)
+    model(x, training=True)
+    named = dict(model.named_parameters())
+    weights = [p for n, p in named.items() if n.endswith('_kernel') or n.endswith('bias')]
+    others = {n: p for n, p in named.items() if p.requires_grad and all(p is not w for w in weights)}
+    assert weights and others
+    state = {n: t.detach().clone() for n, t in model.state_dict().items()}
+
+    def grads(sink):
+        model.load_state_dict(state)
+        for p in named.values():
+            p.grad = None
+            p._hgq_side = None
+        loss = model_loss(model, ops.sparse_ce(model(x, training=True), y))
+        if sink:
+            SGD(weights, lr=0.01).backward(loss)
+        else:
+            loss.backward()
+        return {n: p.grad.detach().clone() for n, p in others.items()}
+
+    plain, with_sink = grads(False), grads(True)
+    for n in others:
+        assert not getattr(others[n], '_hgq_side', None), f'{n}: a piece was parked where no optimizer reads it'
+        assert torch.equal(plain[n], with_sink[n]), n
+
+
 def test_fused_qdense_stack_step_is_the_same_bits_on_every_run(dev):
     """131 072 rows = eight tiles per workgroup: a workgroup's gradient sums run over several tiles and the loss is put
     together from the pieces of ~80 workgroups.  No floating-point sum of the two launches depends on the order in which
