@@ -43,6 +43,12 @@ def _cpu_threads():
     return max(1, min(allowed, share) if share > 0 else allowed)
 
 
+def _lib_bf16_parts():
+    from hgq2_amd import _lib
+
+    return bool(_lib.load().hgq_dense_use_bf16_parts(-1))
+
+
 def _events_ms(fn, iters):
     import torch
 
@@ -526,6 +532,12 @@ def main():
                                'kif WRAP datalanes, EBOPs beta0=1e-5, sparse CE, one fwd+bwd+SGD step; path = ' + args.path
                                + ': ' + labels_of[args.path]},
         'final_loss': float(loss),
+        # which matrix instruction the contractions issued (results are the fp32 contraction either way: fp32 operands are
+        # split exactly into bf16 parts, products exact in fp32, fp32 accumulation)
+        'matrix_instruction': ('v_mfma_f32_32x32x16_bf16 on exact bf16 parts of the fp32 operands'
+                               if _lib_bf16_parts() else 'v_mfma_f32_32x32x2_f32'),
+        'batch_reuse': 'the same resident batch (1.1 MB) is fed every step: the step is latency-bound, its 6 MB working set '
+                       'is served from cache',
     }
     if not args.no_extras:
         # every way the same step can be driven, each on a fresh model, over a few hundred steps

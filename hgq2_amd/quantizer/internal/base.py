@@ -7,6 +7,8 @@ Mirrors reference src/hgq/quantizer/internal/base.py: ``round_conv`` (:19-28),
 
 from __future__ import annotations
 
+import functools
+import math
 from collections.abc import Sequence
 
 import numpy as np
@@ -112,9 +114,13 @@ def bw_layout(bw_shape, x_shape):
     """``(bw_size, bw_inner)`` such that element ``e`` of a contiguous tensor of ``x_shape`` uses
     bit-width entry ``(e // bw_inner) % bw_size`` of a contiguous tensor of ``bw_shape``, or
     ``None`` if the broadcast pattern is not of that form."""
-    bw_shape, x_shape = tuple(bw_shape), tuple(x_shape)
+    return _bw_layout(tuple(bw_shape), tuple(x_shape))
+
+
+@functools.lru_cache(maxsize=4096)
+def _bw_layout(bw_shape, x_shape):  # asked two dozen times per training step with the same few shape pairs
     if len(bw_shape) != len(x_shape):
-        if int(np.prod(bw_shape)) == 1:
+        if math.prod(bw_shape) == 1:
             return 1, 1
         return None
     het = [a for a, (b, s) in enumerate(zip(bw_shape, x_shape)) if b != 1 or s == 1]
@@ -125,7 +131,7 @@ def bw_layout(bw_shape, x_shape):
     for a in range(first, last + 1):
         if bw_shape[a] != x_shape[a]:
             return None
-    return int(np.prod(x_shape[first:last + 1])), int(np.prod(x_shape[last + 1:]))
+    return math.prod(x_shape[first:last + 1]), math.prod(x_shape[last + 1:])
 
 
 class TrainableQuantizerBase(Layer):

@@ -15,7 +15,11 @@
  *   - outputs that are reductions (bit-width gradients, abs-max trackers) are cleared by the
  *     entry point itself with a fill kernel (safe under HIP graph capture), then accumulated;
  *   - bit-width operands (k, i, f or b) must hold integer-valued floats after the optional
- *     rounding selected by HGQ_MODE_ROUND_PARAMS; powers of two are formed exactly from them.
+ *     rounding selected by HGQ_MODE_ROUND_PARAMS; powers of two are formed exactly from them;
+ *   - the entry points keep no state between calls, with two exceptions that are named where they are declared:
+ *     hgq_dense_use_bf16_parts (ONE process-wide switch: which matrix instruction the contractions issue; it
+ *     changes instruction selection only, results stay the fp32 contraction) and the per-GPU scratch array of
+ *     hgq_quantize_bwd_static.
  *
  * Bit-width broadcasting: element `e` of a tensor with `n` elements uses bit-width entry
  * `(e / bw_inner) % bw_size`.  bw_size == n, bw_inner == 1 is the per-element case;
