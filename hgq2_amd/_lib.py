@@ -108,11 +108,11 @@ SIGNATURES = {
     'hgq_qsoftmax_bwd': (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int64, c_float, c_float] + [c_void_p] * 5
                          + [c_void_p] * 4 + [c_void_p]),
     'hgq_qattention_fwd': (c_int, [c_void_p] * 4 + [c_int] * 5 + [c_int64, c_float, c_float] + [c_void_p] * 5 + [c_void_p] * 3
-                           + [c_void_p, c_void_p]),
+                           + [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     'hgq_qattention_fwd_workspace': (c_int64, [c_int] * 5 + [c_int64, c_int]),
     'hgq_qattention_bwd_workspace': (c_int64, [c_int] * 5 + [c_int64, c_int]),
     'hgq_qattention_bwd': (c_int, [c_void_p] * 7 + [c_int] * 5 + [c_int64, c_float, c_float] + [c_void_p] * 5 + [c_void_p] * 4
-                           + [c_void_p]),
+                           + [c_void_p, c_int, c_int, c_void_p]),
     'hgq_attn_scores_fwd': (c_int, [c_void_p] * 3 + [c_int] * 5 + [c_void_p]),
     'hgq_attn_scores_bwd': (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_void_p]),
     'hgq_attn_combine_fwd': (c_int, [c_void_p] * 3 + [c_int] * 5 + [c_void_p]),

@@ -207,6 +207,43 @@ __device__ __forceinline__ void spill_tiles(float *buf, const floatx16 (&acc)[ST
         }
 }
 
+// ---- attention masks (reference src/hgq/layers/softmax.py:118-127: scores <- mask * scores - (1 - mask) * 1e9 ahead of
+// the maximum, exp <- mask * exp behind the table).  A lane keeps one bit per score it owns: bit r of keep[st] is
+// clear where (query t, key qa_row(st, r, hf)) is masked out - by the boolean mask [mask_batch, T, S] (one byte per
+// entry, 0 = masked; four consecutive keys per 32-bit load) and / or by the causal rule key <= query.
+#define QA_MASKED (-1e9f)
+struct QAttnMask {
+    const uint8_t *mask;  // null: no boolean mask
+    int mask_batch;       // 1: the same mask for every batch element, else B
+    int causal;
+};
+
+template <int ST>
+__device__ __forceinline__ void load_keep(const QAttnMask &mk, int b, int T, int S, int t, int hf, uint32_t (&keep)[ST]) {
+#pragma unroll
+    for (int st = 0; st < ST; ++st) keep[st] = 0xffffu;
+    if (mk.mask) {
+        const uint8_t *row = mk.mask + ((int64_t)(mk.mask_batch > 1 ? b : 0) * T + t) * S;
+        uint32_t w[ST][4];
+#pragma unroll
+        for (int st = 0; st < ST; ++st)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) w[st][g] = *(const uint32_t *)(row + st * 32 + 8 * g + 4 * hf);
+#pragma unroll
+        for (int st = 0; st < ST; ++st)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (((w[st][r >> 2] >> (8 * (r & 3))) & 0xffu) == 0) keep[st] &= ~(1u << r);
+    }
+    if (mk.causal) {
+#pragma unroll
+        for (int st = 0; st < ST; ++st)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (qa_row(st, r, hf) > t) keep[st] &= ~(1u << r);
+    }
+}
+
 // ---- the exp stage.  The walk keeps only what turns d = max - x into a table code (ExpCode); the
 // table holds the rest.  Arguments the table does not cover - codes beyond SM_TABLE, an exp input
 // quantizer with an empty range - are rare and go through out-of-line functions that rebuild the
@@ -333,12 +370,13 @@ __device__ __forceinline__ void load_oq_entries(const hgq_qdesc &d, int64_t row,
 
 // OQ_PLAIN: training mode and an output quantizer that only rounds (or none): its fractional bits are
 // packed four to a register; otherwise (k, i, f) take a register per element.
-template <int HD, int TH, int ST, bool TRAIN, bool OQ_PLAIN>
+template <int HD, int TH, int ST, bool TRAIN, bool OQ_PLAIN, bool MASKED>
 __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restrict__ q, const float *__restrict__ k,
                                                           const float *__restrict__ v, float *__restrict__ out, QAttnPlan pl,
                                                           float scale, float eps, hgq_qdesc d1, hgq_qdesc d2, hgq_qdesc d3,
                                                           hgq_qdesc d4, hgq_qdesc dq, uint32_t *amax1, uint32_t *amax3,
-                                                          uint32_t *__restrict__ amax_slices, uint32_t *__restrict__ pair_slices) {
+                                                          uint32_t *__restrict__ amax_slices, uint32_t *__restrict__ pair_slices,
+                                                          QAttnMask mk) {
     static_assert(TRAIN || !OQ_PLAIN, "the packed form is for training mode");
     extern __shared__ __align__(16) float lds[];
     constexpr int T = 32 * TH, S = 32 * ST, NPO = OQ_PLAIN ? 4 : 16;
@@ -413,15 +451,42 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
         for (int st = 0; st < ST; ++st)
 #pragma unroll
             for (int j = 0; j < NPO; ++j) asm volatile("" : "+v"(po[st][j]));
+        uint32_t keep[ST];
+        if (MASKED) load_keep<ST>(mk, b, T, S, t0 + t_l, hf, keep);  // (its loads travel with the contraction below)
         floatx16 acc[ST];
         score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, acc, pl.bf != 0);
+        if (MASKED) {
+#pragma unroll
+            for (int st = 0; st < ST; ++st)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[st][r] = ((keep[st] >> r) & 1u) ? acc[st][r] : QA_MASKED;
+        }
         float mx = acc[0][0];
 #pragma unroll
         for (int st = 0; st < ST; ++st)
 #pragma unroll
             for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc[st][r]);
         mx = fmaxf(mx, xor32(mx));
-        if (TRAIN) {
+        if (TRAIN && MASKED) {
+            // a masked score sits 1e9 below the maximum, far outside the table: it takes the table's place of the maximum
+            // (code 0) and its exp is replaced by zero; what the exp input quantizer makes of it only matters to its tracker
+            bool any_masked = false;
+#pragma unroll
+            for (int st = 0; st < ST; ++st) {
+                floatx16 xm;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) xm[r] = ((keep[st] >> r) & 1u) ? acc[st][r] : mx;
+                exp_tile(tab_e, 1, ec, d1, d2, scale, mx, xm, cmax, m1);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[st][r] = ((keep[st] >> r) & 1u) ? xm[r] : 0.f;
+                any_masked |= keep[st] != 0xffffu;
+            }
+            if (amax1 && any_masked && mx > QA_MASKED) {
+                float a, e;
+                exp_direct(d1, d2, scale, __fsub_rn(mx, QA_MASKED), &a, &e);
+                m1 = max(m1, abs_bits(a));
+            }
+        } else if (TRAIN) {
 #pragma unroll
             for (int st = 0; st < ST; ++st) exp_tile(tab_e, 1, ec, d1, d2, scale, mx, acc[st], cmax, m1);
         } else {
@@ -434,6 +499,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_fwd_kernel(const float *__restric
                     const float a = q1.fwd<false>(__fsub_rn(mx, acc[st][r]));
                     m1 = max(m1, abs_bits(a));
                     acc[st][r] = q2.fwd<false>(ExpTable::t_of(a, scale));
+                    if (MASKED && !((keep[st] >> r) & 1u)) acc[st][r] = 0.f;
                     if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
                 }
         }
@@ -596,12 +662,13 @@ __global__ __launch_bounds__(1024) void qattn_amax_reduce_kernel(const uint32_t 
 // ([n_wg, 8] shared-quantizer sums | [n_wg, N * T * S] d/df of the output quantizer).  The output
 // quantizer, if present, wraps (only rounds in training): its input gradient is the identity and
 // only its fractional bits take gradient; they are packed four to a register.
-template <int HD, int TH, int ST>
+template <int HD, int TH, int ST, bool MASKED>
 __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restrict__ dout, const float *__restrict__ q,
                                                           const float *__restrict__ k, const float *__restrict__ v,
                                                           float *__restrict__ dq_, float *__restrict__ dk_, float *__restrict__ dv_,
                                                           QAttnPlan pl, float scale, float eps, hgq_qdesc d1, hgq_qdesc d2,
-                                                          hgq_qdesc d3, hgq_qdesc d4, hgq_qdesc dq, float *__restrict__ ws) {
+                                                          hgq_qdesc d3, hgq_qdesc d4, hgq_qdesc dq, float *__restrict__ ws,
+                                                          QAttnMask mk) {
     extern __shared__ __align__(16) float lds[];
     constexpr int T = 32 * TH, S = 32 * ST, NW = QA_NT / 64;
     float *Qs = lds, *Ks = Qs + (T + 1) * QA_LD, *Vs = Ks + (S + 1) * QA_LD, *Gs = Vs + (S + 1) * QA_LD;
@@ -680,9 +747,21 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
         for (int st = 0; st < ST; ++st)
 #pragma unroll
             for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(pf[st][g]));
+        uint32_t keep[ST];
+        if (MASKED) {
+#pragma unroll
+            for (int st = 0; st < ST; ++st) keep[st] = 0xffffu;
+        }
         if (active) {
+            if (MASKED) load_keep<ST>(mk, b, T, S, t0 + t_l, hf, keep);
             score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, xs, pl.bf != 0);        // scores, transposed
             score_tiles<HD, ST, true>(Vs, Gs, t0, col0, t_l, hf, ga, pl.bf != 0);  // d probs = dout value^T, transposed
+            if (MASKED) {
+#pragma unroll
+                for (int st = 0; st < ST; ++st)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) xs[st][r] = ((keep[st] >> r) & 1u) ? xs[st][r] : QA_MASKED;
+            }
             // ---- forward chain: e of every element (kept in the wavefront's buffer), row sum, inverse stage
             mx = xs[0][0];
 #pragma unroll
@@ -697,7 +776,15 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
                 for (int st = 0; st < ST; ++st) {
                     floatx16 ev = xs[st];
+                    if (MASKED) {  // masked scores take the maximum's place in the table and give no exp (see the forward kernel)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) ev[r] = ((keep[st] >> r) & 1u) ? ev[r] : mx;
+                    }
                     exp_tile(tab_e, 1, ec, d1, d2, scale, mx, ev, cmax, m1);
+                    if (MASKED) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) ev[r] = ((keep[st] >> r) & 1u) ? ev[r] : 0.f;
+                    }
 #pragma unroll
                     for (int r = 0; r < 16; ++r) s += ev[r];
                     spill_tile(my_buf, st, ev, t_l, hf);  // e waits in the buffer where its prob will go
@@ -750,7 +837,12 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
             for (int st = 0; st < ST; ++st) {
                 float raw[16], cl[16];
-                const bool slow = tile_codes(xs[st], mx, ec, raw, cl);
+                floatx16 xm = xs[st];  // masked entries: the maximum's code, and no gradient (their exp was multiplied by zero)
+                if (MASKED) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) xm[r] = ((keep[st] >> r) & 1u) ? xm[r] : mx;
+                }
+                const bool slow = tile_codes(xm, mx, ec, raw, cl);
 #pragma unroll
                 for (int r0_ = 0; r0_ < 16; r0_ += 4) {
                     if (!slow) {
@@ -760,8 +852,8 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             const int r = r0_ + j;
-                            const float d = __fsub_rn(mx, xs[st][r]);
-                            const float de = ga[st][r] * rr + ds;
+                            const float d = __fsub_rn(mx, xm[r]);
+                            const float de = (!MASKED || ((keep[st] >> r) & 1u)) ? ga[st][r] * rr + ds : 0.f;
                             float dd, gi1, gf1;
                             ec.grad_q1(d, raw[r], en[j].ca * de, dd, gi1, gf1);
                             gs[2] += en[j].ci * de, gs[3] += en[j].cf * de, gs[0] += gi1, gs[1] += gf1;
@@ -773,7 +865,8 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
                         for (int j = 0; j < 4; ++j) {
                             const int r = r0_ + j;
                             float dd, g4[4];
-                            exp_direct_grad(d1, d2, scale, __fsub_rn(mx, xs[st][r]), ga[st][r] * rr + ds, &dd, g4);
+                            exp_direct_grad(d1, d2, scale, __fsub_rn(mx, xm[r]),
+                                            (!MASKED || ((keep[st] >> r) & 1u)) ? ga[st][r] * rr + ds : 0.f, &dd, g4);
                             gs[0] += g4[0], gs[1] += g4[1], gs[2] += g4[2], gs[3] += g4[3];
                             dm += dd;
                             ga[st][r] = dd;
@@ -789,7 +882,10 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
             for (int st = 0; st < ST; ++st)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) ga[st][r] = (xs[st][r] == mx) ? share - ga[st][r] : -ga[st][r];
+                for (int r = 0; r < 16; ++r) {
+                    ga[st][r] = (xs[st][r] == mx) ? share - ga[st][r] : -ga[st][r];
+                    if (MASKED && !((keep[st] >> r) & 1u)) ga[st][r] = 0.f;  // d (mask * scores - ...) / d scores
+                }
         }
         {
             // the next element's operands: issued here, after the register-hungry stages, some eighty MFMAs ahead of their use
@@ -885,6 +981,13 @@ static int raise_lds(K kernel, size_t bytes, const char *who) {
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
 
+static int check_mask(const uint8_t *mask, int mask_batch, int B, const char *who) {
+    if (!mask) return HGQ_OK;
+    if (mask_batch != 1 && mask_batch != B) return fail(HGQ_ERR_ARG, "%s: mask_batch must be 1 or the batch size, got %d", who, mask_batch);
+    if ((uintptr_t)mask & 3u) return fail(HGQ_ERR_ARG, "%s: the mask must be 4-byte aligned", who);
+    return HGQ_OK;
+}
+
 }  // namespace hgq
 
 using namespace hgq;
@@ -906,12 +1009,16 @@ using namespace hgq;
 extern "C" int hgq_qattention_fwd(const float *query, const float *key, const float *value, float *out, int B, int T, int S,
                                   int N, int H, int64_t bw_rows, float input_scaler, float eps, const hgq_qdesc *exp_iq,
                                   const hgq_qdesc *exp_oq, const hgq_qdesc *inv_iq, const hgq_qdesc *inv_oq, const hgq_qdesc *oq,
-                                  uint32_t *amax_exp_iq, uint32_t *amax_inv_iq, uint32_t *amax_oq, void *workspace, void *stream) {
+                                  uint32_t *amax_exp_iq, uint32_t *amax_inv_iq, uint32_t *amax_oq, void *workspace,
+                                  const uint8_t *mask, int mask_batch, int causal, void *stream) {
     hipStream_t s = (hipStream_t)stream;
     const bool has_oq = oq && oq->k;
     QAttnPlan pl;
     int rc = plan_qattn(B, T, S, N, H, bw_rows, has_oq, pl, "hgq_qattention_fwd");
     if (rc) return rc;
+    if ((rc = check_mask(mask, mask_batch, B, "hgq_qattention_fwd"))) return rc;
+    const QAttnMask mk = {mask, mask_batch, causal != 0};
+    const bool masked = mask || causal;
     if (!softmax_desc_ok(exp_iq) || !softmax_desc_ok(exp_oq) || !softmax_desc_ok(inv_iq) || !softmax_desc_ok(inv_oq) || !softmax_desc_ok(oq))
         return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: a quantizer descriptor has k but not i / fb");
     if (amax_oq && !has_oq) return fail(HGQ_ERR_ARG, "hgq_qattention_fwd: amax_oq without an output quantizer");
@@ -932,16 +1039,21 @@ extern "C" int hgq_qattention_fwd(const float *query, const float *key, const fl
     for (const hgq_qdesc *d : all)
         if (d && d->k && !(d->mode & HGQ_MODE_TRAINING)) train = false;
     const size_t lds = qattn_lds_bytes(T, S, false);
-#define QA_FWD(TRAINV, PLAINV)                                                                                                          \
+#define QA_FWD_M(TRAINV, PLAINV, MASKV)                                                                                          \
     QA_DISPATCH(H, T, {                                                                                                         \
-        auto kern = qattn_fwd_kernel<HD, TH, TH, TRAINV, PLAINV>;                                                               \
+        auto kern = qattn_fwd_kernel<HD, TH, TH, TRAINV, PLAINV, MASKV>;                                                        \
         static bool raised = false;                                                                                             \
         if (!raised && (rc = raise_lds(kern, lds, "hgq_qattention_fwd"))) return rc;                                            \
         raised = true;                                                                                                          \
         hipLaunchKernelGGL(kern, dim3(pl.n_wg), dim3(QA_NT), lds, s, query, key, value, out, pl, input_scaler, eps,             \
                            softmax_desc_or_none(exp_iq), softmax_desc_or_none(exp_oq), softmax_desc_or_none(inv_iq),            \
-                           softmax_desc_or_none(inv_oq), softmax_desc_or_none(oq), amax_exp_iq, amax_inv_iq, slices, pairs);    \
+                           softmax_desc_or_none(inv_oq), softmax_desc_or_none(oq), amax_exp_iq, amax_inv_iq, slices, pairs, mk); \
     })
+#define QA_FWD(TRAINV, PLAINV)                  \
+    do {                                        \
+        if (masked) QA_FWD_M(TRAINV, PLAINV, true); \
+        else QA_FWD_M(TRAINV, PLAINV, false);   \
+    } while (0)
     if (train && (!has_oq || ((oq->mode >> 4) & 0xf) == HGQ_WRAP))
         QA_FWD(true, true);
     else if (train)
@@ -949,6 +1061,7 @@ extern "C" int hgq_qattention_fwd(const float *query, const float *key, const fl
     else
         QA_FWD(false, false);
 #undef QA_FWD
+#undef QA_FWD_M
     if ((rc = check_launch("hgq_qattention_fwd"))) return rc;
     if (!slices) return HGQ_OK;
     const int64_t entries = pl.P_table * S;
@@ -973,12 +1086,15 @@ extern "C" int hgq_qattention_bwd(const float *dout, const float *query, const f
                                   float *dkey, float *dvalue, int B, int T, int S, int N, int H, int64_t bw_rows,
                                   float input_scaler, float eps, const hgq_qdesc *exp_iq, const hgq_qdesc *exp_oq,
                                   const hgq_qdesc *inv_iq, const hgq_qdesc *inv_oq, const hgq_qdesc *oq, float *g_shared,
-                                  float *g_oq_i, float *g_oq_fb, float *workspace, void *stream) {
+                                  float *g_oq_i, float *g_oq_fb, float *workspace, const uint8_t *mask, int mask_batch, int causal,
+                                  void *stream) {
     hipStream_t s = (hipStream_t)stream;
     const bool has_oq = oq && oq->k;
     QAttnPlan pl;
     int rc = plan_qattn(B, T, S, N, H, bw_rows, has_oq, pl, "hgq_qattention_bwd");
     if (rc) return rc;
+    if ((rc = check_mask(mask, mask_batch, B, "hgq_qattention_bwd"))) return rc;
+    const QAttnMask mk = {mask, mask_batch, causal != 0};
     if (!softmax_desc_ok(exp_iq) || !softmax_desc_ok(exp_oq) || !softmax_desc_ok(inv_iq) || !softmax_desc_ok(inv_oq) || !softmax_desc_ok(oq))
         return fail(HGQ_ERR_ARG, "hgq_qattention_bwd: a quantizer descriptor has k but not i / fb");
     const hgq_qdesc *all[5] = {exp_iq, exp_oq, inv_iq, inv_oq, oq};
@@ -1001,15 +1117,19 @@ extern "C" int hgq_qattention_bwd(const float *dout, const float *query, const f
           aligned16(dvalue) && aligned16(workspace)))
         return fail(HGQ_ERR_ARG, "hgq_qattention_bwd: operands and workspace must be 16-byte aligned");
     const size_t lds = qattn_lds_bytes(T, S, true);
-    QA_DISPATCH(H, T, {
-        auto kern = qattn_bwd_kernel<HD, TH, TH>;
-        static bool raised = false;
-        if (!raised && (rc = raise_lds(kern, lds, "hgq_qattention_bwd"))) return rc;
-        raised = true;
-        hipLaunchKernelGGL(kern, dim3(pl.n_wg), dim3(QA_NT), lds, s, dout, query, key, value, dquery, dkey, dvalue, pl, input_scaler,
-                           eps, softmax_desc_or_none(exp_iq), softmax_desc_or_none(exp_oq), softmax_desc_or_none(inv_iq),
-                           softmax_desc_or_none(inv_oq), softmax_desc_or_none(oq), workspace);
-    });
+#define QA_BWD(MASKV)                                                                                                            \
+    QA_DISPATCH(H, T, {                                                                                                          \
+        auto kern = qattn_bwd_kernel<HD, TH, TH, MASKV>;                                                                         \
+        static bool raised = false;                                                                                              \
+        if (!raised && (rc = raise_lds(kern, lds, "hgq_qattention_bwd"))) return rc;                                             \
+        raised = true;                                                                                                           \
+        hipLaunchKernelGGL(kern, dim3(pl.n_wg), dim3(QA_NT), lds, s, dout, query, key, value, dquery, dkey, dvalue, pl,          \
+                           input_scaler, eps, softmax_desc_or_none(exp_iq), softmax_desc_or_none(exp_oq),                        \
+                           softmax_desc_or_none(inv_iq), softmax_desc_or_none(inv_oq), softmax_desc_or_none(oq), workspace, mk); \
+    })
+    if (mask || causal) QA_BWD(true);
+    else QA_BWD(false);
+#undef QA_BWD
     if ((rc = check_launch("hgq_qattention_bwd"))) return rc;
     // a wrapping quantizer's integer bits take no gradient: the reduction writes zeros there
     return softmax_reduce_slices(workspace, slices_plan(pl), g_shared, g_oq_i, g_oq_fb, has_oq, false, s);

@@ -210,16 +210,13 @@ class QMultiHeadAttention(QLayerBase):
             value = query
         if key is None:
             key = value
-        if use_causal_mask:
-            if self._n_seq != 1:
-                raise NotImplementedError('use_causal_mask needs a single sequence axis')
-            T, S = query.shape[1], value.shape[1]
-            causal = torch.tril(torch.ones((1, T, S), dtype=torch.bool, device=query.device))
-            attention_mask = causal if attention_mask is None else (attention_mask.bool() & causal)
+        if use_causal_mask and self._n_seq != 1:
+            raise NotImplementedError('use_causal_mask needs a single sequence axis')
         q = self._query_dense(query)
         k = self._key_dense(key)
         v = self._value_dense(value)
-        out, scores = self._compute_attention(q, k, v, attention_mask, training, need_scores=return_attention_scores)
+        out, scores = self._compute_attention(q, k, v, attention_mask, training, need_scores=return_attention_scores,
+                                              causal=bool(use_causal_mask))
         out = self._output_dense(out)
         if self.enable_oq:
             out = self.oq(out, training=training)
@@ -227,14 +224,22 @@ class QMultiHeadAttention(QLayerBase):
             return out, scores
         return out
 
-    def _compute_attention(self, query, key, value, attention_mask=None, training=None, need_scores=True):
+    def _compute_attention(self, query, key, value, attention_mask=None, training=None, need_scores=True, causal=False):
         if self._inverse_sqrt_key_dim != 1.0:  # 1 after build: the scale lives in the softmax's exp table
             query = query * self._inverse_sqrt_key_dim
         flat = self._n_seq == 1
-        if FUSED and flat and not need_scores and attention_mask is None and not (self._dropout and training):
-            stand_in = self._softmax.attention_plan(query, key, value, training)
+        if FUSED and flat and not need_scores and not (self._dropout and training):
+            # a boolean mask [1 or B, T, S] and / or the causal rule are applied inside the kernel
+            m = attention_mask
+            in_kernel = m is None or (m.dim() == 3 and m.dtype == torch.bool and m.shape[0] in (1, query.shape[0])
+                                      and tuple(m.shape[1:]) == (query.shape[1], key.shape[1]))
+            stand_in = self._softmax.attention_plan(query, key, value, training) if in_kernel else None
             if stand_in is not None:  # one kernel each way; scores and probabilities are never written
-                return self._softmax(stand_in, attention=(query, key, value)), None
+                masks = (m, causal) if (m is not None or causal) else None
+                return self._softmax(stand_in, attention=(query, key, value), attention_mask=masks), None
+        if causal:
+            tril = torch.tril(torch.ones((1, query.shape[1], key.shape[1]), dtype=torch.bool, device=query.device))
+            attention_mask = tril if attention_mask is None else (attention_mask.bool() & tril)
         # several sequence axes, all attended: the contractions see them as one axis (same memory), the softmax and its
         # quantizers see [batch, heads, query seq..., key seq...] as the reference builds them
         B, N = query.shape[0], self._num_heads

@@ -147,13 +147,14 @@ class QSoftmax(QLayerBaseSingleInput):
             return None  # a row layout outside the kernel family
         return qs
 
-    def _call_fused(self, x, training, qs, attention=None):
+    def _call_fused(self, x, training, qs, attention=None, attention_mask=None):
         e, v = self.exp_table, self.inv_table
         owners = (e.iq, e.oq, v.iq, v.oq, self.oq if self.enable_oq else None)
         track_mask = sum(bit for bit, q in zip((1, 0, 2, 0, 4), qs) if q is not None and q[4])
         descs = [None if q is None else q[:4] for q in qs]
         if attention is not None:  # scores and probabilities stay inside the kernel; y is the combined output
-            y, a1, a3, ao = ops.qattention(*attention, descs, self.input_scaler, epsilon(), track_mask)
+            mask, causal = attention_mask if attention_mask is not None else (None, False)  # masks are applied inside the kernel
+            y, a1, a3, ao = ops.qattention(*attention, descs, self.input_scaler, epsilon(), track_mask, mask=mask, causal=causal)
         else:
             y, a1, a3, ao = ops.qsoftmax(x, descs, self.input_scaler, epsilon(), track_mask)
         for amax, n in ((a1, 0), (a3, 2), (ao, 4)):
@@ -182,10 +183,10 @@ class QSoftmax(QLayerBaseSingleInput):
         saturates = inner is not None and (inner.overflow_mode != 'WRAP' or isinstance(inner, FixedPointQuantizerKBI))
         return stand_in if ops.qattention_supported(query, key, value, entries, saturates) else None
 
-    def call(self, inputs, training=None, mask=None, attention=None):
+    def call(self, inputs, training=None, mask=None, attention=None, attention_mask=None):
         if attention is not None:  # `inputs` carries the shape of the scores only (see attention_plan)
             self._oq_applied_in_call = self.enable_oq
-            return self._call_fused(inputs, training, self._fused_plan(inputs, training, None), attention)
+            return self._call_fused(inputs, training, self._fused_plan(inputs, training, None), attention, attention_mask)
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
         qs = self._fused_plan(inputs, training, mask)

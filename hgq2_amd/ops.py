@@ -958,10 +958,21 @@ def qattention_supported(q: Tensor, k: Tensor, v: Tensor, oq_entries: int, oq_sa
     return _lib.load().hgq_qattention_bwd_workspace(B, T, S, N, H, max(oq_entries // S, 1), int(oq_entries > 0)) >= 0
 
 
+def _check_attn_mask(mask: Tensor, B: int, T: int, S: int):
+    """An attention mask for the fused kernel: empty (none), or uint8 ``[1 or B, T, S]`` with 0 = masked out."""
+    if mask.numel() == 0:
+        return
+    _need(mask.is_cuda and mask.dtype == torch.uint8 and mask.is_contiguous(), 'the attention mask must be a contiguous uint8 GPU tensor')
+    _need(mask.dim() == 3 and mask.shape[0] in (1, B) and tuple(mask.shape[1:]) == (T, S),
+          f'the attention mask must have shape [1 or {B}, {T}, {S}], got {tuple(mask.shape)}')
+
+
 @torch.library.custom_op('hgq::qattention_fwd', mutates_args=())
 def qattention_fwd(q: Tensor, k: Tensor, v: Tensor, ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor],
-                   modes: Sequence[int], input_scaler: float, eps: float, track_mask: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+                   modes: Sequence[int], input_scaler: float, eps: float, track_mask: int, mask: Tensor,
+                   causal: bool) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     B, T, S, N, H = _qattn_dims(q, k, v)
+    _check_attn_mask(mask, B, T, S)
     descs = _qdescs(ks, is_, fbs, modes)
     bw_rows = _attn_bw_rows(S, is_[4])
     out = torch.empty_like(q)
@@ -974,13 +985,14 @@ def qattention_fwd(q: Tensor, k: Tensor, v: Tensor, ks: Sequence[Tensor], is_: S
     _need(n_ws >= 0, 'hgq_qattention_fwd_workspace rejected the shape')
     ws = torch.empty(int(n_ws), **i32)
     rc = lib.hgq_qattention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), B, T, S, N, H, bw_rows, input_scaler, eps,
-                                *[ctypes.addressof(d) for d in descs], _ptr(a1), _ptr(a3), _ptr(ao), _ptr(ws), _stream())
+                                *[ctypes.addressof(d) for d in descs], _ptr(a1), _ptr(a3), _ptr(ao), _ptr(ws), _ptr(mask),
+                                mask.shape[0] if mask.numel() else 1, int(causal), _stream())
     _lib.check(rc, 'hgq_qattention_fwd')
     return out, a1, a3, ao
 
 
 @qattention_fwd.register_fake
-def _(q, k, v, ks, is_, fbs, modes, input_scaler, eps, track_mask):
+def _(q, k, v, ks, is_, fbs, modes, input_scaler, eps, track_mask, mask, causal):
     n_o = is_[4].numel() if track_mask & 4 else 0
     return (torch.empty_like(q), q.new_empty(1 if track_mask & 1 else 0, dtype=torch.int32),
             q.new_empty(1 if track_mask & 2 else 0, dtype=torch.int32), q.new_empty(n_o, dtype=torch.int32))
@@ -988,9 +1000,10 @@ def _(q, k, v, ks, is_, fbs, modes, input_scaler, eps, track_mask):
 
 @torch.library.custom_op('hgq::qattention_bwd', mutates_args=())
 def qattention_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, ks: Sequence[Tensor], is_: Sequence[Tensor],
-                   fbs: Sequence[Tensor], modes: Sequence[int], input_scaler: float,
-                   eps: float) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
+                   fbs: Sequence[Tensor], modes: Sequence[int], input_scaler: float, eps: float, mask: Tensor,
+                   causal: bool) -> tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
     B, T, S, N, H = _qattn_dims(q, k, v)
+    _check_attn_mask(mask, B, T, S)
     _check_f32('dout', dout)
     _need(dout.shape == q.shape, 'dout and query differ in shape')
     descs = _qdescs(ks, is_, fbs, modes)
@@ -1007,13 +1020,13 @@ def qattention_bwd(dout: Tensor, q: Tensor, k: Tensor, v: Tensor, ks: Sequence[T
     ws = torch.empty(max(int(n_ws), 1), **f32)
     rc = lib.hgq_qattention_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(dq), _ptr(dk), _ptr(dv), B, T, S, N, H, bw_rows,
                                 input_scaler, eps, *[ctypes.addressof(d) for d in descs], _ptr(g_shared), _ptr(g_oi), _ptr(g_of),
-                                _ptr(ws), _stream())
+                                _ptr(ws), _ptr(mask), mask.shape[0] if mask.numel() else 1, int(causal), _stream())
     _lib.check(rc, 'hgq_qattention_bwd')
     return dq, dk, dv, g_shared, g_oi, g_of
 
 
 @qattention_bwd.register_fake
-def _(dout, q, k, v, ks, is_, fbs, modes, input_scaler, eps):
+def _(dout, q, k, v, ks, is_, fbs, modes, input_scaler, eps, mask, causal):
     n_o = is_[4].numel()
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), q.new_empty(8), q.new_empty(n_o), q.new_empty(n_o)
 
@@ -2102,40 +2115,46 @@ class _QAttention(torch.autograd.Function):
     """Arguments after the scalars: k, i, fb of exp_iq, exp_oq, inv_iq, inv_oq, oq (15 tensors, empty = absent)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, modes, input_scaler, eps, track_mask, *qvars):
+    def forward(ctx, q, k, v, modes, input_scaler, eps, track_mask, mask, causal, *qvars):
         ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
-        out, a1, a3, ao = qattention_fwd(q, k, v, ks, is_, fbs, list(modes), input_scaler, eps, track_mask)
-        ctx.save_for_backward(q, k, v, *qvars)
-        ctx.modes, ctx.input_scaler, ctx.eps = tuple(modes), input_scaler, eps
+        out, a1, a3, ao = qattention_fwd(q, k, v, ks, is_, fbs, list(modes), input_scaler, eps, track_mask, mask, causal)
+        ctx.save_for_backward(q, k, v, mask, *qvars)
+        ctx.modes, ctx.input_scaler, ctx.eps, ctx.causal = tuple(modes), input_scaler, eps, causal
         ctx.mark_non_differentiable(a1, a3, ao)
         ctx.set_materialize_grads(False)
         return out, a1, a3, ao
 
     @staticmethod
     def backward(ctx, gout, *_unused):
-        n_in = 7 + 15
+        n_in = 9 + 15
         if gout is None:
             return (None,) * n_in
-        q, k, v, *qvars = ctx.saved_tensors
+        q, k, v, mask, *qvars = ctx.saved_tensors
         ks, is_, fbs = list(qvars[0::3]), list(qvars[1::3]), list(qvars[2::3])
         dq, dk, dv, g_shared, g_oi, g_of = qattention_bwd(gout.contiguous(), q, k, v, ks, is_, fbs, list(ctx.modes),
-                                                          ctx.input_scaler, ctx.eps)
+                                                          ctx.input_scaler, ctx.eps, mask, ctx.causal)
         need = ctx.needs_input_grad
-        grads = [dq if need[0] else None, dk if need[1] else None, dv if need[2] else None, None, None, None, None]
+        grads = [dq if need[0] else None, dk if need[1] else None, dv if need[2] else None, None, None, None, None, None, None]
         for n in range(5):
             gi = g_shared[2 * n] if n < 4 else g_oi
             gf = g_shared[2 * n + 1] if n < 4 else g_of
             present = ks[n].numel() > 0
-            base = 7 + 3 * n
+            base = 9 + 3 * n
             grads.append(None)
             grads.append(gi.view(is_[n].shape) if present and need[base + 1] else None)
             grads.append(gf.view(fbs[n].shape) if present and need[base + 2] else None)
         return tuple(grads)
 
 
-def qattention(q: Tensor, k: Tensor, v: Tensor, quantizers, input_scaler: float, eps: float, track_mask: int = 0):
+def qattention(q: Tensor, k: Tensor, v: Tensor, quantizers, input_scaler: float, eps: float, track_mask: int = 0, mask=None,
+               causal: bool = False):
     """``combine(qsoftmax(scores(q, k)), v)`` without materialising scores or probabilities.  ``quantizers`` as for
-    ``qsoftmax``.  Returns ``(out, amax_exp_iq, amax_inv_iq, amax_oq)``."""
+    ``qsoftmax``.  ``mask``: boolean ``[1 or B, T, S]`` (False = masked out, shared by the heads) or None; ``causal``: key
+    positions beyond the query position are masked as well.  Returns ``(out, amax_exp_iq, amax_inv_iq, amax_oq)``."""
+    if mask is None:
+        mask = torch.empty(0, dtype=torch.uint8, device=q.device)
+    else:
+        mask = mask.to(torch.uint8).contiguous()
     e_f = q.new_empty(0)
     e_k = torch.empty(0, dtype=torch.uint8, device=q.device)
     flat, modes = [], []
@@ -2148,7 +2167,7 @@ def qattention(q: Tensor, k: Tensor, v: Tensor, quantizers, input_scaler: float,
             flat += [kk.contiguous(), i.contiguous(), fb.contiguous()]
             modes.append(int(mode))
     return _QAttention.apply(q.contiguous(), k.contiguous(), v.contiguous(), tuple(modes), float(input_scaler), float(eps),
-                             int(track_mask), *flat)
+                             int(track_mask), mask, bool(causal), *flat)
 
 
 class _Conv2D(torch.autograd.Function):

@@ -808,17 +808,24 @@ int hgq_attn_combine_bwd(const float *dout, const float *probs, const float *val
  * hgq_qsoftmax_* and hgq_attn_combine_*.  Operands and workspaces 16-byte aligned.  The forward
  * workspace (needed with amax_oq only) holds one abs-max slice per workgroup: entries are combined by a
  * second launch, not by atomics.
+ * Masks (QSoftmax.call with `mask`, src/hgq/layers/softmax.py:118-127; `use_causal_mask` and `attention_mask` of
+ * QMultiHeadAttention.call, src/hgq/layers/attn/mha.py:439-461): `mask` (may be NULL) is a boolean mask
+ * [mask_batch, T, S], one byte per entry, 0 = masked out, shared by all heads, mask_batch = 1 or B, 4-byte aligned;
+ * `causal` != 0 masks key positions beyond the query position as well.  A masked score becomes -1e9 ahead of the row
+ * maximum and its exp is multiplied by zero behind the table, as the reference does; it takes no gradient.
  */
 int hgq_qattention_fwd(const float *query, const float *key, const float *value, float *out, int B, int T, int S, int N, int H,
                        int64_t bw_rows, float input_scaler, float eps, const hgq_qdesc *exp_iq, const hgq_qdesc *exp_oq,
                        const hgq_qdesc *inv_iq, const hgq_qdesc *inv_oq, const hgq_qdesc *oq, uint32_t *amax_exp_iq,
-                       uint32_t *amax_inv_iq, uint32_t *amax_oq, void *workspace, void *stream);
+                       uint32_t *amax_inv_iq, uint32_t *amax_oq, void *workspace, const uint8_t *mask, int mask_batch, int causal,
+                       void *stream);
 int64_t hgq_qattention_fwd_workspace(int B, int T, int S, int N, int H, int64_t bw_rows, int track_oq); /* 4-byte words */
 int64_t hgq_qattention_bwd_workspace(int B, int T, int S, int N, int H, int64_t bw_rows, int has_oq);
 int hgq_qattention_bwd(const float *dout, const float *query, const float *key, const float *value, float *dquery, float *dkey,
                        float *dvalue, int B, int T, int S, int N, int H, int64_t bw_rows, float input_scaler, float eps,
                        const hgq_qdesc *exp_iq, const hgq_qdesc *exp_oq, const hgq_qdesc *inv_iq, const hgq_qdesc *inv_oq,
-                       const hgq_qdesc *oq, float *g_shared, float *g_oq_i, float *g_oq_fb, float *workspace, void *stream);
+                       const hgq_qdesc *oq, float *g_shared, float *g_oq_i, float *g_oq_fb, float *workspace, const uint8_t *mask,
+                       int mask_batch, int causal, void *stream);
 
 /*
  * 2-D max / average pooling on channels-last tensors, forward and backward.  Replaces the Keras

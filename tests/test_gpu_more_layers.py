@@ -179,7 +179,9 @@ def test_multi_head_attention(dev):
 
 
 @pytest.mark.parametrize('fuse,shapes,causal', [('none', ((2, 4, 8), (2, 4, 9), (2, 4, 10)), False), ('kv', ((2, 4, 3), (2, 4, 5)), False),
-                                                ('none', ((3, 2, 8), (2, 5, 6)), False), ('qkv', ((9, 8),), True)])
+                                                ('none', ((3, 2, 8), (2, 5, 6)), False), ('qkv', ((9, 8),), True),
+                                                # sequence lengths the one-pass kernels take: the causal rule is applied inside them
+                                                ('none', ((32, 16),), True), ('qkv', ((64, 16),), True)])
 @pytest.mark.parametrize('num_heads', [1, 2])
 def test_multi_head_attention_shapes_of_the_reference_tests(dev, fuse, shapes, causal, num_heads):
     """The input shapes reference tests/test_mha.py:29-37 runs: two sequence axes with separate query / value / key
@@ -579,12 +581,17 @@ def test_bn_fold_matches_the_reference_formula(K, N, with_gamma, is_meansq):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('batch,seq,heads,key_dim,oq_hom', [(2048, 64, 4, 16, None), (300, 32, 2, 8, None), (37, 32, 2, 32, None),
-                                                            (5, 64, 1, 8, None), (70, 64, 2, 16, (0, 1)), (33, 32, 4, 16, (0, 1, 2))])
-def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim, oq_hom):
+@pytest.mark.parametrize('batch,seq,heads,key_dim,oq_hom,masks', [
+    (2048, 64, 4, 16, None, ''), (300, 32, 2, 8, None, ''), (37, 32, 2, 32, None, ''), (5, 64, 1, 8, None, ''),
+    (70, 64, 2, 16, (0, 1), ''), (33, 32, 4, 16, (0, 1, 2), ''),
+    # masks applied inside the one-pass kernels: the causal rule, a boolean mask per batch element or shared, both
+    (300, 64, 4, 16, None, 'causal'), (41, 32, 2, 8, None, 'causal'), (64, 64, 2, 16, None, 'bool'), (37, 32, 2, 32, None, 'bool1'),
+    (50, 64, 1, 8, (0, 1), 'causal+bool')])
+def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim, oq_hom, masks):
     """scores -> table softmax -> combine as one kernel each way (hgq_qattention_fwd / _bwd) against the same
     layer composing hgq_attn_scores_*, hgq_qsoftmax_* and hgq_attn_combine_*: outputs, tracked integer
-    bits and loss terms bit-identical, gradients within fp32 summation noise."""
+    bits and loss terms bit-identical, gradients within fp32 summation noise.  With masks (reference
+    src/hgq/layers/softmax.py:118-127, tests/test_mha.py:54) the composed path runs the softmax stage by stage."""
     import hgq2_amd.layers.attn.mha as mha
     from hgq2_amd.config import QuantizerConfig
     from hgq2_amd.layers import QMultiHeadAttention
@@ -598,8 +605,17 @@ def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim, 
     with readme_scopes():
         layer = QMultiHeadAttention(num_heads=heads, key_dim=key_dim, **kw)
     x = torch.randn(batch, seq, heads * key_dim, generator=g)
+    call_kw = {}
+    if 'causal' in masks:
+        call_kw['use_causal_mask'] = True
+    if 'bool' in masks:
+        m = torch.rand(1 if 'bool1' in masks else batch, seq, seq, generator=g) > 0.3
+        m[..., 0] = True            # (every query keeps a key that the causal rule keeps, too)
+        if batch > 3:
+            m[min(3, m.shape[0] - 1), 5] = False     # ... except one row that is masked out altogether
+        call_kw['attention_mask'] = m.to(dev)
     with torch.no_grad():
-        layer(x.to(dev), training=True)
+        layer(x.to(dev), training=True, **call_kw)
     _perturb(layer, g)
     state = {n: p.detach().clone() for n, p in layer.state_dict().items()}
     w = torch.randn(batch, seq, heads * key_dim, generator=g).to(dev)
@@ -615,7 +631,14 @@ def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim, 
         mha.FUSED = fused
         try:
             xp = x.to(dev).requires_grad_(True)
-            y = layer(xp, training=True)
+            launched = []
+            real = mha.ops.qattention
+            mha.ops.qattention = lambda *a, **k: (launched.append(1), real(*a, **k))[1]
+            try:
+                y = layer(xp, training=True, **call_kw)
+            finally:
+                mha.ops.qattention = real
+            assert bool(launched) == fused, 'the one-pass kernel runs exactly where it is switched on'
             (y * w).sum().backward()
         finally:
             mha.FUSED = True
@@ -627,7 +650,7 @@ def test_one_pass_attention_equals_composed_kernels(batch, seq, heads, key_dim, 
         mha.FUSED = fused
         try:
             with torch.no_grad():
-                y_inf = layer(x.to(dev), training=False)  # inference mode: wrapping quantizers wrap, empty words are zeroed
+                y_inf = layer(x.to(dev), training=False, **call_kw)  # inference mode: wrapping quantizers wrap, empty words are zeroed
         finally:
             mha.FUSED = True
         results.append((y.detach(), grads, i_vars, losses, y_inf))
