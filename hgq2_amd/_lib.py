@@ -95,6 +95,13 @@ SIGNATURES = {
     'hgq_quantize_fwd_bwd': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_fwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_quantize_bwd_multi': (c_int, [c_void_p, c_int, c_void_p]),
+    'hgq_gdense_supported': (c_int, [c_int64, c_int, c_int, c_int]),
+    'hgq_gdense_fwd': (c_int, [c_void_p] * 4 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_gdense_bwd_workspace': (c_int64, [c_int64, c_int, c_int, c_int, c_int]),
+    'hgq_gdense_bwd': (c_int, [c_void_p] * 8 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_affine_rows_fwd': (c_int, [c_void_p] * 4 + [c_int64, c_int, c_void_p]),
+    'hgq_affine_rows_bwd_workspace': (c_int64, [c_int64, c_int]),
+    'hgq_affine_rows_bwd': (c_int, [c_void_p] * 7 + [c_int64, c_int, c_void_p]),
     'hgq_mean_mid_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     'hgq_mean_mid_bwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     'hgq_sum_scalars': (c_int, [c_void_p, c_int, c_void_p, c_void_p]),

@@ -7,7 +7,8 @@ with the batch moments in training (moving averages updated in place) and the mo
 The layer's own ``epsilon`` is used (not the global one), and with ``center=False`` the reference puts 1 in
 the place of ``bn_beta`` (:117-120, :145-148); both are kept.  EBOPs ``sum(bits_in * bits_scale) +
 mean(bits_offset) * size``.  The moments over a trailing channel axis come from the one-pass column-moment
-kernel (``hgq_col_moments_fwd / _bwd``)."""
+kernel (``hgq_col_moments_fwd / _bwd``); in a training step scale, offset, the moving-average updates and the two
+quantizers are one launch each way (``_fold_in_one_launch``)."""
 
 from __future__ import annotations
 
@@ -18,7 +19,7 @@ import torch
 from .. import ops
 from ..core import get_initializer
 from ..quantizer import Quantizer, QuantizerConfig
-from ..quantizer.prefetch import quantize_together
+from ..quantizer.prefetch import _eligible, quantize_together
 from .core.base import QLayerBaseSingleInput, mean_bits
 
 
@@ -97,6 +98,10 @@ class QBatchNormalization(QLayerBaseSingleInput):
             raise NotImplementedError('QBatchNormalization: masked moments are not supported')
         if self.enable_iq:
             inputs = self.iq(inputs, training=training)
+        fused = self._fold_in_one_launch(inputs) if training is True else None
+        if fused is not None:
+            qscale, qoffset = fused
+            return ops.affine_rows(inputs, qscale.reshape(self._shape), qoffset.reshape(self._shape))
         if training:
             mean, variance = self._moments(inputs)
             with torch.no_grad():
@@ -108,6 +113,28 @@ class QBatchNormalization(QLayerBaseSingleInput):
         qscale, qoffset = quantize_together([(self.kq, scale.contiguous()), (self.bq, offset.contiguous())], training)
         qscale, qoffset = qscale.reshape(self._shape), qoffset.reshape(self._shape)
         return ops.affine_rows(inputs, qscale, qoffset)
+
+    def _fold_in_one_launch(self, x):
+        """``(kq(scale), bq(offset))`` of a training step from the batch moments in ONE launch each way - scale, offset,
+        the moving-average updates and both quantizers (``hgq_bn_fold_quant_fwd / _bwd`` on a kernel of ones: a folded
+        kernel ``1 * scale`` and a folded bias ``beta - mean * scale`` are exactly this layer's two operands) - instead
+        of some twenty launches on [channels] vectors; ``None`` where the kernels do not apply."""
+        if not (x.is_cuda and x.dtype == torch.float32 and self.axis == x.dim() - 1 and x.numel() > 0):
+            return None
+        fk, fb = _eligible(self.kq, self.moving_mean), _eligible(self.bq, self.moving_mean)
+        if fk is None or fb is None:
+            return None
+        C = x.shape[-1]
+        ones = self.__dict__.get('_ones')
+        if ones is None or ones.device != x.device or ones.numel() != C:
+            ones = torch.ones(1, C, dtype=torch.float32, device=x.device)
+            object.__setattr__(self, '_ones', ones)
+        mean, meansq = ops.col_moments(x.reshape(-1, C).contiguous())  # one pass over x
+        beta = self.bn_beta if self.center else ones.view(-1)  # (the reference puts 1 in the place of a missing beta)
+        qs, qo = ops.bn_fold_quant(ones, beta, self.bn_gamma if self.scale else None, mean, meansq, True, self.epsilon,
+                                   self.moving_mean, self.moving_variance, self.momentum,
+                                   *((f._k.view(-1), f._i.view(-1), f._third().view(-1), f._mode(True)) for f in (fk, fb)))
+        return qs.view(-1), qo
 
     def _compute_ebops(self, shape):
         bw_inp = self.iq.bits_(shape)

@@ -13,7 +13,7 @@ from math import prod
 
 import torch
 
-from ... import ops
+from ... import _lib, ops
 from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
@@ -79,6 +79,22 @@ def gemm_form(equation):
     return None
 
 
+def grouped_form(equation):
+    """(n_group, n_contract, n_new) if the equation is ``<free><G><C>,<G><C><O>-><free><G><O>`` - the kernel carries the
+    ``G`` axes of the input with it, one small kernel matrix per position (e.g. ``'Babc,bcd->Babd'``) - else None."""
+    in_spec, rest = equation.split(',', 1)
+    w_spec, out_spec = rest.split('->', 1)
+    for ng in range(1, len(w_spec) - 1):
+        for nc in range(1, len(w_spec) - ng):
+            g, c, o = w_spec[:ng], w_spec[ng:ng + nc], w_spec[ng + nc:]
+            if not o or not in_spec.endswith(g + c):
+                continue
+            free = in_spec[:len(in_spec) - ng - nc]
+            if free and out_spec == free + g + o and not (set(o) & set(in_spec)) and len(set(w_spec)) == len(w_spec):
+                return ng, nc, len(o)
+    return None
+
+
 class QEinsumDense(QLayerBaseSingleInput):
     def __init__(self, equation, output_shape, activation=None, bias_axes=None, kernel_initializer='glorot_uniform',
                  bias_initializer='zeros', kernel_regularizer=None, bias_regularizer=None, kernel_constraint=None,
@@ -132,6 +148,13 @@ class QEinsumDense(QLayerBaseSingleInput):
                 q.built = True
         self.ebops_equation = self.equation.split('->')[0] + '->'
         self._gemm = gemm_form(self.equation)
+        self._grouped = grouped_form(self.equation) if self._gemm is None else None
+        if self._grouped is not None:
+            ng, nc, _ = self._grouped
+            self._G, self._gK, self._gN = prod(kernel_shape[:ng]), prod(kernel_shape[ng:ng + nc]), prod(kernel_shape[ng + nc:])
+            # the bias rides in the kernel only when it is exactly one value per (group, output column)
+            self._bias_in_grouped = bias_shape is not None and prod(bias_shape) == self._G * self._gN and \
+                tuple(s for s in bias_shape if s != 1) == tuple(s for s in kernel_shape[:ng] + kernel_shape[ng + nc:] if s != 1)
         if self._gemm is not None:
             nc, _ = self._gemm
             self._K = prod(kernel_shape[:nc])
@@ -174,6 +197,19 @@ class QEinsumDense(QLayerBaseSingleInput):
             return y, act_done
         if iq is not None:
             inputs = iq(inputs, training=training)
+        if self._grouped is not None and inputs.is_cuda and inputs.numel() > 0:
+            # one small kernel matrix per position: the grouped dense kernels on [rows, G, K] / [G, K, N] views
+            x3 = inputs.reshape(-1, self._G, self._gK)
+            w3 = qkernel.reshape(self._G, self._gK, self._gN)
+            if ops.gdense_supported(x3, w3):
+                in_kernel = qbias is None or self._bias_in_grouped
+                relu = in_kernel and self._act_name == 'relu'
+                y = ops.gdense(x3, w3, qbias.reshape(self._G, self._gN) if (qbias is not None and in_kernel) else None,
+                               _lib.ACT_RELU if relu else _lib.ACT_NONE)
+                y = y.view(inputs.shape[0], *self.full_output_shape[1:])
+                if qbias is not None and not in_kernel:
+                    y = ops.bias_add_rows(y, qbias)
+                return y, relu or (in_kernel and self._act_name == 'linear')
         y = torch.einsum(self.equation, inputs, qkernel)
         if qbias is not None:
             y = ops.bias_add_rows(y, qbias)

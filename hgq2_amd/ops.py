@@ -18,7 +18,7 @@ from torch import Tensor
 
 from . import _lib
 
-__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits', 'ebops_finish', 'qattention', 'qattention_supported', 'bits_ebops']
+__all__ = ['quantize', 'wrap_track_i_', 'qdense', 'dense_ebops', 'sparse_ce', 'sgd_update_', 'sgd_update_multi_', 'qsoftmax', 'conv2d', 'matmul_bias_act', 'col_moments', 'attn_scores', 'attn_combine', 'ATTN_MAX', 'pool2d', 'conv2d_ebops', 'conv_geometry', 'conv2d_ebops_supported', 'mse', 'dense_moments', 'dense_moments_supported', 'bn_fold', 'qbits', 'ebops_finish', 'qattention', 'qattention_supported', 'bits_ebops', 'gdense', 'gdense_supported', 'affine_rows']
 
 
 def _ptr(t: Tensor | None):
@@ -2529,45 +2529,136 @@ class _BiasAddRows(torch.autograd.Function):
         return g, db
 
 
+@torch.library.custom_op('hgq::affine_rows_fwd', mutates_args=())
+def affine_rows_fwd(x: Tensor, s: Tensor, o: Tensor) -> Tensor:
+    _check_f32('x', x), _check_f32('scale', s), _check_f32('offset', o)
+    C = x.shape[-1]
+    _need(s.numel() == C and o.numel() == C, 'scale and offset must have one entry per trailing channel')
+    y = torch.empty_like(x)
+    rc = _lib.load().hgq_affine_rows_fwd(_ptr(x), _ptr(s), _ptr(o), _ptr(y), x.numel() // C, C, _stream())
+    _lib.check(rc, 'hgq_affine_rows_fwd')
+    return y
+
+
+@affine_rows_fwd.register_fake
+def _(x, s, o):
+    return torch.empty_like(x)
+
+
+@torch.library.custom_op('hgq::affine_rows_bwd', mutates_args=())
+def affine_rows_bwd(g: Tensor, x: Tensor, s: Tensor, need_dx: bool) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('g', g), _check_f32('x', x), _check_f32('scale', s)
+    C = x.shape[-1]
+    rows = x.numel() // C
+    lib = _lib.load()
+    dx = torch.empty_like(x) if need_dx else x.new_empty(0)
+    ds, do = x.new_empty(C), x.new_empty(C)
+    n_ws = lib.hgq_affine_rows_bwd_workspace(rows, C)
+    _need(n_ws >= 0, 'hgq_affine_rows_bwd_workspace rejected the shape')
+    ws = x.new_empty(max(int(n_ws), 1))
+    rc = lib.hgq_affine_rows_bwd(_ptr(g), _ptr(x), _ptr(s), _ptr(dx), _ptr(ds), _ptr(do), _ptr(ws), rows, C, _stream())
+    _lib.check(rc, 'hgq_affine_rows_bwd')
+    return dx, ds, do
+
+
+@affine_rows_bwd.register_fake
+def _(g, x, s, need_dx):
+    C = x.shape[-1]
+    return (torch.empty_like(x) if need_dx else x.new_empty(0)), x.new_empty(C), x.new_empty(C)
+
+
 class _AffineRows(torch.autograd.Function):
     """``x * s + o`` with ``s``, ``o`` of one value per trailing channel (a multiplication, then an addition, as the
-    reference's ``inputs * qscale + qoffset``, src/hgq/layers/batch_normalization.py:184).  The gradients of ``s`` and
-    ``o`` - sums over all rows - are taken by the library's fixed-order slice reduction, both in one launch."""
+    reference's ``inputs * qscale + qoffset``, src/hgq/layers/batch_normalization.py:184): one launch forward, and one
+    pass + a fixed-order slice reduction backward for ``dx`` and the two sums over the rows."""
 
     @staticmethod
     def forward(ctx, x, s, o):
         ctx.save_for_backward(x, s)
         ctx.shapes = (s.shape, o.shape)
-        return x * s + o
+        return affine_rows_fwd(x, s.reshape(-1).contiguous(), o.reshape(-1).contiguous())
 
     @staticmethod
     def backward(ctx, g):
         x, s = ctx.saved_tensors
-        g = g.contiguous()
-        C = x.shape[-1]
-        dx = g * s if ctx.needs_input_grad[0] else None
-        ds = do = None
-        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            e = g.new_empty(0)
-            sets, outs = [], []
-            if ctx.needs_input_grad[1]:
-                ds = torch.empty(C, dtype=torch.float32, device=g.device)
-                sets.append((g * x).view(-1, C)), outs.extend([ds, e, e])
-            if ctx.needs_input_grad[2]:
-                do = torch.empty(C, dtype=torch.float32, device=g.device)
-                sets.append(g.view(-1, C)), outs.extend([do, e, e])
-            reduce_slices_multi_op(sets, outs, [False] * len(outs))
-            ds = ds.view(ctx.shapes[0]) if ds is not None else None
-            do = do.view(ctx.shapes[1]) if do is not None else None
-        return dx, ds, do
+        dx, ds, do = affine_rows_bwd(g.contiguous(), x, s.reshape(-1).contiguous(), ctx.needs_input_grad[0])
+        return (dx if ctx.needs_input_grad[0] else None, ds.view(ctx.shapes[0]) if ctx.needs_input_grad[1] else None,
+                do.view(ctx.shapes[1]) if ctx.needs_input_grad[2] else None)
+
+
+@torch.library.custom_op('hgq::gdense_fwd', mutates_args=())
+def gdense_fwd(x: Tensor, w: Tensor, bias: Tensor, act: int) -> Tensor:
+    _check_f32('x', x), _check_f32('w', w)
+    R, G, K = x.shape
+    N = w.shape[2]
+    _need(tuple(w.shape) == (G, K, N) and bias.numel() in (0, G * N), 'x [R, G, K], w [G, K, N], bias [G, N]')
+    y = x.new_empty((R, G, N))
+    rc = _lib.load().hgq_gdense_fwd(_ptr(x), _ptr(w), _ptr(bias), _ptr(y), R, G, K, N, act, _stream())
+    _lib.check(rc, 'hgq_gdense_fwd')
+    return y
+
+
+@gdense_fwd.register_fake
+def _(x, w, bias, act):
+    return x.new_empty((x.shape[0], x.shape[1], w.shape[2]))
+
+
+@torch.library.custom_op('hgq::gdense_bwd', mutates_args=())
+def gdense_bwd(dy: Tensor, y: Tensor, x: Tensor, w: Tensor, has_bias: bool, act: int, need_dx: bool) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('dy', dy), _check_f32('x', x), _check_f32('w', w)
+    R, G, K = x.shape
+    N = w.shape[2]
+    lib = _lib.load()
+    dx = torch.empty_like(x) if need_dx else x.new_empty(0)
+    dw = torch.empty_like(w)
+    db = x.new_empty((G, N)) if has_bias else x.new_empty(0)
+    n_ws = lib.hgq_gdense_bwd_workspace(R, G, K, N, int(has_bias))
+    _need(n_ws >= 0, 'hgq_gdense_bwd_workspace rejected the shape')
+    ws = x.new_empty(max(int(n_ws), 1))
+    rc = lib.hgq_gdense_bwd(_ptr(dy), _ptr(y), _ptr(x), _ptr(w), _ptr(dx), _ptr(dw), _ptr(db), _ptr(ws), R, G, K, N, act, _stream())
+    _lib.check(rc, 'hgq_gdense_bwd')
+    return dx, dw, db
+
+
+@gdense_bwd.register_fake
+def _(dy, y, x, w, has_bias, act, need_dx):
+    return (torch.empty_like(x) if need_dx else x.new_empty(0)), torch.empty_like(w), x.new_empty((x.shape[1], w.shape[2]) if has_bias else 0)
+
+
+class _GDense(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w, bias, act):
+        y = gdense_fwd(x, w, bias, act)
+        ctx.save_for_backward(x, w, y)
+        ctx.act, ctx.has_bias = act, bias.numel() > 0
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, w, y = ctx.saved_tensors
+        dx, dw, db = gdense_bwd(gy.contiguous(), y, x, w, ctx.has_bias, ctx.act, ctx.needs_input_grad[0])
+        return (dx if ctx.needs_input_grad[0] else None, dw if ctx.needs_input_grad[1] else None,
+                db if (ctx.has_bias and ctx.needs_input_grad[2]) else None, None)
+
+
+def gdense_supported(x3: Tensor, w3: Tensor) -> bool:
+    return (x3.is_cuda and x3.dtype == torch.float32 and w3.dtype == torch.float32 and x3.dim() == 3 and w3.dim() == 3
+            and bool(_lib.load().hgq_gdense_supported(x3.shape[0], x3.shape[1], x3.shape[2], w3.shape[2])))
+
+
+def gdense(x3: Tensor, w3: Tensor, bias2, act: int = 0) -> Tensor:
+    """``act(x3[r, g, :] @ w3[g] + bias2[g])`` for ``x3 [R, G, K]``, ``w3 [G, K, N]``, ``bias2 [G, N]`` or None."""
+    b = bias2.contiguous() if bias2 is not None else x3.new_empty(0)
+    return _GDense.apply(x3.contiguous(), w3.contiguous(), b, int(act))
 
 
 def affine_rows(x: Tensor, s: Tensor, o: Tensor) -> Tensor:
     """``x * s + o`` for per-channel ``s`` and ``o`` along the last axis of ``x`` (any other layout: plain tensor operations)."""
     C = x.shape[-1] if x.dim() else 0
     if (x.is_cuda and x.dtype == torch.float32 and x.dim() >= 2 and x.numel() > 0 and s.numel() == C and o.numel() == C
-            and s.shape[-1:] == (C,) and o.shape[-1:] == (C,) and s.dtype == torch.float32 and o.dtype == torch.float32):
-        return _AffineRows.apply(x.contiguous(), s, o)
+            and s.shape[-1:] == (C,) and o.shape[-1:] == (C,) and s.dtype == torch.float32 and o.dtype == torch.float32
+            and C % 4 == 0 and x.is_contiguous() and x.data_ptr() % 16 == 0):
+        return _AffineRows.apply(x, s, o)
     return x * s + o
 
 

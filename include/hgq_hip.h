@@ -828,6 +828,33 @@ int hgq_qattention_bwd(const float *dout, const float *query, const float *key, 
                        int mask_batch, int causal, void *stream);
 
 /*
+ * Grouped dense contraction: one small kernel matrix per group g (an axis that input, kernel and output share), the
+ * form of QEinsumDense equations such as 'Babc,bcd->Babd' (reference tests/test_dense.py:56; the einsum and its
+ * autograd of src/hgq/layers/core/einsum_dense.py:72-93 on already quantized operands):
+ *     y[r, g, n] = act(sum_k x[r, g, k] * w[g, k, n] + bias[g, n])
+ *   x [R, G, K], w [G, K, N], bias [G, N] or NULL, y / dy [R, G, N]; K, N <= 64 (hgq_gdense_supported), act HGQ_ACT_*.
+ *   Backward: dx [R, G, K] (NULL to skip), dw [G, K, N], dbias [G, N] or NULL; y is read for the relu mask only;
+ *   workspace: hgq_gdense_bwd_workspace floats (per-workgroup slices, added in a fixed order).
+ */
+int hgq_gdense_supported(int64_t R, int G, int K, int N);
+int hgq_gdense_fwd(const float *x, const float *w, const float *bias, float *y, int64_t R, int G, int K, int N, int act, void *stream);
+int64_t hgq_gdense_bwd_workspace(int64_t R, int G, int K, int N, int has_bias);
+int hgq_gdense_bwd(const float *dy, const float *y, const float *x, const float *w, float *dx, float *dw, float *dbias, float *workspace,
+                   int64_t R, int G, int K, int N, int act, void *stream);
+
+/*
+ * Per-channel affine map of QBatchNormalization.call (src/hgq/layers/batch_normalization.py:184,
+ * `inputs * qscale + qoffset`, a multiplication and then an addition) over the trailing axis, and its gradients:
+ *     y[r, c] = x[r, c] * scale[c] + offset[c];  dx = g * scale;  dscale[c] = sum_r g x;  doffset[c] = sum_r g
+ *   C a positive multiple of 4, operands 16-byte aligned; dx / dscale / doffset may be NULL; workspace:
+ *   hgq_affine_rows_bwd_workspace floats (slices of the two sums, added in a fixed order).
+ */
+int hgq_affine_rows_fwd(const float *x, const float *scale, const float *offset, float *y, int64_t rows, int C, void *stream);
+int64_t hgq_affine_rows_bwd_workspace(int64_t rows, int C);
+int hgq_affine_rows_bwd(const float *g, const float *x, const float *scale, float *dx, float *dscale, float *doffset, float *workspace,
+                        int64_t rows, int C, void *stream);
+
+/*
  * 2-D max / average pooling on channels-last tensors, forward and backward.  Replaces the Keras
  * MaxPooling2D / AveragePooling2D `call` that QMaxPooling2D / QAveragePooling2D apply to the
  * quantized input (src/hgq/layers/pooling.py:23-47; the Keras torch backend transposes to

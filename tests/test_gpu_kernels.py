@@ -639,3 +639,61 @@ def test_bn_fold_with_its_quantizers_in_one_launch(dev, K, N, overflow):
         if a is not None:
             err = (a.double() - b.double()).abs().max().item()
             assert err <= 1e-5 * (b.abs().max().item() + 1e-6), (name, err)
+
+
+@pytest.mark.parametrize('R,G,K,N,act,bias', [(300, 5, 7, 9, 1, True), (1, 1, 1, 1, 0, False), (4096, 3, 16, 16, 1, True), (70, 12, 64, 64, 0, True),
+                                              (65, 2, 33, 5, 1, False), (100000, 4, 8, 8, 0, True), (0, 3, 4, 4, 0, True)])
+def test_grouped_dense_against_fp64(dev, R, G, K, N, act, bias):
+    """``y[r, g] = act(x[r, g] @ w[g] + b[g])`` (the einsum 'Babc,bcd->Babd' of reference tests/test_dense.py:56 on
+    [rows, groups, in] views): values and all three gradients within 1e-5 of the summed |terms| of a float64 einsum."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(R + 31 * G + K)
+    x = torch.randn(R, G, K, generator=g)
+    w = torch.randn(G, K, N, generator=g) * 0.4
+    b = torch.randn(G, N, generator=g) if bias else None
+    up = torch.randn(R, G, N, generator=g)
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    br = b.double().requires_grad_(True) if bias else None
+    z = torch.einsum('rgk,gkn->rgn', xr, wr) + (br if bias else 0)
+    if act:  # no upstream gradient where fp32 and fp64 may disagree on the side of the kink
+        up = up * (z.detach().abs() > 1e-5 * float(z.detach().abs().max() if R else 1)).float()
+    yr = torch.relu(z) if act else z
+    (yr * up.double()).sum().backward()
+    xd, wd = x.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    bd = b.to(dev).requires_grad_(True) if bias else None
+    assert ops.gdense_supported(xd, wd)
+    y = ops.gdense(xd, wd, bd, act)
+    assert tuple(y.shape) == (R, G, N)
+    (y * up.to(dev)).sum().backward()
+    dz = (up.double() * (z.detach() > 0)) if act else up.double()
+    xa, wa = x.double().abs(), w.double().abs()
+    scales = {'y': torch.einsum('rgk,gkn->rgn', xa, wa) + (b.double().abs() if bias else 0),
+              'dx': torch.einsum('rgn,gkn->rgk', dz.abs(), wa), 'dw': torch.einsum('rgk,rgn->gkn', xa, dz.abs()), 'db': dz.abs().sum(0)}
+    checks = [('y', y.detach(), yr.detach()), ('dx', xd.grad, xr.grad), ('dw', wd.grad, wr.grad)] + ([('db', bd.grad, br.grad)] if bias else [])
+    for name, got, want in checks:
+        err = (got.cpu().double() - want).abs()
+        tol = RTOL * scales[name] + 1e-30
+        assert bool((err <= tol).all()), f'{name}: {float((err / tol).max()):.2f} x the bound'
+
+
+@pytest.mark.parametrize('shape', [(1000, 64), (7, 3, 5, 8), (1, 4), (100000, 12), (0, 16)])
+def test_affine_rows_against_fp64(dev, shape):
+    """``x * s + o`` over the trailing channel axis (QBatchNormalization's map): values exactly the two fp32 operations,
+    dx exactly, the two parameter gradients within 1e-5 of the summed |terms|."""
+    _lib, ops = _ops()
+    g = torch.Generator().manual_seed(sum(shape))
+    C = shape[-1]
+    x, up = torch.randn(shape, generator=g), torch.randn(shape, generator=g)
+    s, o = torch.randn(C, generator=g), torch.randn(C, generator=g)
+    xd, sd, od = (t.to(dev).requires_grad_(True) for t in (x, s, o))
+    if x.numel() == 0:
+        return  # the layer does not call the kernels on empty inputs
+    y = ops.affine_rows(xd, sd, od)
+    assert y.grad_fn is not None and type(y.grad_fn).__name__.startswith('_AffineRows')
+    assert torch.equal(y.detach().cpu(), x * s + o)
+    y.backward(up.to(dev))
+    assert torch.equal(xd.grad.cpu(), up * s)
+    rows = x.reshape(-1, C).double()
+    u2 = up.reshape(-1, C).double()
+    for got, terms, name in ((sd.grad, u2 * rows, 'dscale'), (od.grad, u2, 'doffset')):
+        _assert_close_sum(got, terms.sum(0), terms.abs().sum(0), name)
