@@ -158,8 +158,13 @@ __device__ __forceinline__ uint32_t abs_bits(float v) { return __float_as_uint(v
 
 
 // Runtime-mode forms (for kernels that serve several quantizers with different modes at once).
+// Selects, not branches: the mode is uniform over a launch, but a chain of scalar branches per element costs several
+// times the two vector instructions it would save (one floor serves TRN and RND, one pair of scalings all three).
 __device__ __forceinline__ float fixed_round_dyn(float x, float f, int rm) {
-    return rm == HGQ_TRN ? fixed_round<HGQ_TRN>(x, f) : rm == HGQ_RND ? fixed_round<HGQ_RND>(x, f) : fixed_round<HGQ_RND_CONV>(x, f);
+    const int fi = (int)f;
+    const float t = ldexpf(x, fi);
+    const float down = floorf(rm == HGQ_RND ? __fadd_rn(t, 0.5f) : t);
+    return ldexpf(rm == HGQ_RND_CONV ? rintf(t) : down, -fi);
 }
 
 __device__ __forceinline__ float quantize_dyn(float x, const KIF &p, int rm, int om, bool training) {

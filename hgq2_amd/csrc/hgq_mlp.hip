@@ -20,6 +20,16 @@ namespace hgq {
 
 
 #define MLP_BM 64
+// Phase time stamps of workgroup 0, one row per wavefront (measurement builds only: -DMLP_PROF)
+#ifdef MLP_PROF
+__device__ unsigned long long mlp_prof_stamps[8 * 64];
+#define MLP_STAMP(i)                                                                                                  \
+    do {                                                                                                              \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0) mlp_prof_stamps[(threadIdx.x >> 6) * 64 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define MLP_STAMP(i)
+#endif
 // the matrix-core chains: by exact bf16 parts (1) or with the fp32 instruction (0)
 #ifndef MLP_BF16
 #define MLP_BF16 1
@@ -136,7 +146,9 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                                                           const int64_t *__restrict__ labels, int64_t rows,
                                                           float *part, float *aux, uint32_t *ticket) {
     extern __shared__ float lds[];
+    __shared__ float loss_part[MLP_NT / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    MLP_STAMP(0);
     // snapshot for the update pass: workgroup w's last wavefront takes row w; its loads travel with the image fetch below
     const bool snap_wave = __builtin_amdgcn_readfirstlane(wave) == MLP_NT / 64 - 1;
     MlpSnapRow snap;
@@ -153,7 +165,21 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
     const int64_t n_tiles = (rows + MLP_BM - 1) / MLP_BM;
     const float inv_rows = 1.0f / (float)rows;
 
-    // ---- prologue: fetch the quantized kernels / biases / rounded fractional bits (off_raw is a multiple of 4)
+    // ---- prologue.  The first input tile's loads are issued ahead of everything else: they travel while the image is
+    // fetched (the tile can only be quantized once the image's fractional bits are in LDS, but it need not wait to be asked for)
+    const int K0 = d.l[0].h.K, n_el0 = MLP_BM * K0;
+    float pre[4];
+    {
+        const int64_t r0 = (int64_t)blockIdx.x * MLP_BM, left = rows - r0;
+        const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K0, (left < MLP_BM ? (left > 0 ? left : 0) : MLP_BM) * K0 * 4);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int id = u * MLP_NT + tid;
+            pre[u] = buf_ld1(rs, id < n_el0 ? (uint32_t)id * 4u : BUF_OOB);
+        }
+    }
+    MLP_STAMP(1);
+    // fetch the quantized kernels / biases / rounded fractional bits (off_raw is a multiple of 4)
     // (four 128-bit loads per thread in flight: one load per loop trip would cost a memory latency each)
     for (int id0 = 0; id0 < d.off_raw; id0 += 4 * 4 * MLP_NT) {
         float4 v[4];
@@ -168,9 +194,11 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
             if (id < d.off_raw) *(float4 *)(lds + id) = v[u];
         }
     }
+    MLP_STAMP(2);
     for (int id = tid; id < MLP_BM * d.ld_rx; id += MLP_NT) rx[id] = 0.f;  // padding columns stay zero for good
     for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += MLP_NT) dfs[id] = 0.f, dfs[64 * HGQ_MLP_MAX_LAYERS + id] = 0.f, amx[id] = 0u;
     __syncthreads();
+    MLP_STAMP(3);
     if (snap_wave) {
         mlp_snapshot_end(snap, aux, lane);
         // fewer workgroups than rows (small batches): the remaining rows, one after the other
@@ -182,39 +210,46 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const bool first = tile == blockIdx.x;
         const int64_t r0 = tile * MLP_BM;
+        const int live = (int)(rows - r0 < MLP_BM ? rows - r0 : MLP_BM);  // rows of this tile that exist
         // ---- stage the input tile: raw value, quantized value, abs-max
         {
             const MlpLayerDev &l0 = d.l[0];
-            const int K0 = l0.h.K, rm = Mode(l0.h.mode_in).round_mode;
+            const int rm = Mode(l0.h.mode_in).round_mode;
             const float *fl = lds + l0.off_f;
             // the tile's rows are contiguous in x: buffer loads, zeros past the last row, four in flight
-            const int64_t left = rows - r0;
-            const int n_el = MLP_BM * K0;
-            const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K0, (left < MLP_BM ? left : MLP_BM) * K0 * 4);
+            const int n_el = n_el0;
+            const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K0, live * K0 * 4);
+            // id / K0 for id < 64 * 64 and K0 <= 64 as a multiply and a shift (exact: the error term id * (K0 - 1) stays below 2**20)
+            const uint32_t by_k0 = ((1u << 20) + (uint32_t)K0 - 1u) / (uint32_t)K0;
             for (int id0 = 0; id0 < n_el; id0 += 4 * MLP_NT) {
                 float v[4];
+                if (first && id0 == 0) {
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int id = id0 + u * MLP_NT + tid;
-                    v[u] = buf_ld1(rs, id < n_el ? (uint32_t)id * 4u : BUF_OOB);
+                    for (int u = 0; u < 4; ++u) v[u] = pre[u];
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int id = id0 + u * MLP_NT + tid;
+                        v[u] = buf_ld1(rs, id < n_el ? (uint32_t)id * 4u : BUF_OOB);
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int id = id0 + u * MLP_NT + tid;
                     if (id < n_el) {
-                        const int row = id / K0, k = id - row * K0;
-                        float q = 0.f;
-                        if (r0 + row < rows) {
-                            q = fixed_round_dyn(v[u], fl[k], rm);
-                            atomicMax(&amx[k], abs_bits(q));
-                        }
+                        const int row = (int)(((uint32_t)id * by_k0) >> 20), k = id - row * K0;
+                        float q = fixed_round_dyn(v[u], fl[k], rm);
+                        q = row < live ? q : 0.f;  // (a row past the end was read as zeros: its abs-max term is zero too)
+                        atomicMax(&amx[k], abs_bits(q));
                         raw[row * d.ld_raw + l0.acol + k] = v[u];
                         rx[row * d.ld_rx + l0.acol + k] = q;
                     }
                 }
             }
         }
+        MLP_STAMP(32);
         __syncthreads();
+        MLP_STAMP(4);
         // ================= forward =================
         for (int l = 0; l < L; ++l) {
             const MlpLayerDev &ly = d.l[l];
@@ -224,25 +259,30 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                 floatx16 acc = {0};
                 const float *ws = lds + ly.off_w;
                 const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
+                // everything the epilogue needs is asked for ahead of the chain (no branches in between, so the scalar and
+                // LDS loads travel together): the bias, and the next layer's input quantizer, which runs on the accumulator
+                // registers (for the last layer the values are read and not used)
+                const bool last = l + 1 == L;
+                const MlpLayerDev &nx = d.l[last ? l : l + 1];
+                const int ocol = (last ? d.acol_out : nx.acol) + bcol;
+                const int rm = Mode(nx.h.mode_in).round_mode;
+                const bool relu = ly.h.act == HGQ_ACT_RELU;
+                const float bias = lds[ly.off_qb + bcol], fn = lds[nx.off_f + bcol];
                 // input columns and kernel rows are zero padded to a multiple of 32
                 acc = MLP_CHAIN(false, false)(acc, rx + arow * d.ld_rx + ly.acol + kq, 1, ws + kq * ly.ldw + bcol, ly.ldw, (ly.h.K + 15) >> 4);
                 if (bcol < N) {
-                    const float bias = lds[ly.off_qb + bcol];
-                    const bool last = l + 1 == L;
-                    const int ocol = (last ? d.acol_out : d.l[l + 1].acol) + bcol;
-                    // the next layer's input quantizer runs here, on the accumulator registers
-                    const float fn = last ? 0.f : lds[d.l[l + 1].off_f + bcol];
-                    const int rm = last ? 0 : Mode(d.l[l + 1].h.mode_in).round_mode;
                     uint32_t mx = 0;
+                    float *raw_o = raw + (rh * 32 + (lane >> 5) * 4) * d.ld_raw + ocol, *rx_o = rx + (rh * 32 + (lane >> 5) * 4) * d.ld_rx + ocol;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int row = rh * 32 + acc_row_(r, lane);
+                        const int rr = (r >> 2) * 8 + (r & 3);  // acc_row_(r, lane) - 4 * (lane / 32)
                         float v = acc[r] + bias;
-                        if (ly.h.act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
-                        raw[row * d.ld_raw + ocol] = v;
+                        v = relu ? (v > 0.f ? v : 0.f) : v;
+                        raw_o[rr * d.ld_raw] = v;
                         if (!last) {
-                            const float q = (r0 + row < rows) ? fixed_round_dyn(v, fn, rm) : 0.f;
-                            rx[row * d.ld_rx + ocol] = q;
+                            float q = fixed_round_dyn(v, fn, rm);
+                            q = rh * 32 + (lane >> 5) * 4 + rr < live ? q : 0.f;
+                            rx_o[rr * d.ld_rx] = q;
                             const uint32_t a = abs_bits(q);
                             mx = a > mx ? a : mx;
                         }
@@ -254,44 +294,59 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                     }
                 }
             }
+            MLP_STAMP(33 + l);
             __syncthreads();
+            MLP_STAMP(5 + l);
         }
         // ================= loss: mean sparse categorical cross-entropy from logits =================
+        // eight threads per sample, classes j, j + 8, ...: one exponential per thread instead of all of a row's in turn
         float *cur = lds + d.off_dz0, *nxt = lds + d.off_dz1;
         {
             const int C = d.n_classes;
             const int Cp = d.l[L - 1].Np;
+            const int row = tid >> 3, j = tid & 7;
+            const int64_t gr = r0 + row;
+            const float *z = raw + row * d.ld_raw + d.acol_out;
+            float *dz = cur + row * MLP_LDZ;
             float lrow = 0.f;
-            if (tid < MLP_BM) {
-                const int64_t gr = r0 + tid;
-                const float *z = raw + tid * d.ld_raw + d.acol_out;
-                float *dz = cur + tid * MLP_LDZ;
-                if (gr < rows) {
-                    float mx = z[0];
-                    for (int c = 1; c < C; ++c) mx = fmaxf(mx, z[c]);
-                    float se = 0.f;
-                    for (int c = 0; c < C; ++c) se += expf(z[c] - mx);
-                    const int lab = (int)labels[gr];
-                    lrow = logf(se) - (z[lab] - mx);
-                    const float inv = 1.0f / se;
-                    // a relu on the output layer: its mask (z holds the values after the activation)
-                    const bool mask_out = d.l[L - 1].h.act == HGQ_ACT_RELU;
-                    for (int c = 0; c < C; ++c) {
-                        const float gz = (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows;
-                        dz[c] = (!mask_out || z[c] > 0.f) ? gz : 0.f;
+            if (gr < rows) {
+                float mx = -INFINITY;
+                for (int c = j; c < C; c += 8) mx = fmaxf(mx, z[c]);
+                mx = fmaxf(mx, __shfl_xor(mx, 1, 64)), mx = fmaxf(mx, __shfl_xor(mx, 2, 64)), mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+                float se = 0.f;
+                for (int c = j; c < C; c += 8) se += expf(z[c] - mx);
+                // the same association on every lane of the group (and on every run): pairs, then pairs of pairs
+                se += __shfl_xor(se, 1, 64), se += __shfl_xor(se, 2, 64), se += __shfl_xor(se, 4, 64);
+                const int lab = (int)labels[gr];
+                const bool lab_ok = (unsigned)lab < (unsigned)C;  // a label outside [0, C): NaN loss, no gradient for the sample
+                if (j == 0) lrow = lab_ok ? logf(se) - (z[lab_ok ? lab : 0] - mx) : NAN;
+                const float inv = 1.0f / se;
+                // a relu on the output layer: its mask (z holds the values after the activation)
+                const bool mask_out = d.l[L - 1].h.act == HGQ_ACT_RELU;
+                for (int c = j; c < Cp; c += 8) {
+                    float gz = 0.f;
+                    if (c < C && lab_ok) {
+                        gz = (expf(z[c] - mx) * inv - (c == lab ? 1.0f : 0.0f)) * inv_rows;
+                        if (mask_out && !(z[c] > 0.f)) gz = 0.f;
                     }
-                    for (int c = C; c < Cp; ++c) dz[c] = 0.f;
-                } else {
-                    for (int c = 0; c < Cp; ++c) dz[c] = 0.f;
+                    dz[c] = gz;
                 }
+            } else {
+                for (int c = j; c < Cp; c += 8) dz[c] = 0.f;
             }
-            if (wave == 0) {
+            // the tile's loss: the eight samples of a wavefront in lane order, then the wavefronts in order
 #pragma unroll
-                for (int o = 32; o > 0; o >>= 1) lrow += __shfl_xor(lrow, o, 64);
-                if (lane == 0) my[d.p_loss] = (first ? 0.f : my[d.p_loss]) + lrow * inv_rows;
-            }
+            for (int o = 8; o < 64; o <<= 1) lrow += __shfl_xor(lrow, o, 64);
+            if (lane == 0) loss_part[wave] = lrow;
         }
         __syncthreads();
+        MLP_STAMP(16);
+        if (tid == 0) {
+            float t = 0.f;
+#pragma unroll
+            for (int w = 0; w < MLP_NT / 64; ++w) t += loss_part[w];
+            my[d.p_loss] = (first ? 0.f : my[d.p_loss]) + t * inv_rows;
+        }
         // ================= backward =================
         // `cur` holds the gradient at this layer's pre-activation (relu mask already applied) in
         // columns [0, Np); both phases only read it, so one barrier per layer is enough.
@@ -308,25 +363,40 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                 const int kq = lane >> 5, c32 = lane & 31;
                 acc = MLP_CHAIN(false, true)(acc, rx + kq * d.ld_rx + ly.acol + wkb * 32 + c32, d.ld_rx, cur + kq * MLP_LDZ + wnb * 32 + c32, MLP_LDZ,
                                              MLP_BM / 16);
+                MLP_STAMP(48 + (L - 1 - l));
+                // through a descriptor of this layer's K x N section: rows past K fall outside it and are dropped, so
+                // the sixteen stores (or load - add - store triples) go out back to back, without a branch each
                 const int n = wnb * 32 + c32;
-                if (n < N) {
+                const __amdgpu_buffer_rsrc_t rsw = buf_rsrc(my + ly.p_dw, (int64_t)K * N * 4);
+                const uint32_t off0 = (uint32_t)(((wkb * 32 + kq * 4) * N + n) * 4);
+                float old[16];
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int k = wkb * 32 + acc_row_(r, lane);
-                        if (k < K) {
-                            float *dst = my + ly.p_dw + k * N + n;
-                            *dst = first ? acc[r] : *dst + acc[r];
-                        }
-                    }
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t off = n < N ? off0 + (uint32_t)(((r >> 2) * 8 + (r & 3)) * N * 4) : BUF_OOB;
+                    old[r] = first ? 0.f : buf_ld1(rsw, off);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t off = n < N ? off0 + (uint32_t)(((r >> 2) * 8 + (r & 3)) * N * 4) : BUF_OOB;
+                    buf_st1(rsw, off, first ? acc[r] : old[r] + acc[r]);
                 }
             }
-            // ---- bias gradient: the last wave is free of kernel-gradient work unless all four blocks exist
-            if (ly.h.bias && wave == 7 && lane < N) {
+            MLP_STAMP(52 + (L - 1 - l));
+            // ---- bias gradient: the last wave is free of kernel-gradient work unless all four blocks exist.  A layer of
+            // up to 32 outputs: each half of the wavefront adds 32 rows (in row order), the halves are added last
+            if (ly.h.bias && wave == 7) {
+                const bool halves = N <= 32;
+                const int col = halves ? lane & 31 : lane, ra = halves ? (lane >> 5) * (MLP_BM / 2) : 0, nr = halves ? MLP_BM / 2 : MLP_BM;
+                const float *src = cur + ra * MLP_LDZ + (col < N ? col : 0);
                 float s0 = 0.f, s1 = 0.f;
-#pragma unroll 8
-                for (int r = 0; r < MLP_BM; r += 2) s0 += cur[r * MLP_LDZ + lane], s1 += cur[(r + 1) * MLP_LDZ + lane];
-                float *dst = my + ly.p_db + lane;
-                *dst = first ? s0 + s1 : *dst + (s0 + s1);
+#pragma unroll 16
+                for (int r = 0; r < nr; r += 2) s0 += src[r * MLP_LDZ], s1 += src[(r + 1) * MLP_LDZ];
+                float t = s0 + s1;
+                if (halves) t += __shfl_xor(t, 32, 64);
+                if (lane < N) {
+                    float *dst = my + ly.p_db + lane;
+                    *dst = first ? t : *dst + t;
+                }
             }
             // ---- input gradient, the relu mask of the layer below, and this layer's fractional-bit gradient
             {
@@ -337,28 +407,46 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
                     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, wrow = kb * 32 + (lane & 31);
                     // gradient columns and kernel columns are zero padded to a multiple of 32
                     acc = MLP_CHAIN(true, false)(acc, cur + arow * MLP_LDZ + kq, 1, ws + wrow * ly.ldw + kq, 1, (N + 15) >> 4);
+                    MLP_STAMP(56 + (L - 1 - l));
                     const int kcol = kb * 32 + (lane & 31);
                     const bool mask_below = l > 0 && d.l[l - 1].h.act == HGQ_ACT_RELU;
+                    // this lane's sixteen rows are rb + {0..3, 8..11, 16..19, 24..27}: all its LDS reads are asked for first
+                    const int rb = rh * 32 + (lane >> 5) * 4;
+                    const float *raw_i = raw + rb * d.ld_raw + ly.acol + kcol, *rx_i = rx + rb * d.ld_rx + ly.acol + kcol;
+                    float *nxt_o = nxt + rb * MLP_LDZ + kcol;
+                    float a[16], q[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int rr = (r >> 2) * 8 + (r & 3);
+                        a[r] = raw_i[rr * d.ld_raw], q[r] = rx_i[rr * d.ld_rx];
+                    }
                     float dfsum = 0.f;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int row = rh * 32 + acc_row_(r, lane);
-                        const float a = raw[row * d.ld_raw + ly.acol + kcol];
-                        const float delta = rx[row * d.ld_rx + ly.acol + kcol] - a;
-                        if (kcol < K && r0 + row < rows) dfsum += -HGQ_LN2 * delta * acc[r];
-                        nxt[row * MLP_LDZ + kcol] = (kcol < K && (!mask_below || a > 0.f)) ? acc[r] : 0.f;
+                        const int rr = (r >> 2) * 8 + (r & 3);
+                        const float delta = q[r] - a[r];
+                        const float term = -HGQ_LN2 * delta * acc[r];
+                        dfsum += (kcol < K && rb + rr < live) ? term : 0.f;
+                    }
+                    if (l > 0) {  // (nobody reads the gradient at the stack's input)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            nxt_o[((r >> 2) * 8 + (r & 3)) * MLP_LDZ] = (kcol < K && (!mask_below || a[r] > 0.f)) ? acc[r] : 0.f;
                     }
                     dfsum += __shfl_xor(dfsum, 32, 64);
                     if (lane < 32 && kcol < K) dfs[(rh * HGQ_MLP_MAX_LAYERS + l) * 64 + kcol] += dfsum;  // this wavefront's own entry
                 }
             }
+            MLP_STAMP(41 + (L - 1 - l));
             __syncthreads();
+            MLP_STAMP(17 + (L - 1 - l));
             float *t = cur;
             cur = nxt;
             nxt = t;
         }
     }
     // ---- this workgroup's abs-max and fractional-bit sums
+    MLP_STAMP(30);
     for (int l = 0; l < L; ++l) {
         const MlpLayerDev &ly = d.l[l];
         if (tid < ly.h.K) {
@@ -366,6 +454,7 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
             ((uint32_t *)(my + ly.p_amax))[tid] = amx[l * 64 + tid];
         }
     }
+    MLP_STAMP(31);
 }
 
 __device__ __forceinline__ float sgd_clip(float w, float g, float lr, float l1, float lo, float hi) {
@@ -636,6 +725,12 @@ static inline int mlp_parts(int64_t rows) {
 }  // namespace hgq
 
 using namespace hgq;
+
+#ifdef MLP_PROF
+extern "C" int hgq_mlp_prof_read(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(mlp_prof_stamps), sizeof(unsigned long long) * 8 * 64) == hipSuccess ? 0 : -2;
+}
+#endif
 
 extern "C" int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, int64_t rows) {
     MlpDev d;

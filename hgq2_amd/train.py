@@ -8,6 +8,8 @@ propagate; ``w <- w - lr * g``; apply each variable's constraint.
 
 from __future__ import annotations
 
+import operator
+
 import torch
 
 from . import ops
@@ -183,6 +185,15 @@ class GraphedTrainStep:
         return self.loss
 
 
+_version_of = operator.attrgetter('_version')
+
+
+def _raw_stream(device_index: int) -> int:
+    """The current HIP stream of the device as an integer handle (the short way when this torch has it)."""
+    get = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+    return get(device_index) if get is not None else torch.cuda.current_stream(device_index).cuda_stream
+
+
 class FusedQDenseStack:
     """One SGD training step of a stack of :class:`QDense` layers with mean sparse categorical
     cross-entropy, executed by the whole-step kernels (two launches once the quantized weight image of
@@ -268,6 +279,11 @@ class FusedQDenseStack:
         self._versions = None
         self.device = layers[0]._kernel.device
         self.loss = torch.zeros((), dtype=torch.float32, device=self.device)
+        self._loss_ptr, self._ws_ptr = self.loss.data_ptr(), None
+        self._dev_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        self._K0 = int(arr[0].K)
+        self._need = {}  # rows -> workspace floats
+        self._decay_of = [(it, layer.iq.quantizer) for it, layer in zip(arr, layers)]
 
     def invalidate(self):
         """Forget the cached quantized-weight image (after writing the variables in a way neither version counters nor
@@ -285,27 +301,32 @@ class FusedQDenseStack:
     def step(self, x, labels):
         """Run one training step in place; returns the loss tensor (cross-entropy + sum of EBOPs * beta
         + MonoL1 regularisation terms, i.e. the full training loss)."""
-        ct, lib = self._ct, self._lib.load()
-        if not (x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == self._arr[0].K):
+        if not (x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == self._K0):
             raise ValueError('x must be a contiguous float32 GPU tensor [rows, K]')
-        if not (labels.is_cuda and labels.dtype == torch.int64 and labels.is_contiguous() and labels.shape == (x.shape[0],)):
-            raise ValueError('labels must be a contiguous int64 GPU tensor [rows]')
         rows = x.shape[0]
-        need = lib.hgq_mlp_workspace(self._arr, len(self.layers), rows)
-        if need < 0:
-            self._lib.check(-3, 'hgq_mlp_workspace')
-        for it, layer in zip(self._arr, self.layers):
-            it.decay = layer.iq.quantizer._decay_host  # follows the variable
+        if not (labels.is_cuda and labels.dtype == torch.int64 and labels.is_contiguous() and labels.shape == (rows,)):
+            raise ValueError('labels must be a contiguous int64 GPU tensor [rows]')
+        # (the host side of a step is a few microseconds of Python around one foreign call: at 16384 rows the two
+        # launches take the GPU about 30 us, so what is looked up per step is kept to what can change between steps)
+        lib = self._lib.load()
+        need = self._need.get(rows)
+        if need is None:
+            need = lib.hgq_mlp_workspace(self._arr, len(self.layers), rows)
+            if need < 0:
+                self._lib.check(-3, 'hgq_mlp_workspace')
+            self._need[rows] = need
+        for it, q in self._decay_of:
+            it.decay = q._decay_host  # follows the variable
         # the kernels of this class do not move version counters or the state epoch: both unchanged = nobody else wrote
-        versions = [t._version for t in self._vars] + [ops.STATE_EPOCH[0]]
+        versions = (*map(_version_of, self._vars), ops.STATE_EPOCH[0])
         current = self._versions == versions
         if self._ws is None or self._ws.numel() < need:
             self._ws = torch.empty(need, dtype=torch.float32, device=self.device)
-            current = False
-        rc = lib.hgq_mlp_train_step_cached(self._arr, len(self.layers), ct.c_void_p(x.data_ptr()), ct.c_void_p(labels.data_ptr()), rows,
-                                           self.lr, ct.c_void_p(self.loss.data_ptr()), ct.c_void_p(self._ws.data_ptr()), int(current),
-                                           ct.c_void_p(torch.cuda.current_stream().cuda_stream))
-        self._lib.check(rc, 'hgq_mlp_train_step_cached')
+            self._ws_ptr, current = self._ws.data_ptr(), False
+        rc = lib.hgq_mlp_train_step_cached(self._arr, len(self.layers), x.data_ptr(), labels.data_ptr(), rows, self.lr, self._loss_ptr,
+                                           self._ws_ptr, int(current), _raw_stream(self._dev_index))
+        if rc:
+            self._lib.check(rc, 'hgq_mlp_train_step_cached')
         self._versions = versions
         return self.loss
 
