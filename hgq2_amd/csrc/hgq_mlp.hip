@@ -144,17 +144,14 @@ __device__ __forceinline__ void mlp_snapshot_end(MlpSnapRow r, float *aux, int l
 
 __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const float *__restrict__ img, const float *__restrict__ x,
                                                           const int64_t *__restrict__ labels, int64_t rows,
-                                                          float *part, float *aux, uint32_t *ticket) {
+                                                          float *part, float *aux, uint32_t *loss_words) {
     extern __shared__ float lds[];
     __shared__ float loss_part[MLP_NT / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     MLP_STAMP(0);
-    // snapshot for the update pass: workgroup w's last wavefront takes row w; its loads travel with the image fetch below
+    // snapshot for the update pass: workgroup w's last wavefront takes row w, in a forward phase, where it has no other work
     const bool snap_wave = __builtin_amdgcn_readfirstlane(wave) == MLP_NT / 64 - 1;
-    MlpSnapRow snap;
-    snap.l = -1;
-    if (snap_wave) snap = mlp_snapshot_begin(d, (int)blockIdx.x, lane);
-    if (blockIdx.x == 0 && tid == 0) ticket[0] = 0u;  // the update pass counts its finished workgroups here
+    if (blockIdx.x == 0 && tid < 4) loss_words[tid] = 0u;  // the update pass adds up and counts its loss pieces here
     const int L = d.n_layers;
     float *raw = lds + d.off_raw, *rx = lds + d.off_rx;
     // [2][L][64] fractional-bit gradient sums: one set per row half of the tile, each entry owned by one wavefront for the
@@ -180,7 +177,8 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
     }
     MLP_STAMP(1);
     // fetch the quantized kernels / biases / rounded fractional bits (off_raw is a multiple of 4)
-    // (four 128-bit loads per thread in flight: one load per loop trip would cost a memory latency each)
+    // (four 128-bit loads per thread in flight: one load per loop trip would cost a memory latency each; the LDS
+    // clearing is done while the first batch travels)
     for (int id0 = 0; id0 < d.off_raw; id0 += 4 * 4 * MLP_NT) {
         float4 v[4];
 #pragma unroll
@@ -188,30 +186,28 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
             const int id = id0 + (u * MLP_NT + tid) * 4;
             v[u] = *(const float4 *)(img + (id < d.off_raw ? id : 0));
         }
+        if (id0 == 0) {
+            MLP_STAMP(2);
+            // padding columns of rx stay zero for good (rx starts at a multiple of four floats)
+            const int n_rx = MLP_BM * d.ld_rx;
+            for (int id = tid * 4; id + 3 < n_rx; id += 4 * MLP_NT) *(float4 *)(rx + id) = float4{0.f, 0.f, 0.f, 0.f};
+            if (tid < (n_rx & 3)) rx[(n_rx & ~3) + tid] = 0.f;
+            for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += MLP_NT) dfs[id] = 0.f, dfs[64 * HGQ_MLP_MAX_LAYERS + id] = 0.f, amx[id] = 0u;
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int id = id0 + (u * MLP_NT + tid) * 4;
             if (id < d.off_raw) *(float4 *)(lds + id) = v[u];
         }
     }
-    MLP_STAMP(2);
-    for (int id = tid; id < MLP_BM * d.ld_rx; id += MLP_NT) rx[id] = 0.f;  // padding columns stay zero for good
-    for (int id = tid; id < 64 * HGQ_MLP_MAX_LAYERS; id += MLP_NT) dfs[id] = 0.f, dfs[64 * HGQ_MLP_MAX_LAYERS + id] = 0.f, amx[id] = 0u;
     __syncthreads();
     MLP_STAMP(3);
-    if (snap_wave) {
-        mlp_snapshot_end(snap, aux, lane);
-        // fewer workgroups than rows (small batches): the remaining rows, one after the other
-        int total = 0;
-        for (int l = 0; l < L; ++l) total += d.l[l].h.K;
-        for (int row = (int)blockIdx.x + (int)gridDim.x; row < total; row += (int)gridDim.x) mlp_snapshot_end(mlp_snapshot_begin(d, row, lane), aux, lane);
-    }
-
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const bool first = tile == blockIdx.x;
         const int64_t r0 = tile * MLP_BM;
         const int live = (int)(rows - r0 < MLP_BM ? rows - r0 : MLP_BM);  // rows of this tile that exist
         // ---- stage the input tile: raw value, quantized value, abs-max
+        MLP_STAMP(60);
         {
             const MlpLayerDev &l0 = d.l[0];
             const int rm = Mode(l0.h.mode_in).round_mode;
@@ -223,6 +219,7 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
             const uint32_t by_k0 = ((1u << 20) + (uint32_t)K0 - 1u) / (uint32_t)K0;
             for (int id0 = 0; id0 < n_el; id0 += 4 * MLP_NT) {
                 float v[4];
+                MLP_STAMP(61);
                 if (first && id0 == 0) {
 #pragma unroll
                     for (int u = 0; u < 4; ++u) v[u] = pre[u];
@@ -255,6 +252,12 @@ __global__ __launch_bounds__(MLP_NT) void mlp_fwd_bwd_kernel(MlpDev d, const flo
             const MlpLayerDev &ly = d.l[l];
             const int N = ly.h.N;
             const int rh = wave & 1, cb = wave >> 1;
+            if (snap_wave && first && l == 0) {
+                // (fewer workgroups than rows - small batches: the remaining rows, one after the other)
+                int total = 0;
+                for (int j = 0; j < L; ++j) total += d.l[j].h.K;
+                for (int row = (int)blockIdx.x; row < total; row += (int)gridDim.x) mlp_snapshot_end(mlp_snapshot_begin(d, row, lane), aux, lane);
+            }
             if (wave < 4 && cb * 32 < ly.Np) {
                 floatx16 acc = {0};
                 const float *ws = lds + ly.off_w;
@@ -471,30 +474,38 @@ __device__ __forceinline__ float sgd_clip(float w, float g, float lr, float l1, 
 // input bit counts the EBOPs gradients need) without waiting for another workgroup; pre-update values of variables it
 // does not own come from the main kernel's snapshot.
 #define MLP_RG 16
-// The loss is the sum of one piece per workgroup (cross-entropy, a layer's ebops * beta, MonoL1 terms).  Every workgroup
-// leaves its piece in its own slot and draws a ticket; the one that draws the last ticket adds the slots in block order.
-// Slots and ticket are only touched by device-scope atomics (performed where all workgroups meet, no cache write-back),
-// and the ticket's operand depends on the value the slot's exchange returns, so a piece is in place before its
-// workgroup counts as finished.  The main kernel cleared the ticket.
-__device__ __forceinline__ void mlp_loss_piece(float piece, float *slots, uint32_t *ticket, float *loss, int lane) {
-    int last = 0;
-    if (lane == 0) {
-        const float before = __uint_as_float(atomicExch((uint32_t *)slots + blockIdx.x, __float_as_uint(piece)));
-        uint32_t one = 1u;
-        asm volatile("" : "+v"(one) : "v"(before));
-        last = atomicAdd(ticket, one) == gridDim.x - 1;
+// The loss is the sum of one piece per workgroup (cross-entropy, a layer's ebops * beta, MonoL1 terms), taken in fixed
+// point so that it does not depend on the order in which the workgroups arrive: ONE 64-bit atomic addition per workgroup
+// carries its piece (multiples of 2**-28 in bits 12 and up: exact for a piece of magnitude 1/16 and more, within 2**-28
+// otherwise) and counts it (bits 0 .. 10); the workgroup whose addition completes the count converts the sum - one
+// rounding - and clears the word for the next step.  A piece outside +-2**22 or not finite goes beside the sum: it is
+// left in `odd` (an exchange, whose result the addition's operand depends on, so it is in place before it is counted,
+// bit 11) and added to the converted sum by the last workgroup; with several such pieces in one step one of them is
+// reported (NaN if any is NaN ahead of it in arrival, which no run can tell from another NaN).  The main kernel cleared both words.
+#define MLP_LOSS_SCALE 268435456.0f  // 2**28
+__device__ __forceinline__ void mlp_loss_piece(float piece, unsigned long long *word, uint32_t *odd, float *loss, int lane) {
+    if (lane != 0) return;
+    unsigned long long add = 1ull;
+    const bool plain = fabsf(piece) < 4194304.0f;  // (false for NaN)
+    if (plain) {
+        add += (unsigned long long)((long long)(piece * MLP_LOSS_SCALE)) << 12;  // the product is exact, and an integer below 2**50
+    } else {
+        const uint32_t before = atomicExch(odd, __float_as_uint(piece));
+        uint32_t mark = 1u << 11;
+        asm volatile("" : "+v"(mark) : "v"(before));
+        add += mark;
     }
-    if (!__builtin_amdgcn_readfirstlane(last)) return;
-    float v = 0.f;  // lane j adds slots j, j + 64, ... in order; then the lanes in a fixed tree
-    for (int b = lane; b < (int)gridDim.x; b += 64) v += __uint_as_float(atomicOr((uint32_t *)slots + b, 0u));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    if (lane == 0) loss[0] = v;
+    const unsigned long long total = atomicAdd(word, add) + add;
+    if ((uint32_t)(total & 0x7ffull) != gridDim.x) return;
+    float v = (float)((double)((long long)total >> 12) * (1.0 / (double)MLP_LOSS_SCALE));
+    if (total & 0x800ull) v += __uint_as_float(atomicExch(odd, 0u));
+    loss[0] = v;
+    atomicExch(word, 0ull);
 }
 
 __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d, const float *__restrict__ part, int n_parts,
                                                                         const float *__restrict__ aux, float lr, float *loss, float *img,
-                                                                        float *loss_slots, uint32_t *ticket) {
+                                                                        unsigned long long *loss_word, uint32_t *loss_odd) {
     __shared__ float red[64 * MLP_RG];
     __shared__ uint32_t smx[64 * MLP_RG];
     __shared__ float val[64], bits_in[64], dbits_in[64], new_i[64];
@@ -542,6 +553,14 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
             v_w = h.f_in[t];
         }
     }
+    // what the first wavefront needs after the reduction is asked for now as well (the snapshot's column sums, tracked
+    // integer bits and fractional bits of feature t; beta): loads issued behind the barrier would each cost a trip to memory
+    float a_col = 0.f, a_i = 0.f, a_f = 0.f, beta = 0.f;
+    if (grp == 0 && !loss_block) {
+        const float *ax = aux + l * MLP_AUX + (e_local < K ? e_local : 0);
+        a_col = ax[0], a_i = ax[64], a_f = ax[128];
+        if (h.beta) beta = h.beta[0];
+    }
     // both reductions of a thread (its entry's sums, its feature's abs-max) with all loads of a 16-slice run in flight
     {
         float s = 0.f;
@@ -577,12 +596,11 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
             v += (red[e_local + 64 * w] + red[e_local + 64 * (w + 1)]) + (red[e_local + 64 * (w + 2)] + red[e_local + 64 * (w + 3)]);
         val[e_local] = v;
         if (!loss_block && e_local < K) {
-            const float *a = aux + l * MLP_AUX;
             uint32_t mx = smx[e_local];
             for (int w = 1; w < MLP_RG; ++w) mx = max(mx, smx[e_local + 64 * w]);
-            const float f = a[128 + e_local];
+            const float f = a_f;
             const float mi_ = ceil_log2_exact(__fadd_rn(__uint_as_float(mx), pow2(-f)));
-            const float ni = fmaxf(__fsub_rn(a[64 + e_local], h.decay), mi_);
+            const float ni = fmaxf(__fsub_rn(a_i, h.decay), mi_);
             const float sfi = __fadd_rn(rintf(ni), f);
             float b = sfi > 0.f ? sfi : 0.f;
             const Mode mi(h.mode_in);
@@ -596,11 +614,9 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     __builtin_amdgcn_wave_barrier();
     if (loss_block) {
-        if (loss) mlp_loss_piece(val[0], loss_slots, ticket, loss, t);
+        if (loss) mlp_loss_piece(val[0], loss_word, loss_odd, loss, t);
         return;
     }
-    const float *colsum = aux + l * MLP_AUX;
-    const float beta = h.beta ? h.beta[0] : 0.f;
     // d(ebops * beta) / d bits: the chain rule through ((total * par_factor) / n_parallel) * ebops_factor * beta
     const float gs = __fmul_rn(__fdiv_rn(__fmul_rn(beta, h.ebops_factor), h.n_parallel), h.par_factor);
     float reg = 0.f;  // MonoL1 regularisation loss of the trainable bit-width variables (pre-update values)
@@ -625,7 +641,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
                                                                     mk.overflow_mode, true);
         }
     } else if (role == 1) {
-        float part_e = t < K ? bits_in[t] * colsum[t] : 0.f;
+        float part_e = t < K ? bits_in[t] * a_col : 0.f;
         float bsum = 0.f;
         if (h.bias && t < N) {
             bsum = rintf(v_b);
@@ -658,7 +674,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
         if (t < K) {
             h.i_in[t] = new_i[t];
             reg += h.f_in_l1 * v_w;
-            const float f_new = sgd_clip(v_w, val[t] + dbits_in[t] * colsum[t] * gs, lr, h.f_in_l1, h.f_in_lo, h.f_in_hi);
+            const float f_new = sgd_clip(v_w, val[t] + dbits_in[t] * a_col * gs, lr, h.f_in_l1, h.f_in_lo, h.f_in_hi);
             h.f_in[t] = f_new;
             img[ly.off_f + t] = rintf(f_new);
         }
@@ -666,7 +682,7 @@ __global__ __launch_bounds__(64 * MLP_RG) void mlp_reduce_update_kernel(MlpDev d
     if (loss) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) reg += __shfl_xor(reg, o, 64);
-        mlp_loss_piece(ebops_term + reg, loss_slots, ticket, loss, t);
+        mlp_loss_piece(ebops_term + reg, loss_word, loss_odd, loss, t);
     }
 }
 
@@ -736,7 +752,7 @@ extern "C" int64_t hgq_mlp_workspace(const hgq_mlp_layer *layers, int n_layers, 
     MlpDev d;
     size_t lds_bytes;
     if (mlp_plan(layers, n_layers, d, lds_bytes)) return -1;
-    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX + d.off_raw + 4 + 64;  // (+ 64: slots of tiny stacks)
+    return (int64_t)(mlp_parts(rows > 0 ? rows : 1) + 1) * d.M + (int64_t)n_layers * MLP_AUX + d.off_raw + 4 + 64;  // (+ 64: the loss words and their alignment)
 }
 
 extern "C" int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_layers, const float *x, const int64_t *labels,
@@ -764,15 +780,14 @@ extern "C" int hgq_mlp_train_step_cached(const hgq_mlp_layer *layers, int n_laye
         hipLaunchKernelGGL(mlp_prep_kernel, dim3((d.off_raw + 255) / 256), dim3(256), 0, s, d, img);
         if ((rc = check_launch("hgq_mlp_train_step(prep)"))) return rc;
     }
-    // behind the snapshot: one loss slot per workgroup of the update pass and their ticket
-    float *loss_slots = reduced + (int64_t)n_layers * MLP_AUX;
+    // behind the snapshot: the word the update pass adds its loss pieces into (8-byte aligned) and the word beside it
+    uint32_t *loss_words = (uint32_t *)(((uintptr_t)(reduced + (int64_t)n_layers * MLP_AUX) + 7u) & ~(uintptr_t)7u);
     int blocks = 1;
     for (int l = 0; l < n_layers; ++l) blocks += (layers[l].K * layers[l].N + 63) / 64 + 2;
-    uint32_t *ticket = (uint32_t *)(loss_slots + blocks);
-    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, slices, reduced, ticket);
+    hipLaunchKernelGGL(mlp_fwd_bwd_kernel, dim3(parts), dim3(MLP_NT), lds_bytes, s, d, img, x, labels, rows, slices, reduced, loss_words);
     if ((rc = check_launch("hgq_mlp_train_step(fwd_bwd)"))) return rc;
-    hipLaunchKernelGGL(mlp_reduce_update_kernel, dim3(blocks), dim3(64 * MLP_RG), 0, s, d, slices, parts, reduced, lr, loss, img, loss_slots,
-                       ticket);
+    hipLaunchKernelGGL(mlp_reduce_update_kernel, dim3(blocks), dim3(64 * MLP_RG), 0, s, d, slices, parts, reduced, lr, loss, img,
+                       (unsigned long long *)loss_words, loss_words + 2);
     return check_launch("hgq_mlp_train_step(update)");
 }
 

@@ -1,6 +1,8 @@
 """GPU parity of the layer API (hgq2_amd.layers / quantizer / config) against the CPU oracle's
 restatement of the reference's Python, on identical weights and inputs."""
 
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -241,6 +243,35 @@ def test_fused_qdense_stack_step_is_the_same_bits_on_every_run(dev):
     assert s1.keys() == s2.keys()
     for n in s1:
         assert torch.equal(s1[n], s2[n]), n
+
+
+def test_fused_step_reports_a_label_outside_the_classes_and_recovers(dev):
+    """A label outside [0, classes) makes the step's loss NaN (the piece travels beside the fixed-point sum of the loss
+    pieces) and contributes no cross-entropy gradient; the next step with valid labels reports a finite loss again, the
+    one a stack that never saw the bad batch reports from the same variables."""
+    from hgq2_amd.train import FusedQDenseStack
+    from hgq2_amd.utils.models import qdense_mlp
+
+    dims = (16, 64, 32, 32, 5)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4096, dims[0], generator=g).to(dev)
+    labels = torch.randint(0, dims[-1], (4096,), generator=g).to(dev)
+    bad = labels.clone()
+    bad[17] = dims[-1]
+    bad[4000] = -1
+    src = ref.RefMLP(dims=dims, seed=6)
+    model = qdense_mlp(dims, device=dev)
+    _copy_mlp(src, model, dev)
+    fused = FusedQDenseStack(model, lr=0.01)
+    assert math.isfinite(float(fused.step(x, labels)))
+    assert math.isnan(float(fused.step(x, bad)))
+    state = {n: p.detach().clone() for n, p in model.state_dict().items()}
+    assert all(bool(torch.isfinite(v.float()).all()) for v in state.values()), 'the bad labels reached a variable'
+    after = float(fused.step(x, labels))
+    assert math.isfinite(after)
+    twin = qdense_mlp(dims, device=dev)
+    twin.load_state_dict(state)
+    assert float(FusedQDenseStack(twin, lr=0.01).step(x, labels)) == after
 
 
 def test_fused_stack_with_an_activation_on_the_output_layer(dev, acc64):
