@@ -23,12 +23,24 @@ namespace hgq {
 
 #define PG_WS 33  // row stride of the kernel matrix in LDS
 
+// Time stamps of workgroup 0 (measurement builds only: -DPG_PROF): [mode][wavefront][event]
+#ifdef PG_PROF
+__device__ unsigned long long pg_prof_stamps[2 * 8 * 32];
+#define PG_STAMP(i)                                                                                                          \
+    do {                                                                                                                     \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (i) < 32) pg_prof_stamps[(MODE * 8 + (threadIdx.x >> 6)) * 32 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define PG_STAMP(i)
+#endif
+
 __device__ __forceinline__ int pg_acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
 
 struct PatchPlan {
     int TH, TW, tiles_y, tiles_x;  // tile of row-space pixels
     int PH, PW, DS;                // patch of source pixels, pixel stride in words
     int D, N;                      // gathered depth, output channels
+    int patch_words;               // LDS words of the patch (fp32 form: PH * PW * DS; bf16 parts: PH * PW * D * 3 / 2)
     int RH, RW, SH, SW;            // row-space and source-space image sizes
 };
 
@@ -36,9 +48,23 @@ struct PatchPlan {
 // a thread = e * NT + thread.  The first PG_MAXU units of a thread are loaded into registers
 // (buffer loads, zeros outside the image) while the matrix cores still work on the previous
 // tile, and written to LDS afterwards; a larger patch stages the rest in place.
-#define PG_MAXU 6
+// (A workgroup of eight wavefronts keeps four: its threads are twice as many, and two such workgroups share a CU only
+// if a wavefront stays within 128 registers.)
+template <int MAXU>
 struct PatchRegs {
-    f32x4_t v[PG_MAXU], m[PG_MAXU];
+    f32x4_t v[MAXU], m[MAXU];
+    // where unit u of this thread sits in the patch - row << 20 | column << 8 | group of four depths, ~0 past the patch's
+    // end: the same for every tile, so the divisions that find it are done once per launch, not once per tile
+    uint32_t geo[MAXU];
+    template <int NT>
+    __device__ __forceinline__ void init(const PatchPlan &p) {
+        const int D4 = p.D >> 2, n_u = p.PH * p.PW * D4;
+#pragma unroll
+        for (int u = 0; u < MAXU; ++u) {
+            const int e = u * NT + (int)threadIdx.x, px = e / D4, pr = px / p.PW;
+            geo[u] = e < n_u ? ((uint32_t)pr << 20) | ((uint32_t)(px - pr * p.PW) << 8) | (uint32_t)(e - px * D4) : ~0u;
+        }
+    }
 };
 
 __device__ __forceinline__ uint32_t patch_unit_offset(const PatchPlan &p, int e, int n_u, int D4, int b, int sy0, int sx0, int &dst) {
@@ -51,35 +77,64 @@ __device__ __forceinline__ uint32_t patch_unit_offset(const PatchPlan &p, int e,
     return BUF_OOB;
 }
 
-template <bool MASKED, int NT>
-__device__ __forceinline__ void patch_fetch(PatchRegs &r, const __amdgpu_buffer_rsrc_t rs_src, const __amdgpu_buffer_rsrc_t rs_mask,
+template <bool MASKED, int NT, int MAXU>
+__device__ __forceinline__ void patch_fetch(PatchRegs<MAXU> &r, const __amdgpu_buffer_rsrc_t rs_src, const __amdgpu_buffer_rsrc_t rs_mask,
                                             const PatchPlan &p, int b, int sy0, int sx0) {
-    const int D4 = p.D >> 2, n_u = p.PH * p.PW * D4;
 #pragma unroll
-    for (int u = 0; u < PG_MAXU; ++u) {
-        int dst;
-        const uint32_t off = patch_unit_offset(p, u * NT + (int)threadIdx.x, n_u, D4, b, sy0, sx0, dst);
+    for (int u = 0; u < MAXU; ++u) {
+        const uint32_t gq = r.geo[u];
+        const int yy = sy0 + (int)(gq >> 20), xx = sx0 + (int)((gq >> 8) & 0xfffu);
+        const bool in = gq != ~0u && (unsigned)yy < (unsigned)p.SH && (unsigned)xx < (unsigned)p.SW;
+        const uint32_t off = in ? (uint32_t)(((b * p.SH + yy) * p.SW + xx) * p.D + 4 * (int)(gq & 0xffu)) * 4u : BUF_OOB;
         r.v[u] = buf_ld4(rs_src, off);
         if (MASKED) r.m[u] = buf_ld4(rs_mask, off);
     }
 }
 
-template <bool MASKED, int NT>
-__device__ __forceinline__ void patch_stash(float *patch, const PatchRegs &r, const __amdgpu_buffer_rsrc_t rs_src,
-                                            const __amdgpu_buffer_rsrc_t rs_mask, bool use_mask, const PatchPlan &p, int b, int sy0,
-                                            int sx0) {
-    const int D4 = p.D >> 2, n_u = p.PH * p.PW * D4;
+// The patch in LDS, two forms.  fp32: pixel px, depth d at word px * DS + d (DS = D + 1).  bf16 parts (D = 16, 32 or 64): every
+// value as its three exact bf16 parts (hgq_device.h: an fp32 number is the sum of three numbers of eight significant bits),
+// split ONCE here instead of at each of the kh * kw reads; a pixel is 3 * D / 8 slots of 16 bytes - part-major, eight
+// consecutive depths per slot - so a lane's A operand of a 32x32x16 bf16 instruction is one 128-bit read per part.  Slot
+// c of a pixel sits at c ^ ((px >> (4 - j)) & (D / 8 - 1)), j = log2(D / 8): with a pixel stride of 3 * 2**j slots, sixteen
+// consecutive pixels then read sixteen different 16-byte bank groups (no padding: the patch and the kernel matrix of a
+// 3 x 3 x 32 layer fill the 80 KB that let two workgroups share a CU).
+__device__ __forceinline__ void put_unit_f32(float *patch, int DS, int px, int d4, const f32x4_t &v) {
 #pragma unroll
-    for (int u = 0; u < PG_MAXU; ++u) {
-        const int e = u * NT + (int)threadIdx.x;
-        if (e < n_u) {
-            const int px = e / D4, dst = px * p.DS + 4 * (e - px * D4);
+    for (int j = 0; j < 4; ++j) patch[px * DS + 4 * d4 + j] = v[j];
+}
+__device__ __forceinline__ void put_unit_parts(float *patch, int nch, int jbits, int px, int d4, const f32x4_t &v, uint32_t &nz) {
+    uint32_t h[4], m[4], l[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) patch[dst + j] = (!MASKED || !use_mask || r.m[u][j] > 0.f) ? r.v[u][j] : 0.f;
+    for (int j = 0; j < 4; ++j) bf16_parts(v[j], h[j], m[j], l[j]);
+    const int pos = (d4 >> 1) ^ ((px >> (4 - jbits)) & (nch - 1));
+    uint2 *dst = (uint2 *)patch + (px * 3 * nch + pos) * 2 + (d4 & 1);
+    dst[0] = uint2{bf16_pair(h[0], h[1]), bf16_pair(h[2], h[3])};
+    dst[2 * nch] = uint2{bf16_pair(m[0], m[1]), bf16_pair(m[2], m[3])};
+    dst[4 * nch] = uint2{bf16_pair(l[0], l[1]), bf16_pair(l[2], l[3])};
+    // which parts the tile needs at all (bit 0: a second part, bit 1: a third one; a third part implies a second)
+    nz |= ((m[0] | m[1] | m[2] | m[3]) != 0u ? 1u : 0u) | ((l[0] | l[1] | l[2] | l[3]) != 0u ? 2u : 0u);
+}
+
+template <bool MASKED, int NT, int MAXU, bool PARTS>
+__device__ __forceinline__ uint32_t patch_stash(float *patch, const PatchRegs<MAXU> &r, const __amdgpu_buffer_rsrc_t rs_src,
+                                                const __amdgpu_buffer_rsrc_t rs_mask, bool use_mask, const PatchPlan &p, int b, int sy0,
+                                                int sx0) {
+    const int D4 = p.D >> 2, n_u = p.PH * p.PW * D4, nch = p.D >> 3, jbits = 31 - __clz(nch);
+    uint32_t nz = 0u;
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+        const uint32_t gq = r.geo[u];
+        if (gq != ~0u) {
+            const int px = (int)(gq >> 20) * p.PW + (int)((gq >> 8) & 0xfffu), d4 = (int)(gq & 0xffu);
+            f32x4_t v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = (!MASKED || !use_mask || r.m[u][j] > 0.f) ? r.v[u][j] : 0.f;
+            if (PARTS) put_unit_parts(patch, nch, jbits, px, d4, v, nz);
+            else put_unit_f32(patch, p.DS, px, d4, v);
         }
     }
     // the rest of a large patch, four units in flight
-    for (int e0 = PG_MAXU * NT; e0 < n_u; e0 += 4 * NT) {
+    for (int e0 = MAXU * NT; e0 < n_u; e0 += 4 * NT) {
         f32x4_t v[4], m[4];
         int dst[4];
 #pragma unroll
@@ -91,11 +146,40 @@ __device__ __forceinline__ void patch_stash(float *patch, const PatchRegs &r, co
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             if (dst[u] >= 0) {
+                const int e = e0 + u * NT + (int)threadIdx.x, px = e / D4, d4 = e - px * D4;
+                f32x4_t w;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) patch[dst[u] + j] = (!MASKED || !use_mask || m[u][j] > 0.f) ? v[u][j] : 0.f;
+                for (int j = 0; j < 4; ++j) w[j] = (!MASKED || !use_mask || m[u][j] > 0.f) ? v[u][j] : 0.f;
+                if (PARTS) put_unit_parts(patch, nch, jbits, px, d4, w, nz);
+                else put_unit_f32(patch, p.DS, px, d4, w);
             }
         }
     }
+    return nz;
+}
+
+// One batch of sixteen contraction steps with the A operand already in bf16 parts (n_a of them are not all zero in this
+// tile) and B as fp32 values from LDS: B's leading parts are one byte-permute per pair; its further parts are formed only
+// where some lane of the wavefront has them.  Every product of two parts is exact in fp32; only the accumulation rounds.
+__device__ __forceinline__ floatx16 mfma_batch_parts_a(floatx16 acc, const u32x4_t (&a)[3], int n_a, const float (&b)[8]) {
+    u32x4_t pb0;
+    const bool one_b = bf16_lead8(b, pb0);
+    acc = mfma_bf16(a[0], pb0, acc);
+    if (n_a > 1) acc = mfma_bf16(a[1], pb0, acc);
+    if (n_a > 2) acc = mfma_bf16(a[2], pb0, acc);
+    if (!one_b) {
+        u32x4_t p1, p2;
+        const bool third = bf16_rest8(b, p1, p2);
+        acc = mfma_bf16(a[0], p1, acc);
+        if (n_a > 1) acc = mfma_bf16(a[1], p1, acc);
+        if (n_a > 2) acc = mfma_bf16(a[2], p1, acc);
+        if (third) {
+            acc = mfma_bf16(a[0], p2, acc);
+            if (n_a > 1) acc = mfma_bf16(a[1], p2, acc);
+            if (n_a > 2) acc = mfma_bf16(a[2], p2, acc);
+        }
+    }
+    return acc;
 }
 
 // Position (ty << 16 | tx) of tile row `rr` for a tile TW pixels wide.
@@ -110,19 +194,22 @@ __device__ __forceinline__ int tile_pos_advance(int pos, int by, int TW) {  // b
 }
 
 // MODE 0: forward; MODE 1: data gradient.  NW wavefronts, each owning 32 rows of the tile.
-// BF: the contraction runs on the bf16 matrix instruction over exact bf16 parts of the fp32 operands (mfma_chain_bf16: same
-// LDS reads, the same values up to the order of the fp32 additions); the source of the data gradient is an arbitrary fp32 tensor.
-template <int MODE, int NW, bool BF = false>
-__global__ __launch_bounds__(NW * 64) void pgemm_kernel(const float *__restrict__ src, const float *__restrict__ mask,
+// BF = 1: the contraction runs on the bf16 matrix instruction over exact bf16 parts of the fp32 operands, formed at each LDS read
+// (mfma_chain_bf16: same LDS reads, the same values up to the order of the fp32 additions); the source of the data gradient
+// is an arbitrary fp32 tensor.  BF = 2 (D = 16, 32 or 64): the patch is staged as bf16 parts, see put_unit_parts.
+template <int MODE, int NW, int BF = 0>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 4 : 2) void pgemm_kernel(const float *__restrict__ src, const float *__restrict__ mask,
                                                        const float *__restrict__ w, const float *__restrict__ bias,
                                                        float *__restrict__ out, hgq_conv_geom g, int F, int act, PatchPlan p) {
     constexpr int NT = NW * 64;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int taps = g.kh * g.kw, K = taps * p.D;
     float *wl = lds, *patch = lds + ((K * PG_WS + 3) & ~3);
+    uint32_t *part_flags = (uint32_t *)(patch + p.patch_words);  // [2], BF == 2 forward only
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, kq = lane >> 5, n = lane & 31;
     const int64_t src_bytes = (int64_t)g.B * p.SH * p.SW * p.D * 4;
     const __amdgpu_buffer_rsrc_t rs_src = buf_rsrc(src, src_bytes), rs_mask = buf_rsrc(mask ? mask : src, mask ? src_bytes : 0);
+    const __amdgpu_buffer_rsrc_t rs_out = buf_rsrc(out, (int64_t)g.B * p.RH * p.RW * p.N * 4);
     const int tiles_per_image = p.tiles_y * p.tiles_x;
     const int64_t n_tiles = (int64_t)g.B * tiles_per_image;
     // source origin of a tile
@@ -133,54 +220,86 @@ __global__ __launch_bounds__(NW * 64) void pgemm_kernel(const float *__restrict_
         sy0 = MODE == 0 ? ty0 * g.sy - g.py : ty0 + g.py - (g.kh - 1) * g.dly;
         sx0 = MODE == 0 ? tx0 * g.sx - g.px : tx0 + g.px - (g.kw - 1) * g.dlx;
     };
-    PatchRegs pre;
+    PatchRegs<(NW == 8 ? 4 : 6)> pre;
+    pre.template init<NT>(p);
     int64_t tile = blockIdx.x;
     int b, ty0, tx0, sy0, sx0;
+    PG_STAMP(0);
+    if (BF == 2 && MODE == 0 && tid < 2) part_flags[tid] = 0u;
     if (tile < n_tiles) {
         origin(tile, b, ty0, tx0, sy0, sx0);
         patch_fetch<MODE == 1, NT>(pre, rs_src, rs_mask, p, b, sy0, sx0);  // in flight during the set-up below
     }
-    // kernel matrix B[k = (tap, d)][n] -> wl[k][n], zero for n >= N; eight loads per thread in flight
-    // (one load per loop trip would cost a full memory latency each)
+    // kernel matrix B[k = (tap, d)][n] -> wl[k][n], zero for n >= N.  128-bit loads, six or twelve per thread in flight (the matrix
+    // is a few tens of KB in L2: what costs is a memory latency per loop trip, so a trip moves 24 or 48 values per thread);
+    // a forward kernel matrix whose rows are not a multiple of four values wide goes value by value
     {
         const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(w, (int64_t)K * p.N * 4);
         const int dshift = (p.D & (p.D - 1)) == 0 ? __builtin_ctz(p.D) : -1;
-        for (int id0 = 0; id0 < K * 32; id0 += 8 * NT) {
-            float v[8];
-            int dst[8];
+        if (MODE == 1 || (p.N & 3) == 0) {
+            const int D4 = p.D >> 2, n_u = MODE == 0 ? K * 8 : taps * 32 * D4;
+            constexpr int WU = NW == 8 ? 6 : 12;  // units of a thread per trip
+            for (int id0 = 0; id0 < n_u; id0 += WU * NT) {
+                f32x4_t v[WU];
+                int dst[WU];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int id = id0 + u * NT + tid;
-                uint32_t off = BUF_OOB;
-                dst[u] = -1;
-                if (id < K * 32) {
-                    if (MODE == 0) {
+                for (int u = 0; u < WU; ++u) {
+                    const int id = id0 + u * NT + tid;
+                    uint32_t off = BUF_OOB;
+                    dst[u] = -1;
+                    if (id < n_u) {
+                        if (MODE == 0) {
+                            const int k = id >> 3, n4 = (id & 7) * 4;
+                            dst[u] = k * PG_WS + n4;
+                            if (n4 < p.N) off = (uint32_t)(k * p.N + n4) * 4u;
+                        } else {
+                            // W[tap][c = n][f = d]: consecutive threads take consecutive groups of four f
+                            const int r = dshift >= 2 ? id >> (dshift - 2) : id / D4, d = (id - r * D4) * 4, nn = r & 31, tap = r >> 5;
+                            dst[u] = (tap * p.D + d) * PG_WS + nn;
+                            if (nn < p.N) off = (uint32_t)((tap * p.N + nn) * F + d) * 4u;
+                        }
+                    }
+                    v[u] = buf_ld4(rs_w, off);
+                }
+#pragma unroll
+                for (int u = 0; u < WU; ++u)
+                    if (dst[u] >= 0) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) wl[dst[u] + (MODE == 0 ? j : j * PG_WS)] = v[u][j];
+                    }
+            }
+        } else {
+            for (int id0 = 0; id0 < K * 32; id0 += 8 * NT) {
+                float v[8];
+                int dst[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int id = id0 + u * NT + tid;
+                    uint32_t off = BUF_OOB;
+                    dst[u] = -1;
+                    if (id < K * 32) {
                         const int k = id >> 5, nn = id & 31;
                         dst[u] = k * PG_WS + nn;
                         if (nn < p.N) off = (uint32_t)(k * p.N + nn) * 4u;
-                    } else {
-                        // W[tap][c = n][f = d]: consecutive threads take consecutive f
-                        const int r = dshift >= 0 ? id >> dshift : id / p.D, d = id - r * p.D, nn = r & 31, tap = r >> 5;
-                        dst[u] = (tap * p.D + d) * PG_WS + nn;
-                        if (nn < p.N) off = (uint32_t)((tap * p.N + nn) * F + d) * 4u;
                     }
+                    v[u] = buf_ld1(rs_w, off);
                 }
-                v[u] = buf_ld1(rs_w, off);
-            }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (dst[u] >= 0) wl[dst[u]] = v[u];
+                for (int u = 0; u < 8; ++u)
+                    if (dst[u] >= 0) wl[dst[u]] = v[u];
+            }
         }
     }
     // tile-relative position of the row this lane feeds to the matrix cores, and of its 16 result
     // rows (one division, the others follow by stepping)
     const int n_rows = p.TH * p.TW;
     const int r_lane = wave * 32 + (lane & 31);
-    int rowbase = 0;
+    int rowpix = 0;  // the patch pixel under tap (0, 0) of this lane's row
     if (r_lane < n_rows) {
         const int pos = tile_pos(r_lane, p.TW), ty = pos >> 16, tx = pos & 0xffff;
-        rowbase = MODE == 0 ? (ty * g.sy * p.PW + tx * g.sx) * p.DS : (ty * p.PW + tx) * p.DS;
+        rowpix = MODE == 0 ? ty * g.sy * p.PW + tx * g.sx : ty * p.PW + tx;
     }
+    const int rowbase = rowpix * p.DS;
     int rpos[16];
     {
         int pos4 = tile_pos(wave * 32 + (lane >> 5) * 4, p.TW);  // row of register 0
@@ -197,10 +316,27 @@ __global__ __launch_bounds__(NW * 64) void pgemm_kernel(const float *__restrict_
         }
     }
     const float bb = (MODE == 0 && bias && n < p.N) ? bias[n] : 0.f;
-    for (; tile < n_tiles; tile += gridDim.x) {
+    PG_STAMP(1);
+    int it_ = 0;
+    for (; tile < n_tiles; tile += gridDim.x, ++it_) {
         __syncthreads();  // the previous tile's operand reads are done (and, the first time, wl is written)
-        patch_stash<MODE == 1, NT>(patch, pre, rs_src, rs_mask, mask != nullptr, p, b, sy0, sx0);
+        PG_STAMP(2 + 8 * it_);
+        const uint32_t nz = patch_stash<MODE == 1, NT, (NW == 8 ? 4 : 6), BF == 2>(patch, pre, rs_src, rs_mask, mask != nullptr, p, b, sy0, sx0);
+        if (BF == 2 && MODE == 0) {
+            const uint32_t any_nz = (__any((nz & 1u) != 0u) ? 1u : 0u) | (__any((nz & 2u) != 0u) ? 2u : 0u);
+            if (lane == 0 && any_nz) atomicOr(&part_flags[it_ & 1], any_nz);
+        }
+        PG_STAMP(3 + 8 * it_);
         __syncthreads();
+        PG_STAMP(4 + 8 * it_);
+        // parts of the activations this tile needs (the gradient of the data-gradient pass always has three); the other
+        // flag word is cleared for the next tile: its last readers passed the barrier at the top of this trip
+        int n_a = 3;
+        if (BF == 2 && MODE == 0) {
+            const uint32_t f = __builtin_amdgcn_readfirstlane(part_flags[it_ & 1]);
+            n_a = (f & 2u) ? 3 : ((f & 1u) ? 2 : 1);
+            if (tid == 0) part_flags[(it_ + 1) & 1] = 0u;
+        }
         const int cb = b, cty0 = ty0, ctx0 = tx0;
         const int64_t next = tile + gridDim.x;
         if (next < n_tiles) {
@@ -208,16 +344,32 @@ __global__ __launch_bounds__(NW * 64) void pgemm_kernel(const float *__restrict_
             patch_fetch<MODE == 1, NT>(pre, rs_src, rs_mask, p, b, sy0, sx0);  // lands while the matrix cores work
         }
         floatx16 acc = {0};
+        PG_STAMP(5 + 8 * it_);
         if (wave * 32 < n_rows) {
             for (int tap = 0; tap < taps; ++tap) {
                 const int ky = tap / g.kw, kx = tap - ky * g.kw;
-                const int tapoff = MODE == 0 ? (ky * g.dly * p.PW + kx * g.dlx) * p.DS
-                                             : ((g.kh - 1 - ky) * g.dly * p.PW + (g.kw - 1 - kx) * g.dlx) * p.DS;
+                const int tappix = MODE == 0 ? ky * g.dly * p.PW + kx * g.dlx : (g.kh - 1 - ky) * g.dly * p.PW + (g.kw - 1 - kx) * g.dlx;
+                if (BF == 2) {
+                    // lane half kq takes depths 8 kq .. 8 kq + 7 of each batch of sixteen: one 128-bit read per part of A
+                    const int nch = p.D >> 3, px = rowpix + tappix, sw = (px >> (4 - (31 - __clz(nch)))) & (nch - 1);
+                    const u32x4_t *pa = (const u32x4_t *)patch + px * 3 * nch;
+                    const float *bp8 = wl + (tap * p.D + 8 * kq) * PG_WS + n;
+                    for (int bt = 0; bt < (p.D >> 4); ++bt) {
+                        const int pos = (2 * bt + kq) ^ sw;
+                        const u32x4_t a[3] = {pa[pos], pa[nch + pos], pa[2 * nch + pos]};
+                        float bq[8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) bq[e] = bp8[(16 * bt + e) * PG_WS];
+                        acc = mfma_batch_parts_a(acc, a, MODE == 1 ? 3 : n_a, bq);
+                    }
+                    continue;
+                }
+                const int tapoff = tappix * p.DS;
                 const float *ap = patch + rowbase + tapoff + kq;
                 const float *bp = wl + (tap * p.D + kq) * PG_WS + n;
                 // eight depth steps at a time, operands read ahead of the matrix instructions (D is a multiple of 4)
                 int d = 0;
-                if (BF) {
+                if (BF == 1) {
                     for (; d + 16 <= p.D; d += 16) acc = mfma_chain_bf16<MODE == 1, false>(acc, ap + d, 1, bp + d * PG_WS, PG_WS, 1);
                 }
                 for (; d + 16 <= p.D; d += 16) {
@@ -233,26 +385,27 @@ __global__ __launch_bounds__(NW * 64) void pgemm_kernel(const float *__restrict_
                     acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc, 0, 0, 0);
                 }
             }
-            if (n < p.N) {
+            PG_STAMP(6 + 8 * it_);
+            {
+                // through a descriptor: a row outside the tile or the image, or a column past N, is dropped by its offset
                 const int y_end = min(cty0 + p.TH, p.RH);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    if (rpos[r] < 0) continue;
                     const int ry = cty0 + (rpos[r] >> 16), rx = ctx0 + (rpos[r] & 0xffff);
-                    if (ry < y_end && rx < p.RW) {
-                        float v = acc[r] + bb;
-                        if (MODE == 0 && act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
-                        out[(((int64_t)cb * p.RH + ry) * p.RW + rx) * p.N + n] = v;
-                    }
+                    const bool ok = rpos[r] >= 0 && ry < y_end && rx < p.RW && n < p.N;
+                    float v = acc[r] + bb;
+                    if (MODE == 0 && act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
+                    buf_st1(rs_out, ok ? (uint32_t)(((cb * p.RH + ry) * p.RW + rx) * p.N + n) * 4u : BUF_OOB, v);
                 }
             }
+            PG_STAMP(7 + 8 * it_);
         }
     }
 }
 
 #define PG_MAX_LDS (80 * 1024)  // two workgroups per CU
 
-static bool plan_patch(int mode, const hgq_conv_geom &g, int F, PatchPlan &p, size_t &lds) {
+static bool plan_patch(int mode, const hgq_conv_geom &g, int F, bool parts, PatchPlan &p, size_t &lds) {
     p.D = mode == 0 ? g.C : F, p.N = mode == 0 ? F : g.C;
     p.RH = mode == 0 ? g.OH : g.H, p.RW = mode == 0 ? g.OW : g.W;
     p.SH = mode == 0 ? g.H : g.OH, p.SW = mode == 0 ? g.W : g.OW;
@@ -260,6 +413,9 @@ static bool plan_patch(int mode, const hgq_conv_geom &g, int F, PatchPlan &p, si
     if (p.D % 4 != 0 || p.N > 32 || K * PG_WS * 4 > 48 * 1024 || (int64_t)p.RH * p.RW < 32) return false;
     if (mode == 1 && (g.sy != 1 || g.sx != 1)) return false;
     if ((int64_t)g.B * p.SH * p.SW * p.D * 4 >= (1ll << 31) || p.RH >= 32768 || p.RW >= 32768) return false;
+    if ((int64_t)g.B * p.RH * p.RW * p.N * 4 >= (1ll << 31)) return false;
+    if (parts && p.D != 16 && p.D != 32 && p.D != 64) return false;
+    if (p.D > 1020) return false;  // (a thread's place in the patch is packed into one register: 12 + 12 + 8 bits)
     p.DS = p.D + 1;
     p.TW = p.RW < 32 ? p.RW : 32;
     p.tiles_x = (p.RW + p.TW - 1) / p.TW;
@@ -269,8 +425,9 @@ static bool plan_patch(int mode, const hgq_conv_geom &g, int F, PatchPlan &p, si
         p.TH = (p.RH + tiles_y - 1) / tiles_y, p.tiles_y = tiles_y;
         p.PH = mode == 0 ? (p.TH - 1) * g.sy + (g.kh - 1) * g.dly + 1 : p.TH + (g.kh - 1) * g.dly;
         p.PW = mode == 0 ? (p.TW - 1) * g.sx + (g.kw - 1) * g.dlx + 1 : p.TW + (g.kw - 1) * g.dlx;
-        lds = wbytes + (size_t)p.PH * p.PW * p.DS * 4;
-        if (lds <= PG_MAX_LDS) return (int64_t)p.TH * p.TW >= 16;
+        p.patch_words = parts ? p.PH * p.PW * p.D * 3 / 2 : p.PH * p.PW * p.DS;
+        lds = wbytes + (size_t)p.patch_words * 4 + 16;  // (+ 16: the two part-flag words behind the patch)
+        if (lds <= PG_MAX_LDS) return (int64_t)p.TH * p.TW >= 16 && p.PH < 4096 && p.PW < 4096;
     }
     return false;
 }
@@ -282,25 +439,35 @@ static int patch_grid(const hgq_conv_geom &g, const PatchPlan &p, size_t lds) {
     return persistent_grid((int64_t)g.B * p.tiles_y * p.tiles_x, per_cu);
 }
 
+#ifdef PG_PROF
+extern "C" int hgq_pg_prof_read(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(pg_prof_stamps), sizeof(unsigned long long) * 2 * 8 * 32) == hipSuccess ? 0 : -2;
+}
+#endif
+
 bool conv_patch_ok(int mode, const hgq_conv_geom &g, int F) {
     PatchPlan p;
     size_t lds;
-    return plan_patch(mode, g, F, p, lds);
+    return plan_patch(mode, g, F, false, p, lds);
 }
 
 int conv_patch_launch(int mode, const float *src, const float *mask, const float *w, const float *bias, float *out,
                       const hgq_conv_geom &g, int F, int act, hipStream_t s) {
     PatchPlan p;
     size_t lds;
-    if (!plan_patch(mode, g, F, p, lds)) return fail(HGQ_ERR_UNSUPPORTED, "conv_patch_launch: shape not covered");
+    // the form of the patch: bf16 parts where the matrix cores run on them and the depth allows, else fp32
+    const bool bf = hgq_dense_use_bf16_parts(-1) != 0;
+    const bool parts = bf && plan_patch(mode, g, F, true, p, lds);
+    if (!parts && !plan_patch(mode, g, F, false, p, lds)) return fail(HGQ_ERR_UNSUPPORTED, "conv_patch_launch: shape not covered");
     const dim3 grid((unsigned)patch_grid(g, p, lds));
     const bool wide = p.TH * p.TW > 128;  // eight wavefronts of 32 rows
     // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
     static bool allowed = false;
     if (!allowed) {
-        const void *kernels[8] = {(const void *)pgemm_kernel<0, 4>, (const void *)pgemm_kernel<0, 8>, (const void *)pgemm_kernel<1, 4>,
-                                  (const void *)pgemm_kernel<1, 8>, (const void *)pgemm_kernel<0, 4, true>, (const void *)pgemm_kernel<0, 8, true>,
-                                  (const void *)pgemm_kernel<1, 4, true>, (const void *)pgemm_kernel<1, 8, true>};
+        const void *kernels[12] = {(const void *)pgemm_kernel<0, 4, 0>, (const void *)pgemm_kernel<0, 8, 0>, (const void *)pgemm_kernel<1, 4, 0>,
+                                   (const void *)pgemm_kernel<1, 8, 0>, (const void *)pgemm_kernel<0, 4, 1>, (const void *)pgemm_kernel<0, 8, 1>,
+                                   (const void *)pgemm_kernel<1, 4, 1>, (const void *)pgemm_kernel<1, 8, 1>, (const void *)pgemm_kernel<0, 4, 2>,
+                                   (const void *)pgemm_kernel<0, 8, 2>, (const void *)pgemm_kernel<1, 4, 2>, (const void *)pgemm_kernel<1, 8, 2>};
         for (const void *k : kernels)
             if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, PG_MAX_LDS) != hipSuccess)
                 return fail(HGQ_ERR_LAUNCH, "conv_patch_launch: cannot raise the dynamic LDS limit");
@@ -313,8 +480,9 @@ int conv_patch_launch(int mode, const float *src, const float *mask, const float
         else if (wide) hipLaunchKernelGGL((pgemm_kernel<1, 8, BFV>), grid, dim3(512), lds, s, src, mask, w, bias, out, g, F, act, p); \
         else hipLaunchKernelGGL((pgemm_kernel<1, 4, BFV>), grid, dim3(256), lds, s, src, mask, w, bias, out, g, F, act, p); \
     } while (0)
-    if (hgq_dense_use_bf16_parts(-1)) PG_LAUNCH(true);
-    else PG_LAUNCH(false);
+    if (parts) PG_LAUNCH(2);
+    else if (bf) PG_LAUNCH(1);
+    else PG_LAUNCH(0);
 #undef PG_LAUNCH
     return check_launch("conv_patch_launch");
 }
