@@ -1528,6 +1528,7 @@ extern "C" int64_t hgq_conv2d_bwd_workspace(const hgq_conv_geom *g, int F) {
     const WgradCfg c = wgrad_cfg(K, F);
     int64_t slices = wgrad_splits(rows, c.n_kt * c.n_nt);
     if (bwd_smallc_ok(*g, F) && bwd_smallc_grid(*g) > slices) slices = bwd_smallc_grid(*g);
+    if (conv_patch_wgrad_ok(*g, F) && conv_patch_wgrad_slices(*g, F) > slices) slices = conv_patch_wgrad_slices(*g, F);
     return slices * ((int64_t)K * F + F);
 }
 
@@ -1544,6 +1545,7 @@ extern "C" int64_t hgq_conv2d_bwd_slice_count(const hgq_conv_geom *g, int F) {
     const int64_t rows = (int64_t)g->B * g->OH * g->OW;
     if (rows == 0) return 1;
     if (bwd_smallc_ok(*g, F)) return bwd_smallc_grid(*g);
+    if (conv_patch_wgrad_ok(*g, F)) return conv_patch_wgrad_slices(*g, F);
     const WgradCfg c = wgrad_cfg(g->kh * g->kw * g->C, F);
     return wgrad_splits(rows, c.n_kt * c.n_nt);
 }
@@ -1624,8 +1626,22 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
     }
     if (dqw || dqb) {
         if (!workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null workspace");
+        const int64_t M = KF + F;
+        // small feature maps: both operands of a band of an image staged once in LDS (the slice count is a function of the
+        // shape alone, so operands that are not 16-byte aligned keep it and go through the gathered kernels below)
+        const bool patch_shape = conv_patch_wgrad_ok(*g, F);
+        const int64_t patch_slices = patch_shape ? conv_patch_wgrad_slices(*g, F) : 0;
+        if (patch_shape && aligned16(xq) && aligned16(dy) && (!mask || aligned16(mask))) {
+            if ((rc = conv_patch_wgrad_launch(xq, dy, mask, workspace, *g, F, act, s))) return rc;
+            if (reduce && (rc = reduce_parts(workspace, (int)patch_slices, M, dqw, KF, dqb, (int64_t)F, nullptr, 0, s))) return rc;
+            return HGQ_OK;
+        }
         const WgradCfg c = wgrad_cfg(K, F);
-        const int64_t splits = wgrad_splits(rows, c.n_kt * c.n_nt);
+        int64_t splits = wgrad_splits(rows, c.n_kt * c.n_nt);
+        if (patch_shape) {
+            if (splits > patch_slices) splits = patch_slices;
+            if (splits < patch_slices && !reduce && (rc = fill_f32(workspace + splits * M, 0.f, (patch_slices - splits) * M, s))) return rc;
+        }
         int64_t chunk = (rows + splits - 1) / splits;
         chunk = (chunk + 127) / 128 * 128;
         const dim3 grid((unsigned)(c.n_kt * c.n_nt), (unsigned)splits);
@@ -1648,7 +1664,6 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
         else HGQ_WGRAD(4, 1, 1);
 #undef HGQ_WGRAD
         if ((rc = check_launch("hgq_conv2d_bwd(weights)"))) return rc;
-        const int64_t M = KF + F;
         if (reduce && (rc = reduce_parts(workspace, (int)splits, M, dqw, KF, dqb, (int64_t)F, nullptr, 0, s))) return rc;
     }
     return HGQ_OK;

@@ -487,4 +487,278 @@ int conv_patch_launch(int mode, const float *src, const float *mask, const float
     return check_launch("conv_patch_launch");
 }
 
+// ---- weight / bias gradient -------------------------------------------------------------------
+// dW[ky][kx][c][f] = sum over output pixels of x[oy + ky - py][ox + kx - px][c] * dz[oy][ox][f]  (unit stride and dilation).
+// The gathered form reads every source element kh * kw times through L2 and every dz element once per block of the
+// gathered matrix; here a workgroup stages a band of ONE image once - the source patch as fp32 (pixel p of the padded
+// raster, XW = OW + kw - 1 pixels wide, at word p * XS), dz laid out on the SAME raster (zeros in the kw - 1 columns past OW,
+// ReLU mask applied) - so that the contraction index q runs over the raster and tap (ky, kx) reads source pixel
+// q + ky * XW + kx: no index arithmetic in the loop.  dz is an arbitrary fp32 tensor: it is split into its three exact bf16
+// parts ONCE while staging, transposed to [part][f][q], so the B operand of a 32x32x16 bf16 instruction (eight consecutive q of
+// one filter) is one 128-bit read per part.  Wavefront ky owns the kw taps of kernel row ky for the whole launch (kw
+// accumulator blocks [32 c x 32 f] in registers): the taps of a row read the same source values shifted by one pixel, so a
+// lane reads a window of 8 + kw - 1 values per batch of sixteen q and packs kw operands from it.  The source is a quantized
+// tensor: the wavefront looks at the window and multiplies by its first bf16 part only when the others are zero
+// (3 instructions per tap and batch), by two or three parts otherwise (6 / 9) - every product of two parts is exact in fp32,
+// only the accumulation rounds.  Slice blockIdx.x of `part` is [kh kw C F | F] (kernel gradient, bias gradient).
+#ifdef PG_PROF
+__device__ unsigned long long wg_prof_stamps[8 * 32];
+#define WG_STAMP(i)                                                                                                     \
+    do {                                                                                                                \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (i) < 32) wg_prof_stamps[(threadIdx.x >> 6) * 32 + (i)] = clock64(); \
+    } while (0)
+extern "C" int hgq_wg_prof_read(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(wg_prof_stamps), sizeof(unsigned long long) * 8 * 32) == hipSuccess ? 0 : -2;
+}
+#else
+#define WG_STAMP(i)
+#endif
+
+struct WgPlan {
+    int TH, bands;  // output rows per tile, tiles per image
+    int XW, XH;     // the tile's source raster: OW + kw - 1 pixels wide, TH + kh - 1 rows
+    int XP, XS;     // pixel slots of the source patch (the windows of the last batch read past the raster: zeros), words per pixel
+    int QN, QS;     // contraction length of a tile (TH * XW rounded up to 16), bf16 between the rows of a dz plane
+};
+
+template <int KH, int KW>
+__global__ __launch_bounds__(64 * KH, 2) void wgrad_patch_kernel(const float *__restrict__ x, const float *__restrict__ dy,
+                                                              const float *__restrict__ mask, float *__restrict__ part,
+                                                              hgq_conv_geom g, int F, int relu, WgPlan p) {
+    constexpr int NT = 64 * KH, WIN = 8 + KW - 1;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    float *xs = lds;                                    // [XP][XS]
+    uint32_t *zp = (uint32_t *)(lds + p.XP * p.XS);     // [3][32][QS / 2] pairs of bf16
+    const int tid = threadIdx.x, lane = tid & 63, ky = tid >> 6, kq = lane >> 5, c = lane & 31;
+    const int C4 = g.C >> 2, QS2 = p.QS >> 1;
+    const __amdgpu_buffer_rsrc_t rs_x = buf_rsrc(x, (int64_t)g.B * g.H * g.W * g.C * 4);
+    const __amdgpu_buffer_rsrc_t rs_dy = buf_rsrc(dy, (int64_t)g.B * g.OH * g.OW * F * 4);
+    const __amdgpu_buffer_rsrc_t rs_m = buf_rsrc(relu ? mask : dy, relu ? (int64_t)g.B * g.OH * g.OW * F * 4 : 0);
+    const FastDiv dxw((uint32_t)p.XW), dc4((uint32_t)C4);
+    floatx16 acc[KW];
+#pragma unroll
+    for (int kx = 0; kx < KW; ++kx) acc[kx] = floatx16{0};
+    f32x4_t bsum = {0.f, 0.f, 0.f, 0.f};
+    const int f4 = tid & 7;  // NT is a multiple of 8: a thread stages the same four filters in every trip
+    const bool c_counts = c < g.C;
+    const int cc = c_counts ? c : 0;  // lanes past the channel count feed result rows nobody reads
+    const int64_t n_tiles = (int64_t)g.B * p.bands;
+    const int n_xu = p.XP * C4, n_zu = (p.QN >> 1) * 8;
+    // The first XU source units and ZU dz units of a thread are asked for together (one memory latency per tile, not one per
+    // unit; the registers are free again when the matrix cores start, and the other workgroups of the CU cover the wait);
+    // a larger tile stages the rest in place.
+    constexpr int XU = 8, ZU = 3;
+    f32x4_t rx[XU], rz[ZU][2], rm[ZU][2];
+    auto x_off = [&](int u, int b, int oy0, int th, int &dst) -> uint32_t {
+        const uint32_t pix = dc4.div((uint32_t)u), c4 = (uint32_t)u - pix * (uint32_t)C4;
+        const uint32_t pr = dxw.div(pix), pc = pix - pr * (uint32_t)p.XW;
+        const int yy = oy0 + (int)pr - g.py, xx = (int)pc - g.px;
+        const bool in = u < n_xu && (int)pr < th + KH - 1 && (unsigned)yy < (unsigned)g.H && (unsigned)xx < (unsigned)g.W;
+        dst = u < n_xu ? (int)pix * p.XS + 4 * (int)c4 : -1;
+        return in ? (uint32_t)(((b * g.H + yy) * g.W + xx) * g.C + 4 * (int)c4) * 4u : BUF_OOB;
+    };
+    auto z_off = [&](int u, int e, int b, int oy0, int th) -> uint32_t {
+        const uint32_t q = (uint32_t)((u >> 3) * 2 + e), qr = dxw.div(q), qc = q - qr * (uint32_t)p.XW;
+        const bool in = u < n_zu && (int)qr < th && (int)qc < g.OW && 4 * f4 < F;
+        return in ? (uint32_t)(((b * g.OH + oy0 + (int)qr) * g.OW + (int)qc) * F + 4 * f4) * 4u : BUF_OOB;
+    };
+    // one dz unit (q, q + 1 of four filters) into the three planes
+    auto z_put = [&](int u, const f32x4_t (&v)[2], const f32x4_t (&m)[2]) {
+        if (u >= n_zu) return;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float z[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                z[e] = (relu && !(m[e][j] > 0.f)) ? 0.f : v[e][j];
+                bsum[j] += z[e];
+            }
+            uint32_t h0, m0, l0, h1, m1, l1;
+            bf16_parts(z[0], h0, m0, l0), bf16_parts(z[1], h1, m1, l1);
+            uint32_t *dst = zp + (4 * f4 + j) * QS2 + (u >> 3);
+            dst[0] = bf16_pair(h0, h1), dst[32 * QS2] = bf16_pair(m0, m1), dst[64 * QS2] = bf16_pair(l0, l1);
+        }
+    };
+    auto fetch = [&](int64_t tile) {
+        const int b = (int)(tile / p.bands), oy0 = (int)(tile - (int64_t)b * p.bands) * p.TH, th = min(p.TH, g.OH - oy0);
+#pragma unroll
+        for (int i = 0; i < XU; ++i) {
+            int dst;
+            rx[i] = buf_ld4(rs_x, x_off(i * NT + tid, b, oy0, th, dst));
+        }
+#pragma unroll
+        for (int i = 0; i < ZU; ++i)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const uint32_t off = z_off(i * NT + tid, e, b, oy0, th);
+                rz[i][e] = buf_ld4(rs_dy, off);
+                rm[i][e] = buf_ld4(rs_m, off);
+            }
+    };
+    WG_STAMP(0);
+    int it_ = 0;
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x, ++it_) {
+        const int b = (int)(tile / p.bands), oy0 = (int)(tile - (int64_t)b * p.bands) * p.TH;
+        const int th = min(p.TH, g.OH - oy0);
+        WG_STAMP(1 + 8 * it_);
+        fetch(tile);      // every load of the tile is in flight before the first is waited for
+        WG_STAMP(2 + 8 * it_);
+        __syncthreads();  // the previous tile's operands are no longer read
+        WG_STAMP(3 + 8 * it_);
+        // source patch: every slot is written (zeros outside the image and past the raster)
+#pragma unroll
+        for (int i = 0; i < XU; ++i) {
+            const int u = i * NT + tid;
+            if (u < n_xu) {
+                const uint32_t pix = dc4.div((uint32_t)u), c4 = (uint32_t)u - pix * (uint32_t)C4;
+                *(f32x4_t *)(xs + (int)pix * p.XS + 4 * (int)c4) = rx[i];
+            }
+        }
+        for (int u0 = XU * NT; u0 < n_xu; u0 += 4 * NT) {
+            f32x4_t v[4];
+            int dst[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = buf_ld4(rs_x, x_off(u0 + i * NT + tid, b, oy0, th, dst[i]));
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (dst[i] >= 0) *(f32x4_t *)(xs + dst[i]) = v[i];
+        }
+        WG_STAMP(4 + 8 * it_);
+        // dz on the source raster, two neighbouring q of four filters per unit; split into bf16 parts, transposed
+#pragma unroll
+        for (int i = 0; i < ZU; ++i) z_put(i * NT + tid, rz[i], rm[i]);
+        for (int u0 = ZU * NT; u0 < n_zu; u0 += 2 * NT) {
+            f32x4_t v[2][2], m[2][2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const uint32_t off = z_off(u0 + i * NT + tid, e, b, oy0, th);
+                    v[i][e] = buf_ld4(rs_dy, off);
+                    m[i][e] = buf_ld4(rs_m, off);
+                }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) z_put(u0 + i * NT + tid, v[i], m[i]);
+        }
+        WG_STAMP(5 + 8 * it_);
+        __syncthreads();
+        WG_STAMP(6 + 8 * it_);
+        const float *xrow = xs + (8 * kq + ky * p.XW) * p.XS + cc;
+        const u32x4_t *zrow = (const u32x4_t *)zp + (c * QS2 + 4 * kq) / 4;  // this lane's filter is c (= lane % 32)
+        const int n_bt = (th * p.XW + 15) >> 4;
+        for (int bt = 0; bt < n_bt; ++bt) {
+            float w[WIN];
+#pragma unroll
+            for (int e = 0; e < WIN; ++e) w[e] = xrow[(16 * bt + e) * p.XS];
+            const u32x4_t b0 = zrow[2 * bt], b1 = zrow[8 * QS2 + 2 * bt], b2 = zrow[16 * QS2 + 2 * bt];
+            uint32_t low = 0u;
+#pragma unroll
+            for (int e = 0; e < WIN; ++e) low |= __float_as_uint(w[e]);
+            if (!__any(c_counts && (low & 0xffffu) != 0u)) {
+#pragma unroll
+                for (int kx = 0; kx < KW; ++kx) {
+                    u32x4_t a;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) a[e] = bf16_pair(__float_as_uint(w[kx + 2 * e]), __float_as_uint(w[kx + 2 * e + 1]));
+                    acc[kx] = mfma_bf16(a, b0, acc[kx]);
+                    acc[kx] = mfma_bf16(a, b1, acc[kx]);
+                    acc[kx] = mfma_bf16(a, b2, acc[kx]);
+                }
+            } else {
+                uint32_t ph[WIN], pm[WIN], pl[WIN], third = 0u;
+#pragma unroll
+                for (int e = 0; e < WIN; ++e) {
+                    bf16_parts(w[e], ph[e], pm[e], pl[e]);
+                    third |= pl[e];
+                }
+                const bool three = __any(c_counts && third != 0u);
+#pragma unroll
+                for (int kx = 0; kx < KW; ++kx) {
+                    u32x4_t a0, a1, a2;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        a0[e] = bf16_pair(ph[kx + 2 * e], ph[kx + 2 * e + 1]);
+                        a1[e] = bf16_pair(pm[kx + 2 * e], pm[kx + 2 * e + 1]);
+                        a2[e] = bf16_pair(pl[kx + 2 * e], pl[kx + 2 * e + 1]);
+                    }
+                    acc[kx] = mfma_bf16(a0, b0, acc[kx]), acc[kx] = mfma_bf16(a0, b1, acc[kx]), acc[kx] = mfma_bf16(a0, b2, acc[kx]);
+                    acc[kx] = mfma_bf16(a1, b0, acc[kx]), acc[kx] = mfma_bf16(a1, b1, acc[kx]), acc[kx] = mfma_bf16(a1, b2, acc[kx]);
+                    if (three) {
+                        acc[kx] = mfma_bf16(a2, b0, acc[kx]), acc[kx] = mfma_bf16(a2, b1, acc[kx]), acc[kx] = mfma_bf16(a2, b2, acc[kx]);
+                    }
+                }
+            }
+        }
+    }
+    WG_STAMP(30);
+    float *my = part + (int64_t)blockIdx.x * ((int64_t)KH * KW * g.C * F + F);
+    if (c < F) {  // result column = filter
+#pragma unroll
+        for (int kx = 0; kx < KW; ++kx)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ch = pg_acc_row(r, lane);
+                if (ch < g.C) my[(int64_t)((ky * KW + kx) * g.C + ch) * F + c] = acc[kx][r];
+            }
+    }
+    // bias gradient: the threads that stage the same four filters add up in a fixed order
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) lds[tid * 4 + j] = bsum[j];
+    __syncthreads();
+    if (tid < 32 && tid < F) {
+        float sacc = 0.f;
+        for (int u = 0; u < NT / 8; ++u) sacc += lds[(u * 8 + (tid >> 2)) * 4 + (tid & 3)];
+        my[(int64_t)KH * KW * g.C * F + tid] = sacc;
+    }
+    WG_STAMP(31);
+}
+
+#define WG_MAX_LDS (53 * 1024)  // three workgroups per CU
+
+static bool plan_wgrad(const hgq_conv_geom &g, int F, WgPlan &p, size_t &lds) {
+    if (!((g.kh == 3 && g.kw == 3) || (g.kh == 5 && g.kw == 5))) return false;
+    if (g.sy != 1 || g.sx != 1 || g.dly != 1 || g.dlx != 1) return false;
+    if (g.C % 4 != 0 || g.C > 32 || F % 4 != 0 || F > 32 || g.B < 1) return false;
+    if ((int64_t)g.B * g.H * g.W * g.C * 4 >= (1ll << 31) || (int64_t)g.B * g.OH * g.OW * F * 4 >= (1ll << 31)) return false;
+    p.XW = g.OW + g.kw - 1;
+    p.XS = (g.C & 7) == 4 ? g.C : g.C + 4;  // 8 * XS = 32 (mod 64) words: the two halves of a wavefront read disjoint banks
+    for (int th = g.OH; th >= 1; th = th > 1 ? (th + 1) / 2 : 0) {
+        p.TH = th, p.bands = (g.OH + th - 1) / th, p.XH = th + g.kh - 1;
+        p.QN = (th * p.XW + 15) & ~15, p.QS = p.QN + 8;
+        p.XP = p.QN + (g.kh - 1) * p.XW + g.kw - 1;
+        if (p.XP < p.XH * p.XW) p.XP = p.XH * p.XW;
+        if (p.XP * (g.C / 4) >= (1 << 20) || p.QN >= (1 << 20)) continue;
+        lds = (size_t)p.XP * p.XS * 4 + (size_t)3 * 32 * p.QS * 2;
+        if (lds < (size_t)64 * g.kh * 16) lds = (size_t)64 * g.kh * 16;  // the bias sums of the last step
+        if (lds <= WG_MAX_LDS) return true;
+    }
+    return false;
+}
+
+bool conv_patch_wgrad_ok(const hgq_conv_geom &g, int F) {
+    WgPlan p;
+    size_t lds;
+    return hgq_dense_use_bf16_parts(-1) != 0 && plan_wgrad(g, F, p, lds);
+}
+
+int conv_patch_wgrad_slices(const hgq_conv_geom &g, int F) {
+    WgPlan p;
+    size_t lds;
+    if (!plan_wgrad(g, F, p, lds)) return 0;
+    return persistent_grid((int64_t)g.B * p.bands, 2);
+}
+
+int conv_patch_wgrad_launch(const float *x, const float *dy, const float *mask, float *part, const hgq_conv_geom &g, int F, int act,
+                            hipStream_t s) {
+    WgPlan p;
+    size_t lds;
+    if (!plan_wgrad(g, F, p, lds)) return fail(HGQ_ERR_UNSUPPORTED, "conv_patch_wgrad_launch: shape not covered");
+    const dim3 grid((unsigned)conv_patch_wgrad_slices(g, F));
+    const int relu = act == HGQ_ACT_RELU && mask != nullptr;
+    if (g.kh == 3) hipLaunchKernelGGL((wgrad_patch_kernel<3, 3>), grid, dim3(192), lds, s, x, dy, mask, part, g, F, relu, p);
+    else hipLaunchKernelGGL((wgrad_patch_kernel<5, 5>), grid, dim3(320), lds, s, x, dy, mask, part, g, F, relu, p);
+    return check_launch("conv_patch_wgrad_launch");
+}
+
 }  // namespace hgq

@@ -54,5 +54,12 @@ int reduce_parts(const float *part, int n_parts, int64_t M, float *dqw, int64_t 
 bool conv_patch_ok(int mode, const hgq_conv_geom &g, int F);
 int conv_patch_launch(int mode, const float *src, const float *mask, const float *w, const float *bias, float *out,
                       const hgq_conv_geom &g, int F, int act, hipStream_t s);
+// Weight / bias gradient through LDS-resident operands (3 x 3 and 5 x 5 kernels, unit stride and dilation, channel and
+// filter counts multiples of 4 up to 32, 16-byte aligned operands, bf16-part matrix instruction selected): slices
+// [conv_patch_wgrad_slices][kh kw C F + F] into `part`.
+bool conv_patch_wgrad_ok(const hgq_conv_geom &g, int F);
+int conv_patch_wgrad_slices(const hgq_conv_geom &g, int F);
+int conv_patch_wgrad_launch(const float *x, const float *dy, const float *mask, float *part, const hgq_conv_geom &g, int F, int act,
+                            hipStream_t s);
 
 }  // namespace hgq

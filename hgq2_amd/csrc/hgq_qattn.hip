@@ -24,6 +24,8 @@
 // i = (r / 4) * 8 + (lane / 32) * 4 + (r % 4).  The contraction index of a step is free, so a
 // half-wavefront takes one half of the head dimension and reads its operands as 128-bit words.
 // Output rows beyond the head size come from whatever the A operand's lanes read; they are never stored.
+#include <type_traits>
+
 #include "hgq_softmax_dev.h"
 
 namespace hgq {
@@ -31,6 +33,17 @@ namespace hgq {
 #define QA_LD 68    // words between rows of an operand tile in LDS
 #define QA_NT 512   // eight wavefronts
 #define QA_PAD 64   // readable words after the last operand tile
+
+// Time stamps of workgroup 0 in the backward kernel (measurement builds only: -DQA_PROF): [wavefront][element][event], core clock
+#ifdef QA_PROF
+__device__ unsigned long long qa_prof_stamps[8 * 4 * 16];
+#define QA_STAMP(i)                                                                                                       \
+    do {                                                                                                                  \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && it_ < 4) qa_prof_stamps[((threadIdx.x >> 6) * 4 + it_) * 16 + (i)] = clock64(); \
+    } while (0)
+#else
+#define QA_STAMP(i)
+#endif
 
 struct QAttnPlan {
     int B, T, S, N;
@@ -673,8 +686,8 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
     constexpr int T = 32 * TH, S = 32 * ST, NW = QA_NT / 64;
     float *Qs = lds, *Ks = Qs + (T + 1) * QA_LD, *Vs = Ks + (S + 1) * QA_LD, *Gs = Vs + (S + 1) * QA_LD;
     float *Pm = Gs + (T + 1) * QA_LD + QA_PAD;                           // [NW][32][QA_LD]: probs, then dscores
-    ExpTable::Entry *tabp = (ExpTable::Entry *)(Pm + NW * 32 * QA_LD);  // [SM_TABLE]
-    float *tab_e = (float *)(tabp + SM_TABLE);                          // [SM_TABLE]: e alone, one bank per code
+    float *tabp = Pm + NW * 32 * QA_LD;  // [4][SM_TABLE]: planes e, ca, ci, cf of the exp stage's table
+    float *tab_e = tabp;
     __shared__ float part[NW][8];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, t_l = lane & 31, hf = lane >> 5;
@@ -717,10 +730,6 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
         ExpTable tab;
         tab.build_bwd(tabp, q1, q2, scale);
         ec.init(q1, tab);
-        if (tab.on) {
-            for (int n = threadIdx.x; n < SM_TABLE; n += QA_NT) tab_e[n] = tabp[n].e;
-            __syncthreads();
-        }
     }
 
     Stage sq_, sk_, sv_, sg_;
@@ -730,10 +739,14 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
     int b_prev = -1;
     int b = blockIdx.x;
     sq_.fetch(pq, b, b < pl.B), sk_.fetch(pk, b, b < pl.B), sv_.fetch(pv, b, b < pl.B), sg_.fetch(pg, b, b < pl.B);
-    for (; b < pl.B; b += pl.n_wg) {
+    int it_ = 0;
+    for (; b < pl.B; b += pl.n_wg, ++it_) {
+        QA_STAMP(0);
         __syncthreads();  // the previous element's tiles and buffers are no longer read
+        QA_STAMP(1);
         sq_.stash(Qs, T, pq), sk_.stash(Ks, S, pk), sv_.stash(Vs, S, pv), sg_.stash(Gs, T, pg);
         __syncthreads();
+        QA_STAMP(2);
         // the previous element's dkey leaves here, well ahead of the wait at the top of the walk
         if (active && b_prev >= 0) {
 #pragma unroll
@@ -756,6 +769,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
             if (MASKED) load_keep<ST>(mk, b, T, S, t0 + t_l, hf, keep);
             score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, xs, pl.bf != 0);        // scores, transposed
             score_tiles<HD, ST, true>(Vs, Gs, t0, col0, t_l, hf, ga, pl.bf != 0);  // d probs = dout value^T, transposed
+            QA_STAMP(3);
             if (MASKED) {
 #pragma unroll
                 for (int st = 0; st < ST; ++st)
@@ -791,39 +805,51 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
                 }
             }
             s += xor32(s);
+            QA_STAMP(4);
             const float sq = q3.fwd(s);
             const float r0 = __fdiv_rn(1.0f, __fadd_rn(sq, eps));
             rr = q4.fwd(r0);
-            // ---- output quantizer and the product; probs go to the buffer as they are formed
+            // ---- output quantizer and the product; probs go to the buffer as they are formed.  The round mode is the same for
+            // the whole launch: one branch here instead of a select per element.  The fractional-bit gradient keeps its factor
+            // -ln 2 for the end of the walk (gof holds sum (p - y0) * dprob).
             float drr = 0.f;
+            auto oq_stage = [&](auto conv_tag) {
+                constexpr bool CONV = decltype(conv_tag)::value;
 #pragma unroll
-            for (int st = 0; st < ST; ++st)
+                for (int st = 0; st < ST; ++st)
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    float *slot = my_buf + t_l * QA_LD + st * 32 + 8 * g + 4 * hf;
-                    const f32x4_t e4 = *(const f32x4_t *)slot;
-                    f32x4_t p4;
+                    for (int g = 0; g < 4; ++g) {
+                        float *slot = my_buf + t_l * QA_LD + st * 32 + 8 * g + 4 * hf;
+                        const f32x4_t e4 = *(const f32x4_t *)slot;
+                        f32x4_t p4;
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const int r = 4 * g + c;
-                        const float y0 = __fmul_rn(e4[c], rr);
-                        float p = y0;
-                        if (qo.present) {
-                            p = qo.round_at(y0, (int)(int8_t)((pf[st][g] >> (8 * c)) & 0xff));
-                            gof[st][r] += -HGQ_LN2 * (p - y0) * ga[st][r];
+                        for (int c = 0; c < 4; ++c) {
+                            const int r = 4 * g + c;
+                            const float y0 = __fmul_rn(e4[c], rr);
+                            float p = y0;
+                            if (qo.present) {
+                                const int fi = (int)(int8_t)((pf[st][g] >> (8 * c)) & 0xff);
+                                const float t = ldexpf(y0, fi);
+                                p = ldexpf(CONV ? rintf(t) : floorf(__fadd_rn(t, qo.rc)), -fi);
+                                gof[st][r] = fmaf(p - y0, ga[st][r], gof[st][r]);
+                            }
+                            p4[c] = p;
+                            drr = fmaf(ga[st][r], e4[c], drr);
                         }
-                        p4[c] = p;
-                        drr += ga[st][r] * e4[c];
+                        *(f32x4_t *)slot = p4;
                     }
-                    *(f32x4_t *)slot = p4;
-                }
+            };
+            if (qo.conv) oq_stage(std::true_type{});
+            else oq_stage(std::false_type{});
             drr += xor32(drr);
             float dr0, gi4, gf4, gi3, gf3;
             q4.grad(r0, drr, dr0, gi4, gf4);
             q3.grad(s, dr0 * -(r0 * r0), ds, gi3, gf3);
             if (hf == 0) gs[6] += gi4, gs[7] += gf4, gs[4] += gi3, gs[5] += gf3;
         }
+        QA_STAMP(5);
         __syncthreads();  // probs of every head are in the buffers
+        QA_STAMP(6);
         if (active) {
             // dvalue[s][h] = sum_t probs[t][s] dout[t][h]: key-position tile st of a head goes to its wavefront st % TH
 #pragma unroll
@@ -832,8 +858,13 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
                     const floatx16 o = contract_queries<TH, true, false>(Gs, col0, head_buf, st * 32, t_l, hf, pl.bf != 0, HD);
                     store_rows<HD>(o, dv_ + ((int64_t)b * S * pl.N + h) * HD, (int64_t)pl.N * HD, st * 32 + t_l, hf);
                 }
+            QA_STAMP(7);
             // ---- exp stage and the maximum
             float dm = 0.f, cnt = 0.f;
+            // the usual exp input quantizer rounds to nearest (or truncates) and does not saturate: its gradient then has no
+            // bound terms, d/df = -ln 2 * sum (a - d) * da (the factor waits for the end of the element) and d/di = 0
+            const bool plain = ec.on && !ec.conv && ec.code_max == INFINITY;
+            float f1 = 0.f;
 #pragma unroll
             for (int st = 0; st < ST; ++st) {
                 float raw[16], cl[16];
@@ -842,13 +873,43 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
                     for (int r = 0; r < 16; ++r) xm[r] = ((keep[st] >> r) & 1u) ? xm[r] : mx;
                 }
+                if (plain) {
+                    bool big = false;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        raw[r] = floorf(__fadd_rn(ldexpf(__fsub_rn(mx, xm[r]), ec.fi), ec.rc));
+                        big |= !(raw[r] < (float)SM_TABLE);
+                    }
+                    if (!__any(big)) {
+#pragma unroll
+                        for (int r0_ = 0; r0_ < 16; r0_ += 4) {
+                            ExpTable::Entry en[4];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) en[j] = ExpTable::entry_at(tabp, (int)raw[r0_ + j]);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                const int r = r0_ + j;
+                                const float d = __fsub_rn(mx, xm[r]);
+                                const float de = (!MASKED || ((keep[st] >> r) & 1u)) ? fmaf(ga[st][r], rr, ds) : 0.f;
+                                const float da = en[j].ca * de;
+                                f1 = fmaf(ldexpf(raw[r], -ec.fi) - d, da, f1);
+                                gs[2] = fmaf(en[j].ci, de, gs[2]), gs[3] = fmaf(en[j].cf, de, gs[3]);
+                                dm += da;
+                                ga[st][r] = da;
+                            }
+                        }
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) cnt += (xs[st][r] == mx) ? 1.f : 0.f;
+                        continue;
+                    }
+                }
                 const bool slow = tile_codes(xm, mx, ec, raw, cl);
 #pragma unroll
                 for (int r0_ = 0; r0_ < 16; r0_ += 4) {
                     if (!slow) {
                         ExpTable::Entry en[4];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) en[j] = tabp[(int)cl[r0_ + j]];
+                        for (int j = 0; j < 4; ++j) en[j] = ExpTable::entry_at(tabp, (int)cl[r0_ + j]);
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             const int r = r0_ + j;
@@ -876,6 +937,11 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
                 for (int r = 0; r < 16; ++r) cnt += (xs[st][r] == mx) ? 1.f : 0.f;
             }
+            {
+                const float gf1 = -HGQ_LN2 * f1;
+                gs[1] += gf1;
+                if (ec.kbi) gs[0] -= gf1;
+            }
             dm += xor32(dm);
             cnt += xor32(cnt);
             const float share = dm / cnt;  // the maximum's gradient is split evenly among ties
@@ -887,6 +953,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
                     if (MASKED && !((keep[st] >> r) & 1u)) ga[st][r] = 0.f;  // d (mask * scores - ...) / d scores
                 }
         }
+        QA_STAMP(8);
         {
             // the next element's operands: issued here, after the register-hungry stages, some eighty MFMAs ahead of their use
             const int nb = b + pl.n_wg;
@@ -897,9 +964,12 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
             const floatx16 o = contract_keys<ST, true>(Ks, col0, t_l, hf, ga, pl.bf != 0, HD);
             store_rows<HD>(o, dq_ + ((int64_t)b * T * pl.N + h) * HD, (int64_t)pl.N * HD, t0 + t_l, hf);
         }
+        QA_STAMP(9);
         __syncthreads();  // dvalue has read the probs
+        QA_STAMP(10);
         if (active) spill_tiles<ST>(my_buf, ga, t_l, hf);
         __syncthreads();
+        QA_STAMP(11);
         if (active) {
             // dkey[s][h] = sum_t dscores[t][s] query[t][h]
 #pragma unroll
@@ -907,6 +977,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
                 if (st % TH == th) dk_prev = contract_queries<TH, false, true>(Qs, col0, head_buf, st * 32, t_l, hf, pl.bf != 0, HD);
             b_prev = b;
         }
+        QA_STAMP(12);
     }
     if (active && b_prev >= 0) {
 #pragma unroll
@@ -932,16 +1003,22 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             f32x4_t v4;
-            v4.x = gof[st][4 * g], v4.y = gof[st][4 * g + 1], v4.z = gof[st][4 * g + 2], v4.w = gof[st][4 * g + 3];
+            v4.x = -HGQ_LN2 * gof[st][4 * g], v4.y = -HGQ_LN2 * gof[st][4 * g + 1], v4.z = -HGQ_LN2 * gof[st][4 * g + 2], v4.w = -HGQ_LN2 * gof[st][4 * g + 3];
             *(f32x4_t *)(wf + st * 32 + 8 * g + 4 * hf) = v4;
         }
 }
+
+#ifdef QA_PROF
+extern "C" int hgq_qa_prof_read(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(qa_prof_stamps), sizeof(unsigned long long) * 8 * 4 * 16) == hipSuccess ? 0 : -2;
+}
+#endif
 
 static size_t qattn_lds_bytes(int T, int S, bool bwd) {
     size_t words = (size_t)(T + 1 + 2 * (S + 1)) * QA_LD + QA_PAD;
     if (!bwd) return (words + SM_TABLE) * sizeof(float);
     words += (size_t)(T + 1) * QA_LD + (size_t)(QA_NT / 64) * 32 * QA_LD;
-    return words * sizeof(float) + SM_TABLE * (sizeof(ExpTable::Entry) + sizeof(float));
+    return words * sizeof(float) + SM_TABLE * sizeof(ExpTable::Entry);
 }
 
 // Shapes the kernels take: sequence lengths 32 or 64 (both the same number of tiles), head size 8, 16 or

@@ -187,7 +187,7 @@ __global__ __launch_bounds__(64 * SM_WPB) void qsoftmax_bwd_kernel(
     float eps, hgq_qdesc d1, hgq_qdesc d2, hgq_qdesc d3, hgq_qdesc d4, hgq_qdesc dq, float *__restrict__ ws) {
     __shared__ float lds_g[SM_WPB][NP * VEC][64];
     __shared__ float part[SM_WPB][8];
-    __shared__ ExpTable::Entry lds_tab[SM_TABLE];
+    __shared__ float lds_tab[4 * SM_TABLE];
     Walk<SUB, VEC, NP> wk;
     wk.init(pl);
     SharedQ q1, q2, q3, q4;

@@ -190,11 +190,19 @@ struct ExpTable {
         e = n < SM_TABLE ? tab[n] : q2.fwd<true>(t_of(a, scale));
     }
 
-    // backward: tab[n] = (e, d a / d e-gradient, d i2, d fb2) with
-    //   da = -((dt * t) * scale) = ca * de,  gi2 = ci * de,  gf2 = cf * de   for the upstream gradient de of e
+    // backward: entry n = (e, d a / d e-gradient, d i2, d fb2) with
+    //   da = -((dt * t) * scale) = ca * de,  gi2 = ci * de,  gf2 = cf * de   for the upstream gradient de of e.
+    // In LDS the four fields are four planes of SM_TABLE words (field j of code n at tab[j * SM_TABLE + n]): the lanes of a
+    // wavefront look up unrelated codes, and 32-bit reads at unrelated addresses cost a fraction of what 128-bit ones do
+    // (the banks serve them a word at a time; a 128-bit read needs four neighbouring banks free at once).
     struct Entry {
         float e, ca, ci, cf;
     };
+    static __device__ __forceinline__ Entry entry_at(const float *tab, int n) {
+        Entry r;
+        r.e = tab[n], r.ca = tab[SM_TABLE + n], r.ci = tab[2 * SM_TABLE + n], r.cf = tab[3 * SM_TABLE + n];
+        return r;
+    }
     static __device__ __forceinline__ Entry entry_of(float a, const SharedQ &q2, float scale) {
         const float t = t_of(a, scale);
         Entry r;
@@ -204,19 +212,22 @@ struct ExpTable {
         r.ca = -((dt * t) * scale);
         return r;
     }
-    __device__ __forceinline__ void build_bwd(Entry *tab, const SharedQ &q1, const SharedQ &q2, float scale) {
+    __device__ __forceinline__ void build_bwd(float *tab, const SharedQ &q1, const SharedQ &q2, float scale) {
         init(q1);
         if (!on) return;
-        for (int n = threadIdx.x; n < SM_TABLE; n += blockDim.x) tab[n] = entry_of(ldexpf((float)n, -q1.fi), q2, scale);
+        for (int n = threadIdx.x; n < SM_TABLE; n += blockDim.x) {
+            const Entry en = entry_of(ldexpf((float)n, -q1.fi), q2, scale);
+            tab[n] = en.e, tab[SM_TABLE + n] = en.ca, tab[2 * SM_TABLE + n] = en.ci, tab[3 * SM_TABLE + n] = en.cf;
+        }
         __syncthreads();
     }
     // d >= 0 -> r = un-saturated code, entry of the saturated code
-    __device__ __forceinline__ Entry eval_bwd(const Entry *tab, float d, const SharedQ &q1, const SharedQ &q2, float scale,
+    __device__ __forceinline__ Entry eval_bwd(const float *tab, float d, const SharedQ &q1, const SharedQ &q2, float scale,
                                               float &r) const {
         r = code_of(d, q1);
         const float rcl = fminf(r, code_max);
         const unsigned n = (unsigned)(int)rcl;
-        if (n < SM_TABLE) return tab[n];
+        if (n < SM_TABLE) return entry_at(tab, (int)n);
         return entry_of(ldexpf(rcl, -q1.fi), q2, scale);
     }
     // gradients of the exp input quantizer from the un-saturated code r (no lower violation: d >= 0 >= lo)

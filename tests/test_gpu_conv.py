@@ -92,6 +92,57 @@ def test_conv2d_matches_fp64_reference(dev, case):
         assert bool((err <= tol).all()), f'grad {name}: {float((err / tol).max()):.2f} x the bound of 1e-5 of the summed |terms|'
 
 
+WGRAD_PATCH_CASES = [
+    # B, H, W, C, kh, F, padding, bits of the source (0: arbitrary fp32), misaligned source
+    (9, 13, 13, 32, 3, 32, 'valid', 6, False),    # the image configuration's second layer: one bf16 part per source value
+    (9, 13, 13, 32, 3, 32, 'valid', 14, False),   # two parts
+    (9, 13, 13, 32, 3, 32, 'valid', 0, False),    # three parts
+    (700, 9, 10, 8, 3, 20, 'same', 5, False),     # more images than workgroups, padding, filters not a multiple of 32
+    (3, 50, 41, 16, 3, 12, 'same', 7, False),     # several bands per image, the last one short
+    (4, 18, 15, 12, 5, 28, 'same', 6, False),     # 5 x 5, channels not a multiple of 8
+    (3, 12, 12, 24, 5, 8, 'valid', 0, False),
+    (5, 13, 13, 32, 3, 32, 'valid', 6, True),     # a source that is not 16-byte aligned keeps the slice count: gathered kernels
+]
+
+
+@pytest.mark.parametrize('case', WGRAD_PATCH_CASES)
+def test_weight_gradient_from_lds_patches(dev, case):
+    """Kernel / bias gradient of 3 x 3 and 5 x 5 layers with up to 32 channels and filters (both operands of a band of an
+    image staged once in LDS, dz as bf16 parts): against the fp64 reference, error bound 1e-5 of the summed |terms|."""
+    from hgq2_amd import _lib, ops
+
+    B, H, W, C, k, Fo, padding, bits, misaligned = case
+    g = torch.Generator().manual_seed(WGRAD_PATCH_CASES.index(case))
+    if bits:
+        x = torch.randint(-(1 << (bits - 1)), 1 << (bits - 1), (B, H, W, C), generator=g).float() / 16.0
+    else:
+        x = torch.randn(B, H, W, C, generator=g)
+    w = torch.randn(k, k, C, Fo, generator=g) * 0.3
+    b = torch.randn(Fo, generator=g)
+    xr, wr, br = x.clone().requires_grad_(True), w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    want = _ref_conv(xr, wr, br, (1, 1), padding, (1, 1), True)
+    if misaligned:
+        xp = torch.zeros(x.numel() + 1, device=dev)[1:].view(x.shape).copy_(x.to(dev)).requires_grad_(True)
+        assert xp.data_ptr() % 16 != 0
+    else:
+        xp = x.to(dev).requires_grad_(True)
+    wp, bp = w.to(dev).requires_grad_(True), b.to(dev).requires_grad_(True)
+    got = ops.conv2d(xp, wp, bp, (1, 1), padding, (1, 1), _lib.ACT_RELU)
+    scale = want.abs().max().item() + 1e-9
+    up = torch.randn(want.shape, generator=g)
+    pre = _ref_conv(x, w, b, (1, 1), padding, (1, 1), False)
+    up = up * (pre.abs() > 1e-5 * scale)
+    (want * up.double()).sum().backward()
+    (got * up.to(dev)).sum().backward()
+    xa, wa, ba = x.abs().requires_grad_(True), w.abs().requires_grad_(True), b.abs().requires_grad_(True)
+    dz = up.double() * (want.detach() > 0)
+    (_ref_conv(xa, wa, ba, (1, 1), padding, (1, 1), False) * dz.abs()).sum().backward()
+    for name, p_, r, a in (('w', wp, wr, wa), ('b', bp, br, ba), ('x', xp, xr, xa)):
+        err = (p_.grad.cpu().double() - r.grad.double()).abs()
+        tol = 1e-5 * a.grad.double() + 1e-30
+        assert bool((err <= tol).all()), f'grad {name}: {float((err / tol).max()):.2f} x the bound of 1e-5 of the summed |terms|'
+
+
 def test_conv2d_small_integers_exact(dev):
     """Bit-width tensors convolved for EBOPs hold small integers: products and sums are exact in fp32."""
     from hgq2_amd import ops
