@@ -139,6 +139,8 @@ SIGNATURES = {
     'hgq_conv2d_maxpool_bwd_supported': (c_int, [c_void_p, c_int]),
     'hgq_conv2d_maxpool_fwd': (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p]),
     'hgq_conv2d_maxpool_bwd': (c_int, [c_void_p] * 9 + [c_int, c_int, c_int, c_void_p]),
+    'hgq_conv2d_maxpool_fwd_coded': (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p]),
+    'hgq_conv2d_maxpool_bwd_coded': (c_int, [c_void_p] * 9 + [c_int, c_int, c_int, c_void_p]),
 }
 
 

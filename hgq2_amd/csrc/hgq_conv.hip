@@ -498,7 +498,8 @@ __global__ __launch_bounds__(256) void dgrad_patch_kernel(const float *__restric
 template <int KH, int KW, int C>
 __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                          const float *__restrict__ bias, float *__restrict__ out, hgq_conv_geom g,
-                                                         int F, int act, int tiles_x, int tiles_y, float *__restrict__ pooled) {
+                                                         int F, int act, int tiles_x, int tiles_y, float *__restrict__ pooled,
+                                                         uint8_t *__restrict__ code) {
 #pragma clang fp contract(fast)  // multiply-adds of the convolution sum may fuse (see bwd_smallc_kernel)
     constexpr int KC = KH * KW * C;
     extern __shared__ float lds[];  // input patch [XH][XW][C]
@@ -526,11 +527,15 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
         const int oy = oy0 + slot;
         if (oy < g.OH) {
             const int n_x = min(SC_TW, g.OW - ox0);
-            float *orow = out + (((int64_t)b * g.OH + oy) * g.OW + ox0) * F + f;
+            float *orow = out ? out + (((int64_t)b * g.OH + oy) * g.OW + ox0) * F + f : nullptr;
             // `pooled`: also the 2 x 2 / stride 2 maxima, [B, OH / 2, OW / 2, F].  Tiles start on even rows and columns; a
-            // window's two rows are the two halves of one wavefront (slots 2 w and 2 w + 1), its columns two trips of the loop
+            // window's two rows are the two halves of one wavefront (slots 2 w and 2 w + 1), its columns two trips of the loop.
+            // `code` (same shape, one byte per window and filter): bits 0-1 = the place of the window's first maximum in
+            // row-major order, bit 2 = that maximum is positive - all the backward pass needs of the unpooled output.
             const int PHo = g.OH >> 1, PWo = g.OW >> 1;
-            float *prow = pooled ? pooled + (((int64_t)b * PHo + (oy >> 1)) * PWo + (ox0 >> 1)) * F + f : nullptr;
+            const int64_t pbase = (((int64_t)b * PHo + (oy >> 1)) * PWo + (ox0 >> 1)) * F + f;
+            float *prow = pooled ? pooled + pbase : nullptr;
+            uint8_t *crow = code ? code + pbase : nullptr;
             const bool p_row = pooled && (oy >> 1) < PHo;  // both rows of the window exist: both halves are in this loop
             float left = 0.f;
             for (int tx = 0; tx < n_x; ++tx) {
@@ -542,12 +547,18 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
                     acc += xp[(ky * g.dly * XW + kx * g.dlx) * C + c] * wreg[t];
                 }
                 if (act == HGQ_ACT_RELU) acc = acc > 0.f ? acc : 0.f;
-                if (f_on) orow[(int64_t)tx * F] = acc;
+                if (f_on && orow) orow[(int64_t)tx * F] = acc;
                 if (p_row) {
                     if (tx & 1) {
-                        float m = fmaxf(left, acc);
-                        m = fmaxf(m, __shfl_xor(m, 32));
-                        if (!(slot & 1) && f_on && ((ox0 + tx) >> 1) < PWo) prow[(int64_t)(tx >> 1) * F] = m;
+                        const bool right = acc > left;
+                        const float m = right ? acc : left, mo = __shfl_xor(m, 32);
+                        const int j = right ? 1 : 0, jo = __shfl_xor(j, 32);
+                        if (!(slot & 1) && f_on && ((ox0 + tx) >> 1) < PWo) {
+                            const bool lower = mo > m;  // the lower row takes the window only with a larger value
+                            const float best = lower ? mo : m;
+                            prow[(int64_t)(tx >> 1) * F] = best;
+                            if (crow) crow[(int64_t)(tx >> 1) * F] = (uint8_t)((lower ? 2 + jo : j) | (best > 0.f ? 4 : 0));
+                        }
                     } else {
                         left = acc;
                     }
@@ -576,7 +587,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                                                          const float *__restrict__ x, const float *__restrict__ w,
                                                          float *__restrict__ dx, float *__restrict__ part, hgq_conv_geom g, int F,
                                                          int tiles_x, int tiles_y, int vec, const float *__restrict__ dyp, int PHo,
-                                                         int PWo, int relu) {
+                                                         int PWo, int relu, const uint8_t *__restrict__ code) {
     // the multiply-adds of the two contractions below may fuse (the file is built without contraction for the quantizer
     // arithmetic; a convolution sum has no such contract, and unfused it costs two vector instructions per term)
 #pragma clang fp contract(fast)
@@ -590,7 +601,8 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
     const int64_t dy_bytes = (int64_t)g.B * g.OH * g.OW * F * 4;
     const __amdgpu_buffer_rsrc_t rs_dy = buf_rsrc(dy, dy_bytes), rs_mask = buf_rsrc(mask ? mask : dy, mask ? dy_bytes : 0),
                                  rs_x = buf_rsrc(x, (int64_t)g.B * g.H * g.W * C * 4),
-                                 rs_dyp = buf_rsrc(dyp ? dyp : mask, dyp ? (int64_t)g.B * PHo * PWo * F * 4 : 0);
+                                 rs_dyp = buf_rsrc(dyp ? dyp : mask, dyp ? (int64_t)g.B * PHo * PWo * F * 4 : 0),
+                                 rs_code = buf_rsrc(code ? (const void *)code : (const void *)dy, code ? (int64_t)g.B * PHo * PWo * F : 0);
     float wacc[KC], bacc = 0.f;
 #pragma unroll
     for (int t = 0; t < KC; ++t) wacc[t] = 0.f;
@@ -602,7 +614,44 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
         const int oy0 = iy0 + g.py - (KH - 1), ox0 = ix0 + g.px - (KW - 1);
         __syncthreads();
         // buffer loads (zeros outside the tensor, no branch around a load): all units of a batch are in flight together
-        if (dyp) {
+        if (dyp && code) {
+            // the same units from the forward pass's byte per window and filter (place of the first maximum, and whether it
+            // is positive) instead of the four outputs of the window: a sixteenth of the bytes
+            const int f4 = F / 4, wpr = PW / 2, n_u = (PH / 2) * wpr * f4;
+            const FastDiv d_f4((uint32_t)f4), d_wpr((uint32_t)wpr);
+            for (int e0 = 0; e0 < n_u; e0 += 4 * 256) {
+                f32x4_t gv[4];
+                uint32_t cv[4];
+                int dst[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int e = e0 + u * 256 + tid;
+                    uint32_t off_g = BUF_OOB;
+                    dst[u] = -1;
+                    if (e < n_u) {
+                        const int wi = (int)d_f4.div((uint32_t)e), f0 = (e - wi * f4) * 4, wr = (int)d_wpr.div((uint32_t)wi), wc = wi - wr * wpr;
+                        const int oy = oy0 + 2 * wr, ox = ox0 + 2 * wc;
+                        dst[u] = (2 * wr * PW + 2 * wc) * FS + f0;
+                        if ((unsigned)oy < (unsigned)(2 * PHo) && (unsigned)ox < (unsigned)(2 * PWo))
+                            off_g = (uint32_t)(((b * PHo + (oy >> 1)) * PWo + (ox >> 1)) * F + f0) * 4u;
+                    }
+                    gv[u] = buf_ld4(rs_dyp, off_g);
+                    cv[u] = __float_as_uint(buf_ld1(rs_code, off_g == BUF_OOB ? BUF_OOB : off_g >> 2));
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (dst[u] < 0) continue;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const uint32_t cb = (cv[u] >> (8 * c)) & 0xffu;
+                        const int first = (int)(cb & 3u);
+                        const float gz = (!relu || (cb & 4u)) ? gv[u][c] : 0.f;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) zp[dst[u] + ((j >> 1) * PW + (j & 1)) * FS + c] = first == j ? gz : 0.f;
+                    }
+                }
+            }
+        } else if (dyp) {
             // unit = one pooling window x four filters (the patch starts on a window boundary and holds whole windows:
             // the launcher checks it).  An output pixel takes its window's gradient where it holds the window's first
             // maximum in row-major order - what the pooling kernels do - and, behind a ReLU, is positive.
@@ -1497,7 +1546,7 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
         const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
         const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
         const size_t lds = fwd_smallc_lds(*g);
-#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, (float *)nullptr)
+#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, (float *)nullptr, (uint8_t *)nullptr)
         HGQ_SMALLC_DISPATCH(HGQ_FWD_SC);
 #undef HGQ_FWD_SC
         return check_launch("hgq_conv2d_fwd(few channels)");
@@ -1555,7 +1604,7 @@ extern "C" int64_t hgq_conv2d_bwd_slice_count(const hgq_conv_geom *g, int F) {
 // dyp: the gradient behind a 2 x 2 / stride 2 / unpadded maximum pooling of the output ([B, OH / 2, OW / 2, F]) instead of dy
 static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
                            float *workspace, const hgq_conv_geom *g, int F, int act, void *stream, bool reduce,
-                           const float *dyp = nullptr) {
+                           const float *dyp = nullptr, const uint8_t *code = nullptr) {
     int rc = check_geom(g, F, "hgq_conv2d_bwd");
     if (rc) return rc;
     if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: unknown activation %d", act);
@@ -1570,9 +1619,9 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
         return HGQ_OK;
     }
     if ((!dy && !dyp) || !qw || !xq) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: null pointer");
-    if ((act == HGQ_ACT_RELU || dyp) && !y) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: relu / pooling need the forward output");
+    if ((act == HGQ_ACT_RELU || dyp) && !y && !code) return fail(HGQ_ERR_ARG, "hgq_conv2d_bwd: relu / pooling need the forward output");
     const float *mask = (act == HGQ_ACT_RELU || dyp) ? y : nullptr;
-    if (dyp && !(hgq_conv2d_maxpool_bwd_supported(g, F) && aligned16(dyp) && aligned16(y)))
+    if (dyp && !(hgq_conv2d_maxpool_bwd_supported(g, F) && aligned16(dyp) && (code ? ((uintptr_t)code & 3u) == 0 : aligned16(y))))
         return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_maxpool_bwd: shape or alignment not supported (ask hgq_conv2d_maxpool_bwd_supported)");
     if (bwd_smallc_ok(*g, F)) {
         const bool want_w = dqw || dqb;
@@ -1582,7 +1631,7 @@ static int conv2d_bwd_impl(const float *dy, const float *y, const float *xq, con
         const size_t lds = bwd_smallc_lds(*g, F);
         const int vec = F % 4 == 0 && aligned16(dy) && (!mask || aligned16(mask));
 #define HGQ_BWD_SC(KH, KW, CC) \
-    hipLaunchKernelGGL((bwd_smallc_kernel<KH, KW, CC>), dim3((unsigned)grid), dim3(256), lds, s, dy, mask, xq, qw, dxq, want_w ? workspace : (float *)nullptr, *g, F, tiles_x, tiles_y, vec, dyp, g->OH / 2, g->OW / 2, act == HGQ_ACT_RELU)
+    hipLaunchKernelGGL((bwd_smallc_kernel<KH, KW, CC>), dim3((unsigned)grid), dim3(256), lds, s, dy, mask, xq, qw, dxq, want_w ? workspace : (float *)nullptr, *g, F, tiles_x, tiles_y, vec, dyp, g->OH / 2, g->OW / 2, act == HGQ_ACT_RELU, code)
         HGQ_SMALLC_DISPATCH(HGQ_BWD_SC);
 #undef HGQ_BWD_SC
         if ((rc = check_launch("hgq_conv2d_bwd(few channels)"))) return rc;
@@ -1685,22 +1734,34 @@ extern "C" int hgq_conv2d_bwd_slices(const float *dy, const float *y, const floa
     return conv2d_bwd_impl(dy, y, xq, qw, dxq, workspace, workspace, workspace, g, F, act, stream, false);
 }
 
-extern "C" int hgq_conv2d_maxpool_fwd(const float *xq, const float *qw, const float *qb, float *y, float *yp, const hgq_conv_geom *g,
-                                      int F, int act, void *stream) {
-    int rc = check_geom(g, F, "hgq_conv2d_maxpool_fwd");
+static int conv2d_maxpool_fwd_impl(const float *xq, const float *qw, const float *qb, float *y, float *yp, uint8_t *code,
+                                   const hgq_conv_geom *g, int F, int act, void *stream, const char *who) {
+    int rc = check_geom(g, F, who);
     if (rc) return rc;
-    if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_fwd: unknown activation %d", act);
+    if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "%s: unknown activation %d", who, act);
     if (!hgq_conv2d_maxpool_bwd_supported(g, F) || !fwd_smallc_ok(*g, F))
-        return fail(HGQ_ERR_UNSUPPORTED, "hgq_conv2d_maxpool_fwd: shape not supported (ask hgq_conv2d_maxpool_bwd_supported)");
-    if (!xq || !qw || !y || !yp) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_fwd: null pointer");
+        return fail(HGQ_ERR_UNSUPPORTED, "%s: shape not supported (ask hgq_conv2d_maxpool_bwd_supported)", who);
+    if (!xq || !qw || (!y && !code) || !yp) return fail(HGQ_ERR_ARG, "%s: null pointer", who);
     hipStream_t s = (hipStream_t)stream;
     const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
     const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
     const size_t lds = fwd_smallc_lds(*g);
-#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, yp)
+#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, yp, code)
     HGQ_SMALLC_DISPATCH(HGQ_FWD_SC);
 #undef HGQ_FWD_SC
-    return check_launch("hgq_conv2d_maxpool_fwd");
+    return check_launch(who);
+}
+
+extern "C" int hgq_conv2d_maxpool_fwd(const float *xq, const float *qw, const float *qb, float *y, float *yp, const hgq_conv_geom *g,
+                                      int F, int act, void *stream) {
+    if (!y) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_fwd: null pointer");
+    return conv2d_maxpool_fwd_impl(xq, qw, qb, y, yp, nullptr, g, F, act, stream, "hgq_conv2d_maxpool_fwd");
+}
+
+extern "C" int hgq_conv2d_maxpool_fwd_coded(const float *xq, const float *qw, const float *qb, float *yp, uint8_t *code,
+                                            const hgq_conv_geom *g, int F, int act, void *stream) {
+    if (!code) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_fwd_coded: null pointer");
+    return conv2d_maxpool_fwd_impl(xq, qw, qb, nullptr, yp, code, g, F, act, stream, "hgq_conv2d_maxpool_fwd_coded");
 }
 
 extern "C" int hgq_conv2d_maxpool_bwd(const float *dyp, const float *y, const float *xq, const float *qw, float *dxq, float *dqw,
@@ -1709,6 +1770,15 @@ extern "C" int hgq_conv2d_maxpool_bwd(const float *dyp, const float *y, const fl
     if (!reduce && !workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_bwd: null workspace");
     if (reduce) return conv2d_bwd_impl(nullptr, y, xq, qw, dxq, dqw, dqb, workspace, g, F, act, stream, true, dyp);
     return conv2d_bwd_impl(nullptr, y, xq, qw, dxq, workspace, workspace, workspace, g, F, act, stream, false, dyp);
+}
+
+extern "C" int hgq_conv2d_maxpool_bwd_coded(const float *dyp, const uint8_t *code, const float *xq, const float *qw, float *dxq,
+                                            float *dqw, float *dqb, float *workspace, const hgq_conv_geom *g, int F, int act, int reduce,
+                                            void *stream) {
+    if (!dyp || !code) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_bwd_coded: null pointer");
+    if (!reduce && !workspace) return fail(HGQ_ERR_ARG, "hgq_conv2d_maxpool_bwd_coded: null workspace");
+    if (reduce) return conv2d_bwd_impl(nullptr, nullptr, xq, qw, dxq, dqw, dqb, workspace, g, F, act, stream, true, dyp, code);
+    return conv2d_bwd_impl(nullptr, nullptr, xq, qw, dxq, workspace, workspace, workspace, g, F, act, stream, false, dyp, code);
 }
 
 extern "C" int hgq_conv2d_ebops(const float *bits_in, const float *bits_ker, const hgq_conv_geom *g, int F, float *total,

@@ -1160,6 +1160,59 @@ def _(dyp, y, xq, qw, geom, act, need_dx, reduce):
     return xq.new_empty(xq.shape if need_dx else (0,)), xq.new_empty((n,) if reduce else (1, n))
 
 
+@torch.library.custom_op('hgq::conv2d_maxpool_fwd_coded', mutates_args=())
+def conv2d_maxpool_fwd_coded(xq: Tensor, qw: Tensor, qb: Tensor, geom: Sequence[int], act: int) -> tuple[Tensor, Tensor]:
+    """``(code, maxpool2x2(act(conv2d(xq, qw) + qb)))`` in one launch; the unpooled tensor is never written.  ``code`` (uint8,
+    the pooled shape): bits 0-1 the row-major place of each window's first maximum, bit 2 whether it is positive."""
+    _check_f32('xq', xq), _check_f32('qw', qw), _check_f32('qb', qb)
+    g = _geom(geom)
+    F = qw.shape[-1]
+    _need(xq.numel() == g.B * g.H * g.W * g.C and tuple(qw.shape) == (g.kh, g.kw, g.C, F), 'xq / qw do not match the geometry')
+    _need(qb.numel() in (0, F), 'qb must hold one entry per filter')
+    code = torch.empty((g.B, g.OH // 2, g.OW // 2, F), dtype=torch.uint8, device=xq.device)
+    yp = torch.empty((g.B, g.OH // 2, g.OW // 2, F), dtype=torch.float32, device=xq.device)
+    rc = _lib.load().hgq_conv2d_maxpool_fwd_coded(_ptr(xq), _ptr(qw), _ptr(qb) if qb.numel() else None, _ptr(yp), _ptr(code),
+                                                  ctypes.addressof(g), F, act, _stream())
+    _lib.check(rc, 'hgq_conv2d_maxpool_fwd_coded')
+    return code, yp
+
+
+@conv2d_maxpool_fwd_coded.register_fake
+def _(xq, qw, qb, geom, act):
+    F = qw.shape[-1]
+    shape = (geom[0], geom[12] // 2, geom[13] // 2, F)
+    return xq.new_empty(shape, dtype=torch.uint8), xq.new_empty(shape)
+
+
+@torch.library.custom_op('hgq::conv2d_maxpool_bwd_coded', mutates_args=())
+def conv2d_maxpool_bwd_coded(dyp: Tensor, code: Tensor, xq: Tensor, qw: Tensor, geom: Sequence[int], act: int, need_dx: bool,
+                             reduce: bool) -> tuple[Tensor, Tensor]:
+    """``conv2d_maxpool_bwd`` from the forward pass's window codes instead of its unpooled output."""
+    _check_f32('dyp', dyp), _check_f32('xq', xq), _check_f32('qw', qw)
+    g = _geom(geom)
+    F = qw.shape[-1]
+    n_p = g.B * (g.OH // 2) * (g.OW // 2) * F
+    _need(code.dtype == torch.uint8 and code.is_contiguous() and code.numel() == n_p, 'code must be uint8 [B, OH // 2, OW // 2, F]')
+    _need(dyp.numel() == n_p, 'dyp must be [B, OH // 2, OW // 2, F]')
+    lib = _lib.load()
+    dx = torch.empty(xq.shape if need_dx else (0,), dtype=torch.float32, device=xq.device)
+    n = lib.hgq_conv2d_bwd_slice_count(ctypes.addressof(g), F)
+    _need(n >= 1, 'hgq_conv2d_bwd_slice_count rejected the geometry')
+    ws = torch.empty((int(n), qw.numel() + F), dtype=torch.float32, device=xq.device)
+    out = torch.empty(qw.numel() + F, dtype=torch.float32, device=xq.device) if reduce else ws
+    rc = lib.hgq_conv2d_maxpool_bwd_coded(_ptr(dyp), _ptr(code), _ptr(xq), _ptr(qw), _ptr(dx) if need_dx else None, _ptr(out),
+                                          out.data_ptr() + 4 * qw.numel() if reduce else None, _ptr(ws), ctypes.addressof(g), F, act,
+                                          int(reduce), _stream())
+    _lib.check(rc, 'hgq_conv2d_maxpool_bwd_coded')
+    return dx, out
+
+
+@conv2d_maxpool_bwd_coded.register_fake
+def _(dyp, code, xq, qw, geom, act, need_dx, reduce):
+    n = qw.numel() + qw.shape[-1]
+    return xq.new_empty(xq.shape if need_dx else (0,)), xq.new_empty((n,) if reduce else (1, n))
+
+
 def conv2d_maxpool_supported(geom, F: int) -> bool:
     g = _geom(geom)
     return bool(_lib.load().hgq_conv2d_maxpool_bwd_supported(ctypes.addressof(g), int(F)))
@@ -2195,12 +2248,13 @@ class _Conv2D(torch.autograd.Function):
 
 
 class _Conv2DMaxPool(torch.autograd.Function):
-    """Convolution and the 2 x 2 maximum pooling that is its only reader as one node: the unpooled output stays inside
-    (saved for the backward pass, which forms its gradient from the pooled one while it stages its tiles)."""
+    """Convolution and the 2 x 2 maximum pooling that is its only reader as one node: the unpooled output is never
+    written; a byte per window and filter (where the maximum sat, whether it was positive) is saved for the backward
+    pass, which forms the unpooled gradient from the pooled one while it stages its tiles."""
 
     @staticmethod
     def forward(ctx, xq, qw, qb, geom, act):
-        y, yp = conv2d_maxpool_fwd(xq, qw, qb, list(geom), act)
+        y, yp = conv2d_maxpool_fwd_coded(xq, qw, qb, list(geom), act)
         ctx.save_for_backward(xq, qw, y)
         ctx.geom, ctx.act, ctx.has_bias = tuple(geom), act, qb.numel() > 0
         ctx.defer = getattr(qw, '_hgq_single_use', False) and (qb.numel() == 0 or getattr(qb, '_hgq_single_use', False))
@@ -2211,11 +2265,11 @@ class _Conv2DMaxPool(torch.autograd.Function):
         xq, qw, y = ctx.saved_tensors
         need_dx = ctx.needs_input_grad[0]
         if ctx.defer and _SINK['open']:  # as in _Conv2D: the slices join the pass's one reduction launch
-            dx, ws = conv2d_maxpool_bwd(gyp.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, need_dx, False)
+            dx, ws = conv2d_maxpool_bwd_coded(gyp.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, need_dx, False)
             dqw, dqb = torch.empty_like(qw), xq.new_empty(qw.shape[-1])
             _PENDING_REDUCE.append((ws, (dqw.view(-1), dqb, xq.new_empty(0)), (False, not ctx.has_bias, True)))
         else:
-            dx, flat = conv2d_maxpool_bwd(gyp.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, need_dx, True)
+            dx, flat = conv2d_maxpool_bwd_coded(gyp.contiguous(), y, xq, qw, list(ctx.geom), ctx.act, need_dx, True)
             dqw, dqb = flat[:qw.numel()].view(qw.shape), flat[qw.numel():]
         return (dx if need_dx else None, dqw, dqb if ctx.has_bias else None, None, None)
 

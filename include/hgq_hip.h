@@ -624,6 +624,18 @@ int hgq_conv2d_maxpool_fwd(const float *xq, const float *qw, const float *qb, fl
                            int act, void *stream);
 int hgq_conv2d_maxpool_bwd(const float *dyp, const float *y, const float *xq, const float *qw, float *dxq, float *dqw, float *dqb,
                            float *workspace, const hgq_conv_geom *g, int F, int act, int reduce, void *stream);
+/*
+ * The same pair with the unpooled output replaced by what the backward pass needs of it: `code`
+ * [B, OH / 2, OW / 2, F], one byte per pooling window and filter - bits 0-1 the place (row-major, 0..3) of the window's
+ * first maximum, bit 2 set where that maximum is positive.  The forward pass writes yp and code and never writes the
+ * unpooled tensor (four times yp's size); the backward pass reads dyp and code.  Results are those of
+ * hgq_conv2d_maxpool_fwd / _bwd bit for bit.  code must be 4-byte aligned.  Same shapes and errors otherwise.
+ * (No counterpart in the reference, whose Keras layers keep the unpooled tensor: reference src/hgq/layers/conv.py:72-102.)
+ */
+int hgq_conv2d_maxpool_fwd_coded(const float *xq, const float *qw, const float *qb, float *yp, uint8_t *code,
+                                 const hgq_conv_geom *g, int F, int act, void *stream);
+int hgq_conv2d_maxpool_bwd_coded(const float *dyp, const uint8_t *code, const float *xq, const float *qw, float *dxq, float *dqw,
+                                 float *dqb, float *workspace, const hgq_conv_geom *g, int F, int act, int reduce, void *stream);
 
 /*
  * One quantizer's bit-width view for the EBOPs entry points below: `bits` / `fbits` as hgq_qbits_fwd forms

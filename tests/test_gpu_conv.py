@@ -341,6 +341,17 @@ def test_convolution_backward_from_the_pooled_gradient(dev, shape):
     for name, a, f in zip(('pooled output', 'dx', 'dw', 'db'), got[0], got[1]):
         if a is not None:
             assert torch.equal(a, f), f'{name}: {float((a - f).abs().max())}'
+    # the entry points that keep the unpooled output (the node above saves a byte per window and filter instead) give the same bits
+    xs, ws = x.to(dev), w.to(dev)
+    bs = b.to(dev) if bias else xs.new_empty(0)
+    y, yp = ops.conv2d_maxpool_fwd(xs, ws, bs, list(geom), act)
+    assert torch.equal(yp, got[1][0])
+    assert torch.equal(y, ops.conv2d(xs, ws, bs if bias else None, (1, 1), padding, (1, 1), act))
+    dyp = torch.randn(yp.shape, generator=torch.Generator().manual_seed(5)).to(dev)
+    dx, flat = ops.conv2d_maxpool_bwd(dyp, y, xs, ws, list(geom), act, True, True)
+    assert torch.equal(dx, got[1][1]) and torch.equal(flat[:w.numel()].view(w.shape), got[1][2])
+    if bias:
+        assert torch.equal(flat[w.numel():], got[1][3])
     # and against torch's own kernels in fp64 on the CPU
     xd, wd = x.double().requires_grad_(True), w.double().requires_grad_(True)
     pad = (k - 1) // 2 if padding == 'same' else 0
