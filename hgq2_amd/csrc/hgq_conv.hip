@@ -495,7 +495,9 @@ __global__ __launch_bounds__(256) void dgrad_patch_kernel(const float *__restric
 #define SC_TH 8
 #define SC_TW 32
 
-template <int KH, int KW, int C>
+// UNIT: unit stride and dilation - the patch sizes and every tap offset are compile-time constants (the LDS reads of a
+// pixel then differ only in their immediate offsets: no address arithmetic in the loop).
+template <int KH, int KW, int C, bool UNIT = false>
 __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                          const float *__restrict__ bias, float *__restrict__ out, hgq_conv_geom g,
                                                          int F, int act, int tiles_x, int tiles_y, float *__restrict__ pooled,
@@ -503,7 +505,8 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
 #pragma clang fp contract(fast)  // multiply-adds of the convolution sum may fuse (see bwd_smallc_kernel)
     constexpr int KC = KH * KW * C;
     extern __shared__ float lds[];  // input patch [XH][XW][C]
-    const int XH = (SC_TH - 1) * g.sy + (KH - 1) * g.dly + 1, XW = (SC_TW - 1) * g.sx + (KW - 1) * g.dlx + 1;
+    const int sy = UNIT ? 1 : g.sy, sx = UNIT ? 1 : g.sx, dly = UNIT ? 1 : g.dly, dlx = UNIT ? 1 : g.dlx;
+    const int XH = (SC_TH - 1) * sy + (KH - 1) * dly + 1, XW = (SC_TW - 1) * sx + (KW - 1) * dlx + 1;
     const int f = threadIdx.x & 31, slot = threadIdx.x >> 5;
     const bool f_on = f < F;
     float wreg[KC];
@@ -515,7 +518,7 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         const int b = (int)(tile / (tiles_y * tiles_x)), rem = (int)(tile - (int64_t)b * tiles_y * tiles_x);
         const int oy0 = (rem / tiles_x) * SC_TH, ox0 = (rem % tiles_x) * SC_TW;
-        const int iy0 = oy0 * g.sy - g.py, ix0 = ox0 * g.sx - g.px;
+        const int iy0 = oy0 * sy - g.py, ix0 = ox0 * sx - g.px;
         __syncthreads();
         const FastDiv d_xw((uint32_t)(XW * C));
         for (int e = threadIdx.x; e < XH * XW * C; e += 256) {
@@ -537,32 +540,37 @@ __global__ __launch_bounds__(256) void fwd_smallc_kernel(const float *__restrict
             float *prow = pooled ? pooled + pbase : nullptr;
             uint8_t *crow = code ? code + pbase : nullptr;
             const bool p_row = pooled && (oy >> 1) < PHo;  // both rows of the window exist: both halves are in this loop
-            float left = 0.f;
-            for (int tx = 0; tx < n_x; ++tx) {
-                const float *xp = lds + (slot * g.sy * XW + tx * g.sx) * C;
+            auto pixel = [&](int tx) -> float {
+                const float *xp = lds + (slot * sy * XW + tx * sx) * C;
                 float acc = bb;
 #pragma unroll
                 for (int t = 0; t < KC; ++t) {
                     const int ky = t / (KW * C), kx = (t / C) % KW, c = t % C;
-                    acc += xp[(ky * g.dly * XW + kx * g.dlx) * C + c] * wreg[t];
+                    acc += xp[(ky * dly * XW + kx * dlx) * C + c] * wreg[t];
                 }
                 if (act == HGQ_ACT_RELU) acc = acc > 0.f ? acc : 0.f;
-                if (f_on && orow) orow[(int64_t)tx * F] = acc;
+                return acc;
+            };
+            // two pixels - the two columns of a pooling window - per trip: two independent sums in flight
+            int tx = 0;
+            for (; tx + 1 < n_x; tx += 2) {
+                const float left = pixel(tx), acc = pixel(tx + 1);
+                if (f_on && orow) orow[(int64_t)tx * F] = left, orow[(int64_t)(tx + 1) * F] = acc;
                 if (p_row) {
-                    if (tx & 1) {
-                        const bool right = acc > left;
-                        const float m = right ? acc : left, mo = __shfl_xor(m, 32);
-                        const int j = right ? 1 : 0, jo = __shfl_xor(j, 32);
-                        if (!(slot & 1) && f_on && ((ox0 + tx) >> 1) < PWo) {
-                            const bool lower = mo > m;  // the lower row takes the window only with a larger value
-                            const float best = lower ? mo : m;
-                            prow[(int64_t)(tx >> 1) * F] = best;
-                            if (crow) crow[(int64_t)(tx >> 1) * F] = (uint8_t)((lower ? 2 + jo : j) | (best > 0.f ? 4 : 0));
-                        }
-                    } else {
-                        left = acc;
+                    const bool right = acc > left;
+                    const float m = right ? acc : left, mo = __shfl_xor(m, 32);
+                    const int j = right ? 1 : 0, jo = __shfl_xor(j, 32);
+                    if (!(slot & 1) && f_on && ((ox0 + tx) >> 1) < PWo) {
+                        const bool lower = mo > m;  // the lower row takes the window only with a larger value
+                        const float best = lower ? mo : m;
+                        prow[(int64_t)(tx >> 1) * F] = best;
+                        if (crow) crow[(int64_t)(tx >> 1) * F] = (uint8_t)((lower ? 2 + jo : j) | (best > 0.f ? 4 : 0));
                     }
                 }
+            }
+            if (tx < n_x) {  // a last column without a window
+                const float acc = pixel(tx);
+                if (f_on && orow) orow[(int64_t)tx * F] = acc;
             }
         }
     }
@@ -1546,7 +1554,13 @@ extern "C" int hgq_conv2d_fwd(const float *xq, const float *qw, const float *qb,
         const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
         const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
         const size_t lds = fwd_smallc_lds(*g);
-#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, (float *)nullptr, (uint8_t *)nullptr)
+#define HGQ_FWD_SC(KH, KW, CC)                                                                                                                      \
+    do {                                                                                                                                            \
+        if (g->sy == 1 && g->sx == 1 && g->dly == 1 && g->dlx == 1)                                                                                 \
+            hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC, true>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, (float *)nullptr, (uint8_t *)nullptr); \
+        else                                                                                                                                        \
+            hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC, false>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, (float *)nullptr, (uint8_t *)nullptr); \
+    } while (0)
         HGQ_SMALLC_DISPATCH(HGQ_FWD_SC);
 #undef HGQ_FWD_SC
         return check_launch("hgq_conv2d_fwd(few channels)");
@@ -1746,7 +1760,8 @@ static int conv2d_maxpool_fwd_impl(const float *xq, const float *qw, const float
     const int tiles_x = (g->OW + SC_TW - 1) / SC_TW, tiles_y = (g->OH + SC_TH - 1) / SC_TH;
     const dim3 grid((unsigned)persistent_grid((int64_t)g->B * tiles_x * tiles_y, 8));
     const size_t lds = fwd_smallc_lds(*g);
-#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, yp, code)
+    // (hgq_conv2d_maxpool_bwd_supported holds only for unit stride and dilation)
+#define HGQ_FWD_SC(KH, KW, CC) hipLaunchKernelGGL((fwd_smallc_kernel<KH, KW, CC, true>), grid, dim3(256), lds, s, xq, qw, qb, y, *g, F, act, tiles_x, tiles_y, yp, code)
     HGQ_SMALLC_DISPATCH(HGQ_FWD_SC);
 #undef HGQ_FWD_SC
     return check_launch(who);
