@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void qdense_bwd_kernel(const float *__restrict
     const int blk = wave / wpb, sub = wave % wpb;
     const int wkb = blk / N32, wnb = blk % N32;
     const int rows_per = BWD_BM / wpb;
-    floatx16 accw = {0};
+    floatx16 accw = {0}, acc2 = {0};  // acc2: the second block of a wavefront with PAIRS
     float accb = 0.f;
     const int bn = tid & 63, bq = tid >> 6;  // bias column / row quarter
 
@@ -966,7 +966,11 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bf16_kernel(const float 
 // recomputed on the matrix cores (dy = gm, y = gs, both [N]); no activation, no bias, no quantizer.
 // BF: the three contractions run on the bf16 matrix cores by exact splitting (mfma_chain_bf16); the gradient operand is
 // taken in all three parts without looking, the quantized input and the kernel in as many as they need.
-template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true, bool BF = false>
+// PAIRS (with BF; K and N above 32): wavefronts 0 and 1 take the two row halves of dx (both k blocks: the gradient rows they
+// contract are split into bf16 parts once for both), wavefronts 2 and 3 the two column halves of the kernel gradient (both k
+// blocks, all rows of the tile) - every gradient value is split twice per tile instead of four times.  A wavefront's two
+// blocks live in the same registers either way: reset per tile for dx, kept across the tiles for the kernel gradient.
+template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true, bool BF = false, bool PAIRS = false>
 __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
@@ -1026,7 +1030,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     const int blk = wave / wpb, sub = wave % wpb;
     const int wkb = blk / N32, wnb = blk % N32;
     const int rows_per = FAST_BM / wpb;
-    floatx16 accw = {0};
+    floatx16 accw = {0}, acc2 = {0};  // acc2: the second block of a wavefront with PAIRS
     float accb = 0.f;
     const int bn = tid & 63, bq = tid >> 6;
     const bool relu = act == HGQ_ACT_RELU;
@@ -1125,7 +1129,33 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         // ---- dx = dz @ qW^T : blocks (row half, k block), kept in registers until dz is no longer needed
         floatx16 acc = {0};
         const int rh = wave & 1, kb = wave >> 1;
-        if (split_n) {
+        if (PAIRS) {
+            const int kq = lane >> 5, c32 = lane & 31;
+            if (wave < 2) {
+                accw = floatx16{0}, acc2 = floatx16{0};
+#pragma unroll
+                for (int bt = 0; bt < 4; ++bt) {
+                    float a[8], b0[8], b1[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int n = 16 * bt + 2 * u + kq;
+                        a[u] = dzs[wave * 32 + c32][n], b0[u] = ws[c32][n], b1[u] = ws[32 + c32][n];
+                    }
+                    mfma_batch2_bf16<true>(accw, acc2, a, b0, b1);
+                }
+            } else {
+#pragma unroll
+                for (int bt = 0; bt < FAST_BM / 16; ++bt) {
+                    float b[8], a0[8], a1[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int r = 16 * bt + 2 * u + kq;
+                        b[u] = dzs[r][(wave - 2) * 32 + c32], a0[u] = xs[r][c32], a1[u] = xs[r][32 + c32];
+                    }
+                    mfma_batch2_bf16<false>(accw, acc2, b, a0, a1);
+                }
+            }
+        } else if (split_n) {
             // one k block, two column blocks: the two wavefronts of a row half take one half of the contraction each
             const int arow = rh * 32 + (lane & 31), kq = lane >> 5, n0 = kb * 32;
             acc = BF ? mfma_chain_bf16<true, false>(acc, &dzs[arow][n0 + kq], 1, &ws[lane & 31][n0 + kq], 1, 2)
@@ -1136,7 +1166,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                      : mfma_chain(acc, &dzs[arow][kq], 1, &ws[wrow][kq], 1, N32 * 2);
         }
         // ---- dW += xq^T @ dz : this wave's block, its slice of the tile's rows
-        {
+        if (!PAIRS) {
             const int rbeg = sub * rows_per;
             const int kq = lane >> 5, c32 = lane & 31;
             accw = BF ? mfma_chain_bf16<false, true>(accw, &xs[rbeg + kq][wkb * 32 + c32], FAST_LD, &dzs[rbeg + kq][wnb * 32 + c32], FAST_LD, rows_per / 16)
@@ -1147,7 +1177,15 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
             for (int j = 0; j < FAST_BM / 4; ++j) accb += dzs[bq * (FAST_BM / 4) + j][bn];
         }
         __syncthreads();  // dz and xq consumed: the dx tile takes the place of dz (its second partial sum that of xq)
-        if (split_n) {
+        if (PAIRS) {
+            if (wave < 2) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    dzs[wave * 32 + acc_row(r, lane)][lane & 31] = accw[r];
+                    dzs[wave * 32 + acc_row(r, lane)][32 + (lane & 31)] = acc2[r];
+                }
+            }
+        } else if (split_n) {
             float(*dst)[FAST_LD] = kb ? xs : dzs;
 #pragma unroll
             for (int r = 0; r < 16; ++r) dst[rh * 32 + acc_row(r, lane)][lane & 31] = acc[r];
@@ -1186,7 +1224,18 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     // ---- write this workgroup's slice.  Waves sharing a kernel-gradient block combine through LDS.
     __syncthreads();
     float *comb = &xs[0][0];
-    for (int pass = 0; pass < wpb; ++pass) {
+    if (PAIRS) {
+        if (wave >= 2) {
+            const int n = (wave - 2) * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                comb[acc_row(r, lane) * FAST_LD + n] = accw[r];
+                comb[(32 + acc_row(r, lane)) * FAST_LD + n] = acc2[r];
+            }
+        }
+        __syncthreads();
+    }
+    for (int pass = 0; pass < (PAIRS ? 0 : wpb); ++pass) {
         if (sub == pass) {
             const int n = wnb * 32 + (lane & 31);
 #pragma unroll
@@ -1620,7 +1669,10 @@ static int qdense_bwd_impl(const float *dy, const float *y, const float *x, cons
         const bool zvec = N % 4 == 0 && aligned16(dy) && (act != HGQ_ACT_RELU || aligned16(y));
 #define HGQ_BWD_FAST(RMV, QV)                                                                                                          \
     do {                                                                                                                               \
-        if (zvec && g_dense_bf16)                                                                                                      \
+        if (zvec && g_dense_bf16 && K > 32 && N > 32)                                                                                  \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true, true, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
+                               dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
+        else if (zvec && g_dense_bf16)                                                                                                 \
             hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
                                dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
         else if (zvec)                                                                                                                 \

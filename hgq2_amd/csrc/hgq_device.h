@@ -393,6 +393,39 @@ __device__ __forceinline__ floatx16 mfma_batch_bf16(floatx16 acc, const float (&
     return acc;
 }
 
+// Two result blocks that share an operand which is a gradient (arbitrary fp32: all three parts): the shared operand is split
+// ONCE for both.  SHARED_A: acc0 += a * b0, acc1 += a * b1; else acc0 += a0 * b, acc1 += a1 * b (then `a` is unused and
+// b0 / b1 hold a0 / a1).  The other operand of a block takes the bf16 instruction where it has a single part (three
+// instructions) and the eight fp32 instructions otherwise, block by block.
+template <bool SHARED_A>
+__device__ __forceinline__ void mfma_batch2_bf16(floatx16 &acc0, floatx16 &acc1, const float (&sh)[8], const float (&o0)[8],
+                                                 const float (&o1)[8]) {
+    u32x4_t s0, s1, s2, q0, q1;
+    bf16_lead8(sh, s0);
+    bf16_rest8(sh, s1, s2);
+    const bool one0 = bf16_lead8(o0, q0), one1 = bf16_lead8(o1, q1);
+    if (one0) {
+        acc0 = SHARED_A ? mfma_bf16(s0, q0, acc0) : mfma_bf16(q0, s0, acc0);
+        acc0 = SHARED_A ? mfma_bf16(s1, q0, acc0) : mfma_bf16(q0, s1, acc0);
+        acc0 = SHARED_A ? mfma_bf16(s2, q0, acc0) : mfma_bf16(q0, s2, acc0);
+    } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            acc0 = SHARED_A ? __builtin_amdgcn_mfma_f32_32x32x2f32(sh[u], o0[u], acc0, 0, 0, 0)
+                            : __builtin_amdgcn_mfma_f32_32x32x2f32(o0[u], sh[u], acc0, 0, 0, 0);
+    }
+    if (one1) {
+        acc1 = SHARED_A ? mfma_bf16(s0, q1, acc1) : mfma_bf16(q1, s0, acc1);
+        acc1 = SHARED_A ? mfma_bf16(s1, q1, acc1) : mfma_bf16(q1, s1, acc1);
+        acc1 = SHARED_A ? mfma_bf16(s2, q1, acc1) : mfma_bf16(q1, s2, acc1);
+    } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            acc1 = SHARED_A ? __builtin_amdgcn_mfma_f32_32x32x2f32(sh[u], o1[u], acc1, 0, 0, 0)
+                            : __builtin_amdgcn_mfma_f32_32x32x2f32(o1[u], sh[u], acc1, 0, 0, 0);
+    }
+}
+
 // Same arguments and LDS reads as mfma_chain, every batch through mfma_batch_bf16: never slower than mfma_chain by more
 // than the look at the operands.
 template <bool FULL_A, bool FULL_B>
