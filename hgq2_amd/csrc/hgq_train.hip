@@ -210,7 +210,23 @@ __global__ __launch_bounds__(256) void mse_partial_kernel(const float *__restric
     __shared__ float red[4];
     float acc = 0.f;
     const int64_t n4 = n >> 2, stride = (int64_t)gridDim.x * 256;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
+    // four vectors of a thread per trip, every load of the trip in flight before the first is used
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+        f32x4_t p[4], t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            p[u] = ((const f32x4_t *)pred)[i + u * stride];
+            t[u] = target ? ((const f32x4_t *)target)[i + u * stride] : f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const f32x4_t d = p[u] - t[u];
+            acc += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+            if (dpred) ((f32x4_t *)dpred)[i + u * stride] = d * two_over_n;
+        }
+    }
+    for (; i < n4; i += stride) {
         const f32x4_t p = ((const f32x4_t *)pred)[i];
         const f32x4_t t = target ? ((const f32x4_t *)target)[i] : f32x4_t{0.f, 0.f, 0.f, 0.f};
         const f32x4_t d = p - t;

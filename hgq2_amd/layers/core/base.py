@@ -43,20 +43,19 @@ class QLayerBase(Layer):
     def __init__(self, enable_ebops=None, beta0=None, enable_oq=None, enable_iq=None, oq_conf=None,
                  ebops_factor: float = 1.0, **kwargs):
         super().__init__(**kwargs)
-        beta0 = beta0 if beta0 is not None else global_config['beta0']
-        beta0 = Constant(float(beta0)) if not isinstance(beta0, Initializer) else beta0
-        self._enable_iq = enable_iq if enable_iq is not None else global_config['enable_iq']
-        self._enable_oq = enable_oq if enable_oq is not None else global_config['enable_oq']
-        if enable_ebops is None:
-            enable_ebops = global_config['enable_ebops'] and self.enable_iq
-        self._enable_ebops = enable_ebops
-        self._beta0 = beta0
+        # arguments left at None take the scope's defaults (config.layer.global_config)
+        def scoped(value, key):
+            return global_config[key] if value is None else value
+
+        start = scoped(beta0, 'beta0')
+        self._beta0 = start if isinstance(start, Initializer) else Constant(float(start))
+        self._enable_iq, self._enable_oq = scoped(enable_iq, 'enable_iq'), scoped(enable_oq, 'enable_oq')
+        # the resource estimate needs the input bit-widths: without an input quantizer it is off unless asked for
+        self._enable_ebops = (global_config['enable_ebops'] and self._enable_iq) if enable_ebops is None else enable_ebops
         self.ebops_factor = ebops_factor
-        self._beta = None
-        self._ebops = None
-        if self.enable_oq:
-            oq_conf = oq_conf or QuantizerConfig('default', 'datalane')
-            self._oq = Quantizer(oq_conf, name=f'{self.name}_oq')
+        self._beta = self._ebops = None
+        if self._enable_oq:
+            self._oq = Quantizer(oq_conf if oq_conf else QuantizerConfig('default', 'datalane'), name=f'{self.name}_oq')
 
     @property
     def enable_iq(self):
@@ -69,7 +68,7 @@ class QLayerBase(Layer):
     @property
     def oq(self):
         if not self.enable_oq:
-            raise AttributeError(f'oq has been disabled for {self.name}.')
+            raise AttributeError(f'{self.name} was built without an output quantizer (enable_oq=False)')
         return self._oq
 
     @property
@@ -129,9 +128,9 @@ class QLayerBase(Layer):
         self._finish_call()
         if not self.enable_oq or self.__output_quantizer_handled__ or self._oq_applied_in_call:
             return r
-        assert not isinstance(r, (tuple, list)), (
-            f'Layer {self.name}({type(self)}) returns multiple outputs, which must be handled in subclasses.'
-        )
+        if isinstance(r, (tuple, list)):
+            raise AssertionError(f'{type(self).__name__} {self.name!r} returned {len(r)} outputs: a layer with several outputs '
+                                 'applies its output quantizers itself (__output_quantizer_handled__)')
         return self.oq(r, training=training)
 
     def _finish_call(self):
@@ -149,20 +148,19 @@ class QLayerBase(Layer):
         }
 
     def _compute_ebops(self, *args, **kwargs):
-        raise NotImplementedError('This method is abstract and should be implemented in subclasses.')
+        raise NotImplementedError(f'{type(self).__name__} does not define its EBOPs estimate')
 
 
 class QLayerBaseSingleInput(QLayerBase):
     def __init__(self, iq_conf: QuantizerConfig | None = None, **kwargs):
         super().__init__(**kwargs)
-        if self.enable_iq:
-            iq_conf = iq_conf or QuantizerConfig('default', 'datalane')
-            self._iq = Quantizer(iq_conf, name=f'{self.name}_iq')
+        if self._enable_iq:
+            self._iq = Quantizer(iq_conf if iq_conf else QuantizerConfig('default', 'datalane'), name=f'{self.name}_iq')
 
     @property
     def iq(self):
         if not self.enable_iq:
-            raise AttributeError(f'iq has been disabled for {self.name}.')
+            raise AttributeError(f'{self.name} was built without an input quantizer (enable_iq=False)')
         return self._iq
 
     def build(self, input_shape=None):
@@ -179,32 +177,35 @@ class QLayerBaseSingleInput(QLayerBase):
 
 
 class MultipleQuantizers(Layer):
+    """One quantizer per input of a layer that takes several; behaves as the sequence of them."""
+
     def __init__(self, configs: Sequence[QuantizerConfig], **kwargs):
         super().__init__(**kwargs)
-        self.quantizers = nn.ModuleList(Quantizer(config) for config in configs)
+        self.quantizers = nn.ModuleList([Quantizer(c) for c in configs])
 
     def call(self, x, training=None):
-        assert len(self) == len(x), f'{self.name} ({self.__class__.__name__}) expects {len(self)} inputs, got {len(x)}.'
-        return tuple(f(x_, training=training) for f, x_ in zip(self.quantizers, x))
+        if len(x) != len(self.quantizers):
+            raise AssertionError(f'{self.name}: {len(self.quantizers)} quantizers for {len(x)} inputs')
+        return tuple(q(t, training=training) for q, t in zip(self.quantizers, x))
 
     def build(self, shapes):
-        for q, shape in zip(self.quantizers, shapes):
+        for shape, q in zip(shapes, self.quantizers):
             q._build_device = self._build_device
             q.build(tuple(shape))
             q.built = True
         self.built = True
 
-    def __bool__(self):
-        return len(self.quantizers) > 0
-
     def __len__(self):
         return len(self.quantizers)
 
-    def __getitem__(self, item):
-        return self.quantizers[item]
+    def __bool__(self):
+        return len(self) != 0
 
     def __iter__(self):
         return iter(self.quantizers)
+
+    def __getitem__(self, index):
+        return self.quantizers[index]
 
 
 class QLayerBaseMultiInputs(QLayerBase):
@@ -216,28 +217,25 @@ class QLayerBaseMultiInputs(QLayerBase):
     @property
     def iq(self):
         if not self.enable_iq:
-            raise AttributeError(f'iq has been disabled for {self.name}.')
+            raise AttributeError(f'{self.name} was built without input quantizers (enable_iq=False)')
         if not self.built:
-            raise AttributeError(f'iqs is not available before build for {self.name}.')
+            raise AttributeError(f'{self.name}: the input quantizers exist once the layer is built (one per input)')
         return self._iq
 
     @property
     def iq_confs(self):
-        assert self.enable_iq, f'iq_confs has been disabled for {self.name}.'
+        assert self.enable_iq, f'{self.name} has no input quantizers, hence no iq_confs'
         return self._iq_confs
 
     def build(self, input_shape=None):
         super().build(input_shape)
         if not self.enable_iq:
             return
-        n_input = len(input_shape)
-        for s in input_shape:
-            assert isinstance(s, Iterable), f'each element of input_shape must be iterable, got {s}'
-        if isinstance(self.iq_confs, QuantizerConfig):
-            self._iq_confs = [self.iq_confs] * n_input
-        assert len(self.iq_confs) == n_input, (
-            f'number of iq_confs must match number of inputs, got {len(self._iq_confs)} != {n_input}'
-        )
+        for shape in input_shape:
+            assert isinstance(shape, Iterable), f'{self.name}: input_shape must list one shape per input, found {shape!r}'
+        if isinstance(self._iq_confs, QuantizerConfig):  # one configuration for every input
+            self._iq_confs = [self._iq_confs for _ in input_shape]
+        assert len(self._iq_confs) == len(input_shape), f'{self.name}: {len(self._iq_confs)} iq_confs for {len(input_shape)} inputs'
         self._iq = MultipleQuantizers(self._iq_confs)
         self._iq._build_device = self._build_device
         self._iq.build(input_shape)

@@ -55,41 +55,41 @@ class BitwidthMapperBase:
 
 
 def check_axis(axis: Sequence[int], ndim: int):
-    axis = [a if a >= 0 else a + ndim for a in axis]
-    assert all(0 <= a < ndim for a in axis), f'Invalid axis {axis} for shape {ndim}.'
-    return axis
+    """Axes counted from the front (negative ones wrap once); anything outside the rank is refused."""
+    front = [a + ndim if a < 0 else a for a in axis]
+    bad = [a for a in front if not 0 <= a < ndim]
+    assert not bad, f'axes {bad} (of {list(axis)}) do not exist in a tensor of rank {ndim}'
+    return front
 
 
 class DefaultBitwidthMapper(BitwidthMapperBase):
     """Bit-widths are shared along the homogeneous axes and individual along the others."""
 
     def __init__(self, heterogeneous_axis=None, homogeneous_axis=None, **kwargs):
-        _shape_inferenced = kwargs.pop('_shape_inferenced', False)
-        if not _shape_inferenced:
-            assert (heterogeneous_axis is None) ^ (homogeneous_axis is None), (
-                'Only one of quantize_dims and skip_dims can be specified.'
-            )
-        self.heterogeneous_axis = heterogeneous_axis
-        self.homogeneous_axis = homogeneous_axis
-        self._shape_inferenced = _shape_inferenced
+        # a restored mapper (_shape_inferenced) carries both lists; a new one names exactly one of them, the other follows
+        self._shape_inferenced = bool(kwargs.pop('_shape_inferenced', False))
+        if not self._shape_inferenced and (heterogeneous_axis is None) == (homogeneous_axis is None):
+            raise AssertionError('give either heterogeneous_axis or homogeneous_axis, not both and not neither')
+        self.heterogeneous_axis, self.homogeneous_axis = heterogeneous_axis, homogeneous_axis
 
     def inference_weight_shape(self, input_shape):
-        n = len(input_shape)
-        axis = np.arange(n)
+        rank = len(input_shape)
         if self.heterogeneous_axis is not None:
-            self.heterogeneous_axis = tuple(check_axis(self.heterogeneous_axis, n))
-            self.homogeneous_axis = tuple(int(a) for a in np.setdiff1d(axis, self.heterogeneous_axis))
+            own = sorted(check_axis(self.heterogeneous_axis, rank))
+            shared = [a for a in range(rank) if a not in own]
+            self.heterogeneous_axis, self.homogeneous_axis = tuple(check_axis(self.heterogeneous_axis, rank)), tuple(shared)
         elif self.homogeneous_axis is not None:
-            self.homogeneous_axis = tuple(check_axis(self.homogeneous_axis, n))
-            self.heterogeneous_axis = tuple(int(a) for a in np.setdiff1d(axis, self.homogeneous_axis))
-        weight_shape = [1] * n
-        for i in self.heterogeneous_axis:
-            assert input_shape[i] is not None, (
-                f'Unable to heterogeneously quantize axis {i} with unknown shape. Input shape: {input_shape}.'
-            )
-            weight_shape[i] = int(input_shape[i])
+            shared = check_axis(self.homogeneous_axis, rank)
+            self.homogeneous_axis = tuple(shared)
+            self.heterogeneous_axis = tuple(a for a in range(rank) if a not in shared)
+        # one entry per position along the axes with bit-widths of their own, a single one along the shared axes
+        shape = [1] * rank
+        for a in self.heterogeneous_axis:
+            if input_shape[a] is None:
+                raise AssertionError(f'axis {a} of {tuple(input_shape)} has no fixed size: it cannot carry bit-widths of its own')
+            shape[a] = int(input_shape[a])
         self._shape_inferenced = True
-        return tuple(weight_shape)
+        return tuple(shape)
 
     def bw_to_x(self, bw, x_shape):
         return torch.broadcast_to(bw, tuple(x_shape))
