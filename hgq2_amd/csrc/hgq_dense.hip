@@ -577,13 +577,16 @@ __device__ __forceinline__ void bf16_stage(const f32x4_t (&raw)[FAST_NJ], const 
 // returns the number of parts the wavefront has to multiply by.
 template <int NS>
 __device__ __forceinline__ int bf16_kernel_column(const float *__restrict__ qw, int K, int N, int col, int kq, u32x4_t (&wp)[3][NS]) {
+    // through a descriptor: entries outside the matrix read as zero and no load sits inside a branch, so all of them
+    // are in flight together
+    const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(qw, (int64_t)K * N * 4);
     float wv[NS][8];
 #pragma unroll
     for (int st = 0; st < NS; ++st)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int k = 16 * st + 8 * kq + e;
-            wv[st][e] = (k < K && col < N) ? qw[(int64_t)k * N + col] : 0.f;
+            wv[st][e] = buf_ld1(rs_w, (k < K && col < N) ? (uint32_t)(k * N + col) * 4u : BUF_OOB);
         }
     uint32_t wnz1 = 0u, wnz2 = 0u;
 #pragma unroll
@@ -643,14 +646,28 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rh = wave & 1, cb = wave >> 1;
     const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
-    for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;  // columns >= K stay zero
-    if (tid < 3) need[tid] = 0u;
+    // The first tile is asked for before anything else: the kernel matrix, the fractional bits and the LDS clearing below
+    // then run under its latency (a launch of few tiles per workgroup is mostly these start-up round trips).
+    FastMap mp, mo;
+    mp.init(K);
+    f32x4_t raw[FAST_NJ];
+    uint32_t xoff[FAST_NJ];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) xoff[j] = mp.on[j] ? (uint32_t)(mp.row[j] * K + mp.col[j]) * 4u : BUF_OOB;
+    auto load_tile = [&](int64_t t) {
+        const int64_t r0 = t * FAST_BM, left = rows - r0;
+        const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K, (left < FAST_BM ? left : FAST_BM) * K * 4);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) raw[j] = buf_ld4(rs, xoff[j]);
+    };
+    int64_t tile = blockIdx.x;
+    if (tile < n_tiles) load_tile(tile);
     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
     u32x4_t wp[3][NS];
     const int PW = bf16_kernel_column<NS>(qw, K, N, bcol, kq, wp);  // parts of the kernel this wavefront multiplies by
     const float bias = (qb && bcol < N) ? qb[bcol] : 0.f;
-    FastMap mp, mo;
-    mp.init(K);
+    for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;  // columns >= K stay zero
+    if (tid < 3) need[tid] = 0u;
     const bool vec_out = (N & 3) == 0 && ((uintptr_t)y & 15u) == 0;
     mo.init(vec_out ? N : 4);
     // fractional bits of the staged elements, four to a register (unpacked per tile: sixteen values and their negations
@@ -682,18 +699,6 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
             for (int e = 0; e < 4; ++e) oamx[jj][e] = 0;
         }
     }
-    f32x4_t raw[FAST_NJ];
-    uint32_t xoff[FAST_NJ];
-#pragma unroll
-    for (int j = 0; j < FAST_NJ; ++j) xoff[j] = mp.on[j] ? (uint32_t)(mp.row[j] * K + mp.col[j]) * 4u : BUF_OOB;
-    auto load_tile = [&](int64_t t) {
-        const int64_t r0 = t * FAST_BM, left = rows - r0;
-        const __amdgpu_buffer_rsrc_t rs = buf_rsrc(x + r0 * K, (left < FAST_BM ? left : FAST_BM) * K * 4);
-#pragma unroll
-        for (int j = 0; j < FAST_NJ; ++j) raw[j] = buf_ld4(rs, xoff[j]);
-    };
-    int64_t tile = blockIdx.x;
-    if (tile < n_tiles) load_tile(tile);
     __syncthreads();
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     int buf = 0, slot = 0;
@@ -991,36 +996,14 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     float *my_dw = part + (int64_t)blockIdx.x * M;
     float *my_db = my_dw + (int64_t)K * N;
     float *my_df = my_db + N;
-    {
-        // all 16 kernel-matrix loads of a thread in flight (one per loop trip would cost a memory latency each)
-        const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(qw, (int64_t)K * N * 4);
-        float wv[16];
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
-            wv[u] = buf_ld1(rs_w, (kk < K && nn < N) ? (uint32_t)(kk * N + nn) * 4u : BUF_OOB);
-        }
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
-            ws[kk][nn] = wv[u];
-            xs[kk][nn] = 0.f, dzs[kk][nn] = 0.f;
-        }
-    }
     FastMap mx, mz;
     // !ZVEC - N not a multiple of 4, or unaligned gradient rows: the gradient tile is staged in groups of four columns
     // of the width rounded up, each element with a load of its own (columns past N read as zero)
     mx.init(K), mz.init((N + 3) & ~3);
     // fractional bits of the staged elements, four to a register (unpacked per tile: sixteen values and their negations
-    // would otherwise each hold a register for the whole launch)
+    // would otherwise each hold a register for the whole launch); loaded in the start-up block below
     int fip[FAST_NJ];
     float gf[FAST_NJ][4];
-    {
-        int fi[FAST_NJ][4], tix[FAST_NJ];
-        fast_frac_bits<QUANT>(f_in, P, K, mx, m.round_params, fi, tix);
-#pragma unroll
-        for (int j = 0; j < FAST_NJ; ++j) fip[j] = pack_i8x4(fi[j]);
-    }
 #pragma unroll
     for (int j = 0; j < FAST_NJ; ++j)
 #pragma unroll
@@ -1072,7 +1055,29 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         }
     };
     const float inv_rows = 1.0f / (float)rows;
+    // Start-up: the first tile is asked for first, then the kernel matrix and the fractional bits - one round trip for the
+    // three of them instead of three in a row (a launch of one or two tiles per workgroup is mostly start-up).
     if (tile < n_tiles) load_tile(tile);
+    {
+        // all 16 kernel-matrix loads of a thread in flight (one per loop trip would cost a memory latency each)
+        const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(qw, (int64_t)K * N * 4);
+        float wv[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
+            wv[u] = buf_ld1(rs_w, (kk < K && nn < N) ? (uint32_t)(kk * N + nn) * 4u : BUF_OOB);
+        }
+        int fi[FAST_NJ][4], tix[FAST_NJ];
+        fast_frac_bits<QUANT>(f_in, P, K, mx, m.round_params, fi, tix);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) fip[j] = pack_i8x4(fi[j]);
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
+            ws[kk][nn] = wv[u];
+            xs[kk][nn] = 0.f, dzs[kk][nn] = 0.f;
+        }
+    }
     __syncthreads();
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing loaded before the loop is waited for inside it
     for (; tile < n_tiles; tile += gridDim.x) {
