@@ -600,6 +600,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
     // arithmetic; a convolution sum has no such contract, and unfused it costs two vector instructions per term)
 #pragma clang fp contract(fast)
     constexpr int KC = KH * KW * C, PH = SC_TH + KH - 1, PW = SC_TW + KW - 1;
+    constexpr int XWS = PW + KW - 1;  // pixels between the rows of the input patch in LDS (at least PW + px: tap offsets are immediates)
     extern __shared__ float lds[];  // kernel [KC * F] | dz patch [PH * PW][F + 1] (reused for the final sum) | input patch
     const int FS = F + 1, XH = PH + g.py, XW = PW + g.px;
     float *zp = lds + ((KC * F + 3) & ~3), *xp = zp + max(PH * PW * FS, SC_TH * (KC + 1) * 32);
@@ -761,7 +762,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
             for (int e = tid; e < XH * XW * C; e += 256) {
                 const int r = (int)d_xw.div((uint32_t)e), q = e - r * XW * C, iy = iy0 - g.py + r, ix = ix0 - g.px + q / C;
                 const bool ok = (unsigned)iy < (unsigned)g.H && (unsigned)ix < (unsigned)g.W;
-                xp[e] = buf_ld1(rs_x, ok ? (uint32_t)(((b * g.H + iy) * g.W + ix) * C + q % C) * 4u : BUF_OOB);
+                xp[r * XWS * C + q] = buf_ld1(rs_x, ok ? (uint32_t)(((b * g.H + iy) * g.W + ix) * C + q % C) * 4u : BUF_OOB);
             }
         }
         __syncthreads();
@@ -807,7 +808,30 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                 for (int c = 0; c < C; ++c) dx[o + c] = acc[c];
             }
         }
-        if (part) {
+        if (part && dyp) {
+            // Behind the pooling at most ONE pixel of a 2 x 2 window has a gradient per filter: a lane walks the windows its
+            // tile owns (a row slot takes every eighth), finds that pixel from the window's four dz values, and multiplies
+            // the one input window under it - a quarter of the multiply-adds of the walk over pixels below.  (Whole windows
+            // only have gradient, and the tiles' ownership boundaries fall on window boundaries: kh - 1 and kw - 1 are even.)
+            const int pc_lo = ix0 == 0 ? max(0, -ox0) : KW - 1, pc_hi = min(PW, g.OW - ox0);
+            const int wr_lo = iy0 == 0 ? max(0, -oy0 / 2) : (KH - 1) / 2, wr_hi = min(PH / 2, (g.OH - oy0 + 1) >> 1);
+            const int wc_lo = pc_lo >> 1, ncol = min(PW / 2, (pc_hi + 1) >> 1) - wc_lo, n_w = (wr_hi - wr_lo) * ncol;
+            if (ncol > 0 && wr_hi > wr_lo) {
+                const FastDiv d_nc((uint32_t)ncol);
+                for (int wi = slot; wi < n_w; wi += SC_TH) {
+                    const int r = (int)d_nc.div((uint32_t)wi), wr = wr_lo + r, wc = wc_lo + (wi - r * ncol);
+                    const float *zq = zp + (2 * wr * PW + 2 * wc) * FS + f;
+                    const float z0 = f_on ? zq[0] : 0.f, z1 = f_on ? zq[FS] : 0.f, z2 = f_on ? zq[PW * FS] : 0.f,
+                                z3 = f_on ? zq[(PW + 1) * FS] : 0.f;
+                    const float z = (z0 + z1) + (z2 + z3);  // one of them at most is not zero
+                    const int dyb = (z2 != 0.f || z3 != 0.f) ? 1 : 0, dxb = (z1 != 0.f || z3 != 0.f) ? 1 : 0;
+                    bacc += z;
+                    const float *xq = xp + ((2 * wr + dyb - (KH - 1) + g.py) * XWS + (2 * wc + dxb - (KW - 1) + g.px)) * C;
+#pragma unroll
+                    for (int t = 0; t < KC; ++t) wacc[t] += xq[((t / (KW * C)) * XWS + (t / C) % KW) * C + t % C] * z;
+                }
+            }
+        } else if (part) {
             for (int pr = slot; pr < PH; pr += SC_TH) {
                 const int oy = oy0 + pr;
                 if ((unsigned)oy >= (unsigned)g.OH || !(pr >= KH - 1 || iy0 == 0)) continue;
@@ -815,12 +839,12 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
                 // input pixel of tap (ky, kx): patch-relative (pr + ky - (KH - 1) + py, pc + kx - (KW - 1) + px).  The KH x KW
                 // window of a pixel shares all but one column with its left neighbour's: it lives in registers and takes KH * C
                 // new entries per pixel (LDS broadcasts) instead of KC
-                const float *xq = xp + ((pr - (KH - 1) + g.py) * XW + (pc_lo - (KW - 1) + g.px)) * C;
+                const float *xq = xp + ((pr - (KH - 1) + g.py) * XWS + (pc_lo - (KW - 1) + g.px)) * C;
                 float xw[KH][KW * C];
 #pragma unroll
                 for (int ky = 0; ky < KH; ++ky)
 #pragma unroll
-                    for (int j = 0; j < (KW - 1) * C; ++j) xw[ky][j + C] = xq[ky * XW * C + j];
+                    for (int j = 0; j < (KW - 1) * C; ++j) xw[ky][j + C] = xq[ky * XWS * C + j];
                 for (int pc = pc_lo; pc < pc_hi; ++pc, xq += C) {
                     const float z = f_on ? zp[(pr * PW + pc) * FS + f] : 0.f;
                     bacc += z;
@@ -829,7 +853,7 @@ __global__ __launch_bounds__(256) void bwd_smallc_kernel(const float *__restrict
 #pragma unroll
                         for (int j = 0; j < (KW - 1) * C; ++j) xw[ky][j] = xw[ky][j + C];
 #pragma unroll
-                        for (int c = 0; c < C; ++c) xw[ky][(KW - 1) * C + c] = xq[(ky * XW + KW - 1) * C + c];
+                        for (int c = 0; c < C; ++c) xw[ky][(KW - 1) * C + c] = xq[(ky * XWS + KW - 1) * C + c];
                     }
 #pragma unroll
                     for (int t = 0; t < KC; ++t) wacc[t] += xw[t / (KW * C)][t % (KW * C)] * z;
@@ -1419,7 +1443,7 @@ static size_t bwd_smallc_lds(const hgq_conv_geom &g, int F) {
     const size_t KC = (size_t)g.kh * g.kw * g.C, PH = SC_TH + g.kh - 1, PW = SC_TW + g.kw - 1;
     size_t zp = PH * PW * (F + 1), red = SC_TH * (KC + 1) * 32;
     if (red > zp) zp = red;
-    return (((KC * F + 3) & ~(size_t)3) + zp + (PH + g.py) * (PW + g.px) * g.C) * sizeof(float);
+    return (((KC * F + 3) & ~(size_t)3) + zp + (PH + g.py) * (PW + g.kw - 1) * g.C) * sizeof(float);  // (input patch rows PW + kw - 1 pixels apart)
 }
 static bool bwd_smallc_ok(const hgq_conv_geom &g, int F) {
     return smallc_shape(g, F) && g.sy == 1 && g.sx == 1 && g.dly == 1 && g.dlx == 1 && g.py < g.kh && g.px < g.kw &&

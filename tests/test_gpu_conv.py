@@ -338,8 +338,14 @@ def test_convolution_backward_from_the_pooled_gradient(dev, shape):
         dyp = torch.randn(yp.shape, generator=torch.Generator().manual_seed(5)).to(dev)
         yp.backward(dyp)
         got.append((yp.detach(), xs.grad, ws.grad, bs.grad if bias else None))
+    # pooled output and data gradient bit for bit; the kernel / bias gradient walks the pooling windows instead of the pixels
+    # (the same non-zero terms in another order): equal to 1e-5 of the largest entry
     for name, a, f in zip(('pooled output', 'dx', 'dw', 'db'), got[0], got[1]):
-        if a is not None:
+        if a is None:
+            continue
+        if name in ('dw', 'db'):
+            assert float((a - f).abs().max()) <= 1e-5 * float(a.abs().max()) + 1e-30, f'{name}: {float((a - f).abs().max())}'
+        else:
             assert torch.equal(a, f), f'{name}: {float((a - f).abs().max())}'
     # the entry points that keep the unpooled output (the node above saves a byte per window and filter instead) give the same bits
     xs, ws = x.to(dev), w.to(dev)
@@ -380,8 +386,9 @@ def test_unsupported_shapes_of_the_pooled_backward_are_refused(dev):
 
 
 def test_sequential_takes_the_pooling_into_the_convolution(dev):
-    """A QConv2D followed by MaxPooling2D((2, 2)) inside a Sequential runs as one node; outputs, losses and every gradient
-    equal those of the layers called one by one."""
+    """A QConv2D followed by MaxPooling2D((2, 2)) inside a Sequential runs as one node; outputs and losses equal those of the
+    layers called one by one bit for bit, gradients to 1e-5 of the tensor's largest entry (the node's kernel / bias gradient
+    adds the same terms window by window instead of pixel by pixel)."""
     import copy
 
     from hgq2_amd import host, ops
@@ -407,7 +414,7 @@ def test_sequential_takes_the_pooling_into_the_convolution(dev):
     ops.sparse_ce(out_b, labels).backward()
     for (name, pa), (_, pb) in zip(model.named_parameters(), twin.named_parameters()):
         if pa.grad is not None or pb.grad is not None:
-            assert torch.equal(pa.grad, pb.grad), name
+            assert float((pa.grad - pb.grad).abs().max()) <= 1e-5 * float(pb.grad.abs().max()) + 1e-30, name
 
 
 @pytest.mark.parametrize('rows,K,N,relu,bias', [(1024, 3872, 10, False, True), (7, 1500, 16, True, True), (33, 1024, 1, False, False),
