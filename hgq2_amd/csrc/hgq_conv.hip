@@ -1304,6 +1304,47 @@ __device__ __forceinline__ void ce_put(const hgq_bits_desc &d, uint32_t j, bool 
     }
 }
 
+// The bit-widths of n cells of one operand into LDS, a byte per cell (bits 0-6 the width, bit 7 "open": the straight-through
+// gradient is not closed).  Eight cells of a thread per trip, every load of the trip issued before the first value is used:
+// one workgroup sweeping an operand a load at a time pays a memory latency per cell and thread.
+__device__ __forceinline__ void ce_stage_bits(const hgq_bits_desc &d, int n, unsigned char *dst, int *bad) {
+    const bool has_i = !d.kbi, has_k = d.add_mode != 0;
+    for (int e0 = 0; e0 < n; e0 += 8 * 1024) {
+        float iv[8], fv[8];
+        unsigned char kv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int e = e0 + u * 1024 + (int)threadIdx.x, j = e < n ? e : 0;
+            fv[u] = d.fb[j];
+            iv[u] = has_i ? d.i[j] : 0.f;
+            kv[u] = has_k ? d.k[j] : (unsigned char)0;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int e = e0 + u * 1024 + (int)threadIdx.x;
+            float b;
+            bool open = true;
+            if (d.kbi) {
+                b = rintf(fv[u]);
+            } else {
+                const float sum = __fadd_rn(rintf(iv[u]), rintf(fv[u]));
+                open = sum > 0.f;
+                b = open ? sum : 0.f;
+            }
+            if (d.add_mode == 1) b = __fadd_rn(b, (float)kv[u]);
+            else if (d.add_mode == 2) b = __fadd_rn(b, (float)kv[u] * (b > 0.f ? 1.f : 0.f));
+            if (e < n) {
+                if (!(b >= 0.f && b <= 127.f)) *bad = 1;  // a width a byte cannot hold (a negative `_b`): the sweeps read the variables instead
+                dst[e] = (unsigned char)((int)fminf(fmaxf(b, 0.f), 127.f) | (open ? 0x80 : 0));
+            }
+        }
+    }
+}
+
+// STAGED: both operands' bit-widths are formed once into dynamic LDS (H W C + kh kw C F bytes) and every later sweep reads
+// them there; otherwise (operands too large for that, or a width outside 0 .. 127) every sweep forms them from the variables
+// in memory.
+template <bool STAGED>
 __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, hgq_bits_desc dker, hgq_bits_desc dbias, int has_bias,
                                                             hgq_conv_geom g, int F, float conv_scale, float bias_size, float factor,
                                                             const float *beta, uint32_t *ebops_u32, float *loss_term) {
@@ -1311,7 +1352,27 @@ __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, h
     __shared__ int Ws[CE_MAX];
     __shared__ float red[1024];
     __shared__ unsigned char vy[CE_MAXV], vx[CE_MAXV];
+    extern __shared__ unsigned char ce_dyn[];
     const int t = threadIdx.x, taps = g.kh * g.kw, TC = taps * g.C, WC = g.W * g.C;
+    unsigned char *bi = ce_dyn, *bk = ce_dyn + ((g.H * WC + 15) & ~15);
+    __shared__ int ce_bad;
+    bool use_staged = false;
+    auto bits_of = [&](const hgq_bits_desc &d, const unsigned char *staged, uint32_t j, bool &open) -> float {
+        if (STAGED && use_staged) {
+            const unsigned char v = staged[j];
+            open = (v & 0x80) != 0;
+            return (float)(v & 0x7f);
+        }
+        return ce_bits(d, j, open);
+    };
+    if (STAGED) {
+        if (t == 0) ce_bad = 0;
+        __syncthreads();
+        ce_stage_bits(din, g.H * WC, bi, &ce_bad);
+        ce_stage_bits(dker, TC * F, bk, &ce_bad);
+        __syncthreads();
+        use_staged = ce_bad == 0;
+    }
     const FastDiv by_wc((uint32_t)WC), by_f((uint32_t)F), by_c((uint32_t)g.C), by_kw((uint32_t)g.kw);
     for (int e = t; e < TC; e += 1024) Ws[e] = 0;
     for (int e = t; e < g.H * g.kh; e += 1024) {
@@ -1328,7 +1389,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, h
         for (int oy = 0; oy < g.OH; ++oy) {
             const int iy = oy * g.sy - g.py + ky * g.dly;
             bool open;
-            if ((unsigned)iy < (unsigned)g.H) r += ce_bits(din, (uint32_t)(iy * WC + xc), open);
+            if ((unsigned)iy < (unsigned)g.H) r += bits_of(din, bi, (uint32_t)(iy * WC + xc), open);
         }
         R[e] = r;
     }
@@ -1336,7 +1397,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, h
     const int n_w = TC * F;
     for (int e = t; e < n_w; e += 1024) {
         bool open;
-        atomicAdd(&Ws[by_f.div((uint32_t)e)], (int)ce_bits(dker, (uint32_t)e, open));
+        atomicAdd(&Ws[by_f.div((uint32_t)e)], (int)bits_of(dker, bk, (uint32_t)e, open));
     }
     for (int e = t; e < TC; e += 1024) {
         const int tap = (int)by_c.div((uint32_t)e), c = e - tap * g.C, ky = (int)by_kw.div((uint32_t)tap), kx = tap - ky * g.kw;
@@ -1382,7 +1443,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, h
     }
     for (int e = t; e < n_w; e += 1024) {
         bool open;  // a KIF kernel quantizer's width relu(i + f) is flat where i + f <= 0
-        (void)ce_bits(dker, (uint32_t)e, open);
+        (void)bits_of(dker, bk, (uint32_t)e, open);
         ce_put(dker, (uint32_t)e, open, S[by_f.div((uint32_t)e)] * conv_scale * gs);
     }
     for (int e = t; e < g.H * WC; e += 1024) {
@@ -1394,7 +1455,7 @@ __global__ __launch_bounds__(1024) void conv_ebops_q_kernel(hgq_bits_desc din, h
                 if (vx[x * g.kw + kx]) a += (float)Ws[(ky * g.kw + kx) * g.C + c];
         }
         bool open;
-        (void)ce_bits(din, (uint32_t)e, open);
+        (void)bits_of(din, bi, (uint32_t)e, open);
         ce_put(din, (uint32_t)e, open, a * conv_scale * gs);
     }
     if (has_bias)
@@ -1859,7 +1920,19 @@ extern "C" int hgq_conv2d_ebops_q(const hgq_bits_desc *bits_in, const hgq_bits_d
             return fail(HGQ_ERR_ARG, "hgq_conv2d_ebops_q: null pointer in operand %d", t);
     }
     hgq_bits_desc none = *bits_ker;
-    hipLaunchKernelGGL(conv_ebops_q_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, *bits_in, *bits_ker, bits_bias ? *bits_bias : none,
-                       bits_bias ? 1 : 0, *g, F, conv_scale, bias_size, ebops_factor, beta, ebops_u32, loss_term);
+    const size_t staged_bytes = (size_t)((n_in + 15) & ~(int64_t)15) + (size_t)n_w;
+    if (staged_bytes <= 60 * 1024) {
+        static bool allowed = false;  // (static + dynamic LDS of this kernel pass 64 KiB)
+        if (!allowed) {
+            if (hipFuncSetAttribute((const void *)conv_ebops_q_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 60 * 1024) != hipSuccess)
+                return fail(HGQ_ERR_LAUNCH, "hgq_conv2d_ebops_q: cannot raise the dynamic LDS limit");
+            allowed = true;
+        }
+        hipLaunchKernelGGL(conv_ebops_q_kernel<true>, dim3(1), dim3(1024), staged_bytes, (hipStream_t)stream, *bits_in, *bits_ker,
+                           bits_bias ? *bits_bias : none, bits_bias ? 1 : 0, *g, F, conv_scale, bias_size, ebops_factor, beta, ebops_u32, loss_term);
+    } else {
+        hipLaunchKernelGGL(conv_ebops_q_kernel<false>, dim3(1), dim3(1024), 0, (hipStream_t)stream, *bits_in, *bits_ker,
+                           bits_bias ? *bits_bias : none, bits_bias ? 1 : 0, *g, F, conv_scale, bias_size, ebops_factor, beta, ebops_u32, loss_term);
+    }
     return check_launch("hgq_conv2d_ebops_q");
 }
