@@ -42,6 +42,10 @@ SIGNATURES = {
     'hgq_quantize_bwd': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_fwd_stochastic': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int, ctypes.c_uint64, ctypes.c_uint64, c_void_p]),
     'hgq_quantize_bwd_stochastic': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, ctypes.c_uint64, ctypes.c_uint64, c_void_p]),
+    'hgq_quantize_fwd_stochastic_at': (c_int, [c_void_p] * 7 + [c_int64, c_int64, c_int64, c_int, ctypes.c_uint64, ctypes.c_uint64, c_void_p, c_void_p,
+                                               c_void_p]),
+    'hgq_quantize_bwd_stochastic_at': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, ctypes.c_uint64, c_void_p, c_void_p]),
+    'hgq_counters_advance': (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     'hgq_wrap_track_i': (c_int, [c_void_p] * 2 + [c_int] + [c_void_p] * 3 + [c_int64, c_float, c_float, c_float, c_int, c_void_p]),
     'hgq_qdense_fwd_parts': (c_int, [c_int64]),
     'hgq_qdense_bwd_workspace': (c_int64, [c_int64, c_int, c_int, c_int64]),

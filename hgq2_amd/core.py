@@ -314,6 +314,7 @@ class Layer(nn.Module):
             from . import ops
 
             ops.begin_deferred()  # single-workgroup launches that nothing in the forward waits for go out together at the end
+            ops.advance_seed_generators()  # draw counters of stochastic rounding: the previous step's draws are behind them now
         ok = False
         try:
             if top and args and isinstance(args[0], torch.Tensor):

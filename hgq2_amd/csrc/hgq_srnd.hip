@@ -38,8 +38,13 @@ __device__ __forceinline__ float srnd_round(float x, float f, float u) {
 template <int OM>
 __global__ __launch_bounds__(256) void srnd_fwd_kernel(const float *__restrict__ x, const void *k, const float *i, const float *fb,
                                                        float *__restrict__ y, uint32_t *amax, uint32_t *anyneg, int64_t n, int64_t bw_size,
-                                                       int64_t bw_inner, int mode, uint64_t seed, uint64_t offset) {
+                                                       int64_t bw_inner, int mode, uint64_t seed, uint64_t offset, const uint64_t *__restrict__ offset_base,
+                                                       uint64_t *__restrict__ used_offset) {
     const Mode m(mode);
+    // the draw is (seed, offset + *offset_base): a base in device memory lets a recorded launch draw anew on every replay
+    // (the caller advances it between steps); the sum is left for the backward pass, which must repeat this draw
+    if (offset_base) offset += offset_base[0];
+    if (used_offset && blockIdx.x == 0 && threadIdx.x == 0) used_offset[0] = offset;
     for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
         const int64_t b = (e / bw_inner) % bw_size;
         const KIF p = resolve_kif(load_k(k, b, m.k_u8), i[b], fb[b], m.kbi, m.round_params);
@@ -56,8 +61,10 @@ __global__ __launch_bounds__(256) void srnd_fwd_kernel(const float *__restrict__
 template <int OM>
 __global__ __launch_bounds__(256) void srnd_bwd_kernel(const float *__restrict__ dy, const float *__restrict__ x, const void *k, const float *i,
                                                        const float *fb, float *__restrict__ dx, float *di, float *dfb, int64_t n,
-                                                       int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset) {
+                                                       int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset,
+                                                       const uint64_t *__restrict__ offset_base) {
     const Mode m(mode);
+    if (offset_base) offset += offset_base[0];
     for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) {
         const int64_t b = (e / bw_inner) % bw_size;
         const KIF p = resolve_kif(load_k(k, b, m.k_u8), i[b], fb[b], m.kbi, m.round_params);
@@ -111,29 +118,44 @@ using namespace hgq;
         else CALL(HGQ_SAT_SYM);                  \
     } while (0)
 
-extern "C" int hgq_quantize_fwd_stochastic(const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax,
-                                           uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed,
-                                           uint64_t offset, void *stream) {
-    int rc = srnd_check("hgq_quantize_fwd_stochastic", x, k, i, fb, n, bw_size, bw_inner, mode);
+static int srnd_fwd_impl(const char *who, const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax,
+                         uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset,
+                         const uint64_t *offset_base, uint64_t *used_offset, void *stream) {
+    int rc = srnd_check(who, x, k, i, fb, n, bw_size, bw_inner, mode);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
     if (amax && (rc = fill_f32((float *)amax, 0.0f, bw_size, s))) return rc;
     if (anyneg && (rc = fill_f32((float *)anyneg, 0.0f, bw_size, s))) return rc;
-    if (n == 0) return HGQ_OK;
-    if (!y) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_stochastic: null output");
-    const int grid = persistent_grid((n + 255) / 256, 8);
-#define CALL(OMV) hipLaunchKernelGGL((srnd_fwd_kernel<OMV>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n, bw_size, bw_inner, mode, seed, offset)
+    if (n == 0 && !used_offset) return HGQ_OK;
+    if (n > 0 && !y) return fail(HGQ_ERR_ARG, "%s: null output", who);
+    const int grid = persistent_grid((n + 255) / 256, 8);  // (n = 0 with used_offset: one workgroup that only leaves the offset)
+#define CALL(OMV) hipLaunchKernelGGL((srnd_fwd_kernel<OMV>), dim3(grid), dim3(256), 0, s, x, k, i, fb, y, amax, anyneg, n, bw_size, bw_inner, mode, seed, offset, offset_base, used_offset)
     HGQ_SRND_OM(Mode(mode).overflow_mode, CALL);
 #undef CALL
-    return check_launch("hgq_quantize_fwd_stochastic");
+    return check_launch(who);
 }
 
-extern "C" int hgq_quantize_bwd_stochastic(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
-                                           float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset,
-                                           void *stream) {
-    int rc = srnd_check("hgq_quantize_bwd_stochastic", x, k, i, fb, n, bw_size, bw_inner, mode);
+extern "C" int hgq_quantize_fwd_stochastic(const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax,
+                                           uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed,
+                                           uint64_t offset, void *stream) {
+    return srnd_fwd_impl("hgq_quantize_fwd_stochastic", x, k, i, fb, y, amax, anyneg, n, bw_size, bw_inner, mode, seed, offset, nullptr, nullptr,
+                         stream);
+}
+
+extern "C" int hgq_quantize_fwd_stochastic_at(const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax,
+                                              uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed,
+                                              uint64_t offset, const uint64_t *offset_base, uint64_t *used_offset, void *stream) {
+    if (!offset_base || !used_offset) return fail(HGQ_ERR_ARG, "hgq_quantize_fwd_stochastic_at: null pointer");
+    return srnd_fwd_impl("hgq_quantize_fwd_stochastic_at", x, k, i, fb, y, amax, anyneg, n, bw_size, bw_inner, mode, seed, offset, offset_base,
+                         used_offset, stream);
+}
+
+static int srnd_bwd_impl(const char *who, const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
+                         float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset,
+                         const uint64_t *offset_base, void *stream) {
+    int rc = srnd_check(who, x, k, i, fb, n, bw_size, bw_inner, mode);
     if (rc) return rc;
-    if (n > 0 && !dy) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_stochastic: null pointer");
+    if (n > 0 && !dy) return fail(HGQ_ERR_ARG, "%s: null pointer", who);
     hipStream_t s = (hipStream_t)stream;
     const bool per_element = bw_size == n && bw_inner == 1;
     if (!per_element || n == 0) {
@@ -142,8 +164,53 @@ extern "C" int hgq_quantize_bwd_stochastic(const float *dy, const float *x, cons
     }
     if (n == 0) return HGQ_OK;
     const int grid = persistent_grid((n + 255) / 256, 8);
-#define CALL(OMV) hipLaunchKernelGGL((srnd_bwd_kernel<OMV>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n, bw_size, bw_inner, mode, seed, offset)
+#define CALL(OMV) hipLaunchKernelGGL((srnd_bwd_kernel<OMV>), dim3(grid), dim3(256), 0, s, dy, x, k, i, fb, dx, di, dfb, n, bw_size, bw_inner, mode, seed, offset, offset_base)
     HGQ_SRND_OM(Mode(mode).overflow_mode, CALL);
 #undef CALL
-    return check_launch("hgq_quantize_bwd_stochastic");
+    return check_launch(who);
+}
+
+extern "C" int hgq_quantize_bwd_stochastic(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
+                                           float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset,
+                                           void *stream) {
+    return srnd_bwd_impl("hgq_quantize_bwd_stochastic", dy, x, k, i, fb, dx, di, dfb, n, bw_size, bw_inner, mode, seed, offset, nullptr, stream);
+}
+
+extern "C" int hgq_quantize_bwd_stochastic_at(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx,
+                                              float *di, float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed,
+                                              const uint64_t *used_offset, void *stream) {
+    if (!used_offset) return fail(HGQ_ERR_ARG, "hgq_quantize_bwd_stochastic_at: null pointer");
+    return srnd_bwd_impl("hgq_quantize_bwd_stochastic_at", dy, x, k, i, fb, dx, di, dfb, n, bw_size, bw_inner, mode, seed, 0, used_offset, stream);
+}
+
+// counters[j][0] += increments[j]: the draw counters of the seed generators a step used, advanced in one launch
+#define SRND_MAX_COUNTERS 32
+struct CounterBatch {
+    uint64_t *counter[SRND_MAX_COUNTERS];
+    uint64_t increment[SRND_MAX_COUNTERS];
+    int count;
+};
+namespace hgq {
+__global__ __launch_bounds__(64) void counters_advance_kernel(const CounterBatch b) {
+    const int j = threadIdx.x;
+    if (j < b.count) b.counter[j][0] += b.increment[j];
+}
+}  // namespace hgq
+
+extern "C" int hgq_counters_advance(uint64_t *const *counters, const uint64_t *increments, int count, void *stream) {
+    if (count < 0 || (count > 0 && (!counters || !increments))) return fail(HGQ_ERR_ARG, "hgq_counters_advance: bad arguments");
+    for (int j0 = 0; j0 < count; j0 += SRND_MAX_COUNTERS) {
+        CounterBatch b;
+        b.count = count - j0 < SRND_MAX_COUNTERS ? count - j0 : SRND_MAX_COUNTERS;
+        for (int j = 0; j < b.count; ++j) {
+            if (!counters[j0 + j]) return fail(HGQ_ERR_ARG, "hgq_counters_advance: null counter %d", j0 + j);
+            for (int u = 0; u < j; ++u)
+                if (b.counter[u] == counters[j0 + j]) return fail(HGQ_ERR_ARG, "hgq_counters_advance: counter %d is listed twice", j0 + j);
+            b.counter[j] = counters[j0 + j], b.increment[j] = increments[j0 + j];
+        }
+        hipLaunchKernelGGL(counters_advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, b);
+        const int rc = check_launch("hgq_counters_advance");
+        if (rc) return rc;
+    }
+    return HGQ_OK;
 }

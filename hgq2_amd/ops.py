@@ -1796,6 +1796,104 @@ def _(dy, x, k, i, fb, mode, bw_inner, seed, offset):
     return torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
 
 
+@torch.library.custom_op('hgq::quantize_fwd_stochastic_at', mutates_args=())
+def quantize_fwd_stochastic_at(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, track: bool, seed: int,
+                               offset: int, base: Tensor) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """``quantize_fwd_stochastic`` whose draw is ``(seed, offset + base[0])`` with ``base`` an int64 counter in device memory;
+    the fourth result holds the offset that was used (the backward pass repeats that draw)."""
+    _check_f32('x', x), _check_k('k', k), _check_f32('i', i), _check_f32('fb', fb)
+    bw = i.numel()
+    _need(k.numel() == bw and fb.numel() == bw and bw >= 1 and bw_inner >= 1, 'bit-width operands must have equal sizes')
+    _need(base.dtype == torch.int64 and base.numel() == 1 and base.device == x.device, 'base must be one int64 on the device of x')
+    y = torch.empty_like(x)
+    amax = torch.empty(bw if track else 0, dtype=torch.int32, device=x.device)
+    neg = torch.empty(bw if track else 0, dtype=torch.int32, device=x.device)
+    used = torch.empty(1, dtype=torch.int64, device=x.device)
+    m = (_kmode(mode, k) & ~0xf) | _lib.S_RND
+    rc = _lib.load().hgq_quantize_fwd_stochastic_at(_ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(y), _ptr(amax) if track else None,
+                                                    _ptr(neg) if track else None, x.numel(), bw, bw_inner, m, seed, offset, _ptr(base),
+                                                    _ptr(used), _stream())
+    _lib.check(rc, 'hgq_quantize_fwd_stochastic_at')
+    return y, amax, neg, used
+
+
+@quantize_fwd_stochastic_at.register_fake
+def _(x, k, i, fb, mode, bw_inner, track, seed, offset, base):
+    n = i.numel() if track else 0
+    return torch.empty_like(x), x.new_empty(n, dtype=torch.int32), x.new_empty(n, dtype=torch.int32), x.new_empty(1, dtype=torch.int64)
+
+
+@torch.library.custom_op('hgq::quantize_bwd_stochastic_at', mutates_args=())
+def quantize_bwd_stochastic_at(dy: Tensor, x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, bw_inner: int, seed: int,
+                               used: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+    _check_f32('dy', dy), _check_f32('x', x)
+    _need(dy.shape == x.shape, 'dy shape mismatch')
+    _need(used.dtype == torch.int64 and used.numel() == 1 and used.device == x.device, 'used must be one int64 on the device of x')
+    dx, di, dfb = torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+    m = (_kmode(mode, k) & ~0xf) | _lib.S_RND
+    rc = _lib.load().hgq_quantize_bwd_stochastic_at(_ptr(dy), _ptr(x), _ptr(k), _ptr(i), _ptr(fb), _ptr(dx), _ptr(di), _ptr(dfb), x.numel(),
+                                                    i.numel(), bw_inner, m, seed, _ptr(used), _stream())
+    _lib.check(rc, 'hgq_quantize_bwd_stochastic_at')
+    return dx, di, dfb
+
+
+@quantize_bwd_stochastic_at.register_fake
+def _(dy, x, k, i, fb, mode, bw_inner, seed, used):
+    return torch.empty_like(x), torch.empty_like(i), torch.empty_like(fb)
+
+
+@torch.library.custom_op('hgq::counters_advance', mutates_args=('counters',))
+def counters_advance(counters: Sequence[Tensor], increments: Sequence[int]) -> None:
+    """``counters[j] += increments[j]`` for one-element int64 device tensors, one launch."""
+    n = len(counters)
+    _need(len(increments) == n, 'one increment per counter')
+    if n == 0:
+        return
+    for c in counters:
+        _need(c.dtype == torch.int64 and c.numel() == 1 and c.is_cuda, 'counters are one-element int64 device tensors')
+    ptrs = (ctypes.c_void_p * n)(*[c.data_ptr() for c in counters])
+    incs = (ctypes.c_uint64 * n)(*[int(v) for v in increments])
+    _lib.check(_lib.load().hgq_counters_advance(ptrs, incs, n, _stream()), 'hgq_counters_advance')
+
+
+# seed generators that drew on the device since their counters were last advanced (hgq2_amd.quantizer.fixed_point_ops)
+_SEED_PENDING = []
+
+
+def advance_seed_generators():
+    """Advance the device-side draw counters of the seed generators used since the last call by the number of draws each
+    made (one launch).  The outermost layer call of a training step does this before it runs, so a step recorded into a
+    HIP graph - counters advanced, then draws at fixed offsets from them - draws anew on every replay."""
+    if not _SEED_PENDING:
+        return
+    gens = [g for g in _SEED_PENDING if g._drawn]
+    del _SEED_PENDING[:]
+    if gens:
+        counters_advance([g._base for g in gens], [g._drawn for g in gens])
+        for g in gens:
+            g._drawn = 0
+
+
+class _QuantizeStochasticAt(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, k, i, fb, mode, bw_inner, track, seed, offset, base):
+        y, amax, neg, used = quantize_fwd_stochastic_at(x, k, i, fb, mode, bw_inner, track, seed, offset, base)
+        ctx.save_for_backward(x, k, i, fb, used)
+        ctx.mode, ctx.bw_inner, ctx.seed = mode, bw_inner, seed
+        ctx.mark_non_differentiable(amax, neg)
+        ctx.set_materialize_grads(False)
+        return y, amax, neg
+
+    @staticmethod
+    def backward(ctx, gy, _ga, _gn):
+        if gy is None:
+            return (None,) * 10
+        x, k, i, fb, used = ctx.saved_tensors
+        dx, di, dfb = quantize_bwd_stochastic_at(gy.contiguous(), x, k, i, fb, ctx.mode, ctx.bw_inner, ctx.seed, used)
+        return (dx if ctx.needs_input_grad[0] else None, None, di if ctx.needs_input_grad[2] else None,
+                dfb if ctx.needs_input_grad[3] else None, None, None, None, None, None, None)
+
+
 class _QuantizeStochastic(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, k, i, fb, mode, bw_inner, track, seed, offset):
@@ -1817,9 +1915,13 @@ class _QuantizeStochastic(torch.autograd.Function):
 
 
 def quantize_stochastic(x: Tensor, k: Tensor, i: Tensor, fb: Tensor, mode: int, seed: int, offset: int, bw_inner: int = 1,
-                        track: bool = False):
-    """The training-mode quantizer of round modes S_RND / S_RND_CONV; ``(seed, offset)`` names the draw."""
+                        track: bool = False, base: Tensor | None = None):
+    """The training-mode quantizer of round modes S_RND / S_RND_CONV; ``(seed, offset)`` names the draw, or
+    ``(seed, offset + base[0])`` with a counter in device memory (what a seed generator hands over on the GPU)."""
     _need(bool(mode & _lib.MODE_TRAINING), 'stochastic rounding applies to the training-mode forward only')
+    if base is not None:
+        return _QuantizeStochasticAt.apply(x.contiguous(), k.contiguous(), i.contiguous(), fb.contiguous(), mode, bw_inner, track,
+                                           int(seed), int(offset), base)
     return _QuantizeStochastic.apply(x.contiguous(), k.contiguous(), i.contiguous(), fb.contiguous(), mode, bw_inner, track,
                                      int(seed), int(offset))
 

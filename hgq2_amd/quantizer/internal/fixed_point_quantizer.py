@@ -161,8 +161,9 @@ class FixedPointQuantizerBase(TrainableQuantizerBase):
         """``stochastic``: this call is one of those the reference hands ``seed_gen`` to with training on (:147,:279,:404)."""
         k, i, t, (_, inner) = self._operands(x)
         if stochastic and self.stochastic and (mode & _lib.MODE_TRAINING):
-            seed, offset = self._seed_gen.next()
-            return ops.quantize_stochastic(x, k, i, t, mode, seed, offset, bw_inner=inner, track=track)
+            draw = self._seed_gen.next(x.device)  # on a GPU the counter sits in device memory: a recorded step draws anew per replay
+            return ops.quantize_stochastic(x, k, i, t, mode, draw[0], draw[1], bw_inner=inner, track=track,
+                                           base=draw[2] if len(draw) > 2 else None)
         return ops.quantize(x, k, i, t, mode, bw_inner=inner, track=track)
 
     def _constraint_bounds(self):

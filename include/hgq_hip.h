@@ -138,6 +138,21 @@ int hgq_quantize_fwd_stochastic(const float *x, const void *k, const float *i, c
 int hgq_quantize_bwd_stochastic(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
                                 float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed, uint64_t offset,
                                 void *stream);
+/*
+ * The same pair with the draw's offset partly in device memory, so that a launch recorded into a HIP graph draws anew on
+ * every replay: the forward uses offset + offset_base[0] and leaves that sum in used_offset[0]; the backward repeats the draw
+ * named by used_offset[0].  hgq_counters_advance adds increments[j] to counters[j][0] (any number, 32 per launch; a counter
+ * may be listed once): a trainer calls it once per step with the number of draws each seed generator made, which is the
+ * advance keras.random.SeedGenerator makes on the host (reference src/hgq/quantizer/internal/fixed_point_quantizer.py:56-57,
+ * :142-150).  Same shapes, modes and errors as the pair above.
+ */
+int hgq_quantize_fwd_stochastic_at(const float *x, const void *k, const float *i, const float *fb, float *y, uint32_t *amax,
+                                   uint32_t *anyneg, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed,
+                                   uint64_t offset, const uint64_t *offset_base, uint64_t *used_offset, void *stream);
+int hgq_quantize_bwd_stochastic_at(const float *dy, const float *x, const void *k, const float *i, const float *fb, float *dx, float *di,
+                                   float *dfb, int64_t n, int64_t bw_size, int64_t bw_inner, int mode, uint64_t seed,
+                                   const uint64_t *used_offset, void *stream);
+int hgq_counters_advance(uint64_t *const *counters, const uint64_t *increments, int count, void *stream);
 
 /*
  * Measurement aid (no counterpart in the reference): o_j[e] = (j + 1) * (a[e] (+ b[e]) (+ c[e])) for the first n_write

@@ -549,17 +549,99 @@ def test_scaler_division_is_correctly_rounded(dev):
         assert torch.equal(yp.cpu(), yr), f'step {step}: {int((yp.cpu() != yr).sum())} values differ'
 
 
-def test_stochastic_rounding_refuses_graph_capture(dev):
+def test_host_side_draws_refuse_graph_capture(dev):
+    """A draw whose offset travels as a launch argument would repeat on every replay: `next()` without a device refuses a
+    capturing stream, and so does the first device draw of a generator (its counter would be created by a recorded launch)."""
     from hgq2_amd.quantizer.fixed_point_ops import SeedGenerator
 
-    gen = SeedGenerator(1)
-    graph = torch.cuda.CUDAGraph()
-    x = torch.zeros(8, device=dev)
-    s = torch.cuda.Stream()
-    s.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(s):
-        with pytest.raises(RuntimeError, match='HIP graph'):
-            with torch.cuda.graph(graph, stream=s):
-                x.add_(1.0)
-                gen.next()
-    torch.cuda.current_stream().wait_stream(s)
+    for args in ((), (dev,)):
+        gen = SeedGenerator(1)
+        graph = torch.cuda.CUDAGraph()
+        x = torch.zeros(8, device=dev)
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            with pytest.raises(RuntimeError, match='capture'):
+                with torch.cuda.graph(graph, stream=s):
+                    x.add_(1.0)
+                    gen.next(*args)
+        torch.cuda.current_stream().wait_stream(s)
+
+
+def test_device_side_draw_counter_gives_the_host_counters_offsets(dev):
+    """The draws of a seed generator on the GPU - offset = device counter + draws since it was advanced - are those of the
+    host counter 1, 2, 3, ...: values equal the kernel called with the explicit pair, before and after advances."""
+    from hgq2_amd import _lib, ops
+    from hgq2_amd.quantizer.fixed_point_ops import SeedGenerator
+
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(4096, generator=g) * 3).to(dev)
+    k, i, f = torch.ones(1, device=dev), torch.full((1,), 3.0, device=dev), torch.full((1,), 2.0, device=dev)
+    mode = _lib.mode_bits('RND', 'SAT', training=True)
+    gen = SeedGenerator(77)
+    for step in range(1, 7):
+        if step in (3, 4, 6):
+            ops.advance_seed_generators()
+        seed, n, base = gen.next(dev)
+        got, _, _ = ops.quantize_stochastic(x, k, i, f, mode, seed, n, bw_inner=x.numel(), base=base)
+        want, _, _ = ops.quantize_stochastic(x, k, i, f, mode, 77, step, bw_inner=x.numel())
+        assert torch.equal(got, want), step
+        assert gen.offset == step and int(base) + gen._drawn == step
+    # the backward pass repeats the draw the forward pass made, also when the counter has moved on in between
+    xr = x.clone().requires_grad_(True)
+    seed, n, base = gen.next(dev)
+    y, _, _ = ops.quantize_stochastic(xr, k, i, f, mode, seed, n, bw_inner=x.numel(), base=base)
+    ops.advance_seed_generators()
+    gen.next(dev)
+    y.sum().backward()
+    xe = x.clone().requires_grad_(True)
+    ye, _, _ = ops.quantize_stochastic(xe, k, i, f, mode, 77, 7, bw_inner=x.numel())
+    ye.sum().backward()
+    assert torch.equal(y, ye) and torch.equal(xr.grad, xe.grad)
+
+
+def test_stochastic_rounding_in_a_replayed_graph_draws_anew(dev):
+    """A training step with S_RND data quantizers recorded into a HIP graph: every replay draws as the same step run
+    eagerly would - variables after N replays equal those of N eager steps of a twin model, bit for bit - and two
+    replays on the same batch do not repeat each other's draw."""
+    import numpy as np
+
+    from hgq2_amd import ops
+    from hgq2_amd.core import Sequential, set_default_device
+    from hgq2_amd.layers import QDense
+    from hgq2_amd.quantizer.config import QuantizerConfigScope
+    from hgq2_amd.train import SGD, GraphedTrainStep, model_loss
+
+    set_default_device(dev)
+
+    def build():
+        np.random.seed(31)  # the quantizers take their seeds from numpy's generator (reference: internal/base.py seed default)
+        torch.manual_seed(2)
+        with QuantizerConfigScope(place='datalane', round_mode='S_RND'):
+            model = Sequential([QDense(24, activation='relu'), QDense(6)])
+        model(x, training=False)
+        return model
+
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(256, 12, generator=g).to(dev)
+    y = torch.randint(0, 6, (256,), generator=g).to(dev)
+    a, b = build(), build()
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        assert torch.equal(pa, pb)
+    gens = [m.seed_gen for m in a.modules() if getattr(m, 'seed_gen', None) is not None]
+    assert gens, 'no stochastic quantizer in the model'
+    opt_a, opt_b = SGD(a.parameters(), lr=0.05), SGD(b.parameters(), lr=0.05)
+    warmup, replays = 2, 4
+    step_a = GraphedTrainStep(a, ops.sparse_ce, opt_a, x, y, warmup=warmup)
+    losses = [step_a().item() for _ in range(replays)]
+    want = []
+    for _ in range(warmup + replays):  # the recording itself runs nothing
+        opt_b.zero_grad()
+        with ops.overlap_ebops():
+            loss = model_loss(b, ops.sparse_ce(b(x, training=True), y))
+            opt_b.backward(loss)
+            opt_b.step()
+        want.append(loss.item())
+    torch.cuda.synchronize()
+    assert losses == want[warmup:], (losses, want)
+    assert len(set(losses)) > 1
