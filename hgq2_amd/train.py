@@ -144,17 +144,30 @@ class GraphedTrainStep:
     static buffers before each replay.  ``loss_fn(outputs, labels)`` must be built from capturable
     operations (``hgq2_amd.ops.sparse_ce`` is)."""
 
-    def __init__(self, model, loss_fn, optimizer: SGD, example_x, example_y, warmup: int = 3, overlap: bool = True):
+    def __init__(self, model, loss_fn, optimizer: SGD, example_x, example_y, warmup: int = 3, overlap: bool = True,
+                 warmup_data=None):
+        """The recording is preceded by ``warmup`` real training steps on the example batch (operators create their
+        per-stream scratch there, not inside the graph) - or, with ``warmup_data`` (a sequence of ``(x, y)`` of the
+        example's shapes), by one step on each of those: a loop that counts its steps hands over its first batches and
+        starts replaying with the next one; their losses are left in ``warmup_losses``."""
         self.model, self.loss_fn, self.opt = model, loss_fn, optimizer
         self.overlap = overlap  # EBOPs launches and the loss sum on a second branch of the graph, beside loss and backward
         self.x = example_x.clone()
         self.y = example_y.clone()
         self.loss = None
+        self.warmup_losses = []
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            for _ in range(warmup):
-                self._step()
+            if warmup_data is None:
+                for _ in range(warmup):
+                    self._step()
+            else:
+                if len(warmup_data) < 1:
+                    raise ValueError('the recording needs at least one step before it')
+                for wx, wy in warmup_data:
+                    self.x.copy_(wx), self.y.copy_(wy)
+                    self.warmup_losses.append(self._step().clone())
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.opt.zero_grad(set_to_none=True)
@@ -183,6 +196,15 @@ class GraphedTrainStep:
         ops.touch_state()  # the replayed kernels update the variables
         self.graph.replay()
         return self.loss
+
+    def eager(self, x, y):
+        """The same step launched kernel by kernel on a batch of another size (the last, shorter batch of an epoch)."""
+        keep = self.x, self.y
+        self.x, self.y = x, y
+        try:
+            return self._step()
+        finally:
+            self.x, self.y = keep
 
 
 _version_of = operator.attrgetter('_version')
@@ -343,7 +365,8 @@ class _FusedStep:
         return self.stack.step(x, y)
 
 
-def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 'sparse_ce', fused: bool | None = None):
+def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 'sparse_ce', fused: bool | None = None,
+                   warmup_data=None):
     """A callable ``step(x, y) -> loss`` that runs one SGD training step of ``model`` on the fastest path that covers it.
 
     A built stack of :class:`QDense` layers trained with mean sparse categorical cross-entropy and within what
@@ -352,11 +375,13 @@ def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 's
     (:class:`GraphedTrainStep` with :class:`SGD`, regularizers folded into the update).  Both paths update the same
     variables with the same arithmetic (the whole-step kernels restate the per-layer sequence), so the choice changes
     the time per step and nothing else.  ``fused=False`` forces the per-layer path, ``fused=True`` raises where the
-    whole-step path does not apply.  The returned object's ``path`` is ``'fused'`` or ``'layers_graph'``."""
+    whole-step path does not apply.  The returned object's ``path`` is ``'fused'`` or ``'layers_graph'``.
+    ``warmup_data``: see :class:`GraphedTrainStep` (the whole-step path needs no steps before it and takes none:
+    ``warmup_losses`` is then empty)."""
     if loss not in ('sparse_ce', 'mse'):
         raise ValueError(f"loss must be 'sparse_ce' or 'mse', got {loss!r}")
     if not model.built:
-        model(example_x, training=True)
+        model(example_x, training=False)  # creates the variables; an inference call leaves the integer-bit trackers alone
     if fused is not False and loss == 'sparse_ce':
         try:
             stack = FusedQDenseStack(model, lr=lr)
@@ -374,7 +399,90 @@ def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 's
     elif fused:
         raise ValueError('the fused QDense step computes sparse categorical cross-entropy only')
     loss_fn = ops.sparse_ce if loss == 'sparse_ce' else ops.mse
-    step = GraphedTrainStep(model, loss_fn, SGD(model.parameters(), lr=lr, fold_regularizers=True), example_x, example_y)
+    step = GraphedTrainStep(model, loss_fn, SGD(model.parameters(), lr=lr, fold_regularizers=True), example_x, example_y,
+                            warmup_data=warmup_data)
     step.path = 'layers_graph'
     return step
+
+
+def folded_regularizer_loss(model) -> float:
+    """Sum of the MonoL1 terms that :func:`model_loss` leaves out with ``fold_regularizers`` (trainable variables only)."""
+    total = 0.0
+    with torch.no_grad():
+        for p in model.parameters():
+            r = getattr(p, 'regularizer', None)
+            if isinstance(r, MonoL1) and p.requires_grad:
+                total += float(r(p))
+    return total
+
+
+def fit(model, x, y, *, loss: str = 'sparse_ce', lr: float = 0.01, batch_size: int = 1024, epochs: int = 1, callbacks=(),
+        shuffle: bool = True, seed: int | None = None, fused: bool | None = None):
+    """Train ``model`` on the resident tensors ``x`` / ``y`` (first axis: samples) with plain SGD, the way the reference's
+    users call ``model.fit`` (reference tests/base.py:313-331; the epoch hooks of src/hgq/utils/sugar/ drive beta from it):
+    per epoch the callbacks' ``on_epoch_begin``, the batches in order (shuffled anew per epoch with ``shuffle``; the last
+    one may be shorter), ``on_epoch_end`` with ``logs['loss']`` = the mean of the epoch's step losses.  Returns the list
+    of the epochs' logs.
+
+    The steps run on the fastest path that covers the model (:func:`train_step_for`): full batches through the
+    whole-step kernels or a HIP-graph replay - the recording's preparatory steps are the loop's own first batches, so
+    every batch is trained on exactly once - and a shorter last batch through the same kernels launched one by one.
+    The epoch's loss is summed on the device and read once per epoch.  On the per-layer path the MonoL1 terms of the
+    variables are applied inside the update launch and are not part of a step's loss value: their sum
+    (:func:`folded_regularizer_loss`, of the order of 1e-4 with the default 1e-8 factors) is added to ``logs['loss']``
+    once, from the variables as they stand when the epoch ends; the whole-step kernels include it in every step."""
+    n = int(x.shape[0])
+    if n < 1 or int(y.shape[0]) != n:
+        raise ValueError('x and y must hold the same, non-zero number of samples')
+    if not x.is_cuda:
+        raise ValueError('fit trains on GPU tensors: the product has no CPU path')
+    batch_size = min(int(batch_size), n)
+    n_full, tail = divmod(n, batch_size)
+    gen = torch.Generator(device='cpu')
+    if seed is not None:
+        gen.manual_seed(int(seed))
+    for cb in callbacks:
+        cb.set_model(model)
+    for cb in callbacks:
+        cb.on_train_begin({})
+    step = None
+    history = []
+    for epoch in range(epochs):
+        logs: dict = {}
+        for cb in callbacks:
+            cb.on_epoch_begin(epoch, logs)
+        order = torch.randperm(n, generator=gen).to(x.device) if shuffle else None
+
+        def batch(b, size=batch_size):
+            lo = b * batch_size
+            if order is None:
+                return x[lo:lo + size], y[lo:lo + size]
+            idx = order[lo:lo + size]
+            return x.index_select(0, idx), y.index_select(0, idx)
+
+        total = torch.zeros((), dtype=torch.float32, device=x.device)
+        first = 0
+        if step is None:
+            # the steps before the recording are this epoch's first batches
+            warm = [batch(b) for b in range(min(3, n_full))]
+            step = train_step_for(model, *warm[0], lr=lr, loss=loss, fused=fused, warmup_data=warm)
+            done = getattr(step, 'warmup_losses', [])
+            for l in done:
+                total += l.reshape(())
+            first = len(done)
+        for b in range(first, n_full):
+            total += step(*batch(b)).reshape(())
+        if tail:
+            bx, by = batch(n_full, tail)
+            if isinstance(step, _FusedStep):
+                total += step(bx.contiguous(), by.contiguous()).reshape(())
+            else:
+                total += step.eager(bx, by).reshape(())
+        logs['loss'] = float(total) / (n_full + (1 if tail else 0))
+        if not isinstance(step, _FusedStep):
+            logs['loss'] += folded_regularizer_loss(model)
+        for cb in callbacks:
+            cb.on_epoch_end(epoch, logs)
+        history.append(logs)
+    return history
 

@@ -933,3 +933,66 @@ def test_output_quantizer_inside_the_dense_kernel(dev, kind):
     for n in ga:
         err = (ga[n].double() - gb[n].double()).abs().max().item()
         assert err <= 2e-5 * (gb[n].abs().max().item() + 1e-6), (n, err)
+
+
+@pytest.mark.parametrize('fused', [False, None])
+def test_fit_trains_every_batch_once_on_the_fast_path(dev, fused):
+    """`train.fit`: epochs of full batches through the recorded step (or the whole-step kernels) plus a shorter last
+    batch, hooks in Keras' order.  On the per-layer path the variables equal those of the same steps launched one by one,
+    bit for bit and the logged losses agree to 1e-6 (a sum on the device against a sum on the host); on the whole-step path
+    (same arithmetic restated) the epoch losses agree to 1e-5 and the variables to 1e-4 of their largest entry."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import SGD, fit, folded_regularizer_loss, model_loss
+    from hgq2_amd.utils.models import qdense_mlp
+    from hgq2_amd.utils.sugar import BetaScheduler, Callback, FreeEBOPs
+
+    g = torch.Generator().manual_seed(12)
+    n, bs = 5 * 512 + 200, 512
+    x = torch.randn(n, 16, generator=g).to(dev)
+    y = torch.randint(0, 5, (n,), generator=g).to(dev)
+    src = ref.RefMLP(seed=6)
+    model, twin = qdense_mlp(device=dev), qdense_mlp(device=dev)
+    _copy_mlp(src, model, dev), _copy_mlp(src, twin, dev)
+
+    calls = []
+
+    class Spy(Callback):
+        def on_train_begin(self, logs=None):
+            calls.append('train')
+
+        def on_epoch_begin(self, epoch, logs=None):
+            calls.append(f'begin{epoch}')
+
+        def on_epoch_end(self, epoch, logs=None):
+            calls.append(f'end{epoch}')
+
+    betas = [1e-5, 3e-5]
+    history = fit(model, x, y, lr=0.01, batch_size=bs, epochs=2, shuffle=False, fused=fused,
+                  callbacks=[Spy(), BetaScheduler(lambda e: betas[e]), FreeEBOPs()])
+    assert calls == ['train', 'begin0', 'end0', 'begin1', 'end1']
+    assert [h['beta'] for h in history] == betas and all(h['ebops'] > 0 for h in history)
+
+    opt = SGD(twin.parameters(), lr=0.01, fold_regularizers=True)
+    want = []
+    for e in range(2):
+        for layer in twin.layers:
+            layer._beta.fill_(betas[e])
+        total = 0.0
+        for lo in range(0, n, bs):
+            opt.zero_grad()
+            with ops.overlap_ebops():
+                loss = model_loss(twin, ops.sparse_ce(twin(x[lo:lo + bs], training=True), y[lo:lo + bs]), True)
+                opt.backward(loss)
+                opt.step()
+            total += float(loss.detach())
+        want.append(total / 6 + folded_regularizer_loss(twin))
+    torch.cuda.synchronize()
+    for h, w in zip(history, want):
+        assert abs(h['loss'] - w) <= (1e-6 if fused is False else 1e-5) * abs(w)
+    if fused is False:
+        for pm, pt in zip(model.parameters(), twin.parameters()):
+            assert torch.equal(pm, pt)
+    else:
+        for pm, pt in zip(model.parameters(), twin.parameters()):
+            scale = pt.abs().max().item() + 1e-6
+            assert (pm - pt).abs().max().item() <= 1e-4 * scale
