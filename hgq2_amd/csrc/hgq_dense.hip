@@ -508,6 +508,19 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
 // Operand layout of the 32x32x16 instruction (64 lanes, eight bf16 per lane and operand):
 // A[i][k]: i = lane % 32, k = 8 (lane / 32) + e;  B[k][j]: k = 8 (lane / 32) + e, j = lane % 32;  D as for 32x32x2.
 // ------------------------------------------------------------------------------------------
+// Time stamps of workgroup 0 (measurement builds only: -DDB_PROF): [kernel: 0 forward, 1 backward][wavefront][event],
+// in ticks of the constant-rate counter
+#ifdef DB_PROF
+__device__ unsigned long long db_prof_stamps[2 * 4 * 32];
+#define DB_STAMP(k, i)                                                                                                  \
+    do {                                                                                                                \
+        if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (i) < 32)                                                     \
+            db_prof_stamps[((k) * 4 + (threadIdx.x >> 6)) * 32 + (i)] = wall_clock64();                                 \
+    } while (0)
+#else
+#define DB_STAMP(k, i)
+#endif
+
 #define BF_LD 72  // bf16 per LDS row: rows 144 bytes apart keep the 128-bit operand reads of 16 consecutive rows on different banks
 
 typedef uint16_t (*bf16_planes_t)[FAST_BM + 1][BF_LD];  // [part][row][k] of one staged tile
@@ -661,12 +674,16 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         for (int j = 0; j < FAST_NJ; ++j) raw[j] = buf_ld4(rs, xoff[j]);
     };
     int64_t tile = blockIdx.x;
+    DB_STAMP(0, 0);
     if (tile < n_tiles) load_tile(tile);
     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
     u32x4_t wp[3][NS];
     const int PW = bf16_kernel_column<NS>(qw, K, N, bcol, kq, wp);  // parts of the kernel this wavefront multiplies by
     const float bias = (qb && bcol < N) ? qb[bcol] : 0.f;
-    for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;  // columns >= K stay zero
+    // columns from K to the end of the last step of sixteen must read as zero (they are never staged); with K a multiple
+    // of 16 every column a matrix instruction reads is staged in every tile and the 56 KB need no clearing
+    if (K & 15)
+        for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;
     if (tid < 3) need[tid] = 0u;
     const bool vec_out = (N & 3) == 0 && ((uintptr_t)y & 15u) == 0;
     mo.init(vec_out ? N : 4);
@@ -701,8 +718,10 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     }
     __syncthreads();
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    DB_STAMP(0, 1);
     int buf = 0, slot = 0;
-    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1, slot = slot == 2 ? 0 : slot + 1) {
+    [[maybe_unused]] int it_ = 0;
+    for (; tile < n_tiles; tile += gridDim.x, buf ^= 1, slot = slot == 2 ? 0 : slot + 1, ++it_) {
         int fi[FAST_NJ][4];
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
@@ -711,7 +730,9 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
             for (int e = 0; e < 4; ++e) fi[j][e] = unpack_i8(fip[j], e);
         }
         bf16_stage<RM, QUANT, QUANT>(raw, fi, mp, xp[buf], &need[slot], amx);
+        DB_STAMP(0, 2 + 6 * it_);
         __syncthreads();
+        DB_STAMP(0, 3 + 6 * it_);
         if (tid == 0) need[slot == 0 ? 2 : slot - 1] = 0u;  // (slot + 2) % 3
         const int64_t next = tile + gridDim.x;
         if (next < n_tiles) load_tile(next);
@@ -719,6 +740,7 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         if (cb * 32 < N) {
             acc = bf16_chain<NS>(acc, xp[buf], arow, kq, need[slot], wp, PW);
         }
+        DB_STAMP(0, 4 + 6 * it_);
         const int64_t r0 = tile * FAST_BM;
         if (vec_out) {
 #pragma unroll
@@ -727,7 +749,9 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
                 if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
                 ys[rh * 32 + acc_row(r, lane)][bcol] = v;
             }
+            DB_STAMP(0, 5 + 6 * it_);
             __syncthreads();
+            DB_STAMP(0, 6 + 6 * it_);
 #pragma unroll
             for (int j = 0; j < FAST_NJ; ++j) {
                 const int64_t gr = r0 + mo.row[j];
@@ -762,6 +786,7 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
             }
         }
     }
+    DB_STAMP(0, 30);
     if (QUANT && amax_part && P == FAST_BM && ((uintptr_t)amax_part & 15u) == 0) {
         uint32_t *my = amax_part + (int64_t)blockIdx.x * (P * K);
 #pragma unroll
@@ -812,6 +837,7 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
             for (int t = tid; t < PN; t += 256) my[t] = tab[t];
         }
     }
+    DB_STAMP(0, 31);
 }
 
 // Column statistics of the contraction without writing it: sum_r z and sum_r z^2 of z = x W per
@@ -910,7 +936,8 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bf16_kernel(const float 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rh = wave & 1, cb = wave >> 1;
     const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
-    for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;
+    if (K & 15)  // (as in the forward kernel: only the columns between K and the next multiple of 16 need zeros)
+        for (int id = tid; id < 2 * 3 * (FAST_BM + 1) * BF_LD / 2; id += 256) ((uint32_t *)&xp[0][0][0][0])[id] = 0u;
     if (tid < 3) need[tid] = 0u;
     const int arow = rh * 32 + (lane & 31), kq = lane >> 5, bcol = cb * 32 + (lane & 31);
     u32x4_t wp[3][NS];
@@ -1026,6 +1053,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         zoff[j] = mz.on[j] ? (uint32_t)(mz.row[j] * N + mz.col[j]) * 4u : BUF_OOB;
     }
     int64_t tile = blockIdx.x;
+    DB_STAMP(1, 0);
     // descriptors cover the valid rows of one tile (rows past the end read as zero); without ReLU
     // the mask descriptor is empty and is not consulted
     auto load_tile = [&](int64_t t) {
@@ -1080,9 +1108,12 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     }
     __syncthreads();
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing loaded before the loop is waited for inside it
-    for (; tile < n_tiles; tile += gridDim.x) {
+    DB_STAMP(1, 1);
+    [[maybe_unused]] int it_ = 0;
+    for (; tile < n_tiles; tile += gridDim.x, ++it_) {
         float dlt[FAST_NJ][4];  // xq - x of the elements this thread stages
         __syncthreads();        // previous tile's dx has been read back
+        DB_STAMP(1, 2 + 6 * it_);
         // no branch around a staging slot (a wait inside one would cover every load): idle slots
         // hold zeros and write them to the sink row
 #pragma unroll
@@ -1109,7 +1140,9 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                 for (int e = 0; e < 4; ++e) dzs[zr][mz.col[j] + e] = (!relu || a[e] > 0.f) ? g[e] : 0.f;
             }
         }
+        DB_STAMP(1, 3 + 6 * it_);
         __syncthreads();
+        DB_STAMP(1, 4 + 6 * it_);
         if (STATS) {
             // z block (row half, column block) of this wave, then dz into the gradient tile
             const int zrh = wave & 1, zcb = wave >> 1;
@@ -1181,7 +1214,9 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 #pragma unroll
             for (int j = 0; j < FAST_BM / 4; ++j) accb += dzs[bq * (FAST_BM / 4) + j][bn];
         }
+        DB_STAMP(1, 5 + 6 * it_);
         __syncthreads();  // dz and xq consumed: the dx tile takes the place of dz (its second partial sum that of xq)
+        DB_STAMP(1, 6 + 6 * it_);
         if (PAIRS) {
             if (wave < 2) {
 #pragma unroll
@@ -1200,6 +1235,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
             for (int r = 0; r < 16; ++r) dzs[rh * 32 + acc_row(r, lane)][kcol] = acc[r];
         }
         __syncthreads();
+        DB_STAMP(1, 7 + 6 * it_);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
             if (mx.on[j]) {
@@ -1227,6 +1263,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         }
     }
     // ---- write this workgroup's slice.  Waves sharing a kernel-gradient block combine through LDS.
+    DB_STAMP(1, 30);
     __syncthreads();
     float *comb = &xs[0][0];
     if (PAIRS) {
@@ -1273,16 +1310,35 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 #pragma unroll
                 for (int e = 0; e < 4; ++e) gt[mx.row[j] * FAST_LD + mx.col[j] + e] = gf[j][e];
         __syncthreads();
-#pragma unroll 4
-        for (int id = tid; id < P * 64; id += 256) {
-            const int p = id >> 6, c = id & 63;
-            if (c < K) {
+        if (P <= 16) {
+            // few table rows, many tile rows per entry: four threads per entry add a quarter of the tile each (a serial
+            // walk over all 64 rows was three microseconds of every launch), then the quarters are added in order
+            float *quarter = &xs[0][0];  // (the kernel-gradient block has left it)
+            for (int id = tid; id < 4 * P * 64; id += 256) {
+                const int c = id & 63, pq = id >> 6, p = pq & (P - 1), q = pq / P;  // (P is a power of two)
                 float s = 0.f;
-                for (int r = p; r < FAST_BM; r += P) s += gt[r * FAST_LD + c];
-                my_df[p * K + c] = s;
+                for (int r = 16 * q + p; r < 16 * q + 16; r += P) s += gt[r * FAST_LD + c];
+                quarter[pq * 64 + c] = s;
+            }
+            __syncthreads();
+            for (int id = tid; id < P * 64; id += 256) {
+                const int p = id >> 6, c = id & 63;
+                if (c < K)
+                    my_df[p * K + c] = (quarter[p * 64 + c] + quarter[(P + p) * 64 + c]) + (quarter[(2 * P + p) * 64 + c] + quarter[(3 * P + p) * 64 + c]);
+            }
+        } else {
+#pragma unroll 4
+            for (int id = tid; id < P * 64; id += 256) {
+                const int p = id >> 6, c = id & 63;
+                if (c < K) {
+                    float s = 0.f;
+                    for (int r = p; r < FAST_BM; r += P) s += gt[r * FAST_LD + c];
+                    my_df[p * K + c] = s;
+                }
             }
         }
     }
+    DB_STAMP(1, 31);
 }
 
 // out[e] = sum over slices of part[g][e], in slice order.  256 threads = 64 elements x 4 slice groups.
@@ -1416,6 +1472,12 @@ static inline int row_parts(int64_t rows, int bm) {
 }  // namespace hgq
 
 using namespace hgq;
+
+#ifdef DB_PROF
+extern "C" int hgq_db_prof_read(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(db_prof_stamps), sizeof(unsigned long long) * 2 * 4 * 32) == hipSuccess ? 0 : -2;
+}
+#endif
 
 // 1: the streaming dense kernels contract on the bf16 matrix cores by exact splitting; 0: on the fp32 ones
 static int g_dense_bf16 = 1;
