@@ -1341,6 +1341,250 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     DB_STAMP(1, 31);
 }
 
+// ------------------------------------------------------------------------------------------
+// Backward of the column statistics without the pre-activation.  With z = xq W, the upstream gradients gm / gs of the
+// column means / means of squares give  dz[r, c] = (gm[c] + 2 z[r, c] gs[c]) / rows,  and both results are functions of
+// xq through K x K matrices:
+//     dx = dz W^T          = xq A + v,      A = (2 / rows) W diag(gs) W^T,   v = W gm / rows
+//     dW = xq^T dz         = (m gm^T + 2 (S W) diag(gs)) / rows,   S = xq^T xq,  m = column sums of xq  (live rows)
+// so a tile costs one contraction of the quantized input with A (the kernel above recomputes z, forms dz and contracts it
+// twice, each time splitting fresh fp32 values) and one Gram update of the quantized input with itself - operands of one
+// bf16 part each in the usual case.  A and v are formed once per workgroup while the first tile is on its way; S W once
+// per workgroup at the end.  Slices, arguments and results are those of the STATS form of qdense_bwd_fast_kernel
+// (dy = gm, y = gs, no activation, no bias; the [N] section of a slice is zero).
+// ------------------------------------------------------------------------------------------
+template <int RM, bool QUANT>
+__global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const float *__restrict__ gm, const float *__restrict__ gs,
+                                                                     const float *__restrict__ x, const float *__restrict__ f_in,
+                                                                     int P, const float *__restrict__ w, float *__restrict__ dx,
+                                                                     float *part, int64_t rows, int K, int N, int mode,
+                                                                     const float *__restrict__ dx_add) {
+    __shared__ float xs[FAST_BM + 1][FAST_LD];    // the quantized input tile, then the dx tile; row FAST_BM: sink of the idle staging slots
+    __shared__ float adds[FAST_BM + 1][FAST_LD];  // the tile of dx_add (start-up: W diag(2 gs / rows))
+    __shared__ float As[64][FAST_LD];             // A
+    __shared__ float ws[64][FAST_LD];             // W, zero beyond [K, N]
+    __shared__ float vs[64], gms[64], gss[64];
+    const bool has_add = dx_add != nullptr;
+    const Mode m(mode);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, kq = lane >> 5;
+    const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5;
+    const int PK = QUANT ? P * K : 0;
+    const int64_t M = (int64_t)K * N + N + PK;
+    const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
+    float *my_dw = part + (int64_t)blockIdx.x * M;
+    float *my_db = my_dw + (int64_t)K * N;
+    float *my_df = my_db + N;
+    const float inv_rows = 1.0f / (float)rows;
+    FastMap mx;
+    mx.init(K);
+    int fip[FAST_NJ];
+    float gf[FAST_NJ][4];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) gf[j][e] = 0.f;
+    // Gram block of this wavefront: (k block, j block); with one k block the four wavefronts share it, a quarter of the
+    // tile's rows each
+    const int gblk = K32 * K32, gpb = 4 / gblk;
+    const int gb = wave / gpb, gsub = wave % gpb;
+    const int gib = gb / K32, gjb = gb % K32;
+    const int grows = FAST_BM / gpb;
+    floatx16 accS = {0};
+    float accm = 0.f;
+    const int bn = tid & 63, bq = tid >> 6;
+
+    f32x4_t rx[FAST_NJ], rg[FAST_NJ];
+    uint32_t xoff[FAST_NJ];
+#pragma unroll
+    for (int j = 0; j < FAST_NJ; ++j) xoff[j] = mx.on[j] ? (uint32_t)(mx.row[j] * K + mx.col[j]) * 4u : BUF_OOB;
+    int64_t tile = blockIdx.x;
+    auto load_tile = [&](int64_t t) {
+        const int64_t r0 = t * FAST_BM, left = rows - r0, vr = left < FAST_BM ? left : FAST_BM;
+        const __amdgpu_buffer_rsrc_t sx = buf_rsrc(x + r0 * K, vr * K * 4);
+        const __amdgpu_buffer_rsrc_t sg = buf_rsrc(has_add ? dx_add + r0 * K : x, has_add ? vr * K * 4 : 0);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            rx[j] = buf_ld4(sx, xoff[j]);
+            rg[j] = buf_ld4(sg, xoff[j]);  // the other gradient of x, laid out like x (zeros without one)
+        }
+    };
+    if (tile < n_tiles) load_tile(tile);
+    {
+        // start-up under the first tile's latency: W, its scaled copy, the fractional bits; then A and v
+        const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(w, (int64_t)K * N * 4);
+        const __amdgpu_buffer_rsrc_t rs_m = buf_rsrc(gm, (int64_t)N * 4), rs_s = buf_rsrc(gs, (int64_t)N * 4);
+        float wv[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
+            wv[u] = buf_ld1(rs_w, (kk < K && nn < N) ? (uint32_t)(kk * N + nn) * 4u : BUF_OOB);
+        }
+        const float g1 = buf_ld1(rs_m, bn < N ? (uint32_t)bn * 4u : BUF_OOB), g2 = buf_ld1(rs_s, bn < N ? (uint32_t)bn * 4u : BUF_OOB);
+        int fi[FAST_NJ][4], tix[FAST_NJ];
+        fast_frac_bits<QUANT>(f_in, P, K, mx, m.round_params, fi, tix);
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) fip[j] = pack_i8x4(fi[j]);
+        const float sc = 2.0f * g2 * inv_rows;  // column bn = id & 63 of every entry this thread holds
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
+            ws[kk][nn] = wv[u];
+            adds[kk][nn] = wv[u] * sc;
+            xs[kk][nn] = 0.f;
+        }
+        if (tid < 64) gms[tid] = g1, gss[tid] = g2;
+        __syncthreads();
+        // A block (i block, j block) of this wavefront: sum over n of (W diag)[i][n] W[j][n]; blocks past K are zero
+        {
+            const int ib = wave & 1, jb = wave >> 1;
+            floatx16 a = {0};
+            a = mfma_chain(a, &adds[ib * 32 + l32][kq], 1, &ws[jb * 32 + l32][kq], 1, N32 * 2);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) As[ib * 32 + acc_row(r, lane)][jb * 32 + l32] = a[r];
+        }
+        if (tid < 64) {
+            float sacc = 0.f;
+            for (int n = 0; n < N; ++n) sacc += gms[n] * ws[tid][n];
+            vs[tid] = sacc * inv_rows;
+        }
+    }
+    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing loaded before the loop is waited for inside it
+    for (; tile < n_tiles; tile += gridDim.x) {
+        float dlt[FAST_NJ][4];  // xq - x of the elements this thread stages
+        __syncthreads();        // the previous tile's dx has been read back
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            const float v[4] = {rx[j][0], rx[j][1], rx[j][2], rx[j][3]};
+            const int xr = mx.on[j] ? mx.row[j] : FAST_BM;
+            asm volatile("" : "+v"(fip[j]));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int f = unpack_i8(fip[j], e);
+                const float q = QUANT ? ldexpf(round_scaled<RM>(ldexpf(v[e], f)), -f) : v[e];
+                dlt[j][e] = q - v[e];
+                xs[xr][mx.col[j] + e] = q;
+            }
+            if (has_add) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) adds[xr][mx.col[j] + e] = rg[j][e];
+            }
+        }
+        __syncthreads();
+        const int64_t next = tile + gridDim.x;
+        const int64_t r0 = tile * FAST_BM;
+        if (next < n_tiles) load_tile(next);
+        // ---- dx = xq A : (row half, k block); the quantized input usually has one bf16 part, A takes all three
+        floatx16 acc = {0};
+        const int rh = wave & 1, kb = wave >> 1;
+        if (kb < K32) acc = mfma_chain_bf16<false, true>(acc, &xs[rh * 32 + l32][kq], 1, &As[kq][kb * 32 + l32], FAST_LD, K32 * 2);
+        // ---- S += xq^T xq : this wavefront's block over its rows of the tile (rows past the end are zeros)
+        accS = mfma_chain_bf16<false, false>(accS, &xs[gsub * grows + kq][gib * 32 + l32], FAST_LD, &xs[gsub * grows + kq][gjb * 32 + l32], FAST_LD, grows / 16);
+#pragma unroll
+        for (int j = 0; j < FAST_BM / 4; ++j) accm += xs[bq * (FAST_BM / 4) + j][bn];
+        __syncthreads();  // xq consumed: the dx tile takes its place
+        if (kb < K32) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) xs[rh * 32 + acc_row(r, lane)][kb * 32 + l32] = acc[r];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j) {
+            if (mx.on[j]) {
+                const int64_t gr = r0 + mx.row[j];
+                float4 o;
+                o.x = xs[mx.row[j]][mx.col[j]] + vs[mx.col[j]], o.y = xs[mx.row[j]][mx.col[j] + 1] + vs[mx.col[j] + 1];
+                o.z = xs[mx.row[j]][mx.col[j] + 2] + vs[mx.col[j] + 2], o.w = xs[mx.row[j]][mx.col[j] + 3] + vs[mx.col[j] + 3];
+                const float4 og = o;  // this contraction's own gradient: the one the rounding residue meets
+                if (has_add) {
+                    o.x += adds[mx.row[j]][mx.col[j]], o.y += adds[mx.row[j]][mx.col[j] + 1];
+                    o.z += adds[mx.row[j]][mx.col[j] + 2], o.w += adds[mx.row[j]][mx.col[j] + 3];
+                }
+                if (gr < rows) {
+                    st4(dx + gr * K + mx.col[j], o);
+                    if (QUANT) {
+                        gf[j][0] += -HGQ_LN2 * dlt[j][0] * og.x, gf[j][1] += -HGQ_LN2 * dlt[j][1] * og.y;
+                        gf[j][2] += -HGQ_LN2 * dlt[j][2] * og.z, gf[j][3] += -HGQ_LN2 * dlt[j][3] * og.w;
+                    }
+                }
+            }
+        }
+    }
+    // ---- this workgroup's slice: S and m through LDS (wavefronts that share a Gram block add in a fixed order), then
+    // dW = (m gm^T + 2 (S W) diag(gs)) / rows on the fp32 matrix instruction (both operands are arbitrary fp32)
+    __syncthreads();
+    float *Ss = &xs[0][0];
+    for (int pass = 0; pass < gpb; ++pass) {
+        if (gsub == pass) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int k = gib * 32 + acc_row(r, lane), jx = gjb * 32 + l32;
+                if (pass == 0) Ss[k * FAST_LD + jx] = accS[r];
+                else Ss[k * FAST_LD + jx] += accS[r];
+            }
+        }
+        __syncthreads();
+    }
+    float *bred = &adds[0][0];
+    bred[tid] = accm;
+    __syncthreads();
+    if (tid < 64) vs[tid] = (bred[tid] + bred[tid + 64]) + (bred[tid + 128] + bred[tid + 192]);  // m (v is not needed any more)
+    __syncthreads();
+    {
+        const int nb2 = K32 * N32;
+        if (wave < nb2) {
+            const int wkb = wave / N32, wnb = wave % N32;
+            floatx16 t = {0};
+            t = mfma_chain(t, &Ss[(wkb * 32 + l32) * FAST_LD + kq], 1, &ws[kq][wnb * 32 + l32], FAST_LD, K32 * 2);
+            const int c = wnb * 32 + l32;
+            const float g1 = gms[c], g2 = gss[c];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int k = wkb * 32 + acc_row(r, lane);
+                if (k < K && c < N) my_dw[k * N + c] = (vs[k] * g1 + 2.0f * g2 * t[r]) * inv_rows;
+            }
+        }
+    }
+    if (tid < N) my_db[tid] = 0.f;
+    if (QUANT) {
+        // fractional-bit gradient: every (tile row, column) has one owner thread; rows that share a table row are
+        // added in row order (few table rows: four threads per entry, a quarter of the tile each, as in the kernel above)
+        float *gt = &adds[0][0];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < FAST_NJ; ++j)
+            if (mx.on[j])
+#pragma unroll
+                for (int e = 0; e < 4; ++e) gt[mx.row[j] * FAST_LD + mx.col[j] + e] = gf[j][e];
+        __syncthreads();
+        if (P <= 16) {
+            float *quarter = &As[0][0];
+            for (int id = tid; id < 4 * P * 64; id += 256) {
+                const int c = id & 63, pq = id >> 6, p = pq & (P - 1), q = pq / P;
+                float sacc = 0.f;
+                for (int r = 16 * q + p; r < 16 * q + 16; r += P) sacc += gt[r * FAST_LD + c];
+                quarter[pq * 64 + c] = sacc;
+            }
+            __syncthreads();
+            for (int id = tid; id < P * 64; id += 256) {
+                const int p = id >> 6, c = id & 63;
+                if (c < K)
+                    my_df[p * K + c] = (quarter[p * 64 + c] + quarter[(P + p) * 64 + c]) + (quarter[(2 * P + p) * 64 + c] + quarter[(3 * P + p) * 64 + c]);
+            }
+        } else {
+#pragma unroll 4
+            for (int id = tid; id < P * 64; id += 256) {
+                const int p = id >> 6, c = id & 63;
+                if (c < K) {
+                    float sacc = 0.f;
+                    for (int r = p; r < FAST_BM; r += P) sacc += gt[r * FAST_LD + c];
+                    my_df[p * K + c] = sacc;
+                }
+            }
+        }
+    }
+}
+
 // out[e] = sum over slices of part[g][e], in slice order.  256 threads = 64 elements x 4 slice groups.
 #define RP_G 16  // slice groups per entry: 64 entries x 16 groups = 1024 threads, few dependent load batches per thread
 __global__ __launch_bounds__(64 * RP_G) void reduce_parts_kernel(const float *__restrict__ part, int n_parts, int64_t M,
@@ -1683,7 +1927,7 @@ extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t
     const dim3 grid((unsigned)parts);
 #define HGQ_MOM_BWD(RMV, QV) \
     do { \
-        if (g_dense_bf16) hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true, true, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode, dx_add); \
+        if (g_dense_bf16) hipLaunchKernelGGL((dense_moments_bwd_gram_kernel<RMV, QV>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, rows, K, N, mode, dx_add); \
         else hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode, dx_add); \
     } while (0)
     if (!quant) HGQ_MOM_BWD(HGQ_TRN, false);

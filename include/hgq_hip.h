@@ -758,9 +758,11 @@ int hgq_bn_fold_quant_bwd(const float *w, const float *bias, const float *gamma,
 /*
  * Batch statistics of the un-quantized pre-activation z = x W of QEinsumDenseBatchnorm.call
  * (src/hgq/layers/einsum_dense_batchnorm.py:99-124) WITHOUT materialising z: the contraction and the
- * column sums run in one pass over x, and the backward recomputes z tile by tile.
+ * column sums run in one pass over x.
  *   x [rows, K];  w [K, N] (the un-quantized kernel);  mean, meansq [N] = mean_r z, mean_r z^2;
- *   backward: with dz[r, c] = (dmean[c] + 2 z[r, c] dmeansq[c]) / rows,  dx = dz W^T,  dw = x^T dz.
+ *   backward: with dz[r, c] = (dmean[c] + 2 z[r, c] dmeansq[c]) / rows,  dx = dz W^T,  dw = x^T dz - evaluated without z
+ *   on the default matrix instruction:  dx = x A + v,  A = (2 / rows) W diag(dmeansq) W^T,  v = W dmean / rows;
+ *   dw = (m dmean^T + 2 (S W) diag(dmeansq)) / rows  with  S = x^T x  and m the column sums of x.
  *   workspace: hgq_dense_moments_workspace(rows, K, N) floats (per-workgroup slices, fixed-order sum).
  * K, N <= 64 and multiples of 4; x (and dx) 16-byte aligned; otherwise HGQ_ERR_UNSUPPORTED and the
  * caller uses hgq_qdense_fwd + hgq_col_moments_fwd.
