@@ -508,10 +508,10 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_fast_kernel(const float *__
 // Operand layout of the 32x32x16 instruction (64 lanes, eight bf16 per lane and operand):
 // A[i][k]: i = lane % 32, k = 8 (lane / 32) + e;  B[k][j]: k = 8 (lane / 32) + e, j = lane % 32;  D as for 32x32x2.
 // ------------------------------------------------------------------------------------------
-// Time stamps of workgroup 0 (measurement builds only: -DDB_PROF): [kernel: 0 forward, 1 backward][wavefront][event],
+// Time stamps of workgroup 0 (measurement builds only: -DDB_PROF): [kernel: 0 forward, 1 backward, 2 statistics' backward][wavefront][event],
 // in ticks of the constant-rate counter
 #ifdef DB_PROF
-__device__ unsigned long long db_prof_stamps[2 * 4 * 32];
+__device__ unsigned long long db_prof_stamps[3 * 4 * 32];
 #define DB_STAMP(k, i)                                                                                                  \
     do {                                                                                                                \
         if (blockIdx.x == 0 && (threadIdx.x & 63) == 0 && (i) < 32)                                                     \
@@ -1352,29 +1352,36 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
 // bf16 part each in the usual case.  A and v are formed once per workgroup while the first tile is on its way; S W once
 // per workgroup at the end.  Slices, arguments and results are those of the STATS form of qdense_bwd_fast_kernel
 // (dy = gm, y = gs, no activation, no bias; the [N] section of a slice is zero).
+// rep > 1 (a narrow input, K rep = 64): the caller passes the [rows, K] operands as [rows / rep, 64] - the same memory, rep
+// rows side by side, the [P, K] table of fractional bits as [P / rep, 64] - and the kernel works on 64-wide rows with
+// A' = diag(A, ..., A) and v' = (v, ..., v); S and m are the sums of the diagonal blocks / segments of S' and m'.  A tile
+// then holds 64 rep rows of the input, so a narrow layer pays the per-tile latencies a quarter or an eighth as often.
 // ------------------------------------------------------------------------------------------
 template <int RM, bool QUANT>
 __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const float *__restrict__ gm, const float *__restrict__ gs,
                                                                      const float *__restrict__ x, const float *__restrict__ f_in,
                                                                      int P, const float *__restrict__ w, float *__restrict__ dx,
                                                                      float *part, int64_t rows, int K, int N, int mode,
-                                                                     const float *__restrict__ dx_add) {
-    __shared__ float xs[FAST_BM + 1][FAST_LD];    // the quantized input tile, then the dx tile; row FAST_BM: sink of the idle staging slots
+                                                                     const float *__restrict__ dx_add, int rep) {
+    // the quantized input tile, then the dx tile (start-up: A in fp32); rows 68 words apart: 128-bit reads along a row, row
+    // FAST_BM the sink of the idle staging slots
+    __shared__ __attribute__((aligned(16))) float xs[FAST_BM + 1][FAST_XLD];
     __shared__ float adds[FAST_BM + 1][FAST_LD];  // the tile of dx_add (start-up: W diag(2 gs / rows))
-    __shared__ float As[64][FAST_LD];             // A
+    __shared__ __attribute__((aligned(16))) uint16_t Ap[3][64][BF_LD];  // A in bf16 parts, row j = column j (A is symmetric)
     __shared__ float ws[64][FAST_LD];             // W, zero beyond [K, N]
     __shared__ float vs[64], gms[64], gss[64];
     const bool has_add = dx_add != nullptr;
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, kq = lane >> 5;
-    const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5;
+    const int Ko = K / rep;  // rows of W; K is the width of a staged row
+    const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5, Ko32 = (Ko + 31) >> 5;
     const int PK = QUANT ? P * K : 0;
-    const int64_t M = (int64_t)K * N + N + PK;
+    const int64_t M = (int64_t)Ko * N + N + PK;
     const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
     float *my_dw = part + (int64_t)blockIdx.x * M;
-    float *my_db = my_dw + (int64_t)K * N;
+    float *my_db = my_dw + (int64_t)Ko * N;
     float *my_df = my_db + N;
-    const float inv_rows = 1.0f / (float)rows;
+    const float inv_rows = 1.0f / ((float)rows * (float)rep);  // the statistics are over the rows of the input, not over the staged rows
     FastMap mx;
     mx.init(K);
     int fip[FAST_NJ];
@@ -1408,16 +1415,17 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
             rg[j] = buf_ld4(sg, xoff[j]);  // the other gradient of x, laid out like x (zeros without one)
         }
     };
+    DB_STAMP(2, 0);
     if (tile < n_tiles) load_tile(tile);
     {
         // start-up under the first tile's latency: W, its scaled copy, the fractional bits; then A and v
-        const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(w, (int64_t)K * N * 4);
+        const __amdgpu_buffer_rsrc_t rs_w = buf_rsrc(w, (int64_t)Ko * N * 4);
         const __amdgpu_buffer_rsrc_t rs_m = buf_rsrc(gm, (int64_t)N * 4), rs_s = buf_rsrc(gs, (int64_t)N * 4);
         float wv[16];
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
             const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
-            wv[u] = buf_ld1(rs_w, (kk < K && nn < N) ? (uint32_t)(kk * N + nn) * 4u : BUF_OOB);
+            wv[u] = buf_ld1(rs_w, (kk < Ko && nn < N) ? (uint32_t)(kk * N + nn) * 4u : BUF_OOB);
         }
         const float g1 = buf_ld1(rs_m, bn < N ? (uint32_t)bn * 4u : BUF_OOB), g2 = buf_ld1(rs_s, bn < N ? (uint32_t)bn * 4u : BUF_OOB);
         int fi[FAST_NJ][4], tix[FAST_NJ];
@@ -1432,7 +1440,7 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
             adds[kk][nn] = wv[u] * sc;
             xs[kk][nn] = 0.f;
         }
-        if (tid < 64) gms[tid] = g1, gss[tid] = g2;
+        if (tid < 64) gms[tid] = g1, gss[tid] = g2;  // (zero past N: the loads are out of range there)
         __syncthreads();
         // A block (i block, j block) of this wavefront: sum over n of (W diag)[i][n] W[j][n]; blocks past K are zero
         {
@@ -1440,19 +1448,53 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
             floatx16 a = {0};
             a = mfma_chain(a, &adds[ib * 32 + l32][kq], 1, &ws[jb * 32 + l32][kq], 1, N32 * 2);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) As[ib * 32 + acc_row(r, lane)][jb * 32 + l32] = a[r];
+            for (int r = 0; r < 16; ++r) xs[ib * 32 + acc_row(r, lane)][jb * 32 + l32] = a[r];  // A in fp32, for now
         }
-        if (tid < 64) {
+        {
+            // v = W gm / rows: four threads per entry, a quarter of the columns each
             float sacc = 0.f;
-            for (int n = 0; n < N; ++n) sacc += gms[n] * ws[tid][n];
-            vs[tid] = sacc * inv_rows;
+            for (int n = 16 * bq; n < 16 * bq + 16; ++n) sacc += gms[n] * ws[bn][n];  // (gms is zero past N)
+            adds[FAST_BM][0] = 0.f;  // (keeps the sink row defined)
+            __syncthreads();         // the scaled copy of W in `adds` has been read by every A block
+            adds[bq][bn] = sacc;
+            __syncthreads();
+            if (tid < 64) vs[tid] = ((adds[0][tid] + adds[1][tid]) + (adds[2][tid] + adds[3][tid])) * inv_rows;
+        }
+        // A (rep > 1: A' = diag(A, ..., A) and v' = (v, ..., v)) into bf16 parts, 64-bit stores of four entries; then the
+        // input tile's place is cleared again: its columns past K must read as zero
+        __syncthreads();
+        float vv = 0.f;
+        const int seg = rep > 1 ? Ko - 1 : 63;  // (rep > 1: Ko is a power of two, entry (kk, nn) of A' is entry (kk & seg, nn & seg) of A)
+        if (tid < 64) vv = vs[tid & seg];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int id = tid + 256 * u, kk = id >> 4, n4 = (id & 15) << 2;
+            // four consecutive columns lie in one diagonal block or in none (Ko is a multiple of 4)
+            const bool in_block = rep > 1 ? (kk & ~seg) == (n4 & ~seg) : (kk < K && n4 < K);
+            const f32x4_t a4 = *(const f32x4_t *)&xs[kk & seg][n4 & seg];
+            uint32_t h4[4], m4[4], l4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bf16_parts(in_block ? a4[e] : 0.f, h4[e], m4[e], l4[e]);
+            *(uint2 *)&Ap[0][kk][n4] = make_uint2(bf16_pair(h4[0], h4[1]), bf16_pair(h4[2], h4[3]));
+            *(uint2 *)&Ap[1][kk][n4] = make_uint2(bf16_pair(m4[0], m4[1]), bf16_pair(m4[2], m4[3]));
+            *(uint2 *)&Ap[2][kk][n4] = make_uint2(bf16_pair(l4[0], l4[1]), bf16_pair(l4[2], l4[3]));
+        }
+        __syncthreads();
+        if (tid < 64) vs[tid] = vv;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int id = tid + 256 * u, kk = id >> 6, nn = id & 63;
+            xs[kk][nn] = 0.f;
         }
     }
     __syncthreads();
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing loaded before the loop is waited for inside it
-    for (; tile < n_tiles; tile += gridDim.x) {
+    DB_STAMP(2, 1);
+    [[maybe_unused]] int it_ = 0;
+    for (; tile < n_tiles; tile += gridDim.x, ++it_) {
         float dlt[FAST_NJ][4];  // xq - x of the elements this thread stages
         __syncthreads();        // the previous tile's dx has been read back
+        DB_STAMP(2, 2 + 6 * it_);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
             const float v[4] = {rx[j][0], rx[j][1], rx[j][2], rx[j][3]};
@@ -1470,31 +1512,62 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
                 for (int e = 0; e < 4; ++e) adds[xr][mx.col[j] + e] = rg[j][e];
             }
         }
+        DB_STAMP(2, 3 + 6 * it_);
         __syncthreads();
+        DB_STAMP(2, 4 + 6 * it_);
         const int64_t next = tile + gridDim.x;
         const int64_t r0 = tile * FAST_BM;
         if (next < n_tiles) load_tile(next);
         // ---- dx = xq A : (row half, k block); the quantized input usually has one bf16 part, A takes all three
         floatx16 acc = {0};
         const int rh = wave & 1, kb = wave >> 1;
-        if (kb < K32) acc = mfma_chain_bf16<false, true>(acc, &xs[rh * 32 + l32][kq], 1, &As[kq][kb * 32 + l32], FAST_LD, K32 * 2);
+        if (kb < K32) {
+            // steps 16 bt + 8 kq + 0 .. 7 of a batch sit in one lane (both operands in the same order): the input row is read
+            // with two 128-bit loads, A's parts with one each
+#pragma unroll
+            for (int bt = 0; bt < 4; ++bt) {
+                if (bt < K32 * 2) {
+                    const f32x4_t a0 = *(const f32x4_t *)&xs[rh * 32 + l32][16 * bt + 8 * kq], a1 = *(const f32x4_t *)&xs[rh * 32 + l32][16 * bt + 8 * kq + 4];
+                    const float av[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                    u32x4_t pb[3], pa0;
+#pragma unroll
+                    for (int q = 0; q < 3; ++q) pb[q] = *(const u32x4_t *)&Ap[q][kb * 32 + l32][16 * bt + 8 * kq];
+                    const bool one_a = bf16_lead8(av, pa0);
+#pragma unroll
+                    for (int q = 0; q < 3; ++q) acc = mfma_bf16(pa0, pb[q], acc);
+                    if (!one_a) {
+                        u32x4_t p1, p2;
+                        const bool third = bf16_rest8(av, p1, p2);
+#pragma unroll
+                        for (int q = 0; q < 3; ++q) acc = mfma_bf16(p1, pb[q], acc);
+                        if (third) {
+#pragma unroll
+                            for (int q = 0; q < 3; ++q) acc = mfma_bf16(p2, pb[q], acc);
+                        }
+                    }
+                }
+            }
+        }
         // ---- S += xq^T xq : this wavefront's block over its rows of the tile (rows past the end are zeros)
-        accS = mfma_chain_bf16<false, false>(accS, &xs[gsub * grows + kq][gib * 32 + l32], FAST_LD, &xs[gsub * grows + kq][gjb * 32 + l32], FAST_LD, grows / 16);
+        accS = mfma_chain_bf16<false, false>(accS, &xs[gsub * grows + kq][gib * 32 + l32], FAST_XLD, &xs[gsub * grows + kq][gjb * 32 + l32], FAST_XLD, grows / 16);
 #pragma unroll
         for (int j = 0; j < FAST_BM / 4; ++j) accm += xs[bq * (FAST_BM / 4) + j][bn];
+        DB_STAMP(2, 5 + 6 * it_);
         __syncthreads();  // xq consumed: the dx tile takes its place
+        DB_STAMP(2, 6 + 6 * it_);
         if (kb < K32) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) xs[rh * 32 + acc_row(r, lane)][kb * 32 + l32] = acc[r];
         }
         __syncthreads();
+        DB_STAMP(2, 7 + 6 * it_);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
             if (mx.on[j]) {
                 const int64_t gr = r0 + mx.row[j];
+                const f32x4_t t4 = *(const f32x4_t *)&xs[mx.row[j]][mx.col[j]];
                 float4 o;
-                o.x = xs[mx.row[j]][mx.col[j]] + vs[mx.col[j]], o.y = xs[mx.row[j]][mx.col[j] + 1] + vs[mx.col[j] + 1];
-                o.z = xs[mx.row[j]][mx.col[j] + 2] + vs[mx.col[j] + 2], o.w = xs[mx.row[j]][mx.col[j] + 3] + vs[mx.col[j] + 3];
+                o.x = t4[0] + vs[mx.col[j]], o.y = t4[1] + vs[mx.col[j] + 1], o.z = t4[2] + vs[mx.col[j] + 2], o.w = t4[3] + vs[mx.col[j] + 3];
                 const float4 og = o;  // this contraction's own gradient: the one the rounding residue meets
                 if (has_add) {
                     o.x += adds[mx.row[j]][mx.col[j]], o.y += adds[mx.row[j]][mx.col[j] + 1];
@@ -1512,6 +1585,7 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
     }
     // ---- this workgroup's slice: S and m through LDS (wavefronts that share a Gram block add in a fixed order), then
     // dW = (m gm^T + 2 (S W) diag(gs)) / rows on the fp32 matrix instruction (both operands are arbitrary fp32)
+    DB_STAMP(2, 30);
     __syncthreads();
     float *Ss = &xs[0][0];
     for (int pass = 0; pass < gpb; ++pass) {
@@ -1519,8 +1593,8 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int k = gib * 32 + acc_row(r, lane), jx = gjb * 32 + l32;
-                if (pass == 0) Ss[k * FAST_LD + jx] = accS[r];
-                else Ss[k * FAST_LD + jx] += accS[r];
+                if (pass == 0) Ss[k * FAST_XLD + jx] = accS[r];
+                else Ss[k * FAST_XLD + jx] += accS[r];
             }
         }
         __syncthreads();
@@ -1530,18 +1604,33 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
     __syncthreads();
     if (tid < 64) vs[tid] = (bred[tid] + bred[tid + 64]) + (bred[tid + 128] + bred[tid + 192]);  // m (v is not needed any more)
     __syncthreads();
+    if (rep > 1) {
+        // S = sum of the diagonal blocks of S', m = sum of the segments of m', in block order, left in the first block
+        for (int id = tid; id < Ko * Ko; id += 256) {
+            const int i = id / Ko, jx = id % Ko;
+            float sacc = Ss[i * FAST_XLD + jx];
+            for (int q = 1; q < rep; ++q) sacc += Ss[(q * Ko + i) * FAST_XLD + q * Ko + jx];
+            Ss[i * FAST_XLD + jx] = sacc;
+        }
+        float macc = 0.f;
+        if (tid < Ko)
+            for (int q = 0; q < rep; ++q) macc += vs[q * Ko + tid];
+        __syncthreads();
+        if (tid < Ko) vs[tid] = macc;
+        __syncthreads();
+    }
     {
-        const int nb2 = K32 * N32;
+        const int nb2 = Ko32 * N32;
         if (wave < nb2) {
             const int wkb = wave / N32, wnb = wave % N32;
             floatx16 t = {0};
-            t = mfma_chain(t, &Ss[(wkb * 32 + l32) * FAST_LD + kq], 1, &ws[kq][wnb * 32 + l32], FAST_LD, K32 * 2);
+            t = mfma_chain(t, &Ss[(wkb * 32 + l32) * FAST_XLD + kq], 1, &ws[kq][wnb * 32 + l32], FAST_LD, Ko32 * 2);
             const int c = wnb * 32 + l32;
             const float g1 = gms[c], g2 = gss[c];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int k = wkb * 32 + acc_row(r, lane);
-                if (k < K && c < N) my_dw[k * N + c] = (vs[k] * g1 + 2.0f * g2 * t[r]) * inv_rows;
+                if (k < Ko && c < N) my_dw[k * N + c] = (vs[k] * g1 + 2.0f * g2 * t[r]) * inv_rows;
             }
         }
     }
@@ -1558,7 +1647,7 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
                 for (int e = 0; e < 4; ++e) gt[mx.row[j] * FAST_LD + mx.col[j] + e] = gf[j][e];
         __syncthreads();
         if (P <= 16) {
-            float *quarter = &As[0][0];
+            float *quarter = &ws[0][0];  // (W has been used)
             for (int id = tid; id < 4 * P * 64; id += 256) {
                 const int c = id & 63, pq = id >> 6, p = pq & (P - 1), q = pq / P;
                 float sacc = 0.f;
@@ -1583,6 +1672,7 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bwd_gram_kernel(const fl
             }
         }
     }
+    DB_STAMP(2, 31);
 }
 
 // out[e] = sum over slices of part[g][e], in slice order.  256 threads = 64 elements x 4 slice groups.
@@ -1719,7 +1809,7 @@ using namespace hgq;
 
 #ifdef DB_PROF
 extern "C" int hgq_db_prof_read(unsigned long long *out) {
-    return hipMemcpyFromSymbol(out, HIP_SYMBOL(db_prof_stamps), sizeof(unsigned long long) * 2 * 4 * 32) == hipSuccess ? 0 : -2;
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(db_prof_stamps), sizeof(unsigned long long) * 3 * 4 * 32) == hipSuccess ? 0 : -2;
 }
 #endif
 
@@ -1925,9 +2015,12 @@ extern "C" int hgq_qdense_moments_bwd(const float *x, const float *f_in, int64_t
     const int P = quant ? (int)bw_rows : 1;
     const int rm = Mode(mode).round_mode;
     const dim3 grid((unsigned)parts);
+    // a narrow input as rows of 64: rep rows side by side (the table of fractional bits folds the same way)
+    int rep = 1;
+    if (g_dense_bf16 && (K == 8 || K == 16 || K == 32) && rows % (64 / K) == 0 && (!quant || bw_rows % (64 / K) == 0)) rep = 64 / K;
 #define HGQ_MOM_BWD(RMV, QV) \
     do { \
-        if (g_dense_bf16) hipLaunchKernelGGL((dense_moments_bwd_gram_kernel<RMV, QV>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, rows, K, N, mode, dx_add); \
+        if (g_dense_bf16) hipLaunchKernelGGL((dense_moments_bwd_gram_kernel<RMV, QV>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, quant ? P / rep : 1, w, dx, workspace, rows / rep, K * rep, N, mode, dx_add, rep); \
         else hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, true>), grid, dim3(256), 0, s, dmean, dmeansq, x, f_in, P, w, dx, workspace, 0, rows, K, N, HGQ_ACT_NONE, mode, dx_add); \
     } while (0)
     if (!quant) HGQ_MOM_BWD(HGQ_TRN, false);

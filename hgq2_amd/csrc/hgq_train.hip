@@ -451,7 +451,11 @@ __global__ void ebops_finish_bwd_kernel(const float *g, const float *beta, float
 }
 
 // one thread per row; C is small (class count)
-// `state` = {running sum (float), finished workgroups}: both zero at the start and left zero at the end
+// `state` = {sum (64-bit fixed point, two words), finished workgroups, a workgroup's sum was not finite}: all zero at the
+// start and left zero at the end.  The workgroups' sums meet as INTEGERS (2^-40 units): integer addition does not depend on
+// the order in which they arrive, so the loss is the same in every run and in every replay of a recorded step (a float
+// atomic would round differently with every arrival order).  state == NULL: a single workgroup, no meeting at all.
+#define CE_FIX 1099511627776.0f  // 2^40: a sum of up to 2^22 in magnitude keeps 2^-40 resolution in 63 bits
 __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict__ logits,
                                                         const int64_t *__restrict__ labels, float *loss,
                                                         float *__restrict__ dlogits, int64_t rows, int C, uint32_t *state) {
@@ -477,21 +481,28 @@ __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict_
     }
     acc = block_sum_256(acc, red);
     if (threadIdx.x == 0) {
+        const float part = acc * inv_rows;
         if (!state) {
-            atomicAdd(loss, acc * inv_rows);
+            loss[0] = part;  // (launched as one workgroup)
             return;
         }
-        // Both words are only ever touched by device-scope atomics, which are performed where all workgroups meet (not
+        // All four words are only ever touched by device-scope atomics, which are performed where all workgroups meet (not
         // in a cache that would need a write-back).  The ticket is drawn with an operand that depends on the value the
-        // first atomic RETURNS, so it cannot leave this wavefront before this workgroup's part has been added: whoever
+        // sum's atomic RETURNS, so it cannot leave this wavefront before this workgroup's part has been added: whoever
         // draws the last ticket finds every part in the sum.  (A fence of workgroup scope between two non-returning
         // atomics orders nothing for other workgroups; one of device scope costs a cache write-back, ~2 us here.)
-        const float before = atomicAdd((float *)state, acc * inv_rows);
+        const bool finite = fabsf(part) < 4194304.0f;  // (false for NaN too)
+        unsigned long long *sum = (unsigned long long *)state;
+        unsigned long long before = atomicAdd(sum, finite ? (unsigned long long)(long long)rintf(part * CE_FIX) : 0ull);
+        if (!finite) before += atomicOr(state + 3, 1u);
         uint32_t one = 1u;
-        asm volatile("" : "+v"(one) : "v"(before));
-        if (atomicAdd(state + 1, one) == gridDim.x - 1) {
-            loss[0] = __uint_as_float(atomicExch(state, 0u));  // every other workgroup has added its part
-            atomicExch(state + 1, 0u);
+        asm volatile("" : "+v"(one) : "v"((uint32_t)before));
+        if (atomicAdd(state + 2, one) == gridDim.x - 1) {
+            // every other workgroup has added its part
+            const long long total = (long long)atomicExch(sum, 0ull);
+            const uint32_t bad = atomicExch(state + 3, 0u);
+            loss[0] = bad ? NAN : (float)((double)total * (1.0 / (double)CE_FIX));
+            atomicExch(state + 2, 0u);
         }
     }
 }
@@ -739,11 +750,8 @@ extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels,
     if (rows < 1 || C < 1) return fail(HGQ_ERR_ARG, "hgq_sparse_ce_fwd_bwd: bad sizes");
     if (!logits || !labels || !loss) return fail(HGQ_ERR_ARG, "hgq_sparse_ce_fwd_bwd: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    if (!state) {
-        int rc = fill_f32(loss, 0.0f, 1, s);
-        if (rc) return rc;
-    }
-    const int grid = persistent_grid((rows + 255) / 256, 4);
+    if (state && ((uintptr_t)state & 7u)) return fail(HGQ_ERR_ARG, "hgq_sparse_ce_fwd_bwd: state must be 8-byte aligned");
+    const int grid = state ? persistent_grid((rows + 255) / 256, 4) : 1;
     hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C, state);
     return check_launch("hgq_sparse_ce_fwd_bwd");
 }

@@ -711,12 +711,12 @@ def sparse_ce_op(logits: Tensor, labels: Tensor) -> tuple[Tensor, Tensor]:
     _need(labels.dtype == torch.int64 and labels.is_cuda and labels.is_contiguous(), 'labels must be a contiguous int64 GPU tensor')
     loss = torch.empty((), dtype=torch.float32, device=logits.device)
     dlogits = torch.empty_like(logits)
-    # two words per (device, stream), zeroed once: the kernel leaves them zero, so no call clears anything
+    # four words per (device, stream), zeroed once: the kernel leaves them zero, so no call clears anything
     stream = _stream()
     key = (logits.device, stream.value if hasattr(stream, 'value') else stream)
     state = _CE_STATE.get(key)
     if state is None:
-        state = _CE_STATE[key] = torch.zeros(2, dtype=torch.int32, device=logits.device)
+        state = _CE_STATE[key] = torch.zeros(4, dtype=torch.int32, device=logits.device)
     rc = _lib.load().hgq_sparse_ce_fwd_bwd(_ptr(logits), _ptr(labels), _ptr(loss), _ptr(dlogits), logits.shape[0],
                                            logits.shape[1], _ptr(state), stream)
     _lib.check(rc, 'hgq_sparse_ce_fwd_bwd')

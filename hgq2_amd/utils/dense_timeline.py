@@ -1,9 +1,9 @@
 """Time line of the streaming dense kernels' wavefronts (a measurement aid, not part of any compute path).
 
-``make -C hgq2_amd/csrc prof`` builds ``libhgq_hip_prof.so``, in which workgroup 0 of ``qdense_fwd_bf16_kernel`` and of
-``qdense_bwd_fast_kernel`` stamps the constant-rate counter (10 ns ticks) at its phase boundaries, one row of stamps per
-wavefront.  ``python -m hgq2_amd.utils.dense_timeline [rows K N]`` loads that build in place of the product library, runs
-``hgq_qdense_fwd`` and ``hgq_qdense_bwd`` on synthetic operands (a per-column input quantizer, an 8-bit kernel, default
+``make -C hgq2_amd/csrc prof`` builds ``libhgq_hip_prof.so``, in which workgroup 0 of ``qdense_fwd_bf16_kernel``, of
+``qdense_bwd_fast_kernel`` and of ``dense_moments_bwd_gram_kernel`` stamps the constant-rate counter (10 ns ticks) at its phase
+boundaries, one row of stamps per wavefront.  ``python -m hgq2_amd.utils.dense_timeline [rows K N]`` loads that build in place
+of the product library, runs ``hgq_qdense_fwd``, ``hgq_qdense_bwd`` and ``hgq_qdense_moments_bwd`` on synthetic operands (a per-column input quantizer, an 8-bit kernel, default
 131072 x 64 x 64: a projection of the attention configuration) and prints the median time of every stamp since the
 workgroup started, for the first wavefront of each kernel."""
 
@@ -37,6 +37,7 @@ def main(argv=None):
     amax = torch.empty(lib.hgq_qdense_fwd_parts(rows) * K, dtype=torch.int32, device=dev)
     ws = torch.empty(lib.hgq_qdense_bwd_workspace(rows, K, N, 1), dtype=torch.float32, device=dev)
     dqw, dqb, df = torch.empty(K, N, device=dev), torch.empty(N, device=dev), torch.empty(K, device=dev)
+    gm, gsq, dy_in = torch.randn(N, generator=g).to(dev), torch.randn(N, generator=g).to(dev), torch.randn(rows, K, generator=g).to(dev)
 
     def run():
         rc = lib.hgq_qdense_fwd(x.data_ptr(), k_in.data_ptr(), i_in.data_ptr(), f_in.data_ptr(), 1, w.data_ptr(), None, y.data_ptr(),
@@ -45,11 +46,14 @@ def main(argv=None):
         rc = lib.hgq_qdense_bwd(dy.data_ptr(), None, x.data_ptr(), f_in.data_ptr(), 1, w.data_ptr(), dx.data_ptr(), dqw.data_ptr(),
                                 dqb.data_ptr(), df.data_ptr(), ws.data_ptr(), rows, K, N, 0, mode, None)
         _lib.check(rc, 'hgq_qdense_bwd')
+        rc = lib.hgq_qdense_moments_bwd(x.data_ptr(), f_in.data_ptr(), 1, mode, w.data_ptr(), gm.data_ptr(), gsq.data_ptr(), dy_in.data_ptr(),
+                                        dx.data_ptr(), dqw.data_ptr(), df.data_ptr(), ws.data_ptr(), rows, K, N, None)
+        _lib.check(rc, 'hgq_qdense_moments_bwd')
 
     for _ in range(3):
         run()
     torch.cuda.synchronize()
-    buf = (ctypes.c_ulonglong * 256)()
+    buf = (ctypes.c_ulonglong * 384)()
     runs = []
     for _ in range(9):
         run()
@@ -59,18 +63,21 @@ def main(argv=None):
         runs.append(list(buf))
     fwd = {0: 'start', 1: 'kernel matrix, bit-widths, LDS cleared, first tile in', 30: 'tiles done', 31: 'end'}
     bwd = dict(fwd)
+    stats = {0: 'start', 1: 'kernel matrix, A and v, bit-widths, first tile in', 30: 'tiles done', 31: 'end'}
     for it in range(4):
         fwd.update({2 + 6 * it: f'tile {it} staged', 3 + 6 * it: f'tile {it} |barrier', 4 + 6 * it: f'tile {it} matrix instructions',
                     5 + 6 * it: f'tile {it} result in LDS', 6 + 6 * it: f'tile {it} |barrier'})
         bwd.update({2 + 6 * it: f'tile {it} top |barrier', 3 + 6 * it: f'tile {it} staged', 4 + 6 * it: f'tile {it} |barrier',
                     5 + 6 * it: f'tile {it} matrix instructions', 6 + 6 * it: f'tile {it} |barrier', 7 + 6 * it: f'tile {it} dx in LDS |barrier'})
+        stats.update({2 + 6 * it: f'tile {it} top |barrier', 3 + 6 * it: f'tile {it} staged', 4 + 6 * it: f'tile {it} |barrier',
+                      5 + 6 * it: f'tile {it} matrix instructions', 6 + 6 * it: f'tile {it} |barrier', 7 + 6 * it: f'tile {it} dx in LDS |barrier'})
     print(f'rows {rows}, K {K}, N {N}; microseconds since the start of workgroup 0, wavefront 0')
-    for kernel, names in (('forward', fwd), ('backward', bwd)):
-        base = 0 if kernel == 'forward' else 4 * 32
+    for kernel, names in (('forward', fwd), ('backward', bwd), ('statistics', stats)):
+        base = {'forward': 0, 'backward': 4 * 32, 'statistics': 8 * 32}[kernel]
         for k in sorted(names):
             vals = [r[base + k] - r[base] for r in runs if 0 <= r[base + k] - r[base] < 10_000_000]
             if vals and (k == 0 or statistics.median(vals) > 0):
-                print(f'  {kernel:8s} {names[k]:55s} {statistics.median(vals) / 100:8.2f}')
+                print(f'  {kernel:10s} {names[k]:55s} {statistics.median(vals) / 100:8.2f}')
 
 
 if __name__ == '__main__':

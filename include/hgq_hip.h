@@ -421,9 +421,11 @@ int hgq_mse_fwd_bwd(const float *pred, const float *target, float *loss, float *
  * Mean sparse categorical cross-entropy from logits, forward and gradient in one pass.
  *   logits [rows, C]; labels [rows] int64;  loss [1] = mean_r(-log softmax(logits_r)[label_r]);
  *   dlogits [rows, C] = (softmax - onehot) / rows.
- *   state: NULL, or two 32-bit words that are zero when the call starts; the kernel leaves them zero again (the
+ *   state: four 32-bit words, 8-byte aligned, that are zero when the call starts; the kernel leaves them zero again (the
  *   workgroup that finishes last takes the sum out and clears them), so one allocation zeroed once serves every later
- *   call and the launch that would clear `loss` is saved.  Calls that overlap in time need separate words.
+ *   call and no launch clears anything.  The workgroups' sums meet as 64-bit fixed-point integers, so the loss does not
+ *   depend on the order in which they arrive: every run and every replay of a recorded step gives the same bits.  Calls
+ *   that overlap in time need separate words.  NULL: one workgroup computes the whole sum (slower for many rows).
  */
 int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *loss, float *dlogits, int64_t rows,
                           int C, uint32_t *state, void *stream);
