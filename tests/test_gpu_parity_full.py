@@ -602,8 +602,8 @@ def test_device_side_draw_counter_gives_the_host_counters_offsets(dev):
 
 def test_stochastic_rounding_in_a_replayed_graph_draws_anew(dev):
     """A training step with S_RND data quantizers recorded into a HIP graph: every replay draws as the same step run
-    eagerly would - variables after N replays equal those of N eager steps of a twin model, bit for bit - and two
-    replays on the same batch do not repeat each other's draw."""
+    eagerly would - the losses of N replays are those of the same N eager steps of a twin model - and two replays on the
+    same batch do not repeat each other's draw."""
     import numpy as np
 
     from hgq2_amd import ops
@@ -643,5 +643,7 @@ def test_stochastic_rounding_in_a_replayed_graph_draws_anew(dev):
             opt_b.step()
         want.append(loss.item())
     torch.cuda.synchronize()
-    assert losses == want[warmup:], (losses, want)
+    # (the shared bit-widths' gradients of the stochastic kernels are added with float atomics: the trajectories agree to
+    # rounding, not to the bit; a replay that repeated a draw would be off by the rounding noise itself, ~1e-3)
+    assert all(abs(a - b) <= 1e-5 * abs(b) for a, b in zip(losses, want[warmup:])), (losses, want)
     assert len(set(losses)) > 1
