@@ -768,7 +768,9 @@ def test_batch_normalization_layer(shape, axis, center, scale):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('rows,K,N,bw_rows', [(4096, 16, 64, 64), (640, 64, 32, 16), (70 * 64, 64, 64, 1)])
+@pytest.mark.parametrize('rows,K,N,bw_rows', [(4096, 16, 64, 64), (640, 64, 32, 16), (70 * 64, 64, 64, 1),
+                                              # narrow inputs: rows staged side by side (8, 2 and 4 of them), and the same widths where they are not
+                                              (512, 8, 16, 8), (320, 32, 20, 64), (1024, 16, 8, 4), (300, 16, 8, 1), (96, 32, 64, 1), (66, 8, 4, 2)])
 def test_dense_moments_with_the_input_quantizer_inside(rows, K, N, bw_rows):
     """ops.dense_moments(x, w, quant): column moments of q(x) @ w with q a training-mode WRAP quantizer applied while
     the operand is staged, against fp64 on the separately quantized input: moments, dx (straight-through), dw and the
@@ -800,7 +802,7 @@ def test_dense_moments_with_the_input_quantizer_inside(rows, K, N, bw_rows):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('rows,K,N,bw_rows', [(640, 16, 64, 64), (200, 64, 32, 0), (131, 20, 12, 1)])
+@pytest.mark.parametrize('rows,K,N,bw_rows', [(640, 16, 64, 64), (200, 64, 32, 0), (131, 20, 12, 1), (256, 8, 32, 0), (130, 32, 16, 2), (129, 16, 16, 0)])
 def test_dense_moments_chained_input_gradient(rows, K, N, bw_rows):
     """``chain=True``: the third result stands for x in a second consumer, whose gradient is added while the
     statistics' backward writes dx - equal to the unchained gradient plus that of the second consumer; the
