@@ -286,3 +286,21 @@ def test_matrix_instruction_choice_from_the_environment():
         out = subprocess.run([sys.executable, '-c', code], cwd=root, env=env, capture_output=True, text=True, timeout=120)
         assert out.returncode == 0, out.stderr
         assert out.stdout.strip().splitlines()[-1] == want, (value, out.stdout)
+
+
+def test_fit_checks_its_arguments_and_seed_generators_count_on_the_host():
+    """Host logic only: `train.fit` refuses CPU tensors (the product has no CPU path) and mismatched sample counts before
+    anything is built; a seed generator used without a device keeps the host counter 1, 2, 3, ... and never creates the
+    device-side one."""
+    from hgq2_amd.quantizer.fixed_point_ops import SeedGenerator
+    from hgq2_amd.train import fit
+
+    x, y = torch.zeros(8, 4), torch.zeros(8, dtype=torch.int64)
+    with pytest.raises(ValueError, match='GPU'):
+        fit(object(), x, y)
+    with pytest.raises(ValueError, match='same'):
+        fit(object(), x, y[:5])
+    gen = SeedGenerator(9)
+    assert [gen.next() for _ in range(3)] == [(9, 1), (9, 2), (9, 3)]
+    assert gen._base is None and gen.offset == 3
+    assert gen.next(torch.device('cpu')) == (9, 4)
