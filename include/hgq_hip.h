@@ -426,6 +426,7 @@ int hgq_mse_fwd_bwd(const float *pred, const float *target, float *loss, float *
  *   call and no launch clears anything.  The workgroups' sums meet as 64-bit fixed-point integers, so the loss does not
  *   depend on the order in which they arrive: every run and every replay of a recorded step gives the same bits.  Calls
  *   that overlap in time need separate words.  NULL: one workgroup computes the whole sum (slower for many rows).
+ *   A workgroup's share of the mean beyond 2^22 in magnitude (or not finite) makes the loss NaN.
  */
 int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *loss, float *dlogits, int64_t rows,
                           int C, uint32_t *state, void *stream);
