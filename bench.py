@@ -547,6 +547,27 @@ def main():
             el_p, _ = time_steps(make_step(path), n_steps, max(args.warmup, 10))
             paths[path.replace('-', '_')] = {'samples_per_s': BATCH * n_steps / el_p, 'ms_per_step': el_p / n_steps * 1e3, 'steps': n_steps,
                                              'what': labels_of[path]}
+        # the epoch loop a user writes (hgq2_amd.train.fit: batches sliced from a resident data set, callbacks, the loss read
+        # once per epoch), on the path it picks by itself and with the whole-step kernels switched off
+        from hgq2_amd.train import fit
+        n_batches = 64
+        gx = torch.Generator().manual_seed(3)
+        data_x = torch.randn(BATCH * n_batches, DIMS[0], generator=gx).to(dev)
+        data_y = torch.randint(0, DIMS[-1], (BATCH * n_batches,), generator=gx).to(dev)
+        for name, fused in (('fit_loop', None), ('fit_loop_layers', False)):
+            torch.manual_seed(1)
+            model = qdense_mlp(DIMS, beta0=1e-5, device=dev)
+            fit(model, data_x, data_y, lr=0.01, batch_size=BATCH, epochs=1, shuffle=False, fused=fused)  # records / warms up
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            n_epochs = 20
+            hist = fit(model, data_x, data_y, lr=0.01, batch_size=BATCH, epochs=n_epochs, shuffle=False, fused=fused)
+            torch.cuda.synchronize()
+            el_f = time.perf_counter() - t0
+            paths[name] = {'samples_per_s': BATCH * n_batches * n_epochs / el_f, 'ms_per_step': el_f / (n_epochs * n_batches) * 1e3,
+                           'steps': n_epochs * n_batches, 'final_epoch_loss': hist[-1]['loss'],
+                           'what': 'train.fit over 64 resident batches x 20 epochs, the recording of its step included, '
+                                   + ('path chosen by fit' if fused is None else 'per-layer operators replayed from a HIP graph')}
         out['paths'] = paths
 
     qr = quantizer_roofline()
