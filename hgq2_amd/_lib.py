@@ -54,6 +54,11 @@ SIGNATURES = {
     'hgq_qdense_fwd_oq': (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64] + [c_void_p] * 4
                           + [c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     'hgq_qdense_bwd': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 6 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    'hgq_qdense_fwd_mean_supported': (c_int, [c_int64, c_int, c_int, c_int64, c_int64, c_int]),
+    'hgq_qdense_fwd_mean': (c_int, [c_void_p, c_void_p, c_int64] + [c_void_p] * 5 + [c_int64, c_int, c_int, c_int64, c_int, c_int, c_void_p]),
+    'hgq_qdense_bwd_mean': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 6 + [c_int64, c_int, c_int, c_int64, c_int, c_int, c_void_p]),
+    'hgq_qdense_bwd_mean_slices': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 3 + [c_int, c_int64, c_int, c_int, c_int64, c_int, c_int,
+                                           c_void_p]),
     'hgq_dense_ebops': (
         c_int,
         [c_void_p, c_int, c_float, c_void_p, c_void_p] + [c_void_p] * 3 + [c_int64, c_int, c_int] + [c_void_p] * 4

@@ -641,6 +641,9 @@ __device__ __forceinline__ floatx16 bf16_chain(floatx16 acc, bf16_planes_t xp, i
 // OQ: the layer's output quantizer (training-mode WRAP: round only, [Po, N] table of fractional bits, same round mode)
 // runs on the output tile as it leaves: `y` gets the contraction, `yq` its quantized values, slice blockIdx.x of
 // `oamax_part` the abs-max of the quantized values per table entry.
+// ymean (mean_rows = 32 or 64, rows a multiple of it, 128-bit output rows): row g of `ymean` [rows / mean_rows, N] = the
+// mean of the activated output rows g * mean_rows .. (g + 1) * mean_rows - 1, taken from the accumulator registers as the
+// tile leaves (a tile holds two groups or one): sixteen rows per lane in order, the two lane halves, then the two row halves.
 template <int RM, bool QUANT, int NS, bool OQ = false>
 __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw,
@@ -648,10 +651,12 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
                                                               uint32_t *amax_part, int64_t rows, int K, int N, int act,
                                                               int mode, const float *__restrict__ f_out = nullptr, int Po = 1,
                                                               int mode_out = 0, float *__restrict__ yq = nullptr,
-                                                              uint32_t *oamax_part = nullptr) {
+                                                              uint32_t *oamax_part = nullptr, float *__restrict__ ymean = nullptr,
+                                                              int mean_rows = 0) {
     // [buffer][part][row][k]; row FAST_BM: sink of the idle staging slots
     __shared__ __attribute__((aligned(16))) uint16_t xp[2][3][FAST_BM + 1][BF_LD];
     __shared__ __attribute__((aligned(16))) float ys[FAST_BM][FAST_XLD];
+    __shared__ float msum[2][64];  // ymean: column sums of the two row halves of the tile
     // bit 0 / 1: the staged tile has a non-zero second / third part.  Three slots in rotation: the slot of the tile after
     // next is cleared behind this tile's barrier - its last readers passed that barrier, its next writers come after the next one
     __shared__ uint32_t need[3];
@@ -743,15 +748,30 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         DB_STAMP(0, 4 + 6 * it_);
         const int64_t r0 = tile * FAST_BM;
         if (vec_out) {
+            float csum = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 float v = acc[r] + bias;
                 if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
                 ys[rh * 32 + acc_row(r, lane)][bcol] = v;
+                csum += v;
+            }
+            if (ymean) {
+                csum += __shfl_xor(csum, 32);
+                if (lane < 32) msum[rh][bcol] = csum;
             }
             DB_STAMP(0, 5 + 6 * it_);
             __syncthreads();
             DB_STAMP(0, 6 + 6 * it_);
+            // (the next tile's sums are written behind its staging barrier, which these reads precede)
+            if (ymean && tid < 2 * 64) {
+                const int c = tid & 63, h = tid >> 6;
+                if (mean_rows == FAST_BM) {
+                    if (h == 0 && c < N) ymean[tile * N + c] = (msum[0][c] + msum[1][c]) * (1.0f / FAST_BM);
+                } else if (c < N && r0 + h * 32 < rows) {
+                    ymean[(2 * tile + h) * N + c] = msum[h][c] * (1.0f / 32);
+                }
+            }
 #pragma unroll
             for (int j = 0; j < FAST_NJ; ++j) {
                 const int64_t gr = r0 + mo.row[j];
@@ -998,16 +1018,20 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bf16_kernel(const float 
 // recomputed on the matrix cores (dy = gm, y = gs, both [N]); no activation, no bias, no quantizer.
 // BF: the three contractions run on the bf16 matrix cores by exact splitting (mfma_chain_bf16); the gradient operand is
 // taken in all three parts without looking, the quantized input and the kernel in as many as they need.
+// BCAST (32 or 64, not with STATS, ZVEC only, rows a multiple of it; `bcast` below): the output went through a mean over groups of `bcast` rows
+// and dy is the gradient of those means, [rows / bcast, N]: row r of the gradient tile is dy[r / bcast] / bcast, read with a
+// zero row stride instead of from a broadcast copy.
 // PAIRS (with BF; K and N above 32): wavefronts 0 and 1 take the two row halves of dx (both k blocks: the gradient rows they
 // contract are split into bf16 parts once for both), wavefronts 2 and 3 the two column halves of the kernel gradient (both k
 // blocks, all rows of the tile) - every gradient value is split twice per tile instead of four times.  A wavefront's two
 // blocks live in the same registers either way: reset per tile for dx, kept across the tiles for the kernel gradient.
-template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true, bool BF = false, bool PAIRS = false>
+template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true, bool BF = false, bool PAIRS = false, int BCAST = 0>
 __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
                                                               float *part, int has_bias, int64_t rows, int K, int N, int act,
                                                               int mode, const float *__restrict__ dx_add) {
+    constexpr int bcast = BCAST;
     __shared__ float xs[FAST_BM + 1][FAST_LD];   // row FAST_BM: sink of the idle staging slots
     __shared__ float dzs[FAST_BM + 1][FAST_LD];  // dz, then the dx tile
     __shared__ float ws[64][FAST_LD];
@@ -1060,14 +1084,18 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         const int64_t r0 = t * FAST_BM, left = rows - r0, vr = left < FAST_BM ? left : FAST_BM;
         const __amdgpu_buffer_rsrc_t sx = buf_rsrc(x + r0 * K, vr * K * 4);
         const __amdgpu_buffer_rsrc_t sg = STATS ? buf_rsrc(has_add ? dx_add + r0 * K : x, has_add ? vr * K * 4 : 0)
-                                                : buf_rsrc(dy + r0 * N, vr * N * 4);
+                                          : bcast ? buf_rsrc(dy + (r0 / bcast) * N, ((vr + bcast - 1) / bcast) * N * 4)
+                                                  : buf_rsrc(dy + r0 * N, vr * N * 4);
         const __amdgpu_buffer_rsrc_t sy = buf_rsrc((relu && !STATS) ? y + r0 * N : x, (relu && !STATS) ? vr * N * 4 : 0);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
             rx[j] = buf_ld4(sx, xoff[j]);
             if (!STATS) {
                 if (ZVEC) {
-                    rg[j] = buf_ld4(sg, zoff[j]);
+                    // bcast: every row of a group reads the group's one gradient row
+                    const uint32_t goff = !bcast ? zoff[j]
+                                          : mz.on[j] ? (uint32_t)((bcast == 32 ? (mz.row[j] >> 5) : 0) * N + mz.col[j]) * 4u : BUF_OOB;
+                    rg[j] = buf_ld4(sg, goff);
                     ry[j] = buf_ld4(sy, zoff[j]);
                 } else {
 #pragma unroll
@@ -1083,6 +1111,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         }
     };
     const float inv_rows = 1.0f / (float)rows;
+    const float gscale = bcast ? 1.0f / (float)bcast : 1.0f;
     // Start-up: the first tile is asked for first, then the kernel matrix and the fractional bits - one round trip for the
     // three of them instead of three in a row (a launch of one or two tiles per workgroup is mostly start-up).
     if (tile < n_tiles) load_tile(tile);
@@ -1137,7 +1166,7 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                 const float g[4] = {rg[j][0], rg[j][1], rg[j][2], rg[j][3]};
                 const float a[4] = {ry[j][0], ry[j][1], ry[j][2], ry[j][3]};
 #pragma unroll
-                for (int e = 0; e < 4; ++e) dzs[zr][mz.col[j] + e] = (!relu || a[e] > 0.f) ? g[e] : 0.f;
+                for (int e = 0; e < 4; ++e) dzs[zr][mz.col[j] + e] = (!relu || a[e] > 0.f) ? g[e] * gscale : 0.f;
             }
         }
         DB_STAMP(1, 3 + 6 * it_);
@@ -1931,6 +1960,46 @@ extern "C" int hgq_qdense_fwd_oq(const float *x, const float *f_in, int64_t bw_r
     return check_launch("hgq_qdense_fwd_oq");
 }
 
+// 1 if hgq_qdense_fwd_mean covers the shape and mode
+extern "C" int hgq_qdense_fwd_mean_supported(int64_t rows, int K, int N, int64_t bw_rows, int64_t mean_rows, int mode) {
+    const Mode m(mode);
+    const bool quant = bw_rows > 0;
+    const bool wrap_in = m.overflow_mode == HGQ_WRAP && m.training && !m.kbi;
+    return g_dense_bf16 && rows > 0 && K >= 1 && N >= 1 && K <= 64 && N <= 64 && K % 4 == 0 && N % 4 == 0 &&
+           (mean_rows == 32 || mean_rows == 64) && rows % mean_rows == 0 &&
+           (!quant || (wrap_in && (m.round_mode == HGQ_TRN || m.round_mode == HGQ_RND || m.round_mode == HGQ_RND_CONV) && bw_rows <= 64 &&
+                       64 % bw_rows == 0 && rows % bw_rows == 0));
+}
+
+extern "C" int hgq_qdense_fwd_mean(const float *x, const float *f_in, int64_t bw_rows, const float *qw, const float *qb, float *y,
+                                   float *ymean, uint32_t *amax_part, int64_t rows, int K, int N, int64_t mean_rows, int act, int mode,
+                                   void *stream) {
+    hipStream_t s = (hipStream_t)stream;
+    if (rows == 0) return HGQ_OK;
+    if (bw_rows < 0 || !hgq_qdense_fwd_mean_supported(rows, K, N, bw_rows, mean_rows, mode))
+        return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_fwd_mean: shape or mode outside the fused group mean (see hgq_qdense_fwd_mean_supported)");
+    if (!x || !qw || !y || !ymean || (bw_rows > 0 && !f_in)) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: null pointer");
+    if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: unknown activation %d", act);
+    if (!aligned16(x) || !aligned16(y)) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: x and y must be 16-byte aligned");
+    const Mode m(mode);
+    const bool quant = bw_rows > 0;
+    const dim3 fgrid((unsigned)row_parts(rows, FWD_BM));
+    const int P = quant ? (int)bw_rows : 1, mr = (int)mean_rows;
+#define HGQ_FWD_MEAN(NSV) \
+    do { \
+        if (!quant) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, false, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, (uint32_t *)nullptr, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
+        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
+        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
+        else hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND_CONV, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
+    } while (0)
+    if (K <= 16) HGQ_FWD_MEAN(1);
+    else if (K <= 32) HGQ_FWD_MEAN(2);
+    else if (K <= 48) HGQ_FWD_MEAN(3);
+    else HGQ_FWD_MEAN(4);
+#undef HGQ_FWD_MEAN
+    return check_launch("hgq_qdense_fwd_mean");
+}
+
 extern "C" int64_t hgq_qdense_moments_workspace(int64_t rows, int K, int N, int64_t bw_rows) {
     if (rows < 0 || K < 1 || N < 1 || bw_rows < 0) return -1;
     const int64_t parts = rows > 0 ? row_parts(rows, FAST_BM) : 1;
@@ -2042,8 +2111,11 @@ extern "C" int hgq_dense_moments_bwd(const float *x, const float *w, const float
 // Launches the backward kernel; the slices are reduced here (reduce == true) or left in the workspace for the caller.
 static int qdense_bwd_impl(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows, const float *qw, float *dx,
                            float *dqw, float *dqb, float *df_in, float *workspace, int64_t rows, int K, int N, int act, int mode,
-                           void *stream, bool reduce) {
+                           void *stream, bool reduce, int64_t mean_rows = 0) {
     hipStream_t s = (hipStream_t)stream;
+    if (mean_rows != 0 && mean_rows != 32 && mean_rows != 64) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_bwd_mean: groups of 32 or 64 rows only");
+    if (mean_rows && rows % mean_rows != 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd_mean: rows=%lld not a multiple of mean_rows=%lld", (long long)rows, (long long)mean_rows);
+    const int bcast = (int)mean_rows;
     if (rows < 0 || K < 1 || N < 1 || bw_rows < 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: bad sizes");
     if (K > 64 || N > 64) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_bwd: K=%d N=%d exceed the fused kernel's 64 x 64", K, N);
     if (!dy || !x || !qw || !dx || !workspace) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd: null pointer");
@@ -2071,6 +2143,24 @@ static int qdense_bwd_impl(const float *dy, const float *y, const float *x, cons
         const int P = quant ? (int)bw_rows : 1;
         const dim3 fgrid((unsigned)parts);
         const bool zvec = N % 4 == 0 && aligned16(dy) && (act != HGQ_ACT_RELU || aligned16(y));
+        if (bcast && !(zvec && g_dense_bf16))
+            return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_bwd_mean: needs the bf16 matrix instruction, N a multiple of 4 and 16-byte aligned gradients");
+#define HGQ_BWD_BCAST(RMV, QV, BC)                                                                                                     \
+    do {                                                                                                                               \
+        if (K > 32 && N > 32)                                                                                                          \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true, true, true, BC>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, \
+                               workspace, dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                 \
+        else                                                                                                                           \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true, true, false, BC>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, \
+                               workspace, dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                 \
+    } while (0)
+#define HGQ_BWD_BCAST_RM(BC)                                                                                                           \
+    do {                                                                                                                               \
+        if (!quant) HGQ_BWD_BCAST(HGQ_TRN, false, BC);                                                                                 \
+        else if (m.round_mode == HGQ_TRN) HGQ_BWD_BCAST(HGQ_TRN, true, BC);                                                            \
+        else if (m.round_mode == HGQ_RND) HGQ_BWD_BCAST(HGQ_RND, true, BC);                                                            \
+        else HGQ_BWD_BCAST(HGQ_RND_CONV, true, BC);                                                                                    \
+    } while (0)
 #define HGQ_BWD_FAST(RMV, QV)                                                                                                          \
     do {                                                                                                                               \
         if (zvec && g_dense_bf16 && K > 32 && N > 32)                                                                                  \
@@ -2089,15 +2179,20 @@ static int qdense_bwd_impl(const float *dy, const float *y, const float *x, cons
             hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, false>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
                                dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
     } while (0)
-        if (!quant) HGQ_BWD_FAST(HGQ_TRN, false);
+        if (bcast == 64) HGQ_BWD_BCAST_RM(64);
+        else if (bcast == 32) HGQ_BWD_BCAST_RM(32);
+        else if (!quant) HGQ_BWD_FAST(HGQ_TRN, false);
         else if (m.round_mode == HGQ_TRN) HGQ_BWD_FAST(HGQ_TRN, true);
         else if (m.round_mode == HGQ_RND) HGQ_BWD_FAST(HGQ_RND, true);
         else HGQ_BWD_FAST(HGQ_RND_CONV, true);
 #undef HGQ_BWD_FAST
+#undef HGQ_BWD_BCAST_RM
+#undef HGQ_BWD_BCAST
         int rc = check_launch("hgq_qdense_bwd");
         if (rc || !reduce) return rc;
         return reduce_parts(workspace, parts, M, dqw, (int64_t)K * N, dqb, (int64_t)N, quant ? df_in : (float *)nullptr, PK, s);
     }
+    if (bcast) return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_bwd_mean: K must be a multiple of 4 and x / dx 16-byte aligned");
     const int df_lds = (quant && PK <= DF_LDS_MAX) ? 1 : 0;
     const size_t dyn = df_lds ? (size_t)PK * 4 : 0;
     const int parts = row_parts(rows, BWD_BM);
@@ -2138,6 +2233,21 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
                               const float *qw, float *dx, float *dqw, float *dqb, float *df_in, float *workspace,
                               int64_t rows, int K, int N, int act, int mode, void *stream) {
     return qdense_bwd_impl(dy, y, x, f_in, bw_rows, qw, dx, dqw, dqb, df_in, workspace, rows, K, N, act, mode, stream, true);
+}
+
+extern "C" int hgq_qdense_bwd_mean(const float *dmean, const float *y, const float *x, const float *f_in, int64_t bw_rows, const float *qw,
+                                   float *dx, float *dqw, float *dqb, float *df_in, float *workspace, int64_t rows, int K, int N,
+                                   int64_t mean_rows, int act, int mode, void *stream) {
+    if (mean_rows <= 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd_mean: mean_rows must be positive");
+    return qdense_bwd_impl(dmean, y, x, f_in, bw_rows, qw, dx, dqw, dqb, df_in, workspace, rows, K, N, act, mode, stream, true, mean_rows);
+}
+
+extern "C" int hgq_qdense_bwd_mean_slices(const float *dmean, const float *y, const float *x, const float *f_in, int64_t bw_rows,
+                                          const float *qw, float *dx, float *workspace, int has_bias, int64_t rows, int K, int N,
+                                          int64_t mean_rows, int act, int mode, void *stream) {
+    if (mean_rows <= 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd_mean_slices: mean_rows must be positive");
+    return qdense_bwd_impl(dmean, y, x, f_in, bw_rows, qw, dx, nullptr, has_bias ? workspace : nullptr, nullptr, workspace, rows, K, N, act, mode,
+                           stream, false, mean_rows);
 }
 
 extern "C" int hgq_qdense_bwd_slices(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,

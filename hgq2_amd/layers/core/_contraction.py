@@ -112,6 +112,29 @@ def dense_contraction(x, iq, qkernel2d, qbias1d, act_name, training, oq=None, ou
     return y, act_code != _lib.ACT_NONE, None, False
 
 
+def dense_contraction_mean(x, iq, qkernel2d, qbias1d, act_name, training, mean_rows):
+    """``dense_contraction`` followed by a mean over groups of ``mean_rows`` consecutive rows, as one launch each way: returns
+    ``(means [rows / mean_rows, N], DeferredTracking or None)``, or ``None`` where the kernels do not cover the case (the caller
+    then contracts and averages in two steps).  The contraction's own output never leaves the operator."""
+    K, N = qkernel2d.shape
+    if act_name not in (None, 'linear', 'relu') or not x.is_cuda or x.numel() == 0:
+        return None
+    bw_rows = fused_iq_rows(iq, tuple(x.shape), K, training) if iq is not None else 0
+    if iq is not None and not bw_rows:
+        return None  # the quantizer runs as a launch of its own
+    q = iq.quantizer if bw_rows else None
+    mode = q._mode(True) if q is not None else 0
+    x2d = x.reshape(-1, K)
+    if not x2d.is_contiguous():
+        x2d = x2d.contiguous()
+    if not ops.qdense_mean_supported(x2d.shape[0], K, N, bw_rows, mean_rows, mode):
+        return None
+    act_code = _lib.ACT_RELU if act_name == 'relu' else _lib.ACT_NONE
+    ymean, amax = ops.qdense_mean(x2d, q._k.view(-1) if q is not None else None, q._f.view(-1) if q is not None else None, qkernel2d,
+                                  qbias1d, act_code, mode, bw_rows, mean_rows)
+    return ymean, (DeferredTracking(q, amax) if q is not None else None)
+
+
 def dense_ebops_term(layer, iq, kq, bq, K, N, bias_size, deferred):
     """``ebops * beta`` through the fused kernel (which also assigns the layer's ``_ebops`` and, when
     ``deferred`` tracking is pending and small enough, updates the input quantizer's ``_i`` first).

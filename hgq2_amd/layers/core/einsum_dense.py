@@ -17,7 +17,7 @@ from ... import _lib, ops
 from ...core import get_initializer
 from ...quantizer import Quantizer
 from ...quantizer.config import QuantizerConfig
-from ._contraction import dense_contraction, dense_ebops_term, get_activation
+from ._contraction import dense_contraction, dense_contraction_mean, dense_ebops_term, get_activation
 from .base import QLayerBaseSingleInput, mean_bits, scale_ebops
 
 
@@ -170,7 +170,29 @@ class QEinsumDense(QLayerBaseSingleInput):
     def compute_output_shape(self, input_shape):
         return (input_shape[0],) + tuple(self.full_output_shape[1:])
 
-    def _contract(self, inputs, qkernel, qbias, training, oq_ok=False):
+    def absorbs(self, nxt, x) -> bool:
+        """Whether a call may take the layer that follows in a :class:`Sequential` with it (``call(..., then=nxt)``): a mean
+        over the middle axis of a [batch, positions, channels] output (32 or 64 positions) behind a linear or ReLU contraction
+        over the trailing input axis, without output quantizer.  The contraction kernel then writes the means as its tiles leave,
+        and the backward pass reads the means' gradient instead of a broadcast copy."""
+        from ...host import GlobalAveragePooling1D
+
+        if type(nxt) is not GlobalAveragePooling1D or not getattr(type(self).call, '_takes_then', False) or not self.built:
+            return False
+        if self.enable_oq or self._act_name not in (None, 'linear', 'relu') or not torch.is_tensor(x) or not x.is_cuda or x.dim() != 3:
+            return False
+        out = tuple(self.full_output_shape)
+        return (self._gemm is not None and len(out) == 3 and out[-1] == self._N and x.shape[-1] == self._K and out[1] == x.shape[1]
+                and x.shape[1] in (32, 64) and (self.bias is None or self._bias_in_gemm))
+
+    def _contract(self, inputs, qkernel, qbias, training, oq_ok=False, mean_rows=0):
+        """``(outputs, activation applied)``; with ``mean_rows`` (a call that absorbed the mean over the middle axis)
+        ``(outputs, activation applied, mean taken)``."""
+        if mean_rows:
+            y, act_done, mean_done = self._contract_mean(inputs, qkernel, qbias, training, mean_rows)
+            if mean_done:
+                return y, act_done, True
+            return self._contract(inputs, qkernel, qbias, training, oq_ok) + (False,)
         iq = self.iq if self.enable_iq else None
         if self._gemm is not None:
             nc, _ = self._gemm
@@ -215,13 +237,40 @@ class QEinsumDense(QLayerBaseSingleInput):
             y = ops.bias_add_rows(y, qbias)
         return y, False
 
-    def call(self, inputs, training=None):
+    def _contract_mean(self, inputs, qkernel, qbias, training, mean_rows):
+        """The contraction and the mean over the middle axis in one launch each way where the kernels cover it:
+        ``(means, True, True)``, else ``(None, False, False)``."""
+        if self._gemm is None or (qbias is not None and not self._bias_in_gemm):
+            return None, False, False
+        w2d = qkernel.reshape(self._K, self._N)
+        b1d = qbias.reshape(-1) if qbias is not None else None
+        for view, base in ((w2d, qkernel), (b1d, qbias)):
+            if (view is not None and view is not base and getattr(base, '_hgq_single_use', False)
+                    and view._base is not None and view.data_ptr() == base.data_ptr() and view.numel() == base.numel()):
+                view._hgq_single_use = True  # the same elements under another shape
+        r = dense_contraction_mean(inputs, self.iq if self.enable_iq else None, w2d, b1d, self._act_name, training, mean_rows)
+        if r is None:
+            return None, False, False
+        y, self._deferred = r
+        return y, True, True
+
+    def _finish_then(self, y, act_done, mean_done, then):
+        """The tail of a call that absorbed the layer behind it: whatever the kernels did not take."""
+        if self.activation is not None and not act_done:
+            y = self.activation(y)
+        return y if mean_done else then(y)
+
+    def call(self, inputs, training=None, then=None):
         qkernel = self.kq(self._kernel, training=training)
         qbias = self.bq(self.bias, training=training) if self.bias is not None else None
+        if then is not None:
+            return self._finish_then(*self._contract(inputs, qkernel, qbias, training, mean_rows=inputs.shape[1]), then)
         y, act_done = self._contract(inputs, qkernel, qbias, training, oq_ok=True)
         if self.activation is not None and not act_done:
             y = self.activation(y)
         return y
+
+    call._takes_then = True
 
     def _finish_call(self):
         d, self._deferred = getattr(self, '_deferred', None), None

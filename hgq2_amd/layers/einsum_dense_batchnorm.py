@@ -154,7 +154,7 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         q = self.iq.quantizer
         return q._f.view(-1), bw_rows, q._mode(True)
 
-    def call(self, inputs, training=None):
+    def call(self, inputs, training=None, then=None):
         quant = self._fused_iq(inputs, training)
         if quant is None and self.enable_iq:
             inputs = self.iq(inputs, training=training)
@@ -192,9 +192,13 @@ class QEinsumDenseBatchnorm(QEinsumDense):
         # (and leaves the abs-max slices for the integer-bit update, as QEinsumDense does)
         enable_iq, self._enable_iq = self._enable_iq, quant is not None
         try:
+            if then is not None:  # the mean over the middle axis that follows, taken with the contraction where the kernels cover it
+                return self._finish_then(*self._contract(inputs, qkernel, qbias, training, mean_rows=inputs.shape[1]), then)
             y, act_done = self._contract(inputs, qkernel, qbias, training)
         finally:
             self._enable_iq = enable_iq
         if self.activation is not None and not act_done:
             y = self.activation(y)
         return y
+
+    call._takes_then = True

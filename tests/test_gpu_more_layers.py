@@ -862,6 +862,113 @@ def test_mean_over_the_middle_axis(shape):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize('groups,mean_rows,K,N,bw_rows,act,bias', [(4096, 64, 64, 32, 64, 'relu', True), (37, 64, 16, 64, 1, 'relu', True),
+                                                               (9, 32, 32, 20, 32, 'none', True), (130, 32, 8, 4, 0, 'relu', False),
+                                                               (1, 64, 48, 64, 2, 'relu', True), (3, 32, 64, 64, 16, 'none', False)])
+def test_contraction_with_the_mean_over_row_groups(groups, mean_rows, K, N, bw_rows, act, bias):
+    """ops.qdense_mean (the contraction kernel writes the means of groups of 32 / 64 output rows; its backward reads the
+    means' gradient with a zero row stride) against ops.qdense followed by ops.mean_mid: same means, and the same gradients
+    of the input, the kernel, the bias and the fractional bits, to the accumulation order of fp32 sums."""
+    from hgq2_amd import _lib, ops
+
+    dev = torch.device('cuda:0')
+    rows = groups * mean_rows
+    g = torch.Generator().manual_seed(groups + K + N)
+    x = (torch.randn(rows, K, generator=g) * 2).to(dev)
+    w = (torch.randint(-32, 32, (K, N), generator=g).float() / 16).to(dev)
+    b = (torch.randint(-8, 8, (N,), generator=g).float() / 8).to(dev) if bias else None
+    up = torch.randn(groups, N, generator=g).to(dev)
+    act_code = _lib.ACT_RELU if act == 'relu' else _lib.ACT_NONE
+    mode = _lib.mode_bits('RND', 'WRAP', training=True, round_params=True) if bw_rows else 0
+    if bw_rows:
+        f = torch.randint(2, 7, (bw_rows, K), generator=g).float().to(dev)
+        k = torch.ones(bw_rows * K, dtype=torch.uint8, device=dev)
+        i = torch.full((bw_rows * K,), 4.0, device=dev)
+    if not _lib.load().hgq_dense_use_bf16_parts(-1):
+        assert not ops.qdense_mean_supported(rows, K, N, bw_rows, mean_rows, mode)
+        pytest.skip('the fused mean rides on the bf16-part kernels')
+    assert ops.qdense_mean_supported(rows, K, N, bw_rows, mean_rows, mode)
+    res = []
+    for fused in (False, True):
+        xd, wd = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        bd = b.clone().requires_grad_(True) if bias else None
+        fd = f.clone().requires_grad_(True) if bw_rows else None
+        if fused:
+            m, amax = ops.qdense_mean(xd, k if bw_rows else None, fd.view(-1) if bw_rows else None, wd, bd, act_code, mode, bw_rows, mean_rows)
+        else:
+            y, amax = ops.qdense(xd, k if bw_rows else None, i if bw_rows else None, fd.view(-1) if bw_rows else None, wd, bd, act_code, mode,
+                                 bw_rows, bool(bw_rows))
+            m = ops.mean_mid(y.view(groups, mean_rows, N))
+        (m * up).sum().backward()
+        res.append((m.detach(), amax, xd.grad, wd.grad, bd.grad if bias else None, fd.grad if bw_rows else None))
+    assert tuple(res[1][0].shape) == (groups, N)
+    assert torch.equal(res[0][1], res[1][1]), 'abs-max slices of the input quantizer'
+    for name, a, c in zip(('means', 'amax', 'dx', 'dw', 'db', 'df'), *res):
+        if a is None or name == 'amax':
+            continue
+        err = float((a.double() - c.double()).abs().max())
+        assert err <= 2e-6 * float(a.abs().max()) + 1e-9, f'{name}: {err:.3e} of {float(a.abs().max()):.3e}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('with_batchnorm', [True, False])
+def test_a_contraction_layer_takes_the_mean_over_the_positions_with_it(dev, with_batchnorm, monkeypatch):
+    """``Sequential([QEinsumDense(Batchnorm)('bpf,fh->bph', relu), GlobalAveragePooling1D, ...])``: the pair runs as one
+    operator each way (``ops.qdense_mean``); two training steps give the outputs, losses, gradients and states of the same
+    model run layer by layer."""
+    from hgq2_amd import _lib, host, ops
+    from hgq2_amd.core import Sequential
+    from hgq2_amd.layers import QDense, QEinsumDense, QEinsumDenseBatchnorm
+    from hgq2_amd.train import SGD, model_loss
+
+    calls = []
+    real = ops.qdense_mean
+    monkeypatch.setattr(ops, 'qdense_mean', lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(48, 64, 16, generator=g).to(dev)
+    models = []
+    for absorb in (True, False):
+        torch.manual_seed(11)
+        with readme_scopes():
+            cls = QEinsumDenseBatchnorm if with_batchnorm else QEinsumDense
+            first = cls('bpf,fh->bph', (64, 32), bias_axes='h', activation='relu')
+            model = Sequential([first, host.GlobalAveragePooling1D(), QDense(5)])
+        model(x, training=False)
+        _perturb(model, torch.Generator().manual_seed(5))
+        if not absorb:
+            first.absorbs = lambda nxt, xx: False
+        models.append(model)
+    outs = []
+    for model in models:
+        opt = SGD(model.parameters(), lr=0.01)
+        hist = []
+        for t in range(2):
+            opt.zero_grad()
+            out = model(x, training=True)
+            loss = model_loss(model, (out * out).mean())
+            if t == 0:
+                loss.backward()  # every gradient through autograd: the operator's backward with its own slice reduction
+            else:
+                opt.backward(loss)  # gradient sink open: slices left for the joint reduction, pieces parked on the variables
+            grads = {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}
+            opt.step()
+            hist.append((out.detach().clone(), loss.detach().clone(), grads))
+        outs.append((hist, {n: v.detach().clone() for n, v in model.state_dict().items()}))
+    # once per training step of the absorbing model only (never on the fp32 matrix instruction: the pair then runs in two steps)
+    assert len(calls) == (2 if _lib.load().hgq_dense_use_bf16_parts(-1) else 0)
+    (ha, sa), (hb, sb) = outs
+    for (oa, la, ga), (ob, lb, gb) in zip(ha, hb):
+        _close(oa, ob.cpu(), what='output')
+        _close(la, lb.cpu(), what='loss')
+        assert ga.keys() == gb.keys()
+        for n in ga:
+            _close(ga[n], gb[n].cpu(), rtol=2e-5, what=f'grad {n}')
+    assert sa.keys() == sb.keys()
+    for n in sa:
+        _close(sa[n].float(), sb[n].float().cpu(), rtol=2e-5, what=f'state {n}')
+
+
+@pytest.mark.gpu
 def test_global_average_pooling_layers_use_it_and_match_the_library_mean():
     from hgq2_amd.config import QuantizerConfigScope
     from hgq2_amd.layers import QGlobalAveragePooling1D, QGlobalAveragePooling2D
