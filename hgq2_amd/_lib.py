@@ -111,6 +111,9 @@ SIGNATURES = {
     'hgq_affine_rows_fwd': (c_int, [c_void_p] * 4 + [c_int64, c_int, c_void_p]),
     'hgq_affine_rows_bwd_workspace': (c_int64, [c_int64, c_int]),
     'hgq_affine_rows_bwd': (c_int, [c_void_p] * 7 + [c_int64, c_int, c_void_p]),
+    'hgq_quantizer_scale_div': (c_int, [c_void_p, c_void_p, c_int64, c_float, c_void_p]),
+    'hgq_quantizer_tail_fwd': (c_int, [c_void_p] * 3 + [c_int64, c_int, c_float, c_int, c_float, c_int, c_float, c_float, c_void_p]),
+    'hgq_quantizer_tail_bwd': (c_int, [c_void_p] * 3 + [c_int64, c_int, c_float, c_int, c_float, c_int, c_float, c_void_p]),
     'hgq_mean_mid_fwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     'hgq_mean_mid_bwd': (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     'hgq_sum_scalars': (c_int, [c_void_p, c_int, c_void_p, c_void_p]),

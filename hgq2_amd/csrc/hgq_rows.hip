@@ -6,6 +6,10 @@
 //   per-channel affine y[r, c] = x[r, c] * s[c] + o[c]                 (QBatchNormalization, reference
 //                     src/hgq/layers/batch_normalization.py:184) with d/ds, d/do as fixed-order sums over the rows
 //
+// and the elementwise arithmetic the Quantizer wrapper puts around its internal quantizer (reference
+// src/hgq/quantizer/quantizer.py:49-60): the division by the scaler in front, and behind it the multiplication by the scaler,
+// the quantization-noise blend and the affine map as ONE pass each way.
+//
 // K, N <= 64 per group: the operands of a (row tile, group) pair sit in LDS, every output is one thread's sequential sum
 // (a multiplication and an addition per step, in k order), gradients that are sums over the rows leave as one slice per
 // workgroup and are added in a fixed order by reduce_parts.  These are HBM-bound shapes; nothing is reshaped to reach the
@@ -172,6 +176,87 @@ __global__ __launch_bounds__(AF_NT) void affine_rows_bwd_kernel(const float *__r
     }
 }
 
+// ---- Quantizer wrapper: every step is one IEEE fp32 operation, in the order the reference's eager code takes them
+struct WrapTail {
+    float scaler, noise, a0, a1;
+    int has_scaler, has_noise, has_affine;
+};
+
+__device__ __forceinline__ float wrap_tail_value(float q, float xs, const WrapTail &t) {
+    float o = q;
+    if (t.has_scaler) o = __fmul_rn(o, t.scaler);
+    if (t.has_noise) o = __fadd_rn(xs, __fmul_rn(t.noise, __fsub_rn(o, xs)));
+    if (t.has_affine) o = __fadd_rn(__fmul_rn(o, t.a0), t.a1);
+    return o;
+}
+
+// gradients of the quantizer's output and of the scaled input (the blend reads it) for an upstream gradient g, as autograd
+// forms them for the same chain of operations
+__device__ __forceinline__ void wrap_tail_grad(float g, const WrapTail &t, float &dq, float &dxs) {
+    if (t.has_affine) g = __fmul_rn(g, t.a0);
+    dxs = 0.f;
+    if (t.has_noise) {
+        const float go = __fmul_rn(g, t.noise);
+        dxs = __fsub_rn(g, go);
+        g = go;
+    }
+    dq = t.has_scaler ? __fmul_rn(g, t.scaler) : g;
+}
+
+// mode 0: y = x / scaler; 1: y = tail(q = x, xs = x2); 2: (y, y2) = gradients of (q, xs) for the upstream gradient x.
+// Four elements per thread where the arrays are 16-byte aligned (vec), one otherwise.
+__global__ __launch_bounds__(256) void wrap_kernel(const float *__restrict__ x, const float *__restrict__ x2, float *__restrict__ y,
+                                                   float *__restrict__ y2, int64_t n, WrapTail t, int mode, int vec) {
+    const int64_t stride = (int64_t)gridDim.x * 256, first = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n4 = vec ? n / 4 : 0;
+    for (int64_t v = first; v < n4; v += stride) {
+        const f32x4_t a = ((const f32x4_t *)x)[v];
+        f32x4_t o, o2 = {0.f, 0.f, 0.f, 0.f};
+        if (mode == 0) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) o[c] = __fdiv_rn(a[c], t.scaler);
+        } else if (mode == 1) {
+            const f32x4_t b = t.has_noise ? ((const f32x4_t *)x2)[v] : a;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) o[c] = wrap_tail_value(a[c], b[c], t);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float dq, dxs;
+                wrap_tail_grad(a[c], t, dq, dxs);
+                o[c] = dq, o2[c] = dxs;
+            }
+            if (y2) ((f32x4_t *)y2)[v] = o2;
+        }
+        ((f32x4_t *)y)[v] = o;
+    }
+    for (int64_t e = 4 * n4 + first; e < n; e += stride) {
+        const float a = x[e];
+        if (mode == 0) {
+            y[e] = __fdiv_rn(a, t.scaler);
+        } else if (mode == 1) {
+            y[e] = wrap_tail_value(a, t.has_noise ? x2[e] : a, t);
+        } else {
+            float dq, dxs;
+            wrap_tail_grad(a, t, dq, dxs);
+            y[e] = dq;
+            if (y2) y2[e] = dxs;
+        }
+    }
+}
+
+static int wrap_launch(const char *what, const float *x, const float *x2, float *y, float *y2, int64_t n, const WrapTail &t, int mode,
+                       void *stream) {
+    if (n < 0) return fail(HGQ_ERR_ARG, "%s: negative size", what);
+    if (n == 0) return HGQ_OK;
+    if (!x || !y) return fail(HGQ_ERR_ARG, "%s: null pointer", what);
+    const bool vec = (((uintptr_t)x | (uintptr_t)y | (uintptr_t)(x2 ? x2 : x) | (uintptr_t)(y2 ? y2 : y)) & 15u) == 0;
+    const int64_t items = vec ? (n + 3) / 4 : n;
+    hipLaunchKernelGGL(wrap_kernel, dim3((unsigned)persistent_grid((items + 255) / 256, 8)), dim3(256), 0, (hipStream_t)stream, x, x2, y, y2, n, t,
+                       mode, vec ? 1 : 0);
+    return check_launch(what);
+}
+
 static void affine_geometry(int64_t rows, int C, int &TX, int &gx, int64_t &gy, int64_t &rows_per_wg) {
     const int cg = C / 4;
     TX = 1;
@@ -271,4 +356,23 @@ extern "C" int hgq_affine_rows_bwd(const float *g, const float *x, const float *
     int rc = check_launch("hgq_affine_rows_bwd");
     if (rc) return rc;
     return reduce_parts(workspace, (int)gy, 2 * (int64_t)C, dscale, C, doffset, C, nullptr, 0, s);
+}
+
+extern "C" int hgq_quantizer_scale_div(const float *x, float *y, int64_t n, float scaler, void *stream) {
+    WrapTail t = {scaler, 0.f, 1.f, 0.f, 1, 0, 0};
+    return wrap_launch("hgq_quantizer_scale_div", x, nullptr, y, nullptr, n, t, 0, stream);
+}
+
+extern "C" int hgq_quantizer_tail_fwd(const float *q, const float *xs, float *out, int64_t n, int has_scaler, float scaler, int has_noise,
+                                      float noise, int has_affine, float a0, float a1, void *stream) {
+    if (has_noise && !xs) return fail(HGQ_ERR_ARG, "hgq_quantizer_tail_fwd: the noise blend needs the quantizer's input");
+    WrapTail t = {scaler, noise, a0, a1, has_scaler ? 1 : 0, has_noise ? 1 : 0, has_affine ? 1 : 0};
+    return wrap_launch("hgq_quantizer_tail_fwd", q, xs, out, nullptr, n, t, 1, stream);
+}
+
+extern "C" int hgq_quantizer_tail_bwd(const float *g, float *dq, float *dxs, int64_t n, int has_scaler, float scaler, int has_noise,
+                                      float noise, int has_affine, float a0, void *stream) {
+    if (has_noise && !dxs) return fail(HGQ_ERR_ARG, "hgq_quantizer_tail_bwd: the noise blend sends a gradient to the quantizer's input");
+    WrapTail t = {scaler, noise, a0, 0.f, has_scaler ? 1 : 0, has_noise ? 1 : 0, has_affine ? 1 : 0};
+    return wrap_launch("hgq_quantizer_tail_bwd", g, nullptr, dq, has_noise ? dxs : nullptr, n, t, 2, stream);
 }

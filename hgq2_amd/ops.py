@@ -2870,6 +2870,108 @@ class _AffineRows(torch.autograd.Function):
                 do.view(ctx.shapes[1]) if ctx.needs_input_grad[2] else None)
 
 
+@torch.library.custom_op('hgq::quantizer_scale_div', mutates_args=())
+def quantizer_scale_div_op(x: Tensor, scaler: float) -> Tensor:
+    _check_f32('x', x)
+    y = torch.empty_like(x)
+    _lib.check(_lib.load().hgq_quantizer_scale_div(_ptr(x), _ptr(y), x.numel(), scaler, _stream()), 'hgq_quantizer_scale_div')
+    return y
+
+
+@quantizer_scale_div_op.register_fake
+def _(x, scaler):
+    return torch.empty_like(x)
+
+
+@torch.library.custom_op('hgq::quantizer_tail_fwd', mutates_args=())
+def quantizer_tail_fwd(q: Tensor, xs: Tensor, has_scaler: bool, scaler: float, has_noise: bool, noise: float, has_affine: bool, a0: float,
+                       a1: float) -> Tensor:
+    _check_f32('q', q)
+    if has_noise:
+        _check_f32('xs', xs)
+        _need(xs.numel() == q.numel(), 'the quantizer\'s input and output must have the same size')
+    out = torch.empty_like(q)
+    rc = _lib.load().hgq_quantizer_tail_fwd(_ptr(q), _ptr(xs), _ptr(out), q.numel(), int(has_scaler), scaler, int(has_noise), noise,
+                                            int(has_affine), a0, a1, _stream())
+    _lib.check(rc, 'hgq_quantizer_tail_fwd')
+    return out
+
+
+@quantizer_tail_fwd.register_fake
+def _(q, xs, has_scaler, scaler, has_noise, noise, has_affine, a0, a1):
+    return torch.empty_like(q)
+
+
+@torch.library.custom_op('hgq::quantizer_tail_bwd', mutates_args=())
+def quantizer_tail_bwd(g: Tensor, has_scaler: bool, scaler: float, has_noise: bool, noise: float, has_affine: bool,
+                       a0: float) -> tuple[Tensor, Tensor]:
+    _check_f32('g', g)
+    dq = torch.empty_like(g)
+    dxs = torch.empty_like(g) if has_noise else g.new_empty(0)
+    rc = _lib.load().hgq_quantizer_tail_bwd(_ptr(g), _ptr(dq), _ptr(dxs), g.numel(), int(has_scaler), scaler, int(has_noise), noise,
+                                            int(has_affine), a0, _stream())
+    _lib.check(rc, 'hgq_quantizer_tail_bwd')
+    return dq, dxs
+
+
+@quantizer_tail_bwd.register_fake
+def _(g, has_scaler, scaler, has_noise, noise, has_affine, a0):
+    return torch.empty_like(g), (torch.empty_like(g) if has_noise else g.new_empty(0))
+
+
+class _ScaleDiv(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, scaler):
+        ctx.scaler = scaler
+        return quantizer_scale_div_op(x, scaler)
+
+    @staticmethod
+    def backward(ctx, g):
+        return quantizer_scale_div_op(g.contiguous(), ctx.scaler), None
+
+
+class _QuantizerTail(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, xs, scaler, noise, affine):
+        ctx.args = (scaler is not None, float(scaler or 1.0), noise is not None, float(noise or 0.0), affine is not None,
+                    float(affine[0]) if affine is not None else 1.0)
+        return quantizer_tail_fwd(q, xs, *ctx.args, float(affine[1]) if affine is not None else 0.0)
+
+    @staticmethod
+    def backward(ctx, g):
+        dq, dxs = quantizer_tail_bwd(g.contiguous(), *ctx.args)
+        return dq, (dxs if ctx.args[2] and ctx.needs_input_grad[1] else None), None, None, None
+
+
+def _wrapper_on_gpu(*tensors) -> bool:
+    return all(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() > 0 for t in tensors)
+
+
+def quantizer_scale_div(x: Tensor, scaler: float) -> Tensor:
+    """``x / scaler`` as a true division (the first step of the reference's ``Quantizer.call``, src/hgq/quantizer/quantizer.py:50-51)."""
+    if _wrapper_on_gpu(x):
+        return _ScaleDiv.apply(x, float(scaler))
+    return x / torch.full((), float(scaler), dtype=x.dtype, device=x.device)
+
+
+def quantizer_tail(q: Tensor, xs: Tensor, scaler, noise, affine) -> Tensor:
+    """What the reference's ``Quantizer.call`` does behind its internal quantizer (src/hgq/quantizer/quantizer.py:54-59):
+    ``q * scaler``, the blend ``xs + noise * (. - xs)`` with the quantizer's input ``xs``, ``. * affine[0] + affine[1]`` -
+    whichever of the three are not ``None`` - in one pass each way."""
+    if scaler is None and noise is None and affine is None:
+        return q
+    if _wrapper_on_gpu(q, xs) and q.shape == xs.shape:
+        return _QuantizerTail.apply(q, xs, scaler, noise, affine)
+    out = q
+    if scaler is not None:
+        out = out * scaler
+    if noise is not None:
+        out = xs + noise * (out - xs)
+    if affine is not None:
+        out = out * affine[0] + affine[1]
+    return out
+
+
 @torch.library.custom_op('hgq::gdense_fwd', mutates_args=())
 def gdense_fwd(x: Tensor, w: Tensor, bias: Tensor, act: int) -> Tensor:
     _check_f32('x', x), _check_f32('w', w)

@@ -43,23 +43,15 @@ class Quantizer(Layer):
         return QuantizerConfig(*args, **q_kwargs), kwargs
 
     def call(self, inputs, training=None):
+        from .. import ops
+
         if self.scaler is not None:
-            # the divisor goes in as a tensor: on the GPU torch divides by a Python number with a multiplication by its
-            # rounded reciprocal, one ulp away from the quotient for some inputs (and one quantization step after rounding)
-            key = (inputs.device, inputs.dtype, float(self.scaler))
-            cached = getattr(self, '_scaler_tensor', None)
-            if cached is None or cached[0] != key:
-                cached = (key, torch.full((), float(self.scaler), dtype=inputs.dtype, device=inputs.device))
-                object.__setattr__(self, '_scaler_tensor', cached)
-            inputs = inputs / cached[1]
+            # a true division (on the GPU the tensor library divides by a Python number with a multiplication by its rounded
+            # reciprocal, one ulp away from the quotient for some inputs - and one quantization step after rounding)
+            inputs = ops.quantizer_scale_div(inputs, self.scaler)
         outputs = self.quantizer(inputs, training=training)
-        if self.scaler is not None:
-            outputs = outputs * self.scaler
-        if self.qnoise_factor is not None and training:
-            outputs = inputs + self.qnoise_factor * (outputs - inputs)
-        if self.affine is not None:
-            outputs = outputs * self.affine[0] + self.affine[1]
-        return outputs
+        # the multiplication by the scaler, the noise blend of training calls and the affine map: one pass each way
+        return ops.quantizer_tail(outputs, inputs, self.scaler, self.qnoise_factor if training else None, self.affine)
 
     @property
     def plain(self) -> bool:

@@ -46,9 +46,10 @@ def main(argv=None):
         rc = lib.hgq_qdense_bwd(dy.data_ptr(), None, x.data_ptr(), f_in.data_ptr(), 1, w.data_ptr(), dx.data_ptr(), dqw.data_ptr(),
                                 dqb.data_ptr(), df.data_ptr(), ws.data_ptr(), rows, K, N, 0, mode, None)
         _lib.check(rc, 'hgq_qdense_bwd')
-        rc = lib.hgq_qdense_moments_bwd(x.data_ptr(), f_in.data_ptr(), 1, mode, w.data_ptr(), gm.data_ptr(), gsq.data_ptr(), dy_in.data_ptr(),
-                                        dx.data_ptr(), dqw.data_ptr(), df.data_ptr(), ws.data_ptr(), rows, K, N, None)
-        _lib.check(rc, 'hgq_qdense_moments_bwd')
+        if K % 4 == 0 and N % 4 == 0:  # (the statistics' backward takes no other widths)
+            rc = lib.hgq_qdense_moments_bwd(x.data_ptr(), f_in.data_ptr(), 1, mode, w.data_ptr(), gm.data_ptr(), gsq.data_ptr(), dy_in.data_ptr(),
+                                            dx.data_ptr(), dqw.data_ptr(), df.data_ptr(), ws.data_ptr(), rows, K, N, None)
+            _lib.check(rc, 'hgq_qdense_moments_bwd')
 
     for _ in range(3):
         run()

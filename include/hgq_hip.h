@@ -913,6 +913,24 @@ int hgq_affine_rows_bwd(const float *g, const float *x, const float *scale, floa
                         int64_t rows, int C, void *stream);
 
 /*
+ * The arithmetic Quantizer.call puts around its internal quantizer (src/hgq/quantizer/quantizer.py:49-60), every step one
+ * IEEE fp32 operation in the reference's order:
+ *   hgq_quantizer_scale_div:  y = x / scaler                                   (`inputs = inputs / self.scaler`, :50-51)
+ *   hgq_quantizer_tail_fwd:   o = q; o = o * scaler (has_scaler);  o = xs + noise * (o - xs) (has_noise: the
+ *                             quantization-noise blend of training calls, xs = the quantizer's input);  o = o * a0 + a1
+ *                             (has_affine)                                      (:54-59) - one pass for whichever are set
+ *   hgq_quantizer_tail_bwd:   the gradients of (q, xs) for the upstream gradient g, formed as reverse-mode differentiation
+ *                             of that chain forms them: g' = g * a0; dxs = g' - g' * noise, g'' = g' * noise; dq = g'' * scaler.
+ *                             dxs is written only with has_noise (it may be NULL otherwise).
+ * Any n, any alignment (128-bit accesses when every array is 16-byte aligned).
+ */
+int hgq_quantizer_scale_div(const float *x, float *y, int64_t n, float scaler, void *stream);
+int hgq_quantizer_tail_fwd(const float *q, const float *xs, float *out, int64_t n, int has_scaler, float scaler, int has_noise,
+                           float noise, int has_affine, float a0, float a1, void *stream);
+int hgq_quantizer_tail_bwd(const float *g, float *dq, float *dxs, int64_t n, int has_scaler, float scaler, int has_noise, float noise,
+                           int has_affine, float a0, void *stream);
+
+/*
  * 2-D max / average pooling on channels-last tensors, forward and backward.  Replaces the Keras
  * MaxPooling2D / AveragePooling2D `call` that QMaxPooling2D / QAveragePooling2D apply to the
  * quantized input (src/hgq/layers/pooling.py:23-47; the Keras torch backend transposes to

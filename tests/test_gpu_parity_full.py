@@ -305,8 +305,8 @@ def test_kbi_wrap_tracing_matches_oracle_with_many_row_chunks(dev):
 @pytest.mark.parametrize('overflow_mode', ['WRAP', 'SAT'])
 def test_quantizer_wrapper_scaler_qnoise_affine(dev, extras, overflow_mode):
     """Reference src/hgq/quantizer/quantizer.py:49-60 against the oracle twin: the inner quantizer's values are exact,
-    the elementwise stages around it are fp32 ops in the same order, so the outputs are compared bit for bit in
-    inference and at 1e-6 in training (noise blend: one fused multiply-add may differ)."""
+    the elementwise stages around it (one kernel pass in front, one behind, one IEEE operation per step of the reference)
+    are fp32 ops in the same order, so the outputs are compared bit for bit in inference and in training."""
     from hgq2_amd.config import QuantizerConfig
     from hgq2_amd.quantizer import Quantizer
 
@@ -323,7 +323,7 @@ def test_quantizer_wrapper_scaler_qnoise_affine(dev, extras, overflow_mode):
     xp, xr = x.to(dev).requires_grad_(True), x.clone().requires_grad_(True)
     gy = torch.randn(x.shape, generator=g)
     yp, yr = q(xp, training=True), r(xr, training=True)
-    np.testing.assert_allclose(yp.detach().cpu().numpy(), yr.detach().numpy(), rtol=1e-6, atol=1e-6)
+    assert torch.equal(yp.detach().cpu(), yr.detach())
     assert torch.equal(q.quantizer._i.cpu(), r.quantizer._i.detach())
     yp.backward(gy.to(dev))
     yr.backward(gy)
@@ -332,6 +332,46 @@ def test_quantizer_wrapper_scaler_qnoise_affine(dev, extras, overflow_mode):
     _close_scaled(q.quantizer._f.grad, r.quantizer._f.grad, scale, 'd/df')
     if overflow_mode == 'SAT':  # the integer bits are trainable unless the overflow mode is WRAP
         _close_scaled(q.quantizer._i.grad, r.quantizer._i.grad, scale, 'd/di')
+
+
+@pytest.mark.parametrize('n,offset', [(4096, 0), (1001, 0), (1023, 1), (3, 0), (1, 2)])
+@pytest.mark.parametrize('scaler,noise,affine', [(3.0, None, None), (None, 0.3, None), (None, None, (0.25, 0.5)), (0.7, 0.45, (3.0, -1.0))])
+def test_quantizer_wrapper_kernels_equal_the_elementwise_operations(dev, n, offset, scaler, noise, affine):
+    """``ops.quantizer_scale_div`` / ``ops.quantizer_tail`` against the same chain written as separate CPU tensor operations
+    (reference src/hgq/quantizer/quantizer.py:49-60), values and gradients bit for bit, for sizes that are no multiple of
+    four and arrays that are not 16-byte aligned."""
+    from hgq2_amd import ops
+
+    g = torch.Generator().manual_seed(n + offset)
+    base = torch.randn(3, n + offset, generator=g) * 5
+    x, xs, gy = (base[k, offset:].clone() for k in range(3))
+    dev_of = lambda t: torch.zeros(t.numel() + offset, device=dev)[offset:].copy_(t)  # the same misalignment on the device
+    if scaler is not None:
+        xr = x.clone().requires_grad_(True)
+        want = xr / scaler
+        want.backward(gy)
+        xd = dev_of(x).requires_grad_(True)
+        got = ops.quantizer_scale_div(xd, scaler)
+        got.backward(dev_of(gy))
+        assert torch.equal(got.detach().cpu(), want.detach()) and torch.equal(xd.grad.cpu(), xr.grad)
+    qr, xsr = x.clone().requires_grad_(True), xs.clone().requires_grad_(True)
+    out = qr
+    if scaler is not None:
+        out = out * scaler
+    if noise is not None:
+        out = xsr + noise * (out - xsr)
+    if affine is not None:
+        out = out * affine[0] + affine[1]
+    out.backward(gy)
+    qd, xsd = dev_of(x).requires_grad_(True), dev_of(xs).requires_grad_(True)
+    got = ops.quantizer_tail(qd, xsd, scaler, noise, affine)
+    got.backward(dev_of(gy))
+    assert torch.equal(got.detach().cpu(), out.detach())
+    assert torch.equal(qd.grad.cpu(), qr.grad)
+    if noise is not None:
+        assert torch.equal(xsd.grad.cpu(), xsr.grad)
+    else:
+        assert xsd.grad is None
 
 
 # --------------------------------------------------------------------------------------------------------------
