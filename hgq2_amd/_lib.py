@@ -67,6 +67,7 @@ SIGNATURES = {
     'hgq_ebops_finish_fwd': (c_int, [c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_ebops_finish_bwd': (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_void_p]),
     'hgq_lut_ebops': (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
+    'hgq_sum_ebops': (c_int, [c_void_p, c_int64, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_softmax_ebops': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_mha_ebops': (c_int, [c_void_p] * 4 + [c_int] * 5 + [c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p]),
     'hgq_qbits_fwd': (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),

@@ -205,6 +205,37 @@ __global__ __launch_bounds__(EB_NT) void lut_ebops_kernel(hgq_bits_desc d_in, hg
     entry_grads(out, n, gs, [&](uint32_t c) { return ldexpf(1.0f, (int)in.template cell<GENERIC>(c)); }, red);
 }
 
+// Pooling layers: sum over the cells of bits_in, times parallel_factor, divided by n_parallel (a product, then a correctly
+// rounded division, as the reference evaluates it left to right)
+template <bool GENERIC>
+__global__ __launch_bounds__(EB_NT) void sum_ebops_kernel(hgq_bits_desc d_in, uint32_t n, float parallel_factor, float n_parallel, float f2,
+                                                          const float *beta, uint32_t *ebops_u32, float *loss_term) {
+    __shared__ double red[EB_NT];
+    extern __shared__ float pool[];
+    Bits in{d_in};
+    const bool lone = d_in.size == 1;
+    double raw;
+    bool oa = false;
+    if (lone) {
+        if (threadIdx.x != 0) return;
+        raw = (double)n * (double)in.lone(oa);
+    } else {
+        in.stage(pool, n);
+        __syncthreads();
+        double part = 0.0;
+        for (uint32_t c = threadIdx.x; c < n; c += EB_NT) part += (double)in.template cell<GENERIC>(c);
+        raw = block_sum(part, red);
+    }
+    float e = __fmul_rn((float)raw, parallel_factor);
+    if (n_parallel != 1.0f) e = __fdiv_rn(e, n_parallel);
+    const float gs = __fmul_rn(finish((double)e, 1.0f, f2, beta, ebops_u32, loss_term), parallel_factor / n_parallel);
+    if (lone) {
+        in.put_lone(oa, (float)(double)n * gs);
+        return;
+    }
+    entry_grads(in, n, gs, [&](uint32_t) { return 1.0f; }, red);
+}
+
 // QSoftmax over the last axis of [R, L] (stable form):
 //   sum(bits_sub) + sum(bits_exp) - sum_rows min_l bits_exp + sum(bits_exp * bits_inv[row])
 // bits_sub: what the maximum is subtracted from (the layer's input quantizer, else the exp table's); may be absent.
@@ -367,6 +398,25 @@ extern "C" int hgq_lut_ebops(const hgq_bits_desc *bits_in, const hgq_bits_desc *
     const bool generic = !(simple_layout(bits_in, n_cells) && simple_layout(bits_out, n_cells));
     hipLaunchKernelGGL(generic ? lut_ebops_kernel<true> : lut_ebops_kernel<false>, dim3(1), dim3(EB_NT), lds, (hipStream_t)stream, *bits_in, *bits_out, (uint32_t)n_cells, scale,
                        ebops_factor, beta, ebops_u32, loss_term);
+    return check_launch(who);
+}
+
+extern "C" int hgq_sum_ebops(const hgq_bits_desc *bits_in, int64_t n_cells, float parallel_factor, float n_parallel, float ebops_factor,
+                             const float *beta, uint32_t *ebops_u32, float *loss_term, void *stream) {
+    const char *who = "hgq_sum_ebops";
+    if (n_cells < 1 || n_cells >= (1ll << 31)) return fail(HGQ_ERR_UNSUPPORTED, "%s: 1 <= n_cells < 2**31 expected", who);
+    if (!(n_parallel > 0.f)) return fail(HGQ_ERR_ARG, "%s: n_parallel must be positive", who);
+    int rc;
+    if ((rc = check_bits(bits_in, n_cells, who, "bits_in"))) return rc;
+    if (!beta || !loss_term) return fail(HGQ_ERR_ARG, "%s: null pointer", who);
+    size_t lds;
+    static bool raised = false, raised2 = false;
+    if ((rc = pool_bytes(bits_in->size, who, lds)) || (rc = raise_pool(sum_ebops_kernel<true>, raised, who)) ||
+        (rc = raise_pool(sum_ebops_kernel<false>, raised2, who)))
+        return rc;
+    const bool generic = !simple_layout(bits_in, n_cells);
+    hipLaunchKernelGGL(generic ? sum_ebops_kernel<true> : sum_ebops_kernel<false>, dim3(1), dim3(EB_NT), lds, (hipStream_t)stream, *bits_in,
+                       (uint32_t)n_cells, parallel_factor, n_parallel, ebops_factor, beta, ebops_u32, loss_term);
     return check_launch(who);
 }
 

@@ -29,6 +29,16 @@ class QBasePooling(QLayerBaseSingleInput):
         bw_inp = self.iq.bits_(shape)
         return scale_ebops(torch.sum(bw_inp), self.parallelization_factor, self.n_parallel)
 
+    def _ebops_loss_term(self, shape):
+        # value, uint32 variable, loss term and the bit-width gradients in one launch where the quantizer allows it
+        if self.enable_iq and self._beta is not None and self._beta.is_cuda and self.n_parallel:
+            operand = self.iq.bits_operand(shape)
+            n_cells = prod(int(s) for s in shape)
+            if operand is not None and 0 < n_cells < 2**31 and operand[3] <= 30720:
+                return ops.bits_ebops('sum', [operand], (n_cells, float(self.parallelization_factor), float(self.n_parallel),
+                                                         float(self.ebops_factor)), self._beta, self._ebops)
+        return super()._ebops_loss_term(shape)
+
     def pool(self, inputs):
         raise NotImplementedError
 

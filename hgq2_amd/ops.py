@@ -2700,7 +2700,7 @@ def ebops_finish(ebops: Tensor, factor: float, beta: Tensor, ebops_var: Tensor) 
 
 
 class _BitsEbops(torch.autograd.Function):
-    """EBOPs that are algebra on bit-width tensors (``hgq_lut_ebops`` / ``hgq_softmax_ebops`` / ``hgq_mha_ebops``).
+    """EBOPs that are algebra on bit-width tensors (``hgq_lut_ebops`` / ``hgq_sum_ebops`` / ``hgq_softmax_ebops`` / ``hgq_mha_ebops``).
     ``layouts[n]`` = ``(size, inner, kbi, add_mode)`` of operand n or ``None``; ``qvars`` = k, i, fb per operand
     (empty tensors where absent).  The kernel leaves the gradients for a unit upstream gradient; backward scales them."""
 
@@ -2748,6 +2748,9 @@ class _BitsEbops(torch.autograd.Function):
         if kind == 'lut':
             n_cells, scale, factor = params
             rc = lib.hgq_lut_ebops(ptrs[0], ptrs[1], n_cells, scale, factor, _ptr(beta), _ptr(ebops_var), _ptr(out), _stream())
+        elif kind == 'sum':
+            n_cells, parallel_factor, n_parallel, factor = params
+            rc = lib.hgq_sum_ebops(ptrs[0], n_cells, parallel_factor, n_parallel, factor, _ptr(beta), _ptr(ebops_var), _ptr(out), _stream())
         elif kind == 'softmax':
             rows, L, f1, f2 = params
             rc = lib.hgq_softmax_ebops(ptrs[0], ptrs[1], ptrs[2], rows, L, f1, f2, _ptr(beta), _ptr(ebops_var), _ptr(out), _stream())
@@ -3062,7 +3065,7 @@ def bias_add_rows(y: Tensor, b: Tensor) -> Tensor:
 def bits_ebops(kind: str, operands, params, beta: Tensor, ebops_var: Tensor, owners=None) -> Tensor:
     """Loss term ``ebops * beta`` of a layer whose EBOPs are algebra on bit-width tensors, in one launch; also assigns
     the uint32 variable.  ``operands``: per operand ``None`` or ``(k, i, fb, size, inner, kbi, add_mode)`` (``i`` is
-    ``None`` for the (k, b, i) kind); ``params`` as the C entry point of ``kind`` ('lut', 'softmax', 'mha', 'conv') takes them;
+    ``None`` for the (k, b, i) kind); ``params`` as the C entry point of ``kind`` ('lut', 'sum', 'softmax', 'mha', 'conv') takes them;
     ``owners``: per operand ``None`` or the variables ``(i, fb)`` behind it (see :class:`side_gradients`)."""
     e_f = beta.new_empty(0)
     e_k = torch.empty(0, dtype=torch.uint8, device=beta.device)

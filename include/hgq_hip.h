@@ -708,9 +708,14 @@ typedef struct hgq_bits_desc {
  *   hgq_mha_ebops      QMultiHeadAttention._compute_ebops (src/hgq/layers/attn/mha.py:507-524) for rank-3 inputs:
  *                      sum bits_q[t,n,h] bits_k[s,n,h] + sum bits_attn[n,t,s] bits_v[s,n,h]; cells of q / k / v in
  *                      [seq, N, H] order, of attn in [N, T, S] order.  N * H <= 1024, N * S <= 2048.
+ *   hgq_sum_ebops      the pooling layers' QBasePooling._compute_ebops (src/hgq/layers/pooling.py:28-30): sum over
+ *                      n_cells of bits_in, times parallel_factor, divided by n_parallel (a product, then a correctly
+ *                      rounded division; no division when n_parallel is 1), times ebops_factor.
  * Every sum is formed in a fixed order; values are exact while they stay below 2**53.  The operands' entries are
  * staged in LDS: at most 30720 over all operands of a call (HGQ_ERR_UNSUPPORTED beyond, as for the other limits).
  */
+int hgq_sum_ebops(const hgq_bits_desc *bits_in, int64_t n_cells, float parallel_factor, float n_parallel, float ebops_factor,
+                  const float *beta, uint32_t *ebops_u32, float *loss_term, void *stream);
 int hgq_lut_ebops(const hgq_bits_desc *bits_in, const hgq_bits_desc *bits_out, int64_t n_cells, float scale, float ebops_factor,
                   const float *beta, uint32_t *ebops_u32, float *loss_term, void *stream);
 int hgq_softmax_ebops(const hgq_bits_desc *bits_sub, const hgq_bits_desc *bits_exp, const hgq_bits_desc *bits_inv, int64_t rows, int L,

@@ -985,6 +985,46 @@ def test_global_average_pooling_layers_use_it_and_match_the_library_mean():
             assert torch.allclose(y.cpu(), want, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize('factor,het', [(-1, True), (3, True), (7, False)])
+def test_pooling_ebops_in_one_launch(dev, factor, het, monkeypatch):
+    """The pooling layers' EBOPs (reference src/hgq/layers/pooling.py:28-30: sum(bits) * parallelization_factor / n_parallel)
+    through ``hgq_sum_ebops``: the uint32 variable, the loss term and the bit-width gradients equal those of the formula
+    written in tensor operations, also where the factor does not divide."""
+    from hgq2_amd import ops
+    from hgq2_amd.layers import QAveragePooling2D
+    from hgq2_amd.layers.core.base import QLayerBase
+    from hgq2_amd.train import model_loss
+
+    kinds = []
+    real = ops.bits_ebops
+    monkeypatch.setattr(ops, 'bits_ebops', lambda kind, *a, **k: (kinds.append(kind), real(kind, *a, **k))[1])
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(6, 8, 10, 4, generator=g).to(dev)
+    res = []
+    for fused in (True, False):
+        torch.manual_seed(2)
+        with readme_scopes(beta0=1e-3):
+            layer = QAveragePooling2D((2, 2), parallelization_factor=factor)
+        layer(x, training=False)
+        if het:
+            _perturb(layer, torch.Generator().manual_seed(9))
+        if not fused:  # the same layer on the base class's formula
+            layer._ebops_loss_term = lambda shape, layer=layer: QLayerBase._ebops_loss_term(layer, shape)
+        out = layer(x, training=True)
+        loss = model_loss(layer, (out * out).mean())
+        loss.backward()
+        q = layer.iq.quantizer
+        res.append((int(layer._ebops.view(torch.int32)), loss.detach(), q._f.grad.clone(), q._i.grad.clone() if q._i.grad is not None else None))
+    assert kinds == ['sum']
+    (ea, la, fa, ia), (eb, lb, fb, ib) = res
+    assert ea == eb and ea > 0
+    _close(la, lb.cpu(), what='loss')
+    _close(fa, fb.cpu(), what='d/df')
+    if ia is not None:
+        _close(ia, ib.cpu(), what='d/di')
+
+
 @pytest.mark.parametrize('kind', ['conv', 'particle'])
 def test_plain_backward_inside_the_overlap_context(dev, kind):
     """``model_loss`` inside ``ops.overlap_ebops()`` returns a total whose value is written later; ``loss.backward()`` -
