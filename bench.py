@@ -558,15 +558,18 @@ def main():
             torch.manual_seed(1)
             model = qdense_mlp(DIMS, beta0=1e-5, device=dev)
             fit(model, data_x, data_y, lr=0.01, batch_size=BATCH, epochs=1, shuffle=False, fused=fused)  # records / warms up
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            n_epochs = 20
-            hist = fit(model, data_x, data_y, lr=0.01, batch_size=BATCH, epochs=n_epochs, shuffle=False, fused=fused)
-            torch.cuda.synchronize()
-            el_f = time.perf_counter() - t0
-            paths[name] = {'samples_per_s': BATCH * n_batches * n_epochs / el_f, 'ms_per_step': el_f / (n_epochs * n_batches) * 1e3,
-                           'steps': n_epochs * n_batches, 'final_epoch_loss': hist[-1]['loss'],
-                           'what': 'train.fit over 64 resident batches x 20 epochs, the recording of its step included, '
+            times = {}
+            for n_epochs in (5, 25):  # two lengths: their difference is steps only, the rest is the call's own set-up (the recording)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                hist = fit(model, data_x, data_y, lr=0.01, batch_size=BATCH, epochs=n_epochs, shuffle=False, fused=fused)
+                torch.cuda.synchronize()
+                times[n_epochs] = time.perf_counter() - t0
+            per_step = (times[25] - times[5]) / (20 * n_batches)
+            paths[name] = {'samples_per_s': BATCH / per_step, 'ms_per_step': per_step * 1e3, 'steps': 20 * n_batches,
+                           'setup_ms_per_call': (times[5] - 5 * n_batches * per_step) * 1e3, 'final_epoch_loss': hist[-1]['loss'],
+                           'what': 'train.fit over 64 resident batches: time per step from calls of 5 and 25 epochs (setup_ms_per_call = '
+                                   'what a call takes beyond its steps: recording the step, reading the loss), '
                                    + ('path chosen by fit' if fused is None else 'per-layer operators replayed from a HIP graph')}
         out['paths'] = paths
 

@@ -87,6 +87,7 @@ SIGNATURES = {
     'hgq_mse_bwd': (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     'hgq_mse_fwd_bwd': (c_int, [c_void_p] * 5 + [c_int64, c_void_p]),
     'hgq_sparse_ce_fwd_bwd': (c_int, [c_void_p] * 4 + [c_int64, c_int, c_void_p, c_void_p]),
+    'hgq_gather_batch': (c_int, [c_void_p, c_int64, c_void_p, c_int64] + [c_void_p] * 4 + [c_int64, c_int64, c_void_p]),
     'hgq_sgd_update': (c_int, [c_void_p, c_void_p, c_int64, c_float, c_float, c_float, c_float, c_void_p]),
     'hgq_sgd_update_multi': (c_int, [c_void_p, c_int, c_float, c_void_p]),
     'hgq_sgd_update_multi_sum': (c_int, [c_void_p, c_int, c_float, c_void_p, c_int, c_void_p, c_void_p]),

@@ -507,6 +507,48 @@ __global__ __launch_bounds__(256) void sparse_ce_kernel(const float *__restrict_
     }
 }
 
+// The next batch of a data set that lives in device memory: row r of the batch is row order[pos + r] of the source (samples
+// and labels alike), pos = state[0].  The workgroup that finishes last - every other one has read pos by then - moves pos
+// on by `batch` and clears the ticket word state[1], so a recorded launch draws batch after batch as it is replayed.
+// Positions past the end read the last row (the caller resets pos before that happens).  Rows are whole 32-bit words;
+// VEC: 128-bit accesses (row sizes multiples of 16 bytes, aligned arrays).
+template <bool VEC>
+__global__ __launch_bounds__(256) void gather_batch_kernel(const uint32_t *__restrict__ x_src, int64_t x_words,
+                                                           const uint32_t *__restrict__ y_src, int64_t y_words,
+                                                           const int64_t *__restrict__ order, unsigned long long *state,
+                                                           uint32_t *__restrict__ x_dst, uint32_t *__restrict__ y_dst, int64_t batch,
+                                                           int64_t n_rows) {
+    __shared__ int64_t spos;
+    if (threadIdx.x == 0) spos = (int64_t)__hip_atomic_load(state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int64_t pos = spos;
+    const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x, stride = (int64_t)gridDim.x * 256;
+    auto source_row = [&](int64_t r) {
+        int64_t p = pos + r;
+        p = p < n_rows ? p : n_rows - 1;
+        int64_t s = order[p < 0 ? 0 : p];
+        return s < 0 ? 0 : (s < n_rows ? s : n_rows - 1);
+    };
+    const int64_t xw = VEC ? x_words / 4 : x_words;
+    for (int64_t e = first; e < batch * xw; e += stride) {
+        const int64_t r = e / xw, c = e - r * xw, s = source_row(r);
+        if (VEC) ((u32x4_t *)x_dst)[r * xw + c] = ((const u32x4_t *)x_src)[s * xw + c];
+        else x_dst[r * xw + c] = x_src[s * xw + c];
+    }
+    for (int64_t e = first; e < batch * y_words; e += stride) {
+        const int64_t r = e / y_words, c = e - r * y_words;
+        y_dst[e] = y_src[source_row(r) * y_words + c];
+    }
+    __syncthreads();  // every thread of this workgroup has read pos
+    if (threadIdx.x == 0) {
+        uint32_t *ticket = (uint32_t *)(state + 1);
+        if (atomicAdd(ticket, 1u) == gridDim.x - 1) {
+            atomicExch(state, (unsigned long long)(pos + batch));
+            atomicExch(ticket, 0u);
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, int64_t n,
                                                   float lr, float l1, float lo, float hi) {
     for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < n; t += (int64_t)gridDim.x * 256) {
@@ -754,6 +796,27 @@ extern "C" int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels,
     const int grid = state ? persistent_grid((rows + 255) / 256, 4) : 1;
     hipLaunchKernelGGL(sparse_ce_kernel, dim3(grid), dim3(256), 0, s, logits, labels, loss, dlogits, rows, C, state);
     return check_launch("hgq_sparse_ce_fwd_bwd");
+}
+
+extern "C" int hgq_gather_batch(const void *x_src, int64_t x_row_bytes, const void *y_src, int64_t y_row_bytes, const int64_t *order,
+                                void *state, void *x_dst, void *y_dst, int64_t batch, int64_t n_rows, void *stream) {
+    if (batch < 1 || n_rows < 1 || x_row_bytes < 4 || y_row_bytes < 0 || (x_row_bytes & 3) || (y_row_bytes & 3))
+        return fail(HGQ_ERR_ARG, "hgq_gather_batch: sizes must be positive and rows whole 32-bit words");
+    if (batch * (x_row_bytes + y_row_bytes) >= (1ll << 40)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_gather_batch: batch too large");
+    if (!x_src || !x_dst || !order || !state || (y_row_bytes && (!y_src || !y_dst))) return fail(HGQ_ERR_ARG, "hgq_gather_batch: null pointer");
+    if (((uintptr_t)x_src | (uintptr_t)x_dst | (uintptr_t)y_src | (uintptr_t)y_dst) & 3u)
+        return fail(HGQ_ERR_ARG, "hgq_gather_batch: arrays must be 4-byte aligned");
+    if (((uintptr_t)state | (uintptr_t)order) & 7u) return fail(HGQ_ERR_ARG, "hgq_gather_batch: order and state must be 8-byte aligned");
+    const bool vec = (x_row_bytes & 15) == 0 && ((((uintptr_t)x_src | (uintptr_t)x_dst)) & 15u) == 0;
+    const int64_t items = batch * (vec ? x_row_bytes / 16 : x_row_bytes / 4);
+    const dim3 grid((unsigned)persistent_grid((items + 255) / 256, 8));
+    if (vec)
+        hipLaunchKernelGGL(gather_batch_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, (const uint32_t *)x_src, x_row_bytes / 4,
+                           (const uint32_t *)y_src, y_row_bytes / 4, order, (unsigned long long *)state, (uint32_t *)x_dst, (uint32_t *)y_dst, batch, n_rows);
+    else
+        hipLaunchKernelGGL(gather_batch_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, (const uint32_t *)x_src, x_row_bytes / 4,
+                           (const uint32_t *)y_src, y_row_bytes / 4, order, (unsigned long long *)state, (uint32_t *)x_dst, (uint32_t *)y_dst, batch, n_rows);
+    return check_launch("hgq_gather_batch");
 }
 
 extern "C" int hgq_ebops_finish_fwd(const float *ebops, float factor, const float *beta, uint32_t *ebops_u32, float *out, void *stream) {

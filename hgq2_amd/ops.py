@@ -3219,6 +3219,30 @@ def mse(pred: Tensor, target: Tensor | None = None) -> Tensor:
     return _MSE.apply(pred, target.contiguous() if target is not None else pred.new_empty(0))
 
 
+@torch.library.custom_op('hgq::gather_batch', mutates_args=('state', 'x_dst', 'y_dst'))
+def gather_batch(x_src: Tensor, y_src: Tensor, order: Tensor, state: Tensor, x_dst: Tensor, y_dst: Tensor) -> None:
+    """The next batch of a data set in device memory: row r of ``x_dst`` / ``y_dst`` = row ``order[state[0] + r]`` of ``x_src`` /
+    ``y_src``, and ``state[0]`` moves on by the batch size when the launch ends (``state``: two int64 words, zero when an epoch
+    starts).  Recorded in a HIP graph the launch draws batch after batch as the graph is replayed."""
+    n = x_src.shape[0]
+    batch = x_dst.shape[0]
+    for t in (x_src, y_src, x_dst, y_dst):
+        _need(t.is_cuda and t.is_contiguous(), 'the data set and the batch buffers must be contiguous GPU tensors')
+    _need(y_src.shape[0] == n and y_dst.shape[0] == batch and 1 <= batch <= n, 'samples and labels must agree in their first axis')
+    _need(x_dst.dtype == x_src.dtype and y_dst.dtype == y_src.dtype and x_dst.shape[1:] == x_src.shape[1:] and y_dst.shape[1:] == y_src.shape[1:],
+          'the batch buffers must have the data set\'s row shape and type')
+    _need(order.dtype == torch.int64 and order.is_cuda and order.is_contiguous() and order.numel() == n, 'order must hold one int64 per row')
+    _need(state.dtype == torch.int64 and state.is_cuda and state.numel() == 2, 'state must be two int64 words')
+    xb, yb = x_src[0].numel() * x_src.element_size(), y_src[0].numel() * y_src.element_size()
+    rc = _lib.load().hgq_gather_batch(_ptr(x_src), xb, _ptr(y_src), yb, _ptr(order), _ptr(state), _ptr(x_dst), _ptr(y_dst), batch, n, _stream())
+    _lib.check(rc, 'hgq_gather_batch')
+
+
+@gather_batch.register_fake
+def _(x_src, y_src, order, state, x_dst, y_dst):
+    return None
+
+
 def sparse_ce(logits: Tensor, labels: Tensor) -> Tensor:
     """Mean sparse categorical cross-entropy from logits."""
     return _SparseCE.apply(logits.contiguous(), labels)

@@ -145,21 +145,30 @@ class GraphedTrainStep:
     operations (``hgq2_amd.ops.sparse_ce`` is)."""
 
     def __init__(self, model, loss_fn, optimizer: SGD, example_x, example_y, warmup: int = 3, overlap: bool = True,
-                 warmup_data=None):
+                 warmup_data=None, feed: 'ResidentBatches | None' = None):
         """The recording is preceded by ``warmup`` real training steps on the example batch (operators create their
         per-stream scratch there, not inside the graph) - or, with ``warmup_data`` (a sequence of ``(x, y)`` of the
         example's shapes), by one step on each of those: a loop that counts its steps hands over its first batches and
-        starts replaying with the next one; their losses are left in ``warmup_losses``."""
+        starts replaying with the next one; their losses are left in ``warmup_losses``.
+
+        ``feed``: the step draws its batch itself (:class:`ResidentBatches`: a launch at the head of the recorded step
+        that reads the next rows of a data set in device memory) and adds its loss to ``total``; ``step()`` without
+        arguments is then a replay and nothing else.  The ``warmup`` steps draw the feed's first batches."""
         self.model, self.loss_fn, self.opt = model, loss_fn, optimizer
         self.overlap = overlap  # EBOPs launches and the loss sum on a second branch of the graph, beside loss and backward
+        self.feed = feed
         self.x = example_x.clone()
         self.y = example_y.clone()
+        self.total = torch.zeros((), dtype=torch.float32, device=example_x.device)  # with a feed: the sum of the steps' losses
         self.loss = None
         self.warmup_losses = []
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            if warmup_data is None:
+            if feed is not None:
+                for _ in range(warmup):
+                    self.warmup_losses.append(self._step().clone())
+            elif warmup_data is None:
                 for _ in range(warmup):
                     self._step()
             else:
@@ -180,13 +189,18 @@ class GraphedTrainStep:
     def _step(self):
         import contextlib
 
+        if self.feed is not None:
+            self.feed.draw(self.x, self.y)
         with ops.overlap_ebops() if self.overlap else contextlib.nullcontext():
             self.opt.zero_grad(set_to_none=True)
             out = self.model(self.x, training=True)
             loss = model_loss(self.model, self.loss_fn(out, self.y), self.opt.fold_regularizers)
             self.opt.backward(loss)
             self.opt.step()
-        return loss.detach()
+        loss = loss.detach()
+        if self.feed is not None:
+            self.total.add_(loss.reshape(()))
+        return loss
 
     def __call__(self, x=None, y=None):
         if x is not None:
@@ -199,12 +213,41 @@ class GraphedTrainStep:
 
     def eager(self, x, y):
         """The same step launched kernel by kernel on a batch of another size (the last, shorter batch of an epoch)."""
-        keep = self.x, self.y
-        self.x, self.y = x, y
+        keep = self.x, self.y, self.feed
+        self.x, self.y, self.feed = x, y, None
         try:
             return self._step()
         finally:
-            self.x, self.y = keep
+            self.x, self.y, self.feed = keep
+
+
+class ResidentBatches:
+    """The batches of an epoch loop over a data set that lives in device memory, drawn by a launch of their own
+    (``hgq_gather_batch``) so that a recorded step can fetch its batch when it is replayed: ``start_epoch(order)`` lays
+    down the epoch's order (a permutation of the rows, or ``None`` for the rows as they stand) and rewinds; every
+    ``draw(x_buf, y_buf)`` - eager or replayed - fills the buffers with the next ``x_buf.shape[0]`` rows of that order."""
+
+    def __init__(self, x, y):
+        if x.shape[0] != y.shape[0] or x.shape[0] < 1:
+            raise ValueError('x and y must hold the same, non-zero number of samples')
+        self.x, self.y = x.contiguous(), y.contiguous()
+        n = x.shape[0]
+        self._identity = torch.arange(n, dtype=torch.int64, device=x.device)
+        self.order = self._identity.clone()
+        self.state = torch.zeros(2, dtype=torch.int64, device=x.device)
+
+    @staticmethod
+    def covers(x, y) -> bool:
+        """Rows of whole 32-bit words on the GPU."""
+        return all(t.is_cuda and t.dim() >= 1 and t.shape[0] >= 1 and (t[0].numel() * t.element_size()) % 4 == 0 and t[0].numel() > 0
+                   for t in (x, y))
+
+    def start_epoch(self, order=None):
+        self.order.copy_(self._identity if order is None else order)
+        self.state.zero_()
+
+    def draw(self, x_buf, y_buf):
+        ops.gather_batch(self.x, self.y, self.order, self.state, x_buf, y_buf)
 
 
 _version_of = operator.attrgetter('_version')
@@ -366,7 +409,7 @@ class _FusedStep:
 
 
 def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 'sparse_ce', fused: bool | None = None,
-                   warmup_data=None):
+                   warmup_data=None, feed=None, warmup: int = 3):
     """A callable ``step(x, y) -> loss`` that runs one SGD training step of ``model`` on the fastest path that covers it.
 
     A built stack of :class:`QDense` layers trained with mean sparse categorical cross-entropy and within what
@@ -376,8 +419,8 @@ def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 's
     variables with the same arithmetic (the whole-step kernels restate the per-layer sequence), so the choice changes
     the time per step and nothing else.  ``fused=False`` forces the per-layer path, ``fused=True`` raises where the
     whole-step path does not apply.  The returned object's ``path`` is ``'fused'`` or ``'layers_graph'``.
-    ``warmup_data``: see :class:`GraphedTrainStep` (the whole-step path needs no steps before it and takes none:
-    ``warmup_losses`` is then empty)."""
+    ``warmup_data``, ``feed``, ``warmup``: see :class:`GraphedTrainStep` (the whole-step path needs no steps before it and
+    takes none: ``warmup_losses`` is then empty; it does not use a ``feed`` either)."""
     if loss not in ('sparse_ce', 'mse'):
         raise ValueError(f"loss must be 'sparse_ce' or 'mse', got {loss!r}")
     if not model.built:
@@ -400,7 +443,7 @@ def train_step_for(model, example_x, example_y, lr: float = 0.01, loss: str = 's
         raise ValueError('the fused QDense step computes sparse categorical cross-entropy only')
     loss_fn = ops.sparse_ce if loss == 'sparse_ce' else ops.mse
     step = GraphedTrainStep(model, loss_fn, SGD(model.parameters(), lr=lr, fold_regularizers=True), example_x, example_y,
-                            warmup_data=warmup_data)
+                            warmup=warmup, warmup_data=warmup_data, feed=feed)
     step.path = 'layers_graph'
     return step
 
@@ -427,7 +470,9 @@ def fit(model, x, y, *, loss: str = 'sparse_ce', lr: float = 0.01, batch_size: i
     The steps run on the fastest path that covers the model (:func:`train_step_for`): full batches through the
     whole-step kernels or a HIP-graph replay - the recording's preparatory steps are the loop's own first batches, so
     every batch is trained on exactly once - and a shorter last batch through the same kernels launched one by one.
-    The epoch's loss is summed on the device and read once per epoch.  On the per-layer path the MonoL1 terms of the
+    On the replayed path the recorded step fetches its own batch (:class:`ResidentBatches`: the epoch's order lies in
+    device memory and a launch at the head of the step gathers the next rows) and adds its loss to a running sum, so a
+    step costs the host one replay call.  The epoch's loss is summed on the device and read once per epoch.  On the per-layer path the MonoL1 terms of the
     variables are applied inside the update launch and are not part of a step's loss value: their sum
     (:func:`folded_regularizer_loss`, of the order of 1e-4 with the default 1e-8 factors) is added to ``logs['loss']``
     once, from the variables as they stand when the epoch ends; the whole-step kernels include it in every step."""
@@ -447,6 +492,8 @@ def fit(model, x, y, *, loss: str = 'sparse_ce', lr: float = 0.01, batch_size: i
         cb.on_train_begin({})
     step = None
     history = []
+    # a data set of whole 32-bit words per row is fed by a launch inside the recorded step (no copies between replays)
+    feed = ResidentBatches(x, y) if (fused is not True and ResidentBatches.covers(x, y)) else None
     for epoch in range(epochs):
         logs: dict = {}
         for cb in callbacks:
@@ -462,16 +509,26 @@ def fit(model, x, y, *, loss: str = 'sparse_ce', lr: float = 0.01, batch_size: i
 
         total = torch.zeros((), dtype=torch.float32, device=x.device)
         first = 0
+        if feed is not None:
+            feed.start_epoch(order)
         if step is None:
             # the steps before the recording are this epoch's first batches
             warm = [batch(b) for b in range(min(3, n_full))]
-            step = train_step_for(model, *warm[0], lr=lr, loss=loss, fused=fused, warmup_data=warm)
+            step = train_step_for(model, *warm[0], lr=lr, loss=loss, fused=fused, warmup_data=warm, feed=feed, warmup=len(warm))
+            if isinstance(step, _FusedStep):
+                feed = None  # the whole-step kernels read the batch where it lies
             done = getattr(step, 'warmup_losses', [])
             for l in done:
                 total += l.reshape(())
             first = len(done)
-        for b in range(first, n_full):
-            total += step(*batch(b)).reshape(())
+        if feed is not None:
+            step.total.zero_()
+            for b in range(first, n_full):
+                step()
+            total += step.total
+        else:
+            for b in range(first, n_full):
+                total += step(*batch(b)).reshape(())
         if tail:
             bx, by = batch(n_full, tail)
             if isinstance(step, _FusedStep):

@@ -458,6 +458,19 @@ int hgq_sparse_ce_fwd_bwd(const float *logits, const int64_t *labels, float *los
                           int C, uint32_t *state, void *stream);
 
 /*
+ * The batch feed of an epoch loop over a data set that lives in device memory (what `model.fit(x, y, batch_size=,
+ * shuffle=)` of the reference's users does on the host, reference tests/base.py:313-331): row r of the batch =
+ * row order[pos + r] of the source, for the samples (x_row_bytes per row) and the labels (y_row_bytes per row; 0 and NULL
+ * pointers: none) alike; pos = the first of the two 64-bit words of `state`, moved on by `batch` when the launch ends, so
+ * that a launch recorded in a HIP graph draws batch after batch as the graph is replayed.  The caller writes the
+ * permutation (or 0 .. n_rows - 1) into `order` and zeroes `state` when an epoch starts, and launches at most
+ * n_rows / batch times per epoch; positions past the end read the last row.  Row sizes are multiples of 4 bytes;
+ * `order` and `state` 8-byte aligned.  Launches that share `state` must not overlap in time.
+ */
+int hgq_gather_batch(const void *x_src, int64_t x_row_bytes, const void *y_src, int64_t y_row_bytes, const int64_t *order, void *state,
+                     void *x_dst, void *y_dst, int64_t batch, int64_t n_rows, void *stream);
+
+/*
  * Plain SGD update with the reference's post-update constraint and MonoL1 regulariser folded in.
  * Replaces `optimizer.apply` + Constraint.__call__ (src/hgq/constraints/__init__.py:19-21) +
  * the gradient of MonoL1 (src/hgq/regularizers/__init__.py:13-14) for one variable:

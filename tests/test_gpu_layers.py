@@ -935,9 +935,48 @@ def test_output_quantizer_inside_the_dense_kernel(dev, kind):
         assert err <= 2e-5 * (gb[n].abs().max().item() + 1e-6), (n, err)
 
 
-@pytest.mark.parametrize('fused', [False, None])
-def test_fit_trains_every_batch_once_on_the_fast_path(dev, fused):
-    """`train.fit`: epochs of full batches through the recorded step (or the whole-step kernels) plus a shorter last
+@pytest.mark.parametrize('rows,row_shape,dtype,batch', [(1000, (16,), torch.float32, 128), (77, (3, 5), torch.float32, 10),
+                                                        (300, (7,), torch.int32, 64), (64, (4,), torch.float32, 64)])
+def test_batch_feed_draws_the_rows_of_the_order_in_turn(dev, rows, row_shape, dtype, batch):
+    """``ops.gather_batch`` (``hgq_gather_batch``): successive launches fill the buffers with rows
+    ``order[0:batch]``, ``order[batch:2 batch]``, ... of the samples and the labels, eagerly and as a replayed graph."""
+    from hgq2_amd import ops
+    from hgq2_amd.train import ResidentBatches
+
+    g = torch.Generator().manual_seed(rows)
+    x = (torch.randn((rows,) + row_shape, generator=g) * 100).to(dtype).to(dev)
+    y = torch.randint(0, 9, (rows,), generator=g).to(dev)
+    feed = ResidentBatches(x, y)
+    xb, yb = torch.empty((batch,) + row_shape, dtype=dtype, device=dev), torch.empty(batch, dtype=torch.int64, device=dev)
+    for order in (None, torch.randperm(rows, generator=g).to(dev)):
+        feed.start_epoch(order)
+        idx = torch.arange(rows, device=dev) if order is None else order
+        for b in range(rows // batch):
+            feed.draw(xb, yb)
+            sel = idx[b * batch:(b + 1) * batch]
+            assert torch.equal(xb, x[sel]) and torch.equal(yb, y[sel]), (order is None, b)
+        assert int(feed.state[0]) == (rows // batch) * batch and int(feed.state[1]) == 0
+    # recorded once, replayed: every replay draws the next batch
+    feed.start_epoch(None)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        feed.draw(xb, yb)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        feed.draw(xb, yb)
+    for b in range(1, rows // batch):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(xb, x[b * batch:(b + 1) * batch]) and torch.equal(yb, y[b * batch:(b + 1) * batch]), b
+
+
+@pytest.mark.parametrize('fused,shuffle', [(False, False), (None, False), (False, True)])
+def test_fit_trains_every_batch_once_on_the_fast_path(dev, fused, shuffle):
+    """`train.fit`: epochs of full batches (in the rows' order, or shuffled anew per epoch) through the recorded step - which
+    draws its own batches from the data set in device memory - or the whole-step kernels, plus a shorter last
     batch, hooks in Keras' order.  On the per-layer path the variables equal those of the same steps launched one by one,
     bit for bit and the logged losses agree to 1e-6 (a sum on the device against a sum on the host); on the whole-step path
     (same arithmetic restated) the epoch losses agree to 1e-5 and the variables to 1e-4 of their largest entry."""
@@ -967,21 +1006,26 @@ def test_fit_trains_every_batch_once_on_the_fast_path(dev, fused):
             calls.append(f'end{epoch}')
 
     betas = [1e-5, 3e-5]
-    history = fit(model, x, y, lr=0.01, batch_size=bs, epochs=2, shuffle=False, fused=fused,
+    history = fit(model, x, y, lr=0.01, batch_size=bs, epochs=2, shuffle=shuffle, seed=5, fused=fused,
                   callbacks=[Spy(), BetaScheduler(lambda e: betas[e]), FreeEBOPs()])
     assert calls == ['train', 'begin0', 'end0', 'begin1', 'end1']
     assert [h['beta'] for h in history] == betas and all(h['ebops'] > 0 for h in history)
 
     opt = SGD(twin.parameters(), lr=0.01, fold_regularizers=True)
     want = []
+    gen = torch.Generator().manual_seed(5)  # the loop's own generator: one permutation per epoch
     for e in range(2):
         for layer in twin.layers:
             layer._beta.fill_(betas[e])
         total = 0.0
+        xe, ye = x, y
+        if shuffle:
+            order = torch.randperm(n, generator=gen).to(dev)
+            xe, ye = x[order], y[order]
         for lo in range(0, n, bs):
             opt.zero_grad()
             with ops.overlap_ebops():
-                loss = model_loss(twin, ops.sparse_ce(twin(x[lo:lo + bs], training=True), y[lo:lo + bs]), True)
+                loss = model_loss(twin, ops.sparse_ce(twin(xe[lo:lo + bs], training=True), ye[lo:lo + bs]), True)
                 opt.backward(loss)
                 opt.step()
             total += float(loss.detach())
