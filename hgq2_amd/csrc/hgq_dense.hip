@@ -641,9 +641,11 @@ __device__ __forceinline__ floatx16 bf16_chain(floatx16 acc, bf16_planes_t xp, i
 // OQ: the layer's output quantizer (training-mode WRAP: round only, [Po, N] table of fractional bits, same round mode)
 // runs on the output tile as it leaves: `y` gets the contraction, `yq` its quantized values, slice blockIdx.x of
 // `oamax_part` the abs-max of the quantized values per table entry.
-// ymean (mean_rows = 32 or 64, rows a multiple of it, 128-bit output rows): row g of `ymean` [rows / mean_rows, N] = the
-// mean of the activated output rows g * mean_rows .. (g + 1) * mean_rows - 1, taken from the accumulator registers as the
-// tile leaves (a tile holds two groups or one): sixteen rows per lane in order, the two lane halves, then the two row halves.
+// ymean (mean_rows = 32 or 64, rows a multiple of it): the output itself is not written; row g of `ymean`
+// [rows / mean_rows, N] = the mean of the activated output rows g * mean_rows .. (g + 1) * mean_rows - 1, taken from the
+// accumulator registers (a tile holds two groups or one): sixteen rows per lane in order, the two lane halves, then the two
+// row halves.  With ReLU, `relu_mask` [rows][2] gets a bit per output - bit c & 31 of word c >> 5 of a row says that column c
+// was positive - which is all the backward pass needs of the output.
 template <int RM, bool QUANT, int NS, bool OQ = false>
 __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw,
@@ -652,11 +654,14 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
                                                               int mode, const float *__restrict__ f_out = nullptr, int Po = 1,
                                                               int mode_out = 0, float *__restrict__ yq = nullptr,
                                                               uint32_t *oamax_part = nullptr, float *__restrict__ ymean = nullptr,
-                                                              int mean_rows = 0) {
+                                                              int mean_rows = 0, uint32_t *__restrict__ relu_mask = nullptr) {
     // [buffer][part][row][k]; row FAST_BM: sink of the idle staging slots
     __shared__ __attribute__((aligned(16))) uint16_t xp[2][3][FAST_BM + 1][BF_LD];
     __shared__ __attribute__((aligned(16))) float ys[FAST_BM][FAST_XLD];
-    __shared__ float msum[2][64];  // ymean: column sums of the two row halves of the tile
+    // ymean: column sums of the two row halves of a tile and the tile's ReLU mask words (written out as one contiguous run);
+    // two sets in turn - a tile's set is written out behind the NEXT tile's staging barrier, so the tile needs no barrier of its own
+    __shared__ float msum[2][2][64];
+    __shared__ uint32_t mtile[2][FAST_BM][2];
     // bit 0 / 1: the staged tile has a non-zero second / third part.  Three slots in rotation: the slot of the tile after
     // next is cleared behind this tile's barrier - its last readers passed that barrier, its next writers come after the next one
     __shared__ uint32_t need[3];
@@ -726,6 +731,21 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     DB_STAMP(0, 1);
     int buf = 0, slot = 0;
     [[maybe_unused]] int it_ = 0;
+    // ymean: the means and mask words of tile `t`, from set `set` (threads 0 - 127)
+    int64_t mean_tile = -1;
+    int mean_set = 0;
+    auto write_means = [&](int64_t t, int set) __attribute__((always_inline)) {
+        if (tid < 2 * 64) {
+            const int64_t t0 = t * FAST_BM;
+            if (relu_mask && act == HGQ_ACT_RELU && t0 + (tid >> 1) < rows) relu_mask[t0 * 2 + tid] = (&mtile[set][0][0])[tid];
+            const int c = tid & 63, h = tid >> 6;
+            if (mean_rows == FAST_BM) {
+                if (h == 0 && c < N) ymean[t * N + c] = (msum[set][0][c] + msum[set][1][c]) * (1.0f / FAST_BM);
+            } else if (c < N && t0 + h * 32 < rows) {
+                ymean[(2 * t + h) * N + c] = msum[set][h][c] * (1.0f / 32);
+            }
+        }
+    };
     for (; tile < n_tiles; tile += gridDim.x, buf ^= 1, slot = slot == 2 ? 0 : slot + 1, ++it_) {
         int fi[FAST_NJ][4];
 #pragma unroll
@@ -741,37 +761,47 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         if (tid == 0) need[slot == 0 ? 2 : slot - 1] = 0u;  // (slot + 2) % 3
         const int64_t next = tile + gridDim.x;
         if (next < n_tiles) load_tile(next);
+        if (ymean && mean_tile >= 0) write_means(mean_tile, mean_set ^ 1);
         floatx16 acc = {0};
         if (cb * 32 < N) {
             acc = bf16_chain<NS>(acc, xp[buf], arow, kq, need[slot], wp, PW);
         }
         DB_STAMP(0, 4 + 6 * it_);
         const int64_t r0 = tile * FAST_BM;
-        if (vec_out) {
+        if (ymean) {
+            // no branch inside the loop: the mask words are formed whatever the activation and only written out with ReLU
+            const bool relu = act == HGQ_ACT_RELU;
             float csum = 0.f;
+            uint32_t word[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = acc[r] + bias;
+                const bool pos = v > 0.f;
+                v = (relu && !pos) ? 0.f : v;
+                // lanes 0 - 31 hold 32 columns of one row, lanes 32 - 63 the same columns of the row four below
+                const unsigned long long bits = __ballot(pos);
+                word[r] = lane >= 32 ? (uint32_t)(bits >> 32) : (uint32_t)bits;
+                csum += v;
+            }
+            if ((lane & 31) == 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mtile[mean_set][rh * 32 + acc_row(r, lane)][cb] = word[r];
+            }
+            csum += __shfl_xor(csum, 32);
+            if (lane < 32) msum[mean_set][rh][bcol] = csum;
+            // written out behind the next tile's staging barrier (or the one after the loop); this set is written again two
+            // tiles on, behind a barrier that the threads who read it now have passed
+            mean_tile = tile, mean_set ^= 1;
+        } else if (vec_out) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 float v = acc[r] + bias;
                 if (act == HGQ_ACT_RELU) v = v > 0.f ? v : 0.f;
                 ys[rh * 32 + acc_row(r, lane)][bcol] = v;
-                csum += v;
-            }
-            if (ymean) {
-                csum += __shfl_xor(csum, 32);
-                if (lane < 32) msum[rh][bcol] = csum;
             }
             DB_STAMP(0, 5 + 6 * it_);
             __syncthreads();
             DB_STAMP(0, 6 + 6 * it_);
-            // (the next tile's sums are written behind its staging barrier, which these reads precede)
-            if (ymean && tid < 2 * 64) {
-                const int c = tid & 63, h = tid >> 6;
-                if (mean_rows == FAST_BM) {
-                    if (h == 0 && c < N) ymean[tile * N + c] = (msum[0][c] + msum[1][c]) * (1.0f / FAST_BM);
-                } else if (c < N && r0 + h * 32 < rows) {
-                    ymean[(2 * tile + h) * N + c] = msum[h][c] * (1.0f / 32);
-                }
-            }
 #pragma unroll
             for (int j = 0; j < FAST_NJ; ++j) {
                 const int64_t gr = r0 + mo.row[j];
@@ -807,6 +837,10 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         }
     }
     DB_STAMP(0, 30);
+    if (ymean && mean_tile >= 0) {
+        __syncthreads();
+        write_means(mean_tile, mean_set ^ 1);
+    }
     if (QUANT && amax_part && P == FAST_BM && ((uintptr_t)amax_part & 15u) == 0) {
         uint32_t *my = amax_part + (int64_t)blockIdx.x * (P * K);
 #pragma unroll
@@ -1020,7 +1054,8 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bf16_kernel(const float 
 // taken in all three parts without looking, the quantized input and the kernel in as many as they need.
 // BCAST (32 or 64, not with STATS, ZVEC only, rows a multiple of it; `bcast` below): the output went through a mean over groups of `bcast` rows
 // and dy is the gradient of those means, [rows / bcast, N]: row r of the gradient tile is dy[r / bcast] / bcast, read with a
-// zero row stride instead of from a broadcast copy.
+// zero row stride instead of from a broadcast copy; `y` is then not the output but its ReLU mask, two 32-bit words per row
+// (what the forward kernel leaves when it writes the means instead of the output).
 // PAIRS (with BF; K and N above 32): wavefronts 0 and 1 take the two row halves of dx (both k blocks: the gradient rows they
 // contract are split into bf16 parts once for both), wavefronts 2 and 3 the two column halves of the kernel gradient (both k
 // blocks, all rows of the tile) - every gradient value is split twice per tile instead of four times.  A wavefront's two
@@ -1086,7 +1121,8 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
         const __amdgpu_buffer_rsrc_t sg = STATS ? buf_rsrc(has_add ? dx_add + r0 * K : x, has_add ? vr * K * 4 : 0)
                                           : bcast ? buf_rsrc(dy + (r0 / bcast) * N, ((vr + bcast - 1) / bcast) * N * 4)
                                                   : buf_rsrc(dy + r0 * N, vr * N * 4);
-        const __amdgpu_buffer_rsrc_t sy = buf_rsrc((relu && !STATS) ? y + r0 * N : x, (relu && !STATS) ? vr * N * 4 : 0);
+        const __amdgpu_buffer_rsrc_t sy = bcast ? buf_rsrc(relu ? y + r0 * 2 : x, relu ? vr * 2 * 4 : 0)
+                                                : buf_rsrc((relu && !STATS) ? y + r0 * N : x, (relu && !STATS) ? vr * N * 4 : 0);
 #pragma unroll
         for (int j = 0; j < FAST_NJ; ++j) {
             rx[j] = buf_ld4(sx, xoff[j]);
@@ -1096,7 +1132,8 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                     const uint32_t goff = !bcast ? zoff[j]
                                           : mz.on[j] ? (uint32_t)((bcast == 32 ? (mz.row[j] >> 5) : 0) * N + mz.col[j]) * 4u : BUF_OOB;
                     rg[j] = buf_ld4(sg, goff);
-                    ry[j] = buf_ld4(sy, zoff[j]);
+                    if (bcast) ry[j][0] = buf_ld1(sy, mz.on[j] ? (uint32_t)(mz.row[j] * 2 + (mz.col[j] >> 5)) * 4u : BUF_OOB);  // mask word
+                    else ry[j] = buf_ld4(sy, zoff[j]);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -1165,8 +1202,12 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
             } else {
                 const float g[4] = {rg[j][0], rg[j][1], rg[j][2], rg[j][3]};
                 const float a[4] = {ry[j][0], ry[j][1], ry[j][2], ry[j][3]};
+                const uint32_t mbits = __float_as_uint(ry[j][0]) >> (mz.col[j] & 31);  // (BCAST: the mask word of this row and column block)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) dzs[zr][mz.col[j] + e] = (!relu || a[e] > 0.f) ? g[e] * gscale : 0.f;
+                for (int e = 0; e < 4; ++e) {
+                    const bool live = !relu || (bcast ? ((mbits >> e) & 1u) != 0u : a[e] > 0.f);
+                    dzs[zr][mz.col[j] + e] = live ? g[e] * gscale : 0.f;
+                }
             }
         }
         DB_STAMP(1, 3 + 6 * it_);
@@ -1971,26 +2012,27 @@ extern "C" int hgq_qdense_fwd_mean_supported(int64_t rows, int K, int N, int64_t
                        64 % bw_rows == 0 && rows % bw_rows == 0));
 }
 
-extern "C" int hgq_qdense_fwd_mean(const float *x, const float *f_in, int64_t bw_rows, const float *qw, const float *qb, float *y,
-                                   float *ymean, uint32_t *amax_part, int64_t rows, int K, int N, int64_t mean_rows, int act, int mode,
-                                   void *stream) {
+extern "C" int hgq_qdense_fwd_mean(const float *x, const float *f_in, int64_t bw_rows, const float *qw, const float *qb,
+                                   uint32_t *relu_mask, float *ymean, uint32_t *amax_part, int64_t rows, int K, int N, int64_t mean_rows,
+                                   int act, int mode, void *stream) {
     hipStream_t s = (hipStream_t)stream;
     if (rows == 0) return HGQ_OK;
     if (bw_rows < 0 || !hgq_qdense_fwd_mean_supported(rows, K, N, bw_rows, mean_rows, mode))
         return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_fwd_mean: shape or mode outside the fused group mean (see hgq_qdense_fwd_mean_supported)");
-    if (!x || !qw || !y || !ymean || (bw_rows > 0 && !f_in)) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: null pointer");
+    if (!x || !qw || !ymean || (bw_rows > 0 && !f_in)) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: null pointer");
     if (act != HGQ_ACT_NONE && act != HGQ_ACT_RELU) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: unknown activation %d", act);
-    if (!aligned16(x) || !aligned16(y)) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: x and y must be 16-byte aligned");
+    if (act == HGQ_ACT_RELU && !relu_mask) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: a ReLU needs the mask array");
+    if (!aligned16(x)) return fail(HGQ_ERR_ARG, "hgq_qdense_fwd_mean: x must be 16-byte aligned");
     const Mode m(mode);
     const bool quant = bw_rows > 0;
     const dim3 fgrid((unsigned)row_parts(rows, FWD_BM));
     const int P = quant ? (int)bw_rows : 1, mr = (int)mean_rows;
 #define HGQ_FWD_MEAN(NSV) \
     do { \
-        if (!quant) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, false, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, (uint32_t *)nullptr, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
-        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
-        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
-        else hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND_CONV, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, y, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr); \
+        if (!quant) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, false, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, (uint32_t *)nullptr, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
+        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
+        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
+        else hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND_CONV, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
     } while (0)
     if (K <= 16) HGQ_FWD_MEAN(1);
     else if (K <= 32) HGQ_FWD_MEAN(2);
@@ -2142,7 +2184,7 @@ static int qdense_bwd_impl(const float *dy, const float *y, const float *x, cons
         const int parts = row_parts(rows, BWD_BM);
         const int P = quant ? (int)bw_rows : 1;
         const dim3 fgrid((unsigned)parts);
-        const bool zvec = N % 4 == 0 && aligned16(dy) && (act != HGQ_ACT_RELU || aligned16(y));
+        const bool zvec = N % 4 == 0 && aligned16(dy) && (act != HGQ_ACT_RELU || bcast || aligned16(y));
         if (bcast && !(zvec && g_dense_bf16))
             return fail(HGQ_ERR_UNSUPPORTED, "hgq_qdense_bwd_mean: needs the bf16 matrix instruction, N a multiple of 4 and 16-byte aligned gradients");
 #define HGQ_BWD_BCAST(RMV, QV, BC)                                                                                                     \
@@ -2235,19 +2277,20 @@ extern "C" int hgq_qdense_bwd(const float *dy, const float *y, const float *x, c
     return qdense_bwd_impl(dy, y, x, f_in, bw_rows, qw, dx, dqw, dqb, df_in, workspace, rows, K, N, act, mode, stream, true);
 }
 
-extern "C" int hgq_qdense_bwd_mean(const float *dmean, const float *y, const float *x, const float *f_in, int64_t bw_rows, const float *qw,
+extern "C" int hgq_qdense_bwd_mean(const float *dmean, const uint32_t *relu_mask, const float *x, const float *f_in, int64_t bw_rows, const float *qw,
                                    float *dx, float *dqw, float *dqb, float *df_in, float *workspace, int64_t rows, int K, int N,
                                    int64_t mean_rows, int act, int mode, void *stream) {
     if (mean_rows <= 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd_mean: mean_rows must be positive");
-    return qdense_bwd_impl(dmean, y, x, f_in, bw_rows, qw, dx, dqw, dqb, df_in, workspace, rows, K, N, act, mode, stream, true, mean_rows);
+    return qdense_bwd_impl(dmean, (const float *)relu_mask, x, f_in, bw_rows, qw, dx, dqw, dqb, df_in, workspace, rows, K, N, act, mode, stream, true,
+                           mean_rows);
 }
 
-extern "C" int hgq_qdense_bwd_mean_slices(const float *dmean, const float *y, const float *x, const float *f_in, int64_t bw_rows,
+extern "C" int hgq_qdense_bwd_mean_slices(const float *dmean, const uint32_t *relu_mask, const float *x, const float *f_in, int64_t bw_rows,
                                           const float *qw, float *dx, float *workspace, int has_bias, int64_t rows, int K, int N,
                                           int64_t mean_rows, int act, int mode, void *stream) {
     if (mean_rows <= 0) return fail(HGQ_ERR_ARG, "hgq_qdense_bwd_mean_slices: mean_rows must be positive");
-    return qdense_bwd_impl(dmean, y, x, f_in, bw_rows, qw, dx, nullptr, has_bias ? workspace : nullptr, nullptr, workspace, rows, K, N, act, mode,
-                           stream, false, mean_rows);
+    return qdense_bwd_impl(dmean, (const float *)relu_mask, x, f_in, bw_rows, qw, dx, nullptr, has_bias ? workspace : nullptr, nullptr, workspace, rows,
+                           K, N, act, mode, stream, false, mean_rows);
 }
 
 extern "C" int hgq_qdense_bwd_slices(const float *dy, const float *y, const float *x, const float *f_in, int64_t bw_rows,

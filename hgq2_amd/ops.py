@@ -353,11 +353,18 @@ def _(dy, y, x, f_in, qw, has_bias, act, mode, bw_rows):
     return torch.empty_like(x), x.new_empty((max(1, -(-x.shape[0] // 64)), K * N + N + bw_rows * K))
 
 
+def _check_relu_mask(mask: Tensor, rows: int, act: int) -> None:
+    if act == _lib.ACT_RELU:
+        _need(mask.is_cuda and mask.dtype == torch.int32 and mask.is_contiguous() and tuple(mask.shape) == (rows, 2),
+              'the ReLU mask must be the [rows, 2] int32 tensor the forward pass left')
+
+
 @torch.library.custom_op('hgq::qdense_fwd_mean', mutates_args=())
 def qdense_fwd_mean(x: Tensor, k_in: Tensor, f_in: Tensor, qw: Tensor, qb: Tensor, act: int, mode: int, bw_rows: int,
                     mean_rows: int) -> tuple[Tensor, Tensor, Tensor]:
-    """``qdense_fwd`` and the mean over groups of ``mean_rows`` consecutive output rows in one launch:
-    ``(y [rows, N], group means [rows / mean_rows, N], amax slices of the input quantizer)``."""
+    """``qdense_fwd`` and the mean over groups of ``mean_rows`` consecutive output rows in one launch; the output itself is not
+    written: ``(ReLU mask [rows, 2] - a bit per output, empty without ReLU -, group means [rows / mean_rows, N], amax slices of
+    the input quantizer)``."""
     _check_f32('x', x), _check_f32('qw', qw)
     _need(x.dim() == 2 and qw.dim() == 2 and x.shape[1] == qw.shape[0], f'shape mismatch {tuple(x.shape)} @ {tuple(qw.shape)}')
     rows, K = x.shape
@@ -371,67 +378,70 @@ def qdense_fwd_mean(x: Tensor, k_in: Tensor, f_in: Tensor, qw: Tensor, qb: Tenso
         mode = _kmode(mode, k_in)
     _need(mean_rows > 0 and rows % mean_rows == 0, 'rows must be a multiple of mean_rows')
     lib = _lib.load()
-    y = torch.empty((rows, N), dtype=torch.float32, device=x.device)
+    mask = torch.empty((rows if act == _lib.ACT_RELU else 0, 2), dtype=torch.int32, device=x.device)
     ymean = torch.empty((rows // mean_rows, N), dtype=torch.float32, device=x.device)
     amax = torch.empty((lib.hgq_qdense_fwd_parts(rows) if bw_rows > 0 else 0, bw_rows * K), dtype=torch.int32, device=x.device)
-    rc = lib.hgq_qdense_fwd_mean(_ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(qb), _ptr(y), _ptr(ymean), _ptr(amax), rows, K, N, mean_rows,
+    rc = lib.hgq_qdense_fwd_mean(_ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(qb), _ptr(mask), _ptr(ymean), _ptr(amax), rows, K, N, mean_rows,
                                  act, mode, _stream())
     _lib.check(rc, 'hgq_qdense_fwd_mean')
-    return y, ymean, amax
+    return mask, ymean, amax
 
 
 @qdense_fwd_mean.register_fake
 def _(x, k_in, f_in, qw, qb, act, mode, bw_rows, mean_rows):
     rows, N = x.shape[0], qw.shape[1]
-    return x.new_empty((rows, N)), x.new_empty((rows // mean_rows, N)), x.new_empty((1 if bw_rows > 0 else 0, f_in.numel()), dtype=torch.int32)
+    return (x.new_empty((rows if act == _lib.ACT_RELU else 0, 2), dtype=torch.int32), x.new_empty((rows // mean_rows, N)),
+            x.new_empty((1 if bw_rows > 0 else 0, f_in.numel()), dtype=torch.int32))
 
 
 @torch.library.custom_op('hgq::qdense_bwd_mean', mutates_args=())
-def qdense_bwd_mean(dmean: Tensor, y: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_bias: bool, act: int, mode: int,
+def qdense_bwd_mean(dmean: Tensor, mask: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_bias: bool, act: int, mode: int,
                     bw_rows: int, mean_rows: int) -> tuple[Tensor, Tensor, Tensor, Tensor]:
-    """``qdense_bwd`` from the gradient of the group means ``dmean`` [rows / mean_rows, N]."""
-    _check_f32('dmean', dmean), _check_f32('x', x), _check_f32('qw', qw), _check_f32('y', y)
+    """``qdense_bwd`` from the gradient of the group means ``dmean`` [rows / mean_rows, N] and the forward's ReLU mask."""
+    _check_f32('dmean', dmean), _check_f32('x', x), _check_f32('qw', qw)
     rows, K = x.shape
     N = qw.shape[1]
     _need(mean_rows > 0 and rows % mean_rows == 0 and tuple(dmean.shape) == (rows // mean_rows, N), 'dmean shape mismatch')
+    _check_relu_mask(mask, rows, act)
     lib = _lib.load()
     dx = torch.empty_like(x)
     dqw = torch.empty_like(qw)
     dqb = torch.empty(N if has_bias else 0, dtype=torch.float32, device=x.device)
     df = torch.empty(bw_rows * K, dtype=torch.float32, device=x.device)
     ws = torch.empty(lib.hgq_qdense_bwd_workspace(rows, K, N, bw_rows), dtype=torch.float32, device=x.device)
-    rc = lib.hgq_qdense_bwd_mean(_ptr(dmean), _ptr(y), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(dqw), _ptr(dqb), _ptr(df),
+    rc = lib.hgq_qdense_bwd_mean(_ptr(dmean), _ptr(mask), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(dqw), _ptr(dqb), _ptr(df),
                                  _ptr(ws), rows, K, N, mean_rows, act, mode, _stream())
     _lib.check(rc, 'hgq_qdense_bwd_mean')
     return dx, dqw, dqb, df
 
 
 @qdense_bwd_mean.register_fake
-def _(dmean, y, x, f_in, qw, has_bias, act, mode, bw_rows, mean_rows):
+def _(dmean, mask, x, f_in, qw, has_bias, act, mode, bw_rows, mean_rows):
     return (torch.empty_like(x), torch.empty_like(qw), x.new_empty(qw.shape[1] if has_bias else 0),
             x.new_empty(bw_rows * x.shape[1]))
 
 
 @torch.library.custom_op('hgq::qdense_bwd_mean_slices', mutates_args=())
-def qdense_bwd_mean_slices(dmean: Tensor, y: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_bias: bool, act: int, mode: int,
+def qdense_bwd_mean_slices(dmean: Tensor, mask: Tensor, x: Tensor, f_in: Tensor, qw: Tensor, has_bias: bool, act: int, mode: int,
                            bw_rows: int, mean_rows: int) -> tuple[Tensor, Tensor]:
-    """``qdense_bwd_slices`` from the gradient of the group means ``dmean`` [rows / mean_rows, N]."""
-    _check_f32('dmean', dmean), _check_f32('x', x), _check_f32('qw', qw), _check_f32('y', y)
+    """``qdense_bwd_slices`` from the gradient of the group means ``dmean`` [rows / mean_rows, N] and the forward's ReLU mask."""
+    _check_f32('dmean', dmean), _check_f32('x', x), _check_f32('qw', qw)
     rows, K = x.shape
     N = qw.shape[1]
     _need(mean_rows > 0 and rows % mean_rows == 0 and tuple(dmean.shape) == (rows // mean_rows, N), 'dmean shape mismatch')
+    _check_relu_mask(mask, rows, act)
     lib = _lib.load()
     dx = torch.empty_like(x)
     width = K * N + N + bw_rows * K
     ws = torch.empty((lib.hgq_qdense_bwd_workspace(rows, K, N, bw_rows) // width, width), dtype=torch.float32, device=x.device)
-    rc = lib.hgq_qdense_bwd_mean_slices(_ptr(dmean), _ptr(y), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(ws), int(has_bias), rows,
+    rc = lib.hgq_qdense_bwd_mean_slices(_ptr(dmean), _ptr(mask), _ptr(x), _ptr(f_in), bw_rows, _ptr(qw), _ptr(dx), _ptr(ws), int(has_bias), rows,
                                         K, N, mean_rows, act, mode, _stream())
     _lib.check(rc, 'hgq_qdense_bwd_mean_slices')
     return dx, ws
 
 
 @qdense_bwd_mean_slices.register_fake
-def _(dmean, y, x, f_in, qw, has_bias, act, mode, bw_rows, mean_rows):
+def _(dmean, mask, x, f_in, qw, has_bias, act, mode, bw_rows, mean_rows):
     K, N = x.shape[1], qw.shape[1]
     return torch.empty_like(x), x.new_empty((max(1, -(-x.shape[0] // 64)), K * N + N + bw_rows * K))
 
@@ -2174,13 +2184,14 @@ def qdense(x2d, k_in, i_in, f_in, qw, qb, act: int, mode: int, bw_rows: int, tra
 
 class _QDenseMean(torch.autograd.Function):
     """``_QDense`` followed by a mean over groups of ``mean_rows`` rows, as one launch each way: returns
-    ``(group means, amax slices)``; the contraction's own output stays inside (the backward pass reads it as the ReLU mask)."""
+    ``(group means, amax slices)``; the contraction's own output is never written (the backward pass reads a bit per output,
+    the ReLU mask, instead)."""
 
     @staticmethod
     def forward(ctx, x, k_in, f_in, qw, qb, act, mode, bw_rows, mean_rows):
-        y, ymean, amax = qdense_fwd_mean(x, k_in, f_in, qw, qb, act, mode, bw_rows, mean_rows)
+        mask, ymean, amax = qdense_fwd_mean(x, k_in, f_in, qw, qb, act, mode, bw_rows, mean_rows)
         ctx.f_owner = _owner(f_in)
-        ctx.save_for_backward(x, f_in, qw, y)
+        ctx.save_for_backward(x, f_in, qw, mask)
         ctx.has_bias = qb.numel() > 0
         ctx.defer = getattr(qw, '_hgq_single_use', False) and (qb.numel() == 0 or getattr(qb, '_hgq_single_use', False))
         ctx.act, ctx.mode, ctx.bw_rows, ctx.f_shape, ctx.mean_rows = act, _kmode(mode, k_in) if bw_rows > 0 else mode, bw_rows, f_in.shape, mean_rows
@@ -2192,14 +2203,14 @@ class _QDenseMean(torch.autograd.Function):
     def backward(ctx, gm, _ga):
         if gm is None:
             return (None,) * 9
-        x, f_in, qw, y = ctx.saved_tensors
+        x, f_in, qw, mask = ctx.saved_tensors
         if ctx.defer and _SINK['open'] and (ctx.bw_rows == 0 or _can_route(ctx.f_owner, ctx.bw_rows * x.shape[1])):
-            dx, ws = qdense_bwd_mean_slices(gm.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows, ctx.mean_rows)
+            dx, ws = qdense_bwd_mean_slices(gm.contiguous(), mask, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows, ctx.mean_rows)
             K, N = qw.shape
             dqw, dqb, df = torch.empty_like(qw), x.new_empty(N), x.new_empty(ctx.bw_rows * K)
             _PENDING_REDUCE.append((ws, (dqw, dqb, df), (False, not ctx.has_bias, False)))
         else:
-            dx, dqw, dqb, df = qdense_bwd_mean(gm.contiguous(), y, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows, ctx.mean_rows)
+            dx, dqw, dqb, df = qdense_bwd_mean(gm.contiguous(), mask, x, f_in, qw, ctx.has_bias, ctx.act, ctx.mode, ctx.bw_rows, ctx.mean_rows)
         df = _route(ctx.f_owner, df) if ctx.bw_rows > 0 else None
         return (dx, None, df.view(ctx.f_shape) if df is not None else None, dqw, dqb if ctx.has_bias else None, None, None, None, None)
 

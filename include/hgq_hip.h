@@ -306,26 +306,28 @@ int hgq_qdense_fwd(const float *x, const void *k_in, const float *i_in, const fl
  * hgq_qdense_fwd followed by a mean over groups of `mean_rows` consecutive rows, in one launch: a contraction layer whose
  * output [batch, positions, N] goes straight into a mean over the positions (reference src/hgq/layers/core/einsum_dense.py:72-83
  * and src/hgq/layers/einsum_dense_batchnorm.py:185-212 for the layer; the mean is the host framework's
- * GlobalAveragePooling1D behind it).  `y` [rows, N] is written as hgq_qdense_fwd writes it (the backward pass reads it as the
- * ReLU mask), row g of `ymean` [rows / mean_rows, N] = the mean of rows g * mean_rows .. (g + 1) * mean_rows - 1 of `y`, summed
- * in a fixed order from the accumulator registers.  `f_in` / `bw_rows` / `amax_part` as in hgq_qdense_fwd (bw_rows = 0: no
- * input quantizer).  Covers what hgq_qdense_fwd_mean_supported says: mean_rows 32 or 64 dividing the rows, K and N
- * multiples of 4 up to 64, the input quantizer none or KIF on its WRAP training branch with a table whose row count
+ * GlobalAveragePooling1D behind it).  The output itself is not written: row g of `ymean` [rows / mean_rows, N] = the mean of
+ * the activated output rows g * mean_rows .. (g + 1) * mean_rows - 1, summed in a fixed order from the accumulator registers,
+ * and with HGQ_ACT_RELU `relu_mask` [rows][2] (32-bit words) gets what the backward pass needs of the output: bit c & 31 of
+ * word c >> 5 of a row = column c was positive (NULL without ReLU).  `f_in` / `bw_rows` / `amax_part` as in hgq_qdense_fwd
+ * (bw_rows = 0: no input quantizer).  Covers what hgq_qdense_fwd_mean_supported says: mean_rows 32 or 64 dividing the rows,
+ * K and N multiples of 4 up to 64, the input quantizer none or KIF on its WRAP training branch with a table whose row count
  * divides 64 and the rows, the bf16-part kernels selected; HGQ_ERR_UNSUPPORTED otherwise (run hgq_qdense_fwd and
  * hgq_mean_mid_fwd then).
  *
  * hgq_qdense_bwd_mean / hgq_qdense_bwd_mean_slices: hgq_qdense_bwd / hgq_qdense_bwd_slices for that pair, from the gradient
- * of the means `dmean` [rows / mean_rows, N]: row r of the gradient the contraction sees is dmean[r / mean_rows] / mean_rows,
- * read from `dmean` directly (no [rows, N] broadcast copy is made).  All other arguments as in hgq_qdense_bwd(_slices).
+ * of the means `dmean` [rows / mean_rows, N] and the mask: row r of the gradient the contraction sees is
+ * dmean[r / mean_rows] / mean_rows where the mask bit is set (everywhere without ReLU), read from `dmean` directly (no
+ * [rows, N] broadcast copy is made).  All other arguments as in hgq_qdense_bwd(_slices).
  */
 int hgq_qdense_fwd_mean_supported(int64_t rows, int K, int N, int64_t bw_rows, int64_t mean_rows, int mode);
-int hgq_qdense_fwd_mean(const float *x, const float *f_in, int64_t bw_rows, const float *qw, const float *qb, float *y,
+int hgq_qdense_fwd_mean(const float *x, const float *f_in, int64_t bw_rows, const float *qw, const float *qb, uint32_t *relu_mask,
                         float *ymean, uint32_t *amax_part, int64_t rows, int K, int N, int64_t mean_rows, int act, int mode,
                         void *stream);
-int hgq_qdense_bwd_mean(const float *dmean, const float *y, const float *x, const float *f_in, int64_t bw_rows, const float *qw,
+int hgq_qdense_bwd_mean(const float *dmean, const uint32_t *relu_mask, const float *x, const float *f_in, int64_t bw_rows, const float *qw,
                         float *dx, float *dqw, float *dqb, float *df_in, float *workspace, int64_t rows, int K, int N,
                         int64_t mean_rows, int act, int mode, void *stream);
-int hgq_qdense_bwd_mean_slices(const float *dmean, const float *y, const float *x, const float *f_in, int64_t bw_rows,
+int hgq_qdense_bwd_mean_slices(const float *dmean, const uint32_t *relu_mask, const float *x, const float *f_in, int64_t bw_rows,
                                const float *qw, float *dx, float *workspace, int has_bias, int64_t rows, int K, int N,
                                int64_t mean_rows, int act, int mode, void *stream);
 
