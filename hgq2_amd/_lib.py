@@ -101,6 +101,7 @@ SIGNATURES = {
     'hgq_wrap_track_i_multi': (c_int, [c_void_p, c_int, c_void_p]),
     'hgq_qdense_bwd_slices': (c_int, [c_void_p] * 4 + [c_int64] + [c_void_p] * 3 + [c_int, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     'hgq_reduce_slices_multi': (c_int, [c_void_p, c_int, c_void_p]),
+    'hgq_reduce_slices_quant_multi': (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     'hgq_stream_probe': (c_int, [c_void_p] * 7 + [c_int, c_int, c_int64, c_void_p]),
     'hgq_quantize_bwd_static': (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_int64, c_int, c_void_p]),
     'hgq_quantize_fwd_bwd': (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_int64, c_int, c_void_p]),

@@ -1798,7 +1798,15 @@ struct ReduceBatch {
     int count;
 };
 
-__global__ __launch_bounds__(64 * RP_G) void reduce_parts_multi_kernel(const ReduceBatch b) {
+// quantizers whose upstream gradient IS a reduced segment (the kernel / bias quantizers behind a contraction): their surrogate
+// backward runs on the sum as it is formed; attach[t][o] = index into `item` for segment o of slice set t, or -1
+struct ReduceQuants {
+    hgq_quant_grad_item item[HGQ_REDUCE_QUANTS];
+    int8_t attach[HGQ_REDUCE_BATCH][3];
+};
+
+template <bool QUANTS>
+__global__ __launch_bounds__(64 * RP_G) void reduce_parts_multi_kernel(const ReduceBatch b, const ReduceQuants q) {
     __shared__ float red[64 * RP_G];
     int t = 0;
     while (t + 1 < b.count && (int)blockIdx.x >= b.first_block[t + 1]) ++t;
@@ -1833,6 +1841,18 @@ __global__ __launch_bounds__(64 * RP_G) void reduce_parts_multi_kernel(const Red
         for (int o = 0; o < 3; ++o) {
             if (off < it.n_out[o]) {
                 if (it.out[o]) it.out[o][off] = v;
+                if (QUANTS && q.attach[t][o] >= 0) {
+                    // (the arithmetic of quant_bwd_multi_kernel on dy = v)
+                    const hgq_quant_grad_item &qi = q.item[q.attach[t][o]];
+                    const Mode m(qi.mode);
+                    const KIF p = resolve_kif(load_k(qi.k, off, m.k_u8), qi.i[off], qi.fb[off], m.kbi, m.round_params);
+                    float gx, gi, gf;
+                    quantize_grad_dyn(qi.x[off], v, p, m.round_mode, m.overflow_mode, gx, gi, gf);
+                    if (m.kbi) gi -= gf;
+                    if (qi.dx) qi.dx[off] = gx;
+                    if (qi.di) qi.di[off] = gi;
+                    if (qi.dfb) qi.dfb[off] = gf;
+                }
                 break;
             }
             off -= it.n_out[o];
@@ -1840,28 +1860,58 @@ __global__ __launch_bounds__(64 * RP_G) void reduce_parts_multi_kernel(const Red
     }
 }
 
-extern "C" int hgq_reduce_slices_multi(const hgq_reduce_item *items, int count, void *stream) {
-    if (count < 0 || (count > 0 && !items)) return fail(HGQ_ERR_ARG, "hgq_reduce_slices_multi: bad arguments");
+static int reduce_slices_impl(const hgq_reduce_item *items, int count, const hgq_quant_grad_item *quants, const int *quant_set,
+                              const int *quant_segment, int n_quants, void *stream) {
+    const char *who = n_quants ? "hgq_reduce_slices_quant_multi" : "hgq_reduce_slices_multi";
+    if (count < 0 || (count > 0 && !items) || n_quants < 0 || (n_quants > 0 && (!quants || !quant_set || !quant_segment)))
+        return fail(HGQ_ERR_ARG, "%s: bad arguments", who);
+    for (int j = 0; j < n_quants; ++j) {
+        const hgq_quant_grad_item &qi = quants[j];
+        if (quant_set[j] < 0 || quant_set[j] >= count || quant_segment[j] < 0 || quant_segment[j] > 2 || !qi.x || !qi.k || !qi.i || !qi.fb ||
+            qi.n != items[quant_set[j]].n_out[quant_segment[j]])
+            return fail(HGQ_ERR_ARG, "%s: quantizer %d does not fit the segment it is attached to", who, j);
+        if (!Mode(qi.mode).training) return fail(HGQ_ERR_ARG, "%s: quantizer %d: the surrogate gradient is defined for training mode only", who, j);
+    }
     for (int base = 0; base < count; base += HGQ_REDUCE_BATCH) {
         ReduceBatch b;
+        ReduceQuants q;
         b.count = count - base < HGQ_REDUCE_BATCH ? count - base : HGQ_REDUCE_BATCH;
+        for (int t = 0; t < HGQ_REDUCE_BATCH; ++t) q.attach[t][0] = q.attach[t][1] = q.attach[t][2] = -1;
+        int nq = 0;
+        for (int j = 0; j < n_quants; ++j) {
+            if (quant_set[j] < base || quant_set[j] >= base + b.count) continue;
+            if (nq == HGQ_REDUCE_QUANTS) return fail(HGQ_ERR_UNSUPPORTED, "%s: more than %d quantizers on %d slice sets", who, HGQ_REDUCE_QUANTS, HGQ_REDUCE_BATCH);
+            if (q.attach[quant_set[j] - base][quant_segment[j]] >= 0) return fail(HGQ_ERR_ARG, "%s: two quantizers on one segment", who);
+            q.attach[quant_set[j] - base][quant_segment[j]] = (int8_t)nq;
+            q.item[nq++] = quants[j];
+        }
         int64_t blocks = 0;
         for (int t = 0; t < b.count; ++t) {
             const hgq_reduce_item &it = items[base + t];
-            if (it.n_slices < 1 || it.width < 1 || !it.slices) return fail(HGQ_ERR_ARG, "hgq_reduce_slices_multi: bad sizes in item %d", base + t);
+            if (it.n_slices < 1 || it.width < 1 || !it.slices) return fail(HGQ_ERR_ARG, "%s: bad sizes in item %d", who, base + t);
             if (it.n_out[0] < 0 || it.n_out[1] < 0 || it.n_out[2] < 0 || it.n_out[0] + it.n_out[1] + it.n_out[2] != it.width)
-                return fail(HGQ_ERR_ARG, "hgq_reduce_slices_multi: item %d: output lengths do not add up to the slice width", base + t);
+                return fail(HGQ_ERR_ARG, "%s: item %d: output lengths do not add up to the slice width", who, base + t);
             b.item[t] = it;
             b.first_block[t] = (int)blocks;
             blocks += (it.width + 63) / 64;
-            if (blocks > (1 << 24)) return fail(HGQ_ERR_UNSUPPORTED, "hgq_reduce_slices_multi: too many columns");
+            if (blocks > (1 << 24)) return fail(HGQ_ERR_UNSUPPORTED, "%s: too many columns", who);
         }
         for (int t = b.count; t <= HGQ_REDUCE_BATCH; ++t) b.first_block[t] = (int)blocks;
-        hipLaunchKernelGGL(reduce_parts_multi_kernel, dim3((unsigned)blocks), dim3(64 * RP_G), 0, (hipStream_t)stream, b);
-        int rc = check_launch("hgq_reduce_slices_multi");
+        if (nq) hipLaunchKernelGGL(reduce_parts_multi_kernel<true>, dim3((unsigned)blocks), dim3(64 * RP_G), 0, (hipStream_t)stream, b, q);
+        else hipLaunchKernelGGL(reduce_parts_multi_kernel<false>, dim3((unsigned)blocks), dim3(64 * RP_G), 0, (hipStream_t)stream, b, q);
+        int rc = check_launch(who);
         if (rc) return rc;
     }
     return HGQ_OK;
+}
+
+extern "C" int hgq_reduce_slices_multi(const hgq_reduce_item *items, int count, void *stream) {
+    return reduce_slices_impl(items, count, nullptr, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int hgq_reduce_slices_quant_multi(const hgq_reduce_item *items, int count, const hgq_quant_grad_item *quants, const int *quant_set,
+                                             const int *quant_segment, int n_quants, void *stream) {
+    return reduce_slices_impl(items, count, quants, quant_set, quant_segment, n_quants, stream);
 }
 
 static inline bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }

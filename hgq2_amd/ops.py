@@ -455,9 +455,15 @@ class _ReduceItem(ctypes.Structure):
 def reduce_slices_multi_op(slices: Sequence[Tensor], outs: Sequence[Tensor], skip: Sequence[bool]) -> None:
     """``outs[3t .. 3t+2]`` (concatenated) = column sums of ``slices[t]`` [n, width], fixed order, all sets in one launch; a
     segment with ``skip`` set has its length in ``outs`` but is not written."""
+    items = _reduce_items(slices, outs, skip)
+    rc = _lib.load().hgq_reduce_slices_multi(items, len(slices), _stream())
+    _lib.check(rc, 'hgq_reduce_slices_multi')
+
+
+def _reduce_items(slices, outs, skip):
     n = len(slices)
     _need(len(outs) == 3 * n and len(skip) == 3 * n, 'three outputs per slice set')
-    items = (_ReduceItem * n)()
+    items = (_ReduceItem * max(n, 1))()
     for t in range(n):
         sl = slices[t]
         _check_f32('slices', sl)
@@ -470,8 +476,37 @@ def reduce_slices_multi_op(slices: Sequence[Tensor], outs: Sequence[Tensor], ski
         for j in range(3):
             items[t].out[j] = o[j].data_ptr() if (o[j].numel() and not skip[3 * t + j]) else None
             items[t].n_out[j] = o[j].numel()
-    rc = _lib.load().hgq_reduce_slices_multi(items, n, _stream())
-    _lib.check(rc, 'hgq_reduce_slices_multi')
+    return items
+
+
+REDUCE_BATCH, REDUCE_QUANTS = 16, 24  # HGQ_REDUCE_BATCH, HGQ_REDUCE_QUANTS
+
+
+@torch.library.custom_op('hgq::reduce_slices_quant_multi', mutates_args=('outs',))
+def reduce_slices_quant_multi_op(slices: Sequence[Tensor], outs: Sequence[Tensor], skip: Sequence[bool], xs: Sequence[Tensor],
+                                 ks: Sequence[Tensor], is_: Sequence[Tensor], fbs: Sequence[Tensor], modes: Sequence[int],
+                                 q_set: Sequence[int], q_segment: Sequence[int]) -> list[Tensor]:
+    """``reduce_slices_multi_op`` with the backward of quantizers whose upstream gradient is a reduced segment run on the
+    sums as they are formed: quantizer j (per-element bit-widths) reads segment ``q_segment[j]`` of slice set ``q_set[j]``.
+    Returns ``dx_0 .., di_0 .., dfb_0 ..`` as ``quantize_bwd_multi`` does."""
+    items = _reduce_items(slices, outs, skip)
+    _check_multi(xs, ks, is_, fbs, modes)
+    n = len(xs)
+    _need(len(q_set) == n and len(q_segment) == n, 'one slice set and segment per quantizer')
+    dxs, dis, dfs = [torch.empty_like(x) for x in xs], [torch.empty_like(i) for i in is_], [torch.empty_like(f) for f in fbs]
+    quants = (_QuantGradItem * max(n, 1))()
+    for t in range(n):
+        quants[t] = _QuantGradItem(0, xs[t].data_ptr(), ks[t].data_ptr(), is_[t].data_ptr(), fbs[t].data_ptr(), dxs[t].data_ptr(),
+                                   dis[t].data_ptr(), dfs[t].data_ptr(), xs[t].numel(), _kmode(modes[t], ks[t]))
+    sets, segs = (ctypes.c_int * max(n, 1))(*q_set), (ctypes.c_int * max(n, 1))(*q_segment)
+    rc = _lib.load().hgq_reduce_slices_quant_multi(items, len(slices), quants, sets, segs, n, _stream())
+    _lib.check(rc, 'hgq_reduce_slices_quant_multi')
+    return dxs + dis + dfs
+
+
+@reduce_slices_quant_multi_op.register_fake
+def _(slices, outs, skip, xs, ks, is_, fbs, modes, q_set, q_segment):
+    return [torch.empty_like(x) for x in xs] + [torch.empty_like(i) for i in is_] + [torch.empty_like(f) for f in fbs]
 
 
 # ---- slice reductions whose results nothing reads before the kernel / bias quantizers' backward or the optimizer:
@@ -487,6 +522,33 @@ def flush_reductions():
         sl.append(s_), outs.extend(o_), skip.extend(k_)
     _PENDING_REDUCE.clear()
     reduce_slices_multi_op(sl, outs, skip)
+
+
+def _reduce_and_quantize_bwd(dys, xs, ks, is_, fbs, modes):
+    """The pending slice reductions and the backward of the quantizers ``xs`` in ONE launch, when every upstream gradient in
+    ``dys`` is a whole segment of a pending reduction (the kernel / bias gradients a contraction's backward left as slices):
+    the quantizer backward then runs on the sums as they are formed.  Returns what ``quantize_bwd_multi`` returns, or ``None``
+    when the gradients come from elsewhere (the caller flushes and launches the two separately)."""
+    if not _PENDING_REDUCE or not dys or len(dys) > REDUCE_QUANTS or len(_PENDING_REDUCE) > REDUCE_BATCH:
+        return None
+    where = {}
+    for t, (_, outs, _) in enumerate(_PENDING_REDUCE):
+        for seg, o in enumerate(outs):
+            if o.numel():
+                where[(o.data_ptr(), o.numel())] = (t, seg)
+    q_set, q_seg = [], []
+    for dy, x in zip(dys, xs):
+        hit = where.pop((dy.data_ptr(), dy.numel()), None) if dy.numel() == x.numel() and dy.numel() else None
+        if hit is None:
+            return None
+        q_set.append(hit[0]), q_seg.append(hit[1])
+    sl, outs, skip = [], [], []
+    for s_, o_, k_ in _PENDING_REDUCE:
+        sl.append(s_), outs.extend(o_), skip.extend(k_)
+    for t, seg in zip(q_set, q_seg):
+        skip[3 * t + seg] = True  # read by the quantizer's backward inside the launch and by nothing else
+    _PENDING_REDUCE.clear()
+    return reduce_slices_quant_multi_op(sl, outs, skip, list(xs), list(ks), list(is_), list(fbs), list(modes), q_set, q_seg)
 
 
 def _dense_ebops_check(amax, beta, k_in, i_in, f_in, k_ker, b_ker, k_bias, b_bias, ebops_var, P, K, N, mode_in, mode_ker, mode_bias):
@@ -2094,14 +2156,16 @@ class _QuantizeMulti(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, *gys):
-        flush_reductions()
         n, t = ctx.n, ctx.saved_tensors
         xs, ks, is_, fbs = t[:n], t[n:2 * n], t[2 * n:3 * n], t[3 * n:]
         for mode in ctx.modes:
             if not (mode & _lib.MODE_TRAINING):
                 raise RuntimeError('hgq quantizer: gradients are defined for the training-mode forward only')
         dys = [x.new_empty(0) if g is None else g.contiguous() for g, x in zip(gys, xs)]
-        out = quantize_bwd_multi(dys, list(xs), list(ks), list(is_), list(fbs), list(ctx.modes))
+        out = _reduce_and_quantize_bwd(dys, xs, ks, is_, fbs, ctx.modes)
+        if out is None:
+            flush_reductions()
+            out = quantize_bwd_multi(dys, list(xs), list(ks), list(is_), list(fbs), list(ctx.modes))
         need = ctx.needs_input_grad[2:]
         grads = list(out[:n]) + [None] * n + list(out[n:])
         return (None, None) + tuple(g if need[j] else None for j, g in enumerate(grads))

@@ -368,6 +368,17 @@ int hgq_qdense_bwd_slices(const float *dy, const float *y, const float *x, const
                           const float *qw, float *dx, float *workspace, int has_bias, int64_t rows, int K, int N, int act,
                           int mode, void *stream);
 int hgq_reduce_slices_multi(const hgq_reduce_item *items, int count, void *stream);
+/*
+ * hgq_reduce_slices_multi with the backward of quantizers whose upstream gradient is one of the reduced segments - the kernel
+ * and bias quantizers behind a contraction (src/hgq/layers/core/dense.py:60-68: `qkernel = self.kq(self.kernel)`) - run on
+ * the sums as they are formed: quantizer j (hgq_quant_grad_item, its `dy` ignored, n = the segment's length, per-element
+ * bit-widths) reads segment quant_segment[j] of slice set quant_set[j] and writes dx / di / dfb exactly as
+ * hgq_quantize_bwd_multi would from the reduced array.  At most HGQ_REDUCE_QUANTS quantizers per HGQ_REDUCE_BATCH consecutive
+ * slice sets, one per segment; a segment's own output pointer may then be NULL.
+ */
+#define HGQ_REDUCE_QUANTS 24
+int hgq_reduce_slices_quant_multi(const hgq_reduce_item *items, int count, const hgq_quant_grad_item *quants, const int *quant_set,
+                                  const int *quant_segment, int n_quants, void *stream);
 
 /*
  * EBOPs of a dense contraction and its gradient.  Replaces QDense._compute_ebops

@@ -559,9 +559,10 @@ def test_gradient_sink_gives_the_autograd_update(dev, kind, monkeypatch):
     b(xd, training=True)
     b.load_state_dict(a.state_dict())
     opt_a, opt_b = SGD(a.parameters(), lr=0.05, fold_regularizers=True), SGD(b.parameters(), lr=0.05, fold_regularizers=True)
-    joined = []  # slice sets per joint reduction launch
-    plain_reduce = ops.reduce_slices_multi_op
+    joined = []  # slice sets per joint reduction launch (with the kernel / bias quantizers' backward inside it where it applies)
+    plain_reduce, quant_reduce = ops.reduce_slices_multi_op, ops.reduce_slices_quant_multi_op
     monkeypatch.setattr(ops, 'reduce_slices_multi_op', lambda sl, outs, skip: (joined.append(len(sl)), plain_reduce(sl, outs, skip))[1])
+    monkeypatch.setattr(ops, 'reduce_slices_quant_multi_op', lambda sl, *a: (joined.append(len(sl)), quant_reduce(sl, *a))[1])
     for step in range(2):
         opt_a.zero_grad()
         la = model_loss(a, loss_fn(a(xd, training=True)), True)
