@@ -641,12 +641,12 @@ __device__ __forceinline__ floatx16 bf16_chain(floatx16 acc, bf16_planes_t xp, i
 // OQ: the layer's output quantizer (training-mode WRAP: round only, [Po, N] table of fractional bits, same round mode)
 // runs on the output tile as it leaves: `y` gets the contraction, `yq` its quantized values, slice blockIdx.x of
 // `oamax_part` the abs-max of the quantized values per table entry.
-// ymean (mean_rows = 32 or 64, rows a multiple of it): the output itself is not written; row g of `ymean`
+// MEAN (`ymean`; mean_rows = 32 or 64, rows a multiple of it): the output itself is not written; row g of `ymean`
 // [rows / mean_rows, N] = the mean of the activated output rows g * mean_rows .. (g + 1) * mean_rows - 1, taken from the
 // accumulator registers (a tile holds two groups or one): sixteen rows per lane in order, the two lane halves, then the two
 // row halves.  With ReLU, `relu_mask` [rows][2] gets a bit per output - bit c & 31 of word c >> 5 of a row says that column c
 // was positive - which is all the backward pass needs of the output.
-template <int RM, bool QUANT, int NS, bool OQ = false>
+template <int RM, bool QUANT, int NS, bool OQ = false, bool MEAN = false>
 __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw,
                                                               const float *__restrict__ qb, float *__restrict__ y,
@@ -660,8 +660,8 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
     __shared__ __attribute__((aligned(16))) float ys[FAST_BM][FAST_XLD];
     // ymean: column sums of the two row halves of a tile and the tile's ReLU mask words (written out as one contiguous run);
     // two sets in turn - a tile's set is written out behind the NEXT tile's staging barrier, so the tile needs no barrier of its own
-    __shared__ float msum[2][2][64];
-    __shared__ uint32_t mtile[2][FAST_BM][2];
+    __shared__ float msum[MEAN ? 2 : 1][2][64];
+    __shared__ uint32_t mtile[MEAN ? 2 : 1][FAST_BM][2];
     // bit 0 / 1: the staged tile has a non-zero second / third part.  Three slots in rotation: the slot of the tile after
     // next is cleared behind this tile's barrier - its last readers passed that barrier, its next writers come after the next one
     __shared__ uint32_t need[3];
@@ -761,14 +761,14 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         if (tid == 0) need[slot == 0 ? 2 : slot - 1] = 0u;  // (slot + 2) % 3
         const int64_t next = tile + gridDim.x;
         if (next < n_tiles) load_tile(next);
-        if (ymean && mean_tile >= 0) write_means(mean_tile, mean_set ^ 1);
+        if (MEAN && mean_tile >= 0) write_means(mean_tile, mean_set ^ 1);
         floatx16 acc = {0};
         if (cb * 32 < N) {
             acc = bf16_chain<NS>(acc, xp[buf], arow, kq, need[slot], wp, PW);
         }
         DB_STAMP(0, 4 + 6 * it_);
         const int64_t r0 = tile * FAST_BM;
-        if (ymean) {
+        if (MEAN) {
             // no branch inside the loop: the mask words are formed whatever the activation and only written out with ReLU
             const bool relu = act == HGQ_ACT_RELU;
             float csum = 0.f;
@@ -837,7 +837,7 @@ __global__ __launch_bounds__(256, 2) void qdense_fwd_bf16_kernel(const float *__
         }
     }
     DB_STAMP(0, 30);
-    if (ymean && mean_tile >= 0) {
+    if (MEAN && mean_tile >= 0) {
         __syncthreads();
         write_means(mean_tile, mean_set ^ 1);
     }
@@ -2079,10 +2079,10 @@ extern "C" int hgq_qdense_fwd_mean(const float *x, const float *f_in, int64_t bw
     const int P = quant ? (int)bw_rows : 1, mr = (int)mean_rows;
 #define HGQ_FWD_MEAN(NSV) \
     do { \
-        if (!quant) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, false, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, (uint32_t *)nullptr, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
-        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
-        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
-        else hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND_CONV, true, NSV>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
+        if (!quant) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, false, NSV, false, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, (uint32_t *)nullptr, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
+        else if (m.round_mode == HGQ_TRN) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_TRN, true, NSV, false, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
+        else if (m.round_mode == HGQ_RND) hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND, true, NSV, false, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
+        else hipLaunchKernelGGL((qdense_fwd_bf16_kernel<HGQ_RND_CONV, true, NSV, false, true>), fgrid, dim3(256), 0, s, x, f_in, P, qw, qb, (float *)nullptr, amax_part, rows, K, N, act, mode, (const float *)nullptr, 1, 0, (float *)nullptr, (uint32_t *)nullptr, ymean, mr, relu_mask); \
     } while (0)
     if (K <= 16) HGQ_FWD_MEAN(1);
     else if (K <= 32) HGQ_FWD_MEAN(2);
