@@ -1060,7 +1060,7 @@ __global__ __launch_bounds__(256, 2) void dense_moments_bf16_kernel(const float 
 // contract are split into bf16 parts once for both), wavefronts 2 and 3 the two column halves of the kernel gradient (both k
 // blocks, all rows of the tile) - every gradient value is split twice per tile instead of four times.  A wavefront's two
 // blocks live in the same registers either way: reset per tile for dx, kept across the tiles for the kernel gradient.
-template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true, bool BF = false, bool PAIRS = false, int BCAST = 0>
+template <int RM, bool QUANT, bool STATS = false, bool ZVEC = true, bool BF = false, bool PAIRS = false, int BCAST = 0, bool NOACT = false>
 __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__restrict__ dy, const float *__restrict__ y,
                                                               const float *__restrict__ x, const float *__restrict__ f_in,
                                                               int P, const float *__restrict__ qw, float *__restrict__ dx,
@@ -1102,7 +1102,8 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     floatx16 accw = {0}, acc2 = {0};  // acc2: the second block of a wavefront with PAIRS
     float accb = 0.f;
     const int bn = tid & 63, bq = tid >> 6;
-    const bool relu = act == HGQ_ACT_RELU;
+    // NOACT: launched without activation - the forward output is then neither asked for nor kept in registers
+    const bool relu = !NOACT && act == HGQ_ACT_RELU;
 
     f32x4_t rx[FAST_NJ], rg[FAST_NJ], ry[FAST_NJ];
     uint32_t xoff[FAST_NJ], zoff[FAST_NJ];
@@ -1132,7 +1133,8 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
                     const uint32_t goff = !bcast ? zoff[j]
                                           : mz.on[j] ? (uint32_t)((bcast == 32 ? (mz.row[j] >> 5) : 0) * N + mz.col[j]) * 4u : BUF_OOB;
                     rg[j] = buf_ld4(sg, goff);
-                    if (bcast) ry[j][0] = buf_ld1(sy, mz.on[j] ? (uint32_t)(mz.row[j] * 2 + (mz.col[j] >> 5)) * 4u : BUF_OOB);  // mask word
+                    if (NOACT) ry[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    else if (bcast) ry[j][0] = buf_ld1(sy, mz.on[j] ? (uint32_t)(mz.row[j] * 2 + (mz.col[j] >> 5)) * 4u : BUF_OOB);  // mask word
                     else ry[j] = buf_ld4(sy, zoff[j]);
                 } else {
 #pragma unroll
@@ -2255,7 +2257,10 @@ static int qdense_bwd_impl(const float *dy, const float *y, const float *x, cons
     } while (0)
 #define HGQ_BWD_FAST(RMV, QV)                                                                                                          \
     do {                                                                                                                               \
-        if (zvec && g_dense_bf16 && K > 32 && N > 32)                                                                                  \
+        if (zvec && g_dense_bf16 && K > 32 && N > 32 && act == HGQ_ACT_NONE)                                                           \
+            hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true, true, true, 0, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, \
+                               workspace, dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                 \
+        else if (zvec && g_dense_bf16 && K > 32 && N > 32)                                                                             \
             hipLaunchKernelGGL((qdense_bwd_fast_kernel<RMV, QV, false, true, true, true>), fgrid, dim3(256), 0, s, dy, y, x, f_in, P, qw, dx, workspace, \
                                dqb ? 1 : 0, rows, K, N, act, mode, (const float *)nullptr);                                            \
         else if (zvec && g_dense_bf16)                                                                                                 \
