@@ -675,7 +675,9 @@ __global__ __launch_bounds__(1024) void qattn_amax_reduce_kernel(const uint32_t 
 // ([n_wg, 8] shared-quantizer sums | [n_wg, N * T * S] d/df of the output quantizer).  The output
 // quantizer, if present, wraps (only rounds in training): its input gradient is the identity and
 // only its fractional bits take gradient; they are packed four to a register.
-template <int HD, int TH, int ST, bool MASKED>
+// BF: the contractions on the bf16 matrix instruction (exact parts) or on the fp32 one - a template argument, not a branch:
+// with both forms in one kernel the register allocation spilled 80 bytes per lane more
+template <int HD, int TH, int ST, bool MASKED, bool BF>
 __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restrict__ dout, const float *__restrict__ q,
                                                           const float *__restrict__ k, const float *__restrict__ v,
                                                           float *__restrict__ dq_, float *__restrict__ dk_, float *__restrict__ dv_,
@@ -767,8 +769,8 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
         }
         if (active) {
             if (MASKED) load_keep<ST>(mk, b, T, S, t0 + t_l, hf, keep);
-            score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, xs, pl.bf != 0);        // scores, transposed
-            score_tiles<HD, ST, true>(Vs, Gs, t0, col0, t_l, hf, ga, pl.bf != 0);  // d probs = dout value^T, transposed
+            score_tiles<HD, ST>(Ks, Qs, t0, col0, t_l, hf, xs, BF);        // scores, transposed
+            score_tiles<HD, ST, true>(Vs, Gs, t0, col0, t_l, hf, ga, BF);  // d probs = dout value^T, transposed
             QA_STAMP(3);
             if (MASKED) {
 #pragma unroll
@@ -855,7 +857,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
 #pragma unroll
             for (int st = 0; st < ST; ++st)
                 if (st % TH == th) {
-                    const floatx16 o = contract_queries<TH, true, false>(Gs, col0, head_buf, st * 32, t_l, hf, pl.bf != 0, HD);
+                    const floatx16 o = contract_queries<TH, true, false>(Gs, col0, head_buf, st * 32, t_l, hf, BF, HD);
                     store_rows<HD>(o, dv_ + ((int64_t)b * S * pl.N + h) * HD, (int64_t)pl.N * HD, st * 32 + t_l, hf);
                 }
             QA_STAMP(7);
@@ -961,7 +963,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
         }
         if (active) {
             // dquery[t][h] = sum_s dscores[t][s] key[s][h]
-            const floatx16 o = contract_keys<ST, true>(Ks, col0, t_l, hf, ga, pl.bf != 0, HD);
+            const floatx16 o = contract_keys<ST, true>(Ks, col0, t_l, hf, ga, BF, HD);
             store_rows<HD>(o, dq_ + ((int64_t)b * T * pl.N + h) * HD, (int64_t)pl.N * HD, t0 + t_l, hf);
         }
         QA_STAMP(9);
@@ -974,7 +976,7 @@ __global__ __launch_bounds__(QA_NT) void qattn_bwd_kernel(const float *__restric
             // dkey[s][h] = sum_t dscores[t][s] query[t][h]
 #pragma unroll
             for (int st = 0; st < ST; ++st)
-                if (st % TH == th) dk_prev = contract_queries<TH, false, true>(Qs, col0, head_buf, st * 32, t_l, hf, pl.bf != 0, HD);
+                if (st % TH == th) dk_prev = contract_queries<TH, false, true>(Qs, col0, head_buf, st * 32, t_l, hf, BF, HD);
             b_prev = b;
         }
         QA_STAMP(12);
@@ -1194,9 +1196,9 @@ extern "C" int hgq_qattention_bwd(const float *dout, const float *query, const f
           aligned16(dvalue) && aligned16(workspace)))
         return fail(HGQ_ERR_ARG, "hgq_qattention_bwd: operands and workspace must be 16-byte aligned");
     const size_t lds = qattn_lds_bytes(T, S, true);
-#define QA_BWD(MASKV)                                                                                                            \
+#define QA_BWD(MASKV, BFV)                                                                                                       \
     QA_DISPATCH(H, T, {                                                                                                          \
-        auto kern = qattn_bwd_kernel<HD, TH, TH, MASKV>;                                                                         \
+        auto kern = qattn_bwd_kernel<HD, TH, TH, MASKV, BFV>;                                                                    \
         static bool raised = false;                                                                                              \
         if (!raised && (rc = raise_lds(kern, lds, "hgq_qattention_bwd"))) return rc;                                             \
         raised = true;                                                                                                           \
@@ -1204,8 +1206,13 @@ extern "C" int hgq_qattention_bwd(const float *dout, const float *query, const f
                            input_scaler, eps, softmax_desc_or_none(exp_iq), softmax_desc_or_none(exp_oq),                        \
                            softmax_desc_or_none(inv_iq), softmax_desc_or_none(inv_oq), softmax_desc_or_none(oq), workspace, mk); \
     })
-    if (mask || causal) QA_BWD(true);
-    else QA_BWD(false);
+    if (pl.bf) {
+        if (mask || causal) QA_BWD(true, true);
+        else QA_BWD(false, true);
+    } else {
+        if (mask || causal) QA_BWD(true, false);
+        else QA_BWD(false, false);
+    }
 #undef QA_BWD
     if ((rc = check_launch("hgq_qattention_bwd"))) return rc;
     // a wrapping quantizer's integer bits take no gradient: the reduction writes zeros there
