@@ -1074,8 +1074,9 @@ __global__ __launch_bounds__(256, 2) void qdense_bwd_fast_kernel(const float *__
     const bool has_add = STATS && dx_add != nullptr;
     const Mode m(mode);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int K32 = (K + 31) >> 5, N32 = (N + 31) >> 5;
-    const bool split_n = K32 == 1 && N32 == 2;
+    // (PAIRS is launched with K and N above 32 only: both block counts are 2 and known when the kernel is compiled)
+    const int K32 = PAIRS ? 2 : (K + 31) >> 5, N32 = PAIRS ? 2 : (N + 31) >> 5;
+    const bool split_n = !PAIRS && K32 == 1 && N32 == 2;
     const int PK = QUANT ? P * K : 0;
     const int64_t M = (int64_t)K * N + N + PK;
     const int64_t n_tiles = (rows + FAST_BM - 1) / FAST_BM;
