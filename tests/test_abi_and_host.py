@@ -178,6 +178,26 @@ def test_entry_points_validate_arguments_before_any_launch():
     assert lib.hgq_qdense_bwd(none, none, none, none, 0, none, none, none, none, none, none, 128, 80, 10, 0, 0, none) == UNSUPPORTED
     assert lib.hgq_col_moments_workspace(1000, 64) > 0 and lib.hgq_col_moments_workspace(-1, 64) == -1
     assert lib.hgq_col_moments_fwd(none, 0, 64, none, none, none, none) == ARG
+    # contraction + mean over row groups: groups of 32 or 64 rows only, widths multiples of 4 up to 64
+    WRAP_TRAIN = _lib.mode_bits('RND', 'WRAP', training=True)
+    assert lib.hgq_qdense_fwd_mean_supported(4096, 64, 32, 64, 64, WRAP_TRAIN) == 1
+    assert lib.hgq_qdense_fwd_mean_supported(4096, 64, 32, 64, 48, WRAP_TRAIN) == 0    # groups of 48 rows
+    assert lib.hgq_qdense_fwd_mean_supported(4096, 64, 30, 0, 64, 0) == 0              # N not a multiple of 4
+    assert lib.hgq_qdense_fwd_mean_supported(4100, 64, 32, 0, 64, 0) == 0              # rows not whole groups
+    assert lib.hgq_qdense_fwd_mean(none, none, 0, none, none, none, none, none, 4096, 64, 32, 48, 0, 0, none) == UNSUPPORTED
+    assert lib.hgq_qdense_fwd_mean(none, none, 0, none, none, none, none, none, 4096, 64, 32, 64, 0, 0, none) == ARG  # null pointers
+    assert lib.hgq_qdense_fwd_mean(none, none, 0, none, none, none, none, none, 0, 64, 32, 64, 0, 0, none) == OK
+    assert lib.hgq_qdense_bwd_mean_slices(one, none, one, none, 0, one, one, one, 0, 4096, 64, 32, 48, 0, 0, none) == UNSUPPORTED
+    assert lib.hgq_qdense_bwd_mean_slices(one, none, one, none, 0, one, one, one, 0, 4096, 64, 32, 0, 0, 0, none) == ARG
+    # batch feed, quantizer wrapper, pooling EBOPs, reduction with quantizers attached
+    assert lib.hgq_gather_batch(none, 64, none, 8, none, none, none, none, 16, 100, none) == ARG           # null pointers
+    assert lib.hgq_gather_batch(one, 6, one, 8, one, one, one, one, 16, 100, none) == ARG and b'32-bit' in lib.hgq_last_error()
+    assert lib.hgq_quantizer_scale_div(none, none, 0, 2.0, none) == OK and lib.hgq_quantizer_scale_div(none, none, 8, 2.0, none) == ARG
+    assert lib.hgq_quantizer_tail_fwd(one, none, one, 8, 0, 1.0, 1, 0.5, 0, 1.0, 0.0, none) == ARG and b'noise' in lib.hgq_last_error()
+    assert lib.hgq_quantizer_tail_bwd(one, one, none, 8, 0, 1.0, 1, 0.5, 0, 1.0, none) == ARG
+    assert lib.hgq_sum_ebops(none, 0, 1.0, 1.0, 1.0, none, none, none, none) == UNSUPPORTED
+    assert lib.hgq_reduce_slices_quant_multi(none, 1, none, none, none, 0, none) == ARG
+    assert lib.hgq_reduce_slices_quant_multi(none, 0, none, none, none, 2, none) == ARG
 
 
 def test_a_second_thread_inside_a_training_step_is_refused():
